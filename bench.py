@@ -1,0 +1,173 @@
+"""Headline benchmark: multi-step LIF forward+backward, T=16, N=33.5M neurons, fp32, one MI355X.
+
+One "step" is one forward plus one backward of ``LIFNode(step_mode='m', backend='hip',
+store_v_seq=True)`` over x [16,256,128,32,32] (tau=2, hard reset to 0, ATan(2)), with upstream
+gradients for both the spikes and v_seq, inputs resident in HBM.  Prints ONE JSON line:
+``value`` = T*N / seconds per step (neuron-steps/s); ``roofline`` = algorithmic bytes of the slower of
+the two kernels / its mean duration measured with HIP events on the launch stream, against the 8 TB/s
+HBM3E peak; ``cpu_baseline`` = the torch-ops port of the reference's CPU backend timed on this host on
+a bounded sample of the same workload.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+T_STEPS = 16
+SHAPE = (T_STEPS, 256, 128, 32, 32)
+
+
+def cpu_baseline(torch, sample_neurons: int, repeats: int):
+    """torch-ops port of the reference torch backend (oracle/neuron_oracle.py), forward + autograd
+    backward, on ``sample_neurons`` neurons x T=16 of the same input distribution."""
+    from oracle import neuron_oracle as no
+
+    cores = torch.get_num_threads()
+    g = torch.Generator().manual_seed(1002)
+    x = torch.randn((T_STEPS, sample_neurons), generator=g) * 0.8 + 0.3
+    gs = torch.randn((T_STEPS, sample_neurons), generator=g)
+    gv = torch.randn((T_STEPS, sample_neurons), generator=g) * 0.1
+    v0 = torch.zeros(sample_neurons)
+    times = []
+    for i in range(repeats + 1):
+        t0 = time.perf_counter()
+        no.forward_backward("lif", x, v0, gs, gv, None, 2.0, True, 1.0, 0.0, "atan", 2.0, False)
+        dt = time.perf_counter() - t0
+        if i > 0:  # first run is the warm-up
+            times.append(dt)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": T_STEPS * sample_neurons / med,
+        "unit": "neuron-steps/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"N={sample_neurons} neurons x T={T_STEPS}, fwd+autograd bwd, median of {repeats} after 1 warm-up, "
+                  f"{med * 1e3:.0f} ms each",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--cpu-sample-neurons", type=int, default=1 << 23)
+    ap.add_argument("--cpu-repeats", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the path shards over neurons with no exchange, and this build runs "
+              "on single-GPU boxes only; run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from spikingjelly_amd.activation_based import functional, neuron, surrogate
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+
+    L.load()
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm device", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    N = 1
+    for d in SHAPE[1:]:
+        N *= d
+
+    # inputs: CPU generator with the configured seeds, then resident on the device
+    def make(seed, mean, std):
+        g = torch.Generator().manual_seed(seed)
+        return (torch.randn(SHAPE, generator=g) * std + mean).to(dev)
+
+    x = make(1002, 0.3, 0.8).requires_grad_()
+    grad_spike = make(1102, 0.0, 1.0)
+    grad_v = make(1202, 0.0, 0.1)
+
+    node = neuron.LIFNode(tau=2.0, v_threshold=1.0, v_reset=0.0, surrogate_function=surrogate.ATan(2.0),
+                          step_mode="m", backend="hip", store_v_seq=True).to(dev)
+
+    def step():
+        spikes = node(x)
+        torch.autograd.backward([spikes, node.v_seq], [grad_spike, grad_v])
+        x.grad = None
+        functional.reset_net(node)
+        return spikes
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    L.profile_reset()
+    L.profile_enable(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        spikes = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    L.profile_enable(False)
+    rate = float(spikes.mean())
+    n_fwd, ms_fwd = L.profile_read(L.KC_FORWARD)
+    n_bwd, ms_bwd = L.profile_read(L.KC_BACKWARD)
+
+    ms_per_step = elapsed / args.steps * 1e3
+    value = T_STEPS * N / (elapsed / args.steps)
+
+    # algorithmic bytes per launch: each tensor of the operator contract touched once
+    fwd_bytes = 16 * T_STEPS * N + 4 * N  # x, spike, v_seq, h_seq per step + v_init
+    bwd_bytes = 16 * T_STEPS * N + 4 * N  # grad_spike, grad_v, h_seq, grad_x per step + grad_v_init
+    fwd_ms = ms_fwd / max(n_fwd, 1)
+    bwd_ms = ms_bwd / max(n_bwd, 1)
+    dominant = "forward" if fwd_ms >= bwd_ms else "backward"
+    dom_ms, dom_bytes = (fwd_ms, fwd_bytes) if dominant == "forward" else (bwd_ms, bwd_bytes)
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic_lif_fp32_T16_N33554432.json")
+    if os.path.exists(tpath):  # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs
+        with open(tpath) as f:
+            traffic = json.load(f).get(dominant)
+
+    out = {
+        "metric": "neuron-steps/sec LIF fwd+bwd T=16 N=33.5M, 1 MI355X; % of HBM roofline",
+        "value": value,
+        "unit": "neuron-steps/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: LIFNode multi-step fwd+bwd, x [16,256,128,32,32] fp32 ~N(0.3,0.8), tau=2, "
+                               "hard reset 0, ATan(2), store_v_seq=True, grad_spike ~N(0,1), grad_v ~N(0,0.1)",
+                   "T": T_STEPS, "N": N, "backend": "hip", "firing_rate": rate},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": dominant,
+                     "kernel_ms": dom_ms, "algorithmic_bytes": dom_bytes,
+                     "forward_ms": fwd_ms, "backward_ms": bwd_ms,
+                     "forward_GBs": fwd_bytes / (fwd_ms * 1e-3) / 1e9 if fwd_ms else None,
+                     "backward_GBs": bwd_bytes / (bwd_ms * 1e-3) / 1e9 if bwd_ms else None,
+                     "fwd_plus_bwd_frac": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS
+                     if (fwd_ms + bwd_ms) else None},
+    }
+    del x, grad_spike, grad_v, spikes
+    torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, args.cpu_sample_neurons, args.cpu_repeats)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,178 @@
+/*
+ * sjhip.h -- C ABI of libsjhip.so: multi-step spiking-neuron kernels for
+ * AMD MI355X (gfx950), hand-written HIP.
+ *
+ * Every entry point is asynchronous on the HIP stream it is given, owns no
+ * device memory, never synchronises the host and never throws: it returns
+ * SJHIP_OK (0) or a negative sjhip_status and leaves a thread-local message
+ * for sjhip_last_error().  All tensors are dense row-major [T, N] views
+ * ("time outer, neurons contiguous") of device memory owned by the caller.
+ *
+ * Reference interfaces these entry points stand in for (paths relative to the
+ * SpikingJelly source tree):
+ *   sjhip_neuron_forward   <- torch.ops.sj.cupy_multistep_{if,lif,plif}_forward
+ *                             spikingjelly/activation_based/cuda_kernel/neuron_kernel/multi_step/lif.py:144-192,
+ *                             plif.py:288-386, integrate_and_fire.py:76-147; and
+ *                             torch.ops.sj.multistep_{if,lif,plif}_{forward,inference}
+ *                             spikingjelly/activation_based/triton_kernel/neuron_kernel/lif.py:673-763
+ *   sjhip_neuron_backward  <- torch.ops.sj.cupy_multistep_{if,lif,plif}_backward
+ *                             multi_step/lif.py:228-282, plif.py:389-470, integrate_and_fire.py:150-200;
+ *                             BPTT body multi_step/base.py:137-409
+ *   sjhip_plif_workspace_floats / grad_rtau reduction
+ *                          <- shared-memory tree + atomicAdd in multi_step/plif.py:107-237 and the
+ *                             per-neuron partials + torch.sum of triton_kernel/neuron_kernel/plif.py:340-378,1180-1203
+ *   sjhip_bit_pack/unpack  <- bit_spike_compress / bit_spike_decompress,
+ *                             spikingjelly/activation_based/triton_kernel/compress.py:114-221 (torch fallback :19-44),
+ *                             and float2bool/bool2float of cuda_kernel/tensor_cache.py:16-93
+ */
+#ifndef SJHIP_H_
+#define SJHIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SJHIP_ABI_VERSION 1
+
+typedef enum sjhip_status {
+  SJHIP_OK = 0,
+  SJHIP_ERR_INVALID = -1,     /* bad enum / flag / NULL / size / alignment */
+  SJHIP_ERR_UNSUPPORTED = -2, /* valid request this build has no kernel for */
+  SJHIP_ERR_LAUNCH = -3,      /* HIP reported an error at launch */
+  SJHIP_ERR_TOO_LARGE = -4    /* size beyond a documented limit */
+} sjhip_status;
+
+/* Neuron model: charge equation applied before fire/reset. */
+typedef enum sjhip_neuron {
+  SJHIP_NEURON_IF = 0,  /* h = v + x                                  (functional/neuron.py:310)   */
+  SJHIP_NEURON_LIF = 1, /* h = v + (x - (v - vr)) / tau  or  v - (v - vr)/tau + x   (:849-852)     */
+  SJHIP_NEURON_PLIF = 2 /* h = v + (x - (v - vr)) * k    or  v - (v - vr)*k + x     (:1290-1295)   */
+} sjhip_neuron;
+
+/* Storage dtype of every [T,N] / [N] tensor of one call. */
+typedef enum sjhip_dtype {
+  SJHIP_F32 = 0,
+  SJHIP_F16 = 1,
+  SJHIP_BF16 = 2,
+  SJHIP_U8 = 3 /* bit_pack / bit_unpack only */
+} sjhip_dtype;
+
+/* Surrogate gradient used by the backward pass (forward is always Heaviside).
+ * Ids follow triton_kernel/surrogate_kernel.py:26-34. */
+typedef enum sjhip_surrogate {
+  SJHIP_SG_SIGMOID = 0,
+  SJHIP_SG_ATAN = 1,
+  SJHIP_SG_PIECEWISE_QUADRATIC = 2,
+  SJHIP_SG_PIECEWISE_EXP = 3,
+  SJHIP_SG_SOFT_SIGN = 4,
+  SJHIP_SG_SUPER_SPIKE = 5,
+  SJHIP_SG_ERF = 6
+} sjhip_surrogate;
+
+/* Bit flags. */
+#define SJHIP_FLAG_DECAY_INPUT 0x01u  /* LIF/PLIF: input is scaled by 1/tau */
+#define SJHIP_FLAG_SOFT_RESET 0x02u   /* v = h - s*v_th ; otherwise hard reset to v_reset */
+#define SJHIP_FLAG_DETACH_RESET 0x04u /* backward: no gradient through the reset branch */
+#define SJHIP_FLAG_FP32_STATE 0x10u   /* 16-bit storage: keep v and all arithmetic in fp32, round only
+                                         what is stored (the reference's mixed-precision ops,
+                                         triton_kernel/neuron_kernel/lif.py:787-870).  Without it 16-bit
+                                         storage rounds after every arithmetic op, like the torch backend. */
+#define SJHIP_FLAG_RECIPROCAL_TAU 0x20u /* LIF: multiply by fl(1/tau) instead of dividing by tau (what the
+                                           CuPy/Triton kernels and torch-on-GPU do); default is the IEEE
+                                           division of the torch CPU backend. */
+#define SJHIP_FLAG_ATOMIC_REDUCE 0x80u /* PLIF backward: one atomicAdd per block into grad_rtau (caller
+                                          zeroes it) instead of the deterministic two-pass reduction */
+
+/* Scalars of one neuron layer.  `tau` is tau for LIF and the reciprocal k = sigmoid(w) for PLIF
+ * (ignored for IF).  `v_reset` is ignored for IF soft reset and is the charge-equation offset
+ * (0 when the module has v_reset=None) otherwise. */
+typedef struct sjhip_neuron_params {
+  float tau;
+  float v_threshold;
+  float v_reset;
+  float sg_alpha;   /* backward only */
+  int32_t sg_id;    /* backward only, sjhip_surrogate */
+  uint32_t flags;
+} sjhip_neuron_params;
+
+/* ABI version of the loaded library (== SJHIP_ABI_VERSION it was built with). */
+int sjhip_abi_version(void);
+
+/* Thread-local text of the last error returned on this thread ("" if none). */
+const char *sjhip_last_error(void);
+
+/*
+ * Forward over T steps for N neurons.
+ *   x_seq     [T,N] in            v_init  [N] in
+ *   spike_seq [T,N] out (0/1 in the storage dtype)
+ *   v_seq     [T,N] out, membrane potential after reset at every step; NULL = do not write
+ *   v_last    [N] out, membrane potential after the last step; NULL = do not write
+ *             (at least one of v_seq / v_last must be given)
+ *   h_seq     [T,N] out, membrane potential before reset, saved for backward; NULL = do not write
+ *   rtau_device  PLIF only, may be NULL: device address of one fp32 holding k = sigmoid(w); read by the
+ *             kernel in place of p->tau so that no host synchronisation is needed to fetch it
+ * T >= 1, N >= 1, T*N < 2^62.  128-bit accesses are used when N is a multiple of 16/sizeof(dtype)
+ * and every pointer is 16-byte aligned; otherwise an element-wise kernel runs.
+ */
+int sjhip_neuron_forward(int neuron, int dtype, const sjhip_neuron_params *p,
+                         int64_t T, int64_t N,
+                         const void *x_seq, const void *v_init, const float *rtau_device,
+                         void *spike_seq, void *v_seq, void *v_last, void *h_seq,
+                         void *stream);
+
+/* Number of floats of caller-provided workspace the PLIF backward needs for N neurons of `dtype`
+ * (per-block partial sums of the deterministic reduction). */
+int64_t sjhip_plif_workspace_floats(int dtype, int64_t N);
+
+/*
+ * Backward (BPTT) over T steps.
+ *   grad_spike_seq [T,N] in
+ *   grad_v_seq     [T,N] in, gradient w.r.t. v_seq, or NULL
+ *   grad_v_last    [N] in, gradient w.r.t. v_last (enters at t = T-1), or NULL
+ *   h_seq          [T,N] in (from forward)
+ *   v_init         [N] in, PLIF only (NULL otherwise): v before step 0
+ *   grad_x_seq     [T,N] out         grad_v_init [N] out
+ *   grad_rtau      1 float out, PLIF only: dL/dk, k = sigmoid(w)
+ *   workspace      sjhip_plif_workspace_floats() floats, PLIF without SJHIP_FLAG_ATOMIC_REDUCE
+ */
+int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p,
+                          int64_t T, int64_t N,
+                          const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                          const void *h_seq,
+                          const void *v_init, const float *rtau_device,
+                          void *grad_x_seq, void *grad_v_init,
+                          float *grad_rtau, float *workspace,
+                          void *stream);
+
+/*
+ * Spike bit-packing over a flattened tensor, LSB first: byte j bit i = (src[8j+i] != 0).
+ *   src  n elements of `dtype` (F32/F16/BF16/U8)     dst  (n+7)/8 bytes; pad bits of the last byte are 0
+ */
+int sjhip_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, void *stream);
+
+/* Inverse: dst[8j+i] = (src[j] >> i) & 1 as 0/1 of `dtype`, n elements written. */
+int sjhip_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, void *stream);
+
+/*
+ * Launch tuning (process-wide, read at launch).  key = "fwd_block" or "bwd_block", value = work-items
+ * per block (64, 128, 256 or 512).  Returns SJHIP_ERR_INVALID otherwise.  Results never depend on these.
+ */
+int sjhip_set_tuning(const char *key, int value);
+int sjhip_get_tuning(const char *key);
+
+/*
+ * Optional per-kernel timing.  While enabled every launch is bracketed by HIP events on its own
+ * stream.  sjhip_profile_read() synchronises those events and returns, for kernel class `which`
+ * (0 forward, 1 backward, 2 plif-reduce, 3 bit_pack, 4 bit_unpack), the launch count and total
+ * milliseconds since the last sjhip_profile_reset().
+ */
+int sjhip_profile_enable(int on);
+int sjhip_profile_reset(void);
+int sjhip_profile_read(int which, int64_t *launches, double *total_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SJHIP_H_ */

@@ -1,0 +1,53 @@
+"""Closed-form BPTT of IF / LIF / PLIF in numpy float64.  Test infrastructure only.
+
+Derived from the reference's kernels (``cuda_kernel/neuron_kernel/multi_step/base.py:293-409``;
+LIF hooks ``lif.py:89-102``; PLIF ``plif.py:143-203``) and equal to autograd through
+``functional/neuron.py:225-228, 849-852, 1290-1297``:
+
+    sg_t   = surrogate'(h_t - v_th)         s_t = spike used in the reset branch
+    dvdh_t = hard: (1 - s_t) + [not detach] (v_reset - h_t) sg_t     soft: 1 - [not detach] v_th sg_t
+    G_t    = (G_{t+1} (1 - k) + grad_v_seq[t]) dvdh_t + grad_spike[t] sg_t       (G_T (1-k) := grad_v_last)
+    grad_x[t] = G_t (k if decay_input else 1)        grad_v_init = G_0 (1 - k)
+    PLIF: grad_k = sum G_t dh_t/dk,  dh_t/dk = x_t - (v_{t-1} - vr) (decay_input) or vr - v_{t-1}
+
+with k = 1/tau (LIF) or sigmoid(w) (PLIF); IF uses k = 0 in (1 - k) and factor 1 for grad_x.
+"""
+
+from __future__ import annotations
+
+from typing import Callable, Optional
+
+import numpy as np
+
+
+def bptt(kind: str, h_seq: np.ndarray, s_seq: np.ndarray, sg_prime: Callable[[np.ndarray], np.ndarray],
+         grad_spike_seq: np.ndarray, grad_v_seq: Optional[np.ndarray], grad_v_last: Optional[np.ndarray],
+         k: float, decay_input: bool, v_threshold: float, v_reset: Optional[float], detach_reset: bool,
+         v_prev_seq: Optional[np.ndarray] = None, x_seq: Optional[np.ndarray] = None):
+    """Returns (grad_x [T,N], grad_v_init [N], grad_k float or None)."""
+    T = h_seq.shape[0]
+    h_seq = np.asarray(h_seq, dtype=np.float64)
+    s_seq = np.asarray(s_seq, dtype=np.float64)
+    if kind == "if":
+        kx, km = 1.0, 1.0
+    else:
+        kx, km = (k if decay_input else 1.0), 1.0 - k
+    live = 0.0 if detach_reset else 1.0
+    vr = 0.0 if v_reset is None else v_reset
+    carry = np.zeros_like(h_seq[0]) if grad_v_last is None else np.asarray(grad_v_last, dtype=np.float64).copy()
+    grad_x = np.zeros_like(h_seq)
+    grad_k = 0.0
+    for t in range(T - 1, -1, -1):
+        sg = sg_prime(h_seq[t] - v_threshold)
+        if v_reset is None:
+            dvdh = 1.0 - live * v_threshold * sg
+        else:
+            dvdh = (1.0 - s_seq[t]) + live * (v_reset - h_seq[t]) * sg
+        gv = carry if grad_v_seq is None else carry + grad_v_seq[t]
+        G = gv * dvdh + grad_spike_seq[t] * sg
+        grad_x[t] = G * kx
+        carry = G * km
+        if kind == "plif":
+            dh_dk = (x_seq[t] - (v_prev_seq[t] - vr)) if decay_input else (vr - v_prev_seq[t])
+            grad_k += float(np.sum(G * dh_dk))
+    return grad_x, carry, (grad_k if kind == "plif" else None)

@@ -1,0 +1,280 @@
+"""torch-ops restatement of the reference torch backend (CPU).  Test infrastructure only.
+
+Every arithmetic line cites the reference line it follows (paths relative to
+``spikingjelly/activation_based``).  Op order and scalar handling are kept exactly, because the
+HIP kernels are compared bit for bit against what these ops produce on CPU tensors.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Callable, Optional
+
+import torch
+
+# ------------------------------------------------------------------------------------------------
+# surrogate functions
+# ------------------------------------------------------------------------------------------------
+
+
+def heaviside(x: torch.Tensor) -> torch.Tensor:
+    # surrogate.py:60
+    return (x >= 0).to(x)
+
+
+class _SigmoidSG(torch.autograd.Function):
+    # surrogate.py:811-851 (forward = heaviside) with backward :769-771
+    @staticmethod
+    def forward(ctx, x, alpha):
+        ctx.save_for_backward(x)
+        ctx.alpha = alpha
+        return heaviside(x)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (x,) = ctx.saved_tensors
+        sgax = (x * ctx.alpha).sigmoid_()
+        return grad_output * (1.0 - sgax) * sgax * ctx.alpha, None
+
+
+class _ATanSG(torch.autograd.Function):
+    # surrogate.py:1290-1330 with backward :1247-1250
+    @staticmethod
+    def forward(ctx, x, alpha):
+        ctx.save_for_backward(x)
+        ctx.alpha = alpha
+        return heaviside(x)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (x,) = ctx.saved_tensors
+        a = ctx.alpha / 2
+        ax = math.pi * a * x
+        return a / (1 + ax * ax) * grad_output, None
+
+
+def _sg_backward_other(name: str, grad_output, x, alpha):
+    if name == "piecewise_quadratic":  # surrogate.py:401-407
+        x_abs = x.abs()
+        mask = x_abs > (1 / alpha)
+        return (grad_output * (-(alpha**2) * x_abs + alpha)).masked_fill_(mask, 0)
+    if name == "piecewise_exp":  # surrogate.py:595-596
+        return alpha / 2 * (-alpha * x.abs()).exp_() * grad_output
+    if name == "soft_sign":  # surrogate.py:936-937
+        return grad_output / (2 * alpha * (1 / alpha + x.abs()).pow_(2))
+    if name == "super_spike":  # surrogate.py:1101-1102
+        return alpha * grad_output / torch.pow(torch.abs(x) + 1.0, 2)
+    if name == "erf":  # surrogate.py:1610-1613
+        return grad_output * (-(x * alpha).pow_(2)).exp_() * (alpha / math.sqrt(math.pi))
+    raise ValueError(name)
+
+
+class _OtherSG(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, alpha, name):
+        ctx.save_for_backward(x)
+        ctx.alpha = alpha
+        ctx.name = name
+        return heaviside(x)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (x,) = ctx.saved_tensors
+        return _sg_backward_other(ctx.name, grad_output, x, ctx.alpha), None, None
+
+
+SG_NAMES = ("sigmoid", "atan", "piecewise_quadratic", "piecewise_exp", "soft_sign", "super_spike", "erf")
+SG_IDS = {name: i for i, name in enumerate(SG_NAMES)}  # triton_kernel/surrogate_kernel.py:26-34
+SG_DEFAULT_ALPHA = {"sigmoid": 4.0, "atan": 2.0, "piecewise_quadratic": 1.0, "piecewise_exp": 1.0,
+                    "soft_sign": 2.0, "super_spike": 1.0, "erf": 2.0}
+
+
+def surrogate(name: str, alpha: float, spiking: bool = True) -> Callable[[torch.Tensor], torch.Tensor]:
+    """Callable like a reference surrogate module: spiking -> Heaviside forward + surrogate
+    backward; not spiking -> the smooth primitive."""
+    if spiking:
+        if name == "sigmoid":
+            return lambda x: _SigmoidSG.apply(x, alpha)
+        if name == "atan":
+            return lambda x: _ATanSG.apply(x, alpha)
+        if name in SG_IDS:
+            return lambda x: _OtherSG.apply(x, alpha, name)
+        raise ValueError(name)
+    return lambda x: primitive(name, x, alpha)
+
+
+def primitive(name: str, x: torch.Tensor, alpha: float) -> torch.Tensor:
+    if name == "sigmoid":  # surrogate.py:925-926
+        return (x * alpha).sigmoid()
+    if name == "atan":  # surrogate.py:1404-1405
+        return (math.pi / 2 * alpha * x).atan_() / math.pi + 0.5
+    if name == "piecewise_quadratic":  # surrogate.py:582-588
+        mask0 = (x > (1.0 / alpha)).to(x)
+        mask1 = (x.abs() <= (1.0 / alpha)).to(x)
+        return mask0 + mask1 * (-(alpha**2) / 2 * x.square() * x.sign() + alpha * x + 0.5)
+    if name == "piecewise_exp":  # surrogate.py:758-762
+        mask_nonnegative = heaviside(x)
+        mask_sign = mask_nonnegative * 2.0 - 1.0
+        exp_x = (mask_sign * x * -alpha).exp_() / 2.0
+        return mask_nonnegative - exp_x * mask_sign
+    if name == "soft_sign":  # surrogate.py:1093-1094
+        return (torch.nn.functional.softsign(x * alpha) + 1.0) / 2.0
+    if name == "erf":  # surrogate.py:1778-1779
+        return torch.erfc_(-alpha * x) / 2.0
+    raise ValueError(f"{name} has no primitive")
+
+
+def surrogate_grad(name: str, x: torch.Tensor, alpha: float) -> torch.Tensor:
+    """g'(x) as the reference's backward computes it for grad_output = 1."""
+    one = torch.ones_like(x)
+    if name == "sigmoid":
+        sgax = (x * alpha).sigmoid_()
+        return one * (1.0 - sgax) * sgax * alpha
+    if name == "atan":
+        a = alpha / 2
+        ax = math.pi * a * x
+        return a / (1 + ax * ax) * one
+    return _sg_backward_other(name, one, x, alpha)
+
+
+# ------------------------------------------------------------------------------------------------
+# one step
+# ------------------------------------------------------------------------------------------------
+
+
+def voltage_reset(v, spike, v_threshold: float, v_reset: Optional[float], detach_reset: bool):
+    # functional/neuron.py:225-228
+    spike_d = spike.detach() if detach_reset else spike
+    if v_reset is None:
+        return v - spike_d * v_threshold
+    return spike_d * v_reset + (1.0 - spike_d) * v
+
+
+def charge(kind: str, x, v, tau_or_w, decay_input: bool, v_reset: Optional[float]):
+    if kind == "if":
+        return v + x  # functional/neuron.py:310
+    v_reset_value = 0.0 if v_reset is None else v_reset
+    if kind == "lif":
+        # functional/neuron.py:849-852
+        if decay_input:
+            return v + (x - (v - v_reset_value)) / tau_or_w
+        return v - (v - v_reset_value) / tau_or_w + x
+    if kind == "plif":
+        # functional/neuron.py:1290-1295
+        reciprocal_tau = tau_or_w.sigmoid()
+        if decay_input:
+            return v + (x - (v - v_reset_value)) * reciprocal_tau
+        return v - (v - v_reset_value) * reciprocal_tau + x
+    if kind == "plif_k":
+        # same as "plif" but fed k = sigmoid(w) directly (what the kernel operators receive)
+        if decay_input:
+            return v + (x - (v - v_reset_value)) * tau_or_w
+        return v - (v - v_reset_value) * tau_or_w + x
+    raise ValueError(kind)
+
+
+def step(kind: str, x, v, tau_or_w, decay_input: bool, v_threshold: float, v_reset: Optional[float],
+         sg: Callable, detach_reset: bool):
+    """(spike, v_next, h): functional/neuron.py:310-312, 931-933, 1296-1297."""
+    h = charge(kind, x, v, tau_or_w, decay_input, v_reset)
+    spike = sg(h - v_threshold)
+    return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset), h
+
+
+# ------------------------------------------------------------------------------------------------
+# sequences
+# ------------------------------------------------------------------------------------------------
+
+
+def multi_step(kind: str, x_seq: torch.Tensor, v_init: torch.Tensor, tau_or_w=None, decay_input: bool = True,
+               v_threshold: float = 1.0, v_reset: Optional[float] = 0.0, sg: Optional[Callable] = None,
+               detach_reset: bool = False):
+    """Step loop + stack (base.py:594-607, neuron/base_node.py:449-464).
+
+    Returns (spike_seq, v_seq, h_seq); state dtype follows ``x_seq`` as ``full_like`` makes it in
+    ``neuron/base_node.py:474-475``.
+    """
+    sg = heaviside if sg is None else sg
+    v = v_init
+    s_steps, v_steps, h_steps = [], [], []
+    for t in range(x_seq.shape[0]):
+        s, v, h = step(kind, x_seq[t], v, tau_or_w, decay_input, v_threshold, v_reset, sg, detach_reset)
+        s_steps.append(s)
+        v_steps.append(v)
+        h_steps.append(h)
+    return torch.stack(s_steps), torch.stack(v_steps), torch.stack(h_steps)
+
+
+def multi_step_mixed_precision(kind: str, x_seq: torch.Tensor, v_init: torch.Tensor, storage_dtype: torch.dtype,
+                               k: float = 0.5, decay_input: bool = True, v_threshold: float = 1.0,
+                               v_reset: Optional[float] = 0.0, torch_op_order: bool = True):
+    """fp32 state and arithmetic, storage-dtype inputs/outputs
+    (test/activation_based/test_triton_neuron.py:212-247): inputs are quantised to the storage dtype,
+    v is carried in fp32 un-rounded, stored v/h are rounded.  ``torch_op_order`` keeps the torch
+    backend's expression order (what the HIP kernels use); False uses the test's
+    ``v + k*(reset - v + x)`` order -- identical when v_reset is 0 or None.
+    Returns fp32 tensors (spike_seq, v_seq, h_seq) holding storage-representable values.
+    """
+    q = lambda t: t.to(storage_dtype).to(torch.float32)
+    x_seq = q(x_seq)
+    v = q(v_init)
+    k = torch.tensor(k, dtype=torch.float32)
+    reset_value = 0.0 if v_reset is None else v_reset
+    s_seq = torch.empty_like(x_seq)
+    v_seq = torch.empty_like(x_seq)
+    h_seq = torch.empty_like(x_seq)
+    for t in range(x_seq.shape[0]):
+        x = x_seq[t]
+        if kind == "if":
+            h = v + x
+        elif torch_op_order:
+            h = charge("plif_k", x, v, k, decay_input, v_reset)
+        elif decay_input:
+            h = v + k * (reset_value - v + x)
+        else:
+            h = v + k * (reset_value - v) + x
+        s = ((h - v_threshold) >= 0).to(torch.float32)
+        if v_reset is None:
+            v = h - s * v_threshold
+        else:
+            v = s * reset_value + (1.0 - s) * h
+        s_seq[t] = s
+        v_seq[t] = q(v)
+        h_seq[t] = q(h)
+    return s_seq, v_seq, h_seq
+
+
+def forward_backward(kind: str, x_seq: torch.Tensor, v_init: torch.Tensor, grad_spike_seq: Optional[torch.Tensor],
+                     grad_v_seq: Optional[torch.Tensor] = None, grad_v_last: Optional[torch.Tensor] = None,
+                     tau_or_w=None, decay_input: bool = True, v_threshold: float = 1.0,
+                     v_reset: Optional[float] = 0.0, sg_name: str = "atan", sg_alpha: float = 2.0,
+                     detach_reset: bool = False, spiking: bool = True):
+    """Forward with the surrogate, then autograd with the given upstream gradients.
+
+    Returns dict(spike_seq, v_seq, h_seq, grad_x, grad_v_init[, grad_p]) where grad_p is the
+    gradient w.r.t. ``tau_or_w`` when that is a tensor (PLIF's ``w`` or ``k``).
+    """
+    x = x_seq.detach().clone().requires_grad_(True)
+    v0 = v_init.detach().clone().requires_grad_(True)
+    p = tau_or_w
+    if isinstance(p, torch.Tensor):
+        p = p.detach().clone().requires_grad_(True)
+    s_seq, v_seq, h_seq = multi_step(kind, x, v0, p, decay_input, v_threshold, v_reset,
+                                     surrogate(sg_name, sg_alpha, spiking), detach_reset)
+    outs, grads = [], []
+    if grad_spike_seq is not None:
+        outs.append(s_seq)
+        grads.append(grad_spike_seq)
+    if grad_v_seq is not None:
+        outs.append(v_seq)
+        grads.append(grad_v_seq)
+    if grad_v_last is not None:
+        outs.append(v_seq[-1])
+        grads.append(grad_v_last)
+    torch.autograd.backward(outs, grads)
+    res = dict(spike_seq=s_seq.detach(), v_seq=v_seq.detach(), h_seq=h_seq.detach(),
+               grad_x=x.grad if x.grad is not None else torch.zeros_like(x),
+               grad_v_init=v0.grad if v0.grad is not None else torch.zeros_like(v0))
+    if isinstance(p, torch.Tensor):
+        res["grad_p"] = p.grad if p.grad is not None else torch.zeros_like(p)
+    return res

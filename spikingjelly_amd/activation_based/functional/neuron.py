@@ -1,0 +1,180 @@
+"""Functional state transitions of IF / LIF / PLIF neurons.
+
+Two families, as in the reference's ``spikingjelly/activation_based/functional/neuron.py``:
+
+* ``*_step`` / ``voltage_reset`` / ``lif_charge``: the torch-backend math, one step, pure
+  (reference :173-228, :242-312, :797-933, :1215-1297);
+* ``{if,lif,plif}_multi_step_hip``: whole sequences through the HIP kernels, same signature and
+  return convention as the reference's ``*_multi_step_cupy`` / ``*_multi_step_triton``
+  (:1889-2185, :2582-2849): ``(spike_seq, v_next, v_seq or None)``.
+"""
+
+from __future__ import annotations
+
+from typing import Callable, Optional
+
+import torch
+
+from ... import configure
+
+SurrogateFunction = Callable[[torch.Tensor], torch.Tensor]
+
+__all__ = [
+    "voltage_reset",
+    "if_step",
+    "lif_charge",
+    "lif_step",
+    "plif_step",
+    "if_multi_step_hip",
+    "lif_multi_step_hip",
+    "plif_multi_step_hip",
+]
+
+
+# ---- torch backend: one step --------------------------------------------------------------------
+def voltage_reset(v: torch.Tensor, spike: torch.Tensor, v_threshold: float, v_reset: Optional[float],
+                  detach_reset: bool) -> torch.Tensor:
+    """Soft reset ``v - s*v_threshold`` when ``v_reset is None``, else hard reset
+    ``s*v_reset + (1 - s)*v``; ``detach_reset`` cuts the gradient through ``s`` here only."""
+    s = spike.detach() if detach_reset else spike
+    if v_reset is None:
+        return v - s * v_threshold
+    return s * v_reset + (1.0 - s) * v
+
+
+def if_step(x: torch.Tensor, v: torch.Tensor, v_threshold: float, v_reset: Optional[float],
+            surrogate_function: SurrogateFunction, detach_reset: bool = False
+            ) -> tuple[torch.Tensor, torch.Tensor]:
+    """One IF step: ``h = v + x``, fire, reset.  Returns ``(spike, v_next)``."""
+    h = v + x
+    spike = surrogate_function(h - v_threshold)
+    return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset)
+
+
+def lif_charge(x: torch.Tensor, v: torch.Tensor, tau: float, decay_input: bool,
+               v_reset: Optional[float]) -> torch.Tensor:
+    """LIF charge; ``v_reset=None`` counts as 0 here."""
+    rest = 0.0 if v_reset is None else v_reset
+    if decay_input:
+        return v + (x - (v - rest)) / tau
+    return v - (v - rest) / tau + x
+
+
+def lif_step(x: torch.Tensor, v: torch.Tensor, tau: float, decay_input: bool, v_threshold: float,
+             v_reset: Optional[float], surrogate_function: SurrogateFunction, detach_reset: bool = False
+             ) -> tuple[torch.Tensor, torch.Tensor]:
+    """One LIF step.  Returns ``(spike, v_next)``."""
+    h = lif_charge(x, v, tau, decay_input, v_reset)
+    spike = surrogate_function(h - v_threshold)
+    return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset)
+
+
+def plif_step(x: torch.Tensor, v: torch.Tensor, w: torch.Tensor, decay_input: bool, v_threshold: float,
+              v_reset: Optional[float], surrogate_function: SurrogateFunction, detach_reset: bool = False
+              ) -> tuple[torch.Tensor, torch.Tensor]:
+    """One parametric-LIF step with ``1/tau = sigmoid(w)``.  Returns ``(spike, v_next)``."""
+    k = w.sigmoid()
+    rest = 0.0 if v_reset is None else v_reset
+    if decay_input:
+        h = v + (x - (v - rest)) * k
+    else:
+        h = v - (v - rest) * k + x
+    spike = surrogate_function(h - v_threshold)
+    return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset)
+
+
+# ---- hip backend: whole sequence ----------------------------------------------------------------
+def _hip_mode_flags(x_seq: torch.Tensor) -> int:
+    from ..hip_kernel import library as L
+
+    flags = 0
+    if x_seq.dtype != torch.float32:
+        mode = configure.hip_half_precision_mode
+        if mode == "fp32_state":
+            flags |= L.FLAG_FP32_STATE
+        elif mode != "torch":
+            raise ValueError(f"configure.hip_half_precision_mode must be 'torch' or 'fp32_state', got {mode!r}")
+    if configure.hip_lif_reciprocal_tau:
+        flags |= L.FLAG_RECIPROCAL_TAU
+    if configure.hip_plif_atomic_reduce:
+        flags |= L.FLAG_ATOMIC_REDUCE
+    return flags
+
+
+def _needs_grad(*tensors: torch.Tensor) -> bool:
+    return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+
+
+def _finish(x_seq: torch.Tensor, spike_seq: torch.Tensor, v_seq: torch.Tensor, v_last: torch.Tensor,
+            store_v_seq: bool) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    spike_seq = spike_seq.reshape(x_seq.shape)
+    v_last = v_last.reshape(x_seq.shape[1:])
+    return spike_seq, v_last, (v_seq.reshape(x_seq.shape) if store_v_seq else None)
+
+
+def if_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, v_threshold: float, v_reset: Optional[float],
+                      surrogate_function: SurrogateFunction, detach_reset: bool = False,
+                      store_v_seq: bool = False
+                      ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Multi-step IF on the hip backend.  ``x_seq`` is ``[T, *]``, ``v`` has the shape of ``x_seq[0]``."""
+    from ..hip_kernel import neuron_kernel as K
+    from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
+
+    soft = v_reset is None
+    vr = 0.0 if soft else float(v_reset)
+    flags = _hip_mode_flags(x_seq)
+    x2, v1 = x_seq.flatten(1), v.flatten()
+    if _needs_grad(x_seq, v):
+        sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function)
+        s, v_seq, v_last, _ = K.hip_multistep_if_forward(x2, v1, v_threshold, vr, soft, detach_reset, sg_id,
+                                                         sg_alpha, store_v_seq, flags)
+    else:
+        s, v_seq, v_last = K.hip_multistep_if_inference(x2, v1, v_threshold, vr, soft, store_v_seq, flags)
+    return _finish(x_seq, s, v_seq, v_last, store_v_seq)
+
+
+def lif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, decay_input: bool,
+                       v_threshold: float, v_reset: Optional[float], surrogate_function: SurrogateFunction,
+                       detach_reset: bool = False, store_v_seq: bool = False
+                       ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Multi-step LIF on the hip backend."""
+    from ..hip_kernel import neuron_kernel as K
+    from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
+
+    soft = v_reset is None
+    vr = 0.0 if soft else float(v_reset)
+    flags = _hip_mode_flags(x_seq)
+    x2, v1 = x_seq.flatten(1), v.flatten()
+    if _needs_grad(x_seq, v):
+        sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function)
+        s, v_seq, v_last, _ = K.hip_multistep_lif_forward(x2, v1, v_threshold, vr, soft, detach_reset,
+                                                          float(tau), decay_input, sg_id, sg_alpha,
+                                                          store_v_seq, flags)
+    else:
+        s, v_seq, v_last = K.hip_multistep_lif_inference(x2, v1, v_threshold, vr, soft, float(tau),
+                                                         decay_input, store_v_seq, flags)
+    return _finish(x_seq, s, v_seq, v_last, store_v_seq)
+
+
+def plif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Tensor, decay_input: bool,
+                        v_threshold: float, v_reset: Optional[float], surrogate_function: SurrogateFunction,
+                        detach_reset: bool = False, store_v_seq: bool = False
+                        ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Multi-step parametric LIF on the hip backend.  ``w`` is the pre-sigmoid parameter; the
+    sigmoid stays outside the operator so autograd supplies ``dk/dw`` (reference :2173-2182)."""
+    from ..hip_kernel import neuron_kernel as K
+    from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
+
+    soft = v_reset is None
+    vr = 0.0 if soft else float(v_reset)
+    flags = _hip_mode_flags(x_seq)
+    x2, v1 = x_seq.flatten(1), v.flatten()
+    k = w.sigmoid().to(device=x_seq.device, dtype=torch.float32)
+    if _needs_grad(x_seq, v, w):
+        sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function)
+        s, v_seq, v_last, _ = K.hip_multistep_plif_forward(x2, v1, k, v_threshold, vr, soft, detach_reset,
+                                                           decay_input, sg_id, sg_alpha, store_v_seq, flags)
+    else:
+        s, v_seq, v_last = K.hip_multistep_plif_inference(x2, v1, k, v_threshold, vr, soft, decay_input,
+                                                          store_v_seq, flags)
+    return _finish(x_seq, s, v_seq, v_last, store_v_seq)

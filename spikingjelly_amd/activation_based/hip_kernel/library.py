@@ -1,0 +1,178 @@
+"""ctypes binding of the C ABI declared in ``include/sjhip.h``.
+
+The shared library is looked up next to the package (``spikingjelly_amd/libsjhip.so``,
+built in-tree by ``make -C spikingjelly_amd/csrc``).  Nothing here falls back to another
+implementation: a missing library raises, a failing call raises with the library's message.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64, c_uint32, c_void_p
+
+import torch
+
+ABI_VERSION = 1
+
+# enums of include/sjhip.h
+NEURON_IF, NEURON_LIF, NEURON_PLIF = 0, 1, 2
+DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_U8 = 0, 1, 2, 3
+FLAG_DECAY_INPUT = 0x01
+FLAG_SOFT_RESET = 0x02
+FLAG_DETACH_RESET = 0x04
+FLAG_FP32_STATE = 0x10
+FLAG_RECIPROCAL_TAU = 0x20
+FLAG_ATOMIC_REDUCE = 0x80
+
+KC_FORWARD, KC_BACKWARD, KC_PLIF_REDUCE, KC_BIT_PACK, KC_BIT_UNPACK = range(5)
+
+EXPORTED_SYMBOLS = (
+    "sjhip_abi_version",
+    "sjhip_last_error",
+    "sjhip_neuron_forward",
+    "sjhip_plif_workspace_floats",
+    "sjhip_neuron_backward",
+    "sjhip_bit_pack",
+    "sjhip_bit_unpack",
+    "sjhip_set_tuning",
+    "sjhip_get_tuning",
+    "sjhip_profile_enable",
+    "sjhip_profile_reset",
+    "sjhip_profile_read",
+)
+
+
+class NeuronParams(ctypes.Structure):
+    """``struct sjhip_neuron_params``."""
+
+    _fields_ = [
+        ("tau", c_float),
+        ("v_threshold", c_float),
+        ("v_reset", c_float),
+        ("sg_alpha", c_float),
+        ("sg_id", c_int32),
+        ("flags", c_uint32),
+    ]
+
+
+_lock = threading.Lock()
+_lib = None
+
+
+def library_path() -> str:
+    return os.path.join(os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))), "libsjhip.so")
+
+
+def load() -> ctypes.CDLL:
+    """Load (once) and return the library; ``OSError`` if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = library_path()
+        if not os.path.exists(path):
+            raise OSError(f"{path} not found; run `make -C spikingjelly_amd/csrc`")
+        lib = ctypes.CDLL(path)
+        lib.sjhip_abi_version.restype = c_int
+        lib.sjhip_abi_version.argtypes = []
+        if lib.sjhip_abi_version() != ABI_VERSION:
+            raise OSError(f"{path}: ABI version {lib.sjhip_abi_version()} != {ABI_VERSION}")
+        lib.sjhip_last_error.restype = c_char_p
+        lib.sjhip_last_error.argtypes = []
+        lib.sjhip_neuron_forward.restype = c_int
+        lib.sjhip_neuron_forward.argtypes = [
+            c_int, c_int, POINTER(NeuronParams), c_int64, c_int64,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        ]
+        lib.sjhip_plif_workspace_floats.restype = c_int64
+        lib.sjhip_plif_workspace_floats.argtypes = [c_int, c_int64]
+        lib.sjhip_neuron_backward.restype = c_int
+        lib.sjhip_neuron_backward.argtypes = [
+            c_int, c_int, POINTER(NeuronParams), c_int64, c_int64,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        ]
+        lib.sjhip_bit_pack.restype = c_int
+        lib.sjhip_bit_pack.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p]
+        lib.sjhip_bit_unpack.restype = c_int
+        lib.sjhip_bit_unpack.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p]
+        lib.sjhip_set_tuning.restype = c_int
+        lib.sjhip_set_tuning.argtypes = [c_char_p, c_int]
+        lib.sjhip_get_tuning.restype = c_int
+        lib.sjhip_get_tuning.argtypes = [c_char_p]
+        lib.sjhip_profile_enable.restype = c_int
+        lib.sjhip_profile_enable.argtypes = [c_int]
+        lib.sjhip_profile_reset.restype = c_int
+        lib.sjhip_profile_reset.argtypes = []
+        lib.sjhip_profile_read.restype = c_int
+        lib.sjhip_profile_read.argtypes = [c_int, POINTER(c_int64), POINTER(c_double)]
+        _lib = lib
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().sjhip_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"libsjhip {what} failed ({rc}): {msg}")
+
+
+_DTYPE_IDS = {
+    torch.float32: DTYPE_F32,
+    torch.float16: DTYPE_F16,
+    torch.bfloat16: DTYPE_BF16,
+    torch.uint8: DTYPE_U8,
+    torch.bool: DTYPE_U8,
+}
+
+
+def dtype_id(dtype: torch.dtype, *, allow_u8: bool = False) -> int:
+    """Map a torch dtype to ``sjhip_dtype``; ``NotImplementedError(dtype)`` like the
+    reference kernels (cuda_kernel/neuron_kernel/multi_step/base.py:22-27)."""
+    did = _DTYPE_IDS.get(dtype)
+    if did is None or (did == DTYPE_U8 and not allow_u8):
+        raise NotImplementedError(dtype)
+    return did
+
+
+def require_device_tensor(name: str, t: torch.Tensor) -> None:
+    if t.device.type != "cuda":
+        raise RuntimeError(
+            f"backend='hip' runs on a ROCm device only, but {name} is on {t.device}; "
+            "use backend='torch' for CPU tensors."
+        )
+
+
+def current_stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def ptr(t) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def set_tuning(key: str, value: int) -> None:
+    check(load().sjhip_set_tuning(key.encode(), int(value)), f"set_tuning({key})")
+
+
+def get_tuning(key: str) -> int:
+    return load().sjhip_get_tuning(key.encode())
+
+
+def profile_enable(on: bool) -> None:
+    check(load().sjhip_profile_enable(1 if on else 0), "profile_enable")
+
+
+def profile_reset() -> None:
+    check(load().sjhip_profile_reset(), "profile_reset")
+
+
+def profile_read(which: int) -> tuple[int, float]:
+    """(launch count, total milliseconds) of kernel class ``which`` since the last reset."""
+    n = c_int64(0)
+    ms = c_double(0.0)
+    check(load().sjhip_profile_read(which, ctypes.byref(n), ctypes.byref(ms)), "profile_read")
+    return n.value, ms.value

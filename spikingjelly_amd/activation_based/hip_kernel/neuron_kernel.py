@@ -1,0 +1,365 @@
+"""``torch.library`` operators for the multi-step IF / LIF / PLIF kernels of ``libsjhip.so``.
+
+Operator layout follows the reference's kernel backends
+(``cuda_kernel/neuron_kernel/multi_step/lif.py:144-325``: forward op + fake + backward op +
+``register_autograd`` saving ``h_seq``; ``triton_kernel/neuron_kernel/lif.py:673-763``: a separate
+inference op that writes no ``h_seq``):
+
+    sj::hip_multistep_{if,lif,plif}_forward    -> (spike_seq, v_seq, v_last, h_seq)
+    sj::hip_multistep_{if,lif,plif}_inference  -> (spike_seq, v_seq, v_last)
+    sj::hip_multistep_{if,lif,plif}_backward   -> (grad_x_seq, grad_v_init[, grad_k])
+
+All tensors are viewed as ``[T, N]``; ``v_seq`` is an empty tensor when ``store_v_seq`` is false
+(the kernel then writes only ``v_last``).  ``Optional[float]`` is not expressible in an operator
+schema, so soft reset is a bool next to a dummy ``v_reset`` as in the reference (lif.py:342-343).
+The ops run on ROCm tensors only and raise otherwise; there is no fallback path.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import library as L
+
+__all__ = [
+    "hip_multistep_if_forward", "hip_multistep_if_inference", "hip_multistep_if_backward",
+    "hip_multistep_lif_forward", "hip_multistep_lif_inference", "hip_multistep_lif_backward",
+    "hip_multistep_plif_forward", "hip_multistep_plif_inference", "hip_multistep_plif_backward",
+]
+
+
+def _params(tau: float, v_th: float, v_reset: float, sg_alpha: float, sg_id: int, flags: int) -> L.NeuronParams:
+    return L.NeuronParams(tau, v_th, v_reset, sg_alpha, sg_id, flags)
+
+
+def _flags(soft_reset: bool, detach_reset: bool, decay_input: bool, mode_flags: int) -> int:
+    f = int(mode_flags) & (L.FLAG_FP32_STATE | L.FLAG_RECIPROCAL_TAU | L.FLAG_ATOMIC_REDUCE)
+    if soft_reset:
+        f |= L.FLAG_SOFT_RESET
+    if detach_reset:
+        f |= L.FLAG_DETACH_RESET
+    if decay_input:
+        f |= L.FLAG_DECAY_INPUT
+    return f
+
+
+def _check_inputs(x_seq: torch.Tensor, v_init: torch.Tensor) -> None:
+    L.require_device_tensor("x_seq", x_seq)
+    L.require_device_tensor("v_init", v_init)
+    if x_seq.dim() != 2:
+        raise ValueError(f"x_seq must be [T, N], got shape {tuple(x_seq.shape)}")
+    if v_init.shape != x_seq.shape[1:]:
+        raise ValueError(f"v_init shape {tuple(v_init.shape)} does not match x_seq[0] {tuple(x_seq.shape[1:])}")
+    if v_init.dtype != x_seq.dtype:
+        raise ValueError(f"v_init dtype {v_init.dtype} != x_seq dtype {x_seq.dtype}")
+    if x_seq.shape[0] < 1 or x_seq.shape[1] < 1:
+        raise ValueError(f"x_seq must have T >= 1 and N >= 1, got shape {tuple(x_seq.shape)}")
+
+
+def _k_pointer(k: Optional[torch.Tensor], ref: torch.Tensor) -> tuple[Optional[torch.Tensor], Optional[int]]:
+    if k is None:
+        return None, None
+    L.require_device_tensor("k", k)
+    k = k.detach().to(dtype=torch.float32, device=ref.device).reshape(1).contiguous()
+    return k, k.data_ptr()
+
+
+def _run_forward(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: Optional[torch.Tensor],
+                 tau: float, v_th: float, v_reset: float, flags: int, store_v_seq: bool,
+                 save_h: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    _check_inputs(x_seq, v_init)
+    dtype = L.dtype_id(x_seq.dtype)
+    x_seq = x_seq.contiguous()
+    v_init = v_init.contiguous()
+    T, N = x_seq.shape
+    spike_seq = torch.empty_like(x_seq)
+    v_seq = torch.empty_like(x_seq) if store_v_seq else x_seq.new_empty((0,))
+    v_last = torch.empty_like(v_init)
+    h_seq = torch.empty_like(x_seq) if save_h else None
+    k_keep, k_ptr = _k_pointer(k, x_seq)
+    params = _params(tau, v_th, v_reset, 0.0, 0, flags)
+    with torch.cuda.device(x_seq.device):
+        rc = L.load().sjhip_neuron_forward(
+            neuron, dtype, ctypes.byref(params), T, N,
+            x_seq.data_ptr(), v_init.data_ptr(), k_ptr,
+            spike_seq.data_ptr(), v_seq.data_ptr() if store_v_seq else None, v_last.data_ptr(),
+            L.ptr(h_seq), L.current_stream_ptr(x_seq.device),
+        )
+    L.check(rc, "neuron_forward")
+    del k_keep
+    return spike_seq, v_seq, v_last, h_seq
+
+
+def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
+                  grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor, v_init: Optional[torch.Tensor],
+                  k: Optional[torch.Tensor], tau: float, v_th: float, v_reset: float, flags: int,
+                  sg_id: int, sg_alpha: float) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    L.require_device_tensor("h_seq", h_seq)
+    dtype = L.dtype_id(h_seq.dtype)
+    h_seq = h_seq.contiguous()
+    T, N = h_seq.shape
+    if grad_spike_seq is None:
+        grad_spike_seq = torch.zeros_like(h_seq)
+    grad_spike_seq = grad_spike_seq.to(h_seq.dtype).contiguous()
+    if grad_v_seq is not None:
+        grad_v_seq = grad_v_seq.to(h_seq.dtype).contiguous()
+    if grad_v_last is not None:
+        grad_v_last = grad_v_last.to(h_seq.dtype).contiguous()
+    grad_x_seq = torch.empty_like(h_seq)
+    grad_v_init = h_seq.new_empty((N,))
+    grad_k = workspace = None
+    k_keep, k_ptr = _k_pointer(k, h_seq)
+    if neuron == L.NEURON_PLIF:
+        v_init = v_init.contiguous()
+        if flags & L.FLAG_ATOMIC_REDUCE:
+            grad_k = torch.zeros((), dtype=torch.float32, device=h_seq.device)
+        else:
+            grad_k = torch.empty((), dtype=torch.float32, device=h_seq.device)
+            workspace = torch.empty((L.load().sjhip_plif_workspace_floats(dtype, N),), dtype=torch.float32,
+                                    device=h_seq.device)
+    params = _params(tau, v_th, v_reset, sg_alpha, sg_id, flags)
+    with torch.cuda.device(h_seq.device):
+        rc = L.load().sjhip_neuron_backward(
+            neuron, dtype, ctypes.byref(params), T, N,
+            grad_spike_seq.data_ptr(), L.ptr(grad_v_seq), L.ptr(grad_v_last), h_seq.data_ptr(),
+            L.ptr(v_init) if neuron == L.NEURON_PLIF else None, k_ptr,
+            grad_x_seq.data_ptr(), grad_v_init.data_ptr(), L.ptr(grad_k), L.ptr(workspace),
+            L.current_stream_ptr(h_seq.device),
+        )
+    L.check(rc, "neuron_backward")
+    del k_keep
+    return grad_x_seq, grad_v_init, grad_k
+
+
+def _fake_forward(x_seq, v_init, store_v_seq, with_h):
+    outs = [
+        x_seq.new_empty(x_seq.shape),
+        x_seq.new_empty(x_seq.shape) if store_v_seq else x_seq.new_empty((0,)),
+        v_init.new_empty(v_init.shape),
+    ]
+    if with_h:
+        outs.append(x_seq.new_empty(x_seq.shape))
+    return tuple(outs)
+
+
+def _none_if_empty_grad(g: Optional[torch.Tensor], store_v_seq: bool) -> Optional[torch.Tensor]:
+    return g if (store_v_seq and g is not None) else None
+
+
+# =================================================================================================
+# IF
+# =================================================================================================
+@torch.library.custom_op("sj::hip_multistep_if_forward", mutates_args=())
+def hip_multistep_if_forward(x_seq: torch.Tensor, v_init: torch.Tensor, v_th: float, v_reset: float,
+                             soft_reset: bool, detach_reset: bool, sg_id: int, sg_alpha: float,
+                             store_v_seq: bool, mode_flags: int
+                             ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, detach_reset, False, mode_flags)
+    return _run_forward(L.NEURON_IF, x_seq, v_init, None, 0.0, v_th, v_reset, flags, store_v_seq, True)
+
+
+@hip_multistep_if_forward.register_fake
+def _(x_seq, v_init, v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, store_v_seq, mode_flags):
+    return _fake_forward(x_seq, v_init, store_v_seq, True)
+
+
+@torch.library.custom_op("sj::hip_multistep_if_inference", mutates_args=())
+def hip_multistep_if_inference(x_seq: torch.Tensor, v_init: torch.Tensor, v_th: float, v_reset: float,
+                               soft_reset: bool, store_v_seq: bool, mode_flags: int
+                               ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, False, False, mode_flags)
+    return _run_forward(L.NEURON_IF, x_seq, v_init, None, 0.0, v_th, v_reset, flags, store_v_seq, False)[:3]
+
+
+@hip_multistep_if_inference.register_fake
+def _(x_seq, v_init, v_th, v_reset, soft_reset, store_v_seq, mode_flags):
+    return _fake_forward(x_seq, v_init, store_v_seq, False)
+
+
+@torch.library.custom_op("sj::hip_multistep_if_backward", mutates_args=())
+def hip_multistep_if_backward(grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
+                              grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor, v_th: float,
+                              v_reset: float, soft_reset: bool, detach_reset: bool, sg_id: int,
+                              sg_alpha: float, mode_flags: int) -> tuple[torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, detach_reset, False, mode_flags)
+    gx, gvi, _ = _run_backward(L.NEURON_IF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, None, None,
+                               0.0, v_th, v_reset, flags, sg_id, sg_alpha)
+    return gx, gvi
+
+
+@hip_multistep_if_backward.register_fake
+def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_th, v_reset, soft_reset, detach_reset, sg_id,
+      sg_alpha, mode_flags):
+    return torch.empty_like(h_seq), h_seq.new_empty(h_seq.shape[1:])
+
+
+def _if_setup_context(ctx, inputs, output):
+    (_, _, v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, store_v_seq, mode_flags) = inputs
+    ctx.save_for_backward(output[3])
+    ctx.scalars = (v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, mode_flags)
+    ctx.store_v_seq = store_v_seq
+    ctx.set_materialize_grads(False)
+
+
+def _if_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_seq):
+    del grad_h_seq
+    (h_seq,) = ctx.saved_tensors
+    v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, mode_flags = ctx.scalars
+    gx, gvi = hip_multistep_if_backward(
+        grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq,
+        v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, mode_flags)
+    return gx, gvi, None, None, None, None, None, None, None, None
+
+
+torch.library.register_autograd("sj::hip_multistep_if_forward", _if_autograd_backward,
+                                setup_context=_if_setup_context)
+
+
+# =================================================================================================
+# LIF
+# =================================================================================================
+@torch.library.custom_op("sj::hip_multistep_lif_forward", mutates_args=())
+def hip_multistep_lif_forward(x_seq: torch.Tensor, v_init: torch.Tensor, v_th: float, v_reset: float,
+                              soft_reset: bool, detach_reset: bool, tau: float, decay_input: bool,
+                              sg_id: int, sg_alpha: float, store_v_seq: bool, mode_flags: int
+                              ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, detach_reset, decay_input, mode_flags)
+    return _run_forward(L.NEURON_LIF, x_seq, v_init, None, tau, v_th, v_reset, flags, store_v_seq, True)
+
+
+@hip_multistep_lif_forward.register_fake
+def _(x_seq, v_init, v_th, v_reset, soft_reset, detach_reset, tau, decay_input, sg_id, sg_alpha,
+      store_v_seq, mode_flags):
+    return _fake_forward(x_seq, v_init, store_v_seq, True)
+
+
+@torch.library.custom_op("sj::hip_multistep_lif_inference", mutates_args=())
+def hip_multistep_lif_inference(x_seq: torch.Tensor, v_init: torch.Tensor, v_th: float, v_reset: float,
+                                soft_reset: bool, tau: float, decay_input: bool, store_v_seq: bool,
+                                mode_flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, False, decay_input, mode_flags)
+    return _run_forward(L.NEURON_LIF, x_seq, v_init, None, tau, v_th, v_reset, flags, store_v_seq, False)[:3]
+
+
+@hip_multistep_lif_inference.register_fake
+def _(x_seq, v_init, v_th, v_reset, soft_reset, tau, decay_input, store_v_seq, mode_flags):
+    return _fake_forward(x_seq, v_init, store_v_seq, False)
+
+
+@torch.library.custom_op("sj::hip_multistep_lif_backward", mutates_args=())
+def hip_multistep_lif_backward(grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
+                               grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor, v_th: float,
+                               v_reset: float, soft_reset: bool, detach_reset: bool, tau: float,
+                               decay_input: bool, sg_id: int, sg_alpha: float, mode_flags: int
+                               ) -> tuple[torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, detach_reset, decay_input, mode_flags)
+    gx, gvi, _ = _run_backward(L.NEURON_LIF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, None, None,
+                               tau, v_th, v_reset, flags, sg_id, sg_alpha)
+    return gx, gvi
+
+
+@hip_multistep_lif_backward.register_fake
+def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_th, v_reset, soft_reset, detach_reset, tau,
+      decay_input, sg_id, sg_alpha, mode_flags):
+    return torch.empty_like(h_seq), h_seq.new_empty(h_seq.shape[1:])
+
+
+def _lif_setup_context(ctx, inputs, output):
+    (_, _, v_th, v_reset, soft_reset, detach_reset, tau, decay_input, sg_id, sg_alpha, store_v_seq,
+     mode_flags) = inputs
+    ctx.save_for_backward(output[3])
+    ctx.scalars = (v_th, v_reset, soft_reset, detach_reset, tau, decay_input, sg_id, sg_alpha, mode_flags)
+    ctx.store_v_seq = store_v_seq
+    ctx.set_materialize_grads(False)
+
+
+def _lif_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_seq):
+    del grad_h_seq
+    (h_seq,) = ctx.saved_tensors
+    gx, gvi = hip_multistep_lif_backward(
+        grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, *ctx.scalars)
+    return gx, gvi, None, None, None, None, None, None, None, None, None, None
+
+
+torch.library.register_autograd("sj::hip_multistep_lif_forward", _lif_autograd_backward,
+                                setup_context=_lif_setup_context)
+
+
+# =================================================================================================
+# PLIF: k = sigmoid(w) is a 0-dim fp32 tensor on the device; the kernels read it from memory, so no
+# host synchronisation happens (the reference's Triton path calls r_tau.item(), plif.py:666).
+# =================================================================================================
+@torch.library.custom_op("sj::hip_multistep_plif_forward", mutates_args=())
+def hip_multistep_plif_forward(x_seq: torch.Tensor, v_init: torch.Tensor, k: torch.Tensor, v_th: float,
+                               v_reset: float, soft_reset: bool, detach_reset: bool, decay_input: bool,
+                               sg_id: int, sg_alpha: float, store_v_seq: bool, mode_flags: int
+                               ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, detach_reset, decay_input, mode_flags)
+    return _run_forward(L.NEURON_PLIF, x_seq, v_init, k, 0.0, v_th, v_reset, flags, store_v_seq, True)
+
+
+@hip_multistep_plif_forward.register_fake
+def _(x_seq, v_init, k, v_th, v_reset, soft_reset, detach_reset, decay_input, sg_id, sg_alpha,
+      store_v_seq, mode_flags):
+    return _fake_forward(x_seq, v_init, store_v_seq, True)
+
+
+@torch.library.custom_op("sj::hip_multistep_plif_inference", mutates_args=())
+def hip_multistep_plif_inference(x_seq: torch.Tensor, v_init: torch.Tensor, k: torch.Tensor, v_th: float,
+                                 v_reset: float, soft_reset: bool, decay_input: bool, store_v_seq: bool,
+                                 mode_flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, False, decay_input, mode_flags)
+    return _run_forward(L.NEURON_PLIF, x_seq, v_init, k, 0.0, v_th, v_reset, flags, store_v_seq, False)[:3]
+
+
+@hip_multistep_plif_inference.register_fake
+def _(x_seq, v_init, k, v_th, v_reset, soft_reset, decay_input, store_v_seq, mode_flags):
+    return _fake_forward(x_seq, v_init, store_v_seq, False)
+
+
+@torch.library.custom_op("sj::hip_multistep_plif_backward", mutates_args=())
+def hip_multistep_plif_backward(grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
+                                grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor,
+                                v_init: torch.Tensor, k: torch.Tensor, v_th: float, v_reset: float,
+                                soft_reset: bool, detach_reset: bool, decay_input: bool, sg_id: int,
+                                sg_alpha: float, mode_flags: int
+                                ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, detach_reset, decay_input, mode_flags)
+    gx, gvi, gk = _run_backward(L.NEURON_PLIF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, k,
+                                0.0, v_th, v_reset, flags, sg_id, sg_alpha)
+    return gx, gvi, gk
+
+
+@hip_multistep_plif_backward.register_fake
+def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, k, v_th, v_reset, soft_reset, detach_reset,
+      decay_input, sg_id, sg_alpha, mode_flags):
+    return (torch.empty_like(h_seq), h_seq.new_empty(h_seq.shape[1:]),
+            h_seq.new_empty((), dtype=torch.float32))
+
+
+def _plif_setup_context(ctx, inputs, output):
+    (_, v_init, k, v_th, v_reset, soft_reset, detach_reset, decay_input, sg_id, sg_alpha, store_v_seq,
+     mode_flags) = inputs
+    ctx.save_for_backward(output[3], v_init, k)
+    ctx.scalars = (v_th, v_reset, soft_reset, detach_reset, decay_input, sg_id, sg_alpha, mode_flags)
+    ctx.store_v_seq = store_v_seq
+    ctx.k_shape = k.shape
+    ctx.k_dtype = k.dtype
+    ctx.set_materialize_grads(False)
+
+
+def _plif_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_seq):
+    del grad_h_seq
+    h_seq, v_init, k = ctx.saved_tensors
+    gx, gvi, gk = hip_multistep_plif_backward(
+        grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, v_init, k,
+        *ctx.scalars)
+    gk = gk.reshape(ctx.k_shape).to(ctx.k_dtype)
+    return gx, gvi, gk, None, None, None, None, None, None, None, None, None
+
+
+torch.library.register_autograd("sj::hip_multistep_plif_forward", _plif_autograd_backward,
+                                setup_context=_plif_setup_context)

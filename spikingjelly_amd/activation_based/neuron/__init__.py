@@ -1,0 +1,6 @@
+from .base_node import BaseNode
+from .integrate_and_fire import IFNode
+from .lif import LIFNode
+from .plif import ParametricLIFNode
+
+__all__ = ["BaseNode", "IFNode", "LIFNode", "ParametricLIFNode"]

@@ -1,0 +1,24 @@
+"""Process-wide switches of the hip backend (counterpart of the reference's
+``spikingjelly/configure.py``, which holds ``cuda_threads`` and compiler options
+for its CuPy/Triton backends).
+
+``hip_half_precision_mode``
+    How fp16/bf16 inputs are computed by ``backend='hip'``:
+    ``"torch"`` rounds the result of every arithmetic op to the storage dtype and
+    keeps the membrane potential in it -- bit-identical to ``backend='torch'`` on
+    the same half tensors; ``"fp32_state"`` keeps state and arithmetic in fp32 and
+    rounds only what is stored (the reference's mixed-precision Triton ops).
+
+``hip_lif_reciprocal_tau``
+    ``False``: LIF charges with an IEEE division by ``tau`` like the torch CPU
+    backend.  ``True``: multiply by ``fl(1/tau)`` like the reference's CuPy/Triton
+    kernels (identical results when ``tau`` is a power of two).
+
+``hip_plif_atomic_reduce``
+    ``False``: the PLIF ``dL/dk`` sum is reduced in a fixed order (bitwise
+    reproducible).  ``True``: one ``atomicAdd`` per block, order varies run to run.
+"""
+
+hip_half_precision_mode = "torch"
+hip_lif_reciprocal_tau = False
+hip_plif_atomic_reduce = False

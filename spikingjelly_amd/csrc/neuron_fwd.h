@@ -1,0 +1,155 @@
+// Multi-step forward (charge -> fire -> reset over T steps) for IF / LIF / PLIF.
+//
+// One work-item owns V consecutive neurons (one 128-bit access per row) and walks the T rows in
+// order with the membrane potential in registers.  Rows of x are requested SJHIP_FWD_PF steps ahead
+// of their use so several 128-bit loads per lane are always in flight; every tensor is touched
+// exactly once, so loads and stores are non-temporal.
+//
+// The arithmetic restates the torch backend of the reference op for op and in its order
+// (functional/neuron.py:225-228 voltage_reset, :310-312 if_step, :849-852 lif_charge, :1290-1297
+// plif_step, surrogate.py:60 heaviside), with floating-point contraction off, so spikes, h and v are
+// bit-identical to it in fp32.  For 16-bit storage either every op result is rounded to the storage
+// dtype (the torch backend run on half tensors) or state and arithmetic stay fp32 and only stored
+// values are rounded (the reference's mixed-precision kernels).
+#pragma once
+
+#include <type_traits>
+
+#include "sjhip_common.h"
+
+#ifndef SJHIP_FWD_PF
+#define SJHIP_FWD_PF 4
+#endif
+
+namespace sjhip {
+
+enum Charge {
+  CH_IF = 0,
+  CH_DECAY_INPUT_DIV = 1,  // v + (x - (v - vr)) / tau
+  CH_DECAY_INPUT_MUL = 2,  // v + (x - (v - vr)) * k
+  CH_PLAIN_INPUT_DIV = 3,  // v - (v - vr) / tau + x
+  CH_PLAIN_INPUT_MUL = 4   // v - (v - vr) * k + x
+};
+
+struct FwdArgs {
+  const void *x;
+  const void *v_init;
+  void *spike;
+  void *v_seq;           // may be null
+  void *v_last;          // may be null
+  void *h;               // may be null
+  const float *k_device; // may be null: use `tau`
+  int64_t T, N;
+  float tau;     // divisor (DIV charges) or multiplier k (MUL charges)
+  float vr_add;  // v_reset as an addend   (rounded to the storage dtype when every op is rounded)
+  float vr_mul;  // v_reset as a factor    (fp32 always)
+  float vth_sub; // v_threshold as a subtrahend
+  float vth_mul; // v_threshold as a factor
+  int charge;
+  int soft_reset;
+};
+
+// One neuron, one step.  R::round() is applied to the result of every arithmetic op.
+template <typename R, int CH, bool SOFT>
+__device__ __forceinline__ void neuron_step(float x, float &v, float &h, float &s, float tau,
+                                            const FwdArgs &a) {
+#pragma clang fp contract(off)
+  if (CH == CH_IF) {
+    h = Cvt<R>::round(v + x);
+  } else if (CH == CH_DECAY_INPUT_DIV || CH == CH_DECAY_INPUT_MUL) {
+    float d = Cvt<R>::round(v - a.vr_add);
+    float e = Cvt<R>::round(x - d);
+    float f = (CH == CH_DECAY_INPUT_DIV) ? Cvt<R>::round(e / tau) : Cvt<R>::round(e * tau);
+    h = Cvt<R>::round(v + f);
+  } else {
+    float d = Cvt<R>::round(v - a.vr_add);
+    float f = (CH == CH_PLAIN_INPUT_DIV) ? Cvt<R>::round(d / tau) : Cvt<R>::round(d * tau);
+    float g = Cvt<R>::round(v - f);
+    h = Cvt<R>::round(g + x);
+  }
+  float over = Cvt<R>::round(h - a.vth_sub);
+  s = (over >= 0.0f) ? 1.0f : 0.0f;
+  if (SOFT) {
+    float m = Cvt<R>::round(s * a.vth_mul);
+    v = Cvt<R>::round(h - m);
+  } else {
+    // kept in the reference's arithmetic form (not a select): 0 * v_reset and 0 * h keep the
+    // signed-zero / NaN behaviour of  s * v_reset + (1 - s) * h
+    float m = Cvt<R>::round(s * a.vr_mul);
+    float n = Cvt<R>::round(1.0f - s);
+    float o = Cvt<R>::round(n * h);
+    v = Cvt<R>::round(m + o);
+  }
+}
+
+template <typename S, bool VECTOR, bool ROUND_EACH, int CH, bool SOFT>
+__device__ __forceinline__ void forward_body(const FwdArgs &a) {
+  typedef Acc<S, VECTOR> A;
+  typedef typename A::elem_t E;
+  typedef typename std::conditional<ROUND_EACH, S, float>::type R;
+  constexpr int V = A::V;
+  constexpr int PF = SJHIP_FWD_PF;
+
+  const int64_t N = a.N, T = a.T;
+  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
+  if (col >= N) return;
+
+  const E *xp = (const E *)a.x + col;
+  E *sp = (E *)a.spike + col;
+  E *vp = a.v_seq ? (E *)a.v_seq + col : nullptr;
+  E *hp = a.h ? (E *)a.h + col : nullptr;
+  const float tau = a.k_device ? *a.k_device : a.tau;
+
+  typename A::raw_t ahead[PF];
+#pragma unroll
+  for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? A::load(xp + (int64_t)i * N) : A::zero();
+
+  float v[V];
+  A::unpack(A::load((const E *)a.v_init + col), v);
+
+  for (int64_t t0 = 0; t0 < T; t0 += PF) {
+    typename A::raw_t cur[PF];
+#pragma unroll
+    for (int i = 0; i < PF; ++i) cur[i] = ahead[i];
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int64_t tn = t0 + PF + i;
+      if (tn < T) ahead[i] = A::load(xp + tn * N);
+    }
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int64_t t = t0 + i;
+      if (t < T) {
+        float x[V], h[V], s[V];
+        A::unpack(cur[i], x);
+#pragma unroll
+        for (int j = 0; j < V; ++j) neuron_step<R, CH, SOFT>(x[j], v[j], h[j], s[j], tau, a);
+        A::store(sp + t * N, s);
+        if (hp) A::store(hp + t * N, h);
+        if (vp) A::store(vp + t * N, v);
+      }
+    }
+  }
+  if (a.v_last) A::store((E *)a.v_last + col, v);
+}
+
+template <typename S, bool VECTOR, bool ROUND_EACH, int CH>
+__device__ __forceinline__ void forward_reset_dispatch(const FwdArgs &a) {
+  if (a.soft_reset)
+    forward_body<S, VECTOR, ROUND_EACH, CH, true>(a);
+  else
+    forward_body<S, VECTOR, ROUND_EACH, CH, false>(a);
+}
+
+template <typename S, bool VECTOR, bool ROUND_EACH>
+__global__ void __launch_bounds__(512) forward_kernel(const FwdArgs a) {
+  switch (a.charge) {
+    case CH_IF: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_IF>(a); break;
+    case CH_DECAY_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_DIV>(a); break;
+    case CH_DECAY_INPUT_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_MUL>(a); break;
+    case CH_PLAIN_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_DIV>(a); break;
+    default: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_MUL>(a); break;
+  }
+}
+
+}  // namespace sjhip

@@ -1,0 +1,204 @@
+// C ABI of libsjhip.so (declared in include/sjhip.h): argument validation, thread-local error
+// text, launch tuning and the optional event profiler.  No entry point allocates device memory or
+// synchronises the host (sjhip_profile_read excepted, which waits for the events it reports on).
+#include "sjhip_common.h"
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+namespace sjhip {
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+struct TuningStore {
+  std::atomic<int> fwd_block{256};
+  std::atomic<int> bwd_block{256};
+  std::atomic<int> pack_block{256};
+};
+TuningStore g_tuning;
+
+struct EventPair {
+  hipEvent_t start, stop;
+  int kc;
+};
+std::mutex g_prof_mutex;
+std::atomic<int> g_prof_on{0};
+std::vector<EventPair> g_prof_pending;
+int64_t g_prof_count[KC_COUNT] = {0};
+double g_prof_ms[KC_COUNT] = {0};
+constexpr size_t kMaxPending = 4096;
+
+// caller holds g_prof_mutex
+void drain_pending() {
+  for (EventPair &e : g_prof_pending) {
+    float ms = 0.0f;
+    if (hipEventSynchronize(e.stop) == hipSuccess && hipEventElapsedTime(&ms, e.start, e.stop) == hipSuccess) {
+      g_prof_count[e.kc] += 1;
+      g_prof_ms[e.kc] += (double)ms;
+    }
+    (void)hipEventDestroy(e.start);
+    (void)hipEventDestroy(e.stop);
+  }
+  g_prof_pending.clear();
+}
+
+}  // namespace
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(SJHIP_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return SJHIP_OK;
+}
+
+const Tuning &tuning() {
+  thread_local Tuning t;
+  t.fwd_block = g_tuning.fwd_block.load(std::memory_order_relaxed);
+  t.bwd_block = g_tuning.bwd_block.load(std::memory_order_relaxed);
+  t.pack_block = g_tuning.pack_block.load(std::memory_order_relaxed);
+  return t;
+}
+
+ProfileScope::ProfileScope(int kernel_class, hipStream_t stream)
+    : kc_(kernel_class), stream_(stream), start_(nullptr), active_(false) {
+  if (!g_prof_on.load(std::memory_order_relaxed)) return;
+  if (hipEventCreate(&start_) != hipSuccess) return;
+  if (hipEventRecord(start_, stream_) != hipSuccess) { (void)hipEventDestroy(start_); return; }
+  active_ = true;
+}
+
+ProfileScope::~ProfileScope() {
+  if (!active_) return;
+  hipEvent_t stop;
+  if (hipEventCreate(&stop) != hipSuccess) { (void)hipEventDestroy(start_); return; }
+  (void)hipEventRecord(stop, stream_);
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  g_prof_pending.push_back(EventPair{start_, stop, kc_});
+  if (g_prof_pending.size() >= kMaxPending) drain_pending();
+}
+
+}  // namespace sjhip
+
+using namespace sjhip;
+
+namespace {
+
+bool valid_dtype_fp(int dtype) { return dtype == SJHIP_F32 || dtype == SJHIP_F16 || dtype == SJHIP_BF16; }
+
+int check_shape(const char *what, int64_t T, int64_t N) {
+  if (T < 1 || N < 1) return fail(SJHIP_ERR_INVALID, "%s: T=%lld N=%lld must be >= 1", what, (long long)T, (long long)N);
+  if (T > (int64_t(1) << 62) / N) return fail(SJHIP_ERR_TOO_LARGE, "%s: T*N overflows", what);
+  return SJHIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sjhip_abi_version(void) { return SJHIP_ABI_VERSION; }
+
+const char *sjhip_last_error(void) { return g_error; }
+
+int sjhip_neuron_forward(int neuron, int dtype, const sjhip_neuron_params *p, int64_t T, int64_t N,
+                         const void *x_seq, const void *v_init, const float *rtau_device, void *spike_seq,
+                         void *v_seq, void *v_last, void *h_seq, void *stream) {
+  if (!p) return fail(SJHIP_ERR_INVALID, "forward: params is NULL");
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_PLIF) return fail(SJHIP_ERR_INVALID, "forward: neuron %d", neuron);
+  if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "forward: dtype %d", dtype);
+  int rc = check_shape("forward", T, N);
+  if (rc != SJHIP_OK) return rc;
+  if (!x_seq || !v_init || !spike_seq) return fail(SJHIP_ERR_INVALID, "forward: NULL tensor");
+  if (!v_seq && !v_last) return fail(SJHIP_ERR_INVALID, "forward: neither v_seq nor v_last given");
+  return launch_forward(neuron, dtype, *p, T, N, x_seq, v_init, rtau_device, spike_seq, v_seq, v_last, h_seq,
+                        static_cast<hipStream_t>(stream));
+}
+
+int64_t sjhip_plif_workspace_floats(int dtype, int64_t N) {
+  if (N < 1) return 0;
+  return plif_blocks(dtype, N);
+}
+
+int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p, int64_t T, int64_t N,
+                          const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                          const void *h_seq, const void *v_init,
+                          const float *rtau_device, void *grad_x_seq, void *grad_v_init, float *grad_rtau,
+                          float *workspace, void *stream) {
+  if (!p) return fail(SJHIP_ERR_INVALID, "backward: params is NULL");
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_PLIF) return fail(SJHIP_ERR_INVALID, "backward: neuron %d", neuron);
+  if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "backward: dtype %d", dtype);
+  if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_ERF) return fail(SJHIP_ERR_UNSUPPORTED, "backward: surrogate id %d", p->sg_id);
+  int rc = check_shape("backward", T, N);
+  if (rc != SJHIP_OK) return rc;
+  if (!grad_spike_seq || !h_seq || !grad_x_seq || !grad_v_init) return fail(SJHIP_ERR_INVALID, "backward: NULL tensor");
+  if (neuron == SJHIP_NEURON_PLIF) {
+    if (!v_init || !grad_rtau) return fail(SJHIP_ERR_INVALID, "backward: PLIF needs v_init and grad_rtau");
+    if (!(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace) return fail(SJHIP_ERR_INVALID, "backward: PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");
+  }
+  return launch_backward(neuron, dtype, *p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, rtau_device, grad_x_seq,
+                         grad_v_init, grad_rtau, workspace, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, void *stream) {
+  if (n < 0) return fail(SJHIP_ERR_INVALID, "bit_pack: n=%lld", (long long)n);
+  if (n == 0) return SJHIP_OK;
+  if (!src || !dst) return fail(SJHIP_ERR_INVALID, "bit_pack: NULL buffer");
+  return launch_bit_pack(dtype, n, src, dst, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, void *stream) {
+  if (n < 0) return fail(SJHIP_ERR_INVALID, "bit_unpack: n=%lld", (long long)n);
+  if (n == 0) return SJHIP_OK;
+  if (!src || !dst) return fail(SJHIP_ERR_INVALID, "bit_unpack: NULL buffer");
+  return launch_bit_unpack(dtype, n, src, dst, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_set_tuning(const char *key, int value) {
+  if (!key) return fail(SJHIP_ERR_INVALID, "set_tuning: NULL key");
+  const bool block_ok = value == 64 || value == 128 || value == 256 || value == 512;
+  if (!strcmp(key, "fwd_block")) { if (!block_ok) return fail(SJHIP_ERR_INVALID, "set_tuning: fwd_block=%d", value); g_tuning.fwd_block = value; return SJHIP_OK; }
+  if (!strcmp(key, "bwd_block")) { if (!block_ok) return fail(SJHIP_ERR_INVALID, "set_tuning: bwd_block=%d", value); g_tuning.bwd_block = value; return SJHIP_OK; }
+  return fail(SJHIP_ERR_INVALID, "set_tuning: unknown key '%s'", key);
+}
+
+int sjhip_get_tuning(const char *key) {
+  if (!key) return fail(SJHIP_ERR_INVALID, "get_tuning: NULL key");
+  if (!strcmp(key, "fwd_block")) return g_tuning.fwd_block;
+  if (!strcmp(key, "bwd_block")) return g_tuning.bwd_block;
+  return fail(SJHIP_ERR_INVALID, "get_tuning: unknown key '%s'", key);
+}
+
+int sjhip_profile_enable(int on) {
+  g_prof_on.store(on ? 1 : 0);
+  return SJHIP_OK;
+}
+
+int sjhip_profile_reset(void) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  drain_pending();
+  for (int i = 0; i < KC_COUNT; ++i) { g_prof_count[i] = 0; g_prof_ms[i] = 0.0; }
+  return SJHIP_OK;
+}
+
+int sjhip_profile_read(int which, int64_t *launches, double *total_ms) {
+  if (which < 0 || which >= KC_COUNT) return fail(SJHIP_ERR_INVALID, "profile_read: class %d", which);
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  drain_pending();
+  if (launches) *launches = g_prof_count[which];
+  if (total_ms) *total_ms = g_prof_ms[which];
+  return SJHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,64 @@
+"""CPU-only: libsjhip.so loads and exports every symbol include/sjhip.h declares; argument
+validation that needs no device (errors are returned before any launch)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from spikingjelly_amd.activation_based.hip_kernel import library as L
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sjhip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sjhip_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_and_binding_list_the_same_symbols():
+    assert _declared_symbols() == sorted(L.EXPORTED_SYMBOLS)
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    lib = L.load()
+    assert lib.sjhip_abi_version() == L.ABI_VERSION
+    for name in _declared_symbols():
+        assert hasattr(lib, name), name
+
+
+def test_argument_validation_without_a_device():
+    lib = L.load()
+    p = L.NeuronParams(2.0, 1.0, 0.0, 2.0, 1, 0)
+    rc = lib.sjhip_neuron_forward(L.NEURON_LIF, L.DTYPE_F32, ctypes.byref(p), 0, 16, 1, 1, None, 1, 1, 1, None, None)
+    assert rc == -1 and b"T=0" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_forward(7, L.DTYPE_F32, ctypes.byref(p), 4, 16, 1, 1, None, 1, 1, 1, None, None)
+    assert rc == -1 and b"neuron 7" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_forward(L.NEURON_LIF, L.DTYPE_U8, ctypes.byref(p), 4, 16, 1, 1, None, 1, 1, 1, None, None)
+    assert rc == -1
+    rc = lib.sjhip_neuron_forward(L.NEURON_LIF, L.DTYPE_F32, ctypes.byref(p), 4, 16, 1, 1, None, 1, None, None, None, None)
+    assert rc == -1 and b"v_seq" in lib.sjhip_last_error()
+    p_bad = L.NeuronParams(2.0, 1.0, 0.0, 2.0, 9, 0)
+    rc = lib.sjhip_neuron_backward(L.NEURON_LIF, L.DTYPE_F32, ctypes.byref(p_bad), 4, 16, 1, None, None, 1, None, None,
+                                   1, 1, None, None, None)
+    assert rc == -2 and b"surrogate" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_backward(L.NEURON_PLIF, L.DTYPE_F32, ctypes.byref(p), 4, 16, 1, None, None, 1, None, None,
+                                   1, 1, None, None, None)
+    assert rc == -1 and b"PLIF" in lib.sjhip_last_error()
+    assert lib.sjhip_bit_pack(L.DTYPE_F32, -1, 1, 1, None) == -1
+    assert lib.sjhip_bit_pack(L.DTYPE_F32, 0, None, None, None) == 0
+    assert lib.sjhip_plif_workspace_floats(L.DTYPE_F32, 1 << 20) >= (1 << 20) // 1024
+    assert lib.sjhip_set_tuning(b"fwd_block", 100) == -1
+    assert lib.sjhip_set_tuning(b"fwd_block", 256) == 0 and lib.sjhip_get_tuning(b"fwd_block") == 256
+    assert lib.sjhip_set_tuning(b"nope", 1) == -1
+
+
+def test_python_binding_raises_with_library_message():
+    with pytest.raises(RuntimeError, match="set_tuning"):
+        L.set_tuning("fwd_block", 3)
+    with pytest.raises(NotImplementedError):
+        import torch
+
+        L.dtype_id(torch.float64)

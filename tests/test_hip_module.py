@@ -1,0 +1,189 @@
+"""The drop-in boundary on the GPU: ``backend='hip'`` nodes against ``backend='torch'`` nodes and the
+oracle, re-expressing the reference's own consistency tests (test_triton_neuron.py:671-766,
+test_cupy_backend_comprehensive.py:316-424, test_compile_compat.py:380-493, 659-675)."""
+
+import pytest
+import torch
+
+from oracle import neuron_oracle as no
+from spikingjelly_amd import configure
+from spikingjelly_amd.activation_based import functional, neuron, surrogate
+
+from helpers import bits_equal, seeded_randn
+
+pytestmark = pytest.mark.gpu
+
+GRAD_RTOL, GRAD_ATOL = 1e-5, 1e-6
+
+
+def _pair(cls, **kw):
+    a = cls(step_mode="m", backend="torch", **kw)
+    b = cls(step_mode="m", backend="hip", **kw).cuda()
+    return a, b
+
+
+def test_config1_lif_cpu_case():
+    """BASELINE config 1: x [4,64,128] ~ N(0.5,1) seed 1001, grad_spike seed 1101, LIF tau=2, hard reset,
+    ATan(2): spikes and h bit-exact, grad_x within 1e-5."""
+    x = seeded_randn((4, 64, 128), 1001, 0.5, 1.0)
+    gs = seeded_randn((4, 64, 128), 1101)
+    ref = no.forward_backward("lif", x.flatten(1), torch.zeros(64 * 128), gs.flatten(1), None, None, 2.0, True, 1.0,
+                              0.0, "atan", 2.0, False)
+    node = neuron.LIFNode(tau=2.0, surrogate_function=surrogate.ATan(2.0), step_mode="m", backend="hip",
+                          store_v_seq=True).cuda()
+    xd = x.cuda().requires_grad_()
+    s = node(xd)
+    s.backward(gs.cuda())
+    assert 0.05 < float(s.mean()) < 0.15
+    assert bits_equal(s.cpu().flatten(1), ref["spike_seq"])
+    assert bits_equal(node.v_seq.detach().cpu().flatten(1), ref["v_seq"])
+    assert bits_equal(node.v.detach().cpu().flatten(), ref["v_seq"][-1])
+    torch.testing.assert_close(xd.grad.cpu().flatten(1), ref["grad_x"], rtol=GRAD_RTOL, atol=GRAD_ATOL)
+
+
+@pytest.mark.parametrize("cls,kw", [
+    (neuron.IFNode, {}),
+    (neuron.LIFNode, {"tau": 2.0}),
+    (neuron.LIFNode, {"tau": 5.0, "decay_input": False}),
+    (neuron.ParametricLIFNode, {"init_tau": 2.0}),
+    (neuron.ParametricLIFNode, {"init_tau": 2.0, "decay_input": False}),
+])
+@pytest.mark.parametrize("v_reset", [0.0, -0.2, None])
+@pytest.mark.parametrize("detach_reset", [False, True])
+@pytest.mark.parametrize("sg", [surrogate.ATan, surrogate.Sigmoid])
+def test_hip_node_matches_torch_node(cls, kw, v_reset, detach_reset, sg):
+    a, b = _pair(cls, v_threshold=0.5, v_reset=v_reset, detach_reset=detach_reset, surrogate_function=sg(), **kw)
+    x = seeded_randn((6, 4, 12, 4), 20260428, 0.3, 1.0)
+    xa = x.clone().requires_grad_()
+    xb = x.cuda().requires_grad_()
+    sa, sb = a(xa), b(xb)
+    (sa.sum() + 0.5 * a.v.sum()).backward()
+    (sb.sum() + 0.5 * b.v.sum()).backward()
+    assert bits_equal(sb.cpu(), sa.detach())
+    assert bits_equal(b.v.detach().cpu(), a.v.detach())
+    torch.testing.assert_close(xb.grad.cpu(), xa.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+    if cls is neuron.ParametricLIFNode:
+        torch.testing.assert_close(b.w.grad.cpu(), a.w.grad, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("cls", [neuron.IFNode, neuron.LIFNode, neuron.ParametricLIFNode])
+@pytest.mark.parametrize("T,N", [(1, 48), (7, 111), (65, 64)])
+def test_store_v_seq_toggle_is_equivalent(cls, T, N):
+    x = seeded_randn((T, 2, N), 5, 0.4, 1.0).cuda()
+    gs, gv = seeded_randn((T, 2, N), 6).cuda(), seeded_randn((2, N), 7).cuda()
+    outs = []
+    for store in (False, True):
+        node = cls(step_mode="m", backend="hip", store_v_seq=store, surrogate_function=surrogate.ATan()).cuda()
+        xi = x.clone().requires_grad_()
+        s = node(xi)
+        ((s * gs).sum() + (node.v * gv).sum()).backward()
+        if store:
+            assert node.v_seq.shape == x.shape and bits_equal(node.v_seq[-1].detach(), node.v.detach())
+        else:
+            assert node.v_seq is None
+        outs.append((s.detach(), node.v.detach(), xi.grad))
+    for u, w in zip(*outs):
+        assert bits_equal(u, w)
+
+
+def test_non_contiguous_upstream_gradient():
+    x = seeded_randn((8, 16, 32), 8, 0.4, 1.0)
+    a, b = _pair(neuron.LIFNode, surrogate_function=surrogate.ATan())
+    xa, xb = x.clone().requires_grad_(), x.cuda().requires_grad_()
+    g = seeded_randn((32, 16, 8), 9).permute(2, 1, 0)
+    assert not g.is_contiguous()
+    a(xa).backward(g)
+    b(xb).backward(g.cuda())
+    torch.testing.assert_close(xb.grad.cpu(), xa.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+
+
+def test_v_init_gradient_and_user_assigned_state():
+    x = seeded_randn((5, 3, 40), 10, 0.4, 1.0)
+    v0 = seeded_randn((3, 40), 11, 0.0, 0.3)
+    a, b = _pair(neuron.LIFNode, tau=2.5, surrogate_function=surrogate.Sigmoid())
+    va, vb = v0.clone().requires_grad_(), v0.cuda().requires_grad_()
+    a.v, b.v = va, vb
+    sa, sb = a(x), b(x.cuda())
+    (sa.sum() + a.v.sum()).backward()
+    (sb.sum() + b.v.sum()).backward()
+    assert bits_equal(sb.cpu(), sa.detach())
+    torch.testing.assert_close(vb.grad.cpu(), va.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+
+
+def test_state_carries_over_and_batch_size_change_reinitialises():
+    a, b = _pair(neuron.LIFNode, surrogate_function=surrogate.ATan())
+    x1, x2 = seeded_randn((4, 8, 16), 12, 0.4, 1.0), seeded_randn((4, 8, 16), 13, 0.4, 1.0)
+    for x in (x1, x2):  # second call continues from the first call's v
+        assert bits_equal(b(x.cuda()).cpu(), a(x))
+    x3 = seeded_randn((4, 3, 16), 14, 0.4, 1.0)  # batch size changed without reset
+    assert bits_equal(b(x3.cuda()).cpu(), a(x3))
+    functional.reset_net(a)
+    functional.reset_net(b)
+    assert b.v == 0.0 and isinstance(b.v, float)
+    assert bits_equal(b(x1.cuda()).cpu(), a(x1))
+
+
+@pytest.mark.parametrize("ctx", ["eval", "no_grad", "inference_mode"])
+def test_inference_modes(ctx):
+    a, b = _pair(neuron.IFNode, v_reset=None, surrogate_function=surrogate.ATan())
+    x = seeded_randn((6, 4, 32), 15, 0.3, 0.5)
+    if ctx == "eval":
+        a.eval()
+        b.eval()
+        sa, sb = a(x), b(x.cuda())
+    else:
+        cm = torch.no_grad if ctx == "no_grad" else torch.inference_mode
+        with cm():
+            sa, sb = a(x), b(x.cuda())
+    assert bits_equal(sb.cpu(), sa) and bits_equal(b.v.cpu(), a.v)
+
+
+def test_unsupported_surrogate_and_primitive_mode_raise():
+    node = neuron.LIFNode(step_mode="m", backend="hip", surrogate_function=surrogate.PiecewiseLeakyReLU()).cuda()
+    x = torch.randn(4, 2, 8, device="cuda", requires_grad=True)
+    with pytest.raises(NotImplementedError, match="PiecewiseLeakyReLU"):
+        node(x)
+    node = neuron.LIFNode(step_mode="m", backend="hip", surrogate_function=surrogate.ATan(spiking=False)).cuda().eval()
+    with pytest.raises(NotImplementedError, match="spiking"):
+        node(x)
+    with pytest.raises(NotImplementedError):
+        neuron.LIFNode(step_mode="m", backend="hip")(torch.randn(4, 2, 8, device="cuda", dtype=torch.float64))
+
+
+def test_cpu_tensor_is_rejected_not_silently_computed():
+    node = neuron.LIFNode(step_mode="m", backend="hip")
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        node(torch.randn(4, 2, 8))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("cls", [neuron.IFNode, neuron.LIFNode, neuron.ParametricLIFNode])
+def test_half_nodes_match_torch_backend_bitwise(dtype, cls):
+    a, b = _pair(cls, v_reset=None, surrogate_function=surrogate.Sigmoid())
+    x = seeded_randn((8, 4, 64), 16, 0.3, 1.0).to(dtype)
+    with torch.no_grad():
+        sa, sb = a(x), b(x.cuda())
+    assert sb.dtype == dtype and bits_equal(sb.cpu(), sa) and bits_equal(b.v.cpu(), a.v)
+
+
+def test_fp32_state_mode_for_bf16_plif():
+    """Config-3 semantics: bf16 storage, fp32 state; oracle = the reference's mixed-precision recipe."""
+    x = seeded_randn((8, 4, 256), 1003, 0.2, 1.0).bfloat16()
+    es, ev, _ = no.multi_step_mixed_precision("plif", x.float().flatten(1), torch.zeros(4 * 256), torch.bfloat16, 0.5,
+                                              True, 1.0, None)
+    node = neuron.ParametricLIFNode(init_tau=2.0, v_reset=None, step_mode="m", backend="hip", store_v_seq=True).cuda()
+    old = configure.hip_half_precision_mode
+    configure.hip_half_precision_mode = "fp32_state"
+    try:
+        with torch.no_grad():
+            s = node(x.cuda())
+    finally:
+        configure.hip_half_precision_mode = old
+    assert torch.equal(s.cpu().float().flatten(1), es)
+    assert torch.equal(node.v_seq.cpu().float().flatten(1), ev)
+
+
+def test_set_backend_switches_supported_modules_only():
+    net = torch.nn.Sequential(neuron.LIFNode(step_mode="m"), torch.nn.Linear(4, 4), neuron.IFNode(step_mode="s"))
+    functional.set_backend(net, "hip")
+    assert net[0].backend == "hip" and net[2].backend == "torch"

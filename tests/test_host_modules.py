@@ -1,0 +1,208 @@
+"""CPU-only tests of the host-side mirror of the reference interface (torch backend + plumbing):
+function-vs-module consistency, memory semantics, backend validation, surrogate registry, the CPU
+path of the bit compressor, operator schemas / fake kernels."""
+
+import copy
+
+import pytest
+import torch
+
+from oracle import neuron_oracle as no
+from spikingjelly_amd.activation_based import base, functional, neuron, surrogate
+from spikingjelly_amd.activation_based.hip_kernel import neuron_kernel as K
+from spikingjelly_amd.activation_based.hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
+from spikingjelly_amd.activation_based.memopt import BitSpikeCompressor, BooleanSpikeCompressor
+
+from helpers import bits_equal, seeded_randn
+
+NODES = [
+    (neuron.IFNode, {}, "if", None),
+    (neuron.LIFNode, {"tau": 2.5}, "lif", 2.5),
+    (neuron.LIFNode, {"tau": 5.0, "decay_input": False}, "lif", 5.0),
+    (neuron.ParametricLIFNode, {"init_tau": 2.5}, "plif", None),
+]
+
+
+@pytest.mark.parametrize("cls,kw,kind,tau", NODES)
+@pytest.mark.parametrize("v_reset", [0.0, -0.2, None])
+@pytest.mark.parametrize("store_v_seq", [False, True])
+def test_torch_backend_module_equals_oracle(cls, kw, kind, tau, v_reset, store_v_seq):
+    x = seeded_randn((5, 3, 17), 1, 0.4, 1.0)
+    gs = seeded_randn((5, 3, 17), 2)
+    node = cls(v_threshold=0.7, v_reset=v_reset, surrogate_function=surrogate.ATan(), step_mode="m",
+               store_v_seq=store_v_seq, **kw)
+    xi = x.clone().requires_grad_()
+    s = node(xi)
+    s.backward(gs)
+    p = node.w.detach() if kind == "plif" else tau
+    ref = no.forward_backward(kind, x, torch.full((3, 17), 0.0 if v_reset is None else v_reset), gs, None, None, p,
+                              kw.get("decay_input", True), 0.7, v_reset, "atan", 2.0, False)
+    assert bits_equal(s.detach(), ref["spike_seq"])
+    assert bits_equal(node.v.detach(), ref["v_seq"][-1])
+    assert bits_equal(xi.grad, ref["grad_x"])
+    if store_v_seq:
+        assert bits_equal(node.v_seq.detach(), ref["v_seq"])
+    else:
+        assert node.v_seq is None
+
+
+def test_functional_forward_is_pure():
+    node = neuron.LIFNode(step_mode="m")
+    x = seeded_randn((4, 2, 8), 3, 0.5, 1.0)
+    (s,), (v,) = node.functional_forward((x,), (0.0,))
+    assert node.v == 0.0 and isinstance(node.v, float)
+    assert bits_equal(s, node(x)) and bits_equal(v, node.v)
+
+
+def test_single_step_and_multi_step_agree():
+    a = neuron.LIFNode(step_mode="s")
+    b = neuron.LIFNode(step_mode="m")
+    x = seeded_randn((6, 2, 8), 4, 0.5, 1.0)
+    assert bits_equal(torch.stack([a(x[t]) for t in range(6)]), b(x))
+
+
+def test_eval_mode_uses_heaviside_for_if_and_lif_only():
+    x = seeded_randn((3, 4), 5, 0.5, 1.0).requires_grad_()
+    lif = neuron.LIFNode(step_mode="m", surrogate_function=surrogate.ATan()).eval()
+    assert not lif(x).requires_grad  # plain Heaviside: no gradient path through the spike
+    plif = neuron.ParametricLIFNode(step_mode="m", surrogate_function=surrogate.ATan()).eval()
+    assert plif(x).requires_grad  # PLIF keeps its surrogate in eval
+    prim = neuron.LIFNode(step_mode="m", surrogate_function=surrogate.ATan(spiking=False)).eval()
+    out = prim(x)
+    assert ((out > 0) & (out < 1)).any()  # primitive mode stays smooth in eval
+
+
+def test_memory_semantics():
+    node = neuron.IFNode(step_mode="m")
+    assert "v" not in node.state_dict() and dict(node.named_memories()) == {"v": 0.0}
+    node(torch.ones(2, 3, 4))
+    assert isinstance(node.v, torch.Tensor) and node.v.shape == (3, 4)
+    node(torch.ones(2, 5, 4))  # batch size change: re-initialised, no error
+    assert node.v.shape == (5, 4)
+    node.reset()
+    assert node.v == 0.0 and node.v_seq is None
+    node.store_v_seq = True
+    node(torch.ones(2, 3, 4))
+    assert node.v_seq.shape == (2, 3, 4)
+    node.store_v_seq = True
+    assert node.v_seq is None  # setting the property clears it
+    clone = copy.deepcopy(node)
+    clone(torch.ones(2, 3, 4))
+    assert node.v_seq is None
+    with pytest.raises(AssertionError):
+        node.register_memory("v_threshold", 1.0)
+    hard = neuron.IFNode(v_reset=-0.5)
+    assert hard.v == -0.5 and hard.get_reset_value("v") == -0.5
+    x = torch.ones(3, requires_grad=True)
+    hard(x)
+    assert hard.v.requires_grad
+    hard.detach()
+    assert not hard.v.requires_grad
+
+
+def test_backend_and_step_mode_validation():
+    node = neuron.LIFNode()
+    assert node.supported_backends == ("torch",)
+    with pytest.raises(NotImplementedError, match="hip is not a supported backend"):
+        node.backend = "hip"  # single-step mode has no hip backend
+    node.step_mode = "m"
+    assert node.supported_backends == ("torch", "hip")
+    node.backend = "hip"
+    with pytest.raises(NotImplementedError):
+        node.backend = "cupy"
+    with pytest.raises(ValueError):
+        node.step_mode = "x"
+    with pytest.raises(AssertionError):
+        neuron.LIFNode(tau=1.0)
+    with pytest.raises(AssertionError):
+        neuron.IFNode(v_threshold=1)
+    assert "backend=hip" in repr(node) and "tau=2.0" in repr(node)
+
+
+def test_check_backend_library_reports_missing_library(monkeypatch):
+    from spikingjelly_amd.activation_based.hip_kernel import library
+
+    monkeypatch.setattr(library, "_lib", None)
+    monkeypatch.setattr(library, "library_path", lambda: "/nonexistent/libsjhip.so")
+    with pytest.raises(ImportError, match="libsjhip.so"):
+        base.check_backend_library("hip")
+
+
+def test_net_helpers():
+    net = torch.nn.Sequential(neuron.IFNode(), torch.nn.Linear(4, 4), neuron.ParametricLIFNode())
+    functional.set_step_mode(net, "m")
+    assert net[0].step_mode == "m" and net[2].step_mode == "m"
+    functional.set_backend(net, "hip", instance=neuron.IFNode)
+    assert net[0].backend == "hip" and net[2].backend == "torch"
+    net[2](torch.ones(2, 3, 4))
+    functional.reset_net(net)
+    functional.reset_net(net)  # cached module list path
+    assert net[2].v == 0.0
+    x = torch.ones(2, 3, 4, requires_grad=True)
+    net[2](x)
+    functional.detach_net(net)
+    assert not net[2].v.requires_grad
+
+
+def test_surrogate_objects_and_registry():
+    assert repr(surrogate.ATan()) == "ATan(alpha=2.0, spiking=True)"
+    assert resolve_sg_hip_id_and_alpha(surrogate.Sigmoid()) == (0, 4.0)
+    assert resolve_sg_hip_id_and_alpha(surrogate.ATan(alpha=torch.tensor([3.0]))) == (1, 3.0)
+    assert resolve_sg_hip_id_and_alpha(surrogate.Erf()) == (6, 2.0)
+    with pytest.raises(NotImplementedError, match="PiecewiseLeakyReLU"):
+        resolve_sg_hip_id_and_alpha(surrogate.PiecewiseLeakyReLU())
+    with pytest.raises(TypeError):
+        resolve_sg_hip_id_and_alpha(surrogate.ATan(alpha=torch.ones(2)))
+    x = torch.tensor([-0.75, -0.25, 0.25, 0.75], dtype=torch.float64)
+    for cls in (surrogate.Sigmoid, surrogate.ATan, surrogate.PiecewiseQuadratic, surrogate.PiecewiseExp,
+                surrogate.SoftSign, surrogate.Erf, surrogate.PiecewiseLeakyReLU):
+        f = cls()
+        xs = x.clone().requires_grad_()
+        out = f(xs)
+        out.sum().backward()
+        f.set_spiking_mode(False)
+        fd = (f(x + 1e-5) - f(x - 1e-5)) / 2e-5
+        assert torch.equal(out.detach(), surrogate.heaviside(x))
+        torch.testing.assert_close(xs.grad, fd, atol=1e-4, rtol=1e-4)
+
+
+def test_bit_compressor_cpu_path():
+    spikes = torch.tensor([[1.0, 0.0, 1.0], [0.0, 1.0, 0.0]])
+    c = BitSpikeCompressor()
+    packed = c.compress(spikes)
+    assert packed.device.type == "cpu" and packed.tolist() == [0b010101]
+    torch.testing.assert_close(c.decompress(packed, tuple(spikes.shape)), spikes)
+    b = BooleanSpikeCompressor()
+    assert torch.equal(b.decompress(b.compress(spikes.half()), spikes.shape), spikes.half())
+
+
+def test_operator_schemas_and_fake_kernels():
+    """Shapes under fake tensors: (x.shape, x.shape | (0,), v.shape, x.shape), like
+    test_compile_compat.py:496-525 checks for the reference ops."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    assert "Tensor? grad_v_seq" in str(torch.ops.sj.hip_multistep_lif_backward.default._schema)
+    with FakeTensorMode():
+        x = torch.empty(5, 12)
+        v = torch.empty(12)
+        s, v_seq, v_last, h = torch.ops.sj.hip_multistep_lif_forward(x, v, 1.0, 0.0, False, False, 2.0, True, 1, 2.0,
+                                                                     True, 0)
+        assert s.shape == v_seq.shape == h.shape == (5, 12) and v_last.shape == (12,)
+        s, v_seq, v_last = torch.ops.sj.hip_multistep_if_inference(x, v, 1.0, 0.0, True, False, 0)
+        assert v_seq.shape == (0,) and v_last.shape == (12,)
+        gx, gvi, gk = torch.ops.sj.hip_multistep_plif_backward(x, None, None, x, v, torch.empty(()), 1.0, 0.0, False,
+                                                               False, True, 0, 4.0, 0)
+        assert gx.shape == (5, 12) and gvi.shape == (12,) and gk.shape == ()
+
+
+def test_functional_names_follow_the_backend_naming_rule():
+    """<neuron>_multi_step_<backend>, fully annotated, exported (reference
+    test/activation_based/test_functional_neuron.py:709-732)."""
+    import inspect
+
+    for name in ("if_multi_step_hip", "lif_multi_step_hip", "plif_multi_step_hip"):
+        fn = getattr(functional, name)
+        sig = inspect.signature(fn)
+        assert all(p.annotation is not inspect.Parameter.empty for p in sig.parameters.values())
+        assert sig.return_annotation is not inspect.Signature.empty
+        assert list(sig.parameters)[-2:] == ["detach_reset", "store_v_seq"]

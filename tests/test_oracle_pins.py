@@ -1,0 +1,356 @@
+"""Pins the CPU oracle (oracle/) before anything is compared against it.
+
+Each test is chosen so that a plausible mistake in the restatement -- a dropped term, a wrong sign
+or index, a multiplication where the reference divides -- fails it.  None of these tests retypes
+the oracle's own formula: expectations come from exact rational arithmetic (golden fixture),
+closed forms, finite differences, numpy library routines or an independent implementation.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import bitpack_oracle, bptt_oracle
+from oracle import neuron_oracle as no
+
+from helpers import bits_equal, load_dyadic, seeded_randn
+
+torch.set_num_threads(4)
+
+
+# ------------------------------------------------------------------------------------------------
+# 1. known-answer vectors (exact rational arithmetic), reference input test_triton_neuron.py:1207-1216
+# ------------------------------------------------------------------------------------------------
+def _dyadic_cases():
+    doc = load_dyadic()
+    return [(doc, i) for i in range(len(doc["cases"]))]
+
+
+@pytest.mark.parametrize("doc,i", _dyadic_cases(), ids=lambda v: str(v) if isinstance(v, int) else "d")
+def test_torch_oracle_matches_dyadic_golden(doc, i):
+    c = doc["cases"][i]
+    x = torch.tensor(doc["x"], dtype=torch.float32) * c["scale"]
+    v0 = torch.tensor(doc["v_init"], dtype=torch.float32)
+    kind = c["kind"]
+    p = {"if": None, "lif": 1.0 / c["k"], "plif": torch.tensor(math.log(c["k"] / (1 - c["k"])))}[kind]
+    s, v, h = no.multi_step(kind, x, v0, p, c["decay_input"], c["v_threshold"], c["v_reset"])
+    assert torch.equal(s, torch.tensor(c["spike"], dtype=torch.float32))
+    assert torch.equal(h, torch.tensor(c["h"], dtype=torch.float32))
+    assert torch.equal(v, torch.tensor(c["v"], dtype=torch.float32))
+
+
+@pytest.mark.parametrize("doc,i", _dyadic_cases(), ids=lambda v: str(v) if isinstance(v, int) else "d")
+def test_c_oracle_matches_dyadic_golden(doc, i, c_oracle):
+    c = doc["cases"][i]
+    x = np.array(doc["x"], dtype=np.float32) * np.float32(c["scale"])
+    v0 = np.array(doc["v_init"], dtype=np.float32)
+    tau = {"if": 1.0, "lif": 1.0 / c["k"], "plif": c["k"]}[c["kind"]]
+    s, v, h = c_oracle.forward_f32(c["kind"], x, v0, tau, c["decay_input"], c["v_threshold"], c["v_reset"])
+    assert np.array_equal(s, np.array(c["spike"], dtype=np.float32))
+    assert np.array_equal(h, np.array(c["h"], dtype=np.float32))
+    assert np.array_equal(v, np.array(c["v"], dtype=np.float32))
+
+
+@pytest.mark.parametrize("storage", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("doc,i", _dyadic_cases(), ids=lambda v: str(v) if isinstance(v, int) else "d")
+def test_half_precision_oracles_match_dyadic_golden(doc, i, storage):
+    """All golden values fit bf16, so both 16-bit semantics must reproduce them exactly."""
+    c = doc["cases"][i]
+    x = torch.tensor(doc["x"], dtype=torch.float32) * c["scale"]
+    v0 = torch.tensor(doc["v_init"], dtype=torch.float32)
+    kind = c["kind"]
+    for order in (True, False):
+        if not order and c["v_reset"] not in (0.0, None):
+            continue
+        s, v, h = no.multi_step_mixed_precision(kind, x, v0, storage, c["k"], c["decay_input"], c["v_threshold"],
+                                                c["v_reset"], torch_op_order=order)
+        assert torch.equal(s, torch.tensor(c["spike"], dtype=torch.float32))
+        assert torch.equal(h, torch.tensor(c["h"], dtype=torch.float32))
+        assert torch.equal(v, torch.tensor(c["v"], dtype=torch.float32))
+    p = {"if": None, "lif": 1.0 / c["k"], "plif": torch.tensor(math.log(c["k"] / (1 - c["k"])))}[kind]
+    s, v, h = no.multi_step(kind, x.to(storage), v0.to(storage), p, c["decay_input"], c["v_threshold"], c["v_reset"])
+    assert s.dtype == storage and v.dtype == storage
+    assert torch.equal(s.float(), torch.tensor(c["spike"], dtype=torch.float32))
+    assert torch.equal(v.float(), torch.tensor(c["v"], dtype=torch.float32))
+
+
+# ------------------------------------------------------------------------------------------------
+# 2. closed forms and invariants
+# ------------------------------------------------------------------------------------------------
+def test_single_step_from_rest_is_x_over_tau():
+    x = seeded_randn((1, 1000), 1)
+    for tau in (2.0, 3.0, 10.0):
+        _, _, h = no.multi_step("lif", x, torch.zeros(1000), tau, True, 1e9, 0.0)
+        assert torch.equal(h[0], x[0] / tau)
+        _, _, h = no.multi_step("lif", x, torch.zeros(1000), tau, False, 1e9, 0.0)
+        assert torch.equal(h[0], x[0])
+
+
+def test_zero_input_decays_geometrically_towards_v_reset():
+    T, tau, vr = 12, 4.0, -0.5
+    v0 = torch.tensor([0.75, -1.25, 0.0], dtype=torch.float64)
+    x = torch.zeros(T, 3, dtype=torch.float64)
+    for decay_input in (True, False):
+        _, v, h = no.multi_step("lif", x, v0, tau, decay_input, 10.0, vr)
+        expect = torch.stack([vr + (v0 - vr) * (1 - 1 / tau) ** (t + 1) for t in range(T)])
+        torch.testing.assert_close(h, expect, rtol=1e-13, atol=1e-13)
+        torch.testing.assert_close(v, expect, rtol=1e-13, atol=1e-13)
+
+
+def test_if_soft_reset_rate_coding_identity():
+    """Constant dyadic input x in [0,1), v_th=1, soft reset: after T steps the spike count is
+    floor(T x) and the residual potential is T x - count, exactly (ANN2SNN rate coding)."""
+    T = 32
+    xs = torch.arange(0, 64, dtype=torch.float32) / 64.0
+    x = xs.expand(T, -1).contiguous()
+    s, v, _ = no.multi_step("if", x, torch.zeros(64), None, True, 1.0, None)
+    count = s.sum(0)
+    assert torch.equal(count, torch.floor(T * xs))
+    assert torch.equal(v[-1], T * xs - count)
+    # the same in fp16 (all values exact there too)
+    s16, v16, _ = no.multi_step("if", x.half(), torch.zeros(64).half(), None, True, 1.0, None)
+    assert torch.equal(s16.float(), s) and torch.equal(v16.float(), v)
+
+
+@pytest.mark.parametrize("kind,p", [("if", None), ("lif", 3.0), ("plif", torch.tensor(0.3))])
+@pytest.mark.parametrize("v_reset", [0.0, -0.2, None])
+def test_fire_and_reset_invariants(kind, p, v_reset):
+    x = seeded_randn((9, 500), 7, 0.4, 1.0)
+    vth = 0.8
+    s, v, h = no.multi_step(kind, x, torch.zeros(500), p, True, vth, v_reset)
+    assert set(s.unique().tolist()) <= {0.0, 1.0}
+    assert torch.equal(s, (h >= vth).float())
+    fired = s.bool()
+    assert fired.any() and (~fired).any()
+    if v_reset is None:
+        assert torch.equal(v[fired], h[fired] - vth)
+    else:
+        assert torch.equal(v[fired], torch.full_like(v[fired], v_reset))
+    assert torch.equal(v[~fired], h[~fired])
+
+
+def test_plif_equals_lif_when_tau_is_a_power_of_two():
+    """k = sigmoid(-log(tau-1)) = 1/tau; for tau = 2 the product equals the quotient bit for bit."""
+    x = seeded_randn((8, 777), 11, 0.3, 0.8)
+    w = torch.tensor(-math.log(2.0 - 1.0))
+    for decay_input in (True, False):
+        a = no.multi_step("lif", x, torch.zeros(777), 2.0, decay_input, 1.0, 0.0)
+        b = no.multi_step("plif", x, torch.zeros(777), w, decay_input, 1.0, 0.0)
+        for u, w_ in zip(a, b):
+            assert bits_equal(u, w_)
+
+
+def test_lif_divides_rather_than_multiplies():
+    """The torch backend divides by tau; a restatement that multiplies by 1/tau differs for tau=3."""
+    x = seeded_randn((1, 100000), 5)
+    _, _, h = no.multi_step("lif", x, torch.zeros(100000), 3.0, True, 1e9, 0.0)
+    assert torch.equal(h[0], x[0] / 3.0)
+    assert not torch.equal(h[0], x[0] * (1.0 / 3.0))
+
+
+# ------------------------------------------------------------------------------------------------
+# 3. surrogate gradients: finite difference of the primitive (reference
+#    test_neuron_kernel_surrogate_contract.py:25-44) and the values at 0
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["sigmoid", "atan", "piecewise_quadratic", "piecewise_exp", "soft_sign", "erf"])
+def test_surrogate_gradient_is_derivative_of_primitive(name):
+    alpha = no.SG_DEFAULT_ALPHA[name]
+    x = torch.tensor([-0.75, -0.25, 0.25, 0.75], dtype=torch.float64)
+    xs = x.clone().requires_grad_()
+    out = no.surrogate(name, alpha)(xs)
+    out.sum().backward()
+    eps = 1e-5
+    fd = (no.primitive(name, x + eps, alpha) - no.primitive(name, x - eps, alpha)) / (2 * eps)
+    assert torch.equal(out.detach(), no.heaviside(x))
+    torch.testing.assert_close(xs.grad, fd, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(no.surrogate_grad(name, x, alpha), fd, atol=1e-4, rtol=1e-4)
+
+
+def test_surrogate_gradient_values_at_zero():
+    z = torch.zeros(1, dtype=torch.float64)
+    assert no.surrogate_grad("atan", z, 2.0).item() == pytest.approx(1.0)        # alpha/2
+    assert no.surrogate_grad("atan", z, 3.0).item() == pytest.approx(1.5)
+    assert no.surrogate_grad("sigmoid", z, 4.0).item() == pytest.approx(1.0)     # alpha/4
+    assert no.surrogate_grad("super_spike", z, 1.5).item() == pytest.approx(1.5)  # alpha
+    assert no.surrogate_grad("erf", z, 2.0).item() == pytest.approx(2.0 / math.sqrt(math.pi))
+
+
+# ------------------------------------------------------------------------------------------------
+# 4. BPTT: closed-form recurrence == autograd of the restated ops == finite differences
+# ------------------------------------------------------------------------------------------------
+def _np_sg_prime(name, alpha):
+    return lambda z: no.surrogate_grad(name, torch.from_numpy(np.ascontiguousarray(z)), alpha).numpy()
+
+
+GRID = [(kind, sg, di, vr, det)
+        for kind in ("if", "lif", "plif")
+        for sg in ("atan", "sigmoid")
+        for di in ((True,) if kind == "if" else (True, False))
+        for vr in (0.0, -0.2, None)
+        for det in (False, True)]
+
+
+@pytest.mark.parametrize("kind,sg,decay_input,v_reset,detach", GRID)
+def test_recurrence_equals_autograd_float64(kind, sg, decay_input, v_reset, detach):
+    T, N, tau, vth = 6, 257, 3.0, 0.7
+    alpha = no.SG_DEFAULT_ALPHA[sg]
+    x = seeded_randn((T, N), 21, 0.4, 1.0, torch.float64)
+    v0 = seeded_randn((N,), 22, 0.0, 0.3, torch.float64)
+    gs = seeded_randn((T, N), 23, dtype=torch.float64)
+    gv = seeded_randn((T, N), 24, 0.0, 0.1, torch.float64)
+    gl = seeded_randn((N,), 25, 0.0, 0.1, torch.float64)
+    w = torch.tensor(-math.log(tau - 1.0), dtype=torch.float64)
+    p = {"if": None, "lif": tau, "plif": w}[kind]
+    ref = no.forward_backward(kind, x, v0, gs, gv, gl, p, decay_input, vth, v_reset, sg, alpha, detach)
+    k = {"if": 0.0, "lif": 1.0 / tau, "plif": float(w.sigmoid())}[kind]
+    v_prev = torch.cat([v0[None], ref["v_seq"][:-1]]).numpy()
+    gx, gvi, gk = bptt_oracle.bptt(kind, ref["h_seq"].numpy(), ref["spike_seq"].numpy(), _np_sg_prime(sg, alpha),
+                                   gs.numpy(), gv.numpy(), gl.numpy(), k, decay_input, vth, v_reset, detach,
+                                   v_prev, x.numpy())
+    np.testing.assert_allclose(gx, ref["grad_x"].numpy(), rtol=1e-11, atol=1e-13)
+    np.testing.assert_allclose(gvi, ref["grad_v_init"].numpy(), rtol=1e-11, atol=1e-13)
+    if kind == "plif":
+        # dL/dw = dL/dk * k (1 - k)   (reference test_triton_neuron.py:807-809)
+        assert gk * k * (1 - k) == pytest.approx(float(ref["grad_p"]), rel=1e-10)
+
+
+@pytest.mark.parametrize("kind", ["if", "lif", "plif"])
+@pytest.mark.parametrize("v_reset", [0.0, -0.2, None])
+@pytest.mark.parametrize("decay_input", [True, False])
+def test_recurrence_matches_finite_differences_of_the_smooth_network(kind, v_reset, decay_input):
+    """With the primitive (non-spiking) surrogate the network is smooth, autograd is its true
+    gradient and the recurrence (s_t = primitive, sg = primitive') must match central differences."""
+    if kind == "if" and not decay_input:
+        pytest.skip("IF has no decay_input")
+    T, N, tau, vth, alpha = 5, 7, 2.5, 0.6, 2.0
+    x = seeded_randn((T, N), 31, 0.4, 0.8, torch.float64)
+    v0 = seeded_randn((N,), 32, 0.0, 0.3, torch.float64)
+    gs = seeded_randn((T, N), 33, dtype=torch.float64)
+    gv = seeded_randn((T, N), 34, dtype=torch.float64)
+    w = torch.tensor(-math.log(tau - 1.0), dtype=torch.float64)
+    p = {"if": None, "lif": tau, "plif": w}[kind]
+    k = {"if": 0.0, "lif": 1.0 / tau, "plif": float(w.sigmoid())}[kind]
+    smooth = no.surrogate("atan", alpha, spiking=False)
+
+    def loss(x_, v0_, k_=None):
+        pp = p if k_ is None else k_
+        kk = kind if k_ is None else "plif_k"
+        s, v, _ = no.multi_step(kk, x_, v0_, pp, decay_input, vth, v_reset, smooth)
+        return float((s * gs).sum() + (v * gv).sum())
+
+    s, v, h = no.multi_step(kind, x, v0, p, decay_input, vth, v_reset, smooth)
+    v_prev = torch.cat([v0[None], v[:-1]]).numpy()
+    gx, gvi, gk = bptt_oracle.bptt(kind, h.numpy(), s.numpy(), _np_sg_prime("atan", alpha), gs.numpy(), gv.numpy(),
+                                   None, k, decay_input, vth, v_reset, False, v_prev, x.numpy())
+    eps = 1e-6
+    for (t, n) in [(0, 0), (2, 3), (T - 1, N - 1)]:
+        xp, xm = x.clone(), x.clone()
+        xp[t, n] += eps
+        xm[t, n] -= eps
+        assert (loss(xp, v0) - loss(xm, v0)) / (2 * eps) == pytest.approx(gx[t, n], rel=1e-6, abs=1e-8)
+    vp, vm = v0.clone(), v0.clone()
+    vp[2] += eps
+    vm[2] -= eps
+    assert (loss(x, vp) - loss(x, vm)) / (2 * eps) == pytest.approx(gvi[2], rel=1e-6, abs=1e-8)
+    if kind == "plif":
+        kt = torch.tensor(k, dtype=torch.float64)
+        fd = (loss(x, v0, kt + eps) - loss(x, v0, kt - eps)) / (2 * eps)
+        assert fd == pytest.approx(gk, rel=1e-6, abs=1e-8)
+
+
+def test_c_backward_equals_recurrence(c_oracle):
+    T, N, tau, vth = 7, 129, 3.0, 0.9
+    x = seeded_randn((T, N), 41, 0.4, 1.0)
+    v0 = seeded_randn((N,), 42, 0.0, 0.3)
+    gs, gv, gl = seeded_randn((T, N), 43), seeded_randn((T, N), 44, 0, 0.1), seeded_randn((N,), 45, 0, 0.1)
+    for kind in ("if", "lif", "plif"):
+        for sg_id, sg in enumerate(no.SG_NAMES):
+            for v_reset in (0.0, -0.2, None):
+                for detach in (False, True):
+                    for di in ((True,) if kind == "if" else (True, False)):
+                        k = 0.0 if kind == "if" else 1.0 / tau
+                        alpha = no.SG_DEFAULT_ALPHA[sg]
+                        s, v, h = c_oracle.forward_f32(kind, x.numpy(), v0.numpy(), tau if kind == "lif" else k, di,
+                                                       vth, v_reset)
+                        v_prev = np.concatenate([v0.numpy()[None], v[:-1]]).astype(np.float64)
+                        e = bptt_oracle.bptt(kind, h, s, _np_sg_prime(sg, alpha), gs.double().numpy(),
+                                             gv.double().numpy(), gl.double().numpy(), float(np.float32(k)) if kind == "plif" else k,
+                                             di, vth, v_reset, detach, v_prev, x.double().numpy())
+                        a = c_oracle.backward_f64(kind, gs.numpy(), gv.numpy(), gl.numpy(), h,
+                                                  float(np.float32(k)) if kind == "plif" else k, di, vth, v_reset,
+                                                  detach, sg_id, alpha, x.numpy(), v0.numpy(), v)
+                        np.testing.assert_allclose(a[0], e[0], rtol=1e-9, atol=1e-12)
+                        np.testing.assert_allclose(a[1], e[1], rtol=1e-9, atol=1e-12)
+                        if kind == "plif":
+                            assert a[2] == pytest.approx(e[2], rel=1e-9)
+
+
+# ------------------------------------------------------------------------------------------------
+# 5. torch oracle == C oracle bit for bit (two independent implementations of IEEE fp32)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("kind", ["if", "lif", "plif"])
+@pytest.mark.parametrize("v_reset", [0.0, -0.2, None])
+@pytest.mark.parametrize("decay_input", [True, False])
+@pytest.mark.parametrize("tau", [2.0, 3.0, 10.0])
+def test_torch_and_c_oracle_agree_bitwise(kind, v_reset, decay_input, tau, c_oracle):
+    if kind == "if" and (not decay_input or tau != 2.0):
+        pytest.skip("IF has neither tau nor decay_input")
+    T, N = 16, 4099
+    x = seeded_randn((T, N), 51, 0.3, 0.8)
+    v0 = seeded_randn((N,), 52, 0.0, 0.2)
+    if kind == "plif":
+        w = torch.tensor(-math.log(tau - 1.0))
+        kf = float(w.sigmoid())  # the fp32 value torch multiplies by
+        s, v, h = no.multi_step("plif", x, v0, w, decay_input, 0.5, v_reset)
+        cs, cv, ch = c_oracle.forward_f32("plif", x.numpy(), v0.numpy(), kf, decay_input, 0.5, v_reset)
+    else:
+        s, v, h = no.multi_step(kind, x, v0, tau, decay_input, 0.5, v_reset)
+        cs, cv, ch = c_oracle.forward_f32(kind, x.numpy(), v0.numpy(), tau, decay_input, 0.5, v_reset)
+    assert 0.001 < s.mean() < 0.7
+    assert bits_equal(s, torch.from_numpy(cs))
+    assert bits_equal(h, torch.from_numpy(ch))
+    assert bits_equal(v, torch.from_numpy(cv))
+
+
+# ------------------------------------------------------------------------------------------------
+# 6. bit-packing
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [0, 1, 6, 7, 8, 9, 17, 64, 1000, 4097])
+def test_bitpack_oracles_equal_numpy_packbits(n, c_oracle):
+    rng = np.random.default_rng(n)
+    bits = (rng.random(n) < 0.3).astype(np.float32)
+    expect = np.packbits(bits.astype(np.uint8), bitorder="little")
+    got = bitpack_oracle.bit_spike_compress(bits)
+    assert np.array_equal(got, expect)
+    assert np.array_equal(c_oracle.bit_pack(bits), expect)
+    assert np.array_equal(bitpack_oracle.bit_spike_decompress(got, (n,)), bits.astype(np.uint8))
+    assert np.array_equal(c_oracle.bit_unpack(got, n), bits.astype(np.uint8))
+    assert np.array_equal(np.unpackbits(got, bitorder="little")[:n], bits.astype(np.uint8))
+
+
+def test_bitpack_reference_round_trips(c_oracle):
+    # test/activation_based/test_checkpointing.py:275-282 and :647-662
+    spikes = np.array([[1.0, 0.0, 1.0], [0.0, 1.0, 0.0]], dtype=np.float32)
+    packed = bitpack_oracle.bit_spike_compress(spikes)
+    assert packed.tolist() == [0b010101]
+    assert np.array_equal(bitpack_oracle.bit_spike_decompress(packed, spikes.shape), spikes.astype(np.uint8))
+    # test/activation_based/test_cuda_custom_op_migration.py:179-190: 17 elements, every third one set
+    spike = (np.arange(17) % 3 == 0).astype(np.float32)
+    packed = bitpack_oracle.bit_spike_compress(spike)
+    assert packed.tolist() == [0b01001001, 0b10010010, 0b0]
+    assert np.array_equal(c_oracle.bit_pack(spike), packed)
+    assert np.array_equal(bitpack_oracle.bit_spike_decompress(packed, (17,)), spike.astype(np.uint8))
+
+
+def test_bitpack_nonzero_semantics(c_oracle):
+    """`.to(torch.bool)`: -0.0 is no spike, NaN / 2.0 / subnormals are."""
+    vals = np.array([0.0, -0.0, 1.0, 2.0, np.nan, 1e-45, -1.0, 0.0], dtype=np.float32)
+    expect = np.packbits(torch.from_numpy(vals).to(torch.bool).numpy().astype(np.uint8), bitorder="little")
+    assert np.array_equal(bitpack_oracle.bit_spike_compress(vals), expect)
+    assert np.array_equal(c_oracle.bit_pack(vals), expect)
+    for dt in (torch.float16, torch.bfloat16):
+        t = torch.from_numpy(vals).to(dt)
+        e = np.packbits(t.to(torch.bool).numpy().astype(np.uint8), bitorder="little")
+        assert np.array_equal(c_oracle.bit_pack(t.view(torch.int16).numpy()), e)
