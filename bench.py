@@ -115,7 +115,7 @@ def main() -> int:
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     L.profile_enable(False)
-    rate = float(spikes.mean())
+    rate = float(spikes.detach().mean())
     n_fwd, ms_fwd = L.profile_read(L.KC_FORWARD)
     n_bwd, ms_bwd = L.profile_read(L.KC_BACKWARD)
 

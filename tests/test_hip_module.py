@@ -34,7 +34,7 @@ def test_config1_lif_cpu_case():
     xd = x.cuda().requires_grad_()
     s = node(xd)
     s.backward(gs.cuda())
-    assert 0.05 < float(s.mean()) < 0.15
+    assert 0.05 < float(s.detach().mean()) < 0.15
     assert bits_equal(s.cpu().flatten(1), ref["spike_seq"])
     assert bits_equal(node.v_seq.detach().cpu().flatten(1), ref["v_seq"])
     assert bits_equal(node.v.detach().cpu().flatten(), ref["v_seq"][-1])
