@@ -156,8 +156,10 @@ int sjhip_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, void *st
 int sjhip_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, void *stream);
 
 /*
- * Launch tuning (process-wide, read at launch).  key = "fwd_block" or "bwd_block", value = work-items
- * per block (64, 128, 256 or 512).  Returns SJHIP_ERR_INVALID otherwise.  Results never depend on these.
+ * Launch tuning (process-wide, read at launch).  Keys: "fwd_block" / "bwd_block" = work-items per
+ * block (64, 128, 256 or 512); "fwd_blocks_per_cu" / "bwd_blocks_per_cu" = cap on resident blocks per
+ * compute unit (0 = none, else 2..64; enforced through a dynamic-LDS request).  Returns
+ * SJHIP_ERR_INVALID otherwise.  Results never depend on these.
  */
 int sjhip_set_tuning(const char *key, int value);
 int sjhip_get_tuning(const char *key);

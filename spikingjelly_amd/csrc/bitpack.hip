@@ -52,7 +52,7 @@ __global__ void __launch_bounds__(256) pack_vector_kernel(const u32x4 *__restric
 #pragma unroll
   for (int i = 0; i < PACK_R; ++i) {
     const int64_t item = base + (int64_t)i * blockDim.x;
-    r[i] = (item < items) ? stream_load(src + item) : (u32x4)(0u);
+    r[i] = (item < items) ? stream_load<true>(src + item) : (u32x4)(0u);
   }
 #pragma unroll
   for (int i = 0; i < PACK_R; ++i) {
@@ -125,7 +125,7 @@ __global__ void __launch_bounds__(256) unpack_vector_kernel(const uint8_t *__res
       }
     }
     u32x4 r; r.x = w[0]; r.y = w[1]; r.z = w[2]; r.w = w[3];
-    stream_store(dst + item, r);
+    stream_store<true>(dst + item, r);
   }
 }
 

@@ -22,7 +22,10 @@
 #include "sjhip_common.h"
 
 #ifndef SJHIP_BWD_PF
-#define SJHIP_BWD_PF 4
+#define SJHIP_BWD_PF 8
+#endif
+#ifndef SJHIP_BWD_NT
+#define SJHIP_BWD_NT 1
 #endif
 
 namespace sjhip {
@@ -85,7 +88,7 @@ template <int SG> __device__ __forceinline__ float surrogate_grad(float x, float
 
 template <typename S, bool VECTOR, bool PLIF, int SG, bool GVFULL>
 __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, int64_t col, float k) {
-  typedef Acc<S, VECTOR> A;
+  typedef Acc<S, VECTOR, SJHIP_BWD_NT != 0> A;
   typedef typename A::elem_t E;
   constexpr int V = A::V;
   constexpr int PF = SJHIP_BWD_PF;
@@ -192,8 +195,8 @@ __device__ __forceinline__ float backward_gv_dispatch(const BwdArgs &a, bool act
 }
 
 template <typename S, bool VECTOR, bool PLIF>
-__global__ void __launch_bounds__(512) backward_kernel(const BwdArgs a) {
-  constexpr int V = Acc<S, VECTOR>::V;
+__global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_kernel(const BwdArgs a) {
+  constexpr int V = Acc<S, VECTOR, true>::V;
   const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
   const bool active = col < a.N;
   const float k = a.k_device ? *a.k_device : a.k;
@@ -209,7 +212,7 @@ __global__ void __launch_bounds__(512) backward_kernel(const BwdArgs a) {
   }
   if (PLIF) {
     // wavefront (64 lanes) shuffle reduction, then one value per wavefront through LDS
-    __shared__ float wave_sum[8];
+    __shared__ float wave_sum[SJHIP_MAX_BLOCK / 64];
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) part += __shfl_down(part, off, 64);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;

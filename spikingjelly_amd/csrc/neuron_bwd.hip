@@ -10,19 +10,20 @@ namespace {
 template <typename S>
 int launch_typed(BwdArgs &a, bool vector, bool plif, float *grad_k_out, hipStream_t stream) {
   const int block = tuning().bwd_block;
-  const int V = vector ? Acc<S, true>::V : 1;
+  const int V = vector ? Acc<S, true, true>::V : 1;
   const int64_t items = (a.N + V - 1) / V;
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "backward: N=%lld needs %lld blocks", (long long)a.N, (long long)blocks);
   const dim3 grid((unsigned)blocks), threads(block);
+  const unsigned lds = occupancy_cap_lds(tuning().bwd_blocks_per_cu);
   {
     ProfileScope prof(KC_BACKWARD, stream);
     if (plif) {
-      if (vector) hipLaunchKernelGGL((backward_kernel<S, true, true>), grid, threads, 0, stream, a);
-      else hipLaunchKernelGGL((backward_kernel<S, false, true>), grid, threads, 0, stream, a);
+      if (vector) hipLaunchKernelGGL((backward_kernel<S, true, true>), grid, threads, lds, stream, a);
+      else hipLaunchKernelGGL((backward_kernel<S, false, true>), grid, threads, lds, stream, a);
     } else {
-      if (vector) hipLaunchKernelGGL((backward_kernel<S, true, false>), grid, threads, 0, stream, a);
-      else hipLaunchKernelGGL((backward_kernel<S, false, false>), grid, threads, 0, stream, a);
+      if (vector) hipLaunchKernelGGL((backward_kernel<S, true, false>), grid, threads, lds, stream, a);
+      else hipLaunchKernelGGL((backward_kernel<S, false, false>), grid, threads, lds, stream, a);
     }
     int rc = check_launch("backward");
     if (rc != SJHIP_OK) return rc;

@@ -3,7 +3,8 @@
 // One work-item owns V consecutive neurons (one 128-bit access per row) and walks the T rows in
 // order with the membrane potential in registers.  Rows of x are requested SJHIP_FWD_PF steps ahead
 // of their use so several 128-bit loads per lane are always in flight; every tensor is touched
-// exactly once, so loads and stores are non-temporal.
+// exactly once (default cache policy: the write-dominated forward measured slower with
+// non-temporal accesses, the read-dominated backward faster).
 //
 // The arithmetic restates the torch backend of the reference op for op and in its order
 // (functional/neuron.py:225-228 voltage_reset, :310-312 if_step, :849-852 lif_charge, :1290-1297
@@ -18,7 +19,10 @@
 #include "sjhip_common.h"
 
 #ifndef SJHIP_FWD_PF
-#define SJHIP_FWD_PF 4
+#define SJHIP_FWD_PF 8
+#endif
+#ifndef SJHIP_FWD_NT
+#define SJHIP_FWD_NT 0
 #endif
 
 namespace sjhip {
@@ -84,7 +88,7 @@ __device__ __forceinline__ void neuron_step(float x, float &v, float &h, float &
 
 template <typename S, bool VECTOR, bool ROUND_EACH, int CH, bool SOFT>
 __device__ __forceinline__ void forward_body(const FwdArgs &a) {
-  typedef Acc<S, VECTOR> A;
+  typedef Acc<S, VECTOR, SJHIP_FWD_NT != 0> A;
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
@@ -142,7 +146,7 @@ __device__ __forceinline__ void forward_reset_dispatch(const FwdArgs &a) {
 }
 
 template <typename S, bool VECTOR, bool ROUND_EACH>
-__global__ void __launch_bounds__(512) forward_kernel(const FwdArgs a) {
+__global__ void __launch_bounds__(SJHIP_MAX_BLOCK) forward_kernel(const FwdArgs a) {
   switch (a.charge) {
     case CH_IF: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_IF>(a); break;
     case CH_DECAY_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_DIV>(a); break;

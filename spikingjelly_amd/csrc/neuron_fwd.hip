@@ -10,15 +10,16 @@ namespace {
 template <typename S, bool ROUND_EACH>
 int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   const int block = tuning().fwd_block;
-  const int V = vector ? Acc<S, true>::V : 1;
+  const int V = vector ? Acc<S, true, true>::V : 1;
   const int64_t items = (a.N + V - 1) / V;
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "forward: N=%lld needs %lld blocks", (long long)a.N, (long long)blocks);
+  const unsigned lds = occupancy_cap_lds(tuning().fwd_blocks_per_cu);
   ProfileScope prof(KC_FORWARD, stream);
   if (vector)
-    hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH>), dim3((unsigned)blocks), dim3(block), 0, stream, a);
+    hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH>), dim3((unsigned)blocks), dim3(block), lds, stream, a);
   else
-    hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH>), dim3((unsigned)blocks), dim3(block), 0, stream, a);
+    hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH>), dim3((unsigned)blocks), dim3(block), lds, stream, a);
   return check_launch("forward");
 }
 

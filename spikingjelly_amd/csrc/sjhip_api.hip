@@ -17,9 +17,12 @@ namespace {
 thread_local char g_error[512] = "";
 
 struct TuningStore {
-  std::atomic<int> fwd_block{256};
-  std::atomic<int> bwd_block{256};
-  std::atomic<int> pack_block{256};
+  std::atomic<int> fwd_block{128};
+  std::atomic<int> bwd_block{128};
+  // Measured on MI355X at T=16, N=33.5M fp32: 2 blocks of 128 per compute unit (one wavefront per
+  // SIMD) with 8 rows prefetched beat full occupancy by 7 % forward and 7 % backward.
+  std::atomic<int> fwd_blocks_per_cu{2};
+  std::atomic<int> bwd_blocks_per_cu{2};
 };
 TuningStore g_tuning;
 
@@ -68,8 +71,19 @@ const Tuning &tuning() {
   thread_local Tuning t;
   t.fwd_block = g_tuning.fwd_block.load(std::memory_order_relaxed);
   t.bwd_block = g_tuning.bwd_block.load(std::memory_order_relaxed);
-  t.pack_block = g_tuning.pack_block.load(std::memory_order_relaxed);
+  t.fwd_blocks_per_cu = g_tuning.fwd_blocks_per_cu.load(std::memory_order_relaxed);
+  t.bwd_blocks_per_cu = g_tuning.bwd_blocks_per_cu.load(std::memory_order_relaxed);
   return t;
+}
+
+unsigned occupancy_cap_lds(int blocks_per_cu) {
+  // gfx950 has 160 KiB of LDS per compute unit and a block may ask for at most 64 KiB of it:
+  // asking for floor(160 KiB / n) (in 512-byte granules) lets exactly n blocks be resident.
+  if (blocks_per_cu <= 0) return 0;
+  const unsigned total = 160u * 1024u;
+  unsigned bytes = (total / (unsigned)blocks_per_cu) & ~511u;
+  if (bytes > 64u * 1024u) bytes = 64u * 1024u;
+  return bytes;
 }
 
 ProfileScope::ProfileScope(int kernel_class, hipStream_t stream)
@@ -167,9 +181,12 @@ int sjhip_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, void *
 
 int sjhip_set_tuning(const char *key, int value) {
   if (!key) return fail(SJHIP_ERR_INVALID, "set_tuning: NULL key");
-  const bool block_ok = value == 64 || value == 128 || value == 256 || value == 512;
+  const bool block_ok = (value == 64 || value == 128 || value == 256 || value == 512) && value <= SJHIP_MAX_BLOCK;
   if (!strcmp(key, "fwd_block")) { if (!block_ok) return fail(SJHIP_ERR_INVALID, "set_tuning: fwd_block=%d", value); g_tuning.fwd_block = value; return SJHIP_OK; }
   if (!strcmp(key, "bwd_block")) { if (!block_ok) return fail(SJHIP_ERR_INVALID, "set_tuning: bwd_block=%d", value); g_tuning.bwd_block = value; return SJHIP_OK; }
+  const bool cap_ok = value >= 0 && value <= 64;
+  if (!strcmp(key, "fwd_blocks_per_cu")) { if (!cap_ok) return fail(SJHIP_ERR_INVALID, "set_tuning: fwd_blocks_per_cu=%d", value); g_tuning.fwd_blocks_per_cu = value; return SJHIP_OK; }
+  if (!strcmp(key, "bwd_blocks_per_cu")) { if (!cap_ok) return fail(SJHIP_ERR_INVALID, "set_tuning: bwd_blocks_per_cu=%d", value); g_tuning.bwd_blocks_per_cu = value; return SJHIP_OK; }
   return fail(SJHIP_ERR_INVALID, "set_tuning: unknown key '%s'", key);
 }
 
@@ -177,6 +194,8 @@ int sjhip_get_tuning(const char *key) {
   if (!key) return fail(SJHIP_ERR_INVALID, "get_tuning: NULL key");
   if (!strcmp(key, "fwd_block")) return g_tuning.fwd_block;
   if (!strcmp(key, "bwd_block")) return g_tuning.bwd_block;
+  if (!strcmp(key, "fwd_blocks_per_cu")) return g_tuning.fwd_blocks_per_cu;
+  if (!strcmp(key, "bwd_blocks_per_cu")) return g_tuning.bwd_blocks_per_cu;
   return fail(SJHIP_ERR_INVALID, "get_tuning: unknown key '%s'", key);
 }
 

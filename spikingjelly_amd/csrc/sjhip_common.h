@@ -49,60 +49,50 @@ template <> struct Cvt<bf16_t> {
   static __host__ __device__ __forceinline__ float round(float f) { return to_float(from_float(f)); }
 };
 
-#ifndef SJHIP_NT_LOAD
-#define SJHIP_NT_LOAD 1
-#endif
-#ifndef SJHIP_NT_STORE
-#define SJHIP_NT_STORE 1
-#endif
-
-template <typename T> __device__ __forceinline__ T stream_load(const T *p) {
-#if SJHIP_NT_LOAD
-  return __builtin_nontemporal_load(p);
-#else
+// Cache policy of one access: NT marks the line as streaming (non-temporal), otherwise default.
+// Measured on MI355X: read-mostly kernels (backward, unpack) gain from NT on both loads and stores,
+// the write-mostly forward loses with it.
+template <bool NT, typename T> __device__ __forceinline__ T stream_load(const T *p) {
+  if (NT) return __builtin_nontemporal_load(p);
   return *p;
-#endif
 }
-template <typename T> __device__ __forceinline__ void stream_store(T *p, T v) {
-#if SJHIP_NT_STORE
-  __builtin_nontemporal_store(v, p);
-#else
-  *p = v;
-#endif
+template <bool NT, typename T> __device__ __forceinline__ void stream_store(T *p, T v) {
+  if (NT) __builtin_nontemporal_store(v, p);
+  else *p = v;
 }
 
 // Accessor: how one work-item reads/writes its V consecutive neurons of one row.
 // raw_t is what stays in registers between the (early) load and the (late) use.
-template <typename S, bool VECTOR> struct Acc;
+template <typename S, bool VECTOR, bool NT = true> struct Acc;
 
-template <> struct Acc<float, true> {
+template <bool NT> struct Acc<float, true, NT> {
   static constexpr int V = 4;
   typedef float elem_t;
   typedef f32x4 raw_t;
-  static __device__ __forceinline__ raw_t load(const elem_t *p) { return stream_load((const raw_t *)p); }
+  static __device__ __forceinline__ raw_t load(const elem_t *p) { return stream_load<NT>((const raw_t *)p); }
   static __device__ __forceinline__ raw_t zero() { return (raw_t)(0.f); }
   static __device__ __forceinline__ void unpack(raw_t r, float (&f)[V]) {
     f[0] = r.x; f[1] = r.y; f[2] = r.z; f[3] = r.w;
   }
   static __device__ __forceinline__ void store(elem_t *p, const float (&f)[V]) {
     raw_t r; r.x = f[0]; r.y = f[1]; r.z = f[2]; r.w = f[3];
-    stream_store((raw_t *)p, r);
+    stream_store<NT>((raw_t *)p, r);
   }
 };
-template <> struct Acc<float, false> {
+template <bool NT> struct Acc<float, false, NT> {
   static constexpr int V = 1;
   typedef float elem_t;
   typedef float raw_t;
-  static __device__ __forceinline__ raw_t load(const elem_t *p) { return stream_load(p); }
+  static __device__ __forceinline__ raw_t load(const elem_t *p) { return stream_load<NT>(p); }
   static __device__ __forceinline__ raw_t zero() { return 0.f; }
   static __device__ __forceinline__ void unpack(raw_t r, float (&f)[V]) { f[0] = r; }
-  static __device__ __forceinline__ void store(elem_t *p, const float (&f)[V]) { stream_store(p, f[0]); }
+  static __device__ __forceinline__ void store(elem_t *p, const float (&f)[V]) { stream_store<NT>(p, f[0]); }
 };
-template <typename H> struct Acc16v {
+template <typename H, bool NT> struct Acc16v {
   static constexpr int V = 8;
   typedef uint16_t elem_t;
   typedef u32x4 raw_t;
-  static __device__ __forceinline__ raw_t load(const elem_t *p) { return stream_load((const raw_t *)p); }
+  static __device__ __forceinline__ raw_t load(const elem_t *p) { return stream_load<NT>((const raw_t *)p); }
   static __device__ __forceinline__ raw_t zero() { return (raw_t)(0u); }
   static __device__ __forceinline__ void unpack(raw_t r, float (&f)[V]) {
     uint32_t w[4] = {r.x, r.y, r.z, r.w};
@@ -118,24 +108,24 @@ template <typename H> struct Acc16v {
     for (int i = 0; i < 4; ++i)
       w[i] = (uint32_t)Cvt<H>::from_float(f[2 * i]) | ((uint32_t)Cvt<H>::from_float(f[2 * i + 1]) << 16);
     raw_t r; r.x = w[0]; r.y = w[1]; r.z = w[2]; r.w = w[3];
-    stream_store((raw_t *)p, r);
+    stream_store<NT>((raw_t *)p, r);
   }
 };
-template <typename H> struct Acc16s {
+template <typename H, bool NT> struct Acc16s {
   static constexpr int V = 1;
   typedef uint16_t elem_t;
   typedef uint16_t raw_t;
-  static __device__ __forceinline__ raw_t load(const elem_t *p) { return stream_load(p); }
+  static __device__ __forceinline__ raw_t load(const elem_t *p) { return stream_load<NT>(p); }
   static __device__ __forceinline__ raw_t zero() { return 0; }
   static __device__ __forceinline__ void unpack(raw_t r, float (&f)[V]) { f[0] = Cvt<H>::to_float(r); }
   static __device__ __forceinline__ void store(elem_t *p, const float (&f)[V]) {
-    stream_store(p, Cvt<H>::from_float(f[0]));
+    stream_store<NT>(p, Cvt<H>::from_float(f[0]));
   }
 };
-template <> struct Acc<f16_t, true> : Acc16v<f16_t> {};
-template <> struct Acc<f16_t, false> : Acc16s<f16_t> {};
-template <> struct Acc<bf16_t, true> : Acc16v<bf16_t> {};
-template <> struct Acc<bf16_t, false> : Acc16s<bf16_t> {};
+template <bool NT> struct Acc<f16_t, true, NT> : Acc16v<f16_t, NT> {};
+template <bool NT> struct Acc<f16_t, false, NT> : Acc16s<f16_t, NT> {};
+template <bool NT> struct Acc<bf16_t, true, NT> : Acc16v<bf16_t, NT> {};
+template <bool NT> struct Acc<bf16_t, false, NT> : Acc16s<bf16_t, NT> {};
 
 // ----------------------------------------------------------------------------------------------
 // Host-side services (defined in sjhip_api.hip).
@@ -143,11 +133,21 @@ template <> struct Acc<bf16_t, false> : Acc16s<bf16_t> {};
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int check_launch(const char *what);
 
+// Largest block the neuron kernels may be launched with.  Kept small on purpose: the kernels run
+// best with about one fat wavefront per SIMD (few resident waves, many loads in flight each), and a
+// small bound lets the compiler use several hundred VGPRs for the prefetch buffers.
+#ifndef SJHIP_MAX_BLOCK
+#define SJHIP_MAX_BLOCK 128
+#endif
+
 struct Tuning {
   int fwd_block;
   int bwd_block;
-  int pack_block;
+  int fwd_blocks_per_cu;  // 0 = no cap; otherwise dynamic LDS is requested so that at most this many
+  int bwd_blocks_per_cu;  // blocks are resident per compute unit
 };
+// dynamic LDS bytes that cap residency at `blocks_per_cu` blocks (0 for no cap)
+unsigned occupancy_cap_lds(int blocks_per_cu);
 const Tuning &tuning();
 
 enum KernelClass { KC_FORWARD = 0, KC_BACKWARD = 1, KC_PLIF_REDUCE = 2, KC_BIT_PACK = 3, KC_BIT_UNPACK = 4, KC_COUNT = 5 };
