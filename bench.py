@@ -119,6 +119,19 @@ def main() -> int:
     n_fwd, ms_fwd = L.profile_read(L.KC_FORWARD)
     n_bwd, ms_bwd = L.profile_read(L.KC_BACKWARD)
 
+    # measured device-copy ceiling on the same box: torch's copy kernel over one 2.1 GB tensor
+    dst = torch.empty_like(grad_v)
+    for _ in range(2):
+        dst.copy_(grad_v)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        dst.copy_(grad_v)
+    e1.record()
+    torch.cuda.synchronize()
+    copy_gbs = 2 * grad_v.numel() * 4 / (e0.elapsed_time(e1) / 5 * 1e-3) / 1e9
+    del dst
+
     ms_per_step = elapsed / args.steps * 1e3
     value = T_STEPS * N / (elapsed / args.steps)
 
@@ -159,7 +172,8 @@ def main() -> int:
                      "forward_GBs": fwd_bytes / (fwd_ms * 1e-3) / 1e9 if fwd_ms else None,
                      "backward_GBs": bwd_bytes / (bwd_ms * 1e-3) / 1e9 if bwd_ms else None,
                      "fwd_plus_bwd_frac": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS
-                     if (fwd_ms + bwd_ms) else None},
+                     if (fwd_ms + bwd_ms) else None,
+                     "device_copy_GBs": copy_gbs},
     }
     del x, grad_spike, grad_v, spikes
     torch.cuda.empty_cache()
