@@ -51,7 +51,11 @@ def test_argument_validation_without_a_device():
     assert lib.sjhip_bit_pack(L.DTYPE_F32, 0, None, None, None) == 0
     assert lib.sjhip_plif_workspace_floats(L.DTYPE_F32, 1 << 20) >= (1 << 20) // 1024
     assert lib.sjhip_set_tuning(b"fwd_block", 100) == -1
-    assert lib.sjhip_set_tuning(b"fwd_block", 256) == 0 and lib.sjhip_get_tuning(b"fwd_block") == 256
+    assert lib.sjhip_set_tuning(b"fwd_block", 512) == -1  # above the kernels' launch bound
+    assert lib.sjhip_set_tuning(b"fwd_block", 64) == 0 and lib.sjhip_get_tuning(b"fwd_block") == 64
+    assert lib.sjhip_set_tuning(b"fwd_block", 128) == 0
+    assert lib.sjhip_set_tuning(b"bwd_blocks_per_cu", 65) == -1
+    assert lib.sjhip_get_tuning(b"bwd_blocks_per_cu") == 2
     assert lib.sjhip_set_tuning(b"nope", 1) == -1
 
 
