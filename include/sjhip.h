@@ -147,6 +147,28 @@ int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p,
                           void *stream);
 
 /*
+ * Backward that needs no h_seq: it replays the forward from x_seq and v_init (bit-identical h, kept
+ * in LDS) and then runs the same BPTT.  A forward whose backward will use this entry point can be
+ * called with h_seq = NULL, which saves its largest write.  Same argument meaning as
+ * sjhip_neuron_backward with (x_seq, v_init) in place of h_seq; `p` carries the forward flags too
+ * (SJHIP_FLAG_FP32_STATE, SJHIP_FLAG_RECIPROCAL_TAU).  Requires sjhip_recompute_supported() and
+ * 16-byte aligned tensors; returns SJHIP_ERR_UNSUPPORTED / SJHIP_ERR_INVALID otherwise.
+ * Stands in for the same reference backward ops as sjhip_neuron_backward; the reference has no
+ * recomputing variant (its kernels always read the saved h_seq, multi_step/base.py:137-409).
+ */
+int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_params *p,
+                                    int64_t T, int64_t N,
+                                    const void *x_seq, const void *v_init, const float *rtau_device,
+                                    const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                                    void *grad_x_seq, void *grad_v_init,
+                                    float *grad_rtau, float *workspace,
+                                    void *stream);
+
+/* 1 if sjhip_neuron_backward_recompute can serve [T,N] of `dtype` (N a multiple of the 128-bit vector
+ * width and T steps of h fitting in LDS: T <= 159 for fp32, 79 for 16-bit storage), else 0. */
+int sjhip_recompute_supported(int dtype, int64_t T, int64_t N);
+
+/*
  * Spike bit-packing over a flattened tensor, LSB first: byte j bit i = (src[8j+i] != 0).
  *   src  n elements of `dtype` (F32/F16/BF16/U8)     dst  (n+7)/8 bytes; pad bits of the last byte are 0
  */

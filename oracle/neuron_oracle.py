@@ -207,13 +207,15 @@ def multi_step(kind: str, x_seq: torch.Tensor, v_init: torch.Tensor, tau_or_w=No
 
 def multi_step_mixed_precision(kind: str, x_seq: torch.Tensor, v_init: torch.Tensor, storage_dtype: torch.dtype,
                                k: float = 0.5, decay_input: bool = True, v_threshold: float = 1.0,
-                               v_reset: Optional[float] = 0.0, torch_op_order: bool = True):
+                               v_reset: Optional[float] = 0.0, torch_op_order: bool = True,
+                               return_raw_h: bool = False):
     """fp32 state and arithmetic, storage-dtype inputs/outputs
     (test/activation_based/test_triton_neuron.py:212-247): inputs are quantised to the storage dtype,
     v is carried in fp32 un-rounded, stored v/h are rounded.  ``torch_op_order`` keeps the torch
     backend's expression order (what the HIP kernels use); False uses the test's
     ``v + k*(reset - v + x)`` order -- identical when v_reset is 0 or None.
-    Returns fp32 tensors (spike_seq, v_seq, h_seq) holding storage-representable values.
+    Returns fp32 tensors (spike_seq, v_seq, h_seq) holding storage-representable values; with
+    ``return_raw_h`` a fourth tensor holds h before it was rounded for storage.
     """
     q = lambda t: t.to(storage_dtype).to(torch.float32)
     x_seq = q(x_seq)
@@ -223,6 +225,7 @@ def multi_step_mixed_precision(kind: str, x_seq: torch.Tensor, v_init: torch.Ten
     s_seq = torch.empty_like(x_seq)
     v_seq = torch.empty_like(x_seq)
     h_seq = torch.empty_like(x_seq)
+    raw_h_seq = torch.empty_like(x_seq)
     for t in range(x_seq.shape[0]):
         x = x_seq[t]
         if kind == "if":
@@ -241,6 +244,9 @@ def multi_step_mixed_precision(kind: str, x_seq: torch.Tensor, v_init: torch.Ten
         s_seq[t] = s
         v_seq[t] = q(v)
         h_seq[t] = q(h)
+        raw_h_seq[t] = h
+    if return_raw_h:
+        return s_seq, v_seq, h_seq, raw_h_seq
     return s_seq, v_seq, h_seq
 
 

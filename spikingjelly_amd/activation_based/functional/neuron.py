@@ -101,6 +101,13 @@ def _hip_mode_flags(x_seq: torch.Tensor) -> int:
     return flags
 
 
+def _hip_recompute(x2: torch.Tensor) -> bool:
+    """Replay the forward inside the backward kernel instead of saving h_seq, when the shape allows."""
+    from ..hip_kernel import library as L
+
+    return bool(configure.hip_backward_recompute) and L.recompute_supported(x2.dtype, x2.shape[0], x2.shape[1])
+
+
 def _needs_grad(*tensors: torch.Tensor) -> bool:
     return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
 
@@ -127,7 +134,7 @@ def if_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, v_threshold: float, 
     if _needs_grad(x_seq, v):
         sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function)
         s, v_seq, v_last, _ = K.hip_multistep_if_forward(x2, v1, v_threshold, vr, soft, detach_reset, sg_id,
-                                                         sg_alpha, store_v_seq, flags)
+                                                         sg_alpha, store_v_seq, flags, _hip_recompute(x2))
     else:
         s, v_seq, v_last = K.hip_multistep_if_inference(x2, v1, v_threshold, vr, soft, store_v_seq, flags)
     return _finish(x_seq, s, v_seq, v_last, store_v_seq)
@@ -149,7 +156,7 @@ def lif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, decay_i
         sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function)
         s, v_seq, v_last, _ = K.hip_multistep_lif_forward(x2, v1, v_threshold, vr, soft, detach_reset,
                                                           float(tau), decay_input, sg_id, sg_alpha,
-                                                          store_v_seq, flags)
+                                                          store_v_seq, flags, _hip_recompute(x2))
     else:
         s, v_seq, v_last = K.hip_multistep_lif_inference(x2, v1, v_threshold, vr, soft, float(tau),
                                                          decay_input, store_v_seq, flags)
@@ -173,7 +180,8 @@ def plif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Tensor, d
     if _needs_grad(x_seq, v, w):
         sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function)
         s, v_seq, v_last, _ = K.hip_multistep_plif_forward(x2, v1, k, v_threshold, vr, soft, detach_reset,
-                                                           decay_input, sg_id, sg_alpha, store_v_seq, flags)
+                                                           decay_input, sg_id, sg_alpha, store_v_seq, flags,
+                                                           _hip_recompute(x2))
     else:
         s, v_seq, v_last = K.hip_multistep_plif_inference(x2, v1, k, v_threshold, vr, soft, decay_input,
                                                           store_v_seq, flags)

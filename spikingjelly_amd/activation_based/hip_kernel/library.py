@@ -34,6 +34,8 @@ EXPORTED_SYMBOLS = (
     "sjhip_neuron_forward",
     "sjhip_plif_workspace_floats",
     "sjhip_neuron_backward",
+    "sjhip_neuron_backward_recompute",
+    "sjhip_recompute_supported",
     "sjhip_bit_pack",
     "sjhip_bit_unpack",
     "sjhip_set_tuning",
@@ -96,6 +98,14 @@ def load() -> ctypes.CDLL:
             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
         ]
+        lib.sjhip_neuron_backward_recompute.restype = c_int
+        lib.sjhip_neuron_backward_recompute.argtypes = [
+            c_int, c_int, POINTER(NeuronParams), c_int64, c_int64,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        ]
+        lib.sjhip_recompute_supported.restype = c_int
+        lib.sjhip_recompute_supported.argtypes = [c_int, c_int64, c_int64]
         lib.sjhip_bit_pack.restype = c_int
         lib.sjhip_bit_pack.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p]
         lib.sjhip_bit_unpack.restype = c_int
@@ -152,6 +162,17 @@ def current_stream_ptr(device: torch.device) -> int:
 
 def ptr(t) -> int | None:
     return None if t is None else t.data_ptr()
+
+
+def recompute_supported(dtype: torch.dtype, T: int, N: int) -> bool:
+    """Whether the backward can replay the forward from ``x_seq`` instead of reading a saved ``h_seq``."""
+    return bool(load().sjhip_recompute_supported(dtype_id(dtype), T, N))
+
+
+def aligned16(t: torch.Tensor) -> torch.Tensor:
+    """``t`` made contiguous and 16-byte aligned (a fresh allocation always is)."""
+    t = t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
 def set_tuning(key: str, value: int) -> None:

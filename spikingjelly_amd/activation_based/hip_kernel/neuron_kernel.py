@@ -10,7 +10,9 @@ inference op that writes no ``h_seq``):
     sj::hip_multistep_{if,lif,plif}_backward   -> (grad_x_seq, grad_v_init[, grad_k])
 
 All tensors are viewed as ``[T, N]``; ``v_seq`` is an empty tensor when ``store_v_seq`` is false
-(the kernel then writes only ``v_last``).  ``Optional[float]`` is not expressible in an operator
+(the kernel then writes only ``v_last``).  With ``recompute`` the forward writes no ``h_seq`` (an empty
+tensor is returned) and autograd keeps ``x_seq`` and ``v_init`` instead; the backward then replays the
+forward inside the kernel (``sjhip_neuron_backward_recompute``), which removes the forward's largest write.  ``Optional[float]`` is not expressible in an operator
 schema, so soft reset is a bool next to a dummy ``v_reset`` as in the reference (lif.py:342-343).
 The ops run on ROCm tensors only and raise otherwise; there is no fallback path.
 """
@@ -93,21 +95,38 @@ def _run_forward(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: Opti
     return spike_seq, v_seq, v_last, h_seq
 
 
+def _forward_outputs(out, x_seq: torch.Tensor):
+    """custom ops return tensors only: an unsaved h_seq becomes an empty tensor."""
+    s, v_seq, v_last, h = out
+    return s, v_seq, v_last, (h if h is not None else x_seq.new_empty((0,)))
+
+
 def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
-                  grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor, v_init: Optional[torch.Tensor],
-                  k: Optional[torch.Tensor], tau: float, v_th: float, v_reset: float, flags: int,
-                  sg_id: int, sg_alpha: float) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+                  grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor, x_seq: Optional[torch.Tensor],
+                  v_init: Optional[torch.Tensor], k: Optional[torch.Tensor], tau: float, v_th: float,
+                  v_reset: float, flags: int, sg_id: int, sg_alpha: float
+                  ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    recompute = x_seq is not None
+    if not recompute and h_seq is None:
+        raise ValueError("backward needs h_seq, or x_seq and v_init to recompute it")
+    if recompute:
+        # replay path: every buffer must be 16-byte aligned for the 128-bit kernel
+        h_seq = L.aligned16(x_seq)
+        v_init = L.aligned16(v_init)
+        fix = L.aligned16
+    else:
+        h_seq = h_seq.contiguous()
+        fix = lambda t: t.contiguous()
     L.require_device_tensor("h_seq", h_seq)
     dtype = L.dtype_id(h_seq.dtype)
-    h_seq = h_seq.contiguous()
     T, N = h_seq.shape
     if grad_spike_seq is None:
         grad_spike_seq = torch.zeros_like(h_seq)
-    grad_spike_seq = grad_spike_seq.to(h_seq.dtype).contiguous()
+    grad_spike_seq = fix(grad_spike_seq.to(h_seq.dtype))
     if grad_v_seq is not None:
-        grad_v_seq = grad_v_seq.to(h_seq.dtype).contiguous()
+        grad_v_seq = fix(grad_v_seq.to(h_seq.dtype))
     if grad_v_last is not None:
-        grad_v_last = grad_v_last.to(h_seq.dtype).contiguous()
+        grad_v_last = fix(grad_v_last.to(h_seq.dtype))
     grad_x_seq = torch.empty_like(h_seq)
     grad_v_init = h_seq.new_empty((N,))
     grad_k = workspace = None
@@ -122,27 +141,45 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
                                     device=h_seq.device)
     params = _params(tau, v_th, v_reset, sg_alpha, sg_id, flags)
     with torch.cuda.device(h_seq.device):
-        rc = L.load().sjhip_neuron_backward(
-            neuron, dtype, ctypes.byref(params), T, N,
-            grad_spike_seq.data_ptr(), L.ptr(grad_v_seq), L.ptr(grad_v_last), h_seq.data_ptr(),
-            L.ptr(v_init) if neuron == L.NEURON_PLIF else None, k_ptr,
-            grad_x_seq.data_ptr(), grad_v_init.data_ptr(), L.ptr(grad_k), L.ptr(workspace),
-            L.current_stream_ptr(h_seq.device),
-        )
-    L.check(rc, "neuron_backward")
+        if recompute:
+            rc = L.load().sjhip_neuron_backward_recompute(
+                neuron, dtype, ctypes.byref(params), T, N,
+                h_seq.data_ptr(), v_init.data_ptr(), k_ptr,
+                grad_spike_seq.data_ptr(), L.ptr(grad_v_seq), L.ptr(grad_v_last),
+                grad_x_seq.data_ptr(), grad_v_init.data_ptr(), L.ptr(grad_k), L.ptr(workspace),
+                L.current_stream_ptr(h_seq.device),
+            )
+        else:
+            rc = L.load().sjhip_neuron_backward(
+                neuron, dtype, ctypes.byref(params), T, N,
+                grad_spike_seq.data_ptr(), L.ptr(grad_v_seq), L.ptr(grad_v_last), h_seq.data_ptr(),
+                L.ptr(v_init) if neuron == L.NEURON_PLIF else None, k_ptr,
+                grad_x_seq.data_ptr(), grad_v_init.data_ptr(), L.ptr(grad_k), L.ptr(workspace),
+                L.current_stream_ptr(h_seq.device),
+            )
+    L.check(rc, "neuron_backward_recompute" if recompute else "neuron_backward")
     del k_keep
     return grad_x_seq, grad_v_init, grad_k
 
 
-def _fake_forward(x_seq, v_init, store_v_seq, with_h):
+def _fake_forward(x_seq, v_init, store_v_seq, with_h, recompute=False):
     outs = [
         x_seq.new_empty(x_seq.shape),
         x_seq.new_empty(x_seq.shape) if store_v_seq else x_seq.new_empty((0,)),
         v_init.new_empty(v_init.shape),
     ]
     if with_h:
-        outs.append(x_seq.new_empty(x_seq.shape))
+        outs.append(x_seq.new_empty((0,)) if recompute else x_seq.new_empty(x_seq.shape))
     return tuple(outs)
+
+
+def _saved_for_backward(ctx, recompute: bool, x_seq, v_init, h_seq, *extra):
+    """h path keeps h_seq; replay path keeps the op's own inputs x_seq and v_init."""
+    ctx.recompute = recompute
+    if recompute:
+        ctx.save_for_backward(x_seq, v_init, *extra)
+    else:
+        ctx.save_for_backward(h_seq, *extra)
 
 
 def _none_if_empty_grad(g: Optional[torch.Tensor], store_v_seq: bool) -> Optional[torch.Tensor]:
@@ -155,15 +192,16 @@ def _none_if_empty_grad(g: Optional[torch.Tensor], store_v_seq: bool) -> Optiona
 @torch.library.custom_op("sj::hip_multistep_if_forward", mutates_args=())
 def hip_multistep_if_forward(x_seq: torch.Tensor, v_init: torch.Tensor, v_th: float, v_reset: float,
                              soft_reset: bool, detach_reset: bool, sg_id: int, sg_alpha: float,
-                             store_v_seq: bool, mode_flags: int
+                             store_v_seq: bool, mode_flags: int, recompute: bool
                              ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     flags = _flags(soft_reset, detach_reset, False, mode_flags)
-    return _run_forward(L.NEURON_IF, x_seq, v_init, None, 0.0, v_th, v_reset, flags, store_v_seq, True)
+    return _forward_outputs(_run_forward(L.NEURON_IF, x_seq, v_init, None, 0.0, v_th, v_reset, flags, store_v_seq,
+                                         not recompute), x_seq)
 
 
 @hip_multistep_if_forward.register_fake
-def _(x_seq, v_init, v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, store_v_seq, mode_flags):
-    return _fake_forward(x_seq, v_init, store_v_seq, True)
+def _(x_seq, v_init, v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, store_v_seq, mode_flags, recompute):
+    return _fake_forward(x_seq, v_init, store_v_seq, True, recompute)
 
 
 @torch.library.custom_op("sj::hip_multistep_if_inference", mutates_args=())
@@ -181,37 +219,48 @@ def _(x_seq, v_init, v_th, v_reset, soft_reset, store_v_seq, mode_flags):
 
 @torch.library.custom_op("sj::hip_multistep_if_backward", mutates_args=())
 def hip_multistep_if_backward(grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
-                              grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor, v_th: float,
+                              grad_v_last: Optional[torch.Tensor], h_seq: Optional[torch.Tensor],
+                              x_seq: Optional[torch.Tensor], v_init: Optional[torch.Tensor], v_th: float,
                               v_reset: float, soft_reset: bool, detach_reset: bool, sg_id: int,
                               sg_alpha: float, mode_flags: int) -> tuple[torch.Tensor, torch.Tensor]:
     flags = _flags(soft_reset, detach_reset, False, mode_flags)
-    gx, gvi, _ = _run_backward(L.NEURON_IF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, None, None,
+    gx, gvi, _ = _run_backward(L.NEURON_IF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, None,
                                0.0, v_th, v_reset, flags, sg_id, sg_alpha)
     return gx, gvi
 
 
 @hip_multistep_if_backward.register_fake
-def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_th, v_reset, soft_reset, detach_reset, sg_id,
-      sg_alpha, mode_flags):
-    return torch.empty_like(h_seq), h_seq.new_empty(h_seq.shape[1:])
+def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, v_th, v_reset, soft_reset, detach_reset,
+      sg_id, sg_alpha, mode_flags):
+    ref = h_seq if h_seq is not None else x_seq
+    return torch.empty_like(ref), ref.new_empty(ref.shape[1:])
 
 
 def _if_setup_context(ctx, inputs, output):
-    (_, _, v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, store_v_seq, mode_flags) = inputs
-    ctx.save_for_backward(output[3])
+    (x_seq, v_init, v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, store_v_seq, mode_flags,
+     recompute) = inputs
+    _saved_for_backward(ctx, recompute, x_seq, v_init, output[3])
     ctx.scalars = (v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, mode_flags)
     ctx.store_v_seq = store_v_seq
     ctx.set_materialize_grads(False)
 
 
+def _split_saved(ctx):
+    """(h_seq, x_seq, v_init, extra...) from what _saved_for_backward stored."""
+    saved = ctx.saved_tensors
+    if ctx.recompute:
+        return (None, saved[0], saved[1]) + tuple(saved[2:])
+    return (saved[0], None, None) + tuple(saved[1:])
+
+
 def _if_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_seq):
     del grad_h_seq
-    (h_seq,) = ctx.saved_tensors
+    h_seq, x_seq, v_init = _split_saved(ctx)
     v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, mode_flags = ctx.scalars
     gx, gvi = hip_multistep_if_backward(
-        grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq,
+        grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, x_seq, v_init,
         v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, mode_flags)
-    return gx, gvi, None, None, None, None, None, None, None, None
+    return gx, gvi, None, None, None, None, None, None, None, None, None
 
 
 torch.library.register_autograd("sj::hip_multistep_if_forward", _if_autograd_backward,
@@ -224,16 +273,18 @@ torch.library.register_autograd("sj::hip_multistep_if_forward", _if_autograd_bac
 @torch.library.custom_op("sj::hip_multistep_lif_forward", mutates_args=())
 def hip_multistep_lif_forward(x_seq: torch.Tensor, v_init: torch.Tensor, v_th: float, v_reset: float,
                               soft_reset: bool, detach_reset: bool, tau: float, decay_input: bool,
-                              sg_id: int, sg_alpha: float, store_v_seq: bool, mode_flags: int
+                              sg_id: int, sg_alpha: float, store_v_seq: bool, mode_flags: int,
+                              recompute: bool
                               ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     flags = _flags(soft_reset, detach_reset, decay_input, mode_flags)
-    return _run_forward(L.NEURON_LIF, x_seq, v_init, None, tau, v_th, v_reset, flags, store_v_seq, True)
+    return _forward_outputs(_run_forward(L.NEURON_LIF, x_seq, v_init, None, tau, v_th, v_reset, flags, store_v_seq,
+                                         not recompute), x_seq)
 
 
 @hip_multistep_lif_forward.register_fake
 def _(x_seq, v_init, v_th, v_reset, soft_reset, detach_reset, tau, decay_input, sg_id, sg_alpha,
-      store_v_seq, mode_flags):
-    return _fake_forward(x_seq, v_init, store_v_seq, True)
+      store_v_seq, mode_flags, recompute):
+    return _fake_forward(x_seq, v_init, store_v_seq, True, recompute)
 
 
 @torch.library.custom_op("sj::hip_multistep_lif_inference", mutates_args=())
@@ -251,26 +302,28 @@ def _(x_seq, v_init, v_th, v_reset, soft_reset, tau, decay_input, store_v_seq, m
 
 @torch.library.custom_op("sj::hip_multistep_lif_backward", mutates_args=())
 def hip_multistep_lif_backward(grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
-                               grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor, v_th: float,
+                               grad_v_last: Optional[torch.Tensor], h_seq: Optional[torch.Tensor],
+                               x_seq: Optional[torch.Tensor], v_init: Optional[torch.Tensor], v_th: float,
                                v_reset: float, soft_reset: bool, detach_reset: bool, tau: float,
                                decay_input: bool, sg_id: int, sg_alpha: float, mode_flags: int
                                ) -> tuple[torch.Tensor, torch.Tensor]:
     flags = _flags(soft_reset, detach_reset, decay_input, mode_flags)
-    gx, gvi, _ = _run_backward(L.NEURON_LIF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, None, None,
+    gx, gvi, _ = _run_backward(L.NEURON_LIF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, None,
                                tau, v_th, v_reset, flags, sg_id, sg_alpha)
     return gx, gvi
 
 
 @hip_multistep_lif_backward.register_fake
-def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_th, v_reset, soft_reset, detach_reset, tau,
-      decay_input, sg_id, sg_alpha, mode_flags):
-    return torch.empty_like(h_seq), h_seq.new_empty(h_seq.shape[1:])
+def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, v_th, v_reset, soft_reset, detach_reset,
+      tau, decay_input, sg_id, sg_alpha, mode_flags):
+    ref = h_seq if h_seq is not None else x_seq
+    return torch.empty_like(ref), ref.new_empty(ref.shape[1:])
 
 
 def _lif_setup_context(ctx, inputs, output):
-    (_, _, v_th, v_reset, soft_reset, detach_reset, tau, decay_input, sg_id, sg_alpha, store_v_seq,
-     mode_flags) = inputs
-    ctx.save_for_backward(output[3])
+    (x_seq, v_init, v_th, v_reset, soft_reset, detach_reset, tau, decay_input, sg_id, sg_alpha, store_v_seq,
+     mode_flags, recompute) = inputs
+    _saved_for_backward(ctx, recompute, x_seq, v_init, output[3])
     ctx.scalars = (v_th, v_reset, soft_reset, detach_reset, tau, decay_input, sg_id, sg_alpha, mode_flags)
     ctx.store_v_seq = store_v_seq
     ctx.set_materialize_grads(False)
@@ -278,10 +331,11 @@ def _lif_setup_context(ctx, inputs, output):
 
 def _lif_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_seq):
     del grad_h_seq
-    (h_seq,) = ctx.saved_tensors
+    h_seq, x_seq, v_init = _split_saved(ctx)
     gx, gvi = hip_multistep_lif_backward(
-        grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, *ctx.scalars)
-    return gx, gvi, None, None, None, None, None, None, None, None, None, None
+        grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, x_seq, v_init,
+        *ctx.scalars)
+    return gx, gvi, None, None, None, None, None, None, None, None, None, None, None
 
 
 torch.library.register_autograd("sj::hip_multistep_lif_forward", _lif_autograd_backward,
@@ -295,16 +349,18 @@ torch.library.register_autograd("sj::hip_multistep_lif_forward", _lif_autograd_b
 @torch.library.custom_op("sj::hip_multistep_plif_forward", mutates_args=())
 def hip_multistep_plif_forward(x_seq: torch.Tensor, v_init: torch.Tensor, k: torch.Tensor, v_th: float,
                                v_reset: float, soft_reset: bool, detach_reset: bool, decay_input: bool,
-                               sg_id: int, sg_alpha: float, store_v_seq: bool, mode_flags: int
+                               sg_id: int, sg_alpha: float, store_v_seq: bool, mode_flags: int,
+                               recompute: bool
                                ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     flags = _flags(soft_reset, detach_reset, decay_input, mode_flags)
-    return _run_forward(L.NEURON_PLIF, x_seq, v_init, k, 0.0, v_th, v_reset, flags, store_v_seq, True)
+    return _forward_outputs(_run_forward(L.NEURON_PLIF, x_seq, v_init, k, 0.0, v_th, v_reset, flags, store_v_seq,
+                                         not recompute), x_seq)
 
 
 @hip_multistep_plif_forward.register_fake
 def _(x_seq, v_init, k, v_th, v_reset, soft_reset, detach_reset, decay_input, sg_id, sg_alpha,
-      store_v_seq, mode_flags):
-    return _fake_forward(x_seq, v_init, store_v_seq, True)
+      store_v_seq, mode_flags, recompute):
+    return _fake_forward(x_seq, v_init, store_v_seq, True, recompute)
 
 
 @torch.library.custom_op("sj::hip_multistep_plif_inference", mutates_args=())
@@ -322,28 +378,33 @@ def _(x_seq, v_init, k, v_th, v_reset, soft_reset, decay_input, store_v_seq, mod
 
 @torch.library.custom_op("sj::hip_multistep_plif_backward", mutates_args=())
 def hip_multistep_plif_backward(grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
-                                grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor,
-                                v_init: torch.Tensor, k: torch.Tensor, v_th: float, v_reset: float,
+                                grad_v_last: Optional[torch.Tensor], h_seq: Optional[torch.Tensor],
+                                x_seq: Optional[torch.Tensor], v_init: torch.Tensor, k: torch.Tensor,
+                                v_th: float, v_reset: float,
                                 soft_reset: bool, detach_reset: bool, decay_input: bool, sg_id: int,
                                 sg_alpha: float, mode_flags: int
                                 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     flags = _flags(soft_reset, detach_reset, decay_input, mode_flags)
-    gx, gvi, gk = _run_backward(L.NEURON_PLIF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, k,
+    gx, gvi, gk = _run_backward(L.NEURON_PLIF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, k,
                                 0.0, v_th, v_reset, flags, sg_id, sg_alpha)
     return gx, gvi, gk
 
 
 @hip_multistep_plif_backward.register_fake
-def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, k, v_th, v_reset, soft_reset, detach_reset,
-      decay_input, sg_id, sg_alpha, mode_flags):
-    return (torch.empty_like(h_seq), h_seq.new_empty(h_seq.shape[1:]),
-            h_seq.new_empty((), dtype=torch.float32))
+def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, k, v_th, v_reset, soft_reset,
+      detach_reset, decay_input, sg_id, sg_alpha, mode_flags):
+    ref = h_seq if h_seq is not None else x_seq
+    return (torch.empty_like(ref), ref.new_empty(ref.shape[1:]), ref.new_empty((), dtype=torch.float32))
 
 
 def _plif_setup_context(ctx, inputs, output):
-    (_, v_init, k, v_th, v_reset, soft_reset, detach_reset, decay_input, sg_id, sg_alpha, store_v_seq,
-     mode_flags) = inputs
-    ctx.save_for_backward(output[3], v_init, k)
+    (x_seq, v_init, k, v_th, v_reset, soft_reset, detach_reset, decay_input, sg_id, sg_alpha, store_v_seq,
+     mode_flags, recompute) = inputs
+    ctx.recompute = recompute
+    if recompute:
+        ctx.save_for_backward(x_seq, v_init, k)
+    else:
+        ctx.save_for_backward(output[3], v_init, k)
     ctx.scalars = (v_th, v_reset, soft_reset, detach_reset, decay_input, sg_id, sg_alpha, mode_flags)
     ctx.store_v_seq = store_v_seq
     ctx.k_shape = k.shape
@@ -353,12 +414,13 @@ def _plif_setup_context(ctx, inputs, output):
 
 def _plif_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_seq):
     del grad_h_seq
-    h_seq, v_init, k = ctx.saved_tensors
+    first, v_init, k = ctx.saved_tensors
+    h_seq, x_seq = (None, first) if ctx.recompute else (first, None)
     gx, gvi, gk = hip_multistep_plif_backward(
-        grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, v_init, k,
+        grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, x_seq, v_init, k,
         *ctx.scalars)
     gk = gk.reshape(ctx.k_shape).to(ctx.k_dtype)
-    return gx, gvi, gk, None, None, None, None, None, None, None, None, None
+    return gx, gvi, gk, None, None, None, None, None, None, None, None, None, None
 
 
 torch.library.register_autograd("sj::hip_multistep_plif_forward", _plif_autograd_backward,

@@ -17,8 +17,16 @@ for its CuPy/Triton backends).
 ``hip_plif_atomic_reduce``
     ``False``: the PLIF ``dL/dk`` sum is reduced in a fixed order (bitwise
     reproducible).  ``True``: one ``atomicAdd`` per block, order varies run to run.
+
+``hip_backward_recompute``
+    ``True``: training forwards write no ``h_seq``; the backward kernel replays the forward from
+    ``x_seq`` and ``v_init`` (bit-identical ``h``, held in LDS), so autograd keeps ``x_seq`` alive
+    instead of a same-sized ``h_seq`` and the forward's largest write disappears.  Used whenever the
+    shape allows (``N`` a multiple of the 128-bit vector width, ``T`` up to 159 for fp32 / 79 for
+    16-bit storage); other shapes and ``False`` fall back to saving ``h_seq``.
 """
 
 hip_half_precision_mode = "torch"
+hip_backward_recompute = True
 hip_lif_reciprocal_tau = False
 hip_plif_atomic_reduce = False

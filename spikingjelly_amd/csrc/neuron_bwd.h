@@ -19,6 +19,8 @@
 // or one atomicAdd per block.
 #pragma once
 
+#include <cmath>
+
 #include "sjhip_common.h"
 
 #ifndef SJHIP_BWD_PF
@@ -86,8 +88,12 @@ template <int SG> __device__ __forceinline__ float surrogate_grad(float x, float
   }
 }
 
-template <typename S, bool VECTOR, bool PLIF, int SG, bool GVFULL>
-__device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, int64_t col, float k) {
+// HLDS: h_t does not come from h_seq in global memory but from LDS, where the recompute kernel
+// (neuron_bwd_recompute.h) has left it as fp32, V/4 float4 per work-item and step, laid out
+// [step][quarter][lane] so a wavefront reads consecutive 16-byte words.
+template <typename S, bool VECTOR, bool PLIF, int SG, bool GVFULL, bool HLDS = false>
+__device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, int64_t col, float k,
+                                               const f32x4 *lds_h = nullptr) {
   typedef Acc<S, VECTOR, SJHIP_BWD_NT != 0> A;
   typedef typename A::elem_t E;
   constexpr int V = A::V;
@@ -98,7 +104,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
 
   const int64_t N = a.N, T = a.T;
   const E *gsp = (const E *)a.grad_spike + col;
-  const E *hp = (const E *)a.h + col;
+  const E *hp = HLDS ? nullptr : (const E *)a.h + col;
   const E *gvp = GVFULL ? (const E *)a.grad_v_seq + col : nullptr;
   E *gxp = (E *)a.grad_x + col;
 
@@ -111,7 +117,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
   for (int i = 0; i < PF; ++i) {
     const int64_t t = T - 1 - i;
     ahead_gs[i] = (t >= 0) ? A::load(gsp + t * N) : A::zero();
-    ahead_h[i] = (t >= 0) ? A::load(hp + t * N) : A::zero();
+    if (!HLDS) ahead_h[i] = (t >= 0) ? A::load(hp + t * N) : A::zero();
     if (GVFULL) ahead_gv[i] = (t >= 0) ? A::load(gvp + t * N) : A::zero();
   }
 
@@ -132,7 +138,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       cur_gs[i] = ahead_gs[i];
-      cur_h[i] = ahead_h[i];
+      if (!HLDS) cur_h[i] = ahead_h[i];
       if (GVFULL) cur_gv[i] = ahead_gv[i];
     }
 #pragma unroll
@@ -140,7 +146,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
       const int64_t tn = t0 - PF - i;
       if (tn >= 0) {
         ahead_gs[i] = A::load(gsp + tn * N);
-        ahead_h[i] = A::load(hp + tn * N);
+        if (!HLDS) ahead_h[i] = A::load(hp + tn * N);
         if (GVFULL) ahead_gv[i] = A::load(gvp + tn * N);
       }
     }
@@ -150,7 +156,15 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
       if (t >= 0) {
         float gs[V], h[V], gv[V], gx[V];
         A::unpack(cur_gs[i], gs);
-        A::unpack(cur_h[i], h);
+        if (HLDS) {
+#pragma unroll
+          for (int q = 0; q < V / 4; ++q) {
+            const f32x4 w = lds_h[((int)t * (V / 4) + q) * (int)blockDim.x + (int)threadIdx.x];
+            h[4 * q] = w.x; h[4 * q + 1] = w.y; h[4 * q + 2] = w.z; h[4 * q + 3] = w.w;
+          }
+        } else {
+          A::unpack(cur_h[i], h);
+        }
         if (GVFULL) A::unpack(cur_gv[i], gv);
 #pragma unroll
         for (int j = 0; j < V; ++j) {
@@ -188,10 +202,46 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
   return acc_total;
 }
 
-template <typename S, bool VECTOR, bool PLIF, int SG>
-__device__ __forceinline__ float backward_gv_dispatch(const BwdArgs &a, bool active, int64_t col, float k) {
-  if (a.grad_v_seq) return backward_body<S, VECTOR, PLIF, SG, true>(a, active, col, k);
-  return backward_body<S, VECTOR, PLIF, SG, false>(a, active, col, k);
+template <typename S, bool VECTOR, bool PLIF, int SG, bool HLDS = false>
+__device__ __forceinline__ float backward_gv_dispatch(const BwdArgs &a, bool active, int64_t col, float k,
+                                                      const f32x4 *lds_h = nullptr) {
+  if (a.grad_v_seq) return backward_body<S, VECTOR, PLIF, SG, true, HLDS>(a, active, col, k, lds_h);
+  return backward_body<S, VECTOR, PLIF, SG, false, HLDS>(a, active, col, k, lds_h);
+}
+
+template <typename S, bool VECTOR, bool PLIF, bool HLDS>
+__device__ __forceinline__ float backward_sg_dispatch(const BwdArgs &a, bool active, int64_t col, float k,
+                                                      const f32x4 *lds_h) {
+  switch (a.sg) {
+    case SJHIP_SG_SIGMOID: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SIGMOID, HLDS>(a, active, col, k, lds_h);
+    case SJHIP_SG_ATAN: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_ATAN, HLDS>(a, active, col, k, lds_h);
+    case SJHIP_SG_PIECEWISE_QUADRATIC: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_PIECEWISE_QUADRATIC, HLDS>(a, active, col, k, lds_h);
+    case SJHIP_SG_PIECEWISE_EXP: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_PIECEWISE_EXP, HLDS>(a, active, col, k, lds_h);
+    case SJHIP_SG_SOFT_SIGN: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SOFT_SIGN, HLDS>(a, active, col, k, lds_h);
+    case SJHIP_SG_SUPER_SPIKE: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SUPER_SPIKE, HLDS>(a, active, col, k, lds_h);
+    default: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_ERF, HLDS>(a, active, col, k, lds_h);
+  }
+}
+
+// Block-level sum of `part` (PLIF dL/dk): wavefront shuffles, then LDS, then one partial or atomic.
+__device__ __forceinline__ void plif_block_reduce(const BwdArgs &a, float part, float k) {
+  __shared__ float wave_sum[SJHIP_MAX_BLOCK / 64];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) part += __shfl_down(part, off, 64);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) wave_sum[wave] = part;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float total = 0.0f;
+    const int nwaves = (blockDim.x + 63) >> 6;
+    for (int w = 0; w < nwaves; ++w) total += wave_sum[w];
+    if (a.atomic_reduce) {
+      if (a.decay_input) total = total / k;
+      atomicAdd(a.grad_k, total);
+    } else {
+      a.partials[blockIdx.x] = total;
+    }
+  }
 }
 
 template <typename S, bool VECTOR, bool PLIF>
@@ -200,57 +250,45 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_kernel(const BwdArgs
   const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
   const bool active = col < a.N;
   const float k = a.k_device ? *a.k_device : a.k;
-  float part;
-  switch (a.sg) {
-    case SJHIP_SG_SIGMOID: part = backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SIGMOID>(a, active, col, k); break;
-    case SJHIP_SG_ATAN: part = backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_ATAN>(a, active, col, k); break;
-    case SJHIP_SG_PIECEWISE_QUADRATIC: part = backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_PIECEWISE_QUADRATIC>(a, active, col, k); break;
-    case SJHIP_SG_PIECEWISE_EXP: part = backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_PIECEWISE_EXP>(a, active, col, k); break;
-    case SJHIP_SG_SOFT_SIGN: part = backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SOFT_SIGN>(a, active, col, k); break;
-    case SJHIP_SG_SUPER_SPIKE: part = backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SUPER_SPIKE>(a, active, col, k); break;
-    default: part = backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_ERF>(a, active, col, k); break;
-  }
-  if (PLIF) {
-    // wavefront (64 lanes) shuffle reduction, then one value per wavefront through LDS
-    __shared__ float wave_sum[SJHIP_MAX_BLOCK / 64];
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) part += __shfl_down(part, off, 64);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if (lane == 0) wave_sum[wave] = part;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      float total = 0.0f;
-      const int nwaves = (blockDim.x + 63) >> 6;
-      for (int w = 0; w < nwaves; ++w) total += wave_sum[w];
-      if (a.atomic_reduce) {
-        if (a.decay_input) total = total / k;
-        atomicAdd(a.grad_k, total);
-      } else {
-        a.partials[blockIdx.x] = total;
-      }
-    }
-  }
+  const float part = backward_sg_dispatch<S, VECTOR, PLIF, false>(a, active, col, k, nullptr);
+  if (PLIF) plif_block_reduce(a, part, k);
 }
 
-// Fixed-order final sum of the per-block partials: lane i adds partials[i], [i+1024], ... in fp64,
-// then a binary tree over the 1024 lanes through LDS.  Same order on every run.
-__global__ void __launch_bounds__(1024) plif_reduce_kernel(const float *partials, int64_t count,
-                                                            const float *k_device, float k_host,
-                                                            int decay_input, float *out) {
-  __shared__ double tree[1024];
-  double sum = 0.0;
-  for (int64_t i = threadIdx.x; i < count; i += 1024) sum += (double)partials[i];
-  tree[threadIdx.x] = sum;
-  __syncthreads();
-  for (int stride = 512; stride > 0; stride >>= 1) {
-    if ((int)threadIdx.x < stride) tree[threadIdx.x] += tree[threadIdx.x + stride];
-    __syncthreads();
+// ---- host side: turn the ABI parameters into kernel arguments ------------------------------------
+inline int build_bwd_args(BwdArgs &a, int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
+                          const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                          const void *h_seq, const void *v_init, const float *k_device, void *grad_x_seq,
+                          void *grad_v_init, float *grad_rtau, float *workspace) {
+  (void)dtype;
+  a.grad_spike = grad_spike_seq; a.grad_v_seq = grad_v_seq; a.grad_v_last = grad_v_last; a.h = h_seq; a.v_init = v_init;
+  a.k_device = nullptr;
+  a.grad_x = grad_x_seq; a.grad_v_init = grad_v_init;
+  a.partials = workspace; a.grad_k = grad_rtau;
+  a.T = T; a.N = N;
+  a.v_th = p.v_threshold; a.v_reset = p.v_reset; a.alpha = p.sg_alpha;
+  a.sg = p.sg_id;
+  a.soft_reset = (p.flags & SJHIP_FLAG_SOFT_RESET) ? 1 : 0;
+  a.decay_input = (p.flags & SJHIP_FLAG_DECAY_INPUT) ? 1 : 0;
+  a.is_if = neuron == SJHIP_NEURON_IF;
+  a.atomic_reduce = (p.flags & SJHIP_FLAG_ATOMIC_REDUCE) ? 1 : 0;
+  const bool detach = (p.flags & SJHIP_FLAG_DETACH_RESET) != 0;
+  if (a.soft_reset) { a.cB = 0.0f; a.cC = detach ? 0.0f : -p.v_threshold; a.cD = 0.0f; }
+  else { a.cB = 1.0f; a.cC = detach ? 0.0f : p.v_reset; a.cD = detach ? 0.0f : 1.0f; }
+
+  const bool plif = neuron == SJHIP_NEURON_PLIF;
+  if (neuron == SJHIP_NEURON_IF) {
+    a.k = 0.0f;
+  } else if (plif) {
+    a.k = p.tau;
+    a.k_device = k_device;
+  } else {
+    if (!(p.tau > 0.0f) || !std::isfinite(p.tau)) return fail(SJHIP_ERR_INVALID, "backward: tau=%g", (double)p.tau);
+    a.k = (float)(1.0 / (double)p.tau);
   }
-  if (threadIdx.x == 0) {
-    double total = tree[0];
-    if (decay_input) total /= (double)(k_device ? *k_device : k_host);
-    out[0] = (float)total;
-  }
+
+  return SJHIP_OK;
 }
+
+int launch_plif_reduce(const BwdArgs &a, int64_t blocks, float *grad_k_out, hipStream_t stream);
 
 }  // namespace sjhip

@@ -5,6 +5,27 @@
 
 namespace sjhip {
 
+// Fixed-order final sum of the per-block partials: lane i adds partials[i], [i+1024], ... in fp64,
+// then a binary tree over the 1024 lanes through LDS.  Same order on every run.
+__global__ void __launch_bounds__(1024) plif_reduce_kernel(const float *partials, int64_t count,
+                                                            const float *k_device, float k_host,
+                                                            int decay_input, float *out) {
+  __shared__ double tree[1024];
+  double sum = 0.0;
+  for (int64_t i = threadIdx.x; i < count; i += 1024) sum += (double)partials[i];
+  tree[threadIdx.x] = sum;
+  __syncthreads();
+  for (int stride = 512; stride > 0; stride >>= 1) {
+    if ((int)threadIdx.x < stride) tree[threadIdx.x] += tree[threadIdx.x + stride];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    double total = tree[0];
+    if (decay_input) total /= (double)(k_device ? *k_device : k_host);
+    out[0] = (float)total;
+  }
+}
+
 namespace {
 
 template <typename S>
@@ -28,16 +49,18 @@ int launch_typed(BwdArgs &a, bool vector, bool plif, float *grad_k_out, hipStrea
     int rc = check_launch("backward");
     if (rc != SJHIP_OK) return rc;
   }
-  if (plif && !a.atomic_reduce) {
-    ProfileScope prof(KC_PLIF_REDUCE, stream);
-    hipLaunchKernelGGL(plif_reduce_kernel, dim3(1), dim3(1024), 0, stream, (const float *)a.partials, blocks,
-                       a.k_device, a.k, a.decay_input, grad_k_out);
-    return check_launch("plif_reduce");
-  }
+  if (plif && !a.atomic_reduce) return launch_plif_reduce(a, blocks, grad_k_out, stream);
   return SJHIP_OK;
 }
 
 }  // namespace
+
+int launch_plif_reduce(const BwdArgs &a, int64_t blocks, float *grad_k_out, hipStream_t stream) {
+  ProfileScope prof(KC_PLIF_REDUCE, stream);
+  hipLaunchKernelGGL(plif_reduce_kernel, dim3(1), dim3(1024), 0, stream, (const float *)a.partials, blocks,
+                     a.k_device, a.k, a.decay_input, grad_k_out);
+  return check_launch("plif_reduce");
+}
 
 int64_t plif_blocks(int dtype, int64_t N) {
   (void)dtype;
@@ -51,31 +74,10 @@ int launch_backward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t
                     const float *k_device, void *grad_x_seq, void *grad_v_init, float *grad_rtau,
                     float *workspace, hipStream_t stream) {
   BwdArgs a;
-  a.grad_spike = grad_spike_seq; a.grad_v_seq = grad_v_seq; a.grad_v_last = grad_v_last; a.h = h_seq; a.v_init = v_init;
-  a.k_device = nullptr;
-  a.grad_x = grad_x_seq; a.grad_v_init = grad_v_init;
-  a.partials = workspace; a.grad_k = grad_rtau;
-  a.T = T; a.N = N;
-  a.v_th = p.v_threshold; a.v_reset = p.v_reset; a.alpha = p.sg_alpha;
-  a.sg = p.sg_id;
-  a.soft_reset = (p.flags & SJHIP_FLAG_SOFT_RESET) ? 1 : 0;
-  a.decay_input = (p.flags & SJHIP_FLAG_DECAY_INPUT) ? 1 : 0;
-  a.is_if = neuron == SJHIP_NEURON_IF;
-  a.atomic_reduce = (p.flags & SJHIP_FLAG_ATOMIC_REDUCE) ? 1 : 0;
-  const bool detach = (p.flags & SJHIP_FLAG_DETACH_RESET) != 0;
-  if (a.soft_reset) { a.cB = 0.0f; a.cC = detach ? 0.0f : -p.v_threshold; a.cD = 0.0f; }
-  else { a.cB = 1.0f; a.cC = detach ? 0.0f : p.v_reset; a.cD = detach ? 0.0f : 1.0f; }
-
+  int rc = build_bwd_args(a, neuron, dtype, p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, k_device,
+                          grad_x_seq, grad_v_init, grad_rtau, workspace);
+  if (rc != SJHIP_OK) return rc;
   const bool plif = neuron == SJHIP_NEURON_PLIF;
-  if (neuron == SJHIP_NEURON_IF) {
-    a.k = 0.0f;
-  } else if (plif) {
-    a.k = p.tau;
-    a.k_device = k_device;
-  } else {
-    if (!(p.tau > 0.0f) || !std::isfinite(p.tau)) return fail(SJHIP_ERR_INVALID, "backward: tau=%g", (double)p.tau);
-    a.k = (float)(1.0 / (double)p.tau);
-  }
 
   const int esize = dtype == SJHIP_F32 ? 4 : 2;
   const int V = 16 / esize;

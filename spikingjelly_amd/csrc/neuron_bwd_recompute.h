@@ -1,0 +1,95 @@
+// Backward that recomputes h instead of reading a saved h_seq.
+//
+// Phase 1 replays the forward recurrence from x_seq and v_init with the forward's own arithmetic
+// (neuron_step of neuron_fwd.h, so h_t is bit-identical to what the forward computed) and parks h_t
+// for every step in LDS as fp32.  Phase 2 is the ordinary BPTT walk of neuron_bwd.h reading h_t
+// from LDS.  Each work-item touches only its own LDS words, so no barrier is needed.
+//
+// Why: the forward then never writes h_seq (4 B per neuron-step less to write in the slowest,
+// write-dominated kernel) and the backward reads x_seq instead of h_seq (same bytes).  LDS holds
+// T * blockDim * V * 4 bytes per block, which also bounds T (see recompute_block()).
+#pragma once
+
+#include "neuron_bwd.h"
+#include "neuron_fwd.h"
+
+namespace sjhip {
+
+template <typename S, bool ROUND_EACH, int CH, bool SOFT>
+__device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, int64_t col) {
+  typedef Acc<S, true, SJHIP_BWD_NT != 0> A;
+  typedef typename A::elem_t E;
+  typedef typename std::conditional<ROUND_EACH, S, float>::type R;
+  constexpr int V = A::V;
+  constexpr int PF = SJHIP_BWD_PF;
+
+  const int64_t N = a.N, T = a.T;
+  const E *xp = (const E *)a.x + col;
+  const float tau = a.k_device ? *a.k_device : a.tau;
+
+  typename A::raw_t ahead[PF];
+#pragma unroll
+  for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? A::load(xp + (int64_t)i * N) : A::zero();
+  float v[V];
+  A::unpack(A::load((const E *)a.v_init + col), v);
+
+  for (int64_t t0 = 0; t0 < T; t0 += PF) {
+    typename A::raw_t cur[PF];
+#pragma unroll
+    for (int i = 0; i < PF; ++i) cur[i] = ahead[i];
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int64_t tn = t0 + PF + i;
+      if (tn < T) ahead[i] = A::load(xp + tn * N);
+    }
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int64_t t = t0 + i;
+      if (t < T) {
+        float x[V], h[V], s[V];
+        A::unpack(cur[i], x);
+#pragma unroll
+        for (int j = 0; j < V; ++j) neuron_step<R, CH, SOFT>(x[j], v[j], h[j], s[j], tau, a);
+#pragma unroll
+        for (int q = 0; q < V / 4; ++q) {
+          f32x4 w; w.x = h[4 * q]; w.y = h[4 * q + 1]; w.z = h[4 * q + 2]; w.w = h[4 * q + 3];
+          lds_h[((int)t * (V / 4) + q) * (int)blockDim.x + (int)threadIdx.x] = w;
+        }
+      }
+    }
+  }
+}
+
+template <typename S, bool ROUND_EACH, int CH>
+__device__ __forceinline__ void recompute_reset_dispatch(const FwdArgs &a, f32x4 *lds_h, int64_t col) {
+  if (a.soft_reset) recompute_body<S, ROUND_EACH, CH, true>(a, lds_h, col);
+  else recompute_body<S, ROUND_EACH, CH, false>(a, lds_h, col);
+}
+
+template <typename S, bool ROUND_EACH, bool PLIF>
+__global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_kernel(const FwdArgs f, const BwdArgs b) {
+  extern __shared__ f32x4 lds_h[];
+  constexpr int V = Acc<S, true, true>::V;
+  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
+  const bool active = col < b.N;
+  if (active) {
+    switch (f.charge) {
+      case CH_IF: recompute_reset_dispatch<S, ROUND_EACH, CH_IF>(f, lds_h, col); break;
+      case CH_DECAY_INPUT_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_DECAY_INPUT_DIV>(f, lds_h, col); break;
+      case CH_DECAY_INPUT_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_DECAY_INPUT_MUL>(f, lds_h, col); break;
+      case CH_PLAIN_INPUT_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_PLAIN_INPUT_DIV>(f, lds_h, col); break;
+      default: recompute_reset_dispatch<S, ROUND_EACH, CH_PLAIN_INPUT_MUL>(f, lds_h, col); break;
+    }
+  }
+  const float k = b.k_device ? *b.k_device : b.k;
+  const float part = backward_sg_dispatch<S, true, PLIF, true>(b, active, col, k, lds_h);
+  if (PLIF) plif_block_reduce(b, part, k);
+}
+
+// Launches the recompute kernel of storage dtype S; defined in neuron_bwd_recompute_launch.h and
+// instantiated once per dtype (neuron_bwd_recompute_{f32,f16,bf16}.hip).
+template <typename S>
+int launch_recompute_dtype(const FwdArgs &f, const BwdArgs &b, bool round_each, bool plif, int block, unsigned lds,
+                           int64_t blocks, hipStream_t stream);
+
+}  // namespace sjhip

@@ -1,0 +1,79 @@
+// Host launcher of the recompute backward (see neuron_bwd_recompute.h).
+#include "neuron_bwd_recompute.h"
+
+// the kernels of each storage dtype are compiled in their own translation unit
+
+
+namespace sjhip {
+
+extern template int launch_recompute_dtype<float>(const FwdArgs &, const BwdArgs &, bool, bool, int, unsigned, int64_t, hipStream_t);
+extern template int launch_recompute_dtype<f16_t>(const FwdArgs &, const BwdArgs &, bool, bool, int, unsigned, int64_t, hipStream_t);
+extern template int launch_recompute_dtype<bf16_t>(const FwdArgs &, const BwdArgs &, bool, bool, int, unsigned, int64_t, hipStream_t);
+
+namespace {
+
+constexpr unsigned kMaxLds = 159u * 1024u;  // LDS per compute unit on gfx950 minus 1 KiB for static words
+
+// Largest block (128 or 64 lanes) whose h buffer T * block * V * 4 bytes fits in LDS; 0 if none.
+int recompute_block(int dtype, int64_t T) {
+  const int64_t V = dtype == SJHIP_F32 ? 4 : 8;
+  for (int block : {128, 64}) {
+    if (block > SJHIP_MAX_BLOCK) continue;
+    if (T * block * V * 4 <= (int64_t)kMaxLds) return block;
+  }
+  return 0;
+}
+
+}  // namespace
+
+bool recompute_supported(int dtype, int64_t T, int64_t N) {
+  const int64_t V = dtype == SJHIP_F32 ? 4 : 8;
+  return N % V == 0 && recompute_block(dtype, T) != 0;
+}
+
+int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
+                              const void *x_seq, const void *v_init, const float *k_device,
+                              const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                              void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace,
+                              hipStream_t stream) {
+  if (!recompute_supported(dtype, T, N))
+    return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute): T=%lld N=%lld does not fit (N %% %d != 0 or T too large for LDS)",
+                (long long)T, (long long)N, dtype == SJHIP_F32 ? 4 : 8);
+  if (!aligned16(x_seq) || !aligned16(v_init) || !aligned16(grad_spike_seq) || !aligned16(grad_x_seq) ||
+      !aligned16(grad_v_init) || (grad_v_seq && !aligned16(grad_v_seq)) || (grad_v_last && !aligned16(grad_v_last)))
+    return fail(SJHIP_ERR_INVALID, "backward(recompute): every tensor must be 16-byte aligned");
+
+  FwdArgs f;
+  bool round_each = false;
+  // spike/v/h outputs of the replayed forward are never written: the kernel only uses x, v_init and scalars
+  int rc = build_fwd_args(f, round_each, neuron, dtype, p, T, N, x_seq, v_init, k_device, nullptr, nullptr, nullptr, nullptr);
+  if (rc != SJHIP_OK) return rc;
+  BwdArgs b;
+  rc = build_bwd_args(b, neuron, dtype, p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, nullptr, v_init, k_device,
+                      grad_x_seq, grad_v_init, grad_rtau, workspace);
+  if (rc != SJHIP_OK) return rc;
+
+  const int V = dtype == SJHIP_F32 ? 4 : 8;
+  const int block = recompute_block(dtype, T);
+  const int64_t items = N / V;
+  const int64_t blocks = (items + block - 1) / block;
+  if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "backward(recompute): N=%lld", (long long)N);
+  unsigned lds = (unsigned)(T * block * V * 4);
+  const unsigned cap = occupancy_cap_lds(tuning().bwd_blocks_per_cu);
+  if (cap > lds) lds = cap;
+  const bool plif = neuron == SJHIP_NEURON_PLIF;
+  {
+    ProfileScope prof(KC_BACKWARD, stream);
+    switch (dtype) {
+      case SJHIP_F32: rc = launch_recompute_dtype<float>(f, b, false, plif, block, lds, blocks, stream); break;
+      case SJHIP_F16: rc = launch_recompute_dtype<f16_t>(f, b, round_each, plif, block, lds, blocks, stream); break;
+      case SJHIP_BF16: rc = launch_recompute_dtype<bf16_t>(f, b, round_each, plif, block, lds, blocks, stream); break;
+      default: return fail(SJHIP_ERR_INVALID, "backward(recompute): dtype %d", dtype);
+    }
+    if (rc != SJHIP_OK) return rc;
+  }
+  if (plif && !b.atomic_reduce) return launch_plif_reduce(b, blocks, grad_rtau, stream);
+  return SJHIP_OK;
+}
+
+}  // namespace sjhip

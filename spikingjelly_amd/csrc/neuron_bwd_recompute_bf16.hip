@@ -1,0 +1,6 @@
+// Recompute-backward kernels for storage dtype bf16_t.
+#include "neuron_bwd_recompute_launch.h"
+
+namespace sjhip {
+template int launch_recompute_dtype<bf16_t>(const FwdArgs &, const BwdArgs &, bool, bool, int, unsigned, int64_t, hipStream_t);
+}  // namespace sjhip

@@ -1,0 +1,42 @@
+// Kernel launch of the recompute backward for one storage dtype; included by the per-dtype
+// translation units so the three sets of kernels compile in parallel.
+#pragma once
+
+#include <mutex>
+
+#include "neuron_bwd_recompute.h"
+
+namespace sjhip {
+
+// LDS per compute unit on gfx950 is 160 KiB; 1 KiB is left for the statically allocated reduction words
+constexpr unsigned kRecomputeMaxLds = 159u * 1024u;
+
+template <typename S, bool ROUND_EACH, bool PLIF>
+int launch_kernel(const FwdArgs &f, const BwdArgs &b, int block, unsigned lds, int64_t blocks, hipStream_t stream) {
+  auto kernel = backward_recompute_kernel<S, ROUND_EACH, PLIF>;
+  // a block may use more than the default 64 KiB of dynamic LDS only after this opt-in (once per kernel)
+  static std::once_flag once;
+  static hipError_t attr_rc = hipSuccess;
+  std::call_once(once, [&]() {
+    attr_rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)kRecomputeMaxLds);
+    (void)hipGetLastError();  // a refusal is reported below, only if the launch really needs the larger limit
+  });
+  if (lds > 64u * 1024u && attr_rc != hipSuccess)
+    return fail(SJHIP_ERR_LAUNCH, "backward(recompute): cannot raise the dynamic LDS limit: %s", hipGetErrorString(attr_rc));
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(block), lds, stream, f, b);
+  return check_launch("backward(recompute)");
+}
+
+template <typename S>
+int launch_recompute_dtype(const FwdArgs &f, const BwdArgs &b, bool round_each, bool plif, int block, unsigned lds,
+                           int64_t blocks, hipStream_t stream) {
+  if (std::is_same<S, float>::value || !round_each)
+    return plif ? launch_kernel<S, false, true>(f, b, block, lds, blocks, stream)
+                : launch_kernel<S, false, false>(f, b, block, lds, blocks, stream);
+  return plif ? launch_kernel<S, true, true>(f, b, block, lds, blocks, stream)
+              : launch_kernel<S, true, false>(f, b, block, lds, blocks, stream);
+}
+
+
+}  // namespace sjhip

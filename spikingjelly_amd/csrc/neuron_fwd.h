@@ -14,6 +14,7 @@
 // values are rounded (the reference's mixed-precision kernels).
 #pragma once
 
+#include <cmath>
 #include <type_traits>
 
 #include "sjhip_common.h"
@@ -154,6 +155,57 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) forward_kernel(const FwdArgs 
     case CH_PLAIN_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_DIV>(a); break;
     default: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_MUL>(a); break;
   }
+}
+
+// ---- host side: turn the ABI parameters into kernel arguments ------------------------------------
+inline bool is_power_of_two(float f) {
+  int e;
+  return std::isfinite(f) && f > 0.0f && std::frexp(f, &e) == 0.5f;
+}
+
+inline int build_fwd_args(FwdArgs &a, bool &round_each, int neuron, int dtype, const sjhip_neuron_params &p,
+                          int64_t T, int64_t N, const void *x_seq, const void *v_init, const float *k_device,
+                          void *spike_seq, void *v_seq, void *v_last, void *h_seq) {
+  a.x = x_seq; a.v_init = v_init; a.spike = spike_seq; a.v_seq = v_seq; a.v_last = v_last; a.h = h_seq;
+  a.k_device = nullptr;
+  a.T = T; a.N = N;
+  a.soft_reset = (p.flags & SJHIP_FLAG_SOFT_RESET) ? 1 : 0;
+  const bool decay_input = (p.flags & SJHIP_FLAG_DECAY_INPUT) != 0;
+  round_each = dtype != SJHIP_F32 && !(p.flags & SJHIP_FLAG_FP32_STATE);
+
+  a.tau = p.tau;
+  if (neuron == SJHIP_NEURON_IF) {
+    a.charge = CH_IF;
+  } else if (neuron == SJHIP_NEURON_PLIF) {
+    a.charge = decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL;
+    a.k_device = k_device;
+  } else {
+    if (!(p.tau > 0.0f) || !std::isfinite(p.tau)) return fail(SJHIP_ERR_INVALID, "forward: tau=%g", (double)p.tau);
+    if (p.flags & SJHIP_FLAG_RECIPROCAL_TAU) {
+      // fl(1/tau) from the double quotient, as the reference kernels receive it (multi_step/lif.py:338)
+      a.tau = (float)(1.0 / (double)p.tau);
+      a.charge = decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL;
+    } else if (is_power_of_two(p.tau) && p.tau <= 0x1p100f && p.tau >= 0x1p-100f) {
+      // x / 2^e == x * 2^-e bit for bit (both are exact scalings, subnormal results round identically)
+      a.tau = 1.0f / p.tau;
+      a.charge = decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL;
+    } else {
+      a.charge = decay_input ? CH_DECAY_INPUT_DIV : CH_PLAIN_INPUT_DIV;
+    }
+  }
+
+  // The torch CPU backend rounds a Python scalar to the tensor dtype before add/sub and keeps it in
+  // fp32 for mul/div; mirror that when every op is rounded to a 16-bit storage dtype.
+  a.vr_mul = p.v_reset;
+  a.vth_mul = p.v_threshold;
+  a.vr_add = p.v_reset;
+  a.vth_sub = p.v_threshold;
+  if (round_each) {
+    if (dtype == SJHIP_F16) { a.vr_add = Cvt<f16_t>::round(p.v_reset); a.vth_sub = Cvt<f16_t>::round(p.v_threshold); }
+    else { a.vr_add = Cvt<bf16_t>::round(p.v_reset); a.vth_sub = Cvt<bf16_t>::round(p.v_threshold); }
+  }
+
+  return SJHIP_OK;
 }
 
 }  // namespace sjhip

@@ -165,6 +165,32 @@ int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p, i
                          grad_v_init, grad_rtau, workspace, static_cast<hipStream_t>(stream));
 }
 
+int sjhip_recompute_supported(int dtype, int64_t T, int64_t N) {
+  if (!valid_dtype_fp(dtype) || T < 1 || N < 1) return 0;
+  return recompute_supported(dtype, T, N) ? 1 : 0;
+}
+
+int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_params *p, int64_t T, int64_t N,
+                                    const void *x_seq, const void *v_init, const float *rtau_device,
+                                    const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                                    void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace,
+                                    void *stream) {
+  if (!p) return fail(SJHIP_ERR_INVALID, "backward(recompute): params is NULL");
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_PLIF) return fail(SJHIP_ERR_INVALID, "backward(recompute): neuron %d", neuron);
+  if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "backward(recompute): dtype %d", dtype);
+  if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_ERF) return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute): surrogate id %d", p->sg_id);
+  int rc = check_shape("backward(recompute)", T, N);
+  if (rc != SJHIP_OK) return rc;
+  if (!x_seq || !v_init || !grad_spike_seq || !grad_x_seq || !grad_v_init) return fail(SJHIP_ERR_INVALID, "backward(recompute): NULL tensor");
+  if (neuron == SJHIP_NEURON_PLIF) {
+    if (!grad_rtau) return fail(SJHIP_ERR_INVALID, "backward(recompute): PLIF needs grad_rtau");
+    if (!(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace) return fail(SJHIP_ERR_INVALID, "backward(recompute): PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");
+  }
+  return launch_backward_recompute(neuron, dtype, *p, T, N, x_seq, v_init, rtau_device, grad_spike_seq, grad_v_seq,
+                                   grad_v_last, grad_x_seq, grad_v_init, grad_rtau, workspace,
+                                   static_cast<hipStream_t>(stream));
+}
+
 int sjhip_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, void *stream) {
   if (n < 0) return fail(SJHIP_ERR_INVALID, "bit_pack: n=%lld", (long long)n);
   if (n == 0) return SJHIP_OK;

@@ -175,6 +175,12 @@ int launch_backward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t
                     const void *h_seq, const void *v_init,
                     const float *k_device, void *grad_x_seq, void *grad_v_init, float *grad_rtau,
                     float *workspace, hipStream_t stream);
+bool recompute_supported(int dtype, int64_t T, int64_t N);
+int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
+                              const void *x_seq, const void *v_init, const float *k_device,
+                              const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                              void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace,
+                              hipStream_t stream);
 int64_t plif_blocks(int dtype, int64_t N);
 int launch_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, hipStream_t stream);
 int launch_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, hipStream_t stream);

@@ -187,3 +187,41 @@ def test_set_backend_switches_supported_modules_only():
     net = torch.nn.Sequential(neuron.LIFNode(step_mode="m"), torch.nn.Linear(4, 4), neuron.IFNode(step_mode="s"))
     functional.set_backend(net, "hip")
     assert net[0].backend == "hip" and net[2].backend == "torch"
+
+
+@pytest.mark.parametrize("cls", [neuron.IFNode, neuron.LIFNode, neuron.ParametricLIFNode])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_replay_and_h_seq_backward_paths_agree(cls, dtype):
+    """configure.hip_backward_recompute only changes where h comes from in the backward (replayed from x
+    vs read from a saved h_seq); in fp32 both see the same h bit for bit, so gradients must be identical."""
+    x = seeded_randn((16, 4, 256), 31, 0.4, 1.0).to(dtype).cuda()
+    gs = seeded_randn((16, 4, 256), 32).to(dtype).cuda()
+    grads = []
+    old = configure.hip_backward_recompute
+    try:
+        for flag in (True, False):
+            configure.hip_backward_recompute = flag
+            node = cls(step_mode="m", backend="hip", surrogate_function=surrogate.ATan(), store_v_seq=True).cuda()
+            xi = x.clone().requires_grad_()
+            s = node(xi)
+            (s * gs).sum().backward()
+            grads.append((s.detach(), node.v_seq.detach(), xi.grad))
+    finally:
+        configure.hip_backward_recompute = old
+    assert bits_equal(grads[0][0], grads[1][0]) and bits_equal(grads[0][1], grads[1][1])
+    if dtype == torch.float32:
+        assert bits_equal(grads[0][2], grads[1][2])
+    else:
+        torch.testing.assert_close(grads[0][2].float(), grads[1][2].float(), rtol=1e-2, atol=1e-2)
+
+
+def test_replay_path_with_misaligned_and_non_contiguous_input():
+    """A sliced (16-byte misaligned) x_seq and a permuted upstream gradient still take the replay path."""
+    base = seeded_randn((8, 4, 65), 33, 0.4, 1.0)
+    x = base[:, :, 1:]  # [8,4,64] view, rows start 4 bytes off
+    a, b = _pair(neuron.LIFNode, surrogate_function=surrogate.ATan())
+    xa, xb = x.clone().requires_grad_(), base.cuda()[:, :, 1:].requires_grad_()
+    g = seeded_randn((64, 4, 8), 34).permute(2, 1, 0)
+    a(xa).backward(g)
+    b(xb).backward(g.cuda())
+    torch.testing.assert_close(xb.grad.cpu(), xa.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)

@@ -37,24 +37,29 @@ def _flags(fp32_state=False, reciprocal=False, atomic=False):
            (L.FLAG_ATOMIC_REDUCE if atomic else 0)
 
 
-def hip_forward(K, kind, x, v0, tau_or_k, decay_input, vth, v_reset, store_v_seq=True, flags=0, training=True):
+def hip_forward(K, kind, x, v0, tau_or_k, decay_input, vth, v_reset, store_v_seq=True, flags=0, training=True,
+                recompute=False):
     """Calls the forward operator; returns CPU tensors (s, v_seq|None, v_last, h|None)."""
     soft = v_reset is None
     vr = 0.0 if soft else v_reset
     xd, vd = x.cuda(), v0.cuda()
     if kind == "if":
-        out = (K.hip_multistep_if_forward(xd, vd, vth, vr, soft, False, 1, 2.0, store_v_seq, flags) if training
+        out = (K.hip_multistep_if_forward(xd, vd, vth, vr, soft, False, 1, 2.0, store_v_seq, flags, recompute) if training
                else K.hip_multistep_if_inference(xd, vd, vth, vr, soft, store_v_seq, flags))
     elif kind == "lif":
-        out = (K.hip_multistep_lif_forward(xd, vd, vth, vr, soft, False, tau_or_k, decay_input, 1, 2.0, store_v_seq, flags)
+        out = (K.hip_multistep_lif_forward(xd, vd, vth, vr, soft, False, tau_or_k, decay_input, 1, 2.0, store_v_seq, flags,
+                                           recompute)
                if training else K.hip_multistep_lif_inference(xd, vd, vth, vr, soft, tau_or_k, decay_input, store_v_seq, flags))
     else:
         kd = torch.as_tensor(tau_or_k, dtype=torch.float32).cuda()
-        out = (K.hip_multistep_plif_forward(xd, vd, kd, vth, vr, soft, False, decay_input, 1, 2.0, store_v_seq, flags)
+        out = (K.hip_multistep_plif_forward(xd, vd, kd, vth, vr, soft, False, decay_input, 1, 2.0, store_v_seq, flags,
+                                            recompute)
                if training else K.hip_multistep_plif_inference(xd, vd, kd, vth, vr, soft, decay_input, store_v_seq, flags))
     torch.cuda.synchronize()
     s, v_seq, v_last = out[0].cpu(), (out[1].cpu() if store_v_seq else None), out[2].cpu()
-    h = out[3].cpu() if training else None
+    h = out[3].cpu() if training and not recompute else None
+    if training and recompute:
+        assert out[3].numel() == 0  # no h_seq is materialised on the replay path
     return s, v_seq, v_last, h
 
 
@@ -184,18 +189,21 @@ def test_forward_half_storage_fp32_state(K, dtype, kind, v_reset, decay_input):
 # ------------------------------------------------------------------------------------------------
 # backward
 # ------------------------------------------------------------------------------------------------
-def hip_backward(K, kind, gs, gv, gl, h, v0, tau_or_k, decay_input, vth, v_reset, detach, sg_id, alpha, flags=0):
+def hip_backward(K, kind, gs, gv, gl, h, v0, tau_or_k, decay_input, vth, v_reset, detach, sg_id, alpha, flags=0,
+                 x=None):
+    """h given -> the kernel reads h_seq; x given (h None) -> the kernel replays the forward from x, v0."""
     soft = v_reset is None
     vr = 0.0 if soft else v_reset
     d = lambda t: None if t is None else t.cuda()
+    hx = (d(h), None, None) if x is None else (None, d(x), d(v0))
     if kind == "if":
-        out = K.hip_multistep_if_backward(d(gs), d(gv), d(gl), h.cuda(), vth, vr, soft, detach, sg_id, alpha, flags)
+        out = K.hip_multistep_if_backward(d(gs), d(gv), d(gl), *hx, vth, vr, soft, detach, sg_id, alpha, flags)
     elif kind == "lif":
-        out = K.hip_multistep_lif_backward(d(gs), d(gv), d(gl), h.cuda(), vth, vr, soft, detach, tau_or_k, decay_input,
+        out = K.hip_multistep_lif_backward(d(gs), d(gv), d(gl), *hx, vth, vr, soft, detach, tau_or_k, decay_input,
                                            sg_id, alpha, flags)
     else:
         kd = torch.as_tensor(tau_or_k, dtype=torch.float32).cuda()
-        out = K.hip_multistep_plif_backward(d(gs), d(gv), d(gl), h.cuda(), v0.cuda(), kd, vth, vr, soft, detach,
+        out = K.hip_multistep_plif_backward(d(gs), d(gv), d(gl), hx[0], hx[1], d(v0), kd, vth, vr, soft, detach,
                                             decay_input, sg_id, alpha, flags)
     torch.cuda.synchronize()
     return tuple(o.cpu() for o in out)
@@ -211,7 +219,10 @@ BWD_GRID = [(kind, sg, di, vr, det)
 
 @pytest.mark.parametrize("kind,sg,decay_input,v_reset,detach", BWD_GRID)
 @pytest.mark.parametrize("T,N", [(16, 4096), (7, 111)])
-def test_backward_matches_autograd_fp32(K, kind, sg, decay_input, v_reset, detach, T, N):
+@pytest.mark.parametrize("path", ["h_seq", "replay"])
+def test_backward_matches_autograd_fp32(K, kind, sg, decay_input, v_reset, detach, T, N, path):
+    if path == "replay" and N % 4 != 0:
+        pytest.skip("the replay kernel needs N % 4 == 0; such shapes use the h_seq path")
     tau, vth = 3.0, 0.8
     alpha = no.SG_DEFAULT_ALPHA[sg]
     x = seeded_randn((T, N), 600 + T, 0.4, 1.0)
@@ -224,7 +235,9 @@ def test_backward_matches_autograd_fp32(K, kind, sg, decay_input, v_reset, detac
     else:
         ref = no.forward_backward(kind, x, v0, gs, gv, gl, tau, decay_input, vth, v_reset, sg, alpha, detach)
         p = tau
-    out = hip_backward(K, kind, gs, gv, gl, ref["h_seq"], v0, p, decay_input, vth, v_reset, detach, no.SG_IDS[sg], alpha)
+    xr = x if path == "replay" else None
+    out = hip_backward(K, kind, gs, gv, gl, ref["h_seq"], v0, p, decay_input, vth, v_reset, detach, no.SG_IDS[sg], alpha,
+                       x=xr)
     torch.testing.assert_close(out[0], ref["grad_x"], rtol=GRAD_RTOL, atol=GRAD_ATOL)
     torch.testing.assert_close(out[1], ref["grad_v_init"], rtol=GRAD_RTOL, atol=GRAD_ATOL)
     if kind == "plif":
@@ -234,25 +247,28 @@ def test_backward_matches_autograd_fp32(K, kind, sg, decay_input, v_reset, detac
         if torch.equal(ref64["spike_seq"].float(), ref["spike_seq"]):
             assert float(out[2]) == pytest.approx(float(ref64["grad_p"]), rel=1e-4, abs=1e-3)
         out_atomic = hip_backward(K, kind, gs, gv, gl, ref["h_seq"], v0, p, decay_input, vth, v_reset, detach,
-                                  no.SG_IDS[sg], alpha, flags=_flags(atomic=True))
+                                  no.SG_IDS[sg], alpha, flags=_flags(atomic=True), x=xr)
         assert float(out_atomic[2]) == pytest.approx(float(out[2]), rel=1e-4, abs=1e-3)
 
 
 @pytest.mark.parametrize("sg", no.SG_NAMES)
-def test_backward_every_surrogate(K, sg):
+@pytest.mark.parametrize("path", ["h_seq", "replay"])
+def test_backward_every_surrogate(K, sg, path):
     T, N, tau, vth = 6, 2048, 2.0, 1.0
     alpha = no.SG_DEFAULT_ALPHA[sg]
     x = seeded_randn((T, N), 700, 0.5, 1.0)
     v0 = torch.zeros(N)
     gs = seeded_randn((T, N), 701)
     ref = no.forward_backward("lif", x, v0, gs, None, None, tau, True, vth, 0.0, sg, alpha, False)
-    out = hip_backward(K, "lif", gs, None, None, ref["h_seq"], v0, tau, True, vth, 0.0, False, no.SG_IDS[sg], alpha)
+    out = hip_backward(K, "lif", gs, None, None, ref["h_seq"], v0, tau, True, vth, 0.0, False, no.SG_IDS[sg], alpha,
+                       x=x if path == "replay" else None)
     torch.testing.assert_close(out[0], ref["grad_x"], rtol=GRAD_RTOL, atol=GRAD_ATOL)
     torch.testing.assert_close(out[1], ref["grad_v_init"], rtol=GRAD_RTOL, atol=GRAD_ATOL)
 
 
 @pytest.mark.parametrize("which", ["none", "last", "seq", "both"])
-def test_backward_grad_v_variants(K, which):
+@pytest.mark.parametrize("path", ["h_seq", "replay"])
+def test_backward_grad_v_variants(K, which, path):
     T, N = 9, 1024
     x = seeded_randn((T, N), 710, 0.5, 1.0)
     v0 = seeded_randn((N,), 711, 0, 0.2)
@@ -260,7 +276,8 @@ def test_backward_grad_v_variants(K, which):
     gv = seeded_randn((T, N), 713) if which in ("seq", "both") else None
     gl = seeded_randn((N,), 714) if which in ("last", "both") else None
     ref = no.forward_backward("lif", x, v0, gs, gv, gl, 2.0, True, 1.0, 0.0, "atan", 2.0, False)
-    out = hip_backward(K, "lif", gs, gv, gl, ref["h_seq"], v0, 2.0, True, 1.0, 0.0, False, 1, 2.0)
+    out = hip_backward(K, "lif", gs, gv, gl, ref["h_seq"], v0, 2.0, True, 1.0, 0.0, False, 1, 2.0,
+                       x=x if path == "replay" else None)
     torch.testing.assert_close(out[0], ref["grad_x"], rtol=GRAD_RTOL, atol=GRAD_ATOL)
     torch.testing.assert_close(out[1], ref["grad_v_init"], rtol=GRAD_RTOL, atol=GRAD_ATOL)
 
@@ -268,7 +285,8 @@ def test_backward_grad_v_variants(K, which):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("kind", ["if", "lif", "plif"])
 @pytest.mark.parametrize("v_reset", [0.0, None])
-def test_backward_half_storage(K, dtype, kind, v_reset):
+@pytest.mark.parametrize("path", ["h_seq", "replay"])
+def test_backward_half_storage(K, dtype, kind, v_reset, path):
     """16-bit storage: the kernel sees h_seq and the upstream gradients rounded to 16 bits.  Expected
     values come from the float64 recurrence fed exactly those rounded tensors (a spike decided on the
     rounded h is the spike the backward must use), so what is left is fp32 arithmetic plus one final
@@ -280,8 +298,10 @@ def test_backward_half_storage(K, dtype, kind, v_reset):
     v0 = seeded_randn((N,), 722, 0.0, 0.2).to(dtype)
     gs = seeded_randn((T, N), 721).to(dtype)
     gl = seeded_randn((N,), 723, 0.0, 0.1).to(dtype)
-    _, _, h = no.multi_step_mixed_precision(kind, x.float(), v0.float(), dtype, k, True, vth, v_reset)
-    h64 = h.double().numpy()
+    _, _, h, raw_h = no.multi_step_mixed_precision(kind, x.float(), v0.float(), dtype, k, True, vth, v_reset,
+                                                   return_raw_h=True)
+    # the h_seq path sees h rounded to 16 bits, the replay path recomputes the forward's unrounded fp32 h
+    h64 = (h if path == "h_seq" else raw_h).double().numpy()
     s64 = (h64 >= vth).astype(np.float64)
     vr = 0.0 if v_reset is None else v_reset
     v64 = h64 - s64 * vth if v_reset is None else s64 * vr + (1 - s64) * h64
@@ -292,7 +312,7 @@ def test_backward_half_storage(K, dtype, kind, v_reset):
                                       0.0 if kind == "if" else k, True, vth, v_reset, False, v_prev, x_implied)
     p = {"if": 0.0, "lif": 1.0 / k, "plif": k}[kind]
     out = hip_backward(K, kind, gs, None, gl, h.to(dtype), v0, p, True, vth, v_reset, False, 0, 4.0,
-                       flags=_flags(fp32_state=True))
+                       flags=_flags(fp32_state=True), x=x if path == "replay" else None)
     assert out[0].dtype == dtype and out[1].dtype == dtype
     torch.testing.assert_close(out[0].double(), torch.from_numpy(egx), rtol=HALF_RTOL, atol=1e-3)
     torch.testing.assert_close(out[1].double(), torch.from_numpy(egvi), rtol=HALF_RTOL, atol=1e-3)
@@ -300,7 +320,8 @@ def test_backward_half_storage(K, dtype, kind, v_reset):
         assert float(out[2]) == pytest.approx(egk, rel=1e-4)
 
 
-def test_plif_reduction_is_deterministic_and_accurate(K):
+@pytest.mark.parametrize("path", ["h_seq", "replay"])
+def test_plif_reduction_is_deterministic_and_accurate(K, path):
     T, N, k = 8, 1 << 18, 0.5
     x = seeded_randn((T, N), 730, 0.2, 1.0)
     v0 = torch.zeros(N)
@@ -308,7 +329,8 @@ def test_plif_reduction_is_deterministic_and_accurate(K):
     ref = no.forward_backward("plif_k", x.double(), v0.double(), gs.double(), None, None, torch.tensor(k).double(),
                               True, 1.0, None, "sigmoid", 4.0, False)
     h = ref["h_seq"].float()
-    a = hip_backward(K, "plif", gs, None, None, h, v0, k, True, 1.0, None, False, 0, 4.0)
-    b = hip_backward(K, "plif", gs, None, None, h, v0, k, True, 1.0, None, False, 0, 4.0)
+    xr = x if path == "replay" else None
+    a = hip_backward(K, "plif", gs, None, None, h, v0, k, True, 1.0, None, False, 0, 4.0, x=xr)
+    b = hip_backward(K, "plif", gs, None, None, h, v0, k, True, 1.0, None, False, 0, 4.0, x=xr)
     assert bits_equal(a[2], b[2])
     assert float(a[2]) == pytest.approx(float(ref["grad_p"]), rel=1e-5)

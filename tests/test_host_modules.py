@@ -186,12 +186,15 @@ def test_operator_schemas_and_fake_kernels():
         x = torch.empty(5, 12)
         v = torch.empty(12)
         s, v_seq, v_last, h = torch.ops.sj.hip_multistep_lif_forward(x, v, 1.0, 0.0, False, False, 2.0, True, 1, 2.0,
-                                                                     True, 0)
+                                                                     True, 0, False)
         assert s.shape == v_seq.shape == h.shape == (5, 12) and v_last.shape == (12,)
+        _, _, _, h = torch.ops.sj.hip_multistep_lif_forward(x, v, 1.0, 0.0, False, False, 2.0, True, 1, 2.0, True, 0,
+                                                            True)
+        assert h.shape == (0,)  # replay path keeps no h_seq
         s, v_seq, v_last = torch.ops.sj.hip_multistep_if_inference(x, v, 1.0, 0.0, True, False, 0)
         assert v_seq.shape == (0,) and v_last.shape == (12,)
-        gx, gvi, gk = torch.ops.sj.hip_multistep_plif_backward(x, None, None, x, v, torch.empty(()), 1.0, 0.0, False,
-                                                               False, True, 0, 4.0, 0)
+        gx, gvi, gk = torch.ops.sj.hip_multistep_plif_backward(x, None, None, None, x, v, torch.empty(()), 1.0, 0.0,
+                                                               False, False, True, 0, 4.0, 0)
         assert gx.shape == (5, 12) and gvi.shape == (12,) and gk.shape == ()
 
 
