@@ -180,7 +180,8 @@ int sjhip_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, void *
 /*
  * Launch tuning (process-wide, read at launch).  Keys: "fwd_block" / "bwd_block" = work-items per
  * block (64, 128, 256 or 512); "fwd_blocks_per_cu" / "bwd_blocks_per_cu" = cap on resident blocks per
- * compute unit (0 = none, else 2..64; enforced through a dynamic-LDS request).  Returns
+ * compute unit (0 = none, else 2..64; enforced through a dynamic-LDS request), and
+ * "replay_blocks_per_cu" likewise for sjhip_neuron_backward_recompute.  Returns
  * SJHIP_ERR_INVALID otherwise.  Results never depend on these.
  */
 int sjhip_set_tuning(const char *key, int value);

@@ -91,9 +91,27 @@ template <int SG> __device__ __forceinline__ float surrogate_grad(float x, float
 // HLDS: h_t does not come from h_seq in global memory but from LDS, where the recompute kernel
 // (neuron_bwd_recompute.h) has left it as fp32, V/4 float4 per work-item and step, laid out
 // [step][quarter][lane] so a wavefront reads consecutive 16-byte words.
+// First PF rows (t = T-1 downwards) of grad_spike and grad_v_seq, requested ahead of their use.
+template <typename S, bool VECTOR> struct BwdPrologue {
+  typedef Acc<S, VECTOR, SJHIP_BWD_NT != 0> A;
+  typename A::raw_t gs[SJHIP_BWD_PF], gv[SJHIP_BWD_PF];
+  __device__ __forceinline__ void load(const BwdArgs &a, int64_t col) {
+    typedef typename A::elem_t E;
+    const E *gsp = (const E *)a.grad_spike + col;
+    const E *gvp = (const E *)a.grad_v_seq + col;
+#pragma unroll
+    for (int i = 0; i < SJHIP_BWD_PF; ++i) {
+      const int64_t t = a.T - 1 - i;
+      gs[i] = (t >= 0) ? A::load(gsp + t * a.N) : A::zero();
+      if (a.grad_v_seq) gv[i] = (t >= 0) ? A::load(gvp + t * a.N) : A::zero();
+    }
+  }
+};
+
 template <typename S, bool VECTOR, bool PLIF, int SG, bool GVFULL, bool HLDS = false>
 __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, int64_t col, float k,
-                                               const f32x4 *lds_h = nullptr) {
+                                               const f32x4 *lds_h = nullptr,
+                                               const BwdPrologue<S, VECTOR> *pre = nullptr) {
   typedef Acc<S, VECTOR, SJHIP_BWD_NT != 0> A;
   typedef typename A::elem_t E;
   constexpr int V = A::V;
@@ -113,12 +131,21 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
   const float v_th = a.v_th, alpha = a.alpha, cB = a.cB, cC = a.cC, cD = a.cD;
 
   typename A::raw_t ahead_gs[PF], ahead_h[PF], ahead_gv[PF];
+  if (HLDS) {
+    // the replay kernel requested these rows before it started recomputing h
 #pragma unroll
-  for (int i = 0; i < PF; ++i) {
-    const int64_t t = T - 1 - i;
-    ahead_gs[i] = (t >= 0) ? A::load(gsp + t * N) : A::zero();
-    if (!HLDS) ahead_h[i] = (t >= 0) ? A::load(hp + t * N) : A::zero();
-    if (GVFULL) ahead_gv[i] = (t >= 0) ? A::load(gvp + t * N) : A::zero();
+    for (int i = 0; i < PF; ++i) {
+      ahead_gs[i] = pre->gs[i];
+      if (GVFULL) ahead_gv[i] = pre->gv[i];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int64_t t = T - 1 - i;
+      ahead_gs[i] = (t >= 0) ? A::load(gsp + t * N) : A::zero();
+      ahead_h[i] = (t >= 0) ? A::load(hp + t * N) : A::zero();
+      if (GVFULL) ahead_gv[i] = (t >= 0) ? A::load(gvp + t * N) : A::zero();
+    }
   }
 
   float carry[V];
@@ -204,22 +231,24 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
 
 template <typename S, bool VECTOR, bool PLIF, int SG, bool HLDS = false>
 __device__ __forceinline__ float backward_gv_dispatch(const BwdArgs &a, bool active, int64_t col, float k,
-                                                      const f32x4 *lds_h = nullptr) {
-  if (a.grad_v_seq) return backward_body<S, VECTOR, PLIF, SG, true, HLDS>(a, active, col, k, lds_h);
-  return backward_body<S, VECTOR, PLIF, SG, false, HLDS>(a, active, col, k, lds_h);
+                                                      const f32x4 *lds_h = nullptr,
+                                                      const BwdPrologue<S, VECTOR> *pre = nullptr) {
+  if (a.grad_v_seq) return backward_body<S, VECTOR, PLIF, SG, true, HLDS>(a, active, col, k, lds_h, pre);
+  return backward_body<S, VECTOR, PLIF, SG, false, HLDS>(a, active, col, k, lds_h, pre);
 }
 
 template <typename S, bool VECTOR, bool PLIF, bool HLDS>
 __device__ __forceinline__ float backward_sg_dispatch(const BwdArgs &a, bool active, int64_t col, float k,
-                                                      const f32x4 *lds_h) {
+                                                      const f32x4 *lds_h,
+                                                      const BwdPrologue<S, VECTOR> *pre = nullptr) {
   switch (a.sg) {
-    case SJHIP_SG_SIGMOID: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SIGMOID, HLDS>(a, active, col, k, lds_h);
-    case SJHIP_SG_ATAN: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_ATAN, HLDS>(a, active, col, k, lds_h);
-    case SJHIP_SG_PIECEWISE_QUADRATIC: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_PIECEWISE_QUADRATIC, HLDS>(a, active, col, k, lds_h);
-    case SJHIP_SG_PIECEWISE_EXP: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_PIECEWISE_EXP, HLDS>(a, active, col, k, lds_h);
-    case SJHIP_SG_SOFT_SIGN: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SOFT_SIGN, HLDS>(a, active, col, k, lds_h);
-    case SJHIP_SG_SUPER_SPIKE: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SUPER_SPIKE, HLDS>(a, active, col, k, lds_h);
-    default: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_ERF, HLDS>(a, active, col, k, lds_h);
+    case SJHIP_SG_SIGMOID: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SIGMOID, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_ATAN: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_ATAN, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_PIECEWISE_QUADRATIC: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_PIECEWISE_QUADRATIC, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_PIECEWISE_EXP: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_PIECEWISE_EXP, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_SOFT_SIGN: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SOFT_SIGN, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_SUPER_SPIKE: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SUPER_SPIKE, HLDS>(a, active, col, k, lds_h, pre);
+    default: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_ERF, HLDS>(a, active, col, k, lds_h, pre);
   }
 }
 

@@ -59,7 +59,7 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "backward(recompute): N=%lld", (long long)N);
   unsigned lds = (unsigned)(T * block * V * 4);
-  const unsigned cap = occupancy_cap_lds(tuning().bwd_blocks_per_cu);
+  const unsigned cap = occupancy_cap_lds(tuning().replay_blocks_per_cu);
   if (cap > lds) lds = cap;
   const bool plif = neuron == SJHIP_NEURON_PLIF;
   {

@@ -31,11 +31,13 @@ int launch_kernel(const FwdArgs &f, const BwdArgs &b, int block, unsigned lds, i
 template <typename S>
 int launch_recompute_dtype(const FwdArgs &f, const BwdArgs &b, bool round_each, bool plif, int block, unsigned lds,
                            int64_t blocks, hipStream_t stream) {
-  if (std::is_same<S, float>::value || !round_each)
-    return plif ? launch_kernel<S, false, true>(f, b, block, lds, blocks, stream)
-                : launch_kernel<S, false, false>(f, b, block, lds, blocks, stream);
-  return plif ? launch_kernel<S, true, true>(f, b, block, lds, blocks, stream)
-              : launch_kernel<S, true, false>(f, b, block, lds, blocks, stream);
+  if constexpr (!std::is_same<S, float>::value) {
+    if (round_each)
+      return plif ? launch_kernel<S, true, true>(f, b, block, lds, blocks, stream)
+                  : launch_kernel<S, true, false>(f, b, block, lds, blocks, stream);
+  }
+  return plif ? launch_kernel<S, false, true>(f, b, block, lds, blocks, stream)
+              : launch_kernel<S, false, false>(f, b, block, lds, blocks, stream);
 }
 
 

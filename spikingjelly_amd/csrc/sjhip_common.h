@@ -145,6 +145,7 @@ struct Tuning {
   int bwd_block;
   int fwd_blocks_per_cu;  // 0 = no cap; otherwise dynamic LDS is requested so that at most this many
   int bwd_blocks_per_cu;  // blocks are resident per compute unit
+  int replay_blocks_per_cu;  // same for the replay backward (its LDS h buffer already bounds residency)
 };
 // dynamic LDS bytes that cap residency at `blocks_per_cu` blocks (0 for no cap)
 unsigned occupancy_cap_lds(int blocks_per_cu);
