@@ -178,6 +178,22 @@ int sjhip_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, void *st
 int sjhip_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, void *stream);
 
 /*
+ * Spiking self-attention contraction on the matrix cores (stands in for `_ssa_kernel_torch`,
+ * spikingjelly/activation_based/layer/attention.py:346-353:  x = (v @ k^T) @ q * scale).
+ *   qkv      [samples, 3, heads, channels_per_head, tokens] in: binary spikes, q / k / v stacked on dim 1
+ *   out      [samples, heads, channels_per_head, tokens] out = scale * (V K^T) Q, exact (integer sums in fp32)
+ *   grad_out same shape as out, in;  grad_qkv same shape as qkv, out (dq, dk, dv)
+ * bf16 MFMA with fp32 accumulation for the two spike products, fp32 MFMA for the backward products with
+ * real-valued operands.  One wavefront per (sample, head); needs sjhip_ssa_supported(): at most 64 channels
+ * per head, at most 256 tokens (V K^T must stay exact in bf16) and the tiles of one head fitting in LDS.
+ */
+int sjhip_ssa_supported(int dtype, int channels_per_head, int64_t tokens);
+int sjhip_ssa_forward(int dtype, int64_t samples, int heads, int channels_per_head, int64_t tokens, float scale,
+                      const void *qkv, void *out, void *stream);
+int sjhip_ssa_backward(int dtype, int64_t samples, int heads, int channels_per_head, int64_t tokens, float scale,
+                       const void *qkv, const void *grad_out, void *grad_qkv, void *stream);
+
+/*
  * Launch tuning (process-wide, read at launch).  Keys: "fwd_block" / "bwd_block" = work-items per
  * block (64, 128, 256 or 512); "fwd_blocks_per_cu" / "bwd_blocks_per_cu" = cap on resident blocks per
  * compute unit (0 = none, else 2..64; enforced through a dynamic-LDS request), and
@@ -190,7 +206,7 @@ int sjhip_get_tuning(const char *key);
 /*
  * Optional per-kernel timing.  While enabled every launch is bracketed by HIP events on its own
  * stream.  sjhip_profile_read() synchronises those events and returns, for kernel class `which`
- * (0 forward, 1 backward, 2 plif-reduce, 3 bit_pack, 4 bit_unpack), the launch count and total
+ * (0 forward, 1 backward, 2 plif-reduce, 3 bit_pack, 4 bit_unpack, 5 ssa forward, 6 ssa backward), the launch count and total
  * milliseconds since the last sjhip_profile_reset().
  */
 int sjhip_profile_enable(int on);

@@ -26,7 +26,7 @@ FLAG_FP32_STATE = 0x10
 FLAG_RECIPROCAL_TAU = 0x20
 FLAG_ATOMIC_REDUCE = 0x80
 
-KC_FORWARD, KC_BACKWARD, KC_PLIF_REDUCE, KC_BIT_PACK, KC_BIT_UNPACK = range(5)
+KC_FORWARD, KC_BACKWARD, KC_PLIF_REDUCE, KC_BIT_PACK, KC_BIT_UNPACK, KC_SSA_FORWARD, KC_SSA_BACKWARD = range(7)
 
 EXPORTED_SYMBOLS = (
     "sjhip_abi_version",
@@ -36,6 +36,9 @@ EXPORTED_SYMBOLS = (
     "sjhip_neuron_backward",
     "sjhip_neuron_backward_recompute",
     "sjhip_recompute_supported",
+    "sjhip_ssa_supported",
+    "sjhip_ssa_forward",
+    "sjhip_ssa_backward",
     "sjhip_bit_pack",
     "sjhip_bit_unpack",
     "sjhip_set_tuning",
@@ -106,6 +109,13 @@ def load() -> ctypes.CDLL:
         ]
         lib.sjhip_recompute_supported.restype = c_int
         lib.sjhip_recompute_supported.argtypes = [c_int, c_int64, c_int64]
+        lib.sjhip_ssa_supported.restype = c_int
+        lib.sjhip_ssa_supported.argtypes = [c_int, c_int, c_int64]
+        lib.sjhip_ssa_forward.restype = c_int
+        lib.sjhip_ssa_forward.argtypes = [c_int, c_int64, c_int, c_int, c_int64, c_float, c_void_p, c_void_p, c_void_p]
+        lib.sjhip_ssa_backward.restype = c_int
+        lib.sjhip_ssa_backward.argtypes = [c_int, c_int64, c_int, c_int, c_int64, c_float, c_void_p, c_void_p, c_void_p,
+                                           c_void_p]
         lib.sjhip_bit_pack.restype = c_int
         lib.sjhip_bit_pack.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p]
         lib.sjhip_bit_unpack.restype = c_int

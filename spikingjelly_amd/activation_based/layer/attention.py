@@ -1,0 +1,85 @@
+"""Spikformer-style spiking self-attention (reference ``layer/attention.py:245-387``).
+
+``Conv1d+BN -> LIF -> scale * (V K^T) Q -> LIF(v_threshold=0.5) -> Conv1d+BN -> LIF`` on ``[T, N, C, L]``
+input.  With ``backend='hip'`` the three LIF nodes run the HIP neuron kernels and the contraction runs on
+the matrix cores (bf16 MFMA, fp32 accumulation; exact because Q/K/V are binary); the 1x1 convolutions and
+batch norms stay with torch.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from .. import base, neuron
+from .container import SeqToANNContainer
+
+
+class SpikingSelfAttention(nn.Module, base.MultiStepModule):
+    def __init__(self, dim, num_heads=8, backend: str = "torch"):
+        super().__init__()
+        if dim % num_heads != 0:
+            raise ValueError(f"dim {dim} should be divided by num_heads {num_heads}.")
+        self.dim = dim
+        self.num_heads = num_heads
+        self.head_dim = dim // num_heads
+        self.scale = 0.125
+        self.qkv_conv_bn = SeqToANNContainer(
+            nn.Conv1d(dim, dim * 3, kernel_size=1, stride=1, bias=False),
+            nn.BatchNorm1d(dim * 3),
+        )
+        self.qkv_lif = neuron.LIFNode(tau=2.0, detach_reset=True, step_mode="m", backend=backend)
+        self.attn_lif = neuron.LIFNode(tau=2.0, v_threshold=0.5, detach_reset=True, step_mode="m", backend=backend)
+        self.proj_conv_bn = SeqToANNContainer(
+            nn.Conv1d(dim, dim, kernel_size=1, stride=1, bias=False),
+            nn.BatchNorm1d(dim),
+        )
+        self.proj_lif = neuron.LIFNode(tau=2.0, detach_reset=True, step_mode="m", backend=backend)
+
+    @property
+    def backend(self):
+        return self.qkv_lif.backend
+
+    @backend.setter
+    def backend(self, value: str):
+        self.qkv_lif.backend = value
+        self.attn_lif.backend = value
+        self.proj_lif.backend = value
+
+    @property
+    def supported_backends(self):
+        return self.qkv_lif.supported_backends
+
+    @staticmethod
+    def _ssa_kernel_torch(qkv, scale):
+        # qkv [T, N, 3, heads, Cph, L] -> [T, N, heads, Cph, L]
+        qt, kt, vt = qkv.flatten(2, 3).chunk(3, dim=2)
+        x_seq = vt @ kt.transpose(-2, -1)
+        return (x_seq @ qt) * scale
+
+    @staticmethod
+    def _ssa_kernel_hip(qkv, scale):
+        from ..hip_kernel.attention_kernel import hip_ssa_forward
+
+        T, N = qkv.shape[:2]
+        out = hip_ssa_forward(qkv.flatten(0, 1), scale)
+        return out.view(T, N, *out.shape[1:])
+
+    def forward(self, x_seq: torch.Tensor):
+        if x_seq.ndim != 4:
+            raise ValueError(f"expected 4D input with shape [T, N, C, L], but got input with shape {x_seq.shape}")
+        T, N, C, L = x_seq.shape
+        qkv = self.qkv_lif(self.qkv_conv_bn(x_seq))  # [T, N, 3*C, L]
+        local_dim = qkv.shape[2] // 3
+        if local_dim % self.num_heads != 0:
+            raise ValueError(f"local qkv dim {local_dim} is not divisible by num_heads={self.num_heads}.")
+        qkv = qkv.reshape(T, N, 3, self.num_heads, local_dim // self.num_heads, L)
+        if self.backend == "hip":
+            x_seq = self._ssa_kernel_hip(qkv, self.scale)
+        else:
+            x_seq = self._ssa_kernel_torch(qkv, self.scale)
+        x_seq = self.attn_lif(x_seq).reshape(T, N, local_dim, L)
+        return self.proj_lif(self.proj_conv_bn(x_seq))  # [T, N, C, L]
+
+    def extra_repr(self):
+        return f"dim={self.dim}, num_heads={self.num_heads}, backend={self.backend}"

@@ -209,6 +209,24 @@ int sjhip_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, void *
   return launch_bit_unpack(dtype, n, src, dst, static_cast<hipStream_t>(stream));
 }
 
+int sjhip_ssa_supported(int dtype, int channels_per_head, int64_t tokens) {
+  return ssa_supported(dtype, channels_per_head, tokens) ? 1 : 0;
+}
+
+int sjhip_ssa_forward(int dtype, int64_t samples, int heads, int channels_per_head, int64_t tokens, float scale,
+                      const void *qkv, void *out, void *stream) {
+  if (!qkv || !out) return fail(SJHIP_ERR_INVALID, "ssa_forward: NULL tensor");
+  return launch_ssa(false, dtype, samples, heads, channels_per_head, tokens, scale, qkv, nullptr, out, nullptr,
+                    static_cast<hipStream_t>(stream));
+}
+
+int sjhip_ssa_backward(int dtype, int64_t samples, int heads, int channels_per_head, int64_t tokens, float scale,
+                       const void *qkv, const void *grad_out, void *grad_qkv, void *stream) {
+  if (!qkv || !grad_out || !grad_qkv) return fail(SJHIP_ERR_INVALID, "ssa_backward: NULL tensor");
+  return launch_ssa(true, dtype, samples, heads, channels_per_head, tokens, scale, qkv, grad_out, nullptr, grad_qkv,
+                    static_cast<hipStream_t>(stream));
+}
+
 int sjhip_set_tuning(const char *key, int value) {
   if (!key) return fail(SJHIP_ERR_INVALID, "set_tuning: NULL key");
   const bool block_ok = (value == 64 || value == 128 || value == 256 || value == 512) && value <= SJHIP_MAX_BLOCK;

@@ -151,7 +151,8 @@ struct Tuning {
 unsigned occupancy_cap_lds(int blocks_per_cu);
 const Tuning &tuning();
 
-enum KernelClass { KC_FORWARD = 0, KC_BACKWARD = 1, KC_PLIF_REDUCE = 2, KC_BIT_PACK = 3, KC_BIT_UNPACK = 4, KC_COUNT = 5 };
+enum KernelClass { KC_FORWARD = 0, KC_BACKWARD = 1, KC_PLIF_REDUCE = 2, KC_BIT_PACK = 3, KC_BIT_UNPACK = 4,
+                   KC_SSA_FORWARD = 5, KC_SSA_BACKWARD = 6, KC_COUNT = 7 };
 
 // Brackets one launch with events when profiling is on; free otherwise.
 class ProfileScope {
@@ -183,6 +184,9 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
                               void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace,
                               hipStream_t stream);
 int64_t plif_blocks(int dtype, int64_t N);
+bool ssa_supported(int dtype, int cph, int64_t L);
+int launch_ssa(bool backward, int dtype, int64_t samples, int heads, int cph, int64_t L, float scale, const void *qkv,
+               const void *grad_out, void *out, void *grad_qkv, hipStream_t stream);
 int launch_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, hipStream_t stream);
 int launch_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, hipStream_t stream);
 

@@ -354,3 +354,29 @@ def test_bitpack_nonzero_semantics(c_oracle):
         t = torch.from_numpy(vals).to(dt)
         e = np.packbits(t.to(torch.bool).numpy().astype(np.uint8), bitorder="little")
         assert np.array_equal(c_oracle.bit_pack(t.view(torch.int16).numpy()), e)
+
+
+# ------------------------------------------------------------------------------------------------
+# 7. spiking self-attention contraction
+# ------------------------------------------------------------------------------------------------
+def test_ssa_oracle_is_exact_and_associative():
+    """(V K^T) Q == V (K^T Q) in integers; all-ones input has the closed form scale * L * Cph; the float
+    restatement equals the integer one because every partial sum is an integer below 2^24."""
+    from oracle import ssa_oracle
+
+    g = torch.Generator().manual_seed(3)
+    qkv = (torch.rand((5, 3, 4, 32, 50), generator=g) < 0.3).float()
+    exact = ssa_oracle.ssa_exact(qkv, 0.125)
+    q, k, v = (qkv[:, i].to(torch.int64) for i in range(3))
+    other_order = (v @ (k.transpose(-2, -1) @ q)).double() * 0.125
+    assert torch.equal(exact, other_order)
+    assert torch.equal(ssa_oracle.ssa(qkv, 0.125).double(), exact)
+    ones = torch.ones(1, 3, 2, 8, 11)
+    assert torch.equal(ssa_oracle.ssa_exact(ones, 0.125), torch.full((1, 2, 8, 11), 0.125 * 11 * 8, dtype=torch.float64))
+    # a single spike in v[c1, l0], k[c2, l0], q[c2, l1] lights out[c1, l1] only
+    one = torch.zeros(1, 3, 1, 4, 6)
+    one[0, 2, 0, 1, 3] = 1  # v
+    one[0, 1, 0, 2, 3] = 1  # k
+    one[0, 0, 0, 2, 5] = 1  # q
+    out = ssa_oracle.ssa_exact(one, 1.0)
+    assert out[0, 0, 1, 5] == 1 and out.sum() == 1
