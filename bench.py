@@ -56,6 +56,149 @@ def cpu_baseline(torch, sample_neurons: int, repeats: int):
     }
 
 
+def _time_steps(torch, L, step, steps, warmup):
+    """warm-up, then `steps` timed steps bracketed by synchronisation; library event profiler on."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    L.profile_reset()
+    L.profile_enable(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    L.profile_enable(False)
+    return elapsed
+
+
+def _kernel_ms(L, which):
+    n, ms = L.profile_read(which)
+    return ms / max(n, 1)
+
+
+def _emit(args, metric, unit, value, elapsed, dtype, config, roofline):
+    print(json.dumps({
+        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic", "config": config, "roofline": roofline}))
+
+
+def other_workload(args) -> int:
+    """Secondary workloads (BASELINE configs 3-5), same JSON shape; parity for them lives in tests/."""
+    import torch
+
+    from spikingjelly_amd import configure
+    from spikingjelly_amd.activation_based import functional, layer, neuron, surrogate
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+    from spikingjelly_amd.activation_based.hip_kernel.compress import bit_spike_compress, bit_spike_decompress
+
+    L.load()
+    dev = torch.device("cuda:0")
+
+    def randn(shape, seed, mean, std, dtype):
+        g = torch.Generator().manual_seed(seed)
+        return (torch.randn(shape, generator=g) * std + mean).to(dtype).to(dev)
+
+    if args.workload == "config3":
+        shape = (8, 128, 256, 16, 16)
+        T, N = shape[0], 128 * 256 * 16 * 16
+        configure.hip_half_precision_mode = "fp32_state"
+        x = randn(shape, 1003, 0.2, 1.0, torch.bfloat16).requires_grad_()
+        gs = randn(shape, 1103, 0.0, 1.0, torch.bfloat16)
+        gv = randn(shape, 1203, 0.0, 0.1, torch.bfloat16)
+        node = neuron.ParametricLIFNode(init_tau=2.0, v_reset=None, surrogate_function=surrogate.Sigmoid(4.0),
+                                        step_mode="m", backend="hip", store_v_seq=True).to(dev)
+
+        def step():
+            s = node(x)
+            torch.autograd.backward([s, node.v_seq], [gs, gv])
+            x.grad = None
+            node.w.grad = None
+            functional.reset_net(node)
+
+        elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
+        f_ms, b_ms = _kernel_ms(L, L.KC_FORWARD), _kernel_ms(L, L.KC_BACKWARD)
+        bytes_each = 8 * T * N + 2 * N  # 4 tensors x 2 B per step + one [N] state
+        dom = "forward" if f_ms >= b_ms else "backward"
+        d_ms = max(f_ms, b_ms)
+        _emit(args, "neuron-steps/sec PLIF fwd+bwd bf16 storage / fp32 state, T=8 N=8.4M, 1 MI355X", "neuron-steps/s",
+              T * N / (elapsed / args.steps), elapsed, "f32",
+              {"workload": "configs[2]: ParametricLIFNode init_tau=2, soft reset, Sigmoid(4), x [8,128,256,16,16] bf16, "
+                           "store_v_seq=True, incl. dL/dw reduction", "T": T, "N": N},
+              {"bound": "hbm", "achieved": bytes_each / (d_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+               "frac": bytes_each / (d_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": dom,
+               "kernel_ms": d_ms, "algorithmic_bytes": bytes_each, "forward_ms": f_ms, "backward_ms": b_ms,
+               "plif_reduce_ms": _kernel_ms(L, L.KC_PLIF_REDUCE)})
+        return 0
+
+    if args.workload == "config4":
+        shape = (32, 64, 512, 14, 14)
+        T, N = shape[0], 64 * 512 * 14 * 14
+        g = torch.Generator().manual_seed(1004)
+        x = (torch.rand(shape, generator=g) * 0.25).half().to(dev)
+        node = neuron.IFNode(v_threshold=1.0, v_reset=None, step_mode="m", backend="hip").to(dev).eval()
+
+        def step():
+            with torch.no_grad():
+                s = node(x)
+                packed = bit_spike_compress(s)
+                back = bit_spike_decompress(packed, s.shape, dtype=torch.float16)
+            functional.reset_net(node)
+            return s, back
+
+        elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
+        s, back = step()
+        assert torch.equal(s, back)
+        f_ms, p_ms, u_ms = _kernel_ms(L, L.KC_FORWARD), _kernel_ms(L, L.KC_BIT_PACK), _kernel_ms(L, L.KC_BIT_UNPACK)
+        n = T * N
+        fwd_bytes, pack_bytes, unpack_bytes = 4 * n + 4 * N, 2 * n + n // 8, n // 8 + 2 * n
+        _emit(args, "neuron-steps/sec IF inference fp16 + spike bit-pack/unpack, T=32 N=6.4M, 1 MI355X", "neuron-steps/s",
+              n / (elapsed / args.steps), elapsed, "f16",
+              {"workload": "configs[3]: IFNode soft reset eval, x [32,64,512,14,14] fp16 uniform[0,0.25), then "
+                           "bit_spike_compress + bit_spike_decompress(fp16)", "T": T, "N": N,
+               "firing_rate": float(s.float().mean())},
+              {"bound": "hbm", "achieved": fwd_bytes / (f_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+               "frac": fwd_bytes / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "forward(inference)",
+               "kernel_ms": f_ms, "algorithmic_bytes": fwd_bytes,
+               "pack_ms": p_ms, "pack_GBs": pack_bytes / (p_ms * 1e-3) / 1e9,
+               "unpack_ms": u_ms, "unpack_GBs": unpack_bytes / (u_ms * 1e-3) / 1e9})
+        return 0
+
+    if args.workload == "config5":
+        T, B, D, H, tokens = 4, 64, 384, 12, 196
+        torch.manual_seed(1005)
+        block = layer.SpikingSelfAttention(D, H, backend="hip").to(dev)
+        x = randn((T, B, D, tokens), 1105, 0.0, 1.0, torch.float32).requires_grad_()
+        g = randn((T, B, D, tokens), 1205, 0.0, 1.0, torch.float32)
+
+        def step():
+            y = block(x)
+            y.backward(g)
+            x.grad = None
+            block.zero_grad(set_to_none=True)
+            functional.reset_net(block)
+
+        elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
+        sf, sb = _kernel_ms(L, L.KC_SSA_FORWARD), _kernel_ms(L, L.KC_SSA_BACKWARD)
+        cph = D // H
+        probs = T * B * H
+        flops_f = probs * (2 * cph * cph * tokens + 2 * cph * cph * tokens)
+        bytes_f = T * B * D * tokens * 4 * (3 + 1)  # qkv read + out write, fp32 storage
+        _emit(args, "tokens/sec spiking self-attention block fwd+bwd, T=4 B=64 N=196 D=384 12 heads, 1 MI355X",
+              "tokens/s", T * B * tokens / (elapsed / args.steps), elapsed, "bf16",
+              {"workload": "configs[4]: SpikingSelfAttention(384, 12, backend='hip'), x [4,64,384,196] fp32 ~N(0,1), "
+                           "channels per head = 32 (dim // heads, as the reference computes it)"},
+              {"bound": "hbm", "achieved": bytes_f / (sf * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+               "frac": bytes_f / (sf * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "ssa_forward",
+               "kernel_ms": sf, "algorithmic_bytes": bytes_f, "ssa_forward_TFLOPs": flops_f / (sf * 1e-3) / 1e12,
+               "ssa_backward_ms": sb, "lif_forward_ms": _kernel_ms(L, L.KC_FORWARD),
+               "lif_backward_ms": _kernel_ms(L, L.KC_BACKWARD)})
+        return 0
+    raise SystemExit(f"unknown workload {args.workload}")
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -64,6 +207,8 @@ def main() -> int:
     ap.add_argument("--cpu-sample-neurons", type=int, default=1 << 23)
     ap.add_argument("--cpu-repeats", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5"],
+                    help="config2 (default) is the headline metric; the others are secondary measurements")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path shards over neurons with no exchange, and this build runs "
@@ -79,6 +224,8 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm device", file=sys.stderr)
         return 2
+    if args.workload != "config2":
+        return other_workload(args)
     dev = torch.device("cuda:0")
     N = 1
     for d in SHAPE[1:]:
