@@ -3,22 +3,31 @@
 // Layout and order follow the reference (layer/attention.py:346-353, `_ssa_kernel_torch`): qkv is
 // [TB, 3, H, Cph, L] (q, k, v of one sample stacked on dim 1; each head a row-major [Cph, L] tile of
 // binary spikes), S = V K^T is [Cph, Cph] (contraction over the L tokens), out = scale * S Q is
-// [TB, H, Cph, L].  One wavefront owns one (sample, head) problem:
-//   * the three tiles are staged once through LDS as bf16 (0/1 are exact), rows padded with zeros;
-//   * S = V K^T runs on v_mfma_f32_32x32x16_bf16, fp32 accumulation -- exact integers <= L;
-//   * S goes through LDS (accumulator layout -> operand layout) as bf16, exact because L <= 256;
-//   * out = S Q on the same bf16 MFMA; sums are integers <= Cph * L < 2^24, so the fp32 result is the
-//     exact integer and `scale` (a power of two in the reference, 0.125) is applied once.
+// [TB, H, Cph, L].  The work is HBM-bound (about 8 flop per byte), so the kernels are built as streaming
+// kernels whose arithmetic happens to run on the matrix cores:
+//
+//   * one block of four wavefronts owns one (sample, head) problem; each [Cph, L] tile is one contiguous
+//     run in memory and is fetched with 16-byte accesses, all loads of a pass issued before any is used;
+//   * spikes are parked in LDS as one byte each (0 / 1), so the three tiles of a head take 21 KB for
+//     Cph = 32, L = 196 and several blocks are resident per compute unit to overlap load, MFMA and store;
+//   * S = V K^T runs on v_mfma_i32_32x32x32_i8: exact integers <= L;
+//   * S never goes through LDS: it is produced transposed (K V^T), and in the accumulator layout lane
+//     (c1, half) already holds S[c1, c2] for the sixteen c2 = 8 (r / 4) + 4 half + r % 4, which is a valid
+//     A operand of the second product as long as the B operand (Q) is gathered with the same k order;
+//   * out = S Q on v_mfma_f32_32x32x16_bf16 (S <= 256 and spikes are exact in bf16, fp32 accumulation of
+//     integers < 2^24), `scale` (a power of two in the reference, 0.125) is applied once.
 // Hence the forward equals an int64 matmul of the spikes times scale, bit for bit, in fp32 output,
 // and after one rounding in 16-bit output (what torch's bf16 matmuls also produce).
 //
-// The backward has real-valued operands (grad_out, dS), so it uses the fp32 MFMA
-// (v_mfma_f32_32x32x2_f32): dS = scale * dO Q^T, dQ = scale * S^T dO, dV = dS K, dK = dS^T V,
-// with S recomputed on the bf16 MFMA as in the forward.
+// The backward has real-valued operands (grad_out, dS), so those products use the fp32 MFMA:
+//   dS = scale * dO Q^T  (v_mfma_f32_16x16x4_f32, one 16x16 block per wavefront, through LDS),
+//   dQ = scale * S^T dO,  dK = dS^T V,  dV = dS K  (v_mfma_f32_32x32x2_f32, column tiles dealt to wavefronts),
+// with S recomputed on the int8 MFMA where it is needed and kept in registers.
 //
-// The k index of both MFMA operands uses the same lane -> k mapping, so only the row/column mapping of
-// the operands and the accumulator layout (row = 8*(r/4) + 4*(lane/32) + r%4, col = lane%32 for
-// accumulator register r) matter.
+// MFMA layouts used (lane = 0..63):  32x32: A element of lane is row lane % 32, k group lane / 32; B likewise
+// with column lane % 32; accumulator register r sits at row 8 (r / 4) + 4 (lane / 32) + r % 4, column
+// lane % 32.  16x16x4: A row lane % 16, k = lane / 16; accumulator register r at row 4 (lane / 16) + r,
+// column lane % 16.  Which k a lane's operand element stands for is free as long as A and B agree.
 #include "sjhip_common.h"
 
 #include <mutex>
@@ -28,10 +37,14 @@ namespace sjhip {
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
 
 constexpr unsigned kSsaMaxLds = 159u * 1024u;
+constexpr int kSsaThreads = 256;
+constexpr int kSsaWaves = kSsaThreads / 64;
 
 struct SsaArgs {
   const void *qkv;
@@ -42,220 +55,290 @@ struct SsaArgs {
   int heads;
   int cph;    // channels per head (<= 64); tiles are zero-padded to 32 or 64 rows in LDS
   int L;      // tokens
-  int Lp;     // LDS row stride (elements) of the bf16 tiles
+  int Lb;     // LDS row stride (bytes) of the spike tiles = L rounded up to 32
   int Lq;     // LDS row stride (floats) of the grad_out tile
+  int vec;    // tiles may be fetched four elements at a time (L % 4 == 0 and aligned bases)
   float scale;
 };
 
+// Four consecutive elements of a tile, as fetched; and single elements for ragged shapes.
 template <typename S> struct Io;
 template <> struct Io<float> {
   typedef float elem_t;
+  typedef f32x4 quad_t;
   static __device__ __forceinline__ float get(const elem_t *p, int64_t i) { return p[i]; }
   static __device__ __forceinline__ void put(elem_t *p, int64_t i, float v) { p[i] = v; }
+  static __device__ __forceinline__ void unpack(quad_t q, float (&f)[4]) { f[0] = q.x; f[1] = q.y; f[2] = q.z; f[3] = q.w; }
 };
-template <> struct Io<f16_t> {
+template <typename H> struct Io16 {
   typedef uint16_t elem_t;
-  static __device__ __forceinline__ float get(const elem_t *p, int64_t i) { return Cvt<f16_t>::to_float(p[i]); }
-  static __device__ __forceinline__ void put(elem_t *p, int64_t i, float v) { p[i] = Cvt<f16_t>::from_float(v); }
+  typedef u32x2 quad_t;
+  static __device__ __forceinline__ float get(const elem_t *p, int64_t i) { return Cvt<H>::to_float(p[i]); }
+  static __device__ __forceinline__ void put(elem_t *p, int64_t i, float v) { p[i] = Cvt<H>::from_float(v); }
+  static __device__ __forceinline__ void unpack(quad_t q, float (&f)[4]) {
+    f[0] = Cvt<H>::to_float((uint16_t)(q.x & 0xffffu)); f[1] = Cvt<H>::to_float((uint16_t)(q.x >> 16));
+    f[2] = Cvt<H>::to_float((uint16_t)(q.y & 0xffffu)); f[3] = Cvt<H>::to_float((uint16_t)(q.y >> 16));
+  }
 };
-template <> struct Io<bf16_t> {
-  typedef uint16_t elem_t;
-  static __device__ __forceinline__ float get(const elem_t *p, int64_t i) { return Cvt<bf16_t>::to_float(p[i]); }
-  static __device__ __forceinline__ void put(elem_t *p, int64_t i, float v) { p[i] = Cvt<bf16_t>::from_float(v); }
-};
+template <> struct Io<f16_t> : Io16<f16_t> {};
+template <> struct Io<bf16_t> : Io16<bf16_t> {};
 
-__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+__device__ __forceinline__ uint32_t spike_bytes(const float (&f)[4]) {
+  return (f[0] != 0.0f ? 1u : 0u) | (f[1] != 0.0f ? 0x100u : 0u) | (f[2] != 0.0f ? 0x10000u : 0u) |
+         (f[3] != 0.0f ? 0x1000000u : 0u);
+}
 
-// global [rows, L] tile -> LDS bf16 [rows][Lp], columns L..Lp-1 zeroed
-template <typename S>
-__device__ __forceinline__ void stage_bf16(const typename Io<S>::elem_t *src, uint16_t *dst, int rows, int rows_pad,
-                                           int L, int Lp) {
-  const int lane = threadIdx.x;
-  for (int idx = lane; idx < rows_pad * Lp; idx += 64) {
-    const int r = idx / Lp, c = idx - r * Lp;
-    dst[idx] = (c < L && r < rows) ? Cvt<bf16_t>::from_float(Io<S>::get(src, (int64_t)r * L + c)) : (uint16_t)0;
+// Global tiles -> LDS.  NS spike tiles ([cph, L] each) become
+// byte tiles [rows_pad][Lb]; when DO is set the grad_out tile becomes an fp32 tile [rows_pad][Lq].  Rows
+// cph..rows_pad-1 and the columns from L to the row stride are zero-filled, by writes that never overlap the
+// data writes, so one barrier after this function is enough.
+template <typename S, int NS, bool DO, int UN>
+__device__ __forceinline__ void stage_tiles(const typename Io<S>::elem_t *const (&src)[NS], uint8_t *const (&dst)[NS],
+                                            const typename Io<S>::elem_t *do_src, float *do_dst, int cph, int rows_pad,
+                                            int L, int Lb, int Lq, bool vec) {
+  typedef typename Io<S>::quad_t Q;
+  const int tid = threadIdx.x;
+  if (vec) {
+    const int G = cph * L / 4;
+    for (int g0 = tid; g0 < G; g0 += kSsaThreads * UN) {
+      Q buf[UN][NS + (DO ? 1 : 0)];
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int g = g0 + u * kSsaThreads;
+        if (g < G) {
+#pragma unroll
+          for (int s = 0; s < NS; ++s) buf[u][s] = reinterpret_cast<const Q *>(src[s])[g];
+          if (DO) buf[u][NS] = reinterpret_cast<const Q *>(do_src)[g];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int g = g0 + u * kSsaThreads;
+        if (g < G) {
+          const int r = (4 * g) / L, c = 4 * g - r * L;
+          float f[4];
+#pragma unroll
+          for (int s = 0; s < NS; ++s) {
+            Io<S>::unpack(buf[u][s], f);
+            *reinterpret_cast<uint32_t *>(dst[s] + r * Lb + c) = spike_bytes(f);
+          }
+          if (DO) {
+            Io<S>::unpack(buf[u][NS], f);
+            f32x4 w; w.x = f[0]; w.y = f[1]; w.z = f[2]; w.w = f[3];
+            *reinterpret_cast<f32x4 *>(do_dst + r * Lq + c) = w;
+          }
+        }
+      }
+    }
+  } else {
+    const int n = cph * L;
+    for (int i = tid; i < n; i += kSsaThreads) {
+      const int r = i / L, c = i - r * L;
+#pragma unroll
+      for (int s = 0; s < NS; ++s) dst[s][r * Lb + c] = Io<S>::get(src[s], i) != 0.0f ? 1 : 0;
+      if (DO) do_dst[r * Lq + c] = Io<S>::get(do_src, i);
+    }
+  }
+  // zero fill: right margin of the data rows, then the rows below them
+  const int mb = Lb - L;
+  for (int i = tid; i < cph * mb; i += kSsaThreads) {
+    const int r = i / mb, c = L + (i - r * mb);
+#pragma unroll
+    for (int s = 0; s < NS; ++s) dst[s][r * Lb + c] = 0;
+  }
+  for (int i = tid; i < (rows_pad - cph) * (Lb / 4); i += kSsaThreads) {
+#pragma unroll
+    for (int s = 0; s < NS; ++s) reinterpret_cast<uint32_t *>(dst[s] + cph * Lb)[i] = 0u;
+  }
+  if (DO) {
+    const int mq = Lq - L;
+    for (int i = tid; i < cph * mq; i += kSsaThreads) {
+      const int r = i / mq, c = L + (i - r * mq);
+      do_dst[r * Lq + c] = 0.0f;
+    }
+    for (int i = tid; i < (rows_pad - cph) * Lq; i += kSsaThreads) do_dst[cph * Lq + i] = 0.0f;
   }
 }
 
-// global [rows, L] tile -> LDS fp32 [rows][Lq], padded with zeros
-template <typename S>
-__device__ __forceinline__ void stage_f32(const typename Io<S>::elem_t *src, float *dst, int rows, int rows_pad, int L,
-                                          int Lq) {
-  const int lane = threadIdx.x;
-  for (int idx = lane; idx < rows_pad * Lq; idx += 64) {
-    const int r = idx / Lq, c = idx - r * Lq;
-    dst[idx] = (c < L && r < rows) ? Io<S>::get(src, (int64_t)r * L + c) : 0.0f;
-  }
-}
-
-// S block (mi, ni) = V[mi*32.., :] K[ni*32.., :]^T over the padded token axis, bf16 MFMA
-__device__ __forceinline__ f32x16 gemm_vkt(const uint16_t *v_lds, const uint16_t *k_lds, int mi, int ni, int Lp, int Lk) {
-  const int lane = threadIdx.x;
-  const uint16_t *ap = v_lds + (mi * 32 + (lane & 31)) * Lp + 8 * (lane >> 5);
-  const uint16_t *bp = k_lds + (ni * 32 + (lane & 31)) * Lp + 8 * (lane >> 5);
-  f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  for (int k0 = 0; k0 < Lk; k0 += 16) {
-    const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u16x8 *>(ap + k0));
-    const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u16x8 *>(bp + k0));
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
-  }
+// 32x32 block of  A_rows B_rows^T  over the token axis: rows ra.. of tile `a` against rows rb.. of tile `b`
+__device__ __forceinline__ i32x16 spike_gram(const uint8_t *a, int ra, const uint8_t *b, int rb, int Lb, int lane) {
+  const uint8_t *ap = a + (ra + (lane & 31)) * Lb + 16 * (lane >> 5);
+  const uint8_t *bp = b + (rb + (lane & 31)) * Lb + 16 * (lane >> 5);
+  i32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = 0; k0 < Lb; k0 += 32)
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const i32x4 *>(ap + k0),
+                                                *reinterpret_cast<const i32x4 *>(bp + k0), acc, 0, 0, 0);
   return acc;
 }
 
 // accumulator register r of this lane sits at (row, col) of its 32x32 block
-__device__ __forceinline__ int acc_row(int r) { return 8 * (r >> 2) + 4 * ((int)threadIdx.x >> 5) + (r & 3); }
-__device__ __forceinline__ int acc_col() { return (int)threadIdx.x & 31; }
+__device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
 
 template <typename S, int MC>
-__global__ void __launch_bounds__(64) ssa_forward_kernel(const SsaArgs a) {
+__global__ void __launch_bounds__(kSsaThreads) ssa_forward_kernel(const SsaArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char ssa_lds[];
   typedef typename Io<S>::elem_t E;
   constexpr int CPH = 32 * MC;
-  const int L = a.L, Lp = a.Lp;
-  const int Lk = (L + 15) & ~15;
-  constexpr int LS = CPH + 8;  // row stride of the bf16 S tile
-  uint16_t *q_lds = reinterpret_cast<uint16_t *>(ssa_lds);
-  uint16_t *k_lds = q_lds + CPH * Lp;
-  uint16_t *v_lds = k_lds + CPH * Lp;
-  uint16_t *s_lds = v_lds + CPH * Lp;
+  const int L = a.L, Lb = a.Lb, cph = a.cph;
+  uint8_t *q_lds = ssa_lds;
+  uint8_t *k_lds = q_lds + CPH * Lb;
+  uint8_t *v_lds = k_lds + CPH * Lb;
 
   const int64_t p = blockIdx.x;
   const int64_t sample = p / a.heads, head = p - sample * a.heads;
-  const int cph = a.cph;
   const int64_t tile = (int64_t)cph * L;
   const E *qkv = static_cast<const E *>(a.qkv);
-  const E *qg = qkv + ((sample * 3 + 0) * a.heads + head) * tile;
-  const E *kg = qkv + ((sample * 3 + 1) * a.heads + head) * tile;
-  const E *vg = qkv + ((sample * 3 + 2) * a.heads + head) * tile;
-  stage_bf16<S>(qg, q_lds, cph, CPH, L, Lp);
-  stage_bf16<S>(kg, k_lds, cph, CPH, L, Lp);
-  stage_bf16<S>(vg, v_lds, cph, CPH, L, Lp);
+  {
+    const E *const src[3] = {qkv + ((sample * 3 + 0) * a.heads + head) * tile,
+                             qkv + ((sample * 3 + 1) * a.heads + head) * tile,
+                             qkv + ((sample * 3 + 2) * a.heads + head) * tile};
+    uint8_t *const dst[3] = {q_lds, k_lds, v_lds};
+    stage_tiles<S, 3, false, 4>(src, dst, nullptr, nullptr, cph, CPH, L, Lb, 0, a.vec != 0);
+  }
   __syncthreads();
 
-  // S = V K^T, exact integers <= L <= 256 -> bf16 in LDS, operand layout for the second product
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, half = lane >> 5;
+  const int ntiles = (L + 31) / 32;
+  const int units = ntiles * MC;  // unit u: output rows 32 (u % MC).., columns 32 (u / MC)..
+  if (wave >= units) return;
+  const int ni = wave % MC;  // the same for every unit of this wavefront because MC divides the wavefront count
+
+  // S^T blocks (K V^T): lane (c1, half) register r holds S[32 ni + c1, 32 mi + 8 (r/4) + 4 half + r%4]
+  bf16x8 s_op[MC][2];
 #pragma unroll
   for (int mi = 0; mi < MC; ++mi) {
+    const i32x16 acc = spike_gram(k_lds, mi * 32, v_lds, ni * 32, Lb, lane);
 #pragma unroll
-    for (int ni = 0; ni < MC; ++ni) {
-      const f32x16 acc = gemm_vkt(v_lds, k_lds, mi, ni, Lp, Lk);
+    for (int h = 0; h < 2; ++h) {
+      uint16_t w[8];
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        s_lds[(mi * 32 + acc_row(r)) * LS + ni * 32 + acc_col()] = Cvt<bf16_t>::from_float(acc[r]);
+      for (int e = 0; e < 8; ++e) w[e] = (uint16_t)(__builtin_bit_cast(uint32_t, (float)acc[8 * h + e]) >> 16);  // exact: <= 256
+      s_op[mi][h] = __builtin_bit_cast(bf16x8, w);
     }
   }
-  __syncthreads();
 
-  // out[c1, l] = scale * sum_c2 S[c1, c2] Q[c2, l]
-  const int lane = threadIdx.x;
   E *og = static_cast<E *>(a.out) + p * tile;
-  const int ntiles = (L + 31) / 32;
-  for (int nt = 0; nt < ntiles; ++nt) {
+  for (int u = wave; u < units; u += kSsaWaves) {
+    const int nt = u / MC;
+    const int col = nt * 32 + (lane & 31);
+    const int colc = col < L ? col : L - 1;
+    f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int mi = 0; mi < MC; ++mi) {
-      f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-      for (int k0 = 0; k0 < CPH; k0 += 16) {
-        const bf16x8 av = __builtin_bit_cast(
-            bf16x8, *reinterpret_cast<const u16x8 *>(s_lds + (mi * 32 + (lane & 31)) * LS + k0 + 8 * (lane >> 5)));
-        u16x8 bw;
+      for (int h = 0; h < 2; ++h) {
+        uint16_t w[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) bw[j] = q_lds[(k0 + 8 * (lane >> 5) + j) * Lp + nt * 32 + (lane & 31)];
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(bf16x8, bw), acc, 0, 0, 0);
-      }
-      const int col = nt * 32 + acc_col();
-      if (col < L) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = mi * 32 + acc_row(r);
-          if (row < cph) Io<S>::put(og, (int64_t)row * L + col, acc[r] * a.scale);
+        for (int e = 0; e < 8; ++e) {
+          const int c2 = mi * 32 + 16 * h + 8 * (e >> 2) + 4 * half + (e & 3);
+          w[e] = (uint16_t)(q_lds[c2 * Lb + colc] * 0x3f80u);  // 1 -> bf16 1.0
         }
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s_op[mi][h], __builtin_bit_cast(bf16x8, w), acc, 0, 0, 0);
+      }
+    }
+    if (col < L) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = ni * 32 + acc_row(r, lane);
+        if (row < cph) Io<S>::put(og, (int64_t)row * L + col, acc[r] * a.scale);
       }
     }
   }
-}
-
-// D[m, n] (+)= sum_k A(m, k) B(k, n) on the fp32 MFMA, K stepping by 2; fa(m, k) / fb(k, n) fetch operands
-template <typename FA, typename FB>
-__device__ __forceinline__ f32x16 gemm_f32(int K, FA fa, FB fb) {
-  const int lane = threadIdx.x;
-  const int mn = lane & 31, kh = lane >> 5;
-  f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  for (int k0 = 0; k0 < K; k0 += 2) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa(mn, k0 + kh), fb(k0 + kh, mn), acc, 0, 0, 0);
-  return acc;
 }
 
 template <typename S, int MC>
-__global__ void __launch_bounds__(64) ssa_backward_kernel(const SsaArgs a) {
+__global__ void __launch_bounds__(kSsaThreads) ssa_backward_kernel(const SsaArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char ssa_lds[];
   typedef typename Io<S>::elem_t E;
   constexpr int CPH = 32 * MC;
-  constexpr int LS = CPH + 1;  // row stride of the fp32 S / dS tiles
-  const int L = a.L, Lp = a.Lp, Lq = a.Lq;
-  const int Lk = (L + 15) & ~15;
-  const int L2 = (L + 1) & ~1;
+  constexpr int LS = CPH + 1;  // row stride of the fp32 dS tile
+  const int L = a.L, Lb = a.Lb, Lq = a.Lq, cph = a.cph;
   float *do_lds = reinterpret_cast<float *>(ssa_lds);
-  float *s_lds = do_lds + CPH * Lq;
-  float *ds_lds = s_lds + CPH * LS;
-  uint16_t *q_lds = reinterpret_cast<uint16_t *>(ds_lds + CPH * LS);
-  uint16_t *k_lds = q_lds + CPH * Lp;
-  uint16_t *v_lds = k_lds + CPH * Lp;
+  float *ds_lds = do_lds + CPH * Lq;
+  uint8_t *q_lds = reinterpret_cast<uint8_t *>(ds_lds + CPH * LS);  // CPH * LS * 4 is a multiple of 16
+  uint8_t *k_lds = q_lds + CPH * Lb;
+  uint8_t *v_lds = k_lds + CPH * Lb;
 
   const int64_t p = blockIdx.x;
   const int64_t sample = p / a.heads, head = p - sample * a.heads;
-  const int cph = a.cph;
   const int64_t tile = (int64_t)cph * L;
   const E *qkv = static_cast<const E *>(a.qkv);
   const int64_t qoff = ((sample * 3 + 0) * a.heads + head) * tile;
   const int64_t koff = ((sample * 3 + 1) * a.heads + head) * tile;
   const int64_t voff = ((sample * 3 + 2) * a.heads + head) * tile;
-  stage_bf16<S>(qkv + qoff, q_lds, cph, CPH, L, Lp);
-  stage_bf16<S>(qkv + koff, k_lds, cph, CPH, L, Lp);
-  stage_bf16<S>(qkv + voff, v_lds, cph, CPH, L, Lp);
-  stage_f32<S>(static_cast<const E *>(a.grad_out) + p * tile, do_lds, cph, CPH, L, Lq);
+  {
+    const E *const src[3] = {qkv + qoff, qkv + koff, qkv + voff};
+    uint8_t *const dst[3] = {q_lds, k_lds, v_lds};
+    stage_tiles<S, 3, true, 2>(src, dst, static_cast<const E *>(a.grad_out) + p * tile, do_lds, cph, CPH, L, Lb, Lq,
+                               a.vec != 0);
+  }
   __syncthreads();
 
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, half = lane >> 5;
   const float scale = a.scale;
-  // S = V K^T (exact) and dS = scale * dO Q^T, both [CPH, CPH], into LDS
-#pragma unroll
-  for (int mi = 0; mi < MC; ++mi) {
-#pragma unroll
-    for (int ni = 0; ni < MC; ++ni) {
-      const f32x16 s_acc = gemm_vkt(v_lds, k_lds, mi, ni, Lp, Lk);
-      const f32x16 ds_acc = gemm_f32(
-          L2, [&](int m, int k) { return do_lds[(mi * 32 + m) * Lq + k]; },
-          [&](int k, int n) { return bf16_bits_to_float(q_lds[(ni * 32 + n) * Lp + k]); });
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int idx = (mi * 32 + acc_row(r)) * LS + ni * 32 + acc_col();
-        s_lds[idx] = s_acc[r];
-        ds_lds[idx] = ds_acc[r] * scale;
+
+  // dS = scale * dO Q^T, one 16x16 block per wavefront and pass, into LDS
+  {
+    constexpr int NB = CPH / 16;
+    const int Lk = (L + 15) & ~15;
+    const int i16 = lane & 15, kq = lane >> 4;
+    for (int sb = wave; sb < NB * NB; sb += kSsaWaves) {
+      const int bi = sb / NB, bj = sb - bi * NB;
+      const float *ap = do_lds + (16 * bi + i16) * Lq + 4 * kq;
+      const uint8_t *bp = q_lds + (16 * bj + i16) * Lb + 4 * kq;
+      f32x4 acc = {0, 0, 0, 0};
+      for (int k0 = 0; k0 < Lk; k0 += 16) {
+        const f32x4 av = *reinterpret_cast<const f32x4 *>(ap + k0);
+        const uint32_t bw = *reinterpret_cast<const uint32_t *>(bp + k0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, (float)(bw & 0xffu), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, (float)((bw >> 8) & 0xffu), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, (float)((bw >> 16) & 0xffu), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, (float)(bw >> 24), acc, 0, 0, 0);
       }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) ds_lds[(16 * bi + 4 * kq + r) * LS + 16 * bj + i16] = acc[r] * scale;
     }
   }
+
   __syncthreads();
 
   E *gq = static_cast<E *>(a.grad_qkv);
   const int ntiles = (L + 31) / 32;
-  for (int nt = 0; nt < ntiles; ++nt) {
-    const int col = nt * 32 + acc_col();
+  const int m32 = lane & 31;
+  for (int nt = wave; nt < ntiles; nt += kSsaWaves) {
+    const int col = nt * 32 + m32;
+    const int colc = col < L ? col : L - 1;
+#pragma unroll 1
+    for (int b = 0; b < MC; ++b) {
+      // S blocks (V K^T) of column block b, exact, in registers: lane (c2, half) register r of block ai holds
+      // S[32 ai + 8 (r/4) + 4 half + r%4, 32 b + c2]
+      float s_reg[MC][16];
 #pragma unroll
-    for (int mi = 0; mi < MC; ++mi) {
-      // dQ[c2, l] = scale * sum_c1 S[c1, c2] dO[c1, l]
-      const f32x16 dq = gemm_f32(
-          CPH, [&](int m, int k) { return s_lds[k * LS + mi * 32 + m]; },
-          [&](int k, int n) { return do_lds[k * Lq + nt * 32 + n]; });
-      // dV[c1, l] = sum_c2 dS[c1, c2] K[c2, l]
-      const f32x16 dv = gemm_f32(
-          CPH, [&](int m, int k) { return ds_lds[(mi * 32 + m) * LS + k]; },
-          [&](int k, int n) { return bf16_bits_to_float(k_lds[k * Lp + nt * 32 + n]); });
-      // dK[c2, l] = sum_c1 dS[c1, c2] V[c1, l]
-      const f32x16 dk = gemm_f32(
-          CPH, [&](int m, int k) { return ds_lds[k * LS + mi * 32 + m]; },
-          [&](int k, int n) { return bf16_bits_to_float(v_lds[k * Lp + nt * 32 + n]); });
+      for (int ai = 0; ai < MC; ++ai) {
+        const i32x16 acc = spike_gram(v_lds, ai * 32, k_lds, b * 32, Lb, lane);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s_reg[ai][r] = (float)acc[r];
+      }
+      f32x16 dq = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+      f32x16 dk = dq, dv = dq;
+#pragma unroll
+      for (int ai = 0; ai < MC; ++ai) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          // dQ[c2, l] += S[c1, c2] dO[c1, l], c1 in the order the S registers hold it
+          const int c1s = ai * 32 + acc_row(r, lane);
+          dq = __builtin_amdgcn_mfma_f32_32x32x2f32(s_reg[ai][r], do_lds[c1s * Lq + colc], dq, 0, 0, 0);
+          const int kk = ai * 32 + 2 * r + half;
+          // dK[c2, l] += dS[c1 = kk, c2] V[kk, l]
+          dk = __builtin_amdgcn_mfma_f32_32x32x2f32(ds_lds[kk * LS + b * 32 + m32], (float)v_lds[kk * Lb + colc], dk, 0, 0, 0);
+          // dV[c1, l] += dS[c1, c2 = kk] K[kk, l]
+          dv = __builtin_amdgcn_mfma_f32_32x32x2f32(ds_lds[(b * 32 + m32) * LS + kk], (float)k_lds[kk * Lb + colc], dv, 0, 0, 0);
+        }
+      }
       if (col < L) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int row = mi * 32 + acc_row(r);
+          const int row = b * 32 + acc_row(r, lane);
           if (row >= cph) continue;
           const int64_t o = (int64_t)row * L + col;
           Io<S>::put(gq, qoff + o, dq[r] * scale);
@@ -267,17 +350,14 @@ __global__ void __launch_bounds__(64) ssa_backward_kernel(const SsaArgs a) {
   }
 }
 
-int lds_row_bf16(int L) { return ((L + 31) & ~31) + 8; }
-int lds_row_f32(int L) { return ((L + 31) & ~31) + 4; }
+int lds_row_bytes(int L) { return (L + 31) & ~31; }
+int lds_row_f32(int L) { return ((L + 15) & ~15) + 4; }
 
 int padded_rows(int cph) { return cph <= 32 ? 32 : 64; }
-unsigned forward_lds(int cph, int L) {
-  const int c = padded_rows(cph);
-  return (unsigned)((3 * c * lds_row_bf16(L) + c * (c + 8)) * 2);
-}
+unsigned forward_lds(int cph, int L) { return (unsigned)(3 * padded_rows(cph) * lds_row_bytes(L)); }
 unsigned backward_lds(int cph, int L) {
   const int c = padded_rows(cph);
-  return (unsigned)(3 * c * lds_row_bf16(L) * 2 + (c * lds_row_f32(L) + 2 * c * (c + 1)) * 4);
+  return (unsigned)(3 * c * lds_row_bytes(L) + (c * lds_row_f32(L) + c * (c + 1)) * 4);
 }
 
 template <typename K>
@@ -290,7 +370,7 @@ int launch_with_lds(K kernel, const SsaArgs &a, unsigned lds, hipStream_t stream
   });
   if (lds > 64u * 1024u && attr_rc != hipSuccess)
     return fail(SJHIP_ERR_LAUNCH, "%s: cannot raise the dynamic LDS limit: %s", what, hipGetErrorString(attr_rc));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)a.problems), dim3(64), lds, stream, a);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)a.problems), dim3(kSsaThreads), lds, stream, a);
   return check_launch(what);
 }
 
@@ -332,7 +412,11 @@ int launch_ssa(bool backward, int dtype, int64_t samples, int heads, int cph, in
   SsaArgs a;
   a.qkv = qkv; a.grad_out = grad_out; a.out = out; a.grad_qkv = grad_qkv;
   a.problems = samples * heads; a.heads = heads; a.cph = cph; a.L = (int)L;
-  a.Lp = lds_row_bf16((int)L); a.Lq = lds_row_f32((int)L); a.scale = scale;
+  a.Lb = lds_row_bytes((int)L); a.Lq = lds_row_f32((int)L); a.scale = scale;
+  // four elements per access need every tile base on a four-element boundary
+  const uintptr_t quad = dtype == SJHIP_F32 ? 15u : 7u;
+  a.vec = (L % 4 == 0) && (reinterpret_cast<uintptr_t>(qkv) & quad) == 0 &&
+          (grad_out == nullptr || (reinterpret_cast<uintptr_t>(grad_out) & quad) == 0);
   ProfileScope prof(backward ? KC_SSA_BACKWARD : KC_SSA_FORWARD, stream);
   switch (dtype) {
     case SJHIP_F32: return launch_dtype<float>(a, backward, stream);
