@@ -26,6 +26,9 @@
 #ifndef SJHIP_BWD_PF
 #define SJHIP_BWD_PF 8
 #endif
+#ifndef SJHIP_BWD_PF16
+#define SJHIP_BWD_PF16 4
+#endif
 #ifndef SJHIP_BWD_NT
 #define SJHIP_BWD_NT 1
 #endif
@@ -56,10 +59,18 @@ struct BwdArgs {
   int atomic_reduce;
 };
 
-template <int SG> __device__ __forceinline__ float surrogate_grad(float x, float alpha) {
+// FAST (16-bit storage, where the result is rounded to 8 or 11 significant bits anyway) uses the hardware
+// exp2 / reciprocal approximations (about 1 ulp each) in place of the correctly rounded library exp and IEEE
+// division; fp32 storage keeps the latter.
+template <bool FAST> __device__ __forceinline__ float sg_exp(float x) { return FAST ? __expf(x) : expf(x); }
+template <bool FAST> __device__ __forceinline__ float sg_div(float a, float b) {
+  return FAST ? a * __builtin_amdgcn_rcpf(b) : a / b;
+}
+
+template <int SG, bool FAST> __device__ __forceinline__ float surrogate_grad(float x, float alpha) {
   if (SG == SJHIP_SG_SIGMOID) {
     // surrogate.py:769-771:  s = sigmoid(alpha x);  (1 - s) s alpha
-    float s = 1.0f / (1.0f + expf(-alpha * x));
+    float s = sg_div<FAST>(1.0f, 1.0f + sg_exp<FAST>(-alpha * x));
     return (1.0f - s) * s * alpha;
   } else if (SG == SJHIP_SG_ATAN) {
     // surrogate.py:1247-1250:  a = alpha/2;  a / (1 + (pi a x)^2)
@@ -72,19 +83,19 @@ template <int SG> __device__ __forceinline__ float surrogate_grad(float x, float
     return (ax > 1.0f / alpha) ? 0.0f : (alpha - alpha * alpha * ax);
   } else if (SG == SJHIP_SG_PIECEWISE_EXP) {
     // surrogate.py:595-596:  alpha/2 exp(-alpha |x|)
-    return 0.5f * alpha * expf(-alpha * fabsf(x));
+    return 0.5f * alpha * sg_exp<FAST>(-alpha * fabsf(x));
   } else if (SG == SJHIP_SG_SOFT_SIGN) {
     // surrogate.py:936-937:  1 / (2 alpha (1/alpha + |x|)^2)
     float d = 1.0f / alpha + fabsf(x);
-    return 1.0f / (2.0f * alpha * d * d);
+    return sg_div<FAST>(1.0f, 2.0f * alpha * d * d);
   } else if (SG == SJHIP_SG_SUPER_SPIKE) {
     // surrogate.py:1101-1102:  alpha / (|x| + 1)^2
     float d = fabsf(x) + 1.0f;
-    return alpha / (d * d);
+    return sg_div<FAST>(alpha, d * d);
   } else {
     // surrogate.py:1610-1613:  alpha/sqrt(pi) exp(-(alpha x)^2)
     float ax = x * alpha;
-    return 0.56418958354775628695f * alpha * expf(-(ax * ax));
+    return 0.56418958354775628695f * alpha * sg_exp<FAST>(-(ax * ax));
   }
 }
 
@@ -94,13 +105,14 @@ template <int SG> __device__ __forceinline__ float surrogate_grad(float x, float
 // First PF rows (t = T-1 downwards) of grad_spike and grad_v_seq, requested ahead of their use.
 template <typename S, bool VECTOR> struct BwdPrologue {
   typedef Acc<S, VECTOR, SJHIP_BWD_NT != 0> A;
-  typename A::raw_t gs[SJHIP_BWD_PF], gv[SJHIP_BWD_PF];
+  static constexpr int PF = sizeof(S) == 2 ? SJHIP_BWD_PF16 : SJHIP_BWD_PF;
+  typename A::raw_t gs[PF], gv[PF];
   __device__ __forceinline__ void load(const BwdArgs &a, int64_t col) {
     typedef typename A::elem_t E;
     const E *gsp = (const E *)a.grad_spike + col;
     const E *gvp = (const E *)a.grad_v_seq + col;
 #pragma unroll
-    for (int i = 0; i < SJHIP_BWD_PF; ++i) {
+    for (int i = 0; i < PF; ++i) {
       const int64_t t = a.T - 1 - i;
       gs[i] = (t >= 0) ? A::load(gsp + t * a.N) : A::zero();
       if (a.grad_v_seq) gv[i] = (t >= 0) ? A::load(gvp + t * a.N) : A::zero();
@@ -115,7 +127,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
   typedef Acc<S, VECTOR, SJHIP_BWD_NT != 0> A;
   typedef typename A::elem_t E;
   constexpr int V = A::V;
-  constexpr int PF = SJHIP_BWD_PF;
+  constexpr int PF = BwdPrologue<S, VECTOR>::PF;
 
   float acc_total = 0.0f;
   if (!active) return acc_total;
@@ -196,7 +208,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
 #pragma unroll
         for (int j = 0; j < V; ++j) {
           const float over = h[j] - v_th;
-          const float sg = surrogate_grad<SG>(over, alpha);
+          const float sg = surrogate_grad<SG, sizeof(S) == 2>(over, alpha);
           const float s = (over >= 0.0f) ? 1.0f : 0.0f;
           if (PLIF) {
             // v_t from h_t exactly as the forward wrote it

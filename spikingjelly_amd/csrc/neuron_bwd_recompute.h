@@ -17,6 +17,9 @@
 #ifndef SJHIP_REPLAY_PF
 #define SJHIP_REPLAY_PF 8
 #endif
+#ifndef SJHIP_REPLAY_PF16
+#define SJHIP_REPLAY_PF16 4
+#endif
 
 namespace sjhip {
 
@@ -26,7 +29,7 @@ __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, i
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
-  constexpr int PF = SJHIP_REPLAY_PF;
+  constexpr int PF = sizeof(S) == 2 ? SJHIP_REPLAY_PF16 : SJHIP_REPLAY_PF;
 
   const int64_t N = a.N, T = a.T;
   const E *xp = (const E *)a.x + col;

@@ -22,6 +22,11 @@
 #ifndef SJHIP_FWD_PF
 #define SJHIP_FWD_PF 8
 #endif
+// prefetch depth for 16-bit storage: a 16-byte access carries eight neurons there, so the per-lane state is
+// twice as large and fewer rows in flight keep two wavefronts per SIMD resident
+#ifndef SJHIP_FWD_PF16
+#define SJHIP_FWD_PF16 4
+#endif
 #ifndef SJHIP_FWD_NT
 #define SJHIP_FWD_NT 0
 #endif
@@ -93,7 +98,7 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
-  constexpr int PF = SJHIP_FWD_PF;
+  constexpr int PF = sizeof(S) == 2 ? SJHIP_FWD_PF16 : SJHIP_FWD_PF;
 
   const int64_t N = a.N, T = a.T;
   const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
@@ -129,7 +134,7 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
         A::unpack(cur[i], x);
 #pragma unroll
         for (int j = 0; j < V; ++j) neuron_step<R, CH, SOFT>(x[j], v[j], h[j], s[j], tau, a);
-        A::store(sp + t * N, s);
+        A::store_spikes(sp + t * N, s);
         if (hp) A::store(hp + t * N, h);
         if (vp) A::store(vp + t * N, v);
       }

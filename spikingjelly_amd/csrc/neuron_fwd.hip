@@ -14,7 +14,8 @@ int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   const int64_t items = (a.N + V - 1) / V;
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "forward: N=%lld needs %lld blocks", (long long)a.N, (long long)blocks);
-  const unsigned lds = occupancy_cap_lds(tuning().fwd_blocks_per_cu);
+  // the residency cap pays for fp32 storage only: 16-bit storage needs more wavefronts to hide its conversions
+  const unsigned lds = sizeof(S) == 4 ? occupancy_cap_lds(tuning().fwd_blocks_per_cu) : 0u;
   ProfileScope prof(KC_FORWARD, stream);
   if (vector)
     hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH>), dim3((unsigned)blocks), dim3(block), lds, stream, a);

@@ -25,6 +25,7 @@ template <> struct Cvt<float> {
 };
 
 template <> struct Cvt<f16_t> {
+  static constexpr uint16_t kOne = 0x3c00;  // 1.0
   static __host__ __device__ __forceinline__ float to_float(uint16_t b) {
     return (float)__builtin_bit_cast(_Float16, b);
   }
@@ -36,11 +37,16 @@ template <> struct Cvt<f16_t> {
 };
 
 template <> struct Cvt<bf16_t> {
+  static constexpr uint16_t kOne = 0x3f80;  // 1.0
   static __host__ __device__ __forceinline__ float to_float(uint16_t b) {
     return __builtin_bit_cast(float, (uint32_t)b << 16);
   }
-  // round-to-nearest-even on the upper 16 bits; NaN stays a quiet NaN
+  // round-to-nearest-even on the upper 16 bits; NaN stays a quiet NaN.  On the device this is the
+  // hardware conversion (v_cvt_pk_bf16_f32), which rounds the same way.
   static __host__ __device__ __forceinline__ uint16_t from_float(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
+#endif
     uint32_t u = __builtin_bit_cast(uint32_t, f);
     if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
     u += 0x7fffu + ((u >> 16) & 1u);
@@ -78,6 +84,8 @@ template <bool NT> struct Acc<float, true, NT> {
     raw_t r; r.x = f[0]; r.y = f[1]; r.z = f[2]; r.w = f[3];
     stream_store<NT>((raw_t *)p, r);
   }
+  // spikes are exactly 0 or 1: in 16-bit storage the bit pattern is selected instead of converted
+  static __device__ __forceinline__ void store_spikes(elem_t *p, const float (&f)[V]) { store(p, f); }
 };
 template <bool NT> struct Acc<float, false, NT> {
   static constexpr int V = 1;
@@ -87,6 +95,7 @@ template <bool NT> struct Acc<float, false, NT> {
   static __device__ __forceinline__ raw_t zero() { return 0.f; }
   static __device__ __forceinline__ void unpack(raw_t r, float (&f)[V]) { f[0] = r; }
   static __device__ __forceinline__ void store(elem_t *p, const float (&f)[V]) { stream_store<NT>(p, f[0]); }
+  static __device__ __forceinline__ void store_spikes(elem_t *p, const float (&f)[V]) { store(p, f); }
 };
 template <typename H, bool NT> struct Acc16v {
   static constexpr int V = 8;
@@ -110,6 +119,14 @@ template <typename H, bool NT> struct Acc16v {
     raw_t r; r.x = w[0]; r.y = w[1]; r.z = w[2]; r.w = w[3];
     stream_store<NT>((raw_t *)p, r);
   }
+  static __device__ __forceinline__ void store_spikes(elem_t *p, const float (&f)[V]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      w[i] = (f[2 * i] != 0.0f ? (uint32_t)Cvt<H>::kOne : 0u) | (f[2 * i + 1] != 0.0f ? (uint32_t)Cvt<H>::kOne << 16 : 0u);
+    raw_t r; r.x = w[0]; r.y = w[1]; r.z = w[2]; r.w = w[3];
+    stream_store<NT>((raw_t *)p, r);
+  }
 };
 template <typename H, bool NT> struct Acc16s {
   static constexpr int V = 1;
@@ -120,6 +137,9 @@ template <typename H, bool NT> struct Acc16s {
   static __device__ __forceinline__ void unpack(raw_t r, float (&f)[V]) { f[0] = Cvt<H>::to_float(r); }
   static __device__ __forceinline__ void store(elem_t *p, const float (&f)[V]) {
     stream_store<NT>(p, Cvt<H>::from_float(f[0]));
+  }
+  static __device__ __forceinline__ void store_spikes(elem_t *p, const float (&f)[V]) {
+    stream_store<NT>(p, f[0] != 0.0f ? Cvt<H>::kOne : (uint16_t)0);
   }
 };
 template <bool NT> struct Acc<f16_t, true, NT> : Acc16v<f16_t, NT> {};
