@@ -154,6 +154,18 @@ def other_workload(args) -> int:
         f_ms, p_ms, u_ms = _kernel_ms(L, L.KC_FORWARD), _kernel_ms(L, L.KC_BIT_PACK), _kernel_ms(L, L.KC_BIT_UNPACK)
         n = T * N
         fwd_bytes, pack_bytes, unpack_bytes = 4 * n + 4 * N, 2 * n + n // 8, n // 8 + 2 * n
+
+        # the same work with the spikes bit-packed by the neuron kernel itself (no dense spike tensor, no pack pass)
+        v0 = torch.zeros(shape[1:], dtype=torch.float16, device=dev)
+
+        def fused_step():
+            bits, _, _ = functional.if_multi_step_hip_packed(x, v0, 1.0, None)
+            return bits, bit_spike_decompress(bits, x.shape, dtype=torch.float16)
+
+        fused_elapsed = _time_steps(torch, L, fused_step, args.steps, args.warmup)
+        fused_ms = _kernel_ms(L, L.KC_FORWARD)
+        assert torch.equal(fused_step()[1], s)
+        fused_bytes = 2 * n + n // 8 + 4 * N
         _emit(args, "neuron-steps/sec IF inference fp16 + spike bit-pack/unpack, T=32 N=6.4M, 1 MI355X", "neuron-steps/s",
               n / (elapsed / args.steps), elapsed, "f16",
               {"workload": "configs[3]: IFNode soft reset eval, x [32,64,512,14,14] fp16 uniform[0,0.25), then "
@@ -163,7 +175,9 @@ def other_workload(args) -> int:
                "frac": fwd_bytes / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "forward(inference)",
                "kernel_ms": f_ms, "algorithmic_bytes": fwd_bytes,
                "pack_ms": p_ms, "pack_GBs": pack_bytes / (p_ms * 1e-3) / 1e9,
-               "unpack_ms": u_ms, "unpack_GBs": unpack_bytes / (u_ms * 1e-3) / 1e9})
+               "unpack_ms": u_ms, "unpack_GBs": unpack_bytes / (u_ms * 1e-3) / 1e9,
+               "fused_forward_packed_ms": fused_ms, "fused_forward_packed_GBs": fused_bytes / (fused_ms * 1e-3) / 1e9,
+               "fused_ms_per_step": fused_elapsed / args.steps * 1e3})
         return 0
 
     if args.workload == "config5":

@@ -15,6 +15,8 @@
  *                             plif.py:288-386, integrate_and_fire.py:76-147; and
  *                             torch.ops.sj.multistep_{if,lif,plif}_{forward,inference}
  *                             spikingjelly/activation_based/triton_kernel/neuron_kernel/lif.py:673-763
+ *   sjhip_neuron_forward_packed <- the same forward ops followed by BitSpikeCompressor.compress,
+ *                             spikingjelly/activation_based/memopt/compress.py:332-385
  *   sjhip_neuron_backward  <- torch.ops.sj.cupy_multistep_{if,lif,plif}_backward
  *                             multi_step/lif.py:228-282, plif.py:389-470, integrate_and_fire.py:150-200;
  *                             BPTT body multi_step/base.py:137-409
@@ -121,6 +123,23 @@ int sjhip_neuron_forward(int neuron, int dtype, const sjhip_neuron_params *p,
                          const void *x_seq, const void *v_init, const float *rtau_device,
                          void *spike_seq, void *v_seq, void *v_last, void *h_seq,
                          void *stream);
+
+/*
+ * Inference forward that writes the spikes bit-packed instead of as a dense tensor: the fused form of
+ * sjhip_neuron_forward followed by sjhip_bit_pack, i.e. of a kernel-backend neuron feeding the reference's
+ * BitSpikeCompressor (spikingjelly/activation_based/memopt/compress.py:332-385 on top of
+ * triton_kernel/compress.py:114-166).  Per neuron-step it moves sizeof(dtype) + 1/8 bytes instead of
+ * 2 sizeof(dtype) for the forward plus sizeof(dtype) + 1/8 for the pack.
+ *   spike_bits  [(T*N)/8] bytes out: byte j bit i = spike of flattened element 8 j + i (LSB first), exactly
+ *               what sjhip_bit_pack writes for the dense [T,N] spike tensor
+ *   other arguments as sjhip_neuron_forward (no h_seq: this is an inference entry point)
+ * N must be a multiple of 8 so that every time step starts on a byte (SJHIP_ERR_UNSUPPORTED otherwise).
+ */
+int sjhip_neuron_forward_packed(int neuron, int dtype, const sjhip_neuron_params *p,
+                                int64_t T, int64_t N,
+                                const void *x_seq, const void *v_init, const float *rtau_device,
+                                uint8_t *spike_bits, void *v_seq, void *v_last,
+                                void *stream);
 
 /* Number of floats of caller-provided workspace the PLIF backward needs for N neurons of `dtype`
  * (per-block partial sums of the deterministic reduction). */

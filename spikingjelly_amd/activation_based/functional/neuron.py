@@ -6,7 +6,11 @@ Two families, as in the reference's ``spikingjelly/activation_based/functional/n
   (reference :173-228, :242-312, :797-933, :1215-1297);
 * ``{if,lif,plif}_multi_step_hip``: whole sequences through the HIP kernels, same signature and
   return convention as the reference's ``*_multi_step_cupy`` / ``*_multi_step_triton``
-  (:1889-2185, :2582-2849): ``(spike_seq, v_next, v_seq or None)``.
+  (:1889-2185, :2582-2849): ``(spike_seq, v_next, v_seq or None)``;
+* ``{if,lif,plif}_multi_step_hip_packed``: inference only, the spikes come back bit-packed
+  (``bit_spike_compress`` layout) instead of as a dense tensor: ``(spike_bits, v_next, v_seq or None)``.
+  It is the fused form of a kernel-backend neuron followed by the reference's ``BitSpikeCompressor``
+  (``memopt/compress.py:332-385``); unpack with ``bit_spike_decompress(spike_bits, x_seq.shape, dtype)``.
 """
 
 from __future__ import annotations
@@ -28,6 +32,9 @@ __all__ = [
     "if_multi_step_hip",
     "lif_multi_step_hip",
     "plif_multi_step_hip",
+    "if_multi_step_hip_packed",
+    "lif_multi_step_hip_packed",
+    "plif_multi_step_hip_packed",
 ]
 
 
@@ -186,3 +193,76 @@ def plif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Tensor, d
         s, v_seq, v_last = K.hip_multistep_plif_inference(x2, v1, k, v_threshold, vr, soft, decay_input,
                                                           store_v_seq, flags)
     return _finish(x_seq, s, v_seq, v_last, store_v_seq)
+
+
+# ---- hip backend: whole sequence, bit-packed spikes (inference) -----------------------------------
+def _finish_packed(x_seq: torch.Tensor, out, store_v_seq: bool
+                   ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    bits, v_seq, v_last = out
+    return bits, v_last.reshape(x_seq.shape[1:]), (v_seq.reshape(x_seq.shape) if store_v_seq else None)
+
+
+def _packed_by_two_kernels(dense_out) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """N % 8 != 0: a time step does not start on a byte, so the dense kernel runs and its spikes are packed."""
+    from ..hip_kernel.compress import bit_spike_compress
+
+    s, v_seq, v_last = dense_out
+    return bit_spike_compress(s), v_seq, v_last
+
+
+@torch.no_grad()
+def if_multi_step_hip_packed(x_seq: torch.Tensor, v: torch.Tensor, v_threshold: float, v_reset: Optional[float],
+                             store_v_seq: bool = False
+                             ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Multi-step IF inference on the hip backend with bit-packed spike output."""
+    from ..hip_kernel import neuron_kernel as K
+
+    soft = v_reset is None
+    vr = 0.0 if soft else float(v_reset)
+    flags = _hip_mode_flags(x_seq)
+    x2, v1 = x_seq.flatten(1), v.flatten()
+    if K.packed_supported(x2.shape[1]):
+        out = K.hip_multistep_if_inference_packed(x2, v1, v_threshold, vr, soft, store_v_seq, flags)
+    else:
+        out = _packed_by_two_kernels(K.hip_multistep_if_inference(x2, v1, v_threshold, vr, soft, store_v_seq, flags))
+    return _finish_packed(x_seq, out, store_v_seq)
+
+
+@torch.no_grad()
+def lif_multi_step_hip_packed(x_seq: torch.Tensor, v: torch.Tensor, tau: float, decay_input: bool,
+                              v_threshold: float, v_reset: Optional[float], store_v_seq: bool = False
+                              ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Multi-step LIF inference on the hip backend with bit-packed spike output."""
+    from ..hip_kernel import neuron_kernel as K
+
+    soft = v_reset is None
+    vr = 0.0 if soft else float(v_reset)
+    flags = _hip_mode_flags(x_seq)
+    x2, v1 = x_seq.flatten(1), v.flatten()
+    if K.packed_supported(x2.shape[1]):
+        out = K.hip_multistep_lif_inference_packed(x2, v1, v_threshold, vr, soft, float(tau), decay_input,
+                                                   store_v_seq, flags)
+    else:
+        out = _packed_by_two_kernels(K.hip_multistep_lif_inference(x2, v1, v_threshold, vr, soft, float(tau),
+                                                                   decay_input, store_v_seq, flags))
+    return _finish_packed(x_seq, out, store_v_seq)
+
+
+@torch.no_grad()
+def plif_multi_step_hip_packed(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Tensor, decay_input: bool,
+                               v_threshold: float, v_reset: Optional[float], store_v_seq: bool = False
+                               ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Multi-step parametric-LIF inference on the hip backend with bit-packed spike output."""
+    from ..hip_kernel import neuron_kernel as K
+
+    soft = v_reset is None
+    vr = 0.0 if soft else float(v_reset)
+    flags = _hip_mode_flags(x_seq)
+    x2, v1 = x_seq.flatten(1), v.flatten()
+    k = w.sigmoid().to(device=x_seq.device, dtype=torch.float32)
+    if K.packed_supported(x2.shape[1]):
+        out = K.hip_multistep_plif_inference_packed(x2, v1, k, v_threshold, vr, soft, decay_input, store_v_seq, flags)
+    else:
+        out = _packed_by_two_kernels(K.hip_multistep_plif_inference(x2, v1, k, v_threshold, vr, soft, decay_input,
+                                                                    store_v_seq, flags))
+    return _finish_packed(x_seq, out, store_v_seq)

@@ -32,6 +32,7 @@ EXPORTED_SYMBOLS = (
     "sjhip_abi_version",
     "sjhip_last_error",
     "sjhip_neuron_forward",
+    "sjhip_neuron_forward_packed",
     "sjhip_plif_workspace_floats",
     "sjhip_neuron_backward",
     "sjhip_neuron_backward_recompute",
@@ -92,6 +93,11 @@ def load() -> ctypes.CDLL:
         lib.sjhip_neuron_forward.argtypes = [
             c_int, c_int, POINTER(NeuronParams), c_int64, c_int64,
             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        ]
+        lib.sjhip_neuron_forward_packed.restype = c_int
+        lib.sjhip_neuron_forward_packed.argtypes = [
+            c_int, c_int, POINTER(NeuronParams), c_int64, c_int64,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
         ]
         lib.sjhip_plif_workspace_floats.restype = c_int64
         lib.sjhip_plif_workspace_floats.argtypes = [c_int, c_int64]

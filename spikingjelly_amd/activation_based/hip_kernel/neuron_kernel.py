@@ -8,6 +8,10 @@ inference op that writes no ``h_seq``):
     sj::hip_multistep_{if,lif,plif}_forward    -> (spike_seq, v_seq, v_last, h_seq)
     sj::hip_multistep_{if,lif,plif}_inference  -> (spike_seq, v_seq, v_last)
     sj::hip_multistep_{if,lif,plif}_backward   -> (grad_x_seq, grad_v_init[, grad_k])
+    sj::hip_multistep_{if,lif,plif}_inference_packed -> (spike_bits, v_seq, v_last)
+
+The ``_packed`` ops write the spikes bit-packed (uint8, ``T*N/8`` bytes, the layout of
+``bit_spike_compress`` on the dense spike tensor) straight from the neuron kernel; they need ``N % 8 == 0``.
 
 All tensors are viewed as ``[T, N]``; ``v_seq`` is an empty tensor when ``store_v_seq`` is false
 (the kernel then writes only ``v_last``).  With ``recompute`` the forward writes no ``h_seq`` (an empty
@@ -30,6 +34,8 @@ __all__ = [
     "hip_multistep_if_forward", "hip_multistep_if_inference", "hip_multistep_if_backward",
     "hip_multistep_lif_forward", "hip_multistep_lif_inference", "hip_multistep_lif_backward",
     "hip_multistep_plif_forward", "hip_multistep_plif_inference", "hip_multistep_plif_backward",
+    "hip_multistep_if_inference_packed", "hip_multistep_lif_inference_packed", "hip_multistep_plif_inference_packed",
+    "packed_supported",
 ]
 
 
@@ -93,6 +99,44 @@ def _run_forward(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: Opti
     L.check(rc, "neuron_forward")
     del k_keep
     return spike_seq, v_seq, v_last, h_seq
+
+
+def packed_supported(n_neurons: int) -> bool:
+    """The packed-spike forward needs every time step to start on a byte."""
+    return n_neurons % 8 == 0
+
+
+def _run_forward_packed(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: Optional[torch.Tensor],
+                        tau: float, v_th: float, v_reset: float, flags: int, store_v_seq: bool
+                        ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    _check_inputs(x_seq, v_init)
+    dtype = L.dtype_id(x_seq.dtype)
+    x_seq = x_seq.contiguous()
+    v_init = v_init.contiguous()
+    T, N = x_seq.shape
+    if not packed_supported(N):
+        raise NotImplementedError(f"packed spike output needs N % 8 == 0, got N={N}")
+    spike_bits = torch.empty((T * N // 8,), dtype=torch.uint8, device=x_seq.device)
+    v_seq = torch.empty_like(x_seq) if store_v_seq else x_seq.new_empty((0,))
+    v_last = torch.empty_like(v_init)
+    k_keep, k_ptr = _k_pointer(k, x_seq)
+    params = _params(tau, v_th, v_reset, 0.0, 0, flags)
+    with torch.cuda.device(x_seq.device):
+        rc = L.load().sjhip_neuron_forward_packed(
+            neuron, dtype, ctypes.byref(params), T, N,
+            x_seq.data_ptr(), v_init.data_ptr(), k_ptr,
+            spike_bits.data_ptr(), v_seq.data_ptr() if store_v_seq else None, v_last.data_ptr(),
+            L.current_stream_ptr(x_seq.device),
+        )
+    L.check(rc, "neuron_forward_packed")
+    del k_keep
+    return spike_bits, v_seq, v_last
+
+
+def _fake_forward_packed(x_seq, v_init, store_v_seq):
+    return (x_seq.new_empty((x_seq.shape[0] * x_seq.shape[1] // 8,), dtype=torch.uint8),
+            x_seq.new_empty(x_seq.shape) if store_v_seq else x_seq.new_empty((0,)),
+            v_init.new_empty(v_init.shape))
 
 
 def _forward_outputs(out, x_seq: torch.Tensor):
@@ -425,3 +469,45 @@ def _plif_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h
 
 torch.library.register_autograd("sj::hip_multistep_plif_forward", _plif_autograd_backward,
                                 setup_context=_plif_setup_context)
+
+
+# =================================================================================================
+# Inference with bit-packed spike output (all three neurons)
+# =================================================================================================
+@torch.library.custom_op("sj::hip_multistep_if_inference_packed", mutates_args=())
+def hip_multistep_if_inference_packed(x_seq: torch.Tensor, v_init: torch.Tensor, v_th: float, v_reset: float,
+                                      soft_reset: bool, store_v_seq: bool, mode_flags: int
+                                      ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, False, False, mode_flags)
+    return _run_forward_packed(L.NEURON_IF, x_seq, v_init, None, 0.0, v_th, v_reset, flags, store_v_seq)
+
+
+@hip_multistep_if_inference_packed.register_fake
+def _(x_seq, v_init, v_th, v_reset, soft_reset, store_v_seq, mode_flags):
+    return _fake_forward_packed(x_seq, v_init, store_v_seq)
+
+
+@torch.library.custom_op("sj::hip_multistep_lif_inference_packed", mutates_args=())
+def hip_multistep_lif_inference_packed(x_seq: torch.Tensor, v_init: torch.Tensor, v_th: float, v_reset: float,
+                                       soft_reset: bool, tau: float, decay_input: bool, store_v_seq: bool,
+                                       mode_flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, False, decay_input, mode_flags)
+    return _run_forward_packed(L.NEURON_LIF, x_seq, v_init, None, tau, v_th, v_reset, flags, store_v_seq)
+
+
+@hip_multistep_lif_inference_packed.register_fake
+def _(x_seq, v_init, v_th, v_reset, soft_reset, tau, decay_input, store_v_seq, mode_flags):
+    return _fake_forward_packed(x_seq, v_init, store_v_seq)
+
+
+@torch.library.custom_op("sj::hip_multistep_plif_inference_packed", mutates_args=())
+def hip_multistep_plif_inference_packed(x_seq: torch.Tensor, v_init: torch.Tensor, k: torch.Tensor, v_th: float,
+                                        v_reset: float, soft_reset: bool, decay_input: bool, store_v_seq: bool,
+                                        mode_flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, False, decay_input, mode_flags)
+    return _run_forward_packed(L.NEURON_PLIF, x_seq, v_init, k, 0.0, v_th, v_reset, flags, store_v_seq)
+
+
+@hip_multistep_plif_inference_packed.register_fake
+def _(x_seq, v_init, k, v_th, v_reset, soft_reset, decay_input, store_v_seq, mode_flags):
+    return _fake_forward_packed(x_seq, v_init, store_v_seq)

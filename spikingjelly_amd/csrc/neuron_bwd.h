@@ -68,6 +68,7 @@ template <bool FAST> __device__ __forceinline__ float sg_div(float a, float b) {
 }
 
 template <int SG, bool FAST> __device__ __forceinline__ float surrogate_grad(float x, float alpha) {
+#pragma clang fp contract(fast)
   if (SG == SJHIP_SG_SIGMOID) {
     // surrogate.py:769-771:  s = sigmoid(alpha x);  (1 - s) s alpha
     float s = sg_div<FAST>(1.0f, 1.0f + sg_exp<FAST>(-alpha * x));
@@ -97,6 +98,12 @@ template <int SG, bool FAST> __device__ __forceinline__ float surrogate_grad(flo
     float ax = x * alpha;
     return 0.56418958354775628695f * alpha * sg_exp<FAST>(-(ax * ax));
   }
+}
+
+// v_t from h_t exactly as the forward wrote it (no fused multiply-add)
+__device__ __forceinline__ float reset_as_forward(float h, float s, const BwdArgs &a) {
+#pragma clang fp contract(off)
+  return a.soft_reset ? (h - s * a.v_th) : (s * a.v_reset + (1.0f - s) * h);
 }
 
 // HLDS: h_t does not come from h_seq in global memory but from LDS, where the recompute kernel
@@ -208,20 +215,24 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
 #pragma unroll
         for (int j = 0; j < V; ++j) {
           const float over = h[j] - v_th;
-          const float sg = surrogate_grad<SG, sizeof(S) == 2>(over, alpha);
           const float s = (over >= 0.0f) ? 1.0f : 0.0f;
-          if (PLIF) {
-            // v_t from h_t exactly as the forward wrote it
-            const float v_t = a.soft_reset ? (h[j] - s * v_th) : (s * a.v_reset + (1.0f - s) * h[j]);
-            const float dh_dk = a.decay_input ? (h_next[j] - v_t) : (a.v_reset - v_t);
-            acc[j] += g_next[j] * dh_dk;  // g_next is 0 on the first processed step
+          float v_t = 0.0f;
+          if (PLIF) v_t = reset_as_forward(h[j], s, a);
+          {
+            // gradients carry a tolerance, not bit-exactness: let multiply-adds fuse here
+#pragma clang fp contract(fast)
+            const float sg = surrogate_grad<SG, sizeof(S) == 2>(over, alpha);
+            if (PLIF) {
+              const float dh_dk = a.decay_input ? (h_next[j] - v_t) : (a.v_reset - v_t);
+              acc[j] += g_next[j] * dh_dk;  // g_next is 0 on the first processed step
+            }
+            const float dvdh = (1.0f - s * cB) + (cC - h[j] * cD) * sg;
+            const float gvt = GVFULL ? carry[j] + gv[j] : carry[j];
+            const float G = gvt * dvdh + gs[j] * sg;
+            gx[j] = G * kx;
+            carry[j] = G * km;
+            if (PLIF) { g_next[j] = G; h_next[j] = h[j]; }
           }
-          const float dvdh = (1.0f - s * cB) + (cC - h[j] * cD) * sg;
-          const float gvt = GVFULL ? carry[j] + gv[j] : carry[j];
-          const float G = gvt * dvdh + gs[j] * sg;
-          gx[j] = G * kx;
-          carry[j] = G * km;
-          if (PLIF) { g_next[j] = G; h_next[j] = h[j]; }
         }
         A::store(gxp + t * N, gx);
       }

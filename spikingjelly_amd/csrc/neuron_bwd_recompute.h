@@ -38,7 +38,8 @@ __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, i
   typename A::raw_t ahead[PF];
 #pragma unroll
   for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? A::load(xp + (int64_t)i * N) : A::zero();
-  float v[V];
+  typedef typename StepNum<S, ROUND_EACH>::type NUM;
+  NUM v[V];
   A::unpack(A::load((const E *)a.v_init + col), v);
 
   for (int64_t t0 = 0; t0 < T; t0 += PF) {
@@ -54,13 +55,13 @@ __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, i
     for (int i = 0; i < PF; ++i) {
       const int64_t t = t0 + i;
       if (t < T) {
-        float x[V], h[V], s[V];
+        NUM x[V], h[V], s[V];
         A::unpack(cur[i], x);
 #pragma unroll
         for (int j = 0; j < V; ++j) neuron_step<R, CH, SOFT>(x[j], v[j], h[j], s[j], tau, a);
 #pragma unroll
         for (int q = 0; q < V / 4; ++q) {
-          f32x4 w; w.x = h[4 * q]; w.y = h[4 * q + 1]; w.z = h[4 * q + 2]; w.w = h[4 * q + 3];
+          f32x4 w; w.x = (float)h[4 * q]; w.y = (float)h[4 * q + 1]; w.z = (float)h[4 * q + 2]; w.w = (float)h[4 * q + 3];
           lds_h[((int)t * (V / 4) + q) * (int)blockDim.x + (int)threadIdx.x] = w;
         }
       }

@@ -44,7 +44,7 @@ enum Charge {
 struct FwdArgs {
   const void *x;
   const void *v_init;
-  void *spike;
+  void *spike;           // dense spikes in the storage dtype, or the bit-packed byte array
   void *v_seq;           // may be null
   void *v_last;          // may be null
   void *h;               // may be null
@@ -92,7 +92,71 @@ __device__ __forceinline__ void neuron_step(float x, float &v, float &h, float &
   }
 }
 
-template <typename S, bool VECTOR, bool ROUND_EACH, int CH, bool SOFT>
+// fp16 storage with every op rounded: the same step in native half arithmetic.  For two fp16 operands an
+// fp32 add / sub / mul followed by rounding to fp16 equals the correctly rounded fp16 operation (24 >= 2 * 11 + 2
+// significand bits, so the double rounding is harmless; fp16 subnormals are kept), hence these results are
+// bit-identical to neuron_step<f16_t> on floats while needing no conversions.  Python scalars that torch keeps
+// in fp32 (the tau divisor / multiplier, v_threshold and v_reset as factors) still enter through an fp32 product
+// rounded once.
+template <typename R, int CH, bool SOFT>
+__device__ __forceinline__ void neuron_step(_Float16 x, _Float16 &v, _Float16 &h, _Float16 &s, float tau,
+                                            const FwdArgs &a) {
+#pragma clang fp contract(off)
+  typedef _Float16 H;
+  const H vr_add = (H)a.vr_add, vth_sub = (H)a.vth_sub;  // rounded to fp16 by the host already
+  if (CH == CH_IF) {
+    h = v + x;
+  } else if (CH == CH_DECAY_INPUT_DIV || CH == CH_DECAY_INPUT_MUL) {
+    const H d = v - vr_add;
+    const H e = x - d;
+    const H f = (CH == CH_DECAY_INPUT_DIV) ? (H)((float)e / tau) : (H)((float)e * tau);
+    h = v + f;
+  } else {
+    const H d = v - vr_add;
+    const H f = (CH == CH_PLAIN_INPUT_DIV) ? (H)((float)d / tau) : (H)((float)d * tau);
+    const H g = v - f;
+    h = g + x;
+  }
+  const H over = h - vth_sub;
+  s = (over >= (H)0.0f) ? (H)1.0f : (H)0.0f;
+  if (SOFT) {
+    const H m = (H)((float)s * a.vth_mul);
+    v = h - m;
+  } else {
+    const H m = (H)((float)s * a.vr_mul);
+    const H n = (H)1.0f - s;
+    const H o = n * h;
+    v = m + o;
+  }
+}
+
+// register type of x, v, h, s in the step loop
+template <typename S, bool ROUND_EACH> struct StepNum { typedef float type; };
+template <> struct StepNum<f16_t, true> { typedef _Float16 type; };
+
+// Bit-packed spike output (PACKED): a.spike is a byte array holding the flattened [T, N] spikes LSB first,
+// byte j bit i = element 8 j + i, the layout of bit_pack.  N % 8 == 0 makes every row start on a byte.  A
+// work-item with eight neurons writes its byte; with four neurons two neighbouring lanes combine their
+// nibbles; with one neuron a wavefront ballot yields eight bytes written by its first eight lanes.
+template <int V, typename NUM>
+__device__ __forceinline__ void store_spike_bits(uint8_t *row, int64_t col, int64_t N, const NUM (&s)[V]) {
+  uint32_t bits = 0;
+#pragma unroll
+  for (int j = 0; j < V; ++j) bits |= (s[j] != (NUM)0.0f ? 1u : 0u) << j;
+  if (V == 8) {
+    row[col >> 3] = (uint8_t)bits;
+  } else if (V == 4) {
+    const uint32_t other = (uint32_t)__shfl_xor((int)bits, 1, 64);
+    if ((threadIdx.x & 1) == 0) row[col >> 3] = (uint8_t)(bits | (other << 4));
+  } else {
+    const unsigned long long mask = __ballot(bits != 0);
+    const int lane = threadIdx.x & 63;
+    const int64_t col0 = col - lane;  // first neuron of this wavefront, a multiple of 64
+    if (lane < 8 && col0 + 8 * lane < N) row[(col0 >> 3) + lane] = (uint8_t)(mask >> (8 * lane));
+  }
+}
+
+template <typename S, bool VECTOR, bool ROUND_EACH, int CH, bool SOFT, bool PACKED>
 __device__ __forceinline__ void forward_body(const FwdArgs &a) {
   typedef Acc<S, VECTOR, SJHIP_FWD_NT != 0> A;
   typedef typename A::elem_t E;
@@ -114,7 +178,8 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
 #pragma unroll
   for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? A::load(xp + (int64_t)i * N) : A::zero();
 
-  float v[V];
+  typedef typename StepNum<S, ROUND_EACH>::type NUM;
+  NUM v[V];
   A::unpack(A::load((const E *)a.v_init + col), v);
 
   for (int64_t t0 = 0; t0 < T; t0 += PF) {
@@ -130,11 +195,12 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
     for (int i = 0; i < PF; ++i) {
       const int64_t t = t0 + i;
       if (t < T) {
-        float x[V], h[V], s[V];
+        NUM x[V], h[V], s[V];
         A::unpack(cur[i], x);
 #pragma unroll
         for (int j = 0; j < V; ++j) neuron_step<R, CH, SOFT>(x[j], v[j], h[j], s[j], tau, a);
-        A::store_spikes(sp + t * N, s);
+        if (PACKED) store_spike_bits<V>((uint8_t *)a.spike + t * (N >> 3), col, N, s);
+        else A::store_spikes(sp + t * N, s);
         if (hp) A::store(hp + t * N, h);
         if (vp) A::store(vp + t * N, v);
       }
@@ -143,22 +209,22 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
   if (a.v_last) A::store((E *)a.v_last + col, v);
 }
 
-template <typename S, bool VECTOR, bool ROUND_EACH, int CH>
+template <typename S, bool VECTOR, bool ROUND_EACH, int CH, bool PACKED>
 __device__ __forceinline__ void forward_reset_dispatch(const FwdArgs &a) {
   if (a.soft_reset)
-    forward_body<S, VECTOR, ROUND_EACH, CH, true>(a);
+    forward_body<S, VECTOR, ROUND_EACH, CH, true, PACKED>(a);
   else
-    forward_body<S, VECTOR, ROUND_EACH, CH, false>(a);
+    forward_body<S, VECTOR, ROUND_EACH, CH, false, PACKED>(a);
 }
 
-template <typename S, bool VECTOR, bool ROUND_EACH>
+template <typename S, bool VECTOR, bool ROUND_EACH, bool PACKED = false>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) forward_kernel(const FwdArgs a) {
   switch (a.charge) {
-    case CH_IF: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_IF>(a); break;
-    case CH_DECAY_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_DIV>(a); break;
-    case CH_DECAY_INPUT_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_MUL>(a); break;
-    case CH_PLAIN_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_DIV>(a); break;
-    default: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_MUL>(a); break;
+    case CH_IF: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_IF, PACKED>(a); break;
+    case CH_DECAY_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_DIV, PACKED>(a); break;
+    case CH_DECAY_INPUT_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_MUL, PACKED>(a); break;
+    case CH_PLAIN_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_DIV, PACKED>(a); break;
+    default: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_MUL, PACKED>(a); break;
   }
 }
 

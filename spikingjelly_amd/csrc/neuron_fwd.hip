@@ -7,7 +7,7 @@ namespace sjhip {
 
 namespace {
 
-template <typename S, bool ROUND_EACH>
+template <typename S, bool ROUND_EACH, bool PACKED = false>
 int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   const int block = tuning().fwd_block;
   const int V = vector ? Acc<S, true, true>::V : 1;
@@ -18,13 +18,32 @@ int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   const unsigned lds = sizeof(S) == 4 ? occupancy_cap_lds(tuning().fwd_blocks_per_cu) : 0u;
   ProfileScope prof(KC_FORWARD, stream);
   if (vector)
-    hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH>), dim3((unsigned)blocks), dim3(block), lds, stream, a);
+    hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, PACKED>), dim3((unsigned)blocks), dim3(block), lds, stream, a);
   else
-    hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH>), dim3((unsigned)blocks), dim3(block), lds, stream, a);
-  return check_launch("forward");
+    hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH, PACKED>), dim3((unsigned)blocks), dim3(block), lds, stream, a);
+  return check_launch(PACKED ? "forward_packed" : "forward");
 }
 
 }  // namespace
+
+int launch_forward_packed(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
+                          const void *x_seq, const void *v_init, const float *k_device, uint8_t *spike_bits,
+                          void *v_seq, void *v_last, hipStream_t stream) {
+  if (N % 8 != 0)
+    return fail(SJHIP_ERR_UNSUPPORTED, "forward_packed: N=%lld is not a multiple of 8 (rows must start on a byte)", (long long)N);
+  FwdArgs a;
+  bool round_each = false;
+  int rc = build_fwd_args(a, round_each, neuron, dtype, p, T, N, x_seq, v_init, k_device, spike_bits, v_seq, v_last, nullptr);
+  if (rc != SJHIP_OK) return rc;
+  const bool vector = aligned16(x_seq) && aligned16(v_init) && (v_seq == nullptr || aligned16(v_seq)) &&
+                      (v_last == nullptr || aligned16(v_last));
+  switch (dtype) {
+    case SJHIP_F32: return launch_typed<float, false, true>(a, vector, stream);
+    case SJHIP_F16: return round_each ? launch_typed<f16_t, true, true>(a, vector, stream) : launch_typed<f16_t, false, true>(a, vector, stream);
+    case SJHIP_BF16: return round_each ? launch_typed<bf16_t, true, true>(a, vector, stream) : launch_typed<bf16_t, false, true>(a, vector, stream);
+    default: return fail(SJHIP_ERR_INVALID, "forward_packed: dtype %d", dtype);
+  }
+}
 
 int launch_forward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
                    const void *x_seq, const void *v_init, const float *k_device, void *spike_seq,

@@ -144,6 +144,20 @@ int sjhip_neuron_forward(int neuron, int dtype, const sjhip_neuron_params *p, in
                         static_cast<hipStream_t>(stream));
 }
 
+int sjhip_neuron_forward_packed(int neuron, int dtype, const sjhip_neuron_params *p, int64_t T, int64_t N,
+                                const void *x_seq, const void *v_init, const float *rtau_device, uint8_t *spike_bits,
+                                void *v_seq, void *v_last, void *stream) {
+  if (!p) return fail(SJHIP_ERR_INVALID, "forward_packed: params is NULL");
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_PLIF) return fail(SJHIP_ERR_INVALID, "forward_packed: neuron %d", neuron);
+  if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "forward_packed: dtype %d", dtype);
+  int rc = check_shape("forward_packed", T, N);
+  if (rc != SJHIP_OK) return rc;
+  if (!x_seq || !v_init || !spike_bits) return fail(SJHIP_ERR_INVALID, "forward_packed: NULL tensor");
+  if (!v_seq && !v_last) return fail(SJHIP_ERR_INVALID, "forward_packed: neither v_seq nor v_last given");
+  return launch_forward_packed(neuron, dtype, *p, T, N, x_seq, v_init, rtau_device, spike_bits, v_seq, v_last,
+                               static_cast<hipStream_t>(stream));
+}
+
 int64_t sjhip_plif_workspace_floats(int dtype, int64_t N) {
   if (N < 1) return 0;
   return plif_blocks(dtype, N);

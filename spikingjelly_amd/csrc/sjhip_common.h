@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "sjhip.h"
 
 namespace sjhip {
@@ -127,6 +129,26 @@ template <typename H, bool NT> struct Acc16v {
     raw_t r; r.x = w[0]; r.y = w[1]; r.z = w[2]; r.w = w[3];
     stream_store<NT>((raw_t *)p, r);
   }
+  // fp16 values kept as fp16 in registers (native half arithmetic): the stored bits are the register bits
+  static __device__ __forceinline__ void unpack(raw_t r, _Float16 (&f)[V]) {
+    static_assert(std::is_same<H, f16_t>::value, "native half registers are for fp16 storage only");
+    uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __builtin_bit_cast(_Float16, (uint16_t)(w[i] & 0xffffu));
+      f[2 * i + 1] = __builtin_bit_cast(_Float16, (uint16_t)(w[i] >> 16));
+    }
+  }
+  static __device__ __forceinline__ void store(elem_t *p, const _Float16 (&f)[V]) {
+    static_assert(std::is_same<H, f16_t>::value, "native half registers are for fp16 storage only");
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      w[i] = (uint32_t)__builtin_bit_cast(uint16_t, f[2 * i]) | ((uint32_t)__builtin_bit_cast(uint16_t, f[2 * i + 1]) << 16);
+    raw_t r; r.x = w[0]; r.y = w[1]; r.z = w[2]; r.w = w[3];
+    stream_store<NT>((raw_t *)p, r);
+  }
+  static __device__ __forceinline__ void store_spikes(elem_t *p, const _Float16 (&f)[V]) { store(p, f); }
 };
 template <typename H, bool NT> struct Acc16s {
   static constexpr int V = 1;
@@ -141,6 +163,15 @@ template <typename H, bool NT> struct Acc16s {
   static __device__ __forceinline__ void store_spikes(elem_t *p, const float (&f)[V]) {
     stream_store<NT>(p, f[0] != 0.0f ? Cvt<H>::kOne : (uint16_t)0);
   }
+  static __device__ __forceinline__ void unpack(raw_t r, _Float16 (&f)[V]) {
+    static_assert(std::is_same<H, f16_t>::value, "native half registers are for fp16 storage only");
+    f[0] = __builtin_bit_cast(_Float16, r);
+  }
+  static __device__ __forceinline__ void store(elem_t *p, const _Float16 (&f)[V]) {
+    static_assert(std::is_same<H, f16_t>::value, "native half registers are for fp16 storage only");
+    stream_store<NT>(p, __builtin_bit_cast(uint16_t, f[0]));
+  }
+  static __device__ __forceinline__ void store_spikes(elem_t *p, const _Float16 (&f)[V]) { store(p, f); }
 };
 template <bool NT> struct Acc<f16_t, true, NT> : Acc16v<f16_t, NT> {};
 template <bool NT> struct Acc<f16_t, false, NT> : Acc16s<f16_t, NT> {};
@@ -197,6 +228,9 @@ int launch_backward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t
                     const void *h_seq, const void *v_init,
                     const float *k_device, void *grad_x_seq, void *grad_v_init, float *grad_rtau,
                     float *workspace, hipStream_t stream);
+int launch_forward_packed(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
+                          const void *x_seq, const void *v_init, const float *k_device, uint8_t *spike_bits,
+                          void *v_seq, void *v_last, hipStream_t stream);
 bool recompute_supported(int dtype, int64_t T, int64_t N);
 int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
                               const void *x_seq, const void *v_init, const float *k_device,

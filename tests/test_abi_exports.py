@@ -40,6 +40,10 @@ def test_argument_validation_without_a_device():
     assert rc == -1
     rc = lib.sjhip_neuron_forward(L.NEURON_LIF, L.DTYPE_F32, ctypes.byref(p), 4, 16, 1, 1, None, 1, None, None, None, None)
     assert rc == -1 and b"v_seq" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_forward_packed(L.NEURON_IF, L.DTYPE_F16, ctypes.byref(p), 4, 12, 1, 1, None, 1, None, 1, None)
+    assert rc == -2 and b"multiple of 8" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_forward_packed(L.NEURON_IF, L.DTYPE_F16, ctypes.byref(p), 4, 16, 1, 1, None, None, None, 1, None)
+    assert rc == -1 and b"NULL" in lib.sjhip_last_error()
     p_bad = L.NeuronParams(2.0, 1.0, 0.0, 2.0, 9, 0)
     rc = lib.sjhip_neuron_backward(L.NEURON_LIF, L.DTYPE_F32, ctypes.byref(p_bad), 4, 16, 1, None, None, 1, None, None,
                                    1, 1, None, None, None)
