@@ -7,6 +7,8 @@ Two families, as in the reference's ``spikingjelly/activation_based/functional/n
 * ``{if,lif,plif}_multi_step_hip``: whole sequences through the HIP kernels, same signature and
   return convention as the reference's ``*_multi_step_cupy`` / ``*_multi_step_triton``
   (:1889-2185, :2582-2849): ``(spike_seq, v_next, v_seq or None)``;
+* ``{if,lif,plif}_step_hip``: one step through the same kernels (a sequence of length one), signature and
+  return of the reference's ``*_step_cupy`` (:1709-1886): ``(spike, v_next)``;
 * ``{if,lif,plif}_multi_step_hip_packed``: inference only, the spikes come back bit-packed
   (``bit_spike_compress`` layout) instead of as a dense tensor: ``(spike_bits, v_next, v_seq or None)``.
   It is the fused form of a kernel-backend neuron followed by the reference's ``BitSpikeCompressor``
@@ -32,6 +34,9 @@ __all__ = [
     "if_multi_step_hip",
     "lif_multi_step_hip",
     "plif_multi_step_hip",
+    "if_step_hip",
+    "lif_step_hip",
+    "plif_step_hip",
     "if_multi_step_hip_packed",
     "lif_multi_step_hip_packed",
     "plif_multi_step_hip_packed",
@@ -193,6 +198,34 @@ def plif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Tensor, d
         s, v_seq, v_last = K.hip_multistep_plif_inference(x2, v1, k, v_threshold, vr, soft, decay_input,
                                                           store_v_seq, flags)
     return _finish(x_seq, s, v_seq, v_last, store_v_seq)
+
+
+# ---- hip backend: one step (step_mode='s') --------------------------------------------------------
+def if_step_hip(x: torch.Tensor, v: torch.Tensor, v_threshold: float, v_reset: Optional[float],
+                surrogate_function: SurrogateFunction, detach_reset: bool = False
+                ) -> tuple[torch.Tensor, torch.Tensor]:
+    """One IF step on the hip backend: the multi-step kernel on a sequence of length one."""
+    spike_seq, v_next, _ = if_multi_step_hip(x.unsqueeze(0), v, v_threshold, v_reset, surrogate_function,
+                                             detach_reset, False)
+    return spike_seq[0], v_next
+
+
+def lif_step_hip(x: torch.Tensor, v: torch.Tensor, tau: float, decay_input: bool, v_threshold: float,
+                 v_reset: Optional[float], surrogate_function: SurrogateFunction, detach_reset: bool = False
+                 ) -> tuple[torch.Tensor, torch.Tensor]:
+    """One LIF step on the hip backend."""
+    spike_seq, v_next, _ = lif_multi_step_hip(x.unsqueeze(0), v, tau, decay_input, v_threshold, v_reset,
+                                              surrogate_function, detach_reset, False)
+    return spike_seq[0], v_next
+
+
+def plif_step_hip(x: torch.Tensor, v: torch.Tensor, w: torch.Tensor, decay_input: bool, v_threshold: float,
+                  v_reset: Optional[float], surrogate_function: SurrogateFunction, detach_reset: bool = False
+                  ) -> tuple[torch.Tensor, torch.Tensor]:
+    """One parametric-LIF step on the hip backend."""
+    spike_seq, v_next, _ = plif_multi_step_hip(x.unsqueeze(0), v, w, decay_input, v_threshold, v_reset,
+                                               surrogate_function, detach_reset, False)
+    return spike_seq[0], v_next
 
 
 # ---- hip backend: whole sequence, bit-packed spikes (inference) -----------------------------------

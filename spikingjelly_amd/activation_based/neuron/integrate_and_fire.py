@@ -11,7 +11,7 @@ from .base_node import BaseNode
 class IFNode(BaseNode):
     """``h[t] = v[t-1] + x[t]``; fire where ``h >= v_threshold``; hard or soft reset.
 
-    Multi-step mode supports ``backend='torch'`` and ``backend='hip'``.
+    Both step modes support ``backend='torch'`` and ``backend='hip'``.
     """
 
     def __init__(self, v_threshold: float = 1.0, v_reset: Optional[float] = 0.0,
@@ -21,17 +21,20 @@ class IFNode(BaseNode):
 
     @property
     def supported_backends(self):
-        if self.step_mode == "s":
-            return ("torch",)
-        if self.step_mode == "m":
+        if self.step_mode in ("s", "m"):
             return ("torch", "hip")
         raise ValueError(self.step_mode)
 
     def single_step_functional_forward(self, inputs, states, **kwargs):
-        if self.backend != "torch":
+        if self.backend == "hip":
+            self._check_hip_surrogate()
+            spike, v = functional.if_step_hip(inputs[0], states[0], self.v_threshold, self.v_reset,
+                                              self.surrogate_function, self.detach_reset)
+        elif self.backend == "torch":
+            spike, v = functional.if_step(inputs[0], states[0], self.v_threshold, self.v_reset,
+                                          self._torch_surrogate(), self.detach_reset)
+        else:
             raise ValueError(self.backend)
-        spike, v = functional.if_step(inputs[0], states[0], self.v_threshold, self.v_reset,
-                                      self._torch_surrogate(), self.detach_reset)
         return (spike,), (v, *states[1:])
 
     def _hip_multi_step(self, x_seq, v, store_v_seq):

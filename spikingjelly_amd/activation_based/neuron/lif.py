@@ -11,7 +11,7 @@ from .base_node import BaseNode
 class LIFNode(BaseNode):
     """``h = v + (x - (v - v_reset))/tau`` (``decay_input=True``) or ``h = v - (v - v_reset)/tau + x``.
 
-    Multi-step mode supports ``backend='torch'`` and ``backend='hip'``.
+    Both step modes support ``backend='torch'`` and ``backend='hip'``.
     """
 
     def __init__(self, tau: float = 2.0, decay_input: bool = True, v_threshold: float = 1.0,
@@ -25,9 +25,7 @@ class LIFNode(BaseNode):
 
     @property
     def supported_backends(self):
-        if self.step_mode == "s":
-            return ("torch",)
-        if self.step_mode == "m":
+        if self.step_mode in ("s", "m"):
             return ("torch", "hip")
         raise ValueError(self.step_mode)
 
@@ -35,10 +33,15 @@ class LIFNode(BaseNode):
         return super().extra_repr() + f", tau={self.tau}"
 
     def single_step_functional_forward(self, inputs, states, **kwargs):
-        if self.backend != "torch":
+        if self.backend == "hip":
+            self._check_hip_surrogate()
+            spike, v = functional.lif_step_hip(inputs[0], states[0], self.tau, self.decay_input, self.v_threshold,
+                                               self.v_reset, self.surrogate_function, self.detach_reset)
+        elif self.backend == "torch":
+            spike, v = functional.lif_step(inputs[0], states[0], self.tau, self.decay_input, self.v_threshold,
+                                           self.v_reset, self._torch_surrogate(), self.detach_reset)
+        else:
             raise ValueError(self.backend)
-        spike, v = functional.lif_step(inputs[0], states[0], self.tau, self.decay_input, self.v_threshold,
-                                       self.v_reset, self._torch_surrogate(), self.detach_reset)
         return (spike,), (v, *states[1:])
 
     def _hip_multi_step(self, x_seq, v, store_v_seq):

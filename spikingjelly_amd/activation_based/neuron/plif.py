@@ -15,7 +15,7 @@ from .base_node import BaseNode
 class ParametricLIFNode(BaseNode):
     """LIF whose ``1/tau = sigmoid(w)`` is learned; ``w`` starts at ``-log(init_tau - 1)``.
 
-    Multi-step mode supports ``backend='torch'`` and ``backend='hip'``.  Unlike IF/LIF the torch
+    Both step modes support ``backend='torch'`` and ``backend='hip'``.  Unlike IF/LIF the torch
     backend keeps the surrogate in eval mode (reference neuron/plif.py:170-186).
     """
 
@@ -30,9 +30,7 @@ class ParametricLIFNode(BaseNode):
 
     @property
     def supported_backends(self):
-        if self.step_mode == "s":
-            return ("torch",)
-        if self.step_mode == "m":
+        if self.step_mode in ("s", "m"):
             return ("torch", "hip")
         raise ValueError(self.step_mode)
 
@@ -42,10 +40,14 @@ class ParametricLIFNode(BaseNode):
         return super().extra_repr() + f", tau={tau}"
 
     def single_step_functional_forward(self, inputs, states, **kwargs):
-        if self.backend != "torch":
+        if self.backend == "hip":
+            spike, v = functional.plif_step_hip(inputs[0], states[0], self.w, self.decay_input, self.v_threshold,
+                                                self.v_reset, self.surrogate_function, self.detach_reset)
+        elif self.backend == "torch":
+            spike, v = functional.plif_step(inputs[0], states[0], self.w, self.decay_input, self.v_threshold,
+                                            self.v_reset, self.surrogate_function, self.detach_reset)
+        else:
             raise ValueError(self.backend)
-        spike, v = functional.plif_step(inputs[0], states[0], self.w, self.decay_input, self.v_threshold,
-                                        self.v_reset, self.surrogate_function, self.detach_reset)
         return (spike,), (v, *states[1:])
 
     def _check_hip_surrogate(self):

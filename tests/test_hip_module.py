@@ -186,7 +186,50 @@ def test_fp32_state_mode_for_bf16_plif():
 def test_set_backend_switches_supported_modules_only():
     net = torch.nn.Sequential(neuron.LIFNode(step_mode="m"), torch.nn.Linear(4, 4), neuron.IFNode(step_mode="s"))
     functional.set_backend(net, "hip")
-    assert net[0].backend == "hip" and net[2].backend == "torch"
+    assert net[0].backend == "hip" and net[2].backend == "hip" and not hasattr(net[1], "backend")
+
+
+@pytest.mark.parametrize("cls,kw", [
+    (neuron.IFNode, {}),
+    (neuron.LIFNode, {"tau": 3.0}),
+    (neuron.LIFNode, {"tau": 2.0, "decay_input": False}),
+    (neuron.ParametricLIFNode, {"init_tau": 2.0}),
+])
+@pytest.mark.parametrize("v_reset", [0.0, None])
+@pytest.mark.parametrize("detach_reset", [False, True])
+def test_single_step_hip_loop_matches_multi_step_torch(cls, kw, v_reset, detach_reset):
+    """step_mode='s' with backend='hip' (the reference's single-step kernel backends,
+    functional/neuron.py:1709-1886): a Python loop over T single steps, state and its gradient carried
+    through self.v between kernel calls, equals the torch backend's multi-step run."""
+    T = 5
+    a = cls(step_mode="m", backend="torch", v_threshold=0.5, v_reset=v_reset, detach_reset=detach_reset,
+            surrogate_function=surrogate.ATan(), **kw)
+    b = cls(step_mode="s", backend="hip", v_threshold=0.5, v_reset=v_reset, detach_reset=detach_reset,
+            surrogate_function=surrogate.ATan(), **kw).cuda()
+    x = seeded_randn((T, 3, 40), 77, 0.3, 1.0)
+    g = seeded_randn((T, 3, 40), 78)
+    xa, xb = x.clone().requires_grad_(), x.cuda().requires_grad_()
+    sa = a(xa)
+    sb = torch.stack([b(xb[t]) for t in range(T)])
+    assert bits_equal(sb.cpu(), sa.detach())
+    assert bits_equal(b.v.detach().cpu(), a.v.detach())
+    ((sa * g).sum() + 0.5 * a.v.sum()).backward()
+    ((sb * g.cuda()).sum() + 0.5 * b.v.sum()).backward()
+    torch.testing.assert_close(xb.grad.cpu(), xa.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+    if cls is neuron.ParametricLIFNode:
+        torch.testing.assert_close(b.w.grad.cpu(), a.w.grad, rtol=1e-4, atol=1e-5)
+
+
+def test_single_step_functionals_return_spike_and_state():
+    x = seeded_randn((4, 33), 79, 0.6, 1.0).cuda()
+    v = torch.zeros_like(x)
+    es, ev, _ = no.multi_step("lif", x.cpu().unsqueeze(0), v.cpu(), 2.0, True, 1.0, 0.0)
+    s, v_next = functional.lif_step_hip(x, v, 2.0, True, 1.0, 0.0, surrogate.ATan())
+    assert s.shape == x.shape and v_next.shape == x.shape
+    assert bits_equal(s.cpu(), es[0]) and bits_equal(v_next.cpu(), ev[0])
+    s, v_next = functional.if_step_hip(x, v, 1.0, None, surrogate.Sigmoid())
+    es, ev, _ = no.multi_step("if", x.cpu().unsqueeze(0), v.cpu(), None, True, 1.0, None)
+    assert bits_equal(s.cpu(), es[0]) and bits_equal(v_next.cpu(), ev[0])
 
 
 @pytest.mark.parametrize("cls", [neuron.IFNode, neuron.LIFNode, neuron.ParametricLIFNode])

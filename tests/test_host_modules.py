@@ -102,9 +102,9 @@ def test_memory_semantics():
 
 def test_backend_and_step_mode_validation():
     node = neuron.LIFNode()
-    assert node.supported_backends == ("torch",)
-    with pytest.raises(NotImplementedError, match="hip is not a supported backend"):
-        node.backend = "hip"  # single-step mode has no hip backend
+    assert node.supported_backends == ("torch", "hip")  # both step modes have the hip backend
+    with pytest.raises(NotImplementedError, match="triton is not a supported backend"):
+        node.backend = "triton"
     node.step_mode = "m"
     assert node.supported_backends == ("torch", "hip")
     node.backend = "hip"
