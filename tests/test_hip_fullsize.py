@@ -1,4 +1,4 @@
-"""Full-size checks (BASELINE config 2: T=16, N=33.5M fp32) through size-independent properties.
+"""Full-size checks (BASELINE configs 2 to 5 at their real shapes) through size-independent properties.
 
 Neurons are independent, so any subset of columns of the full-size GPU result must equal the C oracle
 run on those columns alone -- that covers every address range of the 2.1 GB tensors without a 30 GB
@@ -54,3 +54,129 @@ def test_config2_full_size_forward_backward(c_oracle):
     assert bool((v_seq[fired] == 0.0).all())
     assert bool((v_seq[~fired] < 1.0).all())
     assert bool(torch.isfinite(x.grad).all())
+
+
+def _column_blocks(n_cols: int, width: int = 4096, count: int = 30, seed: int = 0):
+    rng = np.random.default_rng(seed)
+    starts = np.concatenate([[0, n_cols - width], rng.integers(0, n_cols - width, size=count)])
+    return np.concatenate([np.arange(a, a + width) for a in starts])
+
+
+def test_config3_full_size_plif_bf16_fp32_state(c_oracle):
+    """BASELINE config 3 at full size: ParametricLIF (init_tau=2, so k = 1/2 exactly), soft reset, Sigmoid(4),
+    x [8,128,256,16,16] bf16 with fp32 state.  The C oracle runs the whole tensor (fp32 arithmetic on the
+    bf16-representable inputs is the fp32-state semantics): every spike must match, stored v_seq must be the
+    oracle's v rounded to bf16, grad_x agrees to bf16 accuracy, and the global dL/dw -- one scalar reduced
+    over 67 M terms -- agrees with the float64 recurrence and is additive over a split of the neurons."""
+    from spikingjelly_amd import configure
+    from spikingjelly_amd.activation_based import functional, neuron, surrogate
+
+    Tc, Nc = 8, 128 * 256 * 16 * 16
+    g = torch.Generator().manual_seed(1003)
+    x = (torch.randn((Tc, Nc), generator=g) * 1.0 + 0.2).bfloat16()
+    gs = torch.randn((Tc, Nc), generator=torch.Generator().manual_seed(1103)).bfloat16()
+    gv = (torch.randn((Tc, Nc), generator=torch.Generator().manual_seed(1203)) * 0.1).bfloat16()
+    old = configure.hip_half_precision_mode
+    configure.hip_half_precision_mode = "fp32_state"
+    try:
+        node = neuron.ParametricLIFNode(init_tau=2.0, v_reset=None, surrogate_function=surrogate.Sigmoid(4.0),
+                                        step_mode="m", backend="hip", store_v_seq=True).cuda()
+        xd = x.cuda().requires_grad_()
+        s = node(xd)
+        torch.autograd.backward([s, node.v_seq], [gs.cuda(), gv.cuda()])
+        torch.cuda.synchronize()
+        rate = float(s.detach().float().mean())
+        assert 0.03 < rate < 0.09, rate
+
+        es, ev, eh = c_oracle.forward_f32("plif", x.float().numpy(), np.zeros(Nc, np.float32), 0.5, True, 1.0, None)
+        assert np.array_equal(s.detach().float().cpu().numpy(), es)
+        assert torch.equal(node.v_seq.detach().cpu(), torch.from_numpy(ev).bfloat16())
+        assert torch.equal(node.v.detach().cpu(), torch.from_numpy(ev[-1]).bfloat16())
+
+        gx, _, gk = c_oracle.backward_f64("plif", gs.float().numpy(), gv.float().numpy(), None, eh, 0.5, True, 1.0, None,
+                                          False, 0, 4.0, x_seq=x.float().numpy(), v_init=np.zeros(Nc, np.float32), v_seq=ev)
+        cols = _column_blocks(Nc)
+        np.testing.assert_allclose(xd.grad.float().cpu().numpy()[:, cols], gx[:, cols], rtol=1e-2, atol=2e-3)
+        dw = float(node.w.grad)
+        assert abs(dw - gk * 0.25) <= 2e-3 * abs(gk * 0.25) + 1e-3, (dw, gk * 0.25)  # dL/dw = dL/dk k (1 - k)
+
+        # additivity of the reduction over a split of the neurons
+        parts = []
+        for lo, hi in ((0, Nc // 2), (Nc // 2, Nc)):
+            functional.reset_net(node)
+            node.w.grad = None
+            xi = x[:, lo:hi].contiguous().cuda().requires_grad_()
+            si = node(xi)
+            torch.autograd.backward([si, node.v_seq], [gs[:, lo:hi].contiguous().cuda(), gv[:, lo:hi].contiguous().cuda()])
+            parts.append(float(node.w.grad))
+        assert abs(sum(parts) - dw) <= 1e-4 * abs(dw) + 1e-4, (parts, dw)
+    finally:
+        configure.hip_half_precision_mode = old
+
+
+def test_config4_full_size_if_fp16_inference_and_packing():
+    """BASELINE config 4 at full size: IF, soft reset, fp16, x [32,64,512,14,14] uniform[0,0.25); spikes are
+    bit-packed and unpacked again.  Column blocks must equal the torch-ops oracle on the same half tensors;
+    over the whole tensor the packed bytes must equal numpy.packbits of the spikes, the unpacked tensor the
+    spikes, the fused packed-output kernel the two-kernel result, and the firing rate the input mean."""
+    from oracle import neuron_oracle as no
+    from spikingjelly_amd import configure
+    from spikingjelly_amd.activation_based import functional
+    from spikingjelly_amd.activation_based.hip_kernel.compress import bit_spike_compress, bit_spike_decompress
+
+    Tc, Nc = 32, 64 * 512 * 14 * 14
+    x = (torch.rand((Tc, Nc), generator=torch.Generator().manual_seed(1004)) * 0.25).half()
+    old = configure.hip_half_precision_mode
+    configure.hip_half_precision_mode = "torch"
+    try:
+        xd = x.cuda()
+        v0 = torch.zeros(Nc, dtype=torch.float16, device="cuda")
+        with torch.no_grad():
+            s, v_next, _ = functional.if_multi_step_hip(xd, v0, 1.0, None, None)
+            packed = bit_spike_compress(s)
+            back = bit_spike_decompress(packed, s.shape, dtype=torch.float16)
+            fused, v_next_f, _ = functional.if_multi_step_hip_packed(xd, v0, 1.0, None)
+        torch.cuda.synchronize()
+    finally:
+        configure.hip_half_precision_mode = old
+    assert packed.numel() == Tc * Nc // 8
+    assert torch.equal(back, s)
+    assert torch.equal(fused, packed) and torch.equal(v_next_f, v_next)
+    s_cpu = s.cpu()
+    assert np.array_equal(packed.cpu().numpy(), np.packbits(s_cpu.numpy().reshape(-1).astype(bool), bitorder="little"))
+    rate = float(s_cpu.float().mean())
+    assert 0.10 < rate < 0.125, rate  # tends to the input mean 0.125 once the membranes have charged
+
+    cols = torch.from_numpy(_column_blocks(Nc, width=2048, count=14, seed=4))
+    es, ev, _ = no.multi_step("if", x[:, cols], torch.zeros(cols.numel(), dtype=torch.float16), None, True, 1.0, None)
+    assert torch.equal(s_cpu[:, cols], es)
+    assert torch.equal(v_next.cpu()[cols], ev[-1])
+
+
+def test_config5_full_size_block_matches_torch_backend():
+    """BASELINE config 5 at full size (T=4, B=64, 196 tokens, D=384, 12 heads): the block with backend='hip'
+    against the same block with backend='torch' on the same device and weights.  Convolutions and batch norms
+    are the same torch kernels, the LIF kernels are bit-exact and the contraction is exact, so the output
+    spikes must be identical; gradients agree to fp32 accuracy."""
+    from spikingjelly_amd.activation_based import functional, layer
+
+    from helpers import bits_equal
+
+    torch.manual_seed(1005)
+    a = layer.SpikingSelfAttention(384, 12, backend="torch").cuda()
+    b = layer.SpikingSelfAttention(384, 12, backend="hip").cuda()
+    b.load_state_dict(a.state_dict())
+    x = torch.randn((4, 64, 384, 196), generator=torch.Generator().manual_seed(1105)).cuda()
+    g = torch.randn((4, 64, 384, 196), generator=torch.Generator().manual_seed(1205)).cuda()
+    xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
+    ya = a(xa)
+    ya.backward(g)
+    yb = b(xb)
+    yb.backward(g)
+    torch.cuda.synchronize()
+    assert 0.0 < float(ya.detach().mean()) < 0.5
+    assert bits_equal(yb, ya)
+    torch.testing.assert_close(xb.grad, xa.grad, rtol=1e-3, atol=1e-4)
+    torch.testing.assert_close(b.proj_conv_bn[0].weight.grad, a.proj_conv_bn[0].weight.grad, rtol=1e-3, atol=1e-3)
+    functional.reset_net(a)
+    functional.reset_net(b)
