@@ -87,6 +87,10 @@ typedef enum sjhip_surrogate {
 #define SJHIP_FLAG_ATOMIC_REDUCE 0x80u /* PLIF backward: one atomicAdd per block into grad_rtau (caller
                                           zeroes it) instead of the deterministic two-pass reduction */
 
+#define SJHIP_FLAG_V_INIT_BROADCAST 0x100u /* v_init points to ONE element that every neuron starts from (a
+                                              module state that is still its scalar reset value): no [N]
+                                              tensor has to be filled and read */
+
 /* Scalars of one neuron layer.  `tau` is tau for LIF and the reciprocal k = sigmoid(w) for PLIF
  * (ignored for IF).  `v_reset` is ignored for IF soft reset and is the charge-equation offset
  * (0 when the module has v_reset=None) otherwise. */
@@ -107,7 +111,7 @@ const char *sjhip_last_error(void);
 
 /*
  * Forward over T steps for N neurons.
- *   x_seq     [T,N] in            v_init  [N] in
+ *   x_seq     [T,N] in            v_init  [N] in ([1] with SJHIP_FLAG_V_INIT_BROADCAST)
  *   spike_seq [T,N] out (0/1 in the storage dtype)
  *   v_seq     [T,N] out, membrane potential after reset at every step; NULL = do not write
  *   v_last    [N] out, membrane potential after the last step; NULL = do not write
@@ -151,8 +155,9 @@ int64_t sjhip_plif_workspace_floats(int dtype, int64_t N);
  *   grad_v_seq     [T,N] in, gradient w.r.t. v_seq, or NULL
  *   grad_v_last    [N] in, gradient w.r.t. v_last (enters at t = T-1), or NULL
  *   h_seq          [T,N] in (from forward)
- *   v_init         [N] in, PLIF only (NULL otherwise): v before step 0
- *   grad_x_seq     [T,N] out         grad_v_init [N] out
+ *   v_init         [N] in ([1] with SJHIP_FLAG_V_INIT_BROADCAST), PLIF only (NULL otherwise): v before step 0
+ *   grad_x_seq     [T,N] out
+ *   grad_v_init    [N] out, or NULL when the caller does not need the gradient of the initial state
  *   grad_rtau      1 float out, PLIF only: dL/dk, k = sigmoid(w)
  *   workspace      sjhip_plif_workspace_floats() floats, PLIF without SJHIP_FLAG_ATOMIC_REDUCE
  */

@@ -25,6 +25,7 @@ FLAG_DETACH_RESET = 0x04
 FLAG_FP32_STATE = 0x10
 FLAG_RECIPROCAL_TAU = 0x20
 FLAG_ATOMIC_REDUCE = 0x80
+FLAG_V_INIT_BROADCAST = 0x100
 
 KC_FORWARD, KC_BACKWARD, KC_PLIF_REDUCE, KC_BIT_PACK, KC_BIT_UNPACK, KC_SSA_FORWARD, KC_SSA_BACKWARD = range(7)
 

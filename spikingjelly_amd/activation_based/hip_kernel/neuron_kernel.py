@@ -67,6 +67,19 @@ def _check_inputs(x_seq: torch.Tensor, v_init: torch.Tensor) -> None:
         raise ValueError(f"x_seq must have T >= 1 and N >= 1, got shape {tuple(x_seq.shape)}")
 
 
+def _is_broadcast_state(v: torch.Tensor) -> bool:
+    """An expanded one-element tensor (every stride 0): what a node passes while its state is still the
+    scalar reset value.  The kernels then read that one element instead of an [N] tensor."""
+    return v.numel() > 1 and all(st == 0 for st in v.stride())
+
+
+def _state_arg(v_init: torch.Tensor, align: bool) -> tuple[torch.Tensor, int]:
+    """(tensor to keep alive, SJHIP_FLAG_V_INIT_BROADCAST or 0)."""
+    if _is_broadcast_state(v_init):
+        return v_init, L.FLAG_V_INIT_BROADCAST
+    return (L.aligned16(v_init) if align else v_init.contiguous()), 0
+
+
 def _k_pointer(k: Optional[torch.Tensor], ref: torch.Tensor) -> tuple[Optional[torch.Tensor], Optional[int]]:
     if k is None:
         return None, None
@@ -81,14 +94,14 @@ def _run_forward(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: Opti
     _check_inputs(x_seq, v_init)
     dtype = L.dtype_id(x_seq.dtype)
     x_seq = x_seq.contiguous()
-    v_init = v_init.contiguous()
+    v_init, broadcast = _state_arg(v_init, False)
     T, N = x_seq.shape
     spike_seq = torch.empty_like(x_seq)
     v_seq = torch.empty_like(x_seq) if store_v_seq else x_seq.new_empty((0,))
-    v_last = torch.empty_like(v_init)
+    v_last = x_seq.new_empty((N,))
     h_seq = torch.empty_like(x_seq) if save_h else None
     k_keep, k_ptr = _k_pointer(k, x_seq)
-    params = _params(tau, v_th, v_reset, 0.0, 0, flags)
+    params = _params(tau, v_th, v_reset, 0.0, 0, flags | broadcast)
     with torch.cuda.device(x_seq.device):
         rc = L.load().sjhip_neuron_forward(
             neuron, dtype, ctypes.byref(params), T, N,
@@ -112,15 +125,15 @@ def _run_forward_packed(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, 
     _check_inputs(x_seq, v_init)
     dtype = L.dtype_id(x_seq.dtype)
     x_seq = x_seq.contiguous()
-    v_init = v_init.contiguous()
+    v_init, broadcast = _state_arg(v_init, False)
     T, N = x_seq.shape
     if not packed_supported(N):
         raise NotImplementedError(f"packed spike output needs N % 8 == 0, got N={N}")
     spike_bits = torch.empty((T * N // 8,), dtype=torch.uint8, device=x_seq.device)
     v_seq = torch.empty_like(x_seq) if store_v_seq else x_seq.new_empty((0,))
-    v_last = torch.empty_like(v_init)
+    v_last = x_seq.new_empty((N,))
     k_keep, k_ptr = _k_pointer(k, x_seq)
-    params = _params(tau, v_th, v_reset, 0.0, 0, flags)
+    params = _params(tau, v_th, v_reset, 0.0, 0, flags | broadcast)
     with torch.cuda.device(x_seq.device):
         rc = L.load().sjhip_neuron_forward_packed(
             neuron, dtype, ctypes.byref(params), T, N,
@@ -148,7 +161,7 @@ def _forward_outputs(out, x_seq: torch.Tensor):
 def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
                   grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor, x_seq: Optional[torch.Tensor],
                   v_init: Optional[torch.Tensor], k: Optional[torch.Tensor], tau: float, v_th: float,
-                  v_reset: float, flags: int, sg_id: int, sg_alpha: float
+                  v_reset: float, flags: int, sg_id: int, sg_alpha: float, need_grad_v_init: bool = True
                   ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     recompute = x_seq is not None
     if not recompute and h_seq is None:
@@ -156,11 +169,13 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
     if recompute:
         # replay path: every buffer must be 16-byte aligned for the 128-bit kernel
         h_seq = L.aligned16(x_seq)
-        v_init = L.aligned16(v_init)
         fix = L.aligned16
     else:
         h_seq = h_seq.contiguous()
         fix = lambda t: t.contiguous()
+    if v_init is not None:
+        v_init, broadcast = _state_arg(v_init, recompute)
+        flags |= broadcast
     L.require_device_tensor("h_seq", h_seq)
     dtype = L.dtype_id(h_seq.dtype)
     T, N = h_seq.shape
@@ -172,11 +187,11 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
     if grad_v_last is not None:
         grad_v_last = fix(grad_v_last.to(h_seq.dtype))
     grad_x_seq = torch.empty_like(h_seq)
-    grad_v_init = h_seq.new_empty((N,))
+    # a state that needs no gradient (the usual case: it was the reset value) costs no [N] write
+    grad_v_init = h_seq.new_empty((N,) if need_grad_v_init else (0,))
     grad_k = workspace = None
     k_keep, k_ptr = _k_pointer(k, h_seq)
     if neuron == L.NEURON_PLIF:
-        v_init = v_init.contiguous()
         if flags & L.FLAG_ATOMIC_REDUCE:
             grad_k = torch.zeros((), dtype=torch.float32, device=h_seq.device)
         else:
@@ -190,15 +205,15 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
                 neuron, dtype, ctypes.byref(params), T, N,
                 h_seq.data_ptr(), v_init.data_ptr(), k_ptr,
                 grad_spike_seq.data_ptr(), L.ptr(grad_v_seq), L.ptr(grad_v_last),
-                grad_x_seq.data_ptr(), grad_v_init.data_ptr(), L.ptr(grad_k), L.ptr(workspace),
-                L.current_stream_ptr(h_seq.device),
+                grad_x_seq.data_ptr(), grad_v_init.data_ptr() if need_grad_v_init else None, L.ptr(grad_k),
+                L.ptr(workspace), L.current_stream_ptr(h_seq.device),
             )
         else:
             rc = L.load().sjhip_neuron_backward(
                 neuron, dtype, ctypes.byref(params), T, N,
                 grad_spike_seq.data_ptr(), L.ptr(grad_v_seq), L.ptr(grad_v_last), h_seq.data_ptr(),
                 L.ptr(v_init) if neuron == L.NEURON_PLIF else None, k_ptr,
-                grad_x_seq.data_ptr(), grad_v_init.data_ptr(), L.ptr(grad_k), L.ptr(workspace),
+                grad_x_seq.data_ptr(), grad_v_init.data_ptr() if need_grad_v_init else None, L.ptr(grad_k), L.ptr(workspace),
                 L.current_stream_ptr(h_seq.device),
             )
     L.check(rc, "neuron_backward_recompute" if recompute else "neuron_backward")
@@ -266,18 +281,19 @@ def hip_multistep_if_backward(grad_spike_seq: Optional[torch.Tensor], grad_v_seq
                               grad_v_last: Optional[torch.Tensor], h_seq: Optional[torch.Tensor],
                               x_seq: Optional[torch.Tensor], v_init: Optional[torch.Tensor], v_th: float,
                               v_reset: float, soft_reset: bool, detach_reset: bool, sg_id: int,
-                              sg_alpha: float, mode_flags: int) -> tuple[torch.Tensor, torch.Tensor]:
+                              sg_alpha: float, mode_flags: int, need_grad_v_init: bool = True
+                              ) -> tuple[torch.Tensor, torch.Tensor]:
     flags = _flags(soft_reset, detach_reset, False, mode_flags)
     gx, gvi, _ = _run_backward(L.NEURON_IF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, None,
-                               0.0, v_th, v_reset, flags, sg_id, sg_alpha)
+                               0.0, v_th, v_reset, flags, sg_id, sg_alpha, need_grad_v_init)
     return gx, gvi
 
 
 @hip_multistep_if_backward.register_fake
 def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, v_th, v_reset, soft_reset, detach_reset,
-      sg_id, sg_alpha, mode_flags):
+      sg_id, sg_alpha, mode_flags, need_grad_v_init=True):
     ref = h_seq if h_seq is not None else x_seq
-    return torch.empty_like(ref), ref.new_empty(ref.shape[1:])
+    return torch.empty_like(ref), ref.new_empty(ref.shape[1:] if need_grad_v_init else (0,))
 
 
 def _if_setup_context(ctx, inputs, output):
@@ -301,10 +317,11 @@ def _if_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_s
     del grad_h_seq
     h_seq, x_seq, v_init = _split_saved(ctx)
     v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, mode_flags = ctx.scalars
+    need = bool(ctx.needs_input_grad[1])
     gx, gvi = hip_multistep_if_backward(
         grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, x_seq, v_init,
-        v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, mode_flags)
-    return gx, gvi, None, None, None, None, None, None, None, None, None
+        v_th, v_reset, soft_reset, detach_reset, sg_id, sg_alpha, mode_flags, need)
+    return gx, (gvi if need else None), None, None, None, None, None, None, None, None, None
 
 
 torch.library.register_autograd("sj::hip_multistep_if_forward", _if_autograd_backward,
@@ -349,19 +366,19 @@ def hip_multistep_lif_backward(grad_spike_seq: Optional[torch.Tensor], grad_v_se
                                grad_v_last: Optional[torch.Tensor], h_seq: Optional[torch.Tensor],
                                x_seq: Optional[torch.Tensor], v_init: Optional[torch.Tensor], v_th: float,
                                v_reset: float, soft_reset: bool, detach_reset: bool, tau: float,
-                               decay_input: bool, sg_id: int, sg_alpha: float, mode_flags: int
-                               ) -> tuple[torch.Tensor, torch.Tensor]:
+                               decay_input: bool, sg_id: int, sg_alpha: float, mode_flags: int,
+                               need_grad_v_init: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
     flags = _flags(soft_reset, detach_reset, decay_input, mode_flags)
     gx, gvi, _ = _run_backward(L.NEURON_LIF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, None,
-                               tau, v_th, v_reset, flags, sg_id, sg_alpha)
+                               tau, v_th, v_reset, flags, sg_id, sg_alpha, need_grad_v_init)
     return gx, gvi
 
 
 @hip_multistep_lif_backward.register_fake
 def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, v_th, v_reset, soft_reset, detach_reset,
-      tau, decay_input, sg_id, sg_alpha, mode_flags):
+      tau, decay_input, sg_id, sg_alpha, mode_flags, need_grad_v_init=True):
     ref = h_seq if h_seq is not None else x_seq
-    return torch.empty_like(ref), ref.new_empty(ref.shape[1:])
+    return torch.empty_like(ref), ref.new_empty(ref.shape[1:] if need_grad_v_init else (0,))
 
 
 def _lif_setup_context(ctx, inputs, output):
@@ -376,10 +393,11 @@ def _lif_setup_context(ctx, inputs, output):
 def _lif_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_seq):
     del grad_h_seq
     h_seq, x_seq, v_init = _split_saved(ctx)
+    need = bool(ctx.needs_input_grad[1])
     gx, gvi = hip_multistep_lif_backward(
         grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, x_seq, v_init,
-        *ctx.scalars)
-    return gx, gvi, None, None, None, None, None, None, None, None, None, None, None
+        *ctx.scalars, need)
+    return gx, (gvi if need else None), None, None, None, None, None, None, None, None, None, None, None
 
 
 torch.library.register_autograd("sj::hip_multistep_lif_forward", _lif_autograd_backward,
@@ -426,19 +444,20 @@ def hip_multistep_plif_backward(grad_spike_seq: Optional[torch.Tensor], grad_v_s
                                 x_seq: Optional[torch.Tensor], v_init: torch.Tensor, k: torch.Tensor,
                                 v_th: float, v_reset: float,
                                 soft_reset: bool, detach_reset: bool, decay_input: bool, sg_id: int,
-                                sg_alpha: float, mode_flags: int
+                                sg_alpha: float, mode_flags: int, need_grad_v_init: bool = True
                                 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     flags = _flags(soft_reset, detach_reset, decay_input, mode_flags)
     gx, gvi, gk = _run_backward(L.NEURON_PLIF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, k,
-                                0.0, v_th, v_reset, flags, sg_id, sg_alpha)
+                                0.0, v_th, v_reset, flags, sg_id, sg_alpha, need_grad_v_init)
     return gx, gvi, gk
 
 
 @hip_multistep_plif_backward.register_fake
 def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, k, v_th, v_reset, soft_reset,
-      detach_reset, decay_input, sg_id, sg_alpha, mode_flags):
+      detach_reset, decay_input, sg_id, sg_alpha, mode_flags, need_grad_v_init=True):
     ref = h_seq if h_seq is not None else x_seq
-    return (torch.empty_like(ref), ref.new_empty(ref.shape[1:]), ref.new_empty((), dtype=torch.float32))
+    return (torch.empty_like(ref), ref.new_empty(ref.shape[1:] if need_grad_v_init else (0,)),
+            ref.new_empty((), dtype=torch.float32))
 
 
 def _plif_setup_context(ctx, inputs, output):
@@ -460,11 +479,12 @@ def _plif_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h
     del grad_h_seq
     first, v_init, k = ctx.saved_tensors
     h_seq, x_seq = (None, first) if ctx.recompute else (first, None)
+    need = bool(ctx.needs_input_grad[1])
     gx, gvi, gk = hip_multistep_plif_backward(
         grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, x_seq, v_init, k,
-        *ctx.scalars)
+        *ctx.scalars, need)
     gk = gk.reshape(ctx.k_shape).to(ctx.k_dtype)
-    return gx, gvi, gk, None, None, None, None, None, None, None, None, None, None
+    return gx, (gvi if need else None), gk, None, None, None, None, None, None, None, None, None, None
 
 
 torch.library.register_autograd("sj::hip_multistep_plif_forward", _plif_autograd_backward,

@@ -107,14 +107,23 @@ class BaseNode(base.MemoryModule):
         outputs = tuple(torch.stack(seq) for seq in zip(*per_step, strict=True))
         return outputs[0] if len(outputs) == 1 else outputs
 
+    def _constant_state(self, x: torch.Tensor, value: float) -> torch.Tensor:
+        """The state every neuron starts from, with the shape of ``x`` (reference: ``torch.full_like``,
+        neuron/base_node.py:474-475).  The hip kernels read a constant state from a single element, so for that
+        backend it is a one-element tensor expanded to the shape (read-only, never written back: the next
+        state is the kernel's own output) and no ``[N]`` tensor is filled or read."""
+        if self.backend == "hip" and x.is_cuda and x.numel() > 1:
+            return x.new_full((1,) * x.dim(), value).expand(x.shape)
+        return torch.full_like(x, value, requires_grad=False)
+
     def materialize_states(self, inputs, states, step_mode: str):
         x = inputs[0][0] if step_mode == "m" else inputs[0]
         v = states[0]
         if isinstance(v, float):
-            v = torch.full_like(x, v, requires_grad=False)
+            v = self._constant_state(x, v)
         elif isinstance(v, torch.Tensor):
             if v.shape != x.shape:  # e.g. batch size changed: start again from the reset value
-                v = torch.full_like(x, self.v_reset if self.v_reset is not None else 0.0, requires_grad=False)
+                v = self._constant_state(x, self.v_reset if self.v_reset is not None else 0.0)
             elif v.dtype != x.dtype or v.device != x.device:
                 v = v.to(dtype=x.dtype, device=x.device)
         return (v, *states[1:])

@@ -57,6 +57,7 @@ struct BwdArgs {
   int decay_input;
   int is_if;
   int atomic_reduce;
+  int v_init_broadcast;  // v_init holds one element for all neurons
 };
 
 // FAST (16-bit storage, where the result is rounded to 8 or 11 significant bits anyway) uses the hardware
@@ -238,10 +239,10 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
       }
     }
   }
-  A::store((E *)a.grad_v_init + col, carry);
+  if (a.grad_v_init) A::store((E *)a.grad_v_init + col, carry);
   if (PLIF) {
     float v0[V];
-    A::unpack(A::load((const E *)a.v_init + col), v0);
+    load_state<S, VECTOR, SJHIP_BWD_NT != 0>(a.v_init, col, a.v_init_broadcast != 0, v0);
 #pragma unroll
     for (int j = 0; j < V; ++j) {
       const float dh_dk = a.decay_input ? (h_next[j] - v0[j]) : (a.v_reset - v0[j]);
@@ -323,6 +324,7 @@ inline int build_bwd_args(BwdArgs &a, int neuron, int dtype, const sjhip_neuron_
   a.decay_input = (p.flags & SJHIP_FLAG_DECAY_INPUT) ? 1 : 0;
   a.is_if = neuron == SJHIP_NEURON_IF;
   a.atomic_reduce = (p.flags & SJHIP_FLAG_ATOMIC_REDUCE) ? 1 : 0;
+  a.v_init_broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) ? 1 : 0;
   const bool detach = (p.flags & SJHIP_FLAG_DETACH_RESET) != 0;
   if (a.soft_reset) { a.cB = 0.0f; a.cC = detach ? 0.0f : -p.v_threshold; a.cD = 0.0f; }
   else { a.cB = 1.0f; a.cC = detach ? 0.0f : p.v_reset; a.cD = detach ? 0.0f : 1.0f; }

@@ -82,9 +82,9 @@ int launch_backward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t
   const int esize = dtype == SJHIP_F32 ? 4 : 2;
   const int V = 16 / esize;
   const bool vector = (N % V == 0) && aligned16(grad_spike_seq) && aligned16(h_seq) && aligned16(grad_x_seq) &&
-                      aligned16(grad_v_init) && (grad_v_seq == nullptr || aligned16(grad_v_seq)) &&
+                      (grad_v_init == nullptr || aligned16(grad_v_init)) && (grad_v_seq == nullptr || aligned16(grad_v_seq)) &&
                       (grad_v_last == nullptr || aligned16(grad_v_last)) &&
-                      (v_init == nullptr || aligned16(v_init));
+                      (v_init == nullptr || a.v_init_broadcast || aligned16(v_init));
 
   switch (dtype) {
     case SJHIP_F32: return launch_typed<float>(a, vector, plif, grad_rtau, stream);

@@ -40,7 +40,7 @@ __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, i
   for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? A::load(xp + (int64_t)i * N) : A::zero();
   typedef typename StepNum<S, ROUND_EACH>::type NUM;
   NUM v[V];
-  A::unpack(A::load((const E *)a.v_init + col), v);
+  load_state<S, true, SJHIP_BWD_NT != 0>(a.v_init, col, a.v_init_broadcast != 0, v);
 
   for (int64_t t0 = 0; t0 < T; t0 += PF) {
     typename A::raw_t cur[PF];

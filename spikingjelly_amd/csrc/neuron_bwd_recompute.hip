@@ -39,8 +39,10 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
   if (!recompute_supported(dtype, T, N))
     return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute): T=%lld N=%lld does not fit (N %% %d != 0 or T too large for LDS)",
                 (long long)T, (long long)N, dtype == SJHIP_F32 ? 4 : 8);
-  if (!aligned16(x_seq) || !aligned16(v_init) || !aligned16(grad_spike_seq) || !aligned16(grad_x_seq) ||
-      !aligned16(grad_v_init) || (grad_v_seq && !aligned16(grad_v_seq)) || (grad_v_last && !aligned16(grad_v_last)))
+  const bool broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) != 0;
+  if (!aligned16(x_seq) || (!broadcast && !aligned16(v_init)) || !aligned16(grad_spike_seq) || !aligned16(grad_x_seq) ||
+      (grad_v_init && !aligned16(grad_v_init)) || (grad_v_seq && !aligned16(grad_v_seq)) ||
+      (grad_v_last && !aligned16(grad_v_last)))
     return fail(SJHIP_ERR_INVALID, "backward(recompute): every tensor must be 16-byte aligned");
 
   FwdArgs f;

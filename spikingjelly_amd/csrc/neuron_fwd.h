@@ -57,6 +57,7 @@ struct FwdArgs {
   float vth_mul; // v_threshold as a factor
   int charge;
   int soft_reset;
+  int v_init_broadcast;  // v_init holds one element for all neurons
 };
 
 // One neuron, one step.  R::round() is applied to the result of every arithmetic op.
@@ -180,7 +181,7 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
 
   typedef typename StepNum<S, ROUND_EACH>::type NUM;
   NUM v[V];
-  A::unpack(A::load((const E *)a.v_init + col), v);
+  load_state<S, VECTOR, SJHIP_FWD_NT != 0>(a.v_init, col, a.v_init_broadcast != 0, v);
 
   for (int64_t t0 = 0; t0 < T; t0 += PF) {
     typename A::raw_t cur[PF];
@@ -241,6 +242,7 @@ inline int build_fwd_args(FwdArgs &a, bool &round_each, int neuron, int dtype, c
   a.k_device = nullptr;
   a.T = T; a.N = N;
   a.soft_reset = (p.flags & SJHIP_FLAG_SOFT_RESET) ? 1 : 0;
+  a.v_init_broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) ? 1 : 0;
   const bool decay_input = (p.flags & SJHIP_FLAG_DECAY_INPUT) != 0;
   round_each = dtype != SJHIP_F32 && !(p.flags & SJHIP_FLAG_FP32_STATE);
 

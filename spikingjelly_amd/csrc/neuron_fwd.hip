@@ -35,7 +35,7 @@ int launch_forward_packed(int neuron, int dtype, const sjhip_neuron_params &p, i
   bool round_each = false;
   int rc = build_fwd_args(a, round_each, neuron, dtype, p, T, N, x_seq, v_init, k_device, spike_bits, v_seq, v_last, nullptr);
   if (rc != SJHIP_OK) return rc;
-  const bool vector = aligned16(x_seq) && aligned16(v_init) && (v_seq == nullptr || aligned16(v_seq)) &&
+  const bool vector = aligned16(x_seq) && (a.v_init_broadcast || aligned16(v_init)) && (v_seq == nullptr || aligned16(v_seq)) &&
                       (v_last == nullptr || aligned16(v_last));
   switch (dtype) {
     case SJHIP_F32: return launch_typed<float, false, true>(a, vector, stream);
@@ -55,7 +55,7 @@ int launch_forward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t 
 
   const int esize = dtype == SJHIP_F32 ? 4 : 2;
   const int V = 16 / esize;
-  const bool vector = (N % V == 0) && aligned16(x_seq) && aligned16(v_init) && aligned16(spike_seq) &&
+  const bool vector = (N % V == 0) && aligned16(x_seq) && (a.v_init_broadcast || aligned16(v_init)) && aligned16(spike_seq) &&
                       (v_seq == nullptr || aligned16(v_seq)) && (v_last == nullptr || aligned16(v_last)) &&
                       (h_seq == nullptr || aligned16(h_seq));
 

@@ -174,7 +174,7 @@ int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p, i
   if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_ERF) return fail(SJHIP_ERR_UNSUPPORTED, "backward: surrogate id %d", p->sg_id);
   int rc = check_shape("backward", T, N);
   if (rc != SJHIP_OK) return rc;
-  if (!grad_spike_seq || !h_seq || !grad_x_seq || !grad_v_init) return fail(SJHIP_ERR_INVALID, "backward: NULL tensor");
+  if (!grad_spike_seq || !h_seq || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward: NULL tensor");
   if (neuron == SJHIP_NEURON_PLIF) {
     if (!v_init || !grad_rtau) return fail(SJHIP_ERR_INVALID, "backward: PLIF needs v_init and grad_rtau");
     if (!(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace) return fail(SJHIP_ERR_INVALID, "backward: PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");
@@ -199,7 +199,7 @@ int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_pa
   if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_ERF) return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute): surrogate id %d", p->sg_id);
   int rc = check_shape("backward(recompute)", T, N);
   if (rc != SJHIP_OK) return rc;
-  if (!x_seq || !v_init || !grad_spike_seq || !grad_x_seq || !grad_v_init) return fail(SJHIP_ERR_INVALID, "backward(recompute): NULL tensor");
+  if (!x_seq || !v_init || !grad_spike_seq || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward(recompute): NULL tensor");
   if (neuron == SJHIP_NEURON_PLIF) {
     if (!grad_rtau) return fail(SJHIP_ERR_INVALID, "backward(recompute): PLIF needs grad_rtau");
     if (!(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace) return fail(SJHIP_ERR_INVALID, "backward(recompute): PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");

@@ -178,6 +178,23 @@ template <bool NT> struct Acc<f16_t, false, NT> : Acc16s<f16_t, NT> {};
 template <bool NT> struct Acc<bf16_t, true, NT> : Acc16v<bf16_t, NT> {};
 template <bool NT> struct Acc<bf16_t, false, NT> : Acc16s<bf16_t, NT> {};
 
+// Initial state of this work-item's neurons: its V elements of the [N] tensor, or the one stored element
+// for every neuron when the caller passed a broadcast state.
+template <typename S, bool VECTOR, bool NT, typename NUM, int V>
+__device__ __forceinline__ void load_state(const void *p, int64_t col, bool broadcast, NUM (&v)[V]) {
+  typedef Acc<S, VECTOR, NT> A;
+  static_assert(A::V == V, "state width");
+  if (broadcast) {
+    typedef Acc<S, false, false> A1;
+    NUM one[1];
+    A1::unpack(A1::load((const typename A1::elem_t *)p), one);
+#pragma unroll
+    for (int j = 0; j < V; ++j) v[j] = one[0];
+  } else {
+    A::unpack(A::load((const typename A::elem_t *)p + col), v);
+  }
+}
+
 // ----------------------------------------------------------------------------------------------
 // Host-side services (defined in sjhip_api.hip).
 // ----------------------------------------------------------------------------------------------

@@ -334,3 +334,62 @@ def test_plif_reduction_is_deterministic_and_accurate(K, path):
     b = hip_backward(K, "plif", gs, None, None, h, v0, k, True, 1.0, None, False, 0, 4.0, x=xr)
     assert bits_equal(a[2], b[2])
     assert float(a[2]) == pytest.approx(float(ref["grad_p"]), rel=1e-5)
+
+
+# ------------------------------------------------------------------------------------------------
+# constant initial state passed as one broadcast element; optional grad_v_init
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("kind", ["if", "lif", "plif"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("recompute", [False, True])
+@pytest.mark.parametrize("T,N", [(5, 64), (3, 37)])
+def test_broadcast_initial_state_equals_a_filled_tensor(K, kind, dtype, recompute, T, N):
+    """An expanded one-element v_init (what a node passes while its state is the scalar reset value) must
+    give bit-identical outputs and gradients to the same value filled into an [N] tensor, on the 128-bit and
+    on the element-wise kernels, with h_seq saved or replayed."""
+    if recompute and N % 8 != 0:
+        pytest.skip("the replay kernel needs N % 4 (fp32) / N % 8 (16-bit) == 0; such shapes use the h_seq path")
+    x = seeded_randn((T, N), 41, 0.4, 1.0).to(dtype).cuda()
+    gs = seeded_randn((T, N), 42).to(dtype).cuda()
+    full = torch.full((N,), -0.25, dtype=dtype, device="cuda")
+    bcast = torch.full((1,), -0.25, dtype=dtype, device="cuda").expand(N)
+    assert bcast.stride() == (0,)
+    k = torch.tensor(0.5, device="cuda")
+    res = []
+    for v0 in (full, bcast):
+        xi = x.clone().requires_grad_()
+        ki = k.clone().requires_grad_()
+        if kind == "if":
+            out = K.hip_multistep_if_forward(xi, v0, 0.8, -0.25, False, False, 1, 2.0, True, 0, recompute)
+        elif kind == "lif":
+            out = K.hip_multistep_lif_forward(xi, v0, 0.8, -0.25, False, False, 2.0, True, 1, 2.0, True, 0, recompute)
+        else:
+            out = K.hip_multistep_plif_forward(xi, v0, ki, 0.8, -0.25, False, False, True, 1, 2.0, True, 0, recompute)
+        (out[0] * gs).sum().backward()
+        res.append((out[0].detach(), out[1].detach(), out[2].detach(), xi.grad, ki.grad))
+    for a, b in zip(*res):
+        if a is None:
+            assert b is None
+        else:
+            assert bits_equal(a, b)
+
+
+def test_grad_v_init_is_produced_only_when_asked(K):
+    x = seeded_randn((6, 128), 43, 0.4, 1.0).cuda().requires_grad_()
+    v0 = seeded_randn((128,), 44, 0.0, 0.3).cuda()
+    gs = seeded_randn((6, 128), 45).cuda()
+    # state without requires_grad: the backward op is called with need_grad_v_init=False and returns no [N] tensor
+    s = K.hip_multistep_lif_forward(x, v0, 1.0, 0.0, False, False, 2.0, True, 1, 2.0, False, 0, True)[0]
+    (s * gs).sum().backward()
+    gx_plain = x.grad.clone()
+    x.grad = None
+    v1 = v0.clone().requires_grad_()
+    s = K.hip_multistep_lif_forward(x, v1, 1.0, 0.0, False, False, 2.0, True, 1, 2.0, False, 0, True)[0]
+    (s * gs).sum().backward()
+    assert bits_equal(x.grad, gx_plain) and v1.grad is not None and v1.grad.shape == (128,)
+    gx, gvi = K.hip_multistep_lif_backward(gs, None, None, None, x.detach(), v0, 1.0, 0.0, False, False, 2.0, True, 1, 2.0,
+                                           0, False)
+    assert gvi.numel() == 0 and bits_equal(gx, gx_plain)
+    gx, gvi = K.hip_multistep_lif_backward(gs, None, None, None, x.detach(), v0, 1.0, 0.0, False, False, 2.0, True, 1, 2.0,
+                                           0, True)
+    assert bits_equal(gvi, v1.grad)
