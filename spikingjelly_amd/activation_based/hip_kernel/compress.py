@@ -1,8 +1,9 @@
 """Spike bit-packing on the device: 8 binary spikes per byte, LSB first over the flattened tensor.
 
-Counterpart of the reference's ``triton_kernel/compress.py:114-221`` (``bit_spike_compress`` /
-``bit_spike_decompress``).  Device tensors go through ``libsjhip.so``; CPU tensors take a torch
-path with the same layout, as the reference does for non-CUDA tensors (compress.py:150-151).
+Counterpart of the device kernels of the reference's ``triton_kernel/compress.py:114-221``
+(``bit_spike_compress`` / ``bit_spike_decompress``).  These functions run ``libsjhip.so`` on ROCm tensors only
+and raise for anything else; the torch path the reference keeps for non-CUDA tensors (compress.py:19-44,
+150-151) lives with the compressor classes in ``memopt/compress.py``.
 """
 
 from __future__ import annotations
@@ -14,30 +15,9 @@ from . import library as L
 __all__ = ["bit_spike_compress", "bit_spike_decompress"]
 
 
-def _compress_cpu(s_seq: torch.Tensor) -> torch.Tensor:
-    bits = s_seq.to(dtype=torch.bool).reshape(-1)
-    n_bytes = (bits.numel() + 7) // 8
-    packed = torch.zeros(n_bytes, dtype=torch.uint8, device=bits.device)
-    for i in range(8):
-        lane = bits[i::8].to(torch.uint8)
-        if lane.numel() > 0:
-            packed[: lane.numel()] |= lane << i
-    return packed
-
-
-def _decompress_cpu(packed: torch.Tensor, shape, dtype: torch.dtype) -> torch.Tensor:
-    n = torch.Size(shape).numel()
-    out = torch.zeros(n, dtype=torch.uint8, device=packed.device)
-    for i in range(8):
-        count = (n - i + 7) // 8
-        out[i::8] = ((packed >> i) & 1)[:count]
-    return out.reshape(shape).to(dtype)
-
-
 def bit_spike_compress(s_seq: torch.Tensor) -> torch.Tensor:
     """Pack a strictly binary tensor into ``(numel + 7) // 8`` bytes (uint8, 1-D)."""
-    if s_seq.device.type != "cuda":
-        return _compress_cpu(s_seq)
+    L.require_device_tensor("s_seq", s_seq)
     src = s_seq.contiguous().reshape(-1)
     n = src.numel()
     packed = torch.empty((n + 7) // 8, dtype=torch.uint8, device=src.device)
@@ -54,8 +34,7 @@ def bit_spike_decompress(s_seq_compressed: torch.Tensor, shape, dtype: torch.dty
     """Unpack to a 0/1 tensor of ``shape``.  ``dtype`` defaults to ``uint8`` like the reference's
     device kernel; passing the final dtype saves the separate cast pass."""
     shape = torch.Size(shape)
-    if s_seq_compressed.device.type != "cuda":
-        return _decompress_cpu(s_seq_compressed, shape, dtype)
+    L.require_device_tensor("s_seq_compressed", s_seq_compressed)
     n = shape.numel()
     src = s_seq_compressed.contiguous()
     if src.dtype != torch.uint8 or src.numel() < (n + 7) // 8:

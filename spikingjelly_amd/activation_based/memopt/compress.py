@@ -1,8 +1,10 @@
 """Spike compressors used by input-compressed gradient checkpointing.
 
 Counterpart of the reference's ``memopt/compress.py`` (:57-166 base class, :168-221 Null, :223-275
-Boolean, :278-329 Uint8, :332-385 Bit).  ``BitSpikeCompressor`` packs 8 binary spikes per byte through
-the HIP kernels for device tensors; CPU tensors use the torch path with the same byte layout.
+Boolean, :278-329 Uint8, :332-385 Bit).  ``BitSpikeCompressor`` packs 8 binary spikes per byte: tensors on a
+ROCm device go through the HIP kernels (``hip_kernel/compress.py``, no other path), tensors on the CPU through
+the torch ops below, which restate the reference's torch path for non-CUDA tensors
+(``triton_kernel/compress.py:19-44``) and give the same bytes.
 """
 
 from __future__ import annotations
@@ -11,7 +13,7 @@ import abc
 
 import torch
 
-from ..hip_kernel.compress import bit_spike_compress, bit_spike_decompress
+from ..hip_kernel import compress as _hip
 
 __all__ = [
     "BaseSpikeCompressor",
@@ -19,7 +21,43 @@ __all__ = [
     "BooleanSpikeCompressor",
     "Uint8SpikeCompressor",
     "BitSpikeCompressor",
+    "bit_spike_compress",
+    "bit_spike_decompress",
 ]
+
+
+def _torch_bit_spike_compress(s_seq: torch.Tensor) -> torch.Tensor:
+    bits = s_seq.to(dtype=torch.bool).reshape(-1)
+    n_bytes = (bits.numel() + 7) // 8
+    packed = torch.zeros(n_bytes, dtype=torch.uint8, device=bits.device)
+    for i in range(8):
+        lane = bits[i::8].to(torch.uint8)
+        if lane.numel() > 0:
+            packed[: lane.numel()] |= lane << i
+    return packed
+
+
+def _torch_bit_spike_decompress(packed: torch.Tensor, shape, dtype: torch.dtype) -> torch.Tensor:
+    n = torch.Size(shape).numel()
+    out = torch.zeros(n, dtype=torch.uint8, device=packed.device)
+    for i in range(8):
+        count = (n - i + 7) // 8
+        out[i::8] = ((packed >> i) & 1)[:count]
+    return out.reshape(shape).to(dtype)
+
+
+def bit_spike_compress(s_seq: torch.Tensor) -> torch.Tensor:
+    """Device dispatch of the reference's ``bit_spike_compress`` (triton_kernel/compress.py:114-166)."""
+    if s_seq.device.type == "cuda":
+        return _hip.bit_spike_compress(s_seq)
+    return _torch_bit_spike_compress(s_seq)
+
+
+def bit_spike_decompress(s_seq_compressed: torch.Tensor, shape, dtype: torch.dtype = torch.uint8) -> torch.Tensor:
+    """Device dispatch of the reference's ``bit_spike_decompress`` (triton_kernel/compress.py:169-221)."""
+    if s_seq_compressed.device.type == "cuda":
+        return _hip.bit_spike_decompress(s_seq_compressed, shape, dtype)
+    return _torch_bit_spike_decompress(s_seq_compressed, torch.Size(shape), dtype)
 
 
 class BaseSpikeCompressor(abc.ABC):

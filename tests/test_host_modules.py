@@ -209,3 +209,13 @@ def test_functional_names_follow_the_backend_naming_rule():
         assert all(p.annotation is not inspect.Parameter.empty for p in sig.parameters.values())
         assert sig.return_annotation is not inspect.Signature.empty
         assert list(sig.parameters)[-2:] == ["detach_reset", "store_v_seq"]
+
+
+def test_hip_bit_packing_refuses_cpu_tensors():
+    """The device functions have no other path: a CPU tensor raises instead of being packed by torch ops."""
+    from spikingjelly_amd.activation_based.hip_kernel import compress as hip_compress
+
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        hip_compress.bit_spike_compress(torch.ones(16))
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        hip_compress.bit_spike_decompress(torch.zeros(2, dtype=torch.uint8), (16,))
