@@ -247,7 +247,7 @@ __global__ void __launch_bounds__(kSsaThreads) ssa_forward_kernel(const SsaArgs 
 }
 
 template <typename S, int MC>
-__global__ void __launch_bounds__(kSsaThreads) ssa_backward_kernel(const SsaArgs a) {
+__global__ void __launch_bounds__(kSsaThreads, MC == 1 ? 3 : 1) ssa_backward_kernel(const SsaArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char ssa_lds[];
   typedef typename Io<S>::elem_t E;
   constexpr int CPH = 32 * MC;
