@@ -15,6 +15,8 @@
  *                             plif.py:288-386, integrate_and_fire.py:76-147; and
  *                             torch.ops.sj.multistep_{if,lif,plif}_{forward,inference}
  *                             spikingjelly/activation_based/triton_kernel/neuron_kernel/lif.py:673-763
+ *                             QIF: torch.ops.sj.cupy_multistep_qif_forward and its backward,
+ *                             cuda_kernel/neuron_kernel/multi_step/qif.py:21-277, 628-701
  *   sjhip_neuron_forward_packed <- the same forward ops followed by BitSpikeCompressor.compress,
  *                             spikingjelly/activation_based/memopt/compress.py:332-385
  *   sjhip_neuron_backward  <- torch.ops.sj.cupy_multistep_{if,lif,plif}_backward
@@ -36,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SJHIP_ABI_VERSION 1
+#define SJHIP_ABI_VERSION 2
 
 typedef enum sjhip_status {
   SJHIP_OK = 0,
@@ -50,7 +52,8 @@ typedef enum sjhip_status {
 typedef enum sjhip_neuron {
   SJHIP_NEURON_IF = 0,  /* h = v + x                                  (functional/neuron.py:310)   */
   SJHIP_NEURON_LIF = 1, /* h = v + (x - (v - vr)) / tau  or  v - (v - vr)/tau + x   (:849-852)     */
-  SJHIP_NEURON_PLIF = 2 /* h = v + (x - (v - vr)) * k    or  v - (v - vr)*k + x     (:1290-1295)   */
+  SJHIP_NEURON_PLIF = 2, /* h = v + (x - (v - vr)) * k    or  v - (v - vr)*k + x     (:1290-1295)   */
+  SJHIP_NEURON_QIF = 3  /* h = v + (x + a0 (v - v_rest) (v - v_c)) / tau          (functional/neuron.py:397) */
 } sjhip_neuron;
 
 /* Storage dtype of every [T,N] / [N] tensor of one call. */
@@ -101,6 +104,9 @@ typedef struct sjhip_neuron_params {
   float sg_alpha;   /* backward only */
   int32_t sg_id;    /* backward only, sjhip_surrogate */
   uint32_t flags;
+  float v_rest;     /* QIF only */
+  float v_c;        /* QIF only */
+  float a0;         /* QIF only */
 } sjhip_neuron_params;
 
 /* ABI version of the loaded library (== SJHIP_ABI_VERSION it was built with). */

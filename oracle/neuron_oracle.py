@@ -170,6 +170,10 @@ def charge(kind: str, x, v, tau_or_w, decay_input: bool, v_reset: Optional[float
         if decay_input:
             return v + (x - (v - v_reset_value)) * tau_or_w
         return v - (v - v_reset_value) * tau_or_w + x
+    if kind == "qif":
+        # functional/neuron.py:397; tau_or_w = (tau, a0, v_rest, v_c)
+        tau, a0, v_rest, v_c = tau_or_w
+        return v + (x + a0 * (v - v_rest) * (v - v_c)) / tau
     raise ValueError(kind)
 
 

@@ -31,9 +31,11 @@ __all__ = [
     "lif_charge",
     "lif_step",
     "plif_step",
+    "qif_step",
     "if_multi_step_hip",
     "lif_multi_step_hip",
     "plif_multi_step_hip",
+    "qif_multi_step_hip",
     "if_step_hip",
     "lif_step_hip",
     "plif_step_hip",
@@ -91,6 +93,15 @@ def plif_step(x: torch.Tensor, v: torch.Tensor, w: torch.Tensor, decay_input: bo
         h = v + (x - (v - rest)) * k
     else:
         h = v - (v - rest) * k + x
+    spike = surrogate_function(h - v_threshold)
+    return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset)
+
+
+def qif_step(x: torch.Tensor, v: torch.Tensor, tau: float, a0: float, v_rest: float, v_c: float, v_threshold: float,
+             v_reset: Optional[float], surrogate_function: SurrogateFunction, detach_reset: bool = False
+             ) -> tuple[torch.Tensor, torch.Tensor]:
+    """One quadratic integrate-and-fire step (reference :315-399): ``h = v + (x + a0 (v - v_rest)(v - v_c)) / tau``."""
+    h = v + (x + a0 * (v - v_rest) * (v - v_c)) / tau
     spike = surrogate_function(h - v_threshold)
     return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset)
 
@@ -197,6 +208,29 @@ def plif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Tensor, d
     else:
         s, v_seq, v_last = K.hip_multistep_plif_inference(x2, v1, k, v_threshold, vr, soft, decay_input,
                                                           store_v_seq, flags)
+    return _finish(x_seq, s, v_seq, v_last, store_v_seq)
+
+
+def qif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_threshold: float, v_reset: Optional[float],
+                       v_rest: float, v_c: float, a0: float, detach_reset: bool,
+                       surrogate_function: SurrogateFunction, store_v_seq: bool = False
+                       ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Multi-step QIF on the hip backend; argument order of the reference's ``qif_multi_step_cupy`` (:2188-2200)."""
+    from ..hip_kernel import neuron_kernel as K
+    from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
+
+    soft = v_reset is None
+    vr = 0.0 if soft else float(v_reset)
+    flags = _hip_mode_flags(x_seq)
+    x2, v1 = x_seq.flatten(1), v.flatten()
+    if _needs_grad(x_seq, v):
+        sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function)
+        s, v_seq, v_last, _ = K.hip_multistep_qif_forward(x2, v1, v_threshold, vr, soft, detach_reset, float(tau),
+                                                          float(v_rest), float(v_c), float(a0), sg_id, sg_alpha,
+                                                          store_v_seq, flags, _hip_recompute(x2))
+    else:
+        s, v_seq, v_last = K.hip_multistep_qif_inference(x2, v1, v_threshold, vr, soft, float(tau), float(v_rest),
+                                                         float(v_c), float(a0), store_v_seq, flags)
     return _finish(x_seq, s, v_seq, v_last, store_v_seq)
 
 

@@ -14,10 +14,10 @@ from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64
 
 import torch
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # enums of include/sjhip.h
-NEURON_IF, NEURON_LIF, NEURON_PLIF = 0, 1, 2
+NEURON_IF, NEURON_LIF, NEURON_PLIF, NEURON_QIF = 0, 1, 2, 3
 DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_U8 = 0, 1, 2, 3
 FLAG_DECAY_INPUT = 0x01
 FLAG_SOFT_RESET = 0x02
@@ -61,6 +61,9 @@ class NeuronParams(ctypes.Structure):
         ("sg_alpha", c_float),
         ("sg_id", c_int32),
         ("flags", c_uint32),
+        ("v_rest", c_float),
+        ("v_c", c_float),
+        ("a0", c_float),
     ]
 
 

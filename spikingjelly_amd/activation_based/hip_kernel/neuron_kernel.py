@@ -9,6 +9,7 @@ inference op that writes no ``h_seq``):
     sj::hip_multistep_{if,lif,plif}_inference  -> (spike_seq, v_seq, v_last)
     sj::hip_multistep_{if,lif,plif}_backward   -> (grad_x_seq, grad_v_init[, grad_k])
     sj::hip_multistep_{if,lif,plif}_inference_packed -> (spike_bits, v_seq, v_last)
+    sj::hip_multistep_qif_{forward,inference,backward}   the quadratic integrate-and-fire neuron, same outputs
 
 The ``_packed`` ops write the spikes bit-packed (uint8, ``T*N/8`` bytes, the layout of
 ``bit_spike_compress`` on the dense spike tensor) straight from the neuron kernel; they need ``N % 8 == 0``.
@@ -36,11 +37,14 @@ __all__ = [
     "hip_multistep_plif_forward", "hip_multistep_plif_inference", "hip_multistep_plif_backward",
     "hip_multistep_if_inference_packed", "hip_multistep_lif_inference_packed", "hip_multistep_plif_inference_packed",
     "packed_supported",
+    "hip_multistep_qif_forward", "hip_multistep_qif_inference", "hip_multistep_qif_backward",
 ]
 
 
-def _params(tau: float, v_th: float, v_reset: float, sg_alpha: float, sg_id: int, flags: int) -> L.NeuronParams:
-    return L.NeuronParams(tau, v_th, v_reset, sg_alpha, sg_id, flags)
+def _params(tau: float, v_th: float, v_reset: float, sg_alpha: float, sg_id: int, flags: int,
+            qif: tuple[float, float, float] = (0.0, 0.0, 0.0)) -> L.NeuronParams:
+    """``qif`` is (v_rest, v_c, a0) of the quadratic neuron, unused by the others."""
+    return L.NeuronParams(tau, v_th, v_reset, sg_alpha, sg_id, flags, *qif)
 
 
 def _flags(soft_reset: bool, detach_reset: bool, decay_input: bool, mode_flags: int) -> int:
@@ -90,7 +94,8 @@ def _k_pointer(k: Optional[torch.Tensor], ref: torch.Tensor) -> tuple[Optional[t
 
 def _run_forward(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: Optional[torch.Tensor],
                  tau: float, v_th: float, v_reset: float, flags: int, store_v_seq: bool,
-                 save_h: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+                 save_h: bool, qif: tuple[float, float, float] = (0.0, 0.0, 0.0)
+                 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     _check_inputs(x_seq, v_init)
     dtype = L.dtype_id(x_seq.dtype)
     x_seq = x_seq.contiguous()
@@ -101,7 +106,7 @@ def _run_forward(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: Opti
     v_last = x_seq.new_empty((N,))
     h_seq = torch.empty_like(x_seq) if save_h else None
     k_keep, k_ptr = _k_pointer(k, x_seq)
-    params = _params(tau, v_th, v_reset, 0.0, 0, flags | broadcast)
+    params = _params(tau, v_th, v_reset, 0.0, 0, flags | broadcast, qif)
     with torch.cuda.device(x_seq.device):
         rc = L.load().sjhip_neuron_forward(
             neuron, dtype, ctypes.byref(params), T, N,
@@ -161,7 +166,8 @@ def _forward_outputs(out, x_seq: torch.Tensor):
 def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
                   grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor, x_seq: Optional[torch.Tensor],
                   v_init: Optional[torch.Tensor], k: Optional[torch.Tensor], tau: float, v_th: float,
-                  v_reset: float, flags: int, sg_id: int, sg_alpha: float, need_grad_v_init: bool = True
+                  v_reset: float, flags: int, sg_id: int, sg_alpha: float, need_grad_v_init: bool = True,
+                  qif: tuple[float, float, float] = (0.0, 0.0, 0.0)
                   ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     recompute = x_seq is not None
     if not recompute and h_seq is None:
@@ -198,7 +204,7 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
             grad_k = torch.empty((), dtype=torch.float32, device=h_seq.device)
             workspace = torch.empty((L.load().sjhip_plif_workspace_floats(dtype, N),), dtype=torch.float32,
                                     device=h_seq.device)
-    params = _params(tau, v_th, v_reset, sg_alpha, sg_id, flags)
+    params = _params(tau, v_th, v_reset, sg_alpha, sg_id, flags, qif)
     with torch.cuda.device(h_seq.device):
         if recompute:
             rc = L.load().sjhip_neuron_backward_recompute(
@@ -212,7 +218,7 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
             rc = L.load().sjhip_neuron_backward(
                 neuron, dtype, ctypes.byref(params), T, N,
                 grad_spike_seq.data_ptr(), L.ptr(grad_v_seq), L.ptr(grad_v_last), h_seq.data_ptr(),
-                L.ptr(v_init) if neuron == L.NEURON_PLIF else None, k_ptr,
+                L.ptr(v_init) if neuron in (L.NEURON_PLIF, L.NEURON_QIF) else None, k_ptr,
                 grad_x_seq.data_ptr(), grad_v_init.data_ptr() if need_grad_v_init else None, L.ptr(grad_k), L.ptr(workspace),
                 L.current_stream_ptr(h_seq.device),
             )
@@ -531,3 +537,87 @@ def hip_multistep_plif_inference_packed(x_seq: torch.Tensor, v_init: torch.Tenso
 @hip_multistep_plif_inference_packed.register_fake
 def _(x_seq, v_init, k, v_th, v_reset, soft_reset, decay_input, store_v_seq, mode_flags):
     return _fake_forward_packed(x_seq, v_init, store_v_seq)
+
+
+# =================================================================================================
+# QIF: h = v + (x + a0 (v - v_rest)(v - v_c)) / tau  (reference cuda_kernel/neuron_kernel/multi_step/qif.py)
+# =================================================================================================
+@torch.library.custom_op("sj::hip_multistep_qif_forward", mutates_args=())
+def hip_multistep_qif_forward(x_seq: torch.Tensor, v_init: torch.Tensor, v_th: float, v_reset: float,
+                              soft_reset: bool, detach_reset: bool, tau: float, v_rest: float, v_c: float,
+                              a0: float, sg_id: int, sg_alpha: float, store_v_seq: bool, mode_flags: int,
+                              recompute: bool
+                              ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, detach_reset, True, mode_flags)
+    return _forward_outputs(_run_forward(L.NEURON_QIF, x_seq, v_init, None, tau, v_th, v_reset, flags, store_v_seq,
+                                         not recompute, (v_rest, v_c, a0)), x_seq)
+
+
+@hip_multistep_qif_forward.register_fake
+def _(x_seq, v_init, v_th, v_reset, soft_reset, detach_reset, tau, v_rest, v_c, a0, sg_id, sg_alpha, store_v_seq,
+      mode_flags, recompute):
+    return _fake_forward(x_seq, v_init, store_v_seq, True, recompute)
+
+
+@torch.library.custom_op("sj::hip_multistep_qif_inference", mutates_args=())
+def hip_multistep_qif_inference(x_seq: torch.Tensor, v_init: torch.Tensor, v_th: float, v_reset: float,
+                                soft_reset: bool, tau: float, v_rest: float, v_c: float, a0: float,
+                                store_v_seq: bool, mode_flags: int
+                                ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, False, True, mode_flags)
+    return _run_forward(L.NEURON_QIF, x_seq, v_init, None, tau, v_th, v_reset, flags, store_v_seq, False,
+                        (v_rest, v_c, a0))[:3]
+
+
+@hip_multistep_qif_inference.register_fake
+def _(x_seq, v_init, v_th, v_reset, soft_reset, tau, v_rest, v_c, a0, store_v_seq, mode_flags):
+    return _fake_forward(x_seq, v_init, store_v_seq, False)
+
+
+@torch.library.custom_op("sj::hip_multistep_qif_backward", mutates_args=())
+def hip_multistep_qif_backward(grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
+                               grad_v_last: Optional[torch.Tensor], h_seq: Optional[torch.Tensor],
+                               x_seq: Optional[torch.Tensor], v_init: torch.Tensor, v_th: float,
+                               v_reset: float, soft_reset: bool, detach_reset: bool, tau: float, v_rest: float,
+                               v_c: float, a0: float, sg_id: int, sg_alpha: float, mode_flags: int,
+                               need_grad_v_init: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, detach_reset, True, mode_flags)
+    gx, gvi, _ = _run_backward(L.NEURON_QIF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, None,
+                               tau, v_th, v_reset, flags, sg_id, sg_alpha, need_grad_v_init, (v_rest, v_c, a0))
+    return gx, gvi
+
+
+@hip_multistep_qif_backward.register_fake
+def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, v_th, v_reset, soft_reset, detach_reset,
+      tau, v_rest, v_c, a0, sg_id, sg_alpha, mode_flags, need_grad_v_init=True):
+    ref = h_seq if h_seq is not None else x_seq
+    return torch.empty_like(ref), ref.new_empty(ref.shape[1:] if need_grad_v_init else (0,))
+
+
+def _qif_setup_context(ctx, inputs, output):
+    (x_seq, v_init, v_th, v_reset, soft_reset, detach_reset, tau, v_rest, v_c, a0, sg_id, sg_alpha, store_v_seq,
+     mode_flags, recompute) = inputs
+    ctx.recompute = recompute
+    # the state-dependent dh/dv needs v_init on both paths
+    if recompute:
+        ctx.save_for_backward(x_seq, v_init)
+    else:
+        ctx.save_for_backward(output[3], v_init)
+    ctx.scalars = (v_th, v_reset, soft_reset, detach_reset, tau, v_rest, v_c, a0, sg_id, sg_alpha, mode_flags)
+    ctx.store_v_seq = store_v_seq
+    ctx.set_materialize_grads(False)
+
+
+def _qif_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_seq):
+    del grad_h_seq
+    first, v_init = ctx.saved_tensors
+    h_seq, x_seq = (None, first) if ctx.recompute else (first, None)
+    need = bool(ctx.needs_input_grad[1])
+    gx, gvi = hip_multistep_qif_backward(
+        grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, x_seq, v_init,
+        *ctx.scalars, need)
+    return (gx, (gvi if need else None)) + (None,) * 13
+
+
+torch.library.register_autograd("sj::hip_multistep_qif_forward", _qif_autograd_backward,
+                                setup_context=_qif_setup_context)

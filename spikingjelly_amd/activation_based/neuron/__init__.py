@@ -1,6 +1,7 @@
 from .base_node import BaseNode
 from .integrate_and_fire import IFNode
 from .lif import LIFNode
+from .nonlinear_if import QIFNode
 from .plif import ParametricLIFNode
 
-__all__ = ["BaseNode", "IFNode", "LIFNode", "ParametricLIFNode"]
+__all__ = ["BaseNode", "IFNode", "LIFNode", "ParametricLIFNode", "QIFNode"]

@@ -17,6 +17,9 @@
 // no v_seq has to be stored or read.  The sum is reduced by wavefront shuffles, then through LDS,
 // then either one fp32 partial per block (summed in a fixed order by plif_reduce_kernel, in fp64)
 // or one atomicAdd per block.
+// QIF (h_t = v_{t-1} + k (x_t + a0 (v_{t-1} - v_rest)(v_{t-1} - v_c)), cuda_kernel/neuron_kernel/multi_step/
+// qif.py:138-277) has a state-dependent dh_{t+1}/dv_t = 1 + k a0 ((v_t - v_c) + (v_t - v_rest)); the carry then
+// holds G_{t+1} itself and is scaled when step t has re-derived v_t from h_t; grad_v_init needs v_init.
 #pragma once
 
 #include <cmath>
@@ -58,7 +61,11 @@ struct BwdArgs {
   int is_if;
   int atomic_reduce;
   int v_init_broadcast;  // v_init holds one element for all neurons
+  float q_rest, q_c, q_a0;  // QIF
 };
+
+// Which extra terms the BPTT walk carries.
+enum BwdMode { BWD_PLAIN = 0, BWD_PLIF = 1, BWD_QIF = 2 };
 
 // FAST (16-bit storage, where the result is rounded to 8 or 11 significant bits anyway) uses the hardware
 // exp2 / reciprocal approximations (about 1 ulp each) in place of the correctly rounded library exp and IEEE
@@ -107,6 +114,12 @@ __device__ __forceinline__ float reset_as_forward(float h, float s, const BwdArg
   return a.soft_reset ? (h - s * a.v_th) : (s * a.v_reset + (1.0f - s) * h);
 }
 
+// QIF: d h_{t+1} / d v_t
+__device__ __forceinline__ float qif_dh_dv(float v, float k, const BwdArgs &a) {
+#pragma clang fp contract(fast)
+  return 1.0f + k * a.q_a0 * ((v - a.q_c) + (v - a.q_rest));
+}
+
 // HLDS: h_t does not come from h_seq in global memory but from LDS, where the recompute kernel
 // (neuron_bwd_recompute.h) has left it as fp32, V/4 float4 per work-item and step, laid out
 // [step][quarter][lane] so a wavefront reads consecutive 16-byte words.
@@ -128,7 +141,7 @@ template <typename S, bool VECTOR> struct BwdPrologue {
   }
 };
 
-template <typename S, bool VECTOR, bool PLIF, int SG, bool GVFULL, bool HLDS = false>
+template <typename S, bool VECTOR, int MODE, int SG, bool GVFULL, bool HLDS = false>
 __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, int64_t col, float k,
                                                const f32x4 *lds_h = nullptr,
                                                const BwdPrologue<S, VECTOR> *pre = nullptr) {
@@ -136,6 +149,8 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
   typedef typename A::elem_t E;
   constexpr int V = A::V;
   constexpr int PF = BwdPrologue<S, VECTOR>::PF;
+  constexpr bool PLIF = MODE == BWD_PLIF;
+  constexpr bool QIF = MODE == BWD_QIF;
 
   float acc_total = 0.0f;
   if (!active) return acc_total;
@@ -218,7 +233,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
           const float over = h[j] - v_th;
           const float s = (over >= 0.0f) ? 1.0f : 0.0f;
           float v_t = 0.0f;
-          if (PLIF) v_t = reset_as_forward(h[j], s, a);
+          if (PLIF || QIF) v_t = reset_as_forward(h[j], s, a);
           {
             // gradients carry a tolerance, not bit-exactness: let multiply-adds fuse here
 #pragma clang fp contract(fast)
@@ -228,10 +243,12 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
               acc[j] += g_next[j] * dh_dk;  // g_next is 0 on the first processed step
             }
             const float dvdh = (1.0f - s * cB) + (cC - h[j] * cD) * sg;
-            const float gvt = GVFULL ? carry[j] + gv[j] : carry[j];
+            // QIF: the carry is G_{t+1}; its factor depends on v_t, known only now (grad_v_last enters unscaled)
+            const float cin = (QIF && t != T - 1) ? carry[j] * qif_dh_dv(v_t, k, a) : carry[j];
+            const float gvt = GVFULL ? cin + gv[j] : cin;
             const float G = gvt * dvdh + gs[j] * sg;
             gx[j] = G * kx;
-            carry[j] = G * km;
+            carry[j] = QIF ? G : G * km;
             if (PLIF) { g_next[j] = G; h_next[j] = h[j]; }
           }
         }
@@ -239,7 +256,17 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
       }
     }
   }
-  if (a.grad_v_init) A::store((E *)a.grad_v_init + col, carry);
+  if (QIF) {
+    if (a.grad_v_init) {
+      float v0[V];
+      load_state<S, VECTOR, SJHIP_BWD_NT != 0>(a.v_init, col, a.v_init_broadcast != 0, v0);
+#pragma unroll
+      for (int j = 0; j < V; ++j) carry[j] *= qif_dh_dv(v0[j], k, a);
+      A::store((E *)a.grad_v_init + col, carry);
+    }
+  } else if (a.grad_v_init) {
+    A::store((E *)a.grad_v_init + col, carry);
+  }
   if (PLIF) {
     float v0[V];
     load_state<S, VECTOR, SJHIP_BWD_NT != 0>(a.v_init, col, a.v_init_broadcast != 0, v0);
@@ -253,26 +280,26 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
   return acc_total;
 }
 
-template <typename S, bool VECTOR, bool PLIF, int SG, bool HLDS = false>
+template <typename S, bool VECTOR, int MODE, int SG, bool HLDS = false>
 __device__ __forceinline__ float backward_gv_dispatch(const BwdArgs &a, bool active, int64_t col, float k,
                                                       const f32x4 *lds_h = nullptr,
                                                       const BwdPrologue<S, VECTOR> *pre = nullptr) {
-  if (a.grad_v_seq) return backward_body<S, VECTOR, PLIF, SG, true, HLDS>(a, active, col, k, lds_h, pre);
-  return backward_body<S, VECTOR, PLIF, SG, false, HLDS>(a, active, col, k, lds_h, pre);
+  if (a.grad_v_seq) return backward_body<S, VECTOR, MODE, SG, true, HLDS>(a, active, col, k, lds_h, pre);
+  return backward_body<S, VECTOR, MODE, SG, false, HLDS>(a, active, col, k, lds_h, pre);
 }
 
-template <typename S, bool VECTOR, bool PLIF, bool HLDS>
+template <typename S, bool VECTOR, int MODE, bool HLDS>
 __device__ __forceinline__ float backward_sg_dispatch(const BwdArgs &a, bool active, int64_t col, float k,
                                                       const f32x4 *lds_h,
                                                       const BwdPrologue<S, VECTOR> *pre = nullptr) {
   switch (a.sg) {
-    case SJHIP_SG_SIGMOID: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SIGMOID, HLDS>(a, active, col, k, lds_h, pre);
-    case SJHIP_SG_ATAN: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_ATAN, HLDS>(a, active, col, k, lds_h, pre);
-    case SJHIP_SG_PIECEWISE_QUADRATIC: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_PIECEWISE_QUADRATIC, HLDS>(a, active, col, k, lds_h, pre);
-    case SJHIP_SG_PIECEWISE_EXP: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_PIECEWISE_EXP, HLDS>(a, active, col, k, lds_h, pre);
-    case SJHIP_SG_SOFT_SIGN: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SOFT_SIGN, HLDS>(a, active, col, k, lds_h, pre);
-    case SJHIP_SG_SUPER_SPIKE: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_SUPER_SPIKE, HLDS>(a, active, col, k, lds_h, pre);
-    default: return backward_gv_dispatch<S, VECTOR, PLIF, SJHIP_SG_ERF, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_SIGMOID: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SIGMOID, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_ATAN: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_ATAN, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_PIECEWISE_QUADRATIC: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_PIECEWISE_QUADRATIC, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_PIECEWISE_EXP: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_PIECEWISE_EXP, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_SOFT_SIGN: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SOFT_SIGN, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_SUPER_SPIKE: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SUPER_SPIKE, HLDS>(a, active, col, k, lds_h, pre);
+    default: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_ERF, HLDS>(a, active, col, k, lds_h, pre);
   }
 }
 
@@ -297,14 +324,14 @@ __device__ __forceinline__ void plif_block_reduce(const BwdArgs &a, float part, 
   }
 }
 
-template <typename S, bool VECTOR, bool PLIF>
+template <typename S, bool VECTOR, int MODE>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_kernel(const BwdArgs a) {
   constexpr int V = Acc<S, VECTOR, true>::V;
   const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
   const bool active = col < a.N;
   const float k = a.k_device ? *a.k_device : a.k;
-  const float part = backward_sg_dispatch<S, VECTOR, PLIF, false>(a, active, col, k, nullptr);
-  if (PLIF) plif_block_reduce(a, part, k);
+  const float part = backward_sg_dispatch<S, VECTOR, MODE, false>(a, active, col, k, nullptr);
+  if (MODE == BWD_PLIF) plif_block_reduce(a, part, k);
 }
 
 // ---- host side: turn the ABI parameters into kernel arguments ------------------------------------
@@ -330,6 +357,8 @@ inline int build_bwd_args(BwdArgs &a, int neuron, int dtype, const sjhip_neuron_
   else { a.cB = 1.0f; a.cC = detach ? 0.0f : p.v_reset; a.cD = detach ? 0.0f : 1.0f; }
 
   const bool plif = neuron == SJHIP_NEURON_PLIF;
+  a.q_rest = p.v_rest; a.q_c = p.v_c; a.q_a0 = p.a0;
+  if (neuron == SJHIP_NEURON_QIF) a.decay_input = 1;  // grad_x = G k
   if (neuron == SJHIP_NEURON_IF) {
     a.k = 0.0f;
   } else if (plif) {

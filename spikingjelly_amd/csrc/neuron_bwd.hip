@@ -28,8 +28,15 @@ __global__ void __launch_bounds__(1024) plif_reduce_kernel(const float *partials
 
 namespace {
 
+template <typename S, int MODE>
+void launch_mode(const BwdArgs &a, bool vector, dim3 grid, dim3 threads, unsigned lds, hipStream_t stream) {
+  if (vector) hipLaunchKernelGGL((backward_kernel<S, true, MODE>), grid, threads, lds, stream, a);
+  else hipLaunchKernelGGL((backward_kernel<S, false, MODE>), grid, threads, lds, stream, a);
+}
+
 template <typename S>
-int launch_typed(BwdArgs &a, bool vector, bool plif, float *grad_k_out, hipStream_t stream) {
+int launch_typed(BwdArgs &a, bool vector, int mode, float *grad_k_out, hipStream_t stream) {
+  const bool plif = mode == BWD_PLIF;
   const int block = tuning().bwd_block;
   const int V = vector ? Acc<S, true, true>::V : 1;
   const int64_t items = (a.N + V - 1) / V;
@@ -39,13 +46,9 @@ int launch_typed(BwdArgs &a, bool vector, bool plif, float *grad_k_out, hipStrea
   const unsigned lds = occupancy_cap_lds(tuning().bwd_blocks_per_cu);
   {
     ProfileScope prof(KC_BACKWARD, stream);
-    if (plif) {
-      if (vector) hipLaunchKernelGGL((backward_kernel<S, true, true>), grid, threads, lds, stream, a);
-      else hipLaunchKernelGGL((backward_kernel<S, false, true>), grid, threads, lds, stream, a);
-    } else {
-      if (vector) hipLaunchKernelGGL((backward_kernel<S, true, false>), grid, threads, lds, stream, a);
-      else hipLaunchKernelGGL((backward_kernel<S, false, false>), grid, threads, lds, stream, a);
-    }
+    if (mode == BWD_PLIF) launch_mode<S, BWD_PLIF>(a, vector, grid, threads, lds, stream);
+    else if (mode == BWD_QIF) launch_mode<S, BWD_QIF>(a, vector, grid, threads, lds, stream);
+    else launch_mode<S, BWD_PLAIN>(a, vector, grid, threads, lds, stream);
     int rc = check_launch("backward");
     if (rc != SJHIP_OK) return rc;
   }
@@ -77,7 +80,7 @@ int launch_backward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t
   int rc = build_bwd_args(a, neuron, dtype, p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, k_device,
                           grad_x_seq, grad_v_init, grad_rtau, workspace);
   if (rc != SJHIP_OK) return rc;
-  const bool plif = neuron == SJHIP_NEURON_PLIF;
+  const int mode = neuron == SJHIP_NEURON_PLIF ? BWD_PLIF : (neuron == SJHIP_NEURON_QIF ? BWD_QIF : BWD_PLAIN);
 
   const int esize = dtype == SJHIP_F32 ? 4 : 2;
   const int V = 16 / esize;
@@ -87,9 +90,9 @@ int launch_backward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t
                       (v_init == nullptr || a.v_init_broadcast || aligned16(v_init));
 
   switch (dtype) {
-    case SJHIP_F32: return launch_typed<float>(a, vector, plif, grad_rtau, stream);
-    case SJHIP_F16: return launch_typed<f16_t>(a, vector, plif, grad_rtau, stream);
-    case SJHIP_BF16: return launch_typed<bf16_t>(a, vector, plif, grad_rtau, stream);
+    case SJHIP_F32: return launch_typed<float>(a, vector, mode, grad_rtau, stream);
+    case SJHIP_F16: return launch_typed<f16_t>(a, vector, mode, grad_rtau, stream);
+    case SJHIP_BF16: return launch_typed<bf16_t>(a, vector, mode, grad_rtau, stream);
     default: return fail(SJHIP_ERR_INVALID, "backward: dtype %d", dtype);
   }
 }

@@ -75,7 +75,7 @@ __device__ __forceinline__ void recompute_reset_dispatch(const FwdArgs &a, f32x4
   else recompute_body<S, ROUND_EACH, CH, false>(a, lds_h, col);
 }
 
-template <typename S, bool ROUND_EACH, bool PLIF>
+template <typename S, bool ROUND_EACH, int MODE>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_kernel(const FwdArgs f, const BwdArgs b) {
   extern __shared__ f32x4 lds_h[];
   constexpr int V = Acc<S, true, true>::V;
@@ -90,18 +90,20 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_kernel(con
       case CH_DECAY_INPUT_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_DECAY_INPUT_DIV>(f, lds_h, col); break;
       case CH_DECAY_INPUT_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_DECAY_INPUT_MUL>(f, lds_h, col); break;
       case CH_PLAIN_INPUT_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_PLAIN_INPUT_DIV>(f, lds_h, col); break;
+      case CH_QIF_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_QIF_DIV>(f, lds_h, col); break;
+      case CH_QIF_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_QIF_MUL>(f, lds_h, col); break;
       default: recompute_reset_dispatch<S, ROUND_EACH, CH_PLAIN_INPUT_MUL>(f, lds_h, col); break;
     }
   }
   const float k = b.k_device ? *b.k_device : b.k;
-  const float part = backward_sg_dispatch<S, true, PLIF, true>(b, active, col, k, lds_h, &pre);
-  if (PLIF) plif_block_reduce(b, part, k);
+  const float part = backward_sg_dispatch<S, true, MODE, true>(b, active, col, k, lds_h, &pre);
+  if (MODE == BWD_PLIF) plif_block_reduce(b, part, k);
 }
 
 // Launches the recompute kernel of storage dtype S; defined in neuron_bwd_recompute_launch.h and
 // instantiated once per dtype (neuron_bwd_recompute_{f32,f16,bf16}.hip).
 template <typename S>
-int launch_recompute_dtype(const FwdArgs &f, const BwdArgs &b, bool round_each, bool plif, int block, unsigned lds,
+int launch_recompute_dtype(const FwdArgs &f, const BwdArgs &b, bool round_each, int mode, int block, unsigned lds,
                            int64_t blocks, hipStream_t stream);
 
 }  // namespace sjhip

@@ -6,9 +6,9 @@
 
 namespace sjhip {
 
-extern template int launch_recompute_dtype<float>(const FwdArgs &, const BwdArgs &, bool, bool, int, unsigned, int64_t, hipStream_t);
-extern template int launch_recompute_dtype<f16_t>(const FwdArgs &, const BwdArgs &, bool, bool, int, unsigned, int64_t, hipStream_t);
-extern template int launch_recompute_dtype<bf16_t>(const FwdArgs &, const BwdArgs &, bool, bool, int, unsigned, int64_t, hipStream_t);
+extern template int launch_recompute_dtype<float>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
+extern template int launch_recompute_dtype<f16_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
+extern template int launch_recompute_dtype<bf16_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
 
 namespace {
 
@@ -64,12 +64,13 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
   const unsigned cap = occupancy_cap_lds(tuning().replay_blocks_per_cu);
   if (cap > lds) lds = cap;
   const bool plif = neuron == SJHIP_NEURON_PLIF;
+  const int mode = plif ? BWD_PLIF : (neuron == SJHIP_NEURON_QIF ? BWD_QIF : BWD_PLAIN);
   {
     ProfileScope prof(KC_BACKWARD, stream);
     switch (dtype) {
-      case SJHIP_F32: rc = launch_recompute_dtype<float>(f, b, false, plif, block, lds, blocks, stream); break;
-      case SJHIP_F16: rc = launch_recompute_dtype<f16_t>(f, b, round_each, plif, block, lds, blocks, stream); break;
-      case SJHIP_BF16: rc = launch_recompute_dtype<bf16_t>(f, b, round_each, plif, block, lds, blocks, stream); break;
+      case SJHIP_F32: rc = launch_recompute_dtype<float>(f, b, false, mode, block, lds, blocks, stream); break;
+      case SJHIP_F16: rc = launch_recompute_dtype<f16_t>(f, b, round_each, mode, block, lds, blocks, stream); break;
+      case SJHIP_BF16: rc = launch_recompute_dtype<bf16_t>(f, b, round_each, mode, block, lds, blocks, stream); break;
       default: return fail(SJHIP_ERR_INVALID, "backward(recompute): dtype %d", dtype);
     }
     if (rc != SJHIP_OK) return rc;

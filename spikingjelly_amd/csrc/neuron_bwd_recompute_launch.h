@@ -11,9 +11,9 @@ namespace sjhip {
 // LDS per compute unit on gfx950 is 160 KiB; 1 KiB is left for the statically allocated reduction words
 constexpr unsigned kRecomputeMaxLds = 159u * 1024u;
 
-template <typename S, bool ROUND_EACH, bool PLIF>
+template <typename S, bool ROUND_EACH, int MODE>
 int launch_kernel(const FwdArgs &f, const BwdArgs &b, int block, unsigned lds, int64_t blocks, hipStream_t stream) {
-  auto kernel = backward_recompute_kernel<S, ROUND_EACH, PLIF>;
+  auto kernel = backward_recompute_kernel<S, ROUND_EACH, MODE>;
   // a block may use more than the default 64 KiB of dynamic LDS only after this opt-in (once per kernel)
   static std::once_flag once;
   static hipError_t attr_rc = hipSuccess;
@@ -28,17 +28,20 @@ int launch_kernel(const FwdArgs &f, const BwdArgs &b, int block, unsigned lds, i
   return check_launch("backward(recompute)");
 }
 
-template <typename S>
-int launch_recompute_dtype(const FwdArgs &f, const BwdArgs &b, bool round_each, bool plif, int block, unsigned lds,
-                           int64_t blocks, hipStream_t stream) {
-  if constexpr (!std::is_same<S, float>::value) {
-    if (round_each)
-      return plif ? launch_kernel<S, true, true>(f, b, block, lds, blocks, stream)
-                  : launch_kernel<S, true, false>(f, b, block, lds, blocks, stream);
-  }
-  return plif ? launch_kernel<S, false, true>(f, b, block, lds, blocks, stream)
-              : launch_kernel<S, false, false>(f, b, block, lds, blocks, stream);
+template <typename S, bool ROUND_EACH>
+int launch_mode(const FwdArgs &f, const BwdArgs &b, int mode, int block, unsigned lds, int64_t blocks, hipStream_t stream) {
+  if (mode == BWD_PLIF) return launch_kernel<S, ROUND_EACH, BWD_PLIF>(f, b, block, lds, blocks, stream);
+  if (mode == BWD_QIF) return launch_kernel<S, ROUND_EACH, BWD_QIF>(f, b, block, lds, blocks, stream);
+  return launch_kernel<S, ROUND_EACH, BWD_PLAIN>(f, b, block, lds, blocks, stream);
 }
 
+template <typename S>
+int launch_recompute_dtype(const FwdArgs &f, const BwdArgs &b, bool round_each, int mode, int block, unsigned lds,
+                           int64_t blocks, hipStream_t stream) {
+  if constexpr (!std::is_same<S, float>::value) {
+    if (round_each) return launch_mode<S, true>(f, b, mode, block, lds, blocks, stream);
+  }
+  return launch_mode<S, false>(f, b, mode, block, lds, blocks, stream);
+}
 
 }  // namespace sjhip

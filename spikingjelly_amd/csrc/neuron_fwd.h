@@ -38,7 +38,9 @@ enum Charge {
   CH_DECAY_INPUT_DIV = 1,  // v + (x - (v - vr)) / tau
   CH_DECAY_INPUT_MUL = 2,  // v + (x - (v - vr)) * k
   CH_PLAIN_INPUT_DIV = 3,  // v - (v - vr) / tau + x
-  CH_PLAIN_INPUT_MUL = 4   // v - (v - vr) * k + x
+  CH_PLAIN_INPUT_MUL = 4,  // v - (v - vr) * k + x
+  CH_QIF_DIV = 5,          // v + (x + a0 * (v - v_rest) * (v - v_c)) / tau
+  CH_QIF_MUL = 6           // the same with * k
 };
 
 struct FwdArgs {
@@ -55,6 +57,9 @@ struct FwdArgs {
   float vr_mul;  // v_reset as a factor    (fp32 always)
   float vth_sub; // v_threshold as a subtrahend
   float vth_mul; // v_threshold as a factor
+  float q_rest_sub; // QIF: v_rest and v_c as subtrahends (rounded like vr_add), a0 as a factor
+  float q_c_sub;
+  float q_a0_mul;
   int charge;
   int soft_reset;
   int v_init_broadcast;  // v_init holds one element for all neurons
@@ -71,6 +76,15 @@ __device__ __forceinline__ void neuron_step(float x, float &v, float &h, float &
     float d = Cvt<R>::round(v - a.vr_add);
     float e = Cvt<R>::round(x - d);
     float f = (CH == CH_DECAY_INPUT_DIV) ? Cvt<R>::round(e / tau) : Cvt<R>::round(e * tau);
+    h = Cvt<R>::round(v + f);
+  } else if (CH == CH_QIF_DIV || CH == CH_QIF_MUL) {
+    // functional/neuron.py:397, evaluated left to right: ((a0 * (v - v_rest)) * (v - v_c))
+    float d1 = Cvt<R>::round(v - a.q_rest_sub);
+    float m1 = Cvt<R>::round(a.q_a0_mul * d1);
+    float d2 = Cvt<R>::round(v - a.q_c_sub);
+    float m2 = Cvt<R>::round(m1 * d2);
+    float e = Cvt<R>::round(x + m2);
+    float f = (CH == CH_QIF_DIV) ? Cvt<R>::round(e / tau) : Cvt<R>::round(e * tau);
     h = Cvt<R>::round(v + f);
   } else {
     float d = Cvt<R>::round(v - a.vr_add);
@@ -99,6 +113,17 @@ __device__ __forceinline__ void neuron_step(float x, float &v, float &h, float &
 // bit-identical to neuron_step<f16_t> on floats while needing no conversions.  Python scalars that torch keeps
 // in fp32 (the tau divisor / multiplier, v_threshold and v_reset as factors) still enter through an fp32 product
 // rounded once.
+// fp32 product rounded to fp32, then to fp16: the two roundings torch's CPU kernels perform for a half tensor
+// times a Python scalar.  The product is pinned in a register because the compiler would otherwise fold the
+// multiply and the conversion into v_fma_mixlo_f16, which rounds the exact product once and differs from the
+// double rounding in about one result out of forty (measured).
+__device__ __forceinline__ _Float16 scalar_product_f16(float scalar, _Float16 t) {
+#pragma clang fp contract(off)
+  float p = scalar * (float)t;
+  asm volatile("" : "+v"(p));
+  return (_Float16)p;
+}
+
 template <typename R, int CH, bool SOFT>
 __device__ __forceinline__ void neuron_step(_Float16 x, _Float16 &v, _Float16 &h, _Float16 &s, float tau,
                                             const FwdArgs &a) {
@@ -110,18 +135,26 @@ __device__ __forceinline__ void neuron_step(_Float16 x, _Float16 &v, _Float16 &h
   } else if (CH == CH_DECAY_INPUT_DIV || CH == CH_DECAY_INPUT_MUL) {
     const H d = v - vr_add;
     const H e = x - d;
-    const H f = (CH == CH_DECAY_INPUT_DIV) ? (H)((float)e / tau) : (H)((float)e * tau);
+    const H f = (CH == CH_DECAY_INPUT_DIV) ? (H)((float)e / tau) : scalar_product_f16(tau, e);
+    h = v + f;
+  } else if (CH == CH_QIF_DIV || CH == CH_QIF_MUL) {
+    const H d1 = v - (H)a.q_rest_sub;
+    const H m1 = scalar_product_f16(a.q_a0_mul, d1);
+    const H d2 = v - (H)a.q_c_sub;
+    const H m2 = m1 * d2;
+    const H e = x + m2;
+    const H f = (CH == CH_QIF_DIV) ? (H)((float)e / tau) : scalar_product_f16(tau, e);
     h = v + f;
   } else {
     const H d = v - vr_add;
-    const H f = (CH == CH_PLAIN_INPUT_DIV) ? (H)((float)d / tau) : (H)((float)d * tau);
+    const H f = (CH == CH_PLAIN_INPUT_DIV) ? (H)((float)d / tau) : scalar_product_f16(tau, d);
     const H g = v - f;
     h = g + x;
   }
   const H over = h - vth_sub;
   s = (over >= (H)0.0f) ? (H)1.0f : (H)0.0f;
   if (SOFT) {
-    const H m = (H)((float)s * a.vth_mul);
+    const H m = (H)((float)s * a.vth_mul);  // s is 0 or 1: the product is exact, any rounding order agrees
     v = h - m;
   } else {
     const H m = (H)((float)s * a.vr_mul);
@@ -225,6 +258,8 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) forward_kernel(const FwdArgs 
     case CH_DECAY_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_DIV, PACKED>(a); break;
     case CH_DECAY_INPUT_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_MUL, PACKED>(a); break;
     case CH_PLAIN_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_DIV, PACKED>(a); break;
+    case CH_QIF_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_QIF_DIV, PACKED>(a); break;
+    case CH_QIF_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_QIF_MUL, PACKED>(a); break;
     default: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_MUL, PACKED>(a); break;
   }
 }
@@ -253,17 +288,18 @@ inline int build_fwd_args(FwdArgs &a, bool &round_each, int neuron, int dtype, c
     a.charge = decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL;
     a.k_device = k_device;
   } else {
+    const bool qif = neuron == SJHIP_NEURON_QIF;
     if (!(p.tau > 0.0f) || !std::isfinite(p.tau)) return fail(SJHIP_ERR_INVALID, "forward: tau=%g", (double)p.tau);
     if (p.flags & SJHIP_FLAG_RECIPROCAL_TAU) {
       // fl(1/tau) from the double quotient, as the reference kernels receive it (multi_step/lif.py:338)
       a.tau = (float)(1.0 / (double)p.tau);
-      a.charge = decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL;
+      a.charge = qif ? CH_QIF_MUL : (decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL);
     } else if (is_power_of_two(p.tau) && p.tau <= 0x1p100f && p.tau >= 0x1p-100f) {
       // x / 2^e == x * 2^-e bit for bit (both are exact scalings, subnormal results round identically)
       a.tau = 1.0f / p.tau;
-      a.charge = decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL;
+      a.charge = qif ? CH_QIF_MUL : (decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL);
     } else {
-      a.charge = decay_input ? CH_DECAY_INPUT_DIV : CH_PLAIN_INPUT_DIV;
+      a.charge = qif ? CH_QIF_DIV : (decay_input ? CH_DECAY_INPUT_DIV : CH_PLAIN_INPUT_DIV);
     }
   }
 
@@ -273,9 +309,17 @@ inline int build_fwd_args(FwdArgs &a, bool &round_each, int neuron, int dtype, c
   a.vth_mul = p.v_threshold;
   a.vr_add = p.v_reset;
   a.vth_sub = p.v_threshold;
+  a.q_rest_sub = p.v_rest;
+  a.q_c_sub = p.v_c;
+  a.q_a0_mul = p.a0;
   if (round_each) {
-    if (dtype == SJHIP_F16) { a.vr_add = Cvt<f16_t>::round(p.v_reset); a.vth_sub = Cvt<f16_t>::round(p.v_threshold); }
-    else { a.vr_add = Cvt<bf16_t>::round(p.v_reset); a.vth_sub = Cvt<bf16_t>::round(p.v_threshold); }
+    if (dtype == SJHIP_F16) {
+      a.vr_add = Cvt<f16_t>::round(p.v_reset); a.vth_sub = Cvt<f16_t>::round(p.v_threshold);
+      a.q_rest_sub = Cvt<f16_t>::round(p.v_rest); a.q_c_sub = Cvt<f16_t>::round(p.v_c);
+    } else {
+      a.vr_add = Cvt<bf16_t>::round(p.v_reset); a.vth_sub = Cvt<bf16_t>::round(p.v_threshold);
+      a.q_rest_sub = Cvt<bf16_t>::round(p.v_rest); a.q_c_sub = Cvt<bf16_t>::round(p.v_c);
+    }
   }
 
   return SJHIP_OK;

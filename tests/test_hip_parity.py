@@ -393,3 +393,23 @@ def test_grad_v_init_is_produced_only_when_asked(K):
     gx, gvi = K.hip_multistep_lif_backward(gs, None, None, None, x.detach(), v0, 1.0, 0.0, False, False, 2.0, True, 1, 2.0,
                                            0, True)
     assert bits_equal(gvi, v1.grad)
+
+
+@pytest.mark.parametrize("kind", ["lif", "plif"])
+@pytest.mark.parametrize("decay_input", [True, False])
+def test_fp16_every_op_rounding_with_a_factor_that_is_not_a_half(K, kind, decay_input):
+    """fp16 storage, every op rounded, multiplying by an fp32 scalar that fp16 cannot hold (k = fl(1/3)): torch
+    rounds the fp32 product to fp32 and then to fp16.  A fused mixed-precision multiply would round once and differ
+    in a few percent of the elements, so the kernels must reproduce the two roundings."""
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+
+    T, N = 6, 8192
+    x = seeded_randn((T, N), 61, 0.4, 1.0).half()
+    v0 = seeded_randn((N,), 62, 0.0, 0.5).half()
+    k = torch.tensor(1.0 / 3.0, dtype=torch.float32)
+    es, ev, eh = no.multi_step("plif_k", x, v0, k, decay_input, 0.8, -0.2)
+    if kind == "plif":
+        s, v, vl, h = hip_forward(K, "plif", x, v0, float(k), decay_input, 0.8, -0.2)
+    else:  # LIF told to multiply by fl(1/tau) like the reference's kernels
+        s, v, vl, h = hip_forward(K, "lif", x, v0, 3.0, decay_input, 0.8, -0.2, flags=L.FLAG_RECIPROCAL_TAU)
+    assert bits_equal(h, eh) and bits_equal(s, es) and bits_equal(v, ev)

@@ -380,3 +380,62 @@ def test_ssa_oracle_is_exact_and_associative():
     one[0, 0, 0, 2, 5] = 1  # q
     out = ssa_oracle.ssa_exact(one, 1.0)
     assert out[0, 0, 1, 5] == 1 and out.sum() == 1
+
+
+# ------------------------------------------------------------------------------------------------
+# QIF (functional/neuron.py:397): pins that do not retype the formula
+# ------------------------------------------------------------------------------------------------
+def test_qif_rest_and_critical_potentials_are_fixed_points_without_input():
+    """With x = 0 the quadratic term vanishes at v = v_rest and v = v_c, so both are fixed points of the charge
+    step; between them the potential falls towards v_rest, above v_c it escapes upwards (the defining property of
+    the quadratic integrate-and-fire model)."""
+    tau, a0, v_rest, v_c = 2.0, 1.0, 0.0, 0.5
+    p = (tau, a0, v_rest, v_c)
+    zeros = torch.zeros(1, 4)
+    v0 = torch.tensor([v_rest, v_c, 0.25, 0.75])
+    _, v, h = no.multi_step("qif", zeros, v0, p, True, 10.0, -0.1)
+    assert float(h[0, 0]) == v_rest and float(h[0, 1]) == v_c
+    assert float(h[0, 2]) < 0.25 and float(h[0, 3]) > 0.75
+    # 0.25 -> 0.25 + (0.25)(-0.25)/2 exactly (all dyadic)
+    assert float(h[0, 2]) == 0.25 - 0.03125
+    assert float(h[0, 3]) == 0.75 + 0.09375
+
+
+def test_qif_single_step_closed_form_and_reduction_to_if():
+    """T = 1 from v = 0: h = (x + a0 v_rest v_c) / tau.  A vanishing a0 leaves h = v + x / tau, i.e. an IF neuron
+    driven by x / tau."""
+    x = seeded_randn((1, 64), 11, 0.5, 1.0)
+    v0 = torch.zeros(64)
+    _, _, h = no.multi_step("qif", x, v0, (4.0, 2.0, 0.25, 0.5), True, 100.0, None)
+    assert torch.equal(h[0], (x[0] + 0.25) / 4.0)  # a0 v_rest v_c = 2 * 0.25 * 0.5
+    xs = seeded_randn((6, 64), 12, 0.5, 1.0)
+    s_q, v_q, _ = no.multi_step("qif", xs, v0, (2.0, 0.0, 0.0, 0.5), True, 1.0, 0.0)
+    s_i, v_i, _ = no.multi_step("if", xs / 2.0, v0, None, True, 1.0, 0.0)
+    assert torch.equal(s_q, s_i) and torch.equal(v_q, v_i)
+
+
+@pytest.mark.parametrize("v_reset", [-0.1, None])
+def test_qif_autograd_matches_finite_differences_of_the_smooth_network(v_reset):
+    T, N, vth, alpha = 5, 6, 0.9, 2.0
+    p = (2.5, 1.3, 0.0, 0.6)
+    x = seeded_randn((T, N), 41, 0.4, 0.8, torch.float64)
+    v0 = seeded_randn((N,), 42, 0.0, 0.3, torch.float64)
+    gs = seeded_randn((T, N), 43, dtype=torch.float64)
+    gv = seeded_randn((T, N), 44, dtype=torch.float64)
+    smooth = no.surrogate("atan", alpha, spiking=False)
+
+    def loss(x_, v0_):
+        s, v, _ = no.multi_step("qif", x_, v0_, p, True, vth, v_reset, smooth)
+        return float((s * gs).sum() + (v * gv).sum())
+
+    ref = no.forward_backward("qif", x, v0, gs, gv, None, p, True, vth, v_reset, "atan", alpha, False, spiking=False)
+    eps = 1e-6
+    for (t, n) in [(0, 0), (2, 3), (T - 1, N - 1)]:
+        xp, xm = x.clone(), x.clone()
+        xp[t, n] += eps
+        xm[t, n] -= eps
+        assert (loss(xp, v0) - loss(xm, v0)) / (2 * eps) == pytest.approx(float(ref["grad_x"][t, n]), rel=1e-6, abs=1e-8)
+    vp, vm = v0.clone(), v0.clone()
+    vp[2] += eps
+    vm[2] -= eps
+    assert (loss(x, vp) - loss(x, vm)) / (2 * eps) == pytest.approx(float(ref["grad_v_init"][2]), rel=1e-6, abs=1e-8)
