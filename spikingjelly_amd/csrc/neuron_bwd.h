@@ -120,9 +120,11 @@ __device__ __forceinline__ float qif_dh_dv(float v, float k, const BwdArgs &a) {
   return 1.0f + k * a.q_a0 * ((v - a.q_c) + (v - a.q_rest));
 }
 
-// HLDS: h_t does not come from h_seq in global memory but from LDS, where the recompute kernel
-// (neuron_bwd_recompute.h) has left it as fp32, V/4 float4 per work-item and step, laid out
-// [step][quarter][lane] so a wavefront reads consecutive 16-byte words.
+// HLDS != 0: h_t does not come from h_seq in global memory but from LDS, where the recompute kernel
+// (neuron_bwd_recompute.h) has left it.  HLDS == 1: as fp32, V/4 float4 per work-item and step, laid out
+// [step][quarter][lane] so a wavefront reads consecutive 16-byte words.  HLDS == 2 (16-bit storage with every
+// op rounded, where h is exactly a storage-dtype value): as eight 16-bit patterns in one 16-byte word, laid out
+// [step][lane], half the LDS footprint.
 // First PF rows (t = T-1 downwards) of grad_spike and grad_v_seq, requested ahead of their use.
 template <typename S, bool VECTOR> struct BwdPrologue {
   typedef Acc<S, VECTOR, SJHIP_BWD_NT != 0> A;
@@ -141,7 +143,7 @@ template <typename S, bool VECTOR> struct BwdPrologue {
   }
 };
 
-template <typename S, bool VECTOR, int MODE, int SG, bool GVFULL, bool HLDS = false>
+template <typename S, bool VECTOR, int MODE, int SG, bool GVFULL, int HLDS = 0>
 __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, int64_t col, float k,
                                                const f32x4 *lds_h = nullptr,
                                                const BwdPrologue<S, VECTOR> *pre = nullptr) {
@@ -218,7 +220,11 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
       if (t >= 0) {
         float gs[V], h[V], gv[V], gx[V];
         A::unpack(cur_gs[i], gs);
-        if (HLDS) {
+        if (HLDS == 2) {
+          typedef Acc<S, true, false> AH;
+          if constexpr (AH::V == V && sizeof(S) == 2)
+            AH::unpack(reinterpret_cast<const typename AH::raw_t *>(lds_h)[(int)t * (int)blockDim.x + (int)threadIdx.x], h);
+        } else if (HLDS) {
 #pragma unroll
           for (int q = 0; q < V / 4; ++q) {
             const f32x4 w = lds_h[((int)t * (V / 4) + q) * (int)blockDim.x + (int)threadIdx.x];
@@ -280,7 +286,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
   return acc_total;
 }
 
-template <typename S, bool VECTOR, int MODE, int SG, bool HLDS = false>
+template <typename S, bool VECTOR, int MODE, int SG, int HLDS = 0>
 __device__ __forceinline__ float backward_gv_dispatch(const BwdArgs &a, bool active, int64_t col, float k,
                                                       const f32x4 *lds_h = nullptr,
                                                       const BwdPrologue<S, VECTOR> *pre = nullptr) {
@@ -288,7 +294,7 @@ __device__ __forceinline__ float backward_gv_dispatch(const BwdArgs &a, bool act
   return backward_body<S, VECTOR, MODE, SG, false, HLDS>(a, active, col, k, lds_h, pre);
 }
 
-template <typename S, bool VECTOR, int MODE, bool HLDS>
+template <typename S, bool VECTOR, int MODE, int HLDS>
 __device__ __forceinline__ float backward_sg_dispatch(const BwdArgs &a, bool active, int64_t col, float k,
                                                       const f32x4 *lds_h,
                                                       const BwdPrologue<S, VECTOR> *pre = nullptr) {
@@ -330,7 +336,7 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_kernel(const BwdArgs
   const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
   const bool active = col < a.N;
   const float k = a.k_device ? *a.k_device : a.k;
-  const float part = backward_sg_dispatch<S, VECTOR, MODE, false>(a, active, col, k, nullptr);
+  const float part = backward_sg_dispatch<S, VECTOR, MODE, 0>(a, active, col, k, nullptr);
   if (MODE == BWD_PLIF) plif_block_reduce(a, part, k);
 }
 

@@ -5,6 +5,9 @@
 // for every step in LDS as fp32.  Phase 2 is the ordinary BPTT walk of neuron_bwd.h reading h_t
 // from LDS.  Each work-item touches only its own LDS words, so no barrier is needed.
 //
+// With 16-bit storage and every op rounded, h_t is exactly a storage-dtype value and is parked as 16-bit patterns
+// (half the LDS, twice the resident wavefronts); with fp32 state it stays fp32.
+//
 // Why: the forward then never writes h_seq (4 B per neuron-step less to write in the slowest,
 // write-dominated kernel) and the backward reads x_seq instead of h_seq (same bytes).  LDS holds
 // T * blockDim * V * 4 bytes per block, which also bounds T (see recompute_block()).
@@ -22,6 +25,10 @@
 #endif
 
 namespace sjhip {
+
+// storage-dtype bit pattern of an h that is already a storage-dtype value
+template <typename S> __device__ __forceinline__ uint32_t h_bits(float h) { return Cvt<S>::from_float(h); }
+template <typename S> __device__ __forceinline__ uint32_t h_bits(_Float16 h) { return __builtin_bit_cast(uint16_t, h); }
 
 template <typename S, bool ROUND_EACH, int CH, bool SOFT>
 __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, int64_t col) {
@@ -59,10 +66,17 @@ __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, i
         A::unpack(cur[i], x);
 #pragma unroll
         for (int j = 0; j < V; ++j) neuron_step<R, CH, SOFT>(x[j], v[j], h[j], s[j], tau, a);
+        if constexpr (ROUND_EACH && sizeof(S) == 2) {
+          u32x4 w;
+          w.x = h_bits<S>(h[0]) | (h_bits<S>(h[1]) << 16); w.y = h_bits<S>(h[2]) | (h_bits<S>(h[3]) << 16);
+          w.z = h_bits<S>(h[4]) | (h_bits<S>(h[5]) << 16); w.w = h_bits<S>(h[6]) | (h_bits<S>(h[7]) << 16);
+          reinterpret_cast<u32x4 *>(lds_h)[(int)t * (int)blockDim.x + (int)threadIdx.x] = w;
+        } else {
 #pragma unroll
-        for (int q = 0; q < V / 4; ++q) {
-          f32x4 w; w.x = (float)h[4 * q]; w.y = (float)h[4 * q + 1]; w.z = (float)h[4 * q + 2]; w.w = (float)h[4 * q + 3];
-          lds_h[((int)t * (V / 4) + q) * (int)blockDim.x + (int)threadIdx.x] = w;
+          for (int q = 0; q < V / 4; ++q) {
+            f32x4 w; w.x = (float)h[4 * q]; w.y = (float)h[4 * q + 1]; w.z = (float)h[4 * q + 2]; w.w = (float)h[4 * q + 3];
+            lds_h[((int)t * (V / 4) + q) * (int)blockDim.x + (int)threadIdx.x] = w;
+          }
         }
       }
     }
@@ -96,7 +110,8 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_kernel(con
     }
   }
   const float k = b.k_device ? *b.k_device : b.k;
-  const float part = backward_sg_dispatch<S, true, MODE, true>(b, active, col, k, lds_h, &pre);
+  constexpr int HLDS = (ROUND_EACH && sizeof(S) == 2) ? 2 : 1;
+  const float part = backward_sg_dispatch<S, true, MODE, HLDS>(b, active, col, k, lds_h, &pre);
   if (MODE == BWD_PLIF) plif_block_reduce(b, part, k);
 }
 

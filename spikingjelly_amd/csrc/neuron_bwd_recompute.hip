@@ -14,12 +14,15 @@ namespace {
 
 constexpr unsigned kMaxLds = 159u * 1024u;  // LDS per compute unit on gfx950 minus 1 KiB for static words
 
-// Largest block (128 or 64 lanes) whose h buffer T * block * V * 4 bytes fits in LDS; 0 if none.
-int recompute_block(int dtype, int64_t T) {
-  const int64_t V = dtype == SJHIP_F32 ? 4 : 8;
+// LDS bytes one work-item needs per step for h: its 4 fp32 neurons, its 8 neurons as fp32 (16-bit storage with
+// fp32 state) or its 8 neurons as 16-bit patterns (16-bit storage, every op rounded)
+int64_t h_bytes_per_item(int dtype, bool round_each) { return dtype == SJHIP_F32 ? 16 : (round_each ? 16 : 32); }
+
+// Largest block (128 or 64 lanes) whose h buffer fits in LDS; 0 if none.
+int recompute_block(int dtype, int64_t T, bool round_each) {
   for (int block : {128, 64}) {
     if (block > SJHIP_MAX_BLOCK) continue;
-    if (T * block * V * 4 <= (int64_t)kMaxLds) return block;
+    if (T * block * h_bytes_per_item(dtype, round_each) <= (int64_t)kMaxLds) return block;
   }
   return 0;
 }
@@ -28,7 +31,7 @@ int recompute_block(int dtype, int64_t T) {
 
 bool recompute_supported(int dtype, int64_t T, int64_t N) {
   const int64_t V = dtype == SJHIP_F32 ? 4 : 8;
-  return N % V == 0 && recompute_block(dtype, T) != 0;
+  return N % V == 0 && recompute_block(dtype, T, false) != 0;  // the larger fp32-state footprint: holds for either mode
 }
 
 int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
@@ -56,11 +59,11 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
   if (rc != SJHIP_OK) return rc;
 
   const int V = dtype == SJHIP_F32 ? 4 : 8;
-  const int block = recompute_block(dtype, T);
+  const int block = recompute_block(dtype, T, round_each);
   const int64_t items = N / V;
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "backward(recompute): N=%lld", (long long)N);
-  unsigned lds = (unsigned)(T * block * V * 4);
+  unsigned lds = (unsigned)(T * block * h_bytes_per_item(dtype, round_each));
   const unsigned cap = occupancy_cap_lds(tuning().replay_blocks_per_cu);
   if (cap > lds) lds = cap;
   const bool plif = neuron == SJHIP_NEURON_PLIF;
