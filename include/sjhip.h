@@ -228,7 +228,7 @@ int sjhip_ssa_backward(int dtype, int64_t samples, int heads, int channels_per_h
  * block (64, 128, 256 or 512); "fwd_blocks_per_cu" / "bwd_blocks_per_cu" = cap on resident blocks per
  * compute unit (0 = none, else 2..64; enforced through a dynamic-LDS request), and
  * "replay_blocks_per_cu" likewise for sjhip_neuron_backward_recompute.  The forward cap applies to
- * fp32 storage only (16-bit storage always runs uncapped).  Returns SJHIP_ERR_INVALID otherwise.
+ * fp32 storage with v_seq or h_seq written (spikes-only and 16-bit forwards always run uncapped).  Returns SJHIP_ERR_INVALID otherwise.
  * Results never depend on these.
  */
 int sjhip_set_tuning(const char *key, int value);

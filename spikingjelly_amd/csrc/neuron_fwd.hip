@@ -14,8 +14,10 @@ int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   const int64_t items = (a.N + V - 1) / V;
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "forward: N=%lld needs %lld blocks", (long long)a.N, (long long)blocks);
-  // the residency cap pays for fp32 storage only: 16-bit storage needs more wavefronts to hide its conversions
-  const unsigned lds = sizeof(S) == 4 ? occupancy_cap_lds(tuning().fwd_blocks_per_cu) : 0u;
+  // the residency cap pays for fp32 storage writing two or three [T, N] tensors (spikes plus v_seq and / or h_seq);
+  // with spikes only, and with 16-bit storage (more wavefronts hide its conversions), uncapped is faster (measured)
+  const bool several_outputs = a.v_seq != nullptr || a.h != nullptr;
+  const unsigned lds = (sizeof(S) == 4 && several_outputs) ? occupancy_cap_lds(tuning().fwd_blocks_per_cu) : 0u;
   ProfileScope prof(KC_FORWARD, stream);
   if (vector)
     hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, PACKED>), dim3((unsigned)blocks), dim3(block), lds, stream, a);
