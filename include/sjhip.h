@@ -198,6 +198,11 @@ int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_pa
  * width and T steps of h fitting in LDS: T <= 159 for fp32, 79 for 16-bit storage), else 0. */
 int sjhip_recompute_supported(int dtype, int64_t T, int64_t N);
 
+/* 1 if, beyond being supported, the replay is expected to beat a saved h_seq: its LDS footprint grows with T and
+ * below four resident wavefronts per compute unit (fp32: T > 39) reading h_seq is faster.  `flags` as in
+ * sjhip_neuron_params (only SJHIP_FLAG_FP32_STATE matters).  A policy hint for callers; both paths stay valid. */
+int sjhip_recompute_preferred(int dtype, int64_t T, int64_t N, uint32_t flags);
+
 /*
  * Spike bit-packing over a flattened tensor, LSB first: byte j bit i = (src[8j+i] != 0).
  *   src  n elements of `dtype` (F32/F16/BF16/U8)     dst  (n+7)/8 bytes; pad bits of the last byte are 0
@@ -228,7 +233,8 @@ int sjhip_ssa_backward(int dtype, int64_t samples, int heads, int channels_per_h
  * block (64, 128, 256 or 512); "fwd_blocks_per_cu" / "bwd_blocks_per_cu" = cap on resident blocks per
  * compute unit (0 = none, else 2..64; enforced through a dynamic-LDS request), and
  * "replay_blocks_per_cu" likewise for sjhip_neuron_backward_recompute.  The forward cap applies to
- * fp32 storage with v_seq or h_seq written (spikes-only and 16-bit forwards always run uncapped).  Returns SJHIP_ERR_INVALID otherwise.
+ * fp32 storage with v_seq or h_seq written (spikes-only and 16-bit forwards always run uncapped); it is
+ * doubled for T < 16 and dropped for T < 4, where few rows are in flight per work-item.  Returns SJHIP_ERR_INVALID otherwise.
  * Results never depend on these.
  */
 int sjhip_set_tuning(const char *key, int value);

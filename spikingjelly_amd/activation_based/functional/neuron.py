@@ -125,10 +125,12 @@ def _hip_mode_flags(x_seq: torch.Tensor) -> int:
 
 
 def _hip_recompute(x2: torch.Tensor) -> bool:
-    """Replay the forward inside the backward kernel instead of saving h_seq, when the shape allows."""
+    """Replay the forward inside the backward kernel instead of saving h_seq, when the shape allows and the
+    sequence is short enough for the replay to pay (its LDS footprint grows with T)."""
     from ..hip_kernel import library as L
 
-    return bool(configure.hip_backward_recompute) and L.recompute_supported(x2.dtype, x2.shape[0], x2.shape[1])
+    return bool(configure.hip_backward_recompute) and L.recompute_preferred(x2.dtype, x2.shape[0], x2.shape[1],
+                                                                            _hip_mode_flags(x2))
 
 
 def _needs_grad(*tensors: torch.Tensor) -> bool:

@@ -38,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "sjhip_neuron_backward",
     "sjhip_neuron_backward_recompute",
     "sjhip_recompute_supported",
+    "sjhip_recompute_preferred",
     "sjhip_ssa_supported",
     "sjhip_ssa_forward",
     "sjhip_ssa_backward",
@@ -119,6 +120,8 @@ def load() -> ctypes.CDLL:
         ]
         lib.sjhip_recompute_supported.restype = c_int
         lib.sjhip_recompute_supported.argtypes = [c_int, c_int64, c_int64]
+        lib.sjhip_recompute_preferred.restype = c_int
+        lib.sjhip_recompute_preferred.argtypes = [c_int, c_int64, c_int64, c_uint32]
         lib.sjhip_ssa_supported.restype = c_int
         lib.sjhip_ssa_supported.argtypes = [c_int, c_int, c_int64]
         lib.sjhip_ssa_forward.restype = c_int
@@ -182,6 +185,11 @@ def current_stream_ptr(device: torch.device) -> int:
 
 def ptr(t) -> int | None:
     return None if t is None else t.data_ptr()
+
+
+def recompute_preferred(dtype: torch.dtype, T: int, N: int, flags: int) -> bool:
+    """Whether the replay backward is supported and expected to be faster than a saved ``h_seq`` (short enough T)."""
+    return bool(load().sjhip_recompute_preferred(dtype_id(dtype), T, N, flags))
 
 
 def recompute_supported(dtype: torch.dtype, T: int, N: int) -> bool:

@@ -34,6 +34,13 @@ bool recompute_supported(int dtype, int64_t T, int64_t N) {
   return N % V == 0 && recompute_block(dtype, T, false) != 0;  // the larger fp32-state footprint: holds for either mode
 }
 
+bool recompute_preferred(int dtype, int64_t T, int64_t N, bool round_each) {
+  // the replay needs T * 64 lanes * h_bytes of LDS per wavefront; below four resident wavefronts per compute unit
+  // it is slower than reading a saved h_seq (measured: T = 32 still wins, T = 64 loses, fp32)
+  if (!recompute_supported(dtype, T, N)) return false;
+  return 4 * T * 64 * h_bytes_per_item(dtype, round_each) <= (int64_t)kMaxLds;
+}
+
 int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
                               const void *x_seq, const void *v_init, const float *k_device,
                               const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,

@@ -16,8 +16,13 @@ int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "forward: N=%lld needs %lld blocks", (long long)a.N, (long long)blocks);
   // the residency cap pays for fp32 storage writing two or three [T, N] tensors (spikes plus v_seq and / or h_seq);
   // with spikes only, and with 16-bit storage (more wavefronts hide its conversions), uncapped is faster (measured)
+  // A short sequence has few rows in flight per work-item and needs more resident blocks instead: twice the cap
+  // below 16 steps, none below 4 (measured at T = 1, 2, 4, 8, 16).
   const bool several_outputs = a.v_seq != nullptr || a.h != nullptr;
-  const unsigned lds = (sizeof(S) == 4 && several_outputs) ? occupancy_cap_lds(tuning().fwd_blocks_per_cu) : 0u;
+  int cap = tuning().fwd_blocks_per_cu;
+  if (a.T < 4) cap = 0;
+  else if (a.T < 16) cap *= 2;
+  const unsigned lds = (sizeof(S) == 4 && several_outputs) ? occupancy_cap_lds(cap) : 0u;
   ProfileScope prof(KC_FORWARD, stream);
   if (vector)
     hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, PACKED>), dim3((unsigned)blocks), dim3(block), lds, stream, a);

@@ -189,6 +189,12 @@ int sjhip_recompute_supported(int dtype, int64_t T, int64_t N) {
   return recompute_supported(dtype, T, N) ? 1 : 0;
 }
 
+int sjhip_recompute_preferred(int dtype, int64_t T, int64_t N, uint32_t flags) {
+  if (!valid_dtype_fp(dtype) || T < 1 || N < 1) return 0;
+  const bool round_each = dtype != SJHIP_F32 && !(flags & SJHIP_FLAG_FP32_STATE);
+  return recompute_preferred(dtype, T, N, round_each) ? 1 : 0;
+}
+
 int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_params *p, int64_t T, int64_t N,
                                     const void *x_seq, const void *v_init, const float *rtau_device,
                                     const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,

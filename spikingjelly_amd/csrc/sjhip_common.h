@@ -249,6 +249,7 @@ int launch_forward_packed(int neuron, int dtype, const sjhip_neuron_params &p, i
                           const void *x_seq, const void *v_init, const float *k_device, uint8_t *spike_bits,
                           void *v_seq, void *v_last, hipStream_t stream);
 bool recompute_supported(int dtype, int64_t T, int64_t N);
+bool recompute_preferred(int dtype, int64_t T, int64_t N, bool round_each);
 int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
                               const void *x_seq, const void *v_init, const float *k_device,
                               const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,

@@ -70,3 +70,16 @@ def test_python_binding_raises_with_library_message():
         import torch
 
         L.dtype_id(torch.float64)
+
+
+def test_replay_policy_follows_the_lds_footprint():
+    lib = L.load()
+    N = 1 << 20
+    assert lib.sjhip_recompute_supported(L.DTYPE_F32, 128, N) == 1
+    assert lib.sjhip_recompute_preferred(L.DTYPE_F32, 16, N, 0) == 1
+    assert lib.sjhip_recompute_preferred(L.DTYPE_F32, 39, N, 0) == 1 and lib.sjhip_recompute_preferred(L.DTYPE_F32, 40, N, 0) == 0
+    assert lib.sjhip_recompute_preferred(L.DTYPE_F32, 16, N + 1, 0) == 0  # not supported at all: N % 4
+    # 16-bit: every op rounded parks h as 16-bit (same footprint as fp32), fp32 state needs twice as much
+    assert lib.sjhip_recompute_preferred(L.DTYPE_BF16, 39, N, 0) == 1
+    assert lib.sjhip_recompute_preferred(L.DTYPE_BF16, 19, N, L.FLAG_FP32_STATE) == 1
+    assert lib.sjhip_recompute_preferred(L.DTYPE_BF16, 20, N, L.FLAG_FP32_STATE) == 0
