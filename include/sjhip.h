@@ -195,11 +195,11 @@ int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_pa
                                     void *stream);
 
 /* 1 if sjhip_neuron_backward_recompute can serve [T,N] of `dtype` (N a multiple of the 128-bit vector
- * width and T steps of h fitting in LDS: T <= 159 for fp32, 79 for 16-bit storage), else 0. */
+ * width and T steps of h fitting in LDS: T <= 159), else 0. */
 int sjhip_recompute_supported(int dtype, int64_t T, int64_t N);
 
 /* 1 if, beyond being supported, the replay is expected to beat a saved h_seq: its LDS footprint grows with T and
- * below four resident wavefronts per compute unit (fp32: T > 39) reading h_seq is faster.  `flags` as in
+ * below four resident wavefronts per compute unit (T > 39) reading h_seq is faster.  `flags` as in
  * sjhip_neuron_params (only SJHIP_FLAG_FP32_STATE matters).  A policy hint for callers; both paths stay valid. */
 int sjhip_recompute_preferred(int dtype, int64_t T, int64_t N, uint32_t flags);
 

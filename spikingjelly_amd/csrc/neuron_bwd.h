@@ -128,7 +128,7 @@ __device__ __forceinline__ float qif_dh_dv(float v, float k, const BwdArgs &a) {
 // First PF rows (t = T-1 downwards) of grad_spike and grad_v_seq, requested ahead of their use.
 template <typename S, bool VECTOR> struct BwdPrologue {
   typedef Acc<S, VECTOR, SJHIP_BWD_NT != 0> A;
-  static constexpr int PF = sizeof(S) == 2 ? SJHIP_BWD_PF16 : SJHIP_BWD_PF;
+  static constexpr int PF = (sizeof(S) == 2 && A::V == 8) ? SJHIP_BWD_PF16 : SJHIP_BWD_PF;
   typename A::raw_t gs[PF], gv[PF];
   __device__ __forceinline__ void load(const BwdArgs &a, int64_t col) {
     typedef typename A::elem_t E;

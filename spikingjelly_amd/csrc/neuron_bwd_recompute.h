@@ -36,7 +36,7 @@ __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, i
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
-  constexpr int PF = sizeof(S) == 2 ? SJHIP_REPLAY_PF16 : SJHIP_REPLAY_PF;
+  constexpr int PF = (sizeof(S) == 2 && V == 8) ? SJHIP_REPLAY_PF16 : SJHIP_REPLAY_PF;
 
   const int64_t N = a.N, T = a.T;
   const E *xp = (const E *)a.x + col;

@@ -9,14 +9,17 @@ namespace sjhip {
 extern template int launch_recompute_dtype<float>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
 extern template int launch_recompute_dtype<f16_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
 extern template int launch_recompute_dtype<bf16_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
+extern template int launch_recompute_dtype<f16n_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
+extern template int launch_recompute_dtype<bf16n_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
 
 namespace {
 
 constexpr unsigned kMaxLds = 159u * 1024u;  // LDS per compute unit on gfx950 minus 1 KiB for static words
 
-// LDS bytes one work-item needs per step for h: its 4 fp32 neurons, its 8 neurons as fp32 (16-bit storage with
-// fp32 state) or its 8 neurons as 16-bit patterns (16-bit storage, every op rounded)
-int64_t h_bytes_per_item(int dtype, bool round_each) { return dtype == SJHIP_F32 ? 16 : (round_each ? 16 : 32); }
+// LDS bytes one work-item needs per step for h: its 4 fp32 neurons (fp32 storage, and 16-bit storage with fp32
+// state, which runs four neurons per work-item through 8-byte accesses) or its 8 neurons as 16-bit patterns
+// (16-bit storage, every op rounded)
+int64_t h_bytes_per_item(int dtype, bool round_each) { (void)dtype; (void)round_each; return 16; }
 
 // Largest block (128 or 64 lanes) whose h buffer fits in LDS; 0 if none.
 int recompute_block(int dtype, int64_t T, bool round_each) {
@@ -31,7 +34,7 @@ int recompute_block(int dtype, int64_t T, bool round_each) {
 
 bool recompute_supported(int dtype, int64_t T, int64_t N) {
   const int64_t V = dtype == SJHIP_F32 ? 4 : 8;
-  return N % V == 0 && recompute_block(dtype, T, false) != 0;  // the larger fp32-state footprint: holds for either mode
+  return N % V == 0 && recompute_block(dtype, T, false) != 0;
 }
 
 bool recompute_preferred(int dtype, int64_t T, int64_t N, bool round_each) {
@@ -65,7 +68,8 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
                       grad_x_seq, grad_v_init, grad_rtau, workspace);
   if (rc != SJHIP_OK) return rc;
 
-  const int V = dtype == SJHIP_F32 ? 4 : 8;
+  const bool narrow = dtype != SJHIP_F32 && !round_each;  // 16-bit storage, fp32 state: four neurons per work-item
+  const int V = (dtype == SJHIP_F32 || narrow) ? 4 : 8;
   const int block = recompute_block(dtype, T, round_each);
   const int64_t items = N / V;
   const int64_t blocks = (items + block - 1) / block;
@@ -79,8 +83,14 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
     ProfileScope prof(KC_BACKWARD, stream);
     switch (dtype) {
       case SJHIP_F32: rc = launch_recompute_dtype<float>(f, b, false, mode, block, lds, blocks, stream); break;
-      case SJHIP_F16: rc = launch_recompute_dtype<f16_t>(f, b, round_each, mode, block, lds, blocks, stream); break;
-      case SJHIP_BF16: rc = launch_recompute_dtype<bf16_t>(f, b, round_each, mode, block, lds, blocks, stream); break;
+      case SJHIP_F16:
+        rc = narrow ? launch_recompute_dtype<f16n_t>(f, b, false, mode, block, lds, blocks, stream)
+                    : launch_recompute_dtype<f16_t>(f, b, round_each, mode, block, lds, blocks, stream);
+        break;
+      case SJHIP_BF16:
+        rc = narrow ? launch_recompute_dtype<bf16n_t>(f, b, false, mode, block, lds, blocks, stream)
+                    : launch_recompute_dtype<bf16_t>(f, b, round_each, mode, block, lds, blocks, stream);
+        break;
       default: return fail(SJHIP_ERR_INVALID, "backward(recompute): dtype %d", dtype);
     }
     if (rc != SJHIP_OK) return rc;

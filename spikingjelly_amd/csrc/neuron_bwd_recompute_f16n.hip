@@ -1,0 +1,6 @@
+// Recompute-backward kernels for storage dtype f16n_t (8-byte accesses, fp32 state).
+#include "neuron_bwd_recompute_launch.h"
+
+namespace sjhip {
+template int launch_recompute_dtype<f16n_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
+}  // namespace sjhip

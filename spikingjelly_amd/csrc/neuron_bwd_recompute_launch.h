@@ -38,7 +38,8 @@ int launch_mode(const FwdArgs &f, const BwdArgs &b, int mode, int block, unsigne
 template <typename S>
 int launch_recompute_dtype(const FwdArgs &f, const BwdArgs &b, bool round_each, int mode, int block, unsigned lds,
                            int64_t blocks, hipStream_t stream) {
-  if constexpr (!std::is_same<S, float>::value) {
+  // the 8-byte access tags exist for fp32 state only
+  if constexpr (std::is_same<S, f16_t>::value || std::is_same<S, bf16_t>::value) {
     if (round_each) return launch_mode<S, true>(f, b, mode, block, lds, blocks, stream);
   }
   return launch_mode<S, false>(f, b, mode, block, lds, blocks, stream);

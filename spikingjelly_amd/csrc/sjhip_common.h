@@ -16,9 +16,14 @@ namespace sjhip {
 // ----------------------------------------------------------------------------------------------
 struct f16_t { uint16_t bits; };
 struct bf16_t { uint16_t bits; };
+// The same storage dtypes accessed 8 bytes (four neurons) at a time instead of 16: for kernels whose per-neuron
+// on-chip state, not the access width, limits the resident wavefronts (the fp32-state replay backward).
+struct f16n_t { uint16_t bits; };
+struct bf16n_t { uint16_t bits; };
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 template <typename S> struct Cvt;
 
@@ -56,6 +61,9 @@ template <> struct Cvt<bf16_t> {
   }
   static __host__ __device__ __forceinline__ float round(float f) { return to_float(from_float(f)); }
 };
+
+template <> struct Cvt<f16n_t> : Cvt<f16_t> {};
+template <> struct Cvt<bf16n_t> : Cvt<bf16_t> {};
 
 // Cache policy of one access: NT marks the line as streaming (non-temporal), otherwise default.
 // Measured on MI355X: read-mostly kernels (backward, unpack) gain from NT on both loads and stores,
@@ -150,6 +158,24 @@ template <typename H, bool NT> struct Acc16v {
   }
   static __device__ __forceinline__ void store_spikes(elem_t *p, const _Float16 (&f)[V]) { store(p, f); }
 };
+// four 16-bit neurons per 8-byte access (fp32 arithmetic only)
+template <typename H, bool NT> struct Acc16n {
+  static constexpr int V = 4;
+  typedef uint16_t elem_t;
+  typedef u32x2 raw_t;
+  static __device__ __forceinline__ raw_t load(const elem_t *p) { return stream_load<NT>((const raw_t *)p); }
+  static __device__ __forceinline__ raw_t zero() { return (raw_t)(0u); }
+  static __device__ __forceinline__ void unpack(raw_t r, float (&f)[V]) {
+    f[0] = Cvt<H>::to_float((uint16_t)(r.x & 0xffffu)); f[1] = Cvt<H>::to_float((uint16_t)(r.x >> 16));
+    f[2] = Cvt<H>::to_float((uint16_t)(r.y & 0xffffu)); f[3] = Cvt<H>::to_float((uint16_t)(r.y >> 16));
+  }
+  static __device__ __forceinline__ void store(elem_t *p, const float (&f)[V]) {
+    raw_t r;
+    r.x = (uint32_t)Cvt<H>::from_float(f[0]) | ((uint32_t)Cvt<H>::from_float(f[1]) << 16);
+    r.y = (uint32_t)Cvt<H>::from_float(f[2]) | ((uint32_t)Cvt<H>::from_float(f[3]) << 16);
+    stream_store<NT>((raw_t *)p, r);
+  }
+};
 template <typename H, bool NT> struct Acc16s {
   static constexpr int V = 1;
   typedef uint16_t elem_t;
@@ -177,6 +203,10 @@ template <bool NT> struct Acc<f16_t, true, NT> : Acc16v<f16_t, NT> {};
 template <bool NT> struct Acc<f16_t, false, NT> : Acc16s<f16_t, NT> {};
 template <bool NT> struct Acc<bf16_t, true, NT> : Acc16v<bf16_t, NT> {};
 template <bool NT> struct Acc<bf16_t, false, NT> : Acc16s<bf16_t, NT> {};
+template <bool NT> struct Acc<f16n_t, true, NT> : Acc16n<f16_t, NT> {};
+template <bool NT> struct Acc<f16n_t, false, NT> : Acc16s<f16_t, NT> {};
+template <bool NT> struct Acc<bf16n_t, true, NT> : Acc16n<bf16_t, NT> {};
+template <bool NT> struct Acc<bf16n_t, false, NT> : Acc16s<bf16_t, NT> {};
 
 // Initial state of this work-item's neurons: its V elements of the [N] tensor, or the one stored element
 // for every neuron when the caller passed a broadcast state.

@@ -79,7 +79,8 @@ def test_replay_policy_follows_the_lds_footprint():
     assert lib.sjhip_recompute_preferred(L.DTYPE_F32, 16, N, 0) == 1
     assert lib.sjhip_recompute_preferred(L.DTYPE_F32, 39, N, 0) == 1 and lib.sjhip_recompute_preferred(L.DTYPE_F32, 40, N, 0) == 0
     assert lib.sjhip_recompute_preferred(L.DTYPE_F32, 16, N + 1, 0) == 0  # not supported at all: N % 4
-    # 16-bit: every op rounded parks h as 16-bit (same footprint as fp32), fp32 state needs twice as much
-    assert lib.sjhip_recompute_preferred(L.DTYPE_BF16, 39, N, 0) == 1
-    assert lib.sjhip_recompute_preferred(L.DTYPE_BF16, 19, N, L.FLAG_FP32_STATE) == 1
-    assert lib.sjhip_recompute_preferred(L.DTYPE_BF16, 20, N, L.FLAG_FP32_STATE) == 0
+    # 16-bit storage has the fp32 footprint per work-item: eight neurons parked as 16-bit patterns (every op rounded)
+    # or four neurons parked as fp32 (fp32 state)
+    for flags in (0, L.FLAG_FP32_STATE):
+        assert lib.sjhip_recompute_preferred(L.DTYPE_BF16, 39, N, flags) == 1
+        assert lib.sjhip_recompute_preferred(L.DTYPE_BF16, 40, N, flags) == 0
