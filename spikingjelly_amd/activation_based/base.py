@@ -270,3 +270,132 @@ class MemoryModule(nn.Module, StepModule):
         replica = super()._replicate_for_data_parallel()
         replica._memories = self._memories.copy()
         return replica
+
+
+# ---- memories of a whole module tree -----------------------------------------------------
+def _memory_owners(module: nn.Module, path: Tuple[str, ...] = ()):
+    """Pre-order walk of the tree: a module before its children, children in registration order."""
+    if isinstance(module, MemoryModule):
+        yield path, module
+    for child_name, child in module.named_children():
+        yield from _memory_owners(child, path + (child_name,))
+
+
+def named_memories(module: nn.Module, prefix: str = "") -> Generator:
+    """``(dotted name, value)`` of every memory below ``module``, the tree-wide counterpart of
+    ``named_parameters()``.  Order and naming follow the reference (``base.py:1128-1178``): a
+    module's own memories in registration order, then its children's."""
+    head = (prefix,) if prefix else ()
+    for path, owner in _memory_owners(module):
+        for name, value in owner.named_memories():
+            yield ".".join(head + path + (name,)), value
+
+
+def memories(module: nn.Module) -> Generator:
+    """Values of :func:`named_memories` (reference ``base.py:1181-1221``)."""
+    for _, value in named_memories(module):
+        yield value
+
+
+def extract_memories(module: nn.Module) -> list:
+    """Snapshot (a list of references, nothing is cloned) of every memory below ``module``
+    (reference ``base.py:1224-1262``)."""
+    return [value for _, value in named_memories(module)]
+
+
+def load_memories(module: nn.Module, memory_list: list) -> None:
+    """Inverse of :func:`extract_memories`: assign ``memory_list`` to the memories in the same
+    order.  A list of the wrong length raises ``ValueError`` before anything is written
+    (reference ``base.py:1265-1312``)."""
+    slots = [(owner, name) for _, owner in _memory_owners(module) for name, _ in owner.named_memories()]
+    if len(slots) != len(memory_list):
+        raise ValueError(
+            f"Memory length mismatch: model has {len(slots)} memories but list contains {len(memory_list)}"
+        )
+    for (owner, name), value in zip(slots, memory_list):
+        owner._memories[name] = value
+
+
+def to_functional_forward(module: nn.Module, fn=None):
+    """``f(inputs, states, **kwargs) -> (outputs, new_states)`` for any module tree.
+
+    ``states`` is ordered like :func:`extract_memories`; ``outputs`` is always a tuple.  The module's
+    own memories are the same before and after a call, also when the forward raises.  Three routes, as in
+    the reference (``base.py:1315-1551``): a single ``MemoryModule`` with a pure ``functional_forward`` of
+    its own is called directly; an ``nn.Sequential`` whose direct children own every state and are pure
+    threads ``states`` through them without touching a memory (a child's tuple output becomes the next
+    child's positional arguments, keyword arguments go to the first child only); every other tree runs its
+    ordinary ``forward`` (or ``fn``) between a :func:`load_memories` of ``states`` and a restore of what
+    was there.
+    """
+    owners = [owner for _, owner in _memory_owners(module)]
+    n_states = sum(len(owner._memories) for owner in owners)
+
+    def check(states) -> None:
+        if len(states) != n_states:
+            raise ValueError(f"{module.__class__.__name__} expected {n_states} states, but got {len(states)}.")
+
+    def overrides(owner: MemoryModule, name: str) -> bool:
+        return getattr(type(owner), name) is not getattr(MemoryModule, name)
+
+    def is_pure(owner: nn.Module) -> bool:
+        return isinstance(owner, MemoryModule) and (
+            overrides(owner, "functional_forward")
+            or overrides(owner, "single_step_functional_forward")
+            or (owner.step_mode == "m" and overrides(owner, "multi_step_functional_forward"))
+        )
+
+    def as_tuple(result) -> tuple:
+        return tuple(result) if isinstance(result, (tuple, list)) else (result,)
+
+    if fn is None and len(owners) == 1 and owners[0] is module and is_pure(module):
+
+        def direct(inputs, states, **kwargs):
+            check(states)
+            return module.functional_forward(inputs, states, **kwargs)
+
+        return direct
+
+    if fn is None and isinstance(module, nn.Sequential):
+        stages = list(module.children())
+        counts = [len(stage._memories) if is_pure(stage) else 0 for stage in stages]
+
+        if sum(counts) == n_states:
+
+            def threaded(inputs, states, **kwargs):
+                check(states)
+                flowing, new_states, first = tuple(inputs), [], 0
+                for stage, count in zip(stages, counts):
+                    if count:
+                        flowing, out_states = stage.functional_forward(flowing, states[first:first + count], **kwargs)
+                        new_states.extend(out_states)
+                        first += count
+                    else:
+                        flowing = as_tuple(stage(*flowing, **kwargs))
+                    kwargs = {}
+                return tuple(flowing), tuple(new_states)
+
+            return threaded
+
+        def call(*inputs, **kwargs):
+            flowing = inputs
+            for stage in stages:
+                flowing = as_tuple(stage(*flowing, **kwargs))
+                kwargs = {}
+            return flowing[0] if len(flowing) == 1 else flowing
+
+    else:
+        call = module.forward if fn is None else fn
+
+    def swapped(inputs, states, **kwargs):
+        check(states)
+        saved = extract_memories(module)
+        load_memories(module, list(states))
+        try:
+            outputs = as_tuple(call(*inputs, **kwargs))
+            new_states = tuple(extract_memories(module))
+        finally:
+            load_memories(module, saved)
+        return outputs, new_states
+
+    return swapped

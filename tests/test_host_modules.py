@@ -219,3 +219,150 @@ def test_hip_bit_packing_refuses_cpu_tensors():
         hip_compress.bit_spike_compress(torch.ones(16))
     with pytest.raises(RuntimeError, match="ROCm device"):
         hip_compress.bit_spike_decompress(torch.zeros(2, dtype=torch.uint8), (16,))
+
+
+# ---- tree-wide memory helpers (reference base.py:1128-1551; cases follow test/activation_based/test_memory.py) ----
+class _Counter(base.MemoryModule):
+    """Stateful in the classic style: the forward reads and writes its own memories."""
+
+    def __init__(self, start=0.0):
+        super().__init__()
+        self.register_memory("count", torch.tensor(start))
+        self.register_memory("total", torch.tensor(0.0))
+
+    def single_step_forward(self, x, *, scale=1.0):
+        self.count = self.count + 1.0
+        self.total = self.total + x.sum() * scale
+        return x * self.count
+
+
+def _memory_tree():
+    net = torch.nn.Sequential(_Counter(), torch.nn.Identity(), torch.nn.Sequential(_Counter(5.0)))
+    return net
+
+
+def test_named_memories_walks_the_tree_in_registration_order():
+    net = _memory_tree()
+    names = [n for n, _ in base.named_memories(net)]
+    assert names == ["0.count", "0.total", "2.0.count", "2.0.total"]
+    assert [n for n, _ in base.named_memories(net, prefix="net")] == ["net." + n for n in names]
+    assert [float(v) for v in base.memories(net)] == [0.0, 0.0, 5.0, 0.0]
+    assert list(base.named_memories(torch.nn.Linear(2, 2))) == []
+
+
+def test_extract_and_load_memories_round_trip_and_length_check():
+    net = _memory_tree()
+    net(torch.ones(3))
+    taken = base.extract_memories(net)
+    assert [float(v) for v in taken] == [1.0, 3.0, 6.0, 3.0]
+    base.load_memories(net, [v + 10 for v in taken])
+    assert [float(v) for v in base.extract_memories(net)] == [11.0, 13.0, 16.0, 13.0]
+    assert float(net[2][0].count) == 16.0
+    with pytest.raises(ValueError, match="mismatch"):
+        base.load_memories(net, taken[:-1])
+    with pytest.raises(ValueError, match="mismatch"):
+        base.load_memories(net, taken + [torch.tensor(0.0)])
+    assert [float(v) for v in base.extract_memories(net)] == [11.0, 13.0, 16.0, 13.0]  # nothing half-written
+
+
+def test_to_functional_forward_swaps_states_in_and_restores_them():
+    module = _Counter(7.0)
+    f = base.to_functional_forward(module)
+    x = torch.tensor([1.0, 2.0])
+    outputs, states = f((x,), (torch.tensor(1.0), torch.tensor(4.0)), scale=2.0)
+    assert torch.equal(outputs[0], x * 2.0)
+    assert [float(s) for s in states] == [2.0, 10.0]
+    assert float(module.count) == 7.0 and float(module.total) == 0.0
+    with pytest.raises(ValueError, match="expected 2 states"):
+        f((x,), (torch.tensor(1.0),))
+
+    class Failing(_Counter):
+        def single_step_forward(self, x):
+            self.count = self.count + x
+            raise RuntimeError("expected failure")
+
+    bad = Failing(3.0)
+    with pytest.raises(RuntimeError, match="expected failure"):
+        base.to_functional_forward(bad)((torch.tensor(1.0),), (torch.tensor(0.0), torch.tensor(0.0)))
+    assert float(bad.count) == 3.0
+
+
+def test_to_functional_forward_nested_stateless_and_custom_fn():
+    net = _memory_tree()
+    f = base.to_functional_forward(net)
+    x = torch.ones(2)
+    start = tuple(torch.tensor(v) for v in (1.0, 0.0, 2.0, 0.0))
+    outputs, states = f((x,), start)
+    assert torch.equal(outputs[0], x * 2.0 * 3.0)
+    assert [float(s) for s in states] == [2.0, 2.0, 3.0, 4.0]
+    assert [float(v) for v in base.extract_memories(net)] == [0.0, 0.0, 5.0, 0.0]
+
+    lin = torch.nn.Linear(4, 2)
+    outputs, states = base.to_functional_forward(lin)((torch.ones(3, 4),), ())
+    assert states == () and torch.equal(outputs[0], lin(torch.ones(3, 4)))
+
+    module = _Counter()
+    outputs, states = base.to_functional_forward(module, lambda x: (x + module.count, x))(
+        (torch.tensor(1.0),), (torch.tensor(4.0), torch.tensor(0.0)))
+    assert [float(o) for o in outputs] == [5.0, 1.0] and float(states[0]) == 4.0
+
+
+def test_to_functional_forward_uses_pure_forwards_without_touching_memories():
+    class Pure(base.MemoryModule):
+        def __init__(self):
+            super().__init__()
+            self.register_memory("left", torch.tensor(10.0))
+            self.register_memory("right", torch.tensor(20.0))
+
+        def single_step_functional_forward(self, inputs, states, **kwargs):
+            left, right = states[0] + inputs[0], states[1] + inputs[1]
+            return (left, right), (left, right)
+
+        def forward(self, *args, **kwargs):
+            raise AssertionError("the stateful path was used")
+
+    class Split(torch.nn.Module):
+        def forward(self, x, y, *, scale=1.0):
+            return (x + y) * scale, x - y
+
+    pure = Pure()
+    outputs, states = base.to_functional_forward(torch.nn.Sequential(Split(), pure))(
+        (torch.tensor(3.0), torch.tensor(2.0)), (torch.tensor(1.0), torch.tensor(4.0)), scale=2.0)
+    assert [float(o) for o in outputs] == [11.0, 5.0] and [float(s) for s in states] == [11.0, 5.0]
+    assert float(pure.left) == 10.0 and float(pure.right) == 20.0
+
+    # multi-step mode falls back on the default loop over single_step_functional_forward
+    class Running(base.MemoryModule):
+        def __init__(self):
+            super().__init__()
+            self.register_memory("state", torch.tensor(0.0))
+            self.step_mode = "m"
+
+        def single_step_functional_forward(self, inputs, states, **kwargs):
+            state = states[0] + inputs[0]
+            return (state,), (state,)
+
+        def forward(self, *args, **kwargs):
+            raise AssertionError("the stateful path was used")
+
+    outputs, states = base.to_functional_forward(Running())((torch.tensor([1.0, 2.0, 3.0]),), (torch.tensor(4.0),))
+    assert outputs[0].tolist() == [5.0, 7.0, 10.0] and float(states[0]) == 10.0
+
+    # a sequential of stateless stages passes tuples on as positional arguments
+    class Combine(torch.nn.Module):
+        def forward(self, total, difference):
+            return total + difference
+
+    outputs, states = base.to_functional_forward(torch.nn.Sequential(Split(), Combine()))(
+        (torch.tensor(3.0), torch.tensor(2.0)), (), scale=2.0)
+    assert states == () and float(outputs[0]) == 11.0
+
+
+def test_to_functional_forward_on_a_neuron_matches_the_module():
+    node = neuron.LIFNode(tau=2.0, step_mode="m")
+    node.v = torch.full((5,), 0.25)
+    x_seq = torch.randn(6, 5, generator=torch.Generator().manual_seed(3))
+    outputs, states = base.to_functional_forward(node)((x_seq,), (torch.zeros(5),))
+    ref = neuron.LIFNode(tau=2.0, step_mode="m")
+    assert torch.equal(outputs[0], ref(x_seq)) and torch.equal(states[0], ref.v)
+    assert torch.equal(node.v, torch.full((5,), 0.25))
