@@ -133,16 +133,24 @@ def other_workload(args) -> int:
                "plif_reduce_ms": _kernel_ms(L, L.KC_PLIF_REDUCE)})
         return 0
 
-    if args.workload == "qif":
-        # the config-2 shape with the quadratic integrate-and-fire neuron (state-dependent dh/dv in the backward)
+    if args.workload in ("qif", "ilif"):
+        # the config-2 shape with another neuron of the same kernels: the quadratic integrate-and-fire neuron
+        # (state-dependent dh/dv in the backward) or the integer-valued LIF (multi-level counts, windowed gradient)
         shape = (16, 256, 128, 32, 32)
         T, N = shape[0], 256 * 128 * 32 * 32
         g = torch.Generator(device=dev).manual_seed(1002)
-        x = (torch.randn(shape, generator=g, device=dev) * 0.4 + 0.3).requires_grad_()
+        if args.workload == "qif":
+            x = (torch.randn(shape, generator=g, device=dev) * 0.4 + 0.3).requires_grad_()
+            node = neuron.QIFNode(tau=2.0, surrogate_function=surrogate.ATan(2.0), step_mode="m", backend="hip",
+                                  store_v_seq=True).to(dev)
+            label, what = "QIF", "QIFNode tau=2, v_c=0.8, a0=1, hard reset -0.1, ATan(2), x [16,256,128,32,32] fp32 ~N(0.3,0.4)"
+        else:
+            x = (torch.randn(shape, generator=g, device=dev) * 1.5 + 1.0).requires_grad_()
+            node = neuron.ILIFNode(tau=4.0 / 3.0, surrogate_function=surrogate.MultiLevelSpikeCount(4), step_mode="m",
+                                   backend="hip", store_v_seq=True).to(dev)
+            label, what = "ILIF", "ILIFNode tau=4/3, v_th=1, counts 0..4, x [16,256,128,32,32] fp32 ~N(1.0,1.5)"
         gs = torch.randn(shape, generator=g, device=dev)
         gv = torch.randn(shape, generator=g, device=dev) * 0.1
-        node = neuron.QIFNode(tau=2.0, surrogate_function=surrogate.ATan(2.0), step_mode="m", backend="hip",
-                              store_v_seq=True).to(dev)
 
         def step():
             s = node(x)
@@ -155,10 +163,9 @@ def other_workload(args) -> int:
         bytes_each = 16 * T * N + 4 * N
         dom = "forward" if f_ms >= b_ms else "backward"
         d_ms = max(f_ms, b_ms)
-        _emit(args, "neuron-steps/sec QIF fwd+bwd fp32 T=16 N=33.5M, 1 MI355X", "neuron-steps/s",
+        _emit(args, f"neuron-steps/sec {label} fwd+bwd fp32 T=16 N=33.5M, 1 MI355X", "neuron-steps/s",
               T * N / (elapsed / args.steps), elapsed, "f32",
-              {"workload": "QIFNode tau=2, v_c=0.8, a0=1, hard reset -0.1, ATan(2), x [16,256,128,32,32] fp32 ~N(0.3,0.4), "
-                           "store_v_seq=True, grad_spike ~N(0,1), grad_v ~N(0,0.1)", "T": T, "N": N},
+              {"workload": what + ", store_v_seq=True, grad_spike ~N(0,1), grad_v ~N(0,0.1)", "T": T, "N": N},
               {"bound": "hbm", "achieved": bytes_each / (d_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                "frac": bytes_each / (d_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": dom,
                "kernel_ms": d_ms, "algorithmic_bytes": bytes_each, "forward_ms": f_ms, "backward_ms": b_ms})
@@ -252,7 +259,7 @@ def main() -> int:
     ap.add_argument("--cpu-sample-neurons", type=int, default=1 << 23)
     ap.add_argument("--cpu-repeats", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "qif"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "qif", "ilif"],
                     help="config2 (default) is the headline metric; the others are secondary measurements")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -17,6 +17,8 @@
  *                             spikingjelly/activation_based/triton_kernel/neuron_kernel/lif.py:673-763
  *                             QIF: torch.ops.sj.cupy_multistep_qif_forward and its backward,
  *                             cuda_kernel/neuron_kernel/multi_step/qif.py:21-277, 628-701
+ *                             ILIF: torch.ops.sj.multistep_ilif_forward{,_no_grad} and its backward,
+ *                             triton_kernel/neuron_kernel/ilif.py:37-235, 241-462, 556-726
  *   sjhip_neuron_forward_packed <- the same forward ops followed by BitSpikeCompressor.compress,
  *                             spikingjelly/activation_based/memopt/compress.py:332-385
  *   sjhip_neuron_backward  <- torch.ops.sj.cupy_multistep_{if,lif,plif}_backward
@@ -38,7 +40,7 @@
 extern "C" {
 #endif
 
-#define SJHIP_ABI_VERSION 2
+#define SJHIP_ABI_VERSION 3
 
 typedef enum sjhip_status {
   SJHIP_OK = 0,
@@ -53,7 +55,12 @@ typedef enum sjhip_neuron {
   SJHIP_NEURON_IF = 0,  /* h = v + x                                  (functional/neuron.py:310)   */
   SJHIP_NEURON_LIF = 1, /* h = v + (x - (v - vr)) / tau  or  v - (v - vr)/tau + x   (:849-852)     */
   SJHIP_NEURON_PLIF = 2, /* h = v + (x - (v - vr)) * k    or  v - (v - vr)*k + x     (:1290-1295)   */
-  SJHIP_NEURON_QIF = 3  /* h = v + (x + a0 (v - v_rest) (v - v_c)) / tau          (functional/neuron.py:397) */
+  SJHIP_NEURON_QIF = 3, /* h = v + (x + a0 (v - v_rest) (v - v_c)) / tau          (functional/neuron.py:397) */
+  SJHIP_NEURON_ILIF = 4 /* integer-valued LIF (functional/neuron.py:1097-1099): h = v - v/tau + x (the LIF charge
+                           without input decay and with v_reset = None), fires the count
+                           c = rint(clamp(h / v_th, 0, level_max)) instead of a binary spike and resets softly by
+                           c v_th.  spike_seq holds c.  Always a soft reset; the flags DECAY_INPUT and SOFT_RESET
+                           are ignored.  Backward needs sg_id = SJHIP_SG_MULTI_LEVEL. */
 } sjhip_neuron;
 
 /* Storage dtype of every [T,N] / [N] tensor of one call. */
@@ -73,7 +80,9 @@ typedef enum sjhip_surrogate {
   SJHIP_SG_PIECEWISE_EXP = 3,
   SJHIP_SG_SOFT_SIGN = 4,
   SJHIP_SG_SUPER_SPIKE = 5,
-  SJHIP_SG_ERF = 6
+  SJHIP_SG_ERF = 6,
+  SJHIP_SG_MULTI_LEVEL = 7 /* ILIF only (quantize.py:580-598): straight-through window on z = h / v_th,
+                              dc/dz = [grad_min <= z <= grad_max]; sg_alpha is unused */
 } sjhip_surrogate;
 
 /* Bit flags. */
@@ -107,6 +116,9 @@ typedef struct sjhip_neuron_params {
   float v_rest;     /* QIF only */
   float v_c;        /* QIF only */
   float a0;         /* QIF only */
+  float level_max;  /* ILIF only: largest spike count D, an integer >= 1 */
+  float grad_min;   /* ILIF only, backward: lower end of the gradient window on h / v_th */
+  float grad_max;   /* ILIF only, backward: upper end (grad_min <= grad_max) */
 } sjhip_neuron_params;
 
 /* ABI version of the loaded library (== SJHIP_ABI_VERSION it was built with). */
@@ -118,7 +130,7 @@ const char *sjhip_last_error(void);
 /*
  * Forward over T steps for N neurons.
  *   x_seq     [T,N] in            v_init  [N] in ([1] with SJHIP_FLAG_V_INIT_BROADCAST)
- *   spike_seq [T,N] out (0/1 in the storage dtype)
+ *   spike_seq [T,N] out (0/1 in the storage dtype; ILIF: the count 0..level_max)
  *   v_seq     [T,N] out, membrane potential after reset at every step; NULL = do not write
  *   v_last    [N] out, membrane potential after the last step; NULL = do not write
  *             (at least one of v_seq / v_last must be given)

@@ -51,3 +51,28 @@ def bptt(kind: str, h_seq: np.ndarray, s_seq: np.ndarray, sg_prime: Callable[[np
             dh_dk = (x_seq[t] - (v_prev_seq[t] - vr)) if decay_input else (vr - v_prev_seq[t])
             grad_k += float(np.sum(G * dh_dk))
     return grad_x, carry, (grad_k if kind == "plif" else None)
+
+
+def bptt_ilif(h_seq: np.ndarray, grad_spike_seq: np.ndarray, grad_v_seq: Optional[np.ndarray],
+              grad_v_last: Optional[np.ndarray], k: float, v_threshold: float, grad_min: float, grad_max: float,
+              detach_reset: bool):
+    """ILIF (``triton_kernel/neuron_kernel/ilif.py:300-326``; equal to autograd through
+    ``functional/neuron.py:1097-1099`` and ``quantize.py:594-598``): with w_t = [grad_min <= h_t/v_th <= grad_max]
+
+        G_t = Gv_t + (grad_spike[t] - [not detach] v_th Gv_t) w_t / v_th,   Gv_t = G_{t+1} (1 - k) + grad_v_seq[t]
+        grad_x[t] = G_t        grad_v_init = G_0 (1 - k)
+
+    Returns (grad_x [T,N], grad_v_init [N])."""
+    h_seq = np.asarray(h_seq, dtype=np.float64)
+    T = h_seq.shape[0]
+    carry = np.zeros_like(h_seq[0]) if grad_v_last is None else np.asarray(grad_v_last, dtype=np.float64).copy()
+    grad_x = np.zeros_like(h_seq)
+    live = 0.0 if detach_reset else 1.0
+    for t in range(T - 1, -1, -1):
+        z = h_seq[t] / v_threshold
+        w = ((z >= grad_min) & (z <= grad_max)).astype(np.float64)
+        gv = carry if grad_v_seq is None else carry + grad_v_seq[t]
+        G = gv + (grad_spike_seq[t] - live * v_threshold * gv) * w / v_threshold
+        grad_x[t] = G
+        carry = G * (1.0 - k)
+    return grad_x, carry

@@ -83,6 +83,28 @@ class _OtherSG(torch.autograd.Function):
         return _sg_backward_other(ctx.name, grad_output, x, ctx.alpha), None, None
 
 
+class _MultiLevelCount(torch.autograd.Function):
+    # quantize.py:580-598: forward round(clamp(x, 0, D)), backward passes the gradient inside [grad_min, grad_max]
+    @staticmethod
+    def forward(ctx, x, max_spike_count, grad_min, grad_max):
+        ctx.save_for_backward(x)
+        ctx.grad_min = grad_min
+        ctx.grad_max = grad_max
+        return torch.round(torch.clamp(x, 0, max_spike_count))
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (x,) = ctx.saved_tensors
+        mask = (x >= ctx.grad_min) & (x <= ctx.grad_max)
+        return grad_output * mask.to(grad_output.dtype), None, None, None
+
+
+def multi_level_spike_count(max_spike_count: int, grad_window=None) -> Callable[[torch.Tensor], torch.Tensor]:
+    """Firing function of ILIF (surrogate.py:3107-3160, quantize.py:601-616); default window [0, D]."""
+    grad_min, grad_max = (0.0, float(max_spike_count)) if grad_window is None else grad_window
+    return lambda x: _MultiLevelCount.apply(x, int(max_spike_count), grad_min, grad_max)
+
+
 SG_NAMES = ("sigmoid", "atan", "piecewise_quadratic", "piecewise_exp", "soft_sign", "super_spike", "erf")
 SG_IDS = {name: i for i, name in enumerate(SG_NAMES)}  # triton_kernel/surrogate_kernel.py:26-34
 SG_DEFAULT_ALPHA = {"sigmoid": 4.0, "atan": 2.0, "piecewise_quadratic": 1.0, "piecewise_exp": 1.0,
@@ -179,7 +201,12 @@ def charge(kind: str, x, v, tau_or_w, decay_input: bool, v_reset: Optional[float
 
 def step(kind: str, x, v, tau_or_w, decay_input: bool, v_threshold: float, v_reset: Optional[float],
          sg: Callable, detach_reset: bool):
-    """(spike, v_next, h): functional/neuron.py:310-312, 931-933, 1296-1297."""
+    """(spike, v_next, h): functional/neuron.py:310-312, 931-933, 1296-1297; "ilif" :1097-1099 (sg is the
+    multi-level count, fed h / v_threshold; decay_input and v_reset are fixed to False and None)."""
+    if kind == "ilif":
+        h = charge("lif", x, v, tau_or_w, False, None)
+        spike = sg(h / v_threshold)
+        return spike, voltage_reset(h, spike, v_threshold, None, detach_reset), h
     h = charge(kind, x, v, tau_or_w, decay_input, v_reset)
     spike = sg(h - v_threshold)
     return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset), h
@@ -258,8 +285,9 @@ def forward_backward(kind: str, x_seq: torch.Tensor, v_init: torch.Tensor, grad_
                      grad_v_seq: Optional[torch.Tensor] = None, grad_v_last: Optional[torch.Tensor] = None,
                      tau_or_w=None, decay_input: bool = True, v_threshold: float = 1.0,
                      v_reset: Optional[float] = 0.0, sg_name: str = "atan", sg_alpha: float = 2.0,
-                     detach_reset: bool = False, spiking: bool = True):
-    """Forward with the surrogate, then autograd with the given upstream gradients.
+                     detach_reset: bool = False, spiking: bool = True, sg: Optional[Callable] = None):
+    """Forward with the surrogate, then autograd with the given upstream gradients.  ``sg`` overrides the
+    surrogate named by ``sg_name`` (ILIF: ``multi_level_spike_count(D, window)``).
 
     Returns dict(spike_seq, v_seq, h_seq, grad_x, grad_v_init[, grad_p]) where grad_p is the
     gradient w.r.t. ``tau_or_w`` when that is a tensor (PLIF's ``w`` or ``k``).
@@ -270,7 +298,7 @@ def forward_backward(kind: str, x_seq: torch.Tensor, v_init: torch.Tensor, grad_
     if isinstance(p, torch.Tensor):
         p = p.detach().clone().requires_grad_(True)
     s_seq, v_seq, h_seq = multi_step(kind, x, v0, p, decay_input, v_threshold, v_reset,
-                                     surrogate(sg_name, sg_alpha, spiking), detach_reset)
+                                     surrogate(sg_name, sg_alpha, spiking) if sg is None else sg, detach_reset)
     outs, grads = [], []
     if grad_spike_seq is not None:
         outs.append(s_seq)

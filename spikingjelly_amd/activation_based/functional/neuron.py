@@ -32,10 +32,12 @@ __all__ = [
     "lif_step",
     "plif_step",
     "qif_step",
+    "ilif_step",
     "if_multi_step_hip",
     "lif_multi_step_hip",
     "plif_multi_step_hip",
     "qif_multi_step_hip",
+    "ilif_multi_step_hip",
     "if_step_hip",
     "lif_step_hip",
     "plif_step_hip",
@@ -104,6 +106,17 @@ def qif_step(x: torch.Tensor, v: torch.Tensor, tau: float, a0: float, v_rest: fl
     h = v + (x + a0 * (v - v_rest) * (v - v_c)) / tau
     spike = surrogate_function(h - v_threshold)
     return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset)
+
+
+def ilif_step(x: torch.Tensor, v: torch.Tensor, tau: float, v_threshold: float,
+              surrogate_function: SurrogateFunction, detach_reset: bool = False
+              ) -> tuple[torch.Tensor, torch.Tensor]:
+    """One integer-valued LIF step (reference :1030-1099): the LIF charge without input decay and with
+    ``v_reset=None``, a multi-level count fired from ``h / v_threshold``, a soft reset by ``count * v_threshold``.
+    Returns ``(count, v_next)``."""
+    h = lif_charge(x, v, tau, False, None)
+    count = surrogate_function(h / v_threshold)
+    return count, voltage_reset(h, count, v_threshold, None, detach_reset)
 
 
 # ---- hip backend: whole sequence ----------------------------------------------------------------
@@ -233,6 +246,31 @@ def qif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_thres
     else:
         s, v_seq, v_last = K.hip_multistep_qif_inference(x2, v1, v_threshold, vr, soft, float(tau), float(v_rest),
                                                          float(v_c), float(a0), store_v_seq, flags)
+    return _finish(x_seq, s, v_seq, v_last, store_v_seq)
+
+
+def ilif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_threshold: float,
+                        surrogate_function: SurrogateFunction, detach_reset: bool = False,
+                        store_v_seq: bool = False
+                        ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Multi-step integer-valued LIF on the hip backend; ``surrogate_function`` must be a spiking
+    ``MultiLevelSpikeCount`` (its ``max_spike_count`` and gradient window go to the kernel, as the reference's
+    Triton path passes them, ``neuron/ilif.py:343-353``).  ``spike_seq`` holds the counts."""
+    from .. import surrogate
+    from ..hip_kernel import neuron_kernel as K
+
+    if not isinstance(surrogate_function, surrogate.MultiLevelSpikeCount) or not surrogate_function.spiking:
+        raise ValueError("surrogate_function must be a spiking MultiLevelSpikeCount.")
+    levels = int(surrogate_function.max_spike_count)
+    flags = _hip_mode_flags(x_seq)
+    x2, v1 = x_seq.flatten(1), v.flatten()
+    if _needs_grad(x_seq, v):
+        s, v_seq, v_last, _ = K.hip_multistep_ilif_forward(
+            x2, v1, float(tau), float(v_threshold), levels, float(surrogate_function.grad_min),
+            float(surrogate_function.grad_max), detach_reset, store_v_seq, flags, _hip_recompute(x2))
+    else:
+        s, v_seq, v_last = K.hip_multistep_ilif_inference(x2, v1, float(tau), float(v_threshold), levels,
+                                                          store_v_seq, flags)
     return _finish(x_seq, s, v_seq, v_last, store_v_seq)
 
 

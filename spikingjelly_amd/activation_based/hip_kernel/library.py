@@ -14,10 +14,11 @@ from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64
 
 import torch
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # enums of include/sjhip.h
-NEURON_IF, NEURON_LIF, NEURON_PLIF, NEURON_QIF = 0, 1, 2, 3
+NEURON_IF, NEURON_LIF, NEURON_PLIF, NEURON_QIF, NEURON_ILIF = 0, 1, 2, 3, 4
+SG_MULTI_LEVEL = 7  # ILIF's windowed straight-through estimator; ids 0-6 are listed in surrogate_registry
 DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_U8 = 0, 1, 2, 3
 FLAG_DECAY_INPUT = 0x01
 FLAG_SOFT_RESET = 0x02
@@ -65,6 +66,9 @@ class NeuronParams(ctypes.Structure):
         ("v_rest", c_float),
         ("v_c", c_float),
         ("a0", c_float),
+        ("level_max", c_float),
+        ("grad_min", c_float),
+        ("grad_max", c_float),
     ]
 
 

@@ -10,6 +10,7 @@ inference op that writes no ``h_seq``):
     sj::hip_multistep_{if,lif,plif}_backward   -> (grad_x_seq, grad_v_init[, grad_k])
     sj::hip_multistep_{if,lif,plif}_inference_packed -> (spike_bits, v_seq, v_last)
     sj::hip_multistep_qif_{forward,inference,backward}   the quadratic integrate-and-fire neuron, same outputs
+    sj::hip_multistep_ilif_{forward,inference,backward}  the integer-valued LIF: spike_seq holds counts 0..D
 
 The ``_packed`` ops write the spikes bit-packed (uint8, ``T*N/8`` bytes, the layout of
 ``bit_spike_compress`` on the dense spike tensor) straight from the neuron kernel; they need ``N % 8 == 0``.
@@ -38,13 +39,19 @@ __all__ = [
     "hip_multistep_if_inference_packed", "hip_multistep_lif_inference_packed", "hip_multistep_plif_inference_packed",
     "packed_supported",
     "hip_multistep_qif_forward", "hip_multistep_qif_inference", "hip_multistep_qif_backward",
+    "hip_multistep_ilif_forward", "hip_multistep_ilif_inference", "hip_multistep_ilif_backward",
 ]
 
 
+_NO_EXTRA = (0.0, 0.0, 0.0)
+
+
 def _params(tau: float, v_th: float, v_reset: float, sg_alpha: float, sg_id: int, flags: int,
-            qif: tuple[float, float, float] = (0.0, 0.0, 0.0)) -> L.NeuronParams:
-    """``qif`` is (v_rest, v_c, a0) of the quadratic neuron, unused by the others."""
-    return L.NeuronParams(tau, v_th, v_reset, sg_alpha, sg_id, flags, *qif)
+            qif: tuple[float, float, float] = _NO_EXTRA, levels: tuple[float, float, float] = _NO_EXTRA
+            ) -> L.NeuronParams:
+    """``qif`` is (v_rest, v_c, a0) of the quadratic neuron, ``levels`` is (level_max, grad_min, grad_max) of the
+    integer-valued LIF; both unused by the others."""
+    return L.NeuronParams(tau, v_th, v_reset, sg_alpha, sg_id, flags, *qif, *levels)
 
 
 def _flags(soft_reset: bool, detach_reset: bool, decay_input: bool, mode_flags: int) -> int:
@@ -94,7 +101,8 @@ def _k_pointer(k: Optional[torch.Tensor], ref: torch.Tensor) -> tuple[Optional[t
 
 def _run_forward(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: Optional[torch.Tensor],
                  tau: float, v_th: float, v_reset: float, flags: int, store_v_seq: bool,
-                 save_h: bool, qif: tuple[float, float, float] = (0.0, 0.0, 0.0)
+                 save_h: bool, qif: tuple[float, float, float] = _NO_EXTRA,
+                 levels: tuple[float, float, float] = _NO_EXTRA
                  ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     _check_inputs(x_seq, v_init)
     dtype = L.dtype_id(x_seq.dtype)
@@ -106,7 +114,7 @@ def _run_forward(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: Opti
     v_last = x_seq.new_empty((N,))
     h_seq = torch.empty_like(x_seq) if save_h else None
     k_keep, k_ptr = _k_pointer(k, x_seq)
-    params = _params(tau, v_th, v_reset, 0.0, 0, flags | broadcast, qif)
+    params = _params(tau, v_th, v_reset, 0.0, 0, flags | broadcast, qif, levels)
     with torch.cuda.device(x_seq.device):
         rc = L.load().sjhip_neuron_forward(
             neuron, dtype, ctypes.byref(params), T, N,
@@ -167,7 +175,7 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
                   grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor, x_seq: Optional[torch.Tensor],
                   v_init: Optional[torch.Tensor], k: Optional[torch.Tensor], tau: float, v_th: float,
                   v_reset: float, flags: int, sg_id: int, sg_alpha: float, need_grad_v_init: bool = True,
-                  qif: tuple[float, float, float] = (0.0, 0.0, 0.0)
+                  qif: tuple[float, float, float] = _NO_EXTRA, levels: tuple[float, float, float] = _NO_EXTRA
                   ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     recompute = x_seq is not None
     if not recompute and h_seq is None:
@@ -204,7 +212,7 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
             grad_k = torch.empty((), dtype=torch.float32, device=h_seq.device)
             workspace = torch.empty((L.load().sjhip_plif_workspace_floats(dtype, N),), dtype=torch.float32,
                                     device=h_seq.device)
-    params = _params(tau, v_th, v_reset, sg_alpha, sg_id, flags, qif)
+    params = _params(tau, v_th, v_reset, sg_alpha, sg_id, flags, qif, levels)
     with torch.cuda.device(h_seq.device):
         if recompute:
             rc = L.load().sjhip_neuron_backward_recompute(
@@ -621,3 +629,82 @@ def _qif_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_
 
 torch.library.register_autograd("sj::hip_multistep_qif_forward", _qif_autograd_backward,
                                 setup_context=_qif_setup_context)
+
+
+# =================================================================================================
+# ILIF: h = v - v / tau + x,  c = rint(clamp(h / v_th, 0, D)),  v' = h - c v_th
+# (reference triton_kernel/neuron_kernel/ilif.py:556-726; the op there takes decay = 1 - 1/tau, these take tau
+# because the kernels charge in the torch backend's own arithmetic form)
+# =================================================================================================
+@torch.library.custom_op("sj::hip_multistep_ilif_forward", mutates_args=())
+def hip_multistep_ilif_forward(x_seq: torch.Tensor, v_init: torch.Tensor, tau: float, v_th: float,
+                               max_spike_count: int, grad_min: float, grad_max: float, detach_reset: bool,
+                               store_v_seq: bool, mode_flags: int, recompute: bool
+                               ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(True, detach_reset, False, mode_flags)
+    return _forward_outputs(_run_forward(L.NEURON_ILIF, x_seq, v_init, None, tau, v_th, 0.0, flags, store_v_seq,
+                                         not recompute, levels=(float(max_spike_count), grad_min, grad_max)), x_seq)
+
+
+@hip_multistep_ilif_forward.register_fake
+def _(x_seq, v_init, tau, v_th, max_spike_count, grad_min, grad_max, detach_reset, store_v_seq, mode_flags,
+      recompute):
+    return _fake_forward(x_seq, v_init, store_v_seq, True, recompute)
+
+
+@torch.library.custom_op("sj::hip_multistep_ilif_inference", mutates_args=())
+def hip_multistep_ilif_inference(x_seq: torch.Tensor, v_init: torch.Tensor, tau: float, v_th: float,
+                                 max_spike_count: int, store_v_seq: bool, mode_flags: int
+                                 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(True, False, False, mode_flags)
+    return _run_forward(L.NEURON_ILIF, x_seq, v_init, None, tau, v_th, 0.0, flags, store_v_seq, False,
+                        levels=(float(max_spike_count), 0.0, 0.0))[:3]
+
+
+@hip_multistep_ilif_inference.register_fake
+def _(x_seq, v_init, tau, v_th, max_spike_count, store_v_seq, mode_flags):
+    return _fake_forward(x_seq, v_init, store_v_seq, False)
+
+
+@torch.library.custom_op("sj::hip_multistep_ilif_backward", mutates_args=())
+def hip_multistep_ilif_backward(grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
+                                grad_v_last: Optional[torch.Tensor], h_seq: Optional[torch.Tensor],
+                                x_seq: Optional[torch.Tensor], v_init: Optional[torch.Tensor], tau: float,
+                                v_th: float, max_spike_count: int, grad_min: float, grad_max: float,
+                                detach_reset: bool, mode_flags: int, need_grad_v_init: bool = True
+                                ) -> tuple[torch.Tensor, torch.Tensor]:
+    flags = _flags(True, detach_reset, False, mode_flags)
+    gx, gvi, _ = _run_backward(L.NEURON_ILIF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, None,
+                               tau, v_th, 0.0, flags, L.SG_MULTI_LEVEL, 0.0, need_grad_v_init,
+                               levels=(float(max_spike_count), grad_min, grad_max))
+    return gx, gvi
+
+
+@hip_multistep_ilif_backward.register_fake
+def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, tau, v_th, max_spike_count, grad_min,
+      grad_max, detach_reset, mode_flags, need_grad_v_init=True):
+    ref = h_seq if h_seq is not None else x_seq
+    return torch.empty_like(ref), ref.new_empty(ref.shape[1:] if need_grad_v_init else (0,))
+
+
+def _ilif_setup_context(ctx, inputs, output):
+    (x_seq, v_init, tau, v_th, max_spike_count, grad_min, grad_max, detach_reset, store_v_seq, mode_flags,
+     recompute) = inputs
+    _saved_for_backward(ctx, recompute, x_seq, v_init, output[3])
+    ctx.scalars = (tau, v_th, max_spike_count, grad_min, grad_max, detach_reset, mode_flags)
+    ctx.store_v_seq = store_v_seq
+    ctx.set_materialize_grads(False)
+
+
+def _ilif_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_seq):
+    del grad_h_seq
+    h_seq, x_seq, v_init = _split_saved(ctx)
+    need = bool(ctx.needs_input_grad[1])
+    gx, gvi = hip_multistep_ilif_backward(
+        grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, x_seq, v_init,
+        *ctx.scalars, need)
+    return (gx, (gvi if need else None)) + (None,) * 9
+
+
+torch.library.register_autograd("sj::hip_multistep_ilif_forward", _ilif_autograd_backward,
+                                setup_context=_ilif_setup_context)

@@ -1,7 +1,8 @@
 from .base_node import BaseNode
+from .ilif import ILIFNode
 from .integrate_and_fire import IFNode
 from .lif import LIFNode
 from .nonlinear_if import QIFNode
 from .plif import ParametricLIFNode
 
-__all__ = ["BaseNode", "IFNode", "LIFNode", "ParametricLIFNode", "QIFNode"]
+__all__ = ["BaseNode", "IFNode", "LIFNode", "ParametricLIFNode", "QIFNode", "ILIFNode"]

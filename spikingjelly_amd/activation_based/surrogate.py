@@ -6,12 +6,14 @@ for the surrogates the kernel backends know (ids as in
 ``triton_kernel/surrogate_kernel.py:26-34``): ``Sigmoid`` (:769-933), ``ATan`` (:1247-1412),
 ``PiecewiseQuadratic`` (:401-592), ``PiecewiseExp`` (:595-766), ``SoftSign`` (:936-1098),
 ``SuperSpike`` (:1101-1244), ``Erf`` (:1610-1783), plus ``PiecewiseLeakyReLU`` (:1786-2001) as
-a torch-only surrogate the hip backend must reject by name.
+a torch-only surrogate the hip backend must reject by name, and ``MultiLevelSpikeCount`` (:3107-3160),
+the integer firing function of ``ILIFNode``.
 """
 
 from __future__ import annotations
 
 import math
+import numbers
 
 import torch
 import torch.nn as nn
@@ -28,6 +30,7 @@ __all__ = [
     "SuperSpike",
     "Erf",
     "PiecewiseLeakyReLU",
+    "MultiLevelSpikeCount",
 ]
 
 
@@ -329,3 +332,35 @@ class PiecewiseLeakyReLU(SurrogateFunctionBase):
     @staticmethod
     def backward(grad_output, x, w, c):
         return piecewise_leaky_relu_backward(grad_output, x, w, c)
+
+
+# ---- multi-level spike count (ILIF) ---------------------------------------------------------------
+class MultiLevelSpikeCount(SurrogateFunctionBase):
+    """Firing function of the integer-valued LIF: spiking -> ``round(clamp(x, 0, max_spike_count))`` with a
+    rectangular straight-through gradient on ``grad_window`` (default ``[0, max_spike_count]``); not spiking ->
+    ``clamp(x, 0, max_spike_count)``.  ``x`` is the charged voltage divided by the threshold."""
+
+    def __init__(self, max_spike_count: int, grad_window=None, spiking: bool = True):
+        if isinstance(max_spike_count, bool) or not isinstance(max_spike_count, numbers.Integral):
+            raise TypeError("max_spike_count must be an integer.")
+        max_spike_count = int(max_spike_count)
+        if max_spike_count < 1:
+            raise ValueError("max_spike_count must be >= 1.")
+        if grad_window is None:
+            grad_min, grad_max = 0.0, float(max_spike_count)
+        else:
+            grad_min, grad_max = grad_window
+            if grad_min > grad_max:
+                raise ValueError("grad_window must satisfy grad_min <= grad_max.")
+        super().__init__(spiking=spiking, max_spike_count=max_spike_count, grad_min=grad_min, grad_max=grad_max)
+
+    @staticmethod
+    def spiking_function(x: torch.Tensor, max_spike_count: int, grad_min: float, grad_max: float):
+        from . import quantize
+
+        return quantize.multi_level_spike_count(x, max_spike_count, (grad_min, grad_max))
+
+    @staticmethod
+    def primitive_function(x: torch.Tensor, max_spike_count: int, grad_min: float, grad_max: float):
+        del grad_min, grad_max
+        return torch.clamp(x, 0, max_spike_count)

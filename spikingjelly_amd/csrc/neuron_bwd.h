@@ -1,4 +1,4 @@
-// Multi-step backward (BPTT) for IF / LIF / PLIF with the surrogate gradient inlined.
+// Multi-step backward (BPTT) for IF / LIF / PLIF / QIF / ILIF with the surrogate gradient inlined.
 //
 // Same ownership as the forward: one work-item owns V consecutive neurons and walks the rows from
 // t = T-1 down to 0 with the running gradient in registers.  Per step it reads grad_spike[t], h[t]
@@ -20,6 +20,11 @@
 // QIF (h_t = v_{t-1} + k (x_t + a0 (v_{t-1} - v_rest)(v_{t-1} - v_c)), cuda_kernel/neuron_kernel/multi_step/
 // qif.py:138-277) has a state-dependent dh_{t+1}/dv_t = 1 + k a0 ((v_t - v_c) + (v_t - v_rest)); the carry then
 // holds G_{t+1} itself and is scaled when step t has re-derived v_t from h_t; grad_v_init needs v_init.
+// ILIF (triton_kernel/neuron_kernel/ilif.py:300-326, equal to autograd through functional/neuron.py:1097-1099 and
+// quantize.py:594-598): z_t = h_t / v_th, w_t = [grad_min <= z_t <= grad_max], the count's derivative is w_t / v_th and
+// its soft reset by c_t v_th gives dv_t/dh_t = 1 - [!detach] w_t, so
+//   G_t = (carry_{t+1} + grad_v_seq[t]) (1 - [!detach] w_t) + grad_spike[t] w_t / v_th,   grad_x[t] = G_t.
+// With every op rounded to a 16-bit storage dtype the window is tested on z_t rounded to it, as autograd does.
 #pragma once
 
 #include <cmath>
@@ -62,6 +67,11 @@ struct BwdArgs {
   int atomic_reduce;
   int v_init_broadcast;  // v_init holds one element for all neurons
   float q_rest, q_c, q_a0;  // QIF
+  float grad_min, grad_max; // ILIF: gradient window on h / v_th
+  float vth_inv;            // ILIF: 1 / v_threshold when that is an exact power of two, else 0 (as in FwdArgs)
+  float vth_rcp;            // ILIF: fl(1 / v_threshold), the factor of the count's gradient
+  int detach_reset;
+  int round_each;           // 16-bit storage with every op rounded
 };
 
 // Which extra terms the BPTT walk carries.
@@ -236,6 +246,21 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
         if (GVFULL) A::unpack(cur_gv[i], gv);
 #pragma unroll
         for (int j = 0; j < V; ++j) {
+          if constexpr (SG == SJHIP_SG_MULTI_LEVEL) {
+            float z;
+            {
+#pragma clang fp contract(off)
+              // the forward's own quotient, so both agree on which side of the window it lies
+              z = a.vth_inv != 0.0f ? h[j] * a.vth_inv : h[j] / v_th;
+            }
+            if (a.round_each) z = Cvt<S>::round(z);
+            const bool inside = z >= a.grad_min && z <= a.grad_max;
+            const float gvt = GVFULL ? carry[j] + gv[j] : carry[j];
+            const float G = ((inside && !a.detach_reset) ? 0.0f : gvt) + (inside ? gs[j] * a.vth_rcp : 0.0f);
+            gx[j] = G;
+            carry[j] = G * km;
+            continue;
+          }
           const float over = h[j] - v_th;
           const float s = (over >= 0.0f) ? 1.0f : 0.0f;
           float v_t = 0.0f;
@@ -305,6 +330,9 @@ __device__ __forceinline__ float backward_sg_dispatch(const BwdArgs &a, bool act
     case SJHIP_SG_PIECEWISE_EXP: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_PIECEWISE_EXP, HLDS>(a, active, col, k, lds_h, pre);
     case SJHIP_SG_SOFT_SIGN: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SOFT_SIGN, HLDS>(a, active, col, k, lds_h, pre);
     case SJHIP_SG_SUPER_SPIKE: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SUPER_SPIKE, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_MULTI_LEVEL:
+      if constexpr (MODE == BWD_PLAIN) return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_MULTI_LEVEL, HLDS>(a, active, col, k, lds_h, pre);
+      return 0.0f;
     default: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_ERF, HLDS>(a, active, col, k, lds_h, pre);
   }
 }
@@ -345,7 +373,6 @@ inline int build_bwd_args(BwdArgs &a, int neuron, int dtype, const sjhip_neuron_
                           const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
                           const void *h_seq, const void *v_init, const float *k_device, void *grad_x_seq,
                           void *grad_v_init, float *grad_rtau, float *workspace) {
-  (void)dtype;
   a.grad_spike = grad_spike_seq; a.grad_v_seq = grad_v_seq; a.grad_v_last = grad_v_last; a.h = h_seq; a.v_init = v_init;
   a.k_device = nullptr;
   a.grad_x = grad_x_seq; a.grad_v_init = grad_v_init;
@@ -359,6 +386,12 @@ inline int build_bwd_args(BwdArgs &a, int neuron, int dtype, const sjhip_neuron_
   a.atomic_reduce = (p.flags & SJHIP_FLAG_ATOMIC_REDUCE) ? 1 : 0;
   a.v_init_broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) ? 1 : 0;
   const bool detach = (p.flags & SJHIP_FLAG_DETACH_RESET) != 0;
+  a.detach_reset = detach ? 1 : 0;
+  a.round_each = (dtype != SJHIP_F32 && !(p.flags & SJHIP_FLAG_FP32_STATE)) ? 1 : 0;
+  a.grad_min = p.grad_min; a.grad_max = p.grad_max;
+  a.vth_rcp = 1.0f / p.v_threshold;
+  a.vth_inv = (neuron == SJHIP_NEURON_ILIF && exact_reciprocal(p.v_threshold)) ? a.vth_rcp : 0.0f;
+  if (neuron == SJHIP_NEURON_ILIF) { a.soft_reset = 1; a.decay_input = 0; }
   if (a.soft_reset) { a.cB = 0.0f; a.cC = detach ? 0.0f : -p.v_threshold; a.cD = 0.0f; }
   else { a.cB = 1.0f; a.cC = detach ? 0.0f : p.v_reset; a.cD = detach ? 0.0f : 1.0f; }
 

@@ -30,7 +30,7 @@ namespace sjhip {
 template <typename S> __device__ __forceinline__ uint32_t h_bits(float h) { return Cvt<S>::from_float(h); }
 template <typename S> __device__ __forceinline__ uint32_t h_bits(_Float16 h) { return __builtin_bit_cast(uint16_t, h); }
 
-template <typename S, bool ROUND_EACH, int CH, bool SOFT>
+template <typename S, bool ROUND_EACH, int CH, int RS>
 __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, int64_t col) {
   typedef Acc<S, true, SJHIP_BWD_NT != 0> A;
   typedef typename A::elem_t E;
@@ -65,7 +65,7 @@ __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, i
         NUM x[V], h[V], s[V];
         A::unpack(cur[i], x);
 #pragma unroll
-        for (int j = 0; j < V; ++j) neuron_step<R, CH, SOFT>(x[j], v[j], h[j], s[j], tau, a);
+        for (int j = 0; j < V; ++j) neuron_step<R, CH, RS>(x[j], v[j], h[j], s[j], tau, a);
         if constexpr (ROUND_EACH && sizeof(S) == 2) {
           u32x4 w;
           w.x = h_bits<S>(h[0]) | (h_bits<S>(h[1]) << 16); w.y = h_bits<S>(h[2]) | (h_bits<S>(h[3]) << 16);
@@ -85,8 +85,14 @@ __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, i
 
 template <typename S, bool ROUND_EACH, int CH>
 __device__ __forceinline__ void recompute_reset_dispatch(const FwdArgs &a, f32x4 *lds_h, int64_t col) {
-  if (a.soft_reset) recompute_body<S, ROUND_EACH, CH, true>(a, lds_h, col);
-  else recompute_body<S, ROUND_EACH, CH, false>(a, lds_h, col);
+  if constexpr (CH == CH_PLAIN_INPUT_DIV || CH == CH_PLAIN_INPUT_MUL) {
+    if (a.soft_reset == RESET_COUNT) {
+      recompute_body<S, ROUND_EACH, CH, RESET_COUNT>(a, lds_h, col);
+      return;
+    }
+  }
+  if (a.soft_reset) recompute_body<S, ROUND_EACH, CH, RESET_SOFT>(a, lds_h, col);
+  else recompute_body<S, ROUND_EACH, CH, RESET_HARD>(a, lds_h, col);
 }
 
 template <typename S, bool ROUND_EACH, int MODE>

@@ -1,4 +1,4 @@
-// Multi-step forward (charge -> fire -> reset over T steps) for IF / LIF / PLIF.
+// Multi-step forward (charge -> fire -> reset over T steps) for IF / LIF / PLIF / QIF / ILIF.
 //
 // One work-item owns V consecutive neurons (one 128-bit access per row) and walks the T rows in
 // order with the membrane potential in registers.  Rows of x are requested SJHIP_FWD_PF steps ahead
@@ -60,13 +60,19 @@ struct FwdArgs {
   float q_rest_sub; // QIF: v_rest and v_c as subtrahends (rounded like vr_add), a0 as a factor
   float q_c_sub;
   float q_a0_mul;
+  float level_max;  // ILIF: largest spike count
+  float vth_inv;    // ILIF: 1 / v_threshold when that is an exact power of two (h / v_th == h * vth_inv bit for bit), else 0
   int charge;
-  int soft_reset;
+  int soft_reset;        // a Reset value
   int v_init_broadcast;  // v_init holds one element for all neurons
 };
 
+// Fire-and-reset rule.  RESET_COUNT is ILIF (functional/neuron.py:1097-1099 with quantize.py:592): the neuron fires
+// the count c = rint(clamp(h / v_th, 0, level_max)) and resets softly by c * v_th.
+enum Reset { RESET_HARD = 0, RESET_SOFT = 1, RESET_COUNT = 2 };
+
 // One neuron, one step.  R::round() is applied to the result of every arithmetic op.
-template <typename R, int CH, bool SOFT>
+template <typename R, int CH, int RS>
 __device__ __forceinline__ void neuron_step(float x, float &v, float &h, float &s, float tau,
                                             const FwdArgs &a) {
 #pragma clang fp contract(off)
@@ -92,9 +98,18 @@ __device__ __forceinline__ void neuron_step(float x, float &v, float &h, float &
     float g = Cvt<R>::round(v - f);
     h = Cvt<R>::round(g + x);
   }
+  if (RS == RESET_COUNT) {
+    // written with comparisons so that a NaN stays a NaN, as in torch.clamp
+    float z = Cvt<R>::round(a.vth_inv != 0.0f ? h * a.vth_inv : h / a.vth_mul);
+    z = (z < 0.0f) ? 0.0f : ((z > a.level_max) ? a.level_max : z);
+    s = rintf(z);
+    float m = Cvt<R>::round(s * a.vth_mul);
+    v = Cvt<R>::round(h - m);
+    return;
+  }
   float over = Cvt<R>::round(h - a.vth_sub);
   s = (over >= 0.0f) ? 1.0f : 0.0f;
-  if (SOFT) {
+  if (RS == RESET_SOFT) {
     float m = Cvt<R>::round(s * a.vth_mul);
     v = Cvt<R>::round(h - m);
   } else {
@@ -124,7 +139,7 @@ __device__ __forceinline__ _Float16 scalar_product_f16(float scalar, _Float16 t)
   return (_Float16)p;
 }
 
-template <typename R, int CH, bool SOFT>
+template <typename R, int CH, int RS>
 __device__ __forceinline__ void neuron_step(_Float16 x, _Float16 &v, _Float16 &h, _Float16 &s, float tau,
                                             const FwdArgs &a) {
 #pragma clang fp contract(off)
@@ -151,9 +166,18 @@ __device__ __forceinline__ void neuron_step(_Float16 x, _Float16 &v, _Float16 &h
     const H g = v - f;
     h = g + x;
   }
+  if (RS == RESET_COUNT) {
+    H z = a.vth_inv != 0.0f ? scalar_product_f16(a.vth_inv, h) : (H)((float)h / a.vth_mul);
+    const H top = (H)a.level_max;
+    z = (z < (H)0.0f) ? (H)0.0f : ((z > top) ? top : z);
+    s = (H)rintf((float)z);
+    const H m = scalar_product_f16(a.vth_mul, s);  // a count above 1 times v_th need not be exact
+    v = h - m;
+    return;
+  }
   const H over = h - vth_sub;
   s = (over >= (H)0.0f) ? (H)1.0f : (H)0.0f;
-  if (SOFT) {
+  if (RS == RESET_SOFT) {
     const H m = (H)((float)s * a.vth_mul);  // s is 0 or 1: the product is exact, any rounding order agrees
     v = h - m;
   } else {
@@ -190,7 +214,7 @@ __device__ __forceinline__ void store_spike_bits(uint8_t *row, int64_t col, int6
   }
 }
 
-template <typename S, bool VECTOR, bool ROUND_EACH, int CH, bool SOFT, bool PACKED>
+template <typename S, bool VECTOR, bool ROUND_EACH, int CH, int RS, bool PACKED>
 __device__ __forceinline__ void forward_body(const FwdArgs &a) {
   typedef Acc<S, VECTOR, SJHIP_FWD_NT != 0> A;
   typedef typename A::elem_t E;
@@ -232,8 +256,9 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
         NUM x[V], h[V], s[V];
         A::unpack(cur[i], x);
 #pragma unroll
-        for (int j = 0; j < V; ++j) neuron_step<R, CH, SOFT>(x[j], v[j], h[j], s[j], tau, a);
+        for (int j = 0; j < V; ++j) neuron_step<R, CH, RS>(x[j], v[j], h[j], s[j], tau, a);
         if (PACKED) store_spike_bits<V>((uint8_t *)a.spike + t * (N >> 3), col, N, s);
+        else if (RS == RESET_COUNT) A::store(sp + t * N, s);
         else A::store_spikes(sp + t * N, s);
         if (hp) A::store(hp + t * N, h);
         if (vp) A::store(vp + t * N, v);
@@ -245,10 +270,17 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
 
 template <typename S, bool VECTOR, bool ROUND_EACH, int CH, bool PACKED>
 __device__ __forceinline__ void forward_reset_dispatch(const FwdArgs &a) {
+  // counts exist for the charge ILIF uses (no input decay) and never bit-packed
+  if constexpr ((CH == CH_PLAIN_INPUT_DIV || CH == CH_PLAIN_INPUT_MUL) && !PACKED) {
+    if (a.soft_reset == RESET_COUNT) {
+      forward_body<S, VECTOR, ROUND_EACH, CH, RESET_COUNT, PACKED>(a);
+      return;
+    }
+  }
   if (a.soft_reset)
-    forward_body<S, VECTOR, ROUND_EACH, CH, true, PACKED>(a);
+    forward_body<S, VECTOR, ROUND_EACH, CH, RESET_SOFT, PACKED>(a);
   else
-    forward_body<S, VECTOR, ROUND_EACH, CH, false, PACKED>(a);
+    forward_body<S, VECTOR, ROUND_EACH, CH, RESET_HARD, PACKED>(a);
 }
 
 template <typename S, bool VECTOR, bool ROUND_EACH, bool PACKED = false>
@@ -265,20 +297,19 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) forward_kernel(const FwdArgs 
 }
 
 // ---- host side: turn the ABI parameters into kernel arguments ------------------------------------
-inline bool is_power_of_two(float f) {
-  int e;
-  return std::isfinite(f) && f > 0.0f && std::frexp(f, &e) == 0.5f;
-}
-
 inline int build_fwd_args(FwdArgs &a, bool &round_each, int neuron, int dtype, const sjhip_neuron_params &p,
                           int64_t T, int64_t N, const void *x_seq, const void *v_init, const float *k_device,
                           void *spike_seq, void *v_seq, void *v_last, void *h_seq) {
   a.x = x_seq; a.v_init = v_init; a.spike = spike_seq; a.v_seq = v_seq; a.v_last = v_last; a.h = h_seq;
   a.k_device = nullptr;
   a.T = T; a.N = N;
-  a.soft_reset = (p.flags & SJHIP_FLAG_SOFT_RESET) ? 1 : 0;
+  const bool ilif = neuron == SJHIP_NEURON_ILIF;
+  a.soft_reset = ilif ? RESET_COUNT : ((p.flags & SJHIP_FLAG_SOFT_RESET) ? RESET_SOFT : RESET_HARD);
+  a.level_max = p.level_max;
+  a.vth_inv = (ilif && exact_reciprocal(p.v_threshold))
+                  ? 1.0f / p.v_threshold : 0.0f;
   a.v_init_broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) ? 1 : 0;
-  const bool decay_input = (p.flags & SJHIP_FLAG_DECAY_INPUT) != 0;
+  const bool decay_input = !ilif && (p.flags & SJHIP_FLAG_DECAY_INPUT) != 0;
   round_each = dtype != SJHIP_F32 && !(p.flags & SJHIP_FLAG_FP32_STATE);
 
   a.tau = p.tau;
@@ -294,7 +325,7 @@ inline int build_fwd_args(FwdArgs &a, bool &round_each, int neuron, int dtype, c
       // fl(1/tau) from the double quotient, as the reference kernels receive it (multi_step/lif.py:338)
       a.tau = (float)(1.0 / (double)p.tau);
       a.charge = qif ? CH_QIF_MUL : (decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL);
-    } else if (is_power_of_two(p.tau) && p.tau <= 0x1p100f && p.tau >= 0x1p-100f) {
+    } else if (exact_reciprocal(p.tau)) {
       // x / 2^e == x * 2^-e bit for bit (both are exact scalings, subnormal results round identically)
       a.tau = 1.0f / p.tau;
       a.charge = qif ? CH_QIF_MUL : (decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL);
@@ -307,7 +338,7 @@ inline int build_fwd_args(FwdArgs &a, bool &round_each, int neuron, int dtype, c
   // fp32 for mul/div; mirror that when every op is rounded to a 16-bit storage dtype.
   a.vr_mul = p.v_reset;
   a.vth_mul = p.v_threshold;
-  a.vr_add = p.v_reset;
+  a.vr_add = ilif ? 0.0f : p.v_reset;  // ILIF charges with v_reset = None, i.e. the offset 0.0
   a.vth_sub = p.v_threshold;
   a.q_rest_sub = p.v_rest;
   a.q_c_sub = p.v_c;

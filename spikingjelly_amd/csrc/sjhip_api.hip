@@ -4,6 +4,7 @@
 #include "sjhip_common.h"
 
 #include <atomic>
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -116,6 +117,23 @@ namespace {
 
 bool valid_dtype_fp(int dtype) { return dtype == SJHIP_F32 || dtype == SJHIP_F16 || dtype == SJHIP_BF16; }
 
+// ILIF: the count limit must be a positive integer that every storage dtype holds exactly (bf16: up to 256)
+int check_levels(const char *what, int neuron, const sjhip_neuron_params &p, bool backward) {
+  if (neuron != SJHIP_NEURON_ILIF) {
+    if (backward && p.sg_id == SJHIP_SG_MULTI_LEVEL) return fail(SJHIP_ERR_INVALID, "%s: the multi-level surrogate belongs to ILIF", what);
+    return SJHIP_OK;
+  }
+  if (!(p.level_max >= 1.0f) || p.level_max > 256.0f || p.level_max != std::floor(p.level_max))
+    return fail(SJHIP_ERR_INVALID, "%s: ILIF level_max=%g must be an integer in [1, 256]", what, (double)p.level_max);
+  if (!(p.v_threshold > 0.0f) || !std::isfinite(p.v_threshold))
+    return fail(SJHIP_ERR_INVALID, "%s: ILIF v_threshold=%g must be positive", what, (double)p.v_threshold);
+  if (backward) {
+    if (p.sg_id != SJHIP_SG_MULTI_LEVEL) return fail(SJHIP_ERR_INVALID, "%s: ILIF needs the multi-level surrogate, got id %d", what, p.sg_id);
+    if (!(p.grad_min <= p.grad_max)) return fail(SJHIP_ERR_INVALID, "%s: ILIF gradient window [%g, %g]", what, (double)p.grad_min, (double)p.grad_max);
+  }
+  return SJHIP_OK;
+}
+
 int check_shape(const char *what, int64_t T, int64_t N) {
   if (T < 1 || N < 1) return fail(SJHIP_ERR_INVALID, "%s: T=%lld N=%lld must be >= 1", what, (long long)T, (long long)N);
   if (T > (int64_t(1) << 62) / N) return fail(SJHIP_ERR_TOO_LARGE, "%s: T*N overflows", what);
@@ -134,12 +152,14 @@ int sjhip_neuron_forward(int neuron, int dtype, const sjhip_neuron_params *p, in
                          const void *x_seq, const void *v_init, const float *rtau_device, void *spike_seq,
                          void *v_seq, void *v_last, void *h_seq, void *stream) {
   if (!p) return fail(SJHIP_ERR_INVALID, "forward: params is NULL");
-  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_QIF) return fail(SJHIP_ERR_INVALID, "forward: neuron %d", neuron);
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_ILIF) return fail(SJHIP_ERR_INVALID, "forward: neuron %d", neuron);
   if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "forward: dtype %d", dtype);
   int rc = check_shape("forward", T, N);
   if (rc != SJHIP_OK) return rc;
   if (!x_seq || !v_init || !spike_seq) return fail(SJHIP_ERR_INVALID, "forward: NULL tensor");
   if (!v_seq && !v_last) return fail(SJHIP_ERR_INVALID, "forward: neither v_seq nor v_last given");
+  rc = check_levels("forward", neuron, *p, false);
+  if (rc != SJHIP_OK) return rc;
   return launch_forward(neuron, dtype, *p, T, N, x_seq, v_init, rtau_device, spike_seq, v_seq, v_last, h_seq,
                         static_cast<hipStream_t>(stream));
 }
@@ -148,12 +168,13 @@ int sjhip_neuron_forward_packed(int neuron, int dtype, const sjhip_neuron_params
                                 const void *x_seq, const void *v_init, const float *rtau_device, uint8_t *spike_bits,
                                 void *v_seq, void *v_last, void *stream) {
   if (!p) return fail(SJHIP_ERR_INVALID, "forward_packed: params is NULL");
-  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_QIF) return fail(SJHIP_ERR_INVALID, "forward_packed: neuron %d", neuron);
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_ILIF) return fail(SJHIP_ERR_INVALID, "forward_packed: neuron %d", neuron);
   if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "forward_packed: dtype %d", dtype);
   int rc = check_shape("forward_packed", T, N);
   if (rc != SJHIP_OK) return rc;
   if (!x_seq || !v_init || !spike_bits) return fail(SJHIP_ERR_INVALID, "forward_packed: NULL tensor");
   if (!v_seq && !v_last) return fail(SJHIP_ERR_INVALID, "forward_packed: neither v_seq nor v_last given");
+  if (neuron == SJHIP_NEURON_ILIF) return fail(SJHIP_ERR_UNSUPPORTED, "forward_packed: ILIF fires counts, not bits");
   return launch_forward_packed(neuron, dtype, *p, T, N, x_seq, v_init, rtau_device, spike_bits, v_seq, v_last,
                                static_cast<hipStream_t>(stream));
 }
@@ -169,12 +190,14 @@ int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p, i
                           const float *rtau_device, void *grad_x_seq, void *grad_v_init, float *grad_rtau,
                           float *workspace, void *stream) {
   if (!p) return fail(SJHIP_ERR_INVALID, "backward: params is NULL");
-  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_QIF) return fail(SJHIP_ERR_INVALID, "backward: neuron %d", neuron);
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_ILIF) return fail(SJHIP_ERR_INVALID, "backward: neuron %d", neuron);
   if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "backward: dtype %d", dtype);
-  if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_ERF) return fail(SJHIP_ERR_UNSUPPORTED, "backward: surrogate id %d", p->sg_id);
+  if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_MULTI_LEVEL) return fail(SJHIP_ERR_UNSUPPORTED, "backward: surrogate id %d", p->sg_id);
   int rc = check_shape("backward", T, N);
   if (rc != SJHIP_OK) return rc;
   if (!grad_spike_seq || !h_seq || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward: NULL tensor");
+  rc = check_levels("backward", neuron, *p, true);
+  if (rc != SJHIP_OK) return rc;
   if (neuron == SJHIP_NEURON_QIF && grad_v_init && !v_init) return fail(SJHIP_ERR_INVALID, "backward: QIF needs v_init for grad_v_init");
   if (neuron == SJHIP_NEURON_PLIF) {
     if (!v_init || !grad_rtau) return fail(SJHIP_ERR_INVALID, "backward: PLIF needs v_init and grad_rtau");
@@ -201,12 +224,14 @@ int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_pa
                                     void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace,
                                     void *stream) {
   if (!p) return fail(SJHIP_ERR_INVALID, "backward(recompute): params is NULL");
-  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_QIF) return fail(SJHIP_ERR_INVALID, "backward(recompute): neuron %d", neuron);
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_ILIF) return fail(SJHIP_ERR_INVALID, "backward(recompute): neuron %d", neuron);
   if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "backward(recompute): dtype %d", dtype);
-  if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_ERF) return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute): surrogate id %d", p->sg_id);
+  if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_MULTI_LEVEL) return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute): surrogate id %d", p->sg_id);
   int rc = check_shape("backward(recompute)", T, N);
   if (rc != SJHIP_OK) return rc;
   if (!x_seq || !v_init || !grad_spike_seq || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward(recompute): NULL tensor");
+  rc = check_levels("backward(recompute)", neuron, *p, true);
+  if (rc != SJHIP_OK) return rc;
   if (neuron == SJHIP_NEURON_PLIF) {
     if (!grad_rtau) return fail(SJHIP_ERR_INVALID, "backward(recompute): PLIF needs grad_rtau");
     if (!(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace) return fail(SJHIP_ERR_INVALID, "backward(recompute): PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");

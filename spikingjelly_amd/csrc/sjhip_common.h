@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <cmath>
+
 #include <type_traits>
 
 #include "sjhip.h"
@@ -265,6 +267,13 @@ class ProfileScope {
 };
 
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// True when x / f == x * (1 / f) bit for bit for every x: f is a power of two far from the ends of the exponent
+// range, so both are the same exact scaling and a subnormal result rounds identically.
+static inline bool exact_reciprocal(float f) {
+  int e;
+  return std::isfinite(f) && f > 0.0f && std::frexp(f, &e) == 0.5f && f <= 0x1p100f && f >= 0x1p-100f;
+}
 
 // Launchers (one per translation unit).
 int launch_forward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,

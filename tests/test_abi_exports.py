@@ -51,6 +51,29 @@ def test_argument_validation_without_a_device():
     rc = lib.sjhip_neuron_backward(L.NEURON_PLIF, L.DTYPE_F32, ctypes.byref(p), 4, 16, 1, None, None, 1, None, None,
                                    1, 1, None, None, None)
     assert rc == -1 and b"PLIF" in lib.sjhip_last_error()
+    # ILIF: the count limit, the threshold, the surrogate and the window are checked before anything is launched
+    def ilif(levels, sg=L.SG_MULTI_LEVEL, v_th=1.0, lo=0.0, hi=4.0):
+        return L.NeuronParams(2.0, v_th, 0.0, 0.0, sg, 0, 0.0, 0.0, 0.0, levels, lo, hi)
+
+    for bad in (0.0, 2.5, 300.0, float("nan")):
+        rc = lib.sjhip_neuron_forward(L.NEURON_ILIF, L.DTYPE_F32, ctypes.byref(ilif(bad)), 4, 16, 1, 1, None, 1, 1, 1, None, None)
+        assert rc == -1 and b"level_max" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_forward(L.NEURON_ILIF, L.DTYPE_F32, ctypes.byref(ilif(4.0, v_th=0.0)), 4, 16, 1, 1, None, 1, 1, 1, None, None)
+    assert rc == -1 and b"v_threshold" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_forward_packed(L.NEURON_ILIF, L.DTYPE_F16, ctypes.byref(ilif(4.0)), 4, 16, 1, 1, None, 1, None, 1, None)
+    assert rc == -2 and b"counts" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_backward(L.NEURON_ILIF, L.DTYPE_F32, ctypes.byref(ilif(4.0, sg=1)), 4, 16, 1, None, None, 1, None, None,
+                                   1, 1, None, None, None)
+    assert rc == -1 and b"multi-level" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_backward(L.NEURON_ILIF, L.DTYPE_F32, ctypes.byref(ilif(4.0, lo=2.0, hi=1.0)), 4, 16, 1, None, None, 1,
+                                   None, None, 1, 1, None, None, None)
+    assert rc == -1 and b"window" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_backward(L.NEURON_LIF, L.DTYPE_F32, ctypes.byref(ilif(4.0)), 4, 16, 1, None, None, 1, None, None,
+                                   1, 1, None, None, None)
+    assert rc == -1 and b"belongs to ILIF" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_backward_recompute(L.NEURON_ILIF, L.DTYPE_F32, ctypes.byref(ilif(4.0, sg=0)), 4, 16, 1, 1, None,
+                                             1, None, None, 1, 1, None, None, None)
+    assert rc == -1 and b"multi-level" in lib.sjhip_last_error()
     assert lib.sjhip_bit_pack(L.DTYPE_F32, -1, 1, 1, None) == -1
     assert lib.sjhip_bit_pack(L.DTYPE_F32, 0, None, None, None) == 0
     assert lib.sjhip_plif_workspace_floats(L.DTYPE_F32, 1 << 20) >= (1 << 20) // 1024

@@ -39,6 +39,18 @@ def test_if_and_plif_forward_ops(K):
                           test_utils=TESTS)
 
 
+@pytest.mark.parametrize("recompute", [False, True])
+def test_qif_and_ilif_forward_ops(K, recompute):
+    x = seeded_randn((5, 32), 6, 0.5, 0.6).cuda().requires_grad_()
+    v0 = torch.zeros(32, device="cuda", requires_grad=True)
+    torch.library.opcheck(K.hip_multistep_qif_forward,
+                          (x, v0, 1.0, -0.1, False, False, 2.0, 0.0, 0.8, 1.0, 1, 2.0, True, 0, recompute), test_utils=TESTS)
+    torch.library.opcheck(K.hip_multistep_ilif_forward, (x, v0, 1.6, 0.7, 4, 0.0, 4.0, False, True, 0, recompute),
+                          test_utils=TESTS)
+    torch.library.opcheck(K.hip_multistep_ilif_inference, (x.detach(), v0.detach(), 1.6, 0.7, 4, False, 0),
+                          test_utils=("test_schema", "test_faketensor"))
+
+
 def test_inference_and_packed_ops(K):
     x = seeded_randn((4, 48), 3, 0.5, 1.0).cuda()
     v0 = torch.zeros(48, device="cuda")

@@ -366,3 +366,53 @@ def test_to_functional_forward_on_a_neuron_matches_the_module():
     ref = neuron.LIFNode(tau=2.0, step_mode="m")
     assert torch.equal(outputs[0], ref(x_seq)) and torch.equal(states[0], ref.v)
     assert torch.equal(node.v, torch.full((5,), 0.25))
+
+
+# ---- ILIF (reference neuron/ilif.py, test/activation_based/test_ilif_node.py:314-440) -------------------------------
+def test_ilif_node_construction_and_torch_backend_known_answers():
+    with pytest.raises(ValueError, match="MultiLevelSpikeCount"):
+        neuron.ILIFNode(surrogate_function=surrogate.Sigmoid())
+    with pytest.raises(ValueError, match="MultiLevelSpikeCount"):
+        neuron.ILIFNode(surrogate_function=surrogate.MultiLevelSpikeCount(4, spiking=False))
+    with pytest.raises(TypeError):
+        surrogate.MultiLevelSpikeCount(2.5)
+    with pytest.raises(TypeError):
+        surrogate.MultiLevelSpikeCount(True)
+    with pytest.raises(ValueError):
+        surrogate.MultiLevelSpikeCount(0)
+    with pytest.raises(ValueError):
+        surrogate.MultiLevelSpikeCount(4, grad_window=(2.0, 1.0))
+    node = neuron.ILIFNode()
+    assert isinstance(node, neuron.LIFNode) and node.tau == pytest.approx(4.0 / 3.0)
+    assert node.decay_input is False and node.v_reset is None
+    assert node.surrogate_function.max_spike_count == 4
+    assert (node.surrogate_function.grad_min, node.surrogate_function.grad_max) == (0.0, 4.0)
+    assert node.supported_backends == ("torch", "hip")
+    # non-spiking mode of the surrogate is the clamp itself
+    assert torch.equal(surrogate.MultiLevelSpikeCount(4, spiking=False)(torch.tensor([-1.0, 2.5, 9.0])),
+                       torch.tensor([0.0, 2.5, 4.0]))
+
+    node = neuron.ILIFNode(v_threshold=1.0, tau=4.0 / 3.0)
+    x = torch.tensor([[3.2, 0.4, 5.8]])
+    y = node(x)
+    assert torch.equal(y, torch.tensor([[3.0, 0.0, 4.0]]))
+    torch.testing.assert_close(node.v, x - y)
+    node = neuron.ILIFNode(v_threshold=1.0, tau=4.0 / 3.0)
+    node(torch.tensor([[3.2]]))
+    assert torch.equal(node(torch.tensor([[0.0]])), torch.tensor([[0.0]]))
+    torch.testing.assert_close(node.v, torch.tensor([[0.05]]))
+
+    # train and eval fire the same counts; multi-step equals the oracle
+    kw = dict(v_threshold=0.5, tau=4.0 / 3.0, step_mode="m", store_v_seq=True)
+    a, b = neuron.ILIFNode(**kw), neuron.ILIFNode(**kw).eval()
+    x_seq = torch.tensor([[[1.6, -0.2]], [[0.0, 2.2]], [[0.4, 0.0]]])
+    a.v = torch.tensor([[0.2, -0.1]])
+    b.v = torch.tensor([[0.2, -0.1]])
+    ya, yb = a(x_seq), b(x_seq)
+    assert torch.equal(ya, yb) and torch.equal(a.v_seq, b.v_seq) and float(ya.max()) > 1.0
+    es, ev, _ = no.multi_step("ilif", x_seq, torch.tensor([[0.2, -0.1]]), 4.0 / 3.0, False, 0.5, None,
+                              no.multi_level_spike_count(4))
+    assert torch.equal(ya, es) and torch.equal(a.v_seq, ev)
+
+    with pytest.raises(ValueError, match="MultiLevelSpikeCount"):
+        functional.ilif_multi_step_hip(x_seq, torch.zeros(1, 2), 2.0, 1.0, surrogate.ATan())

@@ -439,3 +439,85 @@ def test_qif_autograd_matches_finite_differences_of_the_smooth_network(v_reset):
     vp[2] += eps
     vm[2] -= eps
     assert (loss(x, vp) - loss(x, vm)) / (2 * eps) == pytest.approx(float(ref["grad_v_init"][2]), rel=1e-6, abs=1e-8)
+
+
+# ------------------------------------------------------------------------------------------------
+# ILIF (functional/neuron.py:1097-1099): the reference's own known-answer values, invariants, recurrence
+# ------------------------------------------------------------------------------------------------
+def _ilif(x_seq, v0, tau=4.0 / 3.0, v_th=1.0, levels=4, window=None, detach=False):
+    return no.multi_step("ilif", x_seq, v0, tau, False, v_th, None, no.multi_level_spike_count(levels, window), detach)
+
+
+def test_ilif_oracle_reproduces_the_reference_tests_literal_values():
+    """Inputs and expected outputs of test/activation_based/test_ilif_node.py:336-344, 354-361, 364-370, 400-413."""
+    s, v, _ = _ilif(torch.tensor([[3.2, 0.4, 5.8]]), torch.zeros(3))
+    assert torch.equal(s, torch.tensor([[3.0, 0.0, 4.0]]))
+    torch.testing.assert_close(v[0], torch.tensor([3.2, 0.4, 5.8]) - torch.tensor([3.0, 0.0, 4.0]))
+    s, v, _ = _ilif(torch.tensor([[3.2], [0.0]]), torch.zeros(1))
+    assert torch.equal(s[1], torch.tensor([0.0]))
+    torch.testing.assert_close(v[1], torch.tensor([0.05]))  # the residual 0.2 decayed by 1 - 1/tau = 0.25
+    s, v, _ = _ilif(torch.tensor([[3.2, 5.8]]), torch.zeros(2))
+    assert torch.equal(s, torch.tensor([[3.0, 4.0]]))
+    torch.testing.assert_close(v[0], torch.tensor([0.2, 1.8]))
+    s, _, _ = _ilif(torch.tensor([[3.2], [0.0], [4.8], [0.0]]), torch.zeros(1))
+    assert torch.equal(s.flatten(), torch.tensor([3.0, 0.0, 4.0, 0.0]))
+
+
+def test_ilif_oracle_gradient_window_matches_the_reference_tests_literal_values():
+    """test_ilif_node.py:416-440: y.sum().backward() through one step from rest."""
+    x = torch.tensor([[-0.5, 0.5, 4.5]])
+    r = no.forward_backward("ilif", x, torch.zeros(3), torch.ones(1, 3), None, None, 2.0, False, 1.0, None,
+                            sg=no.multi_level_spike_count(4))
+    assert torch.equal(r["spike_seq"], torch.tensor([[0.0, 0.0, 4.0]]))
+    torch.testing.assert_close(r["grad_x"], torch.tensor([[0.0, 1.0, 0.0]]))
+    x = torch.tensor([[-0.25, 4.25, 4.75]])
+    r = no.forward_backward("ilif", x, torch.zeros(3), torch.ones(1, 3), None, None, 2.0, False, 1.0, None,
+                            sg=no.multi_level_spike_count(4, (-0.5, 4.5)))
+    assert torch.equal(r["spike_seq"], torch.tensor([[0.0, 4.0, 4.0]]))
+    torch.testing.assert_close(r["grad_x"], torch.tensor([[1.0, 1.0, 0.0]]))
+
+
+def test_ilif_invariants_and_reduction_to_a_soft_reset_lif():
+    """Counts are integers in [0, D]; v = h - c v_th; inside the quantiser's range the residual is at most half a
+    threshold; ties round to even.  With D = 1 the count is [h/v_th > 1/2]: a soft-reset LIF without input decay
+    that fires above v_th/2 but is reset by v_th -- checked against that neuron written out step by step."""
+    x = seeded_randn((12, 500), 71, 0.9, 1.5)
+    v0 = seeded_randn((500,), 72, 0.0, 0.3)
+    for v_th, levels in ((1.0, 4), (0.7, 2), (0.25, 7)):
+        s, v, h = _ilif(x, v0, tau=1.6, v_th=v_th, levels=levels)
+        assert bool(((s >= 0) & (s <= levels) & (s == s.round())).all()) and float(s.max()) == levels
+        assert torch.equal(v, h - s * v_th)
+        inside = (h / v_th >= 0) & (h / v_th <= levels)
+        assert float((v[inside].abs() / v_th).max()) <= 0.5 + 1e-6
+    dyadic = torch.tensor([[0.5, 1.5, 2.5, 3.5, 4.5, -0.5]])
+    s, _, _ = _ilif(dyadic, torch.zeros(6))
+    assert torch.equal(s, torch.tensor([[0.0, 2.0, 2.0, 4.0, 4.0, 0.0]]))
+
+    tau, v_th = 1.6, 0.8
+    s1, v1, _ = _ilif(x, v0, tau=tau, v_th=v_th, levels=1)
+    v = v0
+    for t in range(x.shape[0]):
+        h = v - v / tau + x[t]
+        fired = (h / v_th > 0.5).float()
+        v = h - fired * v_th
+        assert torch.equal(s1[t], fired) and torch.equal(v1[t], v)
+
+
+@pytest.mark.parametrize("detach", [False, True])
+@pytest.mark.parametrize("window", [None, (-0.5, 2.25)])
+def test_ilif_recurrence_equals_autograd_float64(detach, window):
+    T, N, tau, v_th, levels = 6, 257, 1.7, 0.6, 3
+    x = seeded_randn((T, N), 81, 0.5, 1.0, torch.float64)
+    v0 = seeded_randn((N,), 82, 0.0, 0.3, torch.float64)
+    gs = seeded_randn((T, N), 83, dtype=torch.float64)
+    gv = seeded_randn((T, N), 84, 0.0, 0.1, torch.float64)
+    gl = seeded_randn((N,), 85, 0.0, 0.1, torch.float64)
+    ref = no.forward_backward("ilif", x, v0, gs, gv, gl, tau, False, v_th, None, detach_reset=detach,
+                              sg=no.multi_level_spike_count(levels, window))
+    lo, hi = (0.0, float(levels)) if window is None else window
+    gx, gvi = bptt_oracle.bptt_ilif(ref["h_seq"].numpy(), gs.numpy(), gv.numpy(), gl.numpy(), 1.0 / tau, v_th, lo, hi,
+                                    detach)
+    np.testing.assert_allclose(gx, ref["grad_x"].numpy(), rtol=1e-11, atol=1e-13)
+    np.testing.assert_allclose(gvi, ref["grad_v_init"].numpy(), rtol=1e-11, atol=1e-13)
+    z = ref["h_seq"] / v_th
+    assert 0.05 < float(((z >= lo) & (z <= hi)).double().mean()) < 0.95  # both sides of the window are exercised
