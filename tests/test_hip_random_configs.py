@@ -2,7 +2,7 @@
 
 Each case draws the neuron, its parameters, the shape (ragged sizes included), the surrogate, the reset mode,
 store_v_seq, the backward path and a second call that continues from the carried state.  fp32: spikes and
-states bit-exact, gradients to 1e-5; fp16 / bf16 in every-op-rounded mode (IF, LIF, QIF): spikes and states
+states bit-exact, gradients to 1e-5; fp16 / bf16 in every-op-rounded mode (IF, LIF, QIF, ILIF): spikes and states
 bit-exact, gradients to a few 16-bit ulps of the largest gradient (the torch node rounds every backward op).
 """
 
@@ -48,9 +48,33 @@ def _draw(seed):
     return kind, cls, kw, dtype, T, shape, recompute, scale, int(rng.integers(0, 1 << 30))
 
 
+def _draw_ilif(seed):
+    """The integer-valued LIF: time constant, threshold (a power of two or not), count limit, gradient window."""
+    rng = np.random.default_rng(10_000 + seed)
+    dtype = rng.choice([torch.float32, torch.float32, torch.float16, torch.bfloat16])
+    T = int(rng.choice([1, 2, 3, 5, 8, 16, 33, 48]))
+    shape = tuple(int(v) for v in rng.choice([1, 2, 3, 4, 7, 8, 12, 32, 37, 64, 100], size=int(rng.integers(1, 4))))
+    levels = int(rng.choice([1, 2, 4, 7]))
+    window = [None, (-0.5, levels + 0.5), (0.25, levels - 0.25)][int(rng.integers(0, 3))]
+    v_th = float(rng.choice([0.5, 1.0, 0.7, 1.25]))
+    kw = dict(tau=float(rng.choice([4.0 / 3.0, 2.0, 1.6, 10.0])), v_threshold=v_th,
+              surrogate_function=surrogate.MultiLevelSpikeCount(levels, grad_window=window),
+              detach_reset=bool(rng.integers(0, 2)), store_v_seq=bool(rng.integers(0, 2)))
+    # drive the neuron over its whole range of counts
+    return "ilif", neuron.ILIFNode, kw, dtype, T, shape, bool(rng.integers(0, 2)), v_th * levels * 0.6, int(rng.integers(0, 1 << 30))
+
+
 @pytest.mark.parametrize("seed", range(300))
 def test_random_configuration(seed):
-    kind, cls, kw, dtype, T, shape, recompute, scale, data_seed = _draw(seed)
+    _run_case(*_draw(seed))
+
+
+@pytest.mark.parametrize("seed", range(100))
+def test_random_ilif_configuration(seed):
+    _run_case(*_draw_ilif(seed))
+
+
+def _run_case(kind, cls, kw, dtype, T, shape, recompute, scale, data_seed):
     g = torch.Generator().manual_seed(data_seed)
     x = (torch.randn((T,) + shape, generator=g) * scale + 0.4).to(dtype)
     x2 = (torch.randn((T,) + shape, generator=g) * scale + 0.4).to(dtype)
