@@ -171,6 +171,37 @@ def other_workload(args) -> int:
                "kernel_ms": d_ms, "algorithmic_bytes": bytes_each, "forward_ms": f_ms, "backward_ms": b_ms})
         return 0
 
+    if args.workload == "stbif":
+        # SpikeZIP's signed ternary neuron (inference): the config-2 shape, the activation fed at the first step
+        shape = (16, 256, 128, 32, 32)
+        T, N = shape[0], 256 * 128 * 32 * 32
+        g = torch.Generator(device=dev).manual_seed(1002)
+        x = torch.zeros(shape, device=dev)
+        x[0] = torch.randn(shape[1:], generator=g, device=dev) * 0.6
+        node = neuron.STBIFNeuron(0.25, level=8, sym=True, step_mode="m").to(dev)
+        node.backend = "hip"
+
+        def step():
+            with torch.no_grad():
+                out = node(x)
+            functional.reset_net(node)
+            return out
+
+        elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
+        f_ms = _kernel_ms(L, L.KC_FORWARD)
+        out = step()
+        want = torch.clamp(torch.floor(x[0].double() / 0.25 + 0.5), -4, 3) * 0.25
+        assert float((out.sum(0).double() - want).abs().max()) <= 0.25  # the quantiser, up to fp32 boundary cases
+        bytes_each = 8 * T * N + 12 * N  # x in, out_seq out; q, acc_q, cur_output out
+        _emit(args, "neuron-steps/sec ST-BIF inference fp32 T=16 N=33.5M, 1 MI355X", "neuron-steps/s",
+              T * N / (elapsed / args.steps), elapsed, "f32",
+              {"workload": "STBIFNeuron(0.25, level=8, sym=True), x [16,256,128,32,32] fp32, x[0] ~N(0,0.6), zeros after, "
+                           "fresh states; includes the is_work read-back", "T": T, "N": N},
+              {"bound": "hbm", "achieved": bytes_each / (f_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+               "frac": bytes_each / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "stbif_forward",
+               "kernel_ms": f_ms, "algorithmic_bytes": bytes_each})
+        return 0
+
     if args.workload == "config4":
         shape = (32, 64, 512, 14, 14)
         T, N = shape[0], 64 * 512 * 14 * 14
@@ -259,7 +290,7 @@ def main() -> int:
     ap.add_argument("--cpu-sample-neurons", type=int, default=1 << 23)
     ap.add_argument("--cpu-repeats", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "qif", "ilif"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "qif", "ilif", "stbif"],
                     help="config2 (default) is the headline metric; the others are secondary measurements")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -216,6 +216,33 @@ int sjhip_recompute_supported(int dtype, int64_t T, int64_t N);
 int sjhip_recompute_preferred(int dtype, int64_t T, int64_t N, uint32_t flags);
 
 /*
+ * ST-BIF, the signed ternary integrate-and-fire neuron of SpikeZIP's QANN-to-SNN conversion; inference only (the
+ * reference implements no backward either).  Stands in for torch.ops.sj.multi_step_stbif / single_step_stbif,
+ * spikingjelly/activation_based/triton_kernel/neuron_kernel/stbif.py:94-137, 258-316, 337-399, and computes the torch
+ * backend's functional.stbif_step (functional/neuron.py:3234-3247) for every step:
+ *     q += x / s;  acc = round(acc);  pos = (q - 1 >= 0) & (acc < pos_max);  neg = (q < 0) & (acc > neg_min);
+ *     cur = pos - neg;  acc += cur;  q = pos ? q - 1 : (neg ? q + 1 : q);  out = cur * s
+ *   x_seq       [T,N] in
+ *   q_init      [N] in, quantisation residual ([1] with SJHIP_FLAG_Q_BROADCAST; a fresh neuron starts from 0.5)
+ *   acc_q_init  [N] in, integer released so far ([1] with SJHIP_FLAG_ACC_BROADCAST; a fresh neuron starts from 0)
+ *   q_threshold, pos_max, neg_min   device addresses of one fp32 each: the quantiser scale s and the bounds of acc;
+ *               they are rounded to `dtype` before use, like `.to(x)` in the reference
+ *   out_seq     [T,N] out: -s, 0 or +s
+ *   q_final, acc_q_final, cur_output   [N] out: the states after the last step and its ternary output
+ *   work_flag   one int32, or NULL: set to 1 when any input or any output of the call is non-zero, never cleared
+ *               (the caller zeroes it; STBIFNeuron.is_work)
+ * flags: SJHIP_FLAG_FP32_STATE (16-bit storage: fp32 arithmetic, stored values rounded -- the Triton kernel;
+ * without it every op is rounded like torch on half tensors) and the two broadcast flags.
+ */
+#define SJHIP_FLAG_Q_BROADCAST 0x200u
+#define SJHIP_FLAG_ACC_BROADCAST 0x400u
+int sjhip_stbif_forward(int dtype, uint32_t flags, int64_t T, int64_t N,
+                        const void *x_seq, const void *q_init, const void *acc_q_init,
+                        const float *q_threshold, const float *pos_max, const float *neg_min,
+                        void *out_seq, void *q_final, void *acc_q_final, void *cur_output,
+                        int32_t *work_flag, void *stream);
+
+/*
  * Spike bit-packing over a flattened tensor, LSB first: byte j bit i = (src[8j+i] != 0).
  *   src  n elements of `dtype` (F32/F16/BF16/U8)     dst  (n+7)/8 bytes; pad bits of the last byte are 0
  */

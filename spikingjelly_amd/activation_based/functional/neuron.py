@@ -33,11 +33,14 @@ __all__ = [
     "plif_step",
     "qif_step",
     "ilif_step",
+    "stbif_step",
     "if_multi_step_hip",
     "lif_multi_step_hip",
     "plif_multi_step_hip",
     "qif_multi_step_hip",
     "ilif_multi_step_hip",
+    "stbif_multi_step_hip",
+    "stbif_single_step_hip",
     "if_step_hip",
     "lif_step_hip",
     "plif_step_hip",
@@ -117,6 +120,25 @@ def ilif_step(x: torch.Tensor, v: torch.Tensor, tau: float, v_threshold: float,
     h = lif_charge(x, v, tau, False, None)
     count = surrogate_function(h / v_threshold)
     return count, voltage_reset(h, count, v_threshold, None, detach_reset)
+
+
+def stbif_step(x: torch.Tensor, q: torch.Tensor, acc_q: torch.Tensor, q_threshold: torch.Tensor,
+               pos_max: torch.Tensor, neg_min: torch.Tensor
+               ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """One step of SpikeZIP's signed ternary neuron (reference :3144-3247), inference semantics: the input in units
+    of the quantiser scale joins the residual ``q``; a unit is released upwards when ``q >= 1`` and the released
+    total ``acc_q`` is below ``pos_max``, downwards when ``q < 0`` and it is above ``neg_min``.
+    Returns ``(out, q_next, acc_q_next, cur_output_next)`` with ``out = cur_output_next * q_threshold``."""
+    q_threshold, pos_max, neg_min = q_threshold.to(x), pos_max.to(x), neg_min.to(x)
+    q_next = q + (x / q_threshold).detach()
+    acc_next = torch.round(acc_q)
+    up = (q_next - 1 >= 0) & (acc_next < pos_max)
+    down = (q_next < 0) & (acc_next > neg_min)
+    cur = up.to(x.dtype) - down.to(x.dtype)
+    acc_next = acc_next + cur
+    q_next = torch.where(up, q_next - 1, q_next)
+    q_next = torch.where(down, q_next + 1, q_next)
+    return cur * q_threshold, q_next, acc_next, cur
 
 
 # ---- hip backend: whole sequence ----------------------------------------------------------------
@@ -272,6 +294,32 @@ def ilif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_thre
         s, v_seq, v_last = K.hip_multistep_ilif_inference(x2, v1, float(tau), float(v_threshold), levels,
                                                           store_v_seq, flags)
     return _finish(x_seq, s, v_seq, v_last, store_v_seq)
+
+
+@torch.no_grad()
+def stbif_multi_step_hip(x_seq: torch.Tensor, q: torch.Tensor, acc_q: torch.Tensor, q_threshold: torch.Tensor,
+                         pos_max: torch.Tensor, neg_min: torch.Tensor
+                         ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Multi-step ST-BIF on the hip backend (inference only, like the reference's kernels).  Returns
+    ``(out_seq, q_next, acc_q_next, cur_output, work_flag)``, the tuple of the reference's
+    ``triton_kernel.neuron_kernel.stbif.multi_step_stbif`` (:337-399); ``work_flag`` is an int32 device scalar,
+    non-zero when any input or output was non-zero."""
+    from ..hip_kernel import stbif_kernel
+
+    flags = _hip_mode_flags(x_seq)
+    state_shape = x_seq.shape[1:]
+    out, q2, acc2, cur, work = stbif_kernel.hip_multistep_stbif(x_seq.flatten(1), q.flatten(), acc_q.flatten(),
+                                                                q_threshold, pos_max, neg_min, flags)
+    return out.reshape(x_seq.shape), q2.reshape(state_shape), acc2.reshape(state_shape), cur.reshape(state_shape), work
+
+
+def stbif_single_step_hip(x: torch.Tensor, q: torch.Tensor, acc_q: torch.Tensor, q_threshold: torch.Tensor,
+                          pos_max: torch.Tensor, neg_min: torch.Tensor
+                          ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """One ST-BIF step on the hip backend; return convention of the reference's ``stbif_single_step_triton``
+    (:3250-3327)."""
+    out, q2, acc2, cur, work = stbif_multi_step_hip(x.unsqueeze(0), q, acc_q, q_threshold, pos_max, neg_min)
+    return out[0], q2, acc2, cur, work
 
 
 # ---- hip backend: one step (step_mode='s') --------------------------------------------------------

@@ -27,6 +27,8 @@ FLAG_FP32_STATE = 0x10
 FLAG_RECIPROCAL_TAU = 0x20
 FLAG_ATOMIC_REDUCE = 0x80
 FLAG_V_INIT_BROADCAST = 0x100
+FLAG_Q_BROADCAST = 0x200
+FLAG_ACC_BROADCAST = 0x400
 
 KC_FORWARD, KC_BACKWARD, KC_PLIF_REDUCE, KC_BIT_PACK, KC_BIT_UNPACK, KC_SSA_FORWARD, KC_SSA_BACKWARD = range(7)
 
@@ -43,6 +45,7 @@ EXPORTED_SYMBOLS = (
     "sjhip_ssa_supported",
     "sjhip_ssa_forward",
     "sjhip_ssa_backward",
+    "sjhip_stbif_forward",
     "sjhip_bit_pack",
     "sjhip_bit_unpack",
     "sjhip_set_tuning",
@@ -133,6 +136,12 @@ def load() -> ctypes.CDLL:
         lib.sjhip_ssa_backward.restype = c_int
         lib.sjhip_ssa_backward.argtypes = [c_int, c_int64, c_int, c_int, c_int64, c_float, c_void_p, c_void_p, c_void_p,
                                            c_void_p]
+        lib.sjhip_stbif_forward.restype = c_int
+        lib.sjhip_stbif_forward.argtypes = [
+            c_int, c_uint32, c_int64, c_int64,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        ]
         lib.sjhip_bit_pack.restype = c_int
         lib.sjhip_bit_pack.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p]
         lib.sjhip_bit_unpack.restype = c_int

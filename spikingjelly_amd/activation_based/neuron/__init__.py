@@ -4,5 +4,6 @@ from .integrate_and_fire import IFNode
 from .lif import LIFNode
 from .nonlinear_if import QIFNode
 from .plif import ParametricLIFNode
+from .spikezip import STBIFNeuron
 
-__all__ = ["BaseNode", "IFNode", "LIFNode", "ParametricLIFNode", "QIFNode", "ILIFNode"]
+__all__ = ["BaseNode", "IFNode", "LIFNode", "ParametricLIFNode", "QIFNode", "ILIFNode", "STBIFNeuron"]

@@ -241,6 +241,22 @@ int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_pa
                                    static_cast<hipStream_t>(stream));
 }
 
+int sjhip_stbif_forward(int dtype, uint32_t flags, int64_t T, int64_t N, const void *x_seq, const void *q_init,
+                        const void *acc_q_init, const float *q_threshold, const float *pos_max, const float *neg_min,
+                        void *out_seq, void *q_final, void *acc_q_final, void *cur_output, int32_t *work_flag,
+                        void *stream) {
+  if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "stbif_forward: dtype %d", dtype);
+  if (flags & ~(SJHIP_FLAG_FP32_STATE | SJHIP_FLAG_Q_BROADCAST | SJHIP_FLAG_ACC_BROADCAST))
+    return fail(SJHIP_ERR_INVALID, "stbif_forward: flags 0x%x", flags);
+  int rc = check_shape("stbif_forward", T, N);
+  if (rc != SJHIP_OK) return rc;
+  if (!x_seq || !q_init || !acc_q_init || !out_seq || !q_final || !acc_q_final || !cur_output)
+    return fail(SJHIP_ERR_INVALID, "stbif_forward: NULL tensor");
+  if (!q_threshold || !pos_max || !neg_min) return fail(SJHIP_ERR_INVALID, "stbif_forward: NULL scalar address");
+  return launch_stbif_forward(dtype, flags, T, N, x_seq, q_init, acc_q_init, q_threshold, pos_max, neg_min, out_seq,
+                              q_final, acc_q_final, cur_output, work_flag, static_cast<hipStream_t>(stream));
+}
+
 int sjhip_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, void *stream) {
   if (n < 0) return fail(SJHIP_ERR_INVALID, "bit_pack: n=%lld", (long long)n);
   if (n == 0) return SJHIP_OK;

@@ -74,6 +74,16 @@ def test_argument_validation_without_a_device():
     rc = lib.sjhip_neuron_backward_recompute(L.NEURON_ILIF, L.DTYPE_F32, ctypes.byref(ilif(4.0, sg=0)), 4, 16, 1, 1, None,
                                              1, None, None, 1, 1, None, None, None)
     assert rc == -1 and b"multi-level" in lib.sjhip_last_error()
+    rc = lib.sjhip_stbif_forward(L.DTYPE_U8, 0, 4, 16, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, None, None)
+    assert rc == -1 and b"dtype" in lib.sjhip_last_error()
+    rc = lib.sjhip_stbif_forward(L.DTYPE_F32, 0x01, 4, 16, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, None, None)
+    assert rc == -1 and b"flags" in lib.sjhip_last_error()
+    rc = lib.sjhip_stbif_forward(L.DTYPE_F32, 0, 4, 16, 1, 1, 1, 1, None, 1, 1, 1, 1, 1, None, None)
+    assert rc == -1 and b"scalar" in lib.sjhip_last_error()
+    rc = lib.sjhip_stbif_forward(L.DTYPE_F32, 0, 4, 16, 1, 1, 1, 1, 1, 1, 1, None, 1, 1, None, None)
+    assert rc == -1 and b"NULL tensor" in lib.sjhip_last_error()
+    rc = lib.sjhip_stbif_forward(L.DTYPE_F32, 0, 0, 16, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, None, None)
+    assert rc == -1 and b"T=0" in lib.sjhip_last_error()
     assert lib.sjhip_bit_pack(L.DTYPE_F32, -1, 1, 1, None) == -1
     assert lib.sjhip_bit_pack(L.DTYPE_F32, 0, None, None, None) == 0
     assert lib.sjhip_plif_workspace_floats(L.DTYPE_F32, 1 << 20) >= (1 << 20) // 1024

@@ -62,6 +62,15 @@ def test_inference_and_packed_ops(K):
                           test_utils=("test_schema", "test_faketensor"))
 
 
+def test_stbif_op():
+    from spikingjelly_amd.activation_based.hip_kernel.stbif_kernel import hip_multistep_stbif
+
+    x = seeded_randn((5, 40), 7, 0.0, 0.5).cuda()
+    q, acc = torch.full((40,), 0.5, device="cuda"), torch.zeros(40, device="cuda")
+    th = [torch.tensor(v, device="cuda") for v in (0.25, 3.0, -4.0)]
+    torch.library.opcheck(hip_multistep_stbif, (x, q, acc, *th, 0), test_utils=("test_schema", "test_faketensor"))
+
+
 def test_ssa_op():
     from spikingjelly_amd.activation_based.hip_kernel.attention_kernel import hip_ssa_forward
 

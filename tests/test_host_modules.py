@@ -416,3 +416,48 @@ def test_ilif_node_construction_and_torch_backend_known_answers():
 
     with pytest.raises(ValueError, match="MultiLevelSpikeCount"):
         functional.ilif_multi_step_hip(x_seq, torch.zeros(1, 2), 2.0, 1.0, surrogate.ATan())
+
+
+# ---- ST-BIF (reference neuron/spikezip.py, test_ann2snn_transformer.py:792-896, test_functional_neuron.py:690-705) ---
+def test_stbif_neuron_construction_and_torch_backend():
+    for bad in (1, 0, True):
+        with pytest.raises(ValueError, match="level"):
+            neuron.STBIFNeuron(0.25, level=bad, sym=True)
+    node = neuron.STBIFNeuron(0.25, level=8, sym=True)
+    assert node.supported_backends == ("torch", "hip")
+    assert (float(node.pos_max), float(node.neg_min)) == (3.0, -4.0)
+    assert (float(neuron.STBIFNeuron(0.5, level=8).pos_max), float(neuron.STBIFNeuron(0.5, level=8).neg_min)) == (7.0, 0.0)
+    assert "q_threshold" in node.state_dict() and node.q is None and node.is_work is False
+    with pytest.raises(RuntimeError, match="accumulated"):
+        node.accumulated
+
+    class Quantizer(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.s = torch.nn.Parameter(torch.tensor(0.25))
+            self.sym = True
+            self.pos_max, self.neg_min = torch.tensor(3), torch.tensor(-4)
+
+    from_q = neuron.STBIFNeuron.from_quantizer(Quantizer())
+    assert from_q.level == 8 and float(from_q.q_threshold) == 0.25 and not from_q.q_threshold.requires_grad
+
+    x = torch.tensor([[-0.75, -0.2, 0.3, 0.9]])
+    total = sum(node(x if t == 0 else torch.zeros_like(x)) for t in range(16))
+    assert total.tolist() == [[-0.75, -0.25, 0.25, 0.75]]
+    assert torch.equal(node.accumulated, total)
+
+    # multi-step equals the loop of single steps; is_work follows inputs and outputs
+    node.reset()
+    assert node.q is None and node.is_work is False
+    x_seq = torch.cat([x[None], torch.zeros(15, 1, 4)])
+    functional.set_step_mode(node, "m")
+    y_seq = node(x_seq)
+    other = neuron.STBIFNeuron(0.25, level=8, sym=True)
+    assert torch.equal(y_seq, torch.stack([other(v) for v in x_seq])) and node.is_work
+    node.reset()
+    node(torch.zeros(2, 2, 3))
+    assert not node.is_work
+    node(torch.stack([torch.zeros(2, 3), torch.full((2, 3), 0.25)]))
+    assert node.is_work
+    # a changed shape starts from fresh states
+    assert node(torch.zeros(2, 5)).shape == (2, 5) and float(node.q.mean()) == 0.5

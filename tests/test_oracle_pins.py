@@ -521,3 +521,67 @@ def test_ilif_recurrence_equals_autograd_float64(detach, window):
     np.testing.assert_allclose(gvi, ref["grad_v_init"].numpy(), rtol=1e-11, atol=1e-13)
     z = ref["h_seq"] / v_th
     assert 0.05 < float(((z >= lo) & (z <= hi)).double().mean()) < 0.95  # both sides of the window are exercised
+
+
+# ------------------------------------------------------------------------------------------------
+# ST-BIF (functional/neuron.py:3234-3247): the quantiser it must reproduce, literal cases of the reference's tests
+# ------------------------------------------------------------------------------------------------
+def _stbif_tensors(scale, pos_max, neg_min):
+    return torch.tensor(float(scale)), torch.tensor(float(pos_max)), torch.tensor(float(neg_min))
+
+
+@pytest.mark.parametrize("scale,pos_max,neg_min", [(0.25, 3, -4), (0.125, 7, 0), (0.3, 1, -2)])
+def test_stbif_released_total_equals_the_quantiser(scale, pos_max, neg_min):
+    """Defining property (reference test_ann2snn_transformer.py:792-803 with the quantiser of :570-573): feed x once,
+    then zeros; the outputs sum to  s * clamp(floor(x/s + 1/2), neg_min, pos_max)  once enough steps have run.
+    Independent of the step formula: it is the closed form the neuron exists to reproduce."""
+    from oracle import stbif_oracle
+
+    x = seeded_randn((1, 400), 91, 0.0, 1.0, torch.float64)
+    x[0, :4] = torch.tensor([-0.75, -0.2, 0.3, 0.9], dtype=torch.float64)
+    T = 16
+    x_seq = torch.cat([x, torch.zeros((T - 1, 400), dtype=torch.float64)])
+    th = [t.double() for t in _stbif_tensors(scale, pos_max, neg_min)]
+    scale = float(th[0])  # the fp32 value the neuron holds
+    out, q, acc, cur, work = stbif_oracle.multi_step(x_seq, torch.full((400,), 0.5, dtype=torch.float64),
+                                                     torch.zeros(400, dtype=torch.float64), *th)
+    expected = torch.clamp(torch.floor(x[0] / scale + 0.5), neg_min, pos_max) * scale
+    torch.testing.assert_close(out.sum(0), expected, rtol=0, atol=1e-12)
+    assert set(torch.unique(out / scale).round().tolist()) <= {-1.0, 0.0, 1.0} and work
+    assert torch.equal(acc, (expected / scale).round())
+    if scale == 0.25 and pos_max == 3:  # the reference test's literal case: [-0.75, -0.2, 0.3, 0.9] -> [-0.75, -0.25, 0.25, 0.75]
+        assert out.sum(0)[:4].tolist() == [-0.75, -0.25, 0.25, 0.75]
+
+
+def test_stbif_rounds_the_accumulator_half_to_even_and_reports_work():
+    """Literal case of the reference's test_ann2snn_transformer.py:975-1010 (x = 0, q = 1/2, half-integer acc_q) and
+    of test_functional_neuron.py:690-705 (is_work)."""
+    from oracle import stbif_oracle
+
+    x = torch.zeros(6)
+    acc = torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, -2.5])
+    out, q, acc2, cur = stbif_oracle.step(x, torch.full_like(x, 0.5), acc, *_stbif_tensors(0.1, 10, -10))
+    assert torch.equal(acc2, torch.tensor([0.0, 2.0, 2.0, -0.0, -2.0, -2.0]))
+    assert torch.equal(out, torch.zeros(6)) and torch.equal(q, torch.full_like(x, 0.5)) and torch.equal(cur, torch.zeros(6))
+    th = _stbif_tensors(0.25, 3, -4)
+    z = torch.zeros(2, 2, 3)
+    assert stbif_oracle.multi_step(z, torch.full((2, 3), 0.5), torch.zeros(2, 3), *th)[4] is False
+    z[1] = 0.25
+    assert stbif_oracle.multi_step(z, torch.full((2, 3), 0.5), torch.zeros(2, 3), *th)[4] is True
+
+
+def test_stbif_bounds_block_release_and_both_arithmetic_forms_agree_in_fp32():
+    """A saturated accumulator stops releasing in that direction while the residual keeps integrating; the Triton
+    kernel's form (q >= 1, q - pos + neg) equals the torch form in fp32."""
+    from oracle import stbif_oracle
+
+    th = _stbif_tensors(0.5, 2, -1)
+    x_seq = torch.full((8, 1), 1.0)  # two units per step
+    out, q, acc, cur, _ = stbif_oracle.multi_step(x_seq, torch.full((1,), 0.5), torch.zeros(1), *th)
+    assert out.flatten().tolist() == [0.5, 0.5, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0] and float(acc) == 2.0
+    assert float(q) == 0.5 + 16 - 2
+    x = seeded_randn((20, 300), 92, 0.0, 0.6)
+    a = stbif_oracle.multi_step(x, torch.full((300,), 0.5), torch.zeros(300), *_stbif_tensors(0.25, 3, -4))
+    b = stbif_oracle.multi_step_fp32_state(x, torch.full((300,), 0.5), torch.zeros(300), *_stbif_tensors(0.25, 3, -4))
+    for got, want in zip(b, a[:4]):
+        assert torch.equal(got, want)
