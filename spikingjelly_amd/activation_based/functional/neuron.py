@@ -159,13 +159,36 @@ def _hip_mode_flags(x_seq: torch.Tensor) -> int:
     return flags
 
 
+@torch.compiler.assume_constant_result
+def _replay_limits(dtype: torch.dtype, flags: int) -> tuple[int, int]:
+    """``(vector width, longest sequence)`` of the library's replay policy for one dtype and mode: replay is preferred
+    for ``[T, N]`` when ``N`` is a multiple of the width and ``T`` does not exceed the length.  The policy itself lives
+    in the library (``sjhip_recompute_preferred``, monotone in ``T``); it is probed once per ``(dtype, flags)`` and the
+    answer is a constant of any traced graph, so the shape test below is plain integer arithmetic a tracing compiler
+    can follow, also with symbolic shapes."""
+    key = (dtype, flags & _REPLAY_POLICY_FLAGS)
+    if key not in _replay_limits_cache:
+        from ..hip_kernel import library as L
+
+        width = next((n for n in (1, 2, 4, 8, 16) if L.recompute_preferred(dtype, 1, n, key[1])), 0)
+        steps = 0
+        while width and steps < 4096 and L.recompute_preferred(dtype, steps + 1, width, key[1]):
+            steps += 1
+        _replay_limits_cache[key] = (width, steps)
+    return _replay_limits_cache[key]
+
+
+_replay_limits_cache: dict = {}
+_REPLAY_POLICY_FLAGS = 0x10  # FLAG_FP32_STATE: the only flag the policy depends on
+
+
 def _hip_recompute(x2: torch.Tensor) -> bool:
     """Replay the forward inside the backward kernel instead of saving h_seq, when the shape allows and the
     sequence is short enough for the replay to pay (its LDS footprint grows with T)."""
-    from ..hip_kernel import library as L
-
-    return bool(configure.hip_backward_recompute) and L.recompute_preferred(x2.dtype, x2.shape[0], x2.shape[1],
-                                                                            _hip_mode_flags(x2))
+    if not configure.hip_backward_recompute:
+        return False
+    width, steps = _replay_limits(x2.dtype, _hip_mode_flags(x2))
+    return width > 0 and x2.shape[1] % width == 0 and x2.shape[0] <= steps
 
 
 def _needs_grad(*tensors: torch.Tensor) -> bool:

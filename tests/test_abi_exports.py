@@ -117,3 +117,19 @@ def test_replay_policy_follows_the_lds_footprint():
     for flags in (0, L.FLAG_FP32_STATE):
         assert lib.sjhip_recompute_preferred(L.DTYPE_BF16, 39, N, flags) == 1
         assert lib.sjhip_recompute_preferred(L.DTYPE_BF16, 40, N, flags) == 0
+
+
+def test_traceable_replay_policy_mirrors_the_library():
+    """The functionals decide about the replay backward with integer arithmetic on limits probed from the library
+    (a tracing compiler cannot follow a ctypes call): both must agree for every shape."""
+    import torch
+
+    from spikingjelly_amd.activation_based.functional import neuron as F
+
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        for flags in (0, L.FLAG_FP32_STATE, L.FLAG_FP32_STATE | L.FLAG_RECIPROCAL_TAU):
+            width, steps = F._replay_limits(dtype, flags)
+            assert width in (4, 8) and steps == 39
+            for T in (1, 8, 39, 40, 64, 159, 160, 1000):
+                for N in (1, 4, 8, 12, 37, 64, 100, 4096):
+                    assert (N % width == 0 and T <= steps) == L.recompute_preferred(dtype, T, N, flags), (dtype, flags, T, N)

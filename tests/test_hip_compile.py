@@ -1,0 +1,109 @@
+"""``torch.compile(..., fullgraph=True)`` over modules with ``backend='hip'``: the kernels are opaque operators with
+fake (meta) implementations, and everything the host side does around them must be traceable without a graph break,
+as the reference requires of its kernel backends (test/activation_based/test_compile_compat.py:125-170, 496-525).
+The ``aot_eager`` backend traces forward and backward through AOT autograd and then runs the graph with the eager
+kernels, so results must equal the uncompiled module exactly."""
+
+import pytest
+import torch
+
+from spikingjelly_amd.activation_based import layer, neuron, surrogate
+
+from helpers import seeded_randn
+
+pytestmark = pytest.mark.gpu
+
+NODES = {
+    "if": lambda **kw: neuron.IFNode(surrogate_function=surrogate.ATan(), **kw),
+    "lif": lambda **kw: neuron.LIFNode(tau=2.0, surrogate_function=surrogate.ATan(), **kw),
+    "lif_soft_div": lambda **kw: neuron.LIFNode(tau=3.0, v_reset=None, decay_input=False,
+                                                surrogate_function=surrogate.Sigmoid(), **kw),
+    "plif": lambda **kw: neuron.ParametricLIFNode(surrogate_function=surrogate.ATan(), **kw),
+    "qif": lambda **kw: neuron.QIFNode(tau=2.0, surrogate_function=surrogate.ATan(), **kw),
+    "ilif": lambda **kw: neuron.ILIFNode(**kw),
+}
+
+
+@pytest.fixture(autouse=True)
+def fresh_tracer():
+    # every node class shares the code object of MemoryModule.forward, and the recompile limit is per code object
+    torch._dynamo.reset()
+    yield
+    torch._dynamo.reset()
+
+
+def _compiled(module):
+    return torch.compile(module, fullgraph=True, backend="aot_eager")
+
+
+@pytest.mark.parametrize("kind", sorted(NODES))
+@pytest.mark.parametrize("store_v_seq", [False, True])
+def test_multi_step_node_compiles_without_graph_breaks(kind, store_v_seq):
+    scale = {"qif": 0.4, "ilif": 2.0}.get(kind, 0.8)
+    x = (seeded_randn((6, 4, 32), 11, 0.3, scale)).cuda()
+    eager = NODES[kind](step_mode="m", backend="hip", store_v_seq=store_v_seq).cuda()
+    traced = NODES[kind](step_mode="m", backend="hip", store_v_seq=store_v_seq).cuda()
+    fn = _compiled(traced)
+    xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
+    ya, yb = eager(xa), fn(xb)
+    assert torch.equal(ya, yb) and float(ya.detach().abs().sum()) > 0
+    assert torch.equal(eager.v, traced.v)
+    if store_v_seq:
+        assert torch.equal(eager.v_seq, traced.v_seq)
+    (ya.sum() + 0.5 * eager.v.sum()).backward()
+    (yb.sum() + 0.5 * traced.v.sum()).backward()
+    assert torch.equal(xa.grad, xb.grad)
+    if kind == "plif":
+        torch.testing.assert_close(traced.w.grad, eager.w.grad)
+    # the state is an ordinary tensor now: the second call re-traces once and continues from it
+    assert torch.equal(eager(x), fn(x)) and torch.equal(eager.v, traced.v)
+
+
+def test_inference_single_step_and_changing_shapes():
+    """Eval mode, step_mode='s', and a sequence of different shapes (the tracer then treats sizes as symbols: the
+    host-side policy around the operators must stay traceable)."""
+    node = neuron.LIFNode(tau=2.0, surrogate_function=surrogate.ATan(), step_mode="m", backend="hip").cuda().eval()
+    fn = _compiled(node)
+    ref = neuron.LIFNode(tau=2.0, surrogate_function=surrogate.ATan(), step_mode="m", backend="hip").cuda().eval()
+    for shape in ((6, 4, 32), (3, 8, 16), (5, 2, 20), (40, 2, 8), (41, 2, 8)):
+        x = seeded_randn(shape, sum(shape), 0.3, 0.8).cuda()
+        node.reset()
+        ref.reset()
+        with torch.no_grad():
+            assert torch.equal(fn(x), ref(x))
+    train = neuron.LIFNode(tau=2.0, surrogate_function=surrogate.ATan(), step_mode="m", backend="hip").cuda()
+    fn = _compiled(train)
+    for shape in ((6, 4, 32), (3, 8, 16), (5, 2, 20), (39, 2, 8), (40, 2, 8)):  # 39 / 40: either side of the replay limit
+        x = seeded_randn(shape, sum(shape), 0.3, 0.8).cuda().requires_grad_()
+        train.reset()
+        fn(x).sum().backward()
+        assert bool(torch.isfinite(x.grad).all()) and float(x.grad.abs().sum()) > 0
+    single = neuron.LIFNode(tau=2.0, surrogate_function=surrogate.ATan(), step_mode="s", backend="hip").cuda()
+    fn = _compiled(single)
+    ref = neuron.LIFNode(tau=2.0, surrogate_function=surrogate.ATan(), step_mode="s", backend="hip").cuda()
+    x = seeded_randn((4, 64), 3, 0.6, 0.8).cuda()
+    for _ in range(3):
+        assert torch.equal(fn(x), ref(x))
+
+
+def test_spiking_self_attention_block_compiles():
+    def make(backend):
+        torch.manual_seed(1)
+        block = layer.SpikingSelfAttention(128, 4, backend=backend).cuda()
+        with torch.no_grad():  # freshly initialised, the block hardly fires: raise the batch-norm gains
+            block.qkv_conv_bn[1].weight.fill_(2.0)
+            block.proj_conv_bn[1].weight.fill_(3.0)
+        return block
+
+    x = seeded_randn((4, 8, 128, 96), 5).cuda()  # large enough for the attention LIF to receive coincident spikes
+    eager, traced, torch_traced = make("hip"), make("hip"), make("torch")
+    fn, fn_torch = _compiled(traced), _compiled(torch_traced)
+    xa, xb, xc = (x.clone().requires_grad_() for _ in range(3))
+    ya, yb, yc = eager(xa), fn(xb), fn_torch(xc)
+    assert float(ya.detach().mean()) > 0.05
+    assert torch.equal(ya, yb) and torch.equal(yb, yc)
+    ya.sum().backward()
+    yb.sum().backward()
+    yc.sum().backward()
+    torch.testing.assert_close(xb.grad, xa.grad, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(xb.grad, xc.grad, rtol=1e-3, atol=1e-4)
