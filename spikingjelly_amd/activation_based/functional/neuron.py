@@ -207,6 +207,7 @@ def if_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, v_threshold: float, 
                       store_v_seq: bool = False
                       ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     """Multi-step IF on the hip backend.  ``x_seq`` is ``[T, *]``, ``v`` has the shape of ``x_seq[0]``."""
+    from ..hip_kernel import library as L
     from ..hip_kernel import neuron_kernel as K
     from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
 
@@ -214,8 +215,13 @@ def if_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, v_threshold: float, 
     vr = 0.0 if soft else float(v_reset)
     flags = _hip_mode_flags(x_seq)
     x2, v1 = x_seq.flatten(1), v.flatten()
-    if _needs_grad(x_seq, v):
-        sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function)
+    need_grad = _needs_grad(x_seq, v)
+    sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function) if need_grad else (0, 0.0)
+    if not torch.compiler.is_compiling():
+        s, v_seq, v_last = K.eager_multistep(L.NEURON_IF, x2, v1, None, 0.0, v_threshold, vr,
+                                             K._flags(soft, detach_reset, False, flags), sg_id, sg_alpha, store_v_seq,
+                                             need_grad and _hip_recompute(x2), need_grad)
+    elif need_grad:
         s, v_seq, v_last, _ = K.hip_multistep_if_forward(x2, v1, v_threshold, vr, soft, detach_reset, sg_id,
                                                          sg_alpha, store_v_seq, flags, _hip_recompute(x2))
     else:
@@ -228,6 +234,7 @@ def lif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, decay_i
                        detach_reset: bool = False, store_v_seq: bool = False
                        ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     """Multi-step LIF on the hip backend."""
+    from ..hip_kernel import library as L
     from ..hip_kernel import neuron_kernel as K
     from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
 
@@ -235,8 +242,13 @@ def lif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, decay_i
     vr = 0.0 if soft else float(v_reset)
     flags = _hip_mode_flags(x_seq)
     x2, v1 = x_seq.flatten(1), v.flatten()
-    if _needs_grad(x_seq, v):
-        sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function)
+    need_grad = _needs_grad(x_seq, v)
+    sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function) if need_grad else (0, 0.0)
+    if not torch.compiler.is_compiling():
+        s, v_seq, v_last = K.eager_multistep(L.NEURON_LIF, x2, v1, None, float(tau), v_threshold, vr,
+                                             K._flags(soft, detach_reset, decay_input, flags), sg_id, sg_alpha,
+                                             store_v_seq, need_grad and _hip_recompute(x2), need_grad)
+    elif need_grad:
         s, v_seq, v_last, _ = K.hip_multistep_lif_forward(x2, v1, v_threshold, vr, soft, detach_reset,
                                                           float(tau), decay_input, sg_id, sg_alpha,
                                                           store_v_seq, flags, _hip_recompute(x2))
@@ -252,6 +264,7 @@ def plif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Tensor, d
                         ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     """Multi-step parametric LIF on the hip backend.  ``w`` is the pre-sigmoid parameter; the
     sigmoid stays outside the operator so autograd supplies ``dk/dw`` (reference :2173-2182)."""
+    from ..hip_kernel import library as L
     from ..hip_kernel import neuron_kernel as K
     from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
 
@@ -260,8 +273,13 @@ def plif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Tensor, d
     flags = _hip_mode_flags(x_seq)
     x2, v1 = x_seq.flatten(1), v.flatten()
     k = w.sigmoid().to(device=x_seq.device, dtype=torch.float32)
-    if _needs_grad(x_seq, v, w):
-        sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function)
+    need_grad = _needs_grad(x_seq, v, w)
+    sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function) if need_grad else (0, 0.0)
+    if not torch.compiler.is_compiling():
+        s, v_seq, v_last = K.eager_multistep(L.NEURON_PLIF, x2, v1, k, 0.0, v_threshold, vr,
+                                             K._flags(soft, detach_reset, decay_input, flags), sg_id, sg_alpha,
+                                             store_v_seq, need_grad and _hip_recompute(x2), need_grad)
+    elif need_grad:
         s, v_seq, v_last, _ = K.hip_multistep_plif_forward(x2, v1, k, v_threshold, vr, soft, detach_reset,
                                                            decay_input, sg_id, sg_alpha, store_v_seq, flags,
                                                            _hip_recompute(x2))
@@ -276,6 +294,7 @@ def qif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_thres
                        surrogate_function: SurrogateFunction, store_v_seq: bool = False
                        ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     """Multi-step QIF on the hip backend; argument order of the reference's ``qif_multi_step_cupy`` (:2188-2200)."""
+    from ..hip_kernel import library as L
     from ..hip_kernel import neuron_kernel as K
     from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
 
@@ -283,8 +302,14 @@ def qif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_thres
     vr = 0.0 if soft else float(v_reset)
     flags = _hip_mode_flags(x_seq)
     x2, v1 = x_seq.flatten(1), v.flatten()
-    if _needs_grad(x_seq, v):
-        sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function)
+    need_grad = _needs_grad(x_seq, v)
+    sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function) if need_grad else (0, 0.0)
+    if not torch.compiler.is_compiling():
+        s, v_seq, v_last = K.eager_multistep(L.NEURON_QIF, x2, v1, None, float(tau), v_threshold, vr,
+                                             K._flags(soft, detach_reset, True, flags), sg_id, sg_alpha, store_v_seq,
+                                             need_grad and _hip_recompute(x2), need_grad,
+                                             qif=(float(v_rest), float(v_c), float(a0)))
+    elif need_grad:
         s, v_seq, v_last, _ = K.hip_multistep_qif_forward(x2, v1, v_threshold, vr, soft, detach_reset, float(tau),
                                                           float(v_rest), float(v_c), float(a0), sg_id, sg_alpha,
                                                           store_v_seq, flags, _hip_recompute(x2))
@@ -302,6 +327,7 @@ def ilif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_thre
     ``MultiLevelSpikeCount`` (its ``max_spike_count`` and gradient window go to the kernel, as the reference's
     Triton path passes them, ``neuron/ilif.py:343-353``).  ``spike_seq`` holds the counts."""
     from .. import surrogate
+    from ..hip_kernel import library as L
     from ..hip_kernel import neuron_kernel as K
 
     if not isinstance(surrogate_function, surrogate.MultiLevelSpikeCount) or not surrogate_function.spiking:
@@ -309,7 +335,13 @@ def ilif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_thre
     levels = int(surrogate_function.max_spike_count)
     flags = _hip_mode_flags(x_seq)
     x2, v1 = x_seq.flatten(1), v.flatten()
-    if _needs_grad(x_seq, v):
+    need_grad = _needs_grad(x_seq, v)
+    if not torch.compiler.is_compiling():
+        s, v_seq, v_last = K.eager_multistep(
+            L.NEURON_ILIF, x2, v1, None, float(tau), float(v_threshold), 0.0, K._flags(True, detach_reset, False, flags),
+            L.SG_MULTI_LEVEL, 0.0, store_v_seq, need_grad and _hip_recompute(x2), need_grad,
+            levels=(float(levels), float(surrogate_function.grad_min), float(surrogate_function.grad_max)))
+    elif need_grad:
         s, v_seq, v_last, _ = K.hip_multistep_ilif_forward(
             x2, v1, float(tau), float(v_threshold), levels, float(surrogate_function.grad_min),
             float(surrogate_function.grad_max), detach_reset, store_v_seq, flags, _hip_recompute(x2))
