@@ -191,6 +191,12 @@ def _hip_recompute(x2: torch.Tensor) -> bool:
     return width > 0 and x2.shape[1] % width == 0 and x2.shape[0] <= steps
 
 
+def _use_eager_entry() -> bool:
+    """The direct ``autograd.Function`` entry serves ordinary eager calls; a tracing compiler needs the operators
+    (schema, fake kernels)."""
+    return not torch.compiler.is_compiling()
+
+
 def _needs_grad(*tensors: torch.Tensor) -> bool:
     return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
 
@@ -217,7 +223,7 @@ def if_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, v_threshold: float, 
     x2, v1 = x_seq.flatten(1), v.flatten()
     need_grad = _needs_grad(x_seq, v)
     sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function) if need_grad else (0, 0.0)
-    if not torch.compiler.is_compiling():
+    if _use_eager_entry():
         s, v_seq, v_last = K.eager_multistep(L.NEURON_IF, x2, v1, None, 0.0, v_threshold, vr,
                                              K._flags(soft, detach_reset, False, flags), sg_id, sg_alpha, store_v_seq,
                                              need_grad and _hip_recompute(x2), need_grad)
@@ -244,7 +250,7 @@ def lif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, decay_i
     x2, v1 = x_seq.flatten(1), v.flatten()
     need_grad = _needs_grad(x_seq, v)
     sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function) if need_grad else (0, 0.0)
-    if not torch.compiler.is_compiling():
+    if _use_eager_entry():
         s, v_seq, v_last = K.eager_multistep(L.NEURON_LIF, x2, v1, None, float(tau), v_threshold, vr,
                                              K._flags(soft, detach_reset, decay_input, flags), sg_id, sg_alpha,
                                              store_v_seq, need_grad and _hip_recompute(x2), need_grad)
@@ -275,7 +281,7 @@ def plif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Tensor, d
     k = w.sigmoid().to(device=x_seq.device, dtype=torch.float32)
     need_grad = _needs_grad(x_seq, v, w)
     sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function) if need_grad else (0, 0.0)
-    if not torch.compiler.is_compiling():
+    if _use_eager_entry():
         s, v_seq, v_last = K.eager_multistep(L.NEURON_PLIF, x2, v1, k, 0.0, v_threshold, vr,
                                              K._flags(soft, detach_reset, decay_input, flags), sg_id, sg_alpha,
                                              store_v_seq, need_grad and _hip_recompute(x2), need_grad)
@@ -304,7 +310,7 @@ def qif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_thres
     x2, v1 = x_seq.flatten(1), v.flatten()
     need_grad = _needs_grad(x_seq, v)
     sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function) if need_grad else (0, 0.0)
-    if not torch.compiler.is_compiling():
+    if _use_eager_entry():
         s, v_seq, v_last = K.eager_multistep(L.NEURON_QIF, x2, v1, None, float(tau), v_threshold, vr,
                                              K._flags(soft, detach_reset, True, flags), sg_id, sg_alpha, store_v_seq,
                                              need_grad and _hip_recompute(x2), need_grad,
@@ -336,7 +342,7 @@ def ilif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_thre
     flags = _hip_mode_flags(x_seq)
     x2, v1 = x_seq.flatten(1), v.flatten()
     need_grad = _needs_grad(x_seq, v)
-    if not torch.compiler.is_compiling():
+    if _use_eager_entry():
         s, v_seq, v_last = K.eager_multistep(
             L.NEURON_ILIF, x2, v1, None, float(tau), float(v_threshold), 0.0, K._flags(True, detach_reset, False, flags),
             L.SG_MULTI_LEVEL, 0.0, store_v_seq, need_grad and _hip_recompute(x2), need_grad,

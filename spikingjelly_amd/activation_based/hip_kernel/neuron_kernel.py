@@ -719,19 +719,26 @@ class _EagerNeuron(torch.autograd.Function):
     55 us (forward) + 50 us (backward) of host time on top of the 12 us each launch takes, this about 15 + 30."""
 
     @staticmethod
-    def forward(ctx, x_seq, v_init, k, spec):
+    def forward(x_seq, v_init, k, spec):
         neuron, tau, v_th, v_reset, flags, _, _, store_v_seq, recompute, qif, levels = spec
         s, v_seq, v_last, h_seq = _run_forward(neuron, x_seq, v_init, k, tau, v_th, v_reset, flags, store_v_seq,
                                                not recompute, qif, levels)
+        return s, v_seq, v_last, (h_seq if h_seq is not None else x_seq.new_empty((0,)))
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        x_seq, v_init, k, spec = inputs
+        neuron, recompute = spec[0], spec[8]
         ctx.spec = spec
         # PLIF and QIF need the state before the first step in either backward; the replay needs it to start from
         keep_v_init = recompute or neuron in (L.NEURON_PLIF, L.NEURON_QIF)
-        ctx.save_for_backward(x_seq if recompute else h_seq, v_init if keep_v_init else None, k)
+        ctx.save_for_backward(x_seq if recompute else output[3], v_init if keep_v_init else None, k)
+        ctx.mark_non_differentiable(output[3])
         ctx.set_materialize_grads(False)
-        return s, v_seq, v_last
 
     @staticmethod
-    def backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last):
+    def backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_seq):
+        del grad_h_seq
         neuron, tau, v_th, v_reset, flags, sg_id, sg_alpha, store_v_seq, recompute, qif, levels = ctx.spec
         first, v_init, k = ctx.saved_tensors
         h_seq, x_seq = (None, first) if recompute else (first, None)
@@ -753,6 +760,6 @@ def eager_multistep(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: O
     ``h_seq``, or ``x_seq`` and ``v_init`` with ``recompute``) or the inference path (saves nothing)."""
     if need_grad:
         spec = (neuron, tau, v_th, v_reset, flags, sg_id, sg_alpha, store_v_seq, recompute, qif, levels)
-        return _EagerNeuron.apply(x_seq, v_init, k, spec)
+        return _EagerNeuron.apply(x_seq, v_init, k, spec)[:3]
     return _run_forward(neuron, x_seq.detach(), v_init.detach(), None if k is None else k.detach(), tau, v_th, v_reset,
                         flags, store_v_seq, False, qif, levels)[:3]

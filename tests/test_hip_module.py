@@ -268,3 +268,4 @@ def test_replay_path_with_misaligned_and_non_contiguous_input():
     a(xa).backward(g)
     b(xb).backward(g.cuda())
     torch.testing.assert_close(xb.grad.cpu(), xa.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+
