@@ -17,6 +17,8 @@
  *                             spikingjelly/activation_based/triton_kernel/neuron_kernel/lif.py:673-763
  *                             QIF: torch.ops.sj.cupy_multistep_qif_forward and its backward,
  *                             cuda_kernel/neuron_kernel/multi_step/qif.py:21-277, 628-701
+ *                             EIF: torch.ops.sj.cupy_multistep_eif_forward and its backward,
+ *                             cuda_kernel/neuron_kernel/multi_step/eif.py
  *                             ILIF: torch.ops.sj.multistep_ilif_forward{,_no_grad} and its backward,
  *                             triton_kernel/neuron_kernel/ilif.py:37-235, 241-462, 556-726
  *   sjhip_neuron_forward_packed <- the same forward ops followed by BitSpikeCompressor.compress,
@@ -56,6 +58,11 @@ typedef enum sjhip_neuron {
   SJHIP_NEURON_LIF = 1, /* h = v + (x - (v - vr)) / tau  or  v - (v - vr)/tau + x   (:849-852)     */
   SJHIP_NEURON_PLIF = 2, /* h = v + (x - (v - vr)) * k    or  v - (v - vr)*k + x     (:1290-1295)   */
   SJHIP_NEURON_QIF = 3, /* h = v + (x + a0 (v - v_rest) (v - v_c)) / tau          (functional/neuron.py:397) */
+  SJHIP_NEURON_EIF = 5, /* exponential integrate-and-fire (functional/neuron.py:483-485):
+                           h = v + (x + v_rest - v + delta_T exp((v - theta_rh) / delta_T)) / tau; theta_rh travels in
+                           the field v_c and delta_T (> 0) in the field a0.  exp() is the device library's, accurate
+                           to 1 ulp but not bit-identical to a host libm: h agrees with a CPU run to rounding, a
+                           spike may differ where h lands within that distance of v_threshold. */
   SJHIP_NEURON_ILIF = 4 /* integer-valued LIF (functional/neuron.py:1097-1099): h = v - v/tau + x (the LIF charge
                            without input decay and with v_reset = None), fires the count
                            c = rint(clamp(h / v_th, 0, level_max)) instead of a binary spike and resets softly by
@@ -113,9 +120,9 @@ typedef struct sjhip_neuron_params {
   float sg_alpha;   /* backward only */
   int32_t sg_id;    /* backward only, sjhip_surrogate */
   uint32_t flags;
-  float v_rest;     /* QIF only */
-  float v_c;        /* QIF only */
-  float a0;         /* QIF only */
+  float v_rest;     /* QIF and EIF */
+  float v_c;        /* QIF: critical voltage; EIF: theta_rh */
+  float a0;         /* QIF: a0; EIF: delta_T */
   float level_max;  /* ILIF only: largest spike count D, an integer >= 1 */
   float grad_min;   /* ILIF only, backward: lower end of the gradient window on h / v_th */
   float grad_max;   /* ILIF only, backward: upper end (grad_min <= grad_max) */

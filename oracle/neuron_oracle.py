@@ -196,6 +196,10 @@ def charge(kind: str, x, v, tau_or_w, decay_input: bool, v_reset: Optional[float
         # functional/neuron.py:397; tau_or_w = (tau, a0, v_rest, v_c)
         tau, a0, v_rest, v_c = tau_or_w
         return v + (x + a0 * (v - v_rest) * (v - v_c)) / tau
+    if kind == "eif":
+        # functional/neuron.py:483-485; tau_or_w = (tau, delta_t, theta_rh, v_rest)
+        tau, delta_t, theta_rh, v_rest = tau_or_w
+        return v + (x + v_rest - v + delta_t * torch.exp((v - theta_rh) / delta_t)) / tau
     raise ValueError(kind)
 
 

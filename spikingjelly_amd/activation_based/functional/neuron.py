@@ -32,12 +32,14 @@ __all__ = [
     "lif_step",
     "plif_step",
     "qif_step",
+    "eif_step",
     "ilif_step",
     "stbif_step",
     "if_multi_step_hip",
     "lif_multi_step_hip",
     "plif_multi_step_hip",
     "qif_multi_step_hip",
+    "eif_multi_step_hip",
     "ilif_multi_step_hip",
     "stbif_multi_step_hip",
     "stbif_single_step_hip",
@@ -107,6 +109,16 @@ def qif_step(x: torch.Tensor, v: torch.Tensor, tau: float, a0: float, v_rest: fl
              ) -> tuple[torch.Tensor, torch.Tensor]:
     """One quadratic integrate-and-fire step (reference :315-399): ``h = v + (x + a0 (v - v_rest)(v - v_c)) / tau``."""
     h = v + (x + a0 * (v - v_rest) * (v - v_c)) / tau
+    spike = surrogate_function(h - v_threshold)
+    return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset)
+
+
+def eif_step(x: torch.Tensor, v: torch.Tensor, tau: float, delta_t: float, theta_rh: float, v_rest: float,
+             v_threshold: float, v_reset: Optional[float], surrogate_function: SurrogateFunction,
+             detach_reset: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
+    """One exponential integrate-and-fire step (reference :402-487):
+    ``h = v + (x + v_rest - v + delta_t exp((v - theta_rh) / delta_t)) / tau``."""
+    h = v + (x + v_rest - v + delta_t * torch.exp((v - theta_rh) / delta_t)) / tau
     spike = surrogate_function(h - v_threshold)
     return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset)
 
@@ -322,6 +334,36 @@ def qif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_thres
     else:
         s, v_seq, v_last = K.hip_multistep_qif_inference(x2, v1, v_threshold, vr, soft, float(tau), float(v_rest),
                                                          float(v_c), float(a0), store_v_seq, flags)
+    return _finish(x_seq, s, v_seq, v_last, store_v_seq)
+
+
+def eif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_threshold: float, v_reset: Optional[float],
+                       v_rest: float, theta_rh: float, delta_t: float, detach_reset: bool,
+                       surrogate_function: SurrogateFunction, store_v_seq: bool = False
+                       ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Multi-step EIF on the hip backend; argument order of the reference's ``eif_multi_step_cupy`` (:2296-2308)."""
+    from ..hip_kernel import library as L
+    from ..hip_kernel import neuron_kernel as K
+    from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
+
+    soft = v_reset is None
+    vr = 0.0 if soft else float(v_reset)
+    flags = _hip_mode_flags(x_seq)
+    x2, v1 = x_seq.flatten(1), v.flatten()
+    need_grad = _needs_grad(x_seq, v)
+    sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function) if need_grad else (0, 0.0)
+    if _use_eager_entry():
+        s, v_seq, v_last = K.eager_multistep(L.NEURON_EIF, x2, v1, None, float(tau), v_threshold, vr,
+                                             K._flags(soft, detach_reset, True, flags), sg_id, sg_alpha, store_v_seq,
+                                             need_grad and _hip_recompute(x2), need_grad,
+                                             qif=(float(v_rest), float(theta_rh), float(delta_t)))
+    elif need_grad:
+        s, v_seq, v_last, _ = K.hip_multistep_eif_forward(x2, v1, v_threshold, vr, soft, detach_reset, float(tau),
+                                                          float(v_rest), float(theta_rh), float(delta_t), sg_id, sg_alpha,
+                                                          store_v_seq, flags, _hip_recompute(x2))
+    else:
+        s, v_seq, v_last = K.hip_multistep_eif_inference(x2, v1, v_threshold, vr, soft, float(tau), float(v_rest),
+                                                         float(theta_rh), float(delta_t), store_v_seq, flags)
     return _finish(x_seq, s, v_seq, v_last, store_v_seq)
 
 

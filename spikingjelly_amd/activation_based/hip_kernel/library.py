@@ -17,7 +17,7 @@ import torch
 ABI_VERSION = 3
 
 # enums of include/sjhip.h
-NEURON_IF, NEURON_LIF, NEURON_PLIF, NEURON_QIF, NEURON_ILIF = 0, 1, 2, 3, 4
+NEURON_IF, NEURON_LIF, NEURON_PLIF, NEURON_QIF, NEURON_ILIF, NEURON_EIF = 0, 1, 2, 3, 4, 5
 SG_MULTI_LEVEL = 7  # ILIF's windowed straight-through estimator; ids 0-6 are listed in surrogate_registry
 DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_U8 = 0, 1, 2, 3
 FLAG_DECAY_INPUT = 0x01

@@ -10,6 +10,7 @@ inference op that writes no ``h_seq``):
     sj::hip_multistep_{if,lif,plif}_backward   -> (grad_x_seq, grad_v_init[, grad_k])
     sj::hip_multistep_{if,lif,plif}_inference_packed -> (spike_bits, v_seq, v_last)
     sj::hip_multistep_qif_{forward,inference,backward}   the quadratic integrate-and-fire neuron, same outputs
+    sj::hip_multistep_eif_{forward,inference,backward}   the exponential integrate-and-fire neuron
     sj::hip_multistep_ilif_{forward,inference,backward}  the integer-valued LIF: spike_seq holds counts 0..D
 
 The ``_packed`` ops write the spikes bit-packed (uint8, ``T*N/8`` bytes, the layout of
@@ -40,6 +41,7 @@ __all__ = [
     "packed_supported",
     "hip_multistep_qif_forward", "hip_multistep_qif_inference", "hip_multistep_qif_backward",
     "hip_multistep_ilif_forward", "hip_multistep_ilif_inference", "hip_multistep_ilif_backward",
+    "hip_multistep_eif_forward", "hip_multistep_eif_inference", "hip_multistep_eif_backward",
 ]
 
 
@@ -226,7 +228,7 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
             rc = L.load().sjhip_neuron_backward(
                 neuron, dtype, ctypes.byref(params), T, N,
                 grad_spike_seq.data_ptr(), L.ptr(grad_v_seq), L.ptr(grad_v_last), h_seq.data_ptr(),
-                L.ptr(v_init) if neuron in (L.NEURON_PLIF, L.NEURON_QIF) else None, k_ptr,
+                L.ptr(v_init) if neuron in (L.NEURON_PLIF, L.NEURON_QIF, L.NEURON_EIF) else None, k_ptr,
                 grad_x_seq.data_ptr(), grad_v_init.data_ptr() if need_grad_v_init else None, L.ptr(grad_k), L.ptr(workspace),
                 L.current_stream_ptr(h_seq.device),
             )
@@ -632,6 +634,91 @@ torch.library.register_autograd("sj::hip_multistep_qif_forward", _qif_autograd_b
 
 
 # =================================================================================================
+# EIF: h = v + (x + v_rest - v + delta_T exp((v - theta_rh) / delta_T)) / tau
+# (reference cuda_kernel/neuron_kernel/multi_step/eif.py); theta_rh and delta_T travel in the parameter fields v_c and a0
+# =================================================================================================
+@torch.library.custom_op("sj::hip_multistep_eif_forward", mutates_args=())
+def hip_multistep_eif_forward(x_seq: torch.Tensor, v_init: torch.Tensor, v_th: float, v_reset: float,
+                              soft_reset: bool, detach_reset: bool, tau: float, v_rest: float, theta_rh: float,
+                              delta_t: float, sg_id: int, sg_alpha: float, store_v_seq: bool, mode_flags: int,
+                              recompute: bool
+                              ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, detach_reset, True, mode_flags)
+    return _forward_outputs(_run_forward(L.NEURON_EIF, x_seq, v_init, None, tau, v_th, v_reset, flags, store_v_seq,
+                                         not recompute, (v_rest, theta_rh, delta_t)), x_seq)
+
+
+@hip_multistep_eif_forward.register_fake
+def _(x_seq, v_init, v_th, v_reset, soft_reset, detach_reset, tau, v_rest, theta_rh, delta_t, sg_id, sg_alpha, store_v_seq,
+      mode_flags, recompute):
+    return _fake_forward(x_seq, v_init, store_v_seq, True, recompute)
+
+
+@torch.library.custom_op("sj::hip_multistep_eif_inference", mutates_args=())
+def hip_multistep_eif_inference(x_seq: torch.Tensor, v_init: torch.Tensor, v_th: float, v_reset: float,
+                                soft_reset: bool, tau: float, v_rest: float, theta_rh: float, delta_t: float,
+                                store_v_seq: bool, mode_flags: int
+                                ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, False, True, mode_flags)
+    return _run_forward(L.NEURON_EIF, x_seq, v_init, None, tau, v_th, v_reset, flags, store_v_seq, False,
+                        (v_rest, theta_rh, delta_t))[:3]
+
+
+@hip_multistep_eif_inference.register_fake
+def _(x_seq, v_init, v_th, v_reset, soft_reset, tau, v_rest, theta_rh, delta_t, store_v_seq, mode_flags):
+    return _fake_forward(x_seq, v_init, store_v_seq, False)
+
+
+@torch.library.custom_op("sj::hip_multistep_eif_backward", mutates_args=())
+def hip_multistep_eif_backward(grad_spike_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
+                               grad_v_last: Optional[torch.Tensor], h_seq: Optional[torch.Tensor],
+                               x_seq: Optional[torch.Tensor], v_init: torch.Tensor, v_th: float,
+                               v_reset: float, soft_reset: bool, detach_reset: bool, tau: float, v_rest: float,
+                               theta_rh: float, delta_t: float, sg_id: int, sg_alpha: float, mode_flags: int,
+                               need_grad_v_init: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
+    flags = _flags(soft_reset, detach_reset, True, mode_flags)
+    gx, gvi, _ = _run_backward(L.NEURON_EIF, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, None,
+                               tau, v_th, v_reset, flags, sg_id, sg_alpha, need_grad_v_init, (v_rest, theta_rh, delta_t))
+    return gx, gvi
+
+
+@hip_multistep_eif_backward.register_fake
+def _(grad_spike_seq, grad_v_seq, grad_v_last, h_seq, x_seq, v_init, v_th, v_reset, soft_reset, detach_reset,
+      tau, v_rest, theta_rh, delta_t, sg_id, sg_alpha, mode_flags, need_grad_v_init=True):
+    ref = h_seq if h_seq is not None else x_seq
+    return torch.empty_like(ref), ref.new_empty(ref.shape[1:] if need_grad_v_init else (0,))
+
+
+def _eif_setup_context(ctx, inputs, output):
+    (x_seq, v_init, v_th, v_reset, soft_reset, detach_reset, tau, v_rest, theta_rh, delta_t, sg_id, sg_alpha, store_v_seq,
+     mode_flags, recompute) = inputs
+    ctx.recompute = recompute
+    # the state-dependent dh/dv needs v_init on both paths
+    if recompute:
+        ctx.save_for_backward(x_seq, v_init)
+    else:
+        ctx.save_for_backward(output[3], v_init)
+    ctx.scalars = (v_th, v_reset, soft_reset, detach_reset, tau, v_rest, theta_rh, delta_t, sg_id, sg_alpha, mode_flags)
+    ctx.store_v_seq = store_v_seq
+    ctx.set_materialize_grads(False)
+
+
+def _eif_autograd_backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_seq):
+    del grad_h_seq
+    first, v_init = ctx.saved_tensors
+    h_seq, x_seq = (None, first) if ctx.recompute else (first, None)
+    need = bool(ctx.needs_input_grad[1])
+    gx, gvi = hip_multistep_eif_backward(
+        grad_spike_seq, _none_if_empty_grad(grad_v_seq, ctx.store_v_seq), grad_v_last, h_seq, x_seq, v_init,
+        *ctx.scalars, need)
+    return (gx, (gvi if need else None)) + (None,) * 13
+
+
+torch.library.register_autograd("sj::hip_multistep_eif_forward", _eif_autograd_backward,
+                                setup_context=_eif_setup_context)
+
+
+# =================================================================================================
 # ILIF: h = v - v / tau + x,  c = rint(clamp(h / v_th, 0, D)),  v' = h - c v_th
 # (reference triton_kernel/neuron_kernel/ilif.py:556-726; the op there takes decay = 1 - 1/tau, these take tau
 # because the kernels charge in the torch backend's own arithmetic form)
@@ -731,7 +818,7 @@ class _EagerNeuron(torch.autograd.Function):
         neuron, recompute = spec[0], spec[8]
         ctx.spec = spec
         # PLIF and QIF need the state before the first step in either backward; the replay needs it to start from
-        keep_v_init = recompute or neuron in (L.NEURON_PLIF, L.NEURON_QIF)
+        keep_v_init = recompute or neuron in (L.NEURON_PLIF, L.NEURON_QIF, L.NEURON_EIF)
         ctx.save_for_backward(x_seq if recompute else output[3], v_init if keep_v_init else None, k)
         ctx.mark_non_differentiable(output[3])
         ctx.set_materialize_grads(False)

@@ -2,8 +2,8 @@ from .base_node import BaseNode
 from .ilif import ILIFNode
 from .integrate_and_fire import IFNode
 from .lif import LIFNode
-from .nonlinear_if import QIFNode
+from .nonlinear_if import EIFNode, QIFNode
 from .plif import ParametricLIFNode
 from .spikezip import STBIFNeuron
 
-__all__ = ["BaseNode", "IFNode", "LIFNode", "ParametricLIFNode", "QIFNode", "ILIFNode", "STBIFNeuron"]
+__all__ = ["BaseNode", "IFNode", "LIFNode", "ParametricLIFNode", "QIFNode", "EIFNode", "ILIFNode", "STBIFNeuron"]

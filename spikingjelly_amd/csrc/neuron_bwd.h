@@ -66,7 +66,8 @@ struct BwdArgs {
   int is_if;
   int atomic_reduce;
   int v_init_broadcast;  // v_init holds one element for all neurons
-  float q_rest, q_c, q_a0;  // QIF
+  float q_rest, q_c, q_a0;  // QIF, EIF
+  int exponential;          // the state-dependent mode is EIF's, not QIF's
   float grad_min, grad_max; // ILIF: gradient window on h / v_th
   float vth_inv;            // ILIF: 1 / v_threshold when that is an exact power of two, else 0 (as in FwdArgs)
   float vth_rcp;            // ILIF: fl(1 / v_threshold), the factor of the count's gradient
@@ -124,9 +125,11 @@ __device__ __forceinline__ float reset_as_forward(float h, float s, const BwdArg
   return a.soft_reset ? (h - s * a.v_th) : (s * a.v_reset + (1.0f - s) * h);
 }
 
-// QIF: d h_{t+1} / d v_t
+// QIF / EIF: d h_{t+1} / d v_t.  EIF (h = v + k (x + v_rest - v + dT exp((v - theta) / dT)), cuda_kernel/neuron_kernel/
+// multi_step/eif.py): 1 + k (exp((v - theta) / dT) - 1), with theta in q_c and dT in q_a0.
 __device__ __forceinline__ float qif_dh_dv(float v, float k, const BwdArgs &a) {
 #pragma clang fp contract(fast)
+  if (a.exponential) return 1.0f + k * (__expf((v - a.q_c) / a.q_a0) - 1.0f);
   return 1.0f + k * a.q_a0 * ((v - a.q_c) + (v - a.q_rest));
 }
 
@@ -397,7 +400,8 @@ inline int build_bwd_args(BwdArgs &a, int neuron, int dtype, const sjhip_neuron_
 
   const bool plif = neuron == SJHIP_NEURON_PLIF;
   a.q_rest = p.v_rest; a.q_c = p.v_c; a.q_a0 = p.a0;
-  if (neuron == SJHIP_NEURON_QIF) a.decay_input = 1;  // grad_x = G k
+  a.exponential = neuron == SJHIP_NEURON_EIF ? 1 : 0;
+  if (neuron == SJHIP_NEURON_QIF || neuron == SJHIP_NEURON_EIF) a.decay_input = 1;  // grad_x = G k
   if (neuron == SJHIP_NEURON_IF) {
     a.k = 0.0f;
   } else if (plif) {

@@ -80,7 +80,7 @@ int launch_backward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t
   int rc = build_bwd_args(a, neuron, dtype, p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, k_device,
                           grad_x_seq, grad_v_init, grad_rtau, workspace);
   if (rc != SJHIP_OK) return rc;
-  const int mode = neuron == SJHIP_NEURON_PLIF ? BWD_PLIF : (neuron == SJHIP_NEURON_QIF ? BWD_QIF : BWD_PLAIN);
+  const int mode = neuron == SJHIP_NEURON_PLIF ? BWD_PLIF : ((neuron == SJHIP_NEURON_QIF || neuron == SJHIP_NEURON_EIF) ? BWD_QIF : BWD_PLAIN);
 
   const int esize = dtype == SJHIP_F32 ? 4 : 2;
   const int V = 16 / esize;

@@ -112,6 +112,8 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_kernel(con
       case CH_PLAIN_INPUT_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_PLAIN_INPUT_DIV>(f, lds_h, col); break;
       case CH_QIF_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_QIF_DIV>(f, lds_h, col); break;
       case CH_QIF_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_QIF_MUL>(f, lds_h, col); break;
+      case CH_EIF_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_EIF_DIV>(f, lds_h, col); break;
+      case CH_EIF_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_EIF_MUL>(f, lds_h, col); break;
       default: recompute_reset_dispatch<S, ROUND_EACH, CH_PLAIN_INPUT_MUL>(f, lds_h, col); break;
     }
   }

@@ -78,7 +78,7 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
   const unsigned cap = occupancy_cap_lds(tuning().replay_blocks_per_cu);
   if (cap > lds) lds = cap;
   const bool plif = neuron == SJHIP_NEURON_PLIF;
-  const int mode = plif ? BWD_PLIF : (neuron == SJHIP_NEURON_QIF ? BWD_QIF : BWD_PLAIN);
+  const int mode = plif ? BWD_PLIF : ((neuron == SJHIP_NEURON_QIF || neuron == SJHIP_NEURON_EIF) ? BWD_QIF : BWD_PLAIN);
   {
     ProfileScope prof(KC_BACKWARD, stream);
     switch (dtype) {

@@ -40,7 +40,9 @@ enum Charge {
   CH_PLAIN_INPUT_DIV = 3,  // v - (v - vr) / tau + x
   CH_PLAIN_INPUT_MUL = 4,  // v - (v - vr) * k + x
   CH_QIF_DIV = 5,          // v + (x + a0 * (v - v_rest) * (v - v_c)) / tau
-  CH_QIF_MUL = 6           // the same with * k
+  CH_QIF_MUL = 6,          // the same with * k
+  CH_EIF_DIV = 7,          // v + (x + v_rest - v + dT * exp((v - theta) / dT)) / tau
+  CH_EIF_MUL = 8           // the same with * k
 };
 
 struct FwdArgs {
@@ -58,7 +60,7 @@ struct FwdArgs {
   float vth_sub; // v_threshold as a subtrahend
   float vth_mul; // v_threshold as a factor
   float q_rest_sub; // QIF: v_rest and v_c as subtrahends (rounded like vr_add), a0 as a factor
-  float q_c_sub;
+  float q_c_sub;    // EIF: v_rest as an addend, theta_rh as a subtrahend, delta_T as divisor and factor
   float q_a0_mul;
   float level_max;  // ILIF: largest spike count
   float vth_inv;    // ILIF: 1 / v_threshold when that is an exact power of two (h / v_th == h * vth_inv bit for bit), else 0
@@ -91,6 +93,14 @@ __device__ __forceinline__ void neuron_step(float x, float &v, float &h, float &
     float m2 = Cvt<R>::round(m1 * d2);
     float e = Cvt<R>::round(x + m2);
     float f = (CH == CH_QIF_DIV) ? Cvt<R>::round(e / tau) : Cvt<R>::round(e * tau);
+    h = Cvt<R>::round(v + f);
+  } else if (CH == CH_EIF_DIV || CH == CH_EIF_MUL) {
+    // functional/neuron.py:483-485, left to right: ((x + v_rest) - v) + delta_T * exp((v - theta_rh) / delta_T)
+    float b = Cvt<R>::round(Cvt<R>::round(x + a.q_rest_sub) - v);
+    float d = Cvt<R>::round(Cvt<R>::round(v - a.q_c_sub) / a.q_a0_mul);
+    float e = Cvt<R>::round(expf(d));
+    float g = Cvt<R>::round(b + Cvt<R>::round(a.q_a0_mul * e));
+    float f = (CH == CH_EIF_DIV) ? Cvt<R>::round(g / tau) : Cvt<R>::round(g * tau);
     h = Cvt<R>::round(v + f);
   } else {
     float d = Cvt<R>::round(v - a.vr_add);
@@ -159,6 +169,13 @@ __device__ __forceinline__ void neuron_step(_Float16 x, _Float16 &v, _Float16 &h
     const H m2 = m1 * d2;
     const H e = x + m2;
     const H f = (CH == CH_QIF_DIV) ? (H)((float)e / tau) : scalar_product_f16(tau, e);
+    h = v + f;
+  } else if (CH == CH_EIF_DIV || CH == CH_EIF_MUL) {
+    const H b = (x + (H)a.q_rest_sub) - v;
+    const H d = (H)((float)(H)(v - (H)a.q_c_sub) / a.q_a0_mul);
+    const H e = (H)expf((float)d);
+    const H g = b + scalar_product_f16(a.q_a0_mul, e);
+    const H f = (CH == CH_EIF_DIV) ? (H)((float)g / tau) : scalar_product_f16(tau, g);
     h = v + f;
   } else {
     const H d = v - vr_add;
@@ -292,6 +309,8 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) forward_kernel(const FwdArgs 
     case CH_PLAIN_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_DIV, PACKED>(a); break;
     case CH_QIF_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_QIF_DIV, PACKED>(a); break;
     case CH_QIF_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_QIF_MUL, PACKED>(a); break;
+    case CH_EIF_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_EIF_DIV, PACKED>(a); break;
+    case CH_EIF_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_EIF_MUL, PACKED>(a); break;
     default: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_MUL, PACKED>(a); break;
   }
 }
@@ -319,18 +338,18 @@ inline int build_fwd_args(FwdArgs &a, bool &round_each, int neuron, int dtype, c
     a.charge = decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL;
     a.k_device = k_device;
   } else {
-    const bool qif = neuron == SJHIP_NEURON_QIF;
+    const bool qif = neuron == SJHIP_NEURON_QIF, eif = neuron == SJHIP_NEURON_EIF;
     if (!(p.tau > 0.0f) || !std::isfinite(p.tau)) return fail(SJHIP_ERR_INVALID, "forward: tau=%g", (double)p.tau);
     if (p.flags & SJHIP_FLAG_RECIPROCAL_TAU) {
       // fl(1/tau) from the double quotient, as the reference kernels receive it (multi_step/lif.py:338)
       a.tau = (float)(1.0 / (double)p.tau);
-      a.charge = qif ? CH_QIF_MUL : (decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL);
+      a.charge = qif ? CH_QIF_MUL : eif ? CH_EIF_MUL : (decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL);
     } else if (exact_reciprocal(p.tau)) {
       // x / 2^e == x * 2^-e bit for bit (both are exact scalings, subnormal results round identically)
       a.tau = 1.0f / p.tau;
-      a.charge = qif ? CH_QIF_MUL : (decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL);
+      a.charge = qif ? CH_QIF_MUL : eif ? CH_EIF_MUL : (decay_input ? CH_DECAY_INPUT_MUL : CH_PLAIN_INPUT_MUL);
     } else {
-      a.charge = qif ? CH_QIF_DIV : (decay_input ? CH_DECAY_INPUT_DIV : CH_PLAIN_INPUT_DIV);
+      a.charge = qif ? CH_QIF_DIV : eif ? CH_EIF_DIV : (decay_input ? CH_DECAY_INPUT_DIV : CH_PLAIN_INPUT_DIV);
     }
   }
 

@@ -119,6 +119,8 @@ bool valid_dtype_fp(int dtype) { return dtype == SJHIP_F32 || dtype == SJHIP_F16
 
 // ILIF: the count limit must be a positive integer that every storage dtype holds exactly (bf16: up to 256)
 int check_levels(const char *what, int neuron, const sjhip_neuron_params &p, bool backward) {
+  if (neuron == SJHIP_NEURON_EIF && (!(p.a0 > 0.0f) || !std::isfinite(p.a0)))
+    return fail(SJHIP_ERR_INVALID, "%s: EIF delta_T=%g must be positive", what, (double)p.a0);
   if (neuron != SJHIP_NEURON_ILIF) {
     if (backward && p.sg_id == SJHIP_SG_MULTI_LEVEL) return fail(SJHIP_ERR_INVALID, "%s: the multi-level surrogate belongs to ILIF", what);
     return SJHIP_OK;
@@ -152,7 +154,7 @@ int sjhip_neuron_forward(int neuron, int dtype, const sjhip_neuron_params *p, in
                          const void *x_seq, const void *v_init, const float *rtau_device, void *spike_seq,
                          void *v_seq, void *v_last, void *h_seq, void *stream) {
   if (!p) return fail(SJHIP_ERR_INVALID, "forward: params is NULL");
-  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_ILIF) return fail(SJHIP_ERR_INVALID, "forward: neuron %d", neuron);
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_EIF) return fail(SJHIP_ERR_INVALID, "forward: neuron %d", neuron);
   if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "forward: dtype %d", dtype);
   int rc = check_shape("forward", T, N);
   if (rc != SJHIP_OK) return rc;
@@ -168,7 +170,7 @@ int sjhip_neuron_forward_packed(int neuron, int dtype, const sjhip_neuron_params
                                 const void *x_seq, const void *v_init, const float *rtau_device, uint8_t *spike_bits,
                                 void *v_seq, void *v_last, void *stream) {
   if (!p) return fail(SJHIP_ERR_INVALID, "forward_packed: params is NULL");
-  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_ILIF) return fail(SJHIP_ERR_INVALID, "forward_packed: neuron %d", neuron);
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_EIF) return fail(SJHIP_ERR_INVALID, "forward_packed: neuron %d", neuron);
   if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "forward_packed: dtype %d", dtype);
   int rc = check_shape("forward_packed", T, N);
   if (rc != SJHIP_OK) return rc;
@@ -190,7 +192,7 @@ int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p, i
                           const float *rtau_device, void *grad_x_seq, void *grad_v_init, float *grad_rtau,
                           float *workspace, void *stream) {
   if (!p) return fail(SJHIP_ERR_INVALID, "backward: params is NULL");
-  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_ILIF) return fail(SJHIP_ERR_INVALID, "backward: neuron %d", neuron);
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_EIF) return fail(SJHIP_ERR_INVALID, "backward: neuron %d", neuron);
   if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "backward: dtype %d", dtype);
   if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_MULTI_LEVEL) return fail(SJHIP_ERR_UNSUPPORTED, "backward: surrogate id %d", p->sg_id);
   int rc = check_shape("backward", T, N);
@@ -198,7 +200,8 @@ int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p, i
   if (!grad_spike_seq || !h_seq || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward: NULL tensor");
   rc = check_levels("backward", neuron, *p, true);
   if (rc != SJHIP_OK) return rc;
-  if (neuron == SJHIP_NEURON_QIF && grad_v_init && !v_init) return fail(SJHIP_ERR_INVALID, "backward: QIF needs v_init for grad_v_init");
+  if ((neuron == SJHIP_NEURON_QIF || neuron == SJHIP_NEURON_EIF) && grad_v_init && !v_init)
+    return fail(SJHIP_ERR_INVALID, "backward: QIF / EIF need v_init for grad_v_init");
   if (neuron == SJHIP_NEURON_PLIF) {
     if (!v_init || !grad_rtau) return fail(SJHIP_ERR_INVALID, "backward: PLIF needs v_init and grad_rtau");
     if (!(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace) return fail(SJHIP_ERR_INVALID, "backward: PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");
@@ -224,7 +227,7 @@ int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_pa
                                     void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace,
                                     void *stream) {
   if (!p) return fail(SJHIP_ERR_INVALID, "backward(recompute): params is NULL");
-  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_ILIF) return fail(SJHIP_ERR_INVALID, "backward(recompute): neuron %d", neuron);
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_EIF) return fail(SJHIP_ERR_INVALID, "backward(recompute): neuron %d", neuron);
   if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "backward(recompute): dtype %d", dtype);
   if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_MULTI_LEVEL) return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute): surrogate id %d", p->sg_id);
   int rc = check_shape("backward(recompute)", T, N);

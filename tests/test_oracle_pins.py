@@ -585,3 +585,54 @@ def test_stbif_bounds_block_release_and_both_arithmetic_forms_agree_in_fp32():
     b = stbif_oracle.multi_step_fp32_state(x, torch.full((300,), 0.5), torch.zeros(300), *_stbif_tensors(0.25, 3, -4))
     for got, want in zip(b, a[:4]):
         assert torch.equal(got, want)
+
+
+# ------------------------------------------------------------------------------------------------
+# EIF (functional/neuron.py:483-485): pins that do not retype the formula
+# ------------------------------------------------------------------------------------------------
+def test_eif_rheobase_fixed_point_and_lif_limit():
+    """At v = theta_rh the exponential term is exactly delta_T, so x = v - v_rest - delta_T holds the potential
+    still.  Far below theta_rh (in units of delta_T) the exponential vanishes and the neuron is a LIF with input decay
+    resting at v_rest."""
+    tau, dT, theta, v_rest = 2.0, 0.25, 0.5, -0.125  # dyadic: every intermediate value is exact
+    v0 = torch.full((3,), theta)
+    x = torch.full((1, 3), theta - v_rest - dT)
+    _, _, h = no.multi_step("eif", x, v0, (tau, dT, theta, v_rest), True, 10.0, -1.0)
+    assert torch.equal(h[0], v0)
+    xs = seeded_randn((8, 200), 61, 0.0, 0.2, torch.float64)
+    v0 = seeded_randn((200,), 62, 0.0, 0.1, torch.float64)
+    p = (3.0, 0.01, 5.0, 0.1)  # theta_rh 490 delta_T above the potentials: exp() < 1e-200
+    s_e, v_e, h_e = no.multi_step("eif", xs, v0, p, True, 1.0, -0.5)
+    v = v0
+    for t in range(8):
+        h = v + (xs[t] - (v - 0.1)) / 3.0
+        torch.testing.assert_close(h_e[t], h, rtol=1e-13, atol=1e-15)
+        v = h  # no spikes at this drive
+    assert float(s_e.sum()) == 0.0
+
+
+@pytest.mark.parametrize("v_reset", [-0.1, None])
+def test_eif_autograd_matches_finite_differences_of_the_smooth_network(v_reset):
+    T, N, vth, alpha = 5, 6, 0.9, 2.0
+    p = (2.5, 0.5, 0.6, 0.0)
+    x = seeded_randn((T, N), 51, 0.4, 0.6, torch.float64)
+    v0 = seeded_randn((N,), 52, 0.0, 0.3, torch.float64)
+    gs = seeded_randn((T, N), 53, dtype=torch.float64)
+    gv = seeded_randn((T, N), 54, dtype=torch.float64)
+    smooth = no.surrogate("atan", alpha, spiking=False)
+
+    def loss(x_, v0_):
+        s, v, _ = no.multi_step("eif", x_, v0_, p, True, vth, v_reset, smooth)
+        return float((s * gs).sum() + (v * gv).sum())
+
+    ref = no.forward_backward("eif", x, v0, gs, gv, None, p, True, vth, v_reset, "atan", alpha, False, spiking=False)
+    eps = 1e-6
+    for (t, n) in [(0, 0), (2, 3), (T - 1, N - 1)]:
+        xp, xm = x.clone(), x.clone()
+        xp[t, n] += eps
+        xm[t, n] -= eps
+        assert (loss(xp, v0) - loss(xm, v0)) / (2 * eps) == pytest.approx(float(ref["grad_x"][t, n]), rel=1e-6, abs=1e-8)
+    vp, vm = v0.clone(), v0.clone()
+    vp[2] += eps
+    vm[2] -= eps
+    assert (loss(x, vp) - loss(x, vm)) / (2 * eps) == pytest.approx(float(ref["grad_v_init"][2]), rel=1e-6, abs=1e-8)
