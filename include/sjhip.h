@@ -250,6 +250,26 @@ int sjhip_stbif_forward(int dtype, uint32_t flags, int64_t T, int64_t N,
                         int32_t *work_flag, void *stream);
 
 /*
+ * Activation-aware IF (ANN2SNN activation-aware redistribution): an IF neuron whose threshold and membrane offset are
+ * per channel or scalar; inference only.  Stands in for torch.ops.sj.multistep_activation_aware_if_forward,
+ * spikingjelly/activation_based/triton_kernel/neuron_kernel/activation_aware_if.py:44-285, and computes the torch
+ * backend's functional.activation_aware_if_step (functional/neuron.py:577-584) for every step:
+ *     h = v + x;  s = [(h + offset_c) - threshold_c >= 0];  v = h - s threshold_c  or  s v_reset + (1 - s) h
+ * with c = (n / inner_size) % channel_size the channel of neuron n of a flattened time step.
+ *   x_seq [T,N] in        v_init [N] in ([1] with SJHIP_FLAG_V_INIT_BROADCAST)
+ *   v_threshold, v_offset   device fp32 arrays of threshold_count / offset_count elements, each 1 (scalar) or
+ *                           channel_size; rounded to `dtype` before use, like `.to(x)` in the reference
+ *   spike_seq [T,N] out;  v_seq [T,N] out or NULL;  v_last [N] out or NULL (at least one of the two)
+ * flags: SJHIP_FLAG_SOFT_RESET, SJHIP_FLAG_FP32_STATE, SJHIP_FLAG_V_INIT_BROADCAST.
+ */
+int sjhip_aaif_forward(int dtype, uint32_t flags, int64_t T, int64_t N,
+                       const void *x_seq, const void *v_init,
+                       const float *v_threshold, int64_t threshold_count,
+                       const float *v_offset, int64_t offset_count,
+                       int64_t channel_size, int64_t inner_size, float v_reset,
+                       void *spike_seq, void *v_seq, void *v_last, void *stream);
+
+/*
  * Spike bit-packing over a flattened tensor, LSB first: byte j bit i = (src[8j+i] != 0).
  *   src  n elements of `dtype` (F32/F16/BF16/U8)     dst  (n+7)/8 bytes; pad bits of the last byte are 0
  */

@@ -216,6 +216,38 @@ def step(kind: str, x, v, tau_or_w, decay_input: bool, v_threshold: float, v_res
     return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset), h
 
 
+def activation_aware_if_step(x, v, v_threshold, v_offset, v_reset: Optional[float], sg: Callable, detach_reset: bool):
+    """(spike, v_next, h): functional/neuron.py:577-584; v_threshold / v_offset are tensors broadcastable to x."""
+    h = v + x
+    spike = sg(h + v_offset - v_threshold)
+    spike_d = spike.detach() if detach_reset else spike
+    if v_reset is None:
+        v_next = h - spike_d * v_threshold
+    else:
+        v_next = spike_d * v_reset + (1.0 - spike_d) * h
+    return spike, v_next, h
+
+
+def activation_aware_if_multi_step(x_seq, v_init, v_threshold, v_offset, channel_dim: int, v_reset: Optional[float]):
+    """Step loop of neuron/integrate_and_fire.py:1125-1137 with the parameter broadcast of :879-895 (1-D parameters
+    lie along ``channel_dim`` of one time step, cast to the input's dtype).  Returns (spike_seq, v_seq)."""
+    def shaped(param):
+        param = torch.as_tensor(param).to(x_seq.dtype)
+        if param.dim() == 0:
+            return param
+        shape = [1] * (x_seq.dim() - 1)
+        shape[channel_dim] = param.numel()
+        return param.view(shape)
+
+    th, off = shaped(v_threshold), shaped(v_offset)
+    v, s_steps, v_steps = v_init, [], []
+    for t in range(x_seq.shape[0]):
+        s, v, _ = activation_aware_if_step(x_seq[t], v, th, off, v_reset, heaviside, False)
+        s_steps.append(s)
+        v_steps.append(v)
+    return torch.stack(s_steps), torch.stack(v_steps)
+
+
 # ------------------------------------------------------------------------------------------------
 # sequences
 # ------------------------------------------------------------------------------------------------

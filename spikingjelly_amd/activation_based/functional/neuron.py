@@ -35,6 +35,7 @@ __all__ = [
     "eif_step",
     "ilif_step",
     "stbif_step",
+    "activation_aware_if_step",
     "if_multi_step_hip",
     "lif_multi_step_hip",
     "plif_multi_step_hip",
@@ -43,6 +44,7 @@ __all__ = [
     "ilif_multi_step_hip",
     "stbif_multi_step_hip",
     "stbif_single_step_hip",
+    "activation_aware_if_multi_step_hip",
     "if_step_hip",
     "lif_step_hip",
     "plif_step_hip",
@@ -151,6 +153,19 @@ def stbif_step(x: torch.Tensor, q: torch.Tensor, acc_q: torch.Tensor, q_threshol
     q_next = torch.where(up, q_next - 1, q_next)
     q_next = torch.where(down, q_next + 1, q_next)
     return cur * q_threshold, q_next, acc_next, cur
+
+
+def activation_aware_if_step(x: torch.Tensor, v: torch.Tensor, v_threshold: torch.Tensor, v_offset: torch.Tensor,
+                             v_reset: Optional[float], surrogate_function: SurrogateFunction,
+                             detach_reset: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
+    """One step of an IF neuron that fires on ``h + v_offset >= v_threshold`` (reference :502-584); both parameters
+    are already broadcastable to ``x``.  Returns ``(spike, v_next)``."""
+    h = v + x
+    spike = surrogate_function(h + v_offset - v_threshold)
+    s = spike.detach() if detach_reset else spike
+    if v_reset is None:
+        return spike, h - s * v_threshold
+    return spike, s * v_reset + (1.0 - s) * h
 
 
 # ---- hip backend: whole sequence ----------------------------------------------------------------
@@ -423,6 +438,24 @@ def stbif_single_step_hip(x: torch.Tensor, q: torch.Tensor, acc_q: torch.Tensor,
     (:3250-3327)."""
     out, q2, acc2, cur, work = stbif_multi_step_hip(x.unsqueeze(0), q, acc_q, q_threshold, pos_max, neg_min)
     return out[0], q2, acc2, cur, work
+
+
+@torch.no_grad()
+def activation_aware_if_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, v_threshold: torch.Tensor,
+                                       v_offset: torch.Tensor, channel_size: int, inner_size: int,
+                                       v_reset: Optional[float], store_v_seq: bool = False
+                                       ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Multi-step activation-aware IF on the hip backend, inference only; signature and return of the reference's
+    ``activation_aware_if_multi_step_triton`` (:587-660).  ``v_threshold`` / ``v_offset`` are scalars or hold
+    ``channel_size`` values; channel ``(n // inner_size) % channel_size`` belongs to element ``n`` of a flattened
+    step."""
+    from ..hip_kernel import aaif_kernel
+
+    soft = v_reset is None
+    s, v_seq, v_last = aaif_kernel.hip_multistep_activation_aware_if(
+        x_seq.flatten(1), v.flatten(), v_threshold, v_offset, int(channel_size), int(inner_size),
+        0.0 if soft else float(v_reset), soft, store_v_seq, _hip_mode_flags(x_seq))
+    return _finish(x_seq, s, v_seq, v_last, store_v_seq)
 
 
 # ---- hip backend: one step (step_mode='s') --------------------------------------------------------

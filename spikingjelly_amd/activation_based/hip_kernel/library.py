@@ -46,6 +46,7 @@ EXPORTED_SYMBOLS = (
     "sjhip_ssa_forward",
     "sjhip_ssa_backward",
     "sjhip_stbif_forward",
+    "sjhip_aaif_forward",
     "sjhip_bit_pack",
     "sjhip_bit_unpack",
     "sjhip_set_tuning",
@@ -141,6 +142,12 @@ def load() -> ctypes.CDLL:
             c_int, c_uint32, c_int64, c_int64,
             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        ]
+        lib.sjhip_aaif_forward.restype = c_int
+        lib.sjhip_aaif_forward.argtypes = [
+            c_int, c_uint32, c_int64, c_int64, c_void_p, c_void_p,
+            c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_float,
+            c_void_p, c_void_p, c_void_p, c_void_p,
         ]
         lib.sjhip_bit_pack.restype = c_int
         lib.sjhip_bit_pack.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p]

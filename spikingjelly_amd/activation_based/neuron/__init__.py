@@ -1,3 +1,4 @@
+from .activation_aware_if import ActivationAwareIFNode
 from .base_node import BaseNode
 from .ilif import ILIFNode
 from .integrate_and_fire import IFNode
@@ -6,4 +7,4 @@ from .nonlinear_if import EIFNode, QIFNode
 from .plif import ParametricLIFNode
 from .spikezip import STBIFNeuron
 
-__all__ = ["BaseNode", "IFNode", "LIFNode", "ParametricLIFNode", "QIFNode", "EIFNode", "ILIFNode", "STBIFNeuron"]
+__all__ = ["BaseNode", "IFNode", "LIFNode", "ParametricLIFNode", "QIFNode", "EIFNode", "ILIFNode", "STBIFNeuron", "ActivationAwareIFNode"]

@@ -260,6 +260,27 @@ int sjhip_stbif_forward(int dtype, uint32_t flags, int64_t T, int64_t N, const v
                               q_final, acc_q_final, cur_output, work_flag, static_cast<hipStream_t>(stream));
 }
 
+int sjhip_aaif_forward(int dtype, uint32_t flags, int64_t T, int64_t N, const void *x_seq, const void *v_init,
+                       const float *v_threshold, int64_t threshold_count, const float *v_offset, int64_t offset_count,
+                       int64_t channel_size, int64_t inner_size, float v_reset, void *spike_seq, void *v_seq,
+                       void *v_last, void *stream) {
+  if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "aaif_forward: dtype %d", dtype);
+  if (flags & ~(SJHIP_FLAG_SOFT_RESET | SJHIP_FLAG_FP32_STATE | SJHIP_FLAG_V_INIT_BROADCAST))
+    return fail(SJHIP_ERR_INVALID, "aaif_forward: flags 0x%x", flags);
+  int rc = check_shape("aaif_forward", T, N);
+  if (rc != SJHIP_OK) return rc;
+  if (!x_seq || !v_init || !spike_seq || !v_threshold || !v_offset) return fail(SJHIP_ERR_INVALID, "aaif_forward: NULL tensor");
+  if (!v_seq && !v_last) return fail(SJHIP_ERR_INVALID, "aaif_forward: neither v_seq nor v_last given");
+  if (channel_size < 1 || inner_size < 1 || channel_size > N || inner_size > N)
+    return fail(SJHIP_ERR_INVALID, "aaif_forward: channel_size=%lld inner_size=%lld for N=%lld", (long long)channel_size,
+                (long long)inner_size, (long long)N);
+  if ((threshold_count != 1 && threshold_count != channel_size) || (offset_count != 1 && offset_count != channel_size))
+    return fail(SJHIP_ERR_INVALID, "aaif_forward: %lld thresholds and %lld offsets for %lld channels",
+                (long long)threshold_count, (long long)offset_count, (long long)channel_size);
+  return launch_aaif_forward(dtype, flags, T, N, x_seq, v_init, v_threshold, threshold_count, v_offset, offset_count,
+                             channel_size, inner_size, v_reset, spike_seq, v_seq, v_last, static_cast<hipStream_t>(stream));
+}
+
 int sjhip_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, void *stream) {
   if (n < 0) return fail(SJHIP_ERR_INVALID, "bit_pack: n=%lld", (long long)n);
   if (n == 0) return SJHIP_OK;

@@ -283,6 +283,10 @@ int launch_stbif_forward(int dtype, uint32_t flags, int64_t T, int64_t N, const 
                          const void *acc_q_init, const float *q_threshold, const float *pos_max, const float *neg_min,
                          void *out_seq, void *q_final, void *acc_q_final, void *cur_output, int32_t *work_flag,
                          hipStream_t stream);
+int launch_aaif_forward(int dtype, uint32_t flags, int64_t T, int64_t N, const void *x_seq, const void *v_init,
+                        const float *v_threshold, int64_t threshold_count, const float *v_offset, int64_t offset_count,
+                        int64_t channel_size, int64_t inner_size, float v_reset, void *spike_seq, void *v_seq,
+                        void *v_last, hipStream_t stream);
 int launch_backward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
                     const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
                     const void *h_seq, const void *v_init,

@@ -84,6 +84,17 @@ def test_argument_validation_without_a_device():
     assert rc == -1 and b"NULL tensor" in lib.sjhip_last_error()
     rc = lib.sjhip_stbif_forward(L.DTYPE_F32, 0, 0, 16, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, None, None)
     assert rc == -1 and b"T=0" in lib.sjhip_last_error()
+    aaif = lambda *a: lib.sjhip_aaif_forward(*a)
+    rc = aaif(L.DTYPE_F32, 0, 4, 16, 1, 1, 1, 3, 1, 1, 4, 2, 0.0, 1, None, 1, None)
+    assert rc == -1 and b"3 thresholds" in lib.sjhip_last_error()
+    rc = aaif(L.DTYPE_F32, 0, 4, 16, 1, 1, 1, 1, 1, 1, 0, 2, 0.0, 1, None, 1, None)
+    assert rc == -1 and b"channel_size=0" in lib.sjhip_last_error()
+    rc = aaif(L.DTYPE_F32, 0, 4, 16, 1, 1, 1, 1, 1, 1, 4, 2, 0.0, 1, None, None, None)
+    assert rc == -1 and b"v_seq" in lib.sjhip_last_error()
+    rc = aaif(L.DTYPE_F32, L.FLAG_DECAY_INPUT, 4, 16, 1, 1, 1, 1, 1, 1, 4, 2, 0.0, 1, None, 1, None)
+    assert rc == -1 and b"flags" in lib.sjhip_last_error()
+    rc = aaif(L.DTYPE_F32, 0, 4, 16, 1, 1, None, 1, 1, 1, 4, 2, 0.0, 1, None, 1, None)
+    assert rc == -1 and b"NULL" in lib.sjhip_last_error()
     assert lib.sjhip_bit_pack(L.DTYPE_F32, -1, 1, 1, None) == -1
     assert lib.sjhip_bit_pack(L.DTYPE_F32, 0, None, None, None) == 0
     assert lib.sjhip_plif_workspace_floats(L.DTYPE_F32, 1 << 20) >= (1 << 20) // 1024

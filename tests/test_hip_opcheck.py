@@ -71,6 +71,17 @@ def test_stbif_op():
     torch.library.opcheck(hip_multistep_stbif, (x, q, acc, *th, 0), test_utils=("test_schema", "test_faketensor"))
 
 
+def test_activation_aware_if_op():
+    from spikingjelly_amd.activation_based.hip_kernel.aaif_kernel import hip_multistep_activation_aware_if
+
+    x = seeded_randn((5, 48), 8, 0.3, 0.6).cuda()
+    v0 = torch.zeros(48, device="cuda")
+    th, off = torch.tensor([1.0, 1.5, 2.0], device="cuda"), torch.tensor(0.25, device="cuda")
+    for store in (False, True):
+        torch.library.opcheck(hip_multistep_activation_aware_if, (x, v0, th, off, 3, 4, 0.0, True, store, 0),
+                              test_utils=("test_schema", "test_faketensor"))
+
+
 def test_ssa_op():
     from spikingjelly_amd.activation_based.hip_kernel.attention_kernel import hip_ssa_forward
 

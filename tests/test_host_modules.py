@@ -461,3 +461,40 @@ def test_stbif_neuron_construction_and_torch_backend():
     assert node.is_work
     # a changed shape starts from fresh states
     assert node(torch.zeros(2, 5)).shape == (2, 5) and float(node.q.mean()) == 0.5
+
+
+# ---- activation-aware IF (reference neuron/integrate_and_fire.py:536-1150, test_activation_aware_ifnode.py) -----------
+def test_activation_aware_if_node_on_the_torch_backend():
+    for kw in (dict(v_threshold=torch.ones(2, 2)), dict(v_threshold=torch.tensor([1.0, -1.0])), dict(v_offset=float("inf")),
+               dict(v_reset=1), dict(channel_dim=1.0), dict(backend="cupy"), dict(detach_reset=1), dict(store_v_seq=1)):
+        with pytest.raises(ValueError):
+            neuron.ActivationAwareIFNode(**kw)
+    node = neuron.ActivationAwareIFNode(v_threshold=torch.tensor([1.0, 2.0]), v_offset=torch.tensor([0.0, 0.5]))
+    assert node.supported_backends == ("torch",) and "v_threshold" in node.state_dict()
+    node.step_mode = "m"
+    assert node.supported_backends == ("torch", "hip")
+    with pytest.raises(ValueError, match="channels"):
+        node(torch.zeros(2, 3, 5))
+
+    # the reference tests' literal inputs (test_activation_aware_ifnode.py:253-352) against the oracle
+    x = torch.tensor([[[0.8, 1.0], [1.2, 0.2]], [[0.6, 0.2], [0.4, 1.4]], [[0.3, 0.9], [0.1, 0.2]]])
+    node = neuron.ActivationAwareIFNode(v_threshold=1.5, v_offset=0.25, step_mode="m")
+    es, ev = no.activation_aware_if_multi_step(x, torch.zeros(2, 2), 1.5, 0.25, -1, None)
+    assert torch.equal(node(x), es) and torch.equal(node.v, ev[-1])
+    x = torch.tensor([[[1.1, 1.5]], [[0.2, 0.7]], [[0.8, 0.1]]])
+    node = neuron.ActivationAwareIFNode(v_threshold=torch.tensor([1.0, 2.0]), v_reset=0.25, step_mode="m", store_v_seq=True)
+    es, ev = no.activation_aware_if_multi_step(x, torch.full((1, 2), 0.25), torch.tensor([1.0, 2.0]), 0.0, -1, 0.25)
+    assert torch.equal(node(x), es) and torch.equal(node.v_seq, ev)
+    node.store_v_seq = False
+    assert node.v_seq is None
+    # shape change restarts from v_reset; reset restores the scalar
+    node = neuron.ActivationAwareIFNode(v_threshold=1.0, v_reset=0.25)
+    node(torch.tensor([[1.1]]))
+    assert torch.equal(node(torch.tensor([[0.3, 0.3]])), torch.zeros(1, 2)) and torch.equal(node.v, torch.full((1, 2), 0.55))
+    node.reset()
+    assert node.v == 0.25
+    # gradients flow on the torch backend
+    node = neuron.ActivationAwareIFNode(v_threshold=torch.tensor([1.0, 2.0]), v_offset=torch.tensor([0.0, 0.25]))
+    xg = torch.tensor([[0.9, 1.8]], requires_grad=True)
+    node(xg).sum().backward()
+    assert xg.grad is not None and bool((xg.grad != 0).all())

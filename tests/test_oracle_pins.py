@@ -636,3 +636,67 @@ def test_eif_autograd_matches_finite_differences_of_the_smooth_network(v_reset):
     vp[2] += eps
     vm[2] -= eps
     assert (loss(x, vp) - loss(x, vm)) / (2 * eps) == pytest.approx(float(ref["grad_v_init"][2]), rel=1e-6, abs=1e-8)
+
+
+# ------------------------------------------------------------------------------------------------
+# activation-aware IF (functional/neuron.py:577-584)
+# ------------------------------------------------------------------------------------------------
+def _aaif_by_hand(x_seq, threshold, offset, v_reset):
+    """Plain Python floats, one neuron at a time; x_seq [T][n], threshold / offset one value per neuron."""
+    T, n = len(x_seq), len(x_seq[0])
+    v = [0.0 if v_reset is None else v_reset] * n
+    spikes, volts = [], []
+    for t in range(T):
+        row_s, row_v = [], []
+        for i in range(n):
+            h = v[i] + x_seq[t][i]
+            fired = 1.0 if h + offset[i] >= threshold[i] else 0.0
+            v[i] = h - fired * threshold[i] if v_reset is None else (v_reset if fired else h)
+            row_s.append(fired)
+            row_v.append(v[i])
+        spikes.append(row_s)
+        volts.append(row_v)
+    return spikes, volts
+
+
+def test_activation_aware_if_on_the_reference_tests_literal_inputs():
+    """Inputs of the reference's test_activation_aware_ifnode.py:253-352 against a neuron-by-neuron loop in Python
+    floats (no value comes within 0.04 of a threshold, so fp32 and double agree on every spike)."""
+    x = torch.tensor([[[0.8, 1.0], [1.2, 0.2]], [[0.6, 0.2], [0.4, 1.4]], [[0.3, 0.9], [0.1, 0.2]]])
+    s, v = no.activation_aware_if_multi_step(x, torch.zeros(2, 2), 1.5, 0.25, -1, None)
+    es, ev = _aaif_by_hand(x.flatten(1).tolist(), [1.5] * 4, [0.25] * 4, None)
+    assert s.flatten(1).tolist() == es and float(s.sum()) > 0
+    torch.testing.assert_close(v.flatten(1), torch.tensor(ev))
+
+    x = torch.tensor([[[0.6, 1.0, 2.4], [1.1, 1.3, 1.0]], [[0.5, 0.4, 0.7], [0.2, 0.4, 1.3]]])
+    th, off = [1.0, 1.5, 2.0], [0.0, 0.25, -0.25]
+    s, v = no.activation_aware_if_multi_step(x, torch.zeros(2, 3), torch.tensor(th), torch.tensor(off), -1, None)
+    es, ev = _aaif_by_hand(x.flatten(1).tolist(), th * 2, off * 2, None)
+    assert s.flatten(1).tolist() == es and 0 < float(s.sum()) < s.numel()
+
+    x = torch.tensor([[[1.1, 1.5]], [[0.2, 0.7]], [[0.8, 0.1]]])
+    s, v = no.activation_aware_if_multi_step(x, torch.full((1, 2), 0.25), torch.tensor([1.0, 2.0]), 0.0, -1, 0.25)
+    es, ev = _aaif_by_hand(x.flatten(1).tolist(), [1.0, 2.0], [0.0, 0.0], 0.25)
+    assert s.flatten(1).tolist() == es
+    torch.testing.assert_close(v.flatten(1), torch.tensor(ev))
+
+
+def test_activation_aware_if_reduces_to_if():
+    """Zero offset and a scalar threshold is the IF neuron, bit for bit; with a hard reset (where the threshold does
+    not enter the reset) an offset o is the IF neuron with threshold theta - o on dyadic values; a 1-D parameter along
+    channel_dim 0 of an [C, H, W] step treats every channel as its own scalar neuron."""
+    x = seeded_randn((10, 3, 8, 8), 95, 0.3, 0.6)
+    v0 = torch.zeros(3, 8, 8)
+    for v_reset in (None, 0.0, -0.25):
+        s, v = no.activation_aware_if_multi_step(x, v0 if v_reset is None else torch.full_like(v0, v_reset), 0.75, 0.0, 0, v_reset)
+        es, ev, _ = no.multi_step("if", x, v0 if v_reset is None else torch.full_like(v0, v_reset), None, True, 0.75, v_reset)
+        assert torch.equal(s, es) and torch.equal(v, ev)
+    xd = torch.round(x * 64) / 64
+    s, v = no.activation_aware_if_multi_step(xd, v0, 1.0, 0.25, 0, 0.0)
+    es, ev, _ = no.multi_step("if", xd, v0, None, True, 0.75, 0.0)
+    assert torch.equal(s, es) and torch.equal(v, ev)
+    th = torch.tensor([0.5, 1.0, 1.5])
+    s, v = no.activation_aware_if_multi_step(x, v0, th, 0.0, 0, None)
+    for c in range(3):
+        es, ev, _ = no.multi_step("if", x[:, c], v0[c], None, True, float(th[c]), None)
+        assert torch.equal(s[:, c], es) and torch.equal(v[:, c], ev)
