@@ -267,17 +267,22 @@ def other_workload(args) -> int:
         sf, sb = _kernel_ms(L, L.KC_SSA_FORWARD), _kernel_ms(L, L.KC_SSA_BACKWARD)
         cph = D // H
         probs = T * B * H
-        flops_f = probs * (2 * cph * cph * tokens + 2 * cph * cph * tokens)
-        bytes_f = T * B * D * tokens * 4 * (3 + 1)  # qkv read + out write, fp32 storage
+        n = T * B * D * tokens
+        product = probs * 2 * cph * cph * tokens  # flops of one [cph, L] x [L, cph] (or [cph, cph] x [cph, L]) product
+        # the qkv spikes travel bit-packed between the LIF and the contraction: 3 n / 8 bytes; fp32 elsewhere
+        bytes_f = 3 * n // 8 + 4 * n              # bits read, out written
+        bytes_b = 3 * n // 8 + 4 * n + 12 * n     # bits and grad_out read, dq / dk / dv written
         _emit(args, "tokens/sec spiking self-attention block fwd+bwd, T=4 B=64 N=196 D=384 12 heads, 1 MI355X",
               "tokens/s", T * B * tokens / (elapsed / args.steps), elapsed, "bf16",
               {"workload": "configs[4]: SpikingSelfAttention(384, 12, backend='hip'), x [4,64,384,196] fp32 ~N(0,1), "
                            "channels per head = 32 (dim // heads, as the reference computes it)"},
-              {"bound": "hbm", "achieved": bytes_f / (sf * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-               "frac": bytes_f / (sf * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "ssa_forward",
-               "kernel_ms": sf, "algorithmic_bytes": bytes_f, "ssa_forward_TFLOPs": flops_f / (sf * 1e-3) / 1e12,
-               "ssa_backward_ms": sb, "lif_forward_ms": _kernel_ms(L, L.KC_FORWARD),
-               "lif_backward_ms": _kernel_ms(L, L.KC_BACKWARD)})
+              {"bound": "hbm", "achieved": bytes_b / (sb * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+               "frac": bytes_b / (sb * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "ssa_backward",
+               "kernel_ms": sb, "algorithmic_bytes": bytes_b,
+               "ssa_backward_fp32_mfma_TFLOPs": 4 * product / (sb * 1e-3) / 1e12,
+               "ssa_forward_ms": sf, "ssa_forward_GBs": bytes_f / (sf * 1e-3) / 1e9,
+               "ssa_forward_TFLOPs": 2 * product / (sf * 1e-3) / 1e12,
+               "lif_forward_ms": _kernel_ms(L, L.KC_FORWARD), "lif_backward_ms": _kernel_ms(L, L.KC_BACKWARD)})
         return 0
     raise SystemExit(f"unknown workload {args.workload}")
 

@@ -295,6 +295,21 @@ int sjhip_ssa_backward(int dtype, int64_t samples, int heads, int channels_per_h
                        const void *qkv, const void *grad_out, void *grad_qkv, void *stream);
 
 /*
+ * The same contraction with bit-packed operands: the fused form of a kernel-backend LIF (bit-packed spike output,
+ * sjhip_neuron_forward_packed) feeding the contraction, so the dense q / k / v spike tensor is never written or
+ * read.  No counterpart in the reference, whose attention takes dense spike tensors (layer/attention.py:370-383).
+ *   qkv_bits  [(samples*3*heads*channels_per_head*tokens)/8] bytes: the flattened qkv tensor packed LSB first
+ *             (byte j bit i = element 8 j + i, the layout of sjhip_bit_pack)
+ *   dtype     of out / grad_out / grad_qkv
+ * channels_per_head * tokens must be a multiple of 8 so that every head's tile starts on a byte
+ * (SJHIP_ERR_UNSUPPORTED otherwise); results equal the dense entry points' bit for bit.
+ */
+int sjhip_ssa_forward_packed(int dtype, int64_t samples, int heads, int channels_per_head, int64_t tokens, float scale,
+                             const uint8_t *qkv_bits, void *out, void *stream);
+int sjhip_ssa_backward_packed(int dtype, int64_t samples, int heads, int channels_per_head, int64_t tokens, float scale,
+                              const uint8_t *qkv_bits, const void *grad_out, void *grad_qkv, void *stream);
+
+/*
  * Launch tuning (process-wide, read at launch).  Keys: "fwd_block" / "bwd_block" = work-items per
  * block (64, 128, 256 or 512); "fwd_blocks_per_cu" / "bwd_blocks_per_cu" = cap on resident blocks per
  * compute unit (0 = none, else 2..64; enforced through a dynamic-LDS request), and

@@ -85,3 +85,80 @@ def _backward(ctx, grad_out):
 
 
 torch.library.register_autograd("sj::hip_ssa_forward", _backward, setup_context=_setup_context)
+
+
+# =================================================================================================
+# LIF -> contraction with the spikes kept bit-packed in between
+# =================================================================================================
+def ssa_packed_supported(dtype: torch.dtype, channels_per_head: int, tokens: int) -> bool:
+    """The packed-operand contraction needs every head's tile to start on a byte."""
+    return ssa_supported(dtype, channels_per_head, tokens) and (channels_per_head * tokens) % 8 == 0
+
+
+def _ssa_packed(bits: torch.Tensor, grad_out, dtype: torch.dtype, samples: int, heads: int, cph: int, tokens: int,
+                scale: float) -> torch.Tensor:
+    """Forward (``grad_out is None``: returns out) or backward (returns grad_qkv) of the contraction on bit-packed q/k/v."""
+    lib = L.load()
+    with torch.cuda.device(bits.device):
+        if grad_out is None:
+            result = torch.empty((samples, heads, cph, tokens), dtype=dtype, device=bits.device)
+            rc = lib.sjhip_ssa_forward_packed(L.dtype_id(dtype), samples, heads, cph, tokens, scale, bits.data_ptr(),
+                                              result.data_ptr(), L.current_stream_ptr(bits.device))
+        else:
+            grad_out = grad_out.to(dtype).contiguous()
+            result = torch.empty((samples, 3, heads, cph, tokens), dtype=dtype, device=bits.device)
+            rc = lib.sjhip_ssa_backward_packed(L.dtype_id(dtype), samples, heads, cph, tokens, scale, bits.data_ptr(),
+                                               grad_out.data_ptr(), result.data_ptr(), L.current_stream_ptr(bits.device))
+    L.check(rc, "ssa_forward_packed" if grad_out is None else "ssa_backward_packed")
+    return result
+
+
+class _LifSsa(torch.autograd.Function):
+    """``out = scale (V K^T) Q`` of the spikes a multi-step LIF fires from ``x_seq``, with those spikes existing only
+    bit-packed: the LIF forward writes bits (``sjhip_neuron_forward_packed``), the contraction reads bits, and in the
+    backward the contraction writes the dense spike gradient that the replaying LIF backward consumes.  Saves
+    ``x_seq``, ``v_init`` and the bits (1/32 of the fp32 spike tensor)."""
+
+    @staticmethod
+    def forward(x_seq, v_init, spec):
+        from . import neuron_kernel as K
+
+        tau, v_th, v_reset, flags, _, _, samples, heads, cph, tokens, scale = spec
+        bits, _, v_last = K._run_forward_packed(L.NEURON_LIF, x_seq, v_init, None, tau, v_th, v_reset, flags, False)
+        out = _ssa_packed(bits, None, x_seq.dtype, samples, heads, cph, tokens, scale)
+        return out, v_last, bits
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        x_seq, v_init, spec = inputs
+        ctx.spec = spec
+        ctx.save_for_backward(x_seq, v_init, output[2])
+        ctx.mark_non_differentiable(output[2])
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, grad_out, grad_v_last, grad_bits):
+        from . import neuron_kernel as K
+
+        del grad_bits
+        tau, v_th, v_reset, flags, sg_id, sg_alpha, samples, heads, cph, tokens, scale = ctx.spec
+        x_seq, v_init, bits = ctx.saved_tensors
+        grad_spikes = None
+        if grad_out is not None:
+            grad_spikes = _ssa_packed(bits, grad_out, x_seq.dtype, samples, heads, cph, tokens, scale).view(x_seq.shape)
+        need = bool(ctx.needs_input_grad[1])
+        gx, gvi, _ = K._run_backward(L.NEURON_LIF, grad_spikes, None, grad_v_last, None, x_seq, v_init, None, tau, v_th,
+                                     v_reset, flags, sg_id, sg_alpha, need)
+        return gx, (gvi if need else None), None
+
+
+def lif_ssa_fused(x_seq: torch.Tensor, v_init: torch.Tensor, tau: float, v_th: float, v_reset: float, flags: int,
+                  sg_id: int, sg_alpha: float, heads: int, channels_per_head: int, tokens: int, scale: float
+                  ) -> tuple[torch.Tensor, torch.Tensor]:
+    """``x_seq`` is ``[T, N]`` with ``N = B * 3 * heads * channels_per_head * tokens``, ``v_init`` ``[N]``.  Returns
+    ``(out [T*B, heads, channels_per_head, tokens], v_last [N])``.  The caller has checked ``ssa_packed_supported``,
+    ``N % 8 == 0`` and that the replay backward serves the shape."""
+    samples = x_seq.shape[0] * (x_seq.shape[1] // (3 * heads * channels_per_head * tokens))
+    spec = (tau, v_th, v_reset, flags, sg_id, sg_alpha, samples, heads, channels_per_head, tokens, scale)
+    out, v_last, _ = _LifSsa.apply(x_seq, v_init, spec)
+    return out, v_last

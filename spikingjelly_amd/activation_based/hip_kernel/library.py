@@ -45,6 +45,8 @@ EXPORTED_SYMBOLS = (
     "sjhip_ssa_supported",
     "sjhip_ssa_forward",
     "sjhip_ssa_backward",
+    "sjhip_ssa_forward_packed",
+    "sjhip_ssa_backward_packed",
     "sjhip_stbif_forward",
     "sjhip_aaif_forward",
     "sjhip_bit_pack",
@@ -149,6 +151,12 @@ def load() -> ctypes.CDLL:
             c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_float,
             c_void_p, c_void_p, c_void_p, c_void_p,
         ]
+        lib.sjhip_ssa_forward_packed.restype = c_int
+        lib.sjhip_ssa_forward_packed.argtypes = [c_int, c_int64, c_int, c_int, c_int64, c_float, c_void_p, c_void_p,
+                                                 c_void_p]
+        lib.sjhip_ssa_backward_packed.restype = c_int
+        lib.sjhip_ssa_backward_packed.argtypes = [c_int, c_int64, c_int, c_int, c_int64, c_float, c_void_p, c_void_p,
+                                                  c_void_p, c_void_p]
         lib.sjhip_bit_pack.restype = c_int
         lib.sjhip_bit_pack.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p]
         lib.sjhip_bit_unpack.restype = c_int

@@ -65,19 +65,53 @@ class SpikingSelfAttention(nn.Module, base.MultiStepModule):
         out = hip_ssa_forward(qkv.flatten(0, 1), scale)
         return out.view(T, N, *out.shape[1:])
 
+    def _lif_ssa_fused(self, pre: torch.Tensor):
+        """``qkv_lif`` and the contraction as one step whose spikes exist only bit-packed (1/32 of the fp32 spike
+        tensor: the LIF writes bits, the contraction reads bits, the backward keeps bits).  Returns ``None`` when the
+        shape, the mode or the state does not allow it; the two-operator path then runs.  Results are identical."""
+        from ..functional import neuron as F
+        from ..hip_kernel import attention_kernel as A
+        from ..hip_kernel import neuron_kernel as K
+        from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
+
+        node = self.qkv_lif
+        T, N, C3, L = pre.shape
+        cph = C3 // 3 // self.num_heads
+        if (torch.compiler.is_compiling() or node.store_v_seq or not pre.is_cuda
+                or not A.ssa_packed_supported(pre.dtype, cph, L) or (N * C3 * L) % 8 != 0):
+            return None
+        x2 = pre.flatten(1)
+        need_grad = torch.is_grad_enabled() and pre.requires_grad
+        if need_grad and not F._hip_recompute(x2):
+            return None  # the fused backward replays the LIF forward
+        node._check_hip_surrogate()
+        (v,) = node.materialize_states((pre,), (node.v,), "m")
+        if need_grad and v.requires_grad:
+            return None
+        soft = node.v_reset is None
+        flags = K._flags(soft, node.detach_reset, node.decay_input, F._hip_mode_flags(pre))
+        sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(node.surrogate_function) if need_grad else (0, 0.0)
+        with torch.set_grad_enabled(need_grad):
+            out, v_last = A.lif_ssa_fused(x2, v.flatten(), float(node.tau), node.v_threshold, 0.0 if soft else float(node.v_reset),
+                                          flags, sg_id, sg_alpha, self.num_heads, cph, L, self.scale)
+        node.v = v_last.reshape(pre.shape[1:])
+        return out.view(T, N, self.num_heads, cph, L)
+
     def forward(self, x_seq: torch.Tensor):
         if x_seq.ndim != 4:
             raise ValueError(f"expected 4D input with shape [T, N, C, L], but got input with shape {x_seq.shape}")
         T, N, C, L = x_seq.shape
-        qkv = self.qkv_lif(self.qkv_conv_bn(x_seq))  # [T, N, 3*C, L]
-        local_dim = qkv.shape[2] // 3
+        pre = self.qkv_conv_bn(x_seq)  # [T, N, 3*C, L]
+        local_dim = pre.shape[2] // 3
         if local_dim % self.num_heads != 0:
             raise ValueError(f"local qkv dim {local_dim} is not divisible by num_heads={self.num_heads}.")
-        qkv = qkv.reshape(T, N, 3, self.num_heads, local_dim // self.num_heads, L)
-        if self.backend == "hip":
-            x_seq = self._ssa_kernel_hip(qkv, self.scale)
-        else:
-            x_seq = self._ssa_kernel_torch(qkv, self.scale)
+        x_seq = self._lif_ssa_fused(pre) if self.backend == "hip" else None
+        if x_seq is None:
+            qkv = self.qkv_lif(pre).reshape(T, N, 3, self.num_heads, local_dim // self.num_heads, L)
+            if self.backend == "hip":
+                x_seq = self._ssa_kernel_hip(qkv, self.scale)
+            else:
+                x_seq = self._ssa_kernel_torch(qkv, self.scale)
         x_seq = self.attn_lif(x_seq).reshape(T, N, local_dim, L)
         return self.proj_lif(self.proj_conv_bn(x_seq))  # [T, N, C, L]
 

@@ -302,14 +302,28 @@ int sjhip_ssa_supported(int dtype, int channels_per_head, int64_t tokens) {
 int sjhip_ssa_forward(int dtype, int64_t samples, int heads, int channels_per_head, int64_t tokens, float scale,
                       const void *qkv, void *out, void *stream) {
   if (!qkv || !out) return fail(SJHIP_ERR_INVALID, "ssa_forward: NULL tensor");
-  return launch_ssa(false, dtype, samples, heads, channels_per_head, tokens, scale, qkv, nullptr, out, nullptr,
+  return launch_ssa(false, dtype, samples, heads, channels_per_head, tokens, scale, qkv, nullptr, nullptr, out, nullptr,
                     static_cast<hipStream_t>(stream));
+}
+
+int sjhip_ssa_forward_packed(int dtype, int64_t samples, int heads, int channels_per_head, int64_t tokens, float scale,
+                             const uint8_t *qkv_bits, void *out, void *stream) {
+  if (!qkv_bits || !out) return fail(SJHIP_ERR_INVALID, "ssa_forward_packed: NULL tensor");
+  return launch_ssa(false, dtype, samples, heads, channels_per_head, tokens, scale, nullptr, qkv_bits, nullptr, out, nullptr,
+                    static_cast<hipStream_t>(stream));
+}
+
+int sjhip_ssa_backward_packed(int dtype, int64_t samples, int heads, int channels_per_head, int64_t tokens, float scale,
+                              const uint8_t *qkv_bits, const void *grad_out, void *grad_qkv, void *stream) {
+  if (!qkv_bits || !grad_out || !grad_qkv) return fail(SJHIP_ERR_INVALID, "ssa_backward_packed: NULL tensor");
+  return launch_ssa(true, dtype, samples, heads, channels_per_head, tokens, scale, nullptr, qkv_bits, grad_out, nullptr,
+                    grad_qkv, static_cast<hipStream_t>(stream));
 }
 
 int sjhip_ssa_backward(int dtype, int64_t samples, int heads, int channels_per_head, int64_t tokens, float scale,
                        const void *qkv, const void *grad_out, void *grad_qkv, void *stream) {
   if (!qkv || !grad_out || !grad_qkv) return fail(SJHIP_ERR_INVALID, "ssa_backward: NULL tensor");
-  return launch_ssa(true, dtype, samples, heads, channels_per_head, tokens, scale, qkv, grad_out, nullptr, grad_qkv,
+  return launch_ssa(true, dtype, samples, heads, channels_per_head, tokens, scale, qkv, nullptr, grad_out, nullptr, grad_qkv,
                     static_cast<hipStream_t>(stream));
 }
 

@@ -305,7 +305,7 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
 int64_t plif_blocks(int dtype, int64_t N);
 bool ssa_supported(int dtype, int cph, int64_t L);
 int launch_ssa(bool backward, int dtype, int64_t samples, int heads, int cph, int64_t L, float scale, const void *qkv,
-               const void *grad_out, void *out, void *grad_qkv, hipStream_t stream);
+               const uint8_t *qkv_bits, const void *grad_out, void *out, void *grad_qkv, hipStream_t stream);
 int launch_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, hipStream_t stream);
 int launch_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, hipStream_t stream);
 

@@ -47,6 +47,7 @@ constexpr int kSsaThreads = 256;
 constexpr int kSsaWaves = kSsaThreads / 64;
 
 struct SsaArgs {
+  const uint8_t *qkv_bits;  // when set, the spikes come bit-packed (LSB first over the flattened tensor) and qkv is unused
   const void *qkv;
   const void *grad_out;
   void *out;
@@ -160,6 +161,95 @@ __device__ __forceinline__ void stage_tiles(const typename Io<S>::elem_t *const 
   }
 }
 
+// Bit-packed spike tiles -> LDS byte tiles.  The flattened qkv tensor is packed LSB first (byte j bit i = element
+// 8 j + i, what bit_pack and the packed neuron forward write); a [cph, L] tile whose element count is a multiple of 8
+// starts on a byte and is cph L / 8 bytes long, 32 times less to fetch than fp32 spikes.  A byte's eight elements may
+// straddle a row boundary of the tile (L need not be a multiple of 8).
+template <int NS>
+__device__ __forceinline__ void stage_bits(const uint8_t *const (&src)[NS], uint8_t *const (&dst)[NS], int cph,
+                                           int rows_pad, int L, int Lb) {
+  const int tid = threadIdx.x;
+  const int nbytes = cph * L / 8;
+  for (int b = tid; b < nbytes; b += kSsaThreads) {
+    uint32_t w[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) w[s] = src[s][b];
+    if ((L & 3) == 0) {
+      // four elements never straddle a row and land on a 4-byte boundary: one 32-bit store per nibble.  The product
+      // copies bit i of the nibble to bit 8 i (and to other positions the mask drops; no two copies collide).
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int e = 8 * b + 4 * half;
+        const int r = e / L, c = e - r * L;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+          *reinterpret_cast<uint32_t *>(dst[s] + r * Lb + c) = (((w[s] >> (4 * half)) & 15u) * 0x00204081u) & 0x01010101u;
+      }
+    } else {
+      int r = (8 * b) / L, c = 8 * b - r * L;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int s = 0; s < NS; ++s) dst[s][r * Lb + c] = (uint8_t)((w[s] >> i) & 1u);
+        if (++c == L) { c = 0; ++r; }
+      }
+    }
+  }
+  const int mb = Lb - L;
+  for (int i = tid; i < cph * mb; i += kSsaThreads) {
+    const int r = i / mb, c = L + (i - r * mb);
+#pragma unroll
+    for (int s = 0; s < NS; ++s) dst[s][r * Lb + c] = 0;
+  }
+  for (int i = tid; i < (rows_pad - cph) * (Lb / 4); i += kSsaThreads) {
+#pragma unroll
+    for (int s = 0; s < NS; ++s) reinterpret_cast<uint32_t *>(dst[s] + cph * Lb)[i] = 0u;
+  }
+}
+
+// The grad_out tile alone -> fp32 LDS tile [rows_pad][Lq], zero-padded (the packed backward stages its spikes apart).
+template <typename S>
+__device__ __forceinline__ void stage_grad_out(const typename Io<S>::elem_t *do_src, float *do_dst, int cph, int rows_pad,
+                                               int L, int Lq, bool vec) {
+  typedef typename Io<S>::quad_t Q;
+  const int tid = threadIdx.x;
+  if (vec) {
+    const int G = cph * L / 4;
+    constexpr int UN = 4;
+    for (int g0 = tid; g0 < G; g0 += kSsaThreads * UN) {
+      Q buf[UN];
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int g = g0 + u * kSsaThreads;
+        if (g < G) buf[u] = reinterpret_cast<const Q *>(do_src)[g];
+      }
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int g = g0 + u * kSsaThreads;
+        if (g < G) {
+          const int r = (4 * g) / L, c = 4 * g - r * L;
+          float f[4];
+          Io<S>::unpack(buf[u], f);
+          f32x4 w; w.x = f[0]; w.y = f[1]; w.z = f[2]; w.w = f[3];
+          *reinterpret_cast<f32x4 *>(do_dst + r * Lq + c) = w;
+        }
+      }
+    }
+  } else {
+    const int n = cph * L;
+    for (int i = tid; i < n; i += kSsaThreads) {
+      const int r = i / L, c = i - r * L;
+      do_dst[r * Lq + c] = Io<S>::get(do_src, i);
+    }
+  }
+  const int mq = Lq - L;
+  for (int i = tid; i < cph * mq; i += kSsaThreads) {
+    const int r = i / mq, c = L + (i - r * mq);
+    do_dst[r * Lq + c] = 0.0f;
+  }
+  for (int i = tid; i < (rows_pad - cph) * Lq; i += kSsaThreads) do_dst[cph * Lq + i] = 0.0f;
+}
+
 // 32x32 block of  A_rows B_rows^T  over the token axis: rows ra.. of tile `a` against rows rb.. of tile `b`
 __device__ __forceinline__ i32x16 spike_gram(const uint8_t *a, int ra, const uint8_t *b, int rb, int Lb, int lane) {
   const uint8_t *ap = a + (ra + (lane & 31)) * Lb + 16 * (lane >> 5);
@@ -189,11 +279,19 @@ __global__ void __launch_bounds__(kSsaThreads) ssa_forward_kernel(const SsaArgs 
   const int64_t tile = (int64_t)cph * L;
   const E *qkv = static_cast<const E *>(a.qkv);
   {
-    const E *const src[3] = {qkv + ((sample * 3 + 0) * a.heads + head) * tile,
-                             qkv + ((sample * 3 + 1) * a.heads + head) * tile,
-                             qkv + ((sample * 3 + 2) * a.heads + head) * tile};
     uint8_t *const dst[3] = {q_lds, k_lds, v_lds};
-    stage_tiles<S, 3, false, 4>(src, dst, nullptr, nullptr, cph, CPH, L, Lb, 0, a.vec != 0);
+    if (a.qkv_bits) {
+      const int64_t tb = tile / 8;
+      const uint8_t *const src[3] = {a.qkv_bits + ((sample * 3 + 0) * a.heads + head) * tb,
+                                     a.qkv_bits + ((sample * 3 + 1) * a.heads + head) * tb,
+                                     a.qkv_bits + ((sample * 3 + 2) * a.heads + head) * tb};
+      stage_bits<3>(src, dst, cph, CPH, L, Lb);
+    } else {
+      const E *const src[3] = {qkv + ((sample * 3 + 0) * a.heads + head) * tile,
+                               qkv + ((sample * 3 + 1) * a.heads + head) * tile,
+                               qkv + ((sample * 3 + 2) * a.heads + head) * tile};
+      stage_tiles<S, 3, false, 4>(src, dst, nullptr, nullptr, cph, CPH, L, Lb, 0, a.vec != 0);
+    }
   }
   __syncthreads();
 
@@ -267,10 +365,16 @@ __global__ void __launch_bounds__(kSsaThreads, MC == 1 ? 3 : 1) ssa_backward_ker
   const int64_t koff = ((sample * 3 + 1) * a.heads + head) * tile;
   const int64_t voff = ((sample * 3 + 2) * a.heads + head) * tile;
   {
-    const E *const src[3] = {qkv + qoff, qkv + koff, qkv + voff};
     uint8_t *const dst[3] = {q_lds, k_lds, v_lds};
-    stage_tiles<S, 3, true, 2>(src, dst, static_cast<const E *>(a.grad_out) + p * tile, do_lds, cph, CPH, L, Lb, Lq,
-                               a.vec != 0);
+    if (a.qkv_bits) {
+      const uint8_t *const src[3] = {a.qkv_bits + qoff / 8, a.qkv_bits + koff / 8, a.qkv_bits + voff / 8};
+      stage_grad_out<S>(static_cast<const E *>(a.grad_out) + p * tile, do_lds, cph, CPH, L, Lq, a.vec != 0);
+      stage_bits<3>(src, dst, cph, CPH, L, Lb);
+    } else {
+      const E *const src[3] = {qkv + qoff, qkv + koff, qkv + voff};
+      stage_tiles<S, 3, true, 2>(src, dst, static_cast<const E *>(a.grad_out) + p * tile, do_lds, cph, CPH, L, Lb, Lq,
+                                 a.vec != 0);
+    }
   }
   __syncthreads();
 
@@ -403,19 +507,23 @@ bool ssa_supported(int dtype, int cph, int64_t L) {
 }
 
 int launch_ssa(bool backward, int dtype, int64_t samples, int heads, int cph, int64_t L, float scale, const void *qkv,
-               const void *grad_out, void *out, void *grad_qkv, hipStream_t stream) {
+               const uint8_t *qkv_bits, const void *grad_out, void *out, void *grad_qkv, hipStream_t stream) {
   if (!ssa_supported(dtype, cph, L))
     return fail(SJHIP_ERR_UNSUPPORTED, "ssa: dtype %d, %d channels per head, %lld tokens is not supported "
                 "(needs at most 64 channels per head, at most 256 tokens, and the tiles of one head fitting in LDS)", dtype, cph, (long long)L);
   if (samples < 1 || heads < 1 || samples * heads > 0x7fffffffLL)
     return fail(SJHIP_ERR_INVALID, "ssa: samples=%lld heads=%d", (long long)samples, heads);
+  if (qkv_bits && ((int64_t)cph * L) % 8 != 0)
+    return fail(SJHIP_ERR_UNSUPPORTED, "ssa(packed): %d channels x %lld tokens is not a multiple of 8, a tile would not start on a byte",
+                cph, (long long)L);
   SsaArgs a;
+  a.qkv_bits = qkv_bits;
   a.qkv = qkv; a.grad_out = grad_out; a.out = out; a.grad_qkv = grad_qkv;
   a.problems = samples * heads; a.heads = heads; a.cph = cph; a.L = (int)L;
   a.Lb = lds_row_bytes((int)L); a.Lq = lds_row_f32((int)L); a.scale = scale;
   // four elements per access need every tile base on a four-element boundary
   const uintptr_t quad = dtype == SJHIP_F32 ? 15u : 7u;
-  a.vec = (L % 4 == 0) && (reinterpret_cast<uintptr_t>(qkv) & quad) == 0 &&
+  a.vec = (L % 4 == 0) && (qkv_bits != nullptr || (reinterpret_cast<uintptr_t>(qkv) & quad) == 0) &&
           (grad_out == nullptr || (reinterpret_cast<uintptr_t>(grad_out) & quad) == 0);
   ProfileScope prof(backward ? KC_SSA_BACKWARD : KC_SSA_FORWARD, stream);
   switch (dtype) {

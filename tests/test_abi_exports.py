@@ -95,6 +95,12 @@ def test_argument_validation_without_a_device():
     assert rc == -1 and b"flags" in lib.sjhip_last_error()
     rc = aaif(L.DTYPE_F32, 0, 4, 16, 1, 1, None, 1, 1, 1, 4, 2, 0.0, 1, None, 1, None)
     assert rc == -1 and b"NULL" in lib.sjhip_last_error()
+    rc = lib.sjhip_ssa_forward_packed(L.DTYPE_F32, 4, 2, 3, 5, 0.125, 1, 1, None)
+    assert rc == -2 and b"multiple of 8" in lib.sjhip_last_error()
+    rc = lib.sjhip_ssa_backward_packed(L.DTYPE_F32, 4, 2, 32, 196, 0.125, 1, None, 1, None)
+    assert rc == -1 and b"NULL" in lib.sjhip_last_error()
+    rc = lib.sjhip_ssa_forward_packed(L.DTYPE_F32, 4, 2, 128, 196, 0.125, 1, 1, None)
+    assert rc == -2 and b"not supported" in lib.sjhip_last_error()
     assert lib.sjhip_bit_pack(L.DTYPE_F32, -1, 1, 1, None) == -1
     assert lib.sjhip_bit_pack(L.DTYPE_F32, 0, None, None, None) == 0
     assert lib.sjhip_plif_workspace_floats(L.DTYPE_F32, 1 << 20) >= (1 << 20) // 1024

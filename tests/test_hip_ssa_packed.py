@@ -1,0 +1,101 @@
+"""The spiking self-attention contraction with bit-packed operands, and the LIF -> contraction step that keeps the
+spikes bit-packed in between: everything must equal the dense-operand kernels bit for bit (same arithmetic, the
+operands only arrive in another encoding)."""
+
+import pytest
+import torch
+
+from spikingjelly_amd.activation_based import functional, layer
+from spikingjelly_amd.activation_based.hip_kernel import attention_kernel as A
+from spikingjelly_amd.activation_based.hip_kernel.compress import bit_spike_compress
+
+from helpers import bits_equal, seeded_randn
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("samples,heads,cph,tokens", [(6, 12, 32, 196), (3, 2, 64, 196), (5, 4, 32, 20), (2, 3, 16, 44),
+                                                       (4, 2, 24, 256), (1, 1, 8, 1)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_packed_operands_equal_dense_operands(samples, heads, cph, tokens, dtype):
+    g = torch.Generator().manual_seed(samples * 1000 + tokens)
+    qkv = (torch.rand((samples, 3, heads, cph, tokens), generator=g) < 0.3).to(dtype).cuda()
+    grad_out = torch.randn((samples, heads, cph, tokens), generator=g).to(dtype).cuda()
+    bits = bit_spike_compress(qkv)
+    assert A.ssa_packed_supported(dtype, cph, tokens)
+    out_dense = A.hip_ssa_forward(qkv, 0.125)
+    out_packed = A._ssa_packed(bits, None, dtype, samples, heads, cph, tokens, 0.125)
+    assert bits_equal(out_packed, out_dense) and float(out_dense.float().abs().sum()) > 0
+    grad_dense = A.hip_ssa_backward(qkv, grad_out, 0.125)
+    grad_packed = A._ssa_packed(bits, grad_out, dtype, samples, heads, cph, tokens, 0.125)
+    assert bits_equal(grad_packed, grad_dense)
+
+
+def test_tiles_must_start_on_a_byte():
+    assert not A.ssa_packed_supported(torch.float32, 3, 5)
+    bits = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        A._ssa_packed(bits, None, torch.float32, 1, 1, 3, 5, 0.125)
+
+
+def _blocks(dim, heads):
+    torch.manual_seed(dim + heads)
+    fused = layer.SpikingSelfAttention(dim, heads, backend="hip").cuda()
+    plain = layer.SpikingSelfAttention(dim, heads, backend="hip").cuda()
+    plain.load_state_dict(fused.state_dict())
+    for block in (fused, plain):
+        with torch.no_grad():  # freshly initialised, the block hardly fires: raise the batch-norm gains
+            block.qkv_conv_bn[1].weight.fill_(2.0)
+            block.proj_conv_bn[1].weight.fill_(3.0)
+    plain._lif_ssa_fused = lambda pre: None  # the two-operator path
+    return fused, plain
+
+
+@pytest.mark.parametrize("T,B,dim,heads,tokens", [(4, 8, 128, 4, 96), (2, 3, 64, 2, 20), (4, 2, 384, 12, 196)])
+def test_fused_block_equals_two_operator_block(T, B, dim, heads, tokens):
+    fused, plain = _blocks(dim, heads)
+    x = seeded_randn((T, B, dim, tokens), 5)
+    g = seeded_randn((T, B, dim, tokens), 6).cuda()
+    xa, xb = x.cuda().requires_grad_(), x.cuda().requires_grad_()
+    calls = []
+    original = A.lif_ssa_fused
+    A.lif_ssa_fused = lambda *a, **k: (calls.append(1), original(*a, **k))[1]
+    try:
+        ya = fused(xa)
+    finally:
+        A.lif_ssa_fused = original
+    yb = plain(xb)
+    assert calls, "the fused step did not run"
+    assert bits_equal(ya, yb) and float(ya.detach().mean()) > 0.02
+    assert bits_equal(fused.qkv_lif.v, plain.qkv_lif.v)
+    ya.backward(g)
+    yb.backward(g)
+    assert bits_equal(xa.grad, xb.grad)
+    # the input gradient is bit-identical, so the same gradients reached the convolutions; their weight gradients
+    # come from the vendor library's reduction, whose summation order is not fixed from run to run
+    for (name, pa), (_, pb) in zip(fused.named_parameters(), plain.named_parameters()):
+        torch.testing.assert_close(pa.grad, pb.grad, rtol=1e-4, atol=1e-4 * float(pb.grad.abs().max()), msg=name)
+    # second call: the LIF state is a carried tensor now
+    ya2, yb2 = fused(xa.detach()), plain(xb.detach())
+    assert bits_equal(ya2, yb2)
+    # inference
+    functional.reset_net(fused)
+    functional.reset_net(plain)
+    fused.eval()
+    plain.eval()
+    with torch.no_grad():
+        assert bits_equal(fused(x.cuda()), plain(x.cuda()))
+
+
+def test_long_sequences_and_odd_shapes_take_the_two_operator_path():
+    fused, plain = _blocks(64, 2)
+    x = seeded_randn((48, 1, 64, 20), 7).cuda().requires_grad_()   # T = 48: the replay backward is not preferred
+    assert fused._lif_ssa_fused(fused.qkv_conv_bn(x)) is None
+    functional.reset_net(fused)
+    y = fused(x)
+    y.sum().backward()
+    assert bool(torch.isfinite(x.grad).all())
+    functional.reset_net(fused)
+    x = seeded_randn((2, 1, 64, 5), 8).cuda()                      # 32 channels x 5 tokens: tiles start on bytes, N % 8 == 0
+    with torch.no_grad():
+        assert fused(x).shape == x.shape
