@@ -250,6 +250,36 @@ int sjhip_stbif_forward(int dtype, uint32_t flags, int64_t T, int64_t N,
                         int32_t *work_flag, void *stream);
 
 /*
+ * Izhikevich neuron: quadratic membrane v with an adaptation current w (two states).  Stands in for
+ * torch.ops.sj.cupy_multistep_izhikevich_forward / _backward,
+ * spikingjelly/activation_based/cuda_kernel/neuron_kernel/multi_step/izhikevich.py, and computes the torch backend's
+ * functional.izhikevich_step (functional/neuron.py:1514-1522) for every step:
+ *     h = v + (x + a0 (v - v_rest)(v - v_c) - w) / tau;   u = w + (a (h - v_rest) - w) / tau_w;   s = [h >= v_th];
+ *     v' = h - s v_th  or  (1 - s) h + s v_reset;         w' = u + b s
+ * Forward:  x_seq [T,N], v_init / w_init [N] in ([1] with the broadcast flags); spike_seq [T,N], v_last, w_last [N]
+ * out; v_seq, w_seq [T,N] out or NULL; h_seq [T,N] out or NULL (needed by the backward).
+ * Backward: grad_spike_seq [T,N], h_seq [T,N] in; grad_v_seq, grad_w_seq [T,N] and grad_v_last, grad_w_last [N] in or
+ * NULL; v_init in (needed for grad_v_init); grad_x_seq [T,N] out; grad_v_init, grad_w_init [N] out or NULL.
+ * flags: SJHIP_FLAG_SOFT_RESET, SJHIP_FLAG_DETACH_RESET, SJHIP_FLAG_FP32_STATE, SJHIP_FLAG_V_INIT_BROADCAST,
+ * SJHIP_FLAG_W_INIT_BROADCAST.
+ */
+#define SJHIP_FLAG_W_INIT_BROADCAST 0x800u
+typedef struct sjhip_izhikevich_params {
+  float tau, v_threshold, v_reset, v_rest, v_c, a0, tau_w, a, b;
+  float sg_alpha;   /* backward only */
+  int32_t sg_id;    /* backward only, sjhip_surrogate 0..6 */
+  uint32_t flags;
+} sjhip_izhikevich_params;
+int sjhip_izhikevich_forward(int dtype, const sjhip_izhikevich_params *p, int64_t T, int64_t N,
+                             const void *x_seq, const void *v_init, const void *w_init,
+                             void *spike_seq, void *v_seq, void *w_seq, void *v_last, void *w_last, void *h_seq,
+                             void *stream);
+int sjhip_izhikevich_backward(int dtype, const sjhip_izhikevich_params *p, int64_t T, int64_t N,
+                              const void *grad_spike_seq, const void *grad_v_seq, const void *grad_w_seq,
+                              const void *grad_v_last, const void *grad_w_last, const void *h_seq, const void *v_init,
+                              void *grad_x_seq, void *grad_v_init, void *grad_w_init, void *stream);
+
+/*
  * Activation-aware IF (ANN2SNN activation-aware redistribution): an IF neuron whose threshold and membrane offset are
  * per channel or scalar; inference only.  Stands in for torch.ops.sj.multistep_activation_aware_if_forward,
  * spikingjelly/activation_based/triton_kernel/neuron_kernel/activation_aware_if.py:44-285, and computes the torch

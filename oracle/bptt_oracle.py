@@ -76,3 +76,44 @@ def bptt_ilif(h_seq: np.ndarray, grad_spike_seq: np.ndarray, grad_v_seq: Optiona
         grad_x[t] = G
         carry = G * (1.0 - k)
     return grad_x, carry
+
+
+def bptt_izhikevich(h_seq: np.ndarray, v_init: np.ndarray, sg_prime: Callable[[np.ndarray], np.ndarray],
+                    grad_spike_seq: np.ndarray, grad_v_seq: Optional[np.ndarray], grad_w_seq: Optional[np.ndarray],
+                    grad_v_last: Optional[np.ndarray], grad_w_last: Optional[np.ndarray], params, v_threshold: float,
+                    v_reset: Optional[float], detach_reset: bool):
+    """Two coupled states (equal to autograd through ``functional/neuron.py:1514-1522``); ``params`` = (tau, a0,
+    v_rest, v_c, tau_w, a, b), k = 1/tau, kw = 1/tau_w:
+
+        gv_t = grad_v_seq[t] + Gh_{t+1} (1 + k a0 ((v_t - v_c) + (v_t - v_rest)))      gw_t = grad_w_seq[t] + cw_{t+1}
+        dvdh = soft: 1 - [not detach] v_th sg_t        hard: (1 - s_t) + sg_t (v_reset - [not detach] h_t)
+        Gh_t = gv_t dvdh + (grad_spike[t] + b gw_t) sg_t + gw_t kw a          cw_t = gw_t (1 - kw) - Gh_t k
+        grad_x[t] = Gh_t k     grad_v_init = Gh_0 (1 + k a0 (...v_init...))     grad_w_init = cw_0
+
+    Returns (grad_x, grad_v_init, grad_w_init)."""
+    tau, a0, v_rest, v_c, tau_w, a, b = params
+    k, kw = 1.0 / tau, 1.0 / tau_w
+    h_seq = np.asarray(h_seq, dtype=np.float64)
+    T = h_seq.shape[0]
+    live = 0.0 if detach_reset else 1.0
+    gh = np.zeros_like(h_seq[0])
+    cw = np.zeros_like(gh) if grad_w_last is None else np.asarray(grad_w_last, dtype=np.float64).copy()
+    grad_x = np.zeros_like(h_seq)
+    dhdv = lambda v: 1.0 + k * a0 * ((v - v_c) + (v - v_rest))
+    for t in range(T - 1, -1, -1):
+        h = h_seq[t]
+        s = (h - v_threshold >= 0).astype(np.float64)
+        v_t = h - s * v_threshold if v_reset is None else (1.0 - s) * h + s * v_reset
+        sg = sg_prime(h - v_threshold)
+        if t == T - 1:
+            gv = np.zeros_like(h) if grad_v_last is None else np.asarray(grad_v_last, dtype=np.float64)
+        else:
+            gv = gh * dhdv(v_t)
+        if grad_v_seq is not None:
+            gv = gv + grad_v_seq[t]
+        gw = cw if grad_w_seq is None else cw + grad_w_seq[t]
+        dvdh = (1.0 - live * v_threshold * sg) if v_reset is None else ((1.0 - s) + sg * (v_reset - live * h))
+        gh = gv * dvdh + (grad_spike_seq[t] + b * gw) * sg + gw * kw * a
+        grad_x[t] = gh * k
+        cw = gw * (1.0 - kw) - gh * k
+    return grad_x, gh * dhdv(np.asarray(v_init, dtype=np.float64)), cw

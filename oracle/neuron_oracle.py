@@ -216,6 +216,35 @@ def step(kind: str, x, v, tau_or_w, decay_input: bool, v_threshold: float, v_res
     return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset), h
 
 
+def izhikevich_step(x, v, w, tau, a0, v_rest, v_c, tau_w, a, b, v_threshold, v_reset: Optional[float], sg: Callable,
+                    detach_reset: bool):
+    """(spike, v_next, w_next, h): functional/neuron.py:1514-1522."""
+    v_charged = v + (x + a0 * (v - v_rest) * (v - v_c) - w) / tau
+    w_next = w + (a * (v_charged - v_rest) - w) / tau_w
+    spike = sg(v_charged - v_threshold)
+    spike_d = spike.detach() if detach_reset else spike
+    if v_reset is None:
+        v_next = v_charged - spike_d * v_threshold
+    else:
+        v_next = (1.0 - spike_d) * v_charged + spike * v_reset
+    return spike, v_next, w_next + b * spike, v_charged
+
+
+def izhikevich_multi_step(x_seq, v_init, w_init, params, v_threshold: float, v_reset: Optional[float],
+                          sg: Optional[Callable] = None, detach_reset: bool = False):
+    """Step loop (base.py:594-607) over ``izhikevich_step``; ``params`` = (tau, a0, v_rest, v_c, tau_w, a, b).
+    Returns (spike_seq, v_seq, w_seq, h_seq)."""
+    sg = heaviside if sg is None else sg
+    tau, a0, v_rest, v_c, tau_w, a, b = params
+    v, w, out = v_init, w_init, ([], [], [], [])
+    for t in range(x_seq.shape[0]):
+        s, v, w, h = izhikevich_step(x_seq[t], v, w, tau, a0, v_rest, v_c, tau_w, a, b, v_threshold, v_reset, sg,
+                                     detach_reset)
+        for seq, value in zip(out, (s, v, w, h)):
+            seq.append(value)
+    return tuple(torch.stack(seq) for seq in out)
+
+
 def activation_aware_if_step(x, v, v_threshold, v_offset, v_reset: Optional[float], sg: Callable, detach_reset: bool):
     """(spike, v_next, h): functional/neuron.py:577-584; v_threshold / v_offset are tensors broadcastable to x."""
     h = v + x

@@ -33,6 +33,7 @@ __all__ = [
     "plif_step",
     "qif_step",
     "eif_step",
+    "izhikevich_step",
     "ilif_step",
     "stbif_step",
     "activation_aware_if_step",
@@ -41,6 +42,7 @@ __all__ = [
     "plif_multi_step_hip",
     "qif_multi_step_hip",
     "eif_multi_step_hip",
+    "izhikevich_multi_step_hip",
     "ilif_multi_step_hip",
     "stbif_multi_step_hip",
     "stbif_single_step_hip",
@@ -123,6 +125,24 @@ def eif_step(x: torch.Tensor, v: torch.Tensor, tau: float, delta_t: float, theta
     h = v + (x + v_rest - v + delta_t * torch.exp((v - theta_rh) / delta_t)) / tau
     spike = surrogate_function(h - v_threshold)
     return spike, voltage_reset(h, spike, v_threshold, v_reset, detach_reset)
+
+
+def izhikevich_step(x: torch.Tensor, v: torch.Tensor, w: torch.Tensor, tau: float, a0: float, v_rest: float, v_c: float,
+                    tau_w: float, a: float, b: float, v_threshold: float, v_reset: Optional[float],
+                    surrogate_function: SurrogateFunction, detach_reset: bool = False
+                    ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """One Izhikevich step (reference :1412-1522): a quadratic membrane ``v`` with an adaptation current ``w`` that
+    follows the membrane (``a``, ``tau_w``) and jumps by ``b`` at a spike.  Returns ``(spike, v_next, w_next)``.  In the
+    hard reset the ``v_reset`` term carries the undetached spike, as in the reference."""
+    h = v + (x + a0 * (v - v_rest) * (v - v_c) - w) / tau
+    w_next = w + (a * (h - v_rest) - w) / tau_w
+    spike = surrogate_function(h - v_threshold)
+    s = spike.detach() if detach_reset else spike
+    if v_reset is None:
+        v_next = h - s * v_threshold
+    else:
+        v_next = (1.0 - s) * h + spike * v_reset
+    return spike, v_next, w_next + b * spike
 
 
 def ilif_step(x: torch.Tensor, v: torch.Tensor, tau: float, v_threshold: float,
@@ -380,6 +400,31 @@ def eif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_thres
         s, v_seq, v_last = K.hip_multistep_eif_inference(x2, v1, v_threshold, vr, soft, float(tau), float(v_rest),
                                                          float(theta_rh), float(delta_t), store_v_seq, flags)
     return _finish(x_seq, s, v_seq, v_last, store_v_seq)
+
+
+def izhikevich_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Tensor, tau: float, v_threshold: float,
+                              v_reset: Optional[float], v_rest: float, a: float, b: float, tau_w: float, v_c: float,
+                              a0: float, detach_reset: bool, surrogate_function: SurrogateFunction,
+                              store_state_seq: bool = False
+                              ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor],
+                                         Optional[torch.Tensor]]:
+    """Multi-step Izhikevich on the hip backend; arguments and return ``(spike_seq, v_next, w_next, v_seq | None,
+    w_seq | None)`` of the reference's ``izhikevich_multi_step_cupy`` (:2404-2530)."""
+    from ..hip_kernel import izhikevich_kernel as IK
+    from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
+
+    soft = v_reset is None
+    need_grad = _needs_grad(x_seq, v, w)
+    sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function) if need_grad else (0, 0.0)
+    scalars = [float(tau), float(v_threshold), 0.0 if soft else float(v_reset), float(v_rest), float(v_c), float(a0),
+               float(tau_w), float(a), float(b)]
+    s, v_seq, w_seq, v_last, w_last, _ = IK.hip_multistep_izhikevich_forward(
+        x_seq.flatten(1), v.flatten(), w.flatten(), scalars, soft, detach_reset, sg_id, sg_alpha, store_state_seq,
+        need_grad, _hip_mode_flags(x_seq))
+    state = x_seq.shape[1:]
+    return (s.reshape(x_seq.shape), v_last.reshape(state), w_last.reshape(state),
+            v_seq.reshape(x_seq.shape) if store_state_seq else None,
+            w_seq.reshape(x_seq.shape) if store_state_seq else None)
 
 
 def ilif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_threshold: float,

@@ -29,6 +29,7 @@ FLAG_ATOMIC_REDUCE = 0x80
 FLAG_V_INIT_BROADCAST = 0x100
 FLAG_Q_BROADCAST = 0x200
 FLAG_ACC_BROADCAST = 0x400
+FLAG_W_INIT_BROADCAST = 0x800
 
 KC_FORWARD, KC_BACKWARD, KC_PLIF_REDUCE, KC_BIT_PACK, KC_BIT_UNPACK, KC_SSA_FORWARD, KC_SSA_BACKWARD = range(7)
 
@@ -49,6 +50,8 @@ EXPORTED_SYMBOLS = (
     "sjhip_ssa_backward_packed",
     "sjhip_stbif_forward",
     "sjhip_aaif_forward",
+    "sjhip_izhikevich_forward",
+    "sjhip_izhikevich_backward",
     "sjhip_bit_pack",
     "sjhip_bit_unpack",
     "sjhip_set_tuning",
@@ -76,6 +79,13 @@ class NeuronParams(ctypes.Structure):
         ("grad_min", c_float),
         ("grad_max", c_float),
     ]
+
+
+class IzhikevichParams(ctypes.Structure):
+    """``struct sjhip_izhikevich_params``."""
+
+    _fields_ = [(name, c_float) for name in ("tau", "v_threshold", "v_reset", "v_rest", "v_c", "a0", "tau_w", "a", "b",
+                                             "sg_alpha")] + [("sg_id", c_int32), ("flags", c_uint32)]
 
 
 _lock = threading.Lock()
@@ -157,6 +167,10 @@ def load() -> ctypes.CDLL:
         lib.sjhip_ssa_backward_packed.restype = c_int
         lib.sjhip_ssa_backward_packed.argtypes = [c_int, c_int64, c_int, c_int, c_int64, c_float, c_void_p, c_void_p,
                                                   c_void_p, c_void_p]
+        lib.sjhip_izhikevich_forward.restype = c_int
+        lib.sjhip_izhikevich_forward.argtypes = [c_int, POINTER(IzhikevichParams), c_int64, c_int64] + [c_void_p] * 10
+        lib.sjhip_izhikevich_backward.restype = c_int
+        lib.sjhip_izhikevich_backward.argtypes = [c_int, POINTER(IzhikevichParams), c_int64, c_int64] + [c_void_p] * 11
         lib.sjhip_bit_pack.restype = c_int
         lib.sjhip_bit_pack.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p]
         lib.sjhip_bit_unpack.restype = c_int

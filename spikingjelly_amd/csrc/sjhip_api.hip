@@ -260,6 +260,44 @@ int sjhip_stbif_forward(int dtype, uint32_t flags, int64_t T, int64_t N, const v
                               q_final, acc_q_final, cur_output, work_flag, static_cast<hipStream_t>(stream));
 }
 
+namespace {
+int check_izhikevich(const char *what, int dtype, const sjhip_izhikevich_params *p, int64_t T, int64_t N, bool backward) {
+  if (!p) return fail(SJHIP_ERR_INVALID, "%s: params is NULL", what);
+  if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "%s: dtype %d", what, dtype);
+  if (!(p->tau > 0.0f) || !std::isfinite(p->tau) || !(p->tau_w > 0.0f) || !std::isfinite(p->tau_w))
+    return fail(SJHIP_ERR_INVALID, "%s: tau=%g tau_w=%g must be positive", what, (double)p->tau, (double)p->tau_w);
+  if (backward && (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_ERF))
+    return fail(SJHIP_ERR_UNSUPPORTED, "%s: surrogate id %d", what, p->sg_id);
+  const uint32_t known = SJHIP_FLAG_SOFT_RESET | SJHIP_FLAG_DETACH_RESET | SJHIP_FLAG_FP32_STATE |
+                         SJHIP_FLAG_V_INIT_BROADCAST | SJHIP_FLAG_W_INIT_BROADCAST;
+  if (p->flags & ~known) return fail(SJHIP_ERR_INVALID, "%s: flags 0x%x", what, p->flags);
+  return check_shape(what, T, N);
+}
+}  // namespace
+
+int sjhip_izhikevich_forward(int dtype, const sjhip_izhikevich_params *p, int64_t T, int64_t N, const void *x_seq,
+                             const void *v_init, const void *w_init, void *spike_seq, void *v_seq, void *w_seq,
+                             void *v_last, void *w_last, void *h_seq, void *stream) {
+  int rc = check_izhikevich("izhikevich_forward", dtype, p, T, N, false);
+  if (rc != SJHIP_OK) return rc;
+  if (!x_seq || !v_init || !w_init || !spike_seq || !v_last || !w_last)
+    return fail(SJHIP_ERR_INVALID, "izhikevich_forward: NULL tensor");
+  return launch_izhikevich_forward(dtype, *p, T, N, x_seq, v_init, w_init, spike_seq, v_seq, w_seq, v_last, w_last, h_seq,
+                                   static_cast<hipStream_t>(stream));
+}
+
+int sjhip_izhikevich_backward(int dtype, const sjhip_izhikevich_params *p, int64_t T, int64_t N,
+                              const void *grad_spike_seq, const void *grad_v_seq, const void *grad_w_seq,
+                              const void *grad_v_last, const void *grad_w_last, const void *h_seq, const void *v_init,
+                              void *grad_x_seq, void *grad_v_init, void *grad_w_init, void *stream) {
+  int rc = check_izhikevich("izhikevich_backward", dtype, p, T, N, true);
+  if (rc != SJHIP_OK) return rc;
+  if (!grad_spike_seq || !h_seq || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "izhikevich_backward: NULL tensor");
+  if (grad_v_init && !v_init) return fail(SJHIP_ERR_INVALID, "izhikevich_backward: grad_v_init needs v_init");
+  return launch_izhikevich_backward(dtype, *p, T, N, grad_spike_seq, grad_v_seq, grad_w_seq, grad_v_last, grad_w_last, h_seq,
+                                    v_init, grad_x_seq, grad_v_init, grad_w_init, static_cast<hipStream_t>(stream));
+}
+
 int sjhip_aaif_forward(int dtype, uint32_t flags, int64_t T, int64_t N, const void *x_seq, const void *v_init,
                        const float *v_threshold, int64_t threshold_count, const float *v_offset, int64_t offset_count,
                        int64_t channel_size, int64_t inner_size, float v_reset, void *spike_seq, void *v_seq,

@@ -67,6 +67,16 @@ template <> struct Cvt<bf16_t> {
 template <> struct Cvt<f16n_t> : Cvt<f16_t> {};
 template <> struct Cvt<bf16n_t> : Cvt<bf16_t> {};
 
+// (tensor of dtype R) * (Python scalar) as torch's CPU kernels compute it: the fp32 product is rounded to fp32 and then
+// to R.  The register barrier keeps the compiler from fusing the multiply and the conversion into one instruction that
+// rounds the exact product once (v_fma_mixlo_f16), which differs from the double rounding in about one result of forty.
+template <typename R> __device__ __forceinline__ float scalar_product(float scalar, float t) {
+#pragma clang fp contract(off)
+  float p = scalar * t;
+  if constexpr (!std::is_same<R, float>::value) asm volatile("" : "+v"(p));
+  return Cvt<R>::round(p);
+}
+
 // Cache policy of one access: NT marks the line as streaming (non-temporal), otherwise default.
 // Measured on MI355X: read-mostly kernels (backward, unpack) gain from NT on both loads and stores,
 // the write-mostly forward loses with it.
@@ -287,6 +297,13 @@ int launch_aaif_forward(int dtype, uint32_t flags, int64_t T, int64_t N, const v
                         const float *v_threshold, int64_t threshold_count, const float *v_offset, int64_t offset_count,
                         int64_t channel_size, int64_t inner_size, float v_reset, void *spike_seq, void *v_seq,
                         void *v_last, hipStream_t stream);
+int launch_izhikevich_forward(int dtype, const sjhip_izhikevich_params &p, int64_t T, int64_t N, const void *x_seq,
+                              const void *v_init, const void *w_init, void *spike_seq, void *v_seq, void *w_seq,
+                              void *v_last, void *w_last, void *h_seq, hipStream_t stream);
+int launch_izhikevich_backward(int dtype, const sjhip_izhikevich_params &p, int64_t T, int64_t N,
+                               const void *grad_spike_seq, const void *grad_v_seq, const void *grad_w_seq,
+                               const void *grad_v_last, const void *grad_w_last, const void *h_seq, const void *v_init,
+                               void *grad_x_seq, void *grad_v_init, void *grad_w_init, hipStream_t stream);
 int launch_backward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
                     const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
                     const void *h_seq, const void *v_init,

@@ -101,6 +101,17 @@ def test_argument_validation_without_a_device():
     assert rc == -1 and b"NULL" in lib.sjhip_last_error()
     rc = lib.sjhip_ssa_forward_packed(L.DTYPE_F32, 4, 2, 128, 196, 0.125, 1, 1, None)
     assert rc == -2 and b"not supported" in lib.sjhip_last_error()
+    izh = L.IzhikevichParams(2.0, 1.0, 0.0, -0.1, 0.8, 1.0, 2.0, 0.0, 0.0, 2.0, 1, 0)
+    rc = lib.sjhip_izhikevich_forward(L.DTYPE_F32, ctypes.byref(izh), 4, 16, 1, 1, None, 1, None, None, 1, 1, None, None)
+    assert rc == -1 and b"NULL tensor" in lib.sjhip_last_error()
+    bad = L.IzhikevichParams(2.0, 1.0, 0.0, -0.1, 0.8, 1.0, 0.0, 0.0, 0.0, 2.0, 1, 0)
+    rc = lib.sjhip_izhikevich_forward(L.DTYPE_F32, ctypes.byref(bad), 4, 16, 1, 1, 1, 1, None, None, 1, 1, None, None)
+    assert rc == -1 and b"tau_w" in lib.sjhip_last_error()
+    bad = L.IzhikevichParams(2.0, 1.0, 0.0, -0.1, 0.8, 1.0, 2.0, 0.0, 0.0, 2.0, 7, 0)
+    rc = lib.sjhip_izhikevich_backward(L.DTYPE_F32, ctypes.byref(bad), 4, 16, 1, None, None, None, None, 1, 1, 1, 1, 1, None)
+    assert rc == -2 and b"surrogate" in lib.sjhip_last_error()
+    rc = lib.sjhip_izhikevich_backward(L.DTYPE_F32, ctypes.byref(izh), 4, 16, 1, None, None, None, None, 1, None, 1, 1, 1, None)
+    assert rc == -1 and b"v_init" in lib.sjhip_last_error()
     assert lib.sjhip_bit_pack(L.DTYPE_F32, -1, 1, 1, None) == -1
     assert lib.sjhip_bit_pack(L.DTYPE_F32, 0, None, None, None) == 0
     assert lib.sjhip_plif_workspace_floats(L.DTYPE_F32, 1 << 20) >= (1 << 20) // 1024

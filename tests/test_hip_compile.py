@@ -22,6 +22,7 @@ NODES = {
     "qif": lambda **kw: neuron.QIFNode(tau=2.0, surrogate_function=surrogate.ATan(), **kw),
     "eif": lambda **kw: neuron.EIFNode(tau=2.0, surrogate_function=surrogate.ATan(), **kw),
     "ilif": lambda **kw: neuron.ILIFNode(**kw),
+    "izhikevich": lambda **kw: neuron.IzhikevichNode(a=0.3, b=0.2, tau_w=3.0, surrogate_function=surrogate.ATan(), **kw),
 }
 
 
@@ -40,7 +41,7 @@ def _compiled(module):
 @pytest.mark.parametrize("kind", sorted(NODES))
 @pytest.mark.parametrize("store_v_seq", [False, True])
 def test_multi_step_node_compiles_without_graph_breaks(kind, store_v_seq):
-    scale = {"qif": 0.4, "eif": 0.5, "ilif": 2.0}.get(kind, 0.8)
+    scale = {"qif": 0.4, "eif": 0.5, "ilif": 2.0, "izhikevich": 0.5}.get(kind, 0.8)
     x = (seeded_randn((6, 4, 32), 11, 0.3, scale)).cuda()
     eager = NODES[kind](step_mode="m", backend="hip", store_v_seq=store_v_seq).cuda()
     traced = NODES[kind](step_mode="m", backend="hip", store_v_seq=store_v_seq).cuda()

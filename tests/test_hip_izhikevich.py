@@ -1,0 +1,131 @@
+"""Izhikevich neuron (two coupled states) on the hip backend against the oracle and the torch backend.
+
+Bars as for the other polynomial neurons: spikes, h, v and w bit-exact in fp32 and in every-op-rounded 16-bit mode;
+gradients (input, both initial states) within rtol 1e-5 (fp32) of autograd through the oracle.
+"""
+
+import pytest
+import torch
+
+from oracle import neuron_oracle as no
+from spikingjelly_amd.activation_based import functional, neuron, surrogate
+from spikingjelly_amd.activation_based.hip_kernel import izhikevich_kernel as IK
+
+from helpers import bits_equal, seeded_randn
+
+pytestmark = pytest.mark.gpu
+
+GRAD_RTOL, GRAD_ATOL = 1e-5, 2e-6
+
+PARAMS = [  # tau, a0, v_rest, v_c, tau_w, a, b
+    (2.0, 1.0, -0.1, 0.8, 2.0, 0.0, 0.0),
+    (2.5, 0.7, -0.1, 0.6, 3.0, 0.3, 0.2),
+    (10.0, 1.5, 0.0, 0.5, 4.0, -0.2, 0.5),
+]
+
+
+def _scalars(p, vth, v_reset):
+    tau, a0, v_rest, v_c, tau_w, a, b = p
+    return [tau, vth, 0.0 if v_reset is None else v_reset, v_rest, v_c, a0, tau_w, a, b]
+
+
+@pytest.mark.parametrize("p", PARAMS)
+@pytest.mark.parametrize("v_reset", [0.0, -0.2, None])
+@pytest.mark.parametrize("T,N", [(16, 4096), (7, 111), (33, 260), (1, 4)])
+@pytest.mark.parametrize("detach", [False, True])
+def test_forward_bit_exact_and_gradients_fp32(p, v_reset, T, N, detach):
+    # a soft reset leaves v above v_c after a spike, where the quadratic term runs away: keep that drive small
+    x = seeded_randn((T, N), 100 + T, 0.4, 0.6) if v_reset is not None else seeded_randn((T, N), 100 + T, 0.25, 0.25)
+    v0, w0 = seeded_randn((N,), 200 + N, 0.0, 0.2), seeded_randn((N,), 250 + N, 0.0, 0.2)
+    gs, gv, gw = seeded_randn((T, N), 300 + T), seeded_randn((T, N), 400 + T, 0.0, 0.1), seeded_randn((T, N), 500 + T, 0.0, 0.1)
+    vth = 1.0
+    xr, vr, wr = x.clone().requires_grad_(), v0.clone().requires_grad_(), w0.clone().requires_grad_()
+    es, ev, ew, eh = no.izhikevich_multi_step(xr, vr, wr, p, vth, v_reset, no.surrogate("atan", 2.0), detach)
+    assert bool(torch.isfinite(ev).all())
+    torch.autograd.backward([es, ev, ew], [gs, gv, gw])
+    soft = v_reset is None
+    xd, vd, wd = x.cuda().requires_grad_(), v0.cuda().requires_grad_(), w0.cuda().requires_grad_()
+    s, v_seq, w_seq, v_last, w_last, h = IK.hip_multistep_izhikevich_forward(xd, vd, wd, _scalars(p, vth, v_reset), soft,
+                                                                            detach, 1, 2.0, True, True, 0)
+    assert bits_equal(s.cpu(), es.detach()) and bits_equal(h.cpu(), eh.detach())
+    assert bits_equal(v_seq.cpu(), ev.detach()) and bits_equal(w_seq.cpu(), ew.detach())
+    assert bits_equal(v_last.cpu(), ev[-1].detach()) and bits_equal(w_last.cpu(), ew[-1].detach())
+    torch.autograd.backward([s, v_seq, w_seq], [gs.cuda(), gv.cuda(), gw.cuda()])
+    torch.testing.assert_close(xd.grad.cpu(), xr.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+    torch.testing.assert_close(vd.grad.cpu(), vr.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+    torch.testing.assert_close(wd.grad.cpu(), wr.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+
+
+@pytest.mark.parametrize("sg_name,sg_id,alpha", [("sigmoid", 0, 4.0), ("erf", 6, 2.0)])
+def test_last_state_gradients_without_state_sequences(sg_name, sg_id, alpha):
+    T, N = 9, 256
+    p = PARAMS[1]
+    x = seeded_randn((T, N), 7, 0.4, 0.6)
+    v0, w0 = seeded_randn((N,), 8, 0.0, 0.2), seeded_randn((N,), 9, 0.0, 0.2)
+    gs, gvl, gwl = seeded_randn((T, N), 10), seeded_randn((N,), 11), seeded_randn((N,), 12)
+    xr, vr, wr = x.clone().requires_grad_(), v0.clone().requires_grad_(), w0.clone().requires_grad_()
+    es, ev, ew, _ = no.izhikevich_multi_step(xr, vr, wr, p, 1.0, -0.1, no.surrogate(sg_name, alpha), False)
+    torch.autograd.backward([es, ev[-1], ew[-1]], [gs, gvl, gwl])
+    xd, vd, wd = x.cuda().requires_grad_(), v0.cuda().requires_grad_(), w0.cuda().requires_grad_()
+    s, v_seq, w_seq, v_last, w_last, _ = IK.hip_multistep_izhikevich_forward(xd, vd, wd, _scalars(p, 1.0, -0.1), False, False,
+                                                                            sg_id, alpha, False, True, 0)
+    assert v_seq.numel() == 0 and w_seq.numel() == 0
+    torch.autograd.backward([s, v_last, w_last], [gs.cuda(), gvl.cuda(), gwl.cuda()])
+    torch.testing.assert_close(xd.grad.cpu(), xr.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+    torch.testing.assert_close(vd.grad.cpu(), vr.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+    torch.testing.assert_close(wd.grad.cpu(), wr.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("T,N", [(8, 2048), (5, 77)])
+def test_every_op_rounded_16bit_equals_torch_ops_on_half_tensors(dtype, T, N):
+    p = PARAMS[1]
+    x = seeded_randn((T, N), 21, 0.4, 0.6).to(dtype)
+    v0, w0 = seeded_randn((N,), 22, 0.0, 0.2).to(dtype), seeded_randn((N,), 23, 0.0, 0.2).to(dtype)
+    es, ev, ew, eh = no.izhikevich_multi_step(x, v0, w0, p, 1.0, -0.1)
+    s, v_seq, w_seq, _, _, h = IK.hip_multistep_izhikevich_forward(x.cuda(), v0.cuda(), w0.cuda(), _scalars(p, 1.0, -0.1),
+                                                                  False, False, 1, 2.0, True, True, 0)
+    assert bits_equal(s.cpu(), es) and bits_equal(h.cpu(), eh)
+    assert bits_equal(v_seq.cpu(), ev) and bits_equal(w_seq.cpu(), ew)
+
+
+@pytest.mark.parametrize("v_reset", [0.0, None])
+@pytest.mark.parametrize("store_v_seq", [False, True])
+def test_hip_node_matches_torch_node(v_reset, store_v_seq):
+    kw = dict(tau=2.0, v_c=0.8, a0=1.0, v_threshold=1.0, v_reset=v_reset, v_rest=-0.1, w_rest=0.05, tau_w=3.0, a=0.3, b=0.2,
+              surrogate_function=surrogate.ATan(), store_v_seq=store_v_seq)
+    a = neuron.IzhikevichNode(step_mode="m", backend="torch", **kw)
+    b = neuron.IzhikevichNode(step_mode="m", backend="hip", **kw).cuda()
+    x = seeded_randn((6, 4, 12, 4), 20260701, 0.4, 0.6) if v_reset is not None else seeded_randn((6, 4, 12, 4), 20260701, 0.7, 0.4)
+    xa, xb = x.clone().requires_grad_(), x.cuda().requires_grad_()
+    sa, sb = a(xa), b(xb)
+    (sa.sum() + 0.5 * a.v.sum() + 0.25 * a.w.sum()).backward()
+    (sb.sum() + 0.5 * b.v.sum() + 0.25 * b.w.sum()).backward()
+    assert 0.0 < float(sa.detach().mean()) < 0.9 and bool(torch.isfinite(a.v).all())
+    assert bits_equal(sb.cpu(), sa.detach())
+    assert bits_equal(b.v.detach().cpu(), a.v.detach()) and bits_equal(b.w.detach().cpu(), a.w.detach())
+    if store_v_seq:
+        assert bits_equal(b.v_seq.detach().cpu(), a.v_seq.detach())
+    torch.testing.assert_close(xb.grad.cpu(), xa.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+    # a second call continues from both carried states
+    sa2, sb2 = a(xa.detach()), b(xb.detach())
+    assert bits_equal(sb2.cpu(), sa2.detach()) and bits_equal(b.w.detach().cpu(), a.w.detach())
+    functional.reset_net(a)
+    functional.reset_net(b)
+    assert b.w == 0.05 and b.v == (0.0 if v_reset is None else v_reset)
+    # inference
+    with torch.no_grad():
+        assert bits_equal(b(x.cuda()).cpu(), a(x))
+
+
+def test_module_rejects_what_the_reference_rejects():
+    with pytest.raises(AssertionError):
+        neuron.IzhikevichNode(tau=1.0)
+    with pytest.raises(AssertionError):
+        neuron.IzhikevichNode(a0=0.0)
+    node = neuron.IzhikevichNode()
+    assert node.supported_backends == ("torch",)
+    node.step_mode = "m"
+    assert node.supported_backends == ("torch", "hip")
+    assert "tau_w=2.0" in repr(node) and "v_c=0.8" in repr(node)
+    assert dict(node.named_memories()) == {"v": 0.0, "w": 0.0}

@@ -71,6 +71,18 @@ def test_stbif_op():
     torch.library.opcheck(hip_multistep_stbif, (x, q, acc, *th, 0), test_utils=("test_schema", "test_faketensor"))
 
 
+def test_izhikevich_op():
+    from spikingjelly_amd.activation_based.hip_kernel.izhikevich_kernel import hip_multistep_izhikevich_forward
+
+    x = seeded_randn((5, 32), 9, 0.4, 0.5).cuda().requires_grad_()
+    v0 = torch.zeros(32, device="cuda", requires_grad=True)
+    w0 = torch.zeros(32, device="cuda", requires_grad=True)
+    scalars = [2.0, 1.0, 0.0, -0.1, 0.8, 1.0, 3.0, 0.3, 0.2]
+    for store in (False, True):
+        torch.library.opcheck(hip_multistep_izhikevich_forward, (x, v0, w0, scalars, False, False, 1, 2.0, store, True, 0),
+                              test_utils=TESTS)
+
+
 def test_activation_aware_if_op():
     from spikingjelly_amd.activation_based.hip_kernel.aaif_kernel import hip_multistep_activation_aware_if
 

@@ -700,3 +700,79 @@ def test_activation_aware_if_reduces_to_if():
     for c in range(3):
         es, ev, _ = no.multi_step("if", x[:, c], v0[c], None, True, float(th[c]), None)
         assert torch.equal(s[:, c], es) and torch.equal(v[:, c], ev)
+
+
+# ------------------------------------------------------------------------------------------------
+# Izhikevich (functional/neuron.py:1514-1522)
+# ------------------------------------------------------------------------------------------------
+def test_izhikevich_reduces_to_qif_and_the_adaptation_current_decays_geometrically():
+    """Without coupling (a = b = 0) and with w = 0 the membrane is the QIF neuron, bit for bit; a free adaptation
+    current decays by (1 - 1/tau_w) per step; a spike adds b."""
+    x = seeded_randn((10, 300), 111, 0.4, 0.5)
+    v0 = seeded_randn((300,), 112, 0.0, 0.2)
+    for v_reset in (0.0, -0.1):
+        s, v, w, h = no.izhikevich_multi_step(x, v0, torch.zeros(300), (2.0, 1.0, -0.1, 0.8, 2.0, 0.0, 0.0), 1.0, v_reset)
+        es, ev, eh = no.multi_step("qif", x, v0, (2.0, 1.0, -0.1, 0.8), True, 1.0, v_reset)
+        assert torch.equal(s, es) and torch.equal(v, ev) and torch.equal(h, eh) and float(w.abs().max()) == 0.0
+        assert 0.0 < float(s.mean()) < 0.9
+    # x cancels the free current's pull on the membrane so that it never fires: w halves every step (tau_w = 2)
+    w0 = torch.full((4,), 0.5)
+    quiet = torch.zeros(6, 4)
+    s, v, w, _ = no.izhikevich_multi_step(quiet, torch.full((4,), -0.1), w0, (2.0, 1.0, -0.1, 0.8, 2.0, 0.0, 0.0), 10.0, 0.0)
+    assert float(s.sum()) == 0.0
+    assert torch.equal(w[:, 0], torch.tensor([0.5 / 2 ** (t + 1) for t in range(6)]))
+    # a spike adds b to w: drive one neuron over the threshold once
+    x1 = torch.tensor([[3.0], [0.0]])
+    s, v, w, _ = no.izhikevich_multi_step(x1, torch.zeros(1), torch.zeros(1), (2.0, 1.0, -0.1, 0.8, 2.0, 0.0, 0.25), 1.0, 0.0)
+    assert s.flatten().tolist() == [1.0, 0.0] and float(w[0]) == 0.25 and float(w[1]) == 0.125
+
+
+GRID_IZH = [(vr, det, sg) for vr in (0.0, -0.2, None) for det in (False, True) for sg in ("atan", "sigmoid")]
+
+
+@pytest.mark.parametrize("v_reset,detach,sg", GRID_IZH)
+def test_izhikevich_recurrence_equals_autograd_float64(v_reset, detach, sg):
+    T, N, vth = 6, 129, 0.8
+    alpha = no.SG_DEFAULT_ALPHA[sg]
+    params = (2.5, 0.7, -0.1, 0.6, 3.0, 0.3, 0.2)
+    scale = 0.5 if v_reset is not None else 0.25
+    x = seeded_randn((T, N), 121, 0.3, scale, torch.float64).requires_grad_()
+    v0 = seeded_randn((N,), 122, 0.0, 0.2, torch.float64).requires_grad_()
+    w0 = seeded_randn((N,), 123, 0.0, 0.2, torch.float64).requires_grad_()
+    gs, gv, gw = (seeded_randn((T, N), 124 + i, 0.0, 1.0 if i == 0 else 0.2, torch.float64) for i in range(3))
+    gvl, gwl = seeded_randn((N,), 128, dtype=torch.float64), seeded_randn((N,), 129, dtype=torch.float64)
+    s, v, w, h = no.izhikevich_multi_step(x, v0, w0, params, vth, v_reset, no.surrogate(sg, alpha), detach)
+    assert bool(torch.isfinite(v).all())
+    torch.autograd.backward([s, v, w, v[-1], w[-1]], [gs, gv, gw, gvl, gwl])
+    gx, gv0, gw0 = bptt_oracle.bptt_izhikevich(h.detach().numpy(), v0.detach().numpy(), _np_sg_prime(sg, alpha), gs.numpy(),
+                                               gv.numpy(), gw.numpy(), gvl.numpy(), gwl.numpy(), params, vth, v_reset, detach)
+    np.testing.assert_allclose(gx, x.grad.numpy(), rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(gv0, v0.grad.numpy(), rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(gw0, w0.grad.numpy(), rtol=1e-10, atol=1e-12)
+
+
+def test_izhikevich_autograd_matches_finite_differences_of_the_smooth_network():
+    T, N, vth, alpha = 5, 4, 0.9, 2.0
+    params = (2.5, 0.7, -0.1, 0.6, 3.0, 0.3, 0.2)
+    x = seeded_randn((T, N), 131, 0.3, 0.4, torch.float64)
+    v0 = seeded_randn((N,), 132, 0.0, 0.2, torch.float64)
+    w0 = seeded_randn((N,), 133, 0.0, 0.2, torch.float64)
+    gs, gv, gw = (seeded_randn((T, N), 134 + i, dtype=torch.float64) for i in range(3))
+    smooth = no.surrogate("atan", alpha, spiking=False)
+
+    def loss(x_, v_, w_):
+        s, v, w, _ = no.izhikevich_multi_step(x_, v_, w_, params, vth, -0.1, smooth)
+        return (s * gs).sum() + (v * gv).sum() + (w * gw).sum()
+
+    xa, va, wa = x.clone().requires_grad_(), v0.clone().requires_grad_(), w0.clone().requires_grad_()
+    loss(xa, va, wa).backward()
+    eps = 1e-6
+    for (t, n) in [(0, 0), (2, 3), (T - 1, 1)]:
+        xp, xm = x.clone(), x.clone()
+        xp[t, n] += eps
+        xm[t, n] -= eps
+        assert float(loss(xp, v0, w0) - loss(xm, v0, w0)) / (2 * eps) == pytest.approx(float(xa.grad[t, n]), rel=1e-6, abs=1e-8)
+    wp, wm = w0.clone(), w0.clone()
+    wp[2] += eps
+    wm[2] -= eps
+    assert float(loss(x, v0, wp) - loss(x, v0, wm)) / (2 * eps) == pytest.approx(float(wa.grad[2]), rel=1e-6, abs=1e-8)
