@@ -133,7 +133,7 @@ def other_workload(args) -> int:
                "plif_reduce_ms": _kernel_ms(L, L.KC_PLIF_REDUCE)})
         return 0
 
-    if args.workload in ("qif", "ilif"):
+    if args.workload in ("qif", "ilif", "eif", "izhikevich"):
         # the config-2 shape with another neuron of the same kernels: the quadratic integrate-and-fire neuron
         # (state-dependent dh/dv in the backward) or the integer-valued LIF (multi-level counts, windowed gradient)
         shape = (16, 256, 128, 32, 32)
@@ -144,6 +144,17 @@ def other_workload(args) -> int:
             node = neuron.QIFNode(tau=2.0, surrogate_function=surrogate.ATan(2.0), step_mode="m", backend="hip",
                                   store_v_seq=True).to(dev)
             label, what = "QIF", "QIFNode tau=2, v_c=0.8, a0=1, hard reset -0.1, ATan(2), x [16,256,128,32,32] fp32 ~N(0.3,0.4)"
+        elif args.workload == "eif":
+            x = (torch.randn(shape, generator=g, device=dev) * 0.6 + 0.3).requires_grad_()
+            node = neuron.EIFNode(tau=2.0, surrogate_function=surrogate.ATan(2.0), step_mode="m", backend="hip",
+                                  store_v_seq=True).to(dev)
+            label, what = "EIF", "EIFNode tau=2, delta_T=1, theta_rh=0.8, hard reset -0.1, ATan(2), x [16,256,128,32,32] fp32 ~N(0.3,0.6)"
+        elif args.workload == "izhikevich":
+            x = (torch.randn(shape, generator=g, device=dev) * 0.6 + 0.4).requires_grad_()
+            node = neuron.IzhikevichNode(tau=2.0, a=0.3, b=0.2, tau_w=3.0, surrogate_function=surrogate.ATan(2.0),
+                                         step_mode="m", backend="hip", store_v_seq=True).to(dev)
+            label, what = "Izhikevich", ("IzhikevichNode tau=2, v_c=0.8, a0=1, tau_w=3, a=0.3, b=0.2, hard reset 0, ATan(2), "
+                                         "x [16,256,128,32,32] fp32 ~N(0.4,0.6); h_seq saved (no replay)")
         else:
             x = (torch.randn(shape, generator=g, device=dev) * 1.5 + 1.0).requires_grad_()
             node = neuron.ILIFNode(tau=4.0 / 3.0, surrogate_function=surrogate.MultiLevelSpikeCount(4), step_mode="m",
@@ -161,6 +172,8 @@ def other_workload(args) -> int:
         elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
         f_ms, b_ms = _kernel_ms(L, L.KC_FORWARD), _kernel_ms(L, L.KC_BACKWARD)
         bytes_each = 16 * T * N + 4 * N
+        if args.workload == "izhikevich":
+            bytes_each = 16 * T * N + 16 * N  # x, s, v_seq, h_seq / grad_s, grad_v, h_seq, grad_x; two states in and out
         dom = "forward" if f_ms >= b_ms else "backward"
         d_ms = max(f_ms, b_ms)
         _emit(args, f"neuron-steps/sec {label} fwd+bwd fp32 T=16 N=33.5M, 1 MI355X", "neuron-steps/s",
@@ -169,6 +182,34 @@ def other_workload(args) -> int:
               {"bound": "hbm", "achieved": bytes_each / (d_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                "frac": bytes_each / (d_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": dom,
                "kernel_ms": d_ms, "algorithmic_bytes": bytes_each, "forward_ms": f_ms, "backward_ms": b_ms})
+        return 0
+
+    if args.workload == "aaif":
+        # activation-aware IF (inference), per-channel threshold and offset over the channel axis of [B, C, H, W]
+        shape = (16, 256, 128, 32, 32)
+        T, N = shape[0], 256 * 128 * 32 * 32
+        g = torch.Generator(device=dev).manual_seed(1002)
+        x = torch.randn(shape, generator=g, device=dev) * 0.5 + 0.2
+        node = neuron.ActivationAwareIFNode(v_threshold=torch.linspace(0.5, 2.0, 128), v_offset=torch.linspace(-0.2, 0.2, 128),
+                                            channel_dim=1, step_mode="m", backend="hip").to(dev).eval()
+
+        def step():
+            with torch.no_grad():
+                out = node(x)
+            functional.reset_net(node)
+            return out
+
+        elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
+        f_ms = _kernel_ms(L, L.KC_FORWARD)
+        rate = float(step().mean())
+        bytes_each = 8 * T * N + 4 * N  # x in, spike_seq out, v_last out
+        _emit(args, "neuron-steps/sec activation-aware IF inference fp32 T=16 N=33.5M, 1 MI355X", "neuron-steps/s",
+              T * N / (elapsed / args.steps), elapsed, "f32",
+              {"workload": "ActivationAwareIFNode, 128 per-channel thresholds and offsets (channel_dim=1), soft reset, "
+                           "x [16,256,128,32,32] fp32 ~N(0.2,0.5), eval", "T": T, "N": N, "firing_rate": rate},
+              {"bound": "hbm", "achieved": bytes_each / (f_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+               "frac": bytes_each / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "aaif_forward",
+               "kernel_ms": f_ms, "algorithmic_bytes": bytes_each})
         return 0
 
     if args.workload == "stbif":
@@ -295,7 +336,7 @@ def main() -> int:
     ap.add_argument("--cpu-sample-neurons", type=int, default=1 << 23)
     ap.add_argument("--cpu-repeats", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "qif", "ilif", "stbif"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "qif", "eif", "izhikevich", "ilif", "stbif", "aaif"],
                     help="config2 (default) is the headline metric; the others are secondary measurements")
     args = ap.parse_args()
     if args.gpus != 1:

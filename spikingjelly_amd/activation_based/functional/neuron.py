@@ -405,11 +405,12 @@ def eif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_thres
 def izhikevich_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Tensor, tau: float, v_threshold: float,
                               v_reset: Optional[float], v_rest: float, a: float, b: float, tau_w: float, v_c: float,
                               a0: float, detach_reset: bool, surrogate_function: SurrogateFunction,
-                              store_state_seq: bool = False
+                              store_state_seq: bool = False, store_w_seq: Optional[bool] = None
                               ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor],
                                          Optional[torch.Tensor]]:
     """Multi-step Izhikevich on the hip backend; arguments and return ``(spike_seq, v_next, w_next, v_seq | None,
-    w_seq | None)`` of the reference's ``izhikevich_multi_step_cupy`` (:2404-2530)."""
+    w_seq | None)`` of the reference's ``izhikevich_multi_step_cupy`` (:2404-2530).  ``store_w_seq=False`` with
+    ``store_state_seq=True`` keeps only ``v_seq`` (what a node with ``store_v_seq`` needs) and saves the other write."""
     from ..hip_kernel import izhikevich_kernel as IK
     from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
 
@@ -418,13 +419,13 @@ def izhikevich_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Ten
     sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(surrogate_function) if need_grad else (0, 0.0)
     scalars = [float(tau), float(v_threshold), 0.0 if soft else float(v_reset), float(v_rest), float(v_c), float(a0),
                float(tau_w), float(a), float(b)]
+    keep_w = store_state_seq if store_w_seq is None else bool(store_w_seq)
     s, v_seq, w_seq, v_last, w_last, _ = IK.hip_multistep_izhikevich_forward(
-        x_seq.flatten(1), v.flatten(), w.flatten(), scalars, soft, detach_reset, sg_id, sg_alpha, store_state_seq,
+        x_seq.flatten(1), v.flatten(), w.flatten(), scalars, soft, detach_reset, sg_id, sg_alpha, store_state_seq, keep_w,
         need_grad, _hip_mode_flags(x_seq))
     state = x_seq.shape[1:]
     return (s.reshape(x_seq.shape), v_last.reshape(state), w_last.reshape(state),
-            v_seq.reshape(x_seq.shape) if store_state_seq else None,
-            w_seq.reshape(x_seq.shape) if store_state_seq else None)
+            v_seq.reshape(x_seq.shape) if store_state_seq else None, w_seq.reshape(x_seq.shape) if keep_w else None)
 
 
 def ilif_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, tau: float, v_threshold: float,

@@ -6,7 +6,8 @@ Counterpart of the reference's ``sj::cupy_multistep_izhikevich_forward`` / ``_ba
     sj::hip_multistep_izhikevich_forward  -> (spike_seq, v_seq, w_seq, v_last, w_last, h_seq)
     sj::hip_multistep_izhikevich_backward -> (grad_x_seq, grad_v_init, grad_w_init)
 
-``v_seq`` / ``w_seq`` are empty tensors unless ``store_state_seq``; ``h_seq`` is empty unless ``save_h`` (training).
+``v_seq`` / ``w_seq`` are empty tensors unless ``store_v_seq`` / ``store_w_seq``; ``h_seq`` is empty unless ``save_h``
+(training).
 """
 
 from __future__ import annotations
@@ -35,7 +36,8 @@ def _flags(soft_reset: bool, detach_reset: bool, mode_flags: int) -> int:
 @torch.library.custom_op("sj::hip_multistep_izhikevich_forward", mutates_args=())
 def hip_multistep_izhikevich_forward(x_seq: torch.Tensor, v_init: torch.Tensor, w_init: torch.Tensor,
                                      scalars: list[float], soft_reset: bool, detach_reset: bool, sg_id: int,
-                                     sg_alpha: float, store_state_seq: bool, save_h: bool, mode_flags: int
+                                     sg_alpha: float, store_v_seq: bool, store_w_seq: bool, save_h: bool,
+                                     mode_flags: int
                                      ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
                                                 torch.Tensor]:
     """``scalars`` = [tau, v_threshold, v_reset, v_rest, v_c, a0, tau_w, a, b]."""
@@ -54,26 +56,27 @@ def hip_multistep_izhikevich_forward(x_seq: torch.Tensor, v_init: torch.Tensor, 
     flags = _flags(soft_reset, detach_reset, mode_flags) | v_flag | (L.FLAG_W_INIT_BROADCAST if w_flag else 0)
     spike_seq = torch.empty_like(x_seq)
     # outputs of an operator may not alias each other: every unused one is its own empty tensor
-    v_seq = torch.empty_like(x_seq) if store_state_seq else x_seq.new_empty((0,))
-    w_seq = torch.empty_like(x_seq) if store_state_seq else x_seq.new_empty((0,))
+    v_seq = torch.empty_like(x_seq) if store_v_seq else x_seq.new_empty((0,))
+    w_seq = torch.empty_like(x_seq) if store_w_seq else x_seq.new_empty((0,))
     h_seq = torch.empty_like(x_seq) if save_h else x_seq.new_empty((0,))
     v_last, w_last = x_seq.new_empty((N,)), x_seq.new_empty((N,))
     params = _params(scalars, 0, 0.0, flags)
     with torch.cuda.device(x_seq.device):
         rc = L.load().sjhip_izhikevich_forward(
             dtype, ctypes.byref(params), T, N, x_seq.data_ptr(), v_init.data_ptr(), w_init.data_ptr(),
-            spike_seq.data_ptr(), v_seq.data_ptr() if store_state_seq else None,
-            w_seq.data_ptr() if store_state_seq else None, v_last.data_ptr(), w_last.data_ptr(),
+            spike_seq.data_ptr(), v_seq.data_ptr() if store_v_seq else None,
+            w_seq.data_ptr() if store_w_seq else None, v_last.data_ptr(), w_last.data_ptr(),
             h_seq.data_ptr() if save_h else None, L.current_stream_ptr(x_seq.device))
     L.check(rc, "izhikevich_forward")
     return spike_seq, v_seq, w_seq, v_last, w_last, h_seq
 
 
 @hip_multistep_izhikevich_forward.register_fake
-def _(x_seq, v_init, w_init, scalars, soft_reset, detach_reset, sg_id, sg_alpha, store_state_seq, save_h, mode_flags):
+def _(x_seq, v_init, w_init, scalars, soft_reset, detach_reset, sg_id, sg_alpha, store_v_seq, store_w_seq, save_h,
+      mode_flags):
     return (x_seq.new_empty(x_seq.shape),
-            x_seq.new_empty(x_seq.shape) if store_state_seq else x_seq.new_empty((0,)),
-            x_seq.new_empty(x_seq.shape) if store_state_seq else x_seq.new_empty((0,)),
+            x_seq.new_empty(x_seq.shape) if store_v_seq else x_seq.new_empty((0,)),
+            x_seq.new_empty(x_seq.shape) if store_w_seq else x_seq.new_empty((0,)),
             v_init.new_empty(v_init.shape), v_init.new_empty(v_init.shape),
             x_seq.new_empty(x_seq.shape) if save_h else x_seq.new_empty((0,)))
 
@@ -112,24 +115,26 @@ def _(grad_spike_seq, grad_v_seq, grad_w_seq, grad_v_last, grad_w_last, h_seq, v
 
 
 def _setup_context(ctx, inputs, output):
-    (x_seq, v_init, w_init, scalars, soft_reset, detach_reset, sg_id, sg_alpha, store_state_seq, save_h,
+    (x_seq, v_init, w_init, scalars, soft_reset, detach_reset, sg_id, sg_alpha, store_v_seq, store_w_seq, save_h,
      mode_flags) = inputs
     if not save_h:
         raise RuntimeError("hip_multistep_izhikevich_forward was called with save_h=False but needs a gradient")
     ctx.save_for_backward(output[5], v_init)
     ctx.scalars = (list(scalars), soft_reset, detach_reset, sg_id, sg_alpha, mode_flags)
-    ctx.store_state_seq = store_state_seq
+    ctx.store_seq = (store_v_seq, store_w_seq)
     ctx.set_materialize_grads(False)
 
 
 def _backward(ctx, grad_spike_seq, grad_v_seq, grad_w_seq, grad_v_last, grad_w_last, grad_h_seq):
     del grad_h_seq
     h_seq, v_init = ctx.saved_tensors
-    if not ctx.store_state_seq:
-        grad_v_seq = grad_w_seq = None
+    if not ctx.store_seq[0]:
+        grad_v_seq = None
+    if not ctx.store_seq[1]:
+        grad_w_seq = None
     gx, gv, gw = hip_multistep_izhikevich_backward(grad_spike_seq, grad_v_seq, grad_w_seq, grad_v_last, grad_w_last,
                                                    h_seq, v_init, *ctx.scalars)
-    return (gx, gv if ctx.needs_input_grad[1] else None, gw if ctx.needs_input_grad[2] else None) + (None,) * 8
+    return (gx, gv if ctx.needs_input_grad[1] else None, gw if ctx.needs_input_grad[2] else None) + (None,) * 9
 
 
 torch.library.register_autograd("sj::hip_multistep_izhikevich_forward", _backward, setup_context=_setup_context)

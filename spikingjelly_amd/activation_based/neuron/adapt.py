@@ -86,7 +86,7 @@ class IzhikevichNode(AdaptBaseNode):
     def _hip(self, x_seq, v, w, store_state_seq: bool):
         return functional.izhikevich_multi_step_hip(x_seq, v, w, self.tau, self.v_threshold, self.v_reset, self.v_rest,
                                                     self.a, self.b, self.tau_w, self.v_c, self.a0, self.detach_reset,
-                                                    self.surrogate_function, store_state_seq)
+                                                    self.surrogate_function, store_state_seq, False)
 
     def multi_step_functional_forward(self, inputs, states, **kwargs):
         if self.backend == "hip":

@@ -31,7 +31,7 @@ struct AaifArgs {
 
 template <typename S, bool VECTOR, bool ROUND_EACH>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) aaif_forward_kernel(const AaifArgs a) {
-  typedef Acc<S, VECTOR, false> A;
+  typedef Acc<S, VECTOR, true> A;  // one read and one write per element, nothing is reused: streaming policy
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
@@ -59,7 +59,7 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) aaif_forward_kernel(const Aai
   const float reset_mul = a.v_reset;  // a Python scalar in torch: fp32 as a factor
 
   float v[V];
-  load_state<S, VECTOR, false>(a.v_init, col, a.v_init_broadcast != 0, v);
+  load_state<S, VECTOR, true>(a.v_init, col, a.v_init_broadcast != 0, v);
 
   for (int64_t t0 = 0; t0 < T; t0 += PF) {
     typename A::raw_t now[PF];
@@ -108,13 +108,16 @@ int launch_typed(const AaifArgs &a, bool vector, bool round_each, hipStream_t st
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "aaif_forward: N=%lld needs %lld blocks", (long long)a.N, (long long)blocks);
   const dim3 grid((unsigned)blocks), threads(block);
+  // the residency rule measured for the other one-read-one-write walk of this library (the ST-BIF kernel): four
+  // resident blocks per compute unit at T >= 16, more for shorter sequences
+  const unsigned lds = occupancy_cap_lds(a.T < 4 ? 0 : (a.T < 16 ? 8 : 4));
   ProfileScope prof(KC_FORWARD, stream);
   if (vector) {
-    if (round_each) hipLaunchKernelGGL((aaif_forward_kernel<S, true, true>), grid, threads, 0, stream, a);
-    else hipLaunchKernelGGL((aaif_forward_kernel<S, true, false>), grid, threads, 0, stream, a);
+    if (round_each) hipLaunchKernelGGL((aaif_forward_kernel<S, true, true>), grid, threads, lds, stream, a);
+    else hipLaunchKernelGGL((aaif_forward_kernel<S, true, false>), grid, threads, lds, stream, a);
   } else {
-    if (round_each) hipLaunchKernelGGL((aaif_forward_kernel<S, false, true>), grid, threads, 0, stream, a);
-    else hipLaunchKernelGGL((aaif_forward_kernel<S, false, false>), grid, threads, 0, stream, a);
+    if (round_each) hipLaunchKernelGGL((aaif_forward_kernel<S, false, true>), grid, threads, lds, stream, a);
+    else hipLaunchKernelGGL((aaif_forward_kernel<S, false, false>), grid, threads, lds, stream, a);
   }
   return check_launch("aaif_forward");
 }

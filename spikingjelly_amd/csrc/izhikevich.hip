@@ -235,13 +235,18 @@ int launch_fwd_typed(const IzhFwdArgs &a, bool vector, bool round_each, hipStrea
   const int64_t blocks = ((a.N + V - 1) / V + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "izhikevich_forward: N=%lld", (long long)a.N);
   const dim3 grid((unsigned)blocks), threads(block);
+  // write-dominated like the LIF forward that saves h_seq: the same residency cap (twice the tuned value, the step
+  // being a longer dependent chain), scaled with T in the same way
+  int cap = 2 * tuning().fwd_blocks_per_cu;
+  if (a.T < 4) cap = 0; else if (a.T < 16) cap *= 2;
+  const unsigned lds = sizeof(S) == 4 ? occupancy_cap_lds(cap) : 0u;
   ProfileScope prof(KC_FORWARD, stream);
   if (vector) {
-    if (round_each) hipLaunchKernelGGL((izhikevich_forward_kernel<S, true, true>), grid, threads, 0, stream, a);
-    else hipLaunchKernelGGL((izhikevich_forward_kernel<S, true, false>), grid, threads, 0, stream, a);
+    if (round_each) hipLaunchKernelGGL((izhikevich_forward_kernel<S, true, true>), grid, threads, lds, stream, a);
+    else hipLaunchKernelGGL((izhikevich_forward_kernel<S, true, false>), grid, threads, lds, stream, a);
   } else {
-    if (round_each) hipLaunchKernelGGL((izhikevich_forward_kernel<S, false, true>), grid, threads, 0, stream, a);
-    else hipLaunchKernelGGL((izhikevich_forward_kernel<S, false, false>), grid, threads, 0, stream, a);
+    if (round_each) hipLaunchKernelGGL((izhikevich_forward_kernel<S, false, true>), grid, threads, lds, stream, a);
+    else hipLaunchKernelGGL((izhikevich_forward_kernel<S, false, false>), grid, threads, lds, stream, a);
   }
   return check_launch("izhikevich_forward");
 }

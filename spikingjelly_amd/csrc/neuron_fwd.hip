@@ -19,11 +19,11 @@ int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   // A short sequence has few rows in flight per work-item and needs more resident blocks instead: twice the cap
   // below 16 steps, none below 4 (measured at T = 1, 2, 4, 8, 16).  ILIF's step is a longer dependent chain (a
   // quotient, a clamp and a rounding on top of the charge): with two resident blocks that latency shows, with four
-  // it is hidden (measured 1.47 -> 1.24 ms at T = 16, N = 33.5 M).
+  // it is hidden (measured 1.47 -> 1.24 ms at T = 16, N = 33.5 M).  The same holds for EIF's exp().
   const bool several_outputs = a.v_seq != nullptr || a.h != nullptr;
   int cap = tuning().fwd_blocks_per_cu;
   if (a.T < 4) cap = 0;
-  else if (a.T < 16 || a.soft_reset == RESET_COUNT) cap *= 2;
+  else if (a.T < 16 || a.soft_reset == RESET_COUNT || a.charge == CH_EIF_DIV || a.charge == CH_EIF_MUL) cap *= 2;
   const unsigned lds = (sizeof(S) == 4 && several_outputs) ? occupancy_cap_lds(cap) : 0u;
   ProfileScope prof(KC_FORWARD, stream);
   if (vector)

@@ -46,7 +46,7 @@ def test_forward_bit_exact_and_gradients_fp32(p, v_reset, T, N, detach):
     soft = v_reset is None
     xd, vd, wd = x.cuda().requires_grad_(), v0.cuda().requires_grad_(), w0.cuda().requires_grad_()
     s, v_seq, w_seq, v_last, w_last, h = IK.hip_multistep_izhikevich_forward(xd, vd, wd, _scalars(p, vth, v_reset), soft,
-                                                                            detach, 1, 2.0, True, True, 0)
+                                                                            detach, 1, 2.0, True, True, True, 0)
     assert bits_equal(s.cpu(), es.detach()) and bits_equal(h.cpu(), eh.detach())
     assert bits_equal(v_seq.cpu(), ev.detach()) and bits_equal(w_seq.cpu(), ew.detach())
     assert bits_equal(v_last.cpu(), ev[-1].detach()) and bits_equal(w_last.cpu(), ew[-1].detach())
@@ -68,7 +68,7 @@ def test_last_state_gradients_without_state_sequences(sg_name, sg_id, alpha):
     torch.autograd.backward([es, ev[-1], ew[-1]], [gs, gvl, gwl])
     xd, vd, wd = x.cuda().requires_grad_(), v0.cuda().requires_grad_(), w0.cuda().requires_grad_()
     s, v_seq, w_seq, v_last, w_last, _ = IK.hip_multistep_izhikevich_forward(xd, vd, wd, _scalars(p, 1.0, -0.1), False, False,
-                                                                            sg_id, alpha, False, True, 0)
+                                                                            sg_id, alpha, False, False, True, 0)
     assert v_seq.numel() == 0 and w_seq.numel() == 0
     torch.autograd.backward([s, v_last, w_last], [gs.cuda(), gvl.cuda(), gwl.cuda()])
     torch.testing.assert_close(xd.grad.cpu(), xr.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
@@ -84,7 +84,7 @@ def test_every_op_rounded_16bit_equals_torch_ops_on_half_tensors(dtype, T, N):
     v0, w0 = seeded_randn((N,), 22, 0.0, 0.2).to(dtype), seeded_randn((N,), 23, 0.0, 0.2).to(dtype)
     es, ev, ew, eh = no.izhikevich_multi_step(x, v0, w0, p, 1.0, -0.1)
     s, v_seq, w_seq, _, _, h = IK.hip_multistep_izhikevich_forward(x.cuda(), v0.cuda(), w0.cuda(), _scalars(p, 1.0, -0.1),
-                                                                  False, False, 1, 2.0, True, True, 0)
+                                                                  False, False, 1, 2.0, True, True, True, 0)
     assert bits_equal(s.cpu(), es) and bits_equal(h.cpu(), eh)
     assert bits_equal(v_seq.cpu(), ev) and bits_equal(w_seq.cpu(), ew)
 

@@ -79,7 +79,7 @@ def test_izhikevich_op():
     w0 = torch.zeros(32, device="cuda", requires_grad=True)
     scalars = [2.0, 1.0, 0.0, -0.1, 0.8, 1.0, 3.0, 0.3, 0.2]
     for store in (False, True):
-        torch.library.opcheck(hip_multistep_izhikevich_forward, (x, v0, w0, scalars, False, False, 1, 2.0, store, True, 0),
+        torch.library.opcheck(hip_multistep_izhikevich_forward, (x, v0, w0, scalars, False, False, 1, 2.0, store, store, True, 0),
                               test_utils=TESTS)
 
 
