@@ -28,9 +28,13 @@ def _eager_step(node, x, gs):
     (neuron.LIFNode, {"tau": 2.0}),
     (neuron.ParametricLIFNode, {"init_tau": 2.0}),
     (neuron.QIFNode, {"tau": 2.0}),
+    (neuron.EIFNode, {"tau": 2.0}),
+    (neuron.IzhikevichNode, {"tau": 2.0, "a": 0.3, "b": 0.2}),
+    (neuron.ILIFNode, {"surrogate_function": surrogate.MultiLevelSpikeCount(4)}),
 ])
 def test_training_step_replays_from_a_graph(cls, kw):
-    node = cls(step_mode="m", backend="hip", surrogate_function=surrogate.ATan(), **kw).cuda()
+    kw = {"surrogate_function": surrogate.ATan(), **kw}
+    node = cls(step_mode="m", backend="hip", **kw).cuda()
     T, B, C = 4, 64, 128
     static_x = seeded_randn((T, B, C), 1, 0.5, 1.0).cuda().requires_grad_()
     static_gs = seeded_randn((T, B, C), 2).cuda()
@@ -90,3 +94,53 @@ def test_inference_with_packed_spikes_replays_from_a_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(static_bits, want_bits) and bits_equal(static_v, want_v), f"replay {i}"
+
+
+def test_self_attention_block_with_packed_spikes_replays_from_a_graph():
+    """The fused LIF -> contraction step (bit-packed spikes in between) inside a captured training step of the block."""
+    from spikingjelly_amd.activation_based import layer
+
+    torch.manual_seed(3)
+    block = layer.SpikingSelfAttention(128, 4, backend="hip").cuda()
+    with torch.no_grad():
+        block.qkv_conv_bn[1].weight.fill_(2.0)
+        block.proj_conv_bn[1].weight.fill_(3.0)
+    for m in block.modules():  # keep the running statistics out of the comparison
+        if isinstance(m, torch.nn.BatchNorm1d):
+            m.momentum = 0.0
+    shape = (4, 8, 128, 96)
+    static_x = seeded_randn(shape, 1).cuda().requires_grad_()
+    static_g = seeded_randn(shape, 2).cuda()
+
+    def step(x, g):
+        y = block(x)
+        y.backward(g)
+        functional.reset_net(block)
+        return y
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step(static_x, static_g)
+            static_x.grad = None
+            block.zero_grad(set_to_none=True)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = step(static_x, static_g)
+    static_gx = static_x.grad
+    for i in range(3):
+        x, g = seeded_randn(shape, 10 + i).cuda(), seeded_randn(shape, 20 + i).cuda()
+        xi = x.clone().requires_grad_()
+        want = step(xi, g).detach().clone()
+        want_gx = xi.grad.clone()
+        block.zero_grad(set_to_none=True)
+        torch.cuda.synchronize()
+        with torch.no_grad():
+            static_x.copy_(x)
+            static_g.copy_(g)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert bits_equal(static_y.detach(), want) and float(want.mean()) > 0.02, f"replay {i}: output"
+        assert bits_equal(static_gx, want_gx), f"replay {i}: grad_x"
