@@ -154,7 +154,7 @@ def other_workload(args) -> int:
             node = neuron.IzhikevichNode(tau=2.0, a=0.3, b=0.2, tau_w=3.0, surrogate_function=surrogate.ATan(2.0),
                                          step_mode="m", backend="hip", store_v_seq=True).to(dev)
             label, what = "Izhikevich", ("IzhikevichNode tau=2, v_c=0.8, a0=1, tau_w=3, a=0.3, b=0.2, hard reset 0, ATan(2), "
-                                         "x [16,256,128,32,32] fp32 ~N(0.4,0.6); h_seq saved (no replay)")
+                                         "x [16,256,128,32,32] fp32 ~N(0.4,0.6)")
         else:
             x = (torch.randn(shape, generator=g, device=dev) * 1.5 + 1.0).requires_grad_()
             node = neuron.ILIFNode(tau=4.0 / 3.0, surrogate_function=surrogate.MultiLevelSpikeCount(4), step_mode="m",
@@ -173,7 +173,7 @@ def other_workload(args) -> int:
         f_ms, b_ms = _kernel_ms(L, L.KC_FORWARD), _kernel_ms(L, L.KC_BACKWARD)
         bytes_each = 16 * T * N + 4 * N
         if args.workload == "izhikevich":
-            bytes_each = 16 * T * N + 16 * N  # x, s, v_seq, h_seq / grad_s, grad_v, h_seq, grad_x; two states in and out
+            bytes_each = 16 * T * N + 16 * N  # backward: grad_s, grad_v, x (replayed into h) in, grad_x out; two states in and out
         dom = "forward" if f_ms >= b_ms else "backward"
         d_ms = max(f_ms, b_ms)
         _emit(args, f"neuron-steps/sec {label} fwd+bwd fp32 T=16 N=33.5M, 1 MI355X", "neuron-steps/s",

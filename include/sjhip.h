@@ -278,6 +278,15 @@ int sjhip_izhikevich_backward(int dtype, const sjhip_izhikevich_params *p, int64
                               const void *grad_spike_seq, const void *grad_v_seq, const void *grad_w_seq,
                               const void *grad_v_last, const void *grad_w_last, const void *h_seq, const void *v_init,
                               void *grad_x_seq, void *grad_v_init, void *grad_w_init, void *stream);
+/* The same backward without a saved h_seq: the kernel replays the forward from x_seq, v_init and w_init (the forward's
+ * own arithmetic, so the replayed h has its bits), keeps h of every step in LDS and then walks back.  The forward can
+ * then be called with h_seq = NULL.  Limits of sjhip_recompute_supported(dtype, T, N); every tensor 16-byte aligned.
+ * The reference's kernel always saves h_seq (multi_step/izhikevich.py); this variant has no counterpart there. */
+int sjhip_izhikevich_backward_replay(int dtype, const sjhip_izhikevich_params *p, int64_t T, int64_t N,
+                                     const void *x_seq, const void *v_init, const void *w_init,
+                                     const void *grad_spike_seq, const void *grad_v_seq, const void *grad_w_seq,
+                                     const void *grad_v_last, const void *grad_w_last,
+                                     void *grad_x_seq, void *grad_v_init, void *grad_w_init, void *stream);
 
 /*
  * Activation-aware IF (ANN2SNN activation-aware redistribution): an IF neuron whose threshold and membrane offset are

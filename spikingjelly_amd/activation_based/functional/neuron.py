@@ -420,9 +420,11 @@ def izhikevich_multi_step_hip(x_seq: torch.Tensor, v: torch.Tensor, w: torch.Ten
     scalars = [float(tau), float(v_threshold), 0.0 if soft else float(v_reset), float(v_rest), float(v_c), float(a0),
                float(tau_w), float(a), float(b)]
     keep_w = store_state_seq if store_w_seq is None else bool(store_w_seq)
+    x2 = x_seq.flatten(1)
+    replay = need_grad and _hip_recompute(x2)
     s, v_seq, w_seq, v_last, w_last, _ = IK.hip_multistep_izhikevich_forward(
-        x_seq.flatten(1), v.flatten(), w.flatten(), scalars, soft, detach_reset, sg_id, sg_alpha, store_state_seq, keep_w,
-        need_grad, _hip_mode_flags(x_seq))
+        x2, v.flatten(), w.flatten(), scalars, soft, detach_reset, sg_id, sg_alpha, store_state_seq, keep_w,
+        need_grad and not replay, _hip_mode_flags(x_seq), replay)
     state = x_seq.shape[1:]
     return (s.reshape(x_seq.shape), v_last.reshape(state), w_last.reshape(state),
             v_seq.reshape(x_seq.shape) if store_state_seq else None, w_seq.reshape(x_seq.shape) if keep_w else None)

@@ -52,6 +52,7 @@ EXPORTED_SYMBOLS = (
     "sjhip_aaif_forward",
     "sjhip_izhikevich_forward",
     "sjhip_izhikevich_backward",
+    "sjhip_izhikevich_backward_replay",
     "sjhip_bit_pack",
     "sjhip_bit_unpack",
     "sjhip_set_tuning",
@@ -171,6 +172,9 @@ def load() -> ctypes.CDLL:
         lib.sjhip_izhikevich_forward.argtypes = [c_int, POINTER(IzhikevichParams), c_int64, c_int64] + [c_void_p] * 10
         lib.sjhip_izhikevich_backward.restype = c_int
         lib.sjhip_izhikevich_backward.argtypes = [c_int, POINTER(IzhikevichParams), c_int64, c_int64] + [c_void_p] * 11
+        lib.sjhip_izhikevich_backward_replay.restype = c_int
+        lib.sjhip_izhikevich_backward_replay.argtypes = ([c_int, POINTER(IzhikevichParams), c_int64, c_int64]
+                                                         + [c_void_p] * 12)
         lib.sjhip_bit_pack.restype = c_int
         lib.sjhip_bit_pack.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p]
         lib.sjhip_bit_unpack.restype = c_int

@@ -49,8 +49,44 @@ struct IzhBwdArgs {
   int sg, soft_reset, detach_reset, v_broadcast;
 };
 
-template <typename S, bool VECTOR, bool ROUND_EACH>
-__global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_forward_kernel(const IzhFwdArgs a) {
+// The step is compiled once per combination of three launch-uniform choices, so that its body is straight-line code
+// and the V neurons of a work-item interleave (a uniform branch inside the step would serialise them):
+// bit 0: 1/tau is exact, multiply instead of divide; bit 1: the same for tau_w; bit 2: soft reset.
+constexpr int IZH_TAU_MUL = 1, IZH_TAUW_MUL = 2, IZH_SOFT = 4, IZH_VARIANTS = 8;
+__device__ __forceinline__ int izhikevich_variant(const IzhFwdArgs &a) {
+  return (a.tau_mul ? IZH_TAU_MUL : 0) | (a.tau_w_mul ? IZH_TAUW_MUL : 0) | (a.soft_reset ? IZH_SOFT : 0);
+}
+
+// One step of one neuron in torch's op order; every result is rounded to R (the storage dtype when every op is
+// rounded, fp32 otherwise).  The forward kernel and the replaying backward share it, so a replayed h_t has the
+// forward's bits.
+template <typename R, int VAR>
+__device__ __forceinline__ void izhikevich_step(const IzhFwdArgs &a, float x, float &v, float &w, float &h, float &s) {
+#pragma clang fp contract(off)
+  const float d1 = Cvt<R>::round(v - a.rest_sub);
+  const float m1 = scalar_product<R>(a.a0, d1);
+  const float d2 = Cvt<R>::round(v - a.c_sub);
+  const float m2 = Cvt<R>::round(m1 * d2);
+  const float e = Cvt<R>::round(Cvt<R>::round(x + m2) - w);
+  const float f = (VAR & IZH_TAU_MUL) ? scalar_product<R>(a.tau, e) : Cvt<R>::round(e / a.tau);
+  h = Cvt<R>::round(v + f);
+  const float p = Cvt<R>::round(h - a.rest_sub);
+  const float r = Cvt<R>::round(scalar_product<R>(a.a, p) - w);
+  const float u = (VAR & IZH_TAUW_MUL) ? scalar_product<R>(a.tau_w, r) : Cvt<R>::round(r / a.tau_w);
+  const float wn = Cvt<R>::round(w + u);
+  const float over = Cvt<R>::round(h - a.vth_sub);
+  s = (over >= 0.0f) ? 1.0f : 0.0f;
+  if constexpr ((VAR & IZH_SOFT) != 0) {
+    v = Cvt<R>::round(h - scalar_product<R>(a.vth_mul, s));
+  } else {
+    const float keep = Cvt<R>::round(Cvt<R>::round(1.0f - s) * h);
+    v = Cvt<R>::round(keep + scalar_product<R>(a.vr_mul, s));
+  }
+  w = Cvt<R>::round(wn + scalar_product<R>(a.b, s));
+}
+
+template <typename S, bool VECTOR, bool ROUND_EACH, int VAR>
+__device__ __forceinline__ void izhikevich_forward_walk(const IzhFwdArgs &a, int64_t col) {
   typedef Acc<S, VECTOR, false> A;
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
@@ -58,8 +94,6 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_forward_kernel(con
   constexpr int PF = SJHIP_IZH_PF;
 
   const int64_t N = a.N, T = a.T;
-  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
-  if (col >= N) return;
   const E *xp = (const E *)a.x + col;
 
   typename A::raw_t ahead[PF];
@@ -85,29 +119,7 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_forward_kernel(con
         float x[V], h[V], s[V];
         A::unpack(now[i], x);
 #pragma unroll
-        for (int j = 0; j < V; ++j) {
-#pragma clang fp contract(off)
-          const float d1 = Cvt<R>::round(v[j] - a.rest_sub);
-          const float m1 = scalar_product<R>(a.a0, d1);
-          const float d2 = Cvt<R>::round(v[j] - a.c_sub);
-          const float m2 = Cvt<R>::round(m1 * d2);
-          const float e = Cvt<R>::round(Cvt<R>::round(x[j] + m2) - w[j]);
-          const float f = a.tau_mul ? scalar_product<R>(a.tau, e) : Cvt<R>::round(e / a.tau);
-          h[j] = Cvt<R>::round(v[j] + f);
-          const float p = Cvt<R>::round(h[j] - a.rest_sub);
-          const float r = Cvt<R>::round(scalar_product<R>(a.a, p) - w[j]);
-          const float u = a.tau_w_mul ? scalar_product<R>(a.tau_w, r) : Cvt<R>::round(r / a.tau_w);
-          const float wn = Cvt<R>::round(w[j] + u);
-          const float over = Cvt<R>::round(h[j] - a.vth_sub);
-          s[j] = (over >= 0.0f) ? 1.0f : 0.0f;
-          if (a.soft_reset) {
-            v[j] = Cvt<R>::round(h[j] - scalar_product<R>(a.vth_mul, s[j]));
-          } else {
-            const float keep = Cvt<R>::round(Cvt<R>::round(1.0f - s[j]) * h[j]);
-            v[j] = Cvt<R>::round(keep + scalar_product<R>(a.vr_mul, s[j]));
-          }
-          w[j] = Cvt<R>::round(wn + scalar_product<R>(a.b, s[j]));
-        }
+        for (int j = 0; j < V; ++j) izhikevich_step<R, VAR>(a, x[j], v[j], w[j], h[j], s[j]);
         A::store_spikes((E *)a.spike + col + t * N, s);
         if (a.h) A::store((E *)a.h + col + t * N, h);
         if (a.v_seq) A::store((E *)a.v_seq + col + t * N, v);
@@ -119,66 +131,139 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_forward_kernel(con
   A::store((E *)a.w_last + col, w);
 }
 
-__device__ __forceinline__ float surrogate_grad_any(int sg, float x, float alpha) {
-  switch (sg) {
-    case SJHIP_SG_SIGMOID: return surrogate_grad<SJHIP_SG_SIGMOID, false>(x, alpha);
-    case SJHIP_SG_ATAN: return surrogate_grad<SJHIP_SG_ATAN, false>(x, alpha);
-    case SJHIP_SG_PIECEWISE_QUADRATIC: return surrogate_grad<SJHIP_SG_PIECEWISE_QUADRATIC, false>(x, alpha);
-    case SJHIP_SG_PIECEWISE_EXP: return surrogate_grad<SJHIP_SG_PIECEWISE_EXP, false>(x, alpha);
-    case SJHIP_SG_SOFT_SIGN: return surrogate_grad<SJHIP_SG_SOFT_SIGN, false>(x, alpha);
-    case SJHIP_SG_SUPER_SPIKE: return surrogate_grad<SJHIP_SG_SUPER_SPIKE, false>(x, alpha);
-    default: return surrogate_grad<SJHIP_SG_ERF, false>(x, alpha);
+template <typename S, bool VECTOR, bool ROUND_EACH>
+__global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_forward_kernel(const IzhFwdArgs a) {
+  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * Acc<S, VECTOR, false>::V;
+  if (col >= a.N) return;
+  switch (izhikevich_variant(a)) {
+    case 0: izhikevich_forward_walk<S, VECTOR, ROUND_EACH, 0>(a, col); break;
+    case 1: izhikevich_forward_walk<S, VECTOR, ROUND_EACH, 1>(a, col); break;
+    case 2: izhikevich_forward_walk<S, VECTOR, ROUND_EACH, 2>(a, col); break;
+    case 3: izhikevich_forward_walk<S, VECTOR, ROUND_EACH, 3>(a, col); break;
+    case 4: izhikevich_forward_walk<S, VECTOR, ROUND_EACH, 4>(a, col); break;
+    case 5: izhikevich_forward_walk<S, VECTOR, ROUND_EACH, 5>(a, col); break;
+    case 6: izhikevich_forward_walk<S, VECTOR, ROUND_EACH, 6>(a, col); break;
+    default: izhikevich_forward_walk<S, VECTOR, ROUND_EACH, 7>(a, col); break;
   }
 }
 
-template <typename S, bool VECTOR>
-__global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_backward_kernel(const IzhBwdArgs a) {
+// Replays the forward recurrence of one work-item (four neurons) from x_seq, v_init and w_init and parks h_t of every
+// step in LDS as fp32; each work-item touches only its own LDS words, so no barrier is needed.
+template <typename S, bool ROUND_EACH, int VAR>
+__device__ __forceinline__ void izhikevich_replay(const IzhFwdArgs &a, f32x4 *lds_h, int64_t col) {
+  typedef Acc<S, true, true> A;
+  typedef typename A::elem_t E;
+  typedef typename std::conditional<ROUND_EACH, S, float>::type R;
+  constexpr int V = A::V;
+  static_assert(V == 4, "the replay parks one f32x4 per work-item and step");
+  constexpr int PF = SJHIP_IZH_PF;
+
+  const int64_t N = a.N, T = a.T;
+  const E *xp = (const E *)a.x + col;
+  typename A::raw_t ahead[PF];
+#pragma unroll
+  for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? A::load(xp + (int64_t)i * N) : A::zero();
+  float v[V], w[V];
+  load_state<S, true, true>(a.v_init, col, a.v_broadcast != 0, v);
+  load_state<S, true, true>(a.w_init, col, a.w_broadcast != 0, w);
+  for (int64_t t0 = 0; t0 < T; t0 += PF) {
+    typename A::raw_t now[PF];
+#pragma unroll
+    for (int i = 0; i < PF; ++i) now[i] = ahead[i];
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int64_t tn = t0 + PF + i;
+      if (tn < T) ahead[i] = A::load(xp + tn * N);
+    }
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int64_t t = t0 + i;
+      if (t < T) {
+        float x[V], h[V], s[V];
+        A::unpack(now[i], x);
+#pragma unroll
+        for (int j = 0; j < V; ++j) izhikevich_step<R, VAR>(a, x[j], v[j], w[j], h[j], s[j]);
+        f32x4 park; park.x = h[0]; park.y = h[1]; park.z = h[2]; park.w = h[3];
+        lds_h[(int)t * (int)blockDim.x + (int)threadIdx.x] = park;
+      }
+    }
+  }
+}
+
+// The first rows of the upstream gradients (and of a saved h_seq) of one work-item, requested before anything else so
+// that they arrive while h is being replayed.
+template <typename S, bool VECTOR, bool REPLAY>
+struct IzhPrologue {
+  typedef Acc<S, VECTOR, true> A;
+  typedef typename A::elem_t E;
+  static constexpr int V = A::V;
+  static constexpr int PF = SJHIP_IZH_PF;
+  typename A::raw_t gs[PF], h[PF], gv[PF], gw[PF];
+  float gv_last[V], gw_last[V];
+
+  __device__ __forceinline__ void load(const IzhBwdArgs &a, int64_t col) {
+    const int64_t N = a.N, T = a.T;
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int64_t t = T - 1 - i;
+      gs[i] = (t >= 0) ? A::load((const E *)a.grad_spike + col + t * N) : A::zero();
+      if (!REPLAY) h[i] = (t >= 0) ? A::load((const E *)a.h + col + t * N) : A::zero();
+      if (a.grad_v_seq) gv[i] = (t >= 0) ? A::load((const E *)a.grad_v_seq + col + t * N) : A::zero();
+      if (a.grad_w_seq) gw[i] = (t >= 0) ? A::load((const E *)a.grad_w_seq + col + t * N) : A::zero();
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) { gv_last[j] = 0.0f; gw_last[j] = 0.0f; }
+    if (a.grad_v_last) A::unpack(A::load((const E *)a.grad_v_last + col), gv_last);
+    if (a.grad_w_last) A::unpack(A::load((const E *)a.grad_w_last + col), gw_last);
+  }
+};
+
+// The BPTT walk of one work-item for surrogate SG.  REPLAY: h_t comes from LDS, otherwise from the saved h_seq.
+// The two reset rules share one expression whose coefficients are chosen once per launch, so the per-neuron code has
+// no branch:
+//     v_t  = s ? fire_h h + fire_c : h            soft: h - v_th            hard: v_reset
+//     dvdh = (1 - s hard) + sg (d_c + d_h h)      soft: 1 - live v_th sg    hard: (1 - s) + sg (v_reset - live h)
+template <typename S, bool VECTOR, bool REPLAY, int SG>
+__device__ __forceinline__ void izhikevich_bptt_walk(const IzhBwdArgs &a, const f32x4 *lds_h, int64_t col,
+                                                     IzhPrologue<S, VECTOR, REPLAY> &pre) {
   typedef Acc<S, VECTOR, true> A;
   typedef typename A::elem_t E;
   constexpr int V = A::V;
   constexpr int PF = SJHIP_IZH_PF;
 
   const int64_t N = a.N, T = a.T;
-  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
-  if (col >= N) return;
   const E *gsp = (const E *)a.grad_spike + col;
-  const E *hp = (const E *)a.h + col;
+  const E *hp = REPLAY ? nullptr : (const E *)a.h + col;
   const E *gvp = a.grad_v_seq ? (const E *)a.grad_v_seq + col : nullptr;
   const E *gwp = a.grad_w_seq ? (const E *)a.grad_w_seq + col : nullptr;
 
-  typename A::raw_t ahead_gs[PF], ahead_h[PF], ahead_gv[PF], ahead_gw[PF];
-#pragma unroll
-  for (int i = 0; i < PF; ++i) {
-    const int64_t t = T - 1 - i;
-    ahead_gs[i] = (t >= 0) ? A::load(gsp + t * N) : A::zero();
-    ahead_h[i] = (t >= 0) ? A::load(hp + t * N) : A::zero();
-    if (gvp) ahead_gv[i] = (t >= 0) ? A::load(gvp + t * N) : A::zero();
-    if (gwp) ahead_gw[i] = (t >= 0) ? A::load(gwp + t * N) : A::zero();
-  }
+  const float live = a.detach_reset ? 0.0f : 1.0f;
+  const float hard = a.soft_reset ? 0.0f : 1.0f;
+  const float fire_h = a.soft_reset ? 1.0f : 0.0f, fire_c = a.soft_reset ? -a.v_th : a.v_reset;
+  const float d_c = a.soft_reset ? -live * a.v_th : a.v_reset, d_h = a.soft_reset ? 0.0f : -live;
+  const float k = a.k, kw = a.kw, ka0 = a.k * a.a0, kwa = a.kw * a.a;
 
-  float gh_next[V], cw_next[V], gv_last[V];
+  float gh_next[V], cw_next[V];
 #pragma unroll
-  for (int j = 0; j < V; ++j) { gh_next[j] = 0.0f; cw_next[j] = 0.0f; gv_last[j] = 0.0f; }
-  if (a.grad_v_last) A::unpack(A::load((const E *)a.grad_v_last + col), gv_last);
-  if (a.grad_w_last) A::unpack(A::load((const E *)a.grad_w_last + col), cw_next);
+  for (int j = 0; j < V; ++j) { gh_next[j] = 0.0f; cw_next[j] = pre.gw_last[j]; }
 
-  const float k = a.k, kw = a.kw;
   for (int64_t t0 = T - 1; t0 >= 0; t0 -= PF) {
     typename A::raw_t cur_gs[PF], cur_h[PF], cur_gv[PF], cur_gw[PF];
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
-      cur_gs[i] = ahead_gs[i]; cur_h[i] = ahead_h[i];
-      if (gvp) cur_gv[i] = ahead_gv[i];
-      if (gwp) cur_gw[i] = ahead_gw[i];
+      cur_gs[i] = pre.gs[i];
+      if (!REPLAY) cur_h[i] = pre.h[i];
+      if (gvp) cur_gv[i] = pre.gv[i];
+      if (gwp) cur_gw[i] = pre.gw[i];
     }
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int64_t tn = t0 - PF - i;
       if (tn >= 0) {
-        ahead_gs[i] = A::load(gsp + tn * N);
-        ahead_h[i] = A::load(hp + tn * N);
-        if (gvp) ahead_gv[i] = A::load(gvp + tn * N);
-        if (gwp) ahead_gw[i] = A::load(gwp + tn * N);
+        pre.gs[i] = A::load(gsp + tn * N);
+        if (!REPLAY) pre.h[i] = A::load(hp + tn * N);
+        if (gvp) pre.gv[i] = A::load(gvp + tn * N);
+        if (gwp) pre.gw[i] = A::load(gwp + tn * N);
       }
     }
 #pragma unroll
@@ -187,30 +272,36 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_backward_kernel(co
       if (t >= 0) {
         float gs[V], h[V], gvs[V], gws[V], gx[V];
         A::unpack(cur_gs[i], gs);
-        A::unpack(cur_h[i], h);
+        if constexpr (REPLAY) {
+          const f32x4 park = lds_h[(int)t * (int)blockDim.x + (int)threadIdx.x];
+          h[0] = park.x; h[1] = park.y; h[2] = park.z; h[3] = park.w;
+        } else {
+          A::unpack(cur_h[i], h);
+        }
+#pragma unroll
+        for (int j = 0; j < V; ++j) { gvs[j] = 0.0f; gws[j] = 0.0f; }
         if (gvp) A::unpack(cur_gv[i], gvs);
         if (gwp) A::unpack(cur_gw[i], gws);
+        const bool last = t == T - 1;
 #pragma unroll
         for (int j = 0; j < V; ++j) {
           const float over = h[j] - a.v_th;
-          const float s = (over >= 0.0f) ? 1.0f : 0.0f;
+          const bool fired = over >= 0.0f;
+          const float s = fired ? 1.0f : 0.0f;
           float v_t;
           {
 #pragma clang fp contract(off)
-            v_t = a.soft_reset ? (h[j] - s * a.v_th) : ((1.0f - s) * h[j] + s * a.v_reset);
+            v_t = fired ? (fire_h * h[j] + fire_c) : h[j];
           }
-          const float sg = surrogate_grad_any(a.sg, over, a.alpha);
-          const float dhdv = 1.0f + k * a.a0 * ((v_t - a.v_c) + (v_t - a.v_rest));
-          float gv = (t == T - 1) ? gv_last[j] : gh_next[j] * dhdv;
-          if (gvp) gv += gvs[j];
-          float gw = cw_next[j];  // grad_w_last at t = T-1
-          if (gwp) gw += gws[j];
-          const float live = a.detach_reset ? 0.0f : 1.0f;
-          const float dvdh = a.soft_reset ? (1.0f - live * a.v_th * sg) : ((1.0f - s) + sg * (a.v_reset - live * h[j]));
-          const float gh = gv * dvdh + (gs[j] + a.b * gw) * sg + gw * kw * a.a;
+          const float sg = surrogate_grad<SG, false>(over, a.alpha);
+          const float dhdv = 1.0f + ka0 * ((v_t - a.v_c) + (v_t - a.v_rest));
+          const float gv = (last ? pre.gv_last[j] : gh_next[j] * dhdv) + gvs[j];
+          const float gw = cw_next[j] + gws[j];  // cw_next starts from grad_w_last
+          const float dvdh = (1.0f - s * hard) + sg * (d_c + d_h * h[j]);
+          const float gh = gv * dvdh + (gs[j] + a.b * gw) * sg + gw * kwa;
           gx[j] = gh * k;
           gh_next[j] = gh;
-          cw_next[j] = gw * (1.0f - kw) - gh * k;
+          cw_next[j] = gw * (1.0f - kw) - gx[j];
         }
         A::store((E *)a.grad_x + col + t * N, gx);
       }
@@ -220,10 +311,55 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_backward_kernel(co
     float v0[V];
     load_state<S, VECTOR, true>(a.v_init, col, a.v_broadcast != 0, v0);
 #pragma unroll
-    for (int j = 0; j < V; ++j) gh_next[j] *= 1.0f + k * a.a0 * ((v0[j] - a.v_c) + (v0[j] - a.v_rest));
+    for (int j = 0; j < V; ++j) gh_next[j] *= 1.0f + ka0 * ((v0[j] - a.v_c) + (v0[j] - a.v_rest));
     A::store((E *)a.grad_v_init + col, gh_next);
   }
   if (a.grad_w_init) A::store((E *)a.grad_w_init + col, cw_next);
+}
+
+template <typename S, bool VECTOR, bool REPLAY>
+__device__ __forceinline__ void izhikevich_bptt(const IzhBwdArgs &a, const f32x4 *lds_h, int64_t col,
+                                                IzhPrologue<S, VECTOR, REPLAY> &pre) {
+  switch (a.sg) {
+    case SJHIP_SG_SIGMOID: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_SIGMOID>(a, lds_h, col, pre); break;
+    case SJHIP_SG_ATAN: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_ATAN>(a, lds_h, col, pre); break;
+    case SJHIP_SG_PIECEWISE_QUADRATIC: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_PIECEWISE_QUADRATIC>(a, lds_h, col, pre); break;
+    case SJHIP_SG_PIECEWISE_EXP: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_PIECEWISE_EXP>(a, lds_h, col, pre); break;
+    case SJHIP_SG_SOFT_SIGN: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_SOFT_SIGN>(a, lds_h, col, pre); break;
+    case SJHIP_SG_SUPER_SPIKE: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_SUPER_SPIKE>(a, lds_h, col, pre); break;
+    default: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_ERF>(a, lds_h, col, pre); break;
+  }
+}
+
+template <typename S, bool VECTOR>
+__global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_backward_kernel(const IzhBwdArgs a) {
+  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * Acc<S, VECTOR, true>::V;
+  if (col >= a.N) return;
+  IzhPrologue<S, VECTOR, false> pre;
+  pre.load(a, col);
+  izhikevich_bptt<S, VECTOR, false>(a, nullptr, col, pre);
+}
+
+// Backward that recomputes h instead of reading a saved h_seq: the forward then never writes h_seq and this kernel
+// reads x_seq in its place.  S is fp32 or a four-neurons-per-work-item 16-bit type; LDS holds T * blockDim * 16 bytes.
+template <typename S, bool ROUND_EACH>
+__global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_backward_replay_kernel(const IzhFwdArgs f, const IzhBwdArgs a) {
+  extern __shared__ f32x4 izh_lds_h[];
+  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (col >= a.N) return;
+  IzhPrologue<S, true, true> pre;
+  pre.load(a, col);
+  switch (izhikevich_variant(f)) {
+    case 0: izhikevich_replay<S, ROUND_EACH, 0>(f, izh_lds_h, col); break;
+    case 1: izhikevich_replay<S, ROUND_EACH, 1>(f, izh_lds_h, col); break;
+    case 2: izhikevich_replay<S, ROUND_EACH, 2>(f, izh_lds_h, col); break;
+    case 3: izhikevich_replay<S, ROUND_EACH, 3>(f, izh_lds_h, col); break;
+    case 4: izhikevich_replay<S, ROUND_EACH, 4>(f, izh_lds_h, col); break;
+    case 5: izhikevich_replay<S, ROUND_EACH, 5>(f, izh_lds_h, col); break;
+    case 6: izhikevich_replay<S, ROUND_EACH, 6>(f, izh_lds_h, col); break;
+    default: izhikevich_replay<S, ROUND_EACH, 7>(f, izh_lds_h, col); break;
+  }
+  izhikevich_bptt<S, true, true>(a, izh_lds_h, col, pre);
 }
 
 namespace {
@@ -273,14 +409,10 @@ bool all_aligned(std::initializer_list<const void *> ptrs) {
   return true;
 }
 
-}  // namespace
-
-int launch_izhikevich_forward(int dtype, const sjhip_izhikevich_params &p, int64_t T, int64_t N, const void *x_seq,
-                              const void *v_init, const void *w_init, void *spike_seq, void *v_seq, void *w_seq,
-                              void *v_last, void *w_last, void *h_seq, hipStream_t stream) {
-  IzhFwdArgs a;
+bool build_forward_args(IzhFwdArgs &a, int dtype, const sjhip_izhikevich_params &p, int64_t T, int64_t N,
+                        const void *x_seq, const void *v_init, const void *w_init) {
   a.x = x_seq; a.v_init = v_init; a.w_init = w_init;
-  a.spike = spike_seq; a.v_seq = v_seq; a.w_seq = w_seq; a.v_last = v_last; a.w_last = w_last; a.h = h_seq;
+  a.spike = nullptr; a.v_seq = nullptr; a.w_seq = nullptr; a.v_last = nullptr; a.w_last = nullptr; a.h = nullptr;
   a.T = T; a.N = N;
   a.tau_mul = exact_reciprocal(p.tau) ? 1 : 0;
   a.tau = a.tau_mul ? 1.0f / p.tau : p.tau;
@@ -296,6 +428,32 @@ int launch_izhikevich_forward(int dtype, const sjhip_izhikevich_params &p, int64
   a.soft_reset = (p.flags & SJHIP_FLAG_SOFT_RESET) ? 1 : 0;
   a.v_broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) ? 1 : 0;
   a.w_broadcast = (p.flags & SJHIP_FLAG_W_INIT_BROADCAST) ? 1 : 0;
+  return round_each;
+}
+
+void build_backward_args(IzhBwdArgs &a, const sjhip_izhikevich_params &p, int64_t T, int64_t N, const void *grad_spike_seq,
+                         const void *grad_v_seq, const void *grad_w_seq, const void *grad_v_last, const void *grad_w_last,
+                         const void *h_seq, const void *v_init, void *grad_x_seq, void *grad_v_init, void *grad_w_init) {
+  a.grad_spike = grad_spike_seq; a.grad_v_seq = grad_v_seq; a.grad_w_seq = grad_w_seq;
+  a.grad_v_last = grad_v_last; a.grad_w_last = grad_w_last; a.h = h_seq; a.v_init = v_init;
+  a.grad_x = grad_x_seq; a.grad_v_init = grad_v_init; a.grad_w_init = grad_w_init;
+  a.T = T; a.N = N;
+  a.k = (float)(1.0 / (double)p.tau); a.kw = (float)(1.0 / (double)p.tau_w);
+  a.a0 = p.a0; a.a = p.a; a.b = p.b; a.v_rest = p.v_rest; a.v_c = p.v_c;
+  a.v_th = p.v_threshold; a.v_reset = p.v_reset; a.alpha = p.sg_alpha; a.sg = p.sg_id;
+  a.soft_reset = (p.flags & SJHIP_FLAG_SOFT_RESET) ? 1 : 0;
+  a.detach_reset = (p.flags & SJHIP_FLAG_DETACH_RESET) ? 1 : 0;
+  a.v_broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) ? 1 : 0;
+}
+
+}  // namespace
+
+int launch_izhikevich_forward(int dtype, const sjhip_izhikevich_params &p, int64_t T, int64_t N, const void *x_seq,
+                              const void *v_init, const void *w_init, void *spike_seq, void *v_seq, void *w_seq,
+                              void *v_last, void *w_last, void *h_seq, hipStream_t stream) {
+  IzhFwdArgs a;
+  const bool round_each = build_forward_args(a, dtype, p, T, N, x_seq, v_init, w_init);
+  a.spike = spike_seq; a.v_seq = v_seq; a.w_seq = w_seq; a.v_last = v_last; a.w_last = w_last; a.h = h_seq;
   const int V = dtype == SJHIP_F32 ? 4 : 8;
   const bool vector = (N % V == 0) && all_aligned({x_seq, spike_seq, v_seq, w_seq, v_last, w_last, h_seq}) &&
                       (a.v_broadcast || aligned16(v_init)) && (a.w_broadcast || aligned16(w_init));
@@ -312,16 +470,8 @@ int launch_izhikevich_backward(int dtype, const sjhip_izhikevich_params &p, int6
                                const void *grad_v_last, const void *grad_w_last, const void *h_seq, const void *v_init,
                                void *grad_x_seq, void *grad_v_init, void *grad_w_init, hipStream_t stream) {
   IzhBwdArgs a;
-  a.grad_spike = grad_spike_seq; a.grad_v_seq = grad_v_seq; a.grad_w_seq = grad_w_seq;
-  a.grad_v_last = grad_v_last; a.grad_w_last = grad_w_last; a.h = h_seq; a.v_init = v_init;
-  a.grad_x = grad_x_seq; a.grad_v_init = grad_v_init; a.grad_w_init = grad_w_init;
-  a.T = T; a.N = N;
-  a.k = (float)(1.0 / (double)p.tau); a.kw = (float)(1.0 / (double)p.tau_w);
-  a.a0 = p.a0; a.a = p.a; a.b = p.b; a.v_rest = p.v_rest; a.v_c = p.v_c;
-  a.v_th = p.v_threshold; a.v_reset = p.v_reset; a.alpha = p.sg_alpha; a.sg = p.sg_id;
-  a.soft_reset = (p.flags & SJHIP_FLAG_SOFT_RESET) ? 1 : 0;
-  a.detach_reset = (p.flags & SJHIP_FLAG_DETACH_RESET) ? 1 : 0;
-  a.v_broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) ? 1 : 0;
+  build_backward_args(a, p, T, N, grad_spike_seq, grad_v_seq, grad_w_seq, grad_v_last, grad_w_last, h_seq, v_init,
+                      grad_x_seq, grad_v_init, grad_w_init);
   const int V = dtype == SJHIP_F32 ? 4 : 8;
   const bool vector = (N % V == 0) && all_aligned({grad_spike_seq, grad_v_seq, grad_w_seq, grad_v_last, grad_w_last, h_seq,
                                                    grad_x_seq, grad_v_init, grad_w_init}) &&
@@ -332,6 +482,51 @@ int launch_izhikevich_backward(int dtype, const sjhip_izhikevich_params &p, int6
     case SJHIP_BF16: return launch_bwd_typed<bf16_t>(a, vector, stream);
     default: return fail(SJHIP_ERR_INVALID, "izhikevich_backward: dtype %d", dtype);
   }
+}
+
+namespace {
+
+template <typename S>
+void launch_replay_typed(const IzhFwdArgs &f, const IzhBwdArgs &b, bool round_each, int block, unsigned lds,
+                         int64_t blocks, hipStream_t stream) {
+  const dim3 grid((unsigned)blocks), threads(block);
+  if (round_each) hipLaunchKernelGGL((izhikevich_backward_replay_kernel<S, true>), grid, threads, lds, stream, f, b);
+  else hipLaunchKernelGGL((izhikevich_backward_replay_kernel<S, false>), grid, threads, lds, stream, f, b);
+}
+
+}  // namespace
+
+int launch_izhikevich_backward_replay(int dtype, const sjhip_izhikevich_params &p, int64_t T, int64_t N,
+                                      const void *x_seq, const void *v_init, const void *w_init,
+                                      const void *grad_spike_seq, const void *grad_v_seq, const void *grad_w_seq,
+                                      const void *grad_v_last, const void *grad_w_last, void *grad_x_seq,
+                                      void *grad_v_init, void *grad_w_init, hipStream_t stream) {
+  // same LDS footprint per work-item and step as the replay of the one-state neurons (one f32x4), so the same limits
+  if (!recompute_supported(dtype, T, N))
+    return fail(SJHIP_ERR_UNSUPPORTED, "izhikevich_backward(replay): T=%lld N=%lld does not fit (N %% %d != 0 or T too large for LDS)",
+                (long long)T, (long long)N, dtype == SJHIP_F32 ? 4 : 8);
+  IzhFwdArgs f;
+  const bool round_each = build_forward_args(f, dtype, p, T, N, x_seq, v_init, w_init);
+  if (!all_aligned({x_seq, grad_spike_seq, grad_v_seq, grad_w_seq, grad_v_last, grad_w_last, grad_x_seq, grad_v_init, grad_w_init}) ||
+      (!f.v_broadcast && !aligned16(v_init)) || (!f.w_broadcast && !aligned16(w_init)))
+    return fail(SJHIP_ERR_INVALID, "izhikevich_backward(replay): every tensor must be 16-byte aligned");
+  IzhBwdArgs b;
+  build_backward_args(b, p, T, N, grad_spike_seq, grad_v_seq, grad_w_seq, grad_v_last, grad_w_last, nullptr, v_init,
+                      grad_x_seq, grad_v_init, grad_w_init);
+  const int block = recompute_block(dtype, T, round_each);
+  const int64_t blocks = (N / 4 + block - 1) / block;
+  if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "izhikevich_backward(replay): N=%lld", (long long)N);
+  unsigned lds = (unsigned)(T * block * 16);
+  const unsigned cap = occupancy_cap_lds(tuning().replay_blocks_per_cu);
+  if (cap > lds) lds = cap;
+  ProfileScope prof(KC_BACKWARD, stream);
+  switch (dtype) {
+    case SJHIP_F32: launch_replay_typed<float>(f, b, false, block, lds, blocks, stream); break;
+    case SJHIP_F16: launch_replay_typed<f16n_t>(f, b, round_each, block, lds, blocks, stream); break;
+    case SJHIP_BF16: launch_replay_typed<bf16n_t>(f, b, round_each, block, lds, blocks, stream); break;
+    default: return fail(SJHIP_ERR_INVALID, "izhikevich_backward(replay): dtype %d", dtype);
+  }
+  return check_launch("izhikevich_backward(replay)");
 }
 
 }  // namespace sjhip

@@ -21,6 +21,8 @@ constexpr unsigned kMaxLds = 159u * 1024u;  // LDS per compute unit on gfx950 mi
 // (16-bit storage, every op rounded)
 int64_t h_bytes_per_item(int dtype, bool round_each) { (void)dtype; (void)round_each; return 16; }
 
+}  // namespace
+
 // Largest block (128 or 64 lanes) whose h buffer fits in LDS; 0 if none.
 int recompute_block(int dtype, int64_t T, bool round_each) {
   for (int block : {128, 64}) {
@@ -29,8 +31,6 @@ int recompute_block(int dtype, int64_t T, bool round_each) {
   }
   return 0;
 }
-
-}  // namespace
 
 bool recompute_supported(int dtype, int64_t T, int64_t N) {
   const int64_t V = dtype == SJHIP_F32 ? 4 : 8;

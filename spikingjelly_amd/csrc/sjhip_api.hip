@@ -298,6 +298,20 @@ int sjhip_izhikevich_backward(int dtype, const sjhip_izhikevich_params *p, int64
                                     v_init, grad_x_seq, grad_v_init, grad_w_init, static_cast<hipStream_t>(stream));
 }
 
+int sjhip_izhikevich_backward_replay(int dtype, const sjhip_izhikevich_params *p, int64_t T, int64_t N, const void *x_seq,
+                                     const void *v_init, const void *w_init, const void *grad_spike_seq,
+                                     const void *grad_v_seq, const void *grad_w_seq, const void *grad_v_last,
+                                     const void *grad_w_last, void *grad_x_seq, void *grad_v_init, void *grad_w_init,
+                                     void *stream) {
+  int rc = check_izhikevich("izhikevich_backward(replay)", dtype, p, T, N, true);
+  if (rc != SJHIP_OK) return rc;
+  if (!x_seq || !v_init || !w_init || !grad_spike_seq || !grad_x_seq)
+    return fail(SJHIP_ERR_INVALID, "izhikevich_backward(replay): NULL tensor");
+  return launch_izhikevich_backward_replay(dtype, *p, T, N, x_seq, v_init, w_init, grad_spike_seq, grad_v_seq, grad_w_seq,
+                                           grad_v_last, grad_w_last, grad_x_seq, grad_v_init, grad_w_init,
+                                           static_cast<hipStream_t>(stream));
+}
+
 int sjhip_aaif_forward(int dtype, uint32_t flags, int64_t T, int64_t N, const void *x_seq, const void *v_init,
                        const float *v_threshold, int64_t threshold_count, const float *v_offset, int64_t offset_count,
                        int64_t channel_size, int64_t inner_size, float v_reset, void *spike_seq, void *v_seq,

@@ -304,6 +304,11 @@ int launch_izhikevich_backward(int dtype, const sjhip_izhikevich_params &p, int6
                                const void *grad_spike_seq, const void *grad_v_seq, const void *grad_w_seq,
                                const void *grad_v_last, const void *grad_w_last, const void *h_seq, const void *v_init,
                                void *grad_x_seq, void *grad_v_init, void *grad_w_init, hipStream_t stream);
+int launch_izhikevich_backward_replay(int dtype, const sjhip_izhikevich_params &p, int64_t T, int64_t N,
+                                      const void *x_seq, const void *v_init, const void *w_init,
+                                      const void *grad_spike_seq, const void *grad_v_seq, const void *grad_w_seq,
+                                      const void *grad_v_last, const void *grad_w_last, void *grad_x_seq,
+                                      void *grad_v_init, void *grad_w_init, hipStream_t stream);
 int launch_backward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
                     const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
                     const void *h_seq, const void *v_init,
@@ -312,6 +317,8 @@ int launch_backward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t
 int launch_forward_packed(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
                           const void *x_seq, const void *v_init, const float *k_device, uint8_t *spike_bits,
                           void *v_seq, void *v_last, hipStream_t stream);
+// block size (128 or 64 lanes) whose parked h fits in LDS for a sequence of T steps; 0 if none
+int recompute_block(int dtype, int64_t T, bool round_each);
 bool recompute_supported(int dtype, int64_t T, int64_t N);
 bool recompute_preferred(int dtype, int64_t T, int64_t N, bool round_each);
 int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,

@@ -112,6 +112,12 @@ def test_argument_validation_without_a_device():
     assert rc == -2 and b"surrogate" in lib.sjhip_last_error()
     rc = lib.sjhip_izhikevich_backward(L.DTYPE_F32, ctypes.byref(izh), 4, 16, 1, None, None, None, None, 1, None, 1, 1, 1, None)
     assert rc == -1 and b"v_init" in lib.sjhip_last_error()
+    rc = lib.sjhip_izhikevich_backward_replay(L.DTYPE_F32, ctypes.byref(izh), 4, 16, 1, 1, None, 1, None, None, None, None, 1, 1, 1, None)
+    assert rc == -1 and b"NULL tensor" in lib.sjhip_last_error()
+    rc = lib.sjhip_izhikevich_backward_replay(L.DTYPE_F32, ctypes.byref(izh), 4, 18, 16, 16, 16, 16, None, None, None, None, 16, 16, 16, None)
+    assert rc == -2 and b"does not fit" in lib.sjhip_last_error()
+    rc = lib.sjhip_izhikevich_backward_replay(L.DTYPE_F32, ctypes.byref(izh), 4, 16, 16, 16, 16, 8, None, None, None, None, 16, 16, 16, None)
+    assert rc == -1 and b"aligned" in lib.sjhip_last_error()
     assert lib.sjhip_bit_pack(L.DTYPE_F32, -1, 1, 1, None) == -1
     assert lib.sjhip_bit_pack(L.DTYPE_F32, 0, None, None, None) == 0
     assert lib.sjhip_plif_workspace_floats(L.DTYPE_F32, 1 << 20) >= (1 << 20) // 1024

@@ -76,6 +76,68 @@ def test_last_state_gradients_without_state_sequences(sg_name, sg_id, alpha):
     torch.testing.assert_close(wd.grad.cpu(), wr.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
 
 
+def _grads(x, v0, w0, ups, scalars, soft, detach, sg, store, replay, mode_flags=0):
+    xd, vd, wd = x.cuda().requires_grad_(), v0.cuda().requires_grad_(), w0.cuda().requires_grad_()
+    s, v_seq, w_seq, v_last, w_last, h = IK.hip_multistep_izhikevich_forward(
+        xd, vd, wd, scalars, soft, detach, sg[0], sg[1], store, store, not replay, mode_flags, replay)
+    assert (h.numel() == 0) == replay
+    outs = [s, v_seq, w_seq] if store else [s, v_last, w_last]
+    torch.autograd.backward(outs, [u.cuda() for u in ups])
+    return s, xd.grad, vd.grad, wd.grad
+
+
+@pytest.mark.parametrize("p", PARAMS)
+@pytest.mark.parametrize("v_reset", [0.0, -0.2, None])
+@pytest.mark.parametrize("T,N,store", [(16, 4096, True), (7, 132, False), (33, 260, True), (1, 4, True), (64, 1024, False)])
+@pytest.mark.parametrize("detach", [False, True])
+def test_replaying_backward_equals_the_backward_from_a_saved_h_seq(p, v_reset, T, N, store, detach):
+    """Without h_seq the backward kernel recomputes h with the forward's arithmetic, so both routes walk back over the
+    same bits and must return the same gradients bit for bit; the saved-h route is pinned against autograd above."""
+    x = seeded_randn((T, N), 100 + T, 0.4, 0.6) if v_reset is not None else seeded_randn((T, N), 100 + T, 0.25, 0.25)
+    v0, w0 = seeded_randn((N,), 200 + N, 0.0, 0.2), seeded_randn((N,), 250 + N, 0.0, 0.2)
+    ups = ([seeded_randn((T, N), 300 + T), seeded_randn((T, N), 400 + T, 0.0, 0.1), seeded_randn((T, N), 500 + T, 0.0, 0.1)]
+           if store else [seeded_randn((T, N), 300 + T), seeded_randn((N,), 400 + T), seeded_randn((N,), 500 + T)])
+    args = (x, v0, w0, ups, _scalars(p, 1.0, v_reset), v_reset is None, detach, (1, 2.0), store)
+    saved, replayed = _grads(*args, replay=False), _grads(*args, replay=True)
+    for a, b in zip(saved, replayed):
+        assert bits_equal(a.cpu(), b.cpu())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("mode_flags", [0, 0x10])
+def test_replaying_backward_16bit(dtype, mode_flags):
+    T, N = 12, 2048
+    p = PARAMS[1]
+    x = seeded_randn((T, N), 21, 0.4, 0.6).to(dtype)
+    v0, w0 = seeded_randn((N,), 22, 0.0, 0.2).to(dtype), seeded_randn((N,), 23, 0.0, 0.2).to(dtype)
+    ups = [seeded_randn((T, N), 24).to(dtype), seeded_randn((T, N), 25, 0.0, 0.1).to(dtype), seeded_randn((T, N), 26, 0.0, 0.1).to(dtype)]
+    args = (x, v0, w0, ups, _scalars(p, 1.0, -0.1), False, False, (0, 4.0), True)
+    saved, replayed = _grads(*args, replay=False, mode_flags=mode_flags), _grads(*args, replay=True, mode_flags=mode_flags)
+    assert bits_equal(saved[0].cpu(), replayed[0].cpu())
+    if mode_flags == 0:  # h is a storage-dtype value either way: same bits
+        for a, b in zip(saved[1:], replayed[1:]):
+            assert bits_equal(a.cpu(), b.cpu())
+    else:
+        # fp32 state: the replayed h is the forward's fp32 value, while a saved h_seq is rounded to the storage dtype
+        # (and can land on the other side of the threshold), so the replay is checked against fp32 autograd through
+        # the oracle on the same 16-bit-representable inputs
+        xr, vr, wr = (t.float().requires_grad_() for t in (x, v0, w0))
+        es, ev, ew, _ = no.izhikevich_multi_step(xr, vr, wr, p, 1.0, -0.1, no.surrogate("sigmoid", 4.0), False)
+        torch.autograd.backward([es, ev, ew], [u.float() for u in ups])
+        assert bits_equal(replayed[0].float().cpu(), es.detach())
+        for got, want in zip(replayed[1:], (xr.grad, vr.grad, wr.grad)):
+            torch.testing.assert_close(got.float().cpu(), want, rtol=1e-2, atol=1e-2)
+
+
+def test_replay_refuses_shapes_it_cannot_serve():
+    x = torch.zeros((4, 6), device="cuda", requires_grad=True)
+    z = torch.zeros((6,), device="cuda")
+    s = IK.hip_multistep_izhikevich_forward(x, z, z.clone(), _scalars(PARAMS[0], 1.0, 0.0), False, False, 1, 2.0, False,
+                                            False, False, 0, True)[0]
+    with pytest.raises(RuntimeError, match="does not fit"):
+        s.sum().backward()
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("T,N", [(8, 2048), (5, 77)])
 def test_every_op_rounded_16bit_equals_torch_ops_on_half_tensors(dtype, T, N):

@@ -81,6 +81,8 @@ def test_izhikevich_op():
     for store in (False, True):
         torch.library.opcheck(hip_multistep_izhikevich_forward, (x, v0, w0, scalars, False, False, 1, 2.0, store, store, True, 0),
                               test_utils=TESTS)
+        torch.library.opcheck(hip_multistep_izhikevich_forward,
+                              (x, v0, w0, scalars, False, False, 1, 2.0, store, store, False, 0, True), test_utils=TESTS)
 
 
 def test_activation_aware_if_op():
