@@ -126,14 +126,14 @@ def hip_multistep_izhikevich_backward_replay(grad_spike_seq: Optional[torch.Tens
                                              soft_reset: bool, detach_reset: bool, sg_id: int, sg_alpha: float,
                                              mode_flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     L.require_device_tensor("x_seq", x_seq)
-    x_seq = x_seq.contiguous()
+    x_seq = L.aligned16(x_seq)  # the replay kernel has only the 128-bit path
     dtype = L.dtype_id(x_seq.dtype)
     T, N = x_seq.shape
-    fix = lambda t: None if t is None else t.to(x_seq.dtype).contiguous()
+    fix = lambda t: None if t is None else L.aligned16(t.to(x_seq.dtype))
     grad_spike_seq = torch.zeros_like(x_seq) if grad_spike_seq is None else fix(grad_spike_seq)
     grad_v_seq, grad_w_seq, grad_v_last, grad_w_last = map(fix, (grad_v_seq, grad_w_seq, grad_v_last, grad_w_last))
-    v_init, v_flag = _state_arg(v_init, False)
-    w_init, w_flag = _state_arg(w_init, False)
+    v_init, v_flag = _state_arg(v_init, True)
+    w_init, w_flag = _state_arg(w_init, True)
     flags = _flags(soft_reset, detach_reset, mode_flags) | v_flag | (L.FLAG_W_INIT_BROADCAST if w_flag else 0)
     params = _params(scalars, sg_id, sg_alpha, flags)
     grad_x = torch.empty_like(x_seq)

@@ -129,6 +129,32 @@ def test_replaying_backward_16bit(dtype, mode_flags):
             torch.testing.assert_close(got.float().cpu(), want, rtol=1e-2, atol=1e-2)
 
 
+def test_replay_with_misaligned_and_non_contiguous_tensors():
+    """Contiguous tensors that start 4 bytes into an allocation and a permuted upstream gradient: the replaying
+    operator realigns what its 128-bit kernel needs."""
+    T, N = 6, 512
+    p = PARAMS[1]
+    x = seeded_randn((T, N), 31, 0.4, 0.6)
+    v0, w0 = seeded_randn((N,), 32, 0.0, 0.2), seeded_randn((N,), 33, 0.0, 0.2)
+    gs = seeded_randn((N, T), 34)
+    want = _grads(x, v0, w0, [gs.t().contiguous(), seeded_randn((N,), 35), seeded_randn((N,), 36)], _scalars(p, 1.0, 0.0),
+                  False, False, (1, 2.0), False, replay=True)
+
+    def shifted(t):
+        buf = torch.empty(t.numel() + 1, device="cuda")
+        buf[1:].copy_(t.flatten())
+        out = buf[1:].view(t.shape)
+        assert out.data_ptr() % 16 == 4 and out.is_contiguous()
+        return out
+
+    xd, vd, wd = shifted(x).requires_grad_(), shifted(v0).requires_grad_(), shifted(w0).requires_grad_()
+    s, _, _, v_last, w_last, _ = IK.hip_multistep_izhikevich_forward(xd, vd, wd, _scalars(p, 1.0, 0.0), False, False, 1, 2.0,
+                                                                    False, False, False, 0, True)
+    torch.autograd.backward([s, v_last, w_last], [gs.cuda().t(), shifted(seeded_randn((N,), 35)), shifted(seeded_randn((N,), 36))])
+    for got, ref in zip((s, xd.grad, vd.grad, wd.grad), want):
+        assert bits_equal(got.detach().cpu(), ref.detach().cpu())
+
+
 def test_replay_refuses_shapes_it_cannot_serve():
     x = torch.zeros((4, 6), device="cuda", requires_grad=True)
     z = torch.zeros((6,), device="cuda")
