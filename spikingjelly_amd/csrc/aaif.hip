@@ -49,12 +49,27 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) aaif_forward_kernel(const Aai
 #pragma unroll
   for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? A::load(xp + (int64_t)i * N) : A::zero();
 
+  // Channel of the first neuron with one division pair (32-bit when N allows: a 64-bit division is a software loop
+  // of more instructions than the whole walk over T); the neighbours follow by counting.
   float thr[V], off[V];
+  int64_t within, c;
+  if (N <= 0xffffffffLL) {
+    const uint32_t inner = (uint32_t)a.inner_size, q = (uint32_t)col / inner;
+    within = (uint32_t)col - q * inner;
+    c = q % (uint32_t)a.channel_size;
+  } else {
+    const int64_t q = col / a.inner_size;
+    within = col - q * a.inner_size;
+    c = q % a.channel_size;
+  }
 #pragma unroll
   for (int j = 0; j < V; ++j) {
-    const int64_t c = ((col + j) / a.inner_size) % a.channel_size;
     thr[j] = Cvt<S>::round(a.threshold[a.threshold_scalar ? 0 : c]);
     off[j] = Cvt<S>::round(a.offset[a.offset_scalar ? 0 : c]);
+    if (++within == a.inner_size) {
+      within = 0;
+      if (++c == a.channel_size) c = 0;
+    }
   }
   const float reset_mul = a.v_reset;  // a Python scalar in torch: fp32 as a factor
 
