@@ -1,3 +1,12 @@
+from .checkpointing import (  # noqa: F401
+    GCContainer,
+    InputCompressedGC,
+    TCGCContainer,
+    in_gc_1st_forward,
+    input_compressed_gc,
+    query_autocast,
+    to_gc_function,
+)
 from .compress import (  # noqa: F401
     BaseSpikeCompressor,
     BitSpikeCompressor,
