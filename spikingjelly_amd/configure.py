@@ -30,3 +30,8 @@ hip_half_precision_mode = "torch"
 hip_backward_recompute = True
 hip_lif_reciprocal_tau = False
 hip_plif_atomic_reduce = False
+
+# ``save_bool_spike_level`` (same name and meaning as the reference's ``configure.py:59-67``): how the spike operators
+# of ``hip_kernel/spike_op.py`` keep their binary input for the backward.  0: as ``torch.bool`` (one byte per spike);
+# 1: bit-packed, eight spikes per byte (``hip_kernel/tensor_cache.float_spike_to_bool``).
+save_bool_spike_level = 0
