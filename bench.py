@@ -212,6 +212,44 @@ def other_workload(args) -> int:
                "kernel_ms": f_ms, "algorithmic_bytes": bytes_each})
         return 0
 
+    if args.workload == "fp8":
+        # the config-2 shape with 8-bit floating-point storage (mixed precision): x, v_seq, h_seq, grad_v in float8_e4m3fn,
+        # spikes and their gradient in bf16, fp32 recurrence; the two operators are called directly so that the casts
+        # a caller's dtypes may add stay outside the timed region
+        from spikingjelly_amd.activation_based.hip_kernel import neuron_mp_kernel as M
+
+        T, N = 16, 256 * 128 * 32 * 32
+        g = torch.Generator(device=dev).manual_seed(1002)
+        f8, sp = torch.float8_e4m3fn, torch.bfloat16
+        x = (torch.randn((T, N), generator=g, device=dev) * 0.8 + 0.3).to(f8)
+        v0 = torch.zeros((N,), device=dev).to(f8)
+        gs = torch.randn((T, N), generator=g, device=dev).to(sp)
+        gv = (torch.randn((T, N), generator=g, device=dev) * 0.1).to(f8)
+        scalars = (L.NEURON_LIF, 2.0, True, 1.0, 0.0, False, False, 1, 2.0)
+        rate = []
+
+        def step():
+            s, v_seq, h_seq = M.hip_multistep_mp_forward(x, v0, None, *scalars, f8, sp, True)
+            M.hip_multistep_mp_backward(gs, gv, h_seq, v0, None, *scalars, sp)
+            if not rate:
+                rate.append(float(s.float().mean()))
+
+        elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
+        f_ms, b_ms = _kernel_ms(L, L.KC_FORWARD), _kernel_ms(L, L.KC_BACKWARD)
+        fwd_bytes = 5 * T * N + N          # x 1, spikes 2, v_seq 1, h_seq 1; v_init
+        bwd_bytes = 8 * T * N + 4 * N      # grad_spike 2, grad_v 1, h_seq 1, grad_x 4 (fp32); grad_v_init
+        dom, d_ms, d_bytes = ("forward", f_ms, fwd_bytes) if f_ms >= b_ms else ("backward", b_ms, bwd_bytes)
+        _emit(args, "neuron-steps/sec LIF fwd+bwd float8_e4m3fn storage T=16 N=33.5M, 1 MI355X", "neuron-steps/s",
+              T * N / (elapsed / args.steps), elapsed, "f32",
+              {"workload": "sj::hip_multistep_mp_forward + _backward, LIF tau=2, hard reset 0, ATan(2), x [16, 33554432] "
+                           "float8_e4m3fn ~N(0.3,0.8), spikes and grad_spike bf16, v_seq / h_seq / grad_v float8_e4m3fn, "
+                           "grad_x fp32", "T": T, "N": N, "firing_rate": rate[0]},
+              {"bound": "hbm", "achieved": d_bytes / (d_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+               "frac": d_bytes / (d_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": dom, "kernel_ms": d_ms,
+               "algorithmic_bytes": d_bytes, "forward_ms": f_ms, "backward_ms": b_ms,
+               "forward_GBs": fwd_bytes / (f_ms * 1e-3) / 1e9, "backward_GBs": bwd_bytes / (b_ms * 1e-3) / 1e9})
+        return 0
+
     if args.workload == "stbif":
         # SpikeZIP's signed ternary neuron (inference): the config-2 shape, the activation fed at the first step
         shape = (16, 256, 128, 32, 32)
@@ -336,7 +374,7 @@ def main() -> int:
     ap.add_argument("--cpu-sample-neurons", type=int, default=1 << 23)
     ap.add_argument("--cpu-repeats", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "qif", "eif", "izhikevich", "ilif", "stbif", "aaif"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "qif", "eif", "izhikevich", "ilif", "stbif", "aaif", "fp8"],
                     help="config2 (default) is the headline metric; the others are secondary measurements")
     args = ap.parse_args()
     if args.gpus != 1:

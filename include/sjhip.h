@@ -75,7 +75,9 @@ typedef enum sjhip_dtype {
   SJHIP_F32 = 0,
   SJHIP_F16 = 1,
   SJHIP_BF16 = 2,
-  SJHIP_U8 = 3 /* bit_pack / bit_unpack only */
+  SJHIP_U8 = 3, /* bit_pack / bit_unpack only */
+  SJHIP_F8E4M3 = 4, /* float8_e4m3fn, storage dtype of the *_mp entry points only */
+  SJHIP_F8E5M2 = 5  /* float8_e5m2, likewise */
 } sjhip_dtype;
 
 /* Surrogate gradient used by the backward pass (forward is always Heaviside).
@@ -248,6 +250,29 @@ int sjhip_stbif_forward(int dtype, uint32_t flags, int64_t T, int64_t N,
                         const float *q_threshold, const float *pos_max, const float *neg_min,
                         void *out_seq, void *q_final, void *acc_q_final, void *cur_output,
                         int32_t *work_flag, void *stream);
+
+/*
+ * IF / LIF / PLIF with 8-bit floating-point storage (mixed precision).  Stands in for the reference's
+ * torch.ops.sj.multistep_{if,lif,plif}_mp_forward / _mp_inference and their backward with an FP8 storage dtype,
+ * spikingjelly/activation_based/triton_kernel/neuron_kernel/lif.py:788-956, 1103-1150 (plif.py:834-879,
+ * integrate_and_fire.py likewise): x_seq, v_init, v_seq, v_last, h_seq, grad_v_seq and grad_v_last are
+ * `storage_dtype` (SJHIP_F8E4M3 or SJHIP_F8E5M2), spike_seq and grad_spike_seq are `spike_dtype` (SJHIP_F32, SJHIP_F16
+ * or SJHIP_BF16), the recurrence runs in fp32 on the decoded values and only stored values are rounded (round to
+ * nearest even as torch's .to(torch.float8_*): e4m3fn has no infinity and overflows to NaN, e5m2 overflows to
+ * infinity); grad_x_seq [T,N] and grad_v_init [N] are fp32.  Same params, flags and PLIF conventions as
+ * sjhip_neuron_forward / sjhip_neuron_backward (PLIF: rtau_device, grad_rtau and a workspace of
+ * sjhip_plif_workspace_floats(SJHIP_F32, N) floats).  N must be a multiple of 4 and every tensor 16-byte aligned
+ * (a work-item owns four groups of four neurons: one 4-byte access per group of an 8-bit row); callers pad.
+ * neuron: IF, LIF or PLIF.
+ */
+int sjhip_neuron_forward_mp(int neuron, int storage_dtype, int spike_dtype, const sjhip_neuron_params *p,
+                            int64_t T, int64_t N, const void *x_seq, const void *v_init, const float *rtau_device,
+                            void *spike_seq, void *v_seq, void *v_last, void *h_seq, void *stream);
+int sjhip_neuron_backward_mp(int neuron, int storage_dtype, int spike_dtype, const sjhip_neuron_params *p,
+                             int64_t T, int64_t N, const void *grad_spike_seq, const void *grad_v_seq,
+                             const void *grad_v_last, const void *h_seq, const void *v_init,
+                             const float *rtau_device, float *grad_x_seq, float *grad_v_init, float *grad_rtau,
+                             float *workspace, void *stream);
 
 /*
  * Izhikevich neuron: quadratic membrane v with an adaptation current w (two states).  Stands in for

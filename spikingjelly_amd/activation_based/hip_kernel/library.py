@@ -20,6 +20,7 @@ ABI_VERSION = 3
 NEURON_IF, NEURON_LIF, NEURON_PLIF, NEURON_QIF, NEURON_ILIF, NEURON_EIF = 0, 1, 2, 3, 4, 5
 SG_MULTI_LEVEL = 7  # ILIF's windowed straight-through estimator; ids 0-6 are listed in surrogate_registry
 DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_U8 = 0, 1, 2, 3
+DTYPE_F8E4M3, DTYPE_F8E5M2 = 4, 5  # storage dtypes of the mixed-precision entry points only
 FLAG_DECAY_INPUT = 0x01
 FLAG_SOFT_RESET = 0x02
 FLAG_DETACH_RESET = 0x04
@@ -39,6 +40,8 @@ EXPORTED_SYMBOLS = (
     "sjhip_neuron_forward",
     "sjhip_neuron_forward_packed",
     "sjhip_plif_workspace_floats",
+    "sjhip_neuron_forward_mp",
+    "sjhip_neuron_backward_mp",
     "sjhip_neuron_backward",
     "sjhip_neuron_backward_recompute",
     "sjhip_recompute_supported",
@@ -125,6 +128,10 @@ def load() -> ctypes.CDLL:
             c_int, c_int, POINTER(NeuronParams), c_int64, c_int64,
             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
         ]
+        lib.sjhip_neuron_forward_mp.restype = c_int
+        lib.sjhip_neuron_forward_mp.argtypes = [c_int, c_int, c_int, POINTER(NeuronParams), c_int64, c_int64] + [c_void_p] * 8
+        lib.sjhip_neuron_backward_mp.restype = c_int
+        lib.sjhip_neuron_backward_mp.argtypes = [c_int, c_int, c_int, POINTER(NeuronParams), c_int64, c_int64] + [c_void_p] * 11
         lib.sjhip_plif_workspace_floats.restype = c_int64
         lib.sjhip_plif_workspace_floats.argtypes = [c_int, c_int64]
         lib.sjhip_neuron_backward.restype = c_int

@@ -210,6 +210,47 @@ int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p, i
                          grad_v_init, grad_rtau, workspace, static_cast<hipStream_t>(stream));
 }
 
+namespace {
+int check_mp(const char *what, int neuron, int storage_dtype, int spike_dtype, const sjhip_neuron_params *p, int64_t T,
+             int64_t N) {
+  if (!p) return fail(SJHIP_ERR_INVALID, "%s: params is NULL", what);
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_PLIF) return fail(SJHIP_ERR_UNSUPPORTED, "%s: neuron %d (IF, LIF and PLIF only)", what, neuron);
+  if (storage_dtype != SJHIP_F8E4M3 && storage_dtype != SJHIP_F8E5M2)
+    return fail(SJHIP_ERR_INVALID, "%s: storage dtype %d is not an 8-bit float", what, storage_dtype);
+  if (!valid_dtype_fp(spike_dtype)) return fail(SJHIP_ERR_INVALID, "%s: spike dtype %d", what, spike_dtype);
+  return check_shape(what, T, N);
+}
+}  // namespace
+
+int sjhip_neuron_forward_mp(int neuron, int storage_dtype, int spike_dtype, const sjhip_neuron_params *p, int64_t T,
+                            int64_t N, const void *x_seq, const void *v_init, const float *rtau_device, void *spike_seq,
+                            void *v_seq, void *v_last, void *h_seq, void *stream) {
+  int rc = check_mp("forward(mp)", neuron, storage_dtype, spike_dtype, p, T, N);
+  if (rc != SJHIP_OK) return rc;
+  if (!x_seq || !v_init || !spike_seq) return fail(SJHIP_ERR_INVALID, "forward(mp): NULL tensor");
+  if (!v_seq && !v_last) return fail(SJHIP_ERR_INVALID, "forward(mp): neither v_seq nor v_last given");
+  if (neuron == SJHIP_NEURON_PLIF && !rtau_device) return fail(SJHIP_ERR_INVALID, "forward(mp): PLIF needs rtau_device");
+  return launch_forward_mp(neuron, storage_dtype, spike_dtype, *p, T, N, x_seq, v_init, rtau_device, spike_seq, v_seq,
+                           v_last, h_seq, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_neuron_backward_mp(int neuron, int storage_dtype, int spike_dtype, const sjhip_neuron_params *p, int64_t T,
+                             int64_t N, const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                             const void *h_seq, const void *v_init, const float *rtau_device, float *grad_x_seq,
+                             float *grad_v_init, float *grad_rtau, float *workspace, void *stream) {
+  int rc = check_mp("backward(mp)", neuron, storage_dtype, spike_dtype, p, T, N);
+  if (rc != SJHIP_OK) return rc;
+  if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_ERF) return fail(SJHIP_ERR_UNSUPPORTED, "backward(mp): surrogate id %d", p->sg_id);
+  if (!grad_spike_seq || !h_seq || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward(mp): NULL tensor");
+  if (neuron == SJHIP_NEURON_PLIF) {
+    if (!v_init || !grad_rtau || !rtau_device) return fail(SJHIP_ERR_INVALID, "backward(mp): PLIF needs v_init, rtau_device and grad_rtau");
+    if (!(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace) return fail(SJHIP_ERR_INVALID, "backward(mp): PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");
+  }
+  return launch_backward_mp(neuron, storage_dtype, spike_dtype, *p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq,
+                            v_init, rtau_device, grad_x_seq, grad_v_init, grad_rtau, workspace,
+                            static_cast<hipStream_t>(stream));
+}
+
 int sjhip_recompute_supported(int dtype, int64_t T, int64_t N) {
   if (!valid_dtype_fp(dtype) || T < 1 || N < 1) return 0;
   return recompute_supported(dtype, T, N) ? 1 : 0;

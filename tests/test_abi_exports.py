@@ -118,6 +118,23 @@ def test_argument_validation_without_a_device():
     assert rc == -2 and b"does not fit" in lib.sjhip_last_error()
     rc = lib.sjhip_izhikevich_backward_replay(L.DTYPE_F32, ctypes.byref(izh), 4, 16, 16, 16, 16, 8, None, None, None, None, 16, 16, 16, None)
     assert rc == -1 and b"aligned" in lib.sjhip_last_error()
+    mp = L.NeuronParams(2.0, 1.0, 0.0, 2.0, 1, 0)
+    rc = lib.sjhip_neuron_forward_mp(L.NEURON_LIF, L.DTYPE_F16, L.DTYPE_BF16, ctypes.byref(mp), 4, 64, 16, 16, None, 16, 16, None, None, None)
+    assert rc == -1 and b"8-bit float" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_forward_mp(L.NEURON_QIF, L.DTYPE_F8E4M3, L.DTYPE_BF16, ctypes.byref(mp), 4, 64, 16, 16, None, 16, 16, None, None, None)
+    assert rc == -2 and b"IF, LIF and PLIF only" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_forward_mp(L.NEURON_LIF, L.DTYPE_F8E4M3, L.DTYPE_U8, ctypes.byref(mp), 4, 64, 16, 16, None, 16, 16, None, None, None)
+    assert rc == -1 and b"spike dtype" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_forward_mp(L.NEURON_LIF, L.DTYPE_F8E5M2, L.DTYPE_BF16, ctypes.byref(mp), 4, 66, 16, 16, None, 16, 16, None, None, None)
+    assert rc == -2 and b"multiple of 4" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_forward_mp(L.NEURON_LIF, L.DTYPE_F8E5M2, L.DTYPE_BF16, ctypes.byref(mp), 4, 64, 16, 16, None, 8, 16, None, None, None)
+    assert rc == -1 and b"aligned" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_forward_mp(L.NEURON_PLIF, L.DTYPE_F8E5M2, L.DTYPE_BF16, ctypes.byref(mp), 4, 64, 16, 16, None, 16, 16, None, None, None)
+    assert rc == -1 and b"rtau_device" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_backward_mp(L.NEURON_PLIF, L.DTYPE_F8E4M3, L.DTYPE_F32, ctypes.byref(mp), 4, 64, 16, None, None, 16, 16, 16, 16, 16, 16, None, None)
+    assert rc == -1 and b"workspace" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_backward_mp(L.NEURON_IF, L.DTYPE_F8E4M3, L.DTYPE_F32, ctypes.byref(mp), 4, 64, None, None, None, 16, None, None, 16, 16, None, None, None)
+    assert rc == -1 and b"NULL tensor" in lib.sjhip_last_error()
     assert lib.sjhip_bit_pack(L.DTYPE_F32, -1, 1, 1, None) == -1
     assert lib.sjhip_bit_pack(L.DTYPE_F32, 0, None, None, None) == 0
     assert lib.sjhip_plif_workspace_floats(L.DTYPE_F32, 1 << 20) >= (1 << 20) // 1024
