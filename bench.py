@@ -423,12 +423,17 @@ def main() -> int:
     L.profile_reset()
     L.profile_enable(True)
     torch.cuda.synchronize()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for i in range(args.steps):
+        marks[i].record()  # on the stream the kernels are launched on
         spikes = step()
+    marks[-1].record()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     L.profile_enable(False)
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    quantile = lambda q: per_step[min(len(per_step) - 1, int(q * len(per_step)))]
     rate = float(spikes.detach().mean())
     n_fwd, ms_fwd = L.profile_read(L.KC_FORWARD)
     n_bwd, ms_bwd = L.profile_read(L.KC_BACKWARD)
@@ -468,6 +473,7 @@ def main() -> int:
         "value": value,
         "unit": "neuron-steps/s",
         "n_gpus": 1,
+        "step_ms_quantiles": {"p25": quantile(0.25), "median": quantile(0.5), "p75": quantile(0.75)},
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
