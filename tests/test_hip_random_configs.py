@@ -64,6 +64,26 @@ def _draw_ilif(seed):
     return "ilif", neuron.ILIFNode, kw, dtype, T, shape, bool(rng.integers(0, 2)), v_th * levels * 0.6, int(rng.integers(0, 1 << 30))
 
 
+def _draw_izhikevich(seed):
+    """Two coupled states: both time constants (exact reciprocals or not), the coupling, hard reset (a soft reset lets
+    the quadratic term diverge on a random drive), saved-h or replaying backward."""
+    rng = np.random.default_rng(20_000 + seed)
+    dtype = rng.choice([torch.float32, torch.float32, torch.float32, torch.float16, torch.bfloat16])
+    T = int(rng.choice([1, 2, 3, 5, 8, 16, 33]))
+    shape = tuple(int(v) for v in rng.choice([1, 2, 3, 4, 7, 8, 12, 32, 37, 64, 100], size=int(rng.integers(1, 4))))
+    kw = dict(tau=float(rng.choice([2.0, 2.5, 4.0, 10.0])), tau_w=float(rng.choice([2.0, 3.0, 8.0])), v_c=float(rng.choice([0.5, 0.8])),
+              a0=float(rng.choice([0.5, 1.0])), v_rest=float(rng.choice([0.0, -0.1])), w_rest=float(rng.choice([0.0, 0.05])),
+              a=float(rng.choice([0.0, 0.3, -0.2])), b=float(rng.choice([0.0, 0.2])), v_threshold=1.0,
+              v_reset=float(rng.choice([0.0, -0.25])), detach_reset=bool(rng.integers(0, 2)),
+              surrogate_function=SURROGATES[int(rng.integers(0, len(SURROGATES)))](), store_v_seq=bool(rng.integers(0, 2)))
+    return "izhikevich", neuron.IzhikevichNode, kw, dtype, T, shape, bool(rng.integers(0, 2)), 0.5, int(rng.integers(0, 1 << 30))
+
+
+@pytest.mark.parametrize("seed", range(80))
+def test_random_izhikevich_configuration(seed):
+    _run_case(*_draw_izhikevich(seed))
+
+
 @pytest.mark.parametrize("seed", range(300))
 def test_random_configuration(seed):
     _run_case(*_draw(seed))
@@ -88,6 +108,8 @@ def _run_case(kind, cls, kw, dtype, T, shape, recompute, scale, data_seed):
         sa, sb = a(xa), b(xb)
         assert bits_equal(sb.cpu(), sa.detach()), "spikes"
         assert bits_equal(b.v.detach().cpu(), a.v.detach()), "state"
+        if kind == "izhikevich":
+            assert bits_equal(b.w.detach().cpu(), a.w.detach()), "adaptation state"
         if kw["store_v_seq"]:
             assert bits_equal(b.v_seq.detach().cpu(), a.v_seq.detach()), "v_seq"
         la = (sa.float() * gs.float()).sum() + 0.5 * a.v.float().sum()
@@ -107,6 +129,8 @@ def _run_case(kind, cls, kw, dtype, T, shape, recompute, scale, data_seed):
         sa2, sb2 = a(x2), b(x2.cuda())
         assert bits_equal(sb2.cpu(), sa2.detach()), "spikes of the second call"
         assert bits_equal(b.v.detach().cpu(), a.v.detach()), "state after the second call"
+        if kind == "izhikevich":
+            assert bits_equal(b.w.detach().cpu(), a.w.detach()), "adaptation state after the second call"
     finally:
         configure.hip_backward_recompute, configure.hip_half_precision_mode = old
         functional.reset_net(a)
