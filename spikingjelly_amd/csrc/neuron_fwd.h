@@ -30,6 +30,9 @@
 #ifndef SJHIP_FWD_NT
 #define SJHIP_FWD_NT 0
 #endif
+#ifndef SJHIP_FWD_PACKED_NT
+#define SJHIP_FWD_PACKED_NT 1
+#endif
 
 namespace sjhip {
 
@@ -233,11 +236,13 @@ __device__ __forceinline__ void store_spike_bits(uint8_t *row, int64_t col, int6
 
 template <typename S, bool VECTOR, bool ROUND_EACH, int CH, int RS, bool PACKED>
 __device__ __forceinline__ void forward_body(const FwdArgs &a) {
-  typedef Acc<S, VECTOR, SJHIP_FWD_NT != 0> A;
+  // with bit-packed spikes the kernel is read-dominated (x in, one bit out): streaming policy like the backward
+  constexpr bool NT = (SJHIP_FWD_NT != 0) || (PACKED && SJHIP_FWD_PACKED_NT != 0);
+  typedef Acc<S, VECTOR, NT> A;
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
-  constexpr int PF = sizeof(S) == 2 ? SJHIP_FWD_PF16 : SJHIP_FWD_PF;
+  constexpr int PF = sizeof(S) == 2 ? SJHIP_FWD_PF16 : SJHIP_FWD_PF;  // (eight 16-bit rows measured slower, packed too)
 
   const int64_t N = a.N, T = a.T;
   const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
@@ -255,7 +260,7 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
 
   typedef typename StepNum<S, ROUND_EACH>::type NUM;
   NUM v[V];
-  load_state<S, VECTOR, SJHIP_FWD_NT != 0>(a.v_init, col, a.v_init_broadcast != 0, v);
+  load_state<S, VECTOR, NT>(a.v_init, col, a.v_init_broadcast != 0, v);
 
   for (int64_t t0 = 0; t0 < T; t0 += PF) {
     typename A::raw_t cur[PF];
