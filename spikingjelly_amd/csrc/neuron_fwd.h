@@ -234,11 +234,21 @@ __device__ __forceinline__ void store_spike_bits(uint8_t *row, int64_t col, int6
   }
 }
 
-template <typename S, bool VECTOR, bool ROUND_EACH, int CH, int RS, bool PACKED>
+// OUT: what leaves the kernel besides the state, and with it the cache policy of the x loads.  Measured on MI355X with
+// both variants on one machine: bit-packed spikes (nothing but x moves) -> streaming everything (98.7 -> 94 us, fp16
+// T = 32, N = 6.4 M); 16-bit storage with fp32 state writing spikes plus v_seq / h_seq -> streaming x loads (bf16 T = 8,
+// N = 8.4 M: 88 -> 74 us); everything else -> default policy (fp32 with two outputs gained 4 % in a forward-only loop
+// and lost 5 % inside a training step, where the placement of the tensors differs; 16-bit with every op rounded lost
+// 2 %).
+enum FwdOut { FWD_OUT_DENSE = 0, FWD_OUT_PACKED = 1, FWD_OUT_DENSE_STREAM_X = 2 };
+
+template <typename S, bool VECTOR, bool ROUND_EACH, int CH, int RS, int OUT>
 __device__ __forceinline__ void forward_body(const FwdArgs &a) {
+  constexpr bool PACKED = OUT == FWD_OUT_PACKED;
   // with bit-packed spikes the kernel is read-dominated (x in, one bit out): streaming policy like the backward
   constexpr bool NT = (SJHIP_FWD_NT != 0) || (PACKED && SJHIP_FWD_PACKED_NT != 0);
   typedef Acc<S, VECTOR, NT> A;
+  typedef Acc<S, VECTOR, NT || OUT == FWD_OUT_DENSE_STREAM_X> AL;  // policy of the x loads alone
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
@@ -256,7 +266,7 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
 
   typename A::raw_t ahead[PF];
 #pragma unroll
-  for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? A::load(xp + (int64_t)i * N) : A::zero();
+  for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? AL::load(xp + (int64_t)i * N) : A::zero();
 
   typedef typename StepNum<S, ROUND_EACH>::type NUM;
   NUM v[V];
@@ -269,7 +279,7 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int64_t tn = t0 + PF + i;
-      if (tn < T) ahead[i] = A::load(xp + tn * N);
+      if (tn < T) ahead[i] = AL::load(xp + tn * N);
     }
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
@@ -290,33 +300,33 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
   if (a.v_last) A::store((E *)a.v_last + col, v);
 }
 
-template <typename S, bool VECTOR, bool ROUND_EACH, int CH, bool PACKED>
+template <typename S, bool VECTOR, bool ROUND_EACH, int CH, int OUT>
 __device__ __forceinline__ void forward_reset_dispatch(const FwdArgs &a) {
   // counts exist for the charge ILIF uses (no input decay) and never bit-packed
-  if constexpr ((CH == CH_PLAIN_INPUT_DIV || CH == CH_PLAIN_INPUT_MUL) && !PACKED) {
+  if constexpr ((CH == CH_PLAIN_INPUT_DIV || CH == CH_PLAIN_INPUT_MUL) && OUT != FWD_OUT_PACKED) {
     if (a.soft_reset == RESET_COUNT) {
-      forward_body<S, VECTOR, ROUND_EACH, CH, RESET_COUNT, PACKED>(a);
+      forward_body<S, VECTOR, ROUND_EACH, CH, RESET_COUNT, OUT>(a);
       return;
     }
   }
   if (a.soft_reset)
-    forward_body<S, VECTOR, ROUND_EACH, CH, RESET_SOFT, PACKED>(a);
+    forward_body<S, VECTOR, ROUND_EACH, CH, RESET_SOFT, OUT>(a);
   else
-    forward_body<S, VECTOR, ROUND_EACH, CH, RESET_HARD, PACKED>(a);
+    forward_body<S, VECTOR, ROUND_EACH, CH, RESET_HARD, OUT>(a);
 }
 
-template <typename S, bool VECTOR, bool ROUND_EACH, bool PACKED = false>
+template <typename S, bool VECTOR, bool ROUND_EACH, int OUT = FWD_OUT_DENSE>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) forward_kernel(const FwdArgs a) {
   switch (a.charge) {
-    case CH_IF: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_IF, PACKED>(a); break;
-    case CH_DECAY_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_DIV, PACKED>(a); break;
-    case CH_DECAY_INPUT_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_MUL, PACKED>(a); break;
-    case CH_PLAIN_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_DIV, PACKED>(a); break;
-    case CH_QIF_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_QIF_DIV, PACKED>(a); break;
-    case CH_QIF_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_QIF_MUL, PACKED>(a); break;
-    case CH_EIF_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_EIF_DIV, PACKED>(a); break;
-    case CH_EIF_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_EIF_MUL, PACKED>(a); break;
-    default: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_MUL, PACKED>(a); break;
+    case CH_IF: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_IF, OUT>(a); break;
+    case CH_DECAY_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_DIV, OUT>(a); break;
+    case CH_DECAY_INPUT_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_DECAY_INPUT_MUL, OUT>(a); break;
+    case CH_PLAIN_INPUT_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_DIV, OUT>(a); break;
+    case CH_QIF_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_QIF_DIV, OUT>(a); break;
+    case CH_QIF_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_QIF_MUL, OUT>(a); break;
+    case CH_EIF_DIV: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_EIF_DIV, OUT>(a); break;
+    case CH_EIF_MUL: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_EIF_MUL, OUT>(a); break;
+    default: forward_reset_dispatch<S, VECTOR, ROUND_EACH, CH_PLAIN_INPUT_MUL, OUT>(a); break;
   }
 }
 

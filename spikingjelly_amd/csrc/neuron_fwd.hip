@@ -26,10 +26,20 @@ int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   else if (a.T < 16 || a.soft_reset == RESET_COUNT || a.charge == CH_EIF_DIV || a.charge == CH_EIF_MUL) cap *= 2;
   const unsigned lds = (sizeof(S) == 4 && several_outputs) ? occupancy_cap_lds(cap) : 0u;
   ProfileScope prof(KC_FORWARD, stream);
-  if (vector)
-    hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, PACKED>), dim3((unsigned)blocks), dim3(block), lds, stream, a);
-  else
-    hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH, PACKED>), dim3((unsigned)blocks), dim3(block), lds, stream, a);
+  const dim3 grid((unsigned)blocks), threads(block);
+  if constexpr (PACKED) {
+    if (vector) hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, FWD_OUT_PACKED>), grid, threads, lds, stream, a);
+    else hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH, FWD_OUT_PACKED>), grid, threads, lds, stream, a);
+  } else if (sizeof(S) == 2 && !ROUND_EACH && several_outputs) {
+    // 16-bit storage with fp32 state writing spikes plus v_seq / h_seq: see FwdOut
+    if constexpr (sizeof(S) == 2 && !ROUND_EACH) {
+      if (vector) hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, FWD_OUT_DENSE_STREAM_X>), grid, threads, lds, stream, a);
+      else hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH, FWD_OUT_DENSE_STREAM_X>), grid, threads, lds, stream, a);
+    }
+  } else {
+    if (vector) hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, FWD_OUT_DENSE>), grid, threads, lds, stream, a);
+    else hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH, FWD_OUT_DENSE>), grid, threads, lds, stream, a);
+  }
   return check_launch(PACKED ? "forward_packed" : "forward");
 }
 
