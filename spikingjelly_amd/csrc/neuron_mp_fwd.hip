@@ -4,20 +4,24 @@
 #ifndef SJHIP_MP_FWD_NT
 #define SJHIP_MP_FWD_NT 0
 #endif
+#ifndef SJHIP_MP_FWD_X_NT
+#define SJHIP_MP_FWD_X_NT 0
+#endif
 
 namespace sjhip {
 
 template <typename ST, typename SP, int CH, int RS>
 __device__ __forceinline__ void mp_forward_walk(const FwdArgs &a, const MpLane &l) {
   typedef Tile16<ST, SJHIP_MP_FWD_NT != 0> RX;  // streaming policy as measured for the fp32 forward: default wins
+  typedef Tile16<ST, (SJHIP_MP_FWD_NT != 0) || (SJHIP_MP_FWD_X_NT != 0)> RXL;  // the x loads alone
   typedef Tile16<SP, SJHIP_MP_FWD_NT != 0> RSP;
   constexpr int V = 16, PF = SJHIP_MP_PF;
   const int64_t N = a.N, T = a.T;
   const float tau = a.k_device ? *a.k_device : a.tau;
 
-  typename RX::raw_t ahead[PF];
+  typename RXL::raw_t ahead[PF];
 #pragma unroll
-  for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? RX::load(a.x, (int64_t)i * N, l) : RX::zero();
+  for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? RXL::load(a.x, (int64_t)i * N, l) : RXL::zero();
   float v[V];
   if (a.v_init_broadcast) {
     const float v0 = Codec<ST>::dec(*(const uint8_t *)a.v_init);
@@ -27,20 +31,20 @@ __device__ __forceinline__ void mp_forward_walk(const FwdArgs &a, const MpLane &
     RX::unpack(RX::load(a.v_init, 0, l), v);
   }
   for (int64_t t0 = 0; t0 < T; t0 += PF) {
-    typename RX::raw_t now[PF];
+    typename RXL::raw_t now[PF];
 #pragma unroll
     for (int i = 0; i < PF; ++i) now[i] = ahead[i];
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int64_t tn = t0 + PF + i;
-      if (tn < T) ahead[i] = RX::load(a.x, tn * N, l);
+      if (tn < T) ahead[i] = RXL::load(a.x, tn * N, l);
     }
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int64_t t = t0 + i;
       if (t < T) {
         float x[V], h[V], s[V];
-        RX::unpack(now[i], x);
+        RXL::unpack(now[i], x);
 #pragma unroll
         for (int j = 0; j < V; ++j) neuron_step<float, CH, RS>(x[j], v[j], h[j], s[j], tau, a);
         RSP::store(a.spike, t * N, l, s);
