@@ -238,8 +238,8 @@ __device__ __forceinline__ void store_spike_bits(uint8_t *row, int64_t col, int6
 // both variants on one machine: bit-packed spikes (nothing but x moves) -> streaming everything (98.7 -> 94 us, fp16
 // T = 32, N = 6.4 M); 16-bit storage with fp32 state writing spikes plus v_seq / h_seq -> streaming x loads (bf16 T = 8,
 // N = 8.4 M: 88 -> 74 us); everything else -> default policy (fp32 with two outputs gained 4 % in a forward-only loop
-// and lost 5 % inside a training step, where the placement of the tensors differs; 16-bit with every op rounded lost
-// 2 %).
+// but lost 1.2 % inside the training step, forward and backward alternating, which is the case that counts; 16-bit
+// with every op rounded lost 2 %).
 enum FwdOut { FWD_OUT_DENSE = 0, FWD_OUT_PACKED = 1, FWD_OUT_DENSE_STREAM_X = 2 };
 
 template <typename S, bool VECTOR, bool ROUND_EACH, int CH, int RS, int OUT>

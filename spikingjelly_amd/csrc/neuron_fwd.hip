@@ -7,6 +7,12 @@ namespace sjhip {
 
 namespace {
 
+#ifndef SJHIP_FWD_STREAM_X_FP32
+#define SJHIP_FWD_STREAM_X_FP32 0
+#endif
+template <typename S, bool ROUND_EACH>
+constexpr bool kStreamX = (sizeof(S) == 2 && !ROUND_EACH) || (sizeof(S) == 4 && SJHIP_FWD_STREAM_X_FP32 != 0);
+
 template <typename S, bool ROUND_EACH, bool PACKED = false>
 int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   const int block = tuning().fwd_block;
@@ -30,9 +36,9 @@ int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   if constexpr (PACKED) {
     if (vector) hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, FWD_OUT_PACKED>), grid, threads, lds, stream, a);
     else hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH, FWD_OUT_PACKED>), grid, threads, lds, stream, a);
-  } else if (sizeof(S) == 2 && !ROUND_EACH && several_outputs) {
+  } else if (kStreamX<S, ROUND_EACH> && several_outputs) {
     // 16-bit storage with fp32 state writing spikes plus v_seq / h_seq: see FwdOut
-    if constexpr (sizeof(S) == 2 && !ROUND_EACH) {
+    if constexpr (kStreamX<S, ROUND_EACH>) {
       if (vector) hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, FWD_OUT_DENSE_STREAM_X>), grid, threads, lds, stream, a);
       else hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH, FWD_OUT_DENSE_STREAM_X>), grid, threads, lds, stream, a);
     }
