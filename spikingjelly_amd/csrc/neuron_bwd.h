@@ -40,6 +40,14 @@
 #ifndef SJHIP_BWD_NT
 #define SJHIP_BWD_NT 1
 #endif
+// policy of the grad_x stores alone (default: that of the loads)
+#ifndef SJHIP_BWD_STORE_NT
+#define SJHIP_BWD_STORE_NT SJHIP_BWD_NT
+#endif
+// policy of the x loads of the replay phase alone (default: that of the other loads)
+#ifndef SJHIP_REPLAY_X_NT
+#define SJHIP_REPLAY_X_NT SJHIP_BWD_NT
+#endif
 
 namespace sjhip {
 
@@ -286,7 +294,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
             if (PLIF) { g_next[j] = G; h_next[j] = h[j]; }
           }
         }
-        A::store(gxp + t * N, gx);
+        Acc<S, VECTOR, SJHIP_BWD_STORE_NT != 0>::store(gxp + t * N, gx);
       }
     }
   }

@@ -32,7 +32,7 @@ template <typename S> __device__ __forceinline__ uint32_t h_bits(_Float16 h) { r
 
 template <typename S, bool ROUND_EACH, int CH, int RS>
 __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, int64_t col) {
-  typedef Acc<S, true, SJHIP_BWD_NT != 0> A;
+  typedef Acc<S, true, SJHIP_REPLAY_X_NT != 0> A;
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
