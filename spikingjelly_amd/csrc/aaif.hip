@@ -15,6 +15,10 @@
 #define SJHIP_AAIF_PF 8
 #endif
 
+#ifndef SJHIP_AAIF_NT
+#define SJHIP_AAIF_NT 1
+#endif
+
 namespace sjhip {
 
 struct AaifArgs {
@@ -31,7 +35,7 @@ struct AaifArgs {
 
 template <typename S, bool VECTOR, bool ROUND_EACH>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) aaif_forward_kernel(const AaifArgs a) {
-  typedef Acc<S, VECTOR, true> A;  // one read and one write per element, nothing is reused: streaming policy
+  typedef Acc<S, VECTOR, SJHIP_AAIF_NT != 0> A;  // one read and one write per element, nothing is reused: streaming policy
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
@@ -74,7 +78,7 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) aaif_forward_kernel(const Aai
   const float reset_mul = a.v_reset;  // a Python scalar in torch: fp32 as a factor
 
   float v[V];
-  load_state<S, VECTOR, true>(a.v_init, col, a.v_init_broadcast != 0, v);
+  load_state<S, VECTOR, SJHIP_AAIF_NT != 0>(a.v_init, col, a.v_init_broadcast != 0, v);
 
   for (int64_t t0 = 0; t0 < T; t0 += PF) {
     typename A::raw_t now[PF];

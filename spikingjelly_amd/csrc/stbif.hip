@@ -27,6 +27,10 @@
 #define SJHIP_STBIF_PF 8
 #endif
 
+#ifndef SJHIP_STBIF_NT
+#define SJHIP_STBIF_NT 1
+#endif
+
 namespace sjhip {
 
 struct StbifArgs {
@@ -45,7 +49,7 @@ struct StbifArgs {
 
 template <typename S, bool VECTOR, bool ROUND_EACH>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) stbif_forward_kernel(const StbifArgs a) {
-  typedef Acc<S, VECTOR, true> A;  // one read and one write per element, nothing is reused: streaming policy
+  typedef Acc<S, VECTOR, SJHIP_STBIF_NT != 0> A;  // one read and one write per element, nothing is reused: streaming policy
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
@@ -65,8 +69,8 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) stbif_forward_kernel(const St
     for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? A::load(xp + (int64_t)i * N) : A::zero();
 
     float q[V], acc[V], cur[V];
-    load_state<S, VECTOR, true>(a.q_init, col, a.q_broadcast != 0, q);
-    load_state<S, VECTOR, true>(a.acc_init, col, a.acc_broadcast != 0, acc);
+    load_state<S, VECTOR, SJHIP_STBIF_NT != 0>(a.q_init, col, a.q_broadcast != 0, q);
+    load_state<S, VECTOR, SJHIP_STBIF_NT != 0>(a.acc_init, col, a.acc_broadcast != 0, acc);
 #pragma unroll
     for (int j = 0; j < V; ++j) cur[j] = 0.0f;
 
