@@ -180,3 +180,40 @@ def test_config5_full_size_block_matches_torch_backend():
     torch.testing.assert_close(b.proj_conv_bn[0].weight.grad, a.proj_conv_bn[0].weight.grad, rtol=1e-3, atol=1e-3)
     functional.reset_net(a)
     functional.reset_net(b)
+
+
+def test_more_than_two_to_the_32_elements(c_oracle):
+    """T x N beyond 2^32 elements (the reference's kernels index with 32-bit integers and refuse more than 2^31 - 1
+    elements, cuda_kernel/cuda_utils.py:25-30): every element offset is 64-bit here.  Column blocks from every part of
+    the range, the last columns included, against the C oracle, for the forward and the replaying backward."""
+    from spikingjelly_amd.activation_based import neuron, surrogate
+
+    free, _ = torch.cuda.mem_get_info()
+    if free < 100 * (1 << 30):
+        pytest.skip("needs 100 GiB of device memory")
+    T_big, N_big = 16, (1 << 28) + 4096 * 3  # 4 295 163 904 elements per tensor, 17.2 GB in fp32
+    g = torch.Generator(device="cuda").manual_seed(77)
+    x = torch.empty((T_big, N_big), device="cuda")
+    for t in range(T_big):  # row by row: the generator's own kernels need not cope with the full size
+        x[t] = torch.randn((N_big,), generator=g, device="cuda") * 0.8 + 0.3
+    x.requires_grad_()
+    node = neuron.LIFNode(tau=2.0, surrogate_function=surrogate.ATan(2.0), step_mode="m", backend="hip", store_v_seq=False)
+    s = node(x)
+    rng = np.random.default_rng(1)
+    starts = np.concatenate([[0, N_big - 4096, (1 << 28) - 2048], rng.integers(0, N_big - 4096, size=12)])
+    cols = torch.from_numpy(np.concatenate([np.arange(a, a + 4096) for a in starts])).cuda()
+    gs_cols = seeded_randn((T_big, cols.numel()), 78)
+    gs = torch.zeros((T_big, N_big), device="cuda")
+    gs[:, cols] = gs_cols.cuda()
+    s.backward(gs)
+    torch.cuda.synchronize()
+    xs = x.detach()[:, cols].cpu().numpy()
+    es, ev, eh = c_oracle.forward_f32("lif", xs, np.zeros(xs.shape[1], np.float32), 2.0, True, 1.0, 0.0)
+    assert np.array_equal(s.detach()[:, cols].cpu().numpy(), es) and 0.02 < float(es.mean()) < 0.08
+    assert np.array_equal(node.v.detach()[cols].cpu().numpy().view(np.int32), ev[-1].view(np.int32))
+    # duplicate columns in `cols` (blocks may overlap) received the last write of gs_cols: read back what the kernel saw
+    gx, _, _ = c_oracle.backward_f64("lif", gs[:, cols].cpu().numpy(), None, None, eh, 0.5, True, 1.0, 0.0, False, 1, 2.0)
+    np.testing.assert_allclose(x.grad[:, cols].cpu().numpy(), gx, rtol=1e-5, atol=1e-6)
+    # columns that received no upstream gradient have none
+    probe = (1 << 27) + 12345
+    assert probe not in set(cols.tolist()) and float(x.grad[:, probe].abs().max()) == 0.0
