@@ -85,6 +85,18 @@ struct BwdArgs {
 
 // Which extra terms the BPTT walk carries.
 enum BwdMode { BWD_PLAIN = 0, BWD_PLIF = 1, BWD_QIF = 2 };
+// Added to a BwdMode for short sequences: two rows in flight per work-item instead of eight.  The deep prefetch costs
+// registers, i.e. resident wavefronts, and a wavefront with T rows has only T to ask for: at T <= 4 the bytes in flight
+// per compute unit fall below what the memory latency needs (measured, replaying backward, fp32, GB/s of actual
+// traffic with 8 / 2 rows: T = 1: 1.6 / 5.5, T = 2: 2.9 / 6.5, T = 4: 4.7 / 6.2, T = 8: 5.9 / 6.2, T = 16: 6.1 / -).
+constexpr int BWD_SHORT = 4;
+constexpr int kShortRows = 2;
+// sequences up to this length run the BWD_SHORT kernels
+constexpr int64_t kShortSequence = 5;
+template <int MODE> struct BwdModeOf {
+  static constexpr int BASE = MODE & 3;
+  static constexpr bool SHORT = (MODE & BWD_SHORT) != 0;
+};
 
 // FAST (16-bit storage, where the result is rounded to 8 or 11 significant bits anyway) uses the hardware
 // exp2 / reciprocal approximations (about 1 ulp each) in place of the correctly rounded library exp and IEEE
@@ -147,9 +159,9 @@ __device__ __forceinline__ float qif_dh_dv(float v, float k, const BwdArgs &a) {
 // op rounded, where h is exactly a storage-dtype value): as eight 16-bit patterns in one 16-byte word, laid out
 // [step][lane], half the LDS footprint.
 // First PF rows (t = T-1 downwards) of grad_spike and grad_v_seq, requested ahead of their use.
-template <typename S, bool VECTOR> struct BwdPrologue {
+template <typename S, bool VECTOR, bool SHORT = false> struct BwdPrologue {
   typedef Acc<S, VECTOR, SJHIP_BWD_NT != 0> A;
-  static constexpr int PF = (sizeof(S) == 2 && A::V == 8) ? SJHIP_BWD_PF16 : SJHIP_BWD_PF;
+  static constexpr int PF = SHORT ? kShortRows : ((sizeof(S) == 2 && A::V == 8) ? SJHIP_BWD_PF16 : SJHIP_BWD_PF);
   typename A::raw_t gs[PF], gv[PF];
   __device__ __forceinline__ void load(const BwdArgs &a, int64_t col) {
     typedef typename A::elem_t E;
@@ -167,13 +179,13 @@ template <typename S, bool VECTOR> struct BwdPrologue {
 template <typename S, bool VECTOR, int MODE, int SG, bool GVFULL, int HLDS = 0>
 __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, int64_t col, float k,
                                                const f32x4 *lds_h = nullptr,
-                                               const BwdPrologue<S, VECTOR> *pre = nullptr) {
+                                               const BwdPrologue<S, VECTOR, BwdModeOf<MODE>::SHORT> *pre = nullptr) {
   typedef Acc<S, VECTOR, SJHIP_BWD_NT != 0> A;
   typedef typename A::elem_t E;
   constexpr int V = A::V;
-  constexpr int PF = BwdPrologue<S, VECTOR>::PF;
-  constexpr bool PLIF = MODE == BWD_PLIF;
-  constexpr bool QIF = MODE == BWD_QIF;
+  constexpr int PF = BwdPrologue<S, VECTOR, BwdModeOf<MODE>::SHORT>::PF;
+  constexpr bool PLIF = BwdModeOf<MODE>::BASE == BWD_PLIF;
+  constexpr bool QIF = BwdModeOf<MODE>::BASE == BWD_QIF;
 
   float acc_total = 0.0f;
   if (!active) return acc_total;
@@ -325,7 +337,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
 template <typename S, bool VECTOR, int MODE, int SG, int HLDS = 0>
 __device__ __forceinline__ float backward_gv_dispatch(const BwdArgs &a, bool active, int64_t col, float k,
                                                       const f32x4 *lds_h = nullptr,
-                                                      const BwdPrologue<S, VECTOR> *pre = nullptr) {
+                                                      const BwdPrologue<S, VECTOR, BwdModeOf<MODE>::SHORT> *pre = nullptr) {
   if (a.grad_v_seq) return backward_body<S, VECTOR, MODE, SG, true, HLDS>(a, active, col, k, lds_h, pre);
   return backward_body<S, VECTOR, MODE, SG, false, HLDS>(a, active, col, k, lds_h, pre);
 }
@@ -333,7 +345,7 @@ __device__ __forceinline__ float backward_gv_dispatch(const BwdArgs &a, bool act
 template <typename S, bool VECTOR, int MODE, int HLDS>
 __device__ __forceinline__ float backward_sg_dispatch(const BwdArgs &a, bool active, int64_t col, float k,
                                                       const f32x4 *lds_h,
-                                                      const BwdPrologue<S, VECTOR> *pre = nullptr) {
+                                                      const BwdPrologue<S, VECTOR, BwdModeOf<MODE>::SHORT> *pre = nullptr) {
   switch (a.sg) {
     case SJHIP_SG_SIGMOID: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SIGMOID, HLDS>(a, active, col, k, lds_h, pre);
     case SJHIP_SG_ATAN: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_ATAN, HLDS>(a, active, col, k, lds_h, pre);
@@ -342,7 +354,7 @@ __device__ __forceinline__ float backward_sg_dispatch(const BwdArgs &a, bool act
     case SJHIP_SG_SOFT_SIGN: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SOFT_SIGN, HLDS>(a, active, col, k, lds_h, pre);
     case SJHIP_SG_SUPER_SPIKE: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SUPER_SPIKE, HLDS>(a, active, col, k, lds_h, pre);
     case SJHIP_SG_MULTI_LEVEL:
-      if constexpr (MODE == BWD_PLAIN) return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_MULTI_LEVEL, HLDS>(a, active, col, k, lds_h, pre);
+      if constexpr (BwdModeOf<MODE>::BASE == BWD_PLAIN) return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_MULTI_LEVEL, HLDS>(a, active, col, k, lds_h, pre);
       return 0.0f;
     default: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_ERF, HLDS>(a, active, col, k, lds_h, pre);
   }
@@ -376,7 +388,7 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_kernel(const BwdArgs
   const bool active = col < a.N;
   const float k = a.k_device ? *a.k_device : a.k;
   const float part = backward_sg_dispatch<S, VECTOR, MODE, 0>(a, active, col, k, nullptr);
-  if (MODE == BWD_PLIF) plif_block_reduce(a, part, k);
+  if (BwdModeOf<MODE>::BASE == BWD_PLIF) plif_block_reduce(a, part, k);
 }
 
 // ---- host side: turn the ABI parameters into kernel arguments ------------------------------------

@@ -46,7 +46,11 @@ int launch_typed(BwdArgs &a, bool vector, int mode, float *grad_k_out, hipStream
   const unsigned lds = occupancy_cap_lds(tuning().bwd_blocks_per_cu);
   {
     ProfileScope prof(KC_BACKWARD, stream);
-    if (mode == BWD_PLIF) launch_mode<S, BWD_PLIF>(a, vector, grid, threads, lds, stream);
+    if (a.T <= kShortSequence) {
+      if (mode == BWD_PLIF) launch_mode<S, BWD_PLIF | BWD_SHORT>(a, vector, grid, threads, lds, stream);
+      else if (mode == BWD_QIF) launch_mode<S, BWD_QIF | BWD_SHORT>(a, vector, grid, threads, lds, stream);
+      else launch_mode<S, BWD_PLAIN | BWD_SHORT>(a, vector, grid, threads, lds, stream);
+    } else if (mode == BWD_PLIF) launch_mode<S, BWD_PLIF>(a, vector, grid, threads, lds, stream);
     else if (mode == BWD_QIF) launch_mode<S, BWD_QIF>(a, vector, grid, threads, lds, stream);
     else launch_mode<S, BWD_PLAIN>(a, vector, grid, threads, lds, stream);
     int rc = check_launch("backward");

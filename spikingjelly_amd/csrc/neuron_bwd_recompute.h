@@ -30,13 +30,13 @@ namespace sjhip {
 template <typename S> __device__ __forceinline__ uint32_t h_bits(float h) { return Cvt<S>::from_float(h); }
 template <typename S> __device__ __forceinline__ uint32_t h_bits(_Float16 h) { return __builtin_bit_cast(uint16_t, h); }
 
-template <typename S, bool ROUND_EACH, int CH, int RS>
+template <typename S, bool ROUND_EACH, int CH, int RS, bool SHORT>
 __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, int64_t col) {
   typedef Acc<S, true, SJHIP_REPLAY_X_NT != 0> A;
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
-  constexpr int PF = (sizeof(S) == 2 && V == 8) ? SJHIP_REPLAY_PF16 : SJHIP_REPLAY_PF;
+  constexpr int PF = SHORT ? kShortRows : ((sizeof(S) == 2 && V == 8) ? SJHIP_REPLAY_PF16 : SJHIP_REPLAY_PF);
 
   const int64_t N = a.N, T = a.T;
   const E *xp = (const E *)a.x + col;
@@ -83,16 +83,16 @@ __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, i
   }
 }
 
-template <typename S, bool ROUND_EACH, int CH>
+template <typename S, bool ROUND_EACH, int CH, bool SHORT>
 __device__ __forceinline__ void recompute_reset_dispatch(const FwdArgs &a, f32x4 *lds_h, int64_t col) {
   if constexpr (CH == CH_PLAIN_INPUT_DIV || CH == CH_PLAIN_INPUT_MUL) {
     if (a.soft_reset == RESET_COUNT) {
-      recompute_body<S, ROUND_EACH, CH, RESET_COUNT>(a, lds_h, col);
+      recompute_body<S, ROUND_EACH, CH, RESET_COUNT, SHORT>(a, lds_h, col);
       return;
     }
   }
-  if (a.soft_reset) recompute_body<S, ROUND_EACH, CH, RESET_SOFT>(a, lds_h, col);
-  else recompute_body<S, ROUND_EACH, CH, RESET_HARD>(a, lds_h, col);
+  if (a.soft_reset) recompute_body<S, ROUND_EACH, CH, RESET_SOFT, SHORT>(a, lds_h, col);
+  else recompute_body<S, ROUND_EACH, CH, RESET_HARD, SHORT>(a, lds_h, col);
 }
 
 template <typename S, bool ROUND_EACH, int MODE>
@@ -102,25 +102,26 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_kernel(con
   const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
   const bool active = col < b.N;
   // request the last rows of the upstream gradients now, so they arrive while h is being replayed
-  BwdPrologue<S, true> pre;
+  constexpr bool SHORT = BwdModeOf<MODE>::SHORT;
+  BwdPrologue<S, true, SHORT> pre;
   if (active) {
     pre.load(b, col);
     switch (f.charge) {
-      case CH_IF: recompute_reset_dispatch<S, ROUND_EACH, CH_IF>(f, lds_h, col); break;
-      case CH_DECAY_INPUT_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_DECAY_INPUT_DIV>(f, lds_h, col); break;
-      case CH_DECAY_INPUT_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_DECAY_INPUT_MUL>(f, lds_h, col); break;
-      case CH_PLAIN_INPUT_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_PLAIN_INPUT_DIV>(f, lds_h, col); break;
-      case CH_QIF_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_QIF_DIV>(f, lds_h, col); break;
-      case CH_QIF_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_QIF_MUL>(f, lds_h, col); break;
-      case CH_EIF_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_EIF_DIV>(f, lds_h, col); break;
-      case CH_EIF_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_EIF_MUL>(f, lds_h, col); break;
-      default: recompute_reset_dispatch<S, ROUND_EACH, CH_PLAIN_INPUT_MUL>(f, lds_h, col); break;
+      case CH_IF: recompute_reset_dispatch<S, ROUND_EACH, CH_IF, SHORT>(f, lds_h, col); break;
+      case CH_DECAY_INPUT_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_DECAY_INPUT_DIV, SHORT>(f, lds_h, col); break;
+      case CH_DECAY_INPUT_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_DECAY_INPUT_MUL, SHORT>(f, lds_h, col); break;
+      case CH_PLAIN_INPUT_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_PLAIN_INPUT_DIV, SHORT>(f, lds_h, col); break;
+      case CH_QIF_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_QIF_DIV, SHORT>(f, lds_h, col); break;
+      case CH_QIF_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_QIF_MUL, SHORT>(f, lds_h, col); break;
+      case CH_EIF_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_EIF_DIV, SHORT>(f, lds_h, col); break;
+      case CH_EIF_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_EIF_MUL, SHORT>(f, lds_h, col); break;
+      default: recompute_reset_dispatch<S, ROUND_EACH, CH_PLAIN_INPUT_MUL, SHORT>(f, lds_h, col); break;
     }
   }
   const float k = b.k_device ? *b.k_device : b.k;
   constexpr int HLDS = (ROUND_EACH && sizeof(S) == 2) ? 2 : 1;
   const float part = backward_sg_dispatch<S, true, MODE, HLDS>(b, active, col, k, lds_h, &pre);
-  if (MODE == BWD_PLIF) plif_block_reduce(b, part, k);
+  if (BwdModeOf<MODE>::BASE == BWD_PLIF) plif_block_reduce(b, part, k);
 }
 
 // Launches the recompute kernel of storage dtype S; defined in neuron_bwd_recompute_launch.h and

@@ -30,6 +30,11 @@ int launch_kernel(const FwdArgs &f, const BwdArgs &b, int block, unsigned lds, i
 
 template <typename S, bool ROUND_EACH>
 int launch_mode(const FwdArgs &f, const BwdArgs &b, int mode, int block, unsigned lds, int64_t blocks, hipStream_t stream) {
+  if (b.T <= kShortSequence) {
+    if (mode == BWD_PLIF) return launch_kernel<S, ROUND_EACH, BWD_PLIF | BWD_SHORT>(f, b, block, lds, blocks, stream);
+    if (mode == BWD_QIF) return launch_kernel<S, ROUND_EACH, BWD_QIF | BWD_SHORT>(f, b, block, lds, blocks, stream);
+    return launch_kernel<S, ROUND_EACH, BWD_PLAIN | BWD_SHORT>(f, b, block, lds, blocks, stream);
+  }
   if (mode == BWD_PLIF) return launch_kernel<S, ROUND_EACH, BWD_PLIF>(f, b, block, lds, blocks, stream);
   if (mode == BWD_QIF) return launch_kernel<S, ROUND_EACH, BWD_QIF>(f, b, block, lds, blocks, stream);
   return launch_kernel<S, ROUND_EACH, BWD_PLAIN>(f, b, block, lds, blocks, stream);
