@@ -241,18 +241,23 @@ __device__ __forceinline__ void store_spike_bits(uint8_t *row, int64_t col, int6
 // but lost 1.2 % inside the training step, forward and backward alternating, which is the case that counts; 16-bit
 // with every op rounded lost 2 %).
 enum FwdOut { FWD_OUT_DENSE = 0, FWD_OUT_PACKED = 1, FWD_OUT_DENSE_STREAM_X = 2 };
+// Added to a FwdOut for a sequence of one step (what step_mode='s' runs): two rows in flight instead of eight; the
+// registers the deep prefetch would hold go to resident wavefronts instead (T = 1, N = 134 M fp32: 3.7 -> 6.1 TB/s;
+// at T = 2 and 4 the effect is mixed and the deep prefetch stays).
+constexpr int FWD_OUT_SHORT = 4;
 
 template <typename S, bool VECTOR, bool ROUND_EACH, int CH, int RS, int OUT>
 __device__ __forceinline__ void forward_body(const FwdArgs &a) {
-  constexpr bool PACKED = OUT == FWD_OUT_PACKED;
+  constexpr bool PACKED = (OUT & 3) == FWD_OUT_PACKED;
   // with bit-packed spikes the kernel is read-dominated (x in, one bit out): streaming policy like the backward
   constexpr bool NT = (SJHIP_FWD_NT != 0) || (PACKED && SJHIP_FWD_PACKED_NT != 0);
   typedef Acc<S, VECTOR, NT> A;
-  typedef Acc<S, VECTOR, NT || OUT == FWD_OUT_DENSE_STREAM_X> AL;  // policy of the x loads alone
+  typedef Acc<S, VECTOR, NT || (OUT & 3) == FWD_OUT_DENSE_STREAM_X> AL;  // policy of the x loads alone
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
-  constexpr int PF = sizeof(S) == 2 ? SJHIP_FWD_PF16 : SJHIP_FWD_PF;  // (eight 16-bit rows measured slower, packed too)
+  // (eight 16-bit rows measured slower, packed too)
+  constexpr int PF = (OUT & FWD_OUT_SHORT) ? 2 : (sizeof(S) == 2 ? SJHIP_FWD_PF16 : SJHIP_FWD_PF);
 
   const int64_t N = a.N, T = a.T;
   const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
@@ -303,7 +308,7 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
 template <typename S, bool VECTOR, bool ROUND_EACH, int CH, int OUT>
 __device__ __forceinline__ void forward_reset_dispatch(const FwdArgs &a) {
   // counts exist for the charge ILIF uses (no input decay) and never bit-packed
-  if constexpr ((CH == CH_PLAIN_INPUT_DIV || CH == CH_PLAIN_INPUT_MUL) && OUT != FWD_OUT_PACKED) {
+  if constexpr ((CH == CH_PLAIN_INPUT_DIV || CH == CH_PLAIN_INPUT_MUL) && (OUT & 3) != FWD_OUT_PACKED) {
     if (a.soft_reset == RESET_COUNT) {
       forward_body<S, VECTOR, ROUND_EACH, CH, RESET_COUNT, OUT>(a);
       return;

@@ -36,12 +36,15 @@ int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   if constexpr (PACKED) {
     if (vector) hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, FWD_OUT_PACKED>), grid, threads, lds, stream, a);
     else hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH, FWD_OUT_PACKED>), grid, threads, lds, stream, a);
-  } else if (kStreamX<S, ROUND_EACH> && several_outputs) {
+  } else if (kStreamX<S, ROUND_EACH> && several_outputs && a.T > 1) {
     // 16-bit storage with fp32 state writing spikes plus v_seq / h_seq: see FwdOut
     if constexpr (kStreamX<S, ROUND_EACH>) {
       if (vector) hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, FWD_OUT_DENSE_STREAM_X>), grid, threads, lds, stream, a);
       else hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH, FWD_OUT_DENSE_STREAM_X>), grid, threads, lds, stream, a);
     }
+  } else if (a.T == 1) {
+    if (vector) hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, FWD_OUT_DENSE | FWD_OUT_SHORT>), grid, threads, lds, stream, a);
+    else hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH, FWD_OUT_DENSE | FWD_OUT_SHORT>), grid, threads, lds, stream, a);
   } else {
     if (vector) hipLaunchKernelGGL((forward_kernel<S, true, ROUND_EACH, FWD_OUT_DENSE>), grid, threads, lds, stream, a);
     else hipLaunchKernelGGL((forward_kernel<S, false, ROUND_EACH, FWD_OUT_DENSE>), grid, threads, lds, stream, a);
