@@ -88,11 +88,16 @@ enum BwdMode { BWD_PLAIN = 0, BWD_PLIF = 1, BWD_QIF = 2 };
 // Added to a BwdMode for short sequences: two rows in flight per work-item instead of eight.  The deep prefetch costs
 // registers, i.e. resident wavefronts, and a wavefront with T rows has only T to ask for: at T <= 4 the bytes in flight
 // per compute unit fall below what the memory latency needs (measured, replaying backward, fp32, GB/s of actual
-// traffic with 8 / 2 rows: T = 1: 1.6 / 5.5, T = 2: 2.9 / 6.5, T = 4: 4.7 / 6.2, T = 8: 5.9 / 6.2, T = 16: 6.1 / -).
+// traffic with 8 / 2 rows: T = 1: 1.6 / 5.5, T = 2: 2.9 / 6.5, T = 4: 4.7 / 6.2, T = 8: 5.9 / 6.2 without and 6.2 / 6.0 with
+// grad_v_seq; bf16 PLIF with fp32 state at T = 8, N = 8.4 M: 124 -> 110 us; at T = 16 four rows were already 2.5 % slower
+// than eight).
 constexpr int BWD_SHORT = 4;
 constexpr int kShortRows = 2;
 // sequences up to this length run the BWD_SHORT kernels
-constexpr int64_t kShortSequence = 5;
+#ifndef SJHIP_SHORT_SEQUENCE
+#define SJHIP_SHORT_SEQUENCE 8
+#endif
+constexpr int64_t kShortSequence = SJHIP_SHORT_SEQUENCE;
 template <int MODE> struct BwdModeOf {
   static constexpr int BASE = MODE & 3;
   static constexpr bool SHORT = (MODE & BWD_SHORT) != 0;
