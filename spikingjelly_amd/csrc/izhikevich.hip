@@ -149,14 +149,14 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_forward_kernel(con
 
 // Replays the forward recurrence of one work-item (four neurons) from x_seq, v_init and w_init and parks h_t of every
 // step in LDS as fp32; each work-item touches only its own LDS words, so no barrier is needed.
-template <typename S, bool ROUND_EACH, int VAR>
+template <typename S, bool ROUND_EACH, int VAR, bool SHORT>
 __device__ __forceinline__ void izhikevich_replay(const IzhFwdArgs &a, f32x4 *lds_h, int64_t col) {
   typedef Acc<S, true, true> A;
   typedef typename A::elem_t E;
   typedef typename std::conditional<ROUND_EACH, S, float>::type R;
   constexpr int V = A::V;
   static_assert(V == 4, "the replay parks one f32x4 per work-item and step");
-  constexpr int PF = SJHIP_IZH_PF;
+  constexpr int PF = SHORT ? 2 : SJHIP_IZH_PF;
 
   const int64_t N = a.N, T = a.T;
   const E *xp = (const E *)a.x + col;
@@ -192,12 +192,18 @@ __device__ __forceinline__ void izhikevich_replay(const IzhFwdArgs &a, f32x4 *ld
 
 // The first rows of the upstream gradients (and of a saved h_seq) of one work-item, requested before anything else so
 // that they arrive while h is being replayed.
-template <typename S, bool VECTOR, bool REPLAY>
+// RP: IZH_REPLAY (h_t comes from LDS) and / or IZH_SHORT (two rows in flight instead of SJHIP_IZH_PF: for sequences of up
+// to eight steps the registers serve resident wavefronts better; replaying backward fp32, T = 4: 3.4 -> 5.2 TB/s,
+// T = 16: 4.5 -> 4.4)
+constexpr int IZH_REPLAY = 1, IZH_SHORT = 2;
+
+template <typename S, bool VECTOR, int RP>
 struct IzhPrologue {
   typedef Acc<S, VECTOR, true> A;
   typedef typename A::elem_t E;
+  static constexpr bool REPLAY = (RP & IZH_REPLAY) != 0;
   static constexpr int V = A::V;
-  static constexpr int PF = SJHIP_IZH_PF;
+  static constexpr int PF = (RP & IZH_SHORT) ? 2 : SJHIP_IZH_PF;
   typename A::raw_t gs[PF], h[PF], gv[PF], gw[PF];
   float gv_last[V], gw_last[V];
 
@@ -223,13 +229,14 @@ struct IzhPrologue {
 // no branch:
 //     v_t  = s ? fire_h h + fire_c : h            soft: h - v_th            hard: v_reset
 //     dvdh = (1 - s hard) + sg (d_c + d_h h)      soft: 1 - live v_th sg    hard: (1 - s) + sg (v_reset - live h)
-template <typename S, bool VECTOR, bool REPLAY, int SG>
+template <typename S, bool VECTOR, int RP, int SG>
 __device__ __forceinline__ void izhikevich_bptt_walk(const IzhBwdArgs &a, const f32x4 *lds_h, int64_t col,
-                                                     IzhPrologue<S, VECTOR, REPLAY> &pre) {
+                                                     IzhPrologue<S, VECTOR, RP> &pre) {
   typedef Acc<S, VECTOR, true> A;
   typedef typename A::elem_t E;
+  constexpr bool REPLAY = (RP & IZH_REPLAY) != 0;
   constexpr int V = A::V;
-  constexpr int PF = SJHIP_IZH_PF;
+  constexpr int PF = IzhPrologue<S, VECTOR, RP>::PF;
 
   const int64_t N = a.N, T = a.T;
   const E *gsp = (const E *)a.grad_spike + col;
@@ -317,49 +324,51 @@ __device__ __forceinline__ void izhikevich_bptt_walk(const IzhBwdArgs &a, const 
   if (a.grad_w_init) A::store((E *)a.grad_w_init + col, cw_next);
 }
 
-template <typename S, bool VECTOR, bool REPLAY>
+template <typename S, bool VECTOR, int RP>
 __device__ __forceinline__ void izhikevich_bptt(const IzhBwdArgs &a, const f32x4 *lds_h, int64_t col,
-                                                IzhPrologue<S, VECTOR, REPLAY> &pre) {
+                                                IzhPrologue<S, VECTOR, RP> &pre) {
   switch (a.sg) {
-    case SJHIP_SG_SIGMOID: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_SIGMOID>(a, lds_h, col, pre); break;
-    case SJHIP_SG_ATAN: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_ATAN>(a, lds_h, col, pre); break;
-    case SJHIP_SG_PIECEWISE_QUADRATIC: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_PIECEWISE_QUADRATIC>(a, lds_h, col, pre); break;
-    case SJHIP_SG_PIECEWISE_EXP: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_PIECEWISE_EXP>(a, lds_h, col, pre); break;
-    case SJHIP_SG_SOFT_SIGN: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_SOFT_SIGN>(a, lds_h, col, pre); break;
-    case SJHIP_SG_SUPER_SPIKE: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_SUPER_SPIKE>(a, lds_h, col, pre); break;
-    default: izhikevich_bptt_walk<S, VECTOR, REPLAY, SJHIP_SG_ERF>(a, lds_h, col, pre); break;
+    case SJHIP_SG_SIGMOID: izhikevich_bptt_walk<S, VECTOR, RP, SJHIP_SG_SIGMOID>(a, lds_h, col, pre); break;
+    case SJHIP_SG_ATAN: izhikevich_bptt_walk<S, VECTOR, RP, SJHIP_SG_ATAN>(a, lds_h, col, pre); break;
+    case SJHIP_SG_PIECEWISE_QUADRATIC: izhikevich_bptt_walk<S, VECTOR, RP, SJHIP_SG_PIECEWISE_QUADRATIC>(a, lds_h, col, pre); break;
+    case SJHIP_SG_PIECEWISE_EXP: izhikevich_bptt_walk<S, VECTOR, RP, SJHIP_SG_PIECEWISE_EXP>(a, lds_h, col, pre); break;
+    case SJHIP_SG_SOFT_SIGN: izhikevich_bptt_walk<S, VECTOR, RP, SJHIP_SG_SOFT_SIGN>(a, lds_h, col, pre); break;
+    case SJHIP_SG_SUPER_SPIKE: izhikevich_bptt_walk<S, VECTOR, RP, SJHIP_SG_SUPER_SPIKE>(a, lds_h, col, pre); break;
+    default: izhikevich_bptt_walk<S, VECTOR, RP, SJHIP_SG_ERF>(a, lds_h, col, pre); break;
   }
 }
 
-template <typename S, bool VECTOR>
+template <typename S, bool VECTOR, bool SHORT>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_backward_kernel(const IzhBwdArgs a) {
   const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * Acc<S, VECTOR, true>::V;
   if (col >= a.N) return;
-  IzhPrologue<S, VECTOR, false> pre;
+  constexpr int RP = SHORT ? IZH_SHORT : 0;
+  IzhPrologue<S, VECTOR, RP> pre;
   pre.load(a, col);
-  izhikevich_bptt<S, VECTOR, false>(a, nullptr, col, pre);
+  izhikevich_bptt<S, VECTOR, RP>(a, nullptr, col, pre);
 }
 
 // Backward that recomputes h instead of reading a saved h_seq: the forward then never writes h_seq and this kernel
 // reads x_seq in its place.  S is fp32 or a four-neurons-per-work-item 16-bit type; LDS holds T * blockDim * 16 bytes.
-template <typename S, bool ROUND_EACH>
+template <typename S, bool ROUND_EACH, bool SHORT>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) izhikevich_backward_replay_kernel(const IzhFwdArgs f, const IzhBwdArgs a) {
   extern __shared__ f32x4 izh_lds_h[];
   const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (col >= a.N) return;
-  IzhPrologue<S, true, true> pre;
+  constexpr int RP = IZH_REPLAY | (SHORT ? IZH_SHORT : 0);
+  IzhPrologue<S, true, RP> pre;
   pre.load(a, col);
   switch (izhikevich_variant(f)) {
-    case 0: izhikevich_replay<S, ROUND_EACH, 0>(f, izh_lds_h, col); break;
-    case 1: izhikevich_replay<S, ROUND_EACH, 1>(f, izh_lds_h, col); break;
-    case 2: izhikevich_replay<S, ROUND_EACH, 2>(f, izh_lds_h, col); break;
-    case 3: izhikevich_replay<S, ROUND_EACH, 3>(f, izh_lds_h, col); break;
-    case 4: izhikevich_replay<S, ROUND_EACH, 4>(f, izh_lds_h, col); break;
-    case 5: izhikevich_replay<S, ROUND_EACH, 5>(f, izh_lds_h, col); break;
-    case 6: izhikevich_replay<S, ROUND_EACH, 6>(f, izh_lds_h, col); break;
-    default: izhikevich_replay<S, ROUND_EACH, 7>(f, izh_lds_h, col); break;
+    case 0: izhikevich_replay<S, ROUND_EACH, 0, SHORT>(f, izh_lds_h, col); break;
+    case 1: izhikevich_replay<S, ROUND_EACH, 1, SHORT>(f, izh_lds_h, col); break;
+    case 2: izhikevich_replay<S, ROUND_EACH, 2, SHORT>(f, izh_lds_h, col); break;
+    case 3: izhikevich_replay<S, ROUND_EACH, 3, SHORT>(f, izh_lds_h, col); break;
+    case 4: izhikevich_replay<S, ROUND_EACH, 4, SHORT>(f, izh_lds_h, col); break;
+    case 5: izhikevich_replay<S, ROUND_EACH, 5, SHORT>(f, izh_lds_h, col); break;
+    case 6: izhikevich_replay<S, ROUND_EACH, 6, SHORT>(f, izh_lds_h, col); break;
+    default: izhikevich_replay<S, ROUND_EACH, 7, SHORT>(f, izh_lds_h, col); break;
   }
-  izhikevich_bptt<S, true, true>(a, izh_lds_h, col, pre);
+  izhikevich_bptt<S, true, RP>(a, izh_lds_h, col, pre);
 }
 
 namespace {
@@ -394,8 +403,14 @@ int launch_bwd_typed(const IzhBwdArgs &a, bool vector, hipStream_t stream) {
   const int64_t blocks = ((a.N + V - 1) / V + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "izhikevich_backward: N=%lld", (long long)a.N);
   ProfileScope prof(KC_BACKWARD, stream);
-  if (vector) hipLaunchKernelGGL((izhikevich_backward_kernel<S, true>), dim3((unsigned)blocks), dim3(block), 0, stream, a);
-  else hipLaunchKernelGGL((izhikevich_backward_kernel<S, false>), dim3((unsigned)blocks), dim3(block), 0, stream, a);
+  const dim3 grid((unsigned)blocks), threads(block);
+  if (a.T <= kShortSequence) {
+    if (vector) hipLaunchKernelGGL((izhikevich_backward_kernel<S, true, true>), grid, threads, 0, stream, a);
+    else hipLaunchKernelGGL((izhikevich_backward_kernel<S, false, true>), grid, threads, 0, stream, a);
+  } else {
+    if (vector) hipLaunchKernelGGL((izhikevich_backward_kernel<S, true, false>), grid, threads, 0, stream, a);
+    else hipLaunchKernelGGL((izhikevich_backward_kernel<S, false, false>), grid, threads, 0, stream, a);
+  }
   return check_launch("izhikevich_backward");
 }
 
@@ -490,8 +505,13 @@ template <typename S>
 void launch_replay_typed(const IzhFwdArgs &f, const IzhBwdArgs &b, bool round_each, int block, unsigned lds,
                          int64_t blocks, hipStream_t stream) {
   const dim3 grid((unsigned)blocks), threads(block);
-  if (round_each) hipLaunchKernelGGL((izhikevich_backward_replay_kernel<S, true>), grid, threads, lds, stream, f, b);
-  else hipLaunchKernelGGL((izhikevich_backward_replay_kernel<S, false>), grid, threads, lds, stream, f, b);
+  if (b.T <= kShortSequence) {
+    if (round_each) hipLaunchKernelGGL((izhikevich_backward_replay_kernel<S, true, true>), grid, threads, lds, stream, f, b);
+    else hipLaunchKernelGGL((izhikevich_backward_replay_kernel<S, false, true>), grid, threads, lds, stream, f, b);
+  } else {
+    if (round_each) hipLaunchKernelGGL((izhikevich_backward_replay_kernel<S, true, false>), grid, threads, lds, stream, f, b);
+    else hipLaunchKernelGGL((izhikevich_backward_replay_kernel<S, false, false>), grid, threads, lds, stream, f, b);
+  }
 }
 
 }  // namespace
