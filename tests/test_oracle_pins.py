@@ -776,3 +776,51 @@ def test_izhikevich_autograd_matches_finite_differences_of_the_smooth_network():
     wp[2] += eps
     wm[2] -= eps
     assert float(loss(x, v0, wp) - loss(x, v0, wm)) / (2 * eps) == pytest.approx(float(wa.grad[2]), rel=1e-6, abs=1e-8)
+
+
+# ------------------------------------------------------------------------------------------------
+# 8-bit floating-point storage: the conversion the expected values rely on, and the recipe's structure
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("storage", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_torch_float8_conversion_is_round_to_nearest_even_over_the_code_table(storage):
+    """Brute force: the nearest of the 256 decoded codes, ties to the code with an even mantissa; beyond the largest
+    finite value e4m3fn (no infinity) gives NaN once the value rounds past it, e5m2 gives infinity."""
+    codes = torch.arange(256, dtype=torch.uint8)
+    table = codes.view(storage).float().double()
+    finite = torch.isfinite(table)
+    pos = [(float(table[i]), int(codes[i])) for i in range(256) if finite[i] and int(codes[i]) < 128]
+    pos.sort()
+    top, step = pos[-1][0], pos[-1][0] - pos[-2][0]
+    rng = np.random.default_rng(5)
+    samples = np.concatenate([rng.normal(0, 1, 4000), rng.normal(0, 2 ** -7, 2000), rng.normal(0, 100, 2000),
+                              [(a[0] + b[0]) / 2 for a, b in zip(pos[:-1], pos[1:])], [top + step / 2, top + step * 0.51, top * 3]])
+    samples = samples.astype(np.float32)
+    got = torch.from_numpy(samples).to(storage).view(torch.uint8).numpy()
+    for x, code in zip(samples.astype(np.float64), got):
+        mag = abs(x)
+        # the tie between the largest finite value and the first value past it goes to whichever code is even:
+        # e4m3fn's largest finite code (0x7e) is even and keeps it, e5m2's (0x7b) is odd and loses it to infinity
+        top_is_even = (pos[-1][1] & 1) == 0
+        want_special = mag > top + step / 2 or (mag == top + step / 2 and not top_is_even)
+        if want_special:
+            decoded = float(torch.tensor([code], dtype=torch.uint8).view(storage).float())
+            assert math.isnan(decoded) if storage == torch.float8_e4m3fn else math.isinf(decoded), (x, code)
+            continue
+        best = min(pos, key=lambda vc: (abs(vc[0] - mag), vc[1] & 1))  # nearest; on a tie the even code
+        assert (code & 0x7f) == best[1], (x, code, best)
+        assert (code >> 7) == (1 if np.signbit(x) else 0)
+
+
+@pytest.mark.parametrize("storage", [torch.float8_e4m3fn, torch.float8_e5m2, torch.bfloat16])
+@pytest.mark.parametrize("kind,k", [("if", 0.0), ("lif", 0.5), ("plif", 0.25)])
+@pytest.mark.parametrize("v_reset", [0.0, -0.25, None])
+def test_mixed_precision_recipe_is_the_fp32_recurrence_on_rounded_inputs(storage, kind, k, v_reset):
+    """Structure of the recipe: inputs rounded to the storage dtype, the fp32 recurrence (the oracle pinned above) on
+    them with the state never rounded, stored values rounded once.  Rounding what is stored cannot change a spike."""
+    q = lambda t: t.to(storage).float()
+    x, v0 = seeded_randn((9, 300), 61, 0.6, 0.9), seeded_randn((300,), 62, 0.0, 0.3)
+    s, v, h, raw = no.multi_step_mixed_precision(kind, x, v0, storage, k=k, v_reset=v_reset, return_raw_h=True)
+    p = {"if": None, "lif": 1.0 / k if k else None, "plif": torch.tensor(math.log(k / (1 - k))) if k else None}[kind]
+    es, ev, eh = no.multi_step(kind, q(x), q(v0), p, True, 1.0, v_reset)
+    assert torch.equal(s, es) and torch.equal(raw, eh)
+    assert torch.equal(h, q(eh)) and torch.equal(v, q(ev)) and 0.005 < float(s.mean()) < 0.9
