@@ -114,7 +114,8 @@ class InputCompressedGC(torch.autograd.Function):
         x_packed, *args = _combine_args(list(ctx.plain_args), ctx.saved_tensors, ctx.tensor_positions)
         device_type, dtype, enabled = ctx.autocast
         with torch.enable_grad(), torch.autocast(device_type, dtype, enabled):
-            x_seq = ctx.x_compressor.decompress(x_packed, ctx.x_seq_shape).detach().requires_grad_(True)
+            # (the reference always asks for the input's gradient; it is only computed here when somebody wants it)
+            x_seq = ctx.x_compressor.decompress(x_packed, ctx.x_seq_shape).detach().requires_grad_(bool(ctx.needs_input_grad[2]))
             for i, wanted in enumerate(ctx.needs_input_grad[3:]):
                 if torch.is_tensor(args[i]):
                     args[i] = args[i].detach().requires_grad_(wanted and args[i].requires_grad)
@@ -189,17 +190,35 @@ class GCContainer(nn.Sequential):
             flowing = tuple(result) if isinstance(result, (tuple, list)) else (result,)
         return flowing[0] if len(flowing) == 1 else flowing
 
+    def _needs_anchor(self, *values) -> bool:
+        """The segment's parameters are not arguments of the checkpointed function, so when no argument carries a graph
+        (the first segment of a network fed with data) its outputs would be leaves and its parameters would get no
+        gradient: the reference, like ``torch.utils.checkpoint`` in its re-entrant form, has that limitation.  Here an
+        empty tensor that requires a gradient rides along as one more argument in that case."""
+        if not torch.is_grad_enabled() or any(torch.is_tensor(v) and v.requires_grad for v in values):
+            return False
+        return any(p.requires_grad for p in self.parameters())
+
     def stateless_forward(self, x: torch.Tensor, *args: Any) -> Any:
+        if self._needs_anchor(x, *args):
+            anchor = x.new_zeros((0,), dtype=torch.float32).requires_grad_()
+            return input_compressed_gc(lambda x_, *rest: self.super_forward(x_, *rest[:-1]), self.x_compressor, x, *args,
+                                       anchor)
         return input_compressed_gc(self.super_forward, self.x_compressor, x, *args)
 
     def stateful_forward(self, x: torch.Tensor, *args: Any) -> Any:
         n_inputs, n_states = 1 + len(args), self.num_states
+        states = base.extract_memories(self)
+        anchor = ((x.new_zeros((0,), dtype=torch.float32).requires_grad_(),) if self._needs_anchor(x, *args, *states)
+                  else ())
 
         def with_explicit_states(*flat):
+            if anchor:
+                flat = flat[:-1]
             outputs, new_states = self.f_forward(tuple(flat[:n_inputs]), tuple(flat[n_inputs:]))
             return (*outputs, *new_states)
 
-        flat = input_compressed_gc(with_explicit_states, self.x_compressor, x, *args, *base.extract_memories(self))
+        flat = input_compressed_gc(with_explicit_states, self.x_compressor, x, *args, *states, *anchor)
         base.load_memories(self, flat[-n_states:])
         outputs = flat[:-n_states]
         return outputs[0] if len(outputs) == 1 else outputs

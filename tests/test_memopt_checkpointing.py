@@ -185,6 +185,26 @@ def test_stateful_container_equals_the_plain_network(make):
     assert all(not torch.is_tensor(s) for s in base.extract_memories(boxed))
 
 
+@pytest.mark.parametrize("stateful", [False, True])
+def test_first_segment_of_a_network_still_trains_its_parameters(stateful):
+    """Data that requires no gradient into a checkpointed segment: its parameters must get the gradients of the plain
+    segment (the segment's arguments carry no graph then; an anchor argument keeps the function in the graph)."""
+    torch.manual_seed(31)
+    layers = _snn()[:2] if stateful else [nn.Linear(12, 16), nn.ReLU()]
+    plain, boxed = nn.Sequential(*copy.deepcopy(layers)), GCContainer(BitSpikeCompressor(), *copy.deepcopy(layers))
+    x = (seeded_randn((6, 3, 12), 32) > 0.0).float()
+    g = seeded_randn((6, 3, 16), 33)
+    for net in (plain, boxed):
+        out = net(x)
+        assert out.requires_grad
+        out.backward(g)
+    for a, b in zip(boxed.parameters(), plain.parameters()):
+        assert a.grad is not None
+        torch.testing.assert_close(a.grad, b.grad, rtol=1e-6, atol=1e-7)
+    with torch.no_grad():  # and without a graph nothing is anchored
+        assert not boxed(x).requires_grad
+
+
 def test_container_survives_deepcopy_and_pickle():
     box = GCContainer(None, neuron.IFNode(step_mode="m"))
     x = torch.rand(4, 2, 3, generator=torch.Generator().manual_seed(16))
