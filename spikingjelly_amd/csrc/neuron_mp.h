@@ -25,8 +25,13 @@
 
 #include <initializer_list>
 
+// Rows in flight per work-item in the forward and in the backward.  Measured at T = 16, 2^25 neurons, float8 storage:
+// forward 0.514 / 0.527 / 0.537 ms with 2 / 4 / 8 rows, backward 0.83 / 0.81 / 0.87 ms with 1 / 2 / 4.
 #ifndef SJHIP_MP_PF
-#define SJHIP_MP_PF 4
+#define SJHIP_MP_PF 2
+#endif
+#ifndef SJHIP_MP_BWD_PF
+#define SJHIP_MP_BWD_PF 2
 #endif
 #ifndef SJHIP_F8_SOFTWARE
 #define SJHIP_F8_SOFTWARE 0

@@ -10,7 +10,7 @@ __device__ __forceinline__ float mp_backward_walk(const BwdArgs &a, const MpLane
   typedef Tile16<ST> RH;
   typedef Tile16<SP> RG;
   typedef Tile16<float> RO;
-  constexpr int V = 16, PF = 2;
+  constexpr int V = 16, PF = SJHIP_MP_BWD_PF;
   const int64_t N = a.N, T = a.T;
   const float km = a.is_if ? 1.0f : 1.0f - k;
   const float kx = a.is_if ? 1.0f : (a.decay_input ? k : 1.0f);
