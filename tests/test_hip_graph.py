@@ -144,3 +144,53 @@ def test_self_attention_block_with_packed_spikes_replays_from_a_graph():
         torch.cuda.synchronize()
         assert bits_equal(static_y.detach(), want) and float(want.mean()) > 0.02, f"replay {i}: output"
         assert bits_equal(static_gx, want_gx), f"replay {i}: grad_x"
+
+
+@pytest.mark.parametrize("cls,kw", [
+    (neuron.IFNode, {}),
+    (neuron.LIFNode, {"tau": 2.0}),
+    (neuron.ParametricLIFNode, {"init_tau": 2.0}),
+])
+def test_loop_of_single_steps_replays_from_a_graph(cls, kw):
+    """A Python loop over time with ``step_mode='s'`` (state and its gradient carried between the calls), recorded with
+    its backward by the package's helper; a replay costs one launch of the graph instead of 2 T operator calls."""
+    from spikingjelly_amd.activation_based.hip_kernel.graph import GraphedStep
+
+    node = cls(step_mode="s", backend="hip", surrogate_function=surrogate.ATan(), **kw).cuda()
+    reference = cls(step_mode="m", backend="hip", surrogate_function=surrogate.ATan(), **kw).cuda()
+    T, B, C = 6, 32, 96
+
+    def step(x_seq, gs_seq):
+        spikes = torch.stack([node(x_seq[t]) for t in range(x_seq.shape[0])])
+        (spikes * gs_seq).sum().backward()
+        functional.reset_net(node)
+        return spikes.detach()
+
+    x0 = seeded_randn((T, B, C), 1, 0.5, 1.0).cuda().requires_grad_()
+    graphed = GraphedStep(step, [x0, seeded_randn((T, B, C), 2).cuda()], parameters=node.parameters())
+    for i in range(4):
+        x, gs = seeded_randn((T, B, C), 10 + i, 0.5, 1.0).cuda(), seeded_randn((T, B, C), 20 + i).cuda()
+        want_s, want_gx = _eager_step(reference, x, gs)  # the multi-step kernels, eagerly, between the replays
+        want_gw = [p.grad.clone() for p in reference.parameters()]
+        reference.zero_grad(set_to_none=True)
+        torch.cuda.synchronize()
+        got_s = graphed(x, gs)
+        torch.cuda.synchronize()
+        assert bits_equal(got_s, want_s), f"replay {i}: spikes"
+        assert torch.allclose(graphed.static_inputs[0].grad, want_gx, rtol=1e-5, atol=1e-6), f"replay {i}: grad_x"
+        for p, w in zip(node.parameters(), want_gw):
+            assert torch.allclose(p.grad, w, rtol=1e-4, atol=1e-5), f"replay {i}: parameter gradient"
+
+
+def test_graphed_step_checks_what_it_is_given():
+    from spikingjelly_amd.activation_based.hip_kernel.graph import GraphedStep
+
+    x = seeded_randn((4, 64), 1).cuda()
+    graphed = GraphedStep(lambda a: functional.lif_multi_step_hip(a, torch.zeros_like(a[0]), 2.0, True, 1.0, 0.0,
+                                                                  surrogate.ATan())[0], [x])
+    with pytest.raises(ValueError, match="recorded with"):
+        graphed(x[:2])
+    with pytest.raises(ValueError, match="recorded with"):
+        graphed(x, x)
+    with pytest.raises(ValueError, match="on the GPU"):
+        GraphedStep(lambda a: a, [torch.zeros(3)])
