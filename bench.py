@@ -358,7 +358,7 @@ def other_workload(args) -> int:
               {"bound": "hbm", "achieved": bytes_b / (sb * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                "frac": bytes_b / (sb * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "ssa_backward",
                "kernel_ms": sb, "algorithmic_bytes": bytes_b,
-               "ssa_backward_fp32_mfma_TFLOPs": 4 * product / (sb * 1e-3) / 1e12,
+               "ssa_backward_TFLOPs": 4 * product / (sb * 1e-3) / 1e12,
                "ssa_forward_ms": sf, "ssa_forward_GBs": bytes_f / (sf * 1e-3) / 1e9,
                "ssa_forward_TFLOPs": 2 * product / (sf * 1e-3) / 1e12,
                "lif_forward_ms": _kernel_ms(L, L.KC_FORWARD), "lif_backward_ms": _kernel_ms(L, L.KC_BACKWARD)})

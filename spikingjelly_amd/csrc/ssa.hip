@@ -19,10 +19,12 @@
 // Hence the forward equals an int64 matmul of the spikes times scale, bit for bit, in fp32 output,
 // and after one rounding in 16-bit output (what torch's bf16 matmuls also produce).
 //
-// The backward has real-valued operands (grad_out, dS), so those products use the fp32 MFMA:
-//   dS = scale * dO Q^T  (v_mfma_f32_16x16x4_f32, one 16x16 block per wavefront, through LDS),
-//   dQ = scale * S^T dO,  dK = dS^T V,  dV = dS K  (v_mfma_f32_32x32x2_f32, column tiles dealt to wavefronts),
-// with S recomputed on the int8 MFMA where it is needed and kept in registers.
+// The backward has one real-valued operand per product (grad_out or dS) and one exact one (spikes, or S <= 256):
+//   dS = scale * dO Q^T  (v_mfma_f32_16x16x4_f32, one 16x16 block per wavefront, through LDS; the contraction over the
+//        tokens is long and the output small, so splitting dO would cost more VALU work than the fp32 MFMA takes),
+//   dQ = scale * S^T dO,  dK = dS^T V,  dV = dS K  on v_mfma_f32_32x32x16_bf16: the real operand is split into three
+//        bf16 terms that sum to it exactly (Bf16Terms), so the products are the ones an fp32 MFMA would form; column
+//        tiles are dealt to wavefronts, S is recomputed on the int8 MFMA and kept in registers.
 //
 // MFMA layouts used (lane = 0..63):  32x32: A element of lane is row lane % 32, k group lane / 32; B likewise
 // with column lane % 32; accumulator register r sits at row 8 (r / 4) + 4 (lane / 32) + r % 4, column
@@ -31,6 +33,14 @@
 #include "sjhip_common.h"
 
 #include <mutex>
+
+// Resident blocks per compute unit the backward kernel's register allocation is sized for (heads of up to 32
+// channels).  Sized for 2 the kernel takes 124 registers and keeps the split dS operands across the column tiles
+// without spilling, so three blocks are resident anyway (what LDS allows); sized for 3 the allocator spills 40
+// registers around the same code (80 us against 83 us at 256 samples x 12 heads x 32 x 196).
+#ifndef SJHIP_SSA_BWD_RESIDENT
+#define SJHIP_SSA_BWD_RESIDENT 2
+#endif
 
 namespace sjhip {
 
@@ -261,6 +271,28 @@ __device__ __forceinline__ i32x16 spike_gram(const uint8_t *a, int ra, const uin
   return acc;
 }
 
+// Eight fp32 values as three bf16 operands whose sum is the values exactly: every term keeps the next eight significant
+// bits by truncation (24 in all, an fp32 significand), and the differences taken in between are exact.  A product of a
+// term with a spike or with a count <= 256 is exact in fp32, so a bf16 MFMA over the three terms accumulates the same
+// products as an fp32 MFMA would, at sixteen times its rate.
+struct Bf16Terms {
+  uint32_t w[3][4];
+  __device__ __forceinline__ void set(int j, float x0, float x1) {
+    constexpr uint32_t kTop = 0xffff0000u;
+    const uint32_t a0 = __builtin_bit_cast(uint32_t, x0), a1 = __builtin_bit_cast(uint32_t, x1);
+    const float r0 = x0 - __builtin_bit_cast(float, a0 & kTop), r1 = x1 - __builtin_bit_cast(float, a1 & kTop);
+    const uint32_t b0 = __builtin_bit_cast(uint32_t, r0), b1 = __builtin_bit_cast(uint32_t, r1);
+    const float q0 = r0 - __builtin_bit_cast(float, b0 & kTop), q1 = r1 - __builtin_bit_cast(float, b1 & kTop);
+    w[0][j] = (a0 >> 16) | (a1 & kTop);
+    w[1][j] = (b0 >> 16) | (b1 & kTop);
+    w[2][j] = (__builtin_bit_cast(uint32_t, q0) >> 16) | (__builtin_bit_cast(uint32_t, q1) & kTop);
+  }
+  __device__ __forceinline__ bf16x8 term(int t) const {
+    uint32_t v[4] = {w[t][0], w[t][1], w[t][2], w[t][3]};
+    return __builtin_bit_cast(bf16x8, v);
+  }
+};
+
 // accumulator register r of this lane sits at (row, col) of its 32x32 block
 __device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
 
@@ -335,17 +367,23 @@ __global__ void __launch_bounds__(kSsaThreads) ssa_forward_kernel(const SsaArgs 
       }
     }
     if (col < L) {
+      // 32-bit offsets from the uniform tile base; accumulator row r is a constant number of tile rows from the first
+      const uint32_t first = (uint32_t)(ni * 32 + 4 * half) * (uint32_t)L + (uint32_t)col;
+      if (cph == CPH) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = ni * 32 + acc_row(r, lane);
-        if (row < cph) Io<S>::put(og, (int64_t)row * L + col, acc[r] * a.scale);
+        for (int r = 0; r < 16; ++r) Io<S>::put(og, first + (uint32_t)(8 * (r >> 2) + (r & 3)) * (uint32_t)L, acc[r] * a.scale);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (ni * 32 + acc_row(r, lane) < cph)
+            Io<S>::put(og, first + (uint32_t)(8 * (r >> 2) + (r & 3)) * (uint32_t)L, acc[r] * a.scale);
       }
     }
   }
 }
 
 template <typename S, int MC>
-__global__ void __launch_bounds__(kSsaThreads, MC == 1 ? 3 : 1) ssa_backward_kernel(const SsaArgs a) {
+__global__ void __launch_bounds__(kSsaThreads, MC == 1 ? SJHIP_SSA_BWD_RESIDENT : 1) ssa_backward_kernel(const SsaArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char ssa_lds[];
   typedef typename Io<S>::elem_t E;
   constexpr int CPH = 32 * MC;
@@ -409,46 +447,105 @@ __global__ void __launch_bounds__(kSsaThreads, MC == 1 ? 3 : 1) ssa_backward_ker
   E *gq = static_cast<E *>(a.grad_qkv);
   const int ntiles = (L + 31) / 32;
   const int m32 = lane & 31;
-  for (int nt = wave; nt < ntiles; nt += kSsaWaves) {
-    const int col = nt * 32 + m32;
-    const int colc = col < L ? col : L - 1;
 #pragma unroll 1
-    for (int b = 0; b < MC; ++b) {
-      // S blocks (V K^T) of column block b, exact, in registers: lane (c2, half) register r of block ai holds
-      // S[32 ai + 8 (r/4) + 4 half + r%4, 32 b + c2]
-      float s_reg[MC][16];
+  for (int b = 0; b < MC; ++b) {
+    // s_op: S^T blocks (V K^T, exact, <= 256 so exact in bf16) in the order the accumulator holds them: element e of
+    // (ai, h) stands for c1 = 32 ai + 16 h + 8 (e / 4) + 4 half + e % 4.  In the dS operands of dK and dV element e of
+    // (ai, h) stands for c = 32 ai + 16 h + 8 half + e.
+    bf16x8 s_op[MC][2];
 #pragma unroll
-      for (int ai = 0; ai < MC; ++ai) {
-        const i32x16 acc = spike_gram(v_lds, ai * 32, k_lds, b * 32, Lb, lane);
+    for (int ai = 0; ai < MC; ++ai) {
+      const i32x16 acc = spike_gram(v_lds, ai * 32, k_lds, b * 32, Lb, lane);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s_reg[ai][r] = (float)acc[r];
+      for (int h = 0; h < 2; ++h) {
+        uint16_t w[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) w[e] = (uint16_t)(__builtin_bit_cast(uint32_t, (float)acc[8 * h + e]) >> 16);
+        s_op[ai][h] = __builtin_bit_cast(bf16x8, w);
       }
-      f32x16 dq = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-      f32x16 dk = dq, dv = dq;
+    }
+    // One product at a time: sixteen accumulator registers live instead of forty-eight.
+    for (int nt = wave; nt < ntiles; nt += kSsaWaves) {
+      const int col = nt * 32 + m32;
+      const int colc = col < L ? col : L - 1;
+      const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+      // (the dS operands of dK and dV do not depend on the tile: the compiler forms them once, ahead of this loop)
+      // 32-bit offsets from one uniform base per tensor: a row of the accumulator is a constant number of tile rows
+      // away from the lane's first one
+      const uint32_t first = (uint32_t)(b * 32 + 4 * half) * (uint32_t)L + (uint32_t)col;
+      auto store = [&](E *tile_base, const f32x16 &acc, float factor) {
+        if (col >= L) return;
+        if (cph == CPH) {
 #pragma unroll
-      for (int ai = 0; ai < MC; ++ai) {
+          for (int r = 0; r < 16; ++r)
+            Io<S>::put(tile_base, first + (uint32_t)(8 * (r >> 2) + (r & 3)) * (uint32_t)L, acc[r] * factor);
+        } else {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          // dQ[c2, l] += S[c1, c2] dO[c1, l], c1 in the order the S registers hold it
-          const int c1s = ai * 32 + acc_row(r, lane);
-          dq = __builtin_amdgcn_mfma_f32_32x32x2f32(s_reg[ai][r], do_lds[c1s * Lq + colc], dq, 0, 0, 0);
-          const int kk = ai * 32 + 2 * r + half;
-          // dK[c2, l] += dS[c1 = kk, c2] V[kk, l]
-          dk = __builtin_amdgcn_mfma_f32_32x32x2f32(ds_lds[kk * LS + b * 32 + m32], (float)v_lds[kk * Lb + colc], dk, 0, 0, 0);
-          // dV[c1, l] += dS[c1, c2 = kk] K[kk, l]
-          dv = __builtin_amdgcn_mfma_f32_32x32x2f32(ds_lds[(b * 32 + m32) * LS + kk], (float)k_lds[kk * Lb + colc], dv, 0, 0, 0);
+          for (int r = 0; r < 16; ++r)
+            if (b * 32 + acc_row(r, lane) < cph)
+              Io<S>::put(tile_base, first + (uint32_t)(8 * (r >> 2) + (r & 3)) * (uint32_t)L, acc[r] * factor);
         }
+      };
+      {  // dQ[c2, l] = scale * sum_c1 S[c1, c2] dO[c1, l], c1 in the order of s_op
+        f32x16 acc = zero;
+#pragma unroll
+        for (int ai = 0; ai < MC; ++ai) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            Bf16Terms t;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int c1 = ai * 32 + 16 * h + 8 * (j >> 1) + 4 * half + 2 * (j & 1);
+              t.set(j, do_lds[c1 * Lq + colc], do_lds[(c1 + 1) * Lq + colc]);
+            }
+#pragma unroll
+            for (int i = 2; i >= 0; --i)  // smallest terms first
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s_op[ai][h], t.term(i), acc, 0, 0, 0);
+          }
+        }
+        store(gq + qoff, acc, scale);
       }
-      if (col < L) {
+      {  // dK[c2, l] = sum_c dS[c, c2] V[c, l]
+        f32x16 acc = zero;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = b * 32 + acc_row(r, lane);
-          if (row >= cph) continue;
-          const int64_t o = (int64_t)row * L + col;
-          Io<S>::put(gq, qoff + o, dq[r] * scale);
-          Io<S>::put(gq, koff + o, dk[r]);
-          Io<S>::put(gq, voff + o, dv[r]);
+        for (int ai = 0; ai < MC; ++ai) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            Bf16Terms t;
+            uint32_t w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int c = ai * 32 + 16 * h + 8 * half + 2 * j;
+              t.set(j, ds_lds[c * LS + b * 32 + m32], ds_lds[(c + 1) * LS + b * 32 + m32]);
+              w[j] = ((uint32_t)v_lds[c * Lb + colc] | ((uint32_t)v_lds[(c + 1) * Lb + colc] << 16)) * 0x3f80u;  // 1 -> bf16 1.0
+            }
+            const bf16x8 spikes = __builtin_bit_cast(bf16x8, w);
+#pragma unroll
+            for (int i = 2; i >= 0; --i) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.term(i), spikes, acc, 0, 0, 0);
+          }
         }
+        store(gq + koff, acc, 1.0f);
+      }
+      {  // dV[c1, l] = sum_c dS[c1, c] K[c, l]
+        f32x16 acc = zero;
+#pragma unroll
+        for (int ai = 0; ai < MC; ++ai) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            Bf16Terms t;
+            uint32_t w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int c = ai * 32 + 16 * h + 8 * half + 2 * j;
+              t.set(j, ds_lds[(b * 32 + m32) * LS + c], ds_lds[(b * 32 + m32) * LS + c + 1]);
+              w[j] = ((uint32_t)k_lds[c * Lb + colc] | ((uint32_t)k_lds[(c + 1) * Lb + colc] << 16)) * 0x3f80u;
+            }
+            const bf16x8 spikes = __builtin_bit_cast(bf16x8, w);
+#pragma unroll
+            for (int i = 2; i >= 0; --i) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.term(i), spikes, acc, 0, 0, 0);
+          }
+        }
+        store(gq + voff, acc, 1.0f);
       }
     }
   }
