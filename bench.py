@@ -230,20 +230,19 @@ def other_workload(args) -> int:
 
         def step():
             s, v_seq, h_seq = M.hip_multistep_mp_forward(x, v0, None, *scalars, f8, sp, True)
-            M.hip_multistep_mp_backward(gs, gv, h_seq, v0, None, *scalars, sp)
+            M.hip_multistep_mp_backward(gs, gv, h_seq, v0, None, *scalars, sp, True)
             if not rate:
                 rate.append(float(s.float().mean()))
 
         elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
         f_ms, b_ms = _kernel_ms(L, L.KC_FORWARD), _kernel_ms(L, L.KC_BACKWARD)
         fwd_bytes = 5 * T * N + N          # x 1, spikes 2, v_seq 1, h_seq 1; v_init
-        bwd_bytes = 8 * T * N + 4 * N      # grad_spike 2, grad_v 1, h_seq 1, grad_x 4 (fp32); grad_v_init
+        bwd_bytes = 5 * T * N + N          # grad_spike 2, grad_v 1, h_seq 1, grad_x 1 (storage dtype, as x is); grad_v_init
         dom, d_ms, d_bytes = ("forward", f_ms, fwd_bytes) if f_ms >= b_ms else ("backward", b_ms, bwd_bytes)
         _emit(args, "neuron-steps/sec LIF fwd+bwd float8_e4m3fn storage T=16 N=33.5M, 1 MI355X", "neuron-steps/s",
               T * N / (elapsed / args.steps), elapsed, "f32",
               {"workload": "sj::hip_multistep_mp_forward + _backward, LIF tau=2, hard reset 0, ATan(2), x [16, 33554432] "
-                           "float8_e4m3fn ~N(0.3,0.8), spikes and grad_spike bf16, v_seq / h_seq / grad_v float8_e4m3fn, "
-                           "grad_x fp32", "T": T, "N": N, "firing_rate": rate[0]},
+                           "float8_e4m3fn ~N(0.3,0.8), spikes and grad_spike bf16, v_seq / h_seq / grad_v / grad_x float8_e4m3fn", "T": T, "N": N, "firing_rate": rate[0]},
               {"bound": "hbm", "achieved": d_bytes / (d_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                "frac": d_bytes / (d_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": dom, "kernel_ms": d_ms,
                "algorithmic_bytes": d_bytes, "forward_ms": f_ms, "backward_ms": b_ms,

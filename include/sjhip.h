@@ -111,6 +111,8 @@ typedef enum sjhip_surrogate {
 #define SJHIP_FLAG_V_INIT_BROADCAST 0x100u /* v_init points to ONE element that every neuron starts from (a
                                               module state that is still its scalar reset value): no [N]
                                               tensor has to be filled and read */
+#define SJHIP_FLAG_GRAD_STORAGE 0x1000u /* sjhip_neuron_backward_mp: grad_x_seq and grad_v_init are written in the
+                                           storage dtype instead of fp32 (0x200 - 0x800 are taken further down) */
 
 /* Scalars of one neuron layer.  `tau` is tau for LIF and the reciprocal k = sigmoid(w) for PLIF
  * (ignored for IF).  `v_reset` is ignored for IF soft reset and is the charge-equation offset
@@ -259,7 +261,8 @@ int sjhip_stbif_forward(int dtype, uint32_t flags, int64_t T, int64_t N,
  * `storage_dtype` (SJHIP_F8E4M3 or SJHIP_F8E5M2), spike_seq and grad_spike_seq are `spike_dtype` (SJHIP_F32, SJHIP_F16
  * or SJHIP_BF16), the recurrence runs in fp32 on the decoded values and only stored values are rounded (round to
  * nearest even as torch's .to(torch.float8_*): e4m3fn has no infinity and overflows to NaN, e5m2 overflows to
- * infinity); grad_x_seq [T,N] and grad_v_init [N] are fp32.  Same params, flags and PLIF conventions as
+ * infinity); grad_x_seq [T,N] and grad_v_init [N] are fp32, or, with SJHIP_FLAG_GRAD_STORAGE, `storage_dtype` like the
+ * reference's (lif.py:1115-1118 allocates them in the dtypes of x_seq and v_init; the fp32 value is rounded once).  Same params, flags and PLIF conventions as
  * sjhip_neuron_forward / sjhip_neuron_backward (PLIF: rtau_device, grad_rtau and a workspace of
  * sjhip_plif_workspace_floats(SJHIP_F32, N) floats).  N must be a multiple of 4 and every tensor 16-byte aligned
  * (a work-item owns four groups of four neurons: one 4-byte access per group of an 8-bit row); callers pad.
@@ -271,7 +274,7 @@ int sjhip_neuron_forward_mp(int neuron, int storage_dtype, int spike_dtype, cons
 int sjhip_neuron_backward_mp(int neuron, int storage_dtype, int spike_dtype, const sjhip_neuron_params *p,
                              int64_t T, int64_t N, const void *grad_spike_seq, const void *grad_v_seq,
                              const void *grad_v_last, const void *h_seq, const void *v_init,
-                             const float *rtau_device, float *grad_x_seq, float *grad_v_init, float *grad_rtau,
+                             const float *rtau_device, void *grad_x_seq, void *grad_v_init, float *grad_rtau,
                              float *workspace, void *stream);
 
 /*

@@ -31,6 +31,7 @@ FLAG_V_INIT_BROADCAST = 0x100
 FLAG_Q_BROADCAST = 0x200
 FLAG_ACC_BROADCAST = 0x400
 FLAG_W_INIT_BROADCAST = 0x800
+FLAG_GRAD_STORAGE = 0x1000
 
 KC_FORWARD, KC_BACKWARD, KC_PLIF_REDUCE, KC_BIT_PACK, KC_BIT_UNPACK, KC_SSA_FORWARD, KC_SSA_BACKWARD = range(7)
 

@@ -212,9 +212,13 @@ def _(x_seq, v_init, k, neuron, tau, decay_input, v_th, v_reset, soft_reset, det
 def hip_multistep_mp_backward(grad_s_seq: Optional[torch.Tensor], grad_v_seq: Optional[torch.Tensor],
                               h_seq: torch.Tensor, v_init: torch.Tensor, k: Optional[torch.Tensor], neuron: int,
                               tau: float, decay_input: bool, v_th: float, v_reset: float, soft_reset: bool,
-                              detach_reset: bool, sg_id: int, sg_alpha: float, spike_dtype: torch.dtype
-                              ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """-> fp32 ``(grad_x_seq [T, N], grad_v_init [N], grad_k [] )``; ``grad_k`` is zero unless PLIF."""
+                              detach_reset: bool, sg_id: int, sg_alpha: float, spike_dtype: torch.dtype,
+                              grads_in_storage: bool = False) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """-> ``(grad_x_seq [T, N], grad_v_init [N], grad_k [] )``; ``grad_k`` (fp32) is zero unless PLIF.
+
+    The first two are fp32, or, with ``grads_in_storage``, the 8-bit storage dtype: the kernel rounds its fp32 value
+    once, which is what casting the fp32 result gives, and writes a quarter of the bytes (the reference allocates them
+    in the dtypes of ``x_seq`` and ``v_init``, ``triton_kernel/neuron_kernel/lif.py:1115-1118``)."""
     L.require_device_tensor("h_seq", h_seq)
     storage_dtype = h_seq.dtype
     T, N = h_seq.shape
@@ -224,15 +228,17 @@ def hip_multistep_mp_backward(grad_s_seq: Optional[torch.Tensor], grad_v_seq: Op
                  else grad_s_seq.to(spike_dtype)))
     gv = None if grad_v_seq is None else _pad16(grad_v_seq.to(storage_dtype))
     v8 = _pad16(v_init.to(storage_dtype))
-    grad_x = torch.empty((T, Np), dtype=torch.float32, device=h_seq.device)
-    grad_v_init = torch.empty((Np,), dtype=torch.float32, device=h_seq.device)
+    grad_dtype = storage_dtype if grads_in_storage else torch.float32
+    grad_x = torch.empty((T, Np), dtype=grad_dtype, device=h_seq.device)
+    grad_v_init = torch.empty((Np,), dtype=grad_dtype, device=h_seq.device)
     grad_k = torch.zeros((), dtype=torch.float32, device=h_seq.device)
     workspace = None
     if neuron == L.NEURON_PLIF:
         workspace = torch.empty((L.load().sjhip_plif_workspace_floats(L.DTYPE_F32, Np),), dtype=torch.float32,
                                 device=h_seq.device)
     k_keep, k_ptr = K._k_pointer(k, h_seq)
-    params = _mp_params(tau, v_th, v_reset, sg_alpha, sg_id, K._flags(soft_reset, detach_reset, decay_input, 0))
+    flags = K._flags(soft_reset, detach_reset, decay_input, 0) | (L.FLAG_GRAD_STORAGE if grads_in_storage else 0)
+    params = _mp_params(tau, v_th, v_reset, sg_alpha, sg_id, flags)
     with torch.cuda.device(h_seq.device):
         rc = L.load().sjhip_neuron_backward_mp(neuron, _F8_IDS[storage_dtype], L.dtype_id(spike_dtype), ctypes.byref(params),
                                                T, Np, gs.data_ptr(), L.ptr(gv), None, h8.data_ptr(), v8.data_ptr(), k_ptr,
@@ -247,8 +253,9 @@ def hip_multistep_mp_backward(grad_s_seq: Optional[torch.Tensor], grad_v_seq: Op
 
 @hip_multistep_mp_backward.register_fake
 def _(grad_s_seq, grad_v_seq, h_seq, v_init, k, neuron, tau, decay_input, v_th, v_reset, soft_reset, detach_reset, sg_id,
-      sg_alpha, spike_dtype):
-    return (h_seq.new_empty(h_seq.shape, dtype=torch.float32), h_seq.new_empty(h_seq.shape[1:], dtype=torch.float32),
+      sg_alpha, spike_dtype, grads_in_storage=False):
+    grad_dtype = h_seq.dtype if grads_in_storage else torch.float32
+    return (h_seq.new_empty(h_seq.shape, dtype=grad_dtype), h_seq.new_empty(h_seq.shape[1:], dtype=grad_dtype),
             h_seq.new_empty((), dtype=torch.float32))
 
 
@@ -267,7 +274,8 @@ def _mp_backward(ctx, grad_s_seq, grad_v_seq, grad_h_seq):
     del grad_h_seq
     h_seq, v_init, k = ctx.saved_tensors
     x_dtype, v_dtype, spike_dtype = ctx.dtypes
-    gx, gv0, gk = hip_multistep_mp_backward(grad_s_seq, grad_v_seq, h_seq, v_init, k, *ctx.scalars, spike_dtype)
+    in_storage = x_dtype == h_seq.dtype and v_dtype == h_seq.dtype  # otherwise fp32 results, cast below
+    gx, gv0, gk = hip_multistep_mp_backward(grad_s_seq, grad_v_seq, h_seq, v_init, k, *ctx.scalars, spike_dtype, in_storage)
     grad_k = gk.to(k.dtype).reshape(k.shape) if (k is not None and ctx.needs_input_grad[2]) else None
     return (gx.to(x_dtype), gv0.to(v_dtype) if ctx.needs_input_grad[1] else None, grad_k) + (None,) * 12
 

@@ -4,12 +4,13 @@
 namespace sjhip {
 
 // BPTT over the stored (8-bit) h_seq; the recurrence and the PLIF sum are those of neuron_bwd.h.  grad_spike_seq is in
-// the spike dtype, grad_v_seq / grad_v_last in the storage dtype, the results are fp32.
-template <typename ST, typename SP, int SG, bool PLIF>
+// the spike dtype, grad_v_seq / grad_v_last in the storage dtype; the results leave in GO: fp32, or the storage dtype
+// (rounded once from the fp32 value, what a cast of the fp32 result gives; 5 instead of 8 bytes per neuron-step).
+template <typename ST, typename SP, typename GO, int SG, bool PLIF>
 __device__ __forceinline__ float mp_backward_walk(const BwdArgs &a, const MpLane &l, float k) {
   typedef Tile16<ST> RH;
   typedef Tile16<SP> RG;
-  typedef Tile16<float> RO;
+  typedef Tile16<GO> RO;
   constexpr int V = 16, PF = SJHIP_MP_BWD_PF;
   const int64_t N = a.N, T = a.T;
   const float km = a.is_if ? 1.0f : 1.0f - k;
@@ -97,20 +98,20 @@ __device__ __forceinline__ float mp_backward_walk(const BwdArgs &a, const MpLane
   return total;
 }
 
-template <typename ST, typename SP, bool PLIF>
+template <typename ST, typename SP, typename GO, bool PLIF>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) mp_backward_kernel(const BwdArgs a) {
   const MpLane l = mp_lane(a.N);
   const float k = a.k_device ? *a.k_device : a.k;
   float part = 0.0f;
   if (l.groups != 0) {
     switch (a.sg) {
-      case SJHIP_SG_SIGMOID: part = mp_backward_walk<ST, SP, SJHIP_SG_SIGMOID, PLIF>(a, l, k); break;
-      case SJHIP_SG_ATAN: part = mp_backward_walk<ST, SP, SJHIP_SG_ATAN, PLIF>(a, l, k); break;
-      case SJHIP_SG_PIECEWISE_QUADRATIC: part = mp_backward_walk<ST, SP, SJHIP_SG_PIECEWISE_QUADRATIC, PLIF>(a, l, k); break;
-      case SJHIP_SG_PIECEWISE_EXP: part = mp_backward_walk<ST, SP, SJHIP_SG_PIECEWISE_EXP, PLIF>(a, l, k); break;
-      case SJHIP_SG_SOFT_SIGN: part = mp_backward_walk<ST, SP, SJHIP_SG_SOFT_SIGN, PLIF>(a, l, k); break;
-      case SJHIP_SG_SUPER_SPIKE: part = mp_backward_walk<ST, SP, SJHIP_SG_SUPER_SPIKE, PLIF>(a, l, k); break;
-      default: part = mp_backward_walk<ST, SP, SJHIP_SG_ERF, PLIF>(a, l, k); break;
+      case SJHIP_SG_SIGMOID: part = mp_backward_walk<ST, SP, GO, SJHIP_SG_SIGMOID, PLIF>(a, l, k); break;
+      case SJHIP_SG_ATAN: part = mp_backward_walk<ST, SP, GO, SJHIP_SG_ATAN, PLIF>(a, l, k); break;
+      case SJHIP_SG_PIECEWISE_QUADRATIC: part = mp_backward_walk<ST, SP, GO, SJHIP_SG_PIECEWISE_QUADRATIC, PLIF>(a, l, k); break;
+      case SJHIP_SG_PIECEWISE_EXP: part = mp_backward_walk<ST, SP, GO, SJHIP_SG_PIECEWISE_EXP, PLIF>(a, l, k); break;
+      case SJHIP_SG_SOFT_SIGN: part = mp_backward_walk<ST, SP, GO, SJHIP_SG_SOFT_SIGN, PLIF>(a, l, k); break;
+      case SJHIP_SG_SUPER_SPIKE: part = mp_backward_walk<ST, SP, GO, SJHIP_SG_SUPER_SPIKE, PLIF>(a, l, k); break;
+      default: part = mp_backward_walk<ST, SP, GO, SJHIP_SG_ERF, PLIF>(a, l, k); break;
     }
   }
   if (PLIF) plif_block_reduce(a, part, k);
@@ -118,24 +119,34 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) mp_backward_kernel(const BwdA
 
 namespace {
 
-template <typename ST, bool PLIF>
+template <typename ST, typename GO, bool PLIF>
 int launch_bwd_storage(int spike_dtype, const BwdArgs &a, dim3 grid, dim3 threads, hipStream_t stream) {
   // measured at T = 16, N = 33.5 M (blocks of 128): 6 resident blocks per compute unit 0.810 ms, uncapped 0.845, 1-3 1.30
   const unsigned lds = occupancy_cap_lds(6);
   switch (spike_dtype) {
-    case SJHIP_F32: hipLaunchKernelGGL((mp_backward_kernel<ST, float, PLIF>), grid, threads, lds, stream, a); break;
-    case SJHIP_F16: hipLaunchKernelGGL((mp_backward_kernel<ST, f16_t, PLIF>), grid, threads, lds, stream, a); break;
-    case SJHIP_BF16: hipLaunchKernelGGL((mp_backward_kernel<ST, bf16_t, PLIF>), grid, threads, lds, stream, a); break;
+    case SJHIP_F32: hipLaunchKernelGGL((mp_backward_kernel<ST, float, GO, PLIF>), grid, threads, lds, stream, a); break;
+    case SJHIP_F16: hipLaunchKernelGGL((mp_backward_kernel<ST, f16_t, GO, PLIF>), grid, threads, lds, stream, a); break;
+    case SJHIP_BF16: hipLaunchKernelGGL((mp_backward_kernel<ST, bf16_t, GO, PLIF>), grid, threads, lds, stream, a); break;
     default: return fail(SJHIP_ERR_INVALID, "backward(mp): spike dtype %d", spike_dtype);
   }
   return check_launch("backward(mp)");
+}
+
+template <typename ST>
+int launch_bwd_outputs(int spike_dtype, bool plif, bool grads_in_storage, const BwdArgs &a, dim3 grid, dim3 threads,
+                       hipStream_t stream) {
+  if (grads_in_storage)
+    return plif ? launch_bwd_storage<ST, ST, true>(spike_dtype, a, grid, threads, stream)
+                : launch_bwd_storage<ST, ST, false>(spike_dtype, a, grid, threads, stream);
+  return plif ? launch_bwd_storage<ST, float, true>(spike_dtype, a, grid, threads, stream)
+              : launch_bwd_storage<ST, float, false>(spike_dtype, a, grid, threads, stream);
 }
 
 }  // namespace
 
 int launch_backward_mp(int neuron, int storage_dtype, int spike_dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
                        const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last, const void *h_seq,
-                       const void *v_init, const float *k_device, float *grad_x_seq, float *grad_v_init,
+                       const void *v_init, const float *k_device, void *grad_x_seq, void *grad_v_init,
                        float *grad_rtau, float *workspace, hipStream_t stream) {
   if (N % 4 != 0) return fail(SJHIP_ERR_UNSUPPORTED, "backward(mp): N=%lld must be a multiple of 4", (long long)N);
   BwdArgs a;
@@ -152,12 +163,11 @@ int launch_backward_mp(int neuron, int storage_dtype, int spike_dtype, const sjh
   const dim3 grid((unsigned)blocks), threads(block);
   {
     ProfileScope prof(KC_BACKWARD, stream);
+    const bool grads_in_storage = (p.flags & SJHIP_FLAG_GRAD_STORAGE) != 0;
     if (storage_dtype == SJHIP_F8E4M3)
-      rc = plif ? launch_bwd_storage<f8e4m3_t, true>(spike_dtype, a, grid, threads, stream)
-                : launch_bwd_storage<f8e4m3_t, false>(spike_dtype, a, grid, threads, stream);
+      rc = launch_bwd_outputs<f8e4m3_t>(spike_dtype, plif, grads_in_storage, a, grid, threads, stream);
     else if (storage_dtype == SJHIP_F8E5M2)
-      rc = plif ? launch_bwd_storage<f8e5m2_t, true>(spike_dtype, a, grid, threads, stream)
-                : launch_bwd_storage<f8e5m2_t, false>(spike_dtype, a, grid, threads, stream);
+      rc = launch_bwd_outputs<f8e5m2_t>(spike_dtype, plif, grads_in_storage, a, grid, threads, stream);
     else
       return fail(SJHIP_ERR_INVALID, "backward(mp): storage dtype %d is not an 8-bit float", storage_dtype);
     if (rc != SJHIP_OK) return rc;

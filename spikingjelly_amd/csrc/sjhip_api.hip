@@ -236,8 +236,8 @@ int sjhip_neuron_forward_mp(int neuron, int storage_dtype, int spike_dtype, cons
 
 int sjhip_neuron_backward_mp(int neuron, int storage_dtype, int spike_dtype, const sjhip_neuron_params *p, int64_t T,
                              int64_t N, const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
-                             const void *h_seq, const void *v_init, const float *rtau_device, float *grad_x_seq,
-                             float *grad_v_init, float *grad_rtau, float *workspace, void *stream) {
+                             const void *h_seq, const void *v_init, const float *rtau_device, void *grad_x_seq,
+                             void *grad_v_init, float *grad_rtau, float *workspace, void *stream) {
   int rc = check_mp("backward(mp)", neuron, storage_dtype, spike_dtype, p, T, N);
   if (rc != SJHIP_OK) return rc;
   if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_ERF) return fail(SJHIP_ERR_UNSUPPORTED, "backward(mp): surrogate id %d", p->sg_id);

@@ -309,7 +309,7 @@ int launch_forward_mp(int neuron, int storage_dtype, int spike_dtype, const sjhi
                       void *v_last, void *h_seq, hipStream_t stream);
 int launch_backward_mp(int neuron, int storage_dtype, int spike_dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
                        const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last, const void *h_seq,
-                       const void *v_init, const float *k_device, float *grad_x_seq, float *grad_v_init,
+                       const void *v_init, const float *k_device, void *grad_x_seq, void *grad_v_init,
                        float *grad_rtau, float *workspace, hipStream_t stream);
 int launch_izhikevich_backward_replay(int dtype, const sjhip_izhikevich_params &p, int64_t T, int64_t N,
                                       const void *x_seq, const void *v_init, const void *w_init,

@@ -15,6 +15,7 @@ import torch
 from oracle import bptt_oracle as bo
 from oracle import neuron_oracle as no
 from spikingjelly_amd.activation_based import surrogate
+from spikingjelly_amd.activation_based.hip_kernel import library as L
 from spikingjelly_amd.activation_based.hip_kernel import neuron_mp_kernel as M
 
 from helpers import bits_equal, seeded_randn
@@ -228,6 +229,51 @@ def test_fp8_backward_equals_the_closed_form_on_the_stored_h(storage, kind, k, v
     np.testing.assert_allclose(v0.grad.cpu().double().numpy(), want_v0, rtol=2e-5, atol=2e-6)
     if kind == "plif":
         np.testing.assert_allclose(float(kt.grad), want_k, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("storage", F8)
+@pytest.mark.parametrize("neuron_id,k", [(0, None), (1, None), (2, 0.5744425)])
+@pytest.mark.parametrize("N", [512, 520, 37])
+def test_fp8_gradients_written_in_the_storage_dtype_are_the_rounded_fp32_ones(storage, neuron_id, k, N):
+    """What the reference does (it allocates grad_x_seq / grad_v_init in the dtypes of x_seq / v_init,
+    triton_kernel/neuron_kernel/lif.py:1115-1118): the kernel rounds its fp32 value once, so the result is the cast of
+    the fp32 result, at 5 instead of 8 bytes per neuron-step."""
+    T = 6
+    h = seeded_randn((T, N), 61, 0.6, 0.7).cuda().to(storage)
+    v0 = seeded_randn((N,), 62, 0.0, 0.3).cuda().to(storage)
+    gs = seeded_randn((T, N), 63).cuda().to(torch.bfloat16)
+    gv = seeded_randn((T, N), 64, 0.0, 0.2).cuda().to(storage)
+    kt = None if k is None else torch.tensor(k, device="cuda")
+    neuron = (L.NEURON_IF, L.NEURON_LIF, L.NEURON_PLIF)[neuron_id]
+    scalars = (neuron, 2.0, True, 1.0, 0.0, False, False, 1, 2.0)
+    wide = M.hip_multistep_mp_backward(gs, gv, h, v0, kt, *scalars, torch.bfloat16, False)
+    narrow = M.hip_multistep_mp_backward(gs, gv, h, v0, kt, *scalars, torch.bfloat16, True)
+    assert wide[0].dtype == torch.float32 and narrow[0].dtype == storage and narrow[1].dtype == storage
+    assert narrow[0].shape == (T, N) and narrow[1].shape == (N,)
+    assert _same_stored(narrow[0], wide[0].to(storage)) and _same_stored(narrow[1], wide[1].to(storage))
+    assert bits_equal(narrow[2], wide[2]) and float(wide[0].abs().sum()) > 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("storage", F8)
+def test_fp8_inputs_get_fp8_gradients_through_autograd(storage):
+    T, N = 5, 256
+    x32 = seeded_randn((T, N), 71, 0.4, 0.7).cuda()
+    v32 = seeded_randn((N,), 72, 0.0, 0.3).cuda()
+    gs = seeded_randn((T, N), 73).cuda()
+    kw = dict(decay_input=True, tau=2.0, v_threshold=1.0, v_reset=0.0, storage_dtype=storage, spike_dtype=torch.float32,
+              surrogate_function=surrogate.ATan(2.0))
+    x8, v8 = x32.to(storage).requires_grad_(), v32.to(storage).requires_grad_()
+    s8, _, _ = M.multistep_lif_mp(x8, v8, **kw)
+    s8.backward(gs)
+    # the same values fed as fp32 tensors take the fp32 route; its gradients, cast, are the fp8 route's
+    xw, vw = x8.detach().float().requires_grad_(), v8.detach().float().requires_grad_()
+    sw, _, _ = M.multistep_lif_mp(xw, vw, **kw)
+    sw.backward(gs)
+    assert bits_equal(s8.detach(), sw.detach())
+    assert x8.grad.dtype == storage and v8.grad.dtype == storage
+    assert _same_stored(x8.grad, xw.grad.to(storage)) and _same_stored(v8.grad, vw.grad.to(storage))
 
 
 @pytest.mark.gpu
