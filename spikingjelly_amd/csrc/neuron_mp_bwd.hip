@@ -121,8 +121,10 @@ namespace {
 
 template <typename ST, typename GO, bool PLIF>
 int launch_bwd_storage(int spike_dtype, const BwdArgs &a, dim3 grid, dim3 threads, hipStream_t stream) {
-  // measured at T = 16, N = 33.5 M (blocks of 128): 6 resident blocks per compute unit 0.810 ms, uncapped 0.845, 1-3 1.30
-  const unsigned lds = occupancy_cap_lds(6);
+  // resident blocks per compute unit, measured at T = 16, N = 33.5 M (blocks of 128).  fp32 gradients: 6 blocks 0.810 ms,
+  // no cap 0.845, 1-3 1.30; 8-bit gradients (less to write, closer to the arithmetic): 4 blocks 0.722, 6 0.631, 8 0.585,
+  // no cap 0.583
+  const unsigned lds = occupancy_cap_lds(sizeof(GO) == 4 ? 6 : 0);
   switch (spike_dtype) {
     case SJHIP_F32: hipLaunchKernelGGL((mp_backward_kernel<ST, float, GO, PLIF>), grid, threads, lds, stream, a); break;
     case SJHIP_F16: hipLaunchKernelGGL((mp_backward_kernel<ST, f16_t, GO, PLIF>), grid, threads, lds, stream, a); break;
