@@ -151,8 +151,28 @@ def prepare_hip_neuron_execution_plan(*, neuron_type: str, device, storage_dtype
                                   "or in a 16-bit storage dtype itself")
     if backward_name != "fp32":
         raise NotImplementedError(f"backward_compute_dtype={backward_name!r}: the hip backward computes in fp32")
+    if is_fp8_dtype(storage):
+        _check_fp8_capability(storage, device, neuron_type, save_intermediates)
     return HipNeuronExecutionPlan(neuron_type, device, storage, forward_name, backward_name, spike_dtype,
                                   save_intermediates, round_every_op)
+
+
+def _check_fp8_capability(storage: torch.dtype, device: torch.device, neuron_type: str, with_backward: bool) -> None:
+    """The reference's check at plan preparation (``triton_kernel/neuron_kernel/utils.py:99-152``): a forward (and, when
+    intermediates are kept for it, a backward) that the device cannot run is refused here, with the probe's reason.
+    The probes run once per dtype and device; nothing is probed while a HIP graph is being recorded."""
+    from . import fp8_capability as C
+
+    if C.probing() or not torch.cuda.is_available() or torch.cuda.is_current_stream_capturing():
+        return  # (without a device there is nothing to ask; the operators refuse CPU tensors themselves)
+    asks = [("forward", "compute_dtype", C.hip_fp8_neuron_capability)]
+    if with_backward:
+        asks.append(("backward", "backward_compute_dtype", C.hip_fp8_neuron_backward_capability))
+    for pass_name, kw, ask in asks:
+        answer = ask(storage, device, "fp32")
+        if not answer.get("available", False):
+            raise RuntimeError(f"hip FP8 {neuron_type.upper()} {pass_name} is unavailable for {storage} with "
+                               f"{kw}='fp32': {answer.get('reason', 'unknown reason')}")
 
 
 # ---- 8-bit storage: operators over the dedicated kernels -----------------------------------------------------------------
