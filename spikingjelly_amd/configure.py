@@ -35,3 +35,8 @@ hip_plif_atomic_reduce = False
 # of ``hip_kernel/spike_op.py`` keep their binary input for the backward.  0: as ``torch.bool`` (one byte per spike);
 # 1: bit-packed, eight spikes per byte (``hip_kernel/tensor_cache.float_spike_to_bool``).
 save_bool_spike_level = 0
+
+# ``save_spike_as_bool_in_neuron_kernel`` (the reference's ``configure.py:54``: its QIF / EIF / Izhikevich CuPy kernels
+# may keep the forward's spikes as bools for the backward, ``qif.py:437,471``).  Kept for callers that set it; the hip
+# backward keeps no spikes at all (it recomputes them from ``h``), so the value changes nothing here.
+save_spike_as_bool_in_neuron_kernel = False
