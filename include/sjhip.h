@@ -200,6 +200,28 @@ int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p,
                           void *stream);
 
 /*
+ * sjhip_neuron_backward with the PLIF workspace inside the library: for callers that cannot allocate device memory
+ * (code under HIP graph capture, serving loops and harnesses that forbid hipMalloc).  No counterpart in the reference,
+ * whose operators allocate their outputs and partial sums through torch / CuPy on every call.  Same arguments and
+ * results as sjhip_neuron_backward minus `workspace`: the per-block partial sums of dL/dk go to a 4 MiB array that is
+ * part of the library's code object (one copy per GPU, held until the process ends), so the call reaches no
+ * hipMalloc / hipFree.  PLIF without SJHIP_FLAG_ATOMIC_REDUCE accepts N <= SJHIP_STATIC_WORKSPACE_MAX_NEURONS and
+ * returns SJHIP_ERR_TOO_LARGE beyond; other neurons use no workspace and are passed through.  The stream's device must
+ * be the current device.  Every call on one GPU shares that GPU's array: calls that overlap there (two streams, two
+ * threads) race on the partial sums; calls on one stream are ordered and need no clearing in between (each launch
+ * writes every partial it later sums).
+ */
+#define SJHIP_STATIC_WORKSPACE_MAX_NEURONS (INT64_C(1) << 26)
+int sjhip_neuron_backward_static(int neuron, int dtype, const sjhip_neuron_params *p,
+                                 int64_t T, int64_t N,
+                                 const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                                 const void *h_seq,
+                                 const void *v_init, const float *rtau_device,
+                                 void *grad_x_seq, void *grad_v_init,
+                                 float *grad_rtau,
+                                 void *stream);
+
+/*
  * Backward that needs no h_seq: it replays the forward from x_seq and v_init (bit-identical h, kept
  * in LDS) and then runs the same BPTT.  A forward whose backward will use this entry point can be
  * called with h_seq = NULL, which saves its largest write.  Same argument meaning as

@@ -32,6 +32,7 @@ FLAG_Q_BROADCAST = 0x200
 FLAG_ACC_BROADCAST = 0x400
 FLAG_W_INIT_BROADCAST = 0x800
 FLAG_GRAD_STORAGE = 0x1000
+STATIC_WORKSPACE_MAX_NEURONS = 1 << 26
 
 KC_FORWARD, KC_BACKWARD, KC_PLIF_REDUCE, KC_BIT_PACK, KC_BIT_UNPACK, KC_SSA_FORWARD, KC_SSA_BACKWARD = range(7)
 
@@ -44,6 +45,7 @@ EXPORTED_SYMBOLS = (
     "sjhip_neuron_forward_mp",
     "sjhip_neuron_backward_mp",
     "sjhip_neuron_backward",
+    "sjhip_neuron_backward_static",
     "sjhip_neuron_backward_recompute",
     "sjhip_recompute_supported",
     "sjhip_recompute_preferred",
@@ -140,6 +142,12 @@ def load() -> ctypes.CDLL:
             c_int, c_int, POINTER(NeuronParams), c_int64, c_int64,
             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        ]
+        lib.sjhip_neuron_backward_static.restype = c_int
+        lib.sjhip_neuron_backward_static.argtypes = [
+            c_int, c_int, POINTER(NeuronParams), c_int64, c_int64,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+            c_void_p, c_void_p, c_void_p, c_void_p,
         ]
         lib.sjhip_neuron_backward_recompute.restype = c_int
         lib.sjhip_neuron_backward_recompute.argtypes = [

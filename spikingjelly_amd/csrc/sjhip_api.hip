@@ -113,7 +113,37 @@ ProfileScope::~ProfileScope() {
 
 using namespace sjhip;
 
+// Workspace of sjhip_neuron_backward_static: the per-block partial sums of the PLIF dL/dk reduction, held in
+// the code object instead of in memory a caller allocated.  4 MiB on every GPU the library runs on, for as long as the
+// process lives.  In host code the array's name is only a handle for hipGetSymbolAddress; kernels get the address
+// that call returned.
+constexpr int64_t kStaticWorkspaceFloats = int64_t(1) << 20;
+static_assert(kStaticWorkspaceFloats * 64 == SJHIP_STATIC_WORKSPACE_MAX_NEURONS, "plif_blocks() counts one partial per 64 neurons at most");
+static __device__ __align__(256) float scratch[kStaticWorkspaceFloats];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float *g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// Device address of `scratch` on the current device, looked up once per device.
+int static_workspace(const char *what, float **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(SJHIP_ERR_LAUNCH, "%s: hipGetDevice: %s", what, hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(SJHIP_ERR_UNSUPPORTED, "%s: device ordinal %d", what, dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    float *ptr = nullptr;
+    e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return fail(SJHIP_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch) on device %d: %s", what, dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return SJHIP_OK;
+}
 
 bool valid_dtype_fp(int dtype) { return dtype == SJHIP_F32 || dtype == SJHIP_F16 || dtype == SJHIP_BF16; }
 
@@ -208,6 +238,24 @@ int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p, i
   }
   return launch_backward(neuron, dtype, *p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, rtau_device, grad_x_seq,
                          grad_v_init, grad_rtau, workspace, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_neuron_backward_static(int neuron, int dtype, const sjhip_neuron_params *p, int64_t T, int64_t N,
+                                 const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                                 const void *h_seq, const void *v_init, const float *rtau_device, void *grad_x_seq,
+                                 void *grad_v_init, float *grad_rtau, void *stream) {
+  float *workspace = nullptr;
+  const bool needs_workspace = p && neuron == SJHIP_NEURON_PLIF && !(p->flags & SJHIP_FLAG_ATOMIC_REDUCE);
+  if (needs_workspace) {
+    if (N >= 1 && plif_blocks(dtype, N) > kStaticWorkspaceFloats)
+      return fail(SJHIP_ERR_TOO_LARGE, "backward(static): N=%lld needs %lld partial sums, the built-in workspace holds %lld "
+                  "(N <= %lld); use sjhip_neuron_backward with a workspace of the caller's", (long long)N,
+                  (long long)plif_blocks(dtype, N), (long long)kStaticWorkspaceFloats, (long long)(kStaticWorkspaceFloats * 64));
+    int rc = static_workspace("backward(static)", &workspace);
+    if (rc != SJHIP_OK) return rc;
+  }
+  return sjhip_neuron_backward(neuron, dtype, p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, rtau_device,
+                               grad_x_seq, grad_v_init, grad_rtau, workspace, stream);
 }
 
 namespace {
