@@ -43,5 +43,19 @@ def max_rel_err(actual: torch.Tensor, expected: torch.Tensor, floor: float = 1e-
     return float(((a - e).abs() / e.abs().clamp_min(floor)).max())
 
 
+def require_device_memory(gib: int) -> None:
+    """Skip a full-size test on a small card; on an MI355X-class card (192 GiB or more in total) too little free
+    memory is a failure, so that a run there cannot silently drop the benchmark-shape tests."""
+    import pytest
+
+    free, total = torch.cuda.mem_get_info()
+    if free >= gib * (1 << 30):
+        return
+    message = f"needs {gib} GiB of free device memory, {free / (1 << 30):.1f} of {total / (1 << 30):.1f} GiB are free"
+    if total >= 192 * (1 << 30):
+        pytest.fail(message)
+    pytest.skip(message)
+
+
 def np_f32(t: torch.Tensor) -> np.ndarray:
     return t.detach().cpu().to(torch.float32).numpy()

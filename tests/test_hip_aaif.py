@@ -11,7 +11,7 @@ from oracle import neuron_oracle as no
 from spikingjelly_amd import configure
 from spikingjelly_amd.activation_based import functional, neuron
 
-from helpers import bits_equal, seeded_randn
+from helpers import bits_equal, require_device_memory, seeded_randn
 
 pytestmark = pytest.mark.gpu
 
@@ -105,9 +105,7 @@ def test_hip_backend_refuses_what_the_reference_kernel_backend_refuses():
 
 def test_full_size_inference():
     """[T=16, B=64, C=128, 32, 32] fp32 with per-channel parameters: column blocks against the oracle."""
-    free, _ = torch.cuda.mem_get_info()
-    if free < 8 * (1 << 30):
-        pytest.skip("needs 8 GiB of device memory")
+    require_device_memory(8)
     T, B, C, HW = 16, 64, 128, 1024
     g = torch.Generator(device="cuda").manual_seed(9)
     x = torch.randn((T, B, C, HW), generator=g, device="cuda") * 0.5 + 0.2

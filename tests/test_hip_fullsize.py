@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import seeded_randn
+from helpers import require_device_memory, seeded_randn
 
 pytestmark = pytest.mark.gpu
 
@@ -20,9 +20,7 @@ T, N = 16, 256 * 128 * 32 * 32
 def test_config2_full_size_forward_backward(c_oracle):
     from spikingjelly_amd.activation_based import neuron, surrogate
 
-    free, _ = torch.cuda.mem_get_info()
-    if free < 40 * (1 << 30):
-        pytest.skip("needs 40 GiB of device memory")
+    require_device_memory(40)
     g = torch.Generator(device="cuda").manual_seed(1002)
     x = (torch.randn((T, N), generator=g, device="cuda") * 0.8 + 0.3).requires_grad_()
     gs = torch.randn((T, N), generator=g, device="cuda")
@@ -188,9 +186,7 @@ def test_more_than_two_to_the_32_elements(c_oracle):
     the range, the last columns included, against the C oracle, for the forward and the replaying backward."""
     from spikingjelly_amd.activation_based import neuron, surrogate
 
-    free, _ = torch.cuda.mem_get_info()
-    if free < 100 * (1 << 30):
-        pytest.skip("needs 100 GiB of device memory")
+    require_device_memory(100)
     T_big, N_big = 16, (1 << 28) + 4096 * 3  # 4 295 163 904 elements per tensor, 17.2 GB in fp32
     g = torch.Generator(device="cuda").manual_seed(77)
     x = torch.empty((T_big, N_big), device="cuda")

@@ -35,12 +35,10 @@ PARAMS = [  # tau, v_th, levels, gradient window
 
 
 @pytest.mark.parametrize("tau,v_th,levels,window", PARAMS)
-@pytest.mark.parametrize("T,N", [(16, 4096), (7, 111), (33, 260), (1, 4)])
-@pytest.mark.parametrize("recompute", [False, True])
+@pytest.mark.parametrize("T,N,recompute", [(16, 4096, False), (16, 4096, True), (7, 111, False), (33, 260, False),
+                                           (33, 260, True), (1, 4, False), (1, 4, True)])  # replay: N % 4 == 0
 @pytest.mark.parametrize("detach", [False, True])
 def test_forward_bit_exact_and_gradients_fp32(K, tau, v_th, levels, window, T, N, recompute, detach):
-    if recompute and N % 4 != 0:
-        pytest.skip("the replay kernel needs N % 4 == 0; such shapes use the h_seq path")
     x = seeded_randn((T, N), 100 + T, 0.6 * v_th * levels / 2, v_th * levels / 2)
     v0 = seeded_randn((N,), 200 + N, 0.0, 0.3)
     gs, gv = seeded_randn((T, N), 300 + T), seeded_randn((T, N), 400 + T, 0.0, 0.1)

@@ -101,13 +101,11 @@ def _call(kind, x, v0, k, **kw):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("storage", F8)
-@pytest.mark.parametrize("kind,k", [("if", 0.0), ("lif", 0.5), ("lif", 0.25), ("plif", 0.5744425)])
+@pytest.mark.parametrize("kind,k,decay_input", [("if", 0.0, True), ("lif", 0.5, True), ("lif", 0.5, False), ("lif", 0.25, True),
+                                                ("lif", 0.25, False), ("plif", 0.5744425, True), ("plif", 0.5744425, False)])
 @pytest.mark.parametrize("v_reset", [0.0, -0.25, None])
-@pytest.mark.parametrize("decay_input", [True, False])
 @pytest.mark.parametrize("spike_dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_fp8_forward_equals_the_recipe(storage, kind, k, v_reset, decay_input, spike_dtype):
-    if kind == "if" and not decay_input:
-        pytest.skip("IF has no decay_input")
     T, N = 9, 1000  # not a multiple of 16: the operator pads
     x = seeded_randn((T, N), 41, 0.9, 1.0)
     v0 = seeded_randn((N,), 42, 0.0, 0.3)
@@ -187,13 +185,11 @@ SG = {"sigmoid": (surrogate.Sigmoid, 4.0), "atan": (surrogate.ATan, 2.0), "erf":
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("storage", F8)
-@pytest.mark.parametrize("kind,k", [("if", 0.0), ("lif", 0.5), ("plif", 0.5744425)])
+@pytest.mark.parametrize("kind,k,decay_input", [("if", 0.0, True), ("lif", 0.5, True), ("lif", 0.5, False),
+                                                ("plif", 0.5744425, True), ("plif", 0.5744425, False)])
 @pytest.mark.parametrize("v_reset,detach", [(0.0, False), (-0.25, True), (None, False)])
-@pytest.mark.parametrize("decay_input", [True, False])
 @pytest.mark.parametrize("sg_name,spike_dtype", [("sigmoid", torch.float32), ("atan", torch.bfloat16), ("erf", torch.float16)])
 def test_fp8_backward_equals_the_closed_form_on_the_stored_h(storage, kind, k, v_reset, detach, decay_input, sg_name, spike_dtype):
-    if kind == "if" and not decay_input:
-        pytest.skip("IF has no decay_input")
     T, N = 7, 520
     x = seeded_randn((T, N), 51, 0.4, 0.7).cuda().requires_grad_()
     v0 = seeded_randn((N,), 52, 0.0, 0.3).cuda().requires_grad_()

@@ -66,6 +66,28 @@ def test_hip_node_matches_torch_node(cls, kw, v_reset, detach_reset, sg):
         torch.testing.assert_close(b.w.grad.cpu(), a.w.grad, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("decay_input", [True, False])
+@pytest.mark.parametrize("v_reset", [0.0, -0.2, None])
+def test_reciprocal_tau_switch_matches_the_torch_backend_on_the_same_device(decay_input, v_reset, monkeypatch):
+    """tau = 3 is not a power of two.  torch divides a device tensor by a Python scalar as a multiplication by 1/tau,
+    which is also what the reference's CuPy / Triton kernels are handed (multi_step/lif.py:338); with
+    ``configure.hip_lif_reciprocal_tau = True`` the hip backend fires the same spikes as ``backend='torch'`` run on the
+    GPU, while the default (IEEE division) fires the spikes of ``backend='torch'`` run on the CPU."""
+    x = seeded_randn((8, 64, 257), 31, 0.4, 1.0)
+    kw = dict(tau=3.0, decay_input=decay_input, v_reset=v_reset, surrogate_function=surrogate.ATan(), step_mode="m")
+    on_gpu = neuron.LIFNode(backend="torch", store_v_seq=True, **kw).cuda()
+    s_gpu = on_gpu(x.cuda())
+    on_cpu = neuron.LIFNode(backend="torch", store_v_seq=True, **kw)
+    s_cpu = on_cpu(x)
+    for flag, s_ref, node_ref in ((True, s_gpu, on_gpu), (False, s_cpu, on_cpu)):
+        monkeypatch.setattr(configure, "hip_lif_reciprocal_tau", flag)
+        node = neuron.LIFNode(backend="hip", store_v_seq=True, **kw).cuda()
+        s = node(x.cuda())
+        assert bits_equal(s.cpu(), s_ref.cpu()), flag
+        assert bits_equal(node.v_seq.cpu(), node_ref.v_seq.cpu()), flag
+    assert not bits_equal(on_gpu.v_seq.cpu(), on_cpu.v_seq)  # the two torch runs really differ on this input
+
+
 @pytest.mark.parametrize("cls", [neuron.IFNode, neuron.LIFNode, neuron.ParametricLIFNode])
 @pytest.mark.parametrize("T,N", [(1, 48), (7, 111), (65, 64)])
 def test_store_v_seq_toggle_is_equivalent(cls, T, N):

@@ -169,12 +169,9 @@ def test_forward_half_rounds_like_torch_backend(K, dtype, kind, v_reset, decay_i
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("kind", ["if", "lif", "plif"])
+@pytest.mark.parametrize("kind,decay_input", [("if", True), ("lif", True), ("lif", False), ("plif", True), ("plif", False)])
 @pytest.mark.parametrize("v_reset", [0.0, -0.2, None])
-@pytest.mark.parametrize("decay_input", [True, False])
 def test_forward_half_storage_fp32_state(K, dtype, kind, v_reset, decay_input):
-    if kind == "if" and not decay_input:
-        pytest.skip("IF has no decay_input")
     T, N, k = 8, 4096, 0.5
     x = seeded_randn((T, N), 500, 0.3, 1.0).to(dtype)
     v0 = seeded_randn((N,), 501, 0.0, 0.3).to(dtype)
@@ -218,11 +215,8 @@ BWD_GRID = [(kind, sg, di, vr, det)
 
 
 @pytest.mark.parametrize("kind,sg,decay_input,v_reset,detach", BWD_GRID)
-@pytest.mark.parametrize("T,N", [(16, 4096), (7, 111)])
-@pytest.mark.parametrize("path", ["h_seq", "replay"])
+@pytest.mark.parametrize("T,N,path", [(16, 4096, "h_seq"), (16, 4096, "replay"), (7, 111, "h_seq")])  # replay: N % 4 == 0
 def test_backward_matches_autograd_fp32(K, kind, sg, decay_input, v_reset, detach, T, N, path):
-    if path == "replay" and N % 4 != 0:
-        pytest.skip("the replay kernel needs N % 4 == 0; such shapes use the h_seq path")
     tau, vth = 3.0, 0.8
     alpha = no.SG_DEFAULT_ALPHA[sg]
     x = seeded_randn((T, N), 600 + T, 0.4, 1.0)
@@ -341,14 +335,11 @@ def test_plif_reduction_is_deterministic_and_accurate(K, path):
 # ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("kind", ["if", "lif", "plif"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("recompute", [False, True])
-@pytest.mark.parametrize("T,N", [(5, 64), (3, 37)])
+@pytest.mark.parametrize("recompute,T,N", [(False, 5, 64), (True, 5, 64), (False, 3, 37)])  # replay: N % 8 == 0
 def test_broadcast_initial_state_equals_a_filled_tensor(K, kind, dtype, recompute, T, N):
     """An expanded one-element v_init (what a node passes while its state is the scalar reset value) must
     give bit-identical outputs and gradients to the same value filled into an [N] tensor, on the 128-bit and
     on the element-wise kernels, with h_seq saved or replayed."""
-    if recompute and N % 8 != 0:
-        pytest.skip("the replay kernel needs N % 4 (fp32) / N % 8 (16-bit) == 0; such shapes use the h_seq path")
     x = seeded_randn((T, N), 41, 0.4, 1.0).to(dtype).cuda()
     gs = seeded_randn((T, N), 42).to(dtype).cuda()
     full = torch.full((N,), -0.25, dtype=dtype, device="cuda")

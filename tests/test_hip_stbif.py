@@ -12,7 +12,7 @@ from oracle import stbif_oracle
 from spikingjelly_amd import configure
 from spikingjelly_amd.activation_based import functional, neuron
 
-from helpers import bits_equal, seeded_randn
+from helpers import bits_equal, require_device_memory, seeded_randn
 
 pytestmark = pytest.mark.gpu
 
@@ -134,9 +134,7 @@ def test_hip_node_matches_torch_node_and_the_quantiser(sym):
 def test_full_size_against_the_quantiser():
     """T = 16 over 33.5 M neurons: the released total of every neuron equals the quantiser of its input, and column
     blocks equal the torch step bit for bit."""
-    free, _ = torch.cuda.mem_get_info()
-    if free < 12 * (1 << 30):
-        pytest.skip("needs 12 GiB of device memory")
+    require_device_memory(12)
     T, N, scale = 16, 256 * 128 * 32 * 32, 0.25
     g = torch.Generator(device="cuda").manual_seed(3)
     x = torch.zeros((T, N), device="cuda")

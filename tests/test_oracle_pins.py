@@ -177,6 +177,36 @@ def test_surrogate_gradient_values_at_zero():
     assert no.surrogate_grad("erf", z, 2.0).item() == pytest.approx(2.0 / math.sqrt(math.pi))
 
 
+def test_super_spike_gradient_away_from_zero():
+    """alpha / (|x| + 1)^2 (surrogate.py:1101-1102; the reference defines no primitive to difference, :1236-1237):
+    hand-computed values, exact in binary floating point."""
+    x = torch.tensor([1.0, -3.0, 0.5, -0.25], dtype=torch.float64)
+    want = torch.tensor([2.0 / 4.0, 2.0 / 16.0, 2.0 / 2.25, 2.0 / 1.5625], dtype=torch.float64)
+    assert torch.equal(no.surrogate_grad("super_spike", x, 2.0), want)
+    xs = x.clone().requires_grad_()
+    g = torch.tensor([1.0, -2.0, 0.5, 4.0], dtype=torch.float64)
+    no.surrogate("super_spike", 2.0)(xs).backward(g)
+    assert torch.equal(xs.grad, want * g)
+
+
+def test_reciprocal_tau_form_is_a_multiplication_by_the_rounded_reciprocal():
+    """What the reference's kernel backends and torch on a GPU compute for the LIF charge (multi_step/lif.py:338 passes
+    `reciprocal_tau`; a division of a device tensor by a Python scalar runs as a multiplication by 1/b): the oracle's
+    "plif_k" charge fed k = fl32(1/tau).  Pinned against numpy float32 arithmetic written out op by op, and shown to
+    differ from the IEEE division of the CPU backend for tau = 3."""
+    x = seeded_randn((4096,), 77, 0.3, 1.0)
+    v = seeded_randn((4096,), 78, 0.1, 0.5)
+    k32 = np.float32(1.0) / np.float32(3.0)
+    xn, vn, vr = x.numpy(), v.numpy(), np.float32(-0.2)
+    for decay_input in (True, False):
+        want = vn + (xn - (vn - vr)) * k32 if decay_input else vn - (vn - vr) * k32 + xn
+        got = no.charge("plif_k", x, v, torch.tensor(float(k32)), decay_input, -0.2)
+        assert want.dtype == np.float32 and np.array_equal(got.numpy(), want)
+        assert not torch.equal(got, no.charge("lif", x, v, 3.0, decay_input, -0.2))
+    # tau a power of two: both forms agree bit for bit
+    assert torch.equal(no.charge("plif_k", x, v, torch.tensor(0.25), True, -0.2), no.charge("lif", x, v, 4.0, True, -0.2))
+
+
 # ------------------------------------------------------------------------------------------------
 # 4. BPTT: closed-form recurrence == autograd of the restated ops == finite differences
 # ------------------------------------------------------------------------------------------------
@@ -216,14 +246,11 @@ def test_recurrence_equals_autograd_float64(kind, sg, decay_input, v_reset, deta
         assert gk * k * (1 - k) == pytest.approx(float(ref["grad_p"]), rel=1e-10)
 
 
-@pytest.mark.parametrize("kind", ["if", "lif", "plif"])
+@pytest.mark.parametrize("kind,decay_input", [("if", True), ("lif", True), ("lif", False), ("plif", True), ("plif", False)])
 @pytest.mark.parametrize("v_reset", [0.0, -0.2, None])
-@pytest.mark.parametrize("decay_input", [True, False])
 def test_recurrence_matches_finite_differences_of_the_smooth_network(kind, v_reset, decay_input):
     """With the primitive (non-spiking) surrogate the network is smooth, autograd is its true
     gradient and the recurrence (s_t = primitive, sg = primitive') must match central differences."""
-    if kind == "if" and not decay_input:
-        pytest.skip("IF has no decay_input")
     T, N, tau, vth, alpha = 5, 7, 2.5, 0.6, 2.0
     x = seeded_randn((T, N), 31, 0.4, 0.8, torch.float64)
     v0 = seeded_randn((N,), 32, 0.0, 0.3, torch.float64)
@@ -290,13 +317,10 @@ def test_c_backward_equals_recurrence(c_oracle):
 # ------------------------------------------------------------------------------------------------
 # 5. torch oracle == C oracle bit for bit (two independent implementations of IEEE fp32)
 # ------------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("kind", ["if", "lif", "plif"])
+@pytest.mark.parametrize("kind,decay_input,tau", [("if", True, 2.0)] + [(kind, di, tau) for kind in ("lif", "plif")
+                                                  for di in (True, False) for tau in (2.0, 3.0, 10.0)])
 @pytest.mark.parametrize("v_reset", [0.0, -0.2, None])
-@pytest.mark.parametrize("decay_input", [True, False])
-@pytest.mark.parametrize("tau", [2.0, 3.0, 10.0])
 def test_torch_and_c_oracle_agree_bitwise(kind, v_reset, decay_input, tau, c_oracle):
-    if kind == "if" and (not decay_input or tau != 2.0):
-        pytest.skip("IF has neither tau nor decay_input")
     T, N = 16, 4099
     x = seeded_randn((T, N), 51, 0.3, 0.8)
     v0 = seeded_randn((N,), 52, 0.0, 0.2)
