@@ -146,8 +146,9 @@ const char *sjhip_last_error(void);
  *   v_last    [N] out, membrane potential after the last step; NULL = do not write
  *             (at least one of v_seq / v_last must be given)
  *   h_seq     [T,N] out, membrane potential before reset, saved for backward; NULL = do not write
- *   rtau_device  PLIF only, may be NULL: device address of one fp32 holding k = sigmoid(w); read by the
- *             kernel in place of p->tau so that no host synchronisation is needed to fetch it
+ *   rtau_device  PLIF only (required there, SJHIP_ERR_INVALID without it; NULL for the other neurons): device
+ *             address of one fp32 holding k = sigmoid(w), read by the kernel in place of p->tau so that no host
+ *             synchronisation is needed to fetch it
  * T >= 1, N >= 1, T*N < 2^62.  128-bit accesses are used when N is a multiple of 16/sizeof(dtype)
  * and every pointer is 16-byte aligned; otherwise an element-wise kernel runs.
  */
@@ -373,9 +374,12 @@ int sjhip_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, void *
  *   qkv      [samples, 3, heads, channels_per_head, tokens] in: binary spikes, q / k / v stacked on dim 1
  *   out      [samples, heads, channels_per_head, tokens] out = scale * (V K^T) Q, exact (integer sums in fp32)
  *   grad_out same shape as out, in;  grad_qkv same shape as qkv, out (dq, dk, dv)
- * bf16 MFMA with fp32 accumulation for the two spike products, fp32 MFMA for the backward products with
- * real-valued operands.  One wavefront per (sample, head); needs sjhip_ssa_supported(): at most 64 channels
- * per head, at most 256 tokens (V K^T must stay exact in bf16) and the tiles of one head fitting in LDS.
+ * One block of four wavefronts per (sample, head), the spikes of its three tiles parked in LDS as bytes.  Forward:
+ * V K^T on the int8 MFMA (exact integers), then (V K^T) Q on the bf16 MFMA with fp32 accumulation (V K^T <= 256 and
+ * the spikes are exact in bf16), so out equals an integer matmul times scale bit for bit.  Backward: dS = scale dO Q^T
+ * on the fp32 MFMA; dQ, dK, dV on the bf16 MFMA with the real-valued operand split into three bf16 terms that sum to
+ * it exactly.  Needs sjhip_ssa_supported(): at most 64 channels per head, at most 256 tokens (V K^T must stay exact
+ * in bf16) and the tiles of one head fitting in LDS.
  */
 int sjhip_ssa_supported(int dtype, int channels_per_head, int64_t tokens);
 int sjhip_ssa_forward(int dtype, int64_t samples, int heads, int channels_per_head, int64_t tokens, float scale,

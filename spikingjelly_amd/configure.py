@@ -10,9 +10,14 @@ for its CuPy/Triton backends).
     rounds only what is stored (the reference's mixed-precision Triton ops).
 
 ``hip_lif_reciprocal_tau``
-    ``False``: LIF charges with an IEEE division by ``tau`` like the torch CPU
-    backend.  ``True``: multiply by ``fl(1/tau)`` like the reference's CuPy/Triton
-    kernels (identical results when ``tau`` is a power of two).
+    ``False`` (default): LIF charges with an IEEE division by ``tau``: the spikes of
+    ``backend='torch'`` run on the CPU, which is what the parity tests compare with.
+    ``True``: multiply by ``fl(1/tau)``: the spikes of the reference's CuPy / Triton
+    kernels and of ``backend='torch'`` run on a GPU (torch divides a device tensor by
+    a Python scalar as a multiplication by its reciprocal).  Identical when ``tau`` is
+    a power of two; for other values (3.0, 5.0, ...) about a third of the fp32 charges
+    differ in the last bit and a few spikes with them, so pick the one whose results
+    you are reproducing.
 
 ``hip_plif_atomic_reduce``
     ``False``: the PLIF ``dL/dk`` sum is reduced in a fixed order (bitwise
@@ -22,8 +27,9 @@ for its CuPy/Triton backends).
     ``True``: training forwards write no ``h_seq``; the backward kernel replays the forward from
     ``x_seq`` and ``v_init`` (bit-identical ``h``, held in LDS), so autograd keeps ``x_seq`` alive
     instead of a same-sized ``h_seq`` and the forward's largest write disappears.  Used whenever the
-    shape allows (``N`` a multiple of the 128-bit vector width, ``T`` up to 159 for fp32 / 79 for
-    16-bit storage); other shapes and ``False`` fall back to saving ``h_seq``.
+    library prefers it for the shape (``sjhip_recompute_preferred``: ``N`` a multiple of the 128-bit
+    vector width and the sequence short enough for the replayed ``h`` to stay in LDS with enough
+    resident wavefronts); other shapes and ``False`` fall back to saving ``h_seq``.
 """
 
 hip_half_precision_mode = "torch"

@@ -192,6 +192,7 @@ int sjhip_neuron_forward(int neuron, int dtype, const sjhip_neuron_params *p, in
   if (!v_seq && !v_last) return fail(SJHIP_ERR_INVALID, "forward: neither v_seq nor v_last given");
   rc = check_levels("forward", neuron, *p, false);
   if (rc != SJHIP_OK) return rc;
+  if (neuron == SJHIP_NEURON_PLIF && !rtau_device) return fail(SJHIP_ERR_INVALID, "forward: PLIF needs rtau_device");
   return launch_forward(neuron, dtype, *p, T, N, x_seq, v_init, rtau_device, spike_seq, v_seq, v_last, h_seq,
                         static_cast<hipStream_t>(stream));
 }
@@ -207,6 +208,7 @@ int sjhip_neuron_forward_packed(int neuron, int dtype, const sjhip_neuron_params
   if (!x_seq || !v_init || !spike_bits) return fail(SJHIP_ERR_INVALID, "forward_packed: NULL tensor");
   if (!v_seq && !v_last) return fail(SJHIP_ERR_INVALID, "forward_packed: neither v_seq nor v_last given");
   if (neuron == SJHIP_NEURON_ILIF) return fail(SJHIP_ERR_UNSUPPORTED, "forward_packed: ILIF fires counts, not bits");
+  if (neuron == SJHIP_NEURON_PLIF && !rtau_device) return fail(SJHIP_ERR_INVALID, "forward_packed: PLIF needs rtau_device");
   return launch_forward_packed(neuron, dtype, *p, T, N, x_seq, v_init, rtau_device, spike_bits, v_seq, v_last,
                                static_cast<hipStream_t>(stream));
 }
@@ -233,7 +235,7 @@ int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p, i
   if ((neuron == SJHIP_NEURON_QIF || neuron == SJHIP_NEURON_EIF) && grad_v_init && !v_init)
     return fail(SJHIP_ERR_INVALID, "backward: QIF / EIF need v_init for grad_v_init");
   if (neuron == SJHIP_NEURON_PLIF) {
-    if (!v_init || !grad_rtau) return fail(SJHIP_ERR_INVALID, "backward: PLIF needs v_init and grad_rtau");
+    if (!v_init || !grad_rtau || !rtau_device) return fail(SJHIP_ERR_INVALID, "backward: PLIF needs v_init, rtau_device and grad_rtau");
     if (!(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace) return fail(SJHIP_ERR_INVALID, "backward: PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");
   }
   return launch_backward(neuron, dtype, *p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, rtau_device, grad_x_seq,
@@ -325,7 +327,7 @@ int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_pa
   rc = check_levels("backward(recompute)", neuron, *p, true);
   if (rc != SJHIP_OK) return rc;
   if (neuron == SJHIP_NEURON_PLIF) {
-    if (!grad_rtau) return fail(SJHIP_ERR_INVALID, "backward(recompute): PLIF needs grad_rtau");
+    if (!grad_rtau || !rtau_device) return fail(SJHIP_ERR_INVALID, "backward(recompute): PLIF needs rtau_device and grad_rtau");
     if (!(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace) return fail(SJHIP_ERR_INVALID, "backward(recompute): PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");
   }
   return launch_backward_recompute(neuron, dtype, *p, T, N, x_seq, v_init, rtau_device, grad_spike_seq, grad_v_seq,

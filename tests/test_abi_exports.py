@@ -51,6 +51,20 @@ def test_argument_validation_without_a_device():
     rc = lib.sjhip_neuron_backward(L.NEURON_PLIF, L.DTYPE_F32, ctypes.byref(p), 4, 16, 1, None, None, 1, None, None,
                                    1, 1, None, None, None)
     assert rc == -1 and b"PLIF" in lib.sjhip_last_error()
+    # PLIF reads k = sigmoid(w) from device memory: every entry point refuses a call without its address
+    rc = lib.sjhip_neuron_forward(L.NEURON_PLIF, L.DTYPE_F32, ctypes.byref(p), 4, 16, 16, 16, None, 16, 16, 16, None, None)
+    assert rc == -1 and b"rtau_device" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_forward_packed(L.NEURON_PLIF, L.DTYPE_F32, ctypes.byref(p), 4, 16, 16, 16, None, 16, None, 16, None)
+    assert rc == -1 and b"rtau_device" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_backward(L.NEURON_PLIF, L.DTYPE_F32, ctypes.byref(p), 4, 16, 16, None, None, 16, 16, None,
+                                   16, 16, 16, 16, None)
+    assert rc == -1 and b"rtau_device" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_backward_recompute(L.NEURON_PLIF, L.DTYPE_F32, ctypes.byref(p), 4, 16, 16, 16, None,
+                                             16, None, None, 16, 16, 16, 16, None)
+    assert rc == -1 and b"rtau_device" in lib.sjhip_last_error()
+    rc = lib.sjhip_neuron_backward_static(L.NEURON_PLIF, L.DTYPE_F32, ctypes.byref(p), 4, 16, 16, None, None, 16, 16, None,
+                                          16, 16, 16, None)
+    assert rc == -1 and b"rtau_device" in lib.sjhip_last_error()
     # ILIF: the count limit, the threshold, the surrogate and the window are checked before anything is launched
     def ilif(levels, sg=L.SG_MULTI_LEVEL, v_th=1.0, lo=0.0, hi=4.0):
         return L.NeuronParams(2.0, v_th, 0.0, 0.0, sg, 0, 0.0, 0.0, 0.0, levels, lo, hi)
