@@ -218,11 +218,11 @@ int64_t sjhip_plif_workspace_floats(int dtype, int64_t N) {
   return plif_blocks(dtype, N);
 }
 
-int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p, int64_t T, int64_t N,
-                          const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
-                          const void *h_seq, const void *v_init,
-                          const float *rtau_device, void *grad_x_seq, void *grad_v_init, float *grad_rtau,
-                          float *workspace, void *stream) {
+namespace {
+// everything sjhip_neuron_backward checks except the workspace
+int check_backward(int neuron, int dtype, const sjhip_neuron_params *p, int64_t T, int64_t N, const void *grad_spike_seq,
+                   const void *h_seq, const void *v_init, const float *rtau_device, void *grad_x_seq, void *grad_v_init,
+                   float *grad_rtau) {
   if (!p) return fail(SJHIP_ERR_INVALID, "backward: params is NULL");
   if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_EIF) return fail(SJHIP_ERR_INVALID, "backward: neuron %d", neuron);
   if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "backward: dtype %d", dtype);
@@ -234,10 +234,21 @@ int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p, i
   if (rc != SJHIP_OK) return rc;
   if ((neuron == SJHIP_NEURON_QIF || neuron == SJHIP_NEURON_EIF) && grad_v_init && !v_init)
     return fail(SJHIP_ERR_INVALID, "backward: QIF / EIF need v_init for grad_v_init");
-  if (neuron == SJHIP_NEURON_PLIF) {
-    if (!v_init || !grad_rtau || !rtau_device) return fail(SJHIP_ERR_INVALID, "backward: PLIF needs v_init, rtau_device and grad_rtau");
-    if (!(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace) return fail(SJHIP_ERR_INVALID, "backward: PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");
-  }
+  if (neuron == SJHIP_NEURON_PLIF && (!v_init || !grad_rtau || !rtau_device))
+    return fail(SJHIP_ERR_INVALID, "backward: PLIF needs v_init, rtau_device and grad_rtau");
+  return SJHIP_OK;
+}
+}  // namespace
+
+int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p, int64_t T, int64_t N,
+                          const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                          const void *h_seq, const void *v_init,
+                          const float *rtau_device, void *grad_x_seq, void *grad_v_init, float *grad_rtau,
+                          float *workspace, void *stream) {
+  int rc = check_backward(neuron, dtype, p, T, N, grad_spike_seq, h_seq, v_init, rtau_device, grad_x_seq, grad_v_init, grad_rtau);
+  if (rc != SJHIP_OK) return rc;
+  if (neuron == SJHIP_NEURON_PLIF && !(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace)
+    return fail(SJHIP_ERR_INVALID, "backward: PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");
   return launch_backward(neuron, dtype, *p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, rtau_device, grad_x_seq,
                          grad_v_init, grad_rtau, workspace, static_cast<hipStream_t>(stream));
 }
@@ -246,18 +257,19 @@ int sjhip_neuron_backward_static(int neuron, int dtype, const sjhip_neuron_param
                                  const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
                                  const void *h_seq, const void *v_init, const float *rtau_device, void *grad_x_seq,
                                  void *grad_v_init, float *grad_rtau, void *stream) {
+  int rc = check_backward(neuron, dtype, p, T, N, grad_spike_seq, h_seq, v_init, rtau_device, grad_x_seq, grad_v_init, grad_rtau);
+  if (rc != SJHIP_OK) return rc;
   float *workspace = nullptr;
-  const bool needs_workspace = p && neuron == SJHIP_NEURON_PLIF && !(p->flags & SJHIP_FLAG_ATOMIC_REDUCE);
-  if (needs_workspace) {
-    if (N >= 1 && plif_blocks(dtype, N) > kStaticWorkspaceFloats)
+  if (neuron == SJHIP_NEURON_PLIF && !(p->flags & SJHIP_FLAG_ATOMIC_REDUCE)) {
+    if (plif_blocks(dtype, N) > kStaticWorkspaceFloats)
       return fail(SJHIP_ERR_TOO_LARGE, "backward(static): N=%lld needs %lld partial sums, the built-in workspace holds %lld "
                   "(N <= %lld); use sjhip_neuron_backward with a workspace of the caller's", (long long)N,
                   (long long)plif_blocks(dtype, N), (long long)kStaticWorkspaceFloats, (long long)(kStaticWorkspaceFloats * 64));
-    int rc = static_workspace("backward(static)", &workspace);
+    rc = static_workspace("backward(static)", &workspace);
     if (rc != SJHIP_OK) return rc;
   }
-  return sjhip_neuron_backward(neuron, dtype, p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, rtau_device,
-                               grad_x_seq, grad_v_init, grad_rtau, workspace, stream);
+  return launch_backward(neuron, dtype, *p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, rtau_device, grad_x_seq,
+                         grad_v_init, grad_rtau, workspace, static_cast<hipStream_t>(stream));
 }
 
 namespace {
