@@ -47,7 +47,9 @@ def load(name):
 
 
 def grad_tolerance(dtype):
-    return dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-3)
+    # fp16: the reference's autograd rounds every backward op to fp16 (its gradients of O(1) carry a few 1e-3 of
+    # rounding noise of their own and flush to zero below 6e-8); the kernel computes in fp32 and rounds once
+    return dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=1e-2, atol=5e-3)
 
 
 def run_node(name, backend, device):
