@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define SJHIP_ABI_VERSION 3
+#define SJHIP_ABI_VERSION 4
 
 typedef enum sjhip_status {
   SJHIP_OK = 0,
@@ -403,6 +403,71 @@ int sjhip_ssa_backward_packed(int dtype, int64_t samples, int heads, int channel
                               const uint8_t *qkv_bits, const void *grad_out, void *grad_qkv, void *stream);
 
 /*
+ * Kernel-size-1 convolution over [S, C, L] activations (S samples = time steps x batch, L positions, L contiguous) as
+ * GEMMs on the bf16 matrix cores.  Stands in for torch's nn.Conv1d(kernel_size=1, bias=False) inside the reference's
+ * SpikingSelfAttention (spikingjelly/activation_based/layer/attention.py:310-329, applied at :370 and :382 through
+ * SeqToANNContainer) and nn.Conv2d(kernel_size=1) of SpikformerConv2dBN (model/spikformer.py:85-99), forward and both
+ * gradients.  fp32 operands are split into `terms` bf16 terms that sum to the value (3: exactly), and the products whose
+ * combined order is below max(terms) run on v_mfma_f32_32x32x16_bf16 with fp32 accumulation: 3 terms on both sides give
+ * the accuracy of an fp32 GEMM; an operand that bf16 holds exactly (spikes) needs 1 term.  Supported (a_terms, b_terms):
+ * (3,3) (3,1) (2,2) (2,1) (1,1).  L must be a multiple of 4 and the tensors 16-byte aligned (SJHIP_ERR_UNSUPPORTED).
+ *
+ *   sjhip_pwconv_split_weight   planes = bf16 terms [3][rows_pad][cols_pad] (zero padded to multiples of 128 and 32;
+ *                               sjhip_pwconv_planes_elems(rows, cols) elements of 2 bytes) of the matrix A = w
+ *                               ([rows][cols] fp32) or, with transpose != 0, of A = w^T ([cols][rows]): the first operand
+ *                               of sjhip_pwconv_gemm.  For transpose the element count is that of (cols, rows).
+ *   sjhip_pwconv_gemm           c[s][m][l] = sum_k A[m][k] b[s][k][l]: the convolution with A = weight [Cout][Cin]
+ *                               (M = Cout, K = Cin), its input gradient with A = weight^T (M = Cin, K = Cout, b = dY)
+ *   sjhip_pwconv_grad_weight    dw[m][n] = sum_{s,l} dy[s][m][l] x[s][n][l]; workspace of
+ *                               sjhip_pwconv_grad_weight_workspace_floats(M, N, S) floats (partial sums over groups of
+ *                               samples, added in a fixed order)
+ */
+int64_t sjhip_pwconv_planes_elems(int64_t rows, int64_t cols);
+int sjhip_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, void *stream);
+int sjhip_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,
+                      int64_t L, float *c, void *stream);
+int64_t sjhip_pwconv_grad_weight_workspace_floats(int64_t M, int64_t N, int64_t S);
+int sjhip_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int x_terms, int64_t S, int64_t M, int64_t N,
+                             int64_t L, float *dw, float *workspace, void *stream);
+
+/*
+ * Batch normalisation fused with the multi-step IF / LIF neuron behind it, for fp32 activations [T][B][C][L]
+ * (L contiguous, a multiple of 4).  Stands in for nn.BatchNorm1d / nn.BatchNorm2d followed by LIFNode in the reference's
+ * SpikingSelfAttention (layer/attention.py:314-329, 370-384) and SpikformerConv2dBNLIF (model/spikformer.py:196-212),
+ * which torch runs as separate passes; here the normalised tensor is never written.
+ *
+ *   sjhip_bn_stats      partial[s][c] = (sum_l y, sum_l y^2) of every row of y [S][C][L]          (training forward)
+ *   sjhip_bn_finalize   per channel: mean and biased variance from the partial sums (fp64), or, with partial == NULL
+ *                       (evaluation), from running_mean / running_var; writes the affine map z = y scale + shift
+ *                       (scale = gamma / sqrt(var + eps), shift = beta - mean scale; gamma / beta may be NULL = 1 / 0),
+ *                       mean and invstd (kept for the backward), and in training updates running_mean / running_var in
+ *                       place with `momentum` (unbiased variance), when they are given
+ *   sjhip_bn_lif_forward   z = y scale_c + shift_c, then charge / fire / reset over the T steps (same arithmetic and
+ *                       params as sjhip_neuron_forward; neuron IF or LIF); spikes go to spike_seq [T][B][C][L] (fp32) or
+ *                       bit-packed to spike_bits (the layout of sjhip_bit_pack; B*C*L must be a multiple of 8): exactly
+ *                       one of the two is given; v_last [B][C][L] or NULL
+ *   sjhip_bn_lif_backward  replays the neuron from y (T <= 16), runs the BPTT recurrence of sjhip_neuron_backward with
+ *                       grad_spike_seq and (optionally) grad_v_last, writes grad_z = dL/dz [T][B][C][L], grad_v_init
+ *                       (or NULL) and partial[b][c] = (sum g, sum g y) over the row and all steps
+ *   sjhip_bn_backward_finalize   dgamma, dbeta (either may be NULL) and coef [3][C] = (p, q, r) of dy = p g + q y + r;
+ *                       training != 0: batch statistics took part in the forward, else q = r = 0
+ *   sjhip_bn_grad_input    dy = p_c g + q_c y + r_c over [S][C][L]; dy may be g
+ */
+int sjhip_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, void *stream);
+int sjhip_bn_finalize(const float *partial, int64_t S, int64_t C, int64_t L, const float *gamma, const float *beta, float eps,
+                      float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
+                      float *invstd, void *stream);
+int sjhip_bn_lif_forward(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
+                         const float *scale, const float *shift, const float *v_init, float *spike_seq, uint8_t *spike_bits,
+                         float *v_last, void *stream);
+int sjhip_bn_lif_backward(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
+                          const float *scale, const float *shift, const float *v_init, const float *grad_spike_seq,
+                          const float *grad_v_last, float *grad_z, float *grad_v_init, float *partial, void *stream);
+int sjhip_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64_t C, int64_t L, int training, const float *gamma,
+                               const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef, void *stream);
+int sjhip_bn_grad_input(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy, void *stream);
+
+/*
  * Launch tuning (process-wide, read at launch).  Keys: "fwd_block" / "bwd_block" = work-items per
  * block (64, 128, 256 or 512); "fwd_blocks_per_cu" / "bwd_blocks_per_cu" = cap on resident blocks per
  * compute unit (0 = none, else 2..64; enforced through a dynamic-LDS request), and
@@ -417,7 +482,8 @@ int sjhip_get_tuning(const char *key);
 /*
  * Optional per-kernel timing.  While enabled every launch is bracketed by HIP events on its own
  * stream.  sjhip_profile_read() synchronises those events and returns, for kernel class `which`
- * (0 forward, 1 backward, 2 plif-reduce, 3 bit_pack, 4 bit_unpack, 5 ssa forward, 6 ssa backward), the launch count and total
+ * (0 forward, 1 backward, 2 plif-reduce, 3 bit_pack, 4 bit_unpack, 5 ssa forward, 6 ssa backward, 7 pwconv gemm,
+ * 8 pwconv grad_weight, 9 bn stats, 10 bn_lif forward, 11 bn_lif backward, 12 bn grad_input), the launch count and total
  * milliseconds since the last sjhip_profile_reset().
  */
 int sjhip_profile_enable(int on);

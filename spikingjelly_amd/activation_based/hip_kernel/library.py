@@ -14,7 +14,7 @@ from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64
 
 import torch
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 # enums of include/sjhip.h
 NEURON_IF, NEURON_LIF, NEURON_PLIF, NEURON_QIF, NEURON_ILIF, NEURON_EIF = 0, 1, 2, 3, 4, 5
@@ -34,7 +34,8 @@ FLAG_W_INIT_BROADCAST = 0x800
 FLAG_GRAD_STORAGE = 0x1000
 STATIC_WORKSPACE_MAX_NEURONS = 1 << 26
 
-KC_FORWARD, KC_BACKWARD, KC_PLIF_REDUCE, KC_BIT_PACK, KC_BIT_UNPACK, KC_SSA_FORWARD, KC_SSA_BACKWARD = range(7)
+(KC_FORWARD, KC_BACKWARD, KC_PLIF_REDUCE, KC_BIT_PACK, KC_BIT_UNPACK, KC_SSA_FORWARD, KC_SSA_BACKWARD, KC_PW_GEMM,
+ KC_PW_GRAD_WEIGHT, KC_BN_STATS, KC_BN_LIF_FORWARD, KC_BN_LIF_BACKWARD, KC_BN_GRAD_INPUT) = range(13)
 
 EXPORTED_SYMBOLS = (
     "sjhip_abi_version",
@@ -59,6 +60,17 @@ EXPORTED_SYMBOLS = (
     "sjhip_izhikevich_forward",
     "sjhip_izhikevich_backward",
     "sjhip_izhikevich_backward_replay",
+    "sjhip_pwconv_planes_elems",
+    "sjhip_pwconv_split_weight",
+    "sjhip_pwconv_gemm",
+    "sjhip_pwconv_grad_weight_workspace_floats",
+    "sjhip_pwconv_grad_weight",
+    "sjhip_bn_stats",
+    "sjhip_bn_finalize",
+    "sjhip_bn_lif_forward",
+    "sjhip_bn_lif_backward",
+    "sjhip_bn_backward_finalize",
+    "sjhip_bn_grad_input",
     "sjhip_bit_pack",
     "sjhip_bit_unpack",
     "sjhip_set_tuning",
@@ -191,6 +203,31 @@ def load() -> ctypes.CDLL:
         lib.sjhip_izhikevich_backward_replay.restype = c_int
         lib.sjhip_izhikevich_backward_replay.argtypes = ([c_int, POINTER(IzhikevichParams), c_int64, c_int64]
                                                          + [c_void_p] * 12)
+        lib.sjhip_pwconv_planes_elems.restype = c_int64
+        lib.sjhip_pwconv_planes_elems.argtypes = [c_int64, c_int64]
+        lib.sjhip_pwconv_split_weight.restype = c_int
+        lib.sjhip_pwconv_split_weight.argtypes = [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p]
+        lib.sjhip_pwconv_gemm.restype = c_int
+        lib.sjhip_pwconv_gemm.argtypes = [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_void_p,
+                                          c_void_p]
+        lib.sjhip_pwconv_grad_weight_workspace_floats.restype = c_int64
+        lib.sjhip_pwconv_grad_weight_workspace_floats.argtypes = [c_int64, c_int64, c_int64]
+        lib.sjhip_pwconv_grad_weight.restype = c_int
+        lib.sjhip_pwconv_grad_weight.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64,
+                                                 c_void_p, c_void_p, c_void_p]
+        lib.sjhip_bn_stats.restype = c_int
+        lib.sjhip_bn_stats.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]
+        lib.sjhip_bn_finalize.restype = c_int
+        lib.sjhip_bn_finalize.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float, c_float] + \
+                                         [c_void_p] * 7
+        lib.sjhip_bn_lif_forward.restype = c_int
+        lib.sjhip_bn_lif_forward.argtypes = [c_int, POINTER(NeuronParams), c_int64, c_int64, c_int64, c_int64] + [c_void_p] * 8
+        lib.sjhip_bn_lif_backward.restype = c_int
+        lib.sjhip_bn_lif_backward.argtypes = [c_int, POINTER(NeuronParams), c_int64, c_int64, c_int64, c_int64] + [c_void_p] * 10
+        lib.sjhip_bn_backward_finalize.restype = c_int
+        lib.sjhip_bn_backward_finalize.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int] + [c_void_p] * 7
+        lib.sjhip_bn_grad_input.restype = c_int
+        lib.sjhip_bn_grad_input.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]
         lib.sjhip_bit_pack.restype = c_int
         lib.sjhip_bit_pack.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p]
         lib.sjhip_bit_unpack.restype = c_int

@@ -2,8 +2,10 @@
 
 ``Conv1d+BN -> LIF -> scale * (V K^T) Q -> LIF(v_threshold=0.5) -> Conv1d+BN -> LIF`` on ``[T, N, C, L]``
 input.  With ``backend='hip'`` the three LIF nodes run the HIP neuron kernels and the contraction runs on
-the matrix cores (bf16 MFMA, fp32 accumulation; exact because Q/K/V are binary); the 1x1 convolutions and
-batch norms stay with torch.
+the matrix cores (int8 / bf16 MFMA, fp32 accumulation; exact because Q/K/V are binary).  For fp32 device tensors whose
+token count is a multiple of 4 the two ``Conv1d(k=1) -> BatchNorm1d -> LIF`` chains run fused as well (``layer/fused.py``:
+split-bf16 MFMA GEMMs, batch norm and the neuron in two passes over the convolution output); other inputs keep
+torch's convolution and batch norm around the hip neurons.
 """
 
 from __future__ import annotations
@@ -12,6 +14,7 @@ import torch
 import torch.nn as nn
 
 from .. import base, neuron
+from . import fused
 from .container import SeqToANNContainer
 
 
@@ -101,19 +104,29 @@ class SpikingSelfAttention(nn.Module, base.MultiStepModule):
         if x_seq.ndim != 4:
             raise ValueError(f"expected 4D input with shape [T, N, C, L], but got input with shape {x_seq.shape}")
         T, N, C, L = x_seq.shape
-        pre = self.qkv_conv_bn(x_seq)  # [T, N, 3*C, L]
-        local_dim = pre.shape[2] // 3
-        if local_dim % self.num_heads != 0:
-            raise ValueError(f"local qkv dim {local_dim} is not divisible by num_heads={self.num_heads}.")
-        x_seq = self._lif_ssa_fused(pre) if self.backend == "hip" else None
-        if x_seq is None:
-            qkv = self.qkv_lif(pre).reshape(T, N, 3, self.num_heads, local_dim // self.num_heads, L)
-            if self.backend == "hip":
-                x_seq = self._ssa_kernel_hip(qkv, self.scale)
-            else:
-                x_seq = self._ssa_kernel_torch(qkv, self.scale)
-        x_seq = self.attn_lif(x_seq).reshape(T, N, local_dim, L)
-        return self.proj_lif(self.proj_conv_bn(x_seq))  # [T, N, C, L]
+        hip = self.backend == "hip"
+        out = None
+        if hip and len(self.qkv_conv_bn) == 2:
+            # convolution, batch norm, LIF (bit-packed spikes) and the contraction in one autograd node
+            out = fused.conv_bn_lif(x_seq, self.qkv_conv_bn[0], self.qkv_conv_bn[1], self.qkv_lif,
+                                    ssa=(self.num_heads, self.scale))
+        if out is None:
+            pre = self.qkv_conv_bn(x_seq)  # [T, N, 3*C, L]
+            local_dim = pre.shape[2] // 3
+            if local_dim % self.num_heads != 0:
+                raise ValueError(f"local qkv dim {local_dim} is not divisible by num_heads={self.num_heads}.")
+            out = self._lif_ssa_fused(pre) if hip else None
+            if out is None:
+                qkv = self.qkv_lif(pre).reshape(T, N, 3, self.num_heads, local_dim // self.num_heads, L)
+                out = self._ssa_kernel_hip(qkv, self.scale) if hip else self._ssa_kernel_torch(qkv, self.scale)
+        local_dim = out.shape[2] * out.shape[3]
+        x_seq = self.attn_lif(out).reshape(T, N, local_dim, L)
+        y = None
+        if hip and len(self.proj_conv_bn) == 2:
+            y = fused.conv_bn_lif(x_seq, self.proj_conv_bn[0], self.proj_conv_bn[1], self.proj_lif, x_exact=True)
+        if y is None:
+            y = self.proj_lif(self.proj_conv_bn(x_seq))
+        return y  # [T, N, C, L]
 
     def extra_repr(self):
         return f"dim={self.dim}, num_heads={self.num_heads}, backend={self.backend}"

@@ -1,0 +1,106 @@
+"""Host-side glue between modules and the fused convolution / batch-norm / LIF kernels of
+``hip_kernel/conv_bn_lif.py``: decides whether a ``conv -> BatchNorm -> LIFNode`` chain can run fused and, if so, runs
+it and writes the neuron's state back.  Every function returns ``None`` when the chain has to run unfused (the caller
+then calls its sub-modules one after the other, which gives the same result)."""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from .. import neuron
+
+
+def _pointwise(conv: nn.Module) -> bool:
+    """A convolution that is one matrix product per position: kernel 1, stride 1, no padding, one group, no bias."""
+    if not isinstance(conv, (nn.Conv1d, nn.Conv2d)):
+        return False
+    one = all(k == 1 for k in conv.kernel_size) and all(s == 1 for s in conv.stride) and all(d == 1 for d in conv.dilation)
+    no_pad = all(p == 0 for p in conv.padding) if not isinstance(conv.padding, str) else conv.padding == "valid"
+    return one and no_pad and conv.groups == 1 and conv.bias is None
+
+
+def _bn_arguments(bn: nn.Module):
+    """``(gamma, beta, (running_mean, running_var, batch_stats, momentum, eps))`` the way ``_BatchNorm.forward`` derives
+    them, or ``None`` for what the kernels do not cover (cumulative moving average)."""
+    if not isinstance(bn, (nn.BatchNorm1d, nn.BatchNorm2d)):
+        return None
+    batch_stats = bn.training or (bn.running_mean is None and bn.running_var is None)
+    update = bn.training and bn.track_running_stats
+    if update and bn.momentum is None:
+        return None
+    if update and bn.num_batches_tracked is not None:
+        bn.num_batches_tracked.add_(1)
+    running_mean = bn.running_mean if (update or not batch_stats) else None
+    running_var = bn.running_var if (update or not batch_stats) else None
+    return bn.weight, bn.bias, (running_mean, running_var, batch_stats, float(bn.momentum or 0.0), float(bn.eps))
+
+
+def _lif_spec(node: neuron.LIFNode, x_like: torch.Tensor, need_grad: bool):
+    from ..functional import neuron as F
+    from ..hip_kernel import neuron_kernel as K
+    from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
+
+    soft = node.v_reset is None
+    flags = K._flags(soft, node.detach_reset, node.decay_input, F._hip_mode_flags(x_like))
+    sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(node.surrogate_function) if need_grad else (0, 0.0)
+    return (float(node.tau), node.v_threshold, 0.0 if soft else float(node.v_reset), flags, sg_id, sg_alpha)
+
+
+def conv_bn_lif(x_seq: torch.Tensor, conv: Optional[nn.Module], bn: nn.Module, node: nn.Module, x_exact: bool = False,
+                ssa: Optional[tuple] = None) -> Optional[torch.Tensor]:
+    """``node(bn(conv(x_seq)))`` for ``x_seq [T, B, C, *positions]`` in one fused pass, or ``None``.
+
+    ``conv is None``: ``x_seq`` already is the convolution output and only batch norm and the neuron are fused.
+    ``ssa = (heads, scale)``: the spikes feed the spiking self-attention contraction bit-packed and the result is
+    ``scale (V K^T) Q`` as ``[T, B, heads, channels_per_head, L]``.  ``x_exact``: ``x_seq`` holds values that bf16
+    represents exactly (spikes)."""
+    from ..hip_kernel import conv_bn_lif as C
+
+    if (torch.compiler.is_compiling() or type(node) is not neuron.LIFNode or node.backend != "hip" or node.step_mode != "m"
+            or node.store_v_seq or x_seq.dim() < 4):
+        return None
+    if conv is not None and (not _pointwise(conv) or x_seq.shape[2] != conv.in_channels):
+        return None
+    channels = conv.out_channels if conv is not None else x_seq.shape[2]
+    if not isinstance(bn, (nn.BatchNorm1d, nn.BatchNorm2d)) or bn.num_features != channels:
+        return None
+    params = (p for p in (conv.weight if conv is not None else None, bn.weight, bn.bias) if p is not None)
+    need_grad = torch.is_grad_enabled() and (x_seq.requires_grad or any(p.requires_grad for p in params))
+    x4 = x_seq.flatten(3)  # [T, B, C, L]
+    if not C.supported(x4, need_grad):
+        return None
+    T, B, _, Lp = x4.shape
+    if ssa is not None:
+        from ..hip_kernel import attention_kernel as A
+
+        heads, scale = ssa
+        cph = channels // 3 // heads
+        if channels != 3 * heads * cph or not A.ssa_packed_supported(x4.dtype, cph, Lp) or (B * channels * Lp) % 8 != 0:
+            return None
+    node._check_hip_surrogate()
+    state_like = torch.empty((1,), dtype=x4.dtype, device=x4.device).expand(T, B, channels, *x_seq.shape[3:])
+    (v,) = node.materialize_states((state_like,), (node.v,), "m")
+    if need_grad and v.requires_grad:
+        return None
+    bn_args = _bn_arguments(bn)
+    if bn_args is None:
+        return None
+    gamma, beta, bn_cfg = bn_args
+    spec = _lif_spec(node, x4, need_grad)
+    v3 = v.reshape(B, channels, Lp) if v.dim() != 3 else v
+    out_shape = (T, B, channels, *x_seq.shape[3:])
+    with torch.set_grad_enabled(need_grad):
+        if conv is None:
+            spikes, v_last = C.bn_lif(x4, gamma, beta, v3, bn_cfg, spec)
+        elif ssa is None:
+            spikes, v_last = C.conv_bn_lif(x4, conv.weight.view(channels, -1), gamma, beta, v3, bn_cfg, spec, x_exact)
+        else:
+            out, v_last = C.conv_bn_lif_ssa(x4, conv.weight.view(channels, -1), gamma, beta, v3, bn_cfg, spec, x_exact,
+                                            heads, cph, scale)
+            node.v = v_last.reshape(out_shape[1:])
+            return out.view(T, B, heads, cph, Lp)
+    node.v = v_last.reshape(out_shape[1:])
+    return spikes.view(out_shape)

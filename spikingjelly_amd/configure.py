@@ -33,6 +33,10 @@ for its CuPy/Triton backends).
 """
 
 hip_half_precision_mode = "torch"
+# Number of bf16 terms an fp32 operand of the fused kernel-size-1 convolutions is split into (hip_kernel/conv_bn_lif.py):
+# 3 keeps the accuracy of an fp32 GEMM (six matrix-core products per pair of real operands, three when one operand is
+# spikes), 2 gives about 2^-17 relative per product at half the products, 1 is a plain bf16 GEMM.
+hip_conv_terms = 3
 hip_backward_recompute = True
 hip_lif_reciprocal_tau = False
 hip_plif_atomic_reduce = False

@@ -1,0 +1,397 @@
+// Batch normalisation fused with the multi-step neuron that follows it, for activations laid out [T, B, C, L]
+// (time, batch, channels, positions; L contiguous): the block  conv -> BatchNorm1d / BatchNorm2d -> LIFNode  of the
+// reference's spiking self-attention and Spikformer stem (layer/attention.py:310-329, 370-384;
+// model/spikformer.py:16-99, 107-212), where torch runs batch norm and the neuron as separate passes over the tensor.
+//
+// Training forward:  bn_stats_kernel reads the convolution output y once (one wavefront per (sample, channel) row,
+//   fp32 partial sums of y and y^2), bn_finalize_kernel combines them in fp64 into the per-channel affine map
+//   z = y a_c + b_c  (a_c = gamma_c / sqrt(var_c + eps), b_c = beta_c - mean_c a_c) and updates the running statistics,
+//   bn_lif_forward_kernel reads y a second time, applies the map and runs the neuron over the T steps in registers,
+//   writing spikes dense or bit-packed.  The normalised tensor never exists in memory.  In evaluation mode the map
+//   comes from the running statistics and the first pass is skipped.
+// Backward:  bn_lif_backward_kernel replays the neuron from y (the forward's own arithmetic, so the replayed h has its
+//   bits), walks the BPTT recurrence and writes g = dL/dz; a wavefront owns one (batch, channel) row for all T steps and
+//   leaves sum g and sum g y of its row.  bn_backward_finalize_kernel turns those into dgamma, dbeta and the three
+//   per-channel coefficients of  dy = p_c g + q_c y + r_c,  which bn_grad_input_kernel applies (in place over g).
+// Arithmetic of the neuron is neuron_step / surrogate_grad of the plain neuron kernels.
+#include "neuron_bwd.h"
+#include "neuron_fwd.h"
+
+namespace sjhip {
+
+namespace {
+
+struct BnLifFwdArgs {
+  FwdArgs f;           // x = y [T][N], N = B * C * L
+  const float *scale;  // [C]
+  const float *shift;  // [C]
+  int C, L;
+};
+
+struct BnLifBwdArgs {
+  FwdArgs f;
+  BwdArgs b;           // grad_spike, grad_v_last, grad_x (= g out), grad_v_init
+  const float *scale;
+  const float *shift;
+  float *partial;      // [B * C][2]: sum g, sum g y of the row
+  int C, L;
+  int64_t rows;        // B * C
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  return v;
+}
+
+// one wavefront per row of L contiguous elements: sum and sum of squares
+__global__ void __launch_bounds__(256) bn_stats_kernel(const float *y, int64_t rows, int L, float *partial) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const f32x4 *p = reinterpret_cast<const f32x4 *>(y + row * L);
+  float s = 0.0f, q = 0.0f;
+  for (int i = lane; i < L / 4; i += 64) {
+    const f32x4 v = p[i];
+    s += (v.x + v.y) + (v.z + v.w);
+    q = fmaf(v.x, v.x, q); q = fmaf(v.y, v.y, q); q = fmaf(v.z, v.z, q); q = fmaf(v.w, v.w, q);
+  }
+  s = wave_sum(s);
+  q = wave_sum(q);
+  if (lane == 0) { partial[2 * row] = s; partial[2 * row + 1] = q; }
+}
+
+// partial == nullptr: evaluation mode, the map comes from the running statistics (which stay as they are)
+__global__ void __launch_bounds__(256) bn_finalize_kernel(const float *partial, int64_t S, int C, int64_t count,
+                                                           const float *gamma, const float *beta, float eps,
+                                                           float momentum, float *running_mean, float *running_var,
+                                                           float *scale, float *shift, float *mean_out, float *invstd_out) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  double mean, var;
+  if (partial) {
+    double s = 0.0, q = 0.0;
+    for (int64_t i = 0; i < S; ++i) { s += (double)partial[2 * (i * C + c)]; q += (double)partial[2 * (i * C + c) + 1]; }
+    mean = s / (double)count;
+    var = q / (double)count - mean * mean;
+    if (var < 0.0) var = 0.0;
+    if (running_mean) running_mean[c] = (float)((1.0 - (double)momentum) * (double)running_mean[c] + (double)momentum * mean);
+    if (running_var) {
+      const double unbiased = count > 1 ? var * (double)count / (double)(count - 1) : var;
+      running_var[c] = (float)((1.0 - (double)momentum) * (double)running_var[c] + (double)momentum * unbiased);
+    }
+  } else {
+    mean = (double)running_mean[c];
+    var = (double)running_var[c];
+  }
+  const double invstd = 1.0 / sqrt(var + (double)eps);
+  const double g = gamma ? (double)gamma[c] : 1.0, b = beta ? (double)beta[c] : 0.0;
+  const double a = g * invstd;
+  scale[c] = (float)a;
+  shift[c] = (float)(b - mean * a);
+  mean_out[c] = (float)mean;
+  invstd_out[c] = (float)invstd;
+}
+
+template <int CH, int RS, bool PACKED>
+__device__ __forceinline__ void bn_lif_forward_body(const BnLifFwdArgs &a) {
+  typedef Acc<float, true, false> A;
+  const FwdArgs &f = a.f;
+  const int64_t N = f.N, T = f.T;
+  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (col >= N) return;
+  const int c = (int)((col / a.L) % a.C);
+  const float sc = a.scale[c], sh = a.shift[c];
+  const float *yp = (const float *)f.x + col;
+  float *sp = (float *)f.spike + col;
+  float v[4];
+  load_state<float, true, false>(f.v_init, col, f.v_init_broadcast != 0, v);
+  constexpr int PF = 4;
+  for (int64_t t0 = 0; t0 < T; t0 += PF) {
+    f32x4 rows[PF];
+#pragma unroll
+    for (int i = 0; i < PF; ++i) rows[i] = (t0 + i < T) ? A::load(yp + (t0 + i) * N) : A::zero();
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int64_t t = t0 + i;
+      if (t < T) {
+        float y[4], h[4], s[4];
+        A::unpack(rows[i], y);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) neuron_step<float, CH, RS>(fmaf(y[j], sc, sh), v[j], h[j], s[j], f.tau, f);
+        if (PACKED) store_spike_bits<4>((uint8_t *)f.spike + t * (N >> 3), col, N, s);
+        else A::store(sp + t * N, s);
+      }
+    }
+  }
+  if (f.v_last) A::store((float *)f.v_last + col, v);
+}
+
+template <int CH, bool PACKED> __device__ __forceinline__ void bn_lif_forward_reset(const BnLifFwdArgs &a) {
+  if (a.f.soft_reset) bn_lif_forward_body<CH, RESET_SOFT, PACKED>(a);
+  else bn_lif_forward_body<CH, RESET_HARD, PACKED>(a);
+}
+
+template <bool PACKED> __global__ void __launch_bounds__(256) bn_lif_forward_kernel(const BnLifFwdArgs a) {
+  switch (a.f.charge) {
+    case CH_IF: bn_lif_forward_reset<CH_IF, PACKED>(a); break;
+    case CH_DECAY_INPUT_DIV: bn_lif_forward_reset<CH_DECAY_INPUT_DIV, PACKED>(a); break;
+    case CH_DECAY_INPUT_MUL: bn_lif_forward_reset<CH_DECAY_INPUT_MUL, PACKED>(a); break;
+    case CH_PLAIN_INPUT_DIV: bn_lif_forward_reset<CH_PLAIN_INPUT_DIV, PACKED>(a); break;
+    default: bn_lif_forward_reset<CH_PLAIN_INPUT_MUL, PACKED>(a); break;
+  }
+}
+
+// h of every step of this work-item's four neurons, replayed from y
+template <int CH, int RS, int TMAX>
+__device__ __forceinline__ void replay_h(const FwdArgs &f, const f32x4 (&yv)[TMAX], float sc, float sh, float (&v)[4],
+                                         float (&h)[TMAX][4]) {
+#pragma unroll
+  for (int t = 0; t < TMAX; ++t) {
+    if (t < f.T) {
+      const float y[4] = {yv[t].x, yv[t].y, yv[t].z, yv[t].w};
+      float s;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) neuron_step<float, CH, RS>(fmaf(y[j], sc, sh), v[j], h[t][j], s, f.tau, f);
+    }
+  }
+}
+
+template <int CH, int TMAX>
+__device__ __forceinline__ void replay_h_reset(const FwdArgs &f, const f32x4 (&yv)[TMAX], float sc, float sh, float (&v)[4],
+                                               float (&h)[TMAX][4]) {
+  if (f.soft_reset) replay_h<CH, RESET_SOFT, TMAX>(f, yv, sc, sh, v, h);
+  else replay_h<CH, RESET_HARD, TMAX>(f, yv, sc, sh, v, h);
+}
+
+// BPTT over the replayed h (recurrence of neuron_bwd.h); writes g = dL/dz and adds this work-item's share of
+// sum g and sum g y
+template <int SG, int TMAX>
+__device__ __forceinline__ void bptt_rows(const BwdArgs &b, float k, int64_t col, const f32x4 (&yv)[TMAX],
+                                          const float (&h)[TMAX][4], float (&carry)[4], float &acc_g, float &acc_gy) {
+#pragma clang fp contract(fast)
+  typedef Acc<float, true, true> A;
+  const int64_t N = b.N;
+  const float *gsp = (const float *)b.grad_spike + col;
+  float *gxp = (float *)b.grad_x + col;
+  const float kx = b.is_if ? 1.0f : (b.decay_input ? k : 1.0f);
+  const float km = b.is_if ? 1.0f : (1.0f - k);
+#pragma unroll
+  for (int t = TMAX - 1; t >= 0; --t) {
+    if (t < b.T) {
+      float gs[4], gz[4];
+      A::unpack(A::load(gsp + (int64_t)t * N), gs);
+      const float y[4] = {yv[t].x, yv[t].y, yv[t].z, yv[t].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float over = h[t][j] - b.v_th;
+        const float s = (over >= 0.0f) ? 1.0f : 0.0f;
+        const float sg = surrogate_grad<SG, false>(over, b.alpha);
+        const float dvdh = (1.0f - s * b.cB) + (b.cC - h[t][j] * b.cD) * sg;
+        const float G = carry[j] * dvdh + gs[j] * sg;
+        gz[j] = G * kx;
+        carry[j] = G * km;
+        acc_g += gz[j];
+        acc_gy = fmaf(gz[j], y[j], acc_gy);
+      }
+      Acc<float, true, false>::store(gxp + (int64_t)t * N, gz);  // read again by the next kernel
+    }
+  }
+}
+
+template <int TMAX> __global__ void __launch_bounds__(256) bn_lif_backward_kernel(const BnLifBwdArgs a) {
+  typedef Acc<float, true, false> A;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.rows) return;
+  const FwdArgs &f = a.f;
+  const BwdArgs &b = a.b;
+  const int c = (int)(row % a.C);
+  const float sc = a.scale[c], sh = a.shift[c];
+  const float k = b.k;
+  const int64_t N = f.N;
+  float acc_g = 0.0f, acc_gy = 0.0f;
+  for (int q = lane; q < a.L / 4; q += 64) {
+    const int64_t col = row * a.L + 4 * q;
+    const float *yp = (const float *)f.x + col;
+    f32x4 yv[TMAX];
+#pragma unroll
+    for (int t = 0; t < TMAX; ++t) yv[t] = (t < f.T) ? A::load(yp + (int64_t)t * N) : A::zero();
+    float v[4], h[TMAX][4], carry[4];
+    load_state<float, true, false>(f.v_init, col, f.v_init_broadcast != 0, v);
+    if (b.grad_v_last) A::unpack(A::load((const float *)b.grad_v_last + col), carry);
+    else carry[0] = carry[1] = carry[2] = carry[3] = 0.0f;
+    switch (f.charge) {
+      case CH_IF: replay_h_reset<CH_IF, TMAX>(f, yv, sc, sh, v, h); break;
+      case CH_DECAY_INPUT_DIV: replay_h_reset<CH_DECAY_INPUT_DIV, TMAX>(f, yv, sc, sh, v, h); break;
+      case CH_DECAY_INPUT_MUL: replay_h_reset<CH_DECAY_INPUT_MUL, TMAX>(f, yv, sc, sh, v, h); break;
+      case CH_PLAIN_INPUT_DIV: replay_h_reset<CH_PLAIN_INPUT_DIV, TMAX>(f, yv, sc, sh, v, h); break;
+      default: replay_h_reset<CH_PLAIN_INPUT_MUL, TMAX>(f, yv, sc, sh, v, h); break;
+    }
+    switch (b.sg) {
+      case SJHIP_SG_SIGMOID: bptt_rows<SJHIP_SG_SIGMOID, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+      case SJHIP_SG_ATAN: bptt_rows<SJHIP_SG_ATAN, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+      case SJHIP_SG_PIECEWISE_QUADRATIC: bptt_rows<SJHIP_SG_PIECEWISE_QUADRATIC, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+      case SJHIP_SG_PIECEWISE_EXP: bptt_rows<SJHIP_SG_PIECEWISE_EXP, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+      case SJHIP_SG_SOFT_SIGN: bptt_rows<SJHIP_SG_SOFT_SIGN, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+      case SJHIP_SG_SUPER_SPIKE: bptt_rows<SJHIP_SG_SUPER_SPIKE, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+      default: bptt_rows<SJHIP_SG_ERF, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+    }
+    if (b.grad_v_init) A::store((float *)b.grad_v_init + col, carry);
+  }
+  acc_g = wave_sum(acc_g);
+  acc_gy = wave_sum(acc_gy);
+  if (lane == 0) { a.partial[2 * row] = acc_g; a.partial[2 * row + 1] = acc_gy; }
+}
+
+// dgamma, dbeta and the coefficients of dy = p g + q y + r; count = T * B * L elements per channel
+__global__ void __launch_bounds__(256) bn_backward_finalize_kernel(const float *partial, int64_t B, int C, int64_t count,
+                                                                    int training, const float *gamma, const float *mean,
+                                                                    const float *invstd, float *dgamma, float *dbeta,
+                                                                    float *coef) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  double sg = 0.0, sgy = 0.0;
+  for (int64_t i = 0; i < B; ++i) { sg += (double)partial[2 * (i * C + c)]; sgy += (double)partial[2 * (i * C + c) + 1]; }
+  const double m = (double)mean[c], is = (double)invstd[c], g = gamma ? (double)gamma[c] : 1.0;
+  const double dg = is * (sgy - m * sg);  // sum g (y - mean) invstd
+  if (dgamma) dgamma[c] = (float)dg;
+  if (dbeta) dbeta[c] = (float)sg;
+  const double a = g * is;
+  coef[c] = (float)a;
+  if (training) {
+    coef[C + c] = (float)(-a * dg * is / (double)count);
+    coef[2 * C + c] = (float)(a * (dg * is * m - sg) / (double)count);
+  } else {
+    coef[C + c] = 0.0f;
+    coef[2 * C + c] = 0.0f;
+  }
+}
+
+// dy = p_c g + q_c y + r_c over the flattened [S * C * L] tensor; dy may be g itself
+__global__ void __launch_bounds__(256) bn_grad_input_kernel(const float *g, const float *y, const float *coef, int C, int L,
+                                                             int64_t n, float *dy) {
+  const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i >= n) return;
+  const int c = (int)((i / L) % C);
+  const float p = coef[c], q = coef[C + c], r = coef[2 * C + c];
+  const f32x4 gv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(g + i));
+  const f32x4 yv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(y + i));
+  f32x4 o;
+  o.x = fmaf(p, gv.x, fmaf(q, yv.x, r));
+  o.y = fmaf(p, gv.y, fmaf(q, yv.y, r));
+  o.z = fmaf(p, gv.z, fmaf(q, yv.z, r));
+  o.w = fmaf(p, gv.w, fmaf(q, yv.w, r));
+  *reinterpret_cast<f32x4 *>(dy + i) = o;
+}
+
+int check_layout(const char *what, int64_t T, int64_t B, int64_t C, int64_t L) {
+  if (T < 1 || B < 1 || C < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "%s: T=%lld B=%lld C=%lld L=%lld must be >= 1", what, (long long)T, (long long)B, (long long)C, (long long)L);
+  if (L % 4 != 0) return fail(SJHIP_ERR_UNSUPPORTED, "%s: L=%lld must be a multiple of 4", what, (long long)L);
+  if (C > (1 << 24) || L > (1 << 24) || B * C > (int64_t(1) << 40) || T > (int64_t(1) << 40) / (B * C * L))
+    return fail(SJHIP_ERR_TOO_LARGE, "%s: T=%lld B=%lld C=%lld L=%lld", what, (long long)T, (long long)B, (long long)C, (long long)L);
+  return SJHIP_OK;
+}
+
+bool lif_like(int neuron) { return neuron == SJHIP_NEURON_IF || neuron == SJHIP_NEURON_LIF; }
+
+}  // namespace
+
+int launch_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, hipStream_t stream) {
+  int rc = check_layout("bn_stats", 1, S, C, L);
+  if (rc != SJHIP_OK) return rc;
+  if (!aligned16(y)) return fail(SJHIP_ERR_UNSUPPORTED, "bn_stats: y must be 16-byte aligned");
+  const int64_t rows = S * C, blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "bn_stats: %lld rows", (long long)rows);
+  ProfileScope prof(KC_BN_STATS, stream);
+  hipLaunchKernelGGL(bn_stats_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, y, rows, (int)L, partial);
+  return check_launch("bn_stats");
+}
+
+int launch_bn_finalize(const float *partial, int64_t S, int64_t C, int64_t L, const float *gamma, const float *beta, float eps,
+                       float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
+                       float *invstd, hipStream_t stream) {
+  if (C < 1 || C > (1 << 24)) return fail(SJHIP_ERR_INVALID, "bn_finalize: C=%lld", (long long)C);
+  if (!partial && (!running_mean || !running_var)) return fail(SJHIP_ERR_INVALID, "bn_finalize: evaluation mode needs the running statistics");
+  hipLaunchKernelGGL(bn_finalize_kernel, dim3((unsigned)((C + 255) / 256)), dim3(256), 0, stream, partial, S, (int)C, S * L, gamma,
+                     beta, eps, momentum, running_mean, running_var, scale, shift, mean, invstd);
+  return check_launch("bn_finalize");
+}
+
+int launch_bn_lif_forward(int neuron, const sjhip_neuron_params &p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
+                          const float *scale, const float *shift, const float *v_init, float *spike_seq, uint8_t *spike_bits,
+                          float *v_last, hipStream_t stream) {
+  int rc = check_layout("bn_lif_forward", T, B, C, L);
+  if (rc != SJHIP_OK) return rc;
+  if (!lif_like(neuron)) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_forward: neuron %d (IF and LIF only)", neuron);
+  const int64_t N = B * C * L;
+  const bool broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) != 0;
+  if (!aligned16(y) || (!broadcast && !aligned16(v_init)) || (spike_seq && !aligned16(spike_seq)) || (v_last && !aligned16(v_last)))
+    return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_forward: tensors must be 16-byte aligned");
+  if (spike_bits && N % 8 != 0) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_forward: B*C*L=%lld must be a multiple of 8 for bit-packed spikes", (long long)N);
+  BnLifFwdArgs a;
+  bool round_each = false;
+  rc = build_fwd_args(a.f, round_each, neuron, SJHIP_F32, p, T, N, y, v_init, nullptr, spike_bits ? (void *)spike_bits : (void *)spike_seq,
+                      nullptr, v_last, nullptr);
+  if (rc != SJHIP_OK) return rc;
+  a.scale = scale; a.shift = shift; a.C = (int)C; a.L = (int)L;
+  const int64_t blocks = (N / 4 + 255) / 256;
+  if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "bn_lif_forward: N=%lld", (long long)N);
+  ProfileScope prof(KC_BN_LIF_FORWARD, stream);
+  if (spike_bits) hipLaunchKernelGGL((bn_lif_forward_kernel<true>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL((bn_lif_forward_kernel<false>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  return check_launch("bn_lif_forward");
+}
+
+int launch_bn_lif_backward(int neuron, const sjhip_neuron_params &p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
+                           const float *scale, const float *shift, const float *v_init, const float *grad_spike_seq,
+                           const float *grad_v_last, float *grad_z, float *grad_v_init, float *partial, hipStream_t stream) {
+  int rc = check_layout("bn_lif_backward", T, B, C, L);
+  if (rc != SJHIP_OK) return rc;
+  if (!lif_like(neuron)) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: neuron %d (IF and LIF only)", neuron);
+  if (T > 16) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: T=%lld (at most 16 steps are replayed in registers)", (long long)T);
+  if (p.sg_id < SJHIP_SG_SIGMOID || p.sg_id > SJHIP_SG_ERF) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: surrogate id %d", p.sg_id);
+  const int64_t N = B * C * L;
+  const bool broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) != 0;
+  if (!aligned16(y) || (!broadcast && !aligned16(v_init)) || !aligned16(grad_spike_seq) || !aligned16(grad_z) ||
+      (grad_v_last && !aligned16(grad_v_last)) || (grad_v_init && !aligned16(grad_v_init)))
+    return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: tensors must be 16-byte aligned");
+  BnLifBwdArgs a;
+  bool round_each = false;
+  rc = build_fwd_args(a.f, round_each, neuron, SJHIP_F32, p, T, N, y, v_init, nullptr, nullptr, nullptr, nullptr, nullptr);
+  if (rc != SJHIP_OK) return rc;
+  rc = build_bwd_args(a.b, neuron, SJHIP_F32, p, T, N, grad_spike_seq, nullptr, grad_v_last, nullptr, v_init, nullptr, grad_z,
+                      grad_v_init, nullptr, nullptr);
+  if (rc != SJHIP_OK) return rc;
+  a.scale = scale; a.shift = shift; a.partial = partial; a.C = (int)C; a.L = (int)L; a.rows = B * C;
+  const int64_t blocks = (a.rows + 3) / 4;
+  if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "bn_lif_backward: %lld rows", (long long)a.rows);
+  ProfileScope prof(KC_BN_LIF_BACKWARD, stream);
+  if (T <= 4) hipLaunchKernelGGL((bn_lif_backward_kernel<4>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  else if (T <= 8) hipLaunchKernelGGL((bn_lif_backward_kernel<8>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL((bn_lif_backward_kernel<16>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  return check_launch("bn_lif_backward");
+}
+
+int launch_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64_t C, int64_t L, int training, const float *gamma,
+                                const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef,
+                                hipStream_t stream) {
+  if (C < 1 || C > (1 << 24)) return fail(SJHIP_ERR_INVALID, "bn_backward_finalize: C=%lld", (long long)C);
+  hipLaunchKernelGGL(bn_backward_finalize_kernel, dim3((unsigned)((C + 255) / 256)), dim3(256), 0, stream, partial, B, (int)C,
+                     T * B * L, training, gamma, mean, invstd, dgamma, dbeta, coef);
+  return check_launch("bn_backward_finalize");
+}
+
+int launch_bn_grad_input(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy,
+                         hipStream_t stream) {
+  int rc = check_layout("bn_grad_input", 1, S, C, L);
+  if (rc != SJHIP_OK) return rc;
+  if (!aligned16(g) || !aligned16(y) || !aligned16(dy)) return fail(SJHIP_ERR_UNSUPPORTED, "bn_grad_input: tensors must be 16-byte aligned");
+  const int64_t n = S * C * L, blocks = (n / 4 + 255) / 256;
+  if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "bn_grad_input: %lld elements", (long long)n);
+  ProfileScope prof(KC_BN_GRAD_INPUT, stream);
+  hipLaunchKernelGGL(bn_grad_input_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, g, y, coef, (int)C, (int)L, n, dy);
+  return check_launch("bn_grad_input");
+}
+
+}  // namespace sjhip

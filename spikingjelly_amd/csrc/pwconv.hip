@@ -1,0 +1,498 @@
+// Pointwise (kernel size 1) convolution over [S, C, L] activations on the bf16 matrix cores with fp32 accuracy.
+//
+// The reference computes the block Conv1d(k=1) -> BatchNorm1d -> LIF of its spiking self-attention with torch's
+// convolution (layer/attention.py:310-329, 370-384; Conv2d(k=1) in model/spikformer.py:16-99).  A kernel-size-1
+// convolution is the GEMM  Y[s] = W X[s]  per sample s, with X[s] a row-major [K, L] tile (tokens contiguous), and its
+// backward the two GEMMs  dX[s] = W^T dY[s]  and  dW = sum_s dY[s] X[s]^T.  fp32 operands are split on the fly into up to
+// three bf16 terms that sum to the value exactly (round to nearest, remainder, again); the products of the leading
+// terms run on v_mfma_f32_32x32x16_bf16 with fp32 accumulation.  With three terms per operand and the six products
+// whose combined order is at most two, the dropped part is below 2^-24 of each product: the accuracy of an fp32 GEMM
+// at a multiple of the fp32 MFMA rate; an operand that is exact in bf16 (spikes, small counts) needs one term and
+// halves the products.  Fewer terms trade accuracy for speed (two terms: about 2^-17 relative per product).
+//
+//   pw_gemm_kernel     C[s][m][l] = sum_k A[m][k] B[s][k][l]     (forward with A = W, input gradient with A = W^T)
+//       A comes pre-split as bf16 planes [3][M_pad][K_pad] (split_weight_kernel, zero padded), B is fp32 in memory.
+//       The S * L columns of all samples form one column index, so tiles of 128 columns carry no padding whatever L
+//       is.  A block of four wavefronts owns a 128 x 128 tile (each wavefront 64 x 64 = 2 x 2 MFMA tiles) and walks K
+//       in steps of 32: A tiles are copied to LDS as they are, B tiles are split and stored row by row (k rows,
+//       columns contiguous, as in memory) and each lane gathers the eight k values of its column with 16-bit LDS
+//       reads.  The next tile's global loads are in flight while the current one is multiplied.
+//   pw_dw_kernel       dW[m][n] = sum_{s,l} dY[s][m][l] X[s][n][l]
+//       both operands are contiguous along the contraction index l; a block owns a 128 x 128 tile of dW for a chunk
+//       of samples and writes its partial tile, dw_reduce_kernel adds the chunks in a fixed order.
+// Blocks that share operand tiles are numbered so that they run on the same XCD (one L2 each, blocks are dealt
+// round-robin over the eight XCDs).
+#include "sjhip_common.h"
+
+namespace sjhip {
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kPwThreads = 256;
+constexpr int kTile = 128;            // rows and columns of a block's output tile
+constexpr int kTileK = 32;            // contraction elements per LDS stage (two MFMA k steps of 16)
+constexpr int kRowBytes = 80;         // K-contiguous operand row in LDS: 32 bf16 + 16 bytes, so that the 16-byte fragment
+                                      // reads of eight consecutive rows fall on all 32 banks
+constexpr int kRowPlane = kTile * kRowBytes;
+constexpr int kColRowBytes = 264;     // column-contiguous operand: one k row of 128 bf16 + 8 bytes (rows k and k + 8,
+                                      // read by the two halves of a wavefront, then fall on different banks)
+constexpr int kColPlane = kTileK * kColRowBytes;
+constexpr int kXcds = 8;
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  bf16x2 p;
+  p.x = (__bf16)lo;
+  p.y = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, p);
+}
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+
+// Word t holds term t of (x0, x1): term 0 is the value rounded to bf16, term 1 the rounded remainder, term 2 what is
+// left (exact for fp32 inputs: 3 x 8 significant bits).  The remainders are exact differences.
+template <int TERMS> __device__ __forceinline__ void split_pair(float x0, float x1, uint32_t (&w)[TERMS]) {
+#pragma unroll
+  for (int t = 0; t < TERMS; ++t) {
+    w[t] = pack_bf16(x0, x1);
+    if (t + 1 < TERMS) {
+      x0 -= bf16_lo(w[t]);
+      x1 -= bf16_hi(w[t]);
+    }
+  }
+}
+
+// Block number -> position in the order in which blocks that share tiles should be resident together: hardware block b
+// runs on XCD b % 8, so XCD x gets the contiguous range of logical blocks it would get if the grid were cut in eight.
+__device__ __forceinline__ int64_t xcd_order(int64_t b, int64_t n) {
+  const int64_t q = n / kXcds, r = n % kXcds, x = b % kXcds, i = b / kXcds;
+  return x * q + (x < r ? x : r) + i;
+}
+
+// planes[t][r][c] = term t of src[r * ld_r + c * ld_c] for r < rows, c < cols, zero in the padding
+__global__ void __launch_bounds__(256) split_weight_kernel(const float *src, int64_t rows, int64_t cols, int64_t ld_r,
+                                                            int64_t ld_c, int64_t rows_pad, int64_t cols_pad,
+                                                            uint16_t *planes) {
+  const int64_t pairs = rows_pad * (cols_pad / 2);
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= pairs) return;
+  const int64_t r = i / (cols_pad / 2), c = 2 * (i % (cols_pad / 2));
+  float x0 = 0.0f, x1 = 0.0f;
+  if (r < rows) {
+    if (c < cols) x0 = src[r * ld_r + c * ld_c];
+    if (c + 1 < cols) x1 = src[r * ld_r + (c + 1) * ld_c];
+  }
+  uint32_t w[3];
+  split_pair<3>(x0, x1, w);
+#pragma unroll
+  for (int t = 0; t < 3; ++t)
+    reinterpret_cast<uint32_t *>(planes + (int64_t)t * rows_pad * cols_pad)[(r * cols_pad + c) / 2] = w[t];
+}
+
+struct PwGemmArgs {
+  const uint16_t *a_planes;  // [3][M_pad][K_pad] bf16
+  const float *b;            // [S][K][L]
+  float *c;                  // [S][M][L]
+  int64_t plane_stride;      // M_pad * K_pad
+  int64_t ncols;             // S * L
+  int M, K, K_pad, L;
+  int m_blocks;
+};
+
+// Term pairs whose product is kept: combined order at most max(TA, TB) - 1.
+template <int TA, int TB> struct Pairs {
+  static constexpr int kMax = (TA > TB ? TA : TB) - 1;
+  static __device__ __forceinline__ constexpr bool keep(int ta, int tb) { return ta + tb <= kMax; }
+};
+
+// One k step of 16 for a wavefront's 2 x 2 tiles: operands in registers, smallest terms first.
+template <int TA, int TB>
+__device__ __forceinline__ void mfma_step(const bf16x8 (&af)[2][TA], const bf16x8 (&bf)[2][TB], f32x16 (&acc)[2][2]) {
+#pragma unroll
+  for (int order = Pairs<TA, TB>::kMax; order >= 0; --order) {
+#pragma unroll
+    for (int ta = 0; ta < TA; ++ta) {
+      const int tb = order - ta;
+      if (tb < 0 || tb >= TB) continue;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mt][ta], bf[nt][tb], acc[mt][nt], 0, 0, 0);
+    }
+  }
+}
+
+// Fragment of a K-contiguous operand: row `row` of the tile, k group (lane / 32) of k step ks.
+__device__ __forceinline__ bf16x8 row_fragment(const uint8_t *plane, int row, int ks, int lane) {
+  return *reinterpret_cast<const bf16x8 *>(plane + row * kRowBytes + ks * 32 + (lane >> 5) * 16);
+}
+
+template <int TA, int TB>
+__global__ void __launch_bounds__(kPwThreads) pw_gemm_kernel(const PwGemmArgs a) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  uint8_t *As = lds;                   // [TA][128][kRowBytes]
+  uint8_t *Bs = lds + TA * kRowPlane;  // [TB][32][kColRowBytes]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t logical = xcd_order(blockIdx.x, gridDim.x);
+  const int mb = (int)(logical % a.m_blocks);
+  const int64_t nb = logical / a.m_blocks;
+  const int m0 = mb * kTile;
+  const int64_t j0 = nb * kTile;
+  const int M = a.M, K = a.K, L = a.L;
+
+  // A: two 16-byte chunks per term and thread; chunk q = tid + 256 i -> row q / 4, k chunk q % 4
+  const uint16_t *a_src[2];
+  int a_dst[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int q = tid + kPwThreads * i, row = q >> 2, kc = q & 3;
+    a_src[i] = a.a_planes + (int64_t)(m0 + row) * a.K_pad + 8 * kc;
+    a_dst[i] = row * kRowBytes + kc * 16;
+  }
+  // B: four quads (one k row each, rows kr, kr + 8, kr + 16, kr + 24) of the same four columns
+  const int c4 = tid & 31, kr = tid >> 5;
+  const int64_t jq = j0 + 4 * c4;
+  const bool col_ok = jq < a.ncols;  // L % 4 == 0, so a quad is inside one sample and all of it is valid or none
+  const float *b_src = nullptr;
+  if (col_ok) {
+    const int64_t s = jq / L;
+    const int l = (int)(jq - s * L);
+    b_src = a.b + (s * K) * (int64_t)L + l;
+  }
+
+  u32x4 ra[TA][2];
+  f32x4 rb[4];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int t = 0; t < TA; ++t)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        ra[t][i] = *reinterpret_cast<const u32x4 *>(a_src[i] + (int64_t)t * a.plane_stride + k0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + kr + 8 * i;
+      rb[i] = (col_ok && k < K) ? *reinterpret_cast<const f32x4 *>(b_src + (int64_t)k * L) : (f32x4)(0.0f);
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int t = 0; t < TA; ++t)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4 *>(As + t * kRowPlane + a_dst[i]) = ra[t][i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint32_t w01[TB], w23[TB];
+      split_pair<TB>(rb[i].x, rb[i].y, w01);
+      split_pair<TB>(rb[i].z, rb[i].w, w23);
+#pragma unroll
+      for (int t = 0; t < TB; ++t) {
+        u32x2 w;
+        w.x = w01[t];
+        w.y = w23[t];
+        *reinterpret_cast<u32x2 *>(Bs + t * kColPlane + (kr + 8 * i) * kColRowBytes + c4 * 8) = w;
+      }
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.0f;
+
+  fetch(0);
+  for (int k0 = 0; k0 < a.K_pad; k0 += kTileK) {
+    __syncthreads();  // the previous tile has been read by every wavefront
+    stage();
+    __syncthreads();
+    if (k0 + kTileK < a.K_pad) fetch(k0 + kTileK);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      bf16x8 af[2][TA], bf[2][TB];
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int t = 0; t < TA; ++t) af[mt][t] = row_fragment(As + t * kRowPlane, wm * 64 + mt * 32 + (lane & 31), ks, lane);
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int t = 0; t < TB; ++t) {
+          const uint8_t *p = Bs + t * kColPlane + (ks * 16 + 8 * (lane >> 5)) * kColRowBytes +
+                             (wn * 64 + nt * 32 + (lane & 31)) * 2;
+          uint16_t e[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) e[i] = *reinterpret_cast<const uint16_t *>(p + i * kColRowBytes);
+          u32x4 w;
+          w.x = e[0] | ((uint32_t)e[1] << 16);
+          w.y = e[2] | ((uint32_t)e[3] << 16);
+          w.z = e[4] | ((uint32_t)e[5] << 16);
+          w.w = e[6] | ((uint32_t)e[7] << 16);
+          bf[nt][t] = __builtin_bit_cast(bf16x8, w);
+        }
+      mfma_step<TA, TB>(af, bf, acc);
+    }
+  }
+
+  // accumulator register r of a 32 x 32 tile: row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    const int64_t j = j0 + wn * 64 + nt * 32 + (lane & 31);
+    if (j >= a.ncols) continue;
+    const int64_t s = j / L;
+    const int l = (int)(j - s * L);
+    float *cp = a.c + (s * M) * (int64_t)L + l;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const int rbase = m0 + wm * 64 + mt * 32 + 4 * (lane >> 5);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = rbase + 8 * (r >> 2) + (r & 3);
+        if (row < M) cp[(int64_t)row * L] = acc[mt][nt][r];
+      }
+    }
+  }
+}
+
+struct PwDwArgs {
+  const float *dy;   // [S][M][L]
+  const float *x;    // [S][N][L]
+  float *partials;   // [chunks][M][N]
+  int64_t S;
+  int M, N, L;
+  int s_per_chunk;
+  int m_blocks, n_blocks;
+};
+
+template <int TA, int TB>
+__global__ void __launch_bounds__(kPwThreads) pw_dw_kernel(const PwDwArgs a) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  uint8_t *As = lds;                   // [TA][128][kRowBytes]
+  uint8_t *Bs = lds + TA * kRowPlane;  // [TB][128][kRowBytes]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t logical = xcd_order(blockIdx.x, gridDim.x);
+  const int tiles = a.m_blocks * a.n_blocks;
+  const int chunk = (int)(logical / tiles);
+  const int tile = (int)(logical % tiles);
+  const int mb = tile % a.m_blocks, nb = tile / a.m_blocks;
+  const int m0 = mb * kTile, n0 = nb * kTile;
+  const int M = a.M, N = a.N, L = a.L;
+  const int64_t s_begin = (int64_t)chunk * a.s_per_chunk;
+  const int64_t s_end = s_begin + a.s_per_chunk < a.S ? s_begin + a.s_per_chunk : a.S;
+  const int l_steps = (L + kTileK - 1) / kTileK;
+  const int64_t iters = (s_end - s_begin) * l_steps;
+
+  // a thread fetches quad q4 (four consecutive l) of rows rr, rr + 32, rr + 64, rr + 96 of both operand tiles
+  const int q4 = tid & 7, rr = tid >> 3;
+  f32x4 ra[4], rb[4];
+  auto fetch = [&](int64_t it) {
+    const int64_t s = s_begin + it / l_steps;
+    const int l = (int)(it % l_steps) * kTileK + 4 * q4;
+    const bool l_ok = l < L;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = rr + 32 * i;
+      ra[i] = (l_ok && m0 + row < M) ? *reinterpret_cast<const f32x4 *>(a.dy + ((s * M + m0 + row) * (int64_t)L + l))
+                                     : (f32x4)(0.0f);
+      rb[i] = (l_ok && n0 + row < N) ? *reinterpret_cast<const f32x4 *>(a.x + ((s * N + n0 + row) * (int64_t)L + l))
+                                     : (f32x4)(0.0f);
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int off = (rr + 32 * i) * kRowBytes + q4 * 8;
+      {
+        uint32_t w01[TA], w23[TA];
+        split_pair<TA>(ra[i].x, ra[i].y, w01);
+        split_pair<TA>(ra[i].z, ra[i].w, w23);
+#pragma unroll
+        for (int t = 0; t < TA; ++t) {
+          u32x2 w;
+          w.x = w01[t];
+          w.y = w23[t];
+          *reinterpret_cast<u32x2 *>(As + t * kRowPlane + off) = w;
+        }
+      }
+      {
+        uint32_t w01[TB], w23[TB];
+        split_pair<TB>(rb[i].x, rb[i].y, w01);
+        split_pair<TB>(rb[i].z, rb[i].w, w23);
+#pragma unroll
+        for (int t = 0; t < TB; ++t) {
+          u32x2 w;
+          w.x = w01[t];
+          w.y = w23[t];
+          *reinterpret_cast<u32x2 *>(Bs + t * kRowPlane + off) = w;
+        }
+      }
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.0f;
+
+  if (iters > 0) fetch(0);
+  for (int64_t it = 0; it < iters; ++it) {
+    __syncthreads();
+    stage();
+    __syncthreads();
+    const int l0 = (int)(it % l_steps) * kTileK;
+    if (it + 1 < iters) fetch(it + 1);
+    const int ksteps = (l0 + 16 < L) ? 2 : 1;  // the second half of the last stage of a row may hold nothing
+    for (int ks = 0; ks < ksteps; ++ks) {
+      bf16x8 af[2][TA], bf[2][TB];
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int t = 0; t < TA; ++t) af[mt][t] = row_fragment(As + t * kRowPlane, wm * 64 + mt * 32 + (lane & 31), ks, lane);
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int t = 0; t < TB; ++t) bf[nt][t] = row_fragment(Bs + t * kRowPlane, wn * 64 + nt * 32 + (lane & 31), ks, lane);
+      mfma_step<TA, TB>(af, bf, acc);
+    }
+  }
+
+  float *out = a.partials + (int64_t)chunk * M * N;
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    const int col = n0 + wn * 64 + nt * 32 + (lane & 31);
+    if (col >= N) continue;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const int rbase = m0 + wm * 64 + mt * 32 + 4 * (lane >> 5);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = rbase + 8 * (r >> 2) + (r & 3);
+        if (row < M) out[(int64_t)row * N + col] = acc[mt][nt][r];
+      }
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) dw_reduce_kernel(const float *partials, int chunks, int64_t count, float *out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float sum = 0.0f;
+  for (int c = 0; c < chunks; ++c) sum += partials[(int64_t)c * count + i];
+  out[i] = sum;
+}
+
+int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+
+template <int TA, int TB> int launch_gemm_terms(const PwGemmArgs &a, int64_t blocks, hipStream_t stream) {
+  const unsigned lds = TA * kRowPlane + TB * kColPlane;
+  hipLaunchKernelGGL((pw_gemm_kernel<TA, TB>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
+  return check_launch("pwconv_gemm");
+}
+
+template <int TA, int TB> int launch_dw_terms(const PwDwArgs &a, int64_t blocks, hipStream_t stream) {
+  const unsigned lds = (TA + TB) * kRowPlane;
+  hipLaunchKernelGGL((pw_dw_kernel<TA, TB>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
+  return check_launch("pwconv_grad_weight");
+}
+
+// Samples per partial tile of dW: enough chunks to fill the chip a few times over, few enough to keep the partials small.
+int dw_samples_per_chunk(int64_t S, int tiles) {
+  int64_t chunks = (4 * 256 + tiles - 1) / tiles;
+  if (chunks < 1) chunks = 1;
+  if (chunks > S) chunks = S;
+  return (int)((S + chunks - 1) / chunks);
+}
+
+}  // namespace
+
+int64_t pwconv_planes_elems(int64_t rows, int64_t cols) { return 3 * round_up(rows, kTile) * round_up(cols, kTileK); }
+
+int launch_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes,
+                               hipStream_t stream) {
+  // planes hold the matrix A of a later GEMM, K-contiguous: A = W ([rows][cols]) or A = W^T ([cols][rows])
+  const int64_t ar = transpose ? cols : rows, ac = transpose ? rows : cols;
+  const int64_t rows_pad = round_up(ar, kTile), cols_pad = round_up(ac, kTileK);
+  const int64_t pairs = rows_pad * (cols_pad / 2);
+  const int64_t blocks = (pairs + 255) / 256;
+  if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_split_weight: %lld x %lld", (long long)rows, (long long)cols);
+  hipLaunchKernelGGL(split_weight_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, w, ar, ac,
+                     transpose ? (int64_t)1 : cols, transpose ? cols : (int64_t)1, rows_pad, cols_pad, planes);
+  return check_launch("pwconv_split_weight");
+}
+
+int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,
+                       int64_t L, float *c, hipStream_t stream) {
+  if (L % 4 != 0 || !aligned16(b) || !aligned16(a_planes))
+    return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: L=%lld must be a multiple of 4 and the tensors 16-byte aligned", (long long)L);
+  if (M > (1 << 24) || K > (1 << 24) || L > (1 << 24)) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: M=%lld K=%lld L=%lld", (long long)M, (long long)K, (long long)L);
+  PwGemmArgs a;
+  a.a_planes = a_planes; a.b = b; a.c = c;
+  a.M = (int)M; a.K = (int)K; a.K_pad = (int)round_up(K, kTileK); a.L = (int)L;
+  a.plane_stride = round_up(M, kTile) * a.K_pad;
+  a.ncols = S * L;
+  a.m_blocks = (int)(round_up(M, kTile) / kTile);
+  const int64_t blocks = a.m_blocks * ((a.ncols + kTile - 1) / kTile);
+  if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: %lld blocks", (long long)blocks);
+  ProfileScope prof(KC_PW_GEMM, stream);
+  const int key = a_terms * 10 + b_terms;
+  switch (key) {
+    case 33: return launch_gemm_terms<3, 3>(a, blocks, stream);
+    case 31: return launch_gemm_terms<3, 1>(a, blocks, stream);
+    case 22: return launch_gemm_terms<2, 2>(a, blocks, stream);
+    case 21: return launch_gemm_terms<2, 1>(a, blocks, stream);
+    case 11: return launch_gemm_terms<1, 1>(a, blocks, stream);
+    default: return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: %d weight terms with %d activation terms (3/3, 3/1, 2/2, 2/1, 1/1)", a_terms, b_terms);
+  }
+}
+
+int64_t pwconv_dw_workspace_floats(int64_t M, int64_t N, int64_t S) {
+  const int tiles = (int)(round_up(M, kTile) / kTile * (round_up(N, kTile) / kTile));
+  const int spc = dw_samples_per_chunk(S, tiles);
+  return (S + spc - 1) / spc * M * N;
+}
+
+int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int x_terms, int64_t S, int64_t M, int64_t N,
+                              int64_t L, float *dw, float *workspace, hipStream_t stream) {
+  if (L % 4 != 0 || !aligned16(dy) || !aligned16(x))
+    return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight: L=%lld must be a multiple of 4 and the tensors 16-byte aligned", (long long)L);
+  if (M > (1 << 24) || N > (1 << 24) || L > (1 << 24)) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_grad_weight: M=%lld N=%lld L=%lld", (long long)M, (long long)N, (long long)L);
+  PwDwArgs a;
+  a.dy = dy; a.x = x; a.partials = workspace; a.S = S;
+  a.M = (int)M; a.N = (int)N; a.L = (int)L;
+  a.m_blocks = (int)(round_up(M, kTile) / kTile);
+  a.n_blocks = (int)(round_up(N, kTile) / kTile);
+  const int tiles = a.m_blocks * a.n_blocks;
+  a.s_per_chunk = dw_samples_per_chunk(S, tiles);
+  const int chunks = (int)((S + a.s_per_chunk - 1) / a.s_per_chunk);
+  const int64_t blocks = (int64_t)tiles * chunks;
+  int rc;
+  {
+    ProfileScope prof(KC_PW_GRAD_WEIGHT, stream);
+    const int key = dy_terms * 10 + x_terms;
+    switch (key) {
+      case 33: rc = launch_dw_terms<3, 3>(a, blocks, stream); break;
+      case 31: rc = launch_dw_terms<3, 1>(a, blocks, stream); break;
+      case 22: rc = launch_dw_terms<2, 2>(a, blocks, stream); break;
+      case 21: rc = launch_dw_terms<2, 1>(a, blocks, stream); break;
+      case 11: rc = launch_dw_terms<1, 1>(a, blocks, stream); break;
+      default: return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight: %d gradient terms with %d activation terms (3/3, 3/1, 2/2, 2/1, 1/1)", dy_terms, x_terms);
+    }
+    if (rc != SJHIP_OK) return rc;
+    const int64_t count = M * N;
+    hipLaunchKernelGGL(dw_reduce_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, workspace, chunks, count, dw);
+    rc = check_launch("pwconv_grad_weight(reduce)");
+  }
+  return rc;
+}
+
+}  // namespace sjhip

@@ -482,6 +482,83 @@ int sjhip_ssa_backward(int dtype, int64_t samples, int heads, int channels_per_h
                     static_cast<hipStream_t>(stream));
 }
 
+int64_t sjhip_pwconv_planes_elems(int64_t rows, int64_t cols) {
+  if (rows < 1 || cols < 1) return 0;
+  return pwconv_planes_elems(rows, cols);
+}
+
+int sjhip_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, void *stream) {
+  if (!w || !planes) return fail(SJHIP_ERR_INVALID, "pwconv_split_weight: NULL buffer");
+  if (rows < 1 || cols < 1) return fail(SJHIP_ERR_INVALID, "pwconv_split_weight: %lld x %lld", (long long)rows, (long long)cols);
+  return launch_pwconv_split_weight(w, rows, cols, transpose, planes, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,
+                      int64_t L, float *c, void *stream) {
+  if (!a_planes || !b || !c) return fail(SJHIP_ERR_INVALID, "pwconv_gemm: NULL buffer");
+  if (M < 1 || K < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_gemm: M=%lld K=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)K, (long long)S, (long long)L);
+  if (S > (int64_t(1) << 40) / L) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: S*L overflows");
+  return launch_pwconv_gemm(a_planes, a_terms, M, K, b, b_terms, S, L, c, static_cast<hipStream_t>(stream));
+}
+
+int64_t sjhip_pwconv_grad_weight_workspace_floats(int64_t M, int64_t N, int64_t S) {
+  if (M < 1 || N < 1 || S < 1) return 0;
+  return pwconv_dw_workspace_floats(M, N, S);
+}
+
+int sjhip_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int x_terms, int64_t S, int64_t M, int64_t N,
+                             int64_t L, float *dw, float *workspace, void *stream) {
+  if (!dy || !x || !dw || !workspace) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight: NULL buffer");
+  if (M < 1 || N < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight: M=%lld N=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)N, (long long)S, (long long)L);
+  return launch_pwconv_grad_weight(dy, dy_terms, x, x_terms, S, M, N, L, dw, workspace, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, void *stream) {
+  if (!y || !partial) return fail(SJHIP_ERR_INVALID, "bn_stats: NULL buffer");
+  return launch_bn_stats(y, S, C, L, partial, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_bn_finalize(const float *partial, int64_t S, int64_t C, int64_t L, const float *gamma, const float *beta, float eps,
+                      float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
+                      float *invstd, void *stream) {
+  if (!scale || !shift || !mean || !invstd) return fail(SJHIP_ERR_INVALID, "bn_finalize: NULL output");
+  if (partial && (S < 1 || L < 1)) return fail(SJHIP_ERR_INVALID, "bn_finalize: S=%lld L=%lld", (long long)S, (long long)L);
+  return launch_bn_finalize(partial, S, C, L, gamma, beta, eps, momentum, running_mean, running_var, scale, shift, mean, invstd,
+                            static_cast<hipStream_t>(stream));
+}
+
+int sjhip_bn_lif_forward(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
+                         const float *scale, const float *shift, const float *v_init, float *spike_seq, uint8_t *spike_bits,
+                         float *v_last, void *stream) {
+  if (!p) return fail(SJHIP_ERR_INVALID, "bn_lif_forward: params is NULL");
+  if (!y || !scale || !shift || !v_init) return fail(SJHIP_ERR_INVALID, "bn_lif_forward: NULL tensor");
+  if ((spike_seq == nullptr) == (spike_bits == nullptr)) return fail(SJHIP_ERR_INVALID, "bn_lif_forward: exactly one of spike_seq and spike_bits");
+  return launch_bn_lif_forward(neuron, *p, T, B, C, L, y, scale, shift, v_init, spike_seq, spike_bits, v_last,
+                               static_cast<hipStream_t>(stream));
+}
+
+int sjhip_bn_lif_backward(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
+                          const float *scale, const float *shift, const float *v_init, const float *grad_spike_seq,
+                          const float *grad_v_last, float *grad_z, float *grad_v_init, float *partial, void *stream) {
+  if (!p) return fail(SJHIP_ERR_INVALID, "bn_lif_backward: params is NULL");
+  if (!y || !scale || !shift || !v_init || !grad_spike_seq || !grad_z || !partial) return fail(SJHIP_ERR_INVALID, "bn_lif_backward: NULL tensor");
+  return launch_bn_lif_backward(neuron, *p, T, B, C, L, y, scale, shift, v_init, grad_spike_seq, grad_v_last, grad_z, grad_v_init,
+                                partial, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64_t C, int64_t L, int training, const float *gamma,
+                               const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef, void *stream) {
+  if (!partial || !mean || !invstd || !coef) return fail(SJHIP_ERR_INVALID, "bn_backward_finalize: NULL buffer");
+  if (T < 1 || B < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "bn_backward_finalize: T=%lld B=%lld L=%lld", (long long)T, (long long)B, (long long)L);
+  return launch_bn_backward_finalize(partial, T, B, C, L, training, gamma, mean, invstd, dgamma, dbeta, coef,
+                                     static_cast<hipStream_t>(stream));
+}
+
+int sjhip_bn_grad_input(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy, void *stream) {
+  if (!g || !y || !coef || !dy) return fail(SJHIP_ERR_INVALID, "bn_grad_input: NULL buffer");
+  return launch_bn_grad_input(g, y, coef, S, C, L, dy, static_cast<hipStream_t>(stream));
+}
+
 int sjhip_set_tuning(const char *key, int value) {
   if (!key) return fail(SJHIP_ERR_INVALID, "set_tuning: NULL key");
   const bool block_ok = (value == 64 || value == 128 || value == 256 || value == 512) && value <= SJHIP_MAX_BLOCK;

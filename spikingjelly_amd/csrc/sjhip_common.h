@@ -262,7 +262,8 @@ unsigned occupancy_cap_lds(int blocks_per_cu);
 const Tuning &tuning();
 
 enum KernelClass { KC_FORWARD = 0, KC_BACKWARD = 1, KC_PLIF_REDUCE = 2, KC_BIT_PACK = 3, KC_BIT_UNPACK = 4,
-                   KC_SSA_FORWARD = 5, KC_SSA_BACKWARD = 6, KC_COUNT = 7 };
+                   KC_SSA_FORWARD = 5, KC_SSA_BACKWARD = 6, KC_PW_GEMM = 7, KC_PW_GRAD_WEIGHT = 8, KC_BN_STATS = 9,
+                   KC_BN_LIF_FORWARD = 10, KC_BN_LIF_BACKWARD = 11, KC_BN_GRAD_INPUT = 12, KC_COUNT = 13 };
 
 // Brackets one launch with events when profiling is on; free otherwise.
 class ProfileScope {
@@ -339,5 +340,27 @@ int launch_ssa(bool backward, int dtype, int64_t samples, int heads, int cph, in
                const uint8_t *qkv_bits, const void *grad_out, void *out, void *grad_qkv, hipStream_t stream);
 int launch_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, hipStream_t stream);
 int launch_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, hipStream_t stream);
+int64_t pwconv_planes_elems(int64_t rows, int64_t cols);
+int launch_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, hipStream_t stream);
+int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,
+                       int64_t L, float *c, hipStream_t stream);
+int64_t pwconv_dw_workspace_floats(int64_t M, int64_t N, int64_t S);
+int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int x_terms, int64_t S, int64_t M, int64_t N,
+                              int64_t L, float *dw, float *workspace, hipStream_t stream);
+int launch_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, hipStream_t stream);
+int launch_bn_finalize(const float *partial, int64_t S, int64_t C, int64_t L, const float *gamma, const float *beta, float eps,
+                       float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
+                       float *invstd, hipStream_t stream);
+int launch_bn_lif_forward(int neuron, const sjhip_neuron_params &p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
+                          const float *scale, const float *shift, const float *v_init, float *spike_seq, uint8_t *spike_bits,
+                          float *v_last, hipStream_t stream);
+int launch_bn_lif_backward(int neuron, const sjhip_neuron_params &p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
+                           const float *scale, const float *shift, const float *v_init, const float *grad_spike_seq,
+                           const float *grad_v_last, float *grad_z, float *grad_v_init, float *partial, hipStream_t stream);
+int launch_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64_t C, int64_t L, int training, const float *gamma,
+                                const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef,
+                                hipStream_t stream);
+int launch_bn_grad_input(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy,
+                         hipStream_t stream);
 
 }  // namespace sjhip

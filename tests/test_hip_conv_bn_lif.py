@@ -1,0 +1,301 @@
+"""Fused kernel-size-1 convolution / batch norm / LIF kernels against the float64 oracle
+(``oracle/conv_bn_lif_oracle.py``, pinned on the CPU against torch's ``nn.Conv1d`` / ``nn.BatchNorm1d`` and this
+package's torch-backend block).
+
+Bars.  GEMMs with three bf16 terms per fp32 operand: 2e-6 of the row's sum of |products| (an fp32 GEMM's own bound is
+K * 6e-8 of it); exact on operands whose products and sums fp32 holds exactly.  Batch norm + LIF: spikes identical
+wherever the oracle's membrane potential is further than 1e-5 from the threshold (the test inputs are checked to hold
+no closer neuron, so all spikes are compared), running statistics and gradients within 1e-5 relative of float64.
+"""
+
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import conv_bn_lif_oracle as co
+from oracle import neuron_oracle as no
+from spikingjelly_amd import configure
+from spikingjelly_amd.activation_based import functional, layer, neuron, surrogate
+
+from helpers import seeded_randn
+
+pytestmark = pytest.mark.gpu
+
+MARGIN = 1e-5
+
+
+@pytest.fixture(scope="module")
+def C():
+    assert torch.cuda.is_available(), "GPU tests need a ROCm device"
+    from spikingjelly_amd.activation_based.hip_kernel import conv_bn_lif, library
+
+    library.load()
+    return conv_bn_lif
+
+
+# ------------------------------------------------------------------------------------------------
+# the three GEMMs
+# ------------------------------------------------------------------------------------------------
+SHAPES = [(3, 100, 50, 12), (2, 128, 32, 128), (5, 384, 384, 196), (1, 7, 3, 4), (4, 130, 257, 36), (16, 1152, 384, 196)]
+
+
+@pytest.mark.parametrize("S,M,Kd,Lp", SHAPES)
+@pytest.mark.parametrize("transpose", [False, True])
+def test_gemm_with_three_terms_has_fp32_accuracy(C, S, M, Kd, Lp, transpose):
+    w = seeded_randn((Kd, M) if transpose else (M, Kd), 11, 0.0, 1.0)
+    x = seeded_randn((S, Kd, Lp), 12, 0.1, 1.0)
+    planes = C.split_weight(w.cuda(), transpose)
+    got = C.pw_gemm(planes, 3, M, Kd, x.cuda(), 3).cpu().double()
+    a = (w.t() if transpose else w).double()
+    want = torch.einsum("mk,skl->sml", a, x.double())
+    bound = torch.einsum("mk,skl->sml", a.abs(), x.double().abs())
+    assert float(((got - want).abs() / bound).max()) < 2e-6
+    # and better than what two terms give
+    err3 = float((got - want).abs().max())
+    got2 = C.pw_gemm(planes, 2, M, Kd, x.cuda(), 2).cpu().double()
+    assert float(((got2 - want).abs() / bound).max()) < 3e-5
+    assert err3 <= float((got2 - want).abs().max())
+
+
+@pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (4, 384, 384, 196)])
+def test_gemm_is_exact_on_spikes_times_dyadic_weights(C, S, M, Kd, Lp):
+    g = torch.Generator().manual_seed(13)
+    w = torch.randint(-64, 65, (M, Kd), generator=g).float() / 64.0   # 7 significant bits: one bf16 term holds it
+    x = (torch.rand((S, Kd, Lp), generator=g) < 0.3).float()
+    want = torch.einsum("mk,skl->sml", w.double(), x.double()).float()   # sums of multiples of 1/64 below 2^24 / 64: exact
+    for wt, xt in ((3, 1), (2, 1), (1, 1), (3, 3)):
+        got = C.pw_gemm(C.split_weight(w.cuda(), False), wt, M, Kd, x.cuda(), xt).cpu()
+        assert torch.equal(got, want), (wt, xt)
+
+
+@pytest.mark.parametrize("S,M,N,Lp", [(3, 100, 50, 12), (9, 130, 257, 36), (16, 384, 384, 196), (2, 1152, 384, 196), (64, 64, 48, 8)])
+@pytest.mark.parametrize("spikes", [False, True])
+def test_grad_weight_gemm(C, S, M, N, Lp, spikes):
+    dy = seeded_randn((S, M, Lp), 21, 0.0, 1.0)
+    x = (seeded_randn((S, N, Lp), 22, 0.0, 1.0) > 0.5).float() if spikes else seeded_randn((S, N, Lp), 22, 0.2, 1.0)
+    got = C.pw_grad_weight(dy.cuda(), 3, x.cuda(), 1 if spikes else 3).cpu().double()
+    want = torch.einsum("sml,snl->mn", dy.double(), x.double())
+    bound = torch.einsum("sml,snl->mn", dy.double().abs(), x.double().abs()).clamp_min(1e-30)
+    assert float(((got - want).abs() / bound).max()) < 2e-6
+
+
+# ------------------------------------------------------------------------------------------------
+# batch norm + LIF
+# ------------------------------------------------------------------------------------------------
+def _no_borderline(h, v_th):
+    """No membrane potential within the margin of the threshold.  Exact ties are allowed: they occur in the attention
+    neuron, whose inputs are multiples of 1/8 and whose arithmetic is therefore exact in fp32 and float64 alike."""
+    d = (h - v_th).abs()
+    return bool(((d > MARGIN) | (d == 0)).all())
+
+
+@pytest.mark.parametrize("T,B,Cc,Lp", [(4, 3, 10, 12), (1, 2, 5, 4), (7, 2, 33, 20), (16, 2, 6, 260), (4, 2, 12, 196)])
+@pytest.mark.parametrize("training", [True, False])
+@pytest.mark.parametrize("v_reset,decay_input,tau,sg", [(0.0, True, 2.0, "sigmoid"), (None, False, 3.0, "atan"), (-0.2, True, 2.5, "erf")])
+def test_bn_lif_against_float64(C, T, B, Cc, Lp, training, v_reset, decay_input, tau, sg):
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+    from spikingjelly_amd.activation_based.hip_kernel import neuron_kernel as K
+
+    gamma, beta = seeded_randn((Cc,), 32, 1.0, 0.2), seeded_randn((Cc,), 33, 0.6, 0.3)
+    rm, rv = seeded_randn((Cc,), 34, 0.3, 0.2), seeded_randn((Cc,), 35, 2.0, 0.3).abs()
+    gs = seeded_randn((T, B, Cc, Lp), 36)
+    gl = seeded_randn((B, Cc, Lp), 37, 0.0, 0.3)
+    alpha = no.SG_DEFAULT_ALPHA[sg]
+    detach = v_reset is None
+    for seed in range(31, 3100, 100):  # the first input whose membrane potentials all keep the margin from the threshold
+        y = seeded_randn((T, B, Cc, Lp), seed, 0.4, 1.5)
+        y64 = y.double().requires_grad_()
+        g64, b64 = gamma.double().requires_grad_(), beta.double().requires_grad_()
+        z, rm64, rv64 = co.batch_norm(y64, g64, b64, rm.double(), rv.double(), training)
+        s64, v64, h64 = co.lif(z, torch.full((B, Cc, Lp), 0.0 if v_reset is None else v_reset, dtype=torch.float64), tau, 1.0,
+                               v_reset, detach, sg, alpha, decay_input)
+        if _no_borderline(h64.detach(), 1.0):
+            break
+    else:
+        pytest.fail("no input without a neuron within the margin of the threshold")
+    torch.autograd.backward([s64, v64[-1]], [gs.double(), gl.double()])
+
+    soft = v_reset is None
+    flags = K._flags(soft, detach, decay_input, 0)
+    spec = (tau, 1.0, 0.0 if soft else v_reset, flags, no.SG_IDS[sg], alpha)
+    yd = y.cuda().requires_grad_()
+    gd, bd = gamma.cuda().requires_grad_(), beta.cuda().requires_grad_()
+    rmd, rvd = rm.cuda(), rv.cuda()
+    v0 = torch.full((1,), 0.0 if soft else v_reset, device="cuda").expand(B, Cc, Lp)
+    spikes, v_last = C.bn_lif(yd, gd, bd, v0, (rmd, rvd, training, 0.1, 1e-5), spec)
+    torch.autograd.backward([spikes, v_last], [gs.cuda(), gl.cuda()])
+    assert torch.equal(spikes.detach().cpu().double(), s64.detach())
+    torch.testing.assert_close(v_last.detach().cpu().double(), v64[-1].detach(), rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(rmd.cpu().double(), rm64, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(rvd.cpu().double(), rv64, rtol=1e-6, atol=1e-6)
+    scale = float(y64.grad.abs().max())
+    torch.testing.assert_close(yd.grad.cpu().double(), y64.grad, rtol=1e-4, atol=1e-5 * scale)
+    torch.testing.assert_close(gd.grad.cpu().double(), g64.grad, rtol=1e-4, atol=1e-5 * float(g64.grad.abs().max()))
+    torch.testing.assert_close(bd.grad.cpu().double(), b64.grad, rtol=1e-4, atol=1e-5 * float(b64.grad.abs().max()))
+
+
+def test_bn_lif_bit_packed_spikes_equal_the_dense_ones(C):
+    from spikingjelly_amd.activation_based.hip_kernel import neuron_kernel as K
+    from spikingjelly_amd.activation_based.hip_kernel.compress import bit_spike_compress
+
+    T, B, Cc, Lp = 4, 3, 10, 196   # rows of 196 spikes start in the middle of a byte every other row
+    y = seeded_randn((T, B * 2, Cc, Lp), 41, 0.4, 1.5).cuda()
+    beta = torch.full((Cc,), 0.8, device="cuda")
+    bn_map = C._bn_map(y.flatten(0, 1), None, beta, None, None, True, 0.1, 1e-5)
+    spec = (2.0, 1.0, 0.0, K._flags(False, True, True, 0), 0, 4.0)
+    v0 = torch.zeros((B * 2, Cc, Lp), device="cuda")
+    dense, v_a = C._bn_lif_forward(y, bn_map, v0, spec, False)
+    bits, v_b = C._bn_lif_forward(y, bn_map, v0, spec, True)
+    assert torch.equal(bits, bit_spike_compress(dense)) and torch.equal(v_a, v_b)
+    assert 0.05 < float(dense.mean()) < 0.95
+
+
+# ------------------------------------------------------------------------------------------------
+# the whole chain and the attention block
+# ------------------------------------------------------------------------------------------------
+def _block_params(block):
+    params = {}
+    for name, seq in (("qkv", block.qkv_conv_bn), ("proj", block.proj_conv_bn)):
+        params[f"{name}_weight"] = seq[0].weight.detach()[:, :, 0].double().cpu().clone().requires_grad_()
+        params[f"{name}_gamma"] = seq[1].weight.detach().double().cpu().clone().requires_grad_()
+        params[f"{name}_beta"] = seq[1].bias.detach().double().cpu().clone().requires_grad_()
+        params[f"{name}_running_mean"] = seq[1].running_mean.double().cpu().clone()
+        params[f"{name}_running_var"] = seq[1].running_var.double().cpu().clone()
+    return params
+
+
+def _make_block(dim, heads, seed):
+    torch.manual_seed(seed)
+    block = layer.SpikingSelfAttention(dim, heads, backend="hip")
+    with torch.no_grad():
+        for bn in (block.qkv_conv_bn[1], block.proj_conv_bn[1]):
+            bn.running_mean.normal_(0.0, 0.1)
+            bn.running_var.uniform_(0.5, 1.5)
+            bn.weight.normal_(1.0, 0.2)
+            bn.bias.normal_(0.9, 0.3)
+    return block
+
+
+@pytest.mark.parametrize("dim,heads,T,B,tokens", [(16, 2, 3, 2, 8), (64, 2, 4, 2, 36), (48, 3, 4, 1, 196)])
+@pytest.mark.parametrize("training", [True, False])
+def test_attention_block_fused_against_float64(dim, heads, T, B, tokens, training):
+    block = _make_block(dim, heads, 50 + dim).cuda().train(training)
+    params = _block_params(block)
+    g = seeded_randn((T, B, dim, tokens), 52)
+    for seed in range(51, 5100, 100):  # the first input that keeps every neuron of the three layers off its threshold
+        x = seeded_randn((T, B, dim, tokens), seed, 0.0, 2.0)
+        x64 = x.double().requires_grad_()
+        ref = co.attention_block(x64, params, heads, training)
+        if all(_no_borderline(h.detach(), v_th) for h, v_th in ((ref["qkv_h"], 1.0), (ref["attn_h"], 0.5), (ref["proj_h"], 1.0))):
+            break
+    else:
+        pytest.fail("no input without a neuron within the margin of a threshold")
+    ref["out"].backward(g.double())
+
+    xd = x.cuda().requires_grad_()
+    out = block(xd)
+    out.backward(g.cuda())
+    assert torch.equal(out.detach().cpu().double(), ref["out"].detach())
+    assert 0.02 < float(out.detach().mean()) < 0.9
+    assert block.qkv_lif.v.shape == (B, 3 * dim, tokens) and block.proj_lif.v.shape == (B, dim, tokens)
+
+    def close(a, b, what):
+        scale = float(b.abs().max())
+        torch.testing.assert_close(a.cpu().double(), b, rtol=1e-4, atol=2e-5 * scale, msg=lambda m: f"{what}: {m}")
+
+    close(xd.grad, x64.grad, "grad x")
+    for name, seq in (("qkv", block.qkv_conv_bn), ("proj", block.proj_conv_bn)):
+        close(seq[0].weight.grad[:, :, 0], params[f"{name}_weight"].grad, name + " weight")
+        close(seq[1].weight.grad, params[f"{name}_gamma"].grad, name + " gamma")
+        close(seq[1].bias.grad, params[f"{name}_beta"].grad, name + " beta")
+        if training:
+            torch.testing.assert_close(seq[1].running_mean.cpu().double(), ref[f"{name}_running"][0], rtol=1e-5, atol=1e-6)
+            torch.testing.assert_close(seq[1].running_var.cpu().double(), ref[f"{name}_running"][1], rtol=1e-5, atol=1e-6)
+            assert int(seq[1].num_batches_tracked) == 1
+
+
+def test_attention_block_fused_equals_unfused_path(monkeypatch):
+    """The same module with the fusion switched off (torch's convolution and batch norm around the hip neurons)."""
+    from spikingjelly_amd.activation_based.layer import fused
+
+    block = _make_block(64, 2, 60).cuda().train()
+    x = seeded_randn((4, 2, 64, 36), 61, 0.0, 2.0).cuda()
+    calls = []
+    real = fused.conv_bn_lif
+    monkeypatch.setattr(fused, "conv_bn_lif", lambda *a, **k: calls.append(1) or real(*a, **k))
+    a = block(x)
+    assert len(calls) == 2
+    functional.reset_net(block)
+    monkeypatch.setattr(fused, "conv_bn_lif", lambda *a, **k: None)
+    b = block(x)
+    assert float((a != b).float().mean()) < 1e-3   # fp32 convolutions of two libraries: a spike in a thousand may flip
+
+
+def test_eval_mode_spikes_are_bit_identical_to_the_torch_backend_on_exact_inputs():
+    """Binary input, weights that are multiples of 1/64, batch norm in evaluation mode with an exactly representable map
+    (running variance + eps exactly 1, gamma and beta multiples of 1/8): every convolution sum and every normalised value is
+    exact in fp32 in any order, so the hip block must fire exactly the spikes of the torch-backend block on the CPU."""
+    torch.manual_seed(70)
+    dim, heads, T, B, tokens = 64, 2, 4, 2, 36
+    ref = layer.SpikingSelfAttention(dim, heads, backend="torch")
+    g = torch.Generator().manual_seed(71)
+    with torch.no_grad():
+        for seq in (ref.qkv_conv_bn, ref.proj_conv_bn):
+            seq[0].weight.copy_(torch.randint(-16, 17, seq[0].weight.shape, generator=g).float() / 64.0)
+            seq[1].eps = 2.0 ** -10
+            seq[1].running_var.fill_(1.0 - 2.0 ** -10)   # variance + eps is exactly 1
+            seq[1].running_mean.copy_(torch.randint(-4, 5, (seq[1].num_features,), generator=g).float() / 8.0)
+            seq[1].weight.copy_(torch.randint(4, 13, (seq[1].num_features,), generator=g).float() / 8.0)
+            seq[1].bias.copy_(torch.randint(0, 9, (seq[1].num_features,), generator=g).float() / 8.0)
+    ref.eval()
+    hip = layer.SpikingSelfAttention(dim, heads, backend="hip")
+    hip.load_state_dict(ref.state_dict())
+    for a, b in ((hip.qkv_conv_bn, ref.qkv_conv_bn), (hip.proj_conv_bn, ref.proj_conv_bn)):
+        a[1].eps = b[1].eps
+    hip = hip.cuda().eval()
+    x = (torch.rand((T, B, dim, tokens), generator=g) < 0.4).float()
+    with torch.no_grad():
+        want = ref(x)
+        got = hip(x.cuda())
+    assert torch.equal(got.cpu(), want)
+    assert 0.02 < float(want.mean()) < 0.9
+
+
+def test_pointwise_conv2d_bn_lif_module():
+    from spikingjelly_amd.activation_based.model import spikformer
+
+    torch.manual_seed(80)
+    m = spikformer.SpikformerConv2dBNLIF(12, 20, kernel_size=1, backend="hip").cuda().train()
+    x = seeded_randn((4, 2, 12, 6, 6), 81, 0.0, 2.0)
+    ref = co.conv_bn_lif(x.double().flatten(3), m.conv_bn.block[0].weight.detach().double().cpu()[:, :, 0, 0],
+                         m.conv_bn.block[1].weight.detach().double().cpu(), m.conv_bn.block[1].bias.detach().double().cpu(),
+                         torch.zeros(20, dtype=torch.float64), torch.ones(20, dtype=torch.float64), True,
+                         torch.zeros((2, 20, 36), dtype=torch.float64))
+    assert _no_borderline(ref["h_seq"], 1.0)
+    out = m(x.cuda())
+    assert out.shape == (4, 2, 20, 6, 6)
+    assert torch.equal(out.cpu().double().flatten(3), ref["spike_seq"])
+
+
+@pytest.mark.parametrize("pool", [False, True])
+def test_conv2d_3x3_bn_lif_module_against_float64_torch_modules(pool):
+    """A 3x3 convolution stays with torch; batch norm and the neuron run fused when nothing sits between them."""
+    from spikingjelly_amd.activation_based.model import spikformer
+
+    torch.manual_seed(90)
+    m = spikformer.SpikformerConv2dBNLIF(6, 8, kernel_size=3, stride=1, padding=1, pool=pool, backend="hip")
+    ref = spikformer.SpikformerConv2dBNLIF(6, 8, kernel_size=3, stride=1, padding=1, pool=pool, backend="torch").double()
+    ref.load_state_dict({k: v.double() if v.is_floating_point() else v for k, v in m.state_dict().items()})
+    x = seeded_randn((4, 2, 6, 8, 8), 91, 0.0, 2.0)
+    g = seeded_randn((4, 2, 8, 4, 4) if pool else (4, 2, 8, 8, 8), 92)
+    x64 = x.double().requires_grad_()
+    want = ref(x64)
+    want.backward(g.double())
+    m = m.cuda().train()
+    xd = x.cuda().requires_grad_()
+    out = m(xd)
+    out.backward(g.cuda())
+    assert float((out.detach().cpu().double() != want.detach()).float().mean()) == 0.0
+    torch.testing.assert_close(xd.grad.cpu().double(), x64.grad, rtol=1e-3, atol=2e-5 * float(x64.grad.abs().max()))
+    torch.testing.assert_close(m.conv_bn.block[0].weight.grad.cpu().double(), ref.conv_bn.block[0].weight.grad, rtol=1e-3,
+                               atol=2e-5 * float(ref.conv_bn.block[0].weight.grad.abs().max()))
