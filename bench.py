@@ -327,6 +327,35 @@ def other_workload(args) -> int:
                "fused_ms_per_step": fused_elapsed / args.steps * 1e3})
         return 0
 
+    if args.workload == "pwconv":
+        # the three GEMMs of the qkv convolution of configs[4] alone: Y = W X, dX = W^T dY, dW = sum dY X^T
+        from spikingjelly_amd.activation_based.hip_kernel import conv_bn_lif as CB
+
+        S, Cin, Cout, tokens = 256, 384, 1152, 196
+        terms = args.terms
+        x = randn((S, Cin, tokens), 1, 0.0, 1.0, torch.float32)
+        dy = randn((S, Cout, tokens), 2, 0.0, 1.0, torch.float32)
+        w = randn((Cout, Cin), 3, 0.0, 0.05, torch.float32)
+
+        def step():
+            CB.pw_gemm(CB.split_weight(w, False), terms, Cout, Cin, x, terms)
+            CB.pw_gemm(CB.split_weight(w, True), terms, Cin, Cout, dy, terms)
+            CB.pw_grad_weight(dy, terms, x, terms)
+
+        elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
+        g_ms, d_ms = _kernel_ms(L, L.KC_PW_GEMM), _kernel_ms(L, L.KC_PW_GRAD_WEIGHT)
+        flop = 2.0 * S * Cin * Cout * tokens                      # of one GEMM, counted once per fp32 product
+        products = {3: 6, 2: 3, 1: 1}[terms]                      # bf16 matrix-core products per fp32 product
+        _emit(args, "fp32-equivalent TFLOP/s of the kernel-size-1 convolution GEMMs, qkv of configs[4], 1 MI355X", "TFLOP/s",
+              3 * flop / (elapsed / args.steps) / 1e12, elapsed, "bf16",
+              {"workload": f"Y = W X, dX = W^T dY, dW = dY X^T for W [1152, 384], X [256, 384, 196] fp32, {terms} bf16 terms per operand"},
+              {"bound": "mfma", "achieved": products * flop / (g_ms * 1e-3) / 1e12, "peak": 2500.0, "unit": "TFLOP/s",
+               "frac": products * flop / (g_ms * 1e-3) / 1e12 / 2500.0, "traffic": None, "kernel": "pw_gemm",
+               "kernel_ms": g_ms, "grad_weight_ms": d_ms,
+               "grad_weight_TFLOPs": products * flop / (d_ms * 1e-3) / 1e12,
+               "fp32_equivalent_TFLOPs": flop / (g_ms * 1e-3) / 1e12})
+        return 0
+
     if args.workload == "config5":
         T, B, D, H, tokens = 4, 64, 384, 12, 196
         torch.manual_seed(1005)
@@ -373,7 +402,8 @@ def main() -> int:
     ap.add_argument("--cpu-sample-neurons", type=int, default=1 << 23)
     ap.add_argument("--cpu-repeats", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "qif", "eif", "izhikevich", "ilif", "stbif", "aaif", "fp8"],
+    ap.add_argument("--terms", type=int, default=3, choices=[1, 2, 3], help="pwconv workload: bf16 terms per fp32 operand")
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "pwconv", "qif", "eif", "izhikevich", "ilif", "stbif", "aaif", "fp8"],
                     help="config2 (default) is the headline metric; the others are secondary measurements")
     args = ap.parse_args()
     if args.gpus != 1:

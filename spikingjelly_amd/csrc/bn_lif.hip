@@ -43,6 +43,12 @@ __device__ __forceinline__ float wave_sum(float v) {
   for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
   return v;
 }
+// the same for a double, in a fixed order; every lane ends up with the total
+__device__ __forceinline__ double wave_sum_all(double v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
 
 // one wavefront per row of L contiguous elements: sum and sum of squares
 __global__ void __launch_bounds__(256) bn_stats_kernel(const float *y, int64_t rows, int L, float *partial) {
@@ -66,12 +72,17 @@ __global__ void __launch_bounds__(256) bn_finalize_kernel(const float *partial, 
                                                            const float *gamma, const float *beta, float eps,
                                                            float momentum, float *running_mean, float *running_var,
                                                            float *scale, float *shift, float *mean_out, float *invstd_out) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  // one wavefront per channel: lanes stride over the samples, then a butterfly sum
+  const int lane = threadIdx.x & 63;
+  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (c >= C) return;
   double mean, var;
   if (partial) {
     double s = 0.0, q = 0.0;
-    for (int64_t i = 0; i < S; ++i) { s += (double)partial[2 * (i * C + c)]; q += (double)partial[2 * (i * C + c) + 1]; }
+    for (int64_t i = lane; i < S; i += 64) { s += (double)partial[2 * (i * C + c)]; q += (double)partial[2 * (i * C + c) + 1]; }
+    s = wave_sum_all(s);
+    q = wave_sum_all(q);
+    if (lane != 0) return;
     mean = s / (double)count;
     var = q / (double)count - mean * mean;
     if (var < 0.0) var = 0.0;
@@ -81,6 +92,7 @@ __global__ void __launch_bounds__(256) bn_finalize_kernel(const float *partial, 
       running_var[c] = (float)((1.0 - (double)momentum) * (double)running_var[c] + (double)momentum * unbiased);
     }
   } else {
+    if (lane != 0) return;
     mean = (double)running_mean[c];
     var = (double)running_var[c];
   }
@@ -249,10 +261,14 @@ __global__ void __launch_bounds__(256) bn_backward_finalize_kernel(const float *
                                                                     int training, const float *gamma, const float *mean,
                                                                     const float *invstd, float *dgamma, float *dbeta,
                                                                     float *coef) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (c >= C) return;
   double sg = 0.0, sgy = 0.0;
-  for (int64_t i = 0; i < B; ++i) { sg += (double)partial[2 * (i * C + c)]; sgy += (double)partial[2 * (i * C + c) + 1]; }
+  for (int64_t i = lane; i < B; i += 64) { sg += (double)partial[2 * (i * C + c)]; sgy += (double)partial[2 * (i * C + c) + 1]; }
+  sg = wave_sum_all(sg);
+  sgy = wave_sum_all(sgy);
+  if (lane != 0) return;
   const double m = (double)mean[c], is = (double)invstd[c], g = gamma ? (double)gamma[c] : 1.0;
   const double dg = is * (sgy - m * sg);  // sum g (y - mean) invstd
   if (dgamma) dgamma[c] = (float)dg;
@@ -313,7 +329,7 @@ int launch_bn_finalize(const float *partial, int64_t S, int64_t C, int64_t L, co
                        float *invstd, hipStream_t stream) {
   if (C < 1 || C > (1 << 24)) return fail(SJHIP_ERR_INVALID, "bn_finalize: C=%lld", (long long)C);
   if (!partial && (!running_mean || !running_var)) return fail(SJHIP_ERR_INVALID, "bn_finalize: evaluation mode needs the running statistics");
-  hipLaunchKernelGGL(bn_finalize_kernel, dim3((unsigned)((C + 255) / 256)), dim3(256), 0, stream, partial, S, (int)C, S * L, gamma,
+  hipLaunchKernelGGL(bn_finalize_kernel, dim3((unsigned)((C + 3) / 4)), dim3(256), 0, stream, partial, S, (int)C, S * L, gamma,
                      beta, eps, momentum, running_mean, running_var, scale, shift, mean, invstd);
   return check_launch("bn_finalize");
 }
@@ -377,7 +393,7 @@ int launch_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int6
                                 const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef,
                                 hipStream_t stream) {
   if (C < 1 || C > (1 << 24)) return fail(SJHIP_ERR_INVALID, "bn_backward_finalize: C=%lld", (long long)C);
-  hipLaunchKernelGGL(bn_backward_finalize_kernel, dim3((unsigned)((C + 255) / 256)), dim3(256), 0, stream, partial, B, (int)C,
+  hipLaunchKernelGGL(bn_backward_finalize_kernel, dim3((unsigned)((C + 3) / 4)), dim3(256), 0, stream, partial, B, (int)C,
                      T * B * L, training, gamma, mean, invstd, dgamma, dbeta, coef);
   return check_launch("bn_backward_finalize");
 }

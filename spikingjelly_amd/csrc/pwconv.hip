@@ -14,9 +14,16 @@
 //       A comes pre-split as bf16 planes [3][M_pad][K_pad] (split_weight_kernel, zero padded), B is fp32 in memory.
 //       The S * L columns of all samples form one column index, so tiles of 128 columns carry no padding whatever L
 //       is.  A block of four wavefronts owns a 128 x 128 tile (each wavefront 64 x 64 = 2 x 2 MFMA tiles) and walks K
-//       in steps of 32: A tiles are copied to LDS as they are, B tiles are split and stored row by row (k rows,
-//       columns contiguous, as in memory) and each lane gathers the eight k values of its column with 16-bit LDS
-//       reads.  The next tile's global loads are in flight while the current one is multiplied.
+//       in steps of 32.  The matrix cores want, per lane, eight consecutive k of one row (A) or column (B): A tiles are
+//       copied to LDS as they are; for B a work-item fetches eight k of two adjacent columns (consecutive lanes fetch
+//       consecutive column pairs, so every access of a wavefront is one contiguous run), splits them and stores them
+//       k-contiguous, which transposes the tile on the way in and leaves 16-byte fragment reads for both operands.
+//       The global loads of the next two tiles are in flight while the current one is multiplied.
+//       Measured on the qkv convolution of a Spikformer block (M = 1152, K = 384, 50 176 columns): 0.36 ms with six
+//       products, 124 fp32-equivalent TFLOP/s.  Timing the kernel with parts cut out (only the loads 0.12 ms, only the
+//       staging 0.05, only fragment reads + MFMA 0.15, empty loop + stores 0.07) gives parts that add up to the whole,
+//       and neither wavefronts specialised as producers and consumers over two LDS buffers nor fewer, wider loads
+//       changed the total: the phases do not hide behind each other on this chip at this matrix-core load.
 //   pw_dw_kernel       dW[m][n] = sum_{s,l} dY[s][m][l] X[s][n][l]
 //       both operands are contiguous along the contraction index l; a block owns a 128 x 128 tile of dW for a chunk
 //       of samples and writes its partial tile, dw_reduce_kernel adds the chunks in a fixed order.
@@ -38,9 +45,6 @@ constexpr int kTileK = 32;            // contraction elements per LDS stage (two
 constexpr int kRowBytes = 80;         // K-contiguous operand row in LDS: 32 bf16 + 16 bytes, so that the 16-byte fragment
                                       // reads of eight consecutive rows fall on all 32 banks
 constexpr int kRowPlane = kTile * kRowBytes;
-constexpr int kColRowBytes = 264;     // column-contiguous operand: one k row of 128 bf16 + 8 bytes (rows k and k + 8,
-                                      // read by the two halves of a wavefront, then fall on different banks)
-constexpr int kColPlane = kTileK * kColRowBytes;
 constexpr int kXcds = 8;
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
@@ -132,10 +136,10 @@ __device__ __forceinline__ bf16x8 row_fragment(const uint8_t *plane, int row, in
 }
 
 template <int TA, int TB>
-__global__ void __launch_bounds__(kPwThreads) pw_gemm_kernel(const PwGemmArgs a) {
+__global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) pw_gemm_kernel(const PwGemmArgs a) {
   extern __shared__ __align__(16) uint8_t lds[];
   uint8_t *As = lds;                   // [TA][128][kRowBytes]
-  uint8_t *Bs = lds + TA * kRowPlane;  // [TB][32][kColRowBytes]
+  uint8_t *Bs = lds + TA * kRowPlane;  // [TB][128][kRowBytes], column-major: a row holds 32 k of one column
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int64_t logical = xcd_order(blockIdx.x, gridDim.x);
@@ -144,57 +148,79 @@ __global__ void __launch_bounds__(kPwThreads) pw_gemm_kernel(const PwGemmArgs a)
   const int m0 = mb * kTile;
   const int64_t j0 = nb * kTile;
   const int M = a.M, K = a.K, L = a.L;
+  const int K_pad = a.K_pad;
 
+  // Addresses are a wavefront-uniform 64-bit base (scalar registers) plus a 32-bit per-lane byte offset, and every load
+  // is unconditional (a branch per load would serialise them): offsets are clamped into the tensors and what lies
+  // outside the matrices is zeroed, under one uniform branch, when the tile is staged.
   // A: two 16-byte chunks per term and thread; chunk q = tid + 256 i -> row q / 4, k chunk q % 4
-  const uint16_t *a_src[2];
+  uint32_t a_off[2];
   int a_dst[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int q = tid + kPwThreads * i, row = q >> 2, kc = q & 3;
-    a_src[i] = a.a_planes + (int64_t)(m0 + row) * a.K_pad + 8 * kc;
+    a_off[i] = (uint32_t)(((m0 + row) * K_pad + 8 * kc) * 2);
     a_dst[i] = row * kRowBytes + kc * 16;
   }
-  // B: four quads (one k row each, rows kr, kr + 8, kr + 16, kr + 24) of the same four columns
-  const int c4 = tid & 31, kr = tid >> 5;
-  const int64_t jq = j0 + 4 * c4;
-  const bool col_ok = jq < a.ncols;  // L % 4 == 0, so a quad is inside one sample and all of it is valid or none
-  const float *b_src = nullptr;
+  // B: eight k (one fragment) of two adjacent columns, fetched as 8-byte accesses: columns 2 (tid % 64) and the next,
+  // k group = the wavefront's number.  Consecutive lanes fetch consecutive column pairs, so every access of a wavefront
+  // is one contiguous run, and a lane ends up with the eight k of a column that the matrix cores want from it.
+  const int bc = 2 * (tid & 63);
+  const int bk = __builtin_amdgcn_readfirstlane(wave * 8);
+  const int64_t jc = j0 + bc;
+  const bool col_ok = jc < a.ncols;  // L is even, so the two columns are in one sample and both valid or both not
+  uint32_t b_off = 0;
   if (col_ok) {
-    const int64_t s = jq / L;
-    const int l = (int)(jq - s * L);
-    b_src = a.b + (s * K) * (int64_t)L + l;
+    const int64_t s = jc / L;
+    b_off = (uint32_t)(((s * K) * (int64_t)L + (jc - s * L)) * 4);
   }
+  const bool edge_cols = __builtin_amdgcn_readfirstlane(j0 + kTile > a.ncols ? 1 : 0) != 0;
+  const char *a_base = reinterpret_cast<const char *>(a.a_planes);
+  const char *b_base = reinterpret_cast<const char *>(a.b);
 
+  // Two B tiles are in flight in registers (sets 0 and 1): a tile is requested two multiplications before it is staged,
+  // which covers a miss to HBM.  The A tiles (weight planes, a few MB that every block reads) come from L2, one ahead.
   u32x4 ra[TA][2];
-  f32x4 rb[4];
-  auto fetch = [&](int k0) {
+  u32x2 rb[2][8];  // [set][k]: the fp32 bit patterns of the two columns
+  auto fetch_a = [&](int k0) {
 #pragma unroll
-    for (int t = 0; t < TA; ++t)
+    for (int t = 0; t < TA; ++t) {
+      const char *plane = a_base + ((int64_t)t * a.plane_stride + k0) * 2;
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        ra[t][i] = *reinterpret_cast<const u32x4 *>(a_src[i] + (int64_t)t * a.plane_stride + k0);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int k = k0 + kr + 8 * i;
-      rb[i] = (col_ok && k < K) ? *reinterpret_cast<const f32x4 *>(b_src + (int64_t)k * L) : (f32x4)(0.0f);
+      for (int i = 0; i < 2; ++i) ra[t][i] = *reinterpret_cast<const u32x4 *>(plane + a_off[i]);
     }
   };
-  auto stage = [&]() {
+  auto fetch_b = [&](int k0, int set) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int k = k0 + bk + i;
+      const char *row = b_base + (int64_t)(k < K ? k : K - 1) * L * 4;
+      rb[set][i] = *reinterpret_cast<const u32x2 *>(row + b_off);
+    }
+  };
+  auto stage = [&](int k0, int set) {
 #pragma unroll
     for (int t = 0; t < TA; ++t)
 #pragma unroll
       for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4 *>(As + t * kRowPlane + a_dst[i]) = ra[t][i];
+    if (edge_cols || k0 + kTileK > K) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      uint32_t w01[TB], w23[TB];
-      split_pair<TB>(rb[i].x, rb[i].y, w01);
-      split_pair<TB>(rb[i].z, rb[i].w, w23);
+      for (int i = 0; i < 8; ++i)
+        if (!(col_ok && k0 + bk + i < K)) rb[set][i] = (u32x2)(0u);
+    }
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      uint32_t w[4][TB];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const u32x2 lo = rb[set][2 * i], hi = rb[set][2 * i + 1];
+        split_pair<TB>(__builtin_bit_cast(float, c ? lo.y : lo.x), __builtin_bit_cast(float, c ? hi.y : hi.x), w[i]);
+      }
 #pragma unroll
       for (int t = 0; t < TB; ++t) {
-        u32x2 w;
-        w.x = w01[t];
-        w.y = w23[t];
-        *reinterpret_cast<u32x2 *>(Bs + t * kColPlane + (kr + 8 * i) * kColRowBytes + c4 * 8) = w;
+        u32x4 v;
+        v.x = w[0][t]; v.y = w[1][t]; v.z = w[2][t]; v.w = w[3][t];
+        *reinterpret_cast<u32x4 *>(Bs + t * kRowPlane + (bc + c) * kRowBytes + bk * 2) = v;
       }
     }
   };
@@ -207,12 +233,7 @@ __global__ void __launch_bounds__(kPwThreads) pw_gemm_kernel(const PwGemmArgs a)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.0f;
 
-  fetch(0);
-  for (int k0 = 0; k0 < a.K_pad; k0 += kTileK) {
-    __syncthreads();  // the previous tile has been read by every wavefront
-    stage();
-    __syncthreads();
-    if (k0 + kTileK < a.K_pad) fetch(k0 + kTileK);
+  auto multiply = [&]() {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       bf16x8 af[2][TA], bf[2][TB];
@@ -223,21 +244,27 @@ __global__ void __launch_bounds__(kPwThreads) pw_gemm_kernel(const PwGemmArgs a)
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int t = 0; t < TB; ++t) {
-          const uint8_t *p = Bs + t * kColPlane + (ks * 16 + 8 * (lane >> 5)) * kColRowBytes +
-                             (wn * 64 + nt * 32 + (lane & 31)) * 2;
-          uint16_t e[8];
-#pragma unroll
-          for (int i = 0; i < 8; ++i) e[i] = *reinterpret_cast<const uint16_t *>(p + i * kColRowBytes);
-          u32x4 w;
-          w.x = e[0] | ((uint32_t)e[1] << 16);
-          w.y = e[2] | ((uint32_t)e[3] << 16);
-          w.z = e[4] | ((uint32_t)e[5] << 16);
-          w.w = e[6] | ((uint32_t)e[7] << 16);
-          bf[nt][t] = __builtin_bit_cast(bf16x8, w);
-        }
+        for (int t = 0; t < TB; ++t) bf[nt][t] = row_fragment(Bs + t * kRowPlane, wn * 64 + nt * 32 + (lane & 31), ks, lane);
       mfma_step<TA, TB>(af, bf, acc);
     }
+  };
+  fetch_a(0);
+  fetch_b(0, 0);
+  if (kTileK < K_pad) fetch_b(kTileK, 1);
+  for (int k0 = 0; k0 < K_pad; k0 += 2 * kTileK) {
+    __syncthreads();  // the previous tile has been read by every wavefront
+    stage(k0, 0);
+    __syncthreads();
+    if (k0 + kTileK < K_pad) fetch_a(k0 + kTileK);
+    if (k0 + 2 * kTileK < K_pad) fetch_b(k0 + 2 * kTileK, 0);
+    multiply();
+    if (k0 + kTileK >= K_pad) break;
+    __syncthreads();
+    stage(k0 + kTileK, 1);
+    __syncthreads();
+    if (k0 + 2 * kTileK < K_pad) fetch_a(k0 + 2 * kTileK);
+    if (k0 + 3 * kTileK < K_pad) fetch_b(k0 + 3 * kTileK, 1);
+    multiply();
   }
 
   // accumulator register r of a 32 x 32 tile: row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
@@ -271,7 +298,7 @@ struct PwDwArgs {
 };
 
 template <int TA, int TB>
-__global__ void __launch_bounds__(kPwThreads) pw_dw_kernel(const PwDwArgs a) {
+__global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) pw_dw_kernel(const PwDwArgs a) {
   extern __shared__ __align__(16) uint8_t lds[];
   uint8_t *As = lds;                   // [TA][128][kRowBytes]
   uint8_t *Bs = lds + TA * kRowPlane;  // [TB][128][kRowBytes]
@@ -289,30 +316,51 @@ __global__ void __launch_bounds__(kPwThreads) pw_dw_kernel(const PwDwArgs a) {
   const int l_steps = (L + kTileK - 1) / kTileK;
   const int64_t iters = (s_end - s_begin) * l_steps;
 
-  // a thread fetches quad q4 (four consecutive l) of rows rr, rr + 32, rr + 64, rr + 96 of both operand tiles
+  // a thread fetches quad q4 (four consecutive l) of rows rr, rr + 32, rr + 64, rr + 96 of both operand tiles; addresses
+  // are a uniform base (the sample) plus 32-bit per-lane offsets (row; position), loads are unconditional from clamped
+  // offsets and the outside of the matrices is zeroed when the tile is staged
   const int q4 = tid & 7, rr = tid >> 3;
-  f32x4 ra[4], rb[4];
-  auto fetch = [&](int64_t it) {
+  uint32_t a_off[4], b_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = rr + 32 * i;
+    a_off[i] = (uint32_t)((m0 + row < M ? m0 + row : M - 1) * L * 4);
+    b_off[i] = (uint32_t)((n0 + row < N ? n0 + row : N - 1) * L * 4);
+  }
+  const bool edge_rows = __builtin_amdgcn_readfirstlane((m0 + kTile > M || n0 + kTile > N) ? 1 : 0) != 0;
+  const char *dy_base = reinterpret_cast<const char *>(a.dy);
+  const char *x_base = reinterpret_cast<const char *>(a.x);
+  f32x4 ra[2][4], rb[2][4];  // two tiles in flight, as in pw_gemm_kernel
+  auto fetch = [&](int64_t it, int set) {
     const int64_t s = s_begin + it / l_steps;
-    const int l = (int)(it % l_steps) * kTileK + 4 * q4;
-    const bool l_ok = l < L;
+    const int l0 = (int)(it % l_steps) * kTileK;
+    const char *pa = dy_base + (s * M) * (int64_t)L * 4;
+    const char *pb = x_base + (s * N) * (int64_t)L * 4;
+    const int l = l0 + 4 * q4;
+    const uint32_t l_off = (uint32_t)((l < L ? l : L - 4) * 4);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int row = rr + 32 * i;
-      ra[i] = (l_ok && m0 + row < M) ? *reinterpret_cast<const f32x4 *>(a.dy + ((s * M + m0 + row) * (int64_t)L + l))
-                                     : (f32x4)(0.0f);
-      rb[i] = (l_ok && n0 + row < N) ? *reinterpret_cast<const f32x4 *>(a.x + ((s * N + n0 + row) * (int64_t)L + l))
-                                     : (f32x4)(0.0f);
+      ra[set][i] = *reinterpret_cast<const f32x4 *>(pa + (a_off[i] + l_off));
+      rb[set][i] = *reinterpret_cast<const f32x4 *>(pb + (b_off[i] + l_off));
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](int64_t it, int set) {
+    const int l0 = (int)(it % l_steps) * kTileK;
+    const bool l_ok = l0 + 4 * q4 < L;
+    if (edge_rows || l0 + kTileK > L) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (!(l_ok && m0 + rr + 32 * i < M)) ra[set][i] = (f32x4)(0.0f);
+        if (!(l_ok && n0 + rr + 32 * i < N)) rb[set][i] = (f32x4)(0.0f);
+      }
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int off = (rr + 32 * i) * kRowBytes + q4 * 8;
       {
         uint32_t w01[TA], w23[TA];
-        split_pair<TA>(ra[i].x, ra[i].y, w01);
-        split_pair<TA>(ra[i].z, ra[i].w, w23);
+        split_pair<TA>(ra[set][i].x, ra[set][i].y, w01);
+        split_pair<TA>(ra[set][i].z, ra[set][i].w, w23);
 #pragma unroll
         for (int t = 0; t < TA; ++t) {
           u32x2 w;
@@ -323,8 +371,8 @@ __global__ void __launch_bounds__(kPwThreads) pw_dw_kernel(const PwDwArgs a) {
       }
       {
         uint32_t w01[TB], w23[TB];
-        split_pair<TB>(rb[i].x, rb[i].y, w01);
-        split_pair<TB>(rb[i].z, rb[i].w, w23);
+        split_pair<TB>(rb[set][i].x, rb[set][i].y, w01);
+        split_pair<TB>(rb[set][i].z, rb[set][i].w, w23);
 #pragma unroll
         for (int t = 0; t < TB; ++t) {
           u32x2 w;
@@ -344,13 +392,8 @@ __global__ void __launch_bounds__(kPwThreads) pw_dw_kernel(const PwDwArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.0f;
 
-  if (iters > 0) fetch(0);
-  for (int64_t it = 0; it < iters; ++it) {
-    __syncthreads();
-    stage();
-    __syncthreads();
+  auto multiply = [&](int64_t it) {
     const int l0 = (int)(it % l_steps) * kTileK;
-    if (it + 1 < iters) fetch(it + 1);
     const int ksteps = (l0 + 16 < L) ? 2 : 1;  // the second half of the last stage of a row may hold nothing
     for (int ks = 0; ks < ksteps; ++ks) {
       bf16x8 af[2][TA], bf[2][TB];
@@ -364,6 +407,21 @@ __global__ void __launch_bounds__(kPwThreads) pw_dw_kernel(const PwDwArgs a) {
         for (int t = 0; t < TB; ++t) bf[nt][t] = row_fragment(Bs + t * kRowPlane, wn * 64 + nt * 32 + (lane & 31), ks, lane);
       mfma_step<TA, TB>(af, bf, acc);
     }
+  };
+  if (iters > 0) fetch(0, 0);
+  if (iters > 1) fetch(1, 1);
+  for (int64_t it = 0; it < iters; it += 2) {
+    __syncthreads();
+    stage(it, 0);
+    __syncthreads();
+    if (it + 2 < iters) fetch(it + 2, 0);
+    multiply(it);
+    if (it + 1 >= iters) break;
+    __syncthreads();
+    stage(it + 1, 1);
+    __syncthreads();
+    if (it + 3 < iters) fetch(it + 3, 1);
+    multiply(it + 1);
   }
 
   float *out = a.partials + (int64_t)chunk * M * N;
@@ -394,7 +452,7 @@ __global__ void __launch_bounds__(256) dw_reduce_kernel(const float *partials, i
 int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
 template <int TA, int TB> int launch_gemm_terms(const PwGemmArgs &a, int64_t blocks, hipStream_t stream) {
-  const unsigned lds = TA * kRowPlane + TB * kColPlane;
+  const unsigned lds = (TA + TB) * kRowPlane;
   hipLaunchKernelGGL((pw_gemm_kernel<TA, TB>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
   return check_launch("pwconv_gemm");
 }
@@ -432,27 +490,35 @@ int launch_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int t
 
 int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,
                        int64_t L, float *c, hipStream_t stream) {
-  if (L % 4 != 0 || !aligned16(b) || !aligned16(a_planes))
-    return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: L=%lld must be a multiple of 4 and the tensors 16-byte aligned", (long long)L);
-  if (M > (1 << 24) || K > (1 << 24) || L > (1 << 24)) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: M=%lld K=%lld L=%lld", (long long)M, (long long)K, (long long)L);
-  PwGemmArgs a;
-  a.a_planes = a_planes; a.b = b; a.c = c;
-  a.M = (int)M; a.K = (int)K; a.K_pad = (int)round_up(K, kTileK); a.L = (int)L;
-  a.plane_stride = round_up(M, kTile) * a.K_pad;
-  a.ncols = S * L;
-  a.m_blocks = (int)(round_up(M, kTile) / kTile);
-  const int64_t blocks = a.m_blocks * ((a.ncols + kTile - 1) / kTile);
-  if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: %lld blocks", (long long)blocks);
+  if (L % 2 != 0 || !aligned16(a_planes) || (reinterpret_cast<uintptr_t>(b) & 7u))
+    return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: L=%lld must be even, the weight planes 16-byte and the activations 8-byte aligned", (long long)L);
+  const int64_t limit = int64_t(1) << 30;  // per-lane offsets into A and B are 32-bit byte offsets
+  if (round_up(M, kTile) * round_up(K, kTileK) >= limit || K * L >= limit)
+    return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: M=%lld K=%lld L=%lld", (long long)M, (long long)K, (long long)L);
+  const int64_t s_step = (limit - 1) / (K * L);  // samples per launch
   ProfileScope prof(KC_PW_GEMM, stream);
-  const int key = a_terms * 10 + b_terms;
-  switch (key) {
-    case 33: return launch_gemm_terms<3, 3>(a, blocks, stream);
-    case 31: return launch_gemm_terms<3, 1>(a, blocks, stream);
-    case 22: return launch_gemm_terms<2, 2>(a, blocks, stream);
-    case 21: return launch_gemm_terms<2, 1>(a, blocks, stream);
-    case 11: return launch_gemm_terms<1, 1>(a, blocks, stream);
-    default: return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: %d weight terms with %d activation terms (3/3, 3/1, 2/2, 2/1, 1/1)", a_terms, b_terms);
+  for (int64_t s0 = 0; s0 < S; s0 += s_step) {
+    const int64_t s_count = S - s0 < s_step ? S - s0 : s_step;
+    PwGemmArgs a;
+    a.a_planes = a_planes; a.b = b + s0 * K * L; a.c = c + s0 * M * L;
+    a.M = (int)M; a.K = (int)K; a.K_pad = (int)round_up(K, kTileK); a.L = (int)L;
+    a.plane_stride = round_up(M, kTile) * a.K_pad;
+    a.ncols = s_count * L;
+    a.m_blocks = (int)(round_up(M, kTile) / kTile);
+    const int64_t blocks = a.m_blocks * ((a.ncols + kTile - 1) / kTile);
+    if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: %lld blocks", (long long)blocks);
+    int rc;
+    switch (a_terms * 10 + b_terms) {
+      case 33: rc = launch_gemm_terms<3, 3>(a, blocks, stream); break;
+      case 31: rc = launch_gemm_terms<3, 1>(a, blocks, stream); break;
+      case 22: rc = launch_gemm_terms<2, 2>(a, blocks, stream); break;
+      case 21: rc = launch_gemm_terms<2, 1>(a, blocks, stream); break;
+      case 11: rc = launch_gemm_terms<1, 1>(a, blocks, stream); break;
+      default: return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: %d weight terms with %d activation terms (3/3, 3/1, 2/2, 2/1, 1/1)", a_terms, b_terms);
+    }
+    if (rc != SJHIP_OK) return rc;
   }
+  return SJHIP_OK;
 }
 
 int64_t pwconv_dw_workspace_floats(int64_t M, int64_t N, int64_t S) {
@@ -465,7 +531,8 @@ int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int
                               int64_t L, float *dw, float *workspace, hipStream_t stream) {
   if (L % 4 != 0 || !aligned16(dy) || !aligned16(x))
     return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight: L=%lld must be a multiple of 4 and the tensors 16-byte aligned", (long long)L);
-  if (M > (1 << 24) || N > (1 << 24) || L > (1 << 24)) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_grad_weight: M=%lld N=%lld L=%lld", (long long)M, (long long)N, (long long)L);
+  if (M * L >= (int64_t(1) << 30) || N * L >= (int64_t(1) << 30) || M * N >= (int64_t(1) << 40))  // 32-bit per-lane byte offsets
+    return fail(SJHIP_ERR_TOO_LARGE, "pwconv_grad_weight: M=%lld N=%lld L=%lld", (long long)M, (long long)N, (long long)L);
   PwDwArgs a;
   a.dy = dy; a.x = x; a.partials = workspace; a.S = S;
   a.M = (int)M; a.N = (int)N; a.L = (int)L;
