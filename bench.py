@@ -56,6 +56,64 @@ def cpu_baseline(torch, sample_neurons: int, repeats: int):
     }
 
 
+# source files whose kernels the counter-measured traffic in profiles/traffic_*.json belongs to
+TRAFFIC_SOURCES = ("neuron_fwd.h", "neuron_bwd.h", "neuron_bwd_recompute.h", "neuron_bwd_recompute_launch.h", "sjhip_common.h")
+
+
+def kernel_source_digest() -> str:
+    """sha256 over the sources of the forward / backward kernels: the recorded HBM traffic is reported only while it
+    still describes the kernels that run (an edit to any of these files makes it stale)."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in TRAFFIC_SOURCES:
+        with open(os.path.join(ROOT, "spikingjelly_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def recorded_traffic():
+    """The rocprofv3 FETCH_SIZE / WRITE_SIZE record of the headline kernels, or None when it is missing or stale."""
+    path = os.path.join(ROOT, "profiles", "traffic_lif_fp32_T16_N33554432.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        rec = json.load(f)
+    return rec if rec.get("kernel_source_sha256") == kernel_source_digest() else None
+
+
+def measure_ceilings(torch, L, floats_per_stream: int, repeats: int = 5):
+    """GB/s of the library's plain streaming kernel (sjhip_stream_probe) for the access mixes of the neuron kernels,
+    over streams of the size of one [T, N] tensor of the workload; best cache policy of the two for each mix."""
+    dev = torch.device("cuda:0")
+    bufs = [torch.empty(floats_per_stream, dtype=torch.float32, device=dev) for _ in range(4)]
+    for b in bufs[:3]:
+        b.fill_(0.5)
+    mixes = {"read_1r0w": (1, 0), "write_0r1w": (0, 1), "copy_1r1w": (1, 1), "forward_1r2w": (1, 2),
+             "forward_saving_h_1r3w": (1, 3), "backward_3r1w": (3, 1)}
+    out = {}
+    for name, (r, w) in mixes.items():
+        best = 0.0
+        for nt in (False, True):
+            ins, outs = bufs[:r], bufs[r:r + max(w, 1)]  # a read-only probe still takes one (unwritten) output
+            for _ in range(2):
+                L.stream_probe(r, w, nt, ins, outs)
+            torch.cuda.synchronize()
+            L.profile_reset()
+            L.profile_enable(True)
+            for _ in range(repeats):
+                L.stream_probe(r, w, nt, ins, outs)
+            torch.cuda.synchronize()
+            L.profile_enable(False)
+            n, ms = L.profile_read(L.KC_STREAM_PROBE)
+            gbs = (r + w) * floats_per_stream * 4 / (ms / max(n, 1) * 1e-3) / 1e9
+            best = max(best, gbs)
+        out[name] = best
+    del bufs
+    torch.cuda.empty_cache()
+    return out
+
+
 def _time_steps(torch, L, step, steps, warmup):
     """warm-up, then `steps` timed steps bracketed by synchronisation; library event profiler on."""
     for _ in range(warmup):
@@ -327,6 +385,21 @@ def other_workload(args) -> int:
                "fused_ms_per_step": fused_elapsed / args.steps * 1e3})
         return 0
 
+    if args.workload == "ceilings":
+        # what the memory system gives to plain streams of the config-2 tensor size (2.1 GB each)
+        floats = 16 * 256 * 128 * 32 * 32
+        t0 = time.perf_counter()
+        c = measure_ceilings(torch, L, floats, repeats=args.steps)
+        elapsed = time.perf_counter() - t0
+        top = max(c.values())
+        _emit(args, "GB/s of plain fp32 streams (sjhip_stream_probe), 2.1 GB per stream, 1 MI355X", "GB/s", top, elapsed, "f32",
+              {"workload": "one 16-byte access per work-item and stream; read-only, write-only, copy and the read:write "
+                           "mixes of the neuron kernels (1:2 forward, 1:3 forward saving h_seq, 3:1 backward); best of "
+                           "default and streaming cache policy", **{k: round(v, 1) for k, v in c.items()}},
+              {"bound": "hbm", "achieved": top, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": top / HBM_PEAK_GBS,
+               "traffic": None, "kernel": "stream_probe"})
+        return 0
+
     if args.workload == "pwconv":
         # the three GEMMs of the qkv convolution of configs[4] alone: Y = W X, dX = W^T dY, dW = sum dY X^T
         from spikingjelly_amd.activation_based.hip_kernel import conv_bn_lif as CB
@@ -403,7 +476,11 @@ def main() -> int:
     ap.add_argument("--cpu-repeats", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--terms", type=int, default=3, choices=[1, 2, 3], help="pwconv workload: bf16 terms per fp32 operand")
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "pwconv", "qif", "eif", "izhikevich", "ilif", "stbif", "aaif", "fp8"],
+    ap.add_argument("--seq-len", type=int, default=SHAPE[0],
+                    help="config2 variant: T steps over 2^29 / T neurons (the headline is T=16); a secondary measurement")
+    ap.add_argument("--n-offset", type=int, default=0,
+                    help="config2 variant: K more neurons than the power of two, i.e. another row stride (multiple of 4)")
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "pwconv", "ceilings", "qif", "eif", "izhikevich", "ilif", "stbif", "aaif", "fp8"],
                     help="config2 (default) is the headline metric; the others are secondary measurements")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -426,11 +503,18 @@ def main() -> int:
     N = 1
     for d in SHAPE[1:]:
         N *= d
+    T, shape = args.seq_len, SHAPE
+    variant = args.seq_len != SHAPE[0] or args.n_offset != 0
+    if variant:
+        if args.seq_len < 1 or (SHAPE[0] * N) % args.seq_len or args.n_offset % 4 or args.n_offset < 0:
+            raise SystemExit("--seq-len must divide 2^29 and --n-offset must be a non-negative multiple of 4")
+        N = SHAPE[0] * N // args.seq_len + args.n_offset
+        shape = (T, N)
 
     # inputs: CPU generator with the configured seeds, then resident on the device
     def make(seed, mean, std):
         g = torch.Generator().manual_seed(seed)
-        return (torch.randn(SHAPE, generator=g) * std + mean).to(dev)
+        return (torch.randn(shape, generator=g) * std + mean).to(dev)
 
     x = make(1002, 0.3, 0.8).requires_grad_()
     grad_spike = make(1102, 0.0, 1.0)
@@ -467,38 +551,37 @@ def main() -> int:
     n_fwd, ms_fwd = L.profile_read(L.KC_FORWARD)
     n_bwd, ms_bwd = L.profile_read(L.KC_BACKWARD)
 
-    # measured device-copy ceiling on the same box: torch's copy kernel over one 2.1 GB tensor
-    dst = torch.empty_like(grad_v)
-    for _ in range(2):
-        dst.copy_(grad_v)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(5):
-        dst.copy_(grad_v)
-    e1.record()
-    torch.cuda.synchronize()
-    copy_gbs = 2 * grad_v.numel() * 4 / (e0.elapsed_time(e1) / 5 * 1e-3) / 1e9
-    del dst
+    # measured ceilings on the same box: the library's plain streaming kernel over streams of the size of x (2.1 GB)
+    del spikes
+    node.v_seq = None
+    torch.cuda.empty_cache()
+    ceilings = measure_ceilings(torch, L, x.numel())
 
     ms_per_step = elapsed / args.steps * 1e3
-    value = T_STEPS * N / (elapsed / args.steps)
+    value = T * N / (elapsed / args.steps)
 
     # algorithmic bytes per launch: each tensor of the operator contract touched once
-    fwd_bytes = 16 * T_STEPS * N + 4 * N  # x, spike, v_seq, h_seq per step + v_init
-    bwd_bytes = 16 * T_STEPS * N + 4 * N  # grad_spike, grad_v, h_seq, grad_x per step + grad_v_init
+    fwd_bytes = 16 * T * N + 4 * N  # x, spike, v_seq, h_seq per step + v_init
+    bwd_bytes = 16 * T * N + 4 * N  # grad_spike, grad_v, h_seq, grad_x per step + grad_v_init
     fwd_ms = ms_fwd / max(n_fwd, 1)
     bwd_ms = ms_bwd / max(n_bwd, 1)
     dominant = "forward" if fwd_ms >= bwd_ms else "backward"
     dom_ms, dom_bytes = (fwd_ms, fwd_bytes) if dominant == "forward" else (bwd_ms, bwd_bytes)
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic_lif_fp32_T16_N33554432.json")
-    if os.path.exists(tpath):  # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs
-        with open(tpath) as f:
-            traffic = json.load(f).get(dominant)
+    # HBM bytes the kernels actually move, each tensor touched once: the forward writes no h_seq (the backward replays
+    # it) and the module's initial state is one broadcast element, so forward = x in, spikes + v_seq + v_last out;
+    # backward = x, grad_spike, grad_v in, grad_x out.  The counter-measured figures (rocprofv3 FETCH_SIZE / WRITE_SIZE,
+    # profiles/) are reported while they still describe the kernels that ran.
+    fwd_moved = 12 * T * N + 4 * N
+    bwd_moved = 16 * T * N
+    rec = None if variant else recorded_traffic()
+    traffic = rec.get(dominant) if rec else None
+    if rec:
+        fwd_moved, bwd_moved = rec["forward"], rec["backward"]
 
     out = {
-        "metric": "neuron-steps/sec LIF fwd+bwd T=16 N=33.5M, 1 MI355X; % of HBM roofline",
+        "metric": "neuron-steps/sec LIF fwd+bwd T=16 N=33.5M, 1 MI355X; % of HBM roofline" if not variant else
+                  f"neuron-steps/sec LIF fwd+bwd T={T} N={N}, 1 MI355X; % of HBM roofline",
         "value": value,
         "unit": "neuron-steps/s",
         "n_gpus": 1,
@@ -511,9 +594,11 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "configs[1]: LIFNode multi-step fwd+bwd, x [16,256,128,32,32] fp32 ~N(0.3,0.8), tau=2, "
-                               "hard reset 0, ATan(2), store_v_seq=True, grad_spike ~N(0,1), grad_v ~N(0,0.1)",
-                   "T": T_STEPS, "N": N, "backend": "hip", "firing_rate": rate},
+        "config": {"workload": ("configs[1]: LIFNode multi-step fwd+bwd, x [16,256,128,32,32]" if not variant else
+                                f"variant of configs[1] with another shape: LIFNode multi-step fwd+bwd, x [{T},{N}]") +
+                               " fp32 ~N(0.3,0.8), tau=2, hard reset 0, ATan(2), store_v_seq=True, grad_spike ~N(0,1), "
+                               "grad_v ~N(0,0.1)",
+                   "T": T, "N": N, "backend": "hip", "firing_rate": rate},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": dominant,
                      "kernel_ms": dom_ms, "algorithmic_bytes": dom_bytes,
@@ -522,9 +607,13 @@ def main() -> int:
                      "backward_GBs": bwd_bytes / (bwd_ms * 1e-3) / 1e9 if bwd_ms else None,
                      "fwd_plus_bwd_frac": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS
                      if (fwd_ms + bwd_ms) else None,
-                     "device_copy_GBs": copy_gbs},
+                     "forward_traffic_GBs": fwd_moved / (fwd_ms * 1e-3) / 1e9 if fwd_ms else None,
+                     "backward_traffic_GBs": bwd_moved / (bwd_ms * 1e-3) / 1e9 if bwd_ms else None,
+                     "step_traffic_frac": (fwd_moved + bwd_moved) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic_source": "rocprofv3 counters (profiles/)" if rec else "tensor sizes",
+                     "ceilings_GBs": {k: round(v, 1) for k, v in ceilings.items()}},
     }
-    del x, grad_spike, grad_v, spikes
+    del x, grad_spike, grad_v
     torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, args.cpu_sample_neurons, args.cpu_repeats)

@@ -181,7 +181,7 @@ int64_t sjhip_plif_workspace_floats(int dtype, int64_t N);
 
 /*
  * Backward (BPTT) over T steps.
- *   grad_spike_seq [T,N] in
+ *   grad_spike_seq [T,N] in, or NULL for zeros (a loss on the membrane potential alone): nothing is read then
  *   grad_v_seq     [T,N] in, gradient w.r.t. v_seq, or NULL
  *   grad_v_last    [N] in, gradient w.r.t. v_last (enters at t = T-1), or NULL
  *   h_seq          [T,N] in (from forward)
@@ -239,6 +239,37 @@ int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_pa
                                     void *grad_x_seq, void *grad_v_init,
                                     float *grad_rtau, float *workspace,
                                     void *stream);
+
+/*
+ * The replay for sequences of any length, in one launch each way.  The sequence is cut into pieces of `chunk` steps
+ * (the last may be shorter; sjhip_replay_pieces(T, chunk) of them).  sjhip_neuron_forward_pieces is
+ * sjhip_neuron_forward with h_seq = NULL that also leaves the state after every piece but the last in
+ * `checkpoints` [pieces - 1][N] (storage dtype; may be NULL when T <= chunk).  sjhip_neuron_backward_recompute_pieces
+ * is sjhip_neuron_backward_recompute that walks the pieces from the last to the first: each is replayed from its
+ * checkpoint into an LDS buffer of `chunk` steps (so chunk, not T, must satisfy sjhip_recompute_supported) and walked
+ * back; the gradient of a piece's initial state reaches the piece before it through `carry` [N] (storage dtype,
+ * scratch, contents undefined afterwards; may be NULL when T <= chunk).  Results: spikes, states and checkpoints are
+ * bit-identical to sjhip_neuron_forward's; gradients are those of sjhip_neuron_backward_recompute on each piece, with
+ * the carry rounded to the storage dtype between pieces (no rounding for fp32).  N must be a multiple of the 128-bit
+ * vector width and every tensor 16-byte aligned; 16-bit storage with SJHIP_FLAG_FP32_STATE is refused
+ * (SJHIP_ERR_UNSUPPORTED: a checkpoint in the storage dtype would round the state).  The saved state per neuron is 1 / chunk of an h_seq; chunk = 16 keeps
+ * five or more blocks resident per compute unit, which is where the single-piece kernel runs fastest.  No counterpart
+ * in the reference (its kernels always read the saved h_seq, multi_step/base.py:137-409).
+ */
+int64_t sjhip_replay_pieces(int64_t T, int64_t chunk);
+int sjhip_neuron_forward_pieces(int neuron, int dtype, const sjhip_neuron_params *p,
+                                int64_t T, int64_t N, int64_t chunk,
+                                const void *x_seq, const void *v_init, const float *rtau_device,
+                                void *spike_seq, void *v_seq, void *v_last, void *checkpoints,
+                                void *stream);
+int sjhip_neuron_backward_recompute_pieces(int neuron, int dtype, const sjhip_neuron_params *p,
+                                           int64_t T, int64_t N, int64_t chunk,
+                                           const void *x_seq, const void *v_init, const float *rtau_device,
+                                           const void *checkpoints,
+                                           const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                                           void *grad_x_seq, void *grad_v_init,
+                                           float *grad_rtau, float *workspace, void *carry,
+                                           void *stream);
 
 /* 1 if sjhip_neuron_backward_recompute can serve [T,N] of `dtype` (N a multiple of the 128-bit vector
  * width and T steps of h fitting in LDS: T <= 159), else 0. */
@@ -480,10 +511,21 @@ int sjhip_set_tuning(const char *key, int value);
 int sjhip_get_tuning(const char *key);
 
 /*
+ * Bandwidth probe: a plain streaming kernel with `reads` input and `writes` output streams of floats_per_stream fp32
+ * each (0..3 of each; the instantiated mixes are r:w = 1:0 2:0 3:0 0:1 0:2 0:3 1:1 1:2 1:3 2:1 3:1), one 16-byte access
+ * per work-item and stream, default or (nontemporal != 0) streaming cache policy.  in / out are host arrays of device
+ * pointers (a read-only probe still takes one output pointer, which it never writes).  No counterpart in the
+ * reference: it measures the ceilings the neuron kernels' bandwidth is compared with, on the device and in the run
+ * that measures them (kernel class 13 of sjhip_profile_read).
+ */
+int sjhip_stream_probe(int reads, int writes, int nontemporal, int64_t floats_per_stream, const float *const *in,
+                       float *const *out, void *stream);
+
+/*
  * Optional per-kernel timing.  While enabled every launch is bracketed by HIP events on its own
  * stream.  sjhip_profile_read() synchronises those events and returns, for kernel class `which`
  * (0 forward, 1 backward, 2 plif-reduce, 3 bit_pack, 4 bit_unpack, 5 ssa forward, 6 ssa backward, 7 pwconv gemm,
- * 8 pwconv grad_weight, 9 bn stats, 10 bn_lif forward, 11 bn_lif backward, 12 bn grad_input), the launch count and total
+ * 8 pwconv grad_weight, 9 bn stats, 10 bn_lif forward, 11 bn_lif backward, 12 bn grad_input, 13 stream probe), the launch count and total
  * milliseconds since the last sjhip_profile_reset().
  */
 int sjhip_profile_enable(int on);

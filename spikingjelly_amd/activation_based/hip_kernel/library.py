@@ -35,7 +35,7 @@ FLAG_GRAD_STORAGE = 0x1000
 STATIC_WORKSPACE_MAX_NEURONS = 1 << 26
 
 (KC_FORWARD, KC_BACKWARD, KC_PLIF_REDUCE, KC_BIT_PACK, KC_BIT_UNPACK, KC_SSA_FORWARD, KC_SSA_BACKWARD, KC_PW_GEMM,
- KC_PW_GRAD_WEIGHT, KC_BN_STATS, KC_BN_LIF_FORWARD, KC_BN_LIF_BACKWARD, KC_BN_GRAD_INPUT) = range(13)
+ KC_PW_GRAD_WEIGHT, KC_BN_STATS, KC_BN_LIF_FORWARD, KC_BN_LIF_BACKWARD, KC_BN_GRAD_INPUT, KC_STREAM_PROBE) = range(14)
 
 EXPORTED_SYMBOLS = (
     "sjhip_abi_version",
@@ -48,6 +48,9 @@ EXPORTED_SYMBOLS = (
     "sjhip_neuron_backward",
     "sjhip_neuron_backward_static",
     "sjhip_neuron_backward_recompute",
+    "sjhip_replay_pieces",
+    "sjhip_neuron_forward_pieces",
+    "sjhip_neuron_backward_recompute_pieces",
     "sjhip_recompute_supported",
     "sjhip_recompute_preferred",
     "sjhip_ssa_supported",
@@ -60,6 +63,7 @@ EXPORTED_SYMBOLS = (
     "sjhip_izhikevich_forward",
     "sjhip_izhikevich_backward",
     "sjhip_izhikevich_backward_replay",
+    "sjhip_stream_probe",
     "sjhip_pwconv_planes_elems",
     "sjhip_pwconv_split_weight",
     "sjhip_pwconv_gemm",
@@ -167,6 +171,19 @@ def load() -> ctypes.CDLL:
             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
         ]
+        lib.sjhip_replay_pieces.restype = c_int64
+        lib.sjhip_replay_pieces.argtypes = [c_int64, c_int64]
+        lib.sjhip_neuron_forward_pieces.restype = c_int
+        lib.sjhip_neuron_forward_pieces.argtypes = [
+            c_int, c_int, POINTER(NeuronParams), c_int64, c_int64, c_int64,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        ]
+        lib.sjhip_neuron_backward_recompute_pieces.restype = c_int
+        lib.sjhip_neuron_backward_recompute_pieces.argtypes = [
+            c_int, c_int, POINTER(NeuronParams), c_int64, c_int64, c_int64,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        ]
         lib.sjhip_recompute_supported.restype = c_int
         lib.sjhip_recompute_supported.argtypes = [c_int, c_int64, c_int64]
         lib.sjhip_recompute_preferred.restype = c_int
@@ -203,6 +220,8 @@ def load() -> ctypes.CDLL:
         lib.sjhip_izhikevich_backward_replay.restype = c_int
         lib.sjhip_izhikevich_backward_replay.argtypes = ([c_int, POINTER(IzhikevichParams), c_int64, c_int64]
                                                          + [c_void_p] * 12)
+        lib.sjhip_stream_probe.restype = c_int
+        lib.sjhip_stream_probe.argtypes = [c_int, c_int, c_int, c_int64, POINTER(c_void_p), POINTER(c_void_p), c_void_p]
         lib.sjhip_pwconv_planes_elems.restype = c_int64
         lib.sjhip_pwconv_planes_elems.argtypes = [c_int64, c_int64]
         lib.sjhip_pwconv_split_weight.restype = c_int
@@ -300,6 +319,17 @@ def aligned16(t: torch.Tensor) -> torch.Tensor:
     """``t`` made contiguous and 16-byte aligned (a fresh allocation always is)."""
     t = t.contiguous()
     return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
+def stream_probe(reads: int, writes: int, nontemporal: bool, inputs, outputs) -> None:
+    """One launch of the bandwidth probe over equally sized fp32 device tensors (see ``sjhip_stream_probe``)."""
+    ref = (list(inputs) + list(outputs))[0]
+    n = ref.numel()
+    ins = (c_void_p * max(len(inputs), 1))(*[t.data_ptr() for t in inputs])
+    outs = (c_void_p * max(len(outputs), 1))(*[t.data_ptr() for t in outputs])
+    with torch.cuda.device(ref.device):
+        rc = load().sjhip_stream_probe(reads, writes, 1 if nontemporal else 0, n, ins, outs, current_stream_ptr(ref.device))
+    check(rc, "stream_probe")
 
 
 def set_tuning(key: str, value: int) -> None:

@@ -101,32 +101,54 @@ def _k_pointer(k: Optional[torch.Tensor], ref: torch.Tensor) -> tuple[Optional[t
     return k, k.data_ptr()
 
 
+def _chunks(T: int, chunk: int) -> list[tuple[int, int]]:
+    """Row ranges ``[t0, t1)`` of a sequence cut into pieces of at most ``chunk`` steps (one piece for ``chunk <= 0``)."""
+    if chunk <= 0 or T <= chunk:
+        return [(0, T)]
+    return [(t0, min(t0 + chunk, T)) for t0 in range(0, T, chunk)]
+
+
 def _run_forward(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: Optional[torch.Tensor],
                  tau: float, v_th: float, v_reset: float, flags: int, store_v_seq: bool,
                  save_h: bool, qif: tuple[float, float, float] = _NO_EXTRA,
-                 levels: tuple[float, float, float] = _NO_EXTRA
+                 levels: tuple[float, float, float] = _NO_EXTRA, chunk: int = 0
                  ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """``(spike_seq, v_seq, v_last, h_seq)``.  With ``chunk > 0`` (and no ``h_seq``) a sequence longer than ``chunk``
+    runs as pieces of ``chunk`` steps inside one launch, and the fourth result holds the state after every piece but
+    the last, ``[pieces - 1, N]``: the checkpoints from which the backward replays piece by piece."""
     _check_inputs(x_seq, v_init)
     dtype = L.dtype_id(x_seq.dtype)
-    x_seq = x_seq.contiguous()
-    v_init, broadcast = _state_arg(v_init, False)
     T, N = x_seq.shape
+    pieces = len(_chunks(T, 0 if save_h else chunk))
+    x_seq = L.aligned16(x_seq) if pieces > 1 else x_seq.contiguous()
+    v_init, broadcast = _state_arg(v_init, pieces > 1)
     spike_seq = torch.empty_like(x_seq)
     v_seq = torch.empty_like(x_seq) if store_v_seq else x_seq.new_empty((0,))
     v_last = x_seq.new_empty((N,))
     h_seq = torch.empty_like(x_seq) if save_h else None
+    checkpoints = x_seq.new_empty((pieces - 1, N)) if pieces > 1 else None
     k_keep, k_ptr = _k_pointer(k, x_seq)
     params = _params(tau, v_th, v_reset, 0.0, 0, flags | broadcast, qif, levels)
+    lib = L.load()
     with torch.cuda.device(x_seq.device):
-        rc = L.load().sjhip_neuron_forward(
-            neuron, dtype, ctypes.byref(params), T, N,
-            x_seq.data_ptr(), v_init.data_ptr(), k_ptr,
-            spike_seq.data_ptr(), v_seq.data_ptr() if store_v_seq else None, v_last.data_ptr(),
-            L.ptr(h_seq), L.current_stream_ptr(x_seq.device),
-        )
+        stream = L.current_stream_ptr(x_seq.device)
+        if pieces > 1:
+            rc = lib.sjhip_neuron_forward_pieces(
+                neuron, dtype, ctypes.byref(params), T, N, chunk,
+                x_seq.data_ptr(), v_init.data_ptr(), k_ptr,
+                spike_seq.data_ptr(), v_seq.data_ptr() if store_v_seq else None, v_last.data_ptr(),
+                checkpoints.data_ptr(), stream,
+            )
+        else:
+            rc = lib.sjhip_neuron_forward(
+                neuron, dtype, ctypes.byref(params), T, N,
+                x_seq.data_ptr(), v_init.data_ptr(), k_ptr,
+                spike_seq.data_ptr(), v_seq.data_ptr() if store_v_seq else None, v_last.data_ptr(),
+                h_seq.data_ptr() if save_h else None, stream,
+            )
     L.check(rc, "neuron_forward")
     del k_keep
-    return spike_seq, v_seq, v_last, h_seq
+    return spike_seq, v_seq, v_last, (h_seq if checkpoints is None else checkpoints)
 
 
 def packed_supported(n_neurons: int) -> bool:
@@ -177,8 +199,12 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
                   grad_v_last: Optional[torch.Tensor], h_seq: torch.Tensor, x_seq: Optional[torch.Tensor],
                   v_init: Optional[torch.Tensor], k: Optional[torch.Tensor], tau: float, v_th: float,
                   v_reset: float, flags: int, sg_id: int, sg_alpha: float, need_grad_v_init: bool = True,
-                  qif: tuple[float, float, float] = _NO_EXTRA, levels: tuple[float, float, float] = _NO_EXTRA
+                  qif: tuple[float, float, float] = _NO_EXTRA, levels: tuple[float, float, float] = _NO_EXTRA,
+                  chunk: int = 0, checkpoints: Optional[torch.Tensor] = None
                   ) -> tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """``(grad_x_seq, grad_v_init, grad_k)``.  ``x_seq`` given: the replaying backward; with ``chunk > 0`` and the
+    forward's ``checkpoints`` a long sequence is walked piece by piece from the last to the first, each piece replayed
+    from its checkpoint, the gradient of a piece's initial state being the ``grad_v_last`` of the piece before it."""
     recompute = x_seq is not None
     if not recompute and h_seq is None:
         raise ValueError("backward needs h_seq, or x_seq and v_init to recompute it")
@@ -189,15 +215,15 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
     else:
         h_seq = h_seq.contiguous()
         fix = lambda t: t.contiguous()
+    broadcast = 0
     if v_init is not None:
         v_init, broadcast = _state_arg(v_init, recompute)
-        flags |= broadcast
     L.require_device_tensor("h_seq", h_seq)
     dtype = L.dtype_id(h_seq.dtype)
     T, N = h_seq.shape
-    if grad_spike_seq is None:
-        grad_spike_seq = torch.zeros_like(h_seq)
-    grad_spike_seq = fix(grad_spike_seq.to(h_seq.dtype))
+    pieces = len(_chunks(T, chunk if (recompute and checkpoints is not None) else 0))
+    if grad_spike_seq is not None:  # None (a loss on v alone): the kernels read nothing in its place
+        grad_spike_seq = fix(grad_spike_seq.to(h_seq.dtype))
     if grad_v_seq is not None:
         grad_v_seq = fix(grad_v_seq.to(h_seq.dtype))
     if grad_v_last is not None:
@@ -205,6 +231,7 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
     grad_x_seq = torch.empty_like(h_seq)
     # a state that needs no gradient (the usual case: it was the reset value) costs no [N] write
     grad_v_init = h_seq.new_empty((N,) if need_grad_v_init else (0,))
+    carry = h_seq.new_empty((N,)) if pieces > 1 else None  # gradient handed from a piece to the one before
     grad_k = workspace = None
     k_keep, k_ptr = _k_pointer(k, h_seq)
     if neuron == L.NEURON_PLIF:
@@ -214,23 +241,32 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
             grad_k = torch.empty((), dtype=torch.float32, device=h_seq.device)
             workspace = torch.empty((L.load().sjhip_plif_workspace_floats(dtype, N),), dtype=torch.float32,
                                     device=h_seq.device)
-    params = _params(tau, v_th, v_reset, sg_alpha, sg_id, flags, qif, levels)
+    needs_state = neuron in (L.NEURON_PLIF, L.NEURON_QIF, L.NEURON_EIF)
+    params = _params(tau, v_th, v_reset, sg_alpha, sg_id, flags | broadcast, qif, levels)
+    carry_out = grad_v_init.data_ptr() if need_grad_v_init else None
+    lib = L.load()
     with torch.cuda.device(h_seq.device):
-        if recompute:
-            rc = L.load().sjhip_neuron_backward_recompute(
+        stream = L.current_stream_ptr(h_seq.device)
+        if pieces > 1:
+            rc = lib.sjhip_neuron_backward_recompute_pieces(
+                neuron, dtype, ctypes.byref(params), T, N, chunk,
+                h_seq.data_ptr(), v_init.data_ptr(), k_ptr, L.aligned16(checkpoints).data_ptr(),
+                L.ptr(grad_spike_seq), L.ptr(grad_v_seq), L.ptr(grad_v_last),
+                grad_x_seq.data_ptr(), carry_out, L.ptr(grad_k), L.ptr(workspace), carry.data_ptr(), stream,
+            )
+        elif recompute:
+            rc = lib.sjhip_neuron_backward_recompute(
                 neuron, dtype, ctypes.byref(params), T, N,
                 h_seq.data_ptr(), v_init.data_ptr(), k_ptr,
-                grad_spike_seq.data_ptr(), L.ptr(grad_v_seq), L.ptr(grad_v_last),
-                grad_x_seq.data_ptr(), grad_v_init.data_ptr() if need_grad_v_init else None, L.ptr(grad_k),
-                L.ptr(workspace), L.current_stream_ptr(h_seq.device),
+                L.ptr(grad_spike_seq), L.ptr(grad_v_seq), L.ptr(grad_v_last),
+                grad_x_seq.data_ptr(), carry_out, L.ptr(grad_k), L.ptr(workspace), stream,
             )
         else:
-            rc = L.load().sjhip_neuron_backward(
+            rc = lib.sjhip_neuron_backward(
                 neuron, dtype, ctypes.byref(params), T, N,
-                grad_spike_seq.data_ptr(), L.ptr(grad_v_seq), L.ptr(grad_v_last), h_seq.data_ptr(),
-                L.ptr(v_init) if neuron in (L.NEURON_PLIF, L.NEURON_QIF, L.NEURON_EIF) else None, k_ptr,
-                grad_x_seq.data_ptr(), grad_v_init.data_ptr() if need_grad_v_init else None, L.ptr(grad_k), L.ptr(workspace),
-                L.current_stream_ptr(h_seq.device),
+                L.ptr(grad_spike_seq), L.ptr(grad_v_seq), L.ptr(grad_v_last), h_seq.data_ptr(),
+                L.ptr(v_init) if needs_state else None, k_ptr,
+                grad_x_seq.data_ptr(), carry_out, L.ptr(grad_k), L.ptr(workspace), stream,
             )
     L.check(rc, "neuron_backward_recompute" if recompute else "neuron_backward")
     del k_keep
@@ -807,10 +843,11 @@ class _EagerNeuron(torch.autograd.Function):
 
     @staticmethod
     def forward(x_seq, v_init, k, spec):
-        neuron, tau, v_th, v_reset, flags, _, _, store_v_seq, recompute, qif, levels = spec
-        s, v_seq, v_last, h_seq = _run_forward(neuron, x_seq, v_init, k, tau, v_th, v_reset, flags, store_v_seq,
-                                               not recompute, qif, levels)
-        return s, v_seq, v_last, (h_seq if h_seq is not None else x_seq.new_empty((0,)))
+        neuron, tau, v_th, v_reset, flags, _, _, store_v_seq, recompute, qif, levels, chunk = spec
+        s, v_seq, v_last, kept = _run_forward(neuron, x_seq, v_init, k, tau, v_th, v_reset, flags, store_v_seq,
+                                              not recompute, qif, levels, chunk)
+        # kept: h_seq (saved-h route), the checkpoints of a sequence replayed piece by piece, or nothing
+        return s, v_seq, v_last, (kept if kept is not None else x_seq.new_empty((0,)))
 
     @staticmethod
     def setup_context(ctx, inputs, output):
@@ -819,22 +856,38 @@ class _EagerNeuron(torch.autograd.Function):
         ctx.spec = spec
         # PLIF and QIF need the state before the first step in either backward; the replay needs it to start from
         keep_v_init = recompute or neuron in (L.NEURON_PLIF, L.NEURON_QIF, L.NEURON_EIF)
-        ctx.save_for_backward(x_seq if recompute else output[3], v_init if keep_v_init else None, k)
+        ctx.save_for_backward(x_seq if recompute else output[3], v_init if keep_v_init else None, k,
+                              output[3] if (recompute and output[3].numel() > 0) else None)
         ctx.mark_non_differentiable(output[3])
         ctx.set_materialize_grads(False)
 
     @staticmethod
     def backward(ctx, grad_spike_seq, grad_v_seq, grad_v_last, grad_h_seq):
         del grad_h_seq
-        neuron, tau, v_th, v_reset, flags, sg_id, sg_alpha, store_v_seq, recompute, qif, levels = ctx.spec
-        first, v_init, k = ctx.saved_tensors
+        neuron, tau, v_th, v_reset, flags, sg_id, sg_alpha, store_v_seq, recompute, qif, levels, chunk = ctx.spec
+        first, v_init, k, checkpoints = ctx.saved_tensors
         h_seq, x_seq = (None, first) if recompute else (first, None)
         need = bool(ctx.needs_input_grad[1])
         gx, gvi, gk = _run_backward(neuron, grad_spike_seq, _none_if_empty_grad(grad_v_seq, store_v_seq), grad_v_last,
-                                    h_seq, x_seq, v_init, k, tau, v_th, v_reset, flags, sg_id, sg_alpha, need, qif, levels)
+                                    h_seq, x_seq, v_init, k, tau, v_th, v_reset, flags, sg_id, sg_alpha, need, qif, levels,
+                                    chunk, checkpoints)
         if gk is not None:
             gk = gk.reshape(k.shape).to(k.dtype)
         return gx, (gvi if need else None), gk, None
+
+
+def replay_chunk(dtype: torch.dtype, T: int, N: int, flags: int) -> int:
+    """Steps per piece when a sequence of ``T`` steps should be replayed piece by piece in the backward, else 0: the
+    replay is switched on, one piece of the configured length is a shape the replay kernel prefers, and the sequence
+    is longer than that."""
+    from ... import configure
+
+    chunk = int(configure.hip_replay_chunk)
+    if not configure.hip_backward_recompute or chunk <= 0 or T <= chunk:
+        return 0
+    if dtype != torch.float32 and flags & L.FLAG_FP32_STATE:
+        return 0  # a checkpoint in the storage dtype would round the fp32 state
+    return chunk if L.recompute_preferred(dtype, chunk, N, flags) else 0
 
 
 def eager_multistep(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: Optional[torch.Tensor], tau: float,
@@ -846,7 +899,13 @@ def eager_multistep(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: O
     compiler.  ``flags`` is the complete flag word (``_flags``); ``need_grad`` selects the training path (saves
     ``h_seq``, or ``x_seq`` and ``v_init`` with ``recompute``) or the inference path (saves nothing)."""
     if need_grad:
-        spec = (neuron, tau, v_th, v_reset, flags, sg_id, sg_alpha, store_v_seq, recompute, qif, levels)
+        chunk = 0
+        if not recompute:
+            # a sequence too long to replay in one piece (its h would not fit in LDS with enough resident wavefronts) is
+            # replayed in pieces from checkpoints of the state, instead of saving and re-reading h_seq
+            chunk = replay_chunk(x_seq.dtype, x_seq.shape[0], x_seq.shape[1], flags)
+            recompute = chunk > 0
+        spec = (neuron, tau, v_th, v_reset, flags, sg_id, sg_alpha, store_v_seq, recompute, qif, levels, chunk)
         return _EagerNeuron.apply(x_seq, v_init, k, spec)[:3]
     return _run_forward(neuron, x_seq.detach(), v_init.detach(), None if k is None else k.detach(), tau, v_th, v_reset,
                         flags, store_v_seq, False, qif, levels)[:3]

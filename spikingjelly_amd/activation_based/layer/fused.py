@@ -10,6 +10,7 @@ from typing import Optional
 import torch
 import torch.nn as nn
 
+from ... import configure
 from .. import neuron
 
 
@@ -59,7 +60,7 @@ def conv_bn_lif(x_seq: torch.Tensor, conv: Optional[nn.Module], bn: nn.Module, n
     represents exactly (spikes)."""
     from ..hip_kernel import conv_bn_lif as C
 
-    if (torch.compiler.is_compiling() or type(node) is not neuron.LIFNode or node.backend != "hip" or node.step_mode != "m"
+    if (not configure.hip_fuse_conv_bn_lif or torch.compiler.is_compiling() or type(node) is not neuron.LIFNode or node.backend != "hip" or node.step_mode != "m"
             or node.store_v_seq or x_seq.dim() < 4):
         return None
     if conv is not None and (not _pointwise(conv) or x_seq.shape[2] != conv.in_channels):

@@ -37,7 +37,15 @@ hip_half_precision_mode = "torch"
 # 3 keeps the accuracy of an fp32 GEMM (six matrix-core products per pair of real operands, three when one operand is
 # spikes), 2 gives about 2^-17 relative per product at half the products, 1 is a plain bf16 GEMM.
 hip_conv_terms = 3
+# False: modules keep torch's convolution and batch norm around the hip neurons even where the fused
+# convolution / batch norm / LIF kernels could serve the chain (layer/fused.py).
+hip_fuse_conv_bn_lif = True
 hip_backward_recompute = True
+# Sequences longer than the replaying backward prefers in one piece (its LDS buffer for h grows with T) run, outside a
+# tracing compiler, as pieces of this many steps: the forward leaves the state after every piece ([T / chunk, N], in
+# place of a [T, N] h_seq), the backward replays piece by piece from those checkpoints.  0 switches it off (such
+# sequences then save h_seq).
+hip_replay_chunk = 16
 hip_lif_reciprocal_tau = False
 hip_plif_atomic_reduce = False
 

@@ -175,7 +175,7 @@ template <typename S, bool VECTOR, bool SHORT = false> struct BwdPrologue {
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int64_t t = a.T - 1 - i;
-      gs[i] = (t >= 0) ? A::load(gsp + t * a.N) : A::zero();
+      gs[i] = (t >= 0 && a.grad_spike) ? A::load(gsp + t * a.N) : A::zero();  // no spike gradient: zeros, nothing read
       if (a.grad_v_seq) gv[i] = (t >= 0) ? A::load(gvp + t * a.N) : A::zero();
     }
   }
@@ -196,6 +196,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
   if (!active) return acc_total;
 
   const int64_t N = a.N, T = a.T;
+  const bool has_gs = a.grad_spike != nullptr;  // a loss on the membrane potential alone sends no spike gradient
   const E *gsp = (const E *)a.grad_spike + col;
   const E *hp = HLDS ? nullptr : (const E *)a.h + col;
   const E *gvp = GVFULL ? (const E *)a.grad_v_seq + col : nullptr;
@@ -217,7 +218,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int64_t t = T - 1 - i;
-      ahead_gs[i] = (t >= 0) ? A::load(gsp + t * N) : A::zero();
+      ahead_gs[i] = (t >= 0 && has_gs) ? A::load(gsp + t * N) : A::zero();
       ahead_h[i] = (t >= 0) ? A::load(hp + t * N) : A::zero();
       if (GVFULL) ahead_gv[i] = (t >= 0) ? A::load(gvp + t * N) : A::zero();
     }
@@ -247,7 +248,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
     for (int i = 0; i < PF; ++i) {
       const int64_t tn = t0 - PF - i;
       if (tn >= 0) {
-        ahead_gs[i] = A::load(gsp + tn * N);
+        if (has_gs) ahead_gs[i] = A::load(gsp + tn * N);
         if (!HLDS) ahead_h[i] = A::load(hp + tn * N);
         if (GVFULL) ahead_gv[i] = A::load(gvp + tn * N);
       }

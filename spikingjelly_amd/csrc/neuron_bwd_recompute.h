@@ -95,6 +95,88 @@ __device__ __forceinline__ void recompute_reset_dispatch(const FwdArgs &a, f32x4
   else recompute_body<S, ROUND_EACH, CH, RESET_HARD, SHORT>(a, lds_h, col);
 }
 
+// Phase 1 for one work-item: dispatch on the charge equation.
+template <typename S, bool ROUND_EACH, bool SHORT>
+__device__ __forceinline__ void recompute_charge_dispatch(const FwdArgs &f, f32x4 *lds_h, int64_t col) {
+  switch (f.charge) {
+    case CH_IF: recompute_reset_dispatch<S, ROUND_EACH, CH_IF, SHORT>(f, lds_h, col); break;
+    case CH_DECAY_INPUT_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_DECAY_INPUT_DIV, SHORT>(f, lds_h, col); break;
+    case CH_DECAY_INPUT_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_DECAY_INPUT_MUL, SHORT>(f, lds_h, col); break;
+    case CH_PLAIN_INPUT_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_PLAIN_INPUT_DIV, SHORT>(f, lds_h, col); break;
+    case CH_QIF_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_QIF_DIV, SHORT>(f, lds_h, col); break;
+    case CH_QIF_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_QIF_MUL, SHORT>(f, lds_h, col); break;
+    case CH_EIF_DIV: recompute_reset_dispatch<S, ROUND_EACH, CH_EIF_DIV, SHORT>(f, lds_h, col); break;
+    case CH_EIF_MUL: recompute_reset_dispatch<S, ROUND_EACH, CH_EIF_MUL, SHORT>(f, lds_h, col); break;
+    default: recompute_reset_dispatch<S, ROUND_EACH, CH_PLAIN_INPUT_MUL, SHORT>(f, lds_h, col); break;
+  }
+}
+
+// Makes wavefront-uniform scalars opaque to the optimiser at this point, so that values derived from them (copies of
+// scalars into vector registers, folded constants of every surrogate's branch) are formed inside the enclosing loop
+// iteration and die there, instead of being hoisted in front of the loop and held in registers across all of its
+// branches (measured on the kernel below: 256 registers plus 100 to 190 bytes of spills without, 222 and none with).
+template <typename T> __device__ __forceinline__ void keep_scalar_local(T &x) { asm volatile("" : "+s"(x)); }
+template <typename... Ts> __device__ __forceinline__ void keep_uniform_local(Ts &...x) { (keep_scalar_local(x), ...); }
+
+__device__ __forceinline__ void keep_uniform_local(FwdArgs &a) {
+  keep_uniform_local(a.x, a.v_init, a.T, a.N);
+}
+
+__device__ __forceinline__ void keep_uniform_local(BwdArgs &a) {
+  keep_uniform_local(a.grad_spike, a.grad_v_seq, a.grad_v_last, a.v_init, a.grad_x, a.grad_v_init, a.T, a.N, a.sg, a.soft_reset,
+                     a.decay_input, a.is_if, a.exponential, a.detach_reset, a.round_each, a.v_init_broadcast);
+}
+
+// A sequence too long for one LDS buffer, walked piece by piece from the last to the first inside one launch: each
+// piece is replayed from its checkpoint (left by forward_pieces_kernel) into the same LDS buffer of `chunk` steps and
+// walked back; the gradient of the piece's initial state goes through p.carry to the piece before it.  The two phases
+// are the ones of backward_recompute_kernel, called with the pointers and the length of the piece.
+template <typename S, bool ROUND_EACH, int MODE>
+__global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_pieces_kernel(const FwdArgs f0, const BwdArgs b0,
+                                                                                    const PieceArgs p) {
+  extern __shared__ f32x4 lds_h[];
+  typedef typename Acc<S, true, true>::elem_t E;
+  constexpr int V = Acc<S, true, true>::V;
+  static_assert(!BwdModeOf<MODE>::SHORT, "pieces are long enough for the deep prefetch");
+  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
+  const bool active = col < b0.N;
+  const float k = b0.k_device ? *b0.k_device : b0.k;
+  constexpr int HLDS = (ROUND_EACH && sizeof(S) == 2) ? 2 : 1;
+  const int64_t N = b0.N;
+  float part = 0.0f;
+  for (int64_t j = p.pieces - 1; j >= 0; --j) {
+    const int64_t t0 = j * p.chunk;
+    const int64_t len = (b0.T - t0 < p.chunk) ? b0.T - t0 : p.chunk;
+    FwdArgs f = f0;
+    BwdArgs b = b0;
+    f.T = len; b.T = len;
+    f.x = (const E *)f0.x + t0 * N;
+    if (j > 0) {
+      f.v_init = (const E *)p.checkpoints + (j - 1) * N;
+      f.v_init_broadcast = 0;
+      b.grad_v_init = p.carry;
+    }
+    b.v_init = f.v_init;
+    b.v_init_broadcast = f.v_init_broadcast;
+    if (b0.grad_spike) b.grad_spike = (const E *)b0.grad_spike + t0 * N;
+    if (b0.grad_v_seq) b.grad_v_seq = (const E *)b0.grad_v_seq + t0 * N;
+    b.grad_x = (E *)b0.grad_x + t0 * N;
+    if (j + 1 < p.pieces) b.grad_v_last = p.carry;
+    keep_uniform_local(f);
+    keep_uniform_local(b);
+    float kj = k;
+    keep_scalar_local(kj);
+    // request the last rows of the piece's upstream gradients now, so they arrive while h is being replayed
+    BwdPrologue<S, true, false> pre;
+    if (active) {
+      pre.load(b, col);
+      recompute_charge_dispatch<S, ROUND_EACH, false>(f, lds_h, col);
+    }
+    part += backward_sg_dispatch<S, true, MODE, HLDS>(b, active, col, kj, lds_h, &pre);
+  }
+  if (BwdModeOf<MODE>::BASE == BWD_PLIF) plif_block_reduce(b0, part, k);
+}
+
 template <typename S, bool ROUND_EACH, int MODE>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_kernel(const FwdArgs f, const BwdArgs b) {
   extern __shared__ f32x4 lds_h[];
@@ -128,6 +210,6 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_kernel(con
 // instantiated once per dtype (neuron_bwd_recompute_{f32,f16,bf16}.hip).
 template <typename S>
 int launch_recompute_dtype(const FwdArgs &f, const BwdArgs &b, bool round_each, int mode, int block, unsigned lds,
-                           int64_t blocks, hipStream_t stream);
+                           int64_t blocks, hipStream_t stream, const PieceArgs *pieces = nullptr);
 
 }  // namespace sjhip

@@ -6,11 +6,11 @@
 
 namespace sjhip {
 
-extern template int launch_recompute_dtype<float>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
-extern template int launch_recompute_dtype<f16_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
-extern template int launch_recompute_dtype<bf16_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
-extern template int launch_recompute_dtype<f16n_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
-extern template int launch_recompute_dtype<bf16n_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
+extern template int launch_recompute_dtype<float>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t, const PieceArgs *);
+extern template int launch_recompute_dtype<f16_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t, const PieceArgs *);
+extern template int launch_recompute_dtype<bf16_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t, const PieceArgs *);
+extern template int launch_recompute_dtype<f16n_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t, const PieceArgs *);
+extern template int launch_recompute_dtype<bf16n_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t, const PieceArgs *);
 
 namespace {
 
@@ -44,12 +44,16 @@ bool recompute_preferred(int dtype, int64_t T, int64_t N, bool round_each) {
   return 4 * T * 64 * h_bytes_per_item(dtype, round_each) <= (int64_t)kMaxLds;
 }
 
-int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
-                              const void *x_seq, const void *v_init, const float *k_device,
-                              const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
-                              void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace,
-                              hipStream_t stream) {
-  if (!recompute_supported(dtype, T, N))
+namespace {
+
+// One launch over the whole sequence (chunk == 0: T steps of h in LDS) or over pieces of `chunk` steps.
+int launch_replay(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N, int64_t chunk,
+                  const void *x_seq, const void *v_init, const float *k_device, const void *checkpoints,
+                  const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                  void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace, void *carry,
+                  hipStream_t stream) {
+  const int64_t lds_steps = chunk > 0 ? chunk : T;
+  if (!recompute_supported(dtype, lds_steps, N))
     return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute): T=%lld N=%lld does not fit (N %% %d != 0 or T too large for LDS)",
                 (long long)T, (long long)N, dtype == SJHIP_F32 ? 4 : 8);
   const bool broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) != 0;
@@ -70,26 +74,30 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
 
   const bool narrow = dtype != SJHIP_F32 && !round_each;  // 16-bit storage, fp32 state: four neurons per work-item
   const int V = (dtype == SJHIP_F32 || narrow) ? 4 : 8;
-  const int block = recompute_block(dtype, T, round_each);
+  const int block = recompute_block(dtype, lds_steps, round_each);
   const int64_t items = N / V;
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "backward(recompute): N=%lld", (long long)N);
-  unsigned lds = (unsigned)(T * block * h_bytes_per_item(dtype, round_each));
+  unsigned lds = (unsigned)(lds_steps * block * h_bytes_per_item(dtype, round_each));
   const unsigned cap = occupancy_cap_lds(tuning().replay_blocks_per_cu);
   if (cap > lds) lds = cap;
   const bool plif = neuron == SJHIP_NEURON_PLIF;
   const int mode = plif ? BWD_PLIF : ((neuron == SJHIP_NEURON_QIF || neuron == SJHIP_NEURON_EIF) ? BWD_QIF : BWD_PLAIN);
+  PieceArgs piece_args;
+  piece_args.checkpoints = const_cast<void *>(checkpoints); piece_args.carry = carry; piece_args.chunk = chunk;
+  piece_args.pieces = chunk > 0 ? (T + chunk - 1) / chunk : 1;
+  const PieceArgs *pieces = chunk > 0 ? &piece_args : nullptr;
   {
     ProfileScope prof(KC_BACKWARD, stream);
     switch (dtype) {
-      case SJHIP_F32: rc = launch_recompute_dtype<float>(f, b, false, mode, block, lds, blocks, stream); break;
+      case SJHIP_F32: rc = launch_recompute_dtype<float>(f, b, false, mode, block, lds, blocks, stream, pieces); break;
       case SJHIP_F16:
-        rc = narrow ? launch_recompute_dtype<f16n_t>(f, b, false, mode, block, lds, blocks, stream)
-                    : launch_recompute_dtype<f16_t>(f, b, round_each, mode, block, lds, blocks, stream);
+        rc = narrow ? launch_recompute_dtype<f16n_t>(f, b, false, mode, block, lds, blocks, stream, pieces)
+                    : launch_recompute_dtype<f16_t>(f, b, round_each, mode, block, lds, blocks, stream, pieces);
         break;
       case SJHIP_BF16:
-        rc = narrow ? launch_recompute_dtype<bf16n_t>(f, b, false, mode, block, lds, blocks, stream)
-                    : launch_recompute_dtype<bf16_t>(f, b, round_each, mode, block, lds, blocks, stream);
+        rc = narrow ? launch_recompute_dtype<bf16n_t>(f, b, false, mode, block, lds, blocks, stream, pieces)
+                    : launch_recompute_dtype<bf16_t>(f, b, round_each, mode, block, lds, blocks, stream, pieces);
         break;
       default: return fail(SJHIP_ERR_INVALID, "backward(recompute): dtype %d", dtype);
     }
@@ -97,6 +105,28 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
   }
   if (plif && !b.atomic_reduce) return launch_plif_reduce(b, blocks, grad_rtau, stream);
   return SJHIP_OK;
+}
+
+}  // namespace
+
+int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
+                              const void *x_seq, const void *v_init, const float *k_device,
+                              const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                              void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace,
+                              hipStream_t stream) {
+  return launch_replay(neuron, dtype, p, T, N, 0, x_seq, v_init, k_device, nullptr, grad_spike_seq, grad_v_seq, grad_v_last,
+                       grad_x_seq, grad_v_init, grad_rtau, workspace, nullptr, stream);
+}
+
+int launch_backward_recompute_pieces(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N, int64_t chunk,
+                                     const void *x_seq, const void *v_init, const float *k_device, const void *checkpoints,
+                                     const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                                     void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace, void *carry,
+                                     hipStream_t stream) {
+  if (chunk < 1 || (T > chunk && (checkpoints == nullptr || carry == nullptr)) || !aligned16(checkpoints) || !aligned16(carry))
+    return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): chunk=%lld needs 16-byte aligned checkpoints and carry", (long long)chunk);
+  return launch_replay(neuron, dtype, p, T, N, chunk, x_seq, v_init, k_device, checkpoints, grad_spike_seq, grad_v_seq,
+                       grad_v_last, grad_x_seq, grad_v_init, grad_rtau, workspace, carry, stream);
 }
 
 }  // namespace sjhip

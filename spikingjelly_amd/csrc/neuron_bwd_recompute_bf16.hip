@@ -2,5 +2,5 @@
 #include "neuron_bwd_recompute_launch.h"
 
 namespace sjhip {
-template int launch_recompute_dtype<bf16_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t);
+template int launch_recompute_dtype<bf16_t>(const FwdArgs &, const BwdArgs &, bool, int, int, unsigned, int64_t, hipStream_t, const PieceArgs *);
 }  // namespace sjhip

@@ -28,8 +28,22 @@ int launch_kernel(const FwdArgs &f, const BwdArgs &b, int block, unsigned lds, i
   return check_launch("backward(recompute)");
 }
 
+template <typename S, bool ROUND_EACH, int MODE>
+int launch_pieces_kernel(const FwdArgs &f, const BwdArgs &b, const PieceArgs &p, int block, unsigned lds, int64_t blocks,
+                         hipStream_t stream) {
+  hipLaunchKernelGGL((backward_recompute_pieces_kernel<S, ROUND_EACH, MODE>), dim3((unsigned)blocks), dim3(block), lds, stream,
+                     f, b, p);  // a piece's LDS buffer stays below the default 64 KiB limit
+  return check_launch("backward(recompute, pieces)");
+}
+
 template <typename S, bool ROUND_EACH>
-int launch_mode(const FwdArgs &f, const BwdArgs &b, int mode, int block, unsigned lds, int64_t blocks, hipStream_t stream) {
+int launch_mode(const FwdArgs &f, const BwdArgs &b, int mode, int block, unsigned lds, int64_t blocks, hipStream_t stream,
+                const PieceArgs *pieces) {
+  if (pieces) {
+    if (mode == BWD_PLIF) return launch_pieces_kernel<S, ROUND_EACH, BWD_PLIF>(f, b, *pieces, block, lds, blocks, stream);
+    if (mode == BWD_QIF) return launch_pieces_kernel<S, ROUND_EACH, BWD_QIF>(f, b, *pieces, block, lds, blocks, stream);
+    return launch_pieces_kernel<S, ROUND_EACH, BWD_PLAIN>(f, b, *pieces, block, lds, blocks, stream);
+  }
   if (b.T <= kShortSequence) {
     if (mode == BWD_PLIF) return launch_kernel<S, ROUND_EACH, BWD_PLIF | BWD_SHORT>(f, b, block, lds, blocks, stream);
     if (mode == BWD_QIF) return launch_kernel<S, ROUND_EACH, BWD_QIF | BWD_SHORT>(f, b, block, lds, blocks, stream);
@@ -42,12 +56,12 @@ int launch_mode(const FwdArgs &f, const BwdArgs &b, int mode, int block, unsigne
 
 template <typename S>
 int launch_recompute_dtype(const FwdArgs &f, const BwdArgs &b, bool round_each, int mode, int block, unsigned lds,
-                           int64_t blocks, hipStream_t stream) {
+                           int64_t blocks, hipStream_t stream, const PieceArgs *pieces) {
   // the 8-byte access tags exist for fp32 state only
   if constexpr (std::is_same<S, f16_t>::value || std::is_same<S, bf16_t>::value) {
-    if (round_each) return launch_mode<S, true>(f, b, mode, block, lds, blocks, stream);
+    if (round_each) return launch_mode<S, true>(f, b, mode, block, lds, blocks, stream, pieces);
   }
-  return launch_mode<S, false>(f, b, mode, block, lds, blocks, stream);
+  return launch_mode<S, false>(f, b, mode, block, lds, blocks, stream, pieces);
 }
 
 }  // namespace sjhip

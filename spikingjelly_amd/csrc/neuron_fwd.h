@@ -335,6 +335,39 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) forward_kernel(const FwdArgs 
   }
 }
 
+// The same forward over a long sequence cut into pieces, in one launch: piece j runs forward_body on rows
+// [j chunk, (j + 1) chunk) starting from the state piece j - 1 left in the checkpoint row, which the same work-item
+// wrote.  What remains in `checkpoints` is what the replaying backward starts each piece from.
+template <typename S, bool ROUND_EACH>
+__global__ void __launch_bounds__(SJHIP_MAX_BLOCK) forward_pieces_kernel(const FwdArgs a, const PieceArgs p) {
+  typedef typename Acc<S, true, false>::elem_t E;
+  for (int64_t j = 0; j < p.pieces; ++j) {
+    FwdArgs f = a;
+    const int64_t t0 = j * p.chunk;
+    f.T = (a.T - t0 < p.chunk) ? a.T - t0 : p.chunk;
+    f.x = (const E *)a.x + t0 * a.N;
+    f.spike = (E *)a.spike + t0 * a.N;
+    if (a.v_seq) f.v_seq = (E *)a.v_seq + t0 * a.N;
+    f.h = nullptr;
+    if (j > 0) {
+      f.v_init = (const E *)p.checkpoints + (j - 1) * a.N;
+      f.v_init_broadcast = 0;
+    }
+    if (j + 1 < p.pieces) f.v_last = (E *)p.checkpoints + j * a.N;
+    switch (f.charge) {
+      case CH_IF: forward_reset_dispatch<S, true, ROUND_EACH, CH_IF, FWD_OUT_DENSE>(f); break;
+      case CH_DECAY_INPUT_DIV: forward_reset_dispatch<S, true, ROUND_EACH, CH_DECAY_INPUT_DIV, FWD_OUT_DENSE>(f); break;
+      case CH_DECAY_INPUT_MUL: forward_reset_dispatch<S, true, ROUND_EACH, CH_DECAY_INPUT_MUL, FWD_OUT_DENSE>(f); break;
+      case CH_PLAIN_INPUT_DIV: forward_reset_dispatch<S, true, ROUND_EACH, CH_PLAIN_INPUT_DIV, FWD_OUT_DENSE>(f); break;
+      case CH_QIF_DIV: forward_reset_dispatch<S, true, ROUND_EACH, CH_QIF_DIV, FWD_OUT_DENSE>(f); break;
+      case CH_QIF_MUL: forward_reset_dispatch<S, true, ROUND_EACH, CH_QIF_MUL, FWD_OUT_DENSE>(f); break;
+      case CH_EIF_DIV: forward_reset_dispatch<S, true, ROUND_EACH, CH_EIF_DIV, FWD_OUT_DENSE>(f); break;
+      case CH_EIF_MUL: forward_reset_dispatch<S, true, ROUND_EACH, CH_EIF_MUL, FWD_OUT_DENSE>(f); break;
+      default: forward_reset_dispatch<S, true, ROUND_EACH, CH_PLAIN_INPUT_MUL, FWD_OUT_DENSE>(f); break;
+    }
+  }
+}
+
 // ---- host side: turn the ABI parameters into kernel arguments ------------------------------------
 inline int build_fwd_args(FwdArgs &a, bool &round_each, int neuron, int dtype, const sjhip_neuron_params &p,
                           int64_t T, int64_t N, const void *x_seq, const void *v_init, const float *k_device,

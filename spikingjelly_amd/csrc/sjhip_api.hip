@@ -229,7 +229,7 @@ int check_backward(int neuron, int dtype, const sjhip_neuron_params *p, int64_t 
   if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_MULTI_LEVEL) return fail(SJHIP_ERR_UNSUPPORTED, "backward: surrogate id %d", p->sg_id);
   int rc = check_shape("backward", T, N);
   if (rc != SJHIP_OK) return rc;
-  if (!grad_spike_seq || !h_seq || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward: NULL tensor");
+  if (!h_seq || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward: NULL tensor");
   rc = check_levels("backward", neuron, *p, true);
   if (rc != SJHIP_OK) return rc;
   if ((neuron == SJHIP_NEURON_QIF || neuron == SJHIP_NEURON_EIF) && grad_v_init && !v_init)
@@ -335,7 +335,7 @@ int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_pa
   if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_MULTI_LEVEL) return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute): surrogate id %d", p->sg_id);
   int rc = check_shape("backward(recompute)", T, N);
   if (rc != SJHIP_OK) return rc;
-  if (!x_seq || !v_init || !grad_spike_seq || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward(recompute): NULL tensor");
+  if (!x_seq || !v_init || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward(recompute): NULL tensor");
   rc = check_levels("backward(recompute)", neuron, *p, true);
   if (rc != SJHIP_OK) return rc;
   if (neuron == SJHIP_NEURON_PLIF) {
@@ -345,6 +345,56 @@ int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_pa
   return launch_backward_recompute(neuron, dtype, *p, T, N, x_seq, v_init, rtau_device, grad_spike_seq, grad_v_seq,
                                    grad_v_last, grad_x_seq, grad_v_init, grad_rtau, workspace,
                                    static_cast<hipStream_t>(stream));
+}
+
+int64_t sjhip_replay_pieces(int64_t T, int64_t chunk) { return (T < 1 || chunk < 1) ? 0 : (T + chunk - 1) / chunk; }
+
+int sjhip_neuron_forward_pieces(int neuron, int dtype, const sjhip_neuron_params *p, int64_t T, int64_t N, int64_t chunk,
+                                const void *x_seq, const void *v_init, const float *rtau_device, void *spike_seq,
+                                void *v_seq, void *v_last, void *checkpoints, void *stream) {
+  if (!p) return fail(SJHIP_ERR_INVALID, "forward(pieces): params is NULL");
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_EIF) return fail(SJHIP_ERR_INVALID, "forward(pieces): neuron %d", neuron);
+  if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "forward(pieces): dtype %d", dtype);
+  int rc = check_shape("forward(pieces)", T, N);
+  if (rc != SJHIP_OK) return rc;
+  if (chunk < 1) return fail(SJHIP_ERR_INVALID, "forward(pieces): chunk %lld", (long long)chunk);
+  if (!x_seq || !v_init || !spike_seq) return fail(SJHIP_ERR_INVALID, "forward(pieces): NULL tensor");
+  if (!v_seq && !v_last) return fail(SJHIP_ERR_INVALID, "forward(pieces): neither v_seq nor v_last given");
+  if (T > chunk && !checkpoints) return fail(SJHIP_ERR_INVALID, "forward(pieces): %lld pieces need checkpoints", (long long)sjhip_replay_pieces(T, chunk));
+  if (dtype != SJHIP_F32 && (p->flags & SJHIP_FLAG_FP32_STATE))
+    return fail(SJHIP_ERR_UNSUPPORTED, "forward(pieces): an fp32 state does not survive a checkpoint of 16-bit storage");
+  rc = check_levels("forward(pieces)", neuron, *p, false);
+  if (rc != SJHIP_OK) return rc;
+  if (neuron == SJHIP_NEURON_PLIF && !rtau_device) return fail(SJHIP_ERR_INVALID, "forward(pieces): PLIF needs rtau_device");
+  return launch_forward_pieces(neuron, dtype, *p, T, N, chunk, x_seq, v_init, rtau_device, spike_seq, v_seq, v_last, checkpoints,
+                               static_cast<hipStream_t>(stream));
+}
+
+int sjhip_neuron_backward_recompute_pieces(int neuron, int dtype, const sjhip_neuron_params *p, int64_t T, int64_t N,
+                                           int64_t chunk, const void *x_seq, const void *v_init, const float *rtau_device,
+                                           const void *checkpoints, const void *grad_spike_seq, const void *grad_v_seq,
+                                           const void *grad_v_last, void *grad_x_seq, void *grad_v_init, float *grad_rtau,
+                                           float *workspace, void *carry, void *stream) {
+  if (!p) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): params is NULL");
+  if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_EIF) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): neuron %d", neuron);
+  if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): dtype %d", dtype);
+  if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_MULTI_LEVEL) return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute, pieces): surrogate id %d", p->sg_id);
+  int rc = check_shape("backward(recompute, pieces)", T, N);
+  if (rc != SJHIP_OK) return rc;
+  if (chunk < 1) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): chunk %lld", (long long)chunk);
+  if (!x_seq || !v_init || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): NULL tensor");
+  if (T > chunk && (!checkpoints || !carry)) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): several pieces need checkpoints and carry");
+  if (dtype != SJHIP_F32 && (p->flags & SJHIP_FLAG_FP32_STATE))
+    return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute, pieces): an fp32 state does not survive a checkpoint of 16-bit storage");
+  rc = check_levels("backward(recompute, pieces)", neuron, *p, true);
+  if (rc != SJHIP_OK) return rc;
+  if (neuron == SJHIP_NEURON_PLIF) {
+    if (!grad_rtau || !rtau_device) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): PLIF needs rtau_device and grad_rtau");
+    if (!(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");
+  }
+  return launch_backward_recompute_pieces(neuron, dtype, *p, T, N, chunk, x_seq, v_init, rtau_device, checkpoints, grad_spike_seq,
+                                          grad_v_seq, grad_v_last, grad_x_seq, grad_v_init, grad_rtau, workspace, carry,
+                                          static_cast<hipStream_t>(stream));
 }
 
 int sjhip_stbif_forward(int dtype, uint32_t flags, int64_t T, int64_t N, const void *x_seq, const void *q_init,
@@ -480,6 +530,11 @@ int sjhip_ssa_backward(int dtype, int64_t samples, int heads, int channels_per_h
   if (!qkv || !grad_out || !grad_qkv) return fail(SJHIP_ERR_INVALID, "ssa_backward: NULL tensor");
   return launch_ssa(true, dtype, samples, heads, channels_per_head, tokens, scale, qkv, nullptr, grad_out, nullptr, grad_qkv,
                     static_cast<hipStream_t>(stream));
+}
+
+int sjhip_stream_probe(int reads, int writes, int nontemporal, int64_t floats_per_stream, const float *const *in,
+                       float *const *out, void *stream) {
+  return launch_stream_probe(reads, writes, nontemporal, floats_per_stream, in, out, static_cast<hipStream_t>(stream));
 }
 
 int64_t sjhip_pwconv_planes_elems(int64_t rows, int64_t cols) {

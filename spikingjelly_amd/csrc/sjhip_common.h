@@ -263,7 +263,7 @@ const Tuning &tuning();
 
 enum KernelClass { KC_FORWARD = 0, KC_BACKWARD = 1, KC_PLIF_REDUCE = 2, KC_BIT_PACK = 3, KC_BIT_UNPACK = 4,
                    KC_SSA_FORWARD = 5, KC_SSA_BACKWARD = 6, KC_PW_GEMM = 7, KC_PW_GRAD_WEIGHT = 8, KC_BN_STATS = 9,
-                   KC_BN_LIF_FORWARD = 10, KC_BN_LIF_BACKWARD = 11, KC_BN_GRAD_INPUT = 12, KC_COUNT = 13 };
+                   KC_BN_LIF_FORWARD = 10, KC_BN_LIF_BACKWARD = 11, KC_BN_GRAD_INPUT = 12, KC_STREAM_PROBE = 13, KC_COUNT = 14 };
 
 // Brackets one launch with events when profiling is on; free otherwise.
 class ProfileScope {
@@ -285,6 +285,17 @@ static inline bool exact_reciprocal(float f) {
   int e;
   return std::isfinite(f) && f > 0.0f && std::frexp(f, &e) == 0.5f && f <= 0x1p100f && f >= 0x1p-100f;
 }
+
+// A long sequence handled as consecutive pieces of `chunk` steps inside one launch: the forward leaves the state after
+// every piece but the last in `checkpoints` ([pieces - 1][N], storage dtype), the replaying backward starts each piece
+// from there and hands the gradient of a piece's initial state to the piece before it through `carry` ([N]).  A
+// work-item only ever reads back what it wrote itself, so no synchronisation is involved.
+struct PieceArgs {
+  void *checkpoints;
+  void *carry;
+  int64_t chunk;
+  int64_t pieces;
+};
 
 // Launchers (one per translation unit).
 int launch_forward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
@@ -322,6 +333,14 @@ int launch_backward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t
                     const void *h_seq, const void *v_init,
                     const float *k_device, void *grad_x_seq, void *grad_v_init, float *grad_rtau,
                     float *workspace, hipStream_t stream);
+int launch_forward_pieces(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N, int64_t chunk,
+                          const void *x_seq, const void *v_init, const float *k_device, void *spike_seq, void *v_seq,
+                          void *v_last, void *checkpoints, hipStream_t stream);
+int launch_backward_recompute_pieces(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N, int64_t chunk,
+                                     const void *x_seq, const void *v_init, const float *k_device, const void *checkpoints,
+                                     const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
+                                     void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace, void *carry,
+                                     hipStream_t stream);
 int launch_forward_packed(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
                           const void *x_seq, const void *v_init, const float *k_device, uint8_t *spike_bits,
                           void *v_seq, void *v_last, hipStream_t stream);
@@ -340,6 +359,8 @@ int launch_ssa(bool backward, int dtype, int64_t samples, int heads, int cph, in
                const uint8_t *qkv_bits, const void *grad_out, void *out, void *grad_qkv, hipStream_t stream);
 int launch_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, hipStream_t stream);
 int launch_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, hipStream_t stream);
+int launch_stream_probe(int reads, int writes, int nontemporal, int64_t floats_per_stream, const float *const *in,
+                        float *const *out, hipStream_t stream);
 int64_t pwconv_planes_elems(int64_t rows, int64_t cols);
 int launch_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, hipStream_t stream);
 int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,

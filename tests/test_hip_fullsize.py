@@ -151,14 +151,8 @@ def test_config4_full_size_if_fp16_inference_and_packing():
     assert torch.equal(v_next.cpu()[cols], ev[-1])
 
 
-def test_config5_full_size_block_matches_torch_backend():
-    """BASELINE config 5 at full size (T=4, B=64, 196 tokens, D=384, 12 heads): the block with backend='hip'
-    against the same block with backend='torch' on the same device and weights.  Convolutions and batch norms
-    are the same torch kernels, the LIF kernels are bit-exact and the contraction is exact, so the output
-    spikes must be identical; gradients agree to fp32 accuracy."""
-    from spikingjelly_amd.activation_based import functional, layer
-
-    from helpers import bits_equal
+def _config5_blocks():
+    from spikingjelly_amd.activation_based import layer
 
     torch.manual_seed(1005)
     a = layer.SpikingSelfAttention(384, 12, backend="torch").cuda()
@@ -166,6 +160,21 @@ def test_config5_full_size_block_matches_torch_backend():
     b.load_state_dict(a.state_dict())
     x = torch.randn((4, 64, 384, 196), generator=torch.Generator().manual_seed(1105)).cuda()
     g = torch.randn((4, 64, 384, 196), generator=torch.Generator().manual_seed(1205)).cuda()
+    return a, b, x, g
+
+
+def test_config5_full_size_block_matches_torch_backend(monkeypatch):
+    """BASELINE config 5 at full size (T=4, B=64, 196 tokens, D=384, 12 heads): the block with backend='hip' and the
+    convolution / batch-norm fusion switched off, against the same block with backend='torch' on the same device and
+    weights.  Convolutions and batch norms are then the same torch kernels, the LIF kernels are bit-exact and the
+    contraction is exact, so the output spikes must be identical; gradients agree to fp32 accuracy."""
+    from spikingjelly_amd import configure
+    from spikingjelly_amd.activation_based import functional
+
+    from helpers import bits_equal
+
+    monkeypatch.setattr(configure, "hip_fuse_conv_bn_lif", False)
+    a, b, x, g = _config5_blocks()
     xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
     ya = a(xa)
     ya.backward(g)
@@ -176,6 +185,39 @@ def test_config5_full_size_block_matches_torch_backend():
     assert bits_equal(yb, ya)
     torch.testing.assert_close(xb.grad, xa.grad, rtol=1e-3, atol=1e-4)
     torch.testing.assert_close(b.proj_conv_bn[0].weight.grad, a.proj_conv_bn[0].weight.grad, rtol=1e-3, atol=1e-3)
+    functional.reset_net(a)
+    functional.reset_net(b)
+
+
+def test_config5_full_size_fused_block_against_torch_backend():
+    """The same comparison with the fused convolution / batch norm / LIF kernels (the default).  Two fp32 convolutions
+    of different libraries differ in the last bits, so among the 290 million membrane potentials of the block a few
+    hundred land on the other side of a threshold; each such spike changes the attention of its (sample, head) and with
+    it the gradient of that sample's neighbourhood.  Expected values are therefore compared statistically: the output
+    spikes differ in fewer than one in ten thousand positions, the gradients agree within fp32 tolerance on more than
+    97 % of the elements and point the same way."""
+    from spikingjelly_amd.activation_based import functional
+
+    a, b, x, g = _config5_blocks()
+    xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
+    ya = a(xa)
+    ya.backward(g)
+    yb = b(xb)
+    yb.backward(g)
+    torch.cuda.synchronize()
+    assert 0.0 < float(ya.detach().mean()) < 0.5
+    assert float((yb != ya).float().mean()) < 1e-4
+
+    def agree(got, want, rtol, atol):
+        close = (got - want).abs() <= atol + rtol * want.abs()
+        cos = torch.nn.functional.cosine_similarity(got.flatten().double(), want.flatten().double(), dim=0)
+        return float(close.float().mean()), float(cos)
+
+    frac, cos = agree(xb.grad, xa.grad, 1e-3, 1e-4)
+    assert frac > 0.97 and cos > 0.999, (frac, cos)
+    for name in ("qkv_conv_bn", "proj_conv_bn"):
+        frac, cos = agree(getattr(b, name)[0].weight.grad, getattr(a, name)[0].weight.grad, 1e-2, 1e-2)
+        assert frac > 0.97 and cos > 0.999, (name, frac, cos)
     functional.reset_net(a)
     functional.reset_net(b)
 

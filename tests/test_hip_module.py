@@ -108,6 +108,24 @@ def test_store_v_seq_toggle_is_equivalent(cls, T, N):
         assert bits_equal(u, w)
 
 
+@pytest.mark.parametrize("cls", [neuron.IFNode, neuron.LIFNode, neuron.ParametricLIFNode])
+@pytest.mark.parametrize("N,store_v_seq", [(64, False), (64, True), (37, False), (37, True)])  # replay and saved-h kernels
+def test_loss_on_the_membrane_potential_alone(cls, N, store_v_seq):
+    """No gradient reaches the spikes: the kernels are handed no spike gradient at all (nothing is allocated, filled
+    or read in its place) and must give the gradients of the torch backend."""
+    x = seeded_randn((6, 3, N), 12, 0.4, 1.0)
+    gv = seeded_randn((6, 3, N) if store_v_seq else (3, N), 13)
+    a, b = _pair(cls, surrogate_function=surrogate.ATan(), store_v_seq=store_v_seq)
+    xa, xb = x.clone().requires_grad_(), x.cuda().requires_grad_()
+    a(xa)
+    b(xb)
+    ((a.v_seq if store_v_seq else a.v) * gv).sum().backward()
+    ((b.v_seq if store_v_seq else b.v) * gv.cuda()).sum().backward()
+    torch.testing.assert_close(xb.grad.cpu(), xa.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+    if cls is neuron.ParametricLIFNode:
+        torch.testing.assert_close(b.w.grad.cpu(), a.w.grad, rtol=1e-4, atol=1e-5)
+
+
 def test_non_contiguous_upstream_gradient():
     x = seeded_randn((8, 16, 32), 8, 0.4, 1.0)
     a, b = _pair(neuron.LIFNode, surrogate_function=surrogate.ATan())
@@ -278,6 +296,56 @@ def test_replay_and_h_seq_backward_paths_agree(cls, dtype):
         assert bits_equal(grads[0][2], grads[1][2])
     else:
         torch.testing.assert_close(grads[0][2].float(), grads[1][2].float(), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("cls", [neuron.IFNode, neuron.LIFNode, neuron.ParametricLIFNode, neuron.QIFNode])
+@pytest.mark.parametrize("T", [40, 64, 100, 128])
+@pytest.mark.parametrize("store_v_seq", [False, True])
+def test_long_sequences_replayed_in_pieces_equal_the_saved_h_route(cls, T, store_v_seq, monkeypatch):
+    """Beyond the length the replay kernel takes in one piece the forward leaves the state every
+    ``configure.hip_replay_chunk`` steps and the backward replays piece by piece from those checkpoints; with the
+    chunking switched off the same sequence saves and reads h_seq.  fp32: spikes and states identical bit for bit; the
+    gradient crosses a piece boundary as an fp32 tensor, so the two routes perform the same operations and differ at
+    most where the compiler fused a multiply-add in one kernel variant and not in the other (a short last piece runs
+    the short-sequence variant): 1e-6 relative.  The PLIF sum is added in another order."""
+    from spikingjelly_amd.activation_based.hip_kernel import neuron_kernel as K
+
+    x = seeded_randn((T, 2, 512), 33, 0.4, 1.0).cuda()
+    gs = seeded_randn((T, 2, 512), 34).cuda()
+    gv = seeded_randn((T, 2, 512) if store_v_seq else (2, 512), 35, 0.0, 0.2).cuda()
+    v0 = seeded_randn((2, 512), 36, 0.0, 0.3).cuda()
+    pieces = []
+    real = K._run_backward
+    monkeypatch.setattr(K, "_run_backward", lambda *a, **k: (pieces.append(a[17]), real(*a, **k))[1])
+    results = []
+    for chunk in (16, 0):
+        monkeypatch.setattr(configure, "hip_replay_chunk", chunk)
+        node = cls(step_mode="m", backend="hip", surrogate_function=surrogate.ATan(), store_v_seq=store_v_seq).cuda()
+        vi = v0.clone().requires_grad_()
+        node.v = vi
+        xi = x.clone().requires_grad_()
+        s = node(xi)
+        ((s * gs).sum() + ((node.v_seq if store_v_seq else node.v) * gv).sum()).backward()
+        results.append((s.detach(), node.v.detach(), xi.grad, vi.grad, node.w.grad if hasattr(node, "w") else None))
+    assert pieces == [16, 0]  # the first run was chunked, the second was not
+    for a, b in zip(results[0][:2], results[1][:2]):
+        assert bits_equal(a, b)
+    for a, b in zip(results[0][2:4], results[1][2:4]):
+        torch.testing.assert_close(a, b, rtol=1e-6, atol=1e-7)
+    if results[0][4] is not None:
+        torch.testing.assert_close(results[0][4], results[1][4], rtol=1e-5, atol=1e-6)
+
+
+def test_long_sequence_in_pieces_matches_the_torch_backend():
+    x = seeded_randn((70, 3, 64), 37, 0.4, 1.0)
+    gs = seeded_randn((70, 3, 64), 38)
+    a, b = _pair(neuron.LIFNode, tau=2.5, v_reset=-0.1, surrogate_function=surrogate.Sigmoid())
+    xa, xb = x.clone().requires_grad_(), x.cuda().requires_grad_()
+    sa, sb = a(xa), b(xb)
+    (sa * gs).sum().backward()
+    (sb * gs.cuda()).sum().backward()
+    assert bits_equal(sb.cpu(), sa.detach()) and bits_equal(b.v.detach().cpu(), a.v.detach())
+    torch.testing.assert_close(xb.grad.cpu(), xa.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
 
 
 def test_replay_path_with_misaligned_and_non_contiguous_input():

@@ -1,0 +1,183 @@
+"""``sjhip_neuron_forward_pieces`` / ``sjhip_neuron_backward_recompute_pieces`` through the C ABI.
+
+The forward over pieces must equal ``sjhip_neuron_forward`` over the whole sequence bit for bit (spikes, states) and
+its checkpoints must be the states ``v_seq`` holds at the piece boundaries.  The backward over pieces must equal, bit
+for bit, ``sjhip_neuron_backward_recompute`` called once per piece from the last to the first with the gradient of the
+piece's initial state handed on as ``grad_v_last`` (piece lengths above the short-sequence variant's, so both run the
+same device code); PLIF's dL/dk is a sum in another order (rtol 1e-5).  fp32 is also checked against the oracle.
+"""
+
+import ctypes
+
+import pytest
+import torch
+
+from oracle import neuron_oracle as no
+
+from helpers import bits_equal, seeded_randn
+
+pytestmark = pytest.mark.gpu
+
+ERR_INVALID, ERR_UNSUPPORTED = -1, -2  # SJHIP_ERR_INVALID, SJHIP_ERR_UNSUPPORTED
+
+
+@pytest.fixture(scope="module")
+def L():
+    assert torch.cuda.is_available(), "GPU tests need a ROCm device"
+    from spikingjelly_amd.activation_based.hip_kernel import library
+
+    library.load()
+    return library
+
+
+def _case(L, neuron, dtype, T, N, flags, seed):
+    dev = torch.device("cuda:0")
+    c = dict(neuron=neuron, dtype=dtype, T=T, N=N)
+    c["x"] = seeded_randn((T, N), seed, 0.3, 1.0).to(dtype).to(dev)
+    c["v0"] = (seeded_randn((N,), seed + 1) * 0.2).to(dtype).to(dev)
+    c["gs"] = seeded_randn((T, N), seed + 2).to(dtype).to(dev)
+    c["gv"] = (seeded_randn((T, N), seed + 3) * 0.1).to(dtype).to(dev)
+    c["gl"] = (seeded_randn((N,), seed + 4) * 0.1).to(dtype).to(dev)
+    c["k"] = 0.375 if neuron == L.NEURON_PLIF else 0.5
+    c["kd"] = torch.tensor([c["k"]], dtype=torch.float32, device=dev)
+    c["p"] = L.NeuronParams(c["k"] if neuron == L.NEURON_PLIF else 2.0, 1.0, 0.0, 2.0, 1, flags)
+    c["stream"] = L.current_stream_ptr(dev)
+    return c
+
+
+def _kd(L, c):
+    return c["kd"].data_ptr() if c["neuron"] == L.NEURON_PLIF else None
+
+
+def _forward_whole(L, c):
+    s, v, vl = torch.empty_like(c["x"]), torch.empty_like(c["x"]), torch.empty_like(c["v0"])
+    L.check(L.load().sjhip_neuron_forward(c["neuron"], L.dtype_id(c["dtype"]), ctypes.byref(c["p"]), c["T"], c["N"],
+                                          c["x"].data_ptr(), c["v0"].data_ptr(), _kd(L, c), s.data_ptr(), v.data_ptr(),
+                                          vl.data_ptr(), None, c["stream"]), "forward")
+    return s, v, vl
+
+
+def _forward_pieces(L, c, chunk, with_v_seq=True):
+    lib = L.load()
+    pieces = lib.sjhip_replay_pieces(c["T"], chunk)
+    s, vl = torch.empty_like(c["x"]), torch.full_like(c["v0"], float("nan"))
+    v = torch.empty_like(c["x"]) if with_v_seq else None
+    ck = torch.full((max(pieces - 1, 1), c["N"]), float("nan"), dtype=c["dtype"], device=c["x"].device)
+    L.check(lib.sjhip_neuron_forward_pieces(c["neuron"], L.dtype_id(c["dtype"]), ctypes.byref(c["p"]), c["T"], c["N"], chunk,
+                                            c["x"].data_ptr(), c["v0"].data_ptr(), _kd(L, c), s.data_ptr(),
+                                            v.data_ptr() if with_v_seq else None, vl.data_ptr(), ck.data_ptr(),
+                                            c["stream"]), "forward_pieces")
+    return s, v, vl, ck[: pieces - 1]
+
+
+def _plif_buffers(L, c):
+    if c["neuron"] != L.NEURON_PLIF:
+        return None, None
+    ws = torch.empty(L.load().sjhip_plif_workspace_floats(L.dtype_id(c["dtype"]), c["N"]), dtype=torch.float32, device="cuda:0")
+    return torch.full((1,), float("nan"), dtype=torch.float32, device="cuda:0"), ws
+
+
+def _backward_pieces(L, c, chunk, ck, with_gv):
+    gx, gv0 = torch.full_like(c["x"], float("nan")), torch.full_like(c["v0"], float("nan"))
+    carry = torch.full_like(c["v0"], float("nan"))
+    gk, ws = _plif_buffers(L, c)
+    L.check(L.load().sjhip_neuron_backward_recompute_pieces(
+        c["neuron"], L.dtype_id(c["dtype"]), ctypes.byref(c["p"]), c["T"], c["N"], chunk, c["x"].data_ptr(), c["v0"].data_ptr(),
+        _kd(L, c), ck.data_ptr() if ck.numel() else None, c["gs"].data_ptr(), c["gv"].data_ptr() if with_gv else None,
+        c["gl"].data_ptr(), gx.data_ptr(), gv0.data_ptr(), L.ptr(gk), L.ptr(ws), carry.data_ptr(), c["stream"]),
+        "backward_recompute_pieces")
+    return gx, gv0, gk
+
+
+def _backward_piece_by_piece(L, c, chunk, ck, with_gv):
+    """One sjhip_neuron_backward_recompute call per piece, last to first."""
+    lib = L.load()
+    T, N = c["T"], c["N"]
+    row = N * c["x"].element_size()
+    gx, gv0 = torch.full_like(c["x"], float("nan")), torch.full_like(c["v0"], float("nan"))
+    carries = [torch.empty_like(c["v0"]), torch.empty_like(c["v0"])]
+    starts = list(range(0, T, chunk))
+    gk_total = 0.0
+    for j in range(len(starts) - 1, -1, -1):
+        t0 = starts[j]
+        length = min(chunk, T - t0)
+        gk, ws = _plif_buffers(L, c)
+        state = c["v0"] if j == 0 else ck[j - 1]
+        g_last = c["gl"] if j == len(starts) - 1 else carries[(j + 1) & 1]
+        g_init = gv0 if j == 0 else carries[j & 1]
+        L.check(lib.sjhip_neuron_backward_recompute(
+            c["neuron"], L.dtype_id(c["dtype"]), ctypes.byref(c["p"]), length, N, c["x"].data_ptr() + t0 * row, state.data_ptr(),
+            _kd(L, c), c["gs"].data_ptr() + t0 * row, c["gv"].data_ptr() + t0 * row if with_gv else None, g_last.data_ptr(),
+            gx.data_ptr() + t0 * row, g_init.data_ptr(), L.ptr(gk), L.ptr(ws), c["stream"]), "backward_recompute")
+        if gk is not None:
+            gk_total += float(gk.item())
+    return gx, gv0, gk_total
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=lambda v: str(v).replace("torch.", ""))
+@pytest.mark.parametrize("neuron_name", ["IF", "LIF", "PLIF", "QIF"])
+@pytest.mark.parametrize("T,chunk", [(44, 16), (64, 16), (30, 10), (12, 16)])
+def test_pieces_equal_whole_forward_and_piecewise_backward(L, dtype, neuron_name, T, chunk):
+    neuron = getattr(L, "NEURON_" + neuron_name)
+    flags = L.FLAG_DECAY_INPUT
+    N = 8 * 300
+    c = _case(L, neuron, dtype, T, N, flags, 100 + T)
+    if neuron == L.NEURON_QIF:
+        c["p"] = L.NeuronParams(2.0, 1.0, 0.0, 2.0, 1, flags, 0.0, 0.8, 1.0)  # v_rest, v_c, a0 as the Python wrapper lays them out
+    s, v, vl = _forward_whole(L, c)
+    sp, vp, vlp, ck = _forward_pieces(L, c, chunk)
+    torch.cuda.synchronize()
+    assert bits_equal(sp, s) and bits_equal(vp, v) and bits_equal(vlp, vl)
+    for j in range(ck.shape[0]):
+        assert bits_equal(ck[j], v[(j + 1) * chunk - 1]), f"checkpoint {j}"
+    s2, _, vl2, ck2 = _forward_pieces(L, c, chunk, with_v_seq=False)
+    torch.cuda.synchronize()
+    assert bits_equal(s2, s) and bits_equal(vl2, vl) and bits_equal(ck2, ck)
+    for with_gv in (True, False):
+        got = _backward_pieces(L, c, chunk, ck, with_gv)
+        ref = _backward_piece_by_piece(L, c, chunk, ck, with_gv)
+        torch.cuda.synchronize()
+        assert bits_equal(got[0], ref[0]), "grad_x_seq"
+        assert bits_equal(got[1], ref[1]), "grad_v_init"
+        if neuron == L.NEURON_PLIF:
+            assert float(got[2].item()) == pytest.approx(ref[2], rel=1e-3 if dtype != torch.float32 else 1e-5, abs=1e-3)
+
+
+@pytest.mark.parametrize("neuron_name,kind", [("IF", "if"), ("LIF", "lif")])
+def test_pieces_against_the_oracle(L, neuron_name, kind):
+    T, N, chunk = 50, 4 * 257, 16
+    c = _case(L, getattr(L, "NEURON_" + neuron_name), torch.float32, T, N, L.FLAG_DECAY_INPUT, 7)
+    s, v, vl, ck = _forward_pieces(L, c, chunk)
+    gx, gv0, _ = _backward_pieces(L, c, chunk, ck, True)
+    torch.cuda.synchronize()
+    x, v0, gs, gv, gl = (c[n].cpu() for n in ("x", "v0", "gs", "gv", "gl"))
+    want = no.forward_backward(kind, x, v0, gs, gv, gl, 2.0, True, 1.0, 0.0, "atan", 2.0, False)
+    assert torch.equal(want["spike_seq"], s.cpu()) and torch.equal(want["v_seq"], v.cpu())
+    torch.testing.assert_close(gx.cpu(), want["grad_x"], rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(gv0.cpu(), want["grad_v_init"], rtol=1e-5, atol=1e-6)
+
+
+def test_pieces_argument_checks(L):
+    lib = L.load()
+    c = _case(L, L.NEURON_LIF, torch.float32, 40, 64, L.FLAG_DECAY_INPUT, 3)
+    s, vl = torch.empty_like(c["x"]), torch.empty_like(c["v0"])
+    head = (L.NEURON_LIF, L.dtype_id(torch.float32), ctypes.byref(c["p"]), 40, 64)
+    # several pieces without a checkpoint buffer
+    assert lib.sjhip_neuron_forward_pieces(*head, 16, c["x"].data_ptr(), c["v0"].data_ptr(), None, s.data_ptr(), None,
+                                           vl.data_ptr(), None, c["stream"]) == ERR_INVALID
+    assert lib.sjhip_neuron_forward_pieces(*head, 0, c["x"].data_ptr(), c["v0"].data_ptr(), None, s.data_ptr(), None,
+                                           vl.data_ptr(), None, c["stream"]) == ERR_INVALID
+    # a piece too long for LDS
+    ck = torch.empty((1, 64), device="cuda:0")
+    gx = torch.empty_like(c["x"])
+    assert lib.sjhip_neuron_backward_recompute_pieces(*head[:3], 400, 64, 200, c["x"].data_ptr(), c["v0"].data_ptr(), None,
+                                                      ck.data_ptr(), c["gs"].data_ptr(), None, None, gx.data_ptr(), None, None,
+                                                      None, vl.data_ptr(), c["stream"]) == ERR_UNSUPPORTED
+    # an fp32 state over 16-bit storage would be rounded at every checkpoint
+    c = _case(L, L.NEURON_LIF, torch.float16, 40, 64, L.FLAG_DECAY_INPUT | L.FLAG_FP32_STATE, 3)
+    ck16 = torch.empty((2, 64), dtype=torch.float16, device="cuda:0")
+    s16, vl16 = torch.empty_like(c["x"]), torch.empty_like(c["v0"])
+    assert lib.sjhip_neuron_forward_pieces(L.NEURON_LIF, L.dtype_id(torch.float16), ctypes.byref(c["p"]), 40, 64, 16,
+                                           c["x"].data_ptr(), c["v0"].data_ptr(), None, s16.data_ptr(), None, vl16.data_ptr(),
+                                           ck16.data_ptr(), c["stream"]) == ERR_UNSUPPORTED
+    assert lib.sjhip_replay_pieces(40, 16) == 3 and lib.sjhip_replay_pieces(16, 16) == 1 and lib.sjhip_replay_pieces(0, 16) == 0

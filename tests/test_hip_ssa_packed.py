@@ -5,6 +5,7 @@ operands only arrive in another encoding)."""
 import pytest
 import torch
 
+from spikingjelly_amd import configure
 from spikingjelly_amd.activation_based import functional, layer
 from spikingjelly_amd.activation_based.hip_kernel import attention_kernel as A
 from spikingjelly_amd.activation_based.hip_kernel.compress import bit_spike_compress
@@ -52,7 +53,9 @@ def _blocks(dim, heads):
 
 
 @pytest.mark.parametrize("T,B,dim,heads,tokens", [(4, 8, 128, 4, 96), (2, 3, 64, 2, 20), (4, 2, 384, 12, 196)])
-def test_fused_block_equals_two_operator_block(T, B, dim, heads, tokens):
+def test_fused_block_equals_two_operator_block(T, B, dim, heads, tokens, monkeypatch):
+    # torch's convolution and batch norm in both blocks: this test is about the LIF -> contraction step alone
+    monkeypatch.setattr(configure, "hip_fuse_conv_bn_lif", False)
     fused, plain = _blocks(dim, heads)
     x = seeded_randn((T, B, dim, tokens), 5)
     g = seeded_randn((T, B, dim, tokens), 6).cuda()
