@@ -430,7 +430,7 @@ def other_workload(args) -> int:
         return 0
 
     if args.workload == "config5":
-        T, B, D, H, tokens = 4, 64, 384, 12, 196
+        T, B, D, H, tokens = 4, 64, args.dim, 12, 196
         torch.manual_seed(1005)
         block = layer.SpikingSelfAttention(D, H, backend="hip").to(dev)
         x = randn((T, B, D, tokens), 1105, 0.0, 1.0, torch.float32).requires_grad_()
@@ -452,10 +452,10 @@ def other_workload(args) -> int:
         # the qkv spikes travel bit-packed between the LIF and the contraction: 3 n / 8 bytes; fp32 elsewhere
         bytes_f = 3 * n // 8 + 4 * n              # bits read, out written
         bytes_b = 3 * n // 8 + 4 * n + 12 * n     # bits and grad_out read, dq / dk / dv written
-        _emit(args, "tokens/sec spiking self-attention block fwd+bwd, T=4 B=64 N=196 D=384 12 heads, 1 MI355X",
+        _emit(args, f"tokens/sec spiking self-attention block fwd+bwd, T=4 B=64 N=196 D={D} 12 heads, 1 MI355X",
               "tokens/s", T * B * tokens / (elapsed / args.steps), elapsed, "bf16",
-              {"workload": "configs[4]: SpikingSelfAttention(384, 12, backend='hip'), x [4,64,384,196] fp32 ~N(0,1), "
-                           "channels per head = 32 (dim // heads, as the reference computes it)"},
+              {"workload": f"configs[4]: SpikingSelfAttention({D}, 12, backend='hip'), x [4,64,{D},196] fp32 ~N(0,1), "
+                           f"channels per head = {cph} (dim // heads, as the reference computes it)"},
               {"bound": "hbm", "achieved": bytes_b / (sb * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                "frac": bytes_b / (sb * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "ssa_backward",
                "kernel_ms": sb, "algorithmic_bytes": bytes_b,
@@ -476,6 +476,8 @@ def main() -> int:
     ap.add_argument("--cpu-repeats", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--terms", type=int, default=3, choices=[1, 2, 3], help="pwconv workload: bf16 terms per fp32 operand")
+    ap.add_argument("--dim", type=int, default=384, choices=[384, 768],
+                    help="config5 workload: embedding width (12 heads of dim // 12 channels: 32, or 64 with 768)")
     ap.add_argument("--seq-len", type=int, default=SHAPE[0],
                     help="config2 variant: T steps over 2^29 / T neurons (the headline is T=16); a secondary measurement")
     ap.add_argument("--n-offset", type=int, default=0,

@@ -505,6 +505,9 @@ int sjhip_bn_grad_input(const float *g, const float *y, const float *coef, int64
  * "replay_blocks_per_cu" likewise for sjhip_neuron_backward_recompute.  The forward cap applies to
  * fp32 storage with v_seq or h_seq written (spikes-only and 16-bit forwards always run uncapped); it is
  * doubled for T < 16 and dropped for T < 4, where few rows are in flight per work-item.  Returns SJHIP_ERR_INVALID otherwise.
+ * "column_spread" = which columns a block of the neuron kernels takes: 0 = block b takes chunk b of a row (each XCD
+ * every eighth chunk), 1 = each XCD one contiguous eighth of the row, 2 (default) = 1 only for row strides that are a
+ * multiple of 4 KiB with odd parity of address bits 12 and 20, where the default order measured 20 to 35 % slower.
  * Results never depend on these.
  */
 int sjhip_set_tuning(const char *key, int value);

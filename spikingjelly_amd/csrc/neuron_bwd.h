@@ -81,6 +81,7 @@ struct BwdArgs {
   float vth_rcp;            // ILIF: fl(1 / v_threshold), the factor of the count's gradient
   int detach_reset;
   int round_each;           // 16-bit storage with every op rounded
+  int spread;               // block-to-column order, see column_block()
 };
 
 // Which extra terms the BPTT walk carries.
@@ -390,7 +391,7 @@ __device__ __forceinline__ void plif_block_reduce(const BwdArgs &a, float part, 
 template <typename S, bool VECTOR, int MODE>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_kernel(const BwdArgs a) {
   constexpr int V = Acc<S, VECTOR, true>::V;
-  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
+  const int64_t col = ((int64_t)column_block(a.spread) * blockDim.x + threadIdx.x) * V;
   const bool active = col < a.N;
   const float k = a.k_device ? *a.k_device : a.k;
   const float part = backward_sg_dispatch<S, VECTOR, MODE, 0>(a, active, col, k, nullptr);
@@ -407,6 +408,7 @@ inline int build_bwd_args(BwdArgs &a, int neuron, int dtype, const sjhip_neuron_
   a.grad_x = grad_x_seq; a.grad_v_init = grad_v_init;
   a.partials = workspace; a.grad_k = grad_rtau;
   a.T = T; a.N = N;
+  a.spread = column_spread(N * (dtype == SJHIP_F32 ? 4 : 2)) ? 1 : 0;
   a.v_th = p.v_threshold; a.v_reset = p.v_reset; a.alpha = p.sg_alpha;
   a.sg = p.sg_id;
   a.soft_reset = (p.flags & SJHIP_FLAG_SOFT_RESET) ? 1 : 0;

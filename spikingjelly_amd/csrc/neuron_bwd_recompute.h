@@ -138,7 +138,7 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_pieces_ker
   typedef typename Acc<S, true, true>::elem_t E;
   constexpr int V = Acc<S, true, true>::V;
   static_assert(!BwdModeOf<MODE>::SHORT, "pieces are long enough for the deep prefetch");
-  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
+  const int64_t col = ((int64_t)column_block(b0.spread) * blockDim.x + threadIdx.x) * V;
   const bool active = col < b0.N;
   const float k = b0.k_device ? *b0.k_device : b0.k;
   constexpr int HLDS = (ROUND_EACH && sizeof(S) == 2) ? 2 : 1;
@@ -181,7 +181,7 @@ template <typename S, bool ROUND_EACH, int MODE>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_kernel(const FwdArgs f, const BwdArgs b) {
   extern __shared__ f32x4 lds_h[];
   constexpr int V = Acc<S, true, true>::V;
-  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
+  const int64_t col = ((int64_t)column_block(b.spread) * blockDim.x + threadIdx.x) * V;
   const bool active = col < b.N;
   // request the last rows of the upstream gradients now, so they arrive while h is being replayed
   constexpr bool SHORT = BwdModeOf<MODE>::SHORT;

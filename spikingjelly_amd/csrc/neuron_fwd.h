@@ -70,6 +70,7 @@ struct FwdArgs {
   int charge;
   int soft_reset;        // a Reset value
   int v_init_broadcast;  // v_init holds one element for all neurons
+  int spread;            // block-to-column order, see column_block()
 };
 
 // Fire-and-reset rule.  RESET_COUNT is ILIF (functional/neuron.py:1097-1099 with quantize.py:592): the neuron fires
@@ -260,7 +261,7 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
   constexpr int PF = (OUT & FWD_OUT_SHORT) ? 2 : (sizeof(S) == 2 ? SJHIP_FWD_PF16 : SJHIP_FWD_PF);
 
   const int64_t N = a.N, T = a.T;
-  const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
+  const int64_t col = ((int64_t)column_block(a.spread) * blockDim.x + threadIdx.x) * V;
   if (col >= N) return;
 
   const E *xp = (const E *)a.x + col;
@@ -375,6 +376,7 @@ inline int build_fwd_args(FwdArgs &a, bool &round_each, int neuron, int dtype, c
   a.x = x_seq; a.v_init = v_init; a.spike = spike_seq; a.v_seq = v_seq; a.v_last = v_last; a.h = h_seq;
   a.k_device = nullptr;
   a.T = T; a.N = N;
+  a.spread = column_spread(N * (dtype == SJHIP_F32 ? 4 : 2)) ? 1 : 0;
   const bool ilif = neuron == SJHIP_NEURON_ILIF;
   a.soft_reset = ilif ? RESET_COUNT : ((p.flags & SJHIP_FLAG_SOFT_RESET) ? RESET_SOFT : RESET_HARD);
   a.level_max = p.level_max;

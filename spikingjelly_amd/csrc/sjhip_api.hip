@@ -27,6 +27,7 @@ struct TuningStore {
   // The replay backward has two phases per wavefront (recompute h, then BPTT) and needs more waves
   // in flight to overlap them: uncapped (8 waves per CU at T=16 fp32) measured 15 % faster than 2 blocks.
   std::atomic<int> replay_blocks_per_cu{0};
+  std::atomic<int> column_spread{2};
 };
 TuningStore g_tuning;
 
@@ -78,6 +79,7 @@ const Tuning &tuning() {
   t.fwd_blocks_per_cu = g_tuning.fwd_blocks_per_cu.load(std::memory_order_relaxed);
   t.bwd_blocks_per_cu = g_tuning.bwd_blocks_per_cu.load(std::memory_order_relaxed);
   t.replay_blocks_per_cu = g_tuning.replay_blocks_per_cu.load(std::memory_order_relaxed);
+  t.column_spread = g_tuning.column_spread.load(std::memory_order_relaxed);
   return t;
 }
 
@@ -623,6 +625,7 @@ int sjhip_set_tuning(const char *key, int value) {
   if (!strcmp(key, "fwd_blocks_per_cu")) { if (!cap_ok) return fail(SJHIP_ERR_INVALID, "set_tuning: fwd_blocks_per_cu=%d", value); g_tuning.fwd_blocks_per_cu = value; return SJHIP_OK; }
   if (!strcmp(key, "bwd_blocks_per_cu")) { if (!cap_ok) return fail(SJHIP_ERR_INVALID, "set_tuning: bwd_blocks_per_cu=%d", value); g_tuning.bwd_blocks_per_cu = value; return SJHIP_OK; }
   if (!strcmp(key, "replay_blocks_per_cu")) { if (!cap_ok) return fail(SJHIP_ERR_INVALID, "set_tuning: replay_blocks_per_cu=%d", value); g_tuning.replay_blocks_per_cu = value; return SJHIP_OK; }
+  if (!strcmp(key, "column_spread")) { if (value < 0 || value > 2) return fail(SJHIP_ERR_INVALID, "set_tuning: column_spread=%d", value); g_tuning.column_spread = value; return SJHIP_OK; }
   return fail(SJHIP_ERR_INVALID, "set_tuning: unknown key '%s'", key);
 }
 
@@ -633,6 +636,7 @@ int sjhip_get_tuning(const char *key) {
   if (!strcmp(key, "fwd_blocks_per_cu")) return g_tuning.fwd_blocks_per_cu;
   if (!strcmp(key, "bwd_blocks_per_cu")) return g_tuning.bwd_blocks_per_cu;
   if (!strcmp(key, "replay_blocks_per_cu")) return g_tuning.replay_blocks_per_cu;
+  if (!strcmp(key, "column_spread")) return g_tuning.column_spread;
   return fail(SJHIP_ERR_INVALID, "get_tuning: unknown key '%s'", key);
 }
 

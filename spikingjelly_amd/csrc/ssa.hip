@@ -32,12 +32,18 @@
 // column lane % 16.  Which k a lane's operand element stands for is free as long as A and B agree.
 #include "sjhip_common.h"
 
+#include <algorithm>
 #include <mutex>
 
 // Resident blocks per compute unit the backward kernel's register allocation is sized for (heads of up to 32
 // channels).  Sized for 2 the kernel takes 124 registers and keeps the split dS operands across the column tiles
 // without spilling, so three blocks are resident anyway (what LDS allows); sized for 3 the allocator spills 40
 // registers around the same code (80 us against 83 us at 256 samples x 12 heads x 32 x 196).
+// Measured on the same shape with bit-packed spikes (us per launch; fetching with one trip to memory per loop iteration
+// of the stagings and no integer division: 91): requesting all of a head's grad_out and spike bytes before using any
+// (40 registers held): 103; a grid of resident blocks, each fetching its next head into registers while it computes the
+// current one: 108 with two resident blocks (the loop around the products takes the allocator to 256 registers) and
+// 149 with three (60 registers spilled).  The kernel therefore keeps one block per head and the plain stagings.
 #ifndef SJHIP_SSA_BWD_RESIDENT
 #define SJHIP_SSA_BWD_RESIDENT 2
 #endif
@@ -99,6 +105,32 @@ __device__ __forceinline__ uint32_t spike_bytes(const float (&f)[4]) {
          (f[3] != 0.0f ? 0x1000000u : 0u);
 }
 
+// e / L for 0 <= e < 2^16 and 1 <= L <= 256 without the integer-division sequence: (e + 0.5) / L lies at least
+// 0.5 / L away from every integer, far more than the rounding error of the fp32 product.
+__device__ __forceinline__ int div_tokens(int e, float inv_L) { return (int)(((float)e + 0.5f) * inv_L); }
+
+// Zero-fills columns [L, stride) of rows [0, cph) and all of rows [cph, rows_pad) of NS byte tiles or one fp32 tile;
+// eight work-items per row, so no work-item divides.
+template <int NS>
+__device__ __forceinline__ void zero_fill_bytes(uint8_t *const (&dst)[NS], int cph, int rows_pad, int L, int Lb) {
+  const int tid = threadIdx.x;
+  for (int r = tid >> 3; r < cph; r += kSsaThreads / 8)
+    for (int c = L + (tid & 7); c < Lb; c += 8) {
+#pragma unroll
+      for (int s = 0; s < NS; ++s) dst[s][r * Lb + c] = 0;
+    }
+  for (int i = tid; i < (rows_pad - cph) * (Lb / 4); i += kSsaThreads) {
+#pragma unroll
+    for (int s = 0; s < NS; ++s) reinterpret_cast<uint32_t *>(dst[s] + cph * Lb)[i] = 0u;
+  }
+}
+__device__ __forceinline__ void zero_fill_f32(float *dst, int cph, int rows_pad, int L, int Lq) {
+  const int tid = threadIdx.x;
+  for (int r = tid >> 3; r < cph; r += kSsaThreads / 8)
+    for (int c = L + (tid & 7); c < Lq; c += 8) dst[r * Lq + c] = 0.0f;
+  for (int i = tid; i < (rows_pad - cph) * Lq; i += kSsaThreads) dst[cph * Lq + i] = 0.0f;
+}
+
 // Global tiles -> LDS.  NS spike tiles ([cph, L] each) become
 // byte tiles [rows_pad][Lb]; when DO is set the grad_out tile becomes an fp32 tile [rows_pad][Lq].  Rows
 // cph..rows_pad-1 and the columns from L to the row stride are zero-filled, by writes that never overlap the
@@ -111,6 +143,7 @@ __device__ __forceinline__ void stage_tiles(const typename Io<S>::elem_t *const 
   const int tid = threadIdx.x;
   if (vec) {
     const int G = cph * L / 4;
+    const float inv_L = 1.0f / (float)L;
     for (int g0 = tid; g0 < G; g0 += kSsaThreads * UN) {
       Q buf[UN][NS + (DO ? 1 : 0)];
 #pragma unroll
@@ -126,7 +159,7 @@ __device__ __forceinline__ void stage_tiles(const typename Io<S>::elem_t *const 
       for (int u = 0; u < UN; ++u) {
         const int g = g0 + u * kSsaThreads;
         if (g < G) {
-          const int r = (4 * g) / L, c = 4 * g - r * L;
+          const int r = div_tokens(4 * g, inv_L), c = 4 * g - r * L;
           float f[4];
 #pragma unroll
           for (int s = 0; s < NS; ++s) {
@@ -150,71 +183,75 @@ __device__ __forceinline__ void stage_tiles(const typename Io<S>::elem_t *const 
       if (DO) do_dst[r * Lq + c] = Io<S>::get(do_src, i);
     }
   }
-  // zero fill: right margin of the data rows, then the rows below them
-  const int mb = Lb - L;
-  for (int i = tid; i < cph * mb; i += kSsaThreads) {
-    const int r = i / mb, c = L + (i - r * mb);
+  zero_fill_bytes<NS>(dst, cph, rows_pad, L, Lb);
+  if (DO) zero_fill_f32(do_dst, cph, rows_pad, L, Lq);
+}
+
+// Byte b of the bit-packed tiles (its eight elements 8 b ... 8 b + 7) -> LDS byte tiles.
+template <int NS>
+__device__ __forceinline__ void expand_byte(const uint32_t (&w)[NS], int b, uint8_t *const (&dst)[NS], int L, int Lb,
+                                            float inv_L) {
+  if ((L & 3) == 0) {
+    // four elements never straddle a row and land on a 4-byte boundary: one 32-bit store per nibble.  The product
+    // copies bit i of the nibble to bit 8 i (and to other positions the mask drops; no two copies collide).
 #pragma unroll
-    for (int s = 0; s < NS; ++s) dst[s][r * Lb + c] = 0;
-  }
-  for (int i = tid; i < (rows_pad - cph) * (Lb / 4); i += kSsaThreads) {
+    for (int half = 0; half < 2; ++half) {
+      const int e = 8 * b + 4 * half;
+      const int r = div_tokens(e, inv_L), c = e - r * L;
 #pragma unroll
-    for (int s = 0; s < NS; ++s) reinterpret_cast<uint32_t *>(dst[s] + cph * Lb)[i] = 0u;
-  }
-  if (DO) {
-    const int mq = Lq - L;
-    for (int i = tid; i < cph * mq; i += kSsaThreads) {
-      const int r = i / mq, c = L + (i - r * mq);
-      do_dst[r * Lq + c] = 0.0f;
+      for (int s = 0; s < NS; ++s)
+        *reinterpret_cast<uint32_t *>(dst[s] + r * Lb + c) = (((w[s] >> (4 * half)) & 15u) * 0x00204081u) & 0x01010101u;
     }
-    for (int i = tid; i < (rows_pad - cph) * Lq; i += kSsaThreads) do_dst[cph * Lq + i] = 0.0f;
+  } else {
+    int r = div_tokens(8 * b, inv_L), c = 8 * b - r * L;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+      for (int s = 0; s < NS; ++s) dst[s][r * Lb + c] = (uint8_t)((w[s] >> i) & 1u);
+      if (++c == L) { c = 0; ++r; }
+    }
   }
 }
 
 // Bit-packed spike tiles -> LDS byte tiles.  The flattened qkv tensor is packed LSB first (byte j bit i = element
 // 8 j + i, what bit_pack and the packed neuron forward write); a [cph, L] tile whose element count is a multiple of 8
 // starts on a byte and is cph L / 8 bytes long, 32 times less to fetch than fp32 spikes.  A byte's eight elements may
-// straddle a row boundary of the tile (L need not be a multiple of 8).
+// straddle a row boundary of the tile (L need not be a multiple of 8).  All of a work-item's bytes (four cover 32
+// channels of up to 256 tokens) are requested before the first is used: one trip to memory, not one per byte.
 template <int NS>
 __device__ __forceinline__ void stage_bits(const uint8_t *const (&src)[NS], uint8_t *const (&dst)[NS], int cph,
                                            int rows_pad, int L, int Lb) {
+  constexpr int UB = 4;
   const int tid = threadIdx.x;
   const int nbytes = cph * L / 8;
-  for (int b = tid; b < nbytes; b += kSsaThreads) {
-    uint32_t w[NS];
+  const float inv_L = 1.0f / (float)L;
+  for (int b0 = tid; b0 < nbytes; b0 += kSsaThreads * UB) {
+    uint32_t w[UB][NS];
 #pragma unroll
-    for (int s = 0; s < NS; ++s) w[s] = src[s][b];
-    if ((L & 3) == 0) {
-      // four elements never straddle a row and land on a 4-byte boundary: one 32-bit store per nibble.  The product
-      // copies bit i of the nibble to bit 8 i (and to other positions the mask drops; no two copies collide).
+    for (int u = 0; u < UB; ++u) {
+      const int b = b0 + u * kSsaThreads;
+      if (b < nbytes) {
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const int e = 8 * b + 4 * half;
-        const int r = e / L, c = e - r * L;
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-          *reinterpret_cast<uint32_t *>(dst[s] + r * Lb + c) = (((w[s] >> (4 * half)) & 15u) * 0x00204081u) & 0x01010101u;
-      }
-    } else {
-      int r = (8 * b) / L, c = 8 * b - r * L;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-#pragma unroll
-        for (int s = 0; s < NS; ++s) dst[s][r * Lb + c] = (uint8_t)((w[s] >> i) & 1u);
-        if (++c == L) { c = 0; ++r; }
+        for (int s = 0; s < NS; ++s) w[u][s] = src[s][b];
       }
     }
-  }
-  const int mb = Lb - L;
-  for (int i = tid; i < cph * mb; i += kSsaThreads) {
-    const int r = i / mb, c = L + (i - r * mb);
 #pragma unroll
-    for (int s = 0; s < NS; ++s) dst[s][r * Lb + c] = 0;
+    for (int u = 0; u < UB; ++u) {
+      const int b = b0 + u * kSsaThreads;
+      if (b < nbytes) expand_byte<NS>(w[u], b, dst, L, Lb, inv_L);
+    }
   }
-  for (int i = tid; i < (rows_pad - cph) * (Lb / 4); i += kSsaThreads) {
-#pragma unroll
-    for (int s = 0; s < NS; ++s) reinterpret_cast<uint32_t *>(dst[s] + cph * Lb)[i] = 0u;
-  }
+  zero_fill_bytes<NS>(dst, cph, rows_pad, L, Lb);
+}
+
+// Four consecutive grad_out elements -> the fp32 LDS tile [rows_pad][Lq].
+template <typename S>
+__device__ __forceinline__ void put_grad_out_quad(typename Io<S>::quad_t q, int g, float *do_dst, int L, int Lq, float inv_L) {
+  const int r = div_tokens(4 * g, inv_L), c = 4 * g - r * L;
+  float f[4];
+  Io<S>::unpack(q, f);
+  f32x4 w; w.x = f[0]; w.y = f[1]; w.z = f[2]; w.w = f[3];
+  *reinterpret_cast<f32x4 *>(do_dst + r * Lq + c) = w;
 }
 
 // The grad_out tile alone -> fp32 LDS tile [rows_pad][Lq], zero-padded (the packed backward stages its spikes apart).
@@ -225,6 +262,7 @@ __device__ __forceinline__ void stage_grad_out(const typename Io<S>::elem_t *do_
   const int tid = threadIdx.x;
   if (vec) {
     const int G = cph * L / 4;
+    const float inv_L = 1.0f / (float)L;
     constexpr int UN = 4;
     for (int g0 = tid; g0 < G; g0 += kSsaThreads * UN) {
       Q buf[UN];
@@ -236,13 +274,7 @@ __device__ __forceinline__ void stage_grad_out(const typename Io<S>::elem_t *do_
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
         const int g = g0 + u * kSsaThreads;
-        if (g < G) {
-          const int r = (4 * g) / L, c = 4 * g - r * L;
-          float f[4];
-          Io<S>::unpack(buf[u], f);
-          f32x4 w; w.x = f[0]; w.y = f[1]; w.z = f[2]; w.w = f[3];
-          *reinterpret_cast<f32x4 *>(do_dst + r * Lq + c) = w;
-        }
+        if (g < G) put_grad_out_quad<S>(buf[u], g, do_dst, L, Lq, inv_L);
       }
     }
   } else {
@@ -252,12 +284,7 @@ __device__ __forceinline__ void stage_grad_out(const typename Io<S>::elem_t *do_
       do_dst[r * Lq + c] = Io<S>::get(do_src, i);
     }
   }
-  const int mq = Lq - L;
-  for (int i = tid; i < cph * mq; i += kSsaThreads) {
-    const int r = i / mq, c = L + (i - r * mq);
-    do_dst[r * Lq + c] = 0.0f;
-  }
-  for (int i = tid; i < (rows_pad - cph) * Lq; i += kSsaThreads) do_dst[cph * Lq + i] = 0.0f;
+  zero_fill_f32(do_dst, cph, rows_pad, L, Lq);
 }
 
 // 32x32 block of  A_rows B_rows^T  over the token axis: rows ra.. of tile `a` against rows rb.. of tile `b`

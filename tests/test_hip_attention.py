@@ -18,7 +18,7 @@ def _spikes(shape, seed, rate=0.2):
 
 
 @pytest.mark.parametrize("S,H,C,L", [(6, 12, 32, 196), (3, 2, 32, 64), (2, 3, 48, 64), (2, 2, 64, 100), (1, 1, 8, 5),
-                                     (2, 1, 32, 256), (1, 2, 33, 31)])
+                                     (2, 1, 32, 256), (1, 2, 33, 31), (3, 12, 64, 196)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_forward_is_exact(S, H, C, L, dtype):
     qkv = _spikes((S, 3, H, C, L), 7 + L, 0.5 if L * C < 2000 else 0.15)
@@ -39,7 +39,7 @@ def test_forward_maximal_sums_all_ones():
     assert torch.equal(out, torch.full((1, 1, 64, 100), 0.125 * 64 * 100))
 
 
-@pytest.mark.parametrize("S,H,C,L", [(4, 12, 32, 196), (2, 3, 48, 64), (2, 2, 64, 100), (1, 2, 33, 31)])
+@pytest.mark.parametrize("S,H,C,L", [(4, 12, 32, 196), (2, 3, 48, 64), (2, 2, 64, 100), (1, 2, 33, 31), (3, 12, 64, 196)])
 def test_backward_matches_float64_autograd(S, H, C, L):
     qkv = _spikes((S, 3, H, C, L), 11 + L, 0.2)
     g = torch.Generator().manual_seed(5)

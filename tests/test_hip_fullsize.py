@@ -17,10 +17,15 @@ pytestmark = pytest.mark.gpu
 T, N = 16, 256 * 128 * 32 * 32
 
 
-def test_config2_full_size_forward_backward(c_oracle):
+@pytest.mark.parametrize("t_steps,n_neurons", [(T, N), (T, N + 1024), (128, N // 8)],
+                         ids=["config2", "row_stride_off_a_power_of_two", "T128_replayed_in_pieces"])
+def test_config2_full_size_forward_backward(c_oracle, t_steps, n_neurons):
+    """BASELINE config 2, the same element count with rows 4 KiB longer (a row stride that is not a power of two),
+    and the same element count as 128 steps (the forward leaves checkpoints, the backward replays in pieces)."""
     from spikingjelly_amd.activation_based import neuron, surrogate
 
     require_device_memory(40)
+    T, N = t_steps, n_neurons
     g = torch.Generator(device="cuda").manual_seed(1002)
     x = (torch.randn((T, N), generator=g, device="cuda") * 0.8 + 0.3).requires_grad_()
     gs = torch.randn((T, N), generator=g, device="cuda")

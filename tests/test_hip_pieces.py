@@ -181,3 +181,33 @@ def test_pieces_argument_checks(L):
                                            c["x"].data_ptr(), c["v0"].data_ptr(), None, s16.data_ptr(), None, vl16.data_ptr(),
                                            ck16.data_ptr(), c["stream"]) == ERR_UNSUPPORTED
     assert lib.sjhip_replay_pieces(40, 16) == 3 and lib.sjhip_replay_pieces(16, 16) == 1 and lib.sjhip_replay_pieces(0, 16) == 0
+
+
+@pytest.mark.parametrize("N", [8 * 300, 128 * 4 * 8 * 37 + 4, 1 << 20])
+def test_block_to_column_order_does_not_change_results(L, N):
+    """``column_spread`` only permutes which block works on which columns: forward, saved-h backward, replaying backward
+    and the pieces kernels must give the same bits either way (grids of fewer than eight blocks, a grid that is not a
+    multiple of eight, a large one)."""
+    lib = L.load()
+    c = _case(L, L.NEURON_PLIF, torch.float32, 24, N, L.FLAG_DECAY_INPUT, 11)
+    results = []
+    try:
+        for mode in (0, 1):
+            assert lib.sjhip_set_tuning(b"column_spread", mode) == 0
+            s, v, vl = _forward_whole(L, c)
+            sp, vp, vlp, ck = _forward_pieces(L, c, 16)
+            gx, gv0, gk = _backward_pieces(L, c, 16, ck, True)
+            gx1, gv1 = torch.full_like(c["x"], float("nan")), torch.full_like(c["v0"], float("nan"))
+            gk1, ws = _plif_buffers(L, c)
+            L.check(lib.sjhip_neuron_backward_recompute(
+                c["neuron"], L.dtype_id(c["dtype"]), ctypes.byref(c["p"]), c["T"], N, c["x"].data_ptr(), c["v0"].data_ptr(),
+                c["kd"].data_ptr(), c["gs"].data_ptr(), c["gv"].data_ptr(), c["gl"].data_ptr(), gx1.data_ptr(), gv1.data_ptr(),
+                gk1.data_ptr(), ws.data_ptr(), c["stream"]), "backward_recompute")
+            torch.cuda.synchronize()
+            assert bits_equal(sp, s) and bits_equal(vp, v)
+            results.append((s, v, vl, gx, gv0, gx1, gv1, gk1))
+    finally:
+        lib.sjhip_set_tuning(b"column_spread", 2)
+    for a, b in zip(results[0][:7], results[1][:7]):
+        assert bits_equal(a, b)
+    assert float(results[0][7].item()) == pytest.approx(float(results[1][7].item()), rel=1e-5)
