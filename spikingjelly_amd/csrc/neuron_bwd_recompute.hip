@@ -16,10 +16,10 @@ namespace {
 
 constexpr unsigned kMaxLds = 159u * 1024u;  // LDS per compute unit on gfx950 minus 1 KiB for static words
 
-// LDS bytes one work-item needs per step for h: its 4 fp32 neurons (fp32 storage, and 16-bit storage with fp32
-// state, which runs four neurons per work-item through 8-byte accesses) or its 8 neurons as 16-bit patterns
-// (16-bit storage, every op rounded)
-int64_t h_bytes_per_item(int dtype, bool round_each) { (void)dtype; (void)round_each; return 16; }
+// LDS bytes one work-item needs per step for h, the same in every mode: its 4 fp32 neurons (fp32 storage, and 16-bit
+// storage with fp32 state, which runs four neurons per work-item through 8-byte accesses) or its 8 neurons as 16-bit
+// patterns (16-bit storage, every op rounded)
+constexpr int64_t kHBytesPerItem = 16;
 
 }  // namespace
 
@@ -27,7 +27,7 @@ int64_t h_bytes_per_item(int dtype, bool round_each) { (void)dtype; (void)round_
 int recompute_block(int dtype, int64_t T, bool round_each) {
   for (int block : {128, 64}) {
     if (block > SJHIP_MAX_BLOCK) continue;
-    if (T * block * h_bytes_per_item(dtype, round_each) <= (int64_t)kMaxLds) return block;
+    if (T * block * kHBytesPerItem <= (int64_t)kMaxLds) return block;
   }
   return 0;
 }
@@ -41,7 +41,7 @@ bool recompute_preferred(int dtype, int64_t T, int64_t N, bool round_each) {
   // the replay needs T * 64 lanes * h_bytes of LDS per wavefront; below four resident wavefronts per compute unit
   // it is slower than reading a saved h_seq (measured: T = 32 still wins, T = 64 loses, fp32)
   if (!recompute_supported(dtype, T, N)) return false;
-  return 4 * T * 64 * h_bytes_per_item(dtype, round_each) <= (int64_t)kMaxLds;
+  return 4 * T * 64 * kHBytesPerItem <= (int64_t)kMaxLds;
 }
 
 namespace {
@@ -78,7 +78,7 @@ int launch_replay(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T
   const int64_t items = N / V;
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "backward(recompute): N=%lld", (long long)N);
-  unsigned lds = (unsigned)(lds_steps * block * h_bytes_per_item(dtype, round_each));
+  unsigned lds = (unsigned)(lds_steps * block * kHBytesPerItem);
   const unsigned cap = occupancy_cap_lds(tuning().replay_blocks_per_cu);
   if (cap > lds) lds = cap;
   const bool plif = neuron == SJHIP_NEURON_PLIF;

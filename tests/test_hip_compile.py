@@ -109,3 +109,51 @@ def test_spiking_self_attention_block_compiles():
     yc.sum().backward()
     torch.testing.assert_close(xb.grad, xa.grad, rtol=1e-4, atol=1e-5)
     torch.testing.assert_close(xb.grad, xc.grad, rtol=1e-3, atol=1e-4)
+
+
+def _triton_available() -> bool:
+    try:
+        import triton  # noqa: F401
+    except Exception:
+        return False
+    return True
+
+
+@pytest.mark.skipif(not _triton_available(), reason="the inductor backend generates triton kernels and triton is not importable")
+@pytest.mark.parametrize("shape", [(4, 8, 32), (6, 3, 48)])
+def test_inductor_compiles_linear_then_hip_node(shape):
+    """Linear -> multi-step hip LIF -> loss under the code-generating backend, forward and backward, as the reference
+    asks of its kernel backends (test/activation_based/test_compile_compat.py:144-170): the generated code around the
+    opaque operators must hand them contiguous tensors and accept their outputs.  The linear layer runs through
+    generated or library GEMM code, so its output may differ from eager in the last bit and a neuron at the threshold
+    may flip: spikes are compared as a rate of disagreement, gradients with a tolerance."""
+    T, B, D = shape
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc = torch.nn.Linear(D, 2 * D)
+            self.node = neuron.LIFNode(tau=2.0, surrogate_function=surrogate.ATan(), step_mode="m", backend="hip")
+
+        def forward(self, x):
+            return self.node(self.fc(x))
+
+    torch.manual_seed(3)
+    eager = Net().cuda()
+    traced = Net().cuda()
+    traced.load_state_dict(eager.state_dict())
+    fn = torch.compile(traced, fullgraph=True, backend="inductor")
+    x = seeded_randn((T, B, D), 17, 0.2, 1.5).cuda()
+    target = seeded_randn((T, B, 2 * D), 18).cuda()
+    xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
+    ya, yb = eager(xa), fn(xb)
+    assert ya.shape == yb.shape == (T, B, 2 * D)
+    assert 0.02 < float(ya.detach().mean()) < 0.9
+    assert float((ya != yb).float().mean()) < 1e-3
+    ((ya - target) ** 2).mean().backward()
+    ((yb - target) ** 2).mean().backward()
+    scale = float(xa.grad.abs().max())
+    assert scale > 0
+    torch.testing.assert_close(xb.grad, xa.grad, rtol=1e-3, atol=1e-3 * scale)
+    torch.testing.assert_close(traced.fc.weight.grad, eager.fc.weight.grad, rtol=1e-3,
+                               atol=1e-3 * float(eager.fc.weight.grad.abs().max()))
