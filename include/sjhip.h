@@ -441,7 +441,9 @@ int sjhip_ssa_backward_packed(int dtype, int64_t samples, int heads, int channel
  * gradients.  fp32 operands are split into `terms` bf16 terms that sum to the value (3: exactly), and the products whose
  * combined order is below max(terms) run on v_mfma_f32_32x32x16_bf16 with fp32 accumulation: 3 terms on both sides give
  * the accuracy of an fp32 GEMM; an operand that bf16 holds exactly (spikes) needs 1 term.  Supported (a_terms, b_terms):
- * (3,3) (3,1) (2,2) (2,1) (1,1).  L must be a multiple of 4 and the tensors 16-byte aligned (SJHIP_ERR_UNSUPPORTED).
+ * (3,3) (3,1) (2,2) (2,1) (1,1).  sjhip_pwconv_gemm needs an even L, 16-byte aligned weight planes and 8-byte
+ * aligned activations; sjhip_pwconv_grad_weight needs L a multiple of 4 and 16-byte aligned tensors
+ * (SJHIP_ERR_UNSUPPORTED otherwise).
  *
  *   sjhip_pwconv_split_weight   planes = bf16 terms [3][rows_pad][cols_pad] (zero padded to multiples of 128 and 32;
  *                               sjhip_pwconv_planes_elems(rows, cols) elements of 2 bytes) of the matrix A = w
