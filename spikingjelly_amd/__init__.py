@@ -8,3 +8,5 @@ for gfx950 behind the C ABI of ``libsjhip.so``.
 """
 
 __version__ = "0.1.0"
+
+from .install import install  # noqa: E402,F401
