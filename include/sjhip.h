@@ -247,10 +247,10 @@ int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_pa
  * `checkpoints` [pieces - 1][N] (storage dtype; may be NULL when T <= chunk).  sjhip_neuron_backward_recompute_pieces
  * is sjhip_neuron_backward_recompute that walks the pieces from the last to the first: each is replayed from its
  * checkpoint into an LDS buffer of `chunk` steps (so chunk, not T, must satisfy sjhip_recompute_supported) and walked
- * back; the gradient of a piece's initial state reaches the piece before it through `carry` [N] (storage dtype,
- * scratch, contents undefined afterwards; may be NULL when T <= chunk).  Results: spikes, states and checkpoints are
- * bit-identical to sjhip_neuron_forward's; gradients are those of sjhip_neuron_backward_recompute on each piece, with
- * the carry rounded to the storage dtype between pieces (no rounding for fp32).  N must be a multiple of the 128-bit
+ * back; the gradient of a piece's initial state stays in registers (fp32) for the piece before it.  Results: spikes,
+ * states and checkpoints are bit-identical to sjhip_neuron_forward's; gradients are those of the walk over the whole
+ * sequence (in fp32 storage also those of sjhip_neuron_backward_recompute applied piece by piece with grad_v_init
+ * handed on as grad_v_last).  N must be a multiple of the 128-bit
  * vector width and every tensor 16-byte aligned; 16-bit storage with SJHIP_FLAG_FP32_STATE is refused
  * (SJHIP_ERR_UNSUPPORTED: a checkpoint in the storage dtype would round the state).  The saved state per neuron is 1 / chunk of an h_seq; chunk = 16 keeps
  * five or more blocks resident per compute unit, which is where the single-piece kernel runs fastest.  No counterpart
@@ -268,7 +268,7 @@ int sjhip_neuron_backward_recompute_pieces(int neuron, int dtype, const sjhip_ne
                                            const void *checkpoints,
                                            const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
                                            void *grad_x_seq, void *grad_v_init,
-                                           float *grad_rtau, float *workspace, void *carry,
+                                           float *grad_rtau, float *workspace,
                                            void *stream);
 
 /* 1 if sjhip_neuron_backward_recompute can serve [T,N] of `dtype` (N a multiple of the 128-bit vector

@@ -182,7 +182,7 @@ def load() -> ctypes.CDLL:
         lib.sjhip_neuron_backward_recompute_pieces.argtypes = [
             c_int, c_int, POINTER(NeuronParams), c_int64, c_int64, c_int64,
             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
         ]
         lib.sjhip_recompute_supported.restype = c_int
         lib.sjhip_recompute_supported.argtypes = [c_int, c_int64, c_int64]

@@ -231,7 +231,6 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
     grad_x_seq = torch.empty_like(h_seq)
     # a state that needs no gradient (the usual case: it was the reset value) costs no [N] write
     grad_v_init = h_seq.new_empty((N,) if need_grad_v_init else (0,))
-    carry = h_seq.new_empty((N,)) if pieces > 1 else None  # gradient handed from a piece to the one before
     grad_k = workspace = None
     k_keep, k_ptr = _k_pointer(k, h_seq)
     if neuron == L.NEURON_PLIF:
@@ -252,7 +251,7 @@ def _run_backward(neuron: int, grad_spike_seq: Optional[torch.Tensor], grad_v_se
                 neuron, dtype, ctypes.byref(params), T, N, chunk,
                 h_seq.data_ptr(), v_init.data_ptr(), k_ptr, L.aligned16(checkpoints).data_ptr(),
                 L.ptr(grad_spike_seq), L.ptr(grad_v_seq), L.ptr(grad_v_last),
-                grad_x_seq.data_ptr(), carry_out, L.ptr(grad_k), L.ptr(workspace), carry.data_ptr(), stream,
+                grad_x_seq.data_ptr(), carry_out, L.ptr(grad_k), L.ptr(workspace), stream,
             )
         elif recompute:
             rc = lib.sjhip_neuron_backward_recompute(

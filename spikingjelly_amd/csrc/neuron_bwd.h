@@ -182,10 +182,19 @@ template <typename S, bool VECTOR, bool SHORT = false> struct BwdPrologue {
   }
 };
 
+// How the gradient with respect to the state enters and leaves a walk.  Ordinarily through memory (grad_v_last in,
+// grad_v_init out).  A kernel that walks a sequence piece by piece keeps it in registers from one piece to the one
+// before it: `regs` holds the work-item's V values; `from_regs` / `to_regs` say which side of this walk uses them.
+struct StateGradient {
+  float *regs = nullptr;
+  bool from_regs = false, to_regs = false;
+};
+
 template <typename S, bool VECTOR, int MODE, int SG, bool GVFULL, int HLDS = 0>
 __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, int64_t col, float k,
                                                const f32x4 *lds_h = nullptr,
-                                               const BwdPrologue<S, VECTOR, BwdModeOf<MODE>::SHORT> *pre = nullptr) {
+                                               const BwdPrologue<S, VECTOR, BwdModeOf<MODE>::SHORT> *pre = nullptr,
+                                               const StateGradient sgr = StateGradient()) {
   typedef Acc<S, VECTOR, SJHIP_BWD_NT != 0> A;
   typedef typename A::elem_t E;
   constexpr int V = A::V;
@@ -226,7 +235,10 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
   }
 
   float carry[V];
-  if (a.grad_v_last) {
+  if (sgr.from_regs) {
+#pragma unroll
+    for (int j = 0; j < V; ++j) carry[j] = sgr.regs[j];
+  } else if (a.grad_v_last) {
     A::unpack(A::load((const E *)a.grad_v_last + col), carry);
   } else {
 #pragma unroll
@@ -318,15 +330,19 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
     }
   }
   if (QIF) {
-    if (a.grad_v_init) {
+    if (a.grad_v_init || sgr.to_regs) {
       float v0[V];
       load_state<S, VECTOR, SJHIP_BWD_NT != 0>(a.v_init, col, a.v_init_broadcast != 0, v0);
 #pragma unroll
       for (int j = 0; j < V; ++j) carry[j] *= qif_dh_dv(v0[j], k, a);
-      A::store((E *)a.grad_v_init + col, carry);
+      if (!sgr.to_regs) A::store((E *)a.grad_v_init + col, carry);
     }
-  } else if (a.grad_v_init) {
+  } else if (a.grad_v_init && !sgr.to_regs) {
     A::store((E *)a.grad_v_init + col, carry);
+  }
+  if (sgr.to_regs) {
+#pragma unroll
+    for (int j = 0; j < V; ++j) sgr.regs[j] = carry[j];
   }
   if (PLIF) {
     float v0[V];
@@ -344,26 +360,28 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
 template <typename S, bool VECTOR, int MODE, int SG, int HLDS = 0>
 __device__ __forceinline__ float backward_gv_dispatch(const BwdArgs &a, bool active, int64_t col, float k,
                                                       const f32x4 *lds_h = nullptr,
-                                                      const BwdPrologue<S, VECTOR, BwdModeOf<MODE>::SHORT> *pre = nullptr) {
-  if (a.grad_v_seq) return backward_body<S, VECTOR, MODE, SG, true, HLDS>(a, active, col, k, lds_h, pre);
-  return backward_body<S, VECTOR, MODE, SG, false, HLDS>(a, active, col, k, lds_h, pre);
+                                                      const BwdPrologue<S, VECTOR, BwdModeOf<MODE>::SHORT> *pre = nullptr,
+                                                      const StateGradient sgr = StateGradient()) {
+  if (a.grad_v_seq) return backward_body<S, VECTOR, MODE, SG, true, HLDS>(a, active, col, k, lds_h, pre, sgr);
+  return backward_body<S, VECTOR, MODE, SG, false, HLDS>(a, active, col, k, lds_h, pre, sgr);
 }
 
 template <typename S, bool VECTOR, int MODE, int HLDS>
 __device__ __forceinline__ float backward_sg_dispatch(const BwdArgs &a, bool active, int64_t col, float k,
                                                       const f32x4 *lds_h,
-                                                      const BwdPrologue<S, VECTOR, BwdModeOf<MODE>::SHORT> *pre = nullptr) {
+                                                      const BwdPrologue<S, VECTOR, BwdModeOf<MODE>::SHORT> *pre = nullptr,
+                                                      const StateGradient sgr = StateGradient()) {
   switch (a.sg) {
-    case SJHIP_SG_SIGMOID: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SIGMOID, HLDS>(a, active, col, k, lds_h, pre);
-    case SJHIP_SG_ATAN: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_ATAN, HLDS>(a, active, col, k, lds_h, pre);
-    case SJHIP_SG_PIECEWISE_QUADRATIC: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_PIECEWISE_QUADRATIC, HLDS>(a, active, col, k, lds_h, pre);
-    case SJHIP_SG_PIECEWISE_EXP: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_PIECEWISE_EXP, HLDS>(a, active, col, k, lds_h, pre);
-    case SJHIP_SG_SOFT_SIGN: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SOFT_SIGN, HLDS>(a, active, col, k, lds_h, pre);
-    case SJHIP_SG_SUPER_SPIKE: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SUPER_SPIKE, HLDS>(a, active, col, k, lds_h, pre);
+    case SJHIP_SG_SIGMOID: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SIGMOID, HLDS>(a, active, col, k, lds_h, pre, sgr);
+    case SJHIP_SG_ATAN: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_ATAN, HLDS>(a, active, col, k, lds_h, pre, sgr);
+    case SJHIP_SG_PIECEWISE_QUADRATIC: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_PIECEWISE_QUADRATIC, HLDS>(a, active, col, k, lds_h, pre, sgr);
+    case SJHIP_SG_PIECEWISE_EXP: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_PIECEWISE_EXP, HLDS>(a, active, col, k, lds_h, pre, sgr);
+    case SJHIP_SG_SOFT_SIGN: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SOFT_SIGN, HLDS>(a, active, col, k, lds_h, pre, sgr);
+    case SJHIP_SG_SUPER_SPIKE: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_SUPER_SPIKE, HLDS>(a, active, col, k, lds_h, pre, sgr);
     case SJHIP_SG_MULTI_LEVEL:
-      if constexpr (BwdModeOf<MODE>::BASE == BWD_PLAIN) return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_MULTI_LEVEL, HLDS>(a, active, col, k, lds_h, pre);
+      if constexpr (BwdModeOf<MODE>::BASE == BWD_PLAIN) return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_MULTI_LEVEL, HLDS>(a, active, col, k, lds_h, pre, sgr);
       return 0.0f;
-    default: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_ERF, HLDS>(a, active, col, k, lds_h, pre);
+    default: return backward_gv_dispatch<S, VECTOR, MODE, SJHIP_SG_ERF, HLDS>(a, active, col, k, lds_h, pre, sgr);
   }
 }
 

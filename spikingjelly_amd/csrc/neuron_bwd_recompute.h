@@ -129,8 +129,8 @@ __device__ __forceinline__ void keep_uniform_local(BwdArgs &a) {
 
 // A sequence too long for one LDS buffer, walked piece by piece from the last to the first inside one launch: each
 // piece is replayed from its checkpoint (left by forward_pieces_kernel) into the same LDS buffer of `chunk` steps and
-// walked back; the gradient of the piece's initial state goes through p.carry to the piece before it.  The two phases
-// are the ones of backward_recompute_kernel, called with the pointers and the length of the piece.
+// walked back; the gradient of the piece's initial state stays in registers (fp32) for the piece before it.  The two
+// phases are the ones of backward_recompute_kernel, called with the pointers and the length of the piece.
 template <typename S, bool ROUND_EACH, int MODE>
 __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_pieces_kernel(const FwdArgs f0, const BwdArgs b0,
                                                                                     const PieceArgs p) {
@@ -144,6 +144,9 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_pieces_ker
   constexpr int HLDS = (ROUND_EACH && sizeof(S) == 2) ? 2 : 1;
   const int64_t N = b0.N;
   float part = 0.0f;
+  float state_gradient[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) state_gradient[i] = 0.0f;
   for (int64_t j = p.pieces - 1; j >= 0; --j) {
     const int64_t t0 = j * p.chunk;
     const int64_t len = (b0.T - t0 < p.chunk) ? b0.T - t0 : p.chunk;
@@ -154,14 +157,16 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_pieces_ker
     if (j > 0) {
       f.v_init = (const E *)p.checkpoints + (j - 1) * N;
       f.v_init_broadcast = 0;
-      b.grad_v_init = p.carry;
     }
     b.v_init = f.v_init;
     b.v_init_broadcast = f.v_init_broadcast;
     if (b0.grad_spike) b.grad_spike = (const E *)b0.grad_spike + t0 * N;
     if (b0.grad_v_seq) b.grad_v_seq = (const E *)b0.grad_v_seq + t0 * N;
     b.grad_x = (E *)b0.grad_x + t0 * N;
-    if (j + 1 < p.pieces) b.grad_v_last = p.carry;
+    StateGradient sgr;
+    sgr.regs = state_gradient;
+    sgr.from_regs = j + 1 < p.pieces;
+    sgr.to_regs = j > 0;
     keep_uniform_local(f);
     keep_uniform_local(b);
     float kj = k;
@@ -172,7 +177,7 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_pieces_ker
       pre.load(b, col);
       recompute_charge_dispatch<S, ROUND_EACH, false>(f, lds_h, col);
     }
-    part += backward_sg_dispatch<S, true, MODE, HLDS>(b, active, col, kj, lds_h, &pre);
+    part += backward_sg_dispatch<S, true, MODE, HLDS>(b, active, col, kj, lds_h, &pre, sgr);
   }
   if (BwdModeOf<MODE>::BASE == BWD_PLIF) plif_block_reduce(b0, part, k);
 }

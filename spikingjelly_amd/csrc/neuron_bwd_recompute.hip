@@ -50,7 +50,7 @@ namespace {
 int launch_replay(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N, int64_t chunk,
                   const void *x_seq, const void *v_init, const float *k_device, const void *checkpoints,
                   const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
-                  void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace, void *carry,
+                  void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace,
                   hipStream_t stream) {
   const int64_t lds_steps = chunk > 0 ? chunk : T;
   if (!recompute_supported(dtype, lds_steps, N))
@@ -88,7 +88,7 @@ int launch_replay(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T
   // better), unlike the single-piece kernel, which keeps the stride rule of column_spread().
   if (chunk > 0 && T > chunk && tuning().column_spread == 2) b.spread = 1;
   PieceArgs piece_args;
-  piece_args.checkpoints = const_cast<void *>(checkpoints); piece_args.carry = carry; piece_args.chunk = chunk;
+  piece_args.checkpoints = const_cast<void *>(checkpoints); piece_args.chunk = chunk;
   piece_args.pieces = chunk > 0 ? (T + chunk - 1) / chunk : 1;
   const PieceArgs *pieces = chunk > 0 ? &piece_args : nullptr;
   {
@@ -119,18 +119,18 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
                               void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace,
                               hipStream_t stream) {
   return launch_replay(neuron, dtype, p, T, N, 0, x_seq, v_init, k_device, nullptr, grad_spike_seq, grad_v_seq, grad_v_last,
-                       grad_x_seq, grad_v_init, grad_rtau, workspace, nullptr, stream);
+                       grad_x_seq, grad_v_init, grad_rtau, workspace, stream);
 }
 
 int launch_backward_recompute_pieces(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N, int64_t chunk,
                                      const void *x_seq, const void *v_init, const float *k_device, const void *checkpoints,
                                      const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
-                                     void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace, void *carry,
+                                     void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace,
                                      hipStream_t stream) {
-  if (chunk < 1 || (T > chunk && (checkpoints == nullptr || carry == nullptr)) || !aligned16(checkpoints) || !aligned16(carry))
-    return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): chunk=%lld needs 16-byte aligned checkpoints and carry", (long long)chunk);
+  if (chunk < 1 || (T > chunk && checkpoints == nullptr) || !aligned16(checkpoints))
+    return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): chunk=%lld needs 16-byte aligned checkpoints", (long long)chunk);
   return launch_replay(neuron, dtype, p, T, N, chunk, x_seq, v_init, k_device, checkpoints, grad_spike_seq, grad_v_seq,
-                       grad_v_last, grad_x_seq, grad_v_init, grad_rtau, workspace, carry, stream);
+                       grad_v_last, grad_x_seq, grad_v_init, grad_rtau, workspace, stream);
 }
 
 }  // namespace sjhip

@@ -71,6 +71,8 @@ struct FwdArgs {
   int soft_reset;        // a Reset value
   int v_init_broadcast;  // v_init holds one element for all neurons
   int spread;            // block-to-column order, see column_block()
+  void *checkpoints;     // forward_pieces_kernel only: [ceil(T / chunk) - 1][N] states after every chunk steps
+  int64_t chunk;
 };
 
 // Fire-and-reset rule.  RESET_COUNT is ILIF (functional/neuron.py:1097-1099 with quantize.py:592): the neuron fires
@@ -247,7 +249,9 @@ enum FwdOut { FWD_OUT_DENSE = 0, FWD_OUT_PACKED = 1, FWD_OUT_DENSE_STREAM_X = 2 
 // at T = 2 and 4 the effect is mixed and the deep prefetch stays).
 constexpr int FWD_OUT_SHORT = 4;
 
-template <typename S, bool VECTOR, bool ROUND_EACH, int CH, int RS, int OUT>
+// CKPT: besides its outputs the walk leaves the state after every a.chunk steps (but not after the last step) in
+// a.checkpoints, from where the replaying backward starts each piece of a long sequence.
+template <typename S, bool VECTOR, bool ROUND_EACH, int CH, int RS, int OUT, bool CKPT = false>
 __device__ __forceinline__ void forward_body(const FwdArgs &a) {
   constexpr bool PACKED = (OUT & 3) == FWD_OUT_PACKED;
   // with bit-packed spikes the kernel is read-dominated (x in, one bit out): streaming policy like the backward
@@ -278,6 +282,8 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
   NUM v[V];
   load_state<S, VECTOR, NT>(a.v_init, col, a.v_init_broadcast != 0, v);
 
+  int64_t next_checkpoint = CKPT ? a.chunk : 0;  // the step count after which the next checkpoint is due
+  E *cp = CKPT ? (E *)a.checkpoints + col : nullptr;
   for (int64_t t0 = 0; t0 < T; t0 += PF) {
     typename A::raw_t cur[PF];
 #pragma unroll
@@ -300,25 +306,30 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
         else A::store_spikes(sp + t * N, s);
         if (hp) A::store(hp + t * N, h);
         if (vp) A::store(vp + t * N, v);
+        if (CKPT && t + 1 == next_checkpoint && t + 1 < T) {
+          A::store(cp, v);
+          cp += N;
+          next_checkpoint += a.chunk;
+        }
       }
     }
   }
   if (a.v_last) A::store((E *)a.v_last + col, v);
 }
 
-template <typename S, bool VECTOR, bool ROUND_EACH, int CH, int OUT>
+template <typename S, bool VECTOR, bool ROUND_EACH, int CH, int OUT, bool CKPT = false>
 __device__ __forceinline__ void forward_reset_dispatch(const FwdArgs &a) {
   // counts exist for the charge ILIF uses (no input decay) and never bit-packed
   if constexpr ((CH == CH_PLAIN_INPUT_DIV || CH == CH_PLAIN_INPUT_MUL) && (OUT & 3) != FWD_OUT_PACKED) {
     if (a.soft_reset == RESET_COUNT) {
-      forward_body<S, VECTOR, ROUND_EACH, CH, RESET_COUNT, OUT>(a);
+      forward_body<S, VECTOR, ROUND_EACH, CH, RESET_COUNT, OUT, CKPT>(a);
       return;
     }
   }
   if (a.soft_reset)
-    forward_body<S, VECTOR, ROUND_EACH, CH, RESET_SOFT, OUT>(a);
+    forward_body<S, VECTOR, ROUND_EACH, CH, RESET_SOFT, OUT, CKPT>(a);
   else
-    forward_body<S, VECTOR, ROUND_EACH, CH, RESET_HARD, OUT>(a);
+    forward_body<S, VECTOR, ROUND_EACH, CH, RESET_HARD, OUT, CKPT>(a);
 }
 
 template <typename S, bool VECTOR, bool ROUND_EACH, int OUT = FWD_OUT_DENSE>
@@ -336,36 +347,20 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) forward_kernel(const FwdArgs 
   }
 }
 
-// The same forward over a long sequence cut into pieces, in one launch: piece j runs forward_body on rows
-// [j chunk, (j + 1) chunk) starting from the state piece j - 1 left in the checkpoint row, which the same work-item
-// wrote.  What remains in `checkpoints` is what the replaying backward starts each piece from.
+// The forward of a long sequence that the backward will replay in pieces: the ordinary walk over all T steps, which
+// also leaves the state after every a.chunk steps in a.checkpoints.
 template <typename S, bool ROUND_EACH>
-__global__ void __launch_bounds__(SJHIP_MAX_BLOCK) forward_pieces_kernel(const FwdArgs a, const PieceArgs p) {
-  typedef typename Acc<S, true, false>::elem_t E;
-  for (int64_t j = 0; j < p.pieces; ++j) {
-    FwdArgs f = a;
-    const int64_t t0 = j * p.chunk;
-    f.T = (a.T - t0 < p.chunk) ? a.T - t0 : p.chunk;
-    f.x = (const E *)a.x + t0 * a.N;
-    f.spike = (E *)a.spike + t0 * a.N;
-    if (a.v_seq) f.v_seq = (E *)a.v_seq + t0 * a.N;
-    f.h = nullptr;
-    if (j > 0) {
-      f.v_init = (const E *)p.checkpoints + (j - 1) * a.N;
-      f.v_init_broadcast = 0;
-    }
-    if (j + 1 < p.pieces) f.v_last = (E *)p.checkpoints + j * a.N;
-    switch (f.charge) {
-      case CH_IF: forward_reset_dispatch<S, true, ROUND_EACH, CH_IF, FWD_OUT_DENSE>(f); break;
-      case CH_DECAY_INPUT_DIV: forward_reset_dispatch<S, true, ROUND_EACH, CH_DECAY_INPUT_DIV, FWD_OUT_DENSE>(f); break;
-      case CH_DECAY_INPUT_MUL: forward_reset_dispatch<S, true, ROUND_EACH, CH_DECAY_INPUT_MUL, FWD_OUT_DENSE>(f); break;
-      case CH_PLAIN_INPUT_DIV: forward_reset_dispatch<S, true, ROUND_EACH, CH_PLAIN_INPUT_DIV, FWD_OUT_DENSE>(f); break;
-      case CH_QIF_DIV: forward_reset_dispatch<S, true, ROUND_EACH, CH_QIF_DIV, FWD_OUT_DENSE>(f); break;
-      case CH_QIF_MUL: forward_reset_dispatch<S, true, ROUND_EACH, CH_QIF_MUL, FWD_OUT_DENSE>(f); break;
-      case CH_EIF_DIV: forward_reset_dispatch<S, true, ROUND_EACH, CH_EIF_DIV, FWD_OUT_DENSE>(f); break;
-      case CH_EIF_MUL: forward_reset_dispatch<S, true, ROUND_EACH, CH_EIF_MUL, FWD_OUT_DENSE>(f); break;
-      default: forward_reset_dispatch<S, true, ROUND_EACH, CH_PLAIN_INPUT_MUL, FWD_OUT_DENSE>(f); break;
-    }
+__global__ void __launch_bounds__(SJHIP_MAX_BLOCK) forward_pieces_kernel(const FwdArgs a) {
+  switch (a.charge) {
+    case CH_IF: forward_reset_dispatch<S, true, ROUND_EACH, CH_IF, FWD_OUT_DENSE, true>(a); break;
+    case CH_DECAY_INPUT_DIV: forward_reset_dispatch<S, true, ROUND_EACH, CH_DECAY_INPUT_DIV, FWD_OUT_DENSE, true>(a); break;
+    case CH_DECAY_INPUT_MUL: forward_reset_dispatch<S, true, ROUND_EACH, CH_DECAY_INPUT_MUL, FWD_OUT_DENSE, true>(a); break;
+    case CH_PLAIN_INPUT_DIV: forward_reset_dispatch<S, true, ROUND_EACH, CH_PLAIN_INPUT_DIV, FWD_OUT_DENSE, true>(a); break;
+    case CH_QIF_DIV: forward_reset_dispatch<S, true, ROUND_EACH, CH_QIF_DIV, FWD_OUT_DENSE, true>(a); break;
+    case CH_QIF_MUL: forward_reset_dispatch<S, true, ROUND_EACH, CH_QIF_MUL, FWD_OUT_DENSE, true>(a); break;
+    case CH_EIF_DIV: forward_reset_dispatch<S, true, ROUND_EACH, CH_EIF_DIV, FWD_OUT_DENSE, true>(a); break;
+    case CH_EIF_MUL: forward_reset_dispatch<S, true, ROUND_EACH, CH_EIF_MUL, FWD_OUT_DENSE, true>(a); break;
+    default: forward_reset_dispatch<S, true, ROUND_EACH, CH_PLAIN_INPUT_MUL, FWD_OUT_DENSE, true>(a); break;
   }
 }
 
@@ -375,6 +370,7 @@ inline int build_fwd_args(FwdArgs &a, bool &round_each, int neuron, int dtype, c
                           void *spike_seq, void *v_seq, void *v_last, void *h_seq) {
   a.x = x_seq; a.v_init = v_init; a.spike = spike_seq; a.v_seq = v_seq; a.v_last = v_last; a.h = h_seq;
   a.k_device = nullptr;
+  a.checkpoints = nullptr; a.chunk = 0;
   a.T = T; a.N = N;
   a.spread = column_spread(N * (dtype == SJHIP_F32 ? 4 : 2)) ? 1 : 0;
   const bool ilif = neuron == SJHIP_NEURON_ILIF;

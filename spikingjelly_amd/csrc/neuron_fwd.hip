@@ -52,14 +52,14 @@ int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   return check_launch(PACKED ? "forward_packed" : "forward");
 }
 
-template <typename S, bool ROUND_EACH> int launch_pieces_typed(const FwdArgs &a, const PieceArgs &p, hipStream_t stream) {
+template <typename S, bool ROUND_EACH> int launch_pieces_typed(const FwdArgs &a, hipStream_t stream) {
   const int block = tuning().fwd_block;
   const int64_t items = a.N / Acc<S, true, true>::V;
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "forward(pieces): N=%lld", (long long)a.N);
   const unsigned lds = (sizeof(S) == 4 && a.v_seq != nullptr) ? occupancy_cap_lds(tuning().fwd_blocks_per_cu) : 0u;
   ProfileScope prof(KC_FORWARD, stream);
-  hipLaunchKernelGGL((forward_pieces_kernel<S, ROUND_EACH>), dim3((unsigned)blocks), dim3(block), lds, stream, a, p);
+  hipLaunchKernelGGL((forward_pieces_kernel<S, ROUND_EACH>), dim3((unsigned)blocks), dim3(block), lds, stream, a);
   return check_launch("forward(pieces)");
 }
 
@@ -76,12 +76,11 @@ int launch_forward_pieces(int neuron, int dtype, const sjhip_neuron_params &p, i
   if (N % V != 0 || !aligned16(x_seq) || !(a.v_init_broadcast || aligned16(v_init)) || !aligned16(spike_seq) || !aligned16(v_seq) ||
       !aligned16(v_last) || !aligned16(checkpoints))
     return fail(SJHIP_ERR_UNSUPPORTED, "forward(pieces): N=%lld must be a multiple of %d and every tensor 16-byte aligned", (long long)N, V);
-  PieceArgs pieces;
-  pieces.checkpoints = checkpoints; pieces.carry = nullptr; pieces.chunk = chunk; pieces.pieces = (T + chunk - 1) / chunk;
+  a.checkpoints = checkpoints; a.chunk = chunk;
   switch (dtype) {
-    case SJHIP_F32: return launch_pieces_typed<float, false>(a, pieces, stream);
-    case SJHIP_F16: return round_each ? launch_pieces_typed<f16_t, true>(a, pieces, stream) : launch_pieces_typed<f16_t, false>(a, pieces, stream);
-    case SJHIP_BF16: return round_each ? launch_pieces_typed<bf16_t, true>(a, pieces, stream) : launch_pieces_typed<bf16_t, false>(a, pieces, stream);
+    case SJHIP_F32: return launch_pieces_typed<float, false>(a, stream);
+    case SJHIP_F16: return round_each ? launch_pieces_typed<f16_t, true>(a, stream) : launch_pieces_typed<f16_t, false>(a, stream);
+    case SJHIP_BF16: return round_each ? launch_pieces_typed<bf16_t, true>(a, stream) : launch_pieces_typed<bf16_t, false>(a, stream);
     default: return fail(SJHIP_ERR_INVALID, "forward(pieces): dtype %d", dtype);
   }
 }

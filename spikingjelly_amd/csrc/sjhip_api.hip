@@ -376,7 +376,7 @@ int sjhip_neuron_backward_recompute_pieces(int neuron, int dtype, const sjhip_ne
                                            int64_t chunk, const void *x_seq, const void *v_init, const float *rtau_device,
                                            const void *checkpoints, const void *grad_spike_seq, const void *grad_v_seq,
                                            const void *grad_v_last, void *grad_x_seq, void *grad_v_init, float *grad_rtau,
-                                           float *workspace, void *carry, void *stream) {
+                                           float *workspace, void *stream) {
   if (!p) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): params is NULL");
   if (neuron < SJHIP_NEURON_IF || neuron > SJHIP_NEURON_EIF) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): neuron %d", neuron);
   if (!valid_dtype_fp(dtype)) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): dtype %d", dtype);
@@ -385,7 +385,7 @@ int sjhip_neuron_backward_recompute_pieces(int neuron, int dtype, const sjhip_ne
   if (rc != SJHIP_OK) return rc;
   if (chunk < 1) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): chunk %lld", (long long)chunk);
   if (!x_seq || !v_init || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): NULL tensor");
-  if (T > chunk && (!checkpoints || !carry)) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): several pieces need checkpoints and carry");
+  if (T > chunk && !checkpoints) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): several pieces need checkpoints");
   if (dtype != SJHIP_F32 && (p->flags & SJHIP_FLAG_FP32_STATE))
     return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute, pieces): an fp32 state does not survive a checkpoint of 16-bit storage");
   rc = check_levels("backward(recompute, pieces)", neuron, *p, true);
@@ -395,7 +395,7 @@ int sjhip_neuron_backward_recompute_pieces(int neuron, int dtype, const sjhip_ne
     if (!(p->flags & SJHIP_FLAG_ATOMIC_REDUCE) && !workspace) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): PLIF needs a workspace unless SJHIP_FLAG_ATOMIC_REDUCE");
   }
   return launch_backward_recompute_pieces(neuron, dtype, *p, T, N, chunk, x_seq, v_init, rtau_device, checkpoints, grad_spike_seq,
-                                          grad_v_seq, grad_v_last, grad_x_seq, grad_v_init, grad_rtau, workspace, carry,
+                                          grad_v_seq, grad_v_last, grad_x_seq, grad_v_init, grad_rtau, workspace,
                                           static_cast<hipStream_t>(stream));
 }
 

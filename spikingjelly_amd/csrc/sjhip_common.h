@@ -317,11 +317,9 @@ static inline bool exact_reciprocal(float f) {
 
 // A long sequence handled as consecutive pieces of `chunk` steps inside one launch: the forward leaves the state after
 // every piece but the last in `checkpoints` ([pieces - 1][N], storage dtype), the replaying backward starts each piece
-// from there and hands the gradient of a piece's initial state to the piece before it through `carry` ([N]).  A
-// work-item only ever reads back what it wrote itself, so no synchronisation is involved.
+// from there and keeps the gradient of a piece's initial state in registers for the piece before it.
 struct PieceArgs {
   void *checkpoints;
-  void *carry;
   int64_t chunk;
   int64_t pieces;
 };
@@ -368,7 +366,7 @@ int launch_forward_pieces(int neuron, int dtype, const sjhip_neuron_params &p, i
 int launch_backward_recompute_pieces(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N, int64_t chunk,
                                      const void *x_seq, const void *v_init, const float *k_device, const void *checkpoints,
                                      const void *grad_spike_seq, const void *grad_v_seq, const void *grad_v_last,
-                                     void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace, void *carry,
+                                     void *grad_x_seq, void *grad_v_init, float *grad_rtau, float *workspace,
                                      hipStream_t stream);
 int launch_forward_packed(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,
                           const void *x_seq, const void *v_init, const float *k_device, uint8_t *spike_bits,

@@ -1,10 +1,13 @@
 """``sjhip_neuron_forward_pieces`` / ``sjhip_neuron_backward_recompute_pieces`` through the C ABI.
 
 The forward over pieces must equal ``sjhip_neuron_forward`` over the whole sequence bit for bit (spikes, states) and
-its checkpoints must be the states ``v_seq`` holds at the piece boundaries.  The backward over pieces must equal, bit
-for bit, ``sjhip_neuron_backward_recompute`` called once per piece from the last to the first with the gradient of the
-piece's initial state handed on as ``grad_v_last`` (piece lengths above the short-sequence variant's, so both run the
-same device code); PLIF's dL/dk is a sum in another order (rtol 1e-5).  fp32 is also checked against the oracle.
+its checkpoints must be the states ``v_seq`` holds at the piece boundaries.  The backward over pieces keeps the gradient
+of a piece's initial state in fp32 registers for the piece before it.  In fp32 storage it must equal, bit for bit,
+``sjhip_neuron_backward_recompute`` called once per piece from the last to the first with ``grad_v_init`` handed on as
+``grad_v_last`` (piece lengths above the short-sequence variant's, so both run the same device code); in 16-bit storage
+that hand-over through memory rounds, so there the reference is ``sjhip_neuron_backward`` over the whole sequence on a
+saved ``h_seq`` (the same fp32 carry throughout), within one rounding of the storage dtype.  PLIF's dL/dk is a sum in
+another order.  fp32 is also checked against the oracle.
 """
 
 import ctypes
@@ -79,14 +82,28 @@ def _plif_buffers(L, c):
 
 def _backward_pieces(L, c, chunk, ck, with_gv):
     gx, gv0 = torch.full_like(c["x"], float("nan")), torch.full_like(c["v0"], float("nan"))
-    carry = torch.full_like(c["v0"], float("nan"))
     gk, ws = _plif_buffers(L, c)
     L.check(L.load().sjhip_neuron_backward_recompute_pieces(
         c["neuron"], L.dtype_id(c["dtype"]), ctypes.byref(c["p"]), c["T"], c["N"], chunk, c["x"].data_ptr(), c["v0"].data_ptr(),
         _kd(L, c), ck.data_ptr() if ck.numel() else None, c["gs"].data_ptr(), c["gv"].data_ptr() if with_gv else None,
-        c["gl"].data_ptr(), gx.data_ptr(), gv0.data_ptr(), L.ptr(gk), L.ptr(ws), carry.data_ptr(), c["stream"]),
+        c["gl"].data_ptr(), gx.data_ptr(), gv0.data_ptr(), L.ptr(gk), L.ptr(ws), c["stream"]),
         "backward_recompute_pieces")
     return gx, gv0, gk
+
+
+def _backward_whole_saved_h(L, c, with_gv):
+    """sjhip_neuron_forward saving h_seq, then sjhip_neuron_backward over the whole sequence."""
+    lib = L.load()
+    s, v, h = torch.empty_like(c["x"]), torch.empty_like(c["x"]), torch.empty_like(c["x"])
+    L.check(lib.sjhip_neuron_forward(c["neuron"], L.dtype_id(c["dtype"]), ctypes.byref(c["p"]), c["T"], c["N"], c["x"].data_ptr(),
+                                     c["v0"].data_ptr(), _kd(L, c), s.data_ptr(), v.data_ptr(), None, h.data_ptr(), c["stream"]),
+            "forward")
+    gx, gv0 = torch.full_like(c["x"], float("nan")), torch.full_like(c["v0"], float("nan"))
+    gk, ws = _plif_buffers(L, c)
+    L.check(lib.sjhip_neuron_backward(c["neuron"], L.dtype_id(c["dtype"]), ctypes.byref(c["p"]), c["T"], c["N"], c["gs"].data_ptr(),
+                                      c["gv"].data_ptr() if with_gv else None, c["gl"].data_ptr(), h.data_ptr(), c["v0"].data_ptr(),
+                                      _kd(L, c), gx.data_ptr(), gv0.data_ptr(), L.ptr(gk), L.ptr(ws), c["stream"]), "backward")
+    return gx, gv0, (float(gk.item()) if gk is not None else 0.0)
 
 
 def _backward_piece_by_piece(L, c, chunk, ck, with_gv):
@@ -135,10 +152,17 @@ def test_pieces_equal_whole_forward_and_piecewise_backward(L, dtype, neuron_name
     assert bits_equal(s2, s) and bits_equal(vl2, vl) and bits_equal(ck2, ck)
     for with_gv in (True, False):
         got = _backward_pieces(L, c, chunk, ck, with_gv)
-        ref = _backward_piece_by_piece(L, c, chunk, ck, with_gv)
-        torch.cuda.synchronize()
-        assert bits_equal(got[0], ref[0]), "grad_x_seq"
-        assert bits_equal(got[1], ref[1]), "grad_v_init"
+        if dtype == torch.float32:
+            ref = _backward_piece_by_piece(L, c, chunk, ck, with_gv)
+            torch.cuda.synchronize()
+            assert bits_equal(got[0], ref[0]), "grad_x_seq"
+            assert bits_equal(got[1], ref[1]), "grad_v_init"
+        else:
+            ref = _backward_whole_saved_h(L, c, with_gv)
+            torch.cuda.synchronize()
+            ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7  # one rounding of the storage dtype
+            torch.testing.assert_close(got[0].float(), ref[0].float(), rtol=ulp, atol=1e-4)
+            torch.testing.assert_close(got[1].float(), ref[1].float(), rtol=ulp, atol=1e-4)
         if neuron == L.NEURON_PLIF:
             assert float(got[2].item()) == pytest.approx(ref[2], rel=1e-3 if dtype != torch.float32 else 1e-5, abs=1e-3)
 
@@ -172,7 +196,7 @@ def test_pieces_argument_checks(L):
     gx = torch.empty_like(c["x"])
     assert lib.sjhip_neuron_backward_recompute_pieces(*head[:3], 400, 64, 200, c["x"].data_ptr(), c["v0"].data_ptr(), None,
                                                       ck.data_ptr(), c["gs"].data_ptr(), None, None, gx.data_ptr(), None, None,
-                                                      None, vl.data_ptr(), c["stream"]) == ERR_UNSUPPORTED
+                                                      None, c["stream"]) == ERR_UNSUPPORTED
     # an fp32 state over 16-bit storage would be rounded at every checkpoint
     c = _case(L, L.NEURON_LIF, torch.float16, 40, 64, L.FLAG_DECAY_INPUT | L.FLAG_FP32_STATE, 3)
     ck16 = torch.empty((2, 64), dtype=torch.float16, device="cuda:0")
