@@ -198,7 +198,7 @@ __device__ __forceinline__ void bptt_rows(const BwdArgs &b, float k, int64_t col
       for (int j = 0; j < 4; ++j) {
         const float over = h[t][j] - b.v_th;
         const float s = (over >= 0.0f) ? 1.0f : 0.0f;
-        const float sg = surrogate_grad<SG, false>(over, b.alpha);
+        const float sg = surrogate_grad<SG, true>(over, b.alpha);  // hardware exp2 and reciprocal (1 ulp each): this kernel is bound by its arithmetic
         const float dvdh = (1.0f - s * b.cB) + (b.cC - h[t][j] * b.cD) * sg;
         const float G = carry[j] * dvdh + gs[j] * sg;
         gz[j] = G * kx;
