@@ -50,7 +50,34 @@ __device__ __forceinline__ double wave_sum_all(double v) {
   return v;
 }
 
-// one wavefront per row of L contiguous elements: sum and sum of squares
+// Sums of two per-work-item values over the rows of a block in which work-item tid holds a piece of row r_local
+// (consecutive work-items, consecutive rows): per wavefront one masked reduction per row it touches, the results left
+// in LDS, then one work-item per row adds the wavefronts' shares in their order and writes (sum0, sum1) of row
+// first_row + r to out[2 (first_row + r)].  Every work-item of the block must call it.
+constexpr int kBnRowsMax = 16;  // rows per block: rows of at least 16 quads
+__device__ __forceinline__ void block_row_sums(float (&part)[4][kBnRowsMax][2], int r_local, bool valid, int rows_per_block,
+                                               float v0, float v1, float *out, int64_t first_row, int64_t rows) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (lane < rows_per_block) { part[wave][lane][0] = 0.0f; part[wave][lane][1] = 0.0f; }
+  const int r_first = __builtin_amdgcn_readfirstlane(r_local);
+  const int r_last = __builtin_amdgcn_readlane(r_local, 63);
+  for (int r = r_first; r <= r_last; ++r) {
+    const bool mine = valid && r_local == r;
+    const float s0 = wave_sum(mine ? v0 : 0.0f), s1 = wave_sum(mine ? v1 : 0.0f);
+    if (lane == 0) { part[wave][r][0] = s0; part[wave][r][1] = s1; }
+  }
+  __syncthreads();
+  if (tid < rows_per_block && first_row + tid < rows) {
+    float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) { s0 += part[w][tid][0]; s1 += part[w][tid][1]; }
+    out[2 * (first_row + tid)] = s0;
+    out[2 * (first_row + tid) + 1] = s1;
+  }
+}
+
+// one wavefront per row of L contiguous elements: sum and sum of squares (several whole rows per block with the
+// row sums through LDS, as in bn_lif_backward_rows_kernel, measured slower here: 52 against 37 us on [256, 1152, 196])
 __global__ void __launch_bounds__(256) bn_stats_kernel(const float *y, int64_t rows, int L, float *partial) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -211,49 +238,74 @@ __device__ __forceinline__ void bptt_rows(const BwdArgs &b, float k, int64_t col
   }
 }
 
-template <int TMAX> __global__ void __launch_bounds__(256) bn_lif_backward_kernel(const BnLifBwdArgs a) {
+// One work-item's four neurons (quad q of row `row`) for all T steps: replay, BPTT, g written, the sums extended.
+template <int TMAX>
+__device__ __forceinline__ void bn_lif_backward_quad(const BnLifBwdArgs &a, int64_t row, int q, float &acc_g, float &acc_gy) {
   typedef Acc<float, true, false> A;
-  const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= a.rows) return;
   const FwdArgs &f = a.f;
   const BwdArgs &b = a.b;
   const int c = (int)(row % a.C);
   const float sc = a.scale[c], sh = a.shift[c];
   const float k = b.k;
   const int64_t N = f.N;
-  float acc_g = 0.0f, acc_gy = 0.0f;
-  for (int q = lane; q < a.L / 4; q += 64) {
-    const int64_t col = row * a.L + 4 * q;
-    const float *yp = (const float *)f.x + col;
-    f32x4 yv[TMAX];
+  const int64_t col = row * a.L + 4 * q;
+  const float *yp = (const float *)f.x + col;
+  f32x4 yv[TMAX];
 #pragma unroll
-    for (int t = 0; t < TMAX; ++t) yv[t] = (t < f.T) ? A::load(yp + (int64_t)t * N) : A::zero();
-    float v[4], h[TMAX][4], carry[4];
-    load_state<float, true, false>(f.v_init, col, f.v_init_broadcast != 0, v);
-    if (b.grad_v_last) A::unpack(A::load((const float *)b.grad_v_last + col), carry);
-    else carry[0] = carry[1] = carry[2] = carry[3] = 0.0f;
-    switch (f.charge) {
-      case CH_IF: replay_h_reset<CH_IF, TMAX>(f, yv, sc, sh, v, h); break;
-      case CH_DECAY_INPUT_DIV: replay_h_reset<CH_DECAY_INPUT_DIV, TMAX>(f, yv, sc, sh, v, h); break;
-      case CH_DECAY_INPUT_MUL: replay_h_reset<CH_DECAY_INPUT_MUL, TMAX>(f, yv, sc, sh, v, h); break;
-      case CH_PLAIN_INPUT_DIV: replay_h_reset<CH_PLAIN_INPUT_DIV, TMAX>(f, yv, sc, sh, v, h); break;
-      default: replay_h_reset<CH_PLAIN_INPUT_MUL, TMAX>(f, yv, sc, sh, v, h); break;
-    }
-    switch (b.sg) {
-      case SJHIP_SG_SIGMOID: bptt_rows<SJHIP_SG_SIGMOID, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-      case SJHIP_SG_ATAN: bptt_rows<SJHIP_SG_ATAN, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-      case SJHIP_SG_PIECEWISE_QUADRATIC: bptt_rows<SJHIP_SG_PIECEWISE_QUADRATIC, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-      case SJHIP_SG_PIECEWISE_EXP: bptt_rows<SJHIP_SG_PIECEWISE_EXP, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-      case SJHIP_SG_SOFT_SIGN: bptt_rows<SJHIP_SG_SOFT_SIGN, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-      case SJHIP_SG_SUPER_SPIKE: bptt_rows<SJHIP_SG_SUPER_SPIKE, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-      default: bptt_rows<SJHIP_SG_ERF, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-    }
-    if (b.grad_v_init) A::store((float *)b.grad_v_init + col, carry);
+  for (int t = 0; t < TMAX; ++t) yv[t] = (t < f.T) ? A::load(yp + (int64_t)t * N) : A::zero();
+  float v[4], h[TMAX][4], carry[4];
+  load_state<float, true, false>(f.v_init, col, f.v_init_broadcast != 0, v);
+  if (b.grad_v_last) A::unpack(A::load((const float *)b.grad_v_last + col), carry);
+  else carry[0] = carry[1] = carry[2] = carry[3] = 0.0f;
+  switch (f.charge) {
+    case CH_IF: replay_h_reset<CH_IF, TMAX>(f, yv, sc, sh, v, h); break;
+    case CH_DECAY_INPUT_DIV: replay_h_reset<CH_DECAY_INPUT_DIV, TMAX>(f, yv, sc, sh, v, h); break;
+    case CH_DECAY_INPUT_MUL: replay_h_reset<CH_DECAY_INPUT_MUL, TMAX>(f, yv, sc, sh, v, h); break;
+    case CH_PLAIN_INPUT_DIV: replay_h_reset<CH_PLAIN_INPUT_DIV, TMAX>(f, yv, sc, sh, v, h); break;
+    default: replay_h_reset<CH_PLAIN_INPUT_MUL, TMAX>(f, yv, sc, sh, v, h); break;
   }
+  switch (b.sg) {
+    case SJHIP_SG_SIGMOID: bptt_rows<SJHIP_SG_SIGMOID, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+    case SJHIP_SG_ATAN: bptt_rows<SJHIP_SG_ATAN, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+    case SJHIP_SG_PIECEWISE_QUADRATIC: bptt_rows<SJHIP_SG_PIECEWISE_QUADRATIC, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+    case SJHIP_SG_PIECEWISE_EXP: bptt_rows<SJHIP_SG_PIECEWISE_EXP, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+    case SJHIP_SG_SOFT_SIGN: bptt_rows<SJHIP_SG_SOFT_SIGN, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+    case SJHIP_SG_SUPER_SPIKE: bptt_rows<SJHIP_SG_SUPER_SPIKE, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+    default: bptt_rows<SJHIP_SG_ERF, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+  }
+  if (b.grad_v_init) A::store((float *)b.grad_v_init + col, carry);
+}
+
+// A wavefront per row; lanes stride over the row's quads.
+template <int TMAX> __global__ void __launch_bounds__(256) bn_lif_backward_kernel(const BnLifBwdArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.rows) return;
+  float acc_g = 0.0f, acc_gy = 0.0f;
+  for (int q = lane; q < a.L / 4; q += 64) bn_lif_backward_quad<TMAX>(a, row, q, acc_g, acc_gy);
   acc_g = wave_sum(acc_g);
   acc_gy = wave_sum(acc_gy);
   if (lane == 0) { a.partial[2 * row] = acc_g; a.partial[2 * row + 1] = acc_gy; }
+}
+
+// Rows of fewer than 64 quads leave lanes of a wavefront-per-row kernel idle (196 positions: 49 of 64 working), and this
+// kernel is bound by its arithmetic.  Here a block of 256 work-items takes as many whole rows as fit (five rows of 49
+// quads: 245 working); a row's sums are formed per wavefront (a wavefront holds parts of a few rows: one masked
+// reduction per row it touches), left in LDS, and added over the wavefronts in their order by one work-item per row,
+// so the result does not depend on timing.
+template <int TMAX>
+__global__ void __launch_bounds__(256) bn_lif_backward_rows_kernel(const BnLifBwdArgs a, int quads, int rows_per_block,
+                                                                   float inv_quads) {
+  __shared__ float part[4][kBnRowsMax][2];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int r_local = (int)(((float)tid + 0.5f) * inv_quads);  // tid / quads (exact: see div_tokens of ssa.hip)
+  const int q = tid - r_local * quads;
+  const int64_t row = (int64_t)blockIdx.x * rows_per_block + r_local;
+  const bool valid = r_local < rows_per_block && row < a.rows;
+  if (r_local >= rows_per_block) r_local = rows_per_block - 1;
+  float acc_g = 0.0f, acc_gy = 0.0f;
+  if (valid) bn_lif_backward_quad<TMAX>(a, row, q, acc_g, acc_gy);
+  block_row_sums(part, r_local, valid, rows_per_block, acc_g, acc_gy, a.partial, (int64_t)blockIdx.x * rows_per_block, a.rows);
 }
 
 // dgamma, dbeta and the coefficients of dy = p g + q y + r; count = T * B * L elements per channel
@@ -383,6 +435,18 @@ int launch_bn_lif_backward(int neuron, const sjhip_neuron_params &p, int64_t T, 
   const int64_t blocks = (a.rows + 3) / 4;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "bn_lif_backward: %lld rows", (long long)a.rows);
   ProfileScope prof(KC_BN_LIF_BACKWARD, stream);
+  const int quads = (int)(L / 4);
+  const int per = quads > 0 ? 256 / quads : 0;
+  if (quads >= 16 && per > 4) {
+    // more than the four rows a block of the wavefront-per-row kernel takes: more lanes working
+    const int64_t nb = (a.rows + per - 1) / per;
+    if (nb > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "bn_lif_backward: %lld rows", (long long)a.rows);
+    const float inv = 1.0f / (float)quads;
+    if (T <= 4) hipLaunchKernelGGL((bn_lif_backward_rows_kernel<4>), dim3((unsigned)nb), dim3(256), 0, stream, a, quads, per, inv);
+    else if (T <= 8) hipLaunchKernelGGL((bn_lif_backward_rows_kernel<8>), dim3((unsigned)nb), dim3(256), 0, stream, a, quads, per, inv);
+    else hipLaunchKernelGGL((bn_lif_backward_rows_kernel<16>), dim3((unsigned)nb), dim3(256), 0, stream, a, quads, per, inv);
+    return check_launch("bn_lif_backward");
+  }
   if (T <= 4) hipLaunchKernelGGL((bn_lif_backward_kernel<4>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
   else if (T <= 8) hipLaunchKernelGGL((bn_lif_backward_kernel<8>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
   else hipLaunchKernelGGL((bn_lif_backward_kernel<16>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
