@@ -248,24 +248,29 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       mfma_step<TA, TB>(af, bf, acc);
     }
   };
-  fetch_a(0);
-  fetch_b(0, 0);
-  if (kTileK < K_pad) fetch_b(kTileK, 1);
-  for (int k0 = 0; k0 < K_pad; k0 += 2 * kTileK) {
+  // One K step: stage the tile whose loads were requested earlier, request later tiles, multiply.  In the steady state
+  // both requests are unconditional, so the compiler knows how many younger loads are outstanding when it waits for the
+  // tile being staged and leaves them in flight; a request under a condition makes it wait for everything (vmcnt(0)),
+  // which is tolerable only in the last steps.
+  auto step = [&](int k0, int set, bool more_a, bool more_b) {
     __syncthreads();  // the previous tile has been read by every wavefront
-    stage(k0, 0);
+    stage(k0, set);
     __syncthreads();
-    if (k0 + kTileK < K_pad) fetch_a(k0 + kTileK);
-    if (k0 + 2 * kTileK < K_pad) fetch_b(k0 + 2 * kTileK, 0);
+    if (more_a) fetch_a(k0 + kTileK);
+    if (more_b) fetch_b(k0 + 2 * kTileK, set);
     multiply();
-    if (k0 + kTileK >= K_pad) break;
-    __syncthreads();
-    stage(k0 + kTileK, 1);
-    __syncthreads();
-    if (k0 + 2 * kTileK < K_pad) fetch_a(k0 + 2 * kTileK);
-    if (k0 + 3 * kTileK < K_pad) fetch_b(k0 + 3 * kTileK, 1);
-    multiply();
+  };
+  fetch_b(0, 0);
+  fetch_a(0);
+  fetch_b(kTileK, 1);  // rows beyond K are clamped, the tile is never staged then
+  int k0 = 0;
+  for (; k0 + 3 * kTileK < K_pad; k0 += 2 * kTileK) {
+    step(k0, 0, true, true);
+    step(k0 + kTileK, 1, true, true);
   }
+  if (k0 < K_pad) step(k0, 0, k0 + kTileK < K_pad, k0 + 2 * kTileK < K_pad);
+  if (k0 + kTileK < K_pad) step(k0 + kTileK, 1, k0 + 2 * kTileK < K_pad, false);
+  if (k0 + 2 * kTileK < K_pad) step(k0 + 2 * kTileK, 0, false, false);
 
   // accumulator register r of a 32 x 32 tile: row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
 #pragma unroll
@@ -408,21 +413,24 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       mfma_step<TA, TB>(af, bf, acc);
     }
   };
+  // as in pw_gemm_kernel: unconditional requests in the steady state, conditions only in the last steps
+  auto step = [&](int64_t it, int set, bool more) {
+    __syncthreads();
+    stage(it, set);
+    __syncthreads();
+    if (more) fetch(it + 2, set);
+    multiply(it);
+  };
   if (iters > 0) fetch(0, 0);
   if (iters > 1) fetch(1, 1);
-  for (int64_t it = 0; it < iters; it += 2) {
-    __syncthreads();
-    stage(it, 0);
-    __syncthreads();
-    if (it + 2 < iters) fetch(it + 2, 0);
-    multiply(it);
-    if (it + 1 >= iters) break;
-    __syncthreads();
-    stage(it + 1, 1);
-    __syncthreads();
-    if (it + 3 < iters) fetch(it + 3, 1);
-    multiply(it + 1);
+  int64_t it = 0;
+  for (; it + 3 < iters; it += 2) {
+    step(it, 0, true);
+    step(it + 1, 1, true);
   }
+  if (it < iters) step(it, 0, it + 2 < iters);
+  if (it + 1 < iters) step(it + 1, 1, false);
+  if (it + 2 < iters) step(it + 2, 0, false);
 
   float *out = a.partials + (int64_t)chunk * M * N;
 #pragma unroll
