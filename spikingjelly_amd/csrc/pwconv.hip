@@ -23,7 +23,12 @@
 //       products, 124 fp32-equivalent TFLOP/s.  Timing the kernel with parts cut out (only the loads 0.12 ms, only the
 //       staging 0.05, only fragment reads + MFMA 0.15, empty loop + stores 0.07) gives parts that add up to the whole,
 //       and neither wavefronts specialised as producers and consumers over two LDS buffers nor fewer, wider loads
-//       changed the total: the phases do not hide behind each other on this chip at this matrix-core load.
+//       changed the total: the phases do not hide behind each other on this chip at this matrix-core load.  Later
+//       measurements on the same shape: tile requests made unconditional in the steady state of the K loop (a request
+//       under a condition turns every later wait into a wait for all outstanding loads): 0.318 -> 0.301 ms; two LDS
+//       buffers of half the depth with one barrier per step, staging of the next tile and multiplication of the current
+//       one in the same step: 0.334 ms, and 0.352 ms with scheduler hints that ask for the staging instructions between
+//       the matrix-core instructions; not kept.
 //   pw_dw_kernel       dW[m][n] = sum_{s,l} dY[s][m][l] X[s][n][l]
 //       both operands are contiguous along the contraction index l; a block owns a 128 x 128 tile of dW for a chunk
 //       of samples and writes its partial tile, dw_reduce_kernel adds the chunks in a fixed order.
