@@ -59,8 +59,10 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr unsigned kSsaMaxLds = 159u * 1024u;
-constexpr int kSsaThreads = 256;
-constexpr int kSsaWaves = kSsaThreads / 64;
+// Work-items per block: four wavefronts for heads of up to 32 channels, eight for larger ones (measured at 64 channels,
+// 196 tokens: backward 355 -> 290 us; at 32 channels eight wavefronts change nothing backward and cost 20 % forward).
+// Device code asks blockDim.x.
+constexpr int ssa_threads(int mc) { return mc == 1 ? 256 : 512; }
 
 struct SsaArgs {
   const uint8_t *qkv_bits;  // when set, the spikes come bit-packed (LSB first over the flattened tensor) and qkv is unused
@@ -114,21 +116,21 @@ __device__ __forceinline__ int div_tokens(int e, float inv_L) { return (int)(((f
 template <int NS>
 __device__ __forceinline__ void zero_fill_bytes(uint8_t *const (&dst)[NS], int cph, int rows_pad, int L, int Lb) {
   const int tid = threadIdx.x;
-  for (int r = tid >> 3; r < cph; r += kSsaThreads / 8)
+  for (int r = tid >> 3; r < cph; r += ((int)blockDim.x / 8))
     for (int c = L + (tid & 7); c < Lb; c += 8) {
 #pragma unroll
       for (int s = 0; s < NS; ++s) dst[s][r * Lb + c] = 0;
     }
-  for (int i = tid; i < (rows_pad - cph) * (Lb / 4); i += kSsaThreads) {
+  for (int i = tid; i < (rows_pad - cph) * (Lb / 4); i += (int)blockDim.x) {
 #pragma unroll
     for (int s = 0; s < NS; ++s) reinterpret_cast<uint32_t *>(dst[s] + cph * Lb)[i] = 0u;
   }
 }
 __device__ __forceinline__ void zero_fill_f32(float *dst, int cph, int rows_pad, int L, int Lq) {
   const int tid = threadIdx.x;
-  for (int r = tid >> 3; r < cph; r += kSsaThreads / 8)
+  for (int r = tid >> 3; r < cph; r += ((int)blockDim.x / 8))
     for (int c = L + (tid & 7); c < Lq; c += 8) dst[r * Lq + c] = 0.0f;
-  for (int i = tid; i < (rows_pad - cph) * Lq; i += kSsaThreads) dst[cph * Lq + i] = 0.0f;
+  for (int i = tid; i < (rows_pad - cph) * Lq; i += (int)blockDim.x) dst[cph * Lq + i] = 0.0f;
 }
 
 // Global tiles -> LDS.  NS spike tiles ([cph, L] each) become
@@ -144,11 +146,11 @@ __device__ __forceinline__ void stage_tiles(const typename Io<S>::elem_t *const 
   if (vec) {
     const int G = cph * L / 4;
     const float inv_L = 1.0f / (float)L;
-    for (int g0 = tid; g0 < G; g0 += kSsaThreads * UN) {
+    for (int g0 = tid; g0 < G; g0 += (int)blockDim.x * UN) {
       Q buf[UN][NS + (DO ? 1 : 0)];
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
-        const int g = g0 + u * kSsaThreads;
+        const int g = g0 + u * (int)blockDim.x;
         if (g < G) {
 #pragma unroll
           for (int s = 0; s < NS; ++s) buf[u][s] = reinterpret_cast<const Q *>(src[s])[g];
@@ -157,7 +159,7 @@ __device__ __forceinline__ void stage_tiles(const typename Io<S>::elem_t *const 
       }
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
-        const int g = g0 + u * kSsaThreads;
+        const int g = g0 + u * (int)blockDim.x;
         if (g < G) {
           const int r = div_tokens(4 * g, inv_L), c = 4 * g - r * L;
           float f[4];
@@ -176,7 +178,7 @@ __device__ __forceinline__ void stage_tiles(const typename Io<S>::elem_t *const 
     }
   } else {
     const int n = cph * L;
-    for (int i = tid; i < n; i += kSsaThreads) {
+    for (int i = tid; i < n; i += (int)blockDim.x) {
       const int r = i / L, c = i - r * L;
 #pragma unroll
       for (int s = 0; s < NS; ++s) dst[s][r * Lb + c] = Io<S>::get(src[s], i) != 0.0f ? 1 : 0;
@@ -225,11 +227,11 @@ __device__ __forceinline__ void stage_bits(const uint8_t *const (&src)[NS], uint
   const int tid = threadIdx.x;
   const int nbytes = cph * L / 8;
   const float inv_L = 1.0f / (float)L;
-  for (int b0 = tid; b0 < nbytes; b0 += kSsaThreads * UB) {
+  for (int b0 = tid; b0 < nbytes; b0 += (int)blockDim.x * UB) {
     uint32_t w[UB][NS];
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
-      const int b = b0 + u * kSsaThreads;
+      const int b = b0 + u * (int)blockDim.x;
       if (b < nbytes) {
 #pragma unroll
         for (int s = 0; s < NS; ++s) w[u][s] = src[s][b];
@@ -237,7 +239,7 @@ __device__ __forceinline__ void stage_bits(const uint8_t *const (&src)[NS], uint
     }
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
-      const int b = b0 + u * kSsaThreads;
+      const int b = b0 + u * (int)blockDim.x;
       if (b < nbytes) expand_byte<NS>(w[u], b, dst, L, Lb, inv_L);
     }
   }
@@ -264,22 +266,22 @@ __device__ __forceinline__ void stage_grad_out(const typename Io<S>::elem_t *do_
     const int G = cph * L / 4;
     const float inv_L = 1.0f / (float)L;
     constexpr int UN = 4;
-    for (int g0 = tid; g0 < G; g0 += kSsaThreads * UN) {
+    for (int g0 = tid; g0 < G; g0 += (int)blockDim.x * UN) {
       Q buf[UN];
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
-        const int g = g0 + u * kSsaThreads;
+        const int g = g0 + u * (int)blockDim.x;
         if (g < G) buf[u] = reinterpret_cast<const Q *>(do_src)[g];
       }
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
-        const int g = g0 + u * kSsaThreads;
+        const int g = g0 + u * (int)blockDim.x;
         if (g < G) put_grad_out_quad<S>(buf[u], g, do_dst, L, Lq, inv_L);
       }
     }
   } else {
     const int n = cph * L;
-    for (int i = tid; i < n; i += kSsaThreads) {
+    for (int i = tid; i < n; i += (int)blockDim.x) {
       const int r = i / L, c = i - r * L;
       do_dst[r * Lq + c] = Io<S>::get(do_src, i);
     }
@@ -324,7 +326,7 @@ struct Bf16Terms {
 __device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
 
 template <typename S, int MC>
-__global__ void __launch_bounds__(kSsaThreads) ssa_forward_kernel(const SsaArgs a) {
+__global__ void __launch_bounds__(ssa_threads(MC)) ssa_forward_kernel(const SsaArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char ssa_lds[];
   typedef typename Io<S>::elem_t E;
   constexpr int CPH = 32 * MC;
@@ -375,7 +377,7 @@ __global__ void __launch_bounds__(kSsaThreads) ssa_forward_kernel(const SsaArgs 
   }
 
   E *og = static_cast<E *>(a.out) + p * tile;
-  for (int u = wave; u < units; u += kSsaWaves) {
+  for (int u = wave; u < units; u += ((int)blockDim.x >> 6)) {
     const int nt = u / MC;
     const int col = nt * 32 + (lane & 31);
     const int colc = col < L ? col : L - 1;
@@ -410,7 +412,7 @@ __global__ void __launch_bounds__(kSsaThreads) ssa_forward_kernel(const SsaArgs 
 }
 
 template <typename S, int MC>
-__global__ void __launch_bounds__(kSsaThreads, MC == 1 ? SJHIP_SSA_BWD_RESIDENT : 1) ssa_backward_kernel(const SsaArgs a) {
+__global__ void __launch_bounds__(ssa_threads(MC), MC == 1 ? SJHIP_SSA_BWD_RESIDENT : 1) ssa_backward_kernel(const SsaArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char ssa_lds[];
   typedef typename Io<S>::elem_t E;
   constexpr int CPH = 32 * MC;
@@ -451,7 +453,7 @@ __global__ void __launch_bounds__(kSsaThreads, MC == 1 ? SJHIP_SSA_BWD_RESIDENT 
     constexpr int NB = CPH / 16;
     const int Lk = (L + 15) & ~15;
     const int i16 = lane & 15, kq = lane >> 4;
-    for (int sb = wave; sb < NB * NB; sb += kSsaWaves) {
+    for (int sb = wave; sb < NB * NB; sb += ((int)blockDim.x >> 6)) {
       const int bi = sb / NB, bj = sb - bi * NB;
       const float *ap = do_lds + (16 * bi + i16) * Lq + 4 * kq;
       const uint8_t *bp = q_lds + (16 * bj + i16) * Lb + 4 * kq;
@@ -492,7 +494,7 @@ __global__ void __launch_bounds__(kSsaThreads, MC == 1 ? SJHIP_SSA_BWD_RESIDENT 
       }
     }
     // One product at a time: sixteen accumulator registers live instead of forty-eight.
-    for (int nt = wave; nt < ntiles; nt += kSsaWaves) {
+    for (int nt = wave; nt < ntiles; nt += ((int)blockDim.x >> 6)) {
       const int col = nt * 32 + m32;
       const int colc = col < L ? col : L - 1;
       const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -589,8 +591,8 @@ unsigned backward_lds(int cph, int L) {
 }
 
 template <typename K>
-int launch_with_lds(K kernel, const SsaArgs &a, unsigned lds, hipStream_t stream, std::once_flag &once, hipError_t &attr_rc,
-                    const char *what) {
+int launch_with_lds(K kernel, const SsaArgs &a, int threads, unsigned lds, hipStream_t stream, std::once_flag &once,
+                    hipError_t &attr_rc, const char *what) {
   std::call_once(once, [&]() {
     attr_rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)kSsaMaxLds);
@@ -598,7 +600,7 @@ int launch_with_lds(K kernel, const SsaArgs &a, unsigned lds, hipStream_t stream
   });
   if (lds > 64u * 1024u && attr_rc != hipSuccess)
     return fail(SJHIP_ERR_LAUNCH, "%s: cannot raise the dynamic LDS limit: %s", what, hipGetErrorString(attr_rc));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)a.problems), dim3(kSsaThreads), lds, stream, a);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)a.problems), dim3(threads), lds, stream, a);
   return check_launch(what);
 }
 
@@ -606,13 +608,13 @@ template <typename S, int MC>
 int launch_fwd(const SsaArgs &a, hipStream_t stream) {
   static std::once_flag once;
   static hipError_t attr_rc = hipSuccess;
-  return launch_with_lds(ssa_forward_kernel<S, MC>, a, forward_lds(a.cph, a.L), stream, once, attr_rc, "ssa_forward");
+  return launch_with_lds(ssa_forward_kernel<S, MC>, a, ssa_threads(MC), forward_lds(a.cph, a.L), stream, once, attr_rc, "ssa_forward");
 }
 template <typename S, int MC>
 int launch_bwd(const SsaArgs &a, hipStream_t stream) {
   static std::once_flag once;
   static hipError_t attr_rc = hipSuccess;
-  return launch_with_lds(ssa_backward_kernel<S, MC>, a, backward_lds(a.cph, a.L), stream, once, attr_rc, "ssa_backward");
+  return launch_with_lds(ssa_backward_kernel<S, MC>, a, ssa_threads(MC), backward_lds(a.cph, a.L), stream, once, attr_rc, "ssa_backward");
 }
 
 template <typename S>
