@@ -284,19 +284,23 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
 
   int64_t next_checkpoint = CKPT ? a.chunk : 0;  // the step count after which the next checkpoint is due
   E *cp = CKPT ? (E *)a.checkpoints + col : nullptr;
-  for (int64_t t0 = 0; t0 < T; t0 += PF) {
+  // PF steps: requests the rows of the PF steps after them, then walks them.  STEADY: every one of those 2 * PF
+  // rows exists, so no request stands under a condition; a request under a condition would make each later wait
+  // a wait for everything outstanding, the rows just requested included.
+  auto walk = [&](int64_t t0, auto steady) {
+    constexpr bool STEADY = decltype(steady)::value;
     typename A::raw_t cur[PF];
 #pragma unroll
     for (int i = 0; i < PF; ++i) cur[i] = ahead[i];
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int64_t tn = t0 + PF + i;
-      if (tn < T) ahead[i] = AL::load(xp + tn * N);
+      if (STEADY || tn < T) ahead[i] = AL::load(xp + tn * N);
     }
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int64_t t = t0 + i;
-      if (t < T) {
+      if (STEADY || t < T) {
         NUM x[V], h[V], s[V];
         A::unpack(cur[i], x);
 #pragma unroll
@@ -313,7 +317,12 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
         }
       }
     }
+  };
+  int64_t t0 = 0;
+  if constexpr (CKPT) {  // long sequences only: the shorter ones gain nothing from the second copy of the loop
+    for (; t0 + 2 * PF <= T; t0 += PF) walk(t0, std::true_type());
   }
+  for (; t0 < T; t0 += PF) walk(t0, std::false_type());
   if (a.v_last) A::store((E *)a.v_last + col, v);
 }
 

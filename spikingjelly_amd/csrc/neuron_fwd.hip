@@ -53,7 +53,12 @@ int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
 }
 
 template <typename S, bool ROUND_EACH> int launch_pieces_typed(const FwdArgs &a, hipStream_t stream) {
-  const int block = tuning().fwd_block;
+  // From 64 steps on, one wavefront per block: the steady-state loop keeps a block's next rows in flight while it
+  // computes, so half the resident work-items still fill the memory pipeline, and with a fixed number of neuron-steps
+  // a longer sequence means fewer, longer blocks, whose last round leaves less of the chip idle when they are small
+  // (2^29 neuron-steps, fp32, T = 64 / 128 / 512: 1.198 / 1.234 / 1.327 ms against 1.231 / 1.283 / 1.398 with 128
+  // lanes; T = 48: 1.304 against 1.283).
+  const int block = a.T >= 64 && tuning().fwd_block > 64 ? 64 : tuning().fwd_block;
   const int64_t items = a.N / Acc<S, true, true>::V;
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "forward(pieces): N=%lld", (long long)a.N);
