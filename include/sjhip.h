@@ -445,8 +445,9 @@ int sjhip_ssa_backward_packed(int dtype, int64_t samples, int heads, int channel
  * aligned activations; sjhip_pwconv_grad_weight needs L a multiple of 4 and 16-byte aligned tensors
  * (SJHIP_ERR_UNSUPPORTED otherwise).
  *
- *   sjhip_pwconv_split_weight   planes = bf16 terms [3][rows_pad][cols_pad] (zero padded to multiples of 128 and 32;
- *                               sjhip_pwconv_planes_elems(rows, cols) elements of 2 bytes) of the matrix A = w
+ *   sjhip_pwconv_split_weight   planes = bf16 terms [3][rows_pad * cols_pad] (zero padded to multiples of 128 and 32, and
+ *                               stored as tiles of 128 rows x 32 columns in the order sjhip_pwconv_gemm reads them: an
+ *                               opaque buffer of sjhip_pwconv_planes_elems(rows, cols) elements of 2 bytes) of the matrix A = w
  *                               ([rows][cols] fp32) or, with transpose != 0, of A = w^T ([cols][rows]): the first operand
  *                               of sjhip_pwconv_gemm.  For transpose the element count is that of (cols, rows).
  *   sjhip_pwconv_gemm           c[s][m][l] = sum_k A[m][k] b[s][k][l]: the convolution with A = weight [Cout][Cin]

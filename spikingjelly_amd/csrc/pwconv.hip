@@ -11,7 +11,8 @@
 // halves the products.  Fewer terms trade accuracy for speed (two terms: about 2^-17 relative per product).
 //
 //   pw_gemm_kernel     C[s][m][l] = sum_k A[m][k] B[s][k][l]     (forward with A = W, input gradient with A = W^T)
-//       A comes pre-split as bf16 planes [3][M_pad][K_pad] (split_weight_kernel, zero padded), B is fp32 in memory.
+//       A comes pre-split as bf16 planes [3][M_pad / 128][K_pad / 32][128][32] (split_weight_kernel, zero padded), B is
+//       fp32 in memory.
 //       The S * L columns of all samples form one column index, so tiles of 128 columns carry no padding whatever L
 //       is.  A block of four wavefronts owns a 128 x 128 tile (each wavefront 64 x 64 = 2 x 2 MFMA tiles) and walks K
 //       in steps of 32.  The matrix cores want, per lane, eight consecutive k of one row (A) or column (B): A tiles are
@@ -28,7 +29,17 @@
 //       under a condition turns every later wait into a wait for all outstanding loads): 0.318 -> 0.301 ms; two LDS
 //       buffers of half the depth with one barrier per step, staging of the next tile and multiplication of the current
 //       one in the same step: 0.334 ms, and 0.352 ms with scheduler hints that ask for the staging instructions between
-//       the matrix-core instructions; not kept.
+//       the matrix-core instructions; not kept.  Two groups of four wavefronts per block, each with its own tile and
+//       one barrier apart so that one group multiplies while the other stages: 0.339 against 0.345 ms on random data,
+//       not kept either.  Cycle counters around the phases of a K step (one wavefront, steady state): with one block
+//       per compute unit staging 1150, multiplication 2160 (48 matrix-core instructions of 32 cycles: 71 %), barriers
+//       320 cycles, 30.8 us per tile = 1.46 GHz; with two blocks 1280 / 3060 / 360 cycles and 49.3 us per tile =
+//       1.2 GHz.  The chip lowers its clock as the matrix cores fill (the same launch on an all-zero input takes 0.265
+//       instead of 0.330 ms), so what a better overlap of the phases gains in cycles is largely lost in clock rate.
+//       By number of products (M = 1152, K = 384, random data): 1 product 0.15-0.16 ms, 2: 0.17-0.18, 3: 0.22,
+//       6: 0.33-0.35.  The weight planes are stored tile by tile ([row tile][k step][row][k], 8 KiB per staged tile in
+//       a row) so that every 128-byte line a block fetches is used whole: 0.345 -> 0.338 ms, one-term activations
+//       0.229 -> 0.215 ms.
 //   pw_dw_kernel       dW[m][n] = sum_{s,l} dY[s][m][l] X[s][n][l]
 //       both operands are contiguous along the contraction index l; a block owns a 128 x 128 tile of dW for a chunk
 //       of samples and writes its partial tile, dw_reduce_kernel adds the chunks in a fixed order.
@@ -96,13 +107,15 @@ __global__ void __launch_bounds__(256) split_weight_kernel(const float *src, int
   }
   uint32_t w[3];
   split_pair<3>(x0, x1, w);
+  // tile order: the 128 rows x 32 k that a block stages in one step are 8 KiB in a row, [row tile][k step][row][k]
+  const int64_t at = (((r / kTile) * (cols_pad / kTileK) + c / kTileK) * kTile + r % kTile) * kTileK + c % kTileK;
 #pragma unroll
   for (int t = 0; t < 3; ++t)
-    reinterpret_cast<uint32_t *>(planes + (int64_t)t * rows_pad * cols_pad)[(r * cols_pad + c) / 2] = w[t];
+    reinterpret_cast<uint32_t *>(planes + (int64_t)t * rows_pad * cols_pad)[at / 2] = w[t];
 }
 
 struct PwGemmArgs {
-  const uint16_t *a_planes;  // [3][M_pad][K_pad] bf16
+  const uint16_t *a_planes;  // [3][M_pad / 128][K_pad / 32][128][32] bf16
   const float *b;            // [S][K][L]
   float *c;                  // [S][M][L]
   int64_t plane_stride;      // M_pad * K_pad
@@ -164,7 +177,7 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int q = tid + kPwThreads * i, row = q >> 2, kc = q & 3;
-    a_off[i] = (uint32_t)(((m0 + row) * K_pad + 8 * kc) * 2);
+    a_off[i] = (uint32_t)((mb * (K_pad / kTileK) * (kTile * kTileK) + 8 * q) * 2);
     a_dst[i] = row * kRowBytes + kc * 16;
   }
   // B: eight k (one fragment) of two adjacent columns, fetched as 8-byte accesses: columns 2 (tid % 64) and the next,
@@ -190,7 +203,7 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   auto fetch_a = [&](int k0) {
 #pragma unroll
     for (int t = 0; t < TA; ++t) {
-      const char *plane = a_base + ((int64_t)t * a.plane_stride + k0) * 2;
+      const char *plane = a_base + ((int64_t)t * a.plane_stride + (int64_t)(k0 / kTileK) * (kTile * kTileK)) * 2;
 #pragma unroll
       for (int i = 0; i < 2; ++i) ra[t][i] = *reinterpret_cast<const u32x4 *>(plane + a_off[i]);
     }
