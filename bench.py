@@ -115,18 +115,22 @@ def measure_ceilings(torch, L, floats_per_stream: int, repeats: int = 5):
 
 
 def _time_steps(torch, L, step, steps, warmup):
-    """warm-up, then `steps` timed steps bracketed by synchronisation; library event profiler on."""
+    """warm-up, then `steps` timed steps bracketed by synchronisation, then the same steps once more under the library's
+    event profiler for the per-kernel durations: its two events per launch would otherwise sit in the timed region of
+    workloads with dozens of short launches per step (the attention block: 1.88 against 1.77 ms per step)."""
     for _ in range(warmup):
         step()
-    torch.cuda.synchronize()
-    L.profile_reset()
-    L.profile_enable(True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    L.profile_reset()
+    L.profile_enable(True)
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
     L.profile_enable(False)
     return elapsed
 

@@ -460,6 +460,13 @@ int64_t sjhip_pwconv_planes_elems(int64_t rows, int64_t cols);
 int sjhip_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, void *stream);
 int sjhip_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,
                       int64_t L, float *c, void *stream);
+/* sjhip_pwconv_gemm that also leaves the batch-norm statistics of c: partial[r][m] = (sum, sum of squares) of row m of c
+ * over a group of 64 columns (s, l), r < sjhip_pwconv_gemm_stats_rows(K, S, L); sjhip_bn_finalize_rows(partial, rows,
+ * S * L, M, ...) turns them into the affine map, which saves the pass of sjhip_bn_stats over c.  The reference's
+ * nn.Conv1d + nn.BatchNorm1d (layer/attention.py:314-319) read the convolution output once more for this. */
+int64_t sjhip_pwconv_gemm_stats_rows(int64_t K, int64_t S, int64_t L);
+int sjhip_pwconv_gemm_stats(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,
+                            int64_t L, float *c, float *partial, void *stream);
 int64_t sjhip_pwconv_grad_weight_workspace_floats(int64_t M, int64_t N, int64_t S);
 int sjhip_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int x_terms, int64_t S, int64_t M, int64_t N,
                              int64_t L, float *dw, float *workspace, void *stream);
@@ -491,6 +498,10 @@ int sjhip_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *parti
 int sjhip_bn_finalize(const float *partial, int64_t S, int64_t C, int64_t L, const float *gamma, const float *beta, float eps,
                       float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
                       float *invstd, void *stream);
+/* the same from partial [rows][C][2] that sum over `count` elements per channel (training mode only: partial != NULL) */
+int sjhip_bn_finalize_rows(const float *partial, int64_t rows, int64_t count, int64_t C, const float *gamma, const float *beta,
+                           float eps, float momentum, float *running_mean, float *running_var, float *scale, float *shift,
+                           float *mean, float *invstd, void *stream);
 int sjhip_bn_lif_forward(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
                          const float *scale, const float *shift, const float *v_init, float *spike_seq, uint8_t *spike_bits,
                          float *v_last, void *stream);

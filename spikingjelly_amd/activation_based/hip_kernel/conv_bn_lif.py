@@ -69,16 +69,25 @@ def split_weight(weight: torch.Tensor, transpose: bool) -> torch.Tensor:
     return planes
 
 
-def pw_gemm(planes: torch.Tensor, a_terms: int, M: int, Kdim: int, b: torch.Tensor, b_terms: int) -> torch.Tensor:
-    """``c[s] = A b[s]`` for ``b [S, K, L]`` -> ``c [S, M, L]``."""
+def pw_gemm(planes: torch.Tensor, a_terms: int, M: int, Kdim: int, b: torch.Tensor, b_terms: int, stats: bool = False):
+    """``c[s] = A b[s]`` for ``b [S, K, L]`` -> ``c [S, M, L]``.  With ``stats`` the result is ``(c, partial)``:
+    ``partial [rows, M, 2]`` holds sums and sums of squares of every row of ``c`` over groups of its columns, the input
+    of ``_bn_map``."""
     S, Kb, Lp = b.shape
     assert Kb == Kdim
     b = L.aligned16(b)
     c = torch.empty((S, M, Lp), dtype=torch.float32, device=b.device)
+    lib = L.load()
     with torch.cuda.device(b.device):
-        rc = L.load().sjhip_pwconv_gemm(planes.data_ptr(), a_terms, M, Kdim, b.data_ptr(), b_terms, S, Lp, c.data_ptr(), _stream(b))
+        if stats:
+            rows = lib.sjhip_pwconv_gemm_stats_rows(Kdim, S, Lp)
+            partial = torch.empty((rows, M, 2), dtype=torch.float32, device=b.device)
+            rc = lib.sjhip_pwconv_gemm_stats(planes.data_ptr(), a_terms, M, Kdim, b.data_ptr(), b_terms, S, Lp, c.data_ptr(),
+                                             partial.data_ptr(), _stream(b))
+        else:
+            rc = lib.sjhip_pwconv_gemm(planes.data_ptr(), a_terms, M, Kdim, b.data_ptr(), b_terms, S, Lp, c.data_ptr(), _stream(b))
     L.check(rc, "pwconv_gemm")
-    return c
+    return (c, partial) if stats else c
 
 
 def pw_grad_weight(dy: torch.Tensor, dy_terms: int, x: torch.Tensor, x_terms: int) -> torch.Tensor:
@@ -96,13 +105,21 @@ def pw_grad_weight(dy: torch.Tensor, dy_terms: int, x: torch.Tensor, x_terms: in
     return dw
 
 
-def _bn_map(y: torch.Tensor, gamma, beta, running_mean, running_var, batch_stats: bool, momentum: float, eps: float):
+def _bn_map(y: torch.Tensor, gamma, beta, running_mean, running_var, batch_stats: bool, momentum: float, eps: float,
+            partial: Optional[torch.Tensor] = None):
     """Per-channel ``(scale, shift, mean, invstd)`` of ``z = y * scale + shift`` for ``y [S, C, L]``; with
-    ``batch_stats`` from the statistics of ``y`` (and the running statistics, when given, are updated in place)."""
+    ``batch_stats`` from the statistics of ``y`` (and the running statistics, when given, are updated in place).
+    ``partial``: the sums the convolution left behind (``pw_gemm(..., stats=True)``), which save the pass over ``y``."""
     S, C, Lp = y.shape
     lib = L.load()
     out = torch.empty((4, C), dtype=torch.float32, device=y.device)
     with torch.cuda.device(y.device):
+        if batch_stats and partial is not None:
+            rc = lib.sjhip_bn_finalize_rows(partial.data_ptr(), partial.shape[0], S * Lp, C, L.ptr(gamma), L.ptr(beta), eps,
+                                            momentum, L.ptr(running_mean), L.ptr(running_var), out[0].data_ptr(),
+                                            out[1].data_ptr(), out[2].data_ptr(), out[3].data_ptr(), _stream(y))
+            L.check(rc, "bn_finalize_rows")
+            return out
         partial = None
         if batch_stats:
             partial = torch.empty((S * C, 2), dtype=torch.float32, device=y.device)
@@ -171,13 +188,16 @@ def _bn_lif_backward(y: torch.Tensor, bn_map: torch.Tensor, gamma, v_init: torch
 # ------------------------------------------------------------------------------------------------
 # bn: (running_mean | None, running_var | None, batch_stats, momentum, eps)
 # lif spec: (tau, v_threshold, v_reset, flags, sg_id, sg_alpha)
-def _conv_forward(x_seq, weight, x_exact):
+def _conv_forward(x_seq, weight, x_exact, stats: bool = False):
+    """``y [T, B, Cout, L]``, and with ``stats`` the partial batch-norm sums of ``y`` as well."""
     T, B, Cin, Lp = x_seq.shape
     Cout = weight.shape[0]
     terms = _terms()
     planes = split_weight(weight, False)
-    y = pw_gemm(planes, terms, Cout, Cin, x_seq.reshape(T * B, Cin, Lp), 1 if x_exact else terms)
-    return y.view(T, B, Cout, Lp)
+    out = pw_gemm(planes, terms, Cout, Cin, x_seq.reshape(T * B, Cin, Lp), 1 if x_exact else terms, stats)
+    if stats:
+        return out[0].view(T, B, Cout, Lp), out[1]
+    return out.view(T, B, Cout, Lp)
 
 
 def _conv_backward(dy, x_seq, weight, x_exact, need_dx, need_dw):
@@ -223,8 +243,8 @@ class _ConvBnLif(torch.autograd.Function):
     def forward(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact):
         running_mean, running_var, batch_stats, momentum, eps = bn
         x_seq = L.aligned16(x_seq)
-        y = _conv_forward(x_seq, weight, x_exact)
-        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps)
+        y, partial = _conv_forward(x_seq, weight, x_exact, True) if batch_stats else (_conv_forward(x_seq, weight, x_exact), None)
+        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial)
         spikes, v_last = _bn_lif_forward(y, bn_map, v_init, spec, False)
         return spikes, v_last, y, bn_map
 
@@ -258,8 +278,8 @@ class _ConvBnLifSsa(torch.autograd.Function):
         heads, cph, scale = ssa
         x_seq = L.aligned16(x_seq)
         T, B, _, Lp = x_seq.shape
-        y = _conv_forward(x_seq, weight, x_exact)
-        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps)
+        y, partial = _conv_forward(x_seq, weight, x_exact, True) if batch_stats else (_conv_forward(x_seq, weight, x_exact), None)
+        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial)
         bits, v_last = _bn_lif_forward(y, bn_map, v_init, spec, True)
         out = A._ssa_packed(bits, None, torch.float32, T * B, heads, cph, Lp, scale)
         return out, v_last, y, bn_map, bits

@@ -67,10 +67,13 @@ EXPORTED_SYMBOLS = (
     "sjhip_pwconv_planes_elems",
     "sjhip_pwconv_split_weight",
     "sjhip_pwconv_gemm",
+    "sjhip_pwconv_gemm_stats_rows",
+    "sjhip_pwconv_gemm_stats",
     "sjhip_pwconv_grad_weight_workspace_floats",
     "sjhip_pwconv_grad_weight",
     "sjhip_bn_stats",
     "sjhip_bn_finalize",
+    "sjhip_bn_finalize_rows",
     "sjhip_bn_lif_forward",
     "sjhip_bn_lif_backward",
     "sjhip_bn_backward_finalize",
@@ -229,6 +232,11 @@ def load() -> ctypes.CDLL:
         lib.sjhip_pwconv_gemm.restype = c_int
         lib.sjhip_pwconv_gemm.argtypes = [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_void_p,
                                           c_void_p]
+        lib.sjhip_pwconv_gemm_stats_rows.restype = c_int64
+        lib.sjhip_pwconv_gemm_stats_rows.argtypes = [c_int64, c_int64, c_int64]
+        lib.sjhip_pwconv_gemm_stats.restype = c_int
+        lib.sjhip_pwconv_gemm_stats.argtypes = [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_void_p,
+                                                c_void_p, c_void_p]
         lib.sjhip_pwconv_grad_weight_workspace_floats.restype = c_int64
         lib.sjhip_pwconv_grad_weight_workspace_floats.argtypes = [c_int64, c_int64, c_int64]
         lib.sjhip_pwconv_grad_weight.restype = c_int
@@ -239,6 +247,9 @@ def load() -> ctypes.CDLL:
         lib.sjhip_bn_finalize.restype = c_int
         lib.sjhip_bn_finalize.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float, c_float] + \
                                          [c_void_p] * 7
+        lib.sjhip_bn_finalize_rows.restype = c_int
+        lib.sjhip_bn_finalize_rows.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float, c_float] + \
+                                              [c_void_p] * 7
         lib.sjhip_bn_lif_forward.restype = c_int
         lib.sjhip_bn_lif_forward.argtypes = [c_int, POINTER(NeuronParams), c_int64, c_int64, c_int64, c_int64] + [c_void_p] * 8
         lib.sjhip_bn_lif_backward.restype = c_int

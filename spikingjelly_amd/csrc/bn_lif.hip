@@ -400,12 +400,13 @@ int launch_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *part
   return check_launch("bn_stats");
 }
 
-int launch_bn_finalize(const float *partial, int64_t S, int64_t C, int64_t L, const float *gamma, const float *beta, float eps,
+// partial [rows][C][2]: sums over `count` elements per channel in all
+int launch_bn_finalize(const float *partial, int64_t rows, int64_t count, int64_t C, const float *gamma, const float *beta, float eps,
                        float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
                        float *invstd, hipStream_t stream) {
   if (C < 1 || C > (1 << 24)) return fail(SJHIP_ERR_INVALID, "bn_finalize: C=%lld", (long long)C);
   if (!partial && (!running_mean || !running_var)) return fail(SJHIP_ERR_INVALID, "bn_finalize: evaluation mode needs the running statistics");
-  hipLaunchKernelGGL(bn_finalize_kernel, dim3((unsigned)((C + 3) / 4)), dim3(256), 0, stream, partial, S, (int)C, S * L, gamma,
+  hipLaunchKernelGGL(bn_finalize_kernel, dim3((unsigned)((C + 3) / 4)), dim3(256), 0, stream, partial, rows, (int)C, count, gamma,
                      beta, eps, momentum, running_mean, running_var, scale, shift, mean, invstd);
   return check_launch("bn_finalize");
 }

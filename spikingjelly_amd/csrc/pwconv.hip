@@ -122,7 +122,11 @@ struct PwGemmArgs {
   int64_t ncols;             // S * L
   int M, K, K_pad, L;
   int m_blocks;
+  float *stats;              // nullptr, or [2 x column blocks][M][2]: per row of c the sum and the sum of squares over
+                             // each half (64 columns) of every column block
 };
+constexpr int kStatPitch = 33;                             // floats per row of the transposing buffer: no bank conflicts
+constexpr unsigned kStatLds = 4 * 64 * kStatPitch * 4;     // one buffer of 64 rows x 32 column pairs per wavefront
 
 // Term pairs whose product is kept: combined order at most max(TA, TB) - 1.
 template <int TA, int TB> struct Pairs {
@@ -306,6 +310,32 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
         const int row = rbase + 8 * (r >> 2) + (r & 3);
         if (row < M) cp[(int64_t)row * L] = acc[mt][nt][r];
       }
+    }
+  }
+
+  // Batch-norm statistics of the tile, so that no kernel has to read c again for them: per row the sum and the sum of
+  // squares over the wavefront's 64 columns (columns beyond the matrix hold exact zeros).  A lane holds 32 rows of one
+  // column pair; the values go through LDS, transposed, and lane i adds the 32 pairs of row i in a fixed order.
+  if (a.stats) {
+    __syncthreads();  // the operand tiles are no longer read
+    float *buf = reinterpret_cast<float *>(lds) + wave * (64 * kStatPitch);
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float v0 = acc[mt][0][r], v1 = acc[mt][1][r];
+          const int row_local = mt * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          buf[row_local * kStatPitch + (lane & 31)] = pass == 0 ? v0 + v1 : v0 * v0 + v1 * v1;
+        }
+      __syncthreads();
+      float sum = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 32; ++j) sum += buf[lane * kStatPitch + j];
+      const int row = m0 + wm * 64 + lane;
+      if (row < M) a.stats[((2 * nb + wn) * (int64_t)M + row) * 2 + pass] = sum;
+      __syncthreads();
     }
   }
 }
@@ -496,7 +526,8 @@ __global__ void __launch_bounds__(256) dw_reduce_kernel(const float *partials, i
 int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
 template <int TA, int TB> int launch_gemm_terms(const PwGemmArgs &a, int64_t blocks, hipStream_t stream) {
-  const unsigned lds = (TA + TB) * kRowPlane;
+  unsigned lds = (TA + TB) * kRowPlane;
+  if (a.stats && lds < kStatLds) lds = kStatLds;
   hipLaunchKernelGGL((pw_gemm_kernel<TA, TB>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
   return check_launch("pwconv_gemm");
 }
@@ -537,14 +568,30 @@ int launch_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int t
   return check_launch("pwconv_split_weight");
 }
 
+namespace {
+const int64_t kPwOffsetLimit = int64_t(1) << 30;  // per-lane offsets into A and B are 32-bit byte offsets
+int64_t gemm_samples_per_launch(int64_t K, int64_t L) { return (kPwOffsetLimit - 1) / (K * L); }
+}  // namespace
+
+int64_t pwconv_gemm_stats_rows(int64_t K, int64_t S, int64_t L) {
+  if (K < 1 || L < 1 || K * L >= kPwOffsetLimit) return 0;
+  const int64_t s_step = gemm_samples_per_launch(K, L);
+  int64_t rows = 0;
+  for (int64_t s0 = 0; s0 < S; s0 += s_step) {
+    const int64_t s_count = S - s0 < s_step ? S - s0 : s_step;
+    rows += 2 * ((s_count * L + kTile - 1) / kTile);
+  }
+  return rows;
+}
+
 int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,
-                       int64_t L, float *c, hipStream_t stream) {
+                       int64_t L, float *c, float *stats, hipStream_t stream) {
   if (L % 2 != 0 || !aligned16(a_planes) || (reinterpret_cast<uintptr_t>(b) & 7u))
     return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: L=%lld must be even, the weight planes 16-byte and the activations 8-byte aligned", (long long)L);
-  const int64_t limit = int64_t(1) << 30;  // per-lane offsets into A and B are 32-bit byte offsets
+  const int64_t limit = kPwOffsetLimit;
   if (round_up(M, kTile) * round_up(K, kTileK) >= limit || K * L >= limit)
     return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: M=%lld K=%lld L=%lld", (long long)M, (long long)K, (long long)L);
-  const int64_t s_step = (limit - 1) / (K * L);  // samples per launch
+  const int64_t s_step = gemm_samples_per_launch(K, L);
   ProfileScope prof(KC_PW_GEMM, stream);
   for (int64_t s0 = 0; s0 < S; s0 += s_step) {
     const int64_t s_count = S - s0 < s_step ? S - s0 : s_step;
@@ -554,6 +601,8 @@ int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t
     a.plane_stride = round_up(M, kTile) * a.K_pad;
     a.ncols = s_count * L;
     a.m_blocks = (int)(round_up(M, kTile) / kTile);
+    a.stats = stats;
+    if (stats) stats += 2 * ((a.ncols + kTile - 1) / kTile) * M * 2;
     const int64_t blocks = a.m_blocks * ((a.ncols + kTile - 1) / kTile);
     if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: %lld blocks", (long long)blocks);
     int rc;

@@ -555,7 +555,20 @@ int sjhip_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t 
   if (!a_planes || !b || !c) return fail(SJHIP_ERR_INVALID, "pwconv_gemm: NULL buffer");
   if (M < 1 || K < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_gemm: M=%lld K=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)K, (long long)S, (long long)L);
   if (S > (int64_t(1) << 40) / L) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: S*L overflows");
-  return launch_pwconv_gemm(a_planes, a_terms, M, K, b, b_terms, S, L, c, static_cast<hipStream_t>(stream));
+  return launch_pwconv_gemm(a_planes, a_terms, M, K, b, b_terms, S, L, c, nullptr, static_cast<hipStream_t>(stream));
+}
+
+int64_t sjhip_pwconv_gemm_stats_rows(int64_t K, int64_t S, int64_t L) {
+  if (K < 1 || S < 1 || L < 1 || S > (int64_t(1) << 40) / L) return 0;
+  return pwconv_gemm_stats_rows(K, S, L);
+}
+
+int sjhip_pwconv_gemm_stats(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,
+                            int64_t L, float *c, float *partial, void *stream) {
+  if (!a_planes || !b || !c || !partial) return fail(SJHIP_ERR_INVALID, "pwconv_gemm_stats: NULL buffer");
+  if (M < 1 || K < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_gemm_stats: M=%lld K=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)K, (long long)S, (long long)L);
+  if (S > (int64_t(1) << 40) / L) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm_stats: S*L overflows");
+  return launch_pwconv_gemm(a_planes, a_terms, M, K, b, b_terms, S, L, c, partial, static_cast<hipStream_t>(stream));
 }
 
 int64_t sjhip_pwconv_grad_weight_workspace_floats(int64_t M, int64_t N, int64_t S) {
@@ -580,8 +593,17 @@ int sjhip_bn_finalize(const float *partial, int64_t S, int64_t C, int64_t L, con
                       float *invstd, void *stream) {
   if (!scale || !shift || !mean || !invstd) return fail(SJHIP_ERR_INVALID, "bn_finalize: NULL output");
   if (partial && (S < 1 || L < 1)) return fail(SJHIP_ERR_INVALID, "bn_finalize: S=%lld L=%lld", (long long)S, (long long)L);
-  return launch_bn_finalize(partial, S, C, L, gamma, beta, eps, momentum, running_mean, running_var, scale, shift, mean, invstd,
+  return launch_bn_finalize(partial, S, S * L, C, gamma, beta, eps, momentum, running_mean, running_var, scale, shift, mean, invstd,
                             static_cast<hipStream_t>(stream));
+}
+
+int sjhip_bn_finalize_rows(const float *partial, int64_t rows, int64_t count, int64_t C, const float *gamma, const float *beta,
+                           float eps, float momentum, float *running_mean, float *running_var, float *scale, float *shift,
+                           float *mean, float *invstd, void *stream) {
+  if (!partial || !scale || !shift || !mean || !invstd) return fail(SJHIP_ERR_INVALID, "bn_finalize_rows: NULL buffer");
+  if (rows < 1 || count < 1) return fail(SJHIP_ERR_INVALID, "bn_finalize_rows: rows=%lld count=%lld", (long long)rows, (long long)count);
+  return launch_bn_finalize(partial, rows, count, C, gamma, beta, eps, momentum, running_mean, running_var, scale, shift, mean,
+                            invstd, static_cast<hipStream_t>(stream));
 }
 
 int sjhip_bn_lif_forward(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,

@@ -391,12 +391,13 @@ int launch_stream_probe(int reads, int writes, int nontemporal, int64_t floats_p
 int64_t pwconv_planes_elems(int64_t rows, int64_t cols);
 int launch_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, hipStream_t stream);
 int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,
-                       int64_t L, float *c, hipStream_t stream);
+                       int64_t L, float *c, float *stats, hipStream_t stream);
+int64_t pwconv_gemm_stats_rows(int64_t K, int64_t S, int64_t L);
 int64_t pwconv_dw_workspace_floats(int64_t M, int64_t N, int64_t S);
 int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int x_terms, int64_t S, int64_t M, int64_t N,
                               int64_t L, float *dw, float *workspace, hipStream_t stream);
 int launch_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, hipStream_t stream);
-int launch_bn_finalize(const float *partial, int64_t S, int64_t C, int64_t L, const float *gamma, const float *beta, float eps,
+int launch_bn_finalize(const float *partial, int64_t rows, int64_t count, int64_t C, const float *gamma, const float *beta, float eps,
                        float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
                        float *invstd, hipStream_t stream);
 int launch_bn_lif_forward(int neuron, const sjhip_neuron_params &p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,

@@ -202,3 +202,19 @@ def test_traceable_replay_policy_mirrors_the_library():
             for T in (1, 8, 39, 40, 64, 159, 160, 1000):
                 for N in (1, 4, 8, 12, 37, 64, 100, 4096):
                     assert (N % width == 0 and T <= steps) == L.recompute_preferred(dtype, T, N, flags), (dtype, flags, T, N)
+
+
+def test_convolution_statistics_arguments_without_a_device():
+    lib = L.load()
+    # two partial rows per 128 columns of all samples: 256 * 196 columns -> 392 column blocks
+    assert lib.sjhip_pwconv_gemm_stats_rows(384, 256, 196) == 784
+    assert lib.sjhip_pwconv_gemm_stats_rows(3, 1, 4) == 2
+    assert lib.sjhip_pwconv_gemm_stats_rows(0, 1, 4) == 0
+    rc = lib.sjhip_pwconv_gemm_stats(16, 3, 8, 8, 16, 3, 1, 4, 16, None, None)
+    assert rc == -1 and b"NULL" in lib.sjhip_last_error()
+    rc = lib.sjhip_pwconv_gemm_stats(16, 3, 8, 0, 16, 3, 1, 4, 16, 16, None)
+    assert rc == -1 and b"K=0" in lib.sjhip_last_error()
+    rc = lib.sjhip_bn_finalize_rows(None, 4, 16, 8, None, None, 1e-5, 0.1, None, None, 16, 16, 16, 16, None)
+    assert rc == -1 and b"NULL" in lib.sjhip_last_error()
+    rc = lib.sjhip_bn_finalize_rows(16, 0, 16, 8, None, None, 1e-5, 0.1, None, None, 16, 16, 16, 16, None)
+    assert rc == -1 and b"rows=0" in lib.sjhip_last_error()

@@ -68,6 +68,39 @@ def test_gemm_is_exact_on_spikes_times_dyadic_weights(C, S, M, Kd, Lp):
         assert torch.equal(got, want), (wt, xt)
 
 
+@pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (1, 7, 3, 4), (4, 130, 257, 36), (16, 1152, 384, 196), (5, 384, 384, 196)])
+@pytest.mark.parametrize("terms", [(3, 3), (3, 1), (1, 1)])
+def test_gemm_leaves_the_batch_norm_sums_of_its_output(C, S, M, Kd, Lp, terms):
+    """``pw_gemm(..., stats=True)``: the output is the one of the plain call bit for bit, and the partial sums add up to
+    the per-channel sum and sum of squares of that output (float64 sums of the fp32 output; fp32 partial sums over 64
+    columns each: 1e-6 of the sums of absolute values), so that the affine map made from them is the one ``bn_stats``
+    gives."""
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+
+    wt, xt = terms
+    w = seeded_randn((M, Kd), 31, 0.0, 1.0)
+    x = (seeded_randn((S, Kd, Lp), 32, 0.0, 1.0) > 0.3).float() if xt == 1 else seeded_randn((S, Kd, Lp), 32, 0.1, 1.0)
+    planes = C.split_weight(w.cuda(), False)
+    plain = C.pw_gemm(planes, wt, M, Kd, x.cuda(), xt)
+    got, partial = C.pw_gemm(planes, wt, M, Kd, x.cuda(), xt, stats=True)
+    assert torch.equal(got, plain)
+    assert partial.shape == (L.load().sjhip_pwconv_gemm_stats_rows(Kd, S, Lp), M, 2)
+    y = got.double()
+    sums = partial.double().sum(0).cpu()
+    want_s, want_q = y.sum((0, 2)).cpu(), (y * y).sum((0, 2)).cpu()
+    abs_s = y.abs().sum((0, 2)).cpu().clamp_min(1e-30)
+    assert float(((sums[:, 0] - want_s).abs() / abs_s).max()) < 1e-6
+    assert float(((sums[:, 1] - want_q).abs() / want_q.clamp_min(1e-30)).max()) < 1e-6
+    # the affine map from these sums against the one from the pass over y
+    gamma, beta = seeded_randn((M,), 33, 1.0, 0.2).cuda(), seeded_randn((M,), 34, 0.0, 0.2).cuda()
+    a = C._bn_map(got, gamma, beta, None, None, True, 0.1, 1e-5)
+    b = C._bn_map(got, gamma, beta, None, None, True, 0.1, 1e-5, partial)
+    torch.testing.assert_close(b[2], a[2], rtol=1e-6, atol=1e-6)      # mean
+    torch.testing.assert_close(b[3], a[3], rtol=2e-6, atol=0.0)       # 1 / sqrt(var + eps)
+    torch.testing.assert_close(b[0], a[0], rtol=2e-6, atol=0.0)
+    torch.testing.assert_close(b[1], a[1], rtol=1e-5, atol=2e-6)
+
+
 @pytest.mark.parametrize("S,M,N,Lp", [(3, 100, 50, 12), (9, 130, 257, 36), (16, 384, 384, 196), (2, 1152, 384, 196), (64, 64, 48, 8)])
 @pytest.mark.parametrize("spikes", [False, True])
 def test_grad_weight_gemm(C, S, M, N, Lp, spikes):
