@@ -321,7 +321,7 @@ template <int TMAX>
 __global__ void __launch_bounds__(256) bn_lif_backward_rows_kernel(const BnLifBwdArgs a, int quads, int rows_per_block,
                                                                    float inv_quads) {
   __shared__ float part[4][kBnRowsMax][2];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x;
   int r_local = (int)(((float)tid + 0.5f) * inv_quads);  // tid / quads (exact: see div_tokens of ssa.hip)
   const int q = tid - r_local * quads;
   const int64_t row = (int64_t)blockIdx.x * rows_per_block + r_local;
@@ -330,7 +330,7 @@ __global__ void __launch_bounds__(256) bn_lif_backward_rows_kernel(const BnLifBw
   float acc_g = 0.0f, acc_gy = 0.0f;
   if (valid) bn_lif_backward_quad<TMAX>(a, row, q, acc_g, acc_gy);
   block_row_sums(part, r_local, valid, rows_per_block, acc_g, acc_gy, a.partial, (int64_t)blockIdx.x * rows_per_block, a.rows);
-  const int tid = threadIdx.x;
+}
 
 // dgamma, dbeta and the coefficients of dy = p g + q y + r; count = T * B * L elements per channel
 __global__ void __launch_bounds__(256) bn_backward_finalize_kernel(const float *partial, int64_t B, int C, int64_t count,
