@@ -434,6 +434,29 @@ int sjhip_ssa_backward_packed(int dtype, int64_t samples, int heads, int channel
                               const uint8_t *qkv_bits, const void *grad_out, void *grad_qkv, void *stream);
 
 /*
+ * The contraction fused with the multi-step IF / LIF neuron that takes its output as input: `attn_lif` of the
+ * reference's SpikingSelfAttention (layer/attention.py:321-322, 383-384), which there is a separate module call on the
+ * materialised `scale (V K^T) Q`.  fp32, bit-packed q / k / v as for sjhip_ssa_forward_packed with samples = T * B
+ * ordered [T][B]; tokens a multiple of 4.  A block owns one (batch element, head) and walks the T steps with the
+ * membrane potential in registers; the contraction's output is never written.
+ *   forward:  spike_seq [T][B][heads][cph][tokens]; h_seq (same shape: the potential before firing, kept for the
+ *             backward) or NULL; v_init [B][heads][cph][tokens] or one element with SJHIP_FLAG_V_INIT_BROADCAST;
+ *             v_last or NULL.  Same arithmetic as sjhip_ssa_forward_packed followed by sjhip_neuron_forward, bit for bit.
+ *   backward: from h_seq, grad_spike_seq (or NULL) and grad_v_last (or NULL): grad_qkv [T * B][3][heads][cph][tokens]
+ *             (the gradient with respect to the q / k / v spikes) and grad_v_init (or NULL); the recurrence of
+ *             sjhip_neuron_backward and the products of sjhip_ssa_backward_packed.
+ * neuron: SJHIP_NEURON_IF or SJHIP_NEURON_LIF (SJHIP_ERR_UNSUPPORTED otherwise, and for shapes the contraction does
+ * not support).
+ */
+int sjhip_ssa_lif_forward_packed(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int heads, int channels_per_head,
+                                 int64_t tokens, float scale, const uint8_t *qkv_bits, const float *v_init, float *spike_seq,
+                                 float *h_seq, float *v_last, void *stream);
+int sjhip_ssa_lif_backward_packed(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int heads,
+                                  int channels_per_head, int64_t tokens, float scale, const uint8_t *qkv_bits,
+                                  const float *h_seq, const float *grad_spike_seq, const float *grad_v_last, float *grad_qkv,
+                                  float *grad_v_init, void *stream);
+
+/*
  * Kernel-size-1 convolution over [S, C, L] activations (S samples = time steps x batch, L positions, L contiguous) as
  * GEMMs on the bf16 matrix cores.  Stands in for torch's nn.Conv1d(kernel_size=1, bias=False) inside the reference's
  * SpikingSelfAttention (spikingjelly/activation_based/layer/attention.py:310-329, applied at :370 and :382 through

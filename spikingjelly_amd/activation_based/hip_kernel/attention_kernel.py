@@ -9,6 +9,8 @@
 
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import library as L
@@ -111,6 +113,42 @@ def _ssa_packed(bits: torch.Tensor, grad_out, dtype: torch.dtype, samples: int, 
                                                grad_out.data_ptr(), result.data_ptr(), L.current_stream_ptr(bits.device))
     L.check(rc, "ssa_forward_packed" if grad_out is None else "ssa_backward_packed")
     return result
+
+
+def ssa_lif_supported(channels_per_head: int, tokens: int) -> bool:
+    """The contraction fused with the LIF behind it: fp32, bit-packed q / k / v, tokens a multiple of 4."""
+    return ssa_packed_supported(torch.float32, channels_per_head, tokens) and tokens % 4 == 0
+
+
+def _ssa_lif_forward(bits: torch.Tensor, v_init: torch.Tensor, params, T: int, B: int, heads: int, cph: int, tokens: int,
+                     scale: float, save_h: bool):
+    """``(spikes [T, B, heads, cph, tokens], h_seq or None, v_last [B, heads, cph, tokens])`` of the LIF that takes
+    ``scale (V K^T) Q`` of the bit-packed spikes as its input; the contraction's output is never written."""
+    spikes = torch.empty((T, B, heads, cph, tokens), dtype=torch.float32, device=bits.device)
+    h_seq = torch.empty_like(spikes) if save_h else None
+    v_last = torch.empty((B, heads, cph, tokens), dtype=torch.float32, device=bits.device)
+    with torch.cuda.device(bits.device):
+        rc = L.load().sjhip_ssa_lif_forward_packed(L.NEURON_LIF, ctypes.byref(params), T, B, heads, cph, tokens, scale,
+                                                   bits.data_ptr(), v_init.data_ptr(), spikes.data_ptr(), L.ptr(h_seq),
+                                                   v_last.data_ptr(), L.current_stream_ptr(bits.device))
+    L.check(rc, "ssa_lif_forward_packed")
+    return spikes, h_seq, v_last
+
+
+def _ssa_lif_backward(bits: torch.Tensor, h_seq: torch.Tensor, grad_spikes, grad_v_last, params, T: int, B: int, heads: int,
+                      cph: int, tokens: int, scale: float, need_grad_v_init: bool):
+    """``(grad_qkv [T * B, 3, heads, cph, tokens], grad_v_init or None)``."""
+    grad_qkv = torch.empty((T * B, 3, heads, cph, tokens), dtype=torch.float32, device=bits.device)
+    grad_v_init = torch.empty((B, heads, cph, tokens), dtype=torch.float32, device=bits.device) if need_grad_v_init else None
+    gs = L.aligned16(grad_spikes.to(torch.float32)) if grad_spikes is not None else None
+    gvl = L.aligned16(grad_v_last.to(torch.float32)) if grad_v_last is not None else None
+    with torch.cuda.device(bits.device):
+        rc = L.load().sjhip_ssa_lif_backward_packed(L.NEURON_LIF, ctypes.byref(params), T, B, heads, cph, tokens, scale,
+                                                    bits.data_ptr(), h_seq.data_ptr(), L.ptr(gs), L.ptr(gvl),
+                                                    grad_qkv.data_ptr(), L.ptr(grad_v_init),
+                                                    L.current_stream_ptr(bits.device))
+    L.check(rc, "ssa_lif_backward_packed")
+    return grad_qkv, grad_v_init
 
 
 class _LifSsa(torch.autograd.Function):

@@ -30,7 +30,8 @@ from ... import configure
 from . import library as L
 from . import neuron_kernel as K
 
-__all__ = ["supported", "bn_lif", "conv_bn_lif", "conv_bn_lif_ssa", "split_weight", "pw_gemm", "pw_grad_weight"]
+__all__ = ["supported", "bn_lif", "conv_bn_lif", "conv_bn_lif_ssa", "conv_bn_lif_ssa_lif", "split_weight", "pw_gemm",
+           "pw_grad_weight"]
 
 MAX_REPLAY_STEPS = 16  # the backward replays the neuron with h of every step in registers
 
@@ -309,6 +310,58 @@ class _ConvBnLifSsa(torch.autograd.Function):
         return (dx, dw, dgamma if need[2] else None, dbeta if need[3] else None, gvi, None, None, None, None)
 
 
+class _ConvBnLifSsaLif(torch.autograd.Function):
+    """``_ConvBnLifSsa`` followed by the attention's own LIF, whose input ``scale (V K^T) Q`` never leaves the kernel
+    that computes it.  Saves the input, the convolution output, the bits and, when a gradient is wanted, the attention
+    neuron's ``h_seq``."""
+
+    @staticmethod
+    def forward(x_seq, weight, gamma, beta, v_init, attn_v_init, bn, spec, x_exact, ssa, attn_spec, save_h):
+        from . import attention_kernel as A
+
+        running_mean, running_var, batch_stats, momentum, eps = bn
+        heads, cph, scale = ssa
+        x_seq = L.aligned16(x_seq)
+        T, B, _, Lp = x_seq.shape
+        y, partial = _conv_forward(x_seq, weight, x_exact, True) if batch_stats else (_conv_forward(x_seq, weight, x_exact), None)
+        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial)
+        bits, v_last = _bn_lif_forward(y, bn_map, v_init, spec, True)
+        v_keep, broadcast = K._state_arg(attn_v_init, True)
+        spikes, h_seq, attn_v_last = A._ssa_lif_forward(bits, v_keep, _lif_params(attn_spec, broadcast), T, B, heads, cph,
+                                                        Lp, scale, save_h)
+        if h_seq is None:
+            h_seq = spikes.new_empty((0,))
+        return spikes, v_last, attn_v_last, y, bn_map, bits, h_seq
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        x_seq, weight, gamma, beta, v_init, attn_v_init, bn, spec, x_exact, ssa, attn_spec, save_h = inputs
+        ctx.spec, ctx.batch_stats, ctx.x_exact, ctx.ssa, ctx.attn_spec = spec, bn[2], x_exact, ssa, attn_spec
+        ctx.save_for_backward(L.aligned16(x_seq), weight, gamma, v_init, output[3], output[4], output[5], output[6])
+        ctx.mark_non_differentiable(output[3], output[4], output[5], output[6])
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, grad_attn_spikes, grad_v_last, grad_attn_v_last, _y, _map, _bits, _h):
+        from . import attention_kernel as A
+
+        x_seq, weight, gamma, v_init, y, bn_map, bits, h_seq = ctx.saved_tensors
+        if h_seq.numel() == 0:
+            raise RuntimeError("the fused attention block was run without saving h_seq and cannot be differentiated")
+        heads, cph, scale = ctx.ssa
+        T, B, _, Lp = x_seq.shape
+        need = ctx.needs_input_grad
+        grad_spikes = None
+        if grad_attn_spikes is not None or grad_attn_v_last is not None:
+            grad_qkv, _ = A._ssa_lif_backward(bits, h_seq, grad_attn_spikes, grad_attn_v_last, _lif_params(ctx.attn_spec), T, B,
+                                              heads, cph, Lp, scale, False)
+            grad_spikes = grad_qkv.view(y.shape)
+        dy, dgamma, dbeta, gvi = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
+                                                  grad_v_last, bool(need[4]))
+        dx, dw = _conv_backward(dy, x_seq, weight, ctx.x_exact, bool(need[0]), bool(need[1]))
+        return (dx, dw, dgamma if need[2] else None, dbeta if need[3] else None, gvi, None, None, None, None, None, None, None)
+
+
 def bn_lif(y_seq: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec):
     """``y_seq [T, B, C, L]`` (a convolution output) -> ``(spikes, v_last)``."""
     spikes, v_last, _ = _BnLif.apply(y_seq, gamma, beta, v_init, bn, spec)
@@ -329,3 +382,12 @@ def conv_bn_lif_ssa(x_seq: torch.Tensor, weight: torch.Tensor, gamma, beta, v_in
     out, v_last, _, _, _ = _ConvBnLifSsa.apply(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact,
                                                (heads, channels_per_head, scale))
     return out, v_last
+
+
+def conv_bn_lif_ssa_lif(x_seq: torch.Tensor, weight: torch.Tensor, gamma, beta, v_init: torch.Tensor, attn_v_init: torch.Tensor,
+                        bn, spec, x_exact: bool, heads: int, channels_per_head: int, scale: float, attn_spec, save_h: bool):
+    """``conv_bn_lif_ssa`` followed by the LIF of ``attn_spec`` on the contraction's output; returns
+    ``(spikes [T, B, heads, channels_per_head, L], v_last of the first neuron, v_last of the attention neuron)``."""
+    out = _ConvBnLifSsaLif.apply(x_seq, weight, gamma, beta, v_init, attn_v_init, bn, spec, x_exact,
+                                 (heads, channels_per_head, scale), attn_spec, save_h)
+    return out[0], out[1], out[2]

@@ -58,6 +58,8 @@ EXPORTED_SYMBOLS = (
     "sjhip_ssa_backward",
     "sjhip_ssa_forward_packed",
     "sjhip_ssa_backward_packed",
+    "sjhip_ssa_lif_forward_packed",
+    "sjhip_ssa_lif_backward_packed",
     "sjhip_stbif_forward",
     "sjhip_aaif_forward",
     "sjhip_izhikevich_forward",
@@ -225,6 +227,12 @@ def load() -> ctypes.CDLL:
                                                          + [c_void_p] * 12)
         lib.sjhip_stream_probe.restype = c_int
         lib.sjhip_stream_probe.argtypes = [c_int, c_int, c_int, c_int64, POINTER(c_void_p), POINTER(c_void_p), c_void_p]
+        lib.sjhip_ssa_lif_forward_packed.restype = c_int
+        lib.sjhip_ssa_lif_forward_packed.argtypes = [c_int, POINTER(NeuronParams), c_int64, c_int64, c_int, c_int, c_int64, c_float] + \
+                                                    [c_void_p] * 6
+        lib.sjhip_ssa_lif_backward_packed.restype = c_int
+        lib.sjhip_ssa_lif_backward_packed.argtypes = [c_int, POINTER(NeuronParams), c_int64, c_int64, c_int, c_int, c_int64, c_float] + \
+                                                     [c_void_p] * 7
         lib.sjhip_pwconv_planes_elems.restype = c_int64
         lib.sjhip_pwconv_planes_elems.argtypes = [c_int64, c_int64]
         lib.sjhip_pwconv_split_weight.restype = c_int

@@ -13,6 +13,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
+from ... import configure
 from .. import base, neuron
 from . import fused
 from .container import SeqToANNContainer
@@ -106,11 +107,17 @@ class SpikingSelfAttention(nn.Module, base.MultiStepModule):
         T, N, C, L = x_seq.shape
         hip = self.backend == "hip"
         out = None
+        attn_spikes = None
         if hip and len(self.qkv_conv_bn) == 2:
-            # convolution, batch norm, LIF (bit-packed spikes) and the contraction in one autograd node
-            out = fused.conv_bn_lif(x_seq, self.qkv_conv_bn[0], self.qkv_conv_bn[1], self.qkv_lif,
-                                    ssa=(self.num_heads, self.scale))
-        if out is None:
+            # convolution, batch norm, LIF (bit-packed spikes), the contraction and the attention's LIF in one autograd
+            # node; without the last of them when it cannot run inside the contraction
+            if configure.hip_fuse_ssa_lif:
+                attn_spikes = fused.conv_bn_lif(x_seq, self.qkv_conv_bn[0], self.qkv_conv_bn[1], self.qkv_lif,
+                                                ssa=(self.num_heads, self.scale), attn=self.attn_lif)
+            if attn_spikes is None:
+                out = fused.conv_bn_lif(x_seq, self.qkv_conv_bn[0], self.qkv_conv_bn[1], self.qkv_lif,
+                                        ssa=(self.num_heads, self.scale))
+        if out is None and attn_spikes is None:
             pre = self.qkv_conv_bn(x_seq)  # [T, N, 3*C, L]
             local_dim = pre.shape[2] // 3
             if local_dim % self.num_heads != 0:
@@ -119,8 +126,10 @@ class SpikingSelfAttention(nn.Module, base.MultiStepModule):
             if out is None:
                 qkv = self.qkv_lif(pre).reshape(T, N, 3, self.num_heads, local_dim // self.num_heads, L)
                 out = self._ssa_kernel_hip(qkv, self.scale) if hip else self._ssa_kernel_torch(qkv, self.scale)
-        local_dim = out.shape[2] * out.shape[3]
-        x_seq = self.attn_lif(out).reshape(T, N, local_dim, L)
+        if attn_spikes is None:
+            attn_spikes = self.attn_lif(out)
+        local_dim = attn_spikes.shape[2] * attn_spikes.shape[3]
+        x_seq = attn_spikes.reshape(T, N, local_dim, L)
         y = None
         if hip and len(self.proj_conv_bn) == 2:
             y = fused.conv_bn_lif(x_seq, self.proj_conv_bn[0], self.proj_conv_bn[1], self.proj_lif, x_exact=True)

@@ -50,14 +50,19 @@ def _lif_spec(node: neuron.LIFNode, x_like: torch.Tensor, need_grad: bool):
     return (float(node.tau), node.v_threshold, 0.0 if soft else float(node.v_reset), flags, sg_id, sg_alpha)
 
 
+def _plain_hip_lif(node: nn.Module) -> bool:
+    return (type(node) is neuron.LIFNode and node.backend == "hip" and node.step_mode == "m" and not node.store_v_seq)
+
+
 def conv_bn_lif(x_seq: torch.Tensor, conv: Optional[nn.Module], bn: nn.Module, node: nn.Module, x_exact: bool = False,
-                ssa: Optional[tuple] = None) -> Optional[torch.Tensor]:
+                ssa: Optional[tuple] = None, attn: Optional[nn.Module] = None) -> Optional[torch.Tensor]:
     """``node(bn(conv(x_seq)))`` for ``x_seq [T, B, C, *positions]`` in one fused pass, or ``None``.
 
     ``conv is None``: ``x_seq`` already is the convolution output and only batch norm and the neuron are fused.
     ``ssa = (heads, scale)``: the spikes feed the spiking self-attention contraction bit-packed and the result is
-    ``scale (V K^T) Q`` as ``[T, B, heads, channels_per_head, L]``.  ``x_exact``: ``x_seq`` holds values that bf16
-    represents exactly (spikes)."""
+    ``scale (V K^T) Q`` as ``[T, B, heads, channels_per_head, L]``.  With ``attn`` (the neuron that takes that result as
+    its input) the result is ``attn``'s spikes instead, in the same shape, and ``None`` when ``attn`` cannot run inside
+    the contraction.  ``x_exact``: ``x_seq`` holds values that bf16 represents exactly (spikes)."""
     from ..hip_kernel import conv_bn_lif as C
 
     if (not configure.hip_fuse_conv_bn_lif or torch.compiler.is_compiling() or type(node) is not neuron.LIFNode or node.backend != "hip" or node.step_mode != "m"
@@ -81,12 +86,24 @@ def conv_bn_lif(x_seq: torch.Tensor, conv: Optional[nn.Module], bn: nn.Module, n
         cph = channels // 3 // heads
         if channels != 3 * heads * cph or not A.ssa_packed_supported(x4.dtype, cph, Lp) or (B * channels * Lp) % 8 != 0:
             return None
+        if attn is not None and (not configure.hip_fuse_ssa_lif or not _plain_hip_lif(attn)
+                                 or not A.ssa_lif_supported(cph, Lp)):
+            return None
+    elif attn is not None:
+        return None
     node._check_hip_surrogate()
     state_like = torch.empty((1,), dtype=x4.dtype, device=x4.device).expand(T, B, channels, *x_seq.shape[3:])
     (v,) = node.materialize_states((state_like,), (node.v,), "m")
     if need_grad and v.requires_grad:
         return None
-    bn_args = _bn_arguments(bn)
+    attn_v = None
+    if attn is not None:
+        attn._check_hip_surrogate()
+        attn_like = torch.empty((1,), dtype=x4.dtype, device=x4.device).expand(T, B, heads, cph, Lp)
+        (attn_v,) = attn.materialize_states((attn_like,), (attn.v,), "m")
+        if need_grad and attn_v.requires_grad:
+            return None
+    bn_args = _bn_arguments(bn)  # (counts the batch: nothing below may give up)
     if bn_args is None:
         return None
     gamma, beta, bn_cfg = bn_args
@@ -98,10 +115,17 @@ def conv_bn_lif(x_seq: torch.Tensor, conv: Optional[nn.Module], bn: nn.Module, n
             spikes, v_last = C.bn_lif(x4, gamma, beta, v3, bn_cfg, spec)
         elif ssa is None:
             spikes, v_last = C.conv_bn_lif(x4, conv.weight.view(channels, -1), gamma, beta, v3, bn_cfg, spec, x_exact)
-        else:
+        elif attn is None:
             out, v_last = C.conv_bn_lif_ssa(x4, conv.weight.view(channels, -1), gamma, beta, v3, bn_cfg, spec, x_exact,
                                             heads, cph, scale)
             node.v = v_last.reshape(out_shape[1:])
             return out.view(T, B, heads, cph, Lp)
+        else:
+            spikes, v_last, attn_v_last = C.conv_bn_lif_ssa_lif(
+                x4, conv.weight.view(channels, -1), gamma, beta, v3, attn_v, bn_cfg, spec, x_exact, heads, cph, scale,
+                _lif_spec(attn, x4, need_grad), need_grad)
+            node.v = v_last.reshape(out_shape[1:])
+            attn.v = attn_v_last
+            return spikes
     node.v = v_last.reshape(out_shape[1:])
     return spikes.view(out_shape)

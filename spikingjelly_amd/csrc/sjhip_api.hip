@@ -534,6 +534,27 @@ int sjhip_ssa_backward(int dtype, int64_t samples, int heads, int channels_per_h
                     static_cast<hipStream_t>(stream));
 }
 
+int sjhip_ssa_lif_forward_packed(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int heads, int channels_per_head,
+                                 int64_t tokens, float scale, const uint8_t *qkv_bits, const float *v_init, float *spike_seq,
+                                 float *h_seq, float *v_last, void *stream) {
+  if (!p) return fail(SJHIP_ERR_INVALID, "ssa_lif_forward: params is NULL");
+  if (!qkv_bits || !v_init || !spike_seq) return fail(SJHIP_ERR_INVALID, "ssa_lif_forward: NULL tensor");
+  return launch_ssa_lif(false, neuron, *p, T, B, heads, channels_per_head, tokens, scale, qkv_bits, v_init, spike_seq, h_seq,
+                        v_last, nullptr, nullptr, nullptr, nullptr, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_ssa_lif_backward_packed(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int heads,
+                                  int channels_per_head, int64_t tokens, float scale, const uint8_t *qkv_bits,
+                                  const float *h_seq, const float *grad_spike_seq, const float *grad_v_last, float *grad_qkv,
+                                  float *grad_v_init, void *stream) {
+  if (!p) return fail(SJHIP_ERR_INVALID, "ssa_lif_backward: params is NULL");
+  if (!qkv_bits || !h_seq || !grad_qkv) return fail(SJHIP_ERR_INVALID, "ssa_lif_backward: NULL tensor");
+  if (p->sg_id < SJHIP_SG_SIGMOID || p->sg_id > SJHIP_SG_ERF) return fail(SJHIP_ERR_UNSUPPORTED, "ssa_lif_backward: surrogate id %d", p->sg_id);
+  return launch_ssa_lif(true, neuron, *p, T, B, heads, channels_per_head, tokens, scale, qkv_bits, nullptr,
+                        nullptr, const_cast<float *>(h_seq), nullptr, grad_spike_seq, grad_v_last, grad_qkv, grad_v_init,
+                        static_cast<hipStream_t>(stream));
+}
+
 int sjhip_stream_probe(int reads, int writes, int nontemporal, int64_t floats_per_stream, const float *const *in,
                        float *const *out, void *stream) {
   return launch_stream_probe(reads, writes, nontemporal, floats_per_stream, in, out, static_cast<hipStream_t>(stream));

@@ -382,6 +382,10 @@ int launch_backward_recompute(int neuron, int dtype, const sjhip_neuron_params &
                               hipStream_t stream);
 int64_t plif_blocks(int dtype, int64_t N);
 bool ssa_supported(int dtype, int cph, int64_t L);
+int launch_ssa_lif(bool backward, int neuron, const sjhip_neuron_params &p, int64_t T, int64_t B, int heads, int cph, int64_t L,
+                   float scale, const uint8_t *qkv_bits, const float *v_init, float *spikes, float *h_seq, float *v_last,
+                   const float *grad_spikes, const float *grad_v_last, float *grad_qkv, float *grad_v_init,
+                   hipStream_t stream);
 int launch_ssa(bool backward, int dtype, int64_t samples, int heads, int cph, int64_t L, float scale, const void *qkv,
                const uint8_t *qkv_bits, const void *grad_out, void *out, void *grad_qkv, hipStream_t stream);
 int launch_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, hipStream_t stream);

@@ -30,6 +30,8 @@
 // with column lane % 32; accumulator register r sits at row 8 (r / 4) + 4 (lane / 32) + r % 4, column
 // lane % 32.  16x16x4: A row lane % 16, k = lane / 16; accumulator register r at row 4 (lane / 16) + r,
 // column lane % 16.  Which k a lane's operand element stands for is free as long as A and B agree.
+#include "neuron_bwd.h"
+#include "neuron_fwd.h"
 #include "sjhip_common.h"
 
 #include <algorithm>
@@ -46,6 +48,12 @@
 // 149 with three (60 registers spilled).  The kernel therefore keeps one block per head and the plain stagings.
 #ifndef SJHIP_SSA_BWD_RESIDENT
 #define SJHIP_SSA_BWD_RESIDENT 2
+#endif
+// The same for the backward fused with the neuron, which also holds the gradient of the potential (32 registers):
+// sized for 3 it spills 77 registers and takes 155 us on 4 x 64 samples x 12 heads x 32 x 196, sized for 2 it takes all
+// 256 registers, spills nothing and takes 131 us.
+#ifndef SJHIP_SSA_LIF_BWD_RESIDENT
+#define SJHIP_SSA_LIF_BWD_RESIDENT 2
 #endif
 
 namespace sjhip {
@@ -246,6 +254,30 @@ __device__ __forceinline__ void stage_bits(const uint8_t *const (&src)[NS], uint
   zero_fill_bytes<NS>(dst, cph, rows_pad, L, Lb);
 }
 
+// stage_bits in two halves for tiles of at most 4 * blockDim.x bytes (32 channels of 256 tokens with 256 work-items,
+// 64 with 512): the requests, whose results a caller may leave in flight over other work, and the expansion into LDS.
+template <int NS>
+__device__ __forceinline__ void request_bits(const uint8_t *const (&src)[NS], int nbytes, uint32_t (&w)[4][NS]) {
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int b = (int)threadIdx.x + u * (int)blockDim.x;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) w[u][s] = src[s][b < nbytes ? b : nbytes - 1];
+  }
+}
+template <int NS>
+__device__ __forceinline__ void expand_bits(const uint32_t (&w)[4][NS], uint8_t *const (&dst)[NS], int cph, int rows_pad,
+                                            int L, int Lb) {
+  const int nbytes = cph * L / 8;
+  const float inv_L = 1.0f / (float)L;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int b = (int)threadIdx.x + u * (int)blockDim.x;
+    if (b < nbytes) expand_byte<NS>(w[u], b, dst, L, Lb, inv_L);
+  }
+  zero_fill_bytes<NS>(dst, cph, rows_pad, L, Lb);
+}
+
 // Four consecutive grad_out elements -> the fp32 LDS tile [rows_pad][Lq].
 template <typename S>
 __device__ __forceinline__ void put_grad_out_quad(typename Io<S>::quad_t q, int g, float *do_dst, int L, int Lq, float inv_L) {
@@ -411,40 +443,16 @@ __global__ void __launch_bounds__(ssa_threads(MC)) ssa_forward_kernel(const SsaA
   }
 }
 
+// The products of the backward for the head whose tiles are in LDS (grad_out as fp32 in do_lds, spikes as bytes):
+// dS through ds_lds, then dQ, dK, dV stored at gq + qoff / koff / voff.  Every wavefront of the block calls it.
 template <typename S, int MC>
-__global__ void __launch_bounds__(ssa_threads(MC), MC == 1 ? SJHIP_SSA_BWD_RESIDENT : 1) ssa_backward_kernel(const SsaArgs a) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char ssa_lds[];
+__device__ __forceinline__ void ssa_backward_products(const SsaArgs &a, float *do_lds, float *ds_lds, const uint8_t *q_lds,
+                                                      const uint8_t *k_lds, const uint8_t *v_lds, int64_t qoff, int64_t koff,
+                                                      int64_t voff) {
   typedef typename Io<S>::elem_t E;
   constexpr int CPH = 32 * MC;
-  constexpr int LS = CPH + 1;  // row stride of the fp32 dS tile
+  constexpr int LS = CPH + 1;
   const int L = a.L, Lb = a.Lb, Lq = a.Lq, cph = a.cph;
-  float *do_lds = reinterpret_cast<float *>(ssa_lds);
-  float *ds_lds = do_lds + CPH * Lq;
-  uint8_t *q_lds = reinterpret_cast<uint8_t *>(ds_lds + CPH * LS);  // CPH * LS * 4 is a multiple of 16
-  uint8_t *k_lds = q_lds + CPH * Lb;
-  uint8_t *v_lds = k_lds + CPH * Lb;
-
-  const int64_t p = blockIdx.x;
-  const int64_t sample = p / a.heads, head = p - sample * a.heads;
-  const int64_t tile = (int64_t)cph * L;
-  const E *qkv = static_cast<const E *>(a.qkv);
-  const int64_t qoff = ((sample * 3 + 0) * a.heads + head) * tile;
-  const int64_t koff = ((sample * 3 + 1) * a.heads + head) * tile;
-  const int64_t voff = ((sample * 3 + 2) * a.heads + head) * tile;
-  {
-    uint8_t *const dst[3] = {q_lds, k_lds, v_lds};
-    if (a.qkv_bits) {
-      const uint8_t *const src[3] = {a.qkv_bits + qoff / 8, a.qkv_bits + koff / 8, a.qkv_bits + voff / 8};
-      stage_grad_out<S>(static_cast<const E *>(a.grad_out) + p * tile, do_lds, cph, CPH, L, Lq, a.vec != 0);
-      stage_bits<3>(src, dst, cph, CPH, L, Lb);
-    } else {
-      const E *const src[3] = {qkv + qoff, qkv + koff, qkv + voff};
-      stage_tiles<S, 3, true, 2>(src, dst, static_cast<const E *>(a.grad_out) + p * tile, do_lds, cph, CPH, L, Lb, Lq,
-                                 a.vec != 0);
-    }
-  }
-  __syncthreads();
-
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, half = lane >> 5;
   const float scale = a.scale;
 
@@ -580,6 +588,355 @@ __global__ void __launch_bounds__(ssa_threads(MC), MC == 1 ? SJHIP_SSA_BWD_RESID
   }
 }
 
+template <typename S, int MC>
+__global__ void __launch_bounds__(ssa_threads(MC), MC == 1 ? SJHIP_SSA_BWD_RESIDENT : 1) ssa_backward_kernel(const SsaArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char ssa_lds[];
+  typedef typename Io<S>::elem_t E;
+  constexpr int CPH = 32 * MC;
+  constexpr int LS = CPH + 1;  // row stride of the fp32 dS tile
+  const int L = a.L, Lb = a.Lb, Lq = a.Lq, cph = a.cph;
+  float *do_lds = reinterpret_cast<float *>(ssa_lds);
+  float *ds_lds = do_lds + CPH * Lq;
+  uint8_t *q_lds = reinterpret_cast<uint8_t *>(ds_lds + CPH * LS);  // CPH * LS * 4 is a multiple of 16
+  uint8_t *k_lds = q_lds + CPH * Lb;
+  uint8_t *v_lds = k_lds + CPH * Lb;
+
+  const int64_t p = blockIdx.x;
+  const int64_t sample = p / a.heads, head = p - sample * a.heads;
+  const int64_t tile = (int64_t)cph * L;
+  const E *qkv = static_cast<const E *>(a.qkv);
+  const int64_t qoff = ((sample * 3 + 0) * a.heads + head) * tile;
+  const int64_t koff = ((sample * 3 + 1) * a.heads + head) * tile;
+  const int64_t voff = ((sample * 3 + 2) * a.heads + head) * tile;
+  {
+    uint8_t *const dst[3] = {q_lds, k_lds, v_lds};
+    if (a.qkv_bits) {
+      const uint8_t *const src[3] = {a.qkv_bits + qoff / 8, a.qkv_bits + koff / 8, a.qkv_bits + voff / 8};
+      stage_grad_out<S>(static_cast<const E *>(a.grad_out) + p * tile, do_lds, cph, CPH, L, Lq, a.vec != 0);
+      stage_bits<3>(src, dst, cph, CPH, L, Lb);
+    } else {
+      const E *const src[3] = {qkv + qoff, qkv + koff, qkv + voff};
+      stage_tiles<S, 3, true, 2>(src, dst, static_cast<const E *>(a.grad_out) + p * tile, do_lds, cph, CPH, L, Lb, Lq,
+                                 a.vec != 0);
+    }
+  }
+  __syncthreads();
+
+  ssa_backward_products<S, MC>(a, do_lds, ds_lds, q_lds, k_lds, v_lds, qoff, koff, voff);
+}
+
+// ---- the contraction fused with the LIF behind it -------------------------------------------------------------------
+// The reference's attention block feeds  out = scale (V K^T) Q  into a multi-step LIF (`attn_lif`, layer/attention.py:
+// 321-322, 383-384).  A block owns one (batch element, head) and walks the T steps: the product of step t is still in
+// the accumulators when the neuron takes it as its input, the membrane potential of the block's [Cph, L] positions
+// stays in registers in the accumulator layout, and `out` is never written.  For the backward the forward leaves h
+// (the potential before firing) instead; the backward walks the steps from the last to the first with the gradient of
+// the potential in registers, in the layout in which a work-item stages grad_out, forms dL/d out of step t from
+// grad_spike and h on the way into LDS and runs the products of ssa_backward_kernel on it.
+// Measured at T = 4, 64 x 12 heads of [32, 196] (us per launch): forward 49 against 25 (contraction) + 28 (neuron),
+// backward 131 against 82 + 44.  The fused kernels move 8.4 and 20.4 bytes per element instead of 12.4 and 28.4, but
+// both sides are bound by their vector instructions (about 1000 per work-item and step in the forward: the
+// expansion of the bits, the gather of Q, the neuron, the transposition of h), not by memory: requesting the next
+// step's bits during the current step and writing h and the spikes in whole rows changed nothing (49 us either
+// way), and with a block per (batch element, head) only 768 blocks exist.  The callers therefore use these kernels
+// only on request (configure.hip_fuse_ssa_lif).
+// Makes a wavefront-uniform value opaque to the optimiser at this point of a loop body: what is computed from it (LDS
+// addresses, per-row store offsets) is then formed inside the iteration and dies there, instead of being hoisted in
+// front of the loop over the steps and held in registers across it.
+template <typename T> __device__ __forceinline__ void per_step(T &x) { asm volatile("" : "+s"(x)); }
+
+constexpr int kLifUnits = 2;  // accumulator tiles of a wavefront whose potentials are kept: 32 * MC rows x 256 tokens
+constexpr int kLifQuads = 8;  // grad_out quads of a work-item whose potential gradients are kept
+
+struct SsaLifArgs {
+  SsaArgs s;             // qkv_bits, heads, cph, L, Lb, Lq, scale; problems = B * heads
+  FwdArgs f;             // the neuron's constants (forward)
+  BwdArgs b;             // the neuron's constants (backward)
+  int64_t T, B;
+  const float *v_init;   // [B][heads][cph][L], or one element (f.v_init_broadcast)
+  float *spikes;         // [T][B][heads][cph][L]
+  float *h_seq;          // forward: written unless null; backward: read
+  float *v_last;         // [B][heads][cph][L] or null
+  const float *grad_spikes;  // [T][B][heads][cph][L] or null (no gradient reaches the spikes)
+  const float *grad_v_last;  // or null
+  float *grad_v_init;        // or null
+};
+
+template <int MC, int CH, int RS>
+__device__ __forceinline__ void ssa_lif_forward_body(const SsaLifArgs &a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char ssa_lds[];
+  constexpr int CPH = 32 * MC;
+  const int L = a.s.L, Lb = a.s.Lb, cph = a.s.cph;
+  float *h_lds = reinterpret_cast<float *>(ssa_lds);  // [CPH][Lq]: h of the step, on its way out in whole rows
+  uint8_t *q_lds = reinterpret_cast<uint8_t *>(h_lds + CPH * a.s.Lq);
+  uint8_t *k_lds = q_lds + CPH * Lb;
+  uint8_t *v_lds = k_lds + CPH * Lb;
+  uint8_t *const dst[3] = {q_lds, k_lds, v_lds};
+
+  const int64_t bh = blockIdx.x;  // (batch element, head)
+  const int64_t batch = bh / a.s.heads, head = bh - batch * a.s.heads;
+  const int64_t tile = (int64_t)cph * L;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, half = lane >> 5;
+  const int nw = (int)blockDim.x >> 6;
+  const int ntiles = (L + 31) / 32;
+  const int units = ntiles * MC;  // unit u: output rows 32 (u % MC).., columns 32 (u / MC)..
+  const int ni = wave % MC;
+  const float tau = a.f.tau, scale = a.s.scale;
+
+  // the potentials of this wavefront's units, in the accumulator layout
+  float v[kLifUnits][16];
+#pragma unroll
+  for (int j = 0; j < kLifUnits; ++j) {
+    const int u = wave + j * nw;
+    const int col = (u / MC) * 32 + (lane & 31);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = ni * 32 + acc_row(r, lane);
+      const bool in = u < units && col < L && row < cph;
+      v[j][r] = in ? (a.f.v_init_broadcast ? a.v_init[0] : a.v_init[bh * tile + (int64_t)row * L + col]) : 0.0f;
+    }
+  }
+
+  // the bits of a step are requested while the step before it is computed
+  const int64_t tb = tile / 8;
+  uint32_t bits_w[4][3];
+  auto request = [&](int64_t t) {
+    const int64_t sample = t * a.B + batch;
+    const uint8_t *const src[3] = {a.s.qkv_bits + ((sample * 3 + 0) * a.s.heads + head) * tb,
+                                   a.s.qkv_bits + ((sample * 3 + 1) * a.s.heads + head) * tb,
+                                   a.s.qkv_bits + ((sample * 3 + 2) * a.s.heads + head) * tb};
+    request_bits<3>(src, (int)tb, bits_w);
+  };
+  request(0);
+  for (int64_t t = 0; t < a.T; ++t) {
+    int L = a.s.L, Lb = a.s.Lb, Lq = a.s.Lq, cph = a.s.cph;
+    per_step(L); per_step(Lb); per_step(Lq); per_step(cph);
+    const int64_t sample = t * a.B + batch;
+    expand_bits<3>(bits_w, dst, cph, CPH, L, Lb);
+    __syncthreads();
+    request(t + 1 < a.T ? t + 1 : t);  // unconditional: the last step asks for its own bits again
+    if (wave < units) {
+      bf16x8 s_op[MC][2];
+#pragma unroll
+      for (int mi = 0; mi < MC; ++mi) {
+        const i32x16 acc = spike_gram(k_lds, mi * 32, v_lds, ni * 32, Lb, lane);
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+          uint16_t w[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) w[e] = (uint16_t)(__builtin_bit_cast(uint32_t, (float)acc[8 * h2 + e]) >> 16);  // exact: <= 256
+          s_op[mi][h2] = __builtin_bit_cast(bf16x8, w);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kLifUnits; ++j) {
+        const int u = wave + j * nw;
+        if (u < units) {
+          const int nt = u / MC;
+          const int col = nt * 32 + (lane & 31);
+          const int colc = col < L ? col : L - 1;
+          f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+          for (int mi = 0; mi < MC; ++mi) {
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2) {
+              uint16_t w[8];
+#pragma unroll
+              for (int e = 0; e < 8; ++e) {
+                const int c2 = mi * 32 + 16 * h2 + 8 * (e >> 2) + 4 * half + (e & 3);
+                w[e] = (uint16_t)(q_lds[c2 * Lb + colc] * 0x3f80u);  // 1 -> bf16 1.0
+              }
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s_op[mi][h2], __builtin_bit_cast(bf16x8, w), acc, 0, 0, 0);
+            }
+          }
+          float h[16], sp[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) neuron_step<float, CH, RS>(acc[r] * scale, v[j][r], h[r], sp[r], tau, a.f);
+          // h goes to LDS in the accumulator layout (a row of 32 tokens per store) and leaves it below in whole rows
+          if (col < L) {
+            float *hp = h_lds + (ni * 32 + 4 * half) * Lq + col;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) hp[(8 * (r >> 2) + (r & 3)) * Lq] = h[r];
+          }
+        }
+      }
+    }
+    __syncthreads();  // h of the step is complete, and the spike tiles are read no more
+    {
+      // 16 bytes per work-item, consecutive work-items consecutive addresses; the spike is recomputed from h with
+      // the comparison of neuron_step
+      float *sp_tile = a.spikes + (sample * a.s.heads + head) * tile;
+      float *h_tile = a.h_seq ? a.h_seq + (sample * a.s.heads + head) * tile : nullptr;
+      const int G = cph * L / 4;
+      const float inv_L = 1.0f / (float)L;
+      for (int g = threadIdx.x; g < G; g += (int)blockDim.x) {
+        const int r = div_tokens(4 * g, inv_L), c = 4 * g - r * L;
+        const f32x4 hv = *reinterpret_cast<const f32x4 *>(h_lds + r * Lq + c);
+        f32x4 sv;
+        {
+#pragma clang fp contract(off)
+          sv.x = (hv.x - a.f.vth_sub >= 0.0f) ? 1.0f : 0.0f;
+          sv.y = (hv.y - a.f.vth_sub >= 0.0f) ? 1.0f : 0.0f;
+          sv.z = (hv.z - a.f.vth_sub >= 0.0f) ? 1.0f : 0.0f;
+          sv.w = (hv.w - a.f.vth_sub >= 0.0f) ? 1.0f : 0.0f;
+        }
+        reinterpret_cast<f32x4 *>(sp_tile)[g] = sv;
+        if (h_tile) reinterpret_cast<f32x4 *>(h_tile)[g] = hv;
+      }
+    }
+  }
+
+  if (a.v_last) {
+#pragma unroll
+    for (int j = 0; j < kLifUnits; ++j) {
+      const int u = wave + j * nw;
+      const int col = (u / MC) * 32 + (lane & 31);
+      if (u < units && col < L) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = ni * 32 + acc_row(r, lane);
+          if (row < cph) a.v_last[bh * tile + (int64_t)row * L + col] = v[j][r];
+        }
+      }
+    }
+  }
+}
+
+template <int MC, int CH> __device__ __forceinline__ void ssa_lif_forward_reset(const SsaLifArgs &a) {
+  if (a.f.soft_reset) ssa_lif_forward_body<MC, CH, RESET_SOFT>(a);
+  else ssa_lif_forward_body<MC, CH, RESET_HARD>(a);
+}
+// the charge and the reset rule are chosen outside the loop over the steps, so that each copy of the loop holds the
+// constants of one rule only
+template <int MC>
+__global__ void __launch_bounds__(ssa_threads(MC)) ssa_lif_forward_kernel(const SsaLifArgs a) {
+  switch (a.f.charge) {
+    case CH_IF: ssa_lif_forward_reset<MC, CH_IF>(a); break;
+    case CH_DECAY_INPUT_DIV: ssa_lif_forward_reset<MC, CH_DECAY_INPUT_DIV>(a); break;
+    case CH_DECAY_INPUT_MUL: ssa_lif_forward_reset<MC, CH_DECAY_INPUT_MUL>(a); break;
+    case CH_PLAIN_INPUT_DIV: ssa_lif_forward_reset<MC, CH_PLAIN_INPUT_DIV>(a); break;
+    default: ssa_lif_forward_reset<MC, CH_PLAIN_INPUT_MUL>(a); break;
+  }
+}
+
+// dL/d input and the gradient handed to the step before, for four neurons of one step: the recurrence of
+// backward_body (neuron_bwd.h) for IF / LIF with a hard or soft, detached or attached reset.
+template <int SG>
+__device__ __forceinline__ void lif_quad_backward(const float (&gs)[4], const float (&h)[4], float (&gv)[4], float (&gx)[4],
+                                                  const BwdArgs &b, float kx, float km) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+#pragma clang fp contract(fast)
+    const float over = h[j] - b.v_th;
+    const float s = (over >= 0.0f) ? 1.0f : 0.0f;
+    const float sg = surrogate_grad<SG, false>(over, b.alpha);
+    const float dvdh = (1.0f - s * b.cB) + (b.cC - h[j] * b.cD) * sg;
+    const float G = gv[j] * dvdh + gs[j] * sg;
+    gx[j] = G * kx;
+    gv[j] = G * km;
+  }
+}
+template <int MC, int SG>
+__device__ __forceinline__ void ssa_lif_backward_body(const SsaLifArgs &a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char ssa_lds[];
+  constexpr int CPH = 32 * MC;
+  constexpr int LS = CPH + 1;
+  const int L = a.s.L, Lb = a.s.Lb, Lq = a.s.Lq, cph = a.s.cph;
+  float *do_lds = reinterpret_cast<float *>(ssa_lds);
+  float *ds_lds = do_lds + CPH * Lq;
+  uint8_t *q_lds = reinterpret_cast<uint8_t *>(ds_lds + CPH * LS);
+  uint8_t *k_lds = q_lds + CPH * Lb;
+  uint8_t *v_lds = k_lds + CPH * Lb;
+  uint8_t *const dst[3] = {q_lds, k_lds, v_lds};
+
+  const int64_t bh = blockIdx.x;
+  const int64_t batch = bh / a.s.heads, head = bh - batch * a.s.heads;
+  const int64_t tile = (int64_t)cph * L;
+  const int tid = threadIdx.x, nthreads = (int)blockDim.x;
+  const int G = cph * L / 4;  // quads of a tile; L is a multiple of 4
+  const float inv_L = 1.0f / (float)L;
+  const float kx = a.b.is_if ? 1.0f : (a.b.decay_input ? a.b.k : 1.0f);
+  const float km = a.b.is_if ? 1.0f : (1.0f - a.b.k);
+
+  // gradient of the potential after the step being processed, for the quads this work-item stages
+  float gv[kLifQuads][4];
+#pragma unroll
+  for (int j = 0; j < kLifQuads; ++j) {
+    const int g = tid + j * nthreads;
+    f32x4 w = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (a.grad_v_last && g < G) w = reinterpret_cast<const f32x4 *>(a.grad_v_last + bh * tile)[g];
+    gv[j][0] = w.x; gv[j][1] = w.y; gv[j][2] = w.z; gv[j][3] = w.w;
+  }
+  zero_fill_f32(do_lds, cph, CPH, L, Lq);  // the padding of the grad_out tile: written once, never overwritten
+
+  for (int64_t t = a.T - 1; t >= 0; --t) {
+    SsaArgs sa = a.s;
+    per_step(sa.L); per_step(sa.Lb); per_step(sa.Lq); per_step(sa.cph);
+    const int L = sa.L, Lb = sa.Lb, Lq = sa.Lq, cph = sa.cph;
+    const int64_t sample = t * a.B + batch;
+    const int64_t p = sample * a.s.heads + head;
+    const int64_t qoff = ((sample * 3 + 0) * a.s.heads + head) * tile;
+    const int64_t koff = ((sample * 3 + 1) * a.s.heads + head) * tile;
+    const int64_t voff = ((sample * 3 + 2) * a.s.heads + head) * tile;
+    {
+      // dL/d out of this step from grad_spike and h, on its way into LDS
+      const f32x4 *gsp = a.grad_spikes ? reinterpret_cast<const f32x4 *>(a.grad_spikes + p * tile) : nullptr;
+      const f32x4 *hp = reinterpret_cast<const f32x4 *>(a.h_seq + p * tile);
+      f32x4 gs_q[kLifQuads], h_q[kLifQuads];
+#pragma unroll
+      for (int j = 0; j < kLifQuads; ++j) {
+        const int g = tid + j * nthreads;
+        const int gc = g < G ? g : G - 1;  // requests are unconditional; what lies beyond the tile is not used
+        h_q[j] = hp[gc];
+        if (gsp) gs_q[j] = gsp[gc];
+        else gs_q[j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+      }
+#pragma unroll
+      for (int j = 0; j < kLifQuads; ++j) {
+        const int g = tid + j * nthreads;
+        if (g < G) {
+          const float gs[4] = {gs_q[j].x, gs_q[j].y, gs_q[j].z, gs_q[j].w};
+          const float h[4] = {h_q[j].x, h_q[j].y, h_q[j].z, h_q[j].w};
+          float gx[4];
+          lif_quad_backward<SG>(gs, h, gv[j], gx, a.b, kx, km);
+          const int r = div_tokens(4 * g, inv_L), c = 4 * g - r * L;
+          f32x4 w; w.x = gx[0]; w.y = gx[1]; w.z = gx[2]; w.w = gx[3];
+          *reinterpret_cast<f32x4 *>(do_lds + r * Lq + c) = w;
+        }
+      }
+      const uint8_t *const src[3] = {a.s.qkv_bits + qoff / 8, a.s.qkv_bits + koff / 8, a.s.qkv_bits + voff / 8};
+      stage_bits<3>(src, dst, cph, CPH, L, Lb);
+    }
+    __syncthreads();
+    ssa_backward_products<float, MC>(sa, do_lds, ds_lds, q_lds, k_lds, v_lds, qoff, koff, voff);
+    __syncthreads();  // the tiles are read no more: the step before may overwrite them
+  }
+
+  if (a.grad_v_init) {
+#pragma unroll
+    for (int j = 0; j < kLifQuads; ++j) {
+      const int g = tid + j * nthreads;
+      if (g < G) {
+        f32x4 w; w.x = gv[j][0]; w.y = gv[j][1]; w.z = gv[j][2]; w.w = gv[j][3];
+        reinterpret_cast<f32x4 *>(a.grad_v_init + bh * tile)[g] = w;
+      }
+    }
+  }
+}
+
+template <int MC>
+__global__ void __launch_bounds__(ssa_threads(MC), MC == 1 ? SJHIP_SSA_LIF_BWD_RESIDENT : 1) ssa_lif_backward_kernel(const SsaLifArgs a) {
+  switch (a.b.sg) {
+    case SJHIP_SG_SIGMOID: ssa_lif_backward_body<MC, SJHIP_SG_SIGMOID>(a); break;
+    case SJHIP_SG_ATAN: ssa_lif_backward_body<MC, SJHIP_SG_ATAN>(a); break;
+    case SJHIP_SG_PIECEWISE_QUADRATIC: ssa_lif_backward_body<MC, SJHIP_SG_PIECEWISE_QUADRATIC>(a); break;
+    case SJHIP_SG_PIECEWISE_EXP: ssa_lif_backward_body<MC, SJHIP_SG_PIECEWISE_EXP>(a); break;
+    case SJHIP_SG_SOFT_SIGN: ssa_lif_backward_body<MC, SJHIP_SG_SOFT_SIGN>(a); break;
+    case SJHIP_SG_SUPER_SPIKE: ssa_lif_backward_body<MC, SJHIP_SG_SUPER_SPIKE>(a); break;
+    default: ssa_lif_backward_body<MC, SJHIP_SG_ERF>(a); break;
+  }
+}
+
 int lds_row_bytes(int L) { return (L + 31) & ~31; }
 int lds_row_f32(int L) { return ((L + 15) & ~15) + 4; }
 
@@ -657,6 +1014,66 @@ int launch_ssa(bool backward, int dtype, int64_t samples, int heads, int cph, in
     case SJHIP_F16: return launch_dtype<f16_t>(a, backward, stream);
     default: return launch_dtype<bf16_t>(a, backward, stream);
   }
+}
+
+int launch_ssa_lif(bool backward, int neuron, const sjhip_neuron_params &p, int64_t T, int64_t B, int heads, int cph, int64_t L,
+                   float scale, const uint8_t *qkv_bits, const float *v_init, float *spikes, float *h_seq, float *v_last,
+                   const float *grad_spikes, const float *grad_v_last, float *grad_qkv, float *grad_v_init,
+                   hipStream_t stream) {
+  const char *what = backward ? "ssa_lif_backward" : "ssa_lif_forward";
+  if (neuron != SJHIP_NEURON_IF && neuron != SJHIP_NEURON_LIF)
+    return fail(SJHIP_ERR_UNSUPPORTED, "%s: neuron %d (IF and LIF only)", what, neuron);
+  if (!ssa_supported(SJHIP_F32, cph, L) || L % 4 != 0 || ((int64_t)cph * L) % 8 != 0)
+    return fail(SJHIP_ERR_UNSUPPORTED, "%s: %d channels per head x %lld tokens (at most 64 channels, at most 256 tokens, tokens a "
+                "multiple of 4, a tile a multiple of 8 elements)", what, cph, (long long)L);
+  if (T < 1 || B < 1 || heads < 1 || B * heads > 0x7fffffffLL || T > (int64_t(1) << 40) / (B * heads))
+    return fail(SJHIP_ERR_INVALID, "%s: T=%lld B=%lld heads=%d", what, (long long)T, (long long)B, heads);
+  const bool broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) != 0;
+  if (!aligned16(spikes) || !aligned16(h_seq) || !aligned16(grad_spikes) || !aligned16(grad_v_last) || !aligned16(grad_v_init))
+    return fail(SJHIP_ERR_UNSUPPORTED, "%s: spike_seq, h_seq and the gradients must be 16-byte aligned", what);
+  SsaLifArgs a;
+  const int64_t N = B * heads * cph * L;
+  bool round_each = false;
+  int rc = build_fwd_args(a.f, round_each, neuron, SJHIP_F32, p, T, N, nullptr, v_init, nullptr, nullptr, nullptr, nullptr, nullptr);
+  if (rc != SJHIP_OK) return rc;
+  if (backward) {
+    rc = build_bwd_args(a.b, neuron, SJHIP_F32, p, T, N, grad_spikes, nullptr, grad_v_last, h_seq, v_init, nullptr, nullptr,
+                        grad_v_init, nullptr, nullptr);
+    if (rc != SJHIP_OK) return rc;
+  } else {
+    a.b = BwdArgs();
+  }
+  a.f.v_init_broadcast = broadcast ? 1 : 0;
+  a.s.qkv_bits = qkv_bits; a.s.qkv = nullptr; a.s.grad_out = nullptr; a.s.out = nullptr; a.s.grad_qkv = grad_qkv;
+  a.s.problems = B * heads; a.s.heads = heads; a.s.cph = cph; a.s.L = (int)L;
+  a.s.Lb = lds_row_bytes((int)L); a.s.Lq = lds_row_f32((int)L); a.s.vec = 1; a.s.scale = scale;
+  a.T = T; a.B = B;
+  a.v_init = v_init; a.spikes = spikes; a.h_seq = h_seq; a.v_last = v_last;
+  a.grad_spikes = grad_spikes; a.grad_v_last = grad_v_last; a.grad_v_init = grad_v_init;
+  const int mc = cph <= 32 ? 1 : 2;
+  const unsigned lds = backward ? backward_lds(cph, (int)L)
+                                : forward_lds(cph, (int)L) + (unsigned)(padded_rows(cph) * lds_row_f32((int)L) * 4);
+  const void *kernel = backward ? (mc == 1 ? (const void *)ssa_lif_backward_kernel<1> : (const void *)ssa_lif_backward_kernel<2>)
+                                : (mc == 1 ? (const void *)ssa_lif_forward_kernel<1> : (const void *)ssa_lif_forward_kernel<2>);
+  static std::once_flag once[4];
+  static hipError_t attr_rc[4] = {hipSuccess, hipSuccess, hipSuccess, hipSuccess};
+  const int slot = (backward ? 2 : 0) + (mc - 1);
+  std::call_once(once[slot], [&]() {
+    attr_rc[slot] = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSsaMaxLds);
+    (void)hipGetLastError();
+  });
+  if (lds > 64u * 1024u && attr_rc[slot] != hipSuccess)
+    return fail(SJHIP_ERR_LAUNCH, "%s: cannot raise the dynamic LDS limit: %s", what, hipGetErrorString(attr_rc[slot]));
+  ProfileScope prof(backward ? KC_SSA_BACKWARD : KC_SSA_FORWARD, stream);
+  const dim3 grid((unsigned)(B * heads)), threads(ssa_threads(mc));
+  if (backward) {
+    if (mc == 1) hipLaunchKernelGGL(ssa_lif_backward_kernel<1>, grid, threads, lds, stream, a);
+    else hipLaunchKernelGGL(ssa_lif_backward_kernel<2>, grid, threads, lds, stream, a);
+  } else {
+    if (mc == 1) hipLaunchKernelGGL(ssa_lif_forward_kernel<1>, grid, threads, lds, stream, a);
+    else hipLaunchKernelGGL(ssa_lif_forward_kernel<2>, grid, threads, lds, stream, a);
+  }
+  return check_launch(what);
 }
 
 }  // namespace sjhip
