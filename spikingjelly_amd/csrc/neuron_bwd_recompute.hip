@@ -74,7 +74,16 @@ int launch_replay(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T
 
   const bool narrow = dtype != SJHIP_F32 && !round_each;  // 16-bit storage, fp32 state: four neurons per work-item
   const int V = (dtype == SJHIP_F32 || narrow) ? 4 : 8;
-  const int block = recompute_block(dtype, lds_steps, round_each);
+  // The walk over several pieces measured faster with each XCD on a contiguous eighth of the columns at every row
+  // stride tried (T = 128: 1.65 against 1.88 ms at N = 2^22, and likewise at seven other strides; T = 64: equal or
+  // better), unlike the single-piece kernel, which keeps the stride rule of column_spread().  In that order 256
+  // work-items per block are 2 to 4 % faster than 128 when two such blocks still fit a compute unit's LDS
+  // (T = 128: 1.604 -> 1.543 ms; one piece of 16 steps at N = 2^25 + 1024: 1.466 -> 1.455).
+  const bool auto_order = tuning().column_spread == 2;
+  if (chunk > 0 && T > chunk && auto_order) b.spread = 1;
+  int block = recompute_block(dtype, lds_steps, round_each);
+  if (b.spread && auto_order && kSpreadBlock <= SJHIP_MAX_BLOCK && 2 * lds_steps * kSpreadBlock * kHBytesPerItem <= (int64_t)kMaxLds)
+    block = kSpreadBlock;
   const int64_t items = N / V;
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "backward(recompute): N=%lld", (long long)N);
@@ -83,10 +92,6 @@ int launch_replay(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T
   if (cap > lds) lds = cap;
   const bool plif = neuron == SJHIP_NEURON_PLIF;
   const int mode = plif ? BWD_PLIF : ((neuron == SJHIP_NEURON_QIF || neuron == SJHIP_NEURON_EIF) ? BWD_QIF : BWD_PLAIN);
-  // The walk over several pieces measured faster with each XCD on a contiguous eighth of the columns at every row
-  // stride tried (T = 128: 1.65 against 1.88 ms at N = 2^22, and likewise at seven other strides; T = 64: equal or
-  // better), unlike the single-piece kernel, which keeps the stride rule of column_spread().
-  if (chunk > 0 && T > chunk && tuning().column_spread == 2) b.spread = 1;
   PieceArgs piece_args;
   piece_args.checkpoints = const_cast<void *>(checkpoints); piece_args.chunk = chunk;
   piece_args.pieces = chunk > 0 ? (T + chunk - 1) / chunk : 1;

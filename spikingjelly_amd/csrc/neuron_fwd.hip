@@ -15,7 +15,8 @@ constexpr bool kStreamX = (sizeof(S) == 2 && !ROUND_EACH) || (sizeof(S) == 4 && 
 
 template <typename S, bool ROUND_EACH, bool PACKED = false>
 int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
-  const int block = tuning().fwd_block;
+  int block = tuning().fwd_block;
+  if (a.spread && tuning().column_spread == 2 && block < kSpreadBlock && kSpreadBlock <= SJHIP_MAX_BLOCK) block = kSpreadBlock;
   const int V = vector ? Acc<S, true, true>::V : 1;
   const int64_t items = (a.N + V - 1) / V;
   const int64_t blocks = (items + block - 1) / block;

@@ -245,10 +245,14 @@ int check_launch(const char *what);
 
 // Largest block the neuron kernels may be launched with.  Kept small on purpose: the kernels run
 // best with about one fat wavefront per SIMD (few resident waves, many loads in flight each), and a
-// small bound lets the compiler use several hundred VGPRs for the prefetch buffers.
+// small bound lets the compiler use several hundred VGPRs for the prefetch buffers.  128 work-items are the
+// default; 256 are used with the `spread` column order (see column_block()), where a block's longer contiguous run
+// per row measured faster.
 #ifndef SJHIP_MAX_BLOCK
-#define SJHIP_MAX_BLOCK 128
+#define SJHIP_MAX_BLOCK 256
 #endif
+// work-items per block of the neuron kernels in the `spread` order when the order is chosen automatically
+constexpr int kSpreadBlock = 256;
 
 struct Tuning {
   int fwd_block;
@@ -289,7 +293,11 @@ class ProfileScope {
 // 20, and an XCD that otherwise stays on one side of it is sent to both.  A plain four-stream copy shows none of this;
 // it takes the 32 to 64 concurrent row streams of these kernels.  `spread` gives each XCD one contiguous eighth of the
 // columns instead: slower than the default at friendly strides (2.85 against 2.65 on the benchmark step) and
-// insensitive to the stride (2.87 at K = 1024 against 3.57), so it is chosen for the resonant strides only.
+// insensitive to the stride (2.87 at K = 1024 against 3.57), so it is chosen for the resonant strides only.  With 256
+// work-items per block (4 KiB of a row per block and step instead of 2) the spread order loses nothing at the strides
+// where bit 12 is the odd one (forward + backward kernels, ms: K = 0 default order 2.62; spread with 256: K = 0 2.66,
+// K = 1024 2.68, K = 3072 2.70; spread with 128: 2.81 at K = 1024); where bit 20 is the odd one (K = 262 144,
+// 266 240) it stays at 3.10 with either block size (3.14 in the default order).
 inline bool resonant_row_stride(int64_t bytes) {
   return (bytes & 4095) == 0 && (((bytes >> 12) ^ (bytes >> 20)) & 1) != 0;
 }

@@ -54,8 +54,12 @@ def _blocks(dim, heads):
 
 @pytest.mark.parametrize("T,B,dim,heads,tokens", [(4, 8, 128, 4, 96), (2, 3, 64, 2, 20), (4, 2, 384, 12, 196)])
 def test_fused_block_equals_two_operator_block(T, B, dim, heads, tokens, monkeypatch):
-    # torch's convolution and batch norm in both blocks: this test is about the LIF -> contraction step alone
+    # torch's convolution and batch norm in both blocks: this test is about the LIF -> contraction step alone.  The two
+    # blocks must get the same bits out of the vendor library's convolution, so its algorithm choice is pinned (left
+    # free, the second of two identical calls has been seen to take another algorithm after other tests had run)
     monkeypatch.setattr(configure, "hip_fuse_conv_bn_lif", False)
+    monkeypatch.setattr(torch.backends.cudnn, "deterministic", True)
+    monkeypatch.setattr(torch.backends.cudnn, "benchmark", False)
     fused, plain = _blocks(dim, heads)
     x = seeded_randn((T, B, dim, tokens), 5)
     g = seeded_randn((T, B, dim, tokens), 6).cuda()
