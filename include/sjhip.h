@@ -543,9 +543,10 @@ int sjhip_bn_grad_input(const float *g, const float *y, const float *coef, int64
  * fp32 storage with v_seq or h_seq written (spikes-only and 16-bit forwards always run uncapped); it is
  * doubled for T < 16 and dropped for T < 4, where few rows are in flight per work-item.  Returns SJHIP_ERR_INVALID otherwise.
  * "column_spread" = which columns a block of the neuron kernels takes: 0 = block b takes chunk b of a row (each XCD
- * every eighth chunk), 1 = each XCD one contiguous eighth of the row, 2 (default) = 1 only for row strides that are a
- * multiple of 4 KiB with odd parity of address bits 12 and 20, where the default order measured 20 to 35 % slower
- * (in mode 2 the kernels that take the second order also take 256 work-items per block, whatever the block keys say).
+ * every eighth chunk), 1 = each XCD one contiguous eighth of the row, 2 (default) = order 0 except for row strides that
+ * are a multiple of 4 KiB with odd parity of address bits 12 and 20, where it measured 20 to 35 % slower: there the
+ * XCDs take runs of 256 consecutive blocks in turn and the block size follows the stride (256 or 128 work-items,
+ * whatever the block keys say).
  * Results never depend on these.
  */
 int sjhip_set_tuning(const char *key, int value);

@@ -79,11 +79,15 @@ int launch_replay(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T
   // better), unlike the single-piece kernel, which keeps the stride rule of column_spread().  In that order 256
   // work-items per block are 2 to 4 % faster than 128 when two such blocks still fit a compute unit's LDS
   // (T = 128: 1.604 -> 1.543 ms; one piece of 16 steps at N = 2^25 + 1024: 1.466 -> 1.455).
+  // A single piece at a resonant stride takes the order and the block size column_spread() and spread_block() give.
   const bool auto_order = tuning().column_spread == 2;
-  if (chunk > 0 && T > chunk && auto_order) b.spread = 1;
+  const bool several = chunk > 0 && T > chunk;
+  if (several && auto_order) b.spread = 1;
   int block = recompute_block(dtype, lds_steps, round_each);
-  if (b.spread && auto_order && kSpreadBlock <= SJHIP_MAX_BLOCK && 2 * lds_steps * kSpreadBlock * kHBytesPerItem <= (int64_t)kMaxLds)
-    block = kSpreadBlock;
+  if (b.spread && auto_order) {
+    const int want = several ? kSpreadBlock : spread_block(N * (dtype == SJHIP_F32 ? 4 : 2));
+    if (want > block && want <= SJHIP_MAX_BLOCK && 2 * lds_steps * want * kHBytesPerItem <= (int64_t)kMaxLds) block = want;
+  }
   const int64_t items = N / V;
   const int64_t blocks = (items + block - 1) / block;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "backward(recompute): N=%lld", (long long)N);

@@ -265,8 +265,8 @@ struct Tuning {
 // dynamic LDS bytes that cap residency at `blocks_per_cu` blocks (0 for no cap)
 unsigned occupancy_cap_lds(int blocks_per_cu);
 const Tuning &tuning();
-// whether the neuron kernels give each XCD a contiguous eighth of the columns for rows of `row_bytes`
-inline bool column_spread(int64_t row_bytes);
+// the block-to-column order of the neuron kernels for rows of `row_bytes` (see column_block())
+inline int column_spread(int64_t row_bytes);
 
 enum KernelClass { KC_FORWARD = 0, KC_BACKWARD = 1, KC_PLIF_REDUCE = 2, KC_BIT_PACK = 3, KC_BIT_UNPACK = 4,
                    KC_SSA_FORWARD = 5, KC_SSA_BACKWARD = 6, KC_PW_GEMM = 7, KC_PW_GRAD_WEIGHT = 8, KC_BN_STATS = 9,
@@ -298,17 +298,37 @@ class ProfileScope {
 // where bit 12 is the odd one (forward + backward kernels, ms: K = 0 default order 2.62; spread with 256: K = 0 2.66,
 // K = 1024 2.68, K = 3072 2.70; spread with 128: 2.81 at K = 1024); where bit 20 is the odd one (K = 262 144,
 // 266 240) it stays at 3.10 with either block size (3.14 in the default order).
+// A third order deals the XCDs runs of kColumnRun consecutive blocks in turn (XCD x takes run x, 8 + x, ...).  At the
+// resonant strides it is as good as the contiguous eighths where bit 12 is the odd one and better where bit 20 is
+// (forward + backward kernels, ms, K = 262 144: 3.13 eighths, 2.89 runs; K = 266 240: 3.07 and 2.87; K = 1024: 2.70
+// and 2.67; K = 0, for comparison: 2.60 in the default order), with 256 work-items per block in the first case and 128
+// in the second (forward at K = 262 144: 1.27 ms with 128, 1.39 with 256; at K = 1024: 1.38 and 1.21).  At friendly
+// strides the runs are no better than the default order and for some worse (backward at N = 2^25 + 4096: 1.57
+// against 1.44 ms), so the default stays.
 inline bool resonant_row_stride(int64_t bytes) {
   return (bytes & 4095) == 0 && (((bytes >> 12) ^ (bytes >> 20)) & 1) != 0;
 }
-inline bool column_spread(int64_t row_bytes) {
+inline bool resonant_bit_20(int64_t bytes) { return ((bytes >> 20) & 1) != 0; }
+constexpr int kColumnRun = 256;
+// The `spread` argument of column_block() for rows of `row_bytes`: 0 the default order, 1 contiguous eighths, larger
+// values runs of that many blocks.  Tuning key "column_spread": 0 and 1 force those orders, 2 (default) chooses runs
+// of kColumnRun blocks for the resonant strides.
+inline int column_spread(int64_t row_bytes) {
   const int mode = tuning().column_spread;
-  return mode == 2 ? resonant_row_stride(row_bytes) : mode != 0;
+  if (mode != 2) return mode != 0 ? 1 : 0;
+  return resonant_row_stride(row_bytes) ? kColumnRun : 0;
 }
+// work-items per block that go with column_spread() when it chose the order by itself
+inline int spread_block(int64_t row_bytes) { return resonant_bit_20(row_bytes) ? 128 : kSpreadBlock; }
 #ifdef __HIPCC__
 __device__ __forceinline__ unsigned column_block(int spread) {
   const unsigned b = blockIdx.x;
   if (!spread) return b;
+  if (spread > 1) {
+    const unsigned g = (unsigned)spread, x = b % 8u, i = b / 8u;
+    const unsigned full = gridDim.x / (8u * g) * (8u * g);  // blocks beyond the last full round of runs keep their number
+    return b < full ? ((i / g) * 8u + x) * g + i % g : b;
+  }
   const unsigned per = gridDim.x / 8u;
   return b < per * 8u ? (b % 8u) * per + b / 8u : b;
 }
