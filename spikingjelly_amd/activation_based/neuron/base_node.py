@@ -2,11 +2,16 @@
 
 from __future__ import annotations
 
+import math
 from typing import Optional
 
 import torch
 
 from .. import base, surrogate
+
+
+# read-only one-element tensors that stand for a constant initial state on the hip backend (see _constant_state)
+_CONSTANT_STATES: dict = {}
 
 
 class BaseNode(base.MemoryModule):
@@ -113,7 +118,15 @@ class BaseNode(base.MemoryModule):
         backend it is a one-element tensor expanded to the shape (read-only, never written back: the next
         state is the kernel's own output) and no ``[N]`` tensor is filled or read."""
         if self.backend == "hip" and x.is_cuda and x.numel() > 1:
-            return x.new_full((1,) * x.dim(), value).expand(x.shape)
+            if torch.compiler.is_compiling() or torch.cuda.is_current_stream_capturing():
+                # (memory allocated while a graph is being captured belongs to that graph: not kept)
+                return x.new_full((1,) * x.dim(), value).expand(x.shape)
+            # one element per (device, dtype, value), made once: a fill launch per neuron and call otherwise
+            key = (x.device, x.dtype, float(value), math.copysign(1.0, float(value)))
+            one = _CONSTANT_STATES.get(key)
+            if one is None:
+                one = _CONSTANT_STATES[key] = x.new_full((1,), value)
+            return one.view((1,) * x.dim()).expand(x.shape)
         return torch.full_like(x, value, requires_grad=False)
 
     def materialize_states(self, inputs, states, step_mode: str):
