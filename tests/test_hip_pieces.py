@@ -207,16 +207,18 @@ def test_pieces_argument_checks(L):
     assert lib.sjhip_replay_pieces(40, 16) == 3 and lib.sjhip_replay_pieces(16, 16) == 1 and lib.sjhip_replay_pieces(0, 16) == 0
 
 
-@pytest.mark.parametrize("N", [8 * 300, 128 * 4 * 8 * 37 + 4, 1 << 20])
+@pytest.mark.parametrize("N", [8 * 300, 128 * 4 * 8 * 37 + 4, 1 << 20, 1024 * 2049, 262144 * 9])
 def test_block_to_column_order_does_not_change_results(L, N):
     """``column_spread`` only permutes which block works on which columns: forward, saved-h backward, replaying backward
-    and the pieces kernels must give the same bits either way (grids of fewer than eight blocks, a grid that is not a
-    multiple of eight, a large one)."""
+    and the pieces kernels must give the same bits whichever order runs (grids of fewer than eight blocks, a grid that
+    is not a multiple of eight, a large one; the last two row lengths are strides at which the automatic mode deals
+    runs of 256 blocks to the XCDs, with 256 and with 128 work-items per block, over more than 2048 blocks and a
+    remainder)."""
     lib = L.load()
     c = _case(L, L.NEURON_PLIF, torch.float32, 24, N, L.FLAG_DECAY_INPUT, 11)
     results = []
     try:
-        for mode in (0, 1):
+        for mode in (0, 1, 2):
             assert lib.sjhip_set_tuning(b"column_spread", mode) == 0
             s, v, vl = _forward_whole(L, c)
             sp, vp, vlp, ck = _forward_pieces(L, c, 16)
@@ -232,6 +234,7 @@ def test_block_to_column_order_does_not_change_results(L, N):
             results.append((s, v, vl, gx, gv0, gx1, gv1, gk1))
     finally:
         lib.sjhip_set_tuning(b"column_spread", 2)
-    for a, b in zip(results[0][:7], results[1][:7]):
-        assert bits_equal(a, b)
-    assert float(results[0][7].item()) == pytest.approx(float(results[1][7].item()), rel=1e-5)
+    for other in results[1:]:
+        for a, b in zip(results[0][:7], other[:7]):
+            assert bits_equal(a, b)
+        assert float(results[0][7].item()) == pytest.approx(float(other[7].item()), rel=1e-5)
