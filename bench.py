@@ -435,6 +435,7 @@ def other_workload(args) -> int:
 
     if args.workload == "config5":
         T, B, D, H, tokens = 4, 64, args.dim, 12, 196
+        configure.hip_fuse_ssa_lif = bool(args.fuse_ssa_lif)
         torch.manual_seed(1005)
         block = layer.SpikingSelfAttention(D, H, backend="hip").to(dev)
         x = randn((T, B, D, tokens), 1105, 0.0, 1.0, torch.float32).requires_grad_()
@@ -482,6 +483,8 @@ def main() -> int:
     ap.add_argument("--terms", type=int, default=3, choices=[1, 2, 3], help="pwconv workload: bf16 terms per fp32 operand")
     ap.add_argument("--dim", type=int, default=384, choices=[384, 768],
                     help="config5 workload: embedding width (12 heads of dim // 12 channels: 32, or 64 with 768)")
+    ap.add_argument("--fuse-ssa-lif", action="store_true",
+                    help="config5 workload: run the contraction and the attention's LIF as one kernel (configure.hip_fuse_ssa_lif)")
     ap.add_argument("--seq-len", type=int, default=SHAPE[0],
                     help="config2 variant: T steps over 2^29 / T neurons (the headline is T=16); a secondary measurement")
     ap.add_argument("--n-offset", type=int, default=0,

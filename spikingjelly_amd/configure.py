@@ -42,8 +42,8 @@ hip_conv_terms = 3
 hip_fuse_conv_bn_lif = True
 # True: the spiking self-attention feeds the contraction's output of every step straight into its `attn_lif` inside one
 # kernel (`sjhip_ssa_lif_forward_packed` / `_backward_packed`) where that kernel can serve, instead of writing the output
-# and running the neuron as a launch of its own.  Same results; off by default because it measured no faster (the
-# kernels on both sides are bound by their vector instructions, not by the bytes the fusion saves).
+# and running the neuron as a launch of its own.  Same results; off by default because it measured no faster (what
+# bounds the kernels on both sides is not the bytes the fusion saves).
 hip_fuse_ssa_lif = False
 hip_backward_recompute = True
 # Sequences longer than the replaying backward prefers in one piece (its LDS buffer for h grows with T) run, outside a

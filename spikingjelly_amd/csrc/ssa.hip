@@ -635,11 +635,12 @@ __global__ void __launch_bounds__(ssa_threads(MC), MC == 1 ? SJHIP_SSA_BWD_RESID
 // grad_spike and h on the way into LDS and runs the products of ssa_backward_kernel on it.
 // Measured at T = 4, 64 x 12 heads of [32, 196] (us per launch): forward 49 against 25 (contraction) + 28 (neuron),
 // backward 131 against 82 + 44.  The fused kernels move 8.4 and 20.4 bytes per element instead of 12.4 and 28.4, but
-// both sides are bound by their vector instructions (about 1000 per work-item and step in the forward: the
-// expansion of the bits, the gather of Q, the neuron, the transposition of h), not by memory: requesting the next
-// step's bits during the current step and writing h and the spikes in whole rows changed nothing (49 us either
-// way), and with a block per (batch element, head) only 768 blocks exist.  The callers therefore use these kernels
-// only on request (configure.hip_fuse_ssa_lif).
+// bytes are not what bounds either side: the forward runs 1216 vector instructions per wavefront and step (the
+// expansion of the bits, the gather of Q, the neuron, the transposition of h; vector ALU 48 % busy, memory at
+// 3.3 TB/s), a block per (batch element, head) gives only 768 blocks, three or two per compute unit, and each walks
+// its steps phase after phase between barriers.  Requesting the next step's bits during the current step and
+// writing h and the spikes in whole rows changed nothing (49 us either way).  The callers therefore use these
+// kernels only on request (configure.hip_fuse_ssa_lif).
 // Makes a wavefront-uniform value opaque to the optimiser at this point of a loop body: what is computed from it (LDS
 // addresses, per-row store offsets) is then formed inside the iteration and dies there, instead of being hoisted in
 // front of the loop over the steps and held in registers across it.
