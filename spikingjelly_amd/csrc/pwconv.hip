@@ -31,11 +31,13 @@
 //       one in the same step: 0.334 ms, and 0.352 ms with scheduler hints that ask for the staging instructions between
 //       the matrix-core instructions; not kept.  Two groups of four wavefronts per block, each with its own tile and
 //       one barrier apart so that one group multiplies while the other stages: 0.339 against 0.345 ms on random data,
-//       not kept either.  Cycle counters around the phases of a K step (one wavefront, steady state): with one block
-//       per compute unit staging 1150, multiplication 2160 (48 matrix-core instructions of 32 cycles: 71 %), barriers
-//       320 cycles, 30.8 us per tile = 1.46 GHz; with two blocks 1280 / 3060 / 360 cycles and 49.3 us per tile =
-//       1.2 GHz.  The chip lowers its clock as the matrix cores fill (the same launch on an all-zero input takes 0.265
-//       instead of 0.330 ms), so what a better overlap of the phases gains in cycles is largely lost in clock rate.
+//       not kept either.  The timestamp counter (clock64) around the phases of a K step (one wavefront, steady state):
+//       with one block per compute unit staging 1150, multiplication 2160 (48 matrix-core instructions of 32 cycles
+//       would be 1536), barriers 320 ticks, 45 k ticks per tile of 30.8 us; with two blocks 1280 / 3060 / 360 and 59 k
+//       ticks per tile of 49.3 us: the second block adds a third to the throughput, not a factor of two.  How fast
+//       the chip runs depends on what the matrix cores are fed: the same launch on an all-zero input takes 0.265
+//       instead of 0.330 ms, and GRBM_GUI_ACTIVE over the kernel's duration gives 1.93 GHz here against 2.5 GHz in a
+//       kernel that hardly uses them, so what a better overlap of the phases gains in cycles is partly lost in clock.
 //       By number of products (M = 1152, K = 384, random data): 1 product 0.15-0.16 ms, 2: 0.17-0.18, 3: 0.22,
 //       6: 0.33-0.35.  The weight planes are stored tile by tile ([row tile][k step][row][k], 8 KiB per staged tile in
 //       a row) so that every 128-byte line a block fetches is used whole: 0.345 -> 0.338 ms, one-term activations
