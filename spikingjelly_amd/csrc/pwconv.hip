@@ -38,6 +38,8 @@
 //       the chip runs depends on what the matrix cores are fed: the same launch on an all-zero input takes 0.265
 //       instead of 0.330 ms, and GRBM_GUI_ACTIVE over the kernel's duration gives 1.93 GHz here against 2.5 GHz in a
 //       kernel that hardly uses them, so what a better overlap of the phases gains in cycles is partly lost in clock.
+//       Raising the wavefront priority for the multiplication (s_setprio 2 around it): 0.348 and 0.331 ms
+//       (Y = W X and dX) against 0.338 and 0.300; not kept.
 //       By number of products (M = 1152, K = 384, random data): 1 product 0.15-0.16 ms, 2: 0.17-0.18, 3: 0.22,
 //       6: 0.33-0.35.  The weight planes are stored tile by tile ([row tile][k step][row][k], 8 KiB per staged tile in
 //       a row) so that every 128-byte line a block fetches is used whole: 0.345 -> 0.338 ms, one-term activations
