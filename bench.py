@@ -483,6 +483,9 @@ def main() -> int:
     ap.add_argument("--terms", type=int, default=3, choices=[1, 2, 3], help="pwconv workload: bf16 terms per fp32 operand")
     ap.add_argument("--dim", type=int, default=384, choices=[384, 768],
                     help="config5 workload: embedding width (12 heads of dim // 12 channels: 32, or 64 with 768)")
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                    help="launch tuning of the library for this run (sjhip_set_tuning), e.g. --tune column_spread=1 "
+                         "--tune fwd_block=256; may be given several times")
     ap.add_argument("--fuse-ssa-lif", action="store_true",
                     help="config5 workload: run the contraction and the attention's LIF as one kernel (configure.hip_fuse_ssa_lif)")
     ap.add_argument("--seq-len", type=int, default=SHAPE[0],
@@ -503,6 +506,9 @@ def main() -> int:
     from spikingjelly_amd.activation_based.hip_kernel import library as L
 
     L.load()
+    for item in args.tune:
+        key, _, value = item.partition("=")
+        L.set_tuning(key.strip(), int(value))
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm device", file=sys.stderr)
         return 2

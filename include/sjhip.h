@@ -546,7 +546,7 @@ int sjhip_bn_grad_input(const float *g, const float *y, const float *coef, int64
  * every eighth chunk), 1 = each XCD one contiguous eighth of the row, 2 (default) = order 0 except for row strides that
  * are a multiple of 4 KiB with odd parity of address bits 12 and 20, where it measured 20 to 35 % slower: there the
  * XCDs take runs of 256 consecutive blocks in turn and the block size follows the stride (256 or 128 work-items,
- * whatever the block keys say).
+ * whatever the block keys say); 4 ... 65536 = runs of that many blocks at every stride.
  * Results never depend on these.
  */
 int sjhip_set_tuning(const char *key, int value);

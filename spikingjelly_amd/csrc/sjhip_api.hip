@@ -668,7 +668,7 @@ int sjhip_set_tuning(const char *key, int value) {
   if (!strcmp(key, "fwd_blocks_per_cu")) { if (!cap_ok) return fail(SJHIP_ERR_INVALID, "set_tuning: fwd_blocks_per_cu=%d", value); g_tuning.fwd_blocks_per_cu = value; return SJHIP_OK; }
   if (!strcmp(key, "bwd_blocks_per_cu")) { if (!cap_ok) return fail(SJHIP_ERR_INVALID, "set_tuning: bwd_blocks_per_cu=%d", value); g_tuning.bwd_blocks_per_cu = value; return SJHIP_OK; }
   if (!strcmp(key, "replay_blocks_per_cu")) { if (!cap_ok) return fail(SJHIP_ERR_INVALID, "set_tuning: replay_blocks_per_cu=%d", value); g_tuning.replay_blocks_per_cu = value; return SJHIP_OK; }
-  if (!strcmp(key, "column_spread")) { if (value < 0 || value > 2) return fail(SJHIP_ERR_INVALID, "set_tuning: column_spread=%d", value); g_tuning.column_spread = value; return SJHIP_OK; }
+  if (!strcmp(key, "column_spread")) { if (value < 0 || value == 3 || value > 65536) return fail(SJHIP_ERR_INVALID, "set_tuning: column_spread=%d", value); g_tuning.column_spread = value; return SJHIP_OK; }
   return fail(SJHIP_ERR_INVALID, "set_tuning: unknown key '%s'", key);
 }
 

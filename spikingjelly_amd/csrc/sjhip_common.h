@@ -260,7 +260,7 @@ struct Tuning {
   int fwd_blocks_per_cu;  // 0 = no cap; otherwise dynamic LDS is requested so that at most this many
   int bwd_blocks_per_cu;  // blocks are resident per compute unit
   int replay_blocks_per_cu;  // same for the replay backward (its LDS h buffer already bounds residency)
-  int column_spread;         // 0: never, 1: always, 2: by row stride (resonant_row_stride); see column_block()
+  int column_spread;         // 0, 1, >= 4: a fixed order, 2: by row stride (resonant_row_stride); see column_block()
 };
 // dynamic LDS bytes that cap residency at `blocks_per_cu` blocks (0 for no cap)
 unsigned occupancy_cap_lds(int blocks_per_cu);
@@ -311,11 +311,11 @@ inline bool resonant_row_stride(int64_t bytes) {
 inline bool resonant_bit_20(int64_t bytes) { return ((bytes >> 20) & 1) != 0; }
 constexpr int kColumnRun = 256;
 // The `spread` argument of column_block() for rows of `row_bytes`: 0 the default order, 1 contiguous eighths, larger
-// values runs of that many blocks.  Tuning key "column_spread": 0 and 1 force those orders, 2 (default) chooses runs
-// of kColumnRun blocks for the resonant strides.
+// values runs of that many blocks.  Tuning key "column_spread": 0 and 1 force those orders, 4 and more force runs of
+// that many blocks, 2 (default) chooses runs of kColumnRun blocks for the resonant strides.
 inline int column_spread(int64_t row_bytes) {
   const int mode = tuning().column_spread;
-  if (mode != 2) return mode != 0 ? 1 : 0;
+  if (mode != 2) return mode;
   return resonant_row_stride(row_bytes) ? kColumnRun : 0;
 }
 // work-items per block that go with column_spread() when it chose the order by itself

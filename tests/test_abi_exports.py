@@ -160,6 +160,8 @@ def test_argument_validation_without_a_device():
     assert lib.sjhip_get_tuning(b"bwd_blocks_per_cu") == 2
     assert lib.sjhip_get_tuning(b"column_spread") == 2
     assert lib.sjhip_set_tuning(b"column_spread", 3) == -1 and lib.sjhip_set_tuning(b"column_spread", -1) == -1
+    assert lib.sjhip_set_tuning(b"column_spread", 65537) == -1
+    assert lib.sjhip_set_tuning(b"column_spread", 256) == 0 and lib.sjhip_get_tuning(b"column_spread") == 256
     assert lib.sjhip_set_tuning(b"column_spread", 1) == 0 and lib.sjhip_get_tuning(b"column_spread") == 1
     assert lib.sjhip_set_tuning(b"column_spread", 2) == 0
     assert lib.sjhip_set_tuning(b"nope", 1) == -1

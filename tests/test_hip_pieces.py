@@ -218,7 +218,7 @@ def test_block_to_column_order_does_not_change_results(L, N):
     c = _case(L, L.NEURON_PLIF, torch.float32, 24, N, L.FLAG_DECAY_INPUT, 11)
     results = []
     try:
-        for mode in (0, 1, 2):
+        for mode in (0, 1, 2, 4, 64):
             assert lib.sjhip_set_tuning(b"column_spread", mode) == 0
             s, v, vl = _forward_whole(L, c)
             sp, vp, vlp, ck = _forward_pieces(L, c, 16)
