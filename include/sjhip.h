@@ -405,7 +405,8 @@ int sjhip_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, void *
  *   qkv      [samples, 3, heads, channels_per_head, tokens] in: binary spikes, q / k / v stacked on dim 1
  *   out      [samples, heads, channels_per_head, tokens] out = scale * (V K^T) Q, exact (integer sums in fp32)
  *   grad_out same shape as out, in;  grad_qkv same shape as qkv, out (dq, dk, dv)
- * One block of four wavefronts per (sample, head), the spikes of its three tiles parked in LDS as bytes.  Forward:
+ * One block of four wavefronts (eight for heads of more than 32 channels) per (sample, head), the spikes of its three
+ * tiles parked in LDS as bytes.  Forward:
  * V K^T on the int8 MFMA (exact integers), then (V K^T) Q on the bf16 MFMA with fp32 accumulation (V K^T <= 256 and
  * the spikes are exact in bf16), so out equals an integer matmul times scale bit for bit.  Backward: dS = scale dO Q^T
  * on the fp32 MFMA; dQ, dK, dV on the bf16 MFMA with the real-valued operand split into three bf16 terms that sum to
