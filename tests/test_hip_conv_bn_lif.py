@@ -101,6 +101,31 @@ def test_gemm_leaves_the_batch_norm_sums_of_its_output(C, S, M, Kd, Lp, terms):
     torch.testing.assert_close(b[1], a[1], rtol=1e-5, atol=2e-6)
 
 
+def test_gemm_over_several_launches(C):
+    """Per-lane offsets into the activations are 32-bit byte offsets, so a call whose samples span more than 2^30 bytes
+    of ``K * L`` rows runs as several launches over groups of samples (4095 samples of [4096, 64] fp32 and 5 more here): the
+    output and the batch-norm sums must come out as for one launch.  Binary activations and weights that are multiples
+    of 1/64 make every sum of the output exact, so that comparison is exact; samples are compared in slices to bound the
+    memory."""
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+
+    S, M, Kd, Lp = 4100, 8, 4096, 64
+    g = torch.Generator(device="cuda").manual_seed(41)
+    w = (torch.randint(-64, 65, (M, Kd), generator=torch.Generator().manual_seed(42)).float() / 64.0).cuda()
+    x = (torch.rand((S, Kd, Lp), device="cuda", generator=g) < 0.05).float()
+    planes = C.split_weight(w, False)
+    got, partial = C.pw_gemm(planes, 3, M, Kd, x, 1, stats=True)
+    rows = L.load().sjhip_pwconv_gemm_stats_rows(Kd, S, Lp)
+    assert rows == 2 * (-(-4095 * Lp // 128)) + 2 * (-(-5 * Lp // 128)) and partial.shape == (rows, M, 2)
+    for s0 in range(0, S, 410):
+        want = torch.einsum("mk,skl->sml", w.double(), x[s0:s0 + 410].double()).float()
+        assert torch.equal(got[s0:s0 + 410], want), s0
+    sums = partial.double().sum(0)
+    assert torch.equal(sums[:, 0], got.double().sum((0, 2)))
+    want_q = (got.double() ** 2).sum((0, 2))   # the squares' fp32 partial sums are rounded: 1e-6
+    assert float(((sums[:, 1] - want_q).abs() / want_q).max()) < 1e-6
+
+
 @pytest.mark.parametrize("S,M,N,Lp", [(3, 100, 50, 12), (9, 130, 257, 36), (16, 384, 384, 196), (2, 1152, 384, 196), (64, 64, 48, 8)])
 @pytest.mark.parametrize("spikes", [False, True])
 def test_grad_weight_gemm(C, S, M, N, Lp, spikes):
