@@ -244,15 +244,16 @@ int sjhip_neuron_backward_recompute(int neuron, int dtype, const sjhip_neuron_pa
  * The replay for sequences of any length, in one launch each way.  The sequence is cut into pieces of `chunk` steps
  * (the last may be shorter; sjhip_replay_pieces(T, chunk) of them).  sjhip_neuron_forward_pieces is
  * sjhip_neuron_forward with h_seq = NULL that also leaves the state after every piece but the last in
- * `checkpoints` [pieces - 1][N] (storage dtype; may be NULL when T <= chunk).  sjhip_neuron_backward_recompute_pieces
+ * `checkpoints` [pieces - 1][N] (storage dtype, see below; may be NULL when T <= chunk).  sjhip_neuron_backward_recompute_pieces
  * is sjhip_neuron_backward_recompute that walks the pieces from the last to the first: each is replayed from its
  * checkpoint into an LDS buffer of `chunk` steps (so chunk, not T, must satisfy sjhip_recompute_supported) and walked
  * back; the gradient of a piece's initial state stays in registers (fp32) for the piece before it.  Results: spikes,
  * states and checkpoints are bit-identical to sjhip_neuron_forward's; gradients are those of the walk over the whole
  * sequence (in fp32 storage also those of sjhip_neuron_backward_recompute applied piece by piece with grad_v_init
  * handed on as grad_v_last).  N must be a multiple of the 128-bit
- * vector width and every tensor 16-byte aligned; 16-bit storage with SJHIP_FLAG_FP32_STATE is refused
- * (SJHIP_ERR_UNSUPPORTED: a checkpoint in the storage dtype would round the state).  The saved state per neuron is 1 / chunk of an h_seq; chunk = 16 keeps
+ * vector width and every tensor 16-byte aligned.  With 16-bit storage and SJHIP_FLAG_FP32_STATE the checkpoints are
+ * fp32 rows ([pieces - 1][N] floats: a checkpoint in the storage dtype would round the state).  The saved state per
+ * neuron is 1 / chunk of an h_seq; chunk = 16 keeps
  * five or more blocks resident per compute unit, which is where the single-piece kernel runs fastest.  No counterpart
  * in the reference (its kernels always read the saved h_seq, multi_step/base.py:137-409).
  */

@@ -126,7 +126,9 @@ def _run_forward(neuron: int, x_seq: torch.Tensor, v_init: torch.Tensor, k: Opti
     v_seq = torch.empty_like(x_seq) if store_v_seq else x_seq.new_empty((0,))
     v_last = x_seq.new_empty((N,))
     h_seq = torch.empty_like(x_seq) if save_h else None
-    checkpoints = x_seq.new_empty((pieces - 1, N)) if pieces > 1 else None
+    # a state kept in fp32 beside 16-bit storage is checkpointed in fp32
+    ck_dtype = torch.float32 if flags & L.FLAG_FP32_STATE else x_seq.dtype
+    checkpoints = x_seq.new_empty((pieces - 1, N), dtype=ck_dtype) if pieces > 1 else None
     k_keep, k_ptr = _k_pointer(k, x_seq)
     params = _params(tau, v_th, v_reset, 0.0, 0, flags | broadcast, qif, levels)
     lib = L.load()
@@ -884,8 +886,6 @@ def replay_chunk(dtype: torch.dtype, T: int, N: int, flags: int) -> int:
     chunk = int(configure.hip_replay_chunk)
     if not configure.hip_backward_recompute or chunk <= 0 or T <= chunk:
         return 0
-    if dtype != torch.float32 and flags & L.FLAG_FP32_STATE:
-        return 0  # a checkpoint in the storage dtype would round the fp32 state
     return chunk if L.recompute_preferred(dtype, chunk, N, flags) else 0
 
 

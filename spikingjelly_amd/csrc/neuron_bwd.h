@@ -332,7 +332,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
   if (QIF) {
     if (a.grad_v_init || sgr.to_regs) {
       float v0[V];
-      load_state<S, VECTOR, SJHIP_BWD_NT != 0>(a.v_init, col, a.v_init_broadcast != 0, v0);
+      load_state_from<S, VECTOR, SJHIP_BWD_NT != 0>(a.v_init, col, a.v_init_broadcast, v0);
 #pragma unroll
       for (int j = 0; j < V; ++j) carry[j] *= qif_dh_dv(v0[j], k, a);
       if (!sgr.to_regs) A::store((E *)a.grad_v_init + col, carry);
@@ -346,7 +346,7 @@ __device__ __forceinline__ float backward_body(const BwdArgs &a, bool active, in
   }
   if (PLIF) {
     float v0[V];
-    load_state<S, VECTOR, SJHIP_BWD_NT != 0>(a.v_init, col, a.v_init_broadcast != 0, v0);
+    load_state_from<S, VECTOR, SJHIP_BWD_NT != 0>(a.v_init, col, a.v_init_broadcast, v0);
 #pragma unroll
     for (int j = 0; j < V; ++j) {
       const float dh_dk = a.decay_input ? (h_next[j] - v0[j]) : (a.v_reset - v0[j]);

@@ -47,7 +47,7 @@ __device__ __forceinline__ void recompute_body(const FwdArgs &a, f32x4 *lds_h, i
   for (int i = 0; i < PF; ++i) ahead[i] = (i < T) ? A::load(xp + (int64_t)i * N) : A::zero();
   typedef typename StepNum<S, ROUND_EACH>::type NUM;
   NUM v[V];
-  load_state<S, true, SJHIP_BWD_NT != 0>(a.v_init, col, a.v_init_broadcast != 0, v);
+  load_state_from<S, true, SJHIP_BWD_NT != 0>(a.v_init, col, a.v_init_broadcast, v);
 
   for (int64_t t0 = 0; t0 < T; t0 += PF) {
     typename A::raw_t cur[PF];
@@ -155,8 +155,13 @@ __global__ void __launch_bounds__(SJHIP_MAX_BLOCK) backward_recompute_pieces_ker
     f.T = len; b.T = len;
     f.x = (const E *)f0.x + t0 * N;
     if (j > 0) {
-      f.v_init = (const E *)p.checkpoints + (j - 1) * N;
-      f.v_init_broadcast = 0;
+      if (p.checkpoints_f32) {
+        f.v_init = (const float *)p.checkpoints + (j - 1) * N;
+        f.v_init_broadcast = kStateF32;
+      } else {
+        f.v_init = (const E *)p.checkpoints + (j - 1) * N;
+        f.v_init_broadcast = 0;
+      }
     }
     b.v_init = f.v_init;
     b.v_init_broadcast = f.v_init_broadcast;

@@ -98,6 +98,7 @@ int launch_replay(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T
   const int mode = plif ? BWD_PLIF : ((neuron == SJHIP_NEURON_QIF || neuron == SJHIP_NEURON_EIF) ? BWD_QIF : BWD_PLAIN);
   PieceArgs piece_args;
   piece_args.checkpoints = const_cast<void *>(checkpoints); piece_args.chunk = chunk;
+  piece_args.checkpoints_f32 = checkpoints_are_f32(dtype, p.flags) ? 1 : 0;
   piece_args.pieces = chunk > 0 ? (T + chunk - 1) / chunk : 1;
   const PieceArgs *pieces = chunk > 0 ? &piece_args : nullptr;
   {

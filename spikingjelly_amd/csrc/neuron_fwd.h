@@ -311,8 +311,18 @@ __device__ __forceinline__ void forward_body(const FwdArgs &a) {
         if (hp) A::store(hp + t * N, h);
         if (vp) A::store(vp + t * N, v);
         if (CKPT && t + 1 == next_checkpoint && t + 1 < T) {
-          A::store(cp, v);
-          cp += N;
+          if constexpr (sizeof(S) == 2 && !ROUND_EACH) {
+            // the state is kept in fp32 beside 16-bit storage: so is its checkpoint
+            float *cpf = (float *)a.checkpoints + (next_checkpoint / a.chunk - 1) * N + col;
+#pragma unroll
+            for (int q = 0; q < V / 4; ++q) {
+              f32x4 w; w.x = v[4 * q]; w.y = v[4 * q + 1]; w.z = v[4 * q + 2]; w.w = v[4 * q + 3];
+              stream_store<NT>(reinterpret_cast<f32x4 *>(cpf) + q, w);
+            }
+          } else {
+            A::store(cp, v);
+            cp += N;
+          }
           next_checkpoint += a.chunk;
         }
       }

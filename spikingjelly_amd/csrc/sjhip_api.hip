@@ -363,8 +363,6 @@ int sjhip_neuron_forward_pieces(int neuron, int dtype, const sjhip_neuron_params
   if (!x_seq || !v_init || !spike_seq) return fail(SJHIP_ERR_INVALID, "forward(pieces): NULL tensor");
   if (!v_seq && !v_last) return fail(SJHIP_ERR_INVALID, "forward(pieces): neither v_seq nor v_last given");
   if (T > chunk && !checkpoints) return fail(SJHIP_ERR_INVALID, "forward(pieces): %lld pieces need checkpoints", (long long)sjhip_replay_pieces(T, chunk));
-  if (dtype != SJHIP_F32 && (p->flags & SJHIP_FLAG_FP32_STATE))
-    return fail(SJHIP_ERR_UNSUPPORTED, "forward(pieces): an fp32 state does not survive a checkpoint of 16-bit storage");
   rc = check_levels("forward(pieces)", neuron, *p, false);
   if (rc != SJHIP_OK) return rc;
   if (neuron == SJHIP_NEURON_PLIF && !rtau_device) return fail(SJHIP_ERR_INVALID, "forward(pieces): PLIF needs rtau_device");
@@ -386,8 +384,6 @@ int sjhip_neuron_backward_recompute_pieces(int neuron, int dtype, const sjhip_ne
   if (chunk < 1) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): chunk %lld", (long long)chunk);
   if (!x_seq || !v_init || !grad_x_seq) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): NULL tensor");
   if (T > chunk && !checkpoints) return fail(SJHIP_ERR_INVALID, "backward(recompute, pieces): several pieces need checkpoints");
-  if (dtype != SJHIP_F32 && (p->flags & SJHIP_FLAG_FP32_STATE))
-    return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute, pieces): an fp32 state does not survive a checkpoint of 16-bit storage");
   rc = check_levels("backward(recompute, pieces)", neuron, *p, true);
   if (rc != SJHIP_OK) return rc;
   if (neuron == SJHIP_NEURON_PLIF) {

@@ -237,6 +237,28 @@ __device__ __forceinline__ void load_state(const void *p, int64_t col, bool broa
   }
 }
 
+// The same with the source given as the kernels' `v_init_broadcast` field: 0 = [N] in the storage dtype, 1 = one stored
+// element for all, kStateF32 = [N] in fp32 (a checkpoint of a state that is kept in fp32 beside 16-bit storage).
+constexpr int kStateF32 = 2;
+template <typename S, bool VECTOR, bool NT, typename NUM, int V>
+__device__ __forceinline__ void load_state_from(const void *p, int64_t col, int source, NUM (&v)[V]) {
+  if (source == kStateF32) {
+    const float *q = static_cast<const float *>(p) + col;
+    if constexpr (VECTOR && V % 4 == 0) {
+#pragma unroll
+      for (int i = 0; i < V / 4; ++i) {
+        const f32x4 w = stream_load<NT>(reinterpret_cast<const f32x4 *>(q) + i);
+        v[4 * i] = (NUM)w.x; v[4 * i + 1] = (NUM)w.y; v[4 * i + 2] = (NUM)w.z; v[4 * i + 3] = (NUM)w.w;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < V; ++j) v[j] = (NUM)q[j];
+    }
+    return;
+  }
+  load_state<S, VECTOR, NT>(p, col, source != 0, v);
+}
+
 // ----------------------------------------------------------------------------------------------
 // Host-side services (defined in sjhip_api.hip).
 // ----------------------------------------------------------------------------------------------
@@ -350,7 +372,10 @@ struct PieceArgs {
   void *checkpoints;
   int64_t chunk;
   int64_t pieces;
+  int checkpoints_f32;  // the checkpoints hold fp32 (16-bit storage whose state is kept in fp32)
 };
+// whether a checkpoint of the state is an fp32 row rather than one in the storage dtype
+inline bool checkpoints_are_f32(int dtype, uint32_t flags) { return dtype != SJHIP_F32 && (flags & SJHIP_FLAG_FP32_STATE) != 0; }
 
 // Launchers (one per translation unit).
 int launch_forward(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T, int64_t N,

@@ -336,6 +336,42 @@ def test_long_sequences_replayed_in_pieces_equal_the_saved_h_route(cls, T, store
         torch.testing.assert_close(results[0][4], results[1][4], rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("cls", [neuron.IFNode, neuron.LIFNode, neuron.ParametricLIFNode])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=lambda v: str(v).replace("torch.", ""))
+@pytest.mark.parametrize("T", [64, 100])
+def test_long_16_bit_sequences_with_fp32_state_are_replayed_in_pieces(cls, dtype, T, monkeypatch):
+    """16-bit storage with the state kept in fp32: the checkpoints are fp32, so the forward in pieces equals the plain
+    forward bit for bit, and the backward (which replays the unrounded h) is the same at two piece lengths; the PLIF
+    sum is added in another order."""
+    from spikingjelly_amd.activation_based.hip_kernel import neuron_kernel as K
+
+    monkeypatch.setattr(configure, "hip_half_precision_mode", "fp32_state")
+    x = seeded_randn((T, 2, 512), 43, 0.4, 1.0).to(dtype).cuda()
+    gs = seeded_randn((T, 2, 512), 44).to(dtype).cuda()
+    gv = seeded_randn((2, 512), 45, 0.0, 0.2).to(dtype).cuda()
+    v0 = seeded_randn((2, 512), 46, 0.0, 0.3).to(dtype).cuda()
+    pieces = []
+    real = K._run_backward
+    monkeypatch.setattr(K, "_run_backward", lambda *a, **k: (pieces.append(a[17]), real(*a, **k))[1])
+    results = []
+    for chunk in (16, 32, 0):
+        monkeypatch.setattr(configure, "hip_replay_chunk", chunk)
+        node = cls(step_mode="m", backend="hip", surrogate_function=surrogate.ATan()).cuda()
+        vi = v0.clone().requires_grad_()
+        node.v = vi
+        xi = x.clone().requires_grad_()
+        s = node(xi)
+        ((s * gs).sum() + (node.v * gv).sum()).backward()
+        results.append((s.detach(), node.v.detach(), xi.grad, vi.grad, node.w.grad if hasattr(node, "w") else None))
+    assert pieces == [16, 32, 0]
+    for other in results[1:]:
+        assert bits_equal(results[0][0], other[0]) and bits_equal(results[0][1], other[1])
+    assert bits_equal(results[0][2], results[1][2]) and bits_equal(results[0][3], results[1][3])
+    assert not torch.isnan(results[0][2].float()).any() and float(results[0][2].float().abs().sum()) > 0
+    if results[0][4] is not None:
+        torch.testing.assert_close(results[0][4], results[1][4], rtol=1e-4, atol=1e-5)
+
+
 def test_long_sequence_in_pieces_matches_the_torch_backend():
     x = seeded_randn((70, 3, 64), 37, 0.4, 1.0)
     gs = seeded_randn((70, 3, 64), 38)

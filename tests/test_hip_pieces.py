@@ -12,6 +12,8 @@ another order.  fp32 is also checked against the oracle.
 
 import ctypes
 
+import numpy as np
+
 import pytest
 import torch
 
@@ -65,7 +67,9 @@ def _forward_pieces(L, c, chunk, with_v_seq=True):
     pieces = lib.sjhip_replay_pieces(c["T"], chunk)
     s, vl = torch.empty_like(c["x"]), torch.full_like(c["v0"], float("nan"))
     v = torch.empty_like(c["x"]) if with_v_seq else None
-    ck = torch.full((max(pieces - 1, 1), c["N"]), float("nan"), dtype=c["dtype"], device=c["x"].device)
+    # a state kept in fp32 beside 16-bit storage is checkpointed in fp32
+    ck_dtype = torch.float32 if c["p"].flags & L.FLAG_FP32_STATE else c["dtype"]
+    ck = torch.full((max(pieces - 1, 1), c["N"]), float("nan"), dtype=ck_dtype, device=c["x"].device)
     L.check(lib.sjhip_neuron_forward_pieces(c["neuron"], L.dtype_id(c["dtype"]), ctypes.byref(c["p"]), c["T"], c["N"], chunk,
                                             c["x"].data_ptr(), c["v0"].data_ptr(), _kd(L, c), s.data_ptr(),
                                             v.data_ptr() if with_v_seq else None, vl.data_ptr(), ck.data_ptr(),
@@ -167,6 +171,75 @@ def test_pieces_equal_whole_forward_and_piecewise_backward(L, dtype, neuron_name
             assert float(got[2].item()) == pytest.approx(ref[2], rel=1e-3 if dtype != torch.float32 else 1e-5, abs=1e-3)
 
 
+def _backward_whole_replay(L, c, with_gv):
+    """sjhip_neuron_backward_recompute over the whole sequence (it holds every step's h on chip, so T is bounded)."""
+    gx, gv0 = torch.full_like(c["x"], float("nan")), torch.full_like(c["v0"], float("nan"))
+    gk, ws = _plif_buffers(L, c)
+    L.check(L.load().sjhip_neuron_backward_recompute(
+        c["neuron"], L.dtype_id(c["dtype"]), ctypes.byref(c["p"]), c["T"], c["N"], c["x"].data_ptr(), c["v0"].data_ptr(), _kd(L, c),
+        c["gs"].data_ptr(), c["gv"].data_ptr() if with_gv else None, c["gl"].data_ptr(), gx.data_ptr(), gv0.data_ptr(),
+        L.ptr(gk), L.ptr(ws), c["stream"]), "backward_recompute")
+    return gx, gv0, (float(gk.item()) if gk is not None else 0.0)
+
+
+def _fp32_state_oracle(c, kind, with_gv):
+    """float64 backward over the unrounded fp32 h of the mixed-precision forward (what a replay sees)."""
+    from oracle import bptt_oracle
+
+    k = {"if": 0.0, "lif": 0.5, "plif": c["k"]}[kind]
+    x, v0 = c["x"].cpu(), c["v0"].cpu()
+    _, _, _, raw_h = no.multi_step_mixed_precision(kind, x.float(), v0.float(), c["dtype"], k, True, 1.0, 0.0, return_raw_h=True)
+    h64 = raw_h.double().numpy()
+    s64 = (h64 >= 1.0).astype(np.float64)
+    v64 = (1 - s64) * h64
+    v_prev = np.concatenate([v0.double().numpy()[None], v64[:-1]])
+    x_implied = (h64 - v_prev) / k + v_prev if k else None
+    sgp = lambda z: no.surrogate_grad("atan", torch.from_numpy(np.ascontiguousarray(z)), 2.0).numpy()
+    return bptt_oracle.bptt(kind, h64, s64, sgp, c["gs"].cpu().double().numpy(),
+                            c["gv"].cpu().double().numpy() if with_gv else None, c["gl"].cpu().double().numpy(), k, True, 1.0,
+                            0.0, False, v_prev, x_implied)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=lambda v: str(v).replace("torch.", ""))
+@pytest.mark.parametrize("neuron_name", ["IF", "LIF", "PLIF"])
+@pytest.mark.parametrize("T,chunk,other", [(44, 16, 22), (64, 16, 32), (30, 10, 0)])
+def test_pieces_with_16_bit_storage_and_fp32_state(L, dtype, neuron_name, T, chunk, other):
+    """16-bit storage with the state kept in fp32 (``SJHIP_FLAG_FP32_STATE``): the checkpoints are fp32 rows, so the
+    pieces reproduce the whole forward bit for bit (a checkpoint in the storage dtype would round the state).  The
+    backward replays the unrounded h, as the whole-sequence replay does (the route over a saved ``h_seq`` sees h
+    rounded, and decides a few spikes differently): it equals that replay bit for bit where the sequence fits one,
+    equals itself at another piece length, and agrees with the float64 recurrence over the unrounded h."""
+    neuron = getattr(L, "NEURON_" + neuron_name)
+    flags = L.FLAG_DECAY_INPUT | L.FLAG_FP32_STATE
+    c = _case(L, neuron, dtype, T, 8 * 300, flags, 300 + T)
+    s, v, vl = _forward_whole(L, c)
+    sp, vp, vlp, ck = _forward_pieces(L, c, chunk)
+    torch.cuda.synchronize()
+    assert ck.dtype == torch.float32 and not torch.isnan(ck).any()
+    assert bits_equal(sp, s) and bits_equal(vp, v) and bits_equal(vlp, vl)
+    for j in range(ck.shape[0]):  # the stored v_seq row is the checkpoint rounded once
+        assert bits_equal(ck[j].to(dtype), v[(j + 1) * chunk - 1]), f"checkpoint {j}"
+    assert float((ck != ck.to(dtype).float()).float().mean()) > 0.2  # and the checkpoint really holds more bits
+    for with_gv in (True, False):
+        got = _backward_pieces(L, c, chunk, ck, with_gv)
+        if other:
+            ck2 = _forward_pieces(L, c, other)[3]
+            ref = _backward_pieces(L, c, other, ck2, with_gv)
+            ref = (ref[0], ref[1], float(ref[2].item()) if ref[2] is not None else 0.0)
+        else:
+            ref = _backward_whole_replay(L, c, with_gv)
+        torch.cuda.synchronize()
+        assert not torch.isnan(got[0].float()).any() and not torch.isnan(got[1].float()).any()
+        assert bits_equal(got[0], ref[0]), "grad_x_seq"
+        assert bits_equal(got[1], ref[1]), "grad_v_init"
+        egx, egv0, egk = _fp32_state_oracle(c, neuron_name.lower(), with_gv)
+        torch.testing.assert_close(got[0].cpu().double(), torch.from_numpy(egx), rtol=1e-2, atol=1e-3)
+        torch.testing.assert_close(got[1].cpu().double(), torch.from_numpy(egv0), rtol=1e-2, atol=1e-3)
+        if neuron == L.NEURON_PLIF:
+            assert float(got[2].item()) == pytest.approx(ref[2], rel=1e-4, abs=1e-3)
+            assert float(got[2].item()) == pytest.approx(egk, rel=1e-3, abs=1e-2)
+
+
 @pytest.mark.parametrize("neuron_name,kind", [("IF", "if"), ("LIF", "lif")])
 def test_pieces_against_the_oracle(L, neuron_name, kind):
     T, N, chunk = 50, 4 * 257, 16
@@ -197,13 +270,6 @@ def test_pieces_argument_checks(L):
     assert lib.sjhip_neuron_backward_recompute_pieces(*head[:3], 400, 64, 200, c["x"].data_ptr(), c["v0"].data_ptr(), None,
                                                       ck.data_ptr(), c["gs"].data_ptr(), None, None, gx.data_ptr(), None, None,
                                                       None, c["stream"]) == ERR_UNSUPPORTED
-    # an fp32 state over 16-bit storage would be rounded at every checkpoint
-    c = _case(L, L.NEURON_LIF, torch.float16, 40, 64, L.FLAG_DECAY_INPUT | L.FLAG_FP32_STATE, 3)
-    ck16 = torch.empty((2, 64), dtype=torch.float16, device="cuda:0")
-    s16, vl16 = torch.empty_like(c["x"]), torch.empty_like(c["v0"])
-    assert lib.sjhip_neuron_forward_pieces(L.NEURON_LIF, L.dtype_id(torch.float16), ctypes.byref(c["p"]), 40, 64, 16,
-                                           c["x"].data_ptr(), c["v0"].data_ptr(), None, s16.data_ptr(), None, vl16.data_ptr(),
-                                           ck16.data_ptr(), c["stream"]) == ERR_UNSUPPORTED
     assert lib.sjhip_replay_pieces(40, 16) == 3 and lib.sjhip_replay_pieces(16, 16) == 1 and lib.sjhip_replay_pieces(0, 16) == 0
 
 
