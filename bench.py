@@ -409,23 +409,26 @@ def other_workload(args) -> int:
         from spikingjelly_amd.activation_based.hip_kernel import conv_bn_lif as CB
 
         S, Cin, Cout, tokens = 256, 384, 1152, 196
-        terms = args.terms
+        terms = args.terms if args.conv_split == "bf16" else CB.F16 | 2
         x = randn((S, Cin, tokens), 1, 0.0, 1.0, torch.float32)
         dy = randn((S, Cout, tokens), 2, 0.0, 1.0, torch.float32)
         w = randn((Cout, Cin), 3, 0.0, 0.05, torch.float32)
 
-        def step():
-            CB.pw_gemm(CB.split_weight(w, False), terms, Cout, Cin, x, terms)
-            CB.pw_gemm(CB.split_weight(w, True), terms, Cin, Cout, dy, terms)
-            CB.pw_grad_weight(dy, terms, x, terms)
+        def step():  # as the fused block calls them: with fp16 terms one pass per tensor finds its scale
+            x_amax = CB.amax(x) if terms & CB.F16 else None
+            CB.pw_gemm(CB.split_weight(w, False, terms), terms, Cout, Cin, x, terms, False, x_amax)
+            dy_amax = CB.amax(dy) if terms & CB.F16 else None
+            CB.pw_gemm(CB.split_weight(w, True, terms), terms, Cin, Cout, dy, terms, False, dy_amax)
+            CB.pw_grad_weight(dy, terms, x, terms, dy_amax, x_amax)
 
         elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
         g_ms, d_ms = _kernel_ms(L, L.KC_PW_GEMM), _kernel_ms(L, L.KC_PW_GRAD_WEIGHT)
         flop = 2.0 * S * Cin * Cout * tokens                      # of one GEMM, counted once per fp32 product
-        products = {3: 6, 2: 3, 1: 1}[terms]                      # bf16 matrix-core products per fp32 product
+        products = {3: 6, 2: 3, 1: 1, CB.F16 | 2: 3}[terms]      # 16-bit matrix-core products per fp32 product
+        split = "2 fp16 terms per scaled operand" if terms & CB.F16 else f"{terms} bf16 terms per operand"
         _emit(args, "fp32-equivalent TFLOP/s of the kernel-size-1 convolution GEMMs, qkv of configs[4], 1 MI355X", "TFLOP/s",
-              3 * flop / (elapsed / args.steps) / 1e12, elapsed, "bf16",
-              {"workload": f"Y = W X, dX = W^T dY, dW = dY X^T for W [1152, 384], X [256, 384, 196] fp32, {terms} bf16 terms per operand"},
+              3 * flop / (elapsed / args.steps) / 1e12, elapsed, "f16" if terms & CB.F16 else "bf16",
+              {"workload": f"Y = W X, dX = W^T dY, dW = dY X^T for W [1152, 384], X [256, 384, 196] fp32, {split}"},
               {"bound": "mfma", "achieved": products * flop / (g_ms * 1e-3) / 1e12, "peak": 2500.0, "unit": "TFLOP/s",
                "frac": products * flop / (g_ms * 1e-3) / 1e12 / 2500.0, "traffic": None, "kernel": "pw_gemm",
                "kernel_ms": g_ms, "grad_weight_ms": d_ms,
@@ -436,6 +439,7 @@ def other_workload(args) -> int:
     if args.workload == "config5":
         T, B, D, H, tokens = 4, 64, args.dim, 12, 196
         configure.hip_fuse_ssa_lif = bool(args.fuse_ssa_lif)
+        configure.hip_conv_split, configure.hip_conv_terms = args.conv_split, args.terms
         torch.manual_seed(1005)
         block = layer.SpikingSelfAttention(D, H, backend="hip").to(dev)
         x = randn((T, B, D, tokens), 1105, 0.0, 1.0, torch.float32).requires_grad_()
@@ -458,9 +462,10 @@ def other_workload(args) -> int:
         bytes_f = 3 * n // 8 + 4 * n              # bits read, out written
         bytes_b = 3 * n // 8 + 4 * n + 12 * n     # bits and grad_out read, dq / dk / dv written
         _emit(args, f"tokens/sec spiking self-attention block fwd+bwd, T=4 B=64 N=196 D={D} 12 heads, 1 MI355X",
-              "tokens/s", T * B * tokens / (elapsed / args.steps), elapsed, "bf16",
+              "tokens/s", T * B * tokens / (elapsed / args.steps), elapsed, args.conv_split,
               {"workload": f"configs[4]: SpikingSelfAttention({D}, 12, backend='hip'), x [4,64,{D},196] fp32 ~N(0,1), "
-                           f"channels per head = {cph} (dim // heads, as the reference computes it)"},
+                           f"channels per head = {cph} (dim // heads, as the reference computes it); convolution GEMMs on "
+                           f"{'two fp16' if args.conv_split == 'f16' else str(args.terms) + ' bf16'} terms per fp32 operand"},
               {"bound": "hbm", "achieved": bytes_b / (sb * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                "frac": bytes_b / (sb * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "ssa_backward",
                "kernel_ms": sb, "algorithmic_bytes": bytes_b,
@@ -480,7 +485,10 @@ def main() -> int:
     ap.add_argument("--cpu-sample-neurons", type=int, default=1 << 23)
     ap.add_argument("--cpu-repeats", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--terms", type=int, default=3, choices=[1, 2, 3], help="pwconv workload: bf16 terms per fp32 operand")
+    ap.add_argument("--terms", type=int, default=3, choices=[1, 2, 3],
+                    help="pwconv and config5 workloads with --conv-split bf16: bf16 terms per fp32 operand")
+    ap.add_argument("--conv-split", default="f16", choices=["f16", "bf16"],
+                    help="pwconv and config5 workloads: how fp32 operands of the convolution GEMMs are split for the matrix cores")
     ap.add_argument("--dim", type=int, default=384, choices=[384, 768],
                     help="config5 workload: embedding width (12 heads of dim // 12 channels: 32, or 64 with 768)")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",

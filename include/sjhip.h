@@ -497,6 +497,43 @@ int sjhip_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int 
                              int64_t L, float *dw, float *workspace, void *stream);
 
 /*
+ * The same three GEMMs (same reference lines: layer/attention.py:310-329, model/spikformer.py:85-99) with the fp32
+ * operands split into two fp16 terms and the three products hi*hi, hi*lo, lo*hi on v_mfma_f32_32x32x16_f16: half the
+ * matrix-core work of the three-term bf16 split at the same accuracy class.  fp16 has 11 significant bits but a narrow
+ * exponent range, so every operand is scaled by a power of two first (exact) and the scales are taken out of the result
+ * (exact): weights per row of A, inside sjhip_pwconv_split_weight_f16; activations and gradients per tensor, by the power
+ * of two that takes the tensor's largest magnitude `amax` into [2^14, 2^15) (1 for a zero, subnormal or non-finite amax),
+ * which the kernels derive from a device buffer of SJHIP_PW_AMAX_FLOATS non-negative floats whose maximum is amax
+ * (several words, so that the blocks that fold their maxima into it do not meet on one address).  An element above 2^-16 of amax is represented to 2^-23
+ * relative or better, a smaller one to 2^-39 of amax; the dropped product lo*lo is below 2^-22 of hi*hi.  Measured
+ * against float64 on operands whose rows span four decades: 2^-23 of sum |a||b| (three bf16 terms: 2^-26; an fp32 dot
+ * product of 384 terms: 2^-20).  An operand that fp16 holds exactly (spikes, integers up to 2048) takes one term and no
+ * scale (terms = 1, amax = NULL).
+ *
+ *   sjhip_pwconv_split_weight_f16  planes: an opaque buffer of sjhip_pwconv_planes_elems(rows, cols) 2-byte elements,
+ *                                  16-byte aligned (two fp16 planes in the tile order of sjhip_pwconv_split_weight,
+ *                                  then the inverse row scales); amax_reset: NULL, or an amax buffer that the
+ *                                  launch also sets to zero (that of the activations the planes will multiply, so
+ *                                  that no launch is spent on clearing it)
+ *   sjhip_pwconv_amax              folds max |x| over the n elements of x (NaNs ignored) into amax[SJHIP_PW_AMAX_FLOATS]:
+ *                                  afterwards max(amax[]) is the larger of what it was and max |x|; all zero before
+ *                                  the first call for a tensor; one launch
+ *   sjhip_pwconv_gemm_f16          sjhip_pwconv_gemm / sjhip_pwconv_gemm_stats (partial != NULL) on fp16 planes;
+ *                                  b_terms 2 with the b_amax buffer of b (a larger maximum is safe, a smaller one is
+ *                                  not), or 1 with NULL
+ *   sjhip_pwconv_grad_weight_f16   sjhip_pwconv_grad_weight with two terms of dy (dy_amax) and x_terms of x
+ */
+#define SJHIP_PW_F16 16          /* internal term code of an fp16 operand: SJHIP_PW_F16 | terms */
+#define SJHIP_PW_AMAX_FLOATS 256
+int sjhip_pwconv_split_weight_f16(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, float *amax_reset,
+                                  void *stream);
+int sjhip_pwconv_amax(const float *x, int64_t n, float *amax, void *stream);
+int sjhip_pwconv_gemm_f16(const uint16_t *a_planes, int64_t M, int64_t K, const float *b, int b_terms, const float *b_amax,
+                          int64_t S, int64_t L, float *c, float *partial, void *stream);
+int sjhip_pwconv_grad_weight_f16(const float *dy, const float *dy_amax, const float *x, int x_terms, const float *x_amax,
+                                 int64_t S, int64_t M, int64_t N, int64_t L, float *dw, float *workspace, void *stream);
+
+/*
  * Batch normalisation fused with the multi-step IF / LIF neuron behind it, for fp32 activations [T][B][C][L]
  * (L contiguous, a multiple of 4).  Stands in for nn.BatchNorm1d / nn.BatchNorm2d followed by LIFNode in the reference's
  * SpikingSelfAttention (layer/attention.py:314-329, 370-384) and SpikformerConv2dBNLIF (model/spikformer.py:196-212),
@@ -507,7 +544,8 @@ int sjhip_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int 
  *                       (evaluation), from running_mean / running_var; writes the affine map z = y scale + shift
  *                       (scale = gamma / sqrt(var + eps), shift = beta - mean scale; gamma / beta may be NULL = 1 / 0),
  *                       mean and invstd (kept for the backward), and in training updates running_mean / running_var in
- *                       place with `momentum` (unbiased variance), when they are given
+ *                       place with `momentum` (unbiased variance), when they are given, and adds 1 to *batches_tracked
+ *                       (nn.BatchNorm's num_batches_tracked, an int64 on the device), when that is given
  *   sjhip_bn_lif_forward   z = y scale_c + shift_c, then charge / fire / reset over the T steps (same arithmetic and
  *                       params as sjhip_neuron_forward; neuron IF or LIF); spikes go to spike_seq [T][B][C][L] (fp32) or
  *                       bit-packed to spike_bits (the layout of sjhip_bit_pack; B*C*L must be a multiple of 8): exactly
@@ -516,17 +554,18 @@ int sjhip_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int 
  *                       grad_spike_seq and (optionally) grad_v_last, writes grad_z = dL/dz [T][B][C][L], grad_v_init
  *                       (or NULL) and partial[b][c] = (sum g, sum g y) over the row and all steps
  *   sjhip_bn_backward_finalize   dgamma, dbeta (either may be NULL) and coef [3][C] = (p, q, r) of dy = p g + q y + r;
- *                       training != 0: batch statistics took part in the forward, else q = r = 0
+ *                       training != 0: batch statistics took part in the forward, else q = r = 0; amax_reset: NULL, or
+ *                       the amax buffer (SJHIP_PW_AMAX_FLOATS floats) of a following sjhip_bn_grad_input_amax, set to zero
  *   sjhip_bn_grad_input    dy = p_c g + q_c y + r_c over [S][C][L]; dy may be g
  */
 int sjhip_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, void *stream);
 int sjhip_bn_finalize(const float *partial, int64_t S, int64_t C, int64_t L, const float *gamma, const float *beta, float eps,
                       float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
-                      float *invstd, void *stream);
+                      float *invstd, int64_t *batches_tracked, void *stream);
 /* the same from partial [rows][C][2] that sum over `count` elements per channel (training mode only: partial != NULL) */
 int sjhip_bn_finalize_rows(const float *partial, int64_t rows, int64_t count, int64_t C, const float *gamma, const float *beta,
                            float eps, float momentum, float *running_mean, float *running_var, float *scale, float *shift,
-                           float *mean, float *invstd, void *stream);
+                           float *mean, float *invstd, int64_t *batches_tracked, void *stream);
 int sjhip_bn_lif_forward(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
                          const float *scale, const float *shift, const float *v_init, float *spike_seq, uint8_t *spike_bits,
                          float *v_last, void *stream);
@@ -534,8 +573,14 @@ int sjhip_bn_lif_backward(int neuron, const sjhip_neuron_params *p, int64_t T, i
                           const float *scale, const float *shift, const float *v_init, const float *grad_spike_seq,
                           const float *grad_v_last, float *grad_z, float *grad_v_init, float *partial, void *stream);
 int sjhip_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64_t C, int64_t L, int training, const float *gamma,
-                               const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef, void *stream);
+                               const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef, float *amax_reset,
+                               void *stream);
 int sjhip_bn_grad_input(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy, void *stream);
+/* sjhip_bn_grad_input that also folds max |dy| into amax as sjhip_pwconv_amax(dy) would (same contract:
+ * SJHIP_PW_AMAX_FLOATS floats, zero before the call): the fp16 GEMMs that consume dy (the two gradients of the convolution in front of the
+ * batch norm, layer/attention.py:314-319 run backwards) then need no pass of their own over it. */
+int sjhip_bn_grad_input_amax(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy,
+                             float *amax, void *stream);
 
 /*
  * Launch tuning (process-wide, read at launch).  Keys: "fwd_block" / "bwd_block" = work-items per

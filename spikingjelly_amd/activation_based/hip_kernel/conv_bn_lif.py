@@ -6,9 +6,10 @@ The block ``SeqToANNContainer(Conv1d(k=1, bias=False), BatchNorm1d) -> LIFNode``
 layout transposes around them), batch norm and the neuron as separate operators.  Here, for fp32 ``[T, B, C, L]``
 tensors (``L`` the flattened positions, a multiple of 4):
 
-* the convolution and its two gradients are GEMMs on the bf16 matrix cores with the fp32 operands split into up to
-  three bf16 terms (``csrc/pwconv.hip``; ``configure.hip_conv_terms`` = 3 keeps fp32 accuracy, 2 and 1 trade it for speed;
-  an input that is known to be spikes needs one term);
+* the convolution and its two gradients are GEMMs on the 16-bit matrix cores with the fp32 operands split into terms
+  (``csrc/pwconv.hip``): two fp16 terms of power-of-two scaled operands (``configure.hip_conv_split = "f16"``, the
+  default: three products, fp32 accuracy) or up to three bf16 terms (``"bf16"``; ``configure.hip_conv_terms`` = 3 keeps
+  fp32 accuracy with six products, 2 and 1 trade it for speed); an input that is known to be spikes needs one term;
 * batch norm and the neuron are two passes over the convolution output (``csrc/bn_lif.hip``): per-channel statistics,
   then normalise + charge + fire + reset over the T steps in registers, spikes written dense or bit-packed; the
   normalised tensor never exists.  The backward replays the neuron from the convolution output.
@@ -31,16 +32,31 @@ from . import library as L
 from . import neuron_kernel as K
 
 __all__ = ["supported", "bn_lif", "conv_bn_lif", "conv_bn_lif_ssa", "conv_bn_lif_ssa_lif", "split_weight", "pw_gemm",
-           "pw_grad_weight"]
+           "pw_grad_weight", "amax", "F16"]
 
 MAX_REPLAY_STEPS = 16  # the backward replays the neuron with h of every step in registers
 
 
+F16 = 16  # term code of an fp16 operand: F16 | 2 (hi and lo of a scaled value) or F16 | 1 (exact in fp16)
+_AMAX_FLOATS = 256  # SJHIP_PW_AMAX_FLOATS
+
+
 def _terms() -> int:
+    """Term code of an operand with arbitrary fp32 values."""
+    mode = getattr(configure, "hip_conv_split", "f16")
+    if mode == "f16":
+        return F16 | 2
+    if mode != "bf16":
+        raise ValueError(f"configure.hip_conv_split must be 'f16' or 'bf16', got {mode!r}")
     t = int(getattr(configure, "hip_conv_terms", 3))
     if t not in (1, 2, 3):
         raise ValueError(f"configure.hip_conv_terms must be 1, 2 or 3, got {t}")
     return t
+
+
+def _exact(terms: int) -> int:
+    """Term code, in the format of ``terms``, of an operand that 16-bit floats hold exactly (spikes)."""
+    return (terms & F16) | 1
 
 
 def supported(x_seq: torch.Tensor, need_grad: bool) -> bool:
@@ -57,32 +73,62 @@ def _stream(t: torch.Tensor) -> int:
 # ------------------------------------------------------------------------------------------------
 # launch helpers (no autograd)
 # ------------------------------------------------------------------------------------------------
-def split_weight(weight: torch.Tensor, transpose: bool) -> torch.Tensor:
-    """bf16 term planes ``[3, rows_pad, cols_pad]`` of ``weight [Cout, Cin]`` (or of its transpose): the A operand of
-    ``pw_gemm``."""
+def split_weight(weight: torch.Tensor, transpose: bool, terms: int = 3, amax_reset: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Term planes of ``weight [Cout, Cin]`` (or of its transpose), the A operand of ``pw_gemm``: bf16 planes
+    ``[3, rows_pad, cols_pad]``, or with ``terms & F16`` two fp16 planes of the rows scaled by powers of two, followed by
+    the inverse scales (an opaque buffer either way).  ``amax_reset`` (fp16 terms): an ``amax`` buffer that the launch
+    clears on the way."""
     rows, cols = weight.shape
     w = L.aligned16(weight.detach().to(torch.float32))
     planes = torch.empty(L.load().sjhip_pwconv_planes_elems(cols if transpose else rows, rows if transpose else cols),
                          dtype=torch.bfloat16, device=weight.device)
     with torch.cuda.device(weight.device):
-        rc = L.load().sjhip_pwconv_split_weight(w.data_ptr(), rows, cols, 1 if transpose else 0, planes.data_ptr(), _stream(w))
+        if terms & F16:
+            rc = L.load().sjhip_pwconv_split_weight_f16(w.data_ptr(), rows, cols, 1 if transpose else 0, planes.data_ptr(),
+                                                        L.ptr(amax_reset), _stream(w))
+        else:
+            rc = L.load().sjhip_pwconv_split_weight(w.data_ptr(), rows, cols, 1 if transpose else 0, planes.data_ptr(), _stream(w))
     L.check(rc, "pwconv_split_weight")
     return planes
 
 
-def pw_gemm(planes: torch.Tensor, a_terms: int, M: int, Kdim: int, b: torch.Tensor, b_terms: int, stats: bool = False):
+def amax(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The largest magnitude in ``x`` as the maximum of a small device buffer (several words, so that the blocks that
+    write them do not meet on one address): what the fp16 split of a tensor of arbitrary values is scaled by (the
+    kernels turn it into a power of two).  ``out``: a buffer that already holds zeros (or an earlier maximum to keep)."""
+    x = L.aligned16(x)
+    if out is None:
+        out = torch.zeros((_AMAX_FLOATS,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = L.load().sjhip_pwconv_amax(x.data_ptr(), x.numel(), out.data_ptr(), _stream(x))
+    L.check(rc, "pwconv_amax")
+    return out
+
+
+def pw_gemm(planes: torch.Tensor, a_terms: int, M: int, Kdim: int, b: torch.Tensor, b_terms: int, stats: bool = False,
+            b_amax: Optional[torch.Tensor] = None):
     """``c[s] = A b[s]`` for ``b [S, K, L]`` -> ``c [S, M, L]``.  With ``stats`` the result is ``(c, partial)``:
     ``partial [rows, M, 2]`` holds sums and sums of squares of every row of ``c`` over groups of its columns, the input
-    of ``_bn_map``."""
+    of ``_bn_map``.  fp16 terms (``a_terms & F16``, planes from ``split_weight(..., terms)``): ``b_amax`` is
+    ``amax(b)``, computed here when not given."""
     S, Kb, Lp = b.shape
     assert Kb == Kdim
     b = L.aligned16(b)
     c = torch.empty((S, M, Lp), dtype=torch.float32, device=b.device)
     lib = L.load()
+    partial = None
     with torch.cuda.device(b.device):
         if stats:
             rows = lib.sjhip_pwconv_gemm_stats_rows(Kdim, S, Lp)
             partial = torch.empty((rows, M, 2), dtype=torch.float32, device=b.device)
+        if a_terms & F16:
+            if (a_terms & ~F16) != 2 or not b_terms & F16:
+                raise ValueError(f"fp16 weight planes hold two terms and take fp16 activation terms, got {a_terms}, {b_terms}")
+            if (b_terms & ~F16) == 2 and b_amax is None:
+                b_amax = amax(b)
+            rc = lib.sjhip_pwconv_gemm_f16(planes.data_ptr(), M, Kdim, b.data_ptr(), b_terms & ~F16, L.ptr(b_amax), S, Lp,
+                                           c.data_ptr(), L.ptr(partial), _stream(b))
+        elif stats:
             rc = lib.sjhip_pwconv_gemm_stats(planes.data_ptr(), a_terms, M, Kdim, b.data_ptr(), b_terms, S, Lp, c.data_ptr(),
                                              partial.data_ptr(), _stream(b))
         else:
@@ -91,8 +137,10 @@ def pw_gemm(planes: torch.Tensor, a_terms: int, M: int, Kdim: int, b: torch.Tens
     return (c, partial) if stats else c
 
 
-def pw_grad_weight(dy: torch.Tensor, dy_terms: int, x: torch.Tensor, x_terms: int) -> torch.Tensor:
-    """``dw[m, n] = sum_{s, l} dy[s, m, l] x[s, n, l]``."""
+def pw_grad_weight(dy: torch.Tensor, dy_terms: int, x: torch.Tensor, x_terms: int, dy_amax: Optional[torch.Tensor] = None,
+                   x_amax: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``dw[m, n] = sum_{s, l} dy[s, m, l] x[s, n, l]``; with fp16 terms the largest magnitudes (``amax``) are computed
+    here when not given."""
     S, M, Lp = dy.shape
     N = x.shape[1]
     dy, x = L.aligned16(dy), L.aligned16(x)
@@ -100,17 +148,28 @@ def pw_grad_weight(dy: torch.Tensor, dy_terms: int, x: torch.Tensor, x_terms: in
     ws = torch.empty(lib.sjhip_pwconv_grad_weight_workspace_floats(M, N, S), dtype=torch.float32, device=dy.device)
     dw = torch.empty((M, N), dtype=torch.float32, device=dy.device)
     with torch.cuda.device(dy.device):
-        rc = lib.sjhip_pwconv_grad_weight(dy.data_ptr(), dy_terms, x.data_ptr(), x_terms, S, M, N, Lp, dw.data_ptr(),
-                                          ws.data_ptr(), _stream(dy))
+        if dy_terms & F16:
+            if (dy_terms & ~F16) != 2 or not x_terms & F16:
+                raise ValueError(f"the fp16 weight gradient takes two gradient terms and fp16 activation terms, got {dy_terms}, {x_terms}")
+            if dy_amax is None:
+                dy_amax = amax(dy)
+            if (x_terms & ~F16) == 2 and x_amax is None:
+                x_amax = amax(x)
+            rc = lib.sjhip_pwconv_grad_weight_f16(dy.data_ptr(), dy_amax.data_ptr(), x.data_ptr(), x_terms & ~F16, L.ptr(x_amax),
+                                                  S, M, N, Lp, dw.data_ptr(), ws.data_ptr(), _stream(dy))
+        else:
+            rc = lib.sjhip_pwconv_grad_weight(dy.data_ptr(), dy_terms, x.data_ptr(), x_terms, S, M, N, Lp, dw.data_ptr(),
+                                              ws.data_ptr(), _stream(dy))
     L.check(rc, "pwconv_grad_weight")
     return dw
 
 
 def _bn_map(y: torch.Tensor, gamma, beta, running_mean, running_var, batch_stats: bool, momentum: float, eps: float,
-            partial: Optional[torch.Tensor] = None):
+            partial: Optional[torch.Tensor] = None, tracked: Optional[torch.Tensor] = None):
     """Per-channel ``(scale, shift, mean, invstd)`` of ``z = y * scale + shift`` for ``y [S, C, L]``; with
     ``batch_stats`` from the statistics of ``y`` (and the running statistics, when given, are updated in place).
-    ``partial``: the sums the convolution left behind (``pw_gemm(..., stats=True)``), which save the pass over ``y``."""
+    ``partial``: the sums the convolution left behind (``pw_gemm(..., stats=True)``), which save the pass over ``y``.
+    ``tracked``: the batch norm's ``num_batches_tracked`` (int64, on the device), which the same launch increments."""
     S, C, Lp = y.shape
     lib = L.load()
     out = torch.empty((4, C), dtype=torch.float32, device=y.device)
@@ -118,7 +177,7 @@ def _bn_map(y: torch.Tensor, gamma, beta, running_mean, running_var, batch_stats
         if batch_stats and partial is not None:
             rc = lib.sjhip_bn_finalize_rows(partial.data_ptr(), partial.shape[0], S * Lp, C, L.ptr(gamma), L.ptr(beta), eps,
                                             momentum, L.ptr(running_mean), L.ptr(running_var), out[0].data_ptr(),
-                                            out[1].data_ptr(), out[2].data_ptr(), out[3].data_ptr(), _stream(y))
+                                            out[1].data_ptr(), out[2].data_ptr(), out[3].data_ptr(), L.ptr(tracked), _stream(y))
             L.check(rc, "bn_finalize_rows")
             return out
         partial = None
@@ -127,7 +186,7 @@ def _bn_map(y: torch.Tensor, gamma, beta, running_mean, running_var, batch_stats
             L.check(lib.sjhip_bn_stats(y.data_ptr(), S, C, Lp, partial.data_ptr(), _stream(y)), "bn_stats")
         rc = lib.sjhip_bn_finalize(L.ptr(partial), S, C, Lp, L.ptr(gamma), L.ptr(beta), eps, momentum, L.ptr(running_mean),
                                    L.ptr(running_var), out[0].data_ptr(), out[1].data_ptr(), out[2].data_ptr(),
-                                   out[3].data_ptr(), _stream(y))
+                                   out[3].data_ptr(), L.ptr(tracked), _stream(y))
     L.check(rc, "bn_finalize")
     return out
 
@@ -156,8 +215,10 @@ def _bn_lif_forward(y: torch.Tensor, bn_map: torch.Tensor, v_init: torch.Tensor,
 
 
 def _bn_lif_backward(y: torch.Tensor, bn_map: torch.Tensor, gamma, v_init: torch.Tensor, spec, batch_stats: bool,
-                     grad_spikes: Optional[torch.Tensor], grad_v_last: Optional[torch.Tensor], need_grad_v_init: bool):
-    """Returns ``(dy [T, B, C, L], dgamma [C], dbeta [C], grad_v_init or None)``."""
+                     grad_spikes: Optional[torch.Tensor], grad_v_last: Optional[torch.Tensor], need_grad_v_init: bool,
+                     want_amax: bool = False):
+    """Returns ``(dy [T, B, C, L], dgamma [C], dbeta [C], grad_v_init or None)``, and with ``want_amax`` a fifth element:
+    ``amax(dy)``, found by the kernel that writes ``dy``, when the convolution GEMMs run on fp16 terms (else None)."""
     T, B, C, Lp = y.shape
     lib = L.load()
     if grad_spikes is None:
@@ -176,49 +237,106 @@ def _bn_lif_backward(y: torch.Tensor, bn_map: torch.Tensor, gamma, v_init: torch
         L.check(lib.sjhip_bn_lif_backward(L.NEURON_LIF, ctypes.byref(params), T, B, C, Lp, y.data_ptr(), bn_map[0].data_ptr(),
                                           bn_map[1].data_ptr(), v_keep.data_ptr(), grad_spikes.data_ptr(), L.ptr(grad_v_last),
                                           g.data_ptr(), L.ptr(grad_v_init), partial.data_ptr(), stream), "bn_lif_backward")
+        dy_amax = None
+        if want_amax and _terms() & F16:  # (cleared by the launch that makes the coefficients, filled by the next one)
+            dy_amax = torch.empty((_AMAX_FLOATS,), dtype=torch.float32, device=y.device)
         L.check(lib.sjhip_bn_backward_finalize(partial.data_ptr(), T, B, C, Lp, 1 if batch_stats else 0, L.ptr(gamma),
                                                bn_map[2].data_ptr(), bn_map[3].data_ptr(), grads[0].data_ptr(),
-                                               grads[1].data_ptr(), grads[2].data_ptr(), stream), "bn_backward_finalize")
-        L.check(lib.sjhip_bn_grad_input(g.data_ptr(), y.data_ptr(), grads[2].data_ptr(), T * B, C, Lp, g.data_ptr(), stream),
-                "bn_grad_input")
+                                               grads[1].data_ptr(), grads[2].data_ptr(), L.ptr(dy_amax), stream),
+                "bn_backward_finalize")
+        if dy_amax is not None:
+            L.check(lib.sjhip_bn_grad_input_amax(g.data_ptr(), y.data_ptr(), grads[2].data_ptr(), T * B, C, Lp, g.data_ptr(),
+                                                 dy_amax.data_ptr(), stream), "bn_grad_input_amax")
+        else:
+            L.check(lib.sjhip_bn_grad_input(g.data_ptr(), y.data_ptr(), grads[2].data_ptr(), T * B, C, Lp, g.data_ptr(), stream),
+                    "bn_grad_input")
+    if want_amax:
+        return g, grads[0], grads[1], grad_v_init, dy_amax
     return g, grads[0], grads[1], grad_v_init
 
 
 # ------------------------------------------------------------------------------------------------
 # autograd
 # ------------------------------------------------------------------------------------------------
-# bn: (running_mean | None, running_var | None, batch_stats, momentum, eps)
+# bn: (running_mean | None, running_var | None, batch_stats, momentum, eps[, num_batches_tracked | None])
 # lif spec: (tau, v_threshold, v_reset, flags, sg_id, sg_alpha)
-def _conv_forward(x_seq, weight, x_exact, stats: bool = False):
-    """``y [T, B, Cout, L]``, and with ``stats`` the partial batch-norm sums of ``y`` as well."""
+def _bn_config(bn):
+    """The batch-norm tuple with its optional sixth element (the counter of batches, incremented by the launch that
+    updates the running statistics)."""
+    return tuple(bn) if len(bn) == 6 else (*bn, None)
+
+
+def _conv_forward(x_seq, weight, x_exact, stats: bool):
+    """``(y [T, B, Cout, L], partial batch-norm sums of y or None, amax(x_seq) or an empty tensor)``: the last is what the
+    fp16 split of a real-valued input was scaled by, which the weight gradient needs again."""
     T, B, Cin, Lp = x_seq.shape
     Cout = weight.shape[0]
     terms = _terms()
-    planes = split_weight(weight, False)
-    out = pw_gemm(planes, terms, Cout, Cin, x_seq.reshape(T * B, Cin, Lp), 1 if x_exact else terms, stats)
+    x3 = x_seq.reshape(T * B, Cin, Lp)
+    if terms & F16 and not x_exact:  # the split of the weights clears the buffer that the pass over x then fills
+        x_amax = torch.empty((_AMAX_FLOATS,), dtype=torch.float32, device=x_seq.device)
+        planes = split_weight(weight, False, terms, x_amax)
+        amax(x3, x_amax)
+    else:
+        x_amax = x_seq.new_empty((0,))
+        planes = split_weight(weight, False, terms)
+    out = pw_gemm(planes, terms, Cout, Cin, x3, _exact(terms) if x_exact else terms, stats, x_amax if x_amax.numel() else None)
     if stats:
-        return out[0].view(T, B, Cout, Lp), out[1]
-    return out.view(T, B, Cout, Lp)
+        return out[0].view(T, B, Cout, Lp), out[1], x_amax
+    return out.view(T, B, Cout, Lp), None, x_amax
 
 
-def _conv_backward(dy, x_seq, weight, x_exact, need_dx, need_dw):
+def _conv_backward(dy, x_seq, weight, x_exact, need_dx, need_dw, dy_amax=None, x_amax=None):
     T, B, Cin, Lp = x_seq.shape
     Cout = weight.shape[0]
     terms = _terms()
     dy3 = dy.view(T * B, Cout, Lp)
-    dw = pw_grad_weight(dy3, terms, x_seq.reshape(T * B, Cin, Lp), 1 if x_exact else terms) if need_dw else None
-    dx = None
+    if dy_amax is None and terms & F16 and (need_dw or need_dx):
+        dy_amax = amax(dy3)  # one pass for both uses of dy
+    if x_amax is not None and x_amax.numel() == 0:
+        x_amax = None  # the forward ran with an exact input or on bf16 terms (pw_grad_weight finds it if it is needed now)
+    x3 = x_seq.reshape(T * B, Cin, Lp)
+    x_terms = _exact(terms) if x_exact else terms
+    dw = dx = None
+    if need_dw and need_dx and getattr(configure, "hip_conv_overlap_gradients", True):
+        # The two gradients only share their inputs: the weight gradient runs on a second stream, so that the blocks of
+        # one kernel fill the compute units that the last, partly filled round of the other leaves idle.
+        main = torch.cuda.current_stream(dy.device)
+        side = _side_stream(dy.device)
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            dw = pw_grad_weight(dy3, terms, x3, x_terms, dy_amax, x_amax)
+        dx = pw_gemm(split_weight(weight, True, terms), terms, Cin, Cout, dy3, terms, False, dy_amax).view(T, B, Cin, Lp)
+        main.wait_stream(side)
+        dw.record_stream(main)
+        return dx, dw
+    if need_dw:
+        dw = pw_grad_weight(dy3, terms, x3, x_terms, dy_amax, x_amax)
     if need_dx:
-        dx = pw_gemm(split_weight(weight, True), terms, Cin, Cout, dy3, terms).view(T, B, Cin, Lp)
+        dx = pw_gemm(split_weight(weight, True, terms), terms, Cin, Cout, dy3, terms, False, dy_amax).view(T, B, Cin, Lp)
     return dx, dw
+
+
+_SIDE_STREAMS: dict = {}
+
+
+def _side_stream(device: torch.device) -> "torch.cuda.Stream":
+    """One more stream per device (default priority), made on first use."""
+    key = torch.device(device).index
+    if key is None:
+        key = torch.cuda.current_device()
+    stream = _SIDE_STREAMS.get(key)
+    if stream is None:
+        stream = _SIDE_STREAMS[key] = torch.cuda.Stream(device=key)
+    return stream
 
 
 class _BnLif(torch.autograd.Function):
     @staticmethod
     def forward(y, gamma, beta, v_init, bn, spec):
-        running_mean, running_var, batch_stats, momentum, eps = bn
+        running_mean, running_var, batch_stats, momentum, eps, tracked = _bn_config(bn)
         y = L.aligned16(y)
-        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps)
+        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, None, tracked)
         spikes, v_last = _bn_lif_forward(y, bn_map, v_init, spec, False)
         return spikes, v_last, bn_map
 
@@ -242,28 +360,28 @@ class _BnLif(torch.autograd.Function):
 class _ConvBnLif(torch.autograd.Function):
     @staticmethod
     def forward(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact):
-        running_mean, running_var, batch_stats, momentum, eps = bn
+        running_mean, running_var, batch_stats, momentum, eps, tracked = _bn_config(bn)
         x_seq = L.aligned16(x_seq)
-        y, partial = _conv_forward(x_seq, weight, x_exact, True) if batch_stats else (_conv_forward(x_seq, weight, x_exact), None)
-        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial)
+        y, partial, x_amax = _conv_forward(x_seq, weight, x_exact, batch_stats)
+        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial, tracked)
         spikes, v_last = _bn_lif_forward(y, bn_map, v_init, spec, False)
-        return spikes, v_last, y, bn_map
+        return spikes, v_last, y, bn_map, x_amax
 
     @staticmethod
     def setup_context(ctx, inputs, output):
         x_seq, weight, gamma, beta, v_init, bn, spec, x_exact = inputs
         ctx.spec, ctx.batch_stats, ctx.x_exact = spec, bn[2], x_exact
-        ctx.save_for_backward(L.aligned16(x_seq), weight, gamma, v_init, output[2], output[3])
-        ctx.mark_non_differentiable(output[2], output[3])
+        ctx.save_for_backward(L.aligned16(x_seq), weight, gamma, v_init, output[2], output[3], output[4])
+        ctx.mark_non_differentiable(output[2], output[3], output[4])
         ctx.set_materialize_grads(False)
 
     @staticmethod
-    def backward(ctx, grad_spikes, grad_v_last, _y, _map):
-        x_seq, weight, gamma, v_init, y, bn_map = ctx.saved_tensors
+    def backward(ctx, grad_spikes, grad_v_last, _y, _map, _amax):
+        x_seq, weight, gamma, v_init, y, bn_map, x_amax = ctx.saved_tensors
         need = ctx.needs_input_grad
-        dy, dgamma, dbeta, gvi = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
-                                                  grad_v_last, bool(need[4]))
-        dx, dw = _conv_backward(dy, x_seq, weight, ctx.x_exact, bool(need[0]), bool(need[1]))
+        dy, dgamma, dbeta, gvi, dy_amax = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
+                                                            grad_v_last, bool(need[4]), True)
+        dx, dw = _conv_backward(dy, x_seq, weight, ctx.x_exact, bool(need[0]), bool(need[1]), dy_amax, x_amax)
         return (dx, dw, dgamma if need[2] else None, dbeta if need[3] else None, gvi, None, None, None)
 
 
@@ -275,38 +393,38 @@ class _ConvBnLifSsa(torch.autograd.Function):
     def forward(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, ssa):
         from . import attention_kernel as A
 
-        running_mean, running_var, batch_stats, momentum, eps = bn
+        running_mean, running_var, batch_stats, momentum, eps, tracked = _bn_config(bn)
         heads, cph, scale = ssa
         x_seq = L.aligned16(x_seq)
         T, B, _, Lp = x_seq.shape
-        y, partial = _conv_forward(x_seq, weight, x_exact, True) if batch_stats else (_conv_forward(x_seq, weight, x_exact), None)
-        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial)
+        y, partial, x_amax = _conv_forward(x_seq, weight, x_exact, batch_stats)
+        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial, tracked)
         bits, v_last = _bn_lif_forward(y, bn_map, v_init, spec, True)
         out = A._ssa_packed(bits, None, torch.float32, T * B, heads, cph, Lp, scale)
-        return out, v_last, y, bn_map, bits
+        return out, v_last, y, bn_map, bits, x_amax
 
     @staticmethod
     def setup_context(ctx, inputs, output):
         x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, ssa = inputs
         ctx.spec, ctx.batch_stats, ctx.x_exact, ctx.ssa = spec, bn[2], x_exact, ssa
-        ctx.save_for_backward(L.aligned16(x_seq), weight, gamma, v_init, output[2], output[3], output[4])
-        ctx.mark_non_differentiable(output[2], output[3], output[4])
+        ctx.save_for_backward(L.aligned16(x_seq), weight, gamma, v_init, output[2], output[3], output[4], output[5])
+        ctx.mark_non_differentiable(output[2], output[3], output[4], output[5])
         ctx.set_materialize_grads(False)
 
     @staticmethod
-    def backward(ctx, grad_out, grad_v_last, _y, _map, _bits):
+    def backward(ctx, grad_out, grad_v_last, _y, _map, _bits, _amax):
         from . import attention_kernel as A
 
-        x_seq, weight, gamma, v_init, y, bn_map, bits = ctx.saved_tensors
+        x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax = ctx.saved_tensors
         heads, cph, scale = ctx.ssa
         T, B, _, Lp = x_seq.shape
         need = ctx.needs_input_grad
         grad_spikes = None
         if grad_out is not None:
             grad_spikes = A._ssa_packed(bits, grad_out, torch.float32, T * B, heads, cph, Lp, scale).view(y.shape)
-        dy, dgamma, dbeta, gvi = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
-                                                  grad_v_last, bool(need[4]))
-        dx, dw = _conv_backward(dy, x_seq, weight, ctx.x_exact, bool(need[0]), bool(need[1]))
+        dy, dgamma, dbeta, gvi, dy_amax = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
+                                                            grad_v_last, bool(need[4]), True)
+        dx, dw = _conv_backward(dy, x_seq, weight, ctx.x_exact, bool(need[0]), bool(need[1]), dy_amax, x_amax)
         return (dx, dw, dgamma if need[2] else None, dbeta if need[3] else None, gvi, None, None, None, None)
 
 
@@ -319,33 +437,33 @@ class _ConvBnLifSsaLif(torch.autograd.Function):
     def forward(x_seq, weight, gamma, beta, v_init, attn_v_init, bn, spec, x_exact, ssa, attn_spec, save_h):
         from . import attention_kernel as A
 
-        running_mean, running_var, batch_stats, momentum, eps = bn
+        running_mean, running_var, batch_stats, momentum, eps, tracked = _bn_config(bn)
         heads, cph, scale = ssa
         x_seq = L.aligned16(x_seq)
         T, B, _, Lp = x_seq.shape
-        y, partial = _conv_forward(x_seq, weight, x_exact, True) if batch_stats else (_conv_forward(x_seq, weight, x_exact), None)
-        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial)
+        y, partial, x_amax = _conv_forward(x_seq, weight, x_exact, batch_stats)
+        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial, tracked)
         bits, v_last = _bn_lif_forward(y, bn_map, v_init, spec, True)
         v_keep, broadcast = K._state_arg(attn_v_init, True)
         spikes, h_seq, attn_v_last = A._ssa_lif_forward(bits, v_keep, _lif_params(attn_spec, broadcast), T, B, heads, cph,
                                                         Lp, scale, save_h)
         if h_seq is None:
             h_seq = spikes.new_empty((0,))
-        return spikes, v_last, attn_v_last, y, bn_map, bits, h_seq
+        return spikes, v_last, attn_v_last, y, bn_map, bits, h_seq, x_amax
 
     @staticmethod
     def setup_context(ctx, inputs, output):
         x_seq, weight, gamma, beta, v_init, attn_v_init, bn, spec, x_exact, ssa, attn_spec, save_h = inputs
         ctx.spec, ctx.batch_stats, ctx.x_exact, ctx.ssa, ctx.attn_spec = spec, bn[2], x_exact, ssa, attn_spec
-        ctx.save_for_backward(L.aligned16(x_seq), weight, gamma, v_init, output[3], output[4], output[5], output[6])
-        ctx.mark_non_differentiable(output[3], output[4], output[5], output[6])
+        ctx.save_for_backward(L.aligned16(x_seq), weight, gamma, v_init, output[3], output[4], output[5], output[6], output[7])
+        ctx.mark_non_differentiable(output[3], output[4], output[5], output[6], output[7])
         ctx.set_materialize_grads(False)
 
     @staticmethod
-    def backward(ctx, grad_attn_spikes, grad_v_last, grad_attn_v_last, _y, _map, _bits, _h):
+    def backward(ctx, grad_attn_spikes, grad_v_last, grad_attn_v_last, _y, _map, _bits, _h, _amax):
         from . import attention_kernel as A
 
-        x_seq, weight, gamma, v_init, y, bn_map, bits, h_seq = ctx.saved_tensors
+        x_seq, weight, gamma, v_init, y, bn_map, bits, h_seq, x_amax = ctx.saved_tensors
         if h_seq.numel() == 0:
             raise RuntimeError("the fused attention block was run without saving h_seq and cannot be differentiated")
         heads, cph, scale = ctx.ssa
@@ -356,9 +474,9 @@ class _ConvBnLifSsaLif(torch.autograd.Function):
             grad_qkv, _ = A._ssa_lif_backward(bits, h_seq, grad_attn_spikes, grad_attn_v_last, _lif_params(ctx.attn_spec), T, B,
                                               heads, cph, Lp, scale, False)
             grad_spikes = grad_qkv.view(y.shape)
-        dy, dgamma, dbeta, gvi = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
-                                                  grad_v_last, bool(need[4]))
-        dx, dw = _conv_backward(dy, x_seq, weight, ctx.x_exact, bool(need[0]), bool(need[1]))
+        dy, dgamma, dbeta, gvi, dy_amax = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
+                                                            grad_v_last, bool(need[4]), True)
+        dx, dw = _conv_backward(dy, x_seq, weight, ctx.x_exact, bool(need[0]), bool(need[1]), dy_amax, x_amax)
         return (dx, dw, dgamma if need[2] else None, dbeta if need[3] else None, gvi, None, None, None, None, None, None, None)
 
 
@@ -371,7 +489,7 @@ def bn_lif(y_seq: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec):
 def conv_bn_lif(x_seq: torch.Tensor, weight: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec, x_exact: bool):
     """``x_seq [T, B, Cin, L]``, ``weight [Cout, Cin]`` -> ``(spikes [T, B, Cout, L], v_last [B, Cout, L])``.
     ``x_exact``: every element of ``x_seq`` is exactly representable in bf16 (spikes, small integers)."""
-    spikes, v_last, _, _ = _ConvBnLif.apply(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact)
+    spikes, v_last, _, _, _ = _ConvBnLif.apply(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact)
     return spikes, v_last
 
 
@@ -379,7 +497,7 @@ def conv_bn_lif_ssa(x_seq: torch.Tensor, weight: torch.Tensor, gamma, beta, v_in
                     heads: int, channels_per_head: int, scale: float):
     """The same block with ``Cout = 3 * heads * channels_per_head`` followed by the contraction; returns
     ``(out [T * B, heads, channels_per_head, L], v_last)``."""
-    out, v_last, _, _, _ = _ConvBnLifSsa.apply(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact,
+    out, v_last, _, _, _, _ = _ConvBnLifSsa.apply(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact,
                                                (heads, channels_per_head, scale))
     return out, v_last
 

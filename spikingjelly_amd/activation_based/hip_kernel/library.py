@@ -73,6 +73,11 @@ EXPORTED_SYMBOLS = (
     "sjhip_pwconv_gemm_stats",
     "sjhip_pwconv_grad_weight_workspace_floats",
     "sjhip_pwconv_grad_weight",
+    "sjhip_pwconv_split_weight_f16",
+    "sjhip_pwconv_amax",
+    "sjhip_pwconv_gemm_f16",
+    "sjhip_pwconv_grad_weight_f16",
+    "sjhip_bn_grad_input_amax",
     "sjhip_bn_stats",
     "sjhip_bn_finalize",
     "sjhip_bn_finalize_rows",
@@ -250,22 +255,35 @@ def load() -> ctypes.CDLL:
         lib.sjhip_pwconv_grad_weight.restype = c_int
         lib.sjhip_pwconv_grad_weight.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64,
                                                  c_void_p, c_void_p, c_void_p]
+        lib.sjhip_pwconv_split_weight_f16.restype = c_int
+        lib.sjhip_pwconv_split_weight_f16.argtypes = [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p]
+        lib.sjhip_pwconv_amax.restype = c_int
+        lib.sjhip_pwconv_amax.argtypes = [c_void_p, c_int64, c_void_p, c_void_p]
+        lib.sjhip_pwconv_gemm_f16.restype = c_int
+        lib.sjhip_pwconv_gemm_f16.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_int, c_void_p, c_int64, c_int64, c_void_p,
+                                              c_void_p, c_void_p]
+        lib.sjhip_pwconv_grad_weight_f16.restype = c_int
+        lib.sjhip_pwconv_grad_weight_f16.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64,
+                                                     c_int64, c_void_p, c_void_p, c_void_p]
         lib.sjhip_bn_stats.restype = c_int
         lib.sjhip_bn_stats.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]
         lib.sjhip_bn_finalize.restype = c_int
         lib.sjhip_bn_finalize.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float, c_float] + \
-                                         [c_void_p] * 7
+                                         [c_void_p] * 8
         lib.sjhip_bn_finalize_rows.restype = c_int
         lib.sjhip_bn_finalize_rows.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float, c_float] + \
-                                              [c_void_p] * 7
+                                              [c_void_p] * 8
         lib.sjhip_bn_lif_forward.restype = c_int
         lib.sjhip_bn_lif_forward.argtypes = [c_int, POINTER(NeuronParams), c_int64, c_int64, c_int64, c_int64] + [c_void_p] * 8
         lib.sjhip_bn_lif_backward.restype = c_int
         lib.sjhip_bn_lif_backward.argtypes = [c_int, POINTER(NeuronParams), c_int64, c_int64, c_int64, c_int64] + [c_void_p] * 10
         lib.sjhip_bn_backward_finalize.restype = c_int
-        lib.sjhip_bn_backward_finalize.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int] + [c_void_p] * 7
+        lib.sjhip_bn_backward_finalize.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int] + [c_void_p] * 8
         lib.sjhip_bn_grad_input.restype = c_int
         lib.sjhip_bn_grad_input.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]
+        lib.sjhip_bn_grad_input_amax.restype = c_int
+        lib.sjhip_bn_grad_input_amax.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+                                                  c_void_p]
         lib.sjhip_bit_pack.restype = c_int
         lib.sjhip_bit_pack.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p]
         lib.sjhip_bit_unpack.restype = c_int

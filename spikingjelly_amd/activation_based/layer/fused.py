@@ -24,19 +24,22 @@ def _pointwise(conv: nn.Module) -> bool:
 
 
 def _bn_arguments(bn: nn.Module):
-    """``(gamma, beta, (running_mean, running_var, batch_stats, momentum, eps))`` the way ``_BatchNorm.forward`` derives
-    them, or ``None`` for what the kernels do not cover (cumulative moving average)."""
+    """``(gamma, beta, (running_mean, running_var, batch_stats, momentum, eps, num_batches_tracked))`` the way
+    ``_BatchNorm.forward`` derives them, or ``None`` for what the kernels do not cover (cumulative moving average).  The
+    last element is the counter to increment (by the launch that updates the running statistics), or ``None``."""
     if not isinstance(bn, (nn.BatchNorm1d, nn.BatchNorm2d)):
         return None
     batch_stats = bn.training or (bn.running_mean is None and bn.running_var is None)
     update = bn.training and bn.track_running_stats
     if update and bn.momentum is None:
         return None
-    if update and bn.num_batches_tracked is not None:
-        bn.num_batches_tracked.add_(1)
+    tracked = bn.num_batches_tracked if update and bn.num_batches_tracked is not None else None
+    if tracked is not None and not (tracked.is_cuda and tracked.dtype == torch.int64):
+        tracked.add_(1)
+        tracked = None
     running_mean = bn.running_mean if (update or not batch_stats) else None
     running_var = bn.running_var if (update or not batch_stats) else None
-    return bn.weight, bn.bias, (running_mean, running_var, batch_stats, float(bn.momentum or 0.0), float(bn.eps))
+    return bn.weight, bn.bias, (running_mean, running_var, batch_stats, float(bn.momentum or 0.0), float(bn.eps), tracked)
 
 
 def _lif_spec(node: neuron.LIFNode, x_like: torch.Tensor, need_grad: bool):

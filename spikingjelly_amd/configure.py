@@ -33,9 +33,14 @@ for its CuPy/Triton backends).
 """
 
 hip_half_precision_mode = "torch"
-# Number of bf16 terms an fp32 operand of the fused kernel-size-1 convolutions is split into (hip_kernel/conv_bn_lif.py):
-# 3 keeps the accuracy of an fp32 GEMM (six matrix-core products per pair of real operands, three when one operand is
-# spikes), 2 gives about 2^-17 relative per product at half the products, 1 is a plain bf16 GEMM.
+# How the fp32 operands of the fused kernel-size-1 convolutions reach the 16-bit matrix cores (hip_kernel/conv_bn_lif.py).
+# "f16": two fp16 terms of operands scaled by powers of two (weights per row, activations and gradients per tensor, from
+# a pass that finds the largest magnitude), three products per pair of real operands, two when one operand is spikes;
+# accuracy of an fp32 GEMM (2^-23 of sum |a||b| measured).  "bf16": hip_conv_terms bf16 terms, no scaling, no extra pass.
+hip_conv_split = "f16"
+# Number of bf16 terms with hip_conv_split = "bf16": 3 keeps the accuracy of an fp32 GEMM (six matrix-core products per
+# pair of real operands, three when one operand is spikes), 2 gives about 2^-17 relative per product at half the
+# products, 1 is a plain bf16 GEMM.
 hip_conv_terms = 3
 # False: modules keep torch's convolution and batch norm around the hip neurons even where the fused
 # convolution / batch norm / LIF kernels could serve the chain (layer/fused.py).

@@ -122,8 +122,10 @@ __global__ void __launch_bounds__(256) bn_stats_kernel(const float *y, int64_t r
 __global__ void __launch_bounds__(256) bn_finalize_kernel(const float *partial, int64_t S, int C, int64_t count,
                                                            const float *gamma, const float *beta, float eps,
                                                            float momentum, float *running_mean, float *running_var,
-                                                           float *scale, float *shift, float *mean_out, float *invstd_out) {
+                                                           float *scale, float *shift, float *mean_out, float *invstd_out,
+                                                           int64_t *batches_tracked) {
   // one wavefront per channel: lanes stride over the samples, then a butterfly sum
+  if (batches_tracked && blockIdx.x == 0 && threadIdx.x == 0) *batches_tracked += 1;
   const int lane = threadIdx.x & 63;
   const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (c >= C) return;
@@ -336,7 +338,9 @@ __global__ void __launch_bounds__(256) bn_lif_backward_rows_kernel(const BnLifBw
 __global__ void __launch_bounds__(256) bn_backward_finalize_kernel(const float *partial, int64_t B, int C, int64_t count,
                                                                     int training, const float *gamma, const float *mean,
                                                                     const float *invstd, float *dgamma, float *dbeta,
-                                                                    float *coef) {
+                                                                    float *coef, float *amax_reset) {
+  static_assert(SJHIP_PW_AMAX_FLOATS == 256, "one word per work-item of the first block");
+  if (amax_reset && blockIdx.x == 0) amax_reset[threadIdx.x] = 0.0f;
   const int lane = threadIdx.x & 63;
   const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (c >= C) return;
@@ -360,21 +364,39 @@ __global__ void __launch_bounds__(256) bn_backward_finalize_kernel(const float *
   }
 }
 
-// dy = p_c g + q_c y + r_c over the flattened [S * C * L] tensor; dy may be g itself
+// dy = p_c g + q_c y + r_c over the flattened [S * C * L] tensor; dy may be g itself.  With AMAX every block also folds
+// the largest |dy| it wrote into word (block % SJHIP_PW_AMAX_FLOATS) of amax_bits, bit patterns of non-negative floats
+// (they order like unsigned integers, and a maximum does not depend on the order it is taken in), with an atomic whose
+// result is not used, so that the block does not wait for it.
+template <bool AMAX>
 __global__ void __launch_bounds__(256) bn_grad_input_kernel(const float *g, const float *y, const float *coef, int C, int L,
-                                                             int64_t n, float *dy) {
+                                                             int64_t n, float *dy, unsigned *amax_bits) {
   const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
-  if (i >= n) return;
-  const int c = (int)((i / L) % C);
-  const float p = coef[c], q = coef[C + c], r = coef[2 * C + c];
-  const f32x4 gv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(g + i));
-  const f32x4 yv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(y + i));
-  f32x4 o;
-  o.x = fmaf(p, gv.x, fmaf(q, yv.x, r));
-  o.y = fmaf(p, gv.y, fmaf(q, yv.y, r));
-  o.z = fmaf(p, gv.z, fmaf(q, yv.z, r));
-  o.w = fmaf(p, gv.w, fmaf(q, yv.w, r));
-  *reinterpret_cast<f32x4 *>(dy + i) = o;
+  float amax = 0.0f;
+  if (i < n) {
+    const int c = (int)((i / L) % C);
+    const float p = coef[c], q = coef[C + c], r = coef[2 * C + c];
+    const f32x4 gv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(g + i));
+    const f32x4 yv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(y + i));
+    f32x4 o;
+    o.x = fmaf(p, gv.x, fmaf(q, yv.x, r));
+    o.y = fmaf(p, gv.y, fmaf(q, yv.y, r));
+    o.z = fmaf(p, gv.z, fmaf(q, yv.z, r));
+    o.w = fmaf(p, gv.w, fmaf(q, yv.w, r));
+    *reinterpret_cast<f32x4 *>(dy + i) = o;
+    if (AMAX) amax = fmaxf(fmaxf(fabsf(o.x), fabsf(o.y)), fmaxf(fabsf(o.z), fabsf(o.w)));
+  }
+  if (AMAX) {
+    __shared__ float part[4];
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const unsigned bits = __builtin_bit_cast(unsigned, fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3])));
+      atomicMax(amax_bits + blockIdx.x % SJHIP_PW_AMAX_FLOATS, bits);
+    }
+  }
 }
 
 int check_layout(const char *what, int64_t T, int64_t B, int64_t C, int64_t L) {
@@ -403,11 +425,11 @@ int launch_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *part
 // partial [rows][C][2]: sums over `count` elements per channel in all
 int launch_bn_finalize(const float *partial, int64_t rows, int64_t count, int64_t C, const float *gamma, const float *beta, float eps,
                        float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
-                       float *invstd, hipStream_t stream) {
+                       float *invstd, int64_t *batches_tracked, hipStream_t stream) {
   if (C < 1 || C > (1 << 24)) return fail(SJHIP_ERR_INVALID, "bn_finalize: C=%lld", (long long)C);
   if (!partial && (!running_mean || !running_var)) return fail(SJHIP_ERR_INVALID, "bn_finalize: evaluation mode needs the running statistics");
   hipLaunchKernelGGL(bn_finalize_kernel, dim3((unsigned)((C + 3) / 4)), dim3(256), 0, stream, partial, rows, (int)C, count, gamma,
-                     beta, eps, momentum, running_mean, running_var, scale, shift, mean, invstd);
+                     beta, eps, momentum, running_mean, running_var, scale, shift, mean, invstd, batches_tracked);
   return check_launch("bn_finalize");
 }
 
@@ -480,14 +502,14 @@ int launch_bn_lif_backward(int neuron, const sjhip_neuron_params &p, int64_t T, 
 
 int launch_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64_t C, int64_t L, int training, const float *gamma,
                                 const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef,
-                                hipStream_t stream) {
+                                float *amax_reset, hipStream_t stream) {
   if (C < 1 || C > (1 << 24)) return fail(SJHIP_ERR_INVALID, "bn_backward_finalize: C=%lld", (long long)C);
   hipLaunchKernelGGL(bn_backward_finalize_kernel, dim3((unsigned)((C + 3) / 4)), dim3(256), 0, stream, partial, B, (int)C,
-                     T * B * L, training, gamma, mean, invstd, dgamma, dbeta, coef);
+                     T * B * L, training, gamma, mean, invstd, dgamma, dbeta, coef, amax_reset);
   return check_launch("bn_backward_finalize");
 }
 
-int launch_bn_grad_input(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy,
+int launch_bn_grad_input(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy, float *amax,
                          hipStream_t stream) {
   int rc = check_layout("bn_grad_input", 1, S, C, L);
   if (rc != SJHIP_OK) return rc;
@@ -495,7 +517,12 @@ int launch_bn_grad_input(const float *g, const float *y, const float *coef, int6
   const int64_t n = S * C * L, blocks = (n / 4 + 255) / 256;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "bn_grad_input: %lld elements", (long long)n);
   ProfileScope prof(KC_BN_GRAD_INPUT, stream);
-  hipLaunchKernelGGL(bn_grad_input_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, g, y, coef, (int)C, (int)L, n, dy);
+  if (amax)
+    hipLaunchKernelGGL(bn_grad_input_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, g, y, coef, (int)C, (int)L, n, dy,
+                       reinterpret_cast<unsigned *>(amax));
+  else
+    hipLaunchKernelGGL(bn_grad_input_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, g, y, coef, (int)C, (int)L, n, dy,
+                       (unsigned *)nullptr);
   return check_launch("bn_grad_input");
 }
 

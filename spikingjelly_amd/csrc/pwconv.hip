@@ -58,6 +58,8 @@ namespace {
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kPwThreads = 256;
 constexpr int kTile = 128;            // rows and columns of a block's output tile
@@ -78,15 +80,40 @@ __device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast
 
 // Word t holds term t of (x0, x1): term 0 is the value rounded to bf16, term 1 the rounded remainder, term 2 what is
 // left (exact for fp32 inputs: 3 x 8 significant bits).  The remainders are exact differences.
-template <int TERMS> __device__ __forceinline__ void split_pair(float x0, float x1, uint32_t (&w)[TERMS]) {
+// With H the terms are fp16 (round to nearest, subnormals kept): two of them hold 22 to 24 significant bits of a value
+// whose magnitude lies between 2^-2 and 2^16, which the callers arrange by scaling with a power of two.
+template <int TERMS, bool H = false> __device__ __forceinline__ void split_pair(float x0, float x1, uint32_t (&w)[TERMS]) {
 #pragma unroll
   for (int t = 0; t < TERMS; ++t) {
-    w[t] = pack_bf16(x0, x1);
-    if (t + 1 < TERMS) {
-      x0 -= bf16_lo(w[t]);
-      x1 -= bf16_hi(w[t]);
+    if (H) {
+      f16x2 p;
+      p.x = (_Float16)x0;
+      p.y = (_Float16)x1;
+      w[t] = __builtin_bit_cast(uint32_t, p);
+      if (t + 1 < TERMS) {
+        x0 -= (float)p.x;
+        x1 -= (float)p.y;
+      }
+    } else {
+      w[t] = pack_bf16(x0, x1);
+      if (t + 1 < TERMS) {
+        x0 -= bf16_lo(w[t]);
+        x1 -= bf16_hi(w[t]);
+      }
     }
   }
+}
+
+// The power of two that brings a largest magnitude `amax` into [2^14, 2^15), and its inverse; 1 for a zero, subnormal
+// or non-finite amax.  Multiplying by either is exact.
+__device__ __forceinline__ void scale_for(float amax, float &scale, float &inverse) {
+  const int field = (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xffu);
+  scale = inverse = 1.0f;
+  if (field == 0 || field == 255) return;
+  int sf = 268 - field;  // biased exponent of 2^(14 - (field - 127))
+  sf = sf < 1 ? 1 : (sf > 253 ? 253 : sf);
+  scale = __builtin_bit_cast(float, (uint32_t)sf << 23);
+  inverse = __builtin_bit_cast(float, (uint32_t)(254 - sf) << 23);
 }
 
 // Block number -> position in the order in which blocks that share tiles should be resident together: hardware block b
@@ -118,6 +145,83 @@ __global__ void __launch_bounds__(256) split_weight_kernel(const float *src, int
     reinterpret_cast<uint32_t *>(planes + (int64_t)t * rows_pad * cols_pad)[at / 2] = w[t];
 }
 
+// fp16 planes[t][tile order] = term t of scale_r * src[r][c], with a power-of-two scale per row r (a row of A is a row
+// of the product, so the GEMM's epilogue takes the scale out again); the inverse scales follow the two planes as
+// rows_pad floats.  One wavefront per row.
+__global__ void __launch_bounds__(256) split_weight_f16_kernel(const float *src, int64_t rows, int64_t cols, int64_t ld_r,
+                                                                int64_t ld_c, int64_t rows_pad, int64_t cols_pad,
+                                                                uint16_t *planes, float *amax_reset) {
+  static_assert(SJHIP_PW_AMAX_FLOATS == 256, "one word per work-item of the first block");
+  if (amax_reset && blockIdx.x == 0) amax_reset[threadIdx.x] = 0.0f;
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows_pad) return;
+  float amax = 0.0f;
+  if (r < rows)
+    for (int64_t c = lane; c < cols; c += 64) amax = fmaxf(amax, fabsf(src[r * ld_r + c * ld_c]));
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
+  float scale, inverse;
+  scale_for(amax, scale, inverse);
+  for (int64_t c = 2 * lane; c < cols_pad; c += 128) {
+    float x0 = 0.0f, x1 = 0.0f;
+    if (r < rows) {
+      if (c < cols) x0 = src[r * ld_r + c * ld_c] * scale;
+      if (c + 1 < cols) x1 = src[r * ld_r + (c + 1) * ld_c] * scale;
+    }
+    uint32_t w[2];
+    split_pair<2, true>(x0, x1, w);
+    const int64_t at = (((r / kTile) * (cols_pad / kTileK) + c / kTileK) * kTile + r % kTile) * kTileK + c % kTileK;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+      reinterpret_cast<uint32_t *>(planes + (int64_t)t * rows_pad * cols_pad)[at / 2] = w[t];
+  }
+  if (lane == 0) reinterpret_cast<float *>(planes + 2 * rows_pad * cols_pad)[r] = inverse;
+}
+
+// The largest magnitude of a tensor is kept as SJHIP_PW_AMAX_FLOATS non-negative floats whose maximum it is: blocks fold
+// their share into word (block % SJHIP_PW_AMAX_FLOATS) with an integer atomic maximum (the bit patterns of non-negative
+// floats order like unsigned integers, and a maximum does not depend on the order it is taken in).  Several words,
+// and an atomic whose result is not used, so that a block neither meets tens of thousands of others on one address nor
+// waits for memory before it ends: the kernel that writes the gradients of the qkv convolution takes 73 us with it
+// (68 without), against 109 us with one word that a block reads first to skip atomics that would not raise it, and
+// 93 us with that read spread over 256 words.
+__device__ __forceinline__ void fold_amax(unsigned *amax_bits, float block_max) {
+  atomicMax(amax_bits + blockIdx.x % SJHIP_PW_AMAX_FLOATS, __builtin_bit_cast(unsigned, block_max));
+}
+// The maximum of those words, in every lane of a wavefront.
+__device__ __forceinline__ float tensor_amax(const float *amax) {
+  static_assert(SJHIP_PW_AMAX_FLOATS == 256, "one 16-byte load per lane");
+  const f32x4 v = reinterpret_cast<const f32x4 *>(amax)[threadIdx.x & 63];
+  float m = fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w));
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) m = fmaxf(m, __shfl_xor(m, d));
+  return m;
+}
+constexpr int kAmaxBlocks = 1024;
+__global__ void __launch_bounds__(256) amax_kernel(const float *x, int64_t n, unsigned *amax_bits) {
+  __shared__ float part[4];
+  float amax = 0.0f;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  const int64_t i0 = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+    const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
+    const int64_t n4 = n / 4;
+    for (int64_t i = i0; i < n4; i += stride) {
+      const f32x4 v = __builtin_nontemporal_load(x4 + i);
+      amax = fmaxf(fmaxf(amax, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
+    }
+    for (int64_t i = 4 * n4 + i0; i < n; i += stride) amax = fmaxf(amax, fabsf(x[i]));
+  } else {
+    for (int64_t i = i0; i < n; i += stride) amax = fmaxf(amax, fabsf(x[i]));
+  }
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  if (threadIdx.x == 0) fold_amax(amax_bits, fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3])));
+}
+
 struct PwGemmArgs {
   const uint16_t *a_planes;  // [3][M_pad / 128][K_pad / 32][128][32] bf16
   const float *b;            // [S][K][L]
@@ -128,6 +232,8 @@ struct PwGemmArgs {
   int m_blocks;
   float *stats;              // nullptr, or [2 x column blocks][M][2]: per row of c the sum and the sum of squares over
                              // each half (64 columns) of every column block
+  const float *a_inverse;    // fp16 terms: the inverse scale of every (padded) row of A
+  const float *b_amax;       // fp16 terms: nullptr (b needs no scale), or the words whose maximum is max |b|
 };
 constexpr int kStatPitch = 33;                             // floats per row of the transposing buffer: no bank conflicts
 constexpr unsigned kStatLds = 4 * 64 * kStatPitch * 4;     // one buffer of 64 rows x 32 column pairs per wavefront
@@ -139,8 +245,8 @@ template <int TA, int TB> struct Pairs {
 };
 
 // One k step of 16 for a wavefront's 2 x 2 tiles: operands in registers, smallest terms first.
-template <int TA, int TB>
-__device__ __forceinline__ void mfma_step(const bf16x8 (&af)[2][TA], const bf16x8 (&bf)[2][TB], f32x16 (&acc)[2][2]) {
+template <int TA, int TB, bool H>
+__device__ __forceinline__ void mfma_step(const u32x4 (&af)[2][TA], const u32x4 (&bf)[2][TB], f32x16 (&acc)[2][2]) {
 #pragma unroll
   for (int order = Pairs<TA, TB>::kMax; order >= 0; --order) {
 #pragma unroll
@@ -151,17 +257,20 @@ __device__ __forceinline__ void mfma_step(const bf16x8 (&af)[2][TA], const bf16x
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
-          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mt][ta], bf[nt][tb], acc[mt][nt], 0, 0, 0);
+          acc[mt][nt] = H ? __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[mt][ta]),
+                                                                    __builtin_bit_cast(f16x8, bf[nt][tb]), acc[mt][nt], 0, 0, 0)
+                          : __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[mt][ta]),
+                                                                     __builtin_bit_cast(bf16x8, bf[nt][tb]), acc[mt][nt], 0, 0, 0);
     }
   }
 }
 
 // Fragment of a K-contiguous operand: row `row` of the tile, k group (lane / 32) of k step ks.
-__device__ __forceinline__ bf16x8 row_fragment(const uint8_t *plane, int row, int ks, int lane) {
-  return *reinterpret_cast<const bf16x8 *>(plane + row * kRowBytes + ks * 32 + (lane >> 5) * 16);
+__device__ __forceinline__ u32x4 row_fragment(const uint8_t *plane, int row, int ks, int lane) {
+  return *reinterpret_cast<const u32x4 *>(plane + row * kRowBytes + ks * 32 + (lane >> 5) * 16);
 }
 
-template <int TA, int TB>
+template <int TA, int TB, bool H>
 __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) pw_gemm_kernel(const PwGemmArgs a) {
   extern __shared__ __align__(16) uint8_t lds[];
   uint8_t *As = lds;                   // [TA][128][kRowBytes]
@@ -203,6 +312,8 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   const bool edge_cols = __builtin_amdgcn_readfirstlane(j0 + kTile > a.ncols ? 1 : 0) != 0;
   const char *a_base = reinterpret_cast<const char *>(a.a_planes);
   const char *b_base = reinterpret_cast<const char *>(a.b);
+  float b_scale = 1.0f, b_inverse = 1.0f;
+  if (H && TB > 1 && a.b_amax != nullptr) scale_for(tensor_amax(a.b_amax), b_scale, b_inverse);
 
   // Two B tiles are in flight in registers (sets 0 and 1): a tile is requested two multiplications before it is staged,
   // which covers a miss to HBM.  The A tiles (weight planes, a few MB that every block reads) come from L2, one ahead.
@@ -240,7 +351,12 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const u32x2 lo = rb[set][2 * i], hi = rb[set][2 * i + 1];
-        split_pair<TB>(__builtin_bit_cast(float, c ? lo.y : lo.x), __builtin_bit_cast(float, c ? hi.y : hi.x), w[i]);
+        float x0 = __builtin_bit_cast(float, c ? lo.y : lo.x), x1 = __builtin_bit_cast(float, c ? hi.y : hi.x);
+        if (H && TB > 1) {
+          x0 *= b_scale;
+          x1 *= b_scale;
+        }
+        split_pair<TB, H>(x0, x1, w[i]);
       }
 #pragma unroll
       for (int t = 0; t < TB; ++t) {
@@ -262,7 +378,7 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   auto multiply = [&]() {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      bf16x8 af[2][TA], bf[2][TB];
+      u32x4 af[2][TA], bf[2][TB];
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -271,7 +387,7 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int t = 0; t < TB; ++t) bf[nt][t] = row_fragment(Bs + t * kRowPlane, wn * 64 + nt * 32 + (lane & 31), ks, lane);
-      mfma_step<TA, TB>(af, bf, acc);
+      mfma_step<TA, TB, H>(af, bf, acc);
     }
   };
   // One K step: stage the tile whose loads were requested earlier, request later tiles, multiply.  In the steady state
@@ -299,6 +415,16 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   if (k0 + 2 * kTileK < K_pad) step(k0 + 2 * kTileK, 0, false, false);
 
   // accumulator register r of a 32 x 32 tile: row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
+  if (H) {  // take the power-of-two scales of the row of A and of b out again: exact
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float inv = a.a_inverse[m0 + wm * 64 + mt * 32 + 4 * (lane >> 5) + 8 * (r >> 2) + (r & 3)];
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) acc[mt][nt][r] = acc[mt][nt][r] * inv * b_inverse;
+      }
+  }
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
     const int64_t j = j0 + wn * 64 + nt * 32 + (lane & 31);
@@ -352,9 +478,10 @@ struct PwDwArgs {
   int M, N, L;
   int s_per_chunk;
   int m_blocks, n_blocks;
+  const float *dy_amax, *x_amax;  // fp16 terms: nullptr (no scale), or the words whose maximum is the tensor's max |.|
 };
 
-template <int TA, int TB>
+template <int TA, int TB, bool H>
 __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) pw_dw_kernel(const PwDwArgs a) {
   extern __shared__ __align__(16) uint8_t lds[];
   uint8_t *As = lds;                   // [TA][128][kRowBytes]
@@ -387,6 +514,9 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   const bool edge_rows = __builtin_amdgcn_readfirstlane((m0 + kTile > M || n0 + kTile > N) ? 1 : 0) != 0;
   const char *dy_base = reinterpret_cast<const char *>(a.dy);
   const char *x_base = reinterpret_cast<const char *>(a.x);
+  float a_scale = 1.0f, a_inverse = 1.0f, b_scale = 1.0f, b_inverse = 1.0f;
+  if (H && TA > 1 && a.dy_amax != nullptr) scale_for(tensor_amax(a.dy_amax), a_scale, a_inverse);
+  if (H && TB > 1 && a.x_amax != nullptr) scale_for(tensor_amax(a.x_amax), b_scale, b_inverse);
   f32x4 ra[2][4], rb[2][4];  // two tiles in flight, as in pw_gemm_kernel
   auto fetch = [&](int64_t it, int set) {
     const int64_t s = s_begin + it / l_steps;
@@ -416,8 +546,10 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       const int off = (rr + 32 * i) * kRowBytes + q4 * 8;
       {
         uint32_t w01[TA], w23[TA];
-        split_pair<TA>(ra[set][i].x, ra[set][i].y, w01);
-        split_pair<TA>(ra[set][i].z, ra[set][i].w, w23);
+        f32x4 v = ra[set][i];
+        if (H && TA > 1) v *= a_scale;
+        split_pair<TA, H>(v.x, v.y, w01);
+        split_pair<TA, H>(v.z, v.w, w23);
 #pragma unroll
         for (int t = 0; t < TA; ++t) {
           u32x2 w;
@@ -428,8 +560,10 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       }
       {
         uint32_t w01[TB], w23[TB];
-        split_pair<TB>(rb[set][i].x, rb[set][i].y, w01);
-        split_pair<TB>(rb[set][i].z, rb[set][i].w, w23);
+        f32x4 v = rb[set][i];
+        if (H && TB > 1) v *= b_scale;
+        split_pair<TB, H>(v.x, v.y, w01);
+        split_pair<TB, H>(v.z, v.w, w23);
 #pragma unroll
         for (int t = 0; t < TB; ++t) {
           u32x2 w;
@@ -453,7 +587,7 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
     const int l0 = (int)(it % l_steps) * kTileK;
     const int ksteps = (l0 + 16 < L) ? 2 : 1;  // the second half of the last stage of a row may hold nothing
     for (int ks = 0; ks < ksteps; ++ks) {
-      bf16x8 af[2][TA], bf[2][TB];
+      u32x4 af[2][TA], bf[2][TB];
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -462,7 +596,7 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int t = 0; t < TB; ++t) bf[nt][t] = row_fragment(Bs + t * kRowPlane, wn * 64 + nt * 32 + (lane & 31), ks, lane);
-      mfma_step<TA, TB>(af, bf, acc);
+      mfma_step<TA, TB, H>(af, bf, acc);
     }
   };
   // as in pw_gemm_kernel: unconditional requests in the steady state, conditions only in the last steps
@@ -485,6 +619,14 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   if (it + 2 < iters) step(it + 2, 0, false);
 
   float *out = a.partials + (int64_t)chunk * M * N;
+  if (H) {
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[mt][nt][r] = acc[mt][nt][r] * a_inverse * b_inverse;
+  }
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
     const int col = n0 + wn * 64 + nt * 32 + (lane & 31);
@@ -529,16 +671,16 @@ __global__ void __launch_bounds__(256) dw_reduce_kernel(const float *partials, i
 
 int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
-template <int TA, int TB> int launch_gemm_terms(const PwGemmArgs &a, int64_t blocks, hipStream_t stream) {
+template <int TA, int TB, bool H = false> int launch_gemm_terms(const PwGemmArgs &a, int64_t blocks, hipStream_t stream) {
   unsigned lds = (TA + TB) * kRowPlane;
   if (a.stats && lds < kStatLds) lds = kStatLds;
-  hipLaunchKernelGGL((pw_gemm_kernel<TA, TB>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
+  hipLaunchKernelGGL((pw_gemm_kernel<TA, TB, H>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
   return check_launch("pwconv_gemm");
 }
 
-template <int TA, int TB> int launch_dw_terms(const PwDwArgs &a, int64_t blocks, hipStream_t stream) {
+template <int TA, int TB, bool H = false> int launch_dw_terms(const PwDwArgs &a, int64_t blocks, hipStream_t stream) {
   const unsigned lds = (TA + TB) * kRowPlane;
-  hipLaunchKernelGGL((pw_dw_kernel<TA, TB>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
+  hipLaunchKernelGGL((pw_dw_kernel<TA, TB, H>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
   return check_launch("pwconv_grad_weight");
 }
 
@@ -572,6 +714,24 @@ int launch_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int t
   return check_launch("pwconv_split_weight");
 }
 
+int launch_pwconv_split_weight_f16(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes,
+                                   float *amax_reset, hipStream_t stream) {
+  const int64_t ar = transpose ? cols : rows, ac = transpose ? rows : cols;
+  const int64_t rows_pad = round_up(ar, kTile), cols_pad = round_up(ac, kTileK);
+  const int64_t blocks = rows_pad / 4;
+  if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_split_weight_f16: %lld x %lld", (long long)rows, (long long)cols);
+  hipLaunchKernelGGL(split_weight_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, w, ar, ac,
+                     transpose ? (int64_t)1 : cols, transpose ? cols : (int64_t)1, rows_pad, cols_pad, planes, amax_reset);
+  return check_launch("pwconv_split_weight_f16");
+}
+
+int launch_pwconv_amax(const float *x, int64_t n, float *amax, hipStream_t stream) {
+  int64_t blocks = (n / 4 + 255) / 256;
+  blocks = blocks < 1 ? 1 : (blocks > kAmaxBlocks ? kAmaxBlocks : blocks);
+  hipLaunchKernelGGL(amax_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, n, reinterpret_cast<unsigned *>(amax));
+  return check_launch("pwconv_amax");
+}
+
 namespace {
 const int64_t kPwOffsetLimit = int64_t(1) << 30;  // per-lane offsets into A and B are 32-bit byte offsets
 int64_t gemm_samples_per_launch(int64_t K, int64_t L) { return (kPwOffsetLimit - 1) / (K * L); }
@@ -588,8 +748,8 @@ int64_t pwconv_gemm_stats_rows(int64_t K, int64_t S, int64_t L) {
   return rows;
 }
 
-int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,
-                       int64_t L, float *c, float *stats, hipStream_t stream) {
+int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms,
+                       const float *b_amax, int64_t S, int64_t L, float *c, float *stats, hipStream_t stream) {
   if (L % 2 != 0 || !aligned16(a_planes) || (reinterpret_cast<uintptr_t>(b) & 7u))
     return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: L=%lld must be even, the weight planes 16-byte and the activations 8-byte aligned", (long long)L);
   const int64_t limit = kPwOffsetLimit;
@@ -606,6 +766,8 @@ int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t
     a.ncols = s_count * L;
     a.m_blocks = (int)(round_up(M, kTile) / kTile);
     a.stats = stats;
+    a.a_inverse = reinterpret_cast<const float *>(a_planes + 2 * a.plane_stride);
+    a.b_amax = b_amax;
     if (stats) stats += 2 * ((a.ncols + kTile - 1) / kTile) * M * 2;
     const int64_t blocks = a.m_blocks * ((a.ncols + kTile - 1) / kTile);
     if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: %lld blocks", (long long)blocks);
@@ -616,7 +778,9 @@ int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t
       case 22: rc = launch_gemm_terms<2, 2>(a, blocks, stream); break;
       case 21: rc = launch_gemm_terms<2, 1>(a, blocks, stream); break;
       case 11: rc = launch_gemm_terms<1, 1>(a, blocks, stream); break;
-      default: return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: %d weight terms with %d activation terms (3/3, 3/1, 2/2, 2/1, 1/1)", a_terms, b_terms);
+      case (SJHIP_PW_F16 | 2) * 10 + 2: rc = launch_gemm_terms<2, 2, true>(a, blocks, stream); break;
+      case (SJHIP_PW_F16 | 2) * 10 + 1: rc = launch_gemm_terms<2, 1, true>(a, blocks, stream); break;
+      default: return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: %d weight terms with %d activation terms (bf16: 3/3, 3/1, 2/2, 2/1, 1/1; fp16: 2/2, 2/1)", a_terms, b_terms);
     }
     if (rc != SJHIP_OK) return rc;
   }
@@ -629,14 +793,16 @@ int64_t pwconv_dw_workspace_floats(int64_t M, int64_t N, int64_t S) {
   return (S + spc - 1) / spc * M * N;
 }
 
-int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int x_terms, int64_t S, int64_t M, int64_t N,
-                              int64_t L, float *dw, float *workspace, hipStream_t stream) {
+int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *dy_amax, const float *x, int x_terms,
+                              const float *x_amax, int64_t S, int64_t M, int64_t N, int64_t L, float *dw, float *workspace,
+                              hipStream_t stream) {
   if (L % 4 != 0 || !aligned16(dy) || !aligned16(x))
     return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight: L=%lld must be a multiple of 4 and the tensors 16-byte aligned", (long long)L);
   if (M * L >= (int64_t(1) << 30) || N * L >= (int64_t(1) << 30) || M * N >= (int64_t(1) << 40))  // 32-bit per-lane byte offsets
     return fail(SJHIP_ERR_TOO_LARGE, "pwconv_grad_weight: M=%lld N=%lld L=%lld", (long long)M, (long long)N, (long long)L);
   PwDwArgs a;
   a.dy = dy; a.x = x; a.partials = workspace; a.S = S;
+  a.dy_amax = dy_amax; a.x_amax = x_amax;
   a.M = (int)M; a.N = (int)N; a.L = (int)L;
   a.m_blocks = (int)(round_up(M, kTile) / kTile);
   a.n_blocks = (int)(round_up(N, kTile) / kTile);
@@ -654,7 +820,9 @@ int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int
       case 22: rc = launch_dw_terms<2, 2>(a, blocks, stream); break;
       case 21: rc = launch_dw_terms<2, 1>(a, blocks, stream); break;
       case 11: rc = launch_dw_terms<1, 1>(a, blocks, stream); break;
-      default: return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight: %d gradient terms with %d activation terms (3/3, 3/1, 2/2, 2/1, 1/1)", dy_terms, x_terms);
+      case (SJHIP_PW_F16 | 2) * 10 + 2: rc = launch_dw_terms<2, 2, true>(a, blocks, stream); break;
+      case (SJHIP_PW_F16 | 2) * 10 + 1: rc = launch_dw_terms<2, 1, true>(a, blocks, stream); break;
+      default: return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight: %d gradient terms with %d activation terms (bf16: 3/3, 3/1, 2/2, 2/1, 1/1; fp16: 2/2, 2/1)", dy_terms, x_terms);
     }
     if (rc != SJHIP_OK) return rc;
     const int64_t count = M * N;

@@ -572,7 +572,8 @@ int sjhip_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t 
   if (!a_planes || !b || !c) return fail(SJHIP_ERR_INVALID, "pwconv_gemm: NULL buffer");
   if (M < 1 || K < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_gemm: M=%lld K=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)K, (long long)S, (long long)L);
   if (S > (int64_t(1) << 40) / L) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: S*L overflows");
-  return launch_pwconv_gemm(a_planes, a_terms, M, K, b, b_terms, S, L, c, nullptr, static_cast<hipStream_t>(stream));
+  if (a_terms < 1 || a_terms > 3) return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: %d weight terms (1 to 3 bf16 terms; fp16 planes belong to sjhip_pwconv_gemm_f16)", a_terms);
+  return launch_pwconv_gemm(a_planes, a_terms, M, K, b, b_terms, nullptr, S, L, c, nullptr, static_cast<hipStream_t>(stream));
 }
 
 int64_t sjhip_pwconv_gemm_stats_rows(int64_t K, int64_t S, int64_t L) {
@@ -585,7 +586,8 @@ int sjhip_pwconv_gemm_stats(const uint16_t *a_planes, int a_terms, int64_t M, in
   if (!a_planes || !b || !c || !partial) return fail(SJHIP_ERR_INVALID, "pwconv_gemm_stats: NULL buffer");
   if (M < 1 || K < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_gemm_stats: M=%lld K=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)K, (long long)S, (long long)L);
   if (S > (int64_t(1) << 40) / L) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm_stats: S*L overflows");
-  return launch_pwconv_gemm(a_planes, a_terms, M, K, b, b_terms, S, L, c, partial, static_cast<hipStream_t>(stream));
+  if (a_terms < 1 || a_terms > 3) return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm_stats: %d weight terms (1 to 3 bf16 terms; fp16 planes belong to sjhip_pwconv_gemm_f16)", a_terms);
+  return launch_pwconv_gemm(a_planes, a_terms, M, K, b, b_terms, nullptr, S, L, c, partial, static_cast<hipStream_t>(stream));
 }
 
 int64_t sjhip_pwconv_grad_weight_workspace_floats(int64_t M, int64_t N, int64_t S) {
@@ -597,7 +599,43 @@ int sjhip_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int 
                              int64_t L, float *dw, float *workspace, void *stream) {
   if (!dy || !x || !dw || !workspace) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight: NULL buffer");
   if (M < 1 || N < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight: M=%lld N=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)N, (long long)S, (long long)L);
-  return launch_pwconv_grad_weight(dy, dy_terms, x, x_terms, S, M, N, L, dw, workspace, static_cast<hipStream_t>(stream));
+  if (dy_terms < 1 || dy_terms > 3) return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight: %d gradient terms (1 to 3 bf16 terms)", dy_terms);
+  return launch_pwconv_grad_weight(dy, dy_terms, nullptr, x, x_terms, nullptr, S, M, N, L, dw, workspace, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_pwconv_split_weight_f16(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, float *amax_reset,
+                                  void *stream) {
+  if (!w || !planes) return fail(SJHIP_ERR_INVALID, "pwconv_split_weight_f16: NULL buffer");
+  if (rows < 1 || cols < 1) return fail(SJHIP_ERR_INVALID, "pwconv_split_weight_f16: %lld x %lld", (long long)rows, (long long)cols);
+  if (!aligned16(planes)) return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_split_weight_f16: the planes must be 16-byte aligned");
+  return launch_pwconv_split_weight_f16(w, rows, cols, transpose, planes, amax_reset, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_pwconv_amax(const float *x, int64_t n, float *amax, void *stream) {
+  if (!x || !amax) return fail(SJHIP_ERR_INVALID, "pwconv_amax: NULL buffer");
+  if (n < 1) return fail(SJHIP_ERR_INVALID, "pwconv_amax: n=%lld", (long long)n);
+  return launch_pwconv_amax(x, n, amax, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_pwconv_gemm_f16(const uint16_t *a_planes, int64_t M, int64_t K, const float *b, int b_terms, const float *b_amax,
+                          int64_t S, int64_t L, float *c, float *partial, void *stream) {
+  if (!a_planes || !b || !c) return fail(SJHIP_ERR_INVALID, "pwconv_gemm_f16: NULL buffer");
+  if (M < 1 || K < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_gemm_f16: M=%lld K=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)K, (long long)S, (long long)L);
+  if (S > (int64_t(1) << 40) / L) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm_f16: S*L overflows");
+  if (b_terms != 1 && b_terms != 2) return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm_f16: %d activation terms (1 or 2)", b_terms);
+  if (b_terms == 2 && !b_amax) return fail(SJHIP_ERR_INVALID, "pwconv_gemm_f16: two activation terms need the largest magnitude from sjhip_pwconv_amax");
+  return launch_pwconv_gemm(a_planes, SJHIP_PW_F16 | 2, M, K, b, b_terms, b_terms == 2 ? b_amax : nullptr, S, L, c, partial,
+                            static_cast<hipStream_t>(stream));
+}
+
+int sjhip_pwconv_grad_weight_f16(const float *dy, const float *dy_amax, const float *x, int x_terms, const float *x_amax,
+                                 int64_t S, int64_t M, int64_t N, int64_t L, float *dw, float *workspace, void *stream) {
+  if (!dy || !dy_amax || !x || !dw || !workspace) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight_f16: NULL buffer");
+  if (M < 1 || N < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight_f16: M=%lld N=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)N, (long long)S, (long long)L);
+  if (x_terms != 1 && x_terms != 2) return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight_f16: %d activation terms (1 or 2)", x_terms);
+  if (x_terms == 2 && !x_amax) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight_f16: two activation terms need the largest magnitude from sjhip_pwconv_amax");
+  return launch_pwconv_grad_weight(dy, SJHIP_PW_F16 | 2, dy_amax, x, x_terms, x_terms == 2 ? x_amax : nullptr, S, M, N, L, dw,
+                                   workspace, static_cast<hipStream_t>(stream));
 }
 
 int sjhip_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, void *stream) {
@@ -607,20 +645,20 @@ int sjhip_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *parti
 
 int sjhip_bn_finalize(const float *partial, int64_t S, int64_t C, int64_t L, const float *gamma, const float *beta, float eps,
                       float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
-                      float *invstd, void *stream) {
+                      float *invstd, int64_t *batches_tracked, void *stream) {
   if (!scale || !shift || !mean || !invstd) return fail(SJHIP_ERR_INVALID, "bn_finalize: NULL output");
   if (partial && (S < 1 || L < 1)) return fail(SJHIP_ERR_INVALID, "bn_finalize: S=%lld L=%lld", (long long)S, (long long)L);
   return launch_bn_finalize(partial, S, S * L, C, gamma, beta, eps, momentum, running_mean, running_var, scale, shift, mean, invstd,
-                            static_cast<hipStream_t>(stream));
+                            batches_tracked, static_cast<hipStream_t>(stream));
 }
 
 int sjhip_bn_finalize_rows(const float *partial, int64_t rows, int64_t count, int64_t C, const float *gamma, const float *beta,
                            float eps, float momentum, float *running_mean, float *running_var, float *scale, float *shift,
-                           float *mean, float *invstd, void *stream) {
+                           float *mean, float *invstd, int64_t *batches_tracked, void *stream) {
   if (!partial || !scale || !shift || !mean || !invstd) return fail(SJHIP_ERR_INVALID, "bn_finalize_rows: NULL buffer");
   if (rows < 1 || count < 1) return fail(SJHIP_ERR_INVALID, "bn_finalize_rows: rows=%lld count=%lld", (long long)rows, (long long)count);
   return launch_bn_finalize(partial, rows, count, C, gamma, beta, eps, momentum, running_mean, running_var, scale, shift, mean,
-                            invstd, static_cast<hipStream_t>(stream));
+                            invstd, batches_tracked, static_cast<hipStream_t>(stream));
 }
 
 int sjhip_bn_lif_forward(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
@@ -643,16 +681,23 @@ int sjhip_bn_lif_backward(int neuron, const sjhip_neuron_params *p, int64_t T, i
 }
 
 int sjhip_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64_t C, int64_t L, int training, const float *gamma,
-                               const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef, void *stream) {
+                               const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef, float *amax_reset,
+                               void *stream) {
   if (!partial || !mean || !invstd || !coef) return fail(SJHIP_ERR_INVALID, "bn_backward_finalize: NULL buffer");
   if (T < 1 || B < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "bn_backward_finalize: T=%lld B=%lld L=%lld", (long long)T, (long long)B, (long long)L);
-  return launch_bn_backward_finalize(partial, T, B, C, L, training, gamma, mean, invstd, dgamma, dbeta, coef,
+  return launch_bn_backward_finalize(partial, T, B, C, L, training, gamma, mean, invstd, dgamma, dbeta, coef, amax_reset,
                                      static_cast<hipStream_t>(stream));
 }
 
 int sjhip_bn_grad_input(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy, void *stream) {
   if (!g || !y || !coef || !dy) return fail(SJHIP_ERR_INVALID, "bn_grad_input: NULL buffer");
-  return launch_bn_grad_input(g, y, coef, S, C, L, dy, static_cast<hipStream_t>(stream));
+  return launch_bn_grad_input(g, y, coef, S, C, L, dy, nullptr, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_bn_grad_input_amax(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy,
+                             float *amax, void *stream) {
+  if (!g || !y || !coef || !dy || !amax) return fail(SJHIP_ERR_INVALID, "bn_grad_input_amax: NULL buffer");
+  return launch_bn_grad_input(g, y, coef, S, C, L, dy, amax, static_cast<hipStream_t>(stream));
 }
 
 int sjhip_set_tuning(const char *key, int value) {

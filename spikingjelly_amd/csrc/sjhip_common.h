@@ -447,16 +447,20 @@ int launch_stream_probe(int reads, int writes, int nontemporal, int64_t floats_p
                         float *const *out, hipStream_t stream);
 int64_t pwconv_planes_elems(int64_t rows, int64_t cols);
 int launch_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, hipStream_t stream);
-int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms, int64_t S,
-                       int64_t L, float *c, float *stats, hipStream_t stream);
+int launch_pwconv_split_weight_f16(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, float *amax_reset,
+                                   hipStream_t stream);
+int launch_pwconv_amax(const float *x, int64_t n, float *amax, hipStream_t stream);
+int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms,
+                       const float *b_amax, int64_t S, int64_t L, float *c, float *stats, hipStream_t stream);
 int64_t pwconv_gemm_stats_rows(int64_t K, int64_t S, int64_t L);
 int64_t pwconv_dw_workspace_floats(int64_t M, int64_t N, int64_t S);
-int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int x_terms, int64_t S, int64_t M, int64_t N,
-                              int64_t L, float *dw, float *workspace, hipStream_t stream);
+int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *dy_amax, const float *x, int x_terms,
+                              const float *x_amax, int64_t S, int64_t M, int64_t N, int64_t L, float *dw, float *workspace,
+                              hipStream_t stream);
 int launch_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, hipStream_t stream);
 int launch_bn_finalize(const float *partial, int64_t rows, int64_t count, int64_t C, const float *gamma, const float *beta, float eps,
                        float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
-                       float *invstd, hipStream_t stream);
+                       float *invstd, int64_t *batches_tracked, hipStream_t stream);
 int launch_bn_lif_forward(int neuron, const sjhip_neuron_params &p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
                           const float *scale, const float *shift, const float *v_init, float *spike_seq, uint8_t *spike_bits,
                           float *v_last, hipStream_t stream);
@@ -465,8 +469,8 @@ int launch_bn_lif_backward(int neuron, const sjhip_neuron_params &p, int64_t T, 
                            const float *grad_v_last, float *grad_z, float *grad_v_init, float *partial, hipStream_t stream);
 int launch_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64_t C, int64_t L, int training, const float *gamma,
                                 const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef,
-                                hipStream_t stream);
-int launch_bn_grad_input(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy,
+                                float *amax_reset, hipStream_t stream);
+int launch_bn_grad_input(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy, float *amax,
                          hipStream_t stream);
 
 }  // namespace sjhip

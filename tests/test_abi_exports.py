@@ -216,7 +216,31 @@ def test_convolution_statistics_arguments_without_a_device():
     assert rc == -1 and b"NULL" in lib.sjhip_last_error()
     rc = lib.sjhip_pwconv_gemm_stats(16, 3, 8, 0, 16, 3, 1, 4, 16, 16, None)
     assert rc == -1 and b"K=0" in lib.sjhip_last_error()
-    rc = lib.sjhip_bn_finalize_rows(None, 4, 16, 8, None, None, 1e-5, 0.1, None, None, 16, 16, 16, 16, None)
+    rc = lib.sjhip_bn_finalize_rows(None, 4, 16, 8, None, None, 1e-5, 0.1, None, None, 16, 16, 16, 16, None, None)
     assert rc == -1 and b"NULL" in lib.sjhip_last_error()
-    rc = lib.sjhip_bn_finalize_rows(16, 0, 16, 8, None, None, 1e-5, 0.1, None, None, 16, 16, 16, 16, None)
+    rc = lib.sjhip_bn_finalize_rows(16, 0, 16, 8, None, None, 1e-5, 0.1, None, None, 16, 16, 16, 16, None, None)
     assert rc == -1 and b"rows=0" in lib.sjhip_last_error()
+
+
+def test_fp16_split_convolution_arguments_without_a_device():
+    """The fp16 GEMM entry points refuse what they cannot run before anything is launched: bf16 entry points given fp16
+    term codes, activation terms other than 1 or 2, two terms without the scale of their tensor."""
+    lib = L.load()
+    rc = lib.sjhip_pwconv_gemm(16, 18, 8, 8, 16, 2, 1, 4, 16, None)
+    assert rc == -2 and b"sjhip_pwconv_gemm_f16" in lib.sjhip_last_error()
+    rc = lib.sjhip_pwconv_grad_weight(16, 18, 16, 2, 1, 8, 8, 4, 16, 16, None)
+    assert rc == -2 and b"bf16" in lib.sjhip_last_error()
+    rc = lib.sjhip_pwconv_gemm_f16(16, 8, 8, 16, 3, 16, 1, 4, 16, None, None)
+    assert rc == -2 and b"1 or 2" in lib.sjhip_last_error()
+    rc = lib.sjhip_pwconv_gemm_f16(16, 8, 8, 16, 2, None, 1, 4, 16, None, None)
+    assert rc == -1 and b"sjhip_pwconv_amax" in lib.sjhip_last_error()
+    rc = lib.sjhip_pwconv_gemm_f16(None, 8, 8, 16, 1, None, 1, 4, 16, None, None)
+    assert rc == -1 and b"NULL" in lib.sjhip_last_error()
+    rc = lib.sjhip_pwconv_grad_weight_f16(16, None, 16, 1, None, 1, 8, 8, 4, 16, 16, None)
+    assert rc == -1 and b"NULL" in lib.sjhip_last_error()
+    rc = lib.sjhip_pwconv_grad_weight_f16(16, 16, 16, 2, None, 1, 8, 8, 4, 16, 16, None)
+    assert rc == -1 and b"sjhip_pwconv_amax" in lib.sjhip_last_error()
+    rc = lib.sjhip_pwconv_amax(16, 0, 16, None)
+    assert rc == -1 and b"n=0" in lib.sjhip_last_error()
+    rc = lib.sjhip_pwconv_split_weight_f16(16, 8, 8, 0, 8, None, None)
+    assert rc == -2 and b"aligned" in lib.sjhip_last_error()

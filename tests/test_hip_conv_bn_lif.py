@@ -126,6 +126,160 @@ def test_gemm_over_several_launches(C):
     assert float(((sums[:, 1] - want_q).abs() / want_q).max()) < 1e-6
 
 
+# ---- the same GEMMs on two fp16 terms of scaled operands -----------------------------------------------------------
+def _wide(shape, seed, decades, overall):
+    """Normal values whose rows (second to last index) are spread over ``decades`` decades, times ``overall``."""
+    base = seeded_randn(shape, seed, 0.05, 1.0)
+    spread = 10.0 ** (seeded_randn(shape[:-1] + (1,), seed + 1000, 0.0, 1.0).clamp(-1.5, 1.5) * decades / 3.0)
+    return base * spread * overall
+
+
+@pytest.mark.parametrize("S,M,Kd,Lp", SHAPES)
+@pytest.mark.parametrize("transpose", [False, True])
+@pytest.mark.parametrize("w_scale,x_scale", [(1.0, 1.0), (3e-2, 1e-6), (1e-20, 1e12)])
+def test_gemm_with_two_fp16_terms_has_fp32_accuracy(C, S, M, Kd, Lp, transpose, w_scale, x_scale):
+    """Operands spread over four decades per tensor and placed anywhere in the fp32 range: the error stays within the
+    bound of an fp32 dot product (the same bound as the three-term bf16 test), and is on average a few 2^-24 of
+    ``sum |a||b|``."""
+    F = C.F16 | 2
+    w = _wide((Kd, M) if transpose else (M, Kd), 11, 4.0, w_scale)
+    x = _wide((S, Kd, Lp), 12, 4.0, x_scale)
+    planes = C.split_weight(w.cuda(), transpose, F)
+    got = C.pw_gemm(planes, F, M, Kd, x.cuda(), F).cpu().double()
+    a = (w.t() if transpose else w).double()
+    want = torch.einsum("mk,skl->sml", a, x.double())
+    bound = torch.einsum("mk,skl->sml", a.abs(), x.double().abs()).clamp_min(1e-300)
+    rel = (got - want).abs() / bound
+    assert torch.isfinite(got).all()
+    assert float(rel.max()) < 2e-6
+    assert float(rel.mean()) < 2e-7
+    # the largest magnitude handed in is the one found inside; twice as much is still safe (one bit less headroom used)
+    assert torch.equal(C.pw_gemm(planes, F, M, Kd, x.cuda(), F, False, C.amax(x.cuda())).cpu().double(), got)
+    got2 = C.pw_gemm(planes, F, M, Kd, x.cuda(), F, False, C.amax(x.cuda()) * 2.0).cpu().double()
+    assert float(((got2 - want).abs() / bound).max()) < 2e-6
+
+
+@pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (4, 384, 384, 196)])
+def test_fp16_gemm_is_exact_on_spikes_times_dyadic_weights(C, S, M, Kd, Lp):
+    g = torch.Generator().manual_seed(13)
+    w = torch.randint(-64, 65, (M, Kd), generator=g).float() / 64.0
+    w = w * 2.0 ** torch.randint(-30, 20, (M, 1), generator=g).float()   # any power of two per row: the row scale takes it out
+    x = (torch.rand((S, Kd, Lp), generator=g) < 0.3).float()
+    want = torch.einsum("mk,skl->sml", w.double(), x.double()).float()
+    F = C.F16 | 2
+    planes = C.split_weight(w.cuda(), False, F)
+    assert torch.equal(C.pw_gemm(planes, F, M, Kd, x.cuda(), C.F16 | 1).cpu(), want)
+    assert torch.equal(C.pw_gemm(planes, F, M, Kd, x.cuda(), F).cpu(), want)
+    zero = C.pw_gemm(planes, F, M, Kd, torch.zeros_like(x).cuda(), F)
+    assert torch.equal(zero, torch.zeros_like(zero))
+    planes0 = C.split_weight(torch.zeros_like(w).cuda(), False, F)
+    assert not C.pw_gemm(planes0, F, M, Kd, x.cuda(), F).any()
+
+
+def test_amax(C):
+    """``amax(x)`` is the largest magnitude among the numbers of ``x``, for any length and alignment, and folds into what
+    the word already holds."""
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+
+    for n, top in ((1, 1.0), (7, 3.0), (1000, 0.75), (4099, 1e-30), (1 << 20, 262016.0), (5, 0.0), (9, float("inf")),
+                   (3 * (1 << 20) + 5, 17.5)):
+        x = seeded_randn((n + 1,), n, 0.0, 1.0).clamp(-1, 1) * (top if top not in (0.0, float("inf")) else 1.0) * 0.99
+        if top == 0.0:
+            x.zero_()
+        x[n // 2 + 1] = -top
+        top = abs(float(x[n // 2 + 1]))   # as fp32 holds it
+        assert float(C.amax(x.cuda()[1:]).max()) == top, (n, top)
+        words = torch.zeros(256, device="cuda")   # the C entry point on an address 4 bytes past an aligned one
+        xs = x.cuda()[1:]
+        L.check(L.load().sjhip_pwconv_amax(xs.data_ptr(), n, words.data_ptr(), L.current_stream_ptr(xs.device)), "amax")
+        assert float(words.max()) == top and float(words.min()) >= 0.0
+        words[3] = 1e30
+        L.check(L.load().sjhip_pwconv_amax(xs.data_ptr(), n, words.data_ptr(), L.current_stream_ptr(xs.device)), "amax")
+        assert float(words.max()) == max(top, float(torch.tensor(1e30)))
+    nan = torch.tensor([1.0, float("nan"), -2.0, 0.5]).cuda()
+    assert float(C.amax(nan).max()) == 2.0
+
+
+@pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (1, 7, 3, 4), (4, 130, 257, 36), (16, 1152, 384, 196)])
+@pytest.mark.parametrize("spikes", [False, True])
+def test_fp16_gemm_leaves_the_batch_norm_sums_of_its_output(C, S, M, Kd, Lp, spikes):
+    F = C.F16 | 2
+    xt = C.F16 | 1 if spikes else F
+    w = _wide((M, Kd), 31, 2.0, 0.1)
+    x = (seeded_randn((S, Kd, Lp), 32, 0.0, 1.0) > 0.3).float() if spikes else _wide((S, Kd, Lp), 32, 2.0, 5.0)
+    planes = C.split_weight(w.cuda(), False, F)
+    plain = C.pw_gemm(planes, F, M, Kd, x.cuda(), xt)
+    got, partial = C.pw_gemm(planes, F, M, Kd, x.cuda(), xt, stats=True)
+    assert torch.equal(got, plain)
+    y = got.double()
+    sums = partial.double().sum(0).cpu()
+    want_s, want_q = y.sum((0, 2)).cpu(), (y * y).sum((0, 2)).cpu()
+    abs_s = y.abs().sum((0, 2)).cpu().clamp_min(1e-30)
+    assert float(((sums[:, 0] - want_s).abs() / abs_s).max()) < 1e-6
+    assert float(((sums[:, 1] - want_q).abs() / want_q.clamp_min(1e-30)).max()) < 1e-6
+
+
+@pytest.mark.parametrize("S,M,N,Lp", [(3, 100, 50, 12), (9, 130, 257, 36), (16, 384, 384, 196), (2, 1152, 384, 196), (64, 64, 48, 8)])
+@pytest.mark.parametrize("spikes", [False, True])
+@pytest.mark.parametrize("dy_scale", [1.0, 1e-9])
+def test_fp16_grad_weight_gemm(C, S, M, N, Lp, spikes, dy_scale):
+    F = C.F16 | 2
+    dy = _wide((S, M, Lp), 21, 4.0, dy_scale)
+    x = (seeded_randn((S, N, Lp), 22, 0.0, 1.0) > 0.5).float() if spikes else _wide((S, N, Lp), 22, 4.0, 30.0)
+    got = C.pw_grad_weight(dy.cuda(), F, x.cuda(), C.F16 | 1 if spikes else F).cpu().double()
+    want = torch.einsum("sml,snl->mn", dy.double(), x.double())
+    bound = torch.einsum("sml,snl->mn", dy.double().abs(), x.double().abs()).clamp_min(1e-300)
+    rel = (got - want).abs() / bound
+    assert float(rel.max()) < 2e-6 and float(rel.mean()) < 2e-7
+
+
+@pytest.mark.parametrize("S,Cc,Lp", [(3, 5, 12), (16, 384, 196), (7, 33, 4), (300, 64, 100)])
+def test_bn_grad_input_leaves_the_largest_magnitude_of_its_output(C, S, Cc, Lp):
+    """``sjhip_bn_grad_input_amax``: the same ``dy`` as the plain call, and the largest magnitude a pass over it finds."""
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+
+    lib = L.load()
+    g = (seeded_randn((S, Cc, Lp), 51, 0.0, 1.0) * 1e-4).cuda()
+    y = seeded_randn((S, Cc, Lp), 52, 0.3, 2.0).cuda()
+    coef = seeded_randn((3, Cc), 53, 0.0, 1.0).cuda()
+    plain, fused = torch.empty_like(g), torch.empty_like(g)
+    word = torch.zeros((256,), dtype=torch.float32, device="cuda")
+    stream = L.current_stream_ptr(g.device)
+    L.check(lib.sjhip_bn_grad_input(g.data_ptr(), y.data_ptr(), coef.data_ptr(), S, Cc, Lp, plain.data_ptr(), stream), "plain")
+    L.check(lib.sjhip_bn_grad_input_amax(g.data_ptr(), y.data_ptr(), coef.data_ptr(), S, Cc, Lp, fused.data_ptr(),
+                                         word.data_ptr(), stream), "fused")
+    assert torch.equal(plain, fused)
+    assert float(word.max()) == float(plain.abs().max()) == float(C.amax(plain).max())
+
+
+def test_launches_that_clear_an_amax_buffer_and_count_the_batch(C):
+    """The fp16 weight split and the batch-norm backward's coefficient kernel set a given amax buffer to zero (so that the
+    launch that folds the maxima next needs no fill in front of it); the batch-norm forward's finalize adds 1 to the
+    counter of batches."""
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+    from spikingjelly_amd.activation_based.hip_kernel import neuron_kernel as K
+
+    buf = torch.full((256,), 1e30, device="cuda")
+    C.split_weight(seeded_randn((40, 24), 61, 0.0, 1.0).cuda(), False, C.F16 | 2, buf)
+    assert not buf.any()
+    T, B, Cc, Lp = 4, 3, 10, 12
+    y = seeded_randn((T, B, Cc, Lp), 62, 0.4, 1.5).cuda()
+    gamma, beta = seeded_randn((Cc,), 63, 1.0, 0.2).cuda(), seeded_randn((Cc,), 64, 0.6, 0.3).cuda()
+    tracked = torch.tensor(41, dtype=torch.int64, device="cuda")
+    bn_map = C._bn_map(y.flatten(0, 1), gamma, beta, None, None, True, 0.1, 1e-5, None, tracked)
+    assert int(tracked) == 42
+    spec = (2.0, 1.0, 0.0, K._flags(False, False, True, 0), no.SG_IDS["sigmoid"], no.SG_DEFAULT_ALPHA["sigmoid"])
+    v0 = torch.zeros((1,), device="cuda").expand(B, Cc, Lp)
+    gs = seeded_randn((T, B, Cc, Lp), 65).cuda()
+    for _ in range(3):   # the buffer comes from torch.empty: whatever it held before must not survive
+        poison = torch.full((256,), 1e30, device="cuda")
+        del poison
+        dy, _, _, _, dy_amax = C._bn_lif_backward(y, bn_map, gamma, v0, spec, True, gs, None, False, True)
+        assert float(dy_amax.max()) == float(dy.abs().max())
+    plain = C._bn_lif_backward(y, bn_map, gamma, v0, spec, True, gs, None, False)[0]
+    assert torch.equal(plain, dy)
+
+
 @pytest.mark.parametrize("S,M,N,Lp", [(3, 100, 50, 12), (9, 130, 257, 36), (16, 384, 384, 196), (2, 1152, 384, 196), (64, 64, 48, 8)])
 @pytest.mark.parametrize("spikes", [False, True])
 def test_grad_weight_gemm(C, S, M, N, Lp, spikes):
