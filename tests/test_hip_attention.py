@@ -73,10 +73,19 @@ def test_unsupported_shapes_raise():
         hip_ssa_forward(torch.zeros(1, 3, 1, 32, 16), 0.125)
 
 
-def test_block_hip_backend_equals_torch_backend_config5_reduced():
-    """Config 5 at reduced batch: T=4, tokens 196, D=384, 12 heads.  Same weights, same device: the 1x1
-    convolutions are identical, the LIF kernels are bit-exact and the contraction is exact, so the hip block
-    must reproduce the torch block's spikes exactly; gradients agree to fp32 accuracy."""
+@pytest.mark.parametrize("fused", [False, True])
+def test_block_hip_backend_equals_torch_backend_config5_reduced(fused, monkeypatch):
+    """Config 5 at reduced batch: T=4, tokens 196, D=384, 12 heads, same weights, same device.  With torch's
+    convolutions and batch norm around the hip neurons (``hip_fuse_conv_bn_lif = False``) the 1x1 convolutions are
+    identical, the LIF kernels are bit-exact and the contraction is exact, so the hip block reproduces the torch block's
+    spikes exactly and its gradients to fp32 accuracy.  With the library's own convolution GEMMs (the default) the
+    pre-activations differ from torch's in the last bits, so a neuron within rounding of its threshold may fire
+    differently; such a flip changes the gradients of its own sample (and, through the batch statistics, a few elements
+    elsewhere): all but a few of the 8 samples must agree to fp32 accuracy in all but 1e-3 of their elements, and the
+    output spikes in all but 1e-4 of the positions."""
+    from spikingjelly_amd import configure
+
+    monkeypatch.setattr(configure, "hip_fuse_conv_bn_lif", fused)
     torch.manual_seed(1005)
     a = layer.SpikingSelfAttention(384, 12, backend="torch").cuda()
     b = layer.SpikingSelfAttention(384, 12, backend="hip").cuda()
@@ -85,12 +94,21 @@ def test_block_hip_backend_equals_torch_backend_config5_reduced():
     xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
     ya, yb = a(xa), b(xb)
     assert 0.0 < float(ya.detach().mean()) < 0.5
-    assert bits_equal(yb, ya)
     g = torch.randn(ya.shape, generator=torch.Generator().manual_seed(7)).cuda()
     ya.backward(g)
     yb.backward(g)
-    torch.testing.assert_close(xb.grad, xa.grad, rtol=1e-3, atol=1e-4)
     wa, wb = a.qkv_conv_bn[0].weight.grad, b.qkv_conv_bn[0].weight.grad
-    torch.testing.assert_close(wb, wa, rtol=1e-3, atol=1e-3)
+    if not fused:
+        assert bits_equal(yb, ya)
+        torch.testing.assert_close(xb.grad, xa.grad, rtol=1e-3, atol=1e-4)
+        torch.testing.assert_close(wb, wa, rtol=1e-3, atol=1e-3)
+    else:
+        assert float((yb != ya).float().mean()) < 1e-4
+        close = torch.isclose(xb.grad, xa.grad, rtol=1e-3, atol=1e-4)
+        off = (~close).float().transpose(0, 1).flatten(1).mean(1)    # fraction of elements off, per batch sample
+        assert int((off > 1e-3).sum()) <= 2, off   # (the batch statistics carry a trace of a flip into the other samples)
+        assert float((~close).float().mean()) < 0.05
+        scale = float(wa.abs().max())
+        assert float((wb - wa).abs().max()) < 0.05 * scale            # a flipped spike moves a weight gradient a little
     functional.reset_net(a)
     functional.reset_net(b)
