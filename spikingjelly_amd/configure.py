@@ -38,6 +38,10 @@ hip_half_precision_mode = "torch"
 # a pass that finds the largest magnitude), three products per pair of real operands, two when one operand is spikes;
 # accuracy of an fp32 GEMM (2^-23 of sum |a||b| measured).  "bf16": hip_conv_terms bf16 terms, no scaling, no extra pass.
 hip_conv_split = "f16"
+# True: the weight gradient of a fused convolution runs on a second stream beside its input gradient (they only share
+# their inputs), so that the blocks of one kernel fill the compute units that the last, partly filled round of the
+# other leaves idle (config 5: 1.53 -> 1.49 ms per step).  False: one after the other on the caller's stream.
+hip_conv_overlap_gradients = True
 # Number of bf16 terms with hip_conv_split = "bf16": 3 keeps the accuracy of an fp32 GEMM (six matrix-core products per
 # pair of real operands, three when one operand is spikes), 2 gives about 2^-17 relative per product at half the
 # products, 1 is a plain bf16 GEMM.
