@@ -390,7 +390,12 @@ def _make_block(dim, heads, seed):
 
 @pytest.mark.parametrize("dim,heads,T,B,tokens", [(16, 2, 3, 2, 8), (64, 2, 4, 2, 36), (48, 3, 4, 1, 196)])
 @pytest.mark.parametrize("training", [True, False])
-def test_attention_block_fused_against_float64(dim, heads, T, B, tokens, training):
+@pytest.mark.parametrize("split,overlap", [("f16", True), ("f16", False), ("bf16", True)])
+def test_attention_block_fused_against_float64(dim, heads, T, B, tokens, training, split, overlap, monkeypatch):
+    """Both splits of the convolution GEMMs' operands, and the two gradients of a convolution on two streams or one."""
+
+    monkeypatch.setattr(configure, "hip_conv_split", split)
+    monkeypatch.setattr(configure, "hip_conv_overlap_gradients", overlap)
     block = _make_block(dim, heads, 50 + dim).cuda().train(training)
     params = _block_params(block)
     g = seeded_randn((T, B, dim, tokens), 52)
@@ -424,6 +429,30 @@ def test_attention_block_fused_against_float64(dim, heads, T, B, tokens, trainin
             torch.testing.assert_close(seq[1].running_mean.cpu().double(), ref[f"{name}_running"][0], rtol=1e-5, atol=1e-6)
             torch.testing.assert_close(seq[1].running_var.cpu().double(), ref[f"{name}_running"][1], rtol=1e-5, atol=1e-6)
             assert int(seq[1].num_batches_tracked) == 1
+
+
+def test_convolution_gradients_on_two_streams_equal_those_on_one(monkeypatch):
+    """The weight gradient on a second stream beside the input gradient: the same kernels on the same data, so the same
+    bits, also when other work is queued behind them and the step is repeated."""
+
+    block = _make_block(64, 2, 61).cuda().train()
+    x = seeded_randn((4, 3, 64, 36), 62, 0.0, 2.0).cuda()
+    g = seeded_randn((4, 3, 64, 36), 63).cuda()
+    results = []
+    for overlap in (False, True, True):
+        monkeypatch.setattr(configure, "hip_conv_overlap_gradients", overlap)
+        xi = x.clone().requires_grad_()
+        for p_ in block.parameters():
+            p_.grad = None
+        functional.reset_net(block)
+        out = block(xi)
+        out.backward(g)
+        busy = (xi.grad * 2.0).sum()   # work queued right behind the backward
+        results.append([xi.grad.clone()] + [p_.grad.clone() for p_ in block.parameters()] + [busy])
+    torch.cuda.synchronize()
+    for other in results[1:]:
+        for a, b in zip(results[0], other):
+            assert torch.equal(a, b)
 
 
 def test_attention_block_fused_equals_unfused_path(monkeypatch):
