@@ -440,7 +440,7 @@ def other_workload(args) -> int:
         T, B, D, H, tokens = 4, 64, args.dim, 12, 196
         configure.hip_fuse_ssa_lif = bool(args.fuse_ssa_lif)
         configure.hip_conv_split, configure.hip_conv_terms = args.conv_split, args.terms
-        configure.hip_conv_overlap_gradients = not args.no_overlap
+        configure.hip_conv_overlap_gradients = bool(args.overlap)
         torch.manual_seed(1005)
         block = layer.SpikingSelfAttention(D, H, backend="hip").to(dev)
         x = randn((T, B, D, tokens), 1105, 0.0, 1.0, torch.float32).requires_grad_()
@@ -488,9 +488,9 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--terms", type=int, default=3, choices=[1, 2, 3],
                     help="pwconv and config5 workloads with --conv-split bf16: bf16 terms per fp32 operand")
-    ap.add_argument("--no-overlap", action="store_true",
-                    help="config5 workload: run the two gradients of a convolution one after the other on one stream (per-kernel "
-                         "durations of a trace then add up to the step)")
+    ap.add_argument("--overlap", action="store_true",
+                    help="config5 workload: run the weight gradient of a convolution on a second stream beside its input gradient "
+                         "(configure.hip_conv_overlap_gradients)")
     ap.add_argument("--conv-split", default="f16", choices=["f16", "bf16"],
                     help="pwconv and config5 workloads: how fp32 operands of the convolution GEMMs are split for the matrix cores")
     ap.add_argument("--dim", type=int, default=384, choices=[384, 768],

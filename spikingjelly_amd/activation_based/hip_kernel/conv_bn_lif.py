@@ -298,7 +298,7 @@ def _conv_backward(dy, x_seq, weight, x_exact, need_dx, need_dw, dy_amax=None, x
     x3 = x_seq.reshape(T * B, Cin, Lp)
     x_terms = _exact(terms) if x_exact else terms
     dw = dx = None
-    if (need_dw and need_dx and getattr(configure, "hip_conv_overlap_gradients", True)
+    if (need_dw and need_dx and getattr(configure, "hip_conv_overlap_gradients", False)
             and not torch.cuda.is_current_stream_capturing()):  # (a recorded graph keeps the step on the stream it records)
         # The two gradients only share their inputs: the weight gradient runs on a second stream, so that the blocks of
         # one kernel fill the compute units that the last, partly filled round of the other leaves idle.

@@ -40,8 +40,10 @@ hip_half_precision_mode = "torch"
 hip_conv_split = "f16"
 # True: the weight gradient of a fused convolution runs on a second stream beside its input gradient (they only share
 # their inputs), so that the blocks of one kernel fill the compute units that the last, partly filled round of the
-# other leaves idle (config 5: 1.53 -> 1.49 ms per step).  False: one after the other on the caller's stream.
-hip_conv_overlap_gradients = True
+# other leaves idle.  False (default): one after the other on the caller's stream.  It paid while the GEMM kernel kept
+# two blocks per compute unit (config 5: 1.51 -> 1.49 ms per step); with three it measures 1.47 ms either way (1.473,
+# 1.477, 1.467 against 1.466, 1.462, 1.463), so the simpler schedule is the default.
+hip_conv_overlap_gradients = False
 # Number of bf16 terms with hip_conv_split = "bf16": 3 keeps the accuracy of an fp32 GEMM (six matrix-core products per
 # pair of real operands, three when one operand is spikes), 2 gives about 2^-17 relative per product at half the
 # products, 1 is a plain bf16 GEMM.

@@ -79,6 +79,13 @@ constexpr int kRowBytes = 80;         // K-contiguous operand row in LDS: 32 bf1
                                       // reads of eight consecutive rows fall on all 32 banks
 constexpr int kRowPlane = kTile * kRowBytes;
 constexpr int kXcds = 8;
+#ifndef SJHIP_PW_F16_WAVES
+#define SJHIP_PW_F16_WAVES 3
+#endif
+// Wavefronts per SIMD of pw_gemm_kernel: with the fp16 split (two operand planes instead of three) 168 registers hold a
+// wavefront's state (3 spilled), and a third resident block per compute unit is worth 9 % (191 -> 174 us on the qkv
+// shape).  Not so for pw_dw_kernel, which splits both operands on the fly: 22 registers spilled, 237 -> 344 us.
+constexpr int pw_waves(bool h) { return h ? SJHIP_PW_F16_WAVES : 2; }
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   bf16x2 p;
@@ -282,7 +289,7 @@ __device__ __forceinline__ u32x4 row_fragment(const uint8_t *plane, int row, int
 }
 
 template <int TA, int TB, bool H>
-__global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) pw_gemm_kernel(const PwGemmArgs a) {
+__global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu(pw_waves(H), pw_waves(H)))) pw_gemm_kernel(const PwGemmArgs a) {
   extern __shared__ __align__(16) uint8_t lds[];
   uint8_t *As = lds;                   // [TA][128][kRowBytes]
   uint8_t *Bs = lds + TA * kRowPlane;  // [TB][128][kRowBytes], column-major: a row holds 32 k of one column
