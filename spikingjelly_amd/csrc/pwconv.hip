@@ -84,7 +84,9 @@ constexpr int kXcds = 8;
 #endif
 // Wavefronts per SIMD of pw_gemm_kernel: with the fp16 split (two operand planes instead of three) 168 registers hold a
 // wavefront's state (3 spilled), and a third resident block per compute unit is worth 9 % (191 -> 174 us on the qkv
-// shape).  Not so for pw_dw_kernel, which splits both operands on the fly: 22 registers spilled, 237 -> 344 us.
+// shape).  Not so for pw_dw_kernel, which splits both operands on the fly: 22 registers spilled, 237 -> 344 us; with
+// one tile in flight instead of two it fits without spilling and takes the same 244 us, and the attention block's
+// step 1.50 instead of 1.46 ms.
 constexpr int pw_waves(bool h) { return h ? SJHIP_PW_F16_WAVES : 2; }
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
