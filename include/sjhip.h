@@ -502,7 +502,8 @@ int sjhip_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int 
  * matrix-core work of the three-term bf16 split at the same accuracy class.  fp16 has 11 significant bits but a narrow
  * exponent range, so every operand is scaled by a power of two first (exact) and the scales are taken out of the result
  * (exact): weights per row of A, inside sjhip_pwconv_split_weight_f16; activations and gradients per tensor, by the power
- * of two that takes the tensor's largest magnitude `amax` into [2^14, 2^15) (1 for a zero, subnormal or non-finite amax),
+ * of two that takes the tensor's largest finite magnitude `amax` into [2^14, 2^15) (1 for a zero or subnormal amax;
+ * infinities and NaNs take no part in it and propagate through the products as in fp32),
  * which the kernels derive from a device buffer of SJHIP_PW_AMAX_FLOATS non-negative floats whose maximum is amax
  * (several words, so that the blocks that fold their maxima into it do not meet on one address).  An element above 2^-16 of amax is represented to 2^-23
  * relative or better, a smaller one to 2^-39 of amax; the dropped product lo*lo is below 2^-22 of hi*hi.  Measured
@@ -515,7 +516,7 @@ int sjhip_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int 
  *                                  then the inverse row scales); amax_reset: NULL, or an amax buffer that the
  *                                  launch also sets to zero (that of the activations the planes will multiply, so
  *                                  that no launch is spent on clearing it)
- *   sjhip_pwconv_amax              folds max |x| over the n elements of x (NaNs ignored) into amax[SJHIP_PW_AMAX_FLOATS]:
+ *   sjhip_pwconv_amax              folds max |x| over the finite ones of the n elements of x into amax[SJHIP_PW_AMAX_FLOATS]:
  *                                  afterwards max(amax[]) is the larger of what it was and max |x|; all zero before
  *                                  the first call for a tensor; one launch
  *   sjhip_pwconv_gemm_f16          sjhip_pwconv_gemm / sjhip_pwconv_gemm_stats (partial != NULL) on fp16 planes;

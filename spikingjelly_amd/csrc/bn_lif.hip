@@ -364,6 +364,12 @@ __global__ void __launch_bounds__(256) bn_backward_finalize_kernel(const float *
   }
 }
 
+// |x| of a number, 0 for an infinity or a NaN (they take no part in choosing the scale of the tensor)
+__device__ __forceinline__ float finite_abs(float x) {
+  const float a = fabsf(x);
+  return a <= 3.4028234663852886e38f ? a : 0.0f;
+}
+
 // dy = p_c g + q_c y + r_c over the flattened [S * C * L] tensor; dy may be g itself.  With AMAX every block also folds
 // the largest |dy| it wrote into word (block % SJHIP_PW_AMAX_FLOATS) of amax_bits, bit patterns of non-negative floats
 // (they order like unsigned integers, and a maximum does not depend on the order it is taken in), with an atomic whose
@@ -384,7 +390,7 @@ __global__ void __launch_bounds__(256) bn_grad_input_kernel(const float *g, cons
     o.z = fmaf(p, gv.z, fmaf(q, yv.z, r));
     o.w = fmaf(p, gv.w, fmaf(q, yv.w, r));
     *reinterpret_cast<f32x4 *>(dy + i) = o;
-    if (AMAX) amax = fmaxf(fmaxf(fabsf(o.x), fabsf(o.y)), fmaxf(fabsf(o.z), fabsf(o.w)));
+    if (AMAX) amax = fmaxf(fmaxf(finite_abs(o.x), finite_abs(o.y)), fmaxf(finite_abs(o.z), finite_abs(o.w)));
   }
   if (AMAX) {
     __shared__ float part[4];

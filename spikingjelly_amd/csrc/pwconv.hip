@@ -124,6 +124,13 @@ template <int TERMS, bool H = false> __device__ __forceinline__ void split_pair(
   }
 }
 
+// |x| of a number, 0 for an infinity or a NaN: non-finite elements take no part in choosing a scale (they still
+// propagate through the products as they would in fp32).
+__device__ __forceinline__ float finite_abs(float x) {
+  const float a = fabsf(x);
+  return a <= 3.4028234663852886e38f ? a : 0.0f;
+}
+
 // The power of two that brings a largest magnitude `amax` into [2^14, 2^15), and its inverse; 1 for a zero, subnormal
 // or non-finite amax.  Multiplying by either is exact.
 __device__ __forceinline__ void scale_for(float amax, float &scale, float &inverse) {
@@ -177,12 +184,15 @@ __global__ void __launch_bounds__(256) split_weight_f16_kernel(const float *src,
   const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= rows_pad) return;
   float amax = 0.0f;
-  if (r < rows)
-    for (int64_t c = lane; c < cols; c += 64) amax = fmaxf(amax, fabsf(src[r * ld_r + c * ld_c]));
+  if (r < rows) {
+#pragma unroll 8
+    for (int64_t c = lane; c < cols; c += 64) amax = fmaxf(amax, finite_abs(src[r * ld_r + c * ld_c]));
+  }
 #pragma unroll
   for (int d = 32; d > 0; d >>= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
   float scale, inverse;
   scale_for(amax, scale, inverse);
+#pragma unroll 4
   for (int64_t c = 2 * lane; c < cols_pad; c += 128) {
     float x0 = 0.0f, x1 = 0.0f;
     if (r < rows) {
@@ -229,11 +239,11 @@ __global__ void __launch_bounds__(256) amax_kernel(const float *x, int64_t n, un
     const int64_t n4 = n / 4;
     for (int64_t i = i0; i < n4; i += stride) {
       const f32x4 v = __builtin_nontemporal_load(x4 + i);
-      amax = fmaxf(fmaxf(amax, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
+      amax = fmaxf(fmaxf(amax, fmaxf(finite_abs(v.x), finite_abs(v.y))), fmaxf(finite_abs(v.z), finite_abs(v.w)));
     }
-    for (int64_t i = 4 * n4 + i0; i < n; i += stride) amax = fmaxf(amax, fabsf(x[i]));
+    for (int64_t i = 4 * n4 + i0; i < n; i += stride) amax = fmaxf(amax, finite_abs(x[i]));
   } else {
-    for (int64_t i = i0; i < n; i += stride) amax = fmaxf(amax, fabsf(x[i]));
+    for (int64_t i = i0; i < n; i += stride) amax = fmaxf(amax, finite_abs(x[i]));
   }
 #pragma unroll
   for (int d = 32; d > 0; d >>= 1) amax = fmaxf(amax, __shfl_xor(amax, d));

@@ -176,14 +176,32 @@ def test_fp16_gemm_is_exact_on_spikes_times_dyadic_weights(C, S, M, Kd, Lp):
     assert not C.pw_gemm(planes0, F, M, Kd, x.cuda(), F).any()
 
 
+def test_fp16_gemm_with_an_infinity_in_the_activations(C):
+    """An infinity (or NaN) takes no part in the scale: the outputs that do not touch it are as accurate as without it,
+    those that do are non-finite as in fp32."""
+    F = C.F16 | 2
+    S, M, Kd, Lp = 2, 40, 24, 8
+    w = seeded_randn((M, Kd), 71, 0.0, 1.0)
+    x = seeded_randn((S, Kd, Lp), 72, 0.0, 3e4)   # finite values beyond fp16's range when left unscaled
+    x[1, 5, 3] = float("inf")
+    x[0, 2, 6] = float("nan")
+    got = C.pw_gemm(C.split_weight(w.cuda(), False, F), F, M, Kd, x.cuda(), F).cpu().double()
+    want = torch.einsum("mk,skl->sml", w.double(), x.double())
+    touched = torch.zeros((S, Lp), dtype=torch.bool)
+    touched[1, 3] = touched[0, 6] = True
+    clean = ~touched[:, None, :].expand(S, M, Lp)
+    assert not torch.isfinite(got[~clean]).any()
+    bound = torch.einsum("mk,skl->sml", w.double().abs(), torch.nan_to_num(x.double(), nan=0.0, posinf=0.0).abs())
+    assert float(((got - want).abs() / bound)[clean].max()) < 2e-6
+
+
 def test_amax(C):
     """``amax(x)`` is the largest magnitude among the numbers of ``x``, for any length and alignment, and folds into what
     the word already holds."""
     from spikingjelly_amd.activation_based.hip_kernel import library as L
 
-    for n, top in ((1, 1.0), (7, 3.0), (1000, 0.75), (4099, 1e-30), (1 << 20, 262016.0), (5, 0.0), (9, float("inf")),
-                   (3 * (1 << 20) + 5, 17.5)):
-        x = seeded_randn((n + 1,), n, 0.0, 1.0).clamp(-1, 1) * (top if top not in (0.0, float("inf")) else 1.0) * 0.99
+    for n, top in ((1, 1.0), (7, 3.0), (1000, 0.75), (4099, 1e-30), (1 << 20, 262016.0), (5, 0.0), (3 * (1 << 20) + 5, 17.5)):
+        x = seeded_randn((n + 1,), n, 0.0, 1.0).clamp(-1, 1) * (top if top != 0.0 else 1.0) * 0.99
         if top == 0.0:
             x.zero_()
         x[n // 2 + 1] = -top
@@ -196,8 +214,8 @@ def test_amax(C):
         words[3] = 1e30
         L.check(L.load().sjhip_pwconv_amax(xs.data_ptr(), n, words.data_ptr(), L.current_stream_ptr(xs.device)), "amax")
         assert float(words.max()) == max(top, float(torch.tensor(1e30)))
-    nan = torch.tensor([1.0, float("nan"), -2.0, 0.5]).cuda()
-    assert float(C.amax(nan).max()) == 2.0
+    odd = torch.tensor([1.0, float("nan"), -2.0, 0.5, float("-inf"), float("inf")]).cuda()
+    assert float(C.amax(odd).max()) == 2.0   # the largest magnitude among the finite elements
 
 
 @pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (1, 7, 3, 4), (4, 130, 257, 36), (16, 1152, 384, 196)])
