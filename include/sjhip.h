@@ -533,6 +533,15 @@ int sjhip_pwconv_gemm_f16(const uint16_t *a_planes, int64_t M, int64_t K, const 
                           int64_t S, int64_t L, float *c, float *partial, void *stream);
 int sjhip_pwconv_grad_weight_f16(const float *dy, const float *dy_amax, const float *x, int x_terms, const float *x_amax,
                                  int64_t S, int64_t M, int64_t N, int64_t L, float *dw, float *workspace, void *stream);
+/* The two of them that read a spike tensor, with the spikes bit-packed (the layout of sjhip_bit_pack over the flattened
+ * [S][K][L] or [S][N][L] tensor: 1/32 of the bytes of fp32 spikes): the projection convolution of the reference's
+ * SpikingSelfAttention reads the attention neuron's spikes (layer/attention.py:378-384), which that neuron can write as
+ * bits (sjhip_neuron_forward_packed).  K * L (N * L) must be a multiple of 8, L even (a multiple of 4 for the weight
+ * gradient); results equal those of the fp32-spike calls bit for bit. */
+int sjhip_pwconv_gemm_f16_bits(const uint16_t *a_planes, int64_t M, int64_t K, const uint8_t *b_bits, int64_t S, int64_t L,
+                               float *c, float *partial, void *stream);
+int sjhip_pwconv_grad_weight_f16_bits(const float *dy, const float *dy_amax, const uint8_t *x_bits, int64_t S, int64_t M,
+                                      int64_t N, int64_t L, float *dw, float *workspace, void *stream);
 
 /*
  * Batch normalisation fused with the multi-step IF / LIF neuron behind it, for fp32 activations [T][B][C][L]

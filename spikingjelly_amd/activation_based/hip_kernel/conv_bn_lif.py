@@ -32,7 +32,7 @@ from . import library as L
 from . import neuron_kernel as K
 
 __all__ = ["supported", "bn_lif", "conv_bn_lif", "conv_bn_lif_ssa", "conv_bn_lif_ssa_lif", "split_weight", "pw_gemm",
-           "pw_grad_weight", "amax", "F16"]
+           "pw_grad_weight", "pw_gemm_bits", "pw_grad_weight_bits", "amax", "F16"]
 
 MAX_REPLAY_STEPS = 16  # the backward replays the neuron with h of every step in registers
 
@@ -161,6 +161,37 @@ def pw_grad_weight(dy: torch.Tensor, dy_terms: int, x: torch.Tensor, x_terms: in
             rc = lib.sjhip_pwconv_grad_weight(dy.data_ptr(), dy_terms, x.data_ptr(), x_terms, S, M, N, Lp, dw.data_ptr(),
                                               ws.data_ptr(), _stream(dy))
     L.check(rc, "pwconv_grad_weight")
+    return dw
+
+
+def pw_gemm_bits(planes: torch.Tensor, M: int, Kdim: int, bits: torch.Tensor, S: int, Lp: int, stats: bool = False):
+    """``pw_gemm`` on fp16 weight planes for a spike tensor ``[S, K, L]`` that arrives bit-packed (``bits``: the byte
+    array of ``bit_spike_compress`` / ``sjhip_neuron_forward_packed``); ``K * L`` a multiple of 8."""
+    c = torch.empty((S, M, Lp), dtype=torch.float32, device=bits.device)
+    lib = L.load()
+    partial = None
+    with torch.cuda.device(bits.device):
+        if stats:
+            partial = torch.empty((lib.sjhip_pwconv_gemm_stats_rows(Kdim, S, Lp), M, 2), dtype=torch.float32, device=bits.device)
+        rc = lib.sjhip_pwconv_gemm_f16_bits(planes.data_ptr(), M, Kdim, bits.data_ptr(), S, Lp, c.data_ptr(), L.ptr(partial),
+                                            _stream(bits))
+    L.check(rc, "pwconv_gemm_f16_bits")
+    return (c, partial) if stats else c
+
+
+def pw_grad_weight_bits(dy: torch.Tensor, bits: torch.Tensor, N: int, dy_amax: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``pw_grad_weight`` with two fp16 terms of ``dy [S, M, L]`` and the spike tensor ``x [S, N, L]`` bit-packed."""
+    S, M, Lp = dy.shape
+    dy = L.aligned16(dy)
+    lib = L.load()
+    ws = torch.empty(lib.sjhip_pwconv_grad_weight_workspace_floats(M, N, S), dtype=torch.float32, device=dy.device)
+    dw = torch.empty((M, N), dtype=torch.float32, device=dy.device)
+    if dy_amax is None:
+        dy_amax = amax(dy)
+    with torch.cuda.device(dy.device):
+        rc = lib.sjhip_pwconv_grad_weight_f16_bits(dy.data_ptr(), dy_amax.data_ptr(), bits.data_ptr(), S, M, N, Lp, dw.data_ptr(),
+                                                   ws.data_ptr(), _stream(dy))
+    L.check(rc, "pwconv_grad_weight_f16_bits")
     return dw
 
 

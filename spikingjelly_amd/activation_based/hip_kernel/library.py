@@ -78,6 +78,8 @@ EXPORTED_SYMBOLS = (
     "sjhip_pwconv_gemm_f16",
     "sjhip_pwconv_grad_weight_f16",
     "sjhip_bn_grad_input_amax",
+    "sjhip_pwconv_gemm_f16_bits",
+    "sjhip_pwconv_grad_weight_f16_bits",
     "sjhip_bn_stats",
     "sjhip_bn_finalize",
     "sjhip_bn_finalize_rows",
@@ -265,6 +267,12 @@ def load() -> ctypes.CDLL:
         lib.sjhip_pwconv_grad_weight_f16.restype = c_int
         lib.sjhip_pwconv_grad_weight_f16.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64,
                                                      c_int64, c_void_p, c_void_p, c_void_p]
+        lib.sjhip_pwconv_gemm_f16_bits.restype = c_int
+        lib.sjhip_pwconv_gemm_f16_bits.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p,
+                                                   c_void_p]
+        lib.sjhip_pwconv_grad_weight_f16_bits.restype = c_int
+        lib.sjhip_pwconv_grad_weight_f16_bits.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                                          c_void_p, c_void_p, c_void_p]
         lib.sjhip_bn_stats.restype = c_int
         lib.sjhip_bn_stats.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]
         lib.sjhip_bn_finalize.restype = c_int

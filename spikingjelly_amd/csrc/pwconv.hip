@@ -300,8 +300,11 @@ __device__ __forceinline__ u32x4 row_fragment(const uint8_t *plane, int row, int
   return *reinterpret_cast<const u32x4 *>(plane + row * kRowBytes + ks * 32 + (lane >> 5) * 16);
 }
 
-template <int TA, int TB, bool H>
+// BITS: b is a spike tensor that arrives bit-packed (the layout of sjhip_bit_pack over [S][K][L]: bit e % 8 of byte e / 8
+// is element e), 1/32 of the bytes of fp32 spikes; a work-item fetches the byte that holds its two columns of a row.
+template <int TA, int TB, bool H, bool BITS = false>
 __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu(pw_waves(H), pw_waves(H)))) pw_gemm_kernel(const PwGemmArgs a) {
+  static_assert(!BITS || TB == 1, "a bit-packed operand has one term");
   extern __shared__ __align__(16) uint8_t lds[];
   uint8_t *As = lds;                   // [TA][128][kRowBytes]
   uint8_t *Bs = lds + TA * kRowPlane;  // [TB][128][kRowBytes], column-major: a row holds 32 k of one column
@@ -334,10 +337,10 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   const int bk = __builtin_amdgcn_readfirstlane(wave * 8);
   const int64_t jc = j0 + bc;
   const bool col_ok = jc < a.ncols;  // L is even, so the two columns are in one sample and both valid or both not
-  uint32_t b_off = 0;
+  uint32_t b_off = 0;  // byte offset of the column pair in row 0 of its sample; with BITS the bit index
   if (col_ok) {
     const int64_t s = jc / L;
-    b_off = (uint32_t)(((s * K) * (int64_t)L + (jc - s * L)) * 4);
+    b_off = (uint32_t)(((s * K) * (int64_t)L + (jc - s * L)) * (BITS ? 1 : 4));
   }
   const bool edge_cols = __builtin_amdgcn_readfirstlane(j0 + kTile > a.ncols ? 1 : 0) != 0;
   const char *a_base = reinterpret_cast<const char *>(a.a_planes);
@@ -361,6 +364,12 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int k = k0 + bk + i;
+      if (BITS) {  // K * L is a multiple of 8 and L is even: the two bits share a byte
+        const uint32_t e = b_off + (uint32_t)(k < K ? k : K - 1) * (uint32_t)L;
+        rb[set][i].x = *reinterpret_cast<const uint8_t *>(b_base + (e >> 3));
+        rb[set][i].y = e & 7u;
+        continue;
+      }
       const char *row = b_base + (int64_t)(k < K ? k : K - 1) * L * 4;
       rb[set][i] = *reinterpret_cast<const u32x2 *>(row + b_off);
     }
@@ -382,6 +391,10 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       for (int i = 0; i < 4; ++i) {
         const u32x2 lo = rb[set][2 * i], hi = rb[set][2 * i + 1];
         float x0 = __builtin_bit_cast(float, c ? lo.y : lo.x), x1 = __builtin_bit_cast(float, c ? hi.y : hi.x);
+        if (BITS) {
+          x0 = (float)((lo.x >> (lo.y + c)) & 1u);
+          x1 = (float)((hi.x >> (hi.y + c)) & 1u);
+        }
         if (H && TB > 1) {
           x0 *= b_scale;
           x1 *= b_scale;
@@ -511,8 +524,11 @@ struct PwDwArgs {
   const float *dy_amax, *x_amax;  // fp16 terms: nullptr (no scale), or the words whose maximum is the tensor's max |.|
 };
 
-template <int TA, int TB, bool H>
+// BITS: x is a spike tensor that arrives bit-packed (as in pw_gemm_kernel); a work-item fetches the byte whose low or
+// high half holds its four consecutive positions of a row (L and N * L are multiples of 4 and 8).
+template <int TA, int TB, bool H, bool BITS = false>
 __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) pw_dw_kernel(const PwDwArgs a) {
+  static_assert(!BITS || TB == 1, "a bit-packed operand has one term");
   extern __shared__ __align__(16) uint8_t lds[];
   uint8_t *As = lds;                   // [TA][128][kRowBytes]
   uint8_t *Bs = lds + TA * kRowPlane;  // [TB][128][kRowBytes]
@@ -539,7 +555,7 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   for (int i = 0; i < 4; ++i) {
     const int row = rr + 32 * i;
     a_off[i] = (uint32_t)((m0 + row < M ? m0 + row : M - 1) * L * 4);
-    b_off[i] = (uint32_t)((n0 + row < N ? n0 + row : N - 1) * L * 4);
+    b_off[i] = (uint32_t)((n0 + row < N ? n0 + row : N - 1) * L * (BITS ? 1 : 4));  // bytes; with BITS bits
   }
   const bool edge_rows = __builtin_amdgcn_readfirstlane((m0 + kTile > M || n0 + kTile > N) ? 1 : 0) != 0;
   const char *dy_base = reinterpret_cast<const char *>(a.dy);
@@ -552,13 +568,18 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
     const int64_t s = s_begin + it / l_steps;
     const int l0 = (int)(it % l_steps) * kTileK;
     const char *pa = dy_base + (s * M) * (int64_t)L * 4;
-    const char *pb = x_base + (s * N) * (int64_t)L * 4;
+    const char *pb = x_base + (BITS ? ((s * N) * (int64_t)L >> 3) : (s * N) * (int64_t)L * 4);
     const int l = l0 + 4 * q4;
     const uint32_t l_off = (uint32_t)((l < L ? l : L - 4) * 4);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       ra[set][i] = *reinterpret_cast<const f32x4 *>(pa + (a_off[i] + l_off));
-      rb[set][i] = *reinterpret_cast<const f32x4 *>(pb + (b_off[i] + l_off));
+      if (BITS) {
+        const uint32_t e = b_off[i] + (l_off >> 2);
+        rb[set][i].x = __builtin_bit_cast(float, (uint32_t)*reinterpret_cast<const uint8_t *>(pb + (e >> 3)));
+      } else {
+        rb[set][i] = *reinterpret_cast<const f32x4 *>(pb + (b_off[i] + l_off));
+      }
     }
   };
   auto stage = [&](int64_t it, int set) {
@@ -591,6 +612,15 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       {
         uint32_t w01[TB], w23[TB];
         f32x4 v = rb[set][i];
+        if (BITS) {
+          const int l = l0 + 4 * q4;
+          const uint32_t e = b_off[i] + (uint32_t)(l < L ? l : L - 4);
+          const uint32_t four = __builtin_bit_cast(uint32_t, rb[set][i].x) >> (e & 7u);
+          v.x = (float)(four & 1u);
+          v.y = (float)((four >> 1) & 1u);
+          v.z = (float)((four >> 2) & 1u);
+          v.w = (float)((four >> 3) & 1u);
+        }
         if (H && TB > 1) v *= b_scale;
         split_pair<TB, H>(v.x, v.y, w01);
         split_pair<TB, H>(v.z, v.w, w23);
@@ -701,16 +731,18 @@ __global__ void __launch_bounds__(256) dw_reduce_kernel(const float *partials, i
 
 int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
-template <int TA, int TB, bool H = false> int launch_gemm_terms(const PwGemmArgs &a, int64_t blocks, hipStream_t stream) {
+template <int TA, int TB, bool H = false, bool BITS = false>
+int launch_gemm_terms(const PwGemmArgs &a, int64_t blocks, hipStream_t stream) {
   unsigned lds = (TA + TB) * kRowPlane;
   if (a.stats && lds < kStatLds) lds = kStatLds;
-  hipLaunchKernelGGL((pw_gemm_kernel<TA, TB, H>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
+  hipLaunchKernelGGL((pw_gemm_kernel<TA, TB, H, BITS>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
   return check_launch("pwconv_gemm");
 }
 
-template <int TA, int TB, bool H = false> int launch_dw_terms(const PwDwArgs &a, int64_t blocks, hipStream_t stream) {
+template <int TA, int TB, bool H = false, bool BITS = false>
+int launch_dw_terms(const PwDwArgs &a, int64_t blocks, hipStream_t stream) {
   const unsigned lds = (TA + TB) * kRowPlane;
-  hipLaunchKernelGGL((pw_dw_kernel<TA, TB, H>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
+  hipLaunchKernelGGL((pw_dw_kernel<TA, TB, H, BITS>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
   return check_launch("pwconv_grad_weight");
 }
 
@@ -779,9 +811,11 @@ int64_t pwconv_gemm_stats_rows(int64_t K, int64_t S, int64_t L) {
 }
 
 int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms,
-                       const float *b_amax, int64_t S, int64_t L, float *c, float *stats, hipStream_t stream) {
-  if (L % 2 != 0 || !aligned16(a_planes) || (reinterpret_cast<uintptr_t>(b) & 7u))
+                       const float *b_amax, int64_t S, int64_t L, float *c, float *stats, hipStream_t stream, bool b_bits) {
+  if (L % 2 != 0 || !aligned16(a_planes) || (!b_bits && (reinterpret_cast<uintptr_t>(b) & 7u)))
     return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: L=%lld must be even, the weight planes 16-byte and the activations 8-byte aligned", (long long)L);
+  if (b_bits && ((K * L) % 8 != 0 || a_terms != (SJHIP_PW_F16 | 2) || b_terms != 1))
+    return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: bit-packed activations need K*L=%lld to be a multiple of 8, fp16 weight planes and one activation term", (long long)(K * L));
   const int64_t limit = kPwOffsetLimit;
   if (round_up(M, kTile) * round_up(K, kTileK) >= limit || K * L >= limit)
     return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: M=%lld K=%lld L=%lld", (long long)M, (long long)K, (long long)L);
@@ -790,7 +824,8 @@ int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t
   for (int64_t s0 = 0; s0 < S; s0 += s_step) {
     const int64_t s_count = S - s0 < s_step ? S - s0 : s_step;
     PwGemmArgs a;
-    a.a_planes = a_planes; a.b = b + s0 * K * L; a.c = c + s0 * M * L;
+    a.a_planes = a_planes; a.c = c + s0 * M * L;
+    a.b = b_bits ? reinterpret_cast<const float *>(reinterpret_cast<const uint8_t *>(b) + s0 * K * L / 8) : b + s0 * K * L;
     a.M = (int)M; a.K = (int)K; a.K_pad = (int)round_up(K, kTileK); a.L = (int)L;
     a.plane_stride = round_up(M, kTile) * a.K_pad;
     a.ncols = s_count * L;
@@ -809,7 +844,9 @@ int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t
       case 21: rc = launch_gemm_terms<2, 1>(a, blocks, stream); break;
       case 11: rc = launch_gemm_terms<1, 1>(a, blocks, stream); break;
       case (SJHIP_PW_F16 | 2) * 10 + 2: rc = launch_gemm_terms<2, 2, true>(a, blocks, stream); break;
-      case (SJHIP_PW_F16 | 2) * 10 + 1: rc = launch_gemm_terms<2, 1, true>(a, blocks, stream); break;
+      case (SJHIP_PW_F16 | 2) * 10 + 1:
+        rc = b_bits ? launch_gemm_terms<2, 1, true, true>(a, blocks, stream) : launch_gemm_terms<2, 1, true>(a, blocks, stream);
+        break;
       default: return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: %d weight terms with %d activation terms (bf16: 3/3, 3/1, 2/2, 2/1, 1/1; fp16: 2/2, 2/1)", a_terms, b_terms);
     }
     if (rc != SJHIP_OK) return rc;
@@ -825,8 +862,10 @@ int64_t pwconv_dw_workspace_floats(int64_t M, int64_t N, int64_t S) {
 
 int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *dy_amax, const float *x, int x_terms,
                               const float *x_amax, int64_t S, int64_t M, int64_t N, int64_t L, float *dw, float *workspace,
-                              hipStream_t stream) {
-  if (L % 4 != 0 || !aligned16(dy) || !aligned16(x))
+                              hipStream_t stream, bool x_bits) {
+  if (x_bits && ((N * L) % 8 != 0 || dy_terms != (SJHIP_PW_F16 | 2) || x_terms != 1))
+    return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight: bit-packed activations need N*L=%lld to be a multiple of 8, two fp16 gradient terms and one activation term", (long long)(N * L));
+  if (L % 4 != 0 || !aligned16(dy) || (!x_bits && !aligned16(x)))
     return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight: L=%lld must be a multiple of 4 and the tensors 16-byte aligned", (long long)L);
   if (M * L >= (int64_t(1) << 30) || N * L >= (int64_t(1) << 30) || M * N >= (int64_t(1) << 40))  // 32-bit per-lane byte offsets
     return fail(SJHIP_ERR_TOO_LARGE, "pwconv_grad_weight: M=%lld N=%lld L=%lld", (long long)M, (long long)N, (long long)L);
@@ -851,7 +890,9 @@ int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *dy_ama
       case 21: rc = launch_dw_terms<2, 1>(a, blocks, stream); break;
       case 11: rc = launch_dw_terms<1, 1>(a, blocks, stream); break;
       case (SJHIP_PW_F16 | 2) * 10 + 2: rc = launch_dw_terms<2, 2, true>(a, blocks, stream); break;
-      case (SJHIP_PW_F16 | 2) * 10 + 1: rc = launch_dw_terms<2, 1, true>(a, blocks, stream); break;
+      case (SJHIP_PW_F16 | 2) * 10 + 1:
+        rc = x_bits ? launch_dw_terms<2, 1, true, true>(a, blocks, stream) : launch_dw_terms<2, 1, true>(a, blocks, stream);
+        break;
       default: return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight: %d gradient terms with %d activation terms (bf16: 3/3, 3/1, 2/2, 2/1, 1/1; fp16: 2/2, 2/1)", dy_terms, x_terms);
     }
     if (rc != SJHIP_OK) return rc;

@@ -638,6 +638,23 @@ int sjhip_pwconv_grad_weight_f16(const float *dy, const float *dy_amax, const fl
                                    workspace, static_cast<hipStream_t>(stream));
 }
 
+int sjhip_pwconv_gemm_f16_bits(const uint16_t *a_planes, int64_t M, int64_t K, const uint8_t *b_bits, int64_t S, int64_t L,
+                               float *c, float *partial, void *stream) {
+  if (!a_planes || !b_bits || !c) return fail(SJHIP_ERR_INVALID, "pwconv_gemm_f16_bits: NULL buffer");
+  if (M < 1 || K < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_gemm_f16_bits: M=%lld K=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)K, (long long)S, (long long)L);
+  if (S > (int64_t(1) << 40) / L) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm_f16_bits: S*L overflows");
+  return launch_pwconv_gemm(a_planes, SJHIP_PW_F16 | 2, M, K, reinterpret_cast<const float *>(b_bits), 1, nullptr, S, L, c, partial,
+                            static_cast<hipStream_t>(stream), true);
+}
+
+int sjhip_pwconv_grad_weight_f16_bits(const float *dy, const float *dy_amax, const uint8_t *x_bits, int64_t S, int64_t M,
+                                      int64_t N, int64_t L, float *dw, float *workspace, void *stream) {
+  if (!dy || !dy_amax || !x_bits || !dw || !workspace) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight_f16_bits: NULL buffer");
+  if (M < 1 || N < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight_f16_bits: M=%lld N=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)N, (long long)S, (long long)L);
+  return launch_pwconv_grad_weight(dy, SJHIP_PW_F16 | 2, dy_amax, reinterpret_cast<const float *>(x_bits), 1, nullptr, S, M, N, L, dw,
+                                   workspace, static_cast<hipStream_t>(stream), true);
+}
+
 int sjhip_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, void *stream) {
   if (!y || !partial) return fail(SJHIP_ERR_INVALID, "bn_stats: NULL buffer");
   return launch_bn_stats(y, S, C, L, partial, static_cast<hipStream_t>(stream));

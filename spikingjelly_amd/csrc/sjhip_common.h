@@ -451,12 +451,12 @@ int launch_pwconv_split_weight_f16(const float *w, int64_t rows, int64_t cols, i
                                    hipStream_t stream);
 int launch_pwconv_amax(const float *x, int64_t n, float *amax, hipStream_t stream);
 int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms,
-                       const float *b_amax, int64_t S, int64_t L, float *c, float *stats, hipStream_t stream);
+                       const float *b_amax, int64_t S, int64_t L, float *c, float *stats, hipStream_t stream, bool b_bits = false);
 int64_t pwconv_gemm_stats_rows(int64_t K, int64_t S, int64_t L);
 int64_t pwconv_dw_workspace_floats(int64_t M, int64_t N, int64_t S);
 int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *dy_amax, const float *x, int x_terms,
                               const float *x_amax, int64_t S, int64_t M, int64_t N, int64_t L, float *dw, float *workspace,
-                              hipStream_t stream);
+                              hipStream_t stream, bool x_bits = false);
 int launch_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, hipStream_t stream);
 int launch_bn_finalize(const float *partial, int64_t rows, int64_t count, int64_t C, const float *gamma, const float *beta, float eps,
                        float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,

@@ -195,6 +195,25 @@ def test_fp16_gemm_with_an_infinity_in_the_activations(C):
     assert float(((got - want).abs() / bound)[clean].max()) < 2e-6
 
 
+@pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (1, 7, 6, 4), (4, 130, 258, 36), (16, 384, 384, 196), (5, 1152, 384, 196)])
+def test_fp16_gemms_read_bit_packed_spikes(C, S, M, Kd, Lp):
+    """The GEMMs that take a spike tensor as bits give the results of the fp32-spike calls bit for bit: the forward with
+    its batch-norm sums, and the weight gradient."""
+    from spikingjelly_amd.activation_based.hip_kernel.compress import bit_spike_compress
+
+    F = C.F16 | 2
+    w = _wide((M, Kd), 81, 2.0, 0.1).cuda()
+    x = (seeded_randn((S, Kd, Lp), 82, 0.0, 1.0) > 0.4).float().cuda()
+    bits = bit_spike_compress(x)
+    planes = C.split_weight(w, False, F)
+    want, want_partial = C.pw_gemm(planes, F, M, Kd, x, C.F16 | 1, stats=True)
+    got, partial = C.pw_gemm_bits(planes, M, Kd, bits, S, Lp, stats=True)
+    assert torch.equal(got, want) and torch.equal(partial, want_partial)
+    assert torch.equal(C.pw_gemm_bits(planes, M, Kd, bits, S, Lp), want)
+    dy = _wide((S, M, Lp), 83, 3.0, 1e-3).cuda()
+    assert torch.equal(C.pw_grad_weight_bits(dy, bits, Kd), C.pw_grad_weight(dy, F, x, C.F16 | 1))
+
+
 def test_amax(C):
     """``amax(x)`` is the largest magnitude among the numbers of ``x``, for any length and alignment, and folds into what
     the word already holds."""
