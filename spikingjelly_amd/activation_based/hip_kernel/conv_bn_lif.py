@@ -31,7 +31,8 @@ from ... import configure
 from . import library as L
 from . import neuron_kernel as K
 
-__all__ = ["supported", "bn_lif", "conv_bn_lif", "conv_bn_lif_ssa", "conv_bn_lif_ssa_lif", "split_weight", "pw_gemm",
+__all__ = ["supported", "bn_lif", "conv_bn_lif", "conv_bn_lif_ssa", "conv_bn_lif_ssa_lif", "lif_conv_bn_lif",
+           "lif_conv_bn_lif_supported", "split_weight", "pw_gemm",
            "pw_grad_weight", "pw_gemm_bits", "pw_grad_weight_bits", "amax", "F16"]
 
 MAX_REPLAY_STEPS = 16  # the backward replays the neuron with h of every step in registers
@@ -510,6 +511,83 @@ class _ConvBnLifSsaLif(torch.autograd.Function):
                                                             grad_v_last, bool(need[4]), True)
         dx, dw = _conv_backward(dy, x_seq, weight, ctx.x_exact, bool(need[0]), bool(need[1]), dy_amax, x_amax)
         return (dx, dw, dgamma if need[2] else None, dbeta if need[3] else None, gvi, None, None, None, None, None, None, None)
+
+
+class _LifConvBnLif(torch.autograd.Function):
+    """A multi-step LIF whose spikes feed a kernel-size-1 convolution, batch norm and a second LIF, with those spikes
+    existing only bit-packed: the first neuron writes bits (``sjhip_neuron_forward_packed``), the convolution and its
+    weight gradient read bits, and the first neuron's backward replays its forward from its input.  This is the
+    ``attn_lif -> proj_conv -> proj_bn -> proj_lif`` tail of the spiking self-attention (reference
+    layer/attention.py:376-384).  Saves the first neuron's input, the bits (1/32 of the fp32 spike tensor), the
+    convolution output and the batch-norm map."""
+
+    @staticmethod
+    def forward(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec):
+        running_mean, running_var, batch_stats, momentum, eps, tracked = _bn_config(bn)
+        pre_seq = L.aligned16(pre_seq)
+        T, B, Cin, Lp = pre_seq.shape
+        Cout = weight.shape[0]
+        tau, v_th, v_reset, flags, _, _ = pre_spec
+        bits, _, pre_v_last = K._run_forward_packed(L.NEURON_LIF, pre_seq.view(T, -1), pre_v_init.flatten(), None, tau, v_th,
+                                                    v_reset, flags, False)
+        terms = _terms()
+        planes = split_weight(weight, False, terms)
+        out = pw_gemm_bits(planes, Cout, Cin, bits, T * B, Lp, batch_stats)
+        y, partial = (out[0], out[1]) if batch_stats else (out, None)
+        y = y.view(T, B, Cout, Lp)
+        bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial, tracked)
+        spikes, v_last = _bn_lif_forward(y, bn_map, v_init, spec, False)
+        return spikes, v_last, pre_v_last.view(B, Cin, Lp), y, bn_map, bits
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec = inputs
+        ctx.pre_spec, ctx.spec, ctx.batch_stats = pre_spec, spec, _bn_config(bn)[2]
+        ctx.save_for_backward(L.aligned16(pre_seq), pre_v_init, weight, gamma, v_init, output[3], output[4], output[5])
+        ctx.mark_non_differentiable(output[3], output[4], output[5])
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, grad_spikes, grad_v_last, grad_pre_v_last, _y, _map, _bits):
+        pre_seq, pre_v_init, weight, gamma, v_init, y, bn_map, bits = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        T, B, Cin, Lp = pre_seq.shape
+        Cout = weight.shape[0]
+        terms = _terms()
+        dy, dgamma, dbeta, gvi, dy_amax = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
+                                                            grad_v_last, bool(need[5]), True)
+        dy3 = dy.view(T * B, Cout, Lp)
+        if dy_amax is None:
+            dy_amax = amax(dy3)
+        dw = pw_grad_weight_bits(dy3, bits, Cin, dy_amax) if need[2] else None
+        gx = gpv = None
+        if need[0] or need[1]:
+            grad_pre_spikes = pw_gemm(split_weight(weight, True, terms), terms, Cin, Cout, dy3, terms, False, dy_amax)
+            tau, v_th, v_reset, flags, sg_id, sg_alpha = ctx.pre_spec
+            glast = grad_pre_v_last.flatten() if grad_pre_v_last is not None else None
+            gx, gpv, _ = K._run_backward(L.NEURON_LIF, grad_pre_spikes.view(T, -1), None, glast, None, pre_seq.view(T, -1),
+                                         pre_v_init.flatten(), None, tau, v_th, v_reset, flags, sg_id, sg_alpha, bool(need[1]))
+            gx = gx.view(pre_seq.shape) if need[0] else None
+            gpv = gpv.view(B, Cin, Lp) if need[1] else None
+        return (gx, gpv, dw, dgamma if need[3] else None, dbeta if need[4] else None, gvi, None, None, None)
+
+
+def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_v_init: torch.Tensor, weight: torch.Tensor, gamma, beta, v_init: torch.Tensor,
+                    bn, pre_spec, spec):
+    """``pre_seq [T, B, Cin, L]`` is the input of a LIF (``pre_spec``, state ``pre_v_init [B, Cin, L]``) whose spikes go
+    through ``weight [Cout, Cin]``, batch norm and a second LIF (``spec``, ``v_init [B, Cout, L]``).  Returns
+    ``(spikes [T, B, Cout, L], v_last, v_last of the first neuron)``.  The caller has checked ``lif_conv_bn_lif_supported``."""
+    out = _LifConvBnLif.apply(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec)
+    return out[0], out[1], out[2]
+
+
+def lif_conv_bn_lif_supported(pre_seq: torch.Tensor, need_grad: bool) -> bool:
+    """What ``supported`` asks, the fp16 split of the GEMM operands (the kernels that read bits belong to it) and a
+    spike tensor whose samples start on a byte."""
+    if not supported(pre_seq, need_grad) or not (_terms() & F16):
+        return False
+    T, B, Cin, Lp = pre_seq.shape
+    return (Cin * Lp) % 8 == 0
 
 
 def bn_lif(y_seq: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec):

@@ -126,11 +126,16 @@ class SpikingSelfAttention(nn.Module, base.MultiStepModule):
             if out is None:
                 qkv = self.qkv_lif(pre).reshape(T, N, 3, self.num_heads, local_dim // self.num_heads, L)
                 out = self._ssa_kernel_hip(qkv, self.scale) if hip else self._ssa_kernel_torch(qkv, self.scale)
+        y = None
+        if attn_spikes is None and hip and len(self.proj_conv_bn) == 2:
+            # the attention's LIF writes its spikes as bits, the projection's convolution reads bits
+            y = fused.lif_conv_bn_lif(out, self.attn_lif, self.proj_conv_bn[0], self.proj_conv_bn[1], self.proj_lif)
+            if y is not None:
+                return y
         if attn_spikes is None:
             attn_spikes = self.attn_lif(out)
         local_dim = attn_spikes.shape[2] * attn_spikes.shape[3]
         x_seq = attn_spikes.reshape(T, N, local_dim, L)
-        y = None
         if hip and len(self.proj_conv_bn) == 2:
             y = fused.conv_bn_lif(x_seq, self.proj_conv_bn[0], self.proj_conv_bn[1], self.proj_lif, x_exact=True)
         if y is None:

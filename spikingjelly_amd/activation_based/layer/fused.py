@@ -132,3 +132,60 @@ def conv_bn_lif(x_seq: torch.Tensor, conv: Optional[nn.Module], bn: nn.Module, n
             return spikes
     node.v = v_last.reshape(out_shape[1:])
     return spikes.view(out_shape)
+
+
+def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_node: nn.Module, conv: nn.Module, bn: nn.Module, node: nn.Module
+                    ) -> Optional[torch.Tensor]:
+    """``node(bn(conv(pre_node(pre_seq))))`` for ``pre_seq [T, B, C, *positions]`` (or ``[T, B, heads, C / heads, L]``,
+    as the attention's neuron sees it: its state keeps that shape) in one autograd node whose first
+    neuron writes its spikes bit-packed and whose convolution reads them as bits (the spikes never exist as a float
+    tensor), or ``None`` when the chain does not qualify (the caller then runs the modules one by one).  This is the
+    ``attn_lif -> proj_conv -> proj_bn -> proj_lif`` tail of the reference's ``SpikingSelfAttention.forward``
+    (layer/attention.py:376-384)."""
+    from ..functional import neuron as F
+    from ..hip_kernel import conv_bn_lif as C
+
+    if (not configure.hip_fuse_conv_bn_lif or not getattr(configure, "hip_conv_bit_spikes", True) or torch.compiler.is_compiling()
+            or type(node) is not neuron.LIFNode or node.backend != "hip" or node.step_mode != "m" or node.store_v_seq
+            or not _plain_hip_lif(pre_node) or pre_seq.dim() < 4):
+        return None
+    Cin = conv.in_channels
+    if not _pointwise(conv) or pre_seq[0, 0].numel() % Cin != 0:
+        return None
+    if pre_seq.shape[2] == Cin:
+        positions = tuple(pre_seq.shape[3:])
+    elif pre_seq.dim() == 5 and pre_seq.shape[2] * pre_seq.shape[3] == Cin:
+        positions = (pre_seq.shape[4],)
+    else:
+        return None
+    channels = conv.out_channels
+    if not isinstance(bn, (nn.BatchNorm1d, nn.BatchNorm2d)) or bn.num_features != channels:
+        return None
+    params = (p for p in (conv.weight, bn.weight, bn.bias) if p is not None)
+    need_grad = torch.is_grad_enabled() and (pre_seq.requires_grad or any(p.requires_grad for p in params))
+    x4 = pre_seq.reshape(pre_seq.shape[0], pre_seq.shape[1], Cin, -1)  # [T, B, Cin, L]
+    T, B, _, Lp = x4.shape
+    if not C.lif_conv_bn_lif_supported(x4, need_grad) or (B * Cin * Lp) % 8 != 0:
+        return None
+    if need_grad and not F._hip_recompute(x4.flatten(1)):
+        return None  # the first neuron's backward replays its forward
+    node._check_hip_surrogate()
+    pre_node._check_hip_surrogate()
+    (pre_v,) = pre_node.materialize_states((pre_seq,), (pre_node.v,), "m")
+    state_like = torch.empty((1,), dtype=x4.dtype, device=x4.device).expand(T, B, channels, *positions)
+    (v,) = node.materialize_states((state_like,), (node.v,), "m")
+    if need_grad and (v.requires_grad or pre_v.requires_grad):
+        return None
+    bn_args = _bn_arguments(bn)  # (counts the batch: nothing below may give up)
+    if bn_args is None:
+        return None
+    gamma, beta, bn_cfg = bn_args
+    v3 = v.reshape(B, channels, Lp) if v.dim() != 3 else v
+    pre_v3 = pre_v.reshape(B, Cin, Lp)
+    with torch.set_grad_enabled(need_grad):
+        spikes, v_last, pre_v_last = C.lif_conv_bn_lif(x4, pre_v3, conv.weight.view(channels, -1), gamma, beta, v3, bn_cfg,
+                                                       _lif_spec(pre_node, x4, need_grad), _lif_spec(node, x4, need_grad))
+    node.v = v_last.reshape(B, channels, *positions)
+    pre_node.v = pre_v_last.reshape(pre_seq.shape[1:])
+    return spikes.view(T, B, channels, *positions)
+

@@ -38,6 +38,10 @@ hip_half_precision_mode = "torch"
 # a pass that finds the largest magnitude), three products per pair of real operands, two when one operand is spikes;
 # accuracy of an fp32 GEMM (2^-23 of sum |a||b| measured).  "bf16": hip_conv_terms bf16 terms, no scaling, no extra pass.
 hip_conv_split = "f16"
+# True: where a hip LIF feeds a fused kernel-size-1 convolution + batch norm + LIF (the attention neuron and the projection
+# of the spiking self-attention), the first neuron writes its spikes bit-packed and the convolution GEMMs read the bits:
+# the spikes never exist as a float tensor (needs hip_conv_split = "f16").  False: dense fp32 spikes between the two.
+hip_conv_bit_spikes = True
 # True: the weight gradient of a fused convolution runs on a second stream beside its input gradient (they only share
 # their inputs), so that the blocks of one kernel fill the compute units that the last, partly filled round of the
 # other leaves idle.  False (default): one after the other on the caller's stream.  It paid while the GEMM kernel kept

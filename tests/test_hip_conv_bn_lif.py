@@ -492,6 +492,36 @@ def test_convolution_gradients_on_two_streams_equal_those_on_one(monkeypatch):
             assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("training", [True, False])
+def test_bit_packed_spikes_between_attention_neuron_and_projection_change_nothing(training, monkeypatch):
+    """``configure.hip_conv_bit_spikes``: the attention neuron writes bits and the projection's GEMMs read bits, or the
+    spikes travel as fp32; the same arithmetic on the same values, so outputs, states and gradients are the same bits,
+    over two consecutive calls (the second starts from the states of the first)."""
+    block = _make_block(64, 2, 65).cuda().train(training)
+    xs = [seeded_randn((4, 3, 64, 36), 66 + i, 0.0, 2.0).cuda() for i in range(2)]
+    g = seeded_randn((4, 3, 64, 36), 68).cuda()
+    results = []
+    for bits in (False, True):
+        monkeypatch.setattr(configure, "hip_conv_bit_spikes", bits)
+        functional.reset_net(block)
+        got = []
+        for x in xs:
+            for p_ in block.parameters():
+                p_.grad = None
+            xi = x.clone().requires_grad_()
+            out = block(xi)
+            out.backward(g)
+            got += [out.detach().clone(), xi.grad.clone(), block.attn_lif.v.detach().clone(), block.proj_lif.v.detach().clone()]
+            got += [p_.grad.clone() for p_ in block.parameters()]
+            for node in (block.qkv_lif, block.attn_lif, block.proj_lif):   # the next call starts from these states
+                node.v = node.v.detach()
+        results.append(got)
+    assert results[0][2].shape == results[1][2].shape == (3, 2, 32, 36)   # the attention neuron's state keeps its shape
+    assert 0.02 < float(results[0][0].mean()) < 0.9
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+
+
 def test_attention_block_fused_equals_unfused_path(monkeypatch):
     """The same module with the fusion switched off (torch's convolution and batch norm around the hip neurons)."""
     from spikingjelly_amd.activation_based.layer import fused
@@ -499,12 +529,14 @@ def test_attention_block_fused_equals_unfused_path(monkeypatch):
     block = _make_block(64, 2, 60).cuda().train()
     x = seeded_randn((4, 2, 64, 36), 61, 0.0, 2.0).cuda()
     calls = []
-    real = fused.conv_bn_lif
+    real, real_tail = fused.conv_bn_lif, fused.lif_conv_bn_lif
     monkeypatch.setattr(fused, "conv_bn_lif", lambda *a, **k: calls.append(1) or real(*a, **k))
+    monkeypatch.setattr(fused, "lif_conv_bn_lif", lambda *a, **k: calls.append(2) or real_tail(*a, **k))
     a = block(x)
-    assert len(calls) == 2
+    assert calls == [1, 2]   # the qkv chain with the contraction, then the attention neuron with the projection chain
     functional.reset_net(block)
     monkeypatch.setattr(fused, "conv_bn_lif", real)
+    monkeypatch.setattr(fused, "lif_conv_bn_lif", real_tail)
     monkeypatch.setattr(configure, "hip_fuse_conv_bn_lif", False)
     b = block(x)
     assert float((a != b).float().mean()) < 1e-3   # fp32 convolutions of two libraries: a spike in a thousand may flip
