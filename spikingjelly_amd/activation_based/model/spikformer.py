@@ -3,7 +3,7 @@ path (reference ``model/spikformer.py:16-99`` ``SpikformerConv2dBN`` and ``:107-
 rest of that model (patch stem, MLP, classifier) is built from these two, ``SpikingSelfAttention`` and torch layers.
 
 With ``backend='hip'`` and no pooling between batch norm and the neuron, ``SpikformerConv2dBNLIF`` runs batch norm and
-the LIF fused (``layer/fused.py``); a kernel-size-1 convolution runs on the split-bf16 GEMM kernels as well, any other
+the LIF fused (``layer/fused.py``); a kernel-size-1 convolution runs on the library's split-operand GEMM kernels as well, any other
 convolution stays with torch and hands its output to the fused batch norm + LIF.
 """
 
