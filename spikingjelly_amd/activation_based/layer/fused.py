@@ -150,7 +150,7 @@ def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_node: nn.Module, conv: nn.Module,
             or not _plain_hip_lif(pre_node) or pre_seq.dim() < 4):
         return None
     Cin = conv.in_channels
-    if not _pointwise(conv) or pre_seq[0, 0].numel() % Cin != 0:
+    if not _pointwise(conv) or pre_seq.numel() == 0:
         return None
     if pre_seq.shape[2] == Cin:
         positions = tuple(pre_seq.shape[3:])
