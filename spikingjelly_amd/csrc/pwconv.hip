@@ -520,6 +520,7 @@ struct PwDwArgs {
   int64_t S;
   int M, N, L;
   int s_per_chunk;
+  int flat;  // the K steps run over the positions of all samples of a chunk in a row (see pw_dw_kernel)
   int m_blocks, n_blocks;
   const float *dy_amax, *x_amax;  // fp16 terms: nullptr (no scale), or the words whose maximum is the tensor's max |.|
 };
@@ -544,7 +545,18 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   const int64_t s_begin = (int64_t)chunk * a.s_per_chunk;
   const int64_t s_end = s_begin + a.s_per_chunk < a.S ? s_begin + a.s_per_chunk : a.S;
   const int l_steps = (L + kTileK - 1) / kTileK;
-  const int64_t iters = (s_end - s_begin) * l_steps;
+  // flat: the contraction index runs over the quads (four positions) of all samples of the chunk in a row, so a K step of
+  // eight quads may take the last quads of one sample and the first of the next, and only the last step of a chunk is
+  // partly empty (a row of 196 positions is 6.125 steps instead of 7).  Needs at least eight quads per sample (a step
+  // then touches two samples at most) and samples of less than 2^31 bytes (a lane's offset reaches into the second).
+  const bool flat = a.flat != 0;
+  const int Q = L >> 2;
+  const int n_samples = (int)(s_end - s_begin);
+  const int64_t total_quads = (int64_t)n_samples * Q;
+  const int64_t iters = flat ? (total_quads + 7) / 8 : (int64_t)n_samples * l_steps;
+  const uint32_t a_sample = (uint32_t)(M * L * 4), b_sample = (uint32_t)(N * L * (BITS ? 1 : 4));  // bytes; with BITS bits
+  int f_s = 0, f_q = 0;  // flat: sample and quad at which the next step to be fetched begins
+  int g_s = 0, g_q = 0;  // flat: the same for the next step to be staged
 
   // a thread fetches quad q4 (four consecutive l) of rows rr, rr + 32, rr + 64, rr + 96 of both operand tiles; addresses
   // are a uniform base (the sample) plus 32-bit per-lane offsets (row; position), loads are unconditional from clamped
@@ -564,28 +576,65 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   if (H && TA > 1 && a.dy_amax != nullptr) scale_for(tensor_amax(a.dy_amax), a_scale, a_inverse);
   if (H && TB > 1 && a.x_amax != nullptr) scale_for(tensor_amax(a.x_amax), b_scale, b_inverse);
   f32x4 ra[2][4], rb[2][4];  // two tiles in flight, as in pw_gemm_kernel
-  auto fetch = [&](int64_t it, int set) {
-    const int64_t s = s_begin + it / l_steps;
-    const int l0 = (int)(it % l_steps) * kTileK;
+  auto fetch = [&](int64_t it, int set) {  // (called for it = 0, 1, 2, ... in this order)
+    int64_t s;
+    uint32_t l_off, sa = 0, sb = 0;
+    if (flat) {
+      int q = f_q + q4;
+      const bool second = q >= Q;
+      if (second) q -= Q;
+      const bool ok = f_s + (second ? 1 : 0) < n_samples;
+      s = s_begin + f_s;
+      l_off = ok ? (uint32_t)q * 16u : 0u;
+      if (ok && second) {
+        sa = a_sample;
+        sb = b_sample;
+      }
+      f_q += 8;
+      if (f_q >= Q) {
+        f_q -= Q;
+        ++f_s;
+      }
+    } else {
+      s = s_begin + it / l_steps;
+      const int l = (int)(it % l_steps) * kTileK + 4 * q4;
+      l_off = (uint32_t)((l < L ? l : L - 4) * 4);
+    }
     const char *pa = dy_base + (s * M) * (int64_t)L * 4;
     const char *pb = x_base + (BITS ? ((s * N) * (int64_t)L >> 3) : (s * N) * (int64_t)L * 4);
-    const int l = l0 + 4 * q4;
-    const uint32_t l_off = (uint32_t)((l < L ? l : L - 4) * 4);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      ra[set][i] = *reinterpret_cast<const f32x4 *>(pa + (a_off[i] + l_off));
+      ra[set][i] = *reinterpret_cast<const f32x4 *>(pa + (a_off[i] + sa + l_off));
       if (BITS) {
-        const uint32_t e = b_off[i] + (l_off >> 2);
+        const uint32_t e = b_off[i] + sb + (l_off >> 2);
         rb[set][i].x = __builtin_bit_cast(float, (uint32_t)*reinterpret_cast<const uint8_t *>(pb + (e >> 3)));
       } else {
-        rb[set][i] = *reinterpret_cast<const f32x4 *>(pb + (b_off[i] + l_off));
+        rb[set][i] = *reinterpret_cast<const f32x4 *>(pb + (b_off[i] + sb + l_off));
       }
     }
   };
-  auto stage = [&](int64_t it, int set) {
-    const int l0 = (int)(it % l_steps) * kTileK;
-    const bool l_ok = l0 + 4 * q4 < L;
-    if (edge_rows || l0 + kTileK > L) {
+  auto stage = [&](int64_t it, int set) {  // (called for it = 0, 1, 2, ... in this order)
+    bool l_ok, tail;
+    int lq;  // the position of the work-item's quad in its row (for the bit offset)
+    if (flat) {
+      int q = g_q + q4;
+      const bool second = q >= Q;
+      if (second) q -= Q;
+      l_ok = g_s + (second ? 1 : 0) < n_samples;
+      lq = l_ok ? 4 * q : 0;
+      tail = (int64_t)g_s * Q + g_q + 8 > total_quads;
+      g_q += 8;
+      if (g_q >= Q) {
+        g_q -= Q;
+        ++g_s;
+      }
+    } else {
+      const int l0 = (int)(it % l_steps) * kTileK;
+      l_ok = l0 + 4 * q4 < L;
+      lq = l_ok ? l0 + 4 * q4 : L - 4;
+      tail = l0 + kTileK > L;
+    }
+    if (edge_rows || tail) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (!(l_ok && m0 + rr + 32 * i < M)) ra[set][i] = (f32x4)(0.0f);
@@ -612,9 +661,8 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       {
         uint32_t w01[TB], w23[TB];
         f32x4 v = rb[set][i];
-        if (BITS) {
-          const int l = l0 + 4 * q4;
-          const uint32_t e = b_off[i] + (uint32_t)(l < L ? l : L - 4);
+        if (BITS) {  // (a whole sample is a multiple of 8 bits: the shift does not depend on the sample)
+          const uint32_t e = b_off[i] + (uint32_t)lq;
           const uint32_t four = __builtin_bit_cast(uint32_t, rb[set][i].x) >> (e & 7u);
           v.x = (float)(four & 1u);
           v.y = (float)((four >> 1) & 1u);
@@ -644,8 +692,9 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.0f;
 
   auto multiply = [&](int64_t it) {
-    const int l0 = (int)(it % l_steps) * kTileK;
-    const int ksteps = (l0 + 16 < L) ? 2 : 1;  // the second half of the last stage of a row may hold nothing
+    // the second half of the last stage of a row (flat: of the chunk) may hold nothing
+    const int ksteps = flat ? ((it + 1 == iters && total_quads - 8 * it <= 4) ? 1 : 2)
+                            : (((int)(it % l_steps) * kTileK + 16 < L) ? 2 : 1);
     for (int ks = 0; ks < ksteps; ++ks) {
       u32x4 af[2][TA], bf[2][TB];
 #pragma unroll
@@ -872,6 +921,7 @@ int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *dy_ama
   PwDwArgs a;
   a.dy = dy; a.x = x; a.partials = workspace; a.S = S;
   a.dy_amax = dy_amax; a.x_amax = x_amax;
+  a.flat = (L >= 32 && M * L < (int64_t(1) << 29) && N * L < (int64_t(1) << 29)) ? 1 : 0;
   a.M = (int)M; a.N = (int)N; a.L = (int)L;
   a.m_blocks = (int)(round_up(M, kTile) / kTile);
   a.n_blocks = (int)(round_up(N, kTile) / kTile);
