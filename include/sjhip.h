@@ -505,7 +505,7 @@ int sjhip_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int 
  * of two that takes the tensor's largest finite magnitude `amax` into [2^14, 2^15) (1 for a zero or subnormal amax;
  * infinities and NaNs take no part in it and propagate through the products as in fp32),
  * which the kernels derive from a device buffer of SJHIP_PW_AMAX_FLOATS non-negative floats whose maximum is amax
- * (several words, so that the blocks that fold their maxima into it do not meet on one address).  An element above 2^-16 of amax is represented to 2^-23
+ * (several words, so that the blocks that fold their maxima into it do not meet on one address; 16-byte aligned).  An element above 2^-16 of amax is represented to 2^-23
  * relative or better, a smaller one to 2^-39 of amax; the dropped product lo*lo is below 2^-22 of hi*hi.  Measured
  * against float64 on operands whose rows span four decades: 2^-23 of sum |a||b| (three bf16 terms: 2^-26; an fp32 dot
  * product of 384 terms: 2^-20).  An operand that fp16 holds exactly (spikes, integers up to 2048) takes one term and no

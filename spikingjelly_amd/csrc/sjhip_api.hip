@@ -624,6 +624,7 @@ int sjhip_pwconv_gemm_f16(const uint16_t *a_planes, int64_t M, int64_t K, const 
   if (S > (int64_t(1) << 40) / L) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm_f16: S*L overflows");
   if (b_terms != 1 && b_terms != 2) return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm_f16: %d activation terms (1 or 2)", b_terms);
   if (b_terms == 2 && !b_amax) return fail(SJHIP_ERR_INVALID, "pwconv_gemm_f16: two activation terms need the largest magnitude from sjhip_pwconv_amax");
+  if (b_terms == 2 && !aligned16(b_amax)) return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm_f16: the amax buffer must be 16-byte aligned");
   return launch_pwconv_gemm(a_planes, SJHIP_PW_F16 | 2, M, K, b, b_terms, b_terms == 2 ? b_amax : nullptr, S, L, c, partial,
                             static_cast<hipStream_t>(stream));
 }
@@ -634,6 +635,8 @@ int sjhip_pwconv_grad_weight_f16(const float *dy, const float *dy_amax, const fl
   if (M < 1 || N < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight_f16: M=%lld N=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)N, (long long)S, (long long)L);
   if (x_terms != 1 && x_terms != 2) return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight_f16: %d activation terms (1 or 2)", x_terms);
   if (x_terms == 2 && !x_amax) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight_f16: two activation terms need the largest magnitude from sjhip_pwconv_amax");
+  if (!aligned16(dy_amax) || (x_terms == 2 && !aligned16(x_amax)))
+    return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight_f16: the amax buffers must be 16-byte aligned");
   return launch_pwconv_grad_weight(dy, SJHIP_PW_F16 | 2, dy_amax, x, x_terms, x_terms == 2 ? x_amax : nullptr, S, M, N, L, dw,
                                    workspace, static_cast<hipStream_t>(stream));
 }
@@ -651,6 +654,7 @@ int sjhip_pwconv_grad_weight_f16_bits(const float *dy, const float *dy_amax, con
                                       int64_t N, int64_t L, float *dw, float *workspace, void *stream) {
   if (!dy || !dy_amax || !x_bits || !dw || !workspace) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight_f16_bits: NULL buffer");
   if (M < 1 || N < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight_f16_bits: M=%lld N=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)N, (long long)S, (long long)L);
+  if (!aligned16(dy_amax)) return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight_f16_bits: the amax buffer must be 16-byte aligned");
   return launch_pwconv_grad_weight(dy, SJHIP_PW_F16 | 2, dy_amax, reinterpret_cast<const float *>(x_bits), 1, nullptr, S, M, N, L, dw,
                                    workspace, static_cast<hipStream_t>(stream), true);
 }

@@ -240,6 +240,10 @@ def test_fp16_split_convolution_arguments_without_a_device():
     assert rc == -1 and b"NULL" in lib.sjhip_last_error()
     rc = lib.sjhip_pwconv_grad_weight_f16(16, 16, 16, 2, None, 1, 8, 8, 4, 16, 16, None)
     assert rc == -1 and b"sjhip_pwconv_amax" in lib.sjhip_last_error()
+    rc = lib.sjhip_pwconv_gemm_f16(16, 8, 8, 16, 2, 20, 1, 4, 16, None, None)
+    assert rc == -2 and b"16-byte aligned" in lib.sjhip_last_error()
+    rc = lib.sjhip_pwconv_grad_weight_f16_bits(16, 20, 16, 1, 8, 8, 4, 16, 16, None)
+    assert rc == -2 and b"16-byte aligned" in lib.sjhip_last_error()
     rc = lib.sjhip_pwconv_amax(16, 0, 16, None)
     assert rc == -1 and b"n=0" in lib.sjhip_last_error()
     rc = lib.sjhip_pwconv_split_weight_f16(16, 8, 8, 0, 8, None, None)
