@@ -26,11 +26,22 @@ T_STEPS = 16
 SHAPE = (T_STEPS, 256, 128, 32, 32)
 
 
-def cpu_baseline(torch, sample_neurons: int, repeats: int):
+def cpu_baseline(torch, sample_neurons: int, repeats: int, threads: int = 0):
     """torch-ops port of the reference torch backend (oracle/neuron_oracle.py), forward + autograd
-    backward, on ``sample_neurons`` neurons x T=16 of the same input distribution."""
+    backward, on ``sample_neurons`` neurons x T=16 of the same input distribution; ``threads``: intra-op threads for
+    this measurement (0: as torch is configured)."""
     from oracle import neuron_oracle as no
 
+    before = torch.get_num_threads()
+    if threads > 0:
+        torch.set_num_threads(threads)
+    try:
+        return _cpu_baseline(torch, no, sample_neurons, repeats)
+    finally:
+        torch.set_num_threads(before)
+
+
+def _cpu_baseline(torch, no, sample_neurons: int, repeats: int):
     cores = torch.get_num_threads()
     g = torch.Generator().manual_seed(1002)
     x = torch.randn((T_STEPS, sample_neurons), generator=g) * 0.8 + 0.3
@@ -141,10 +152,38 @@ def _kernel_ms(L, which):
 
 
 def _emit(args, metric, unit, value, elapsed, dtype, config, roofline):
-    print(json.dumps({
+    line = {
         "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": dtype, "data": "synthetic", "config": config, "roofline": roofline}))
+        "dtype": dtype, "data": "synthetic", "config": config, "roofline": roofline}
+    collect = getattr(args, "collect", None)
+    if collect is not None:  # a secondary measurement inside the default run: kept for the headline's JSON line
+        collect.append(line)
+    else:
+        print(json.dumps(line))
+
+
+def secondary_measurements(args):
+    """BASELINE configs[2], [3] and [4] timed after the headline (a few hundred ms in all), condensed for the
+    ``secondary`` object of the default JSON line: ms per step, the metric value, and the dominant kernel with its
+    duration and its fraction of the roofline that bounds it."""
+    import copy
+
+    out = {}
+    for name in ("config3", "config4", "config5"):
+        sub = copy.copy(args)
+        sub.workload, sub.steps, sub.warmup, sub.collect = name, 10, 3, []
+        other_workload(sub)
+        line = sub.collect[0]
+        r = line["roofline"]
+        out[name] = {"metric": line["metric"], "value": line["value"], "unit": line["unit"], "ms_per_step": line["ms_per_step"],
+                     "kernel": r["kernel"], "kernel_ms": r["kernel_ms"], "bound": r["bound"], "achieved": r["achieved"],
+                     "peak": r["peak"], "roofline_unit": r["unit"], "frac": r["frac"]}
+        for extra in ("forward_ms", "backward_ms", "fused_forward_packed_ms", "fused_forward_packed_GBs", "gemm_ms_per_step",
+                      "ssa_backward_ms", "ssa_backward_GBs"):
+            if extra in r:
+                out[name][extra] = r[extra]
+    return out
 
 
 def other_workload(args) -> int:
@@ -455,6 +494,18 @@ def other_workload(args) -> int:
 
         elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
         sf, sb = _kernel_ms(L, L.KC_SSA_FORWARD), _kernel_ms(L, L.KC_SSA_BACKWARD)
+        # The convolution GEMMs are the largest share of the step and the part that the matrix cores bound: 16-bit
+        # products per step (three per pair of real operands, two when one operand is spikes; bf16 terms: six and
+        # three) over the time of all their launches.  qkv: Y = W X (real), dX (real), dW (real x real);
+        # projection: Y (spikes), dX (real), dW (real x spikes).
+        S_ = T * B
+        flop_qkv, flop_proj = 2.0 * S_ * D * 3 * D * tokens, 2.0 * S_ * D * D * tokens
+        real, spk = (3, 2) if args.conv_split == "f16" else ({3: 6, 2: 3, 1: 1}[args.terms], {3: 3, 2: 2, 1: 1}[args.terms])
+        gemm_products = flop_qkv * 3 * real + flop_proj * (2 * spk + real)
+        n_g, ms_g = L.profile_read(L.KC_PW_GEMM)
+        n_d, ms_d = L.profile_read(L.KC_PW_GRAD_WEIGHT)
+        gemm_ms_per_step = (ms_g + ms_d) / args.steps
+        gemm_tflops = gemm_products / (gemm_ms_per_step * 1e-3) / 1e12 if gemm_ms_per_step else 0.0
         cph = D // H
         probs = T * B * H
         n = T * B * D * tokens
@@ -467,9 +518,12 @@ def other_workload(args) -> int:
               {"workload": f"configs[4]: SpikingSelfAttention({D}, 12, backend='hip'), x [4,64,{D},196] fp32 ~N(0,1), "
                            f"channels per head = {cph} (dim // heads, as the reference computes it); convolution GEMMs on "
                            f"{'two fp16' if args.conv_split == 'f16' else str(args.terms) + ' bf16'} terms per fp32 operand"},
-              {"bound": "hbm", "achieved": bytes_b / (sb * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-               "frac": bytes_b / (sb * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "ssa_backward",
-               "kernel_ms": sb, "algorithmic_bytes": bytes_b,
+              {"bound": "mfma", "achieved": gemm_tflops, "peak": 2500.0, "unit": "TFLOP/s", "frac": gemm_tflops / 2500.0,
+               "traffic": None, "kernel": "pw_gemm + pw_dw (the six convolution GEMM launches of a step)",
+               "kernel_ms": gemm_ms_per_step / max((n_g + n_d) / args.steps, 1), "gemm_ms_per_step": gemm_ms_per_step,
+               "gemm_launches_per_step": (n_g + n_d) / args.steps, "gemm_16bit_product_flops_per_step": gemm_products,
+               "ssa_backward_ms": sb, "ssa_backward_GBs": bytes_b / (sb * 1e-3) / 1e9,
+               "ssa_backward_frac_of_hbm": bytes_b / (sb * 1e-3) / 1e9 / HBM_PEAK_GBS, "ssa_backward_bytes": bytes_b,
                "ssa_backward_TFLOPs": 4 * product / (sb * 1e-3) / 1e12,
                "ssa_forward_ms": sf, "ssa_forward_GBs": bytes_f / (sf * 1e-3) / 1e9,
                "ssa_forward_TFLOPs": 2 * product / (sf * 1e-3) / 1e12,
@@ -486,6 +540,8 @@ def main() -> int:
     ap.add_argument("--cpu-sample-neurons", type=int, default=1 << 23)
     ap.add_argument("--cpu-repeats", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="default workload: skip the condensed measurements of BASELINE configs 3-5 after the headline")
     ap.add_argument("--terms", type=int, default=3, choices=[1, 2, 3],
                     help="pwconv and config5 workloads with --conv-split bf16: bf16 terms per fp32 operand")
     ap.add_argument("--overlap", action="store_true",
@@ -630,10 +686,6 @@ def main() -> int:
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": dominant,
                      "kernel_ms": dom_ms, "algorithmic_bytes": dom_bytes,
                      "forward_ms": fwd_ms, "backward_ms": bwd_ms,
-                     "forward_GBs": fwd_bytes / (fwd_ms * 1e-3) / 1e9 if fwd_ms else None,
-                     "backward_GBs": bwd_bytes / (bwd_ms * 1e-3) / 1e9 if bwd_ms else None,
-                     "fwd_plus_bwd_frac": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS
-                     if (fwd_ms + bwd_ms) else None,
                      "forward_traffic_GBs": fwd_moved / (fwd_ms * 1e-3) / 1e9 if fwd_ms else None,
                      "backward_traffic_GBs": bwd_moved / (bwd_ms * 1e-3) / 1e9 if bwd_ms else None,
                      "step_traffic_frac": (fwd_moved + bwd_moved) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
@@ -642,8 +694,12 @@ def main() -> int:
     }
     del x, grad_spike, grad_v
     torch.cuda.empty_cache()
+    if not variant and not args.no_secondary:
+        out["secondary"] = secondary_measurements(args)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, args.cpu_sample_neurons, args.cpu_repeats)
+        # the same port on one thread (a quarter of the sample: about as long as the run above)
+        out["cpu_baseline_1thread"] = cpu_baseline(torch, max(args.cpu_sample_neurons // 4, 1 << 16), 2, threads=1)
     print(json.dumps(out))
     return 0
 

@@ -81,7 +81,7 @@ class SpikingSelfAttention(nn.Module, base.MultiStepModule):
         node = self.qkv_lif
         T, N, C3, L = pre.shape
         cph = C3 // 3 // self.num_heads
-        if (torch.compiler.is_compiling() or node.store_v_seq or not pre.is_cuda
+        if (torch.compiler.is_compiling() or not fused.unobserved(node) or node.store_v_seq or not pre.is_cuda
                 or not A.ssa_packed_supported(pre.dtype, cph, L) or (N * C3 * L) % 8 != 0):
             return None
         x2 = pre.flatten(1)
@@ -113,10 +113,11 @@ class SpikingSelfAttention(nn.Module, base.MultiStepModule):
             # node; without the last of them when it cannot run inside the contraction
             if configure.hip_fuse_ssa_lif:
                 attn_spikes = fused.conv_bn_lif(x_seq, self.qkv_conv_bn[0], self.qkv_conv_bn[1], self.qkv_lif,
-                                                ssa=(self.num_heads, self.scale), attn=self.attn_lif)
+                                                ssa=(self.num_heads, self.scale), attn=self.attn_lif,
+                                                container=self.qkv_conv_bn)
             if attn_spikes is None:
                 out = fused.conv_bn_lif(x_seq, self.qkv_conv_bn[0], self.qkv_conv_bn[1], self.qkv_lif,
-                                        ssa=(self.num_heads, self.scale))
+                                        ssa=(self.num_heads, self.scale), container=self.qkv_conv_bn)
         if out is None and attn_spikes is None:
             pre = self.qkv_conv_bn(x_seq)  # [T, N, 3*C, L]
             local_dim = pre.shape[2] // 3
@@ -129,7 +130,8 @@ class SpikingSelfAttention(nn.Module, base.MultiStepModule):
         y = None
         if attn_spikes is None and hip and len(self.proj_conv_bn) == 2:
             # the attention's LIF writes its spikes as bits, the projection's convolution reads bits
-            y = fused.lif_conv_bn_lif(out, self.attn_lif, self.proj_conv_bn[0], self.proj_conv_bn[1], self.proj_lif)
+            y = fused.lif_conv_bn_lif(out, self.attn_lif, self.proj_conv_bn[0], self.proj_conv_bn[1], self.proj_lif,
+                                      container=self.proj_conv_bn)
             if y is not None:
                 return y
         if attn_spikes is None:
@@ -137,7 +139,8 @@ class SpikingSelfAttention(nn.Module, base.MultiStepModule):
         local_dim = attn_spikes.shape[2] * attn_spikes.shape[3]
         x_seq = attn_spikes.reshape(T, N, local_dim, L)
         if hip and len(self.proj_conv_bn) == 2:
-            y = fused.conv_bn_lif(x_seq, self.proj_conv_bn[0], self.proj_conv_bn[1], self.proj_lif, x_exact=True)
+            y = fused.conv_bn_lif(x_seq, self.proj_conv_bn[0], self.proj_conv_bn[1], self.proj_lif, x_exact=True,
+                                  container=self.proj_conv_bn)
         if y is None:
             y = self.proj_lif(self.proj_conv_bn(x_seq))
         return y  # [T, N, C, L]

@@ -14,6 +14,28 @@ from ... import configure
 from .. import neuron
 
 
+def unobserved(*modules: Optional[nn.Module]) -> bool:
+    """True when running ``modules`` as one fused kernel chain is indistinguishable from calling them one by one: none
+    of them (and no global registration) has a forward, pre-forward or backward hook, which only ``Module.__call__``
+    fires (output monitors, old-style ``weight_norm`` that rebuilds ``conv.weight`` in a pre-hook), and autocast is off
+    (torch would run the convolution in the autocast dtype; the fused GEMMs keep fp32 operands)."""
+    import torch.nn.modules.module as M
+
+    if torch.is_autocast_enabled():
+        return False
+    for name in ("_global_forward_hooks", "_global_forward_pre_hooks", "_global_backward_hooks", "_global_backward_pre_hooks",
+                 "_global_forward_hooks_always_called"):
+        if len(getattr(M, name, ())):
+            return False
+    for m in modules:
+        if m is None:
+            continue
+        for name in ("_forward_hooks", "_forward_pre_hooks", "_backward_hooks", "_backward_pre_hooks"):
+            if len(getattr(m, name, ())):
+                return False
+    return True
+
+
 def _pointwise(conv: nn.Module) -> bool:
     """A convolution that is one matrix product per position: kernel 1, stride 1, no padding, one group, no bias."""
     if not isinstance(conv, (nn.Conv1d, nn.Conv2d)):
@@ -58,16 +80,20 @@ def _plain_hip_lif(node: nn.Module) -> bool:
 
 
 def conv_bn_lif(x_seq: torch.Tensor, conv: Optional[nn.Module], bn: nn.Module, node: nn.Module, x_exact: bool = False,
-                ssa: Optional[tuple] = None, attn: Optional[nn.Module] = None) -> Optional[torch.Tensor]:
+                ssa: Optional[tuple] = None, attn: Optional[nn.Module] = None, container: Optional[nn.Module] = None
+                ) -> Optional[torch.Tensor]:
     """``node(bn(conv(x_seq)))`` for ``x_seq [T, B, C, *positions]`` in one fused pass, or ``None``.
 
     ``conv is None``: ``x_seq`` already is the convolution output and only batch norm and the neuron are fused.
     ``ssa = (heads, scale)``: the spikes feed the spiking self-attention contraction bit-packed and the result is
     ``scale (V K^T) Q`` as ``[T, B, heads, channels_per_head, L]``.  With ``attn`` (the neuron that takes that result as
     its input) the result is ``attn``'s spikes instead, in the same shape, and ``None`` when ``attn`` cannot run inside
-    the contraction.  ``x_exact``: ``x_seq`` holds values that bf16 represents exactly (spikes)."""
+    the contraction.  ``x_exact``: ``x_seq`` holds values that bf16 represents exactly (spikes).  ``container``: the
+    module through which the caller would otherwise call ``conv`` and ``bn`` (its hooks count like theirs)."""
     from ..hip_kernel import conv_bn_lif as C
 
+    if not unobserved(conv, bn, node, attn, container):
+        return None
     if (not configure.hip_fuse_conv_bn_lif or torch.compiler.is_compiling() or type(node) is not neuron.LIFNode or node.backend != "hip" or node.step_mode != "m"
             or node.store_v_seq or x_seq.dim() < 4):
         return None
@@ -134,8 +160,8 @@ def conv_bn_lif(x_seq: torch.Tensor, conv: Optional[nn.Module], bn: nn.Module, n
     return spikes.view(out_shape)
 
 
-def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_node: nn.Module, conv: nn.Module, bn: nn.Module, node: nn.Module
-                    ) -> Optional[torch.Tensor]:
+def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_node: nn.Module, conv: nn.Module, bn: nn.Module, node: nn.Module,
+                    container: Optional[nn.Module] = None) -> Optional[torch.Tensor]:
     """``node(bn(conv(pre_node(pre_seq))))`` for ``pre_seq [T, B, C, *positions]`` (or ``[T, B, heads, C / heads, L]``,
     as the attention's neuron sees it: its state keeps that shape) in one autograd node whose first
     neuron writes its spikes bit-packed and whose convolution reads them as bits (the spikes never exist as a float
@@ -145,6 +171,8 @@ def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_node: nn.Module, conv: nn.Module,
     from ..functional import neuron as F
     from ..hip_kernel import conv_bn_lif as C
 
+    if not unobserved(pre_node, conv, bn, node, container):
+        return None
     if (not configure.hip_fuse_conv_bn_lif or not getattr(configure, "hip_conv_bit_spikes", True) or torch.compiler.is_compiling()
             or type(node) is not neuron.LIFNode or node.backend != "hip" or node.step_mode != "m" or node.store_v_seq
             or not _plain_hip_lif(pre_node) or pre_seq.dim() < 4):

@@ -47,7 +47,8 @@ class SpikformerConv2dBNLIF(nn.Module, base.MultiStepModule):
 
     def forward(self, x_seq: torch.Tensor):
         block = self.conv_bn.block
-        if self.neuron.backend == "hip" and len(block) == 2 and x_seq.dim() == 5:
+        if (self.neuron.backend == "hip" and len(block) == 2 and x_seq.dim() == 5
+                and fused.unobserved(self.conv_bn, block, block[0], block[1], self.neuron)):
             conv, bn = block[0], block[1]
             out = fused.conv_bn_lif(x_seq, conv, bn, self.neuron)
             if out is None:

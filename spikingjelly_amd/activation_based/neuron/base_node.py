@@ -125,7 +125,13 @@ class BaseNode(base.MemoryModule):
             key = (x.device, x.dtype, float(value), math.copysign(1.0, float(value)))
             one = _CONSTANT_STATES.get(key)
             if one is None:
-                one = _CONSTANT_STATES[key] = x.new_full((1,), value)
+                # The element outlives this call: it must be an ordinary tensor even when the first call comes under
+                # torch.inference_mode() (an inference tensor could not be saved for a later training backward), and
+                # its fill must have finished before a call on another stream reads it (made once: the wait is free).
+                with torch.inference_mode(False):
+                    one = torch.full((1,), value, dtype=x.dtype, device=x.device)
+                torch.cuda.current_stream(x.device).synchronize()
+                _CONSTANT_STATES[key] = one
             return one.view((1,) * x.dim()).expand(x.shape)
         return torch.full_like(x, value, requires_grad=False)
 

@@ -31,8 +31,21 @@ int launch_kernel(const FwdArgs &f, const BwdArgs &b, int block, unsigned lds, i
 template <typename S, bool ROUND_EACH, int MODE>
 int launch_pieces_kernel(const FwdArgs &f, const BwdArgs &b, const PieceArgs &p, int block, unsigned lds, int64_t blocks,
                          hipStream_t stream) {
-  hipLaunchKernelGGL((backward_recompute_pieces_kernel<S, ROUND_EACH, MODE>), dim3((unsigned)blocks), dim3(block), lds, stream,
-                     f, b, p);  // a piece's LDS buffer stays below the default 64 KiB limit
+  auto kernel = backward_recompute_pieces_kernel<S, ROUND_EACH, MODE>;
+  // pieces of 16 steps stay below the default 64 KiB of dynamic LDS; longer pieces (17 steps and more at 256 lanes,
+  // 33 and more at 128) do not and need the same opt-in as launch_kernel
+  static std::once_flag once;
+  static hipError_t attr_rc = hipSuccess;
+  std::call_once(once, [&]() {
+    attr_rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)kRecomputeMaxLds);
+    (void)hipGetLastError();
+  });
+  if (lds > kRecomputeMaxLds)
+    return fail(SJHIP_ERR_UNSUPPORTED, "backward(recompute, pieces): %u bytes of LDS per block exceed %u", lds, kRecomputeMaxLds);
+  if (lds > 64u * 1024u && attr_rc != hipSuccess)
+    return fail(SJHIP_ERR_LAUNCH, "backward(recompute, pieces): cannot raise the dynamic LDS limit: %s", hipGetErrorString(attr_rc));
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(block), lds, stream, f, b, p);
   return check_launch("backward(recompute, pieces)");
 }
 

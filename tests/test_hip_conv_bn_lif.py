@@ -270,6 +270,97 @@ def test_fp16_grad_weight_gemm(C, S, M, N, Lp, spikes, dy_scale):
     assert float(rel.max()) < 2e-6 and float(rel.mean()) < 2e-7
 
 
+# ---- operands that arrive as fp16 term planes (split once by their producer, not by every block of a GEMM) ---------------
+PLANE_SHAPES = [(3, 100, 50, 12), (2, 128, 32, 128), (1, 7, 3, 4), (4, 130, 257, 36), (5, 384, 384, 196), (16, 1152, 384, 196),
+                (3, 40, 9, 20)]
+
+
+@pytest.mark.parametrize("S,M,Kd,Lp", PLANE_SHAPES)
+@pytest.mark.parametrize("x_scale", [1.0, 1e-6, 1e12])
+def test_plane_layout_is_the_split_of_the_scaled_tensor(C, S, M, Kd, Lp, x_scale):
+    """``split_planes``: plane 0 is fp16(scale x), plane 1 fp16 of the remainder, rows of channels with the columns of all
+    samples in a row; scale = the power of two that takes amax into [2^14, 2^15)."""
+    x = _wide((S, Kd, Lp), 31, 4.0, x_scale).cuda()
+    xa = C.amax(x)
+    planes = C.split_planes(x, xa)
+    ld = -(-S * Lp // 8) * 8
+    assert planes.numel() == 2 * Kd * ld
+    top = float(xa.max())
+    scale = 2.0 ** (14 - int(torch.tensor(top).log2().floor()))
+    xs = (x.double() * scale).permute(1, 0, 2).reshape(Kd, S * Lp)
+    hi = planes[:Kd * ld].view(Kd, ld)[:, :S * Lp]
+    lo = planes[Kd * ld:].view(Kd, ld)[:, :S * Lp]
+    assert torch.equal(hi, xs.float().half())
+    assert torch.equal(lo, (xs.float() - hi.float()).half())
+    # two terms hold 22 significant bits of a value, down to the subnormal spacing 2^-24 of the second
+    assert bool(((hi.double() + lo.double() - xs).abs() <= xs.abs() * 2.0 ** -22 + 2.0 ** -25).all())
+
+
+@pytest.mark.parametrize("S,M,Kd,Lp", PLANE_SHAPES)
+@pytest.mark.parametrize("transpose", [False, True])
+def test_gemm_from_planes_has_fp32_accuracy_and_leaves_the_batch_norm_sums(C, S, M, Kd, Lp, transpose):
+    F = C.F16 | 2
+    w = _wide((Kd, M) if transpose else (M, Kd), 32, 4.0, 0.05)
+    x = _wide((S, Kd, Lp), 33, 4.0, 3.0)
+    wp = C.split_weight(w.cuda(), transpose, F)
+    xa = C.amax(x.cuda())
+    xp = C.split_planes(x.cuda(), xa)
+    got, part = C.pw_gemm_planes(wp, M, Kd, xp, 2, xa, S, Lp, True)
+    assert torch.equal(C.pw_gemm_planes(wp, M, Kd, xp, 2, xa, S, Lp), got)
+    got = got.cpu().double()
+    a = (w.t() if transpose else w).double()
+    want = torch.einsum("mk,skl->sml", a, x.double())
+    bound = torch.einsum("mk,skl->sml", a.abs(), x.double().abs()).clamp_min(1e-300)
+    rel = (got - want).abs() / bound
+    assert torch.isfinite(got).all() and float(rel.max()) < 2e-6 and float(rel.mean()) < 2e-7
+    # the same operands through the kernels that split while they stage: equal up to the fp32 accumulation order
+    ref = C.pw_gemm(wp, F, M, Kd, x.cuda(), F, False, xa).cpu().double()
+    assert float(((got - ref).abs() / bound).max()) < 1e-6
+    sums = part.double().sum(0).cpu()
+    want_s, abs_s, want_q = got.sum((0, 2)), got.abs().sum((0, 2)).clamp_min(1e-30), (got ** 2).sum((0, 2))
+    assert float(((sums[:, 0] - want_s).abs() / abs_s).max()) < 1e-6
+    assert float(((sums[:, 1] - want_q).abs() / want_q.clamp_min(1e-30)).max()) < 1e-6
+
+
+@pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (4, 384, 384, 196)])
+def test_gemm_from_a_plane_of_spikes_is_exact(C, S, M, Kd, Lp):
+    g = torch.Generator().manual_seed(34)
+    w = torch.randint(-64, 65, (M, Kd), generator=g).float() / 64.0
+    x = (torch.rand((S, Kd, Lp), generator=g) < 0.3).float()
+    wp = C.split_weight(w.cuda(), False, C.F16 | 2)
+    xp = C.split_planes(x.cuda(), None, 1)
+    got = C.pw_gemm_planes(wp, M, Kd, xp, 1, None, S, Lp)
+    assert torch.equal(got.cpu().double(), torch.einsum("mk,skl->sml", w.double(), x.double()))
+
+
+@pytest.mark.parametrize("S,M,N,Lp", [(3, 100, 50, 12), (9, 130, 257, 36), (16, 384, 384, 196), (2, 1152, 384, 196), (64, 64, 48, 8),
+                                      (1, 5, 3, 4)])
+@pytest.mark.parametrize("spikes", [False, True])
+def test_grad_weight_from_planes(C, S, M, N, Lp, spikes):
+    dy = _wide((S, M, Lp), 35, 4.0, 1e-3)
+    x = (seeded_randn((S, N, Lp), 36, 0.0, 1.0) > 0.5).float() if spikes else _wide((S, N, Lp), 36, 4.0, 30.0)
+    dya = C.amax(dy.cuda())
+    xa = None if spikes else C.amax(x.cuda())
+    dyp, xp = C.split_planes(dy.cuda(), dya), C.split_planes(x.cuda(), xa, 1 if spikes else 2)
+    got = C.pw_grad_weight_planes(dyp, dya, xp, 1 if spikes else 2, xa, S, M, N, Lp).cpu().double()
+    want = torch.einsum("sml,snl->mn", dy.double(), x.double())
+    bound = torch.einsum("sml,snl->mn", dy.double().abs(), x.double().abs()).clamp_min(1e-300)
+    rel = (got - want).abs() / bound
+    assert float(rel.max()) < 2e-6 and float(rel.mean()) < 2e-7
+
+
+def test_plane_calls_refuse_what_they_cannot_run(C):
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+
+    x = torch.randn(2, 8, 6, device="cuda")  # rows of six positions: not a multiple of 4
+    with pytest.raises(RuntimeError, match="multiple of 4"):
+        C.split_planes(x, C.amax(x))
+    x = torch.randn(2, 8, 8, device="cuda")
+    with pytest.raises(RuntimeError, match="amax"):
+        C.split_planes(x, None, 2)
+    assert L.load().sjhip_pwconv_plane_elems(2, 8, 8, 3) == 0
+
+
 @pytest.mark.parametrize("S,Cc,Lp", [(3, 5, 12), (16, 384, 196), (7, 33, 4), (300, 64, 100)])
 def test_bn_grad_input_leaves_the_largest_magnitude_of_its_output(C, S, Cc, Lp):
     """``sjhip_bn_grad_input_amax``: the same ``dy`` as the plain call, and the largest magnitude a pass over it finds."""
@@ -540,6 +631,51 @@ def test_attention_block_fused_equals_unfused_path(monkeypatch):
     monkeypatch.setattr(configure, "hip_fuse_conv_bn_lif", False)
     b = block(x)
     assert float((a != b).float().mean()) < 1e-3   # fp32 convolutions of two libraries: a spike in a thousand may flip
+
+
+@pytest.mark.parametrize("where", ["proj_lif", "attn_lif", "qkv_lif", "proj_bn", "qkv_conv_pre", "qkv_container"])
+def test_hooks_on_sub_modules_fire_and_see_the_spikes_of_the_unfused_path(where, monkeypatch):
+    """A module with a hook is called the way the reference's forward calls it (layer/attention.py:370-384): the fused
+    chain steps aside, the hook fires once per forward and sees what the same block computes with the fusion off."""
+    block = _make_block(64, 2, 62).cuda().train()
+    x = seeded_randn((4, 2, 64, 36), 63, 0.0, 2.0).cuda()
+    seen = []
+    target = {"proj_lif": block.proj_lif, "attn_lif": block.attn_lif, "qkv_lif": block.qkv_lif, "proj_bn": block.proj_conv_bn[1],
+              "qkv_conv_pre": block.qkv_conv_bn[0], "qkv_container": block.qkv_conv_bn}[where]
+    if where == "qkv_conv_pre":
+        handle = target.register_forward_pre_hook(lambda m, args: seen.append(args[0].detach().clone()))
+    else:
+        handle = target.register_forward_hook(lambda m, args, out: seen.append(out.detach().clone()))
+    out_hooked = block(x)
+    assert len(seen) == 1
+    handle.remove()
+    functional.reset_net(block)
+    monkeypatch.setattr(configure, "hip_fuse_conv_bn_lif", False)
+    handle = (target.register_forward_pre_hook(lambda m, args: seen.append(args[0].detach().clone())) if where == "qkv_conv_pre"
+              else target.register_forward_hook(lambda m, args, out: seen.append(out.detach().clone())))
+    out_plain = block(x)
+    handle.remove()
+    assert len(seen) == 2 and seen[0].shape == seen[1].shape
+    if where in ("qkv_conv_pre", "qkv_container", "qkv_lif"):  # nothing fused ran in front of these: identical
+        assert torch.equal(seen[0], seen[1])
+    else:  # (a fused qkv chain ran in front of the hooked module: a spike in a thousand may differ, as between libraries)
+        assert float((seen[0] != seen[1]).float().mean()) < 2e-3
+    assert float((out_hooked != out_plain).float().mean()) < 2e-3
+
+
+def test_autocast_keeps_the_modules_in_charge(monkeypatch):
+    """Under autocast torch runs the convolution in the autocast dtype; the fused fp32 GEMMs would not, so they step aside."""
+    from spikingjelly_amd.activation_based.layer import fused
+
+    block = _make_block(64, 2, 64).cuda().train()
+    x = seeded_randn((4, 2, 64, 36), 65, 0.0, 2.0).cuda()
+    calls = []
+    from spikingjelly_amd.activation_based.hip_kernel import conv_bn_lif as Ck
+    monkeypatch.setattr(Ck, "conv_bn_lif_ssa", lambda *a, **k: calls.append(1))
+    monkeypatch.setattr(Ck, "lif_conv_bn_lif", lambda *a, **k: calls.append(2))
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = block(x)
+    assert calls == [] and out.shape == x.shape
 
 
 def test_eval_mode_spikes_are_bit_identical_to_the_torch_backend_on_exact_inputs():

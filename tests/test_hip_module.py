@@ -178,6 +178,25 @@ def test_inference_modes(ctx):
     assert bits_equal(sb.cpu(), sa) and bits_equal(b.v.cpu(), a.v)
 
 
+def test_training_after_a_first_forward_under_inference_mode():
+    """The shared one-element initial state (one per device, dtype and value; -0.37 is used by no other test) is first
+    made under ``torch.inference_mode()``: a later training forward saves its expanded view for the backward, which an
+    inference tensor would refuse."""
+    kw = dict(v_reset=-0.37, surrogate_function=surrogate.ATan())
+    x = seeded_randn((6, 4, 32), 16, 0.3, 0.5)
+    first = neuron.LIFNode(step_mode="m", backend="hip", **kw).cuda()
+    with torch.inference_mode():
+        first(x.cuda())
+    a, b = _pair(neuron.LIFNode, **kw)
+    xa, xb = x.clone().requires_grad_(), x.cuda().requires_grad_()
+    sa, sb = a(xa), b(xb)
+    g = seeded_randn(sa.shape, 17)
+    sa.backward(g)
+    sb.backward(g.cuda())
+    assert bits_equal(sb.detach().cpu(), sa.detach())
+    torch.testing.assert_close(xb.grad.cpu(), xa.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
+
+
 def test_unsupported_surrogate_and_primitive_mode_raise():
     node = neuron.LIFNode(step_mode="m", backend="hip", surrogate_function=surrogate.PiecewiseLeakyReLU()).cuda()
     x = torch.randn(4, 2, 8, device="cuda", requires_grad=True)

@@ -137,7 +137,8 @@ def _backward_piece_by_piece(L, c, chunk, ck, with_gv):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=lambda v: str(v).replace("torch.", ""))
 @pytest.mark.parametrize("neuron_name", ["IF", "LIF", "PLIF", "QIF"])
-@pytest.mark.parametrize("T,chunk", [(44, 16), (64, 16), (30, 10), (12, 16)])
+# (pieces of 18 and 40 steps need more than 64 KiB of dynamic LDS per block at 256 and 128 work-items)
+@pytest.mark.parametrize("T,chunk", [(44, 16), (64, 16), (30, 10), (12, 16), (40, 18), (90, 40)])
 def test_pieces_equal_whole_forward_and_piecewise_backward(L, dtype, neuron_name, T, chunk):
     neuron = getattr(L, "NEURON_" + neuron_name)
     flags = L.FLAG_DECAY_INPUT

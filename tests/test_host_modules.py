@@ -498,3 +498,28 @@ def test_activation_aware_if_node_on_the_torch_backend():
     xg = torch.tensor([[0.9, 1.8]], requires_grad=True)
     node(xg).sum().backward()
     assert xg.grad is not None and bool((xg.grad != 0).all())
+
+
+def test_fused_chain_steps_aside_for_hooks_and_autocast():
+    """``layer.fused.unobserved``: hooks only fire through ``Module.__call__`` and autocast would change the convolution's
+    dtype, so either keeps the modules of a chain in charge (reference forward: layer/attention.py:370-384)."""
+    import torch.nn as nn
+
+    from spikingjelly_amd.activation_based.layer import fused
+
+    conv, bn, node = nn.Conv1d(4, 4, 1, bias=False), nn.BatchNorm1d(4), neuron.LIFNode(step_mode="m")
+    assert fused.unobserved(conv, bn, node, None)
+    for module, register in ((node, "register_forward_hook"), (conv, "register_forward_pre_hook"),
+                             (bn, "register_full_backward_hook"), (conv, "register_full_backward_pre_hook")):
+        handle = getattr(module, register)(lambda *a: None)
+        assert not fused.unobserved(conv, bn, node)
+        handle.remove()
+        assert fused.unobserved(conv, bn, node)
+    handle = nn.modules.module.register_module_forward_hook(lambda *a: None)
+    try:
+        assert not fused.unobserved(conv)
+    finally:
+        handle.remove()
+    with torch.autocast("cpu", dtype=torch.bfloat16):
+        assert fused.unobserved(conv)  # (autocast of another device type does not concern device tensors)
+    assert fused.unobserved(conv, bn, node)
