@@ -544,6 +544,39 @@ int sjhip_pwconv_grad_weight_f16_bits(const float *dy, const float *dy_amax, con
                                       int64_t N, int64_t L, float *dw, float *workspace, void *stream);
 
 /*
+ * The same GEMMs with the activations / gradients arriving as fp16 term planes that their producer wrote already scaled
+ * and split (sjhip_pwconv_split_planes, or the kernel that computes the tensor: sjhip_bn_grad_input_planes), instead of
+ * fp32 tensors that every block of a GEMM splits again while it stages them (same reference lines:
+ * layer/attention.py:310-329, model/spikformer.py:85-99).  A plane buffer of a tensor x [S][C][L] holds `terms` planes
+ * [C][ld] of fp16, ld = S * L rounded up to a multiple of 8 (16-byte aligned rows): element (c, s * L + l) of plane 0 is
+ * fp16(scale x[s][c][l]), of plane 1 fp16 of the remainder; scale is the power of two that the tensor's amax buffer gives
+ * (as for sjhip_pwconv_gemm_f16), so the same amax buffer must accompany the planes into every GEMM that reads them.  The
+ * columns beyond S * L are never read as data.  The channel-major layout makes the columns of all samples one contiguous
+ * contraction (weight gradient) or output (forward, input gradient) index; results agree with the *_f16 calls to the
+ * rounding of the fp32 accumulation order.
+ *
+ *   sjhip_pwconv_plane_elems       2-byte elements of the plane buffer of x [S][C][L] with `terms` (1 or 2) terms
+ *   sjhip_pwconv_split_planes      planes of x; terms 2 with the amax buffer of x (sjhip_pwconv_amax), or 1 (values that
+ *                                  fp16 holds exactly; amax NULL); L a multiple of 4, 16-byte aligned buffers
+ *   sjhip_pwconv_gemm_planes       c[s][m][l] = sum_k A[m][k] b[s][k][l] from fp16 weight planes
+ *                                  (sjhip_pwconv_split_weight_f16) and the planes of b; partial as in
+ *                                  sjhip_pwconv_gemm_stats with sjhip_pwconv_gemm_planes_stats_rows(S, L) rows, or NULL;
+ *                                  any L
+ *   sjhip_pwconv_grad_weight_planes  dw[m][n] = sum_{s,l} dy[s][m][l] x[s][n][l] from the planes of dy (two terms) and of
+ *                                  x (x_terms); workspace of sjhip_pwconv_grad_weight_planes_workspace_floats floats
+ */
+int64_t sjhip_pwconv_plane_elems(int64_t S, int64_t C, int64_t L, int terms);
+int sjhip_pwconv_split_planes(const float *x, int64_t S, int64_t C, int64_t L, int terms, const float *amax, uint16_t *planes,
+                              void *stream);
+int64_t sjhip_pwconv_gemm_planes_stats_rows(int64_t S, int64_t L);
+int sjhip_pwconv_gemm_planes(const uint16_t *a_planes, int64_t M, int64_t K, const uint16_t *b_planes, int b_terms,
+                             const float *b_amax, int64_t S, int64_t L, float *c, float *partial, void *stream);
+int64_t sjhip_pwconv_grad_weight_planes_workspace_floats(int64_t M, int64_t N, int64_t S, int64_t L);
+int sjhip_pwconv_grad_weight_planes(const uint16_t *dy_planes, const float *dy_amax, const uint16_t *x_planes, int x_terms,
+                                    const float *x_amax, int64_t S, int64_t M, int64_t N, int64_t L, float *dw, float *workspace,
+                                    void *stream);
+
+/*
  * Batch normalisation fused with the multi-step IF / LIF neuron behind it, for fp32 activations [T][B][C][L]
  * (L contiguous, a multiple of 4).  Stands in for nn.BatchNorm1d / nn.BatchNorm2d followed by LIFNode in the reference's
  * SpikingSelfAttention (layer/attention.py:314-329, 370-384) and SpikformerConv2dBNLIF (model/spikformer.py:196-212),

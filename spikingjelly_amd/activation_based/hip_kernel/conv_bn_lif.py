@@ -33,7 +33,8 @@ from . import neuron_kernel as K
 
 __all__ = ["supported", "bn_lif", "conv_bn_lif", "conv_bn_lif_ssa", "conv_bn_lif_ssa_lif", "lif_conv_bn_lif",
            "lif_conv_bn_lif_supported", "split_weight", "pw_gemm",
-           "pw_grad_weight", "pw_gemm_bits", "pw_grad_weight_bits", "amax", "F16"]
+           "pw_grad_weight", "pw_gemm_bits", "pw_grad_weight_bits", "amax", "F16", "split_planes", "pw_gemm_planes",
+           "pw_grad_weight_planes"]
 
 MAX_REPLAY_STEPS = 16  # the backward replays the neuron with h of every step in registers
 
@@ -193,6 +194,50 @@ def pw_grad_weight_bits(dy: torch.Tensor, bits: torch.Tensor, N: int, dy_amax: O
         rc = lib.sjhip_pwconv_grad_weight_f16_bits(dy.data_ptr(), dy_amax.data_ptr(), bits.data_ptr(), S, M, N, Lp, dw.data_ptr(),
                                                    ws.data_ptr(), _stream(dy))
     L.check(rc, "pwconv_grad_weight_f16_bits")
+    return dw
+
+
+def split_planes(x: torch.Tensor, x_amax: Optional[torch.Tensor], terms: int = 2) -> torch.Tensor:
+    """fp16 term planes of ``x [S, C, L]`` (``L`` a multiple of 4): ``terms`` planes ``[C, ld]`` with the columns
+    ``s * L + l`` of all samples in a row, scaled by the power of two that ``x_amax`` (``amax(x)``) gives; one term and no
+    scale for values that fp16 holds exactly.  The operand format of ``pw_gemm_planes`` / ``pw_grad_weight_planes``."""
+    S, C, Lp = x.shape
+    x = L.aligned16(x)
+    lib = L.load()
+    planes = torch.empty((lib.sjhip_pwconv_plane_elems(S, C, Lp, terms),), dtype=torch.float16, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.sjhip_pwconv_split_planes(x.data_ptr(), S, C, Lp, terms, L.ptr(x_amax), planes.data_ptr(), _stream(x))
+    L.check(rc, "pwconv_split_planes")
+    return planes
+
+
+def pw_gemm_planes(w_planes: torch.Tensor, M: int, Kdim: int, b_planes: torch.Tensor, b_terms: int, b_amax: Optional[torch.Tensor],
+                   S: int, Lp: int, stats: bool = False):
+    """``pw_gemm`` on fp16 weight planes with the activations as term planes (``split_planes`` or a kernel that writes
+    them): ``c [S, M, L]``, and with ``stats`` the partial batch-norm sums as well."""
+    c = torch.empty((S, M, Lp), dtype=torch.float32, device=b_planes.device)
+    lib = L.load()
+    partial = None
+    with torch.cuda.device(b_planes.device):
+        if stats:
+            partial = torch.empty((lib.sjhip_pwconv_gemm_planes_stats_rows(S, Lp), M, 2), dtype=torch.float32, device=c.device)
+        rc = lib.sjhip_pwconv_gemm_planes(w_planes.data_ptr(), M, Kdim, b_planes.data_ptr(), b_terms, L.ptr(b_amax), S, Lp,
+                                          c.data_ptr(), L.ptr(partial), _stream(c))
+    L.check(rc, "pwconv_gemm_planes")
+    return (c, partial) if stats else c
+
+
+def pw_grad_weight_planes(dy_planes: torch.Tensor, dy_amax: torch.Tensor, x_planes: torch.Tensor, x_terms: int,
+                          x_amax: Optional[torch.Tensor], S: int, M: int, N: int, Lp: int) -> torch.Tensor:
+    """``dw [M, N] = sum_{s, l} dy[s, m, l] x[s, n, l]`` from the term planes of ``dy`` (two terms) and of ``x``."""
+    lib = L.load()
+    dev = dy_planes.device
+    ws = torch.empty(lib.sjhip_pwconv_grad_weight_planes_workspace_floats(M, N, S, Lp), dtype=torch.float32, device=dev)
+    dw = torch.empty((M, N), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.sjhip_pwconv_grad_weight_planes(dy_planes.data_ptr(), dy_amax.data_ptr(), x_planes.data_ptr(), x_terms,
+                                                 L.ptr(x_amax), S, M, N, Lp, dw.data_ptr(), ws.data_ptr(), _stream(dw))
+    L.check(rc, "pwconv_grad_weight_planes")
     return dw
 
 

@@ -80,6 +80,12 @@ EXPORTED_SYMBOLS = (
     "sjhip_bn_grad_input_amax",
     "sjhip_pwconv_gemm_f16_bits",
     "sjhip_pwconv_grad_weight_f16_bits",
+    "sjhip_pwconv_plane_elems",
+    "sjhip_pwconv_split_planes",
+    "sjhip_pwconv_gemm_planes_stats_rows",
+    "sjhip_pwconv_gemm_planes",
+    "sjhip_pwconv_grad_weight_planes_workspace_floats",
+    "sjhip_pwconv_grad_weight_planes",
     "sjhip_bn_stats",
     "sjhip_bn_finalize",
     "sjhip_bn_finalize_rows",
@@ -273,6 +279,20 @@ def load() -> ctypes.CDLL:
         lib.sjhip_pwconv_grad_weight_f16_bits.restype = c_int
         lib.sjhip_pwconv_grad_weight_f16_bits.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                                           c_void_p, c_void_p, c_void_p]
+        lib.sjhip_pwconv_plane_elems.restype = c_int64
+        lib.sjhip_pwconv_plane_elems.argtypes = [c_int64, c_int64, c_int64, c_int]
+        lib.sjhip_pwconv_split_planes.restype = c_int
+        lib.sjhip_pwconv_split_planes.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p]
+        lib.sjhip_pwconv_gemm_planes_stats_rows.restype = c_int64
+        lib.sjhip_pwconv_gemm_planes_stats_rows.argtypes = [c_int64, c_int64]
+        lib.sjhip_pwconv_gemm_planes.restype = c_int
+        lib.sjhip_pwconv_gemm_planes.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_int, c_void_p, c_int64, c_int64,
+                                                 c_void_p, c_void_p, c_void_p]
+        lib.sjhip_pwconv_grad_weight_planes_workspace_floats.restype = c_int64
+        lib.sjhip_pwconv_grad_weight_planes_workspace_floats.argtypes = [c_int64, c_int64, c_int64, c_int64]
+        lib.sjhip_pwconv_grad_weight_planes.restype = c_int
+        lib.sjhip_pwconv_grad_weight_planes.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64,
+                                                        c_int64, c_void_p, c_void_p, c_void_p]
         lib.sjhip_bn_stats.restype = c_int
         lib.sjhip_bn_stats.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]
         lib.sjhip_bn_finalize.restype = c_int

@@ -78,7 +78,16 @@ constexpr int kTileK = 32;            // contraction elements per LDS stage (two
 constexpr int kRowBytes = 80;         // K-contiguous operand row in LDS: 32 bf16 + 16 bytes, so that the 16-byte fragment
                                       // reads of eight consecutive rows fall on all 32 banks
 constexpr int kRowPlane = kTile * kRowBytes;
+constexpr int kPlanePitch = 320;      // a k row of a B tile kept as it lies in memory (128 columns of fp16, n contiguous): 256
+                                      // bytes + 64, so that the four k rows a transposing read of 32 lanes touches (64 bytes
+                                      // of each) fall on distinct banks
+static_assert(kTileK * kPlanePitch == kRowPlane, "a B tile takes the same LDS in either layout");
 constexpr int kXcds = 8;
+// where the B operand of pw_gemm_kernel comes from
+constexpr int kBFloat = 0;   // fp32 [S][K][L], split into terms while it is staged
+constexpr int kBBits = 1;    // bit-packed spikes over [S][K][L]
+constexpr int kBPlanes = 2;  // fp16 term planes [TB][K][ld] with the columns of all samples in a row (split_planes_kernel)
+typedef short s16x4 __attribute__((ext_vector_type(4)));
 #ifndef SJHIP_PW_F16_WAVES
 #define SJHIP_PW_F16_WAVES 3
 #endif
@@ -264,6 +273,9 @@ struct PwGemmArgs {
                              // each half (64 columns) of every column block
   const float *a_inverse;    // fp16 terms: the inverse scale of every (padded) row of A
   const float *b_amax;       // fp16 terms: nullptr (b needs no scale), or the words whose maximum is max |b|
+  const uint16_t *b_planes;  // kBPlanes: fp16 terms of b, [TB][K][ld], column s * L + l of row k holds b[s][k][l]
+  int64_t b_plane_stride;    // K * ld
+  int ld;                    // columns per row of a plane: a multiple of 8, at least ncols
 };
 constexpr int kStatPitch = 33;                             // floats per row of the transposing buffer: no bank conflicts
 constexpr unsigned kStatLds = 4 * 64 * kStatPitch * 4;     // one buffer of 64 rows x 32 column pairs per wavefront
@@ -300,11 +312,21 @@ __device__ __forceinline__ u32x4 row_fragment(const uint8_t *plane, int row, int
   return *reinterpret_cast<const u32x4 *>(plane + row * kRowBytes + ks * 32 + (lane >> 5) * 16);
 }
 
-// BITS: b is a spike tensor that arrives bit-packed (the layout of sjhip_bit_pack over [S][K][L]: bit e % 8 of byte e / 8
-// is element e), 1/32 of the bytes of fp32 spikes; a work-item fetches the byte that holds its two columns of a row.
-template <int TA, int TB, bool H, bool BITS = false>
+// BSRC == kBBits: b is a spike tensor that arrives bit-packed (the layout of sjhip_bit_pack over [S][K][L]: bit e % 8 of
+// byte e / 8 is element e), 1/32 of the bytes of fp32 spikes; a work-item fetches the byte that holds its two columns of
+// a row.
+// BSRC == kBPlanes: b arrives as fp16 term planes that its producer wrote already scaled and split, rows of K with the
+// columns of all samples in a row.  A tile of 32 k x 128 columns is copied to LDS as it lies in memory (16 bytes per
+// work-item and row, no arithmetic), and the wavefronts fetch their fragments with the transposing LDS read
+// (ds_read_b64_tr_b16: the 16 lanes of a group each point at four consecutive columns of a k row, four rows of 16
+// columns in all, and lane j of the group receives column j of the four rows), which delivers the eight consecutive k of
+// a column that the matrix cores want from a tile whose rows run along the columns.
+template <int TA, int TB, bool H, int BSRC = kBFloat>
 __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu(pw_waves(H), pw_waves(H)))) pw_gemm_kernel(const PwGemmArgs a) {
+  constexpr bool BITS = BSRC == kBBits;
+  constexpr bool PLANES = BSRC == kBPlanes;
   static_assert(!BITS || TB == 1, "a bit-packed operand has one term");
+  static_assert(!PLANES || H, "term planes are fp16");
   extern __shared__ __align__(16) uint8_t lds[];
   uint8_t *As = lds;                   // [TA][128][kRowBytes]
   uint8_t *Bs = lds + TA * kRowPlane;  // [TB][128][kRowBytes], column-major: a row holds 32 k of one column
@@ -347,11 +369,17 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   const char *b_base = reinterpret_cast<const char *>(a.b);
   float b_scale = 1.0f, b_inverse = 1.0f;
   if (H && TB > 1 && a.b_amax != nullptr) scale_for(tensor_amax(a.b_amax), b_scale, b_inverse);
+  // planes: 16-byte chunk pc (eight columns) of the k rows pr and pr + 16 of every plane
+  const int pc = tid & 15, pr = tid >> 4;
+  const uint32_t ld2 = PLANES ? (uint32_t)a.ld * 2u : 0u;
+  const uint32_t p_col = (PLANES && j0 + 8 * pc < a.ld) ? 16u * pc : 0u;  // (ld is a multiple of 8: a chunk is inside a row or not)
+  const char *bp_base = reinterpret_cast<const char *>(a.b_planes) + j0 * 2;
 
   // Two B tiles are in flight in registers (sets 0 and 1): a tile is requested two multiplications before it is staged,
   // which covers a miss to HBM.  The A tiles (weight planes, a few MB that every block reads) come from L2, one ahead.
   u32x4 ra[TA][2];
-  u32x2 rb[2][8];  // [set][k]: the fp32 bit patterns of the two columns
+  u32x2 rb[2][8];       // [set][k]: the fp32 bit patterns of the two columns
+  u32x4 rbp[2][TB][2];  // planes: [set][term][row pr + 16 i]  (of rb and rbp only the one that the mode uses exists)
   auto fetch_a = [&](int k0) {
 #pragma unroll
     for (int t = 0; t < TA; ++t) {
@@ -361,6 +389,17 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
     }
   };
   auto fetch_b = [&](int k0, int set) {
+    if constexpr (PLANES) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int k = k0 + pr + 16 * i;
+        const uint32_t off = (uint32_t)(k < K ? k : K - 1) * ld2 + p_col;
+#pragma unroll
+        for (int t = 0; t < TB; ++t)
+          rbp[set][t][i] = *reinterpret_cast<const u32x4 *>(bp_base + (int64_t)t * a.b_plane_stride * 2 + off);
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int k = k0 + bk + i;
@@ -379,6 +418,30 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
     for (int t = 0; t < TA; ++t)
 #pragma unroll
       for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4 *>(As + t * kRowPlane + a_dst[i]) = ra[t][i];
+    if constexpr (PLANES) {
+      if (edge_cols || k0 + kTileK > K) {  // rows beyond K and columns beyond the matrix hold zeros
+        const int64_t left = a.ncols - (j0 + 8 * pc);
+        const int nvalid = left < 0 ? 0 : (left > 8 ? 8 : (int)left);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int n = (k0 + pr + 16 * i < K) ? nvalid : 0;
+#pragma unroll
+          for (int t = 0; t < TB; ++t) {
+            u32x4 &v = rbp[set][t][i];
+            v.x &= n >= 2 ? 0xffffffffu : (n == 1 ? 0xffffu : 0u);
+            v.y &= n >= 4 ? 0xffffffffu : (n == 3 ? 0xffffu : 0u);
+            v.z &= n >= 6 ? 0xffffffffu : (n == 5 ? 0xffffu : 0u);
+            v.w &= n >= 8 ? 0xffffffffu : (n == 7 ? 0xffffu : 0u);
+          }
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < TB; ++t)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          *reinterpret_cast<u32x4 *>(Bs + t * kRowPlane + (pr + 16 * i) * kPlanePitch + pc * 16) = rbp[set][t][i];
+      return;
+    }
     if (edge_cols || k0 + kTileK > K) {
 #pragma unroll
       for (int i = 0; i < 8; ++i)
@@ -429,7 +492,21 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int t = 0; t < TB; ++t) bf[nt][t] = row_fragment(Bs + t * kRowPlane, wn * 64 + nt * 32 + (lane & 31), ks, lane);
+        for (int t = 0; t < TB; ++t) {
+          if constexpr (PLANES) {
+            // group g = lane / 16 of a transposing read: columns 16 (g % 2) + 0..15 of the 32, k rows 8 (g / 2) + 0..3 (and + 4
+            // in the second read) of the 16; lane i of the group points at columns 4 (i % 4) + 0..3 of row i / 4
+            const int g = lane >> 4, i = lane & 15;
+            const uint8_t *src = Bs + t * kRowPlane + (ks * 16 + 8 * (g >> 1) + (i >> 2)) * kPlanePitch +
+                                 (wn * 64 + nt * 32 + 16 * (g & 1) + 4 * (i & 3)) * 2;
+            typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+            const u32x2 k03 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(src)));
+            const u32x2 k47 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(src + 4 * kPlanePitch)));
+            bf[nt][t].x = k03.x; bf[nt][t].y = k03.y; bf[nt][t].z = k47.x; bf[nt][t].w = k47.y;
+          } else {
+            bf[nt][t] = row_fragment(Bs + t * kRowPlane, wn * 64 + nt * 32 + (lane & 31), ks, lane);
+          }
+        }
       mfma_step<TA, TB, H>(af, bf, acc);
     }
   };
@@ -752,6 +829,202 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   }
 }
 
+
+struct PwDwPlanesArgs {
+  const uint16_t *dy_planes;  // [2][M][ld] fp16 terms of dy, column s * L + l of row m holds dy[s][m][l]
+  const uint16_t *x_planes;   // [TB][N][ld], likewise
+  float *partials;            // [chunks][M][N]
+  int64_t dy_plane_stride, x_plane_stride;  // M * ld, N * ld
+  int64_t ncols;              // S * L
+  int ld;
+  int M, N;
+  int64_t steps_per_chunk;    // K steps (32 columns each) per partial tile
+  int m_blocks, n_blocks;
+  const float *dy_amax, *x_amax;
+};
+
+// The weight gradient from term planes: dW[m][n] = sum_j dy[m][j] x[n][j] with both operands contiguous along the
+// contraction index j (the columns of all samples in a row), so a tile of either is copied to LDS as it lies in memory,
+// 16 bytes per work-item and row, and read back as fragments; no arithmetic on the way, and no sample boundaries.
+template <int TB>
+__global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) pw_dw_planes_kernel(const PwDwPlanesArgs a) {
+  constexpr int TA = 2;
+  extern __shared__ __align__(16) uint8_t lds[];
+  uint8_t *As = lds;                   // [TA][128][kRowBytes]
+  uint8_t *Bs = lds + TA * kRowPlane;  // [TB][128][kRowBytes]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t logical = xcd_order(blockIdx.x, gridDim.x);
+  const int tiles = a.m_blocks * a.n_blocks;
+  const int chunk = (int)(logical / tiles);
+  const int tile = (int)(logical % tiles);
+  const int mb = tile % a.m_blocks, nb = tile / a.m_blocks;
+  const int m0 = mb * kTile, n0 = nb * kTile;
+  const int M = a.M, N = a.N;
+  const int64_t steps_total = (a.ncols + kTileK - 1) / kTileK;
+  const int64_t it_begin = (int64_t)chunk * a.steps_per_chunk;
+  const int64_t it_end = it_begin + a.steps_per_chunk < steps_total ? it_begin + a.steps_per_chunk : steps_total;
+  const int64_t iters = it_end - it_begin;
+
+  // a work-item copies the 16-byte chunks q = tid and tid + 256 of a tile: row q / 4, eight columns 8 (q % 4)
+  const uint32_t ld2 = (uint32_t)a.ld * 2u;
+  uint32_t a_off[2], b_off[2];
+  int dst[2];
+  const int kc = tid & 3;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = (tid >> 2) + 64 * i;
+    a_off[i] = (uint32_t)(m0 + row < M ? m0 + row : M - 1) * ld2;
+    b_off[i] = (uint32_t)(n0 + row < N ? n0 + row : N - 1) * ld2;
+    dst[i] = row * kRowBytes + kc * 16;
+  }
+  const bool edge_rows = __builtin_amdgcn_readfirstlane((m0 + kTile > M || n0 + kTile > N) ? 1 : 0) != 0;
+  const char *dy_base = reinterpret_cast<const char *>(a.dy_planes);
+  const char *x_base = reinterpret_cast<const char *>(a.x_planes);
+  float a_scale, a_inverse = 1.0f, b_scale, b_inverse = 1.0f;
+  if (a.dy_amax != nullptr) scale_for(tensor_amax(a.dy_amax), a_scale, a_inverse);
+  if (TB > 1 && a.x_amax != nullptr) scale_for(tensor_amax(a.x_amax), b_scale, b_inverse);
+  u32x4 ra[2][TA][2], rb[2][TB][2];  // two tiles in flight
+  auto fetch = [&](int64_t it, int set) {
+    const int64_t j = (it_begin + it) * kTileK;  // first column of the step; a chunk beyond the row is fetched from its start
+    const uint32_t col = (j + 8 * kc < a.ld) ? (uint32_t)kc * 16u : 0u;
+    const char *pa = dy_base + j * 2, *pb = x_base + j * 2;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int t = 0; t < TA; ++t) ra[set][t][i] = *reinterpret_cast<const u32x4 *>(pa + (int64_t)t * a.dy_plane_stride * 2 + (a_off[i] + col));
+#pragma unroll
+      for (int t = 0; t < TB; ++t) rb[set][t][i] = *reinterpret_cast<const u32x4 *>(pb + (int64_t)t * a.x_plane_stride * 2 + (b_off[i] + col));
+    }
+  };
+  auto stage = [&](int64_t it, int set) {
+    const int64_t j = (it_begin + it) * kTileK;
+    const bool tail = j + kTileK > a.ncols;
+    if (edge_rows || tail) {  // rows beyond the matrices and columns beyond the last sample hold zeros
+      const int64_t left = a.ncols - (j + 8 * kc);
+      const int nvalid = left < 0 ? 0 : (left > 8 ? 8 : (int)left);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int row = (tid >> 2) + 64 * i;
+        const int na = m0 + row < M ? nvalid : 0, nb_ = n0 + row < N ? nvalid : 0;
+#pragma unroll
+        for (int t = 0; t < TA; ++t) {
+          u32x4 &v = ra[set][t][i];
+          v.x &= na >= 2 ? 0xffffffffu : (na == 1 ? 0xffffu : 0u);
+          v.y &= na >= 4 ? 0xffffffffu : (na == 3 ? 0xffffu : 0u);
+          v.z &= na >= 6 ? 0xffffffffu : (na == 5 ? 0xffffu : 0u);
+          v.w &= na >= 8 ? 0xffffffffu : (na == 7 ? 0xffffu : 0u);
+        }
+#pragma unroll
+        for (int t = 0; t < TB; ++t) {
+          u32x4 &v = rb[set][t][i];
+          v.x &= nb_ >= 2 ? 0xffffffffu : (nb_ == 1 ? 0xffffu : 0u);
+          v.y &= nb_ >= 4 ? 0xffffffffu : (nb_ == 3 ? 0xffffu : 0u);
+          v.z &= nb_ >= 6 ? 0xffffffffu : (nb_ == 5 ? 0xffffu : 0u);
+          v.w &= nb_ >= 8 ? 0xffffffffu : (nb_ == 7 ? 0xffffu : 0u);
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int t = 0; t < TA; ++t) *reinterpret_cast<u32x4 *>(As + t * kRowPlane + dst[i]) = ra[set][t][i];
+#pragma unroll
+      for (int t = 0; t < TB; ++t) *reinterpret_cast<u32x4 *>(Bs + t * kRowPlane + dst[i]) = rb[set][t][i];
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.0f;
+
+  auto multiply = [&](int64_t it) {
+    // the second half of the last step of the matrix may hold nothing
+    const int ksteps = (a.ncols - (it_begin + it) * kTileK <= 16) ? 1 : 2;
+    for (int ks = 0; ks < ksteps; ++ks) {
+      u32x4 af[2][TA], bf[2][TB];
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int t = 0; t < TA; ++t) af[mt][t] = row_fragment(As + t * kRowPlane, wm * 64 + mt * 32 + (lane & 31), ks, lane);
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int t = 0; t < TB; ++t) bf[nt][t] = row_fragment(Bs + t * kRowPlane, wn * 64 + nt * 32 + (lane & 31), ks, lane);
+      mfma_step<TA, TB, true>(af, bf, acc);
+    }
+  };
+  // as in pw_gemm_kernel: unconditional requests in the steady state, conditions only in the last steps
+  auto step = [&](int64_t it, int set, bool more) {
+    __syncthreads();
+    stage(it, set);
+    __syncthreads();
+    if (more) fetch(it + 2, set);
+    multiply(it);
+  };
+  if (iters > 0) fetch(0, 0);
+  if (iters > 1) fetch(1, 1);
+  int64_t it = 0;
+  for (; it + 3 < iters; it += 2) {
+    step(it, 0, true);
+    step(it + 1, 1, true);
+  }
+  if (it < iters) step(it, 0, it + 2 < iters);
+  if (it + 1 < iters) step(it + 1, 1, false);
+  if (it + 2 < iters) step(it + 2, 0, false);
+
+  float *out = a.partials + (int64_t)chunk * M * N;
+  const float inv = a_inverse * b_inverse;
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    const int col = n0 + wn * 64 + nt * 32 + (lane & 31);
+    if (col >= N) continue;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const int rbase = m0 + wm * 64 + mt * 32 + 4 * (lane >> 5);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = rbase + 8 * (r >> 2) + (r & 3);
+        if (row < M) out[(int64_t)row * N + col] = acc[mt][nt][r] * inv;
+      }
+    }
+  }
+}
+
+// planes[t][c][s * L + l] = term t of scale * x[s][c][l] for x [S][C][L] fp32: two fp16 terms (TERMS == 2: the scale is the
+// power of two that the words of amax give, as in the kernels that split on the fly) or one (TERMS == 1: values that
+// fp16 holds exactly, no scale).  A work-item takes four consecutive l.
+template <int TERMS>
+__global__ void __launch_bounds__(256) split_planes_kernel(const float *x, int64_t quads, int C, int L, const float *amax,
+                                                            uint16_t *planes, int64_t plane_stride, int ld) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  float scale = 1.0f, inverse = 1.0f;
+  if (TERMS > 1 && amax != nullptr) scale_for(tensor_amax(amax), scale, inverse);
+  if (i >= quads) return;
+  const int qpr = L >> 2;
+  const int64_t row = i / qpr;  // s * C + c
+  const int l = (int)(i - row * qpr) * 4;
+  const int64_t s = row / C;
+  const int c = (int)(row - s * C);
+  f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x) + i);
+  v *= scale;
+  uint32_t w01[TERMS], w23[TERMS];
+  split_pair<TERMS, true>(v.x, v.y, w01);
+  split_pair<TERMS, true>(v.z, v.w, w23);
+  uint16_t *dst = planes + (int64_t)c * ld + s * L + l;
+#pragma unroll
+  for (int t = 0; t < TERMS; ++t) {
+    u32x2 w;
+    w.x = w01[t];
+    w.y = w23[t];
+    *reinterpret_cast<u32x2 *>(dst + (int64_t)t * plane_stride) = w;
+  }
+}
+
 __global__ void __launch_bounds__(256) dw_reduce_scalar_kernel(const float *partials, int chunks, int64_t count, float *out) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= count) return;
@@ -780,11 +1053,11 @@ __global__ void __launch_bounds__(256) dw_reduce_kernel(const float *partials, i
 
 int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
-template <int TA, int TB, bool H = false, bool BITS = false>
+template <int TA, int TB, bool H = false, int BSRC = kBFloat>
 int launch_gemm_terms(const PwGemmArgs &a, int64_t blocks, hipStream_t stream) {
   unsigned lds = (TA + TB) * kRowPlane;
   if (a.stats && lds < kStatLds) lds = kStatLds;
-  hipLaunchKernelGGL((pw_gemm_kernel<TA, TB, H, BITS>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
+  hipLaunchKernelGGL((pw_gemm_kernel<TA, TB, H, BSRC>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
   return check_launch("pwconv_gemm");
 }
 
@@ -845,6 +1118,7 @@ int launch_pwconv_amax(const float *x, int64_t n, float *amax, hipStream_t strea
 
 namespace {
 const int64_t kPwOffsetLimit = int64_t(1) << 30;  // per-lane offsets into A and B are 32-bit byte offsets
+const int64_t kPwPlaneLimit = int64_t(1) << 30;   // elements of one fp16 plane: 32-bit byte offsets within it
 int64_t gemm_samples_per_launch(int64_t K, int64_t L) { return (kPwOffsetLimit - 1) / (K * L); }
 }  // namespace
 
@@ -882,6 +1156,7 @@ int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t
     a.stats = stats;
     a.a_inverse = reinterpret_cast<const float *>(a_planes + 2 * a.plane_stride);
     a.b_amax = b_amax;
+    a.b_planes = nullptr; a.b_plane_stride = 0; a.ld = 0;
     if (stats) stats += 2 * ((a.ncols + kTile - 1) / kTile) * M * 2;
     const int64_t blocks = a.m_blocks * ((a.ncols + kTile - 1) / kTile);
     if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: %lld blocks", (long long)blocks);
@@ -894,7 +1169,7 @@ int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t
       case 11: rc = launch_gemm_terms<1, 1>(a, blocks, stream); break;
       case (SJHIP_PW_F16 | 2) * 10 + 2: rc = launch_gemm_terms<2, 2, true>(a, blocks, stream); break;
       case (SJHIP_PW_F16 | 2) * 10 + 1:
-        rc = b_bits ? launch_gemm_terms<2, 1, true, true>(a, blocks, stream) : launch_gemm_terms<2, 1, true>(a, blocks, stream);
+        rc = b_bits ? launch_gemm_terms<2, 1, true, kBBits>(a, blocks, stream) : launch_gemm_terms<2, 1, true>(a, blocks, stream);
         break;
       default: return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm: %d weight terms with %d activation terms (bf16: 3/3, 3/1, 2/2, 2/1, 1/1; fp16: 2/2, 2/1)", a_terms, b_terms);
     }
@@ -954,6 +1229,109 @@ int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *dy_ama
     rc = check_launch("pwconv_grad_weight(reduce)");
   }
   return rc;
+}
+
+// ---- operands that arrive as fp16 term planes -------------------------------------------------------------------------
+namespace {
+// K steps per partial tile of the weight gradient from planes: as dw_samples_per_chunk, over the steps of 32 columns
+int64_t dw_planes_steps_per_chunk(int64_t ncols, int tiles) {
+  const int64_t steps = (ncols + kTileK - 1) / kTileK;
+  const int rounds = tiles >= 16 ? 2 : 1;
+  int64_t chunks = (int64_t)rounds * 512 / tiles;
+  if (chunks < 1) chunks = 1;
+  if (chunks > steps) chunks = steps > 0 ? steps : 1;
+  return (steps + chunks - 1) / chunks;
+}
+}  // namespace
+
+int64_t pwconv_plane_ld(int64_t S, int64_t L) { return round_up(S * L, 8); }
+
+int launch_pwconv_split_planes(const float *x, int64_t S, int64_t C, int64_t L, int terms, const float *amax, uint16_t *planes,
+                               hipStream_t stream) {
+  if (S < 1 || C < 1 || L < 1 || L % 4 != 0 || !aligned16(x) || !aligned16(planes) || (terms != 1 && terms != 2))
+    return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_split_planes: S=%lld C=%lld L=%lld (a multiple of 4), %d terms (1 or 2), 16-byte aligned buffers", (long long)S, (long long)C, (long long)L, terms);
+  if (terms == 2 && (amax == nullptr || !aligned16(amax)))
+    return fail(SJHIP_ERR_INVALID, "pwconv_split_planes: two terms need the 16-byte aligned amax buffer of the tensor");
+  const int64_t ld = pwconv_plane_ld(S, L);
+  if (C > (1 << 24) || L > (1 << 24) || C * ld >= kPwPlaneLimit)
+    return fail(SJHIP_ERR_TOO_LARGE, "pwconv_split_planes: S=%lld C=%lld L=%lld", (long long)S, (long long)C, (long long)L);
+  const int64_t quads = S * C * (L / 4), blocks = (quads + 255) / 256;
+  if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_split_planes: %lld elements", (long long)(quads * 4));
+  if (terms == 2)
+    hipLaunchKernelGGL(split_planes_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, stream, x, quads, (int)C, (int)L, amax, planes, C * ld, (int)ld);
+  else
+    hipLaunchKernelGGL(split_planes_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, stream, x, quads, (int)C, (int)L, amax, planes, C * ld, (int)ld);
+  return check_launch("pwconv_split_planes");
+}
+
+int64_t pwconv_gemm_planes_stats_rows(int64_t S, int64_t L) { return 2 * ((S * L + kTile - 1) / kTile); }
+
+int launch_pwconv_gemm_planes(const uint16_t *a_planes, int64_t M, int64_t K, const uint16_t *b_planes, int b_terms,
+                              const float *b_amax, int64_t S, int64_t L, float *c, float *stats, hipStream_t stream) {
+  if (M < 1 || K < 1 || S < 1 || L < 1 || !aligned16(a_planes) || !aligned16(b_planes) || (b_terms != 1 && b_terms != 2))
+    return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_gemm_planes: M=%lld K=%lld S=%lld L=%lld, %d activation terms (1 or 2), 16-byte aligned planes", (long long)M, (long long)K, (long long)S, (long long)L, b_terms);
+  if (b_terms == 2 && (b_amax == nullptr || !aligned16(b_amax)))
+    return fail(SJHIP_ERR_INVALID, "pwconv_gemm_planes: two activation terms need the 16-byte aligned amax buffer they were scaled by");
+  const int64_t ld = pwconv_plane_ld(S, L);
+  if (round_up(M, kTile) * round_up(K, kTileK) >= kPwOffsetLimit || K * ld >= kPwPlaneLimit || M * L >= (int64_t(1) << 40))
+    return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm_planes: M=%lld K=%lld S=%lld L=%lld", (long long)M, (long long)K, (long long)S, (long long)L);
+  PwGemmArgs a;
+  a.a_planes = a_planes; a.b = nullptr; a.c = c;
+  a.M = (int)M; a.K = (int)K; a.K_pad = (int)round_up(K, kTileK); a.L = (int)L;
+  a.plane_stride = round_up(M, kTile) * a.K_pad;
+  a.ncols = S * L;
+  a.m_blocks = (int)(round_up(M, kTile) / kTile);
+  a.stats = stats;
+  a.a_inverse = reinterpret_cast<const float *>(a_planes + 2 * a.plane_stride);
+  a.b_amax = b_terms == 2 ? b_amax : nullptr;
+  a.b_planes = b_planes; a.b_plane_stride = K * ld; a.ld = (int)ld;
+  const int64_t blocks = a.m_blocks * ((a.ncols + kTile - 1) / kTile);
+  if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm_planes: %lld blocks", (long long)blocks);
+  ProfileScope prof(KC_PW_GEMM, stream);
+  return b_terms == 2 ? launch_gemm_terms<2, 2, true, kBPlanes>(a, blocks, stream)
+                      : launch_gemm_terms<2, 1, true, kBPlanes>(a, blocks, stream);
+}
+
+int64_t pwconv_dw_planes_workspace_floats(int64_t M, int64_t N, int64_t S, int64_t L) {
+  const int tiles = (int)(round_up(M, kTile) / kTile * (round_up(N, kTile) / kTile));
+  const int64_t steps = (S * L + kTileK - 1) / kTileK, spc = dw_planes_steps_per_chunk(S * L, tiles);
+  return (steps + spc - 1) / spc * M * N;
+}
+
+int launch_pwconv_grad_weight_planes(const uint16_t *dy_planes, const float *dy_amax, const uint16_t *x_planes, int x_terms,
+                                     const float *x_amax, int64_t S, int64_t M, int64_t N, int64_t L, float *dw,
+                                     float *workspace, hipStream_t stream) {
+  if (M < 1 || N < 1 || S < 1 || L < 1 || !aligned16(dy_planes) || !aligned16(x_planes) || (x_terms != 1 && x_terms != 2))
+    return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_grad_weight_planes: M=%lld N=%lld S=%lld L=%lld, %d activation terms (1 or 2), 16-byte aligned planes", (long long)M, (long long)N, (long long)S, (long long)L, x_terms);
+  if (dy_amax == nullptr || !aligned16(dy_amax) || (x_terms == 2 && (x_amax == nullptr || !aligned16(x_amax))))
+    return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight_planes: operands of two terms need the 16-byte aligned amax buffers they were scaled by");
+  const int64_t ld = pwconv_plane_ld(S, L);
+  if (M * ld >= kPwPlaneLimit || N * ld >= kPwPlaneLimit || M * N >= (int64_t(1) << 40))
+    return fail(SJHIP_ERR_TOO_LARGE, "pwconv_grad_weight_planes: M=%lld N=%lld S=%lld L=%lld", (long long)M, (long long)N, (long long)S, (long long)L);
+  PwDwPlanesArgs a;
+  a.dy_planes = dy_planes; a.x_planes = x_planes; a.partials = workspace;
+  a.dy_plane_stride = M * ld; a.x_plane_stride = N * ld; a.ncols = S * L; a.ld = (int)ld;
+  a.M = (int)M; a.N = (int)N;
+  a.m_blocks = (int)(round_up(M, kTile) / kTile);
+  a.n_blocks = (int)(round_up(N, kTile) / kTile);
+  a.dy_amax = dy_amax; a.x_amax = x_terms == 2 ? x_amax : nullptr;
+  const int tiles = a.m_blocks * a.n_blocks;
+  a.steps_per_chunk = dw_planes_steps_per_chunk(a.ncols, tiles);
+  const int64_t steps = (a.ncols + kTileK - 1) / kTileK;
+  const int chunks = (int)((steps + a.steps_per_chunk - 1) / a.steps_per_chunk);
+  const int64_t blocks = (int64_t)tiles * chunks;
+  ProfileScope prof(KC_PW_GRAD_WEIGHT, stream);
+  const unsigned lds = (2 + x_terms) * kRowPlane;
+  if (x_terms == 2) hipLaunchKernelGGL(pw_dw_planes_kernel<2>, dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
+  else hipLaunchKernelGGL(pw_dw_planes_kernel<1>, dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
+  int rc = check_launch("pwconv_grad_weight_planes");
+  if (rc != SJHIP_OK) return rc;
+  const int64_t count = M * N;
+  if (count % 4 == 0 && aligned16(workspace) && aligned16(dw))
+    hipLaunchKernelGGL(dw_reduce_kernel, dim3((unsigned)((count / 4 + 255) / 256)), dim3(256), 0, stream, workspace, chunks, count, dw);
+  else
+    hipLaunchKernelGGL(dw_reduce_scalar_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, workspace, chunks, count, dw);
+  return check_launch("pwconv_grad_weight_planes(reduce)");
 }
 
 }  // namespace sjhip

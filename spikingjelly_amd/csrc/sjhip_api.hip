@@ -659,6 +659,46 @@ int sjhip_pwconv_grad_weight_f16_bits(const float *dy, const float *dy_amax, con
                                    workspace, static_cast<hipStream_t>(stream), true);
 }
 
+int64_t sjhip_pwconv_plane_elems(int64_t S, int64_t C, int64_t L, int terms) {
+  if (S < 1 || C < 1 || L < 1 || terms < 1 || terms > 2 || S > (int64_t(1) << 40) / L) return 0;
+  return terms * C * pwconv_plane_ld(S, L);
+}
+
+int sjhip_pwconv_split_planes(const float *x, int64_t S, int64_t C, int64_t L, int terms, const float *amax, uint16_t *planes,
+                              void *stream) {
+  if (!x || !planes) return fail(SJHIP_ERR_INVALID, "pwconv_split_planes: NULL buffer");
+  if (S < 1 || C < 1 || L < 1 || S > (int64_t(1) << 40) / L) return fail(SJHIP_ERR_INVALID, "pwconv_split_planes: S=%lld C=%lld L=%lld", (long long)S, (long long)C, (long long)L);
+  return launch_pwconv_split_planes(x, S, C, L, terms, amax, planes, static_cast<hipStream_t>(stream));
+}
+
+int64_t sjhip_pwconv_gemm_planes_stats_rows(int64_t S, int64_t L) {
+  if (S < 1 || L < 1 || S > (int64_t(1) << 40) / L) return 0;
+  return pwconv_gemm_planes_stats_rows(S, L);
+}
+
+int sjhip_pwconv_gemm_planes(const uint16_t *a_planes, int64_t M, int64_t K, const uint16_t *b_planes, int b_terms,
+                             const float *b_amax, int64_t S, int64_t L, float *c, float *partial, void *stream) {
+  if (!a_planes || !b_planes || !c) return fail(SJHIP_ERR_INVALID, "pwconv_gemm_planes: NULL buffer");
+  if (M < 1 || K < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_gemm_planes: M=%lld K=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)K, (long long)S, (long long)L);
+  if (S > (int64_t(1) << 40) / L) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm_planes: S*L overflows");
+  return launch_pwconv_gemm_planes(a_planes, M, K, b_planes, b_terms, b_amax, S, L, c, partial, static_cast<hipStream_t>(stream));
+}
+
+int64_t sjhip_pwconv_grad_weight_planes_workspace_floats(int64_t M, int64_t N, int64_t S, int64_t L) {
+  if (M < 1 || N < 1 || S < 1 || L < 1 || S > (int64_t(1) << 40) / L) return 0;
+  return pwconv_dw_planes_workspace_floats(M, N, S, L);
+}
+
+int sjhip_pwconv_grad_weight_planes(const uint16_t *dy_planes, const float *dy_amax, const uint16_t *x_planes, int x_terms,
+                                    const float *x_amax, int64_t S, int64_t M, int64_t N, int64_t L, float *dw, float *workspace,
+                                    void *stream) {
+  if (!dy_planes || !x_planes || !dw || !workspace) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight_planes: NULL buffer");
+  if (M < 1 || N < 1 || S < 1 || L < 1) return fail(SJHIP_ERR_INVALID, "pwconv_grad_weight_planes: M=%lld N=%lld S=%lld L=%lld must be >= 1", (long long)M, (long long)N, (long long)S, (long long)L);
+  if (S > (int64_t(1) << 40) / L) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_grad_weight_planes: S*L overflows");
+  return launch_pwconv_grad_weight_planes(dy_planes, dy_amax, x_planes, x_terms, x_amax, S, M, N, L, dw, workspace,
+                                          static_cast<hipStream_t>(stream));
+}
+
 int sjhip_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, void *stream) {
   if (!y || !partial) return fail(SJHIP_ERR_INVALID, "bn_stats: NULL buffer");
   return launch_bn_stats(y, S, C, L, partial, static_cast<hipStream_t>(stream));

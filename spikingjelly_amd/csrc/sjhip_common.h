@@ -457,6 +457,16 @@ int64_t pwconv_dw_workspace_floats(int64_t M, int64_t N, int64_t S);
 int launch_pwconv_grad_weight(const float *dy, int dy_terms, const float *dy_amax, const float *x, int x_terms,
                               const float *x_amax, int64_t S, int64_t M, int64_t N, int64_t L, float *dw, float *workspace,
                               hipStream_t stream, bool x_bits = false);
+int64_t pwconv_plane_ld(int64_t S, int64_t L);
+int launch_pwconv_split_planes(const float *x, int64_t S, int64_t C, int64_t L, int terms, const float *amax, uint16_t *planes,
+                               hipStream_t stream);
+int64_t pwconv_gemm_planes_stats_rows(int64_t S, int64_t L);
+int launch_pwconv_gemm_planes(const uint16_t *a_planes, int64_t M, int64_t K, const uint16_t *b_planes, int b_terms,
+                              const float *b_amax, int64_t S, int64_t L, float *c, float *stats, hipStream_t stream);
+int64_t pwconv_dw_planes_workspace_floats(int64_t M, int64_t N, int64_t S, int64_t L);
+int launch_pwconv_grad_weight_planes(const uint16_t *dy_planes, const float *dy_amax, const uint16_t *x_planes, int x_terms,
+                                     const float *x_amax, int64_t S, int64_t M, int64_t N, int64_t L, float *dw,
+                                     float *workspace, hipStream_t stream);
 int launch_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, hipStream_t stream);
 int launch_bn_finalize(const float *partial, int64_t rows, int64_t count, int64_t C, const float *gamma, const float *beta, float eps,
                        float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
