@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define SJHIP_ABI_VERSION 4
+#define SJHIP_ABI_VERSION 5
 
 typedef enum sjhip_status {
   SJHIP_OK = 0,
@@ -501,34 +501,47 @@ int sjhip_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int 
  * operands split into two fp16 terms and the three products hi*hi, hi*lo, lo*hi on v_mfma_f32_32x32x16_f16: half the
  * matrix-core work of the three-term bf16 split at the same accuracy class.  fp16 has 11 significant bits but a narrow
  * exponent range, so every operand is scaled by a power of two first (exact) and the scales are taken out of the result
- * (exact): weights per row of A, inside sjhip_pwconv_split_weight_f16; activations and gradients per tensor, by the power
- * of two that takes the tensor's largest finite magnitude `amax` into [2^14, 2^15) (1 for a zero or subnormal amax;
- * infinities and NaNs take no part in it and propagate through the products as in fp32),
- * which the kernels derive from a device buffer of SJHIP_PW_AMAX_FLOATS non-negative floats whose maximum is amax
- * (several words, so that the blocks that fold their maxima into it do not meet on one address; 16-byte aligned).  An element above 2^-16 of amax is represented to 2^-23
- * relative or better, a smaller one to 2^-39 of amax; the dropped product lo*lo is below 2^-22 of hi*hi.  Measured
+ * (exact): weights per row of A, inside sjhip_pwconv_split_weight_f16; activations and gradients by the power of two
+ * that takes a largest finite magnitude `amax` into [2^14, 2^15) (1 for a zero or subnormal amax; infinities and NaNs take
+ * no part in it and propagate through the products as in fp32).  Which magnitude: in sjhip_pwconv_gemm_f16, whose output
+ * columns are (sample, position) pairs, every sample s of b is scaled by its own amax (the scale leaves the sum over k
+ * of a column untouched), so a sample whose values are all small beside another's keeps its significant bits; in the
+ * weight gradient, which sums over samples and positions, by the amax of the whole tensor (what a small sample adds to
+ * that sum is small beside the rest).  The kernels derive both from one device buffer per tensor of
+ * sjhip_pwconv_amax_floats(S) = SJHIP_PW_AMAX_FLOATS + SJHIP_PW_AMAX_SAMPLE_WORDS * S non-negative floats, 16-byte
+ * aligned: the first SJHIP_PW_AMAX_FLOATS words have the tensor's amax as their maximum (several words, so that the
+ * blocks that fold their maxima into it do not meet on one address), and the amax of sample s is the maximum of the
+ * words SJHIP_PW_AMAX_FLOATS + SJHIP_PW_AMAX_SAMPLE_WORDS * s + r, r < SJHIP_PW_AMAX_SAMPLE_WORDS.  An element above
+ * 2^-16 of the amax it is scaled by is represented to 2^-23 relative or better, a smaller one to 2^-39 of that amax
+ * (within one sample the spread between positions is not compensated: a token column whose values all lie below 2^-17
+ * of its sample's amax loses significant bits; configure the bf16 split, which has fp32's exponent range, for such
+ * data); the dropped product lo*lo is below 2^-22 of hi*hi.  Measured
  * against float64 on operands whose rows span four decades: 2^-23 of sum |a||b| (three bf16 terms: 2^-26; an fp32 dot
  * product of 384 terms: 2^-20).  An operand that fp16 holds exactly (spikes, integers up to 2048) takes one term and no
  * scale (terms = 1, amax = NULL).
  *
  *   sjhip_pwconv_split_weight_f16  planes: an opaque buffer of sjhip_pwconv_planes_elems(rows, cols) 2-byte elements,
  *                                  16-byte aligned (two fp16 planes in the tile order of sjhip_pwconv_split_weight,
- *                                  then the inverse row scales); amax_reset: NULL, or an amax buffer that the
- *                                  launch also sets to zero (that of the activations the planes will multiply, so
- *                                  that no launch is spent on clearing it)
- *   sjhip_pwconv_amax              folds max |x| over the finite ones of the n elements of x into amax[SJHIP_PW_AMAX_FLOATS]:
- *                                  afterwards max(amax[]) is the larger of what it was and max |x|; all zero before
- *                                  the first call for a tensor; one launch
+ *                                  then the inverse row scales); amax_reset: NULL, or an amax buffer for
+ *                                  amax_reset_samples samples that the launch also sets to zero (that of the
+ *                                  activations the planes will multiply, so that no launch is spent on clearing it)
+ *   sjhip_pwconv_amax              folds max |x| over the finite ones of the elements of x (S samples of per_sample
+ *                                  elements each) into amax[sjhip_pwconv_amax_floats(S)]: afterwards the maximum of
+ *                                  the first SJHIP_PW_AMAX_FLOATS words is the larger of what it was and max |x|, and
+ *                                  the maximum of the words of sample s likewise for that sample; all zero before the
+ *                                  first call for a tensor; one launch
  *   sjhip_pwconv_gemm_f16          sjhip_pwconv_gemm / sjhip_pwconv_gemm_stats (partial != NULL) on fp16 planes;
- *                                  b_terms 2 with the b_amax buffer of b (a larger maximum is safe, a smaller one is
- *                                  not), or 1 with NULL
+ *                                  b_terms 2 with the b_amax buffer of b (sjhip_pwconv_amax_floats(S) floats; larger
+ *                                  maxima are safe, smaller ones are not), or 1 with NULL
  *   sjhip_pwconv_grad_weight_f16   sjhip_pwconv_grad_weight with two terms of dy (dy_amax) and x_terms of x
  */
 #define SJHIP_PW_F16 16          /* internal term code of an fp16 operand: SJHIP_PW_F16 | terms */
 #define SJHIP_PW_AMAX_FLOATS 256
+#define SJHIP_PW_AMAX_SAMPLE_WORDS 16 /* words per sample (blocks that meet on one address fold one after the other) */
+int64_t sjhip_pwconv_amax_floats(int64_t S);
 int sjhip_pwconv_split_weight_f16(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, float *amax_reset,
-                                  void *stream);
-int sjhip_pwconv_amax(const float *x, int64_t n, float *amax, void *stream);
+                                  int64_t amax_reset_samples, void *stream);
+int sjhip_pwconv_amax(const float *x, int64_t S, int64_t per_sample, float *amax, void *stream);
 int sjhip_pwconv_gemm_f16(const uint16_t *a_planes, int64_t M, int64_t K, const float *b, int b_terms, const float *b_amax,
                           int64_t S, int64_t L, float *c, float *partial, void *stream);
 int sjhip_pwconv_grad_weight_f16(const float *dy, const float *dy_amax, const float *x, int x_terms, const float *x_amax,
@@ -550,7 +563,8 @@ int sjhip_pwconv_grad_weight_f16_bits(const float *dy, const float *dy_amax, con
  * layer/attention.py:310-329, model/spikformer.py:85-99).  A plane buffer of a tensor x [S][C][L] holds `terms` planes
  * [C][ld] of fp16, ld = S * L rounded up to a multiple of 8 (16-byte aligned rows): element (c, s * L + l) of plane 0 is
  * fp16(scale x[s][c][l]), of plane 1 fp16 of the remainder; scale is the power of two that the tensor's amax buffer gives
- * (as for sjhip_pwconv_gemm_f16), so the same amax buffer must accompany the planes into every GEMM that reads them.  The
+ * (the tensor's amax, the first SJHIP_PW_AMAX_FLOATS words of its buffer: planes carry one scale for all their uses), so the
+ * same amax buffer must accompany the planes into every GEMM that reads them.  The
  * columns beyond S * L are never read as data.  The channel-major layout makes the columns of all samples one contiguous
  * contraction (weight gradient) or output (forward, input gradient) index; results agree with the *_f16 calls to the
  * rounding of the fp32 accumulation order.
@@ -598,7 +612,8 @@ int sjhip_pwconv_grad_weight_planes(const uint16_t *dy_planes, const float *dy_a
  *                       (or NULL) and partial[b][c] = (sum g, sum g y) over the row and all steps
  *   sjhip_bn_backward_finalize   dgamma, dbeta (either may be NULL) and coef [3][C] = (p, q, r) of dy = p g + q y + r;
  *                       training != 0: batch statistics took part in the forward, else q = r = 0; amax_reset: NULL, or
- *                       the amax buffer (SJHIP_PW_AMAX_FLOATS floats) of a following sjhip_bn_grad_input_amax, set to zero
+ *                       the amax buffer (sjhip_pwconv_amax_floats(T * B) floats) of a following sjhip_bn_grad_input_amax,
+ *                       set to zero
  *   sjhip_bn_grad_input    dy = p_c g + q_c y + r_c over [S][C][L]; dy may be g
  */
 int sjhip_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *partial, void *stream);
@@ -619,8 +634,8 @@ int sjhip_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64
                                const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef, float *amax_reset,
                                void *stream);
 int sjhip_bn_grad_input(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy, void *stream);
-/* sjhip_bn_grad_input that also folds max |dy| into amax as sjhip_pwconv_amax(dy) would (same contract:
- * SJHIP_PW_AMAX_FLOATS floats, zero before the call): the fp16 GEMMs that consume dy (the two gradients of the convolution in front of the
+/* sjhip_bn_grad_input that also folds max |dy| into amax as sjhip_pwconv_amax(dy, S, C * L) would (same contract:
+ * sjhip_pwconv_amax_floats(S) floats, zero before the call): the fp16 GEMMs that consume dy (the two gradients of the convolution in front of the
  * batch norm, layer/attention.py:314-319 run backwards) then need no pass of their own over it. */
 int sjhip_bn_grad_input_amax(const float *g, const float *y, const float *coef, int64_t S, int64_t C, int64_t L, float *dy,
                              float *amax, void *stream);

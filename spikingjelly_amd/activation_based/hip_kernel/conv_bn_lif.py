@@ -40,7 +40,18 @@ MAX_REPLAY_STEPS = 16  # the backward replays the neuron with h of every step in
 
 
 F16 = 16  # term code of an fp16 operand: F16 | 2 (hi and lo of a scaled value) or F16 | 1 (exact in fp16)
-_AMAX_FLOATS = 256  # SJHIP_PW_AMAX_FLOATS
+_AMAX_FLOATS = 256  # SJHIP_PW_AMAX_FLOATS: the words of a tensor's largest magnitude
+_AMAX_SAMPLE_WORDS = 16  # SJHIP_PW_AMAX_SAMPLE_WORDS: then so many adjacent words per sample
+
+
+def amax_floats(samples: int) -> int:
+    """Length of the amax buffer of a tensor of ``samples`` samples (``sjhip_pwconv_amax_floats``)."""
+    return _AMAX_FLOATS + _AMAX_SAMPLE_WORDS * int(samples)
+
+
+def sample_amax(words: torch.Tensor) -> torch.Tensor:
+    """The largest magnitude of every sample, from the amax buffer of a tensor."""
+    return words[_AMAX_FLOATS:].view(-1, _AMAX_SAMPLE_WORDS).amax(dim=1)
 
 
 def _terms() -> int:
@@ -78,16 +89,17 @@ def _stream(t: torch.Tensor) -> int:
 def split_weight(weight: torch.Tensor, transpose: bool, terms: int = 3, amax_reset: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Term planes of ``weight [Cout, Cin]`` (or of its transpose), the A operand of ``pw_gemm``: bf16 planes
     ``[3, rows_pad, cols_pad]``, or with ``terms & F16`` two fp16 planes of the rows scaled by powers of two, followed by
-    the inverse scales (an opaque buffer either way).  ``amax_reset`` (fp16 terms): an ``amax`` buffer that the launch
-    clears on the way."""
+    the inverse scales (an opaque buffer either way).  ``amax_reset`` (fp16 terms): an ``amax`` buffer (of
+    ``amax_floats(S)`` words) that the launch clears on the way."""
     rows, cols = weight.shape
     w = L.aligned16(weight.detach().to(torch.float32))
     planes = torch.empty(L.load().sjhip_pwconv_planes_elems(cols if transpose else rows, rows if transpose else cols),
                          dtype=torch.bfloat16, device=weight.device)
     with torch.cuda.device(weight.device):
         if terms & F16:
+            reset_samples = (amax_reset.numel() - _AMAX_FLOATS) // _AMAX_SAMPLE_WORDS if amax_reset is not None else 0
             rc = L.load().sjhip_pwconv_split_weight_f16(w.data_ptr(), rows, cols, 1 if transpose else 0, planes.data_ptr(),
-                                                        L.ptr(amax_reset), _stream(w))
+                                                        L.ptr(amax_reset), reset_samples, _stream(w))
         else:
             rc = L.load().sjhip_pwconv_split_weight(w.data_ptr(), rows, cols, 1 if transpose else 0, planes.data_ptr(), _stream(w))
     L.check(rc, "pwconv_split_weight")
@@ -95,14 +107,20 @@ def split_weight(weight: torch.Tensor, transpose: bool, terms: int = 3, amax_res
 
 
 def amax(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The largest magnitude in ``x`` as the maximum of a small device buffer (several words, so that the blocks that
-    write them do not meet on one address): what the fp16 split of a tensor of arbitrary values is scaled by (the
-    kernels turn it into a power of two).  ``out``: a buffer that already holds zeros (or an earlier maximum to keep)."""
+    """The largest magnitudes in ``x [S, ...]`` as a small device buffer: the maximum of its first ``_AMAX_FLOATS`` words
+    is that of the whole tensor (several words, so that the blocks that write them do not meet on one address), and
+    ``sample_amax(words)[s]`` is that of sample ``s``: what the fp16 split of a tensor of arbitrary values is scaled by (the
+    kernels turn it into a power of two; per sample where a GEMM's columns are samples, per tensor where it sums over
+    them).  A tensor without a sample axis is one sample.  ``out``: a buffer of ``amax_floats(S)`` words that already holds
+    zeros (or earlier maxima to keep)."""
     x = L.aligned16(x)
+    S = x.shape[0] if x.dim() >= 2 else 1
     if out is None:
-        out = torch.zeros((_AMAX_FLOATS,), dtype=torch.float32, device=x.device)
+        out = torch.zeros((amax_floats(S),), dtype=torch.float32, device=x.device)
+    elif out.numel() != amax_floats(S):
+        raise ValueError(f"the amax buffer of {S} samples has {amax_floats(S)} words, got {out.numel()}")
     with torch.cuda.device(x.device):
-        rc = L.load().sjhip_pwconv_amax(x.data_ptr(), x.numel(), out.data_ptr(), _stream(x))
+        rc = L.load().sjhip_pwconv_amax(x.data_ptr(), S, x.numel() // S, out.data_ptr(), _stream(x))
     L.check(rc, "pwconv_amax")
     return out
 
@@ -316,7 +334,7 @@ def _bn_lif_backward(y: torch.Tensor, bn_map: torch.Tensor, gamma, v_init: torch
                                           g.data_ptr(), L.ptr(grad_v_init), partial.data_ptr(), stream), "bn_lif_backward")
         dy_amax = None
         if want_amax and _terms() & F16:  # (cleared by the launch that makes the coefficients, filled by the next one)
-            dy_amax = torch.empty((_AMAX_FLOATS,), dtype=torch.float32, device=y.device)
+            dy_amax = torch.empty((amax_floats(T * B),), dtype=torch.float32, device=y.device)
         L.check(lib.sjhip_bn_backward_finalize(partial.data_ptr(), T, B, C, Lp, 1 if batch_stats else 0, L.ptr(gamma),
                                                bn_map[2].data_ptr(), bn_map[3].data_ptr(), grads[0].data_ptr(),
                                                grads[1].data_ptr(), grads[2].data_ptr(), L.ptr(dy_amax), stream),
@@ -351,7 +369,7 @@ def _conv_forward(x_seq, weight, x_exact, stats: bool):
     terms = _terms()
     x3 = x_seq.reshape(T * B, Cin, Lp)
     if terms & F16 and not x_exact:  # the split of the weights clears the buffer that the pass over x then fills
-        x_amax = torch.empty((_AMAX_FLOATS,), dtype=torch.float32, device=x_seq.device)
+        x_amax = torch.empty((amax_floats(T * B),), dtype=torch.float32, device=x_seq.device)
         planes = split_weight(weight, False, terms, x_amax)
         amax(x3, x_amax)
     else:

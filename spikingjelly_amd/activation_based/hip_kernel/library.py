@@ -14,7 +14,7 @@ from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64
 
 import torch
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 # enums of include/sjhip.h
 NEURON_IF, NEURON_LIF, NEURON_PLIF, NEURON_QIF, NEURON_ILIF, NEURON_EIF = 0, 1, 2, 3, 4, 5
@@ -75,6 +75,7 @@ EXPORTED_SYMBOLS = (
     "sjhip_pwconv_grad_weight",
     "sjhip_pwconv_split_weight_f16",
     "sjhip_pwconv_amax",
+    "sjhip_pwconv_amax_floats",
     "sjhip_pwconv_gemm_f16",
     "sjhip_pwconv_grad_weight_f16",
     "sjhip_bn_grad_input_amax",
@@ -264,9 +265,11 @@ def load() -> ctypes.CDLL:
         lib.sjhip_pwconv_grad_weight.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64,
                                                  c_void_p, c_void_p, c_void_p]
         lib.sjhip_pwconv_split_weight_f16.restype = c_int
-        lib.sjhip_pwconv_split_weight_f16.argtypes = [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p]
+        lib.sjhip_pwconv_split_weight_f16.argtypes = [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_int64, c_void_p]
+        lib.sjhip_pwconv_amax_floats.restype = c_int64
+        lib.sjhip_pwconv_amax_floats.argtypes = [c_int64]
         lib.sjhip_pwconv_amax.restype = c_int
-        lib.sjhip_pwconv_amax.argtypes = [c_void_p, c_int64, c_void_p, c_void_p]
+        lib.sjhip_pwconv_amax.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p]
         lib.sjhip_pwconv_gemm_f16.restype = c_int
         lib.sjhip_pwconv_gemm_f16.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_int, c_void_p, c_int64, c_int64, c_void_p,
                                               c_void_p, c_void_p]

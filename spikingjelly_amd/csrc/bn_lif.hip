@@ -338,9 +338,9 @@ __global__ void __launch_bounds__(256) bn_lif_backward_rows_kernel(const BnLifBw
 __global__ void __launch_bounds__(256) bn_backward_finalize_kernel(const float *partial, int64_t B, int C, int64_t count,
                                                                     int training, const float *gamma, const float *mean,
                                                                     const float *invstd, float *dgamma, float *dbeta,
-                                                                    float *coef, float *amax_reset) {
-  static_assert(SJHIP_PW_AMAX_FLOATS == 256, "one word per work-item of the first block");
-  if (amax_reset && blockIdx.x == 0) amax_reset[threadIdx.x] = 0.0f;
+                                                                    float *coef, float *amax_reset, int64_t amax_floats) {
+  if (amax_reset && blockIdx.x == 0)
+    for (int64_t i = threadIdx.x; i < amax_floats; i += 256) amax_reset[i] = 0.0f;
   const int lane = threadIdx.x & 63;
   const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (c >= C) return;
@@ -373,14 +373,19 @@ __device__ __forceinline__ float finite_abs(float x) {
 // dy = p_c g + q_c y + r_c over the flattened [S * C * L] tensor; dy may be g itself.  With AMAX every block also folds
 // the largest |dy| it wrote into word (block % SJHIP_PW_AMAX_FLOATS) of amax_bits, bit patterns of non-negative floats
 // (they order like unsigned integers, and a maximum does not depend on the order it is taken in), with an atomic whose
-// result is not used, so that the block does not wait for it.
+// result is not used, so that the block does not wait for it; and every wavefront the largest |dy| of its sample into
+// that sample's word, which follow the tensor's (one atomic when its lanes share a sample, else one per lane).
 template <bool AMAX>
-__global__ void __launch_bounds__(256) bn_grad_input_kernel(const float *g, const float *y, const float *coef, int C, int L,
-                                                             int64_t n, float *dy, unsigned *amax_bits) {
+__global__ void __launch_bounds__(256) bn_grad_input_kernel(const float *g, const float *y, const float *coef, int64_t S, int C,
+                                                             int L, int64_t n, float *dy, unsigned *amax_bits) {
   const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   float amax = 0.0f;
+  int sample = -1;
   if (i < n) {
-    const int c = (int)((i / L) % C);
+    const int64_t row = i / L;  // sample * C + channel
+    const int64_t smp = row / C;
+    const int c = (int)(row - smp * C);
+    sample = (int)smp;
     const float p = coef[c], q = coef[C + c], r = coef[2 * C + c];
     const f32x4 gv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(g + i));
     const f32x4 yv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(y + i));
@@ -393,14 +398,39 @@ __global__ void __launch_bounds__(256) bn_grad_input_kernel(const float *g, cons
     if (AMAX) amax = fmaxf(fmaxf(finite_abs(o.x), finite_abs(o.y)), fmaxf(finite_abs(o.z), finite_abs(o.w)));
   }
   if (AMAX) {
+    // One atomic per block for the tensor's words and, when the block lies in one sample (nearly always: a sample is
+    // many blocks long), one for that sample's word.
     __shared__ float part[4];
+    __shared__ int part_sample[4];
+    // (blocks that run at the same time belong to one sample: they fold into different words of it)
+    unsigned *sample_bits = amax_bits + SJHIP_PW_AMAX_FLOATS + blockIdx.x % SJHIP_PW_AMAX_SAMPLE_WORDS;
+    constexpr int64_t kW = SJHIP_PW_AMAX_SAMPLE_WORDS;
+    const int first = __builtin_amdgcn_readfirstlane(sample);
+    const bool one_sample = __all(sample == first || sample < 0);
+    if (!one_sample && sample >= 0) atomicMax(sample_bits + kW * sample, __builtin_bit_cast(unsigned, amax));
 #pragma unroll
     for (int d = 32; d > 0; d >>= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = amax;
+    if ((threadIdx.x & 63) == 0) {
+      part[threadIdx.x >> 6] = amax;
+      part_sample[threadIdx.x >> 6] = one_sample ? first : -1;  // (-1: nothing left to fold for this wavefront)
+    }
     __syncthreads();
     if (threadIdx.x == 0) {
-      const unsigned bits = __builtin_bit_cast(unsigned, fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3])));
-      atomicMax(amax_bits + blockIdx.x % SJHIP_PW_AMAX_FLOATS, bits);
+      float all = 0.0f, run = 0.0f;
+      int run_sample = -1;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        all = fmaxf(all, part[w]);
+        if (part_sample[w] < 0) continue;
+        if (part_sample[w] != run_sample) {
+          if (run_sample >= 0) atomicMax(sample_bits + kW * run_sample, __builtin_bit_cast(unsigned, run));
+          run_sample = part_sample[w];
+          run = 0.0f;
+        }
+        run = fmaxf(run, part[w]);
+      }
+      if (run_sample >= 0) atomicMax(sample_bits + kW * run_sample, __builtin_bit_cast(unsigned, run));
+      atomicMax(amax_bits + blockIdx.x % SJHIP_PW_AMAX_FLOATS, __builtin_bit_cast(unsigned, all));
     }
   }
 }
@@ -510,8 +540,9 @@ int launch_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int6
                                 const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef,
                                 float *amax_reset, hipStream_t stream) {
   if (C < 1 || C > (1 << 24)) return fail(SJHIP_ERR_INVALID, "bn_backward_finalize: C=%lld", (long long)C);
+  // (the amax buffer of the dy that sjhip_bn_grad_input_amax writes next: the tensor's words and one per sample)
   hipLaunchKernelGGL(bn_backward_finalize_kernel, dim3((unsigned)((C + 3) / 4)), dim3(256), 0, stream, partial, B, (int)C,
-                     T * B * L, training, gamma, mean, invstd, dgamma, dbeta, coef, amax_reset);
+                     T * B * L, training, gamma, mean, invstd, dgamma, dbeta, coef, amax_reset, SJHIP_PW_AMAX_FLOATS + SJHIP_PW_AMAX_SAMPLE_WORDS * T * B);
   return check_launch("bn_backward_finalize");
 }
 
@@ -524,10 +555,10 @@ int launch_bn_grad_input(const float *g, const float *y, const float *coef, int6
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "bn_grad_input: %lld elements", (long long)n);
   ProfileScope prof(KC_BN_GRAD_INPUT, stream);
   if (amax)
-    hipLaunchKernelGGL(bn_grad_input_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, g, y, coef, (int)C, (int)L, n, dy,
+    hipLaunchKernelGGL(bn_grad_input_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, g, y, coef, S, (int)C, (int)L, n, dy,
                        reinterpret_cast<unsigned *>(amax));
   else
-    hipLaunchKernelGGL(bn_grad_input_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, g, y, coef, (int)C, (int)L, n, dy,
+    hipLaunchKernelGGL(bn_grad_input_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, g, y, coef, S, (int)C, (int)L, n, dy,
                        (unsigned *)nullptr);
   return check_launch("bn_grad_input");
 }

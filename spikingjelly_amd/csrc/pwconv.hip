@@ -186,9 +186,9 @@ __global__ void __launch_bounds__(256) split_weight_kernel(const float *src, int
 // rows_pad floats.  One wavefront per row.
 __global__ void __launch_bounds__(256) split_weight_f16_kernel(const float *src, int64_t rows, int64_t cols, int64_t ld_r,
                                                                 int64_t ld_c, int64_t rows_pad, int64_t cols_pad,
-                                                                uint16_t *planes, float *amax_reset) {
-  static_assert(SJHIP_PW_AMAX_FLOATS == 256, "one word per work-item of the first block");
-  if (amax_reset && blockIdx.x == 0) amax_reset[threadIdx.x] = 0.0f;
+                                                                uint16_t *planes, float *amax_reset, int64_t amax_floats) {
+  if (amax_reset && blockIdx.x == 0)
+    for (int64_t i = threadIdx.x; i < amax_floats; i += 256) amax_reset[i] = 0.0f;
   const int lane = threadIdx.x & 63;
   const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= rows_pad) return;
@@ -237,28 +237,76 @@ __device__ __forceinline__ float tensor_amax(const float *amax) {
   for (int d = 32; d > 0; d >>= 1) m = fmaxf(m, __shfl_xor(m, d));
   return m;
 }
-constexpr int kAmaxBlocks = 1024;
-__global__ void __launch_bounds__(256) amax_kernel(const float *x, int64_t n, unsigned *amax_bits) {
-  __shared__ float part[4];
-  float amax = 0.0f;
-  const int64_t stride = (int64_t)gridDim.x * 256;
-  const int64_t i0 = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
-    const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
-    const int64_t n4 = n / 4;
-    for (int64_t i = i0; i < n4; i += stride) {
-      const f32x4 v = __builtin_nontemporal_load(x4 + i);
-      amax = fmaxf(fmaxf(amax, fmaxf(finite_abs(v.x), finite_abs(v.y))), fmaxf(finite_abs(v.z), finite_abs(v.w)));
+// The words of every sample's own largest magnitude follow the SJHIP_PW_AMAX_FLOATS words of the tensor's
+// (SJHIP_PW_AMAX_SAMPLE_WORDS adjacent words per sample, whose maximum is the sample's amax: blocks that run at the
+// same time belong to one sample, and atomics on one address are served one after the other): the GEMMs whose
+// columns are (sample, position) pairs scale every sample by its own power of two (a sample whose values are all small
+// beside another's keeps its significant bits), the weight gradient, which sums over the samples, by the tensor's.
+__device__ __forceinline__ float sample_amax(const float *sample_words, int64_t s) {
+  static_assert(SJHIP_PW_AMAX_SAMPLE_WORDS == 16, "four 16-byte loads per sample");
+  const f32x4 *p = reinterpret_cast<const f32x4 *>(sample_words) + 4 * s;
+  const f32x4 a = p[0], b = p[1], c = p[2], d = p[3];
+  const f32x4 m = {fmaxf(fmaxf(a.x, b.x), fmaxf(c.x, d.x)), fmaxf(fmaxf(a.y, b.y), fmaxf(c.y, d.y)),
+                   fmaxf(fmaxf(a.z, b.z), fmaxf(c.z, d.z)), fmaxf(fmaxf(a.w, b.w), fmaxf(c.w, d.w))};
+  return fmaxf(fmaxf(m.x, m.y), fmaxf(m.z, m.w));
+}
+// x holds samples of per_sample elements each (a multiple of 4 when x is 16-byte aligned, so that a 16-byte access lies
+// in one sample); a block takes 4096 consecutive elements.  One atomic per block for the tensor's words and one for
+// a word of each of the (nearly always one, at most two) samples it lies in; what lies in further samples (samples
+// shorter than a block) the work-items fold themselves.
+constexpr int kAmaxChunk = 4096;
+__global__ void __launch_bounds__(256) amax_kernel(const float *x, int64_t S, int64_t per_sample, unsigned *amax_bits) {
+  const int64_t n = S * per_sample;
+  __shared__ float part[4], part_first[4], part_second[4];
+  unsigned *sample_bits = amax_bits + SJHIP_PW_AMAX_FLOATS + blockIdx.x % SJHIP_PW_AMAX_SAMPLE_WORDS;
+  constexpr int64_t kW = SJHIP_PW_AMAX_SAMPLE_WORDS;
+  const int64_t e0 = (int64_t)blockIdx.x * kAmaxChunk;
+  const int64_t s0 = e0 / per_sample;                // the block's first sample (the same for every work-item)
+  const int64_t next = (s0 + 1) * per_sample;        // first element of the following sample
+  float amax = 0.0f;                                 // over everything the work-item reads
+  float first = 0.0f, second = 0.0f;                 // over its elements of samples s0 and s0 + 1
+  auto take = [&](int64_t e, float m) {
+    amax = fmaxf(amax, m);
+    if (e < next) first = fmaxf(first, m);
+    else if (e < next + per_sample) second = fmaxf(second, m);
+    else atomicMax(sample_bits + kW * (e / per_sample), __builtin_bit_cast(unsigned, m));  // (samples shorter than a block)
+  };
+  if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0 && per_sample % 4 == 0) {
+    f32x4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int64_t e = e0 + (int64_t)(k * 256 + threadIdx.x) * 4;
+      v[k] = e + 4 <= n ? __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x + e)) : (f32x4)(0.0f);
     }
-    for (int64_t i = 4 * n4 + i0; i < n; i += stride) amax = fmaxf(amax, finite_abs(x[i]));
-  } else {
-    for (int64_t i = i0; i < n; i += stride) amax = fmaxf(amax, finite_abs(x[i]));
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int64_t e = e0 + (int64_t)(k * 256 + threadIdx.x) * 4;
+      if (e + 4 <= n) take(e, fmaxf(fmaxf(finite_abs(v[k].x), finite_abs(v[k].y)), fmaxf(finite_abs(v[k].z), finite_abs(v[k].w))));
+    }
+  } else {  // any alignment, any sample length: element by element
+    for (int k = 0; k < 16; ++k) {
+      const int64_t e = e0 + (int64_t)k * 256 + threadIdx.x;
+      if (e < n) take(e, finite_abs(x[e]));
+    }
   }
 #pragma unroll
-  for (int d = 32; d > 0; d >>= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
-  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = amax;
+  for (int d = 32; d > 0; d >>= 1) {
+    amax = fmaxf(amax, __shfl_xor(amax, d));
+    first = fmaxf(first, __shfl_xor(first, d));
+    second = fmaxf(second, __shfl_xor(second, d));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    part[threadIdx.x >> 6] = amax;
+    part_first[threadIdx.x >> 6] = first;
+    part_second[threadIdx.x >> 6] = second;
+  }
   __syncthreads();
-  if (threadIdx.x == 0) fold_amax(amax_bits, fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3])));
+  if (threadIdx.x == 0) {
+    fold_amax(amax_bits, fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3])));
+    if (e0 < n) atomicMax(sample_bits + kW * s0, __builtin_bit_cast(unsigned, fmaxf(fmaxf(part_first[0], part_first[1]), fmaxf(part_first[2], part_first[3]))));
+    if (next < n && next < e0 + kAmaxChunk)
+      atomicMax(sample_bits + kW * (s0 + 1), __builtin_bit_cast(unsigned, fmaxf(fmaxf(part_second[0], part_second[1]), fmaxf(part_second[2], part_second[3]))));
+  }
 }
 
 struct PwGemmArgs {
@@ -273,6 +321,8 @@ struct PwGemmArgs {
                              // each half (64 columns) of every column block
   const float *a_inverse;    // fp16 terms: the inverse scale of every (padded) row of A
   const float *b_amax;       // fp16 terms: nullptr (b needs no scale), or the words whose maximum is max |b|
+  const float *b_amax_samples;  // kBFloat with two fp16 terms: the per-sample words of b's amax buffer (they follow b_amax's words)
+  int64_t amax_s0, amax_S;      // the first sample of this launch, the samples of the tensor
   const uint16_t *b_planes;  // kBPlanes: fp16 terms of b, [TB][K][ld], column s * L + l of row k holds b[s][k][l]
   int64_t b_plane_stride;    // K * ld
   int ld;                    // columns per row of a plane: a multiple of 8, at least ncols
@@ -367,8 +417,25 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   const bool edge_cols = __builtin_amdgcn_readfirstlane(j0 + kTile > a.ncols ? 1 : 0) != 0;
   const char *a_base = reinterpret_cast<const char *>(a.a_planes);
   const char *b_base = reinterpret_cast<const char *>(a.b);
+  // The scale of b: a sample's own power of two when b is split here (a work-item stages columns of one sample), the
+  // tensor's when b arrives as planes (split with it).
+  constexpr bool SAMPLE_SCALE = H && TB > 1 && BSRC == kBFloat;
   float b_scale = 1.0f, b_inverse = 1.0f;
-  if (H && TB > 1 && a.b_amax != nullptr) scale_for(tensor_amax(a.b_amax), b_scale, b_inverse);
+  if (H && TB > 1 && !SAMPLE_SCALE && a.b_amax != nullptr) scale_for(tensor_amax(a.b_amax), b_scale, b_inverse);
+  // A tile of 128 columns lies in at most two samples when a sample has that many positions: their two maxima are
+  // fetched once per block from addresses that do not depend on the lane; shorter samples are looked up per column.
+  const bool two_samples = L >= kTile;
+  const int64_t tile_sample = j0 / L, next_sample_col = (tile_sample + 1) * L;
+  float tile_amax[2] = {0.0f, 0.0f};
+  if (SAMPLE_SCALE && a.b_amax_samples != nullptr && two_samples) {
+    const int64_t s_a = a.amax_s0 + tile_sample, s_b = s_a + 1 < a.amax_S ? s_a + 1 : s_a;
+    tile_amax[0] = sample_amax(a.b_amax_samples, s_a);
+    tile_amax[1] = sample_amax(a.b_amax_samples, s_b);
+  }
+  auto column_amax = [&](int64_t j) {
+    return two_samples ? (j < next_sample_col ? tile_amax[0] : tile_amax[1]) : sample_amax(a.b_amax_samples, a.amax_s0 + j / L);
+  };
+  if (SAMPLE_SCALE && a.b_amax_samples != nullptr && col_ok) scale_for(column_amax(jc), b_scale, b_inverse);
   // planes: 16-byte chunk pc (eight columns) of the k rows pr and pr + 16 of every plane
   const int pc = tid & 15, pr = tid >> 4;
   const uint32_t ld2 = PLANES ? (uint32_t)a.ld * 2u : 0u;
@@ -535,6 +602,16 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   if (k0 + 2 * kTileK < K_pad) step(k0 + 2 * kTileK, 0, false, false);
 
   // accumulator register r of a 32 x 32 tile: row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
+  float b_inv_col[2] = {b_inverse, b_inverse};  // of the two columns whose results this lane holds
+  if (SAMPLE_SCALE && a.b_amax_samples != nullptr) {
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int64_t j = j0 + wn * 64 + nt * 32 + (lane & 31);
+      float unused;
+      b_inv_col[nt] = 1.0f;
+      if (j < a.ncols) scale_for(column_amax(j), unused, b_inv_col[nt]);
+    }
+  }
   if (H) {  // take the power-of-two scales of the row of A and of b out again: exact
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
@@ -542,7 +619,7 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       for (int r = 0; r < 16; ++r) {
         const float inv = a.a_inverse[m0 + wm * 64 + mt * 32 + 4 * (lane >> 5) + 8 * (r >> 2) + (r & 3)];
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) acc[mt][nt][r] = acc[mt][nt][r] * inv * b_inverse;
+        for (int nt = 0; nt < 2; ++nt) acc[mt][nt][r] = acc[mt][nt][r] * inv * b_inv_col[nt];
       }
   }
 #pragma unroll
@@ -1099,20 +1176,20 @@ int launch_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int t
 }
 
 int launch_pwconv_split_weight_f16(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes,
-                                   float *amax_reset, hipStream_t stream) {
+                                   float *amax_reset, int64_t amax_floats, hipStream_t stream) {
   const int64_t ar = transpose ? cols : rows, ac = transpose ? rows : cols;
   const int64_t rows_pad = round_up(ar, kTile), cols_pad = round_up(ac, kTileK);
   const int64_t blocks = rows_pad / 4;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_split_weight_f16: %lld x %lld", (long long)rows, (long long)cols);
   hipLaunchKernelGGL(split_weight_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, w, ar, ac,
-                     transpose ? (int64_t)1 : cols, transpose ? cols : (int64_t)1, rows_pad, cols_pad, planes, amax_reset);
+                     transpose ? (int64_t)1 : cols, transpose ? cols : (int64_t)1, rows_pad, cols_pad, planes, amax_reset, amax_floats);
   return check_launch("pwconv_split_weight_f16");
 }
 
-int launch_pwconv_amax(const float *x, int64_t n, float *amax, hipStream_t stream) {
-  int64_t blocks = (n / 4 + 255) / 256;
-  blocks = blocks < 1 ? 1 : (blocks > kAmaxBlocks ? kAmaxBlocks : blocks);
-  hipLaunchKernelGGL(amax_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, n, reinterpret_cast<unsigned *>(amax));
+int launch_pwconv_amax(const float *x, int64_t S, int64_t per_sample, float *amax, hipStream_t stream) {
+  const int64_t n = S * per_sample, blocks = (n + kAmaxChunk - 1) / kAmaxChunk;
+  if (S > 0x7fffffffLL || blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_amax: %lld samples of %lld elements", (long long)S, (long long)per_sample);
+  hipLaunchKernelGGL(amax_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, S, per_sample, reinterpret_cast<unsigned *>(amax));
   return check_launch("pwconv_amax");
 }
 
@@ -1156,6 +1233,8 @@ int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t
     a.stats = stats;
     a.a_inverse = reinterpret_cast<const float *>(a_planes + 2 * a.plane_stride);
     a.b_amax = b_amax;
+    a.b_amax_samples = b_amax ? b_amax + SJHIP_PW_AMAX_FLOATS : nullptr;
+    a.amax_s0 = s0; a.amax_S = S;
     a.b_planes = nullptr; a.b_plane_stride = 0; a.ld = 0;
     if (stats) stats += 2 * ((a.ncols + kTile - 1) / kTile) * M * 2;
     const int64_t blocks = a.m_blocks * ((a.ncols + kTile - 1) / kTile);
@@ -1284,6 +1363,7 @@ int launch_pwconv_gemm_planes(const uint16_t *a_planes, int64_t M, int64_t K, co
   a.stats = stats;
   a.a_inverse = reinterpret_cast<const float *>(a_planes + 2 * a.plane_stride);
   a.b_amax = b_terms == 2 ? b_amax : nullptr;
+  a.b_amax_samples = nullptr; a.amax_s0 = 0; a.amax_S = 0;
   a.b_planes = b_planes; a.b_plane_stride = K * ld; a.ld = (int)ld;
   const int64_t blocks = a.m_blocks * ((a.ncols + kTile - 1) / kTile);
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm_planes: %lld blocks", (long long)blocks);

@@ -603,18 +603,23 @@ int sjhip_pwconv_grad_weight(const float *dy, int dy_terms, const float *x, int 
   return launch_pwconv_grad_weight(dy, dy_terms, nullptr, x, x_terms, nullptr, S, M, N, L, dw, workspace, static_cast<hipStream_t>(stream));
 }
 
+int64_t sjhip_pwconv_amax_floats(int64_t S) { return S < 0 ? 0 : SJHIP_PW_AMAX_FLOATS + SJHIP_PW_AMAX_SAMPLE_WORDS * S; }
+
 int sjhip_pwconv_split_weight_f16(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, float *amax_reset,
-                                  void *stream) {
+                                  int64_t amax_reset_samples, void *stream) {
   if (!w || !planes) return fail(SJHIP_ERR_INVALID, "pwconv_split_weight_f16: NULL buffer");
   if (rows < 1 || cols < 1) return fail(SJHIP_ERR_INVALID, "pwconv_split_weight_f16: %lld x %lld", (long long)rows, (long long)cols);
   if (!aligned16(planes)) return fail(SJHIP_ERR_UNSUPPORTED, "pwconv_split_weight_f16: the planes must be 16-byte aligned");
-  return launch_pwconv_split_weight_f16(w, rows, cols, transpose, planes, amax_reset, static_cast<hipStream_t>(stream));
+  if (amax_reset && amax_reset_samples < 0) return fail(SJHIP_ERR_INVALID, "pwconv_split_weight_f16: amax_reset_samples=%lld", (long long)amax_reset_samples);
+  return launch_pwconv_split_weight_f16(w, rows, cols, transpose, planes, amax_reset, SJHIP_PW_AMAX_FLOATS + SJHIP_PW_AMAX_SAMPLE_WORDS * amax_reset_samples,
+                                        static_cast<hipStream_t>(stream));
 }
 
-int sjhip_pwconv_amax(const float *x, int64_t n, float *amax, void *stream) {
+int sjhip_pwconv_amax(const float *x, int64_t S, int64_t per_sample, float *amax, void *stream) {
   if (!x || !amax) return fail(SJHIP_ERR_INVALID, "pwconv_amax: NULL buffer");
-  if (n < 1) return fail(SJHIP_ERR_INVALID, "pwconv_amax: n=%lld", (long long)n);
-  return launch_pwconv_amax(x, n, amax, static_cast<hipStream_t>(stream));
+  if (S < 1 || per_sample < 1 || S > (int64_t(1) << 40) / per_sample)
+    return fail(SJHIP_ERR_INVALID, "pwconv_amax: S=%lld samples of per_sample=%lld elements", (long long)S, (long long)per_sample);
+  return launch_pwconv_amax(x, S, per_sample, amax, static_cast<hipStream_t>(stream));
 }
 
 int sjhip_pwconv_gemm_f16(const uint16_t *a_planes, int64_t M, int64_t K, const float *b, int b_terms, const float *b_amax,

@@ -448,8 +448,8 @@ int launch_stream_probe(int reads, int writes, int nontemporal, int64_t floats_p
 int64_t pwconv_planes_elems(int64_t rows, int64_t cols);
 int launch_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, hipStream_t stream);
 int launch_pwconv_split_weight_f16(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, float *amax_reset,
-                                   hipStream_t stream);
-int launch_pwconv_amax(const float *x, int64_t n, float *amax, hipStream_t stream);
+                                   int64_t amax_floats, hipStream_t stream);
+int launch_pwconv_amax(const float *x, int64_t S, int64_t per_sample, float *amax, hipStream_t stream);
 int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t K, const float *b, int b_terms,
                        const float *b_amax, int64_t S, int64_t L, float *c, float *stats, hipStream_t stream, bool b_bits = false);
 int64_t pwconv_gemm_stats_rows(int64_t K, int64_t S, int64_t L);

@@ -244,7 +244,8 @@ def test_fp16_split_convolution_arguments_without_a_device():
     assert rc == -2 and b"16-byte aligned" in lib.sjhip_last_error()
     rc = lib.sjhip_pwconv_grad_weight_f16_bits(16, 20, 16, 1, 8, 8, 4, 16, 16, None)
     assert rc == -2 and b"16-byte aligned" in lib.sjhip_last_error()
-    rc = lib.sjhip_pwconv_amax(16, 0, 16, None)
-    assert rc == -1 and b"n=0" in lib.sjhip_last_error()
-    rc = lib.sjhip_pwconv_split_weight_f16(16, 8, 8, 0, 8, None, None)
+    rc = lib.sjhip_pwconv_amax(16, 0, 4, 16, None)
+    assert rc == -1 and b"S=0" in lib.sjhip_last_error()
+    assert lib.sjhip_pwconv_amax_floats(10) == 256 + 16 * 10
+    rc = lib.sjhip_pwconv_split_weight_f16(16, 8, 8, 0, 8, None, 0, None)
     assert rc == -2 and b"aligned" in lib.sjhip_last_error()

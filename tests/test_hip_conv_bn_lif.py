@@ -159,6 +159,70 @@ def test_gemm_with_two_fp16_terms_has_fp32_accuracy(C, S, M, Kd, Lp, transpose, 
     assert float(((got2 - want).abs() / bound).max()) < 2e-6
 
 
+def _column_errors(got, w, x):
+    """Per output element: |got - float64| over the sum of |a||b| of its dot product."""
+    want = torch.einsum("mk,skl->sml", w.double(), x.double())
+    bound = torch.einsum("mk,skl->sml", w.double().abs(), x.double().abs()).clamp_min(1e-300)
+    return (got.cpu().double() - want).abs() / bound
+
+
+@pytest.mark.parametrize("S,M,Kd,Lp", [(24, 130, 96, 36), (16, 384, 384, 196)])
+@pytest.mark.parametrize("what", ["samples", "outlier"])
+def test_fp16_gemm_keeps_fp32_accuracy_over_a_wide_dynamic_range(C, S, M, Kd, Lp, what):
+    """Activations (or gradients) whose samples are spread over eight decades (a batch in which some samples have
+    converged), and a tensor with one element a million times the rest: every output column stays within 2e-6 of its
+    own sum of |a||b|, because every sample is scaled by its own largest magnitude (with one scale per tensor a sample
+    six decades below the largest would keep 2^-19 of relative accuracy, an eight-decade one 2^-12)."""
+    F = C.F16 | 2
+    w = seeded_randn((M, Kd), 93, 0.0, 0.05)
+    x = seeded_randn((S, Kd, Lp), 94, 0.0, 1.0)
+    if what == "samples":
+        x = x * 10.0 ** torch.linspace(-8.0, 0.0, S)[:, None, None]
+    else:
+        x[S // 3, Kd // 2, Lp // 2] = 1e6
+    planes = C.split_weight(w.cuda(), False, F)
+    rel = _column_errors(C.pw_gemm(planes, F, M, Kd, x.cuda(), F), w, x)
+    assert float(rel.max()) < 2e-6, float(rel.max())
+    # the weight gradient sums over the samples: the tensor's scale, and what small samples add is small beside the rest
+    # (holds when the samples that are small in one operand are not the only large ones in the other: gradients that
+    # fade with the samples they belong to, against activations of any spread)
+    dy = seeded_randn((S, M, Lp), 95, 0.0, 1.0)
+    if what == "samples":
+        dy = dy * 10.0 ** torch.linspace(-8.0, 0.0, S)[:, None, None]
+    for xs in (x, seeded_randn((S, Kd, Lp), 98, 0.0, 1.0)):
+        got = C.pw_grad_weight(dy.cuda(), F, xs.cuda(), F).cpu().double()
+        want = torch.einsum("sml,snl->mn", dy.double(), xs.double())
+        bound = torch.einsum("sml,snl->mn", dy.double().abs(), xs.double().abs())
+        assert float(((got - want).abs() / bound).max()) < 2e-6
+    # and the gradient with respect to the input, whose columns are samples again
+    planes_t = C.split_weight(w.cuda(), True, F)
+    rel = _column_errors(C.pw_gemm(planes_t, F, Kd, M, dy.cuda(), F), w.t(), dy)
+    assert float(rel.max()) < 2e-6, float(rel.max())
+
+
+@pytest.mark.parametrize("split", ["bf16", "f16"])
+def test_gemm_with_token_columns_spread_over_eight_decades(C, split):
+    """Positions of one sample spread over eight decades: the three-term bf16 split (fp32's exponent range) keeps every
+    column within the fp32 bound; the fp16 split, whose scale is per sample, keeps the bound for columns above 2^-17 of
+    their sample's largest magnitude and an absolute floor of 2^-38 of that magnitude times sum |a| below."""
+    S, M, Kd, Lp = 4, 130, 96, 64
+    F = C.F16 | 2 if split == "f16" else 3
+    w = seeded_randn((M, Kd), 96, 0.0, 0.05)
+    x = seeded_randn((S, Kd, Lp), 97, 0.0, 1.0) * 10.0 ** torch.linspace(-8.0, 0.0, Lp)[None, None, :]
+    planes = C.split_weight(w.cuda(), False, F)
+    got = C.pw_gemm(planes, F, M, Kd, x.cuda(), F).cpu().double()
+    want = torch.einsum("mk,skl->sml", w.double(), x.double())
+    bound = torch.einsum("mk,skl->sml", w.double().abs(), x.double().abs())
+    err = (got - want).abs()
+    if split == "bf16":
+        assert float((err / bound).max()) < 2e-6
+    else:
+        floor = 2.0 ** -38 * x.double().abs().amax(dim=(1, 2))[:, None, None] * w.double().abs().sum(dim=1)[None, :, None]
+        assert bool((err <= 2e-6 * bound + floor).all())
+        large = (x.abs().amax(dim=1, keepdim=True) >= 2.0 ** -16 * x.abs().amax(dim=(1, 2), keepdim=True)).expand(S, M, Lp)
+        assert float((err / bound)[large].max()) < 2e-6
+
+
 @pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (4, 384, 384, 196)])
 def test_fp16_gemm_is_exact_on_spikes_times_dyadic_weights(C, S, M, Kd, Lp):
     g = torch.Generator().manual_seed(13)
@@ -215,8 +279,8 @@ def test_fp16_gemms_read_bit_packed_spikes(C, S, M, Kd, Lp):
 
 
 def test_amax(C):
-    """``amax(x)`` is the largest magnitude among the numbers of ``x``, for any length and alignment, and folds into what
-    the word already holds."""
+    """``amax(x)``: the maximum of the first 256 words is the largest magnitude among the numbers of ``x``, for any length
+    and alignment, ``sample_amax`` of the words that of every sample, and both fold into what the words already hold."""
     from spikingjelly_amd.activation_based.hip_kernel import library as L
 
     for n, top in ((1, 1.0), (7, 3.0), (1000, 0.75), (4099, 1e-30), (1 << 20, 262016.0), (5, 0.0), (3 * (1 << 20) + 5, 17.5)):
@@ -225,16 +289,38 @@ def test_amax(C):
             x.zero_()
         x[n // 2 + 1] = -top
         top = abs(float(x[n // 2 + 1]))   # as fp32 holds it
-        assert float(C.amax(x.cuda()[1:]).max()) == top, (n, top)
-        words = torch.zeros(256, device="cuda")   # the C entry point on an address 4 bytes past an aligned one
+        got = C.amax(x.cuda()[1:])        # one sample
+        assert got.numel() == C.amax_floats(1) and float(got[:256].max()) == top == float(C.sample_amax(got)), (n, top)
+        words = torch.zeros(C.amax_floats(1), device="cuda")   # the C entry point on an address 4 bytes past an aligned one
         xs = x.cuda()[1:]
-        L.check(L.load().sjhip_pwconv_amax(xs.data_ptr(), n, words.data_ptr(), L.current_stream_ptr(xs.device)), "amax")
+        L.check(L.load().sjhip_pwconv_amax(xs.data_ptr(), 1, n, words.data_ptr(), L.current_stream_ptr(xs.device)), "amax")
         assert float(words.max()) == top and float(words.min()) >= 0.0
         words[3] = 1e30
-        L.check(L.load().sjhip_pwconv_amax(xs.data_ptr(), n, words.data_ptr(), L.current_stream_ptr(xs.device)), "amax")
-        assert float(words.max()) == max(top, float(torch.tensor(1e30)))
+        L.check(L.load().sjhip_pwconv_amax(xs.data_ptr(), 1, n, words.data_ptr(), L.current_stream_ptr(xs.device)), "amax")
+        assert float(words[:256].max()) == max(top, float(torch.tensor(1e30))) and float(C.sample_amax(words)) == top
     odd = torch.tensor([1.0, float("nan"), -2.0, 0.5, float("-inf"), float("inf")]).cuda()
     assert float(C.amax(odd).max()) == 2.0   # the largest magnitude among the finite elements
+
+
+@pytest.mark.parametrize("S,per_sample,offset", [(5, 12, 0), (3, 75264, 0), (300, 40, 0), (7, 4100, 0), (6, 10, 1), (4, 5000, 1),
+                                                 (70000, 4, 0)])
+def test_amax_per_sample(C, S, per_sample, offset):
+    """Samples shorter and longer than the 4096 elements a block takes, sample lengths that are no multiple of 4 and a
+    tensor that starts 4 bytes past an aligned address: every sample's word holds that sample's largest magnitude."""
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+
+    x = seeded_randn((S * per_sample + offset,), 91, 0.0, 1.0)
+    x = (x[offset:].view(S, per_sample) * (10.0 ** (seeded_randn((S, 1), 92, 0.0, 3.0)))).contiguous()
+    x[S // 2] = 0.0
+    flat = torch.empty(S * per_sample + offset, device="cuda")
+    flat[offset:] = x.flatten().cuda()
+    xd = flat[offset:].view(S, per_sample)
+    words = torch.zeros(C.amax_floats(S), device="cuda")
+    L.check(L.load().sjhip_pwconv_amax(xd.data_ptr(), S, per_sample, words.data_ptr(), L.current_stream_ptr(xd.device)), "amax")
+    assert torch.equal(C.sample_amax(words).cpu(), x.abs().amax(dim=1))
+    assert float(words[:256].max()) == float(x.abs().max())
+    if offset == 0:
+        assert torch.equal(C.sample_amax(C.amax(xd)), C.sample_amax(words))
 
 
 @pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (1, 7, 3, 4), (4, 130, 257, 36), (16, 1152, 384, 196)])
@@ -371,13 +457,15 @@ def test_bn_grad_input_leaves_the_largest_magnitude_of_its_output(C, S, Cc, Lp):
     y = seeded_randn((S, Cc, Lp), 52, 0.3, 2.0).cuda()
     coef = seeded_randn((3, Cc), 53, 0.0, 1.0).cuda()
     plain, fused = torch.empty_like(g), torch.empty_like(g)
-    word = torch.zeros((256,), dtype=torch.float32, device="cuda")
+    word = torch.zeros((C.amax_floats(S),), dtype=torch.float32, device="cuda")
     stream = L.current_stream_ptr(g.device)
     L.check(lib.sjhip_bn_grad_input(g.data_ptr(), y.data_ptr(), coef.data_ptr(), S, Cc, Lp, plain.data_ptr(), stream), "plain")
     L.check(lib.sjhip_bn_grad_input_amax(g.data_ptr(), y.data_ptr(), coef.data_ptr(), S, Cc, Lp, fused.data_ptr(),
                                          word.data_ptr(), stream), "fused")
     assert torch.equal(plain, fused)
-    assert float(word.max()) == float(plain.abs().max()) == float(C.amax(plain).max())
+    assert float(word[:256].max()) == float(plain.abs().max())
+    assert torch.equal(C.sample_amax(word), plain.abs().amax(dim=(1, 2)))   # every sample's own largest magnitude
+    assert torch.equal(C.sample_amax(C.amax(plain)), C.sample_amax(word))
 
 
 def test_launches_that_clear_an_amax_buffer_and_count_the_batch(C):
@@ -387,9 +475,10 @@ def test_launches_that_clear_an_amax_buffer_and_count_the_batch(C):
     from spikingjelly_amd.activation_based.hip_kernel import library as L
     from spikingjelly_amd.activation_based.hip_kernel import neuron_kernel as K
 
-    buf = torch.full((256,), 1e30, device="cuda")
-    C.split_weight(seeded_randn((40, 24), 61, 0.0, 1.0).cuda(), False, C.F16 | 2, buf)
-    assert not buf.any()
+    for samples in (0, 5, 1000):
+        buf = torch.full((C.amax_floats(samples),), 1e30, device="cuda")
+        C.split_weight(seeded_randn((40, 24), 61, 0.0, 1.0).cuda(), False, C.F16 | 2, buf)
+        assert not buf.any()
     T, B, Cc, Lp = 4, 3, 10, 12
     y = seeded_randn((T, B, Cc, Lp), 62, 0.4, 1.5).cuda()
     gamma, beta = seeded_randn((Cc,), 63, 1.0, 0.2).cuda(), seeded_randn((Cc,), 64, 0.6, 0.3).cuda()
@@ -400,10 +489,11 @@ def test_launches_that_clear_an_amax_buffer_and_count_the_batch(C):
     v0 = torch.zeros((1,), device="cuda").expand(B, Cc, Lp)
     gs = seeded_randn((T, B, Cc, Lp), 65).cuda()
     for _ in range(3):   # the buffer comes from torch.empty: whatever it held before must not survive
-        poison = torch.full((256,), 1e30, device="cuda")
+        poison = torch.full((C.amax_floats(T * B),), 1e30, device="cuda")
         del poison
         dy, _, _, _, dy_amax = C._bn_lif_backward(y, bn_map, gamma, v0, spec, True, gs, None, False, True)
-        assert float(dy_amax.max()) == float(dy.abs().max())
+        assert float(dy_amax[:256].max()) == float(dy.abs().max())
+        assert torch.equal(C.sample_amax(dy_amax), dy.abs().amax(dim=(2, 3)).flatten())
     plain = C._bn_lif_backward(y, bn_map, gamma, v0, spec, True, gs, None, False)[0]
     assert torch.equal(plain, dy)
 
