@@ -18,7 +18,9 @@ from . import library as L
 __all__ = ["hip_ssa_forward", "hip_ssa_backward", "ssa_supported"]
 
 
+@torch.compiler.assume_constant_result
 def ssa_supported(dtype: torch.dtype, channels_per_head: int, tokens: int) -> bool:
+    """(asks the library; a constant of any traced graph, like the shapes it is asked about)"""
     try:
         did = L.dtype_id(dtype)
     except NotImplementedError:
@@ -176,18 +178,25 @@ class _LifSsa(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_out, grad_v_last, grad_bits):
-        from . import neuron_kernel as K
-
         del grad_bits
-        tau, v_th, v_reset, flags, sg_id, sg_alpha, samples, heads, cph, tokens, scale = ctx.spec
         x_seq, v_init, bits = ctx.saved_tensors
-        grad_spikes = None
-        if grad_out is not None:
-            grad_spikes = _ssa_packed(bits, grad_out, x_seq.dtype, samples, heads, cph, tokens, scale).view(x_seq.shape)
         need = bool(ctx.needs_input_grad[1])
-        gx, gvi, _ = K._run_backward(L.NEURON_LIF, grad_spikes, None, grad_v_last, None, x_seq, v_init, None, tau, v_th,
-                                     v_reset, flags, sg_id, sg_alpha, need)
+        gx, gvi = _lif_ssa_backward(x_seq, v_init, bits, ctx.spec, grad_out, grad_v_last, need)
         return gx, (gvi if need else None), None
+
+
+def _lif_ssa_backward(x_seq, v_init, bits, spec, grad_out, grad_v_last, need_gvi: bool):
+    """``(grad_x_seq, grad_v_init or None)`` of ``_LifSsa``: the contraction writes the dense spike gradient from the
+    bits, the LIF backward replays its forward from ``x_seq``."""
+    from . import neuron_kernel as K
+
+    tau, v_th, v_reset, flags, sg_id, sg_alpha, samples, heads, cph, tokens, scale = spec
+    grad_spikes = None
+    if grad_out is not None:
+        grad_spikes = _ssa_packed(bits, grad_out, x_seq.dtype, samples, heads, cph, tokens, scale).view(x_seq.shape)
+    gx, gvi, _ = K._run_backward(L.NEURON_LIF, grad_spikes, None, grad_v_last, None, x_seq, v_init, None, tau, v_th,
+                                 v_reset, flags, sg_id, sg_alpha, need_gvi)
+    return gx, (gvi if need_gvi else None)
 
 
 def lif_ssa_fused(x_seq: torch.Tensor, v_init: torch.Tensor, tau: float, v_th: float, v_reset: float, flags: int,
@@ -198,5 +207,9 @@ def lif_ssa_fused(x_seq: torch.Tensor, v_init: torch.Tensor, tau: float, v_th: f
     ``N % 8 == 0`` and that the replay backward serves the shape."""
     samples = x_seq.shape[0] * (x_seq.shape[1] // (3 * heads * channels_per_head * tokens))
     spec = (tau, v_th, v_reset, flags, sg_id, sg_alpha, samples, heads, channels_per_head, tokens, scale)
+    if torch.compiler.is_compiling():  # the same launches as torch.library operators (schema, fake kernels)
+        from . import fused_ops as O
+
+        return O.lif_ssa(x_seq, v_init, spec)
     out, v_last, _ = _LifSsa.apply(x_seq, v_init, spec)
     return out, v_last

@@ -14,6 +14,11 @@ tensors (``L`` the flattened positions, a multiple of 4):
   then normalise + charge + fire + reset over the T steps in registers, spikes written dense or bit-packed; the
   normalised tensor never exists.  The backward replays the neuron from the convolution output.
 
+Ordinary eager calls go through ``autograd.Function`` s; under a tracing compiler (``torch.compile``) the same launch
+helpers run as ``torch.library`` operators with fake kernels and registered backward formulas (``fused_ops.py``), so a
+compiled module keeps the fused chain (reference: the kernel backends are compile-transparent custom operators,
+``cuda_kernel/neuron_kernel/multi_step/lif.py:144-225``, ``test/activation_based/test_compile_compat.py:125-170``).
+
 Three entries share the pieces: ``bn_lif`` (any convolution output, e.g. a 3x3 ``Conv2d`` run by torch),
 ``conv_bn_lif`` (the whole block) and ``conv_bn_lif_ssa`` (the block feeding the spiking self-attention contraction
 through bit-packed spikes).  All are ``autograd.Function`` s around plain launch helpers; nothing here falls back to
@@ -427,6 +432,49 @@ def _side_stream(device: torch.device) -> "torch.cuda.Stream":
     return stream
 
 
+def _conv_chain_backward(x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax, spec, batch_stats: bool, x_exact: bool, ssa,
+                         grad_out, grad_v_last, need_dx: bool, need_dw: bool, need_gvi: bool):
+    """Backward of convolution -> batch norm -> LIF (-> contraction on the bit-packed spikes when ``ssa = (heads,
+    channels per head, scale)``): ``(dx, dw, dgamma, dbeta, grad_v_init)``, ``None`` where not needed."""
+    grad_spikes = grad_out
+    if ssa is not None and grad_out is not None:
+        from . import attention_kernel as A
+
+        heads, cph, scale = ssa
+        T, B, _, Lp = x_seq.shape
+        grad_spikes = A._ssa_packed(bits, grad_out, torch.float32, T * B, heads, cph, Lp, scale).view(y.shape)
+    dy, dgamma, dbeta, gvi, dy_amax = _bn_lif_backward(y, bn_map, gamma, v_init, spec, batch_stats, grad_spikes, grad_v_last,
+                                                        need_gvi, True)
+    dx, dw = _conv_backward(dy, x_seq, weight, x_exact, need_dx, need_dw, dy_amax, x_amax)
+    return dx, dw, dgamma, dbeta, gvi
+
+
+def _lif_conv_chain_backward(pre_seq, pre_v_init, weight, gamma, v_init, y, bn_map, bits, pre_spec, spec, batch_stats: bool,
+                             grad_spikes, grad_v_last, grad_pre_v_last, need_gx: bool, need_gpv: bool, need_dw: bool,
+                             need_gvi: bool):
+    """Backward of LIF -> convolution -> batch norm -> LIF with the first neuron's spikes as bits:
+    ``(grad of the first neuron's input, of its state, dw, dgamma, dbeta, grad_v_init)``."""
+    T, B, Cin, Lp = pre_seq.shape
+    Cout = weight.shape[0]
+    terms = _terms()
+    dy, dgamma, dbeta, gvi, dy_amax = _bn_lif_backward(y, bn_map, gamma, v_init, spec, batch_stats, grad_spikes, grad_v_last,
+                                                        need_gvi, True)
+    dy3 = dy.view(T * B, Cout, Lp)
+    if dy_amax is None:
+        dy_amax = amax(dy3)
+    dw = pw_grad_weight_bits(dy3, bits, Cin, dy_amax) if need_dw else None
+    gx = gpv = None
+    if need_gx or need_gpv:
+        grad_pre_spikes = pw_gemm(split_weight(weight, True, terms), terms, Cin, Cout, dy3, terms, False, dy_amax)
+        tau, v_th, v_reset, flags, sg_id, sg_alpha = pre_spec
+        glast = grad_pre_v_last.flatten() if grad_pre_v_last is not None else None
+        gx, gpv, _ = K._run_backward(L.NEURON_LIF, grad_pre_spikes.view(T, -1), None, glast, None, pre_seq.view(T, -1),
+                                     pre_v_init.flatten(), None, tau, v_th, v_reset, flags, sg_id, sg_alpha, need_gpv)
+        gx = gx.view(pre_seq.shape) if need_gx else None
+        gpv = gpv.view(B, Cin, Lp) if need_gpv else None
+    return gx, gpv, dw, dgamma, dbeta, gvi
+
+
 class _BnLif(torch.autograd.Function):
     @staticmethod
     def forward(y, gamma, beta, v_init, bn, spec):
@@ -475,9 +523,9 @@ class _ConvBnLif(torch.autograd.Function):
     def backward(ctx, grad_spikes, grad_v_last, _y, _map, _amax):
         x_seq, weight, gamma, v_init, y, bn_map, x_amax = ctx.saved_tensors
         need = ctx.needs_input_grad
-        dy, dgamma, dbeta, gvi, dy_amax = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
-                                                            grad_v_last, bool(need[4]), True)
-        dx, dw = _conv_backward(dy, x_seq, weight, ctx.x_exact, bool(need[0]), bool(need[1]), dy_amax, x_amax)
+        dx, dw, dgamma, dbeta, gvi = _conv_chain_backward(x_seq, weight, gamma, v_init, y, bn_map, None, x_amax, ctx.spec,
+                                                          ctx.batch_stats, ctx.x_exact, None, grad_spikes, grad_v_last,
+                                                          bool(need[0]), bool(need[1]), bool(need[4]))
         return (dx, dw, dgamma if need[2] else None, dbeta if need[3] else None, gvi, None, None, None)
 
 
@@ -512,15 +560,10 @@ class _ConvBnLifSsa(torch.autograd.Function):
         from . import attention_kernel as A
 
         x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax = ctx.saved_tensors
-        heads, cph, scale = ctx.ssa
-        T, B, _, Lp = x_seq.shape
         need = ctx.needs_input_grad
-        grad_spikes = None
-        if grad_out is not None:
-            grad_spikes = A._ssa_packed(bits, grad_out, torch.float32, T * B, heads, cph, Lp, scale).view(y.shape)
-        dy, dgamma, dbeta, gvi, dy_amax = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
-                                                            grad_v_last, bool(need[4]), True)
-        dx, dw = _conv_backward(dy, x_seq, weight, ctx.x_exact, bool(need[0]), bool(need[1]), dy_amax, x_amax)
+        dx, dw, dgamma, dbeta, gvi = _conv_chain_backward(x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax, ctx.spec,
+                                                          ctx.batch_stats, ctx.x_exact, ctx.ssa, grad_out, grad_v_last,
+                                                          bool(need[0]), bool(need[1]), bool(need[4]))
         return (dx, dw, dgamma if need[2] else None, dbeta if need[3] else None, gvi, None, None, None, None)
 
 
@@ -614,24 +657,9 @@ class _LifConvBnLif(torch.autograd.Function):
     def backward(ctx, grad_spikes, grad_v_last, grad_pre_v_last, _y, _map, _bits):
         pre_seq, pre_v_init, weight, gamma, v_init, y, bn_map, bits = ctx.saved_tensors
         need = ctx.needs_input_grad
-        T, B, Cin, Lp = pre_seq.shape
-        Cout = weight.shape[0]
-        terms = _terms()
-        dy, dgamma, dbeta, gvi, dy_amax = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
-                                                            grad_v_last, bool(need[5]), True)
-        dy3 = dy.view(T * B, Cout, Lp)
-        if dy_amax is None:
-            dy_amax = amax(dy3)
-        dw = pw_grad_weight_bits(dy3, bits, Cin, dy_amax) if need[2] else None
-        gx = gpv = None
-        if need[0] or need[1]:
-            grad_pre_spikes = pw_gemm(split_weight(weight, True, terms), terms, Cin, Cout, dy3, terms, False, dy_amax)
-            tau, v_th, v_reset, flags, sg_id, sg_alpha = ctx.pre_spec
-            glast = grad_pre_v_last.flatten() if grad_pre_v_last is not None else None
-            gx, gpv, _ = K._run_backward(L.NEURON_LIF, grad_pre_spikes.view(T, -1), None, glast, None, pre_seq.view(T, -1),
-                                         pre_v_init.flatten(), None, tau, v_th, v_reset, flags, sg_id, sg_alpha, bool(need[1]))
-            gx = gx.view(pre_seq.shape) if need[0] else None
-            gpv = gpv.view(B, Cin, Lp) if need[1] else None
+        gx, gpv, dw, dgamma, dbeta, gvi = _lif_conv_chain_backward(
+            pre_seq, pre_v_init, weight, gamma, v_init, y, bn_map, bits, ctx.pre_spec, ctx.spec, ctx.batch_stats, grad_spikes,
+            grad_v_last, grad_pre_v_last, bool(need[0]), bool(need[1]), bool(need[2]), bool(need[5]))
         return (gx, gpv, dw, dgamma if need[3] else None, dbeta if need[4] else None, gvi, None, None, None)
 
 
@@ -640,6 +668,10 @@ def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_v_init: torch.Tensor, weight: tor
     """``pre_seq [T, B, Cin, L]`` is the input of a LIF (``pre_spec``, state ``pre_v_init [B, Cin, L]``) whose spikes go
     through ``weight [Cout, Cin]``, batch norm and a second LIF (``spec``, ``v_init [B, Cout, L]``).  Returns
     ``(spikes [T, B, Cout, L], v_last, v_last of the first neuron)``.  The caller has checked ``lif_conv_bn_lif_supported``."""
+    if torch.compiler.is_compiling():
+        from . import fused_ops as O
+
+        return O.lif_conv_bn_lif(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec)
     out = _LifConvBnLif.apply(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec)
     return out[0], out[1], out[2]
 
@@ -655,6 +687,10 @@ def lif_conv_bn_lif_supported(pre_seq: torch.Tensor, need_grad: bool) -> bool:
 
 def bn_lif(y_seq: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec):
     """``y_seq [T, B, C, L]`` (a convolution output) -> ``(spikes, v_last)``."""
+    if torch.compiler.is_compiling():
+        from . import fused_ops as O
+
+        return O.bn_lif(y_seq, gamma, beta, v_init, bn, spec)
     spikes, v_last, _ = _BnLif.apply(y_seq, gamma, beta, v_init, bn, spec)
     return spikes, v_last
 
@@ -662,6 +698,10 @@ def bn_lif(y_seq: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec):
 def conv_bn_lif(x_seq: torch.Tensor, weight: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec, x_exact: bool):
     """``x_seq [T, B, Cin, L]``, ``weight [Cout, Cin]`` -> ``(spikes [T, B, Cout, L], v_last [B, Cout, L])``.
     ``x_exact``: every element of ``x_seq`` is exactly representable in bf16 (spikes, small integers)."""
+    if torch.compiler.is_compiling():
+        from . import fused_ops as O
+
+        return O.conv_bn_lif(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, None)
     spikes, v_last, _, _, _ = _ConvBnLif.apply(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact)
     return spikes, v_last
 
@@ -670,6 +710,10 @@ def conv_bn_lif_ssa(x_seq: torch.Tensor, weight: torch.Tensor, gamma, beta, v_in
                     heads: int, channels_per_head: int, scale: float):
     """The same block with ``Cout = 3 * heads * channels_per_head`` followed by the contraction; returns
     ``(out [T * B, heads, channels_per_head, L], v_last)``."""
+    if torch.compiler.is_compiling():
+        from . import fused_ops as O
+
+        return O.conv_bn_lif(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, (heads, channels_per_head, scale))
     out, v_last, _, _, _, _ = _ConvBnLifSsa.apply(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact,
                                                (heads, channels_per_head, scale))
     return out, v_last

@@ -94,9 +94,11 @@ def conv_bn_lif(x_seq: torch.Tensor, conv: Optional[nn.Module], bn: nn.Module, n
 
     if not unobserved(conv, bn, node, attn, container):
         return None
-    if (not configure.hip_fuse_conv_bn_lif or torch.compiler.is_compiling() or type(node) is not neuron.LIFNode or node.backend != "hip" or node.step_mode != "m"
+    if (not configure.hip_fuse_conv_bn_lif or type(node) is not neuron.LIFNode or node.backend != "hip" or node.step_mode != "m"
             or node.store_v_seq or x_seq.dim() < 4):
         return None
+    if attn is not None and torch.compiler.is_compiling():
+        return None  # (the contraction with the attention's neuron inside has no operator form: eager only)
     if conv is not None and (not _pointwise(conv) or x_seq.shape[2] != conv.in_channels):
         return None
     channels = conv.out_channels if conv is not None else x_seq.shape[2]
@@ -173,7 +175,7 @@ def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_node: nn.Module, conv: nn.Module,
 
     if not unobserved(pre_node, conv, bn, node, container):
         return None
-    if (not configure.hip_fuse_conv_bn_lif or not getattr(configure, "hip_conv_bit_spikes", True) or torch.compiler.is_compiling()
+    if (not configure.hip_fuse_conv_bn_lif or not getattr(configure, "hip_conv_bit_spikes", True)
             or type(node) is not neuron.LIFNode or node.backend != "hip" or node.step_mode != "m" or node.store_v_seq
             or not _plain_hip_lif(pre_node) or pre_seq.dim() < 4):
         return None

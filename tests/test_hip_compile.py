@@ -157,3 +157,63 @@ def test_inductor_compiles_linear_then_hip_node(shape):
     torch.testing.assert_close(xb.grad, xa.grad, rtol=1e-3, atol=1e-3 * scale)
     torch.testing.assert_close(traced.fc.weight.grad, eager.fc.weight.grad, rtol=1e-3,
                                atol=1e-3 * float(eager.fc.weight.grad.abs().max()))
+
+
+def _attention_block(dim, heads, seed):
+    torch.manual_seed(seed)
+    block = layer.SpikingSelfAttention(dim, heads, backend="hip").cuda().train()
+    with torch.no_grad():
+        block.qkv_conv_bn[1].weight.fill_(2.0)
+        block.proj_conv_bn[1].weight.fill_(3.0)
+    return block
+
+
+def _launch_counts(L):
+    return {name: L.profile_read(getattr(L, name))[0] for name in
+            ("KC_PW_GEMM", "KC_PW_GRAD_WEIGHT", "KC_BN_LIF_FORWARD", "KC_BN_LIF_BACKWARD", "KC_BN_GRAD_INPUT", "KC_SSA_FORWARD",
+             "KC_SSA_BACKWARD", "KC_FORWARD", "KC_BACKWARD")}
+
+
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
+@pytest.mark.parametrize("dim,heads,T,B,tokens", [(64, 2, 4, 2, 36), (384, 12, 4, 2, 196)])
+def test_compiled_attention_block_keeps_the_fused_chain(backend, dim, heads, T, B, tokens):
+    """``torch.compile(SpikingSelfAttention(..., backend='hip'), fullgraph=True)`` launches the kernels of the fused
+    convolution / batch norm / LIF chain that the eager module launches (counted by the library's own launch counters:
+    the convolution GEMMs, the batch-norm + LIF kernels, the contraction), in forward and backward, with results equal
+    to eager bit for bit: the chain is a set of opaque operators to the tracer, as the reference's kernel backends are
+    (test/activation_based/test_compile_compat.py:125-170)."""
+    from spikingjelly_amd.activation_based import functional
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+
+    if backend == "inductor" and not _triton_available():
+        pytest.skip("the inductor backend generates triton kernels and triton is not importable")
+    eager, traced = _attention_block(dim, heads, 7), _attention_block(dim, heads, 7)
+    fn = torch.compile(traced, fullgraph=True, backend=backend)
+    x = seeded_randn((T, B, dim, tokens), 19).cuda()
+    g = seeded_randn((T, B, dim, tokens), 20).cuda()
+    results = []
+    for module, call in ((eager, eager), (traced, fn)):
+        xi = x.clone().requires_grad_()
+        call(xi).backward(g)  # (first call: compilation; its launches are not counted; both modules take the same step)
+        functional.reset_net(module)
+        module.zero_grad(set_to_none=True)
+        xi = x.clone().requires_grad_()
+        torch.cuda.synchronize()
+        L.profile_reset()
+        L.profile_enable(True)
+        out = call(xi)
+        out.backward(g)
+        torch.cuda.synchronize()
+        L.profile_enable(False)
+        results.append((out.detach(), xi.grad, [p.grad for p in module.parameters()], _launch_counts(L),
+                        [b.clone() for b in module.buffers()]))
+        functional.reset_net(module)
+    (out_e, gx_e, gp_e, counts_e, buf_e), (out_c, gx_c, gp_c, counts_c, buf_c) = results
+    assert counts_e["KC_PW_GEMM"] == 4 and counts_e["KC_PW_GRAD_WEIGHT"] == 2 and counts_e["KC_BN_LIF_FORWARD"] == 2
+    assert counts_c == counts_e, (counts_c, counts_e)
+    assert float(out_e.mean()) > 0.02
+    assert torch.equal(out_c, out_e) and torch.equal(gx_c, gx_e)
+    for a, b in zip(gp_c, gp_e):
+        assert torch.equal(a, b)
+    for a, b in zip(buf_c, buf_e):   # running statistics and the batch counter
+        assert torch.equal(a, b)

@@ -116,3 +116,44 @@ def test_module_traces_under_torch_compile_with_the_eager_backend():
     fn = torch.compile(lambda t: functional.lif_multi_step_hip(t, torch.zeros_like(t[0]), 2.0, True, 1.0, 0.0,
                                                                surrogate.ATan(), False, False)[0], backend="eager")
     assert torch.equal(fn(x), eager)
+
+
+def _chain_inputs(T=3, B=2, Cin=8, Cout=12, Lp=8):
+    x = seeded_randn((T, B, Cin, Lp), 31, 0.0, 1.5).cuda().requires_grad_()
+    w = (seeded_randn((Cout, Cin), 32, 0.0, 0.4)).cuda().requires_grad_()
+    gamma = seeded_randn((Cout,), 33, 1.5, 0.2).cuda().requires_grad_()
+    beta = seeded_randn((Cout,), 34, 0.5, 0.3).cuda().requires_grad_()
+    v0 = torch.zeros((1,), device="cuda").expand(B, Cout, Lp)
+    rm, rv = torch.zeros(Cout, device="cuda"), torch.ones(Cout, device="cuda")
+    tracked = torch.zeros((), dtype=torch.int64, device="cuda")
+    return x, w, gamma, beta, v0, rm, rv, tracked
+
+
+def test_fused_chain_ops():
+    """The operators a tracing compiler sees in place of the fused convolution / batch norm / LIF chains
+    (``hip_kernel/fused_ops.py``): schema (including the mutated running statistics), fake kernels, autograd
+    registration and AOT dispatch."""
+    from spikingjelly_amd.activation_based.hip_kernel import conv_bn_lif as C
+    from spikingjelly_amd.activation_based.hip_kernel import fused_ops as O
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+    from spikingjelly_amd.activation_based.hip_kernel import neuron_kernel as K
+
+    flags = K._flags(False, True, True, 0)
+    spec = (2.0, 1.0, 0.0, flags, 0, 4.0)
+    x, w, gamma, beta, v0, rm, rv, tracked = _chain_inputs()
+    terms = C._terms()
+    for heads, cph in ((0, 0), (2, 2)):
+        torch.library.opcheck(O.hip_conv_bn_lif_forward,
+                              (x, w, gamma, beta, v0, rm, rv, True, 0.1, 1e-5, *spec, False, terms, heads, cph, 0.125),
+                              test_utils=TESTS)
+    y = seeded_randn((3, 2, 12, 8), 35, 0.4, 1.5).cuda().requires_grad_()
+    torch.library.opcheck(O.hip_bn_lif_forward, (y, gamma, beta, v0, rm, rv, True, 0.1, 1e-5, *spec), test_utils=TESTS)
+    torch.library.opcheck(O.hip_bn_lif_forward, (y, None, None, v0, rm, rv, False, 0.1, 1e-5, *spec), test_utils=TESTS)
+    assert float(rm.abs().max()) == 0.0 and float((rv - 1).abs().max()) == 0.0   # the operators write to no argument
+    pre = seeded_randn((3, 2, 8, 8), 36, 0.6, 1.0).cuda().requires_grad_()
+    pre_v0 = torch.zeros((2, 8, 8), device="cuda")
+    torch.library.opcheck(O.hip_lif_conv_bn_lif_forward,
+                          (pre, pre_v0, w, gamma, beta, v0, rm, rv, True, 0.1, 1e-5, *spec, *spec, terms), test_utils=TESTS)
+    x2 = seeded_randn((3, 2 * 3 * 2 * 2 * 8), 37, 0.6, 1.0).cuda().requires_grad_()   # B = 2, 3 x 2 heads x 2 channels x 8 tokens
+    torch.library.opcheck(O.hip_lif_ssa_forward, (x2, torch.zeros(x2.shape[1], device="cuda"), *spec, 6, 2, 2, 8, 0.125),
+                          test_utils=TESTS)
