@@ -208,9 +208,11 @@ int sjhip_neuron_backward(int neuron, int dtype, const sjhip_neuron_params *p,
  * part of the library's code object (one copy per GPU, held until the process ends), so the call reaches no
  * hipMalloc / hipFree.  PLIF without SJHIP_FLAG_ATOMIC_REDUCE accepts N <= SJHIP_STATIC_WORKSPACE_MAX_NEURONS and
  * returns SJHIP_ERR_TOO_LARGE beyond; other neurons use no workspace and are passed through.  The stream's device must
- * be the current device.  Every call on one GPU shares that GPU's array: calls that overlap there (two streams, two
- * threads) race on the partial sums; calls on one stream are ordered and need no clearing in between (each launch
- * writes every partial it later sums).
+ * be the current device.  Every call on one GPU shares that GPU's array: calls on one stream are ordered and need no
+ * clearing in between (each launch writes every partial it later sums); a call on another stream of the GPU while the
+ * last call's work has not finished is refused with SJHIP_ERR_INVALID (an event recorded behind every launch that uses
+ * the array, created once per GPU, tells), so order such calls with one stream or an event.  A stream that is being
+ * captured into a graph is neither checked nor recorded: the caller orders the replays of graphs that use the array.
  */
 #define SJHIP_STATIC_WORKSPACE_MAX_NEURONS (INT64_C(1) << 26)
 int sjhip_neuron_backward_static(int neuron, int dtype, const sjhip_neuron_params *p,

@@ -47,21 +47,28 @@ def _pointwise(conv: nn.Module) -> bool:
 
 def _bn_arguments(bn: nn.Module):
     """``(gamma, beta, (running_mean, running_var, batch_stats, momentum, eps, num_batches_tracked))`` the way
-    ``_BatchNorm.forward`` derives them, or ``None`` for what the kernels do not cover (cumulative moving average).  The
-    last element is the counter to increment (by the launch that updates the running statistics), or ``None``."""
+    ``_BatchNorm.forward`` derives them (``None`` for another kind of module).  The last element is the counter to
+    increment (by the launch that updates the running statistics), or ``None``.  With ``momentum=None`` (cumulative
+    moving average) the factor is ``1 / num_batches_tracked`` after the increment, which torch reads back to the host
+    at this point of ``_BatchNorm.forward`` as well; the counter is then incremented here."""
     if not isinstance(bn, (nn.BatchNorm1d, nn.BatchNorm2d)):
         return None
     batch_stats = bn.training or (bn.running_mean is None and bn.running_var is None)
     update = bn.training and bn.track_running_stats
-    if update and bn.momentum is None:
-        return None
     tracked = bn.num_batches_tracked if update and bn.num_batches_tracked is not None else None
+    momentum = float(bn.momentum or 0.0)
+    if update and bn.momentum is None:
+        if tracked is None or torch.compiler.is_compiling():  # (a value read back from the device is no part of a traced graph)
+            return None
+        tracked.add_(1)
+        momentum = 1.0 / float(tracked)
+        tracked = None
     if tracked is not None and not (tracked.is_cuda and tracked.dtype == torch.int64):
         tracked.add_(1)
         tracked = None
     running_mean = bn.running_mean if (update or not batch_stats) else None
     running_var = bn.running_var if (update or not batch_stats) else None
-    return bn.weight, bn.bias, (running_mean, running_var, batch_stats, float(bn.momentum or 0.0), float(bn.eps), tracked)
+    return bn.weight, bn.bias, (running_mean, running_var, batch_stats, momentum, float(bn.eps), tracked)
 
 
 def _lif_spec(node: neuron.LIFNode, x_like: torch.Tensor, need_grad: bool):

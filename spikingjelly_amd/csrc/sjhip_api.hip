@@ -128,9 +128,27 @@ namespace {
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 float *g_scratch_ptr[kMaxDevices] = {nullptr};
+// Every call on a device shares that device's array, so two calls whose kernels overlap would corrupt each other's
+// partial sums.  Calls on one stream are ordered; a call on another stream is refused while the last call's work has not
+// finished.  `g_scratch_done` is recorded behind every launch that uses the array (made once per device, beside the
+// address look-up); a stream that is being captured into a graph records and checks nothing (the caller orders the
+// graph's replays).
+hipEvent_t g_scratch_done[kMaxDevices] = {nullptr};
+hipStream_t g_scratch_stream[kMaxDevices] = {nullptr};
+bool g_scratch_used[kMaxDevices] = {false};
 
-// Device address of `scratch` on the current device, looked up once per device.
-int static_workspace(const char *what, float **out) {
+bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+
+// Device address of `scratch` on the current device, looked up once per device; refuses a call on `stream` while a call
+// made on another stream of the device is still running.
+int static_workspace(const char *what, hipStream_t stream, float **out, int *device) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return fail(SJHIP_ERR_LAUNCH, "%s: hipGetDevice: %s", what, hipGetErrorString(e));
@@ -141,10 +159,32 @@ int static_workspace(const char *what, float **out) {
     e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !ptr)
       return fail(SJHIP_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch) on device %d: %s", what, dev, hipGetErrorString(e));
+    e = hipEventCreateWithFlags(&g_scratch_done[dev], hipEventDisableTiming);
+    if (e != hipSuccess) return fail(SJHIP_ERR_LAUNCH, "%s: hipEventCreateWithFlags on device %d: %s", what, dev, hipGetErrorString(e));
     g_scratch_ptr[dev] = ptr;
   }
+  if (g_scratch_used[dev] && g_scratch_stream[dev] != stream && !stream_is_capturing(stream)) {
+    e = hipEventQuery(g_scratch_done[dev]);
+    if (e == hipErrorNotReady)
+      return fail(SJHIP_ERR_INVALID, "%s: the built-in workspace of device %d is in use by a call on another stream that has not "
+                  "finished; order the calls (one stream, or an event between them)", what, dev);
+    if (e != hipSuccess) (void)hipGetLastError();
+  }
   *out = g_scratch_ptr[dev];
+  *device = dev;
   return SJHIP_OK;
+}
+
+// After the launch that uses the array: remember the stream and when its work ends.
+void static_workspace_launched(int dev, hipStream_t stream) {
+  if (stream_is_capturing(stream)) return;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (hipEventRecord(g_scratch_done[dev], stream) != hipSuccess) {
+    (void)hipGetLastError();
+    return;
+  }
+  g_scratch_stream[dev] = stream;
+  g_scratch_used[dev] = true;
 }
 
 bool valid_dtype_fp(int dtype) { return dtype == SJHIP_F32 || dtype == SJHIP_F16 || dtype == SJHIP_BF16; }
@@ -262,16 +302,19 @@ int sjhip_neuron_backward_static(int neuron, int dtype, const sjhip_neuron_param
   int rc = check_backward(neuron, dtype, p, T, N, grad_spike_seq, h_seq, v_init, rtau_device, grad_x_seq, grad_v_init, grad_rtau);
   if (rc != SJHIP_OK) return rc;
   float *workspace = nullptr;
+  int device = 0;
   if (neuron == SJHIP_NEURON_PLIF && !(p->flags & SJHIP_FLAG_ATOMIC_REDUCE)) {
     if (plif_blocks(dtype, N) > kStaticWorkspaceFloats)
       return fail(SJHIP_ERR_TOO_LARGE, "backward(static): N=%lld needs %lld partial sums, the built-in workspace holds %lld "
                   "(N <= %lld); use sjhip_neuron_backward with a workspace of the caller's", (long long)N,
                   (long long)plif_blocks(dtype, N), (long long)kStaticWorkspaceFloats, (long long)(kStaticWorkspaceFloats * 64));
-    rc = static_workspace("backward(static)", &workspace);
+    rc = static_workspace("backward(static)", static_cast<hipStream_t>(stream), &workspace, &device);
     if (rc != SJHIP_OK) return rc;
   }
-  return launch_backward(neuron, dtype, *p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, rtau_device, grad_x_seq,
-                         grad_v_init, grad_rtau, workspace, static_cast<hipStream_t>(stream));
+  rc = launch_backward(neuron, dtype, *p, T, N, grad_spike_seq, grad_v_seq, grad_v_last, h_seq, v_init, rtau_device, grad_x_seq,
+                       grad_v_init, grad_rtau, workspace, static_cast<hipStream_t>(stream));
+  if (rc == SJHIP_OK && workspace) static_workspace_launched(device, static_cast<hipStream_t>(stream));
+  return rc;
 }
 
 namespace {

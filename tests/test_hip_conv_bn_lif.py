@@ -768,6 +768,33 @@ def test_autocast_keeps_the_modules_in_charge(monkeypatch):
     assert calls == [] and out.shape == x.shape
 
 
+def test_cumulative_moving_average_batch_norm_runs_fused(monkeypatch):
+    """``BatchNorm1d(momentum=None)``: the running statistics are the plain average over the batches seen, with the
+    factor 1 / num_batches_tracked (nn.modules.batchnorm._BatchNorm.forward); the fused chain follows it step by step."""
+    from spikingjelly_amd.activation_based.layer import fused
+
+    fused_block, plain_block = _make_block(64, 2, 66).cuda().train(), _make_block(64, 2, 66).cuda().train()
+    for block in (fused_block, plain_block):
+        for bn in (block.qkv_conv_bn[1], block.proj_conv_bn[1]):
+            bn.momentum = None
+    calls = []
+    real = fused.conv_bn_lif
+    monkeypatch.setattr(fused, "conv_bn_lif", lambda *a, **k: (lambda r: calls.append(r is not None) or r)(real(*a, **k)))
+    for step in range(3):
+        x = seeded_randn((4, 2, 64, 36), 67 + step, 0.1 * step, 1.0 + step).cuda()
+        monkeypatch.setattr(configure, "hip_fuse_conv_bn_lif", True)
+        fused_block(x)
+        monkeypatch.setattr(configure, "hip_fuse_conv_bn_lif", False)
+        plain_block(x)
+        functional.reset_net(fused_block)
+        functional.reset_net(plain_block)
+        for a, b in zip((fused_block.qkv_conv_bn[1], fused_block.proj_conv_bn[1]), (plain_block.qkv_conv_bn[1], plain_block.proj_conv_bn[1])):
+            assert int(a.num_batches_tracked) == int(b.num_batches_tracked) == step + 1
+            torch.testing.assert_close(a.running_mean, b.running_mean, rtol=1e-4, atol=1e-5)
+            torch.testing.assert_close(a.running_var, b.running_var, rtol=1e-4, atol=1e-5)
+    assert calls[0] is True and all(calls[::2])   # the qkv chain ran fused in every step
+
+
 def test_eval_mode_spikes_are_bit_identical_to_the_torch_backend_on_exact_inputs():
     """Binary input, weights that are multiples of 1/64, batch norm in evaluation mode with an exactly representable map
     (running variance + eps exactly 1, gamma and beta multiples of 1/8): every convolution sum and every normalised value is

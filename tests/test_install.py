@@ -250,3 +250,50 @@ def test_installed_classes_run_the_hip_kernels(stand_in, kind, store_v_seq):
     single_b = getattr(neuron, kind)(step_mode="s", backend="hip", surrogate_function=surrogate.ATan(), **kw).cuda()
     for t in range(3):
         assert bits_equal(single_a(x[t]), single_b(x[t]))
+
+
+def test_stand_in_and_install_agree_with_the_reference_interface(stand_in):
+    """``tests/golden/reference_install_facts.json`` (written by ``tests/golden/make_install_facts.py`` from the
+    reference's source text: ``neuron/lif.py:231-398``, ``neuron/integrate_and_fire.py``, ``neuron/plif.py``,
+    ``base.py:35-90, 398-440``) lists what ``install`` relies on.  The stand-in package of these tests must have that
+    interface, and what ``install`` replaces must exist in the reference under the same names and parameter lists."""
+    import inspect
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_install_facts.json")) as f:
+        facts = json.load(f)
+    sn = importlib.import_module("sj_stand_in.activation_based.neuron")
+    sb = importlib.import_module("sj_stand_in.activation_based.base")
+
+    def parameters(fn):
+        out = []
+        for p in inspect.signature(fn).parameters.values():
+            out.append({p.VAR_POSITIONAL: "*", p.VAR_KEYWORD: "**"}.get(p.kind, "") + p.name)
+        return out
+
+    assert parameters(sb.check_backend_library) == facts["check_backend_library"]["parameters"]
+    assert facts["MemoryModule"]["backend_setter_calls_check_backend_library"]
+    assert facts["MemoryModule"]["backend_setter_not_implemented_message"] == ["f'{value} is not a supported backend of {self._get_name()}!'"]
+    for name, ref in facts["classes"].items():
+        cls = getattr(sn, name)
+        assert ref["supported_backends_is_property"] and isinstance(inspect.getattr_static(cls, "supported_backends"), property)
+        for forward, params in ref["forwards"].items():
+            assert parameters(getattr(cls, forward)) == params, (name, forward)
+        assert parameters(cls.materialize_states) == facts["MemoryModule"]["materialize_states"]
+        # the stand-in offers a subset of the reference's backends in either step mode, 'torch' among them
+        for mode in ("s", "m"):
+            assert set(cls(step_mode=mode).supported_backends) - {"hip"} <= set(ref["supported_backends"][mode]) | {"cupy"}
+            assert "torch" in ref["supported_backends"][mode]
+        with pytest.raises(NotImplementedError, match="is not a supported backend of"):
+            cls(step_mode="m").backend = "no-such-backend"
+    spikingjelly_amd.install(stand_in)
+    for name, ref in facts["classes"].items():
+        cls = getattr(sn, name)
+        assert isinstance(inspect.getattr_static(cls, "supported_backends"), property)
+        for forward, params in ref["forwards"].items():   # the replaced methods keep the reference's parameter lists
+            assert parameters(getattr(cls, forward)) == params, (name, forward)
+        for mode in ("s", "m"):
+            node = cls(step_mode=mode)
+            assert node.supported_backends[-1] == "hip" and "hip" not in ref["supported_backends"][mode]
+    assert parameters(sb.check_backend_library) == facts["check_backend_library"]["parameters"]

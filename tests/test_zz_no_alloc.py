@@ -124,3 +124,41 @@ def test_static_workspace_backward_passes_other_neurons_through(L):
         torch.cuda.synchronize()
         out.append((gx.cpu(), gv0.cpu()))
     assert bits_equal(out[0][0], out[1][0]) and bits_equal(out[0][1], out[1][1])
+
+
+def test_a_call_on_another_stream_is_refused_while_the_array_is_in_use(L):
+    """Calls on one GPU share its array.  A call on a second stream while the first call's kernels still run would mix
+    two sets of partial sums: the library refuses it (SJHIP_ERR_INVALID) instead; after the first stream has finished,
+    or on the first stream itself, the call goes through."""
+    lib = L.load()
+    c = _plif_case(L, 16, 1 << 24, 31)   # a backward of about a millisecond
+    small = _plif_case(L, 4, 4 * 1024, 32)
+    torch.cuda.synchronize()
+    other = torch.cuda.Stream()
+
+    def buffers(case):
+        return (torch.empty_like(case["x"]), torch.empty_like(case["v0"]),
+                torch.empty((1,), dtype=torch.float32, device=case["x"].device))
+
+    def call(case, out, stream_ptr):
+        gx, gv0, gk = out
+        return lib.sjhip_neuron_backward_static(L.NEURON_PLIF, L.dtype_id(case["dtype"]), ctypes.byref(case["p"]), case["T"],
+                                                case["N"], case["gs"].data_ptr(), case["gv"].data_ptr(), None, case["h"].data_ptr(),
+                                                case["v0"].data_ptr(), case["kd"].data_ptr(), gx.data_ptr(), gv0.data_ptr(),
+                                                gk.data_ptr(), stream_ptr)
+
+    # every buffer exists before the first launch: nothing between the launches below waits for the device
+    big_out, same_out, other_out, out = buffers(c), buffers(small), buffers(small), buffers(small)
+    torch.cuda.synchronize()
+    for _ in range(20):   # some fifteen milliseconds of work on the first stream
+        assert call(c, big_out, c["stream"]) == 0
+    rc_same = call(small, same_out, c["stream"])          # same stream: ordered behind the calls before
+    rc_other = call(small, other_out, other.cuda_stream)  # another stream while the first one still works
+    message = lib.sjhip_last_error()
+    torch.cuda.synchronize()
+    assert rc_same == 0
+    assert rc_other == -1 and b"another stream" in message
+    assert call(small, out, other.cuda_stream) == 0       # everything has finished: the other stream may use the array
+    torch.cuda.synchronize()
+    ref = _backward(L, small, False)
+    assert bits_equal(out[0].cpu(), ref[0]) and bits_equal(out[1].cpu(), ref[1]) and bits_equal(out[2].cpu(), ref[2])
