@@ -426,7 +426,7 @@ inline int build_bwd_args(BwdArgs &a, int neuron, int dtype, const sjhip_neuron_
   a.grad_x = grad_x_seq; a.grad_v_init = grad_v_init;
   a.partials = workspace; a.grad_k = grad_rtau;
   a.T = T; a.N = N;
-  a.spread = column_spread(N * (dtype == SJHIP_F32 ? 4 : 2));
+  a.spread = column_spread(N * (dtype == SJHIP_F32 ? 4 : 2), T);
   a.v_th = p.v_threshold; a.v_reset = p.v_reset; a.alpha = p.sg_alpha;
   a.sg = p.sg_id;
   a.soft_reset = (p.flags & SJHIP_FLAG_SOFT_RESET) ? 1 : 0;

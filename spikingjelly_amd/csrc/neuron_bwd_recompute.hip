@@ -84,7 +84,7 @@ int launch_replay(int neuron, int dtype, const sjhip_neuron_params &p, int64_t T
   const bool several = chunk > 0 && T > chunk;
   if (several && auto_order) b.spread = 1;
   int block = recompute_block(dtype, lds_steps, round_each);
-  if (b.spread && auto_order) {
+  if ((several || b.spread > 1) && auto_order) {
     const int want = several ? kSpreadBlock : spread_block(N * (dtype == SJHIP_F32 ? 4 : 2));
     if (want > block && want <= SJHIP_MAX_BLOCK && 2 * lds_steps * want * kHBytesPerItem <= (int64_t)kMaxLds) block = want;
   }

@@ -391,7 +391,7 @@ inline int build_fwd_args(FwdArgs &a, bool &round_each, int neuron, int dtype, c
   a.k_device = nullptr;
   a.checkpoints = nullptr; a.chunk = 0;
   a.T = T; a.N = N;
-  a.spread = column_spread(N * (dtype == SJHIP_F32 ? 4 : 2));
+  a.spread = column_spread(N * (dtype == SJHIP_F32 ? 4 : 2), T);
   const bool ilif = neuron == SJHIP_NEURON_ILIF;
   a.soft_reset = ilif ? RESET_COUNT : ((p.flags & SJHIP_FLAG_SOFT_RESET) ? RESET_SOFT : RESET_HARD);
   a.level_max = p.level_max;

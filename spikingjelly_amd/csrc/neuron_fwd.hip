@@ -16,7 +16,8 @@ constexpr bool kStreamX = (sizeof(S) == 2 && !ROUND_EACH) || (sizeof(S) == 4 && 
 template <typename S, bool ROUND_EACH, bool PACKED = false>
 int launch_typed(const FwdArgs &a, bool vector, hipStream_t stream) {
   int block = tuning().fwd_block;
-  if (a.spread && tuning().column_spread == 2) block = spread_block(a.N * (int64_t)sizeof(S));
+  // (the block size changes only with the runs that answer a resonant row stride, not with the contiguous eighths)
+  if (a.spread > 1 && tuning().column_spread == 2) block = spread_block(a.N * (int64_t)sizeof(S));
   const int V = vector ? Acc<S, true, true>::V : 1;
   const int64_t items = (a.N + V - 1) / V;
   const int64_t blocks = (items + block - 1) / block;
