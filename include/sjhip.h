@@ -560,7 +560,7 @@ int sjhip_pwconv_grad_weight_f16_bits(const float *dy, const float *dy_amax, con
 
 /*
  * The same GEMMs with the activations / gradients arriving as fp16 term planes that their producer wrote already scaled
- * and split (sjhip_pwconv_split_planes, or the kernel that computes the tensor: sjhip_bn_grad_input_planes), instead of
+ * and split (sjhip_pwconv_split_planes), instead of
  * fp32 tensors that every block of a GEMM splits again while it stages them (same reference lines:
  * layer/attention.py:310-329, model/spikformer.py:85-99).  A plane buffer of a tensor x [S][C][L] holds `terms` planes
  * [C][ld] of fp16, ld = S * L rounded up to a multiple of 8 (16-byte aligned rows): element (c, s * L + l) of plane 0 is
