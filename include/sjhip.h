@@ -609,7 +609,7 @@ int sjhip_pwconv_grad_weight_planes(const uint16_t *dy_planes, const float *dy_a
  *                       params as sjhip_neuron_forward; neuron IF or LIF); spikes go to spike_seq [T][B][C][L] (fp32) or
  *                       bit-packed to spike_bits (the layout of sjhip_bit_pack; B*C*L must be a multiple of 8): exactly
  *                       one of the two is given; v_last [B][C][L] or NULL
- *   sjhip_bn_lif_backward  replays the neuron from y (T <= 16), runs the BPTT recurrence of sjhip_neuron_backward with
+ *   sjhip_bn_lif_backward  replays the neuron from y (T <= 256; beyond 16 steps in pieces of 16), runs the BPTT recurrence of sjhip_neuron_backward with
  *                       grad_spike_seq and (optionally) grad_v_last, writes grad_z = dL/dz [T][B][C][L], grad_v_init
  *                       (or NULL) and partial[b][c] = (sum g, sum g y) over the row and all steps
  *   sjhip_bn_backward_finalize   dgamma, dbeta (either may be NULL) and coef [3][C] = (p, q, r) of dy = p g + q y + r;

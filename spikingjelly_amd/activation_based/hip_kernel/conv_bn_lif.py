@@ -41,7 +41,7 @@ __all__ = ["supported", "bn_lif", "conv_bn_lif", "conv_bn_lif_ssa", "conv_bn_lif
            "pw_grad_weight", "pw_gemm_bits", "pw_grad_weight_bits", "amax", "F16", "split_planes", "pw_gemm_planes",
            "pw_grad_weight_planes"]
 
-MAX_REPLAY_STEPS = 16  # the backward replays the neuron with h of every step in registers
+MAX_REPLAY_STEPS = 256  # the backward replays the neuron in pieces of 16 steps, one parked state per piece in LDS
 
 
 F16 = 16  # term code of an fp16 operand: F16 | 2 (hi and lo of a scaled value) or F16 | 1 (exact in fp16)
@@ -78,7 +78,7 @@ def _exact(terms: int) -> int:
 
 
 def supported(x_seq: torch.Tensor, need_grad: bool) -> bool:
-    """fp32 device tensor ``[T, B, C, L]`` whose rows of ``L`` elements start on 16 bytes; at most 16 steps when a
+    """fp32 device tensor ``[T, B, C, L]`` whose rows of ``L`` elements start on 16 bytes; at most ``MAX_REPLAY_STEPS`` steps when a
     backward will follow."""
     return (x_seq.is_cuda and x_seq.dtype == torch.float32 and x_seq.dim() == 4 and x_seq.shape[-1] % 4 == 0
             and x_seq.numel() > 0 and (not need_grad or x_seq.shape[0] <= MAX_REPLAY_STEPS))

@@ -209,11 +209,11 @@ template <bool PACKED> __global__ void __launch_bounds__(256) bn_lif_forward_ker
 
 // h of every step of this work-item's four neurons, replayed from y
 template <int CH, int RS, int TMAX>
-__device__ __forceinline__ void replay_h(const FwdArgs &f, const f32x4 (&yv)[TMAX], float sc, float sh, float (&v)[4],
+__device__ __forceinline__ void replay_h(const FwdArgs &f, int len, const f32x4 (&yv)[TMAX], float sc, float sh, float (&v)[4],
                                          float (&h)[TMAX][4]) {
 #pragma unroll
   for (int t = 0; t < TMAX; ++t) {
-    if (t < f.T) {
+    if (t < len) {
       const float y[4] = {yv[t].x, yv[t].y, yv[t].z, yv[t].w};
       float s;
 #pragma unroll
@@ -223,27 +223,40 @@ __device__ __forceinline__ void replay_h(const FwdArgs &f, const f32x4 (&yv)[TMA
 }
 
 template <int CH, int TMAX>
-__device__ __forceinline__ void replay_h_reset(const FwdArgs &f, const f32x4 (&yv)[TMAX], float sc, float sh, float (&v)[4],
-                                               float (&h)[TMAX][4]) {
-  if (f.soft_reset) replay_h<CH, RESET_SOFT, TMAX>(f, yv, sc, sh, v, h);
-  else replay_h<CH, RESET_HARD, TMAX>(f, yv, sc, sh, v, h);
+__device__ __forceinline__ void replay_h_reset(const FwdArgs &f, int len, const f32x4 (&yv)[TMAX], float sc, float sh,
+                                               float (&v)[4], float (&h)[TMAX][4]) {
+  if (f.soft_reset) replay_h<CH, RESET_SOFT, TMAX>(f, len, yv, sc, sh, v, h);
+  else replay_h<CH, RESET_HARD, TMAX>(f, len, yv, sc, sh, v, h);
+}
+
+// the steps t0 .. t0 + len - 1 (len <= TMAX) of this work-item's four neurons from the state v in front of step t0
+template <int TMAX>
+__device__ __forceinline__ void replay_h_charge(const FwdArgs &f, int len, const f32x4 (&yv)[TMAX], float sc, float sh,
+                                                float (&v)[4], float (&h)[TMAX][4]) {
+  switch (f.charge) {
+    case CH_IF: replay_h_reset<CH_IF, TMAX>(f, len, yv, sc, sh, v, h); break;
+    case CH_DECAY_INPUT_DIV: replay_h_reset<CH_DECAY_INPUT_DIV, TMAX>(f, len, yv, sc, sh, v, h); break;
+    case CH_DECAY_INPUT_MUL: replay_h_reset<CH_DECAY_INPUT_MUL, TMAX>(f, len, yv, sc, sh, v, h); break;
+    case CH_PLAIN_INPUT_DIV: replay_h_reset<CH_PLAIN_INPUT_DIV, TMAX>(f, len, yv, sc, sh, v, h); break;
+    default: replay_h_reset<CH_PLAIN_INPUT_MUL, TMAX>(f, len, yv, sc, sh, v, h); break;
+  }
 }
 
 // BPTT over the replayed h (recurrence of neuron_bwd.h); writes g = dL/dz and adds this work-item's share of
 // sum g and sum g y
 template <int SG, int TMAX>
-__device__ __forceinline__ void bptt_rows(const BwdArgs &b, float k, int64_t col, const f32x4 (&yv)[TMAX],
+__device__ __forceinline__ void bptt_rows(const BwdArgs &b, float k, int64_t col, int64_t t0, int len, const f32x4 (&yv)[TMAX],
                                           const float (&h)[TMAX][4], float (&carry)[4], float &acc_g, float &acc_gy) {
 #pragma clang fp contract(fast)
   typedef Acc<float, true, true> A;
   const int64_t N = b.N;
-  const float *gsp = (const float *)b.grad_spike + col;
-  float *gxp = (float *)b.grad_x + col;
+  const float *gsp = (const float *)b.grad_spike + col + t0 * N;
+  float *gxp = (float *)b.grad_x + col + t0 * N;
   const float kx = b.is_if ? 1.0f : (b.decay_input ? k : 1.0f);
   const float km = b.is_if ? 1.0f : (1.0f - k);
 #pragma unroll
   for (int t = TMAX - 1; t >= 0; --t) {
-    if (t < b.T) {
+    if (t < len) {
       float gs[4], gz[4];
       A::unpack(A::load(gsp + (int64_t)t * N), gs);
       const float y[4] = {yv[t].x, yv[t].y, yv[t].z, yv[t].w};
@@ -261,6 +274,21 @@ __device__ __forceinline__ void bptt_rows(const BwdArgs &b, float k, int64_t col
       }
       Acc<float, true, false>::store(gxp + (int64_t)t * N, gz);  // read again by the next kernel
     }
+  }
+}
+
+template <int TMAX>
+__device__ __forceinline__ void bptt_rows_surrogate(const BwdArgs &b, float k, int64_t col, int64_t t0, int len,
+                                                    const f32x4 (&yv)[TMAX], const float (&h)[TMAX][4], float (&carry)[4],
+                                                    float &acc_g, float &acc_gy) {
+  switch (b.sg) {
+    case SJHIP_SG_SIGMOID: bptt_rows<SJHIP_SG_SIGMOID, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
+    case SJHIP_SG_ATAN: bptt_rows<SJHIP_SG_ATAN, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
+    case SJHIP_SG_PIECEWISE_QUADRATIC: bptt_rows<SJHIP_SG_PIECEWISE_QUADRATIC, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
+    case SJHIP_SG_PIECEWISE_EXP: bptt_rows<SJHIP_SG_PIECEWISE_EXP, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
+    case SJHIP_SG_SOFT_SIGN: bptt_rows<SJHIP_SG_SOFT_SIGN, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
+    case SJHIP_SG_SUPER_SPIKE: bptt_rows<SJHIP_SG_SUPER_SPIKE, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
+    default: bptt_rows<SJHIP_SG_ERF, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
   }
 }
 
@@ -283,32 +311,64 @@ __device__ __forceinline__ void bn_lif_backward_quad(const BnLifBwdArgs &a, int6
   load_state<float, true, false>(f.v_init, col, f.v_init_broadcast != 0, v);
   if (b.grad_v_last) A::unpack(A::load((const float *)b.grad_v_last + col), carry);
   else carry[0] = carry[1] = carry[2] = carry[3] = 0.0f;
-  switch (f.charge) {
-    case CH_IF: replay_h_reset<CH_IF, TMAX>(f, yv, sc, sh, v, h); break;
-    case CH_DECAY_INPUT_DIV: replay_h_reset<CH_DECAY_INPUT_DIV, TMAX>(f, yv, sc, sh, v, h); break;
-    case CH_DECAY_INPUT_MUL: replay_h_reset<CH_DECAY_INPUT_MUL, TMAX>(f, yv, sc, sh, v, h); break;
-    case CH_PLAIN_INPUT_DIV: replay_h_reset<CH_PLAIN_INPUT_DIV, TMAX>(f, yv, sc, sh, v, h); break;
-    default: replay_h_reset<CH_PLAIN_INPUT_MUL, TMAX>(f, yv, sc, sh, v, h); break;
+  replay_h_charge<TMAX>(f, (int)f.T, yv, sc, sh, v, h);
+  bptt_rows_surrogate<TMAX>(b, k, col, 0, (int)b.T, yv, h, carry, acc_g, acc_gy);
+  if (b.grad_v_init) A::store((float *)b.grad_v_init + col, carry);
+}
+
+// The same for a sequence of more than kBnPiece steps, walked in pieces of kBnPiece as the plain neuron's replay over
+// pieces does: a first pass replays the whole sequence and parks the state in front of every piece in LDS (each
+// work-item its own 16 bytes per piece, no barrier), then the pieces are taken from the last to the first, each
+// replayed from its parked state into registers and walked backwards; y is read twice.
+constexpr int kBnPiece = 16;
+constexpr int kBnMaxPieces = 16;  // 256 work-items x 16 bytes x 16 pieces = 64 KiB of LDS
+__device__ __forceinline__ void bn_lif_backward_quad_long(const BnLifBwdArgs &a, int64_t row, int q, float &acc_g, float &acc_gy,
+                                                          f32x4 *parked) {
+  typedef Acc<float, true, false> A;
+  const FwdArgs &f = a.f;
+  const BwdArgs &b = a.b;
+  const int c = (int)(row % a.C);
+  const float sc = a.scale[c], sh = a.shift[c];
+  const int64_t N = f.N;
+  const int64_t col = row * a.L + 4 * q;
+  const float *yp = (const float *)f.x + col;
+  const int T = (int)f.T, pieces = (T + kBnPiece - 1) / kBnPiece;
+  f32x4 yv[kBnPiece];
+  float v[4], h[kBnPiece][4], carry[4];
+  load_state<float, true, false>(f.v_init, col, f.v_init_broadcast != 0, v);
+  for (int p = 0; p + 1 < pieces; ++p) {  // (the pieces in front of the last one are whole)
+    parked[p * blockDim.x] = f32x4{v[0], v[1], v[2], v[3]};
+#pragma unroll
+    for (int t = 0; t < kBnPiece; ++t) yv[t] = A::load(yp + (int64_t)(p * kBnPiece + t) * N);
+    replay_h_charge<kBnPiece>(f, kBnPiece, yv, sc, sh, v, h);
   }
-  switch (b.sg) {
-    case SJHIP_SG_SIGMOID: bptt_rows<SJHIP_SG_SIGMOID, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-    case SJHIP_SG_ATAN: bptt_rows<SJHIP_SG_ATAN, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-    case SJHIP_SG_PIECEWISE_QUADRATIC: bptt_rows<SJHIP_SG_PIECEWISE_QUADRATIC, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-    case SJHIP_SG_PIECEWISE_EXP: bptt_rows<SJHIP_SG_PIECEWISE_EXP, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-    case SJHIP_SG_SOFT_SIGN: bptt_rows<SJHIP_SG_SOFT_SIGN, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-    case SJHIP_SG_SUPER_SPIKE: bptt_rows<SJHIP_SG_SUPER_SPIKE, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
-    default: bptt_rows<SJHIP_SG_ERF, TMAX>(b, k, col, yv, h, carry, acc_g, acc_gy); break;
+  parked[(pieces - 1) * blockDim.x] = f32x4{v[0], v[1], v[2], v[3]};
+  if (b.grad_v_last) A::unpack(A::load((const float *)b.grad_v_last + col), carry);
+  else carry[0] = carry[1] = carry[2] = carry[3] = 0.0f;
+  for (int p = pieces - 1; p >= 0; --p) {
+    const int t0 = p * kBnPiece, len = min(kBnPiece, T - t0);
+#pragma unroll
+    for (int t = 0; t < kBnPiece; ++t) yv[t] = (t < len) ? A::load(yp + (int64_t)(t0 + t) * N) : A::zero();
+    const f32x4 s = parked[p * blockDim.x];
+    v[0] = s.x; v[1] = s.y; v[2] = s.z; v[3] = s.w;
+    replay_h_charge<kBnPiece>(f, len, yv, sc, sh, v, h);
+    bptt_rows_surrogate<kBnPiece>(b, b.k, col, t0, len, yv, h, carry, acc_g, acc_gy);
   }
   if (b.grad_v_init) A::store((float *)b.grad_v_init + col, carry);
 }
 
 // A wavefront per row; lanes stride over the row's quads.
+// (TMAX = 0: the walk in pieces, with pieces x 256 x 16 bytes of dynamic LDS)
 template <int TMAX> __global__ void __launch_bounds__(256) bn_lif_backward_kernel(const BnLifBwdArgs a) {
+  extern __shared__ f32x4 parked_states[];
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= a.rows) return;
   float acc_g = 0.0f, acc_gy = 0.0f;
-  for (int q = lane; q < a.L / 4; q += 64) bn_lif_backward_quad<TMAX>(a, row, q, acc_g, acc_gy);
+  for (int q = lane; q < a.L / 4; q += 64) {
+    if constexpr (TMAX == 0) bn_lif_backward_quad_long(a, row, q, acc_g, acc_gy, parked_states + threadIdx.x);
+    else bn_lif_backward_quad<TMAX>(a, row, q, acc_g, acc_gy);
+  }
   acc_g = wave_sum(acc_g);
   acc_gy = wave_sum(acc_gy);
   if (lane == 0) { a.partial[2 * row] = acc_g; a.partial[2 * row + 1] = acc_gy; }
@@ -323,6 +383,7 @@ template <int TMAX>
 __global__ void __launch_bounds__(256) bn_lif_backward_rows_kernel(const BnLifBwdArgs a, int quads, int rows_per_block,
                                                                    float inv_quads) {
   __shared__ float part[4][kBnRowsMax][2];
+  extern __shared__ f32x4 parked_states[];
   const int tid = threadIdx.x;
   int r_local = (int)(((float)tid + 0.5f) * inv_quads);  // tid / quads (exact: see div_tokens of ssa.hip)
   const int q = tid - r_local * quads;
@@ -330,7 +391,10 @@ __global__ void __launch_bounds__(256) bn_lif_backward_rows_kernel(const BnLifBw
   const bool valid = r_local < rows_per_block && row < a.rows;
   if (r_local >= rows_per_block) r_local = rows_per_block - 1;
   float acc_g = 0.0f, acc_gy = 0.0f;
-  if (valid) bn_lif_backward_quad<TMAX>(a, row, q, acc_g, acc_gy);
+  if (valid) {
+    if constexpr (TMAX == 0) bn_lif_backward_quad_long(a, row, q, acc_g, acc_gy, parked_states + tid);
+    else bn_lif_backward_quad<TMAX>(a, row, q, acc_g, acc_gy);
+  }
   block_row_sums(part, r_local, valid, rows_per_block, acc_g, acc_gy, a.partial, (int64_t)blockIdx.x * rows_per_block, a.rows);
 }
 
@@ -500,7 +564,8 @@ int launch_bn_lif_backward(int neuron, const sjhip_neuron_params &p, int64_t T, 
   int rc = check_layout("bn_lif_backward", T, B, C, L);
   if (rc != SJHIP_OK) return rc;
   if (!lif_like(neuron)) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: neuron %d (IF and LIF only)", neuron);
-  if (T > 16) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: T=%lld (at most 16 steps are replayed in registers)", (long long)T);
+  if (T > kBnPiece * kBnMaxPieces)
+    return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: T=%lld (at most %d steps)", (long long)T, kBnPiece * kBnMaxPieces);
   if (p.sg_id < SJHIP_SG_SIGMOID || p.sg_id > SJHIP_SG_ERF) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: surrogate id %d", p.sg_id);
   const int64_t N = B * C * L;
   const bool broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) != 0;
@@ -518,6 +583,8 @@ int launch_bn_lif_backward(int neuron, const sjhip_neuron_params &p, int64_t T, 
   const int64_t blocks = (a.rows + 3) / 4;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "bn_lif_backward: %lld rows", (long long)a.rows);
   ProfileScope prof(KC_BN_LIF_BACKWARD, stream);
+  // (the walk in pieces parks one state per piece and work-item in LDS: at most 64 KiB, no opt-in needed)
+  const unsigned parked = T > kBnPiece ? (unsigned)((T + kBnPiece - 1) / kBnPiece) * 256u * 16u : 0u;
   const int quads = (int)(L / 4);
   const int per = quads > 0 ? 256 / quads : 0;
   if (quads >= 16 && per > 4) {
@@ -527,12 +594,14 @@ int launch_bn_lif_backward(int neuron, const sjhip_neuron_params &p, int64_t T, 
     const float inv = 1.0f / (float)quads;
     if (T <= 4) hipLaunchKernelGGL((bn_lif_backward_rows_kernel<4>), dim3((unsigned)nb), dim3(256), 0, stream, a, quads, per, inv);
     else if (T <= 8) hipLaunchKernelGGL((bn_lif_backward_rows_kernel<8>), dim3((unsigned)nb), dim3(256), 0, stream, a, quads, per, inv);
-    else hipLaunchKernelGGL((bn_lif_backward_rows_kernel<16>), dim3((unsigned)nb), dim3(256), 0, stream, a, quads, per, inv);
+    else if (T <= 16) hipLaunchKernelGGL((bn_lif_backward_rows_kernel<16>), dim3((unsigned)nb), dim3(256), 0, stream, a, quads, per, inv);
+    else hipLaunchKernelGGL((bn_lif_backward_rows_kernel<0>), dim3((unsigned)nb), dim3(256), parked, stream, a, quads, per, inv);
     return check_launch("bn_lif_backward");
   }
   if (T <= 4) hipLaunchKernelGGL((bn_lif_backward_kernel<4>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
   else if (T <= 8) hipLaunchKernelGGL((bn_lif_backward_kernel<8>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
-  else hipLaunchKernelGGL((bn_lif_backward_kernel<16>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  else if (T <= 16) hipLaunchKernelGGL((bn_lif_backward_kernel<16>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL((bn_lif_backward_kernel<0>), dim3((unsigned)blocks), dim3(256), parked, stream, a);
   return check_launch("bn_lif_backward");
 }
 

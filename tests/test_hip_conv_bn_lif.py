@@ -519,7 +519,9 @@ def _no_borderline(h, v_th):
     return bool(((d > MARGIN) | (d == 0)).all())
 
 
-@pytest.mark.parametrize("T,B,Cc,Lp", [(4, 3, 10, 12), (1, 2, 5, 4), (7, 2, 33, 20), (16, 2, 6, 260), (4, 2, 12, 196)])
+# (more than 16 steps: the backward walks the sequence in pieces of 16, one kernel variant per row shape)
+@pytest.mark.parametrize("T,B,Cc,Lp", [(4, 3, 10, 12), (1, 2, 5, 4), (7, 2, 33, 20), (16, 2, 6, 260), (4, 2, 12, 196),
+                                       (17, 2, 5, 36), (33, 1, 6, 196), (40, 1, 3, 260), (64, 2, 3, 8)])
 @pytest.mark.parametrize("training", [True, False])
 @pytest.mark.parametrize("v_reset,decay_input,tau,sg", [(0.0, True, 2.0, "sigmoid"), (None, False, 3.0, "atan"), (-0.2, True, 2.5, "erf")])
 def test_bn_lif_against_float64(C, T, B, Cc, Lp, training, v_reset, decay_input, tau, sg):
@@ -606,7 +608,7 @@ def _make_block(dim, heads, seed):
     return block
 
 
-@pytest.mark.parametrize("dim,heads,T,B,tokens", [(16, 2, 3, 2, 8), (64, 2, 4, 2, 36), (48, 3, 4, 1, 196)])
+@pytest.mark.parametrize("dim,heads,T,B,tokens", [(16, 2, 3, 2, 8), (64, 2, 4, 2, 36), (48, 3, 4, 1, 196), (32, 2, 20, 1, 36)])
 @pytest.mark.parametrize("training", [True, False])
 @pytest.mark.parametrize("split,overlap", [("f16", True), ("f16", False), ("bf16", True)])
 def test_attention_block_fused_against_float64(dim, heads, T, B, tokens, training, split, overlap, monkeypatch):
@@ -799,6 +801,25 @@ def test_cumulative_moving_average_batch_norm_runs_fused(monkeypatch):
             torch.testing.assert_close(a.running_mean, b.running_mean, rtol=1e-4, atol=1e-5)
             torch.testing.assert_close(a.running_var, b.running_var, rtol=1e-4, atol=1e-5)
     assert len(calls) == 3   # the fused block's qkv chain ran fused in every step
+
+
+def test_sequences_longer_than_one_piece_stay_fused(monkeypatch):
+    """T = 20 with gradients: the chain's backward walks the sequence in pieces of 16 steps, so the block keeps its
+    fused path (the float64 comparison of this shape is a case of ``test_attention_block_fused_against_float64``)."""
+    from spikingjelly_amd.activation_based.layer import fused
+
+    block = _make_block(32, 2, 91).cuda().train()
+    results, real = [], fused.conv_bn_lif
+
+    def recorded(*a, **k):
+        r = real(*a, **k)
+        results.append(r is not None)
+        return r
+
+    monkeypatch.setattr(fused, "conv_bn_lif", recorded)
+    x = seeded_randn((20, 2, 32, 36), 92, 0.0, 2.0).cuda().requires_grad_()
+    block(x).sum().backward()
+    assert results and results[0] and x.grad is not None and bool(torch.isfinite(x.grad).all())
 
 
 def test_eval_mode_spikes_are_bit_identical_to_the_torch_backend_on_exact_inputs():
