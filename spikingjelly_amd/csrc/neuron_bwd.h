@@ -93,7 +93,10 @@ enum BwdMode { BWD_PLAIN = 0, BWD_PLIF = 1, BWD_QIF = 2 };
 // grad_v_seq; bf16 PLIF with fp32 state at T = 8, N = 8.4 M: 124 -> 110 us; at T = 16 four rows were already 2.5 % slower
 // than eight).
 constexpr int BWD_SHORT = 4;
-constexpr int kShortRows = 2;
+#ifndef SJHIP_SHORT_ROWS
+#define SJHIP_SHORT_ROWS 2
+#endif
+constexpr int kShortRows = SJHIP_SHORT_ROWS;
 // sequences up to this length run the BWD_SHORT kernels
 #ifndef SJHIP_SHORT_SEQUENCE
 #define SJHIP_SHORT_SEQUENCE 8
