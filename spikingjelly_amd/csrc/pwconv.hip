@@ -4,9 +4,11 @@
 //   * two fp16 terms (H): x is scaled by a power of two, hi = fp16(x), lo = fp16(x - hi); hi + lo holds x to 2^-23 or
 //     better, and hi*hi + hi*lo + lo*hi (three v_mfma_f32_32x32x16_f16 products, fp32 accumulation) drops only lo*lo,
 //     below 2^-22 of the product.  The scale keeps the terms inside fp16's exponent range: per row of A for the weights
-//     (split_weight_f16_kernel, taken out per row of the result), per tensor for activations and gradients (the power
-//     of two that takes the largest magnitude into [2^14, 2^15); amax_kernel or the producer of the tensor finds that
-//     magnitude, the kernels read it from a small device buffer).  Measured: 2^-23 of sum |a||b| against float64.
+//     (split_weight_f16_kernel, taken out per row of the result); for activations and gradients the power of two that
+//     takes a largest magnitude into [2^14, 2^15): that of the sample in pw_gemm_kernel, whose columns are (sample,
+//     position) pairs, that of the whole tensor in the weight gradient, which sums over samples (amax_kernel or the
+//     producer of the tensor finds both, the kernels read them from a small device buffer).  Measured: 2^-23 of
+//     sum |a||b| against float64.
 //   * up to three bf16 terms: no scaling (bf16 has fp32's exponent range), six products for fp32 accuracy; described
 //     next, and what the measurements below were taken with unless they say otherwise.  The fp16 split runs the qkv
 //     shape in 0.19 ms (forward / input gradient) and 0.24 ms (weight gradient) against 0.27 and 0.30 ms.
@@ -326,7 +328,13 @@ struct PwGemmArgs {
   const uint16_t *b_planes;  // kBPlanes: fp16 terms of b, [TB][K][ld], column s * L + l of row k holds b[s][k][l]
   int64_t b_plane_stride;    // K * ld
   int ld;                    // columns per row of a plane: a multiple of 8, at least ncols
+  int wide_out;              // L is a multiple of 4 and c is 16-byte aligned: the tile leaves through LDS as 16-byte row pieces
 };
+#ifndef SJHIP_PW_WIDE_OUT
+#define SJHIP_PW_WIDE_OUT 1
+#endif
+constexpr int kOutPitch = 68;                              // floats per row of the output staging buffer (64 columns + 4)
+constexpr unsigned kOutLds = 4 * 32 * kOutPitch * 4;       // 32 rows x 64 columns per wavefront
 constexpr int kStatPitch = 33;                             // floats per row of the transposing buffer: no bank conflicts
 constexpr unsigned kStatLds = 4 * 64 * kStatPitch * 4;     // one buffer of 64 rows x 32 column pairs per wavefront
 
@@ -622,23 +630,74 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
         for (int nt = 0; nt < 2; ++nt) acc[mt][nt][r] = acc[mt][nt][r] * inv * b_inv_col[nt];
       }
   }
-#pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
-    const int64_t j = j0 + wn * 64 + nt * 32 + (lane & 31);
-    if (j >= a.ncols) continue;
-    const int64_t s = j / L;
-    const int l = (int)(j - s * L);
-    float *cp = a.c + (s * M) * (int64_t)L + l;
+  if (a.wide_out) {
+    // The accumulators hold four rows of one column per group of registers, so a direct store writes 4-byte pieces of
+    // 128-byte row segments, 64 instructions per wavefront.  Through LDS a wavefront's 64 x 64 tile leaves in two halves
+    // of 32 rows as 16-byte pieces: a store instruction writes four rows of 256 contiguous bytes, 16 per wavefront.  A
+    // piece of four columns lies in one sample (L is a multiple of 4).
+    float *buf = reinterpret_cast<float *>(lds) + wave * (32 * kOutPitch);
+    const int c4 = 4 * (lane & 15), rsub = lane >> 4;
+    const int64_t j4 = j0 + wn * 64 + c4;
+    const bool ok4 = j4 < a.ncols;
+    const int64_t s4 = ok4 ? j4 / L : 0;
+    float *cp4 = a.c + (s4 * M) * (int64_t)L + (ok4 ? (int)(j4 - s4 * L) : 0);
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
-      const int rbase = m0 + wm * 64 + mt * 32 + 4 * (lane >> 5);
+      __syncthreads();  // the operand tiles (first half) or the rows of the first half (second) are no longer read
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = rbase + 8 * (r >> 2) + (r & 3);
-        if (row < M) cp[(int64_t)row * L] = acc[mt][nt][r];
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          buf[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * kOutPitch + nt * 32 + (lane & 31)] = acc[mt][nt][r];
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int row_local = 4 * i + rsub;
+        const int row = m0 + wm * 64 + mt * 32 + row_local;
+        const f32x4 v = *reinterpret_cast<const f32x4 *>(buf + row_local * kOutPitch + c4);
+        if (ok4 && row < M) *reinterpret_cast<f32x4 *>(cp4 + (int64_t)row * L) = v;
+      }
+      // the batch-norm sums of these 32 rows over the wavefront's 64 columns (columns beyond the matrix hold exact
+      // zeros): lane i adds row i from the staged half, in a fixed order
+      if (a.stats && lane < 32) {
+        const float *rowp = buf + lane * kOutPitch;
+        float sum = 0.0f, squares = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const f32x4 v = *reinterpret_cast<const f32x4 *>(rowp + 4 * j);
+          sum += (v.x + v.y) + (v.z + v.w);
+          squares = fmaf(v.x, v.x, squares); squares = fmaf(v.y, v.y, squares);
+          squares = fmaf(v.z, v.z, squares); squares = fmaf(v.w, v.w, squares);
+        }
+        const int row = m0 + wm * 64 + mt * 32 + lane;
+        if (row < M) {
+          float *out = a.stats + ((2 * nb + wn) * (int64_t)M + row) * 2;
+          out[0] = sum;
+          out[1] = squares;
+        }
       }
     }
-  }
+    return;
+  } else {
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int64_t j = j0 + wn * 64 + nt * 32 + (lane & 31);
+      if (j >= a.ncols) continue;
+      const int64_t s = j / L;
+      const int l = (int)(j - s * L);
+      float *cp = a.c + (s * M) * (int64_t)L + l;
+  #pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        const int rbase = m0 + wm * 64 + mt * 32 + 4 * (lane >> 5);
+  #pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = rbase + 8 * (r >> 2) + (r & 3);
+          if (row < M) cp[(int64_t)row * L] = acc[mt][nt][r];
+        }
+      }
+    }
+  
+}
 
   // Batch-norm statistics of the tile, so that no kernel has to read c again for them: per row the sum and the sum of
   // squares over the wavefront's 64 columns (columns beyond the matrix hold exact zeros).  A lane holds 32 rows of one
@@ -1134,6 +1193,7 @@ template <int TA, int TB, bool H = false, int BSRC = kBFloat>
 int launch_gemm_terms(const PwGemmArgs &a, int64_t blocks, hipStream_t stream) {
   unsigned lds = (TA + TB) * kRowPlane;
   if (a.stats && lds < kStatLds) lds = kStatLds;
+  if (a.wide_out && lds < kOutLds) lds = kOutLds;
   hipLaunchKernelGGL((pw_gemm_kernel<TA, TB, H, BSRC>), dim3((unsigned)blocks), dim3(kPwThreads), lds, stream, a);
   return check_launch("pwconv_gemm");
 }
@@ -1236,6 +1296,7 @@ int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t
     a.b_amax_samples = b_amax ? b_amax + SJHIP_PW_AMAX_FLOATS : nullptr;
     a.amax_s0 = s0; a.amax_S = S;
     a.b_planes = nullptr; a.b_plane_stride = 0; a.ld = 0;
+    a.wide_out = (SJHIP_PW_WIDE_OUT != 0 && L % 4 == 0 && aligned16(c)) ? 1 : 0;
     if (stats) stats += 2 * ((a.ncols + kTile - 1) / kTile) * M * 2;
     const int64_t blocks = a.m_blocks * ((a.ncols + kTile - 1) / kTile);
     if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: %lld blocks", (long long)blocks);
@@ -1365,6 +1426,7 @@ int launch_pwconv_gemm_planes(const uint16_t *a_planes, int64_t M, int64_t K, co
   a.b_amax = b_terms == 2 ? b_amax : nullptr;
   a.b_amax_samples = nullptr; a.amax_s0 = 0; a.amax_S = 0;
   a.b_planes = b_planes; a.b_plane_stride = K * ld; a.ld = (int)ld;
+  a.wide_out = (SJHIP_PW_WIDE_OUT != 0 && L % 4 == 0 && aligned16(c)) ? 1 : 0;
   const int64_t blocks = a.m_blocks * ((a.ncols + kTile - 1) / kTile);
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm_planes: %lld blocks", (long long)blocks);
   ProfileScope prof(KC_PW_GEMM, stream);
