@@ -334,16 +334,17 @@ inline bool resonant_bit_20(int64_t bytes) { return ((bytes >> 20) & 1) != 0; }
 constexpr int kColumnRun = 256;
 // The `spread` argument of column_block() for T rows of `row_bytes`: 0 the default order, 1 contiguous eighths, larger
 // values runs of that many blocks.  Tuning key "column_spread": 0 and 1 force those orders, 4 and more force runs of
-// that many blocks, 2 (default) chooses: contiguous eighths for small tensors (rows of at most 16 MiB, or T rows of at
-// most 256 MiB together), runs of kColumnRun blocks for the resonant strides, the default order otherwise.
-// Measured (forward / backward, us; default order -> eighths): fp32 [16, 2^22] 165 / 214 -> 163 / 177, fp32 [8, 2^23]
-// 167 / 198 -> 161 / 180, bf16 [8, 2^23] 73 / 108 -> 65 / 102, fp16 [32, 6.4 M] inference 153 -> 145; larger tensors the
-// other way: fp32 [16, 2^23] 292 / 370 -> 316 / 369, fp32 [16, 2^24] 579 / 702 -> 626 / 739, fp32 [4, 2^25] 318 / 352 ->
-// 331 / 369.
+// that many blocks, 2 (default) chooses: contiguous eighths for small tensors whose rows are a multiple of 256 KiB apart
+// (at least four rows of at most 256 MiB together), runs of kColumnRun blocks for the resonant strides, the default
+// order otherwise.  Measured (forward / backward, us; default order -> eighths): fp32 [16, 2^22] 165 / 214 -> 163 / 177,
+// fp32 [16, 2^21] 99 / 109 -> 87 / 90, fp32 [8, 2^23] 167 / 198 -> 161 / 180, bf16 [8, 2^23] 73 / 108 -> 65 / 102, bf16 [4, 2^24]
+// 83 / 94 -> 66 / 91, fp16 [32, 49 * 2^17] inference 153 -> 145.  The other way: larger tensors (fp32 [16, 2^23] 292 / 370 ->
+// 316 / 369, [16, 2^24] 579 / 702 -> 626 / 739, [4, 2^25] 318 / 352 -> 331 / 369), rows that are not such a multiple apart (fp32
+// [16, 147 * 2^15] 182 / 228 -> 228 / 245, [4, 147 * 2^15] 51 / 52 -> 55 / 58) and single rows (fp32 [1, 2^24] 45 -> 53).
 inline int column_spread(int64_t row_bytes, int64_t T) {
   const int mode = tuning().column_spread;
   if (mode != 2) return mode;
-  if (row_bytes <= (int64_t(16) << 20) || T * row_bytes <= (int64_t(256) << 20)) return 1;
+  if ((row_bytes & ((int64_t(1) << 18) - 1)) == 0 && T >= 4 && T * row_bytes <= (int64_t(256) << 20)) return 1;
   return resonant_row_stride(row_bytes) ? kColumnRun : 0;
 }
 // work-items per block that go with column_spread() when it chose the order by itself
