@@ -36,7 +36,9 @@ def C():
 # ------------------------------------------------------------------------------------------------
 # the three GEMMs
 # ------------------------------------------------------------------------------------------------
-SHAPES = [(3, 100, 50, 12), (2, 128, 32, 128), (5, 384, 384, 196), (1, 7, 3, 4), (4, 130, 257, 36), (16, 1152, 384, 196)]
+# (token counts that are a multiple of 4 leave through the 16-byte epilogue, the others, which must be even, element by element)
+SHAPES = [(3, 100, 50, 12), (2, 128, 32, 128), (5, 384, 384, 196), (1, 7, 3, 4), (4, 130, 257, 36), (16, 1152, 384, 196),
+          (3, 70, 33, 6), (5, 200, 64, 198)]
 
 
 @pytest.mark.parametrize("S,M,Kd,Lp", SHAPES)
@@ -68,7 +70,8 @@ def test_gemm_is_exact_on_spikes_times_dyadic_weights(C, S, M, Kd, Lp):
         assert torch.equal(got, want), (wt, xt)
 
 
-@pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (1, 7, 3, 4), (4, 130, 257, 36), (16, 1152, 384, 196), (5, 384, 384, 196)])
+@pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (1, 7, 3, 4), (4, 130, 257, 36), (16, 1152, 384, 196), (5, 384, 384, 196), (3, 70, 33, 6),
+                                       (5, 200, 64, 198)])
 @pytest.mark.parametrize("terms", [(3, 3), (3, 1), (1, 1)])
 def test_gemm_leaves_the_batch_norm_sums_of_its_output(C, S, M, Kd, Lp, terms):
     """``pw_gemm(..., stats=True)``: the output is the one of the plain call bit for bit, and the partial sums add up to
@@ -91,6 +94,8 @@ def test_gemm_leaves_the_batch_norm_sums_of_its_output(C, S, M, Kd, Lp, terms):
     abs_s = y.abs().sum((0, 2)).cpu().clamp_min(1e-30)
     assert float(((sums[:, 0] - want_s).abs() / abs_s).max()) < 1e-6
     assert float(((sums[:, 1] - want_q).abs() / want_q.clamp_min(1e-30)).max()) < 1e-6
+    if Lp % 4 != 0:
+        return  # (the pass over y of the batch-norm kernels takes rows of whole quads only)
     # the affine map from these sums against the one from the pass over y
     gamma, beta = seeded_randn((M,), 33, 1.0, 0.2).cuda(), seeded_randn((M,), 34, 0.0, 0.2).cuda()
     a = C._bn_map(got, gamma, beta, None, None, True, 0.1, 1e-5)
@@ -323,7 +328,7 @@ def test_amax_per_sample(C, S, per_sample, offset):
         assert torch.equal(C.sample_amax(C.amax(xd)), C.sample_amax(words))
 
 
-@pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (1, 7, 3, 4), (4, 130, 257, 36), (16, 1152, 384, 196)])
+@pytest.mark.parametrize("S,M,Kd,Lp", [(3, 100, 50, 12), (1, 7, 3, 4), (4, 130, 257, 36), (16, 1152, 384, 196), (3, 70, 33, 6), (5, 200, 64, 198)])
 @pytest.mark.parametrize("spikes", [False, True])
 def test_fp16_gemm_leaves_the_batch_norm_sums_of_its_output(C, S, M, Kd, Lp, spikes):
     F = C.F16 | 2
