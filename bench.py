@@ -125,6 +125,25 @@ def measure_ceilings(torch, L, floats_per_stream: int, repeats: int = 5):
     return out
 
 
+class _quiet_collector:
+    """Python's cyclic garbage collector off for a timed region (as ``timeit`` does): with torch imported a full
+    collection takes 70-80 ms of host time, and whether one falls among twenty timed steps depends on how many objects
+    the process happened to allocate before (measured: 0.29 against 4.4 ms per step for the same 20 steps of configs[2])."""
+
+    def __enter__(self):
+        import gc
+
+        gc.collect()
+        self.was_enabled = gc.isenabled()
+        gc.disable()
+
+    def __exit__(self, *exc):
+        import gc
+
+        if self.was_enabled:
+            gc.enable()
+
+
 def _time_steps(torch, L, step, steps, warmup):
     """warm-up, then `steps` timed steps bracketed by synchronisation, then the same steps once more under the library's
     event profiler for the per-kernel durations: its two events per launch would otherwise sit in the timed region of
@@ -132,11 +151,12 @@ def _time_steps(torch, L, step, steps, warmup):
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    with _quiet_collector():
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
     L.profile_reset()
     L.profile_enable(True)
     for _ in range(steps):
@@ -172,7 +192,7 @@ def secondary_measurements(args):
     out = {}
     for name in ("config3", "config4", "config5"):
         sub = copy.copy(args)
-        sub.workload, sub.steps, sub.warmup, sub.collect = name, 10, 3, []
+        sub.workload, sub.steps, sub.warmup, sub.collect = name, 20, 5, []
         other_workload(sub)
         line = sub.collect[0]
         r = line["roofline"]
@@ -620,13 +640,14 @@ def main() -> int:
     L.profile_enable(True)
     torch.cuda.synchronize()
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        marks[i].record()  # on the stream the kernels are launched on
-        spikes = step()
-    marks[-1].record()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    with _quiet_collector():
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            marks[i].record()  # on the stream the kernels are launched on
+            spikes = step()
+        marks[-1].record()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
     L.profile_enable(False)
     per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
     quantile = lambda q: per_step[min(len(per_step) - 1, int(q * len(per_step)))]
