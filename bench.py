@@ -199,7 +199,7 @@ def secondary_measurements(args):
         out[name] = {"metric": line["metric"], "value": line["value"], "unit": line["unit"], "ms_per_step": line["ms_per_step"],
                      "kernel": r["kernel"], "kernel_ms": r["kernel_ms"], "bound": r["bound"], "achieved": r["achieved"],
                      "peak": r["peak"], "roofline_unit": r["unit"], "frac": r["frac"]}
-        for extra in ("forward_ms", "backward_ms", "fused_forward_packed_ms", "fused_forward_packed_GBs", "gemm_ms_per_step",
+        for extra in ("forward_ms", "backward_ms", "graph_replay_ms_per_step", "fused_forward_packed_ms", "fused_forward_packed_GBs", "gemm_ms_per_step",
                       "ssa_backward_ms", "ssa_backward_GBs"):
             if extra in r:
                 out[name][extra] = r[extra]
@@ -241,6 +241,32 @@ def other_workload(args) -> int:
 
         elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
         f_ms, b_ms = _kernel_ms(L, L.KC_FORWARD), _kernel_ms(L, L.KC_BACKWARD)
+        plif_reduce_ms = _kernel_ms(L, L.KC_PLIF_REDUCE)
+        # The same step recorded into a HIP graph and replayed: at this size the Python around the launches (0.2-0.3 ms
+        # per step) is longer than the kernels (0.17 ms), and a replay issues them without it.  (Replays of the recorded
+        # step on its static input; a caller with new data per step adds the copy into that buffer.)
+        from spikingjelly_amd.activation_based.hip_kernel.graph import GraphedStep
+
+        eager_spikes = node(x).detach().clone()
+        functional.reset_net(node)
+
+        def recorded(xs):
+            s = node(xs)
+            torch.autograd.backward([s, node.v_seq], [gs, gv])
+            functional.reset_net(node)
+            return s
+
+        graphed = GraphedStep(recorded, [x], parameters=[node.w])
+        for _ in range(args.warmup):
+            graphed.graph.replay()
+        torch.cuda.synchronize()
+        with _quiet_collector():
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                graphed.graph.replay()
+            torch.cuda.synchronize()
+            graph_elapsed = time.perf_counter() - t0
+        assert torch.equal(graphed.static_outputs.detach(), eager_spikes)
         bytes_each = 8 * T * N + 2 * N  # 4 tensors x 2 B per step + one [N] state
         dom = "forward" if f_ms >= b_ms else "backward"
         d_ms = max(f_ms, b_ms)
@@ -251,7 +277,8 @@ def other_workload(args) -> int:
               {"bound": "hbm", "achieved": bytes_each / (d_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                "frac": bytes_each / (d_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": dom,
                "kernel_ms": d_ms, "algorithmic_bytes": bytes_each, "forward_ms": f_ms, "backward_ms": b_ms,
-               "plif_reduce_ms": _kernel_ms(L, L.KC_PLIF_REDUCE)})
+               "plif_reduce_ms": plif_reduce_ms, "graph_replay_ms_per_step": graph_elapsed / args.steps * 1e3,
+               "graph_replay_neuron_steps_per_s": T * N / (graph_elapsed / args.steps)})
         return 0
 
     if args.workload in ("qif", "ilif", "eif", "izhikevich"):
