@@ -149,14 +149,28 @@ def test_a_call_on_another_stream_is_refused_while_the_array_is_in_use(L):
 
     # every buffer exists before the first launch: nothing between the launches below waits for the device
     big_out, same_out, other_out, out = buffers(c), buffers(small), buffers(small), buffers(small)
-    torch.cuda.synchronize()
-    for _ in range(20):   # some fifteen milliseconds of work on the first stream
-        assert call(c, big_out, c["stream"]) == 0
-    rc_same = call(small, same_out, c["stream"])          # same stream: ordered behind the calls before
-    rc_other = call(small, other_out, other.cuda_stream)  # another stream while the first one still works
-    message = lib.sjhip_last_error()
-    torch.cuda.synchronize()
-    assert rc_same == 0
+    import gc
+
+    main = torch.cuda.current_stream()
+    for calls in (20, 80, 320):   # some fifteen milliseconds of work on the first stream, more if the host was held up
+        torch.cuda.synchronize()
+        gc.collect()
+        gc.disable()   # (a full collection takes longer than the queued work)
+        try:
+            for _ in range(calls):
+                assert call(c, big_out, c["stream"]) == 0
+            rc_same = call(small, same_out, c["stream"])          # same stream: ordered behind the calls before
+            rc_other = call(small, other_out, other.cuda_stream)  # another stream while the first one still works
+            message = lib.sjhip_last_error()
+            still_busy = not main.query()
+        finally:
+            gc.enable()
+        torch.cuda.synchronize()
+        assert rc_same == 0
+        if still_busy:   # the premise held: the first stream was still working after the call on the other one returned
+            break
+    else:
+        pytest.fail("the first stream finished 320 backward calls before the host could issue the next call")
     assert rc_other == -1 and b"another stream" in message
     assert call(small, out, other.cuda_stream) == 0       # everything has finished: the other stream may use the array
     torch.cuda.synchronize()
