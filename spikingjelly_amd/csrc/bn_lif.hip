@@ -165,7 +165,9 @@ __device__ __forceinline__ void bn_lif_forward_body(const BnLifFwdArgs &a) {
   const int64_t N = f.N, T = f.T;
   const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (col >= N) return;
-  const int c = (int)((col / a.L) % a.C);
+  // (32-bit quotients where the tensor allows it: a 64-bit integer division is some hundred instructions, as many as
+  // the four steps of a short sequence)
+  const int c = N <= 0x7fffffffLL ? (int)(((uint32_t)col / (uint32_t)a.L) % (uint32_t)a.C) : (int)((col / a.L) % a.C);
   const float sc = a.scale[c], sh = a.shift[c];
   const float *yp = (const float *)f.x + col;
   float *sp = (float *)f.spike + col;
@@ -446,10 +448,16 @@ __global__ void __launch_bounds__(256) bn_grad_input_kernel(const float *g, cons
   float amax = 0.0f;
   int sample = -1;
   if (i < n) {
-    const int64_t row = i / L;  // sample * C + channel
-    const int64_t smp = row / C;
-    const int c = (int)(row - smp * C);
-    sample = (int)smp;
+    int c;  // i = ((sample * C) + channel) * L + position
+    if (n <= 0x7fffffffLL) {
+      const uint32_t row = (uint32_t)i / (uint32_t)L, smp = row / (uint32_t)C;
+      c = (int)(row - smp * (uint32_t)C);
+      sample = (int)smp;
+    } else {
+      const int64_t row = i / L, smp = row / C;
+      c = (int)(row - smp * C);
+      sample = (int)smp;
+    }
     const float p = coef[c], q = coef[C + c], r = coef[2 * C + c];
     const f32x4 gv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(g + i));
     const f32x4 yv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(y + i));
