@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define SJHIP_ABI_VERSION 5
+#define SJHIP_ABI_VERSION 6
 
 typedef enum sjhip_status {
   SJHIP_OK = 0,
@@ -632,6 +632,19 @@ int sjhip_bn_lif_forward(int neuron, const sjhip_neuron_params *p, int64_t T, in
 int sjhip_bn_lif_backward(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
                           const float *scale, const float *shift, const float *v_init, const float *grad_spike_seq,
                           const float *grad_v_last, float *grad_z, float *grad_v_init, float *partial, void *stream);
+/* The same two calls with a ParametricLIFNode behind the batch norm (neuron/plif.py:14-261 in the place of the LIF of
+ * layer/attention.py:310-329): k = sigmoid(w) is read from device memory (k_device, one float, as sjhip_neuron_forward
+ * takes it), and the backward also leaves dL/dk in grad_k[0]: every wavefront writes its share of sum G_t dh_t/dk to
+ * workspace (sjhip_bn_plif_backward_workspace_floats(B, C, L) floats), and one more launch adds the shares in fp64 in a
+ * fixed order, as sjhip_neuron_backward does for PLIF.  params: as for SJHIP_NEURON_PLIF (tau is ignored). */
+int sjhip_bn_plif_forward(const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
+                          const float *scale, const float *shift, const float *v_init, const float *k_device, float *spike_seq,
+                          uint8_t *spike_bits, float *v_last, void *stream);
+int64_t sjhip_bn_plif_backward_workspace_floats(int64_t B, int64_t C, int64_t L);
+int sjhip_bn_plif_backward(const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
+                           const float *scale, const float *shift, const float *v_init, const float *k_device,
+                           const float *grad_spike_seq, const float *grad_v_last, float *grad_z, float *grad_v_init,
+                           float *partial, float *grad_k, float *workspace, void *stream);
 int sjhip_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64_t C, int64_t L, int training, const float *gamma,
                                const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef, float *amax_reset,
                                void *stream);

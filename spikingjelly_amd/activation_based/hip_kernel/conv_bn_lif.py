@@ -296,8 +296,10 @@ def _lif_params(spec, flags_extra: int = 0) -> L.NeuronParams:
     return K._params(tau, v_th, v_reset, sg_alpha, sg_id, flags | flags_extra)
 
 
-def _bn_lif_forward(y: torch.Tensor, bn_map: torch.Tensor, v_init: torch.Tensor, spec, packed: bool):
-    """``y [T, B, C, L]`` -> (spikes ``[T, B, C, L]`` fp32 or the bit-packed byte array, ``v_last [B, C, L]``)."""
+def _bn_lif_forward(y: torch.Tensor, bn_map: torch.Tensor, v_init: torch.Tensor, spec, packed: bool,
+                    k: Optional[torch.Tensor] = None):
+    """``y [T, B, C, L]`` -> (spikes ``[T, B, C, L]`` fp32 or the bit-packed byte array, ``v_last [B, C, L]``).
+    ``k``: one fp32 element on the device, ``sigmoid(w)`` of a parametric LIF (``spec[0]`` is then unused)."""
     T, B, C, Lp = y.shape
     v_keep, broadcast = K._state_arg(v_init, True)
     params = _lif_params(spec, broadcast)
@@ -306,19 +308,27 @@ def _bn_lif_forward(y: torch.Tensor, bn_map: torch.Tensor, v_init: torch.Tensor,
         spikes = torch.empty((T * B * C * Lp // 8,), dtype=torch.uint8, device=y.device)
     else:
         spikes = torch.empty_like(y)
+    k_keep, k_ptr = K._k_pointer(k, y)
     with torch.cuda.device(y.device):
-        rc = L.load().sjhip_bn_lif_forward(L.NEURON_LIF, ctypes.byref(params), T, B, C, Lp, y.data_ptr(), bn_map[0].data_ptr(),
-                                           bn_map[1].data_ptr(), v_keep.data_ptr(), None if packed else spikes.data_ptr(),
-                                           spikes.data_ptr() if packed else None, v_last.data_ptr(), _stream(y))
+        if k is None:
+            rc = L.load().sjhip_bn_lif_forward(L.NEURON_LIF, ctypes.byref(params), T, B, C, Lp, y.data_ptr(), bn_map[0].data_ptr(),
+                                               bn_map[1].data_ptr(), v_keep.data_ptr(), None if packed else spikes.data_ptr(),
+                                               spikes.data_ptr() if packed else None, v_last.data_ptr(), _stream(y))
+        else:
+            rc = L.load().sjhip_bn_plif_forward(ctypes.byref(params), T, B, C, Lp, y.data_ptr(), bn_map[0].data_ptr(),
+                                                bn_map[1].data_ptr(), v_keep.data_ptr(), k_ptr,
+                                                None if packed else spikes.data_ptr(), spikes.data_ptr() if packed else None,
+                                                v_last.data_ptr(), _stream(y))
     L.check(rc, "bn_lif_forward")
     return spikes, v_last
 
 
 def _bn_lif_backward(y: torch.Tensor, bn_map: torch.Tensor, gamma, v_init: torch.Tensor, spec, batch_stats: bool,
                      grad_spikes: Optional[torch.Tensor], grad_v_last: Optional[torch.Tensor], need_grad_v_init: bool,
-                     want_amax: bool = False):
+                     want_amax: bool = False, k: Optional[torch.Tensor] = None):
     """Returns ``(dy [T, B, C, L], dgamma [C], dbeta [C], grad_v_init or None)``, and with ``want_amax`` a fifth element:
-    ``amax(dy)``, found by the kernel that writes ``dy``, when the convolution GEMMs run on fp16 terms (else None)."""
+    ``amax(dy)``, found by the kernel that writes ``dy``, when the convolution GEMMs run on fp16 terms (else None).
+    With ``k`` (parametric LIF) one more element follows: ``dL/dk``, one fp32 element."""
     T, B, C, Lp = y.shape
     lib = L.load()
     if grad_spikes is None:
@@ -334,9 +344,19 @@ def _bn_lif_backward(y: torch.Tensor, bn_map: torch.Tensor, gamma, v_init: torch
     grad_v_init = torch.empty((B, C, Lp), dtype=torch.float32, device=y.device) if need_grad_v_init else None
     with torch.cuda.device(y.device):
         stream = _stream(y)
-        L.check(lib.sjhip_bn_lif_backward(L.NEURON_LIF, ctypes.byref(params), T, B, C, Lp, y.data_ptr(), bn_map[0].data_ptr(),
-                                          bn_map[1].data_ptr(), v_keep.data_ptr(), grad_spikes.data_ptr(), L.ptr(grad_v_last),
-                                          g.data_ptr(), L.ptr(grad_v_init), partial.data_ptr(), stream), "bn_lif_backward")
+        grad_k = None
+        if k is None:
+            L.check(lib.sjhip_bn_lif_backward(L.NEURON_LIF, ctypes.byref(params), T, B, C, Lp, y.data_ptr(), bn_map[0].data_ptr(),
+                                              bn_map[1].data_ptr(), v_keep.data_ptr(), grad_spikes.data_ptr(), L.ptr(grad_v_last),
+                                              g.data_ptr(), L.ptr(grad_v_init), partial.data_ptr(), stream), "bn_lif_backward")
+        else:
+            k_keep, k_ptr = K._k_pointer(k, y)
+            grad_k = torch.empty((1,), dtype=torch.float32, device=y.device)
+            shares = torch.empty((lib.sjhip_bn_plif_backward_workspace_floats(B, C, Lp),), dtype=torch.float32, device=y.device)
+            L.check(lib.sjhip_bn_plif_backward(ctypes.byref(params), T, B, C, Lp, y.data_ptr(), bn_map[0].data_ptr(),
+                                               bn_map[1].data_ptr(), v_keep.data_ptr(), k_ptr, grad_spikes.data_ptr(),
+                                               L.ptr(grad_v_last), g.data_ptr(), L.ptr(grad_v_init), partial.data_ptr(),
+                                               grad_k.data_ptr(), shares.data_ptr(), stream), "bn_plif_backward")
         dy_amax = None
         if want_amax and _terms() & F16:  # (cleared by the launch that makes the coefficients, filled by the next one)
             dy_amax = torch.empty((amax_floats(T * B),), dtype=torch.float32, device=y.device)
@@ -350,9 +370,8 @@ def _bn_lif_backward(y: torch.Tensor, bn_map: torch.Tensor, gamma, v_init: torch
         else:
             L.check(lib.sjhip_bn_grad_input(g.data_ptr(), y.data_ptr(), grads[2].data_ptr(), T * B, C, Lp, g.data_ptr(), stream),
                     "bn_grad_input")
-    if want_amax:
-        return g, grads[0], grads[1], grad_v_init, dy_amax
-    return g, grads[0], grads[1], grad_v_init
+    out = (g, grads[0], grads[1], grad_v_init, dy_amax) if want_amax else (g, grads[0], grads[1], grad_v_init)
+    return out if k is None else (*out, grad_k)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -433,9 +452,10 @@ def _side_stream(device: torch.device) -> "torch.cuda.Stream":
 
 
 def _conv_chain_backward(x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax, spec, batch_stats: bool, x_exact: bool, ssa,
-                         grad_out, grad_v_last, need_dx: bool, need_dw: bool, need_gvi: bool):
+                         grad_out, grad_v_last, need_dx: bool, need_dw: bool, need_gvi: bool, k=None):
     """Backward of convolution -> batch norm -> LIF (-> contraction on the bit-packed spikes when ``ssa = (heads,
-    channels per head, scale)``): ``(dx, dw, dgamma, dbeta, grad_v_init)``, ``None`` where not needed."""
+    channels per head, scale)``): ``(dx, dw, dgamma, dbeta, grad_v_init)``, ``None`` where not needed; with ``k``
+    (parametric LIF) a sixth element, ``dL/dk``."""
     grad_spikes = grad_out
     if ssa is not None and grad_out is not None:
         from . import attention_kernel as A
@@ -443,22 +463,23 @@ def _conv_chain_backward(x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax, 
         heads, cph, scale = ssa
         T, B, _, Lp = x_seq.shape
         grad_spikes = A._ssa_packed(bits, grad_out, torch.float32, T * B, heads, cph, Lp, scale).view(y.shape)
-    dy, dgamma, dbeta, gvi, dy_amax = _bn_lif_backward(y, bn_map, gamma, v_init, spec, batch_stats, grad_spikes, grad_v_last,
-                                                        need_gvi, True)
+    dy, dgamma, dbeta, gvi, dy_amax, *grad_k = _bn_lif_backward(y, bn_map, gamma, v_init, spec, batch_stats, grad_spikes,
+                                                                 grad_v_last, need_gvi, True, k)
     dx, dw = _conv_backward(dy, x_seq, weight, x_exact, need_dx, need_dw, dy_amax, x_amax)
-    return dx, dw, dgamma, dbeta, gvi
+    return (dx, dw, dgamma, dbeta, gvi, *grad_k)
 
 
 def _lif_conv_chain_backward(pre_seq, pre_v_init, weight, gamma, v_init, y, bn_map, bits, pre_spec, spec, batch_stats: bool,
                              grad_spikes, grad_v_last, grad_pre_v_last, need_gx: bool, need_gpv: bool, need_dw: bool,
-                             need_gvi: bool):
+                             need_gvi: bool, k=None):
     """Backward of LIF -> convolution -> batch norm -> LIF with the first neuron's spikes as bits:
-    ``(grad of the first neuron's input, of its state, dw, dgamma, dbeta, grad_v_init)``."""
+    ``(grad of the first neuron's input, of its state, dw, dgamma, dbeta, grad_v_init)``; with ``k`` (the second neuron
+    is a parametric LIF) a seventh element, ``dL/dk``."""
     T, B, Cin, Lp = pre_seq.shape
     Cout = weight.shape[0]
     terms = _terms()
-    dy, dgamma, dbeta, gvi, dy_amax = _bn_lif_backward(y, bn_map, gamma, v_init, spec, batch_stats, grad_spikes, grad_v_last,
-                                                        need_gvi, True)
+    dy, dgamma, dbeta, gvi, dy_amax, *grad_k = _bn_lif_backward(y, bn_map, gamma, v_init, spec, batch_stats, grad_spikes,
+                                                                 grad_v_last, need_gvi, True, k)
     dy3 = dy.view(T * B, Cout, Lp)
     if dy_amax is None:
         dy_amax = amax(dy3)
@@ -472,61 +493,63 @@ def _lif_conv_chain_backward(pre_seq, pre_v_init, weight, gamma, v_init, y, bn_m
                                      pre_v_init.flatten(), None, tau, v_th, v_reset, flags, sg_id, sg_alpha, need_gpv)
         gx = gx.view(pre_seq.shape) if need_gx else None
         gpv = gpv.view(B, Cin, Lp) if need_gpv else None
-    return gx, gpv, dw, dgamma, dbeta, gvi
+    return (gx, gpv, dw, dgamma, dbeta, gvi, *grad_k)
 
 
 class _BnLif(torch.autograd.Function):
     @staticmethod
-    def forward(y, gamma, beta, v_init, bn, spec):
+    def forward(y, gamma, beta, v_init, bn, spec, k=None):
         running_mean, running_var, batch_stats, momentum, eps, tracked = _bn_config(bn)
         y = L.aligned16(y)
         bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, None, tracked)
-        spikes, v_last = _bn_lif_forward(y, bn_map, v_init, spec, False)
+        spikes, v_last = _bn_lif_forward(y, bn_map, v_init, spec, False, k)
         return spikes, v_last, bn_map
 
     @staticmethod
     def setup_context(ctx, inputs, output):
-        y, gamma, beta, v_init, bn, spec = inputs
+        y, gamma, beta, v_init, bn, spec, k = inputs
         ctx.spec, ctx.batch_stats = spec, bn[2]
-        ctx.save_for_backward(L.aligned16(y), gamma, v_init, output[2])
+        ctx.save_for_backward(L.aligned16(y), gamma, v_init, output[2], k)
         ctx.mark_non_differentiable(output[2])
         ctx.set_materialize_grads(False)
 
     @staticmethod
     def backward(ctx, grad_spikes, grad_v_last, _):
-        y, gamma, v_init, bn_map = ctx.saved_tensors
+        y, gamma, v_init, bn_map, k = ctx.saved_tensors
         need = ctx.needs_input_grad
-        dy, dgamma, dbeta, gvi = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
-                                                  grad_v_last, bool(need[3]))
-        return (dy if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None, gvi, None, None)
+        dy, dgamma, dbeta, gvi, *grad_k = _bn_lif_backward(y, bn_map, gamma, v_init, ctx.spec, ctx.batch_stats, grad_spikes,
+                                                           grad_v_last, bool(need[3]), False, k)
+        return (dy if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None, gvi, None, None,
+                grad_k[0] if grad_k and need[6] else None)
 
 
 class _ConvBnLif(torch.autograd.Function):
     @staticmethod
-    def forward(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact):
+    def forward(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, k=None):
         running_mean, running_var, batch_stats, momentum, eps, tracked = _bn_config(bn)
         x_seq = L.aligned16(x_seq)
         y, partial, x_amax = _conv_forward(x_seq, weight, x_exact, batch_stats)
         bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial, tracked)
-        spikes, v_last = _bn_lif_forward(y, bn_map, v_init, spec, False)
+        spikes, v_last = _bn_lif_forward(y, bn_map, v_init, spec, False, k)
         return spikes, v_last, y, bn_map, x_amax
 
     @staticmethod
     def setup_context(ctx, inputs, output):
-        x_seq, weight, gamma, beta, v_init, bn, spec, x_exact = inputs
+        x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, k = inputs
         ctx.spec, ctx.batch_stats, ctx.x_exact = spec, bn[2], x_exact
-        ctx.save_for_backward(L.aligned16(x_seq), weight, gamma, v_init, output[2], output[3], output[4])
+        ctx.save_for_backward(L.aligned16(x_seq), weight, gamma, v_init, output[2], output[3], output[4], k)
         ctx.mark_non_differentiable(output[2], output[3], output[4])
         ctx.set_materialize_grads(False)
 
     @staticmethod
     def backward(ctx, grad_spikes, grad_v_last, _y, _map, _amax):
-        x_seq, weight, gamma, v_init, y, bn_map, x_amax = ctx.saved_tensors
+        x_seq, weight, gamma, v_init, y, bn_map, x_amax, k = ctx.saved_tensors
         need = ctx.needs_input_grad
-        dx, dw, dgamma, dbeta, gvi = _conv_chain_backward(x_seq, weight, gamma, v_init, y, bn_map, None, x_amax, ctx.spec,
-                                                          ctx.batch_stats, ctx.x_exact, None, grad_spikes, grad_v_last,
-                                                          bool(need[0]), bool(need[1]), bool(need[4]))
-        return (dx, dw, dgamma if need[2] else None, dbeta if need[3] else None, gvi, None, None, None)
+        dx, dw, dgamma, dbeta, gvi, *grad_k = _conv_chain_backward(x_seq, weight, gamma, v_init, y, bn_map, None, x_amax,
+                                                                   ctx.spec, ctx.batch_stats, ctx.x_exact, None, grad_spikes,
+                                                                   grad_v_last, bool(need[0]), bool(need[1]), bool(need[4]), k)
+        return (dx, dw, dgamma if need[2] else None, dbeta if need[3] else None, gvi, None, None, None,
+                grad_k[0] if grad_k and need[8] else None)
 
 
 class _ConvBnLifSsa(torch.autograd.Function):
@@ -534,7 +557,7 @@ class _ConvBnLifSsa(torch.autograd.Function):
     contraction ``scale (V K^T) Q`` reading those bits.  Saves the input, the convolution output and the bits."""
 
     @staticmethod
-    def forward(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, ssa):
+    def forward(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, ssa, k=None):
         from . import attention_kernel as A
 
         running_mean, running_var, batch_stats, momentum, eps, tracked = _bn_config(bn)
@@ -543,15 +566,15 @@ class _ConvBnLifSsa(torch.autograd.Function):
         T, B, _, Lp = x_seq.shape
         y, partial, x_amax = _conv_forward(x_seq, weight, x_exact, batch_stats)
         bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial, tracked)
-        bits, v_last = _bn_lif_forward(y, bn_map, v_init, spec, True)
+        bits, v_last = _bn_lif_forward(y, bn_map, v_init, spec, True, k)
         out = A._ssa_packed(bits, None, torch.float32, T * B, heads, cph, Lp, scale)
         return out, v_last, y, bn_map, bits, x_amax
 
     @staticmethod
     def setup_context(ctx, inputs, output):
-        x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, ssa = inputs
+        x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, ssa, k = inputs
         ctx.spec, ctx.batch_stats, ctx.x_exact, ctx.ssa = spec, bn[2], x_exact, ssa
-        ctx.save_for_backward(L.aligned16(x_seq), weight, gamma, v_init, output[2], output[3], output[4], output[5])
+        ctx.save_for_backward(L.aligned16(x_seq), weight, gamma, v_init, output[2], output[3], output[4], output[5], k)
         ctx.mark_non_differentiable(output[2], output[3], output[4], output[5])
         ctx.set_materialize_grads(False)
 
@@ -559,12 +582,13 @@ class _ConvBnLifSsa(torch.autograd.Function):
     def backward(ctx, grad_out, grad_v_last, _y, _map, _bits, _amax):
         from . import attention_kernel as A
 
-        x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax = ctx.saved_tensors
+        x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax, k = ctx.saved_tensors
         need = ctx.needs_input_grad
-        dx, dw, dgamma, dbeta, gvi = _conv_chain_backward(x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax, ctx.spec,
-                                                          ctx.batch_stats, ctx.x_exact, ctx.ssa, grad_out, grad_v_last,
-                                                          bool(need[0]), bool(need[1]), bool(need[4]))
-        return (dx, dw, dgamma if need[2] else None, dbeta if need[3] else None, gvi, None, None, None, None)
+        dx, dw, dgamma, dbeta, gvi, *grad_k = _conv_chain_backward(x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax,
+                                                                   ctx.spec, ctx.batch_stats, ctx.x_exact, ctx.ssa, grad_out,
+                                                                   grad_v_last, bool(need[0]), bool(need[1]), bool(need[4]), k)
+        return (dx, dw, dgamma if need[2] else None, dbeta if need[3] else None, gvi, None, None, None, None,
+                grad_k[0] if grad_k and need[9] else None)
 
 
 class _ConvBnLifSsaLif(torch.autograd.Function):
@@ -628,7 +652,7 @@ class _LifConvBnLif(torch.autograd.Function):
     convolution output and the batch-norm map."""
 
     @staticmethod
-    def forward(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec):
+    def forward(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec, k=None):
         running_mean, running_var, batch_stats, momentum, eps, tracked = _bn_config(bn)
         pre_seq = L.aligned16(pre_seq)
         T, B, Cin, Lp = pre_seq.shape
@@ -642,37 +666,39 @@ class _LifConvBnLif(torch.autograd.Function):
         y, partial = (out[0], out[1]) if batch_stats else (out, None)
         y = y.view(T, B, Cout, Lp)
         bn_map = _bn_map(y.flatten(0, 1), gamma, beta, running_mean, running_var, batch_stats, momentum, eps, partial, tracked)
-        spikes, v_last = _bn_lif_forward(y, bn_map, v_init, spec, False)
+        spikes, v_last = _bn_lif_forward(y, bn_map, v_init, spec, False, k)
         return spikes, v_last, pre_v_last.view(B, Cin, Lp), y, bn_map, bits
 
     @staticmethod
     def setup_context(ctx, inputs, output):
-        pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec = inputs
+        pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec, k = inputs
         ctx.pre_spec, ctx.spec, ctx.batch_stats = pre_spec, spec, _bn_config(bn)[2]
-        ctx.save_for_backward(L.aligned16(pre_seq), pre_v_init, weight, gamma, v_init, output[3], output[4], output[5])
+        ctx.save_for_backward(L.aligned16(pre_seq), pre_v_init, weight, gamma, v_init, output[3], output[4], output[5], k)
         ctx.mark_non_differentiable(output[3], output[4], output[5])
         ctx.set_materialize_grads(False)
 
     @staticmethod
     def backward(ctx, grad_spikes, grad_v_last, grad_pre_v_last, _y, _map, _bits):
-        pre_seq, pre_v_init, weight, gamma, v_init, y, bn_map, bits = ctx.saved_tensors
+        pre_seq, pre_v_init, weight, gamma, v_init, y, bn_map, bits, k = ctx.saved_tensors
         need = ctx.needs_input_grad
-        gx, gpv, dw, dgamma, dbeta, gvi = _lif_conv_chain_backward(
+        gx, gpv, dw, dgamma, dbeta, gvi, *grad_k = _lif_conv_chain_backward(
             pre_seq, pre_v_init, weight, gamma, v_init, y, bn_map, bits, ctx.pre_spec, ctx.spec, ctx.batch_stats, grad_spikes,
-            grad_v_last, grad_pre_v_last, bool(need[0]), bool(need[1]), bool(need[2]), bool(need[5]))
-        return (gx, gpv, dw, dgamma if need[3] else None, dbeta if need[4] else None, gvi, None, None, None)
+            grad_v_last, grad_pre_v_last, bool(need[0]), bool(need[1]), bool(need[2]), bool(need[5]), k)
+        return (gx, gpv, dw, dgamma if need[3] else None, dbeta if need[4] else None, gvi, None, None, None,
+                grad_k[0] if grad_k and need[9] else None)
 
 
 def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_v_init: torch.Tensor, weight: torch.Tensor, gamma, beta, v_init: torch.Tensor,
-                    bn, pre_spec, spec):
+                    bn, pre_spec, spec, k: Optional[torch.Tensor] = None):
     """``pre_seq [T, B, Cin, L]`` is the input of a LIF (``pre_spec``, state ``pre_v_init [B, Cin, L]``) whose spikes go
     through ``weight [Cout, Cin]``, batch norm and a second LIF (``spec``, ``v_init [B, Cout, L]``).  Returns
     ``(spikes [T, B, Cout, L], v_last, v_last of the first neuron)``.  The caller has checked ``lif_conv_bn_lif_supported``."""
     if torch.compiler.is_compiling():
         from . import fused_ops as O
 
+        _eager_only(k)
         return O.lif_conv_bn_lif(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec)
-    out = _LifConvBnLif.apply(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec)
+    out = _LifConvBnLif.apply(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec, k)
     return out[0], out[1], out[2]
 
 
@@ -685,37 +711,48 @@ def lif_conv_bn_lif_supported(pre_seq: torch.Tensor, need_grad: bool) -> bool:
     return (Cin * Lp) % 8 == 0
 
 
-def bn_lif(y_seq: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec):
-    """``y_seq [T, B, C, L]`` (a convolution output) -> ``(spikes, v_last)``."""
+def _eager_only(k):
+    if k is not None:
+        raise NotImplementedError("the fused chain with a parametric LIF has no traceable operator form: run it eagerly "
+                                  "(layer/fused.py steps aside for it while a graph is traced)")
+
+
+def bn_lif(y_seq: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec, k: Optional[torch.Tensor] = None):
+    """``y_seq [T, B, C, L]`` (a convolution output) -> ``(spikes, v_last)``.  ``k``: ``sigmoid(w)`` of a parametric LIF
+    (one element on the device; its gradient comes back through autograd), in which case ``spec[0]`` is unused."""
     if torch.compiler.is_compiling():
         from . import fused_ops as O
 
+        _eager_only(k)
         return O.bn_lif(y_seq, gamma, beta, v_init, bn, spec)
-    spikes, v_last, _ = _BnLif.apply(y_seq, gamma, beta, v_init, bn, spec)
+    spikes, v_last, _ = _BnLif.apply(y_seq, gamma, beta, v_init, bn, spec, k)
     return spikes, v_last
 
 
-def conv_bn_lif(x_seq: torch.Tensor, weight: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec, x_exact: bool):
+def conv_bn_lif(x_seq: torch.Tensor, weight: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec, x_exact: bool,
+                k: Optional[torch.Tensor] = None):
     """``x_seq [T, B, Cin, L]``, ``weight [Cout, Cin]`` -> ``(spikes [T, B, Cout, L], v_last [B, Cout, L])``.
     ``x_exact``: every element of ``x_seq`` is exactly representable in bf16 (spikes, small integers)."""
     if torch.compiler.is_compiling():
         from . import fused_ops as O
 
+        _eager_only(k)
         return O.conv_bn_lif(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, None)
-    spikes, v_last, _, _, _ = _ConvBnLif.apply(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact)
+    spikes, v_last, _, _, _ = _ConvBnLif.apply(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, k)
     return spikes, v_last
 
 
 def conv_bn_lif_ssa(x_seq: torch.Tensor, weight: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec, x_exact: bool,
-                    heads: int, channels_per_head: int, scale: float):
+                    heads: int, channels_per_head: int, scale: float, k: Optional[torch.Tensor] = None):
     """The same block with ``Cout = 3 * heads * channels_per_head`` followed by the contraction; returns
     ``(out [T * B, heads, channels_per_head, L], v_last)``."""
     if torch.compiler.is_compiling():
         from . import fused_ops as O
 
+        _eager_only(k)
         return O.conv_bn_lif(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, (heads, channels_per_head, scale))
     out, v_last, _, _, _, _ = _ConvBnLifSsa.apply(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact,
-                                               (heads, channels_per_head, scale))
+                                               (heads, channels_per_head, scale), k)
     return out, v_last
 
 

@@ -14,7 +14,7 @@ from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64
 
 import torch
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 # enums of include/sjhip.h
 NEURON_IF, NEURON_LIF, NEURON_PLIF, NEURON_QIF, NEURON_ILIF, NEURON_EIF = 0, 1, 2, 3, 4, 5
@@ -92,6 +92,9 @@ EXPORTED_SYMBOLS = (
     "sjhip_bn_finalize_rows",
     "sjhip_bn_lif_forward",
     "sjhip_bn_lif_backward",
+    "sjhip_bn_plif_forward",
+    "sjhip_bn_plif_backward_workspace_floats",
+    "sjhip_bn_plif_backward",
     "sjhip_bn_backward_finalize",
     "sjhip_bn_grad_input",
     "sjhip_bit_pack",
@@ -308,6 +311,12 @@ def load() -> ctypes.CDLL:
         lib.sjhip_bn_lif_forward.argtypes = [c_int, POINTER(NeuronParams), c_int64, c_int64, c_int64, c_int64] + [c_void_p] * 8
         lib.sjhip_bn_lif_backward.restype = c_int
         lib.sjhip_bn_lif_backward.argtypes = [c_int, POINTER(NeuronParams), c_int64, c_int64, c_int64, c_int64] + [c_void_p] * 10
+        lib.sjhip_bn_plif_forward.restype = c_int
+        lib.sjhip_bn_plif_forward.argtypes = [POINTER(NeuronParams), c_int64, c_int64, c_int64, c_int64] + [c_void_p] * 9
+        lib.sjhip_bn_plif_backward_workspace_floats.restype = c_int64
+        lib.sjhip_bn_plif_backward_workspace_floats.argtypes = [c_int64, c_int64, c_int64]
+        lib.sjhip_bn_plif_backward.restype = c_int
+        lib.sjhip_bn_plif_backward.argtypes = [POINTER(NeuronParams), c_int64, c_int64, c_int64, c_int64] + [c_void_p] * 13
         lib.sjhip_bn_backward_finalize.restype = c_int
         lib.sjhip_bn_backward_finalize.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int] + [c_void_p] * 8
         lib.sjhip_bn_grad_input.restype = c_int

@@ -81,7 +81,7 @@ class SpikingSelfAttention(nn.Module, base.MultiStepModule):
         node = self.qkv_lif
         T, N, C3, L = pre.shape
         cph = C3 // 3 // self.num_heads
-        if (not fused.unobserved(node) or node.store_v_seq or not pre.is_cuda
+        if (not fused._plain_hip_lif(node) or not fused.unobserved(node) or not pre.is_cuda
                 or not A.ssa_packed_supported(pre.dtype, cph, L) or (N * C3 * L) % 8 != 0):
             return None
         x2 = pre.flatten(1)

@@ -71,7 +71,7 @@ def _bn_arguments(bn: nn.Module):
     return bn.weight, bn.bias, (running_mean, running_var, batch_stats, momentum, float(bn.eps), tracked)
 
 
-def _lif_spec(node: neuron.LIFNode, x_like: torch.Tensor, need_grad: bool):
+def _lif_spec(node: nn.Module, x_like: torch.Tensor, need_grad: bool):
     from ..functional import neuron as F
     from ..hip_kernel import neuron_kernel as K
     from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
@@ -79,7 +79,24 @@ def _lif_spec(node: neuron.LIFNode, x_like: torch.Tensor, need_grad: bool):
     soft = node.v_reset is None
     flags = K._flags(soft, node.detach_reset, node.decay_input, F._hip_mode_flags(x_like))
     sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(node.surrogate_function) if need_grad else (0, 0.0)
-    return (float(node.tau), node.v_threshold, 0.0 if soft else float(node.v_reset), flags, sg_id, sg_alpha)
+    tau = 0.0 if type(node) is neuron.ParametricLIFNode else float(node.tau)  # (a parametric LIF's k travels as a tensor)
+    return (tau, node.v_threshold, 0.0 if soft else float(node.v_reset), flags, sg_id, sg_alpha)
+
+
+def _chain_neuron(node: nn.Module) -> bool:
+    """The neuron at the end of a fused chain: a plain LIF, or a parametric LIF outside a traced graph (the operator
+    forms of the chain take no learnable ``k``)."""
+    if type(node) is neuron.ParametricLIFNode:
+        return not torch.compiler.is_compiling()
+    return type(node) is neuron.LIFNode
+
+
+def _neuron_k(node: nn.Module, x_like: torch.Tensor) -> Optional[torch.Tensor]:
+    """``k = sigmoid(w)`` of a parametric LIF as the kernels read it (the sigmoid stays with autograd, which supplies
+    ``dk/dw``; reference functional/neuron.py:2173-2182), ``None`` for a plain LIF."""
+    if type(node) is not neuron.ParametricLIFNode:
+        return None
+    return node.w.sigmoid().to(device=x_like.device, dtype=torch.float32).reshape(1)
 
 
 def _plain_hip_lif(node: nn.Module) -> bool:
@@ -101,17 +118,18 @@ def conv_bn_lif(x_seq: torch.Tensor, conv: Optional[nn.Module], bn: nn.Module, n
 
     if not unobserved(conv, bn, node, attn, container):
         return None
-    if (not configure.hip_fuse_conv_bn_lif or type(node) is not neuron.LIFNode or node.backend != "hip" or node.step_mode != "m"
+    if (not configure.hip_fuse_conv_bn_lif or not _chain_neuron(node) or node.backend != "hip" or node.step_mode != "m"
             or node.store_v_seq or x_seq.dim() < 4):
         return None
-    if attn is not None and torch.compiler.is_compiling():
-        return None  # (the contraction with the attention's neuron inside has no operator form: eager only)
+    if attn is not None and (torch.compiler.is_compiling() or type(node) is not neuron.LIFNode):
+        return None  # (the contraction with the attention's neuron inside: eager only, plain LIF in front of it)
     if conv is not None and (not _pointwise(conv) or x_seq.shape[2] != conv.in_channels):
         return None
     channels = conv.out_channels if conv is not None else x_seq.shape[2]
     if not isinstance(bn, (nn.BatchNorm1d, nn.BatchNorm2d)) or bn.num_features != channels:
         return None
-    params = (p for p in (conv.weight if conv is not None else None, bn.weight, bn.bias) if p is not None)
+    params = (p for p in (conv.weight if conv is not None else None, bn.weight, bn.bias, getattr(node, "w", None))
+              if p is not None)
     need_grad = torch.is_grad_enabled() and (x_seq.requires_grad or any(p.requires_grad for p in params))
     x4 = x_seq.flatten(3)  # [T, B, C, L]
     if not C.supported(x4, need_grad):
@@ -149,13 +167,14 @@ def conv_bn_lif(x_seq: torch.Tensor, conv: Optional[nn.Module], bn: nn.Module, n
     v3 = v.reshape(B, channels, Lp) if v.dim() != 3 else v
     out_shape = (T, B, channels, *x_seq.shape[3:])
     with torch.set_grad_enabled(need_grad):
+        k = _neuron_k(node, x4)
         if conv is None:
-            spikes, v_last = C.bn_lif(x4, gamma, beta, v3, bn_cfg, spec)
+            spikes, v_last = C.bn_lif(x4, gamma, beta, v3, bn_cfg, spec, k)
         elif ssa is None:
-            spikes, v_last = C.conv_bn_lif(x4, conv.weight.view(channels, -1), gamma, beta, v3, bn_cfg, spec, x_exact)
+            spikes, v_last = C.conv_bn_lif(x4, conv.weight.view(channels, -1), gamma, beta, v3, bn_cfg, spec, x_exact, k)
         elif attn is None:
             out, v_last = C.conv_bn_lif_ssa(x4, conv.weight.view(channels, -1), gamma, beta, v3, bn_cfg, spec, x_exact,
-                                            heads, cph, scale)
+                                            heads, cph, scale, k)
             node.v = v_last.reshape(out_shape[1:])
             return out.view(T, B, heads, cph, Lp)
         else:
@@ -183,7 +202,7 @@ def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_node: nn.Module, conv: nn.Module,
     if not unobserved(pre_node, conv, bn, node, container):
         return None
     if (not configure.hip_fuse_conv_bn_lif or not getattr(configure, "hip_conv_bit_spikes", True)
-            or type(node) is not neuron.LIFNode or node.backend != "hip" or node.step_mode != "m" or node.store_v_seq
+            or not _chain_neuron(node) or node.backend != "hip" or node.step_mode != "m" or node.store_v_seq
             or not _plain_hip_lif(pre_node) or pre_seq.dim() < 4):
         return None
     Cin = conv.in_channels
@@ -198,7 +217,7 @@ def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_node: nn.Module, conv: nn.Module,
     channels = conv.out_channels
     if not isinstance(bn, (nn.BatchNorm1d, nn.BatchNorm2d)) or bn.num_features != channels:
         return None
-    params = (p for p in (conv.weight, bn.weight, bn.bias) if p is not None)
+    params = (p for p in (conv.weight, bn.weight, bn.bias, getattr(node, "w", None)) if p is not None)
     need_grad = torch.is_grad_enabled() and (pre_seq.requires_grad or any(p.requires_grad for p in params))
     x4 = pre_seq.reshape(pre_seq.shape[0], pre_seq.shape[1], Cin, -1)  # [T, B, Cin, L]
     T, B, _, Lp = x4.shape
@@ -221,7 +240,8 @@ def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_node: nn.Module, conv: nn.Module,
     pre_v3 = pre_v.reshape(B, Cin, Lp)
     with torch.set_grad_enabled(need_grad):
         spikes, v_last, pre_v_last = C.lif_conv_bn_lif(x4, pre_v3, conv.weight.view(channels, -1), gamma, beta, v3, bn_cfg,
-                                                       _lif_spec(pre_node, x4, need_grad), _lif_spec(node, x4, need_grad))
+                                                       _lif_spec(pre_node, x4, need_grad), _lif_spec(node, x4, need_grad),
+                                                       _neuron_k(node, x4))
     node.v = v_last.reshape(B, channels, *positions)
     pre_node.v = pre_v_last.reshape(pre_seq.shape[1:])
     return spikes.view(T, B, channels, *positions)

@@ -34,6 +34,7 @@ struct BnLifBwdArgs {
   const float *scale;
   const float *shift;
   float *partial;      // [B * C][2]: sum g, sum g y of the row
+  float *k_partial;    // PLIF: [4 x blocks] shares of dL/dk, one per wavefront
   int C, L;
   int64_t rows;        // B * C
 };
@@ -169,6 +170,7 @@ __device__ __forceinline__ void bn_lif_forward_body(const BnLifFwdArgs &a) {
   // the four steps of a short sequence)
   const int c = N <= 0x7fffffffLL ? (int)(((uint32_t)col / (uint32_t)a.L) % (uint32_t)a.C) : (int)((col / a.L) % a.C);
   const float sc = a.scale[c], sh = a.shift[c];
+  const float tau = f.k_device ? *f.k_device : f.tau;  // PLIF: k = sigmoid(w), read where torch left it
   const float *yp = (const float *)f.x + col;
   float *sp = (float *)f.spike + col;
   float v[4];
@@ -185,7 +187,7 @@ __device__ __forceinline__ void bn_lif_forward_body(const BnLifFwdArgs &a) {
         float y[4], h[4], s[4];
         A::unpack(rows[i], y);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) neuron_step<float, CH, RS>(fmaf(y[j], sc, sh), v[j], h[j], s[j], f.tau, f);
+        for (int j = 0; j < 4; ++j) neuron_step<float, CH, RS>(fmaf(y[j], sc, sh), v[j], h[j], s[j], tau, f);
         if (PACKED) store_spike_bits<4>((uint8_t *)f.spike + t * (N >> 3), col, N, s);
         else A::store(sp + t * N, s);
       }
@@ -213,13 +215,14 @@ template <bool PACKED> __global__ void __launch_bounds__(256) bn_lif_forward_ker
 template <int CH, int RS, int TMAX>
 __device__ __forceinline__ void replay_h(const FwdArgs &f, int len, const f32x4 (&yv)[TMAX], float sc, float sh, float (&v)[4],
                                          float (&h)[TMAX][4]) {
+  const float tau = f.k_device ? *f.k_device : f.tau;
 #pragma unroll
   for (int t = 0; t < TMAX; ++t) {
     if (t < len) {
       const float y[4] = {yv[t].x, yv[t].y, yv[t].z, yv[t].w};
       float s;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) neuron_step<float, CH, RS>(fmaf(y[j], sc, sh), v[j], h[t][j], s, f.tau, f);
+      for (int j = 0; j < 4; ++j) neuron_step<float, CH, RS>(fmaf(y[j], sc, sh), v[j], h[t][j], s, tau, f);
     }
   }
 }
@@ -245,10 +248,13 @@ __device__ __forceinline__ void replay_h_charge(const FwdArgs &f, int len, const
 }
 
 // BPTT over the replayed h (recurrence of neuron_bwd.h); writes g = dL/dz and adds this work-item's share of
-// sum g and sum g y
-template <int SG, int TMAX>
+// sum g and sum g y.  PLIF: also of dL/dk = sum G_t dh_t/dk, dh_t/dk = (h_t - v_{t-1}) / k with input decay (the division
+// is left to the final reduction) or v_reset - v_{t-1} without; v_{t-1} is re-derived from h_{t-1} with the forward's
+// reset arithmetic, v0 is the state in front of the first of these steps.
+template <int SG, int TMAX, bool PLIF>
 __device__ __forceinline__ void bptt_rows(const BwdArgs &b, float k, int64_t col, int64_t t0, int len, const f32x4 (&yv)[TMAX],
-                                          const float (&h)[TMAX][4], float (&carry)[4], float &acc_g, float &acc_gy) {
+                                          const float (&h)[TMAX][4], const float (&v0)[4], float (&carry)[4], float &acc_g,
+                                          float &acc_gy, float &acc_k) {
 #pragma clang fp contract(fast)
   typedef Acc<float, true, true> A;
   const int64_t N = b.N;
@@ -273,36 +279,45 @@ __device__ __forceinline__ void bptt_rows(const BwdArgs &b, float k, int64_t col
         carry[j] = G * km;
         acc_g += gz[j];
         acc_gy = fmaf(gz[j], y[j], acc_gy);
+        if constexpr (PLIF) {
+          float v_prev = v0[j];
+          if (t > 0) {
+            const float h_prev = h[t > 0 ? t - 1 : 0][j];
+            v_prev = reset_as_forward(h_prev, (h_prev - b.v_th >= 0.0f) ? 1.0f : 0.0f, b);
+          }
+          acc_k = fmaf(G, b.decay_input ? (h[t][j] - v_prev) : (b.v_reset - v_prev), acc_k);
+        }
       }
       Acc<float, true, false>::store(gxp + (int64_t)t * N, gz);  // read again by the next kernel
     }
   }
 }
 
-template <int TMAX>
+template <int TMAX, bool PLIF>
 __device__ __forceinline__ void bptt_rows_surrogate(const BwdArgs &b, float k, int64_t col, int64_t t0, int len,
-                                                    const f32x4 (&yv)[TMAX], const float (&h)[TMAX][4], float (&carry)[4],
-                                                    float &acc_g, float &acc_gy) {
+                                                    const f32x4 (&yv)[TMAX], const float (&h)[TMAX][4], const float (&v0)[4],
+                                                    float (&carry)[4], float &acc_g, float &acc_gy, float &acc_k) {
   switch (b.sg) {
-    case SJHIP_SG_SIGMOID: bptt_rows<SJHIP_SG_SIGMOID, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
-    case SJHIP_SG_ATAN: bptt_rows<SJHIP_SG_ATAN, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
-    case SJHIP_SG_PIECEWISE_QUADRATIC: bptt_rows<SJHIP_SG_PIECEWISE_QUADRATIC, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
-    case SJHIP_SG_PIECEWISE_EXP: bptt_rows<SJHIP_SG_PIECEWISE_EXP, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
-    case SJHIP_SG_SOFT_SIGN: bptt_rows<SJHIP_SG_SOFT_SIGN, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
-    case SJHIP_SG_SUPER_SPIKE: bptt_rows<SJHIP_SG_SUPER_SPIKE, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
-    default: bptt_rows<SJHIP_SG_ERF, TMAX>(b, k, col, t0, len, yv, h, carry, acc_g, acc_gy); break;
+    case SJHIP_SG_SIGMOID: bptt_rows<SJHIP_SG_SIGMOID, TMAX, PLIF>(b, k, col, t0, len, yv, h, v0, carry, acc_g, acc_gy, acc_k); break;
+    case SJHIP_SG_ATAN: bptt_rows<SJHIP_SG_ATAN, TMAX, PLIF>(b, k, col, t0, len, yv, h, v0, carry, acc_g, acc_gy, acc_k); break;
+    case SJHIP_SG_PIECEWISE_QUADRATIC: bptt_rows<SJHIP_SG_PIECEWISE_QUADRATIC, TMAX, PLIF>(b, k, col, t0, len, yv, h, v0, carry, acc_g, acc_gy, acc_k); break;
+    case SJHIP_SG_PIECEWISE_EXP: bptt_rows<SJHIP_SG_PIECEWISE_EXP, TMAX, PLIF>(b, k, col, t0, len, yv, h, v0, carry, acc_g, acc_gy, acc_k); break;
+    case SJHIP_SG_SOFT_SIGN: bptt_rows<SJHIP_SG_SOFT_SIGN, TMAX, PLIF>(b, k, col, t0, len, yv, h, v0, carry, acc_g, acc_gy, acc_k); break;
+    case SJHIP_SG_SUPER_SPIKE: bptt_rows<SJHIP_SG_SUPER_SPIKE, TMAX, PLIF>(b, k, col, t0, len, yv, h, v0, carry, acc_g, acc_gy, acc_k); break;
+    default: bptt_rows<SJHIP_SG_ERF, TMAX, PLIF>(b, k, col, t0, len, yv, h, v0, carry, acc_g, acc_gy, acc_k); break;
   }
 }
 
 // One work-item's four neurons (quad q of row `row`) for all T steps: replay, BPTT, g written, the sums extended.
-template <int TMAX>
-__device__ __forceinline__ void bn_lif_backward_quad(const BnLifBwdArgs &a, int64_t row, int q, float &acc_g, float &acc_gy) {
+template <int TMAX, bool PLIF>
+__device__ __forceinline__ void bn_lif_backward_quad(const BnLifBwdArgs &a, int64_t row, int q, float &acc_g, float &acc_gy,
+                                                     float &acc_k) {
   typedef Acc<float, true, false> A;
   const FwdArgs &f = a.f;
   const BwdArgs &b = a.b;
   const int c = (int)(row % a.C);
   const float sc = a.scale[c], sh = a.shift[c];
-  const float k = b.k;
+  const float k = (PLIF && b.k_device) ? *b.k_device : b.k;
   const int64_t N = f.N;
   const int64_t col = row * a.L + 4 * q;
   const float *yp = (const float *)f.x + col;
@@ -311,10 +326,11 @@ __device__ __forceinline__ void bn_lif_backward_quad(const BnLifBwdArgs &a, int6
   for (int t = 0; t < TMAX; ++t) yv[t] = (t < f.T) ? A::load(yp + (int64_t)t * N) : A::zero();
   float v[4], h[TMAX][4], carry[4];
   load_state<float, true, false>(f.v_init, col, f.v_init_broadcast != 0, v);
+  const float v0[4] = {v[0], v[1], v[2], v[3]};
   if (b.grad_v_last) A::unpack(A::load((const float *)b.grad_v_last + col), carry);
   else carry[0] = carry[1] = carry[2] = carry[3] = 0.0f;
   replay_h_charge<TMAX>(f, (int)f.T, yv, sc, sh, v, h);
-  bptt_rows_surrogate<TMAX>(b, k, col, 0, (int)b.T, yv, h, carry, acc_g, acc_gy);
+  bptt_rows_surrogate<TMAX, PLIF>(b, k, col, 0, (int)b.T, yv, h, v0, carry, acc_g, acc_gy, acc_k);
   if (b.grad_v_init) A::store((float *)b.grad_v_init + col, carry);
 }
 
@@ -324,8 +340,9 @@ __device__ __forceinline__ void bn_lif_backward_quad(const BnLifBwdArgs &a, int6
 // replayed from its parked state into registers and walked backwards; y is read twice.
 constexpr int kBnPiece = 16;
 constexpr int kBnMaxPieces = 16;  // 256 work-items x 16 bytes x 16 pieces = 64 KiB of LDS
+template <bool PLIF>
 __device__ __forceinline__ void bn_lif_backward_quad_long(const BnLifBwdArgs &a, int64_t row, int q, float &acc_g, float &acc_gy,
-                                                          f32x4 *parked) {
+                                                          float &acc_k, f32x4 *parked) {
   typedef Acc<float, true, false> A;
   const FwdArgs &f = a.f;
   const BwdArgs &b = a.b;
@@ -353,27 +370,39 @@ __device__ __forceinline__ void bn_lif_backward_quad_long(const BnLifBwdArgs &a,
     for (int t = 0; t < kBnPiece; ++t) yv[t] = (t < len) ? A::load(yp + (int64_t)(t0 + t) * N) : A::zero();
     const f32x4 s = parked[p * blockDim.x];
     v[0] = s.x; v[1] = s.y; v[2] = s.z; v[3] = s.w;
+    const float v0[4] = {s.x, s.y, s.z, s.w};
     replay_h_charge<kBnPiece>(f, len, yv, sc, sh, v, h);
-    bptt_rows_surrogate<kBnPiece>(b, b.k, col, t0, len, yv, h, carry, acc_g, acc_gy);
+    bptt_rows_surrogate<kBnPiece, PLIF>(b, (PLIF && b.k_device) ? *b.k_device : b.k, col, t0, len, yv, h, v0, carry, acc_g,
+                                        acc_gy, acc_k);
   }
   if (b.grad_v_init) A::store((float *)b.grad_v_init + col, carry);
 }
 
 // A wavefront per row; lanes stride over the row's quads.
 // (TMAX = 0: the walk in pieces, with pieces x 256 x 16 bytes of dynamic LDS)
-template <int TMAX> __global__ void __launch_bounds__(256) bn_lif_backward_kernel(const BnLifBwdArgs a) {
+// PLIF: every wavefront also leaves its share of dL/dk in k_partial[4 * block + wavefront] (summed afterwards in a fixed
+// order by plif_reduce_kernel, which also divides by k where the charge calls for it).
+template <int TMAX, bool PLIF> __global__ void __launch_bounds__(256) bn_lif_backward_kernel(const BnLifBwdArgs a) {
   extern __shared__ f32x4 parked_states[];
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= a.rows) return;
-  float acc_g = 0.0f, acc_gy = 0.0f;
+  if (row >= a.rows) {
+    if (PLIF && lane == 0) a.k_partial[(int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)] = 0.0f;
+    return;
+  }
+  float acc_g = 0.0f, acc_gy = 0.0f, acc_k = 0.0f;
   for (int q = lane; q < a.L / 4; q += 64) {
-    if constexpr (TMAX == 0) bn_lif_backward_quad_long(a, row, q, acc_g, acc_gy, parked_states + threadIdx.x);
-    else bn_lif_backward_quad<TMAX>(a, row, q, acc_g, acc_gy);
+    if constexpr (TMAX == 0) bn_lif_backward_quad_long<PLIF>(a, row, q, acc_g, acc_gy, acc_k, parked_states + threadIdx.x);
+    else bn_lif_backward_quad<TMAX, PLIF>(a, row, q, acc_g, acc_gy, acc_k);
   }
   acc_g = wave_sum(acc_g);
   acc_gy = wave_sum(acc_gy);
-  if (lane == 0) { a.partial[2 * row] = acc_g; a.partial[2 * row + 1] = acc_gy; }
+  if (PLIF) acc_k = wave_sum(acc_k);
+  if (lane == 0) {
+    a.partial[2 * row] = acc_g;
+    a.partial[2 * row + 1] = acc_gy;
+    if (PLIF) a.k_partial[(int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)] = acc_k;
+  }
 }
 
 // Rows of fewer than 64 quads leave lanes of a wavefront-per-row kernel idle (196 positions: 49 of 64 working), and this
@@ -381,7 +410,7 @@ template <int TMAX> __global__ void __launch_bounds__(256) bn_lif_backward_kerne
 // quads: 245 working); a row's sums are formed per wavefront (a wavefront holds parts of a few rows: one masked
 // reduction per row it touches), left in LDS, and added over the wavefronts in their order by one work-item per row,
 // so the result does not depend on timing.
-template <int TMAX>
+template <int TMAX, bool PLIF>
 __global__ void __launch_bounds__(256) bn_lif_backward_rows_kernel(const BnLifBwdArgs a, int quads, int rows_per_block,
                                                                    float inv_quads) {
   __shared__ float part[4][kBnRowsMax][2];
@@ -392,10 +421,14 @@ __global__ void __launch_bounds__(256) bn_lif_backward_rows_kernel(const BnLifBw
   const int64_t row = (int64_t)blockIdx.x * rows_per_block + r_local;
   const bool valid = r_local < rows_per_block && row < a.rows;
   if (r_local >= rows_per_block) r_local = rows_per_block - 1;
-  float acc_g = 0.0f, acc_gy = 0.0f;
+  float acc_g = 0.0f, acc_gy = 0.0f, acc_k = 0.0f;
   if (valid) {
-    if constexpr (TMAX == 0) bn_lif_backward_quad_long(a, row, q, acc_g, acc_gy, parked_states + tid);
-    else bn_lif_backward_quad<TMAX>(a, row, q, acc_g, acc_gy);
+    if constexpr (TMAX == 0) bn_lif_backward_quad_long<PLIF>(a, row, q, acc_g, acc_gy, acc_k, parked_states + tid);
+    else bn_lif_backward_quad<TMAX, PLIF>(a, row, q, acc_g, acc_gy, acc_k);
+  }
+  if (PLIF) {
+    acc_k = wave_sum(acc_k);
+    if ((tid & 63) == 0) a.k_partial[(int64_t)blockIdx.x * 4 + (tid >> 6)] = acc_k;
   }
   block_row_sums(part, r_local, valid, rows_per_block, acc_g, acc_gy, a.partial, (int64_t)blockIdx.x * rows_per_block, a.rows);
 }
@@ -515,7 +548,7 @@ int check_layout(const char *what, int64_t T, int64_t B, int64_t C, int64_t L) {
   return SJHIP_OK;
 }
 
-bool lif_like(int neuron) { return neuron == SJHIP_NEURON_IF || neuron == SJHIP_NEURON_LIF; }
+bool lif_like(int neuron) { return neuron == SJHIP_NEURON_IF || neuron == SJHIP_NEURON_LIF || neuron == SJHIP_NEURON_PLIF; }
 
 }  // namespace
 
@@ -542,11 +575,13 @@ int launch_bn_finalize(const float *partial, int64_t rows, int64_t count, int64_
 }
 
 int launch_bn_lif_forward(int neuron, const sjhip_neuron_params &p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
-                          const float *scale, const float *shift, const float *v_init, float *spike_seq, uint8_t *spike_bits,
-                          float *v_last, hipStream_t stream) {
+                          const float *scale, const float *shift, const float *v_init, const float *k_device, float *spike_seq,
+                          uint8_t *spike_bits, float *v_last, hipStream_t stream) {
   int rc = check_layout("bn_lif_forward", T, B, C, L);
   if (rc != SJHIP_OK) return rc;
-  if (!lif_like(neuron)) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_forward: neuron %d (IF and LIF only)", neuron);
+  if (!lif_like(neuron)) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_forward: neuron %d (IF, LIF and PLIF only)", neuron);
+  if ((neuron == SJHIP_NEURON_PLIF) != (k_device != nullptr))
+    return fail(SJHIP_ERR_INVALID, "bn_lif_forward: k in device memory goes with PLIF and only with it");
   const int64_t N = B * C * L;
   const bool broadcast = (p.flags & SJHIP_FLAG_V_INIT_BROADCAST) != 0;
   if (!aligned16(y) || (!broadcast && !aligned16(v_init)) || (spike_seq && !aligned16(spike_seq)) || (v_last && !aligned16(v_last)))
@@ -554,8 +589,8 @@ int launch_bn_lif_forward(int neuron, const sjhip_neuron_params &p, int64_t T, i
   if (spike_bits && N % 8 != 0) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_forward: B*C*L=%lld must be a multiple of 8 for bit-packed spikes", (long long)N);
   BnLifFwdArgs a;
   bool round_each = false;
-  rc = build_fwd_args(a.f, round_each, neuron, SJHIP_F32, p, T, N, y, v_init, nullptr, spike_bits ? (void *)spike_bits : (void *)spike_seq,
-                      nullptr, v_last, nullptr);
+  rc = build_fwd_args(a.f, round_each, neuron, SJHIP_F32, p, T, N, y, v_init, k_device,
+                      spike_bits ? (void *)spike_bits : (void *)spike_seq, nullptr, v_last, nullptr);
   if (rc != SJHIP_OK) return rc;
   a.scale = scale; a.shift = shift; a.C = (int)C; a.L = (int)L;
   const int64_t blocks = (N / 4 + 255) / 256;
@@ -566,12 +601,22 @@ int launch_bn_lif_forward(int neuron, const sjhip_neuron_params &p, int64_t T, i
   return check_launch("bn_lif_forward");
 }
 
+// wavefront shares of dL/dk: four per block of either backward kernel (the one with fewer rows per block bounds it)
+int64_t bn_lif_backward_k_workspace_floats(int64_t B, int64_t C, int64_t L) {
+  (void)L;
+  return 4 * ((B * C + 3) / 4) + 4;
+}
+
 int launch_bn_lif_backward(int neuron, const sjhip_neuron_params &p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
-                           const float *scale, const float *shift, const float *v_init, const float *grad_spike_seq,
-                           const float *grad_v_last, float *grad_z, float *grad_v_init, float *partial, hipStream_t stream) {
+                           const float *scale, const float *shift, const float *v_init, const float *k_device,
+                           const float *grad_spike_seq, const float *grad_v_last, float *grad_z, float *grad_v_init, float *partial,
+                           float *grad_k, float *k_workspace, hipStream_t stream) {
   int rc = check_layout("bn_lif_backward", T, B, C, L);
   if (rc != SJHIP_OK) return rc;
-  if (!lif_like(neuron)) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: neuron %d (IF and LIF only)", neuron);
+  if (!lif_like(neuron)) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: neuron %d (IF, LIF and PLIF only)", neuron);
+  const bool plif = neuron == SJHIP_NEURON_PLIF;
+  if (plif != (k_device != nullptr) || (plif && (!grad_k || !k_workspace)))
+    return fail(SJHIP_ERR_INVALID, "bn_lif_backward: k in device memory, grad_k and the workspace go with PLIF and only with it");
   if (T > kBnPiece * kBnMaxPieces)
     return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: T=%lld (at most %d steps)", (long long)T, kBnPiece * kBnMaxPieces);
   if (p.sg_id < SJHIP_SG_SIGMOID || p.sg_id > SJHIP_SG_ERF) return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: surrogate id %d", p.sg_id);
@@ -582,12 +627,12 @@ int launch_bn_lif_backward(int neuron, const sjhip_neuron_params &p, int64_t T, 
     return fail(SJHIP_ERR_UNSUPPORTED, "bn_lif_backward: tensors must be 16-byte aligned");
   BnLifBwdArgs a;
   bool round_each = false;
-  rc = build_fwd_args(a.f, round_each, neuron, SJHIP_F32, p, T, N, y, v_init, nullptr, nullptr, nullptr, nullptr, nullptr);
+  rc = build_fwd_args(a.f, round_each, neuron, SJHIP_F32, p, T, N, y, v_init, k_device, nullptr, nullptr, nullptr, nullptr);
   if (rc != SJHIP_OK) return rc;
-  rc = build_bwd_args(a.b, neuron, SJHIP_F32, p, T, N, grad_spike_seq, nullptr, grad_v_last, nullptr, v_init, nullptr, grad_z,
-                      grad_v_init, nullptr, nullptr);
+  rc = build_bwd_args(a.b, neuron, SJHIP_F32, p, T, N, grad_spike_seq, nullptr, grad_v_last, nullptr, v_init, k_device, grad_z,
+                      grad_v_init, grad_k, k_workspace);
   if (rc != SJHIP_OK) return rc;
-  a.scale = scale; a.shift = shift; a.partial = partial; a.C = (int)C; a.L = (int)L; a.rows = B * C;
+  a.scale = scale; a.shift = shift; a.partial = partial; a.k_partial = k_workspace; a.C = (int)C; a.L = (int)L; a.rows = B * C;
   const int64_t blocks = (a.rows + 3) / 4;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "bn_lif_backward: %lld rows", (long long)a.rows);
   ProfileScope prof(KC_BN_LIF_BACKWARD, stream);
@@ -595,22 +640,34 @@ int launch_bn_lif_backward(int neuron, const sjhip_neuron_params &p, int64_t T, 
   const unsigned parked = T > kBnPiece ? (unsigned)((T + kBnPiece - 1) / kBnPiece) * 256u * 16u : 0u;
   const int quads = (int)(L / 4);
   const int per = quads > 0 ? 256 / quads : 0;
-  if (quads >= 16 && per > 4) {
-    // more than the four rows a block of the wavefront-per-row kernel takes: more lanes working
-    const int64_t nb = (a.rows + per - 1) / per;
-    if (nb > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "bn_lif_backward: %lld rows", (long long)a.rows);
-    const float inv = 1.0f / (float)quads;
-    if (T <= 4) hipLaunchKernelGGL((bn_lif_backward_rows_kernel<4>), dim3((unsigned)nb), dim3(256), 0, stream, a, quads, per, inv);
-    else if (T <= 8) hipLaunchKernelGGL((bn_lif_backward_rows_kernel<8>), dim3((unsigned)nb), dim3(256), 0, stream, a, quads, per, inv);
-    else if (T <= 16) hipLaunchKernelGGL((bn_lif_backward_rows_kernel<16>), dim3((unsigned)nb), dim3(256), 0, stream, a, quads, per, inv);
-    else hipLaunchKernelGGL((bn_lif_backward_rows_kernel<0>), dim3((unsigned)nb), dim3(256), parked, stream, a, quads, per, inv);
-    return check_launch("bn_lif_backward");
-  }
-  if (T <= 4) hipLaunchKernelGGL((bn_lif_backward_kernel<4>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
-  else if (T <= 8) hipLaunchKernelGGL((bn_lif_backward_kernel<8>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
-  else if (T <= 16) hipLaunchKernelGGL((bn_lif_backward_kernel<16>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
-  else hipLaunchKernelGGL((bn_lif_backward_kernel<0>), dim3((unsigned)blocks), dim3(256), parked, stream, a);
-  return check_launch("bn_lif_backward");
+  // TMAX by sequence length (0: the walk in pieces), with or without the dL/dk term
+  auto launch = [&](auto rows_kernel, auto plif_flag) {
+    constexpr bool ROWS = decltype(rows_kernel)::value, P = decltype(plif_flag)::value;
+    const int64_t nb = ROWS ? (a.rows + per - 1) / per : blocks;
+    const float inv = quads > 0 ? 1.0f / (float)quads : 0.0f;
+    const dim3 grid((unsigned)nb), threads(256);
+    if constexpr (ROWS) {
+      if (T <= 4) hipLaunchKernelGGL((bn_lif_backward_rows_kernel<4, P>), grid, threads, 0, stream, a, quads, per, inv);
+      else if (T <= 8) hipLaunchKernelGGL((bn_lif_backward_rows_kernel<8, P>), grid, threads, 0, stream, a, quads, per, inv);
+      else if (T <= 16) hipLaunchKernelGGL((bn_lif_backward_rows_kernel<16, P>), grid, threads, 0, stream, a, quads, per, inv);
+      else hipLaunchKernelGGL((bn_lif_backward_rows_kernel<0, P>), grid, threads, parked, stream, a, quads, per, inv);
+    } else {
+      if (T <= 4) hipLaunchKernelGGL((bn_lif_backward_kernel<4, P>), grid, threads, 0, stream, a);
+      else if (T <= 8) hipLaunchKernelGGL((bn_lif_backward_kernel<8, P>), grid, threads, 0, stream, a);
+      else if (T <= 16) hipLaunchKernelGGL((bn_lif_backward_kernel<16, P>), grid, threads, 0, stream, a);
+      else hipLaunchKernelGGL((bn_lif_backward_kernel<0, P>), grid, threads, parked, stream, a);
+    }
+    return nb;
+  };
+  // more than the four rows a block of the wavefront-per-row kernel takes: more lanes working
+  const bool by_rows = quads >= 16 && per > 4;
+  if (by_rows && (a.rows + per - 1) / per > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "bn_lif_backward: %lld rows", (long long)a.rows);
+  int64_t nb;
+  if (by_rows) nb = plif ? launch(std::true_type(), std::true_type()) : launch(std::true_type(), std::false_type());
+  else nb = plif ? launch(std::false_type(), std::true_type()) : launch(std::false_type(), std::false_type());
+  rc = check_launch("bn_lif_backward");
+  if (rc != SJHIP_OK || !plif) return rc;
+  return launch_plif_reduce(a.b, 4 * nb, grad_k, stream);
 }
 
 int launch_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64_t C, int64_t L, int training, const float *gamma,

@@ -773,20 +773,42 @@ int sjhip_bn_finalize_rows(const float *partial, int64_t rows, int64_t count, in
 int sjhip_bn_lif_forward(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
                          const float *scale, const float *shift, const float *v_init, float *spike_seq, uint8_t *spike_bits,
                          float *v_last, void *stream) {
-  if (!p) return fail(SJHIP_ERR_INVALID, "bn_lif_forward: params is NULL");
-  if (!y || !scale || !shift || !v_init) return fail(SJHIP_ERR_INVALID, "bn_lif_forward: NULL tensor");
-  if ((spike_seq == nullptr) == (spike_bits == nullptr)) return fail(SJHIP_ERR_INVALID, "bn_lif_forward: exactly one of spike_seq and spike_bits");
-  return launch_bn_lif_forward(neuron, *p, T, B, C, L, y, scale, shift, v_init, spike_seq, spike_bits, v_last,
+  if (!p || !y || !scale || !shift || !v_init || (spike_seq == nullptr) == (spike_bits == nullptr))
+    return fail(SJHIP_ERR_INVALID, "bn_lif_forward: NULL buffer, or not exactly one of spike_seq / spike_bits");
+  return launch_bn_lif_forward(neuron, *p, T, B, C, L, y, scale, shift, v_init, nullptr, spike_seq, spike_bits, v_last,
                                static_cast<hipStream_t>(stream));
 }
 
 int sjhip_bn_lif_backward(int neuron, const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
                           const float *scale, const float *shift, const float *v_init, const float *grad_spike_seq,
                           const float *grad_v_last, float *grad_z, float *grad_v_init, float *partial, void *stream) {
-  if (!p) return fail(SJHIP_ERR_INVALID, "bn_lif_backward: params is NULL");
-  if (!y || !scale || !shift || !v_init || !grad_spike_seq || !grad_z || !partial) return fail(SJHIP_ERR_INVALID, "bn_lif_backward: NULL tensor");
-  return launch_bn_lif_backward(neuron, *p, T, B, C, L, y, scale, shift, v_init, grad_spike_seq, grad_v_last, grad_z, grad_v_init,
-                                partial, static_cast<hipStream_t>(stream));
+  if (!p || !y || !scale || !shift || !v_init || !grad_spike_seq || !grad_z || !partial)
+    return fail(SJHIP_ERR_INVALID, "bn_lif_backward: NULL buffer");
+  return launch_bn_lif_backward(neuron, *p, T, B, C, L, y, scale, shift, v_init, nullptr, grad_spike_seq, grad_v_last, grad_z,
+                                grad_v_init, partial, nullptr, nullptr, static_cast<hipStream_t>(stream));
+}
+
+int sjhip_bn_plif_forward(const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
+                          const float *scale, const float *shift, const float *v_init, const float *k_device, float *spike_seq,
+                          uint8_t *spike_bits, float *v_last, void *stream) {
+  if (!p || !y || !scale || !shift || !v_init || !k_device || (spike_seq == nullptr) == (spike_bits == nullptr))
+    return fail(SJHIP_ERR_INVALID, "bn_plif_forward: NULL buffer, or not exactly one of spike_seq / spike_bits");
+  return launch_bn_lif_forward(SJHIP_NEURON_PLIF, *p, T, B, C, L, y, scale, shift, v_init, k_device, spike_seq, spike_bits, v_last,
+                               static_cast<hipStream_t>(stream));
+}
+
+int64_t sjhip_bn_plif_backward_workspace_floats(int64_t B, int64_t C, int64_t L) {
+  return bn_lif_backward_k_workspace_floats(B, C, L);
+}
+
+int sjhip_bn_plif_backward(const sjhip_neuron_params *p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
+                           const float *scale, const float *shift, const float *v_init, const float *k_device,
+                           const float *grad_spike_seq, const float *grad_v_last, float *grad_z, float *grad_v_init,
+                           float *partial, float *grad_k, float *workspace, void *stream) {
+  if (!p || !y || !scale || !shift || !v_init || !k_device || !grad_spike_seq || !grad_z || !partial || !grad_k || !workspace)
+    return fail(SJHIP_ERR_INVALID, "bn_plif_backward: NULL buffer");
+  return launch_bn_lif_backward(SJHIP_NEURON_PLIF, *p, T, B, C, L, y, scale, shift, v_init, k_device, grad_spike_seq, grad_v_last,
+                                grad_z, grad_v_init, partial, grad_k, workspace, static_cast<hipStream_t>(stream));
 }
 
 int sjhip_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64_t C, int64_t L, int training, const float *gamma,

@@ -478,12 +478,15 @@ int launch_bn_stats(const float *y, int64_t S, int64_t C, int64_t L, float *part
 int launch_bn_finalize(const float *partial, int64_t rows, int64_t count, int64_t C, const float *gamma, const float *beta, float eps,
                        float momentum, float *running_mean, float *running_var, float *scale, float *shift, float *mean,
                        float *invstd, int64_t *batches_tracked, hipStream_t stream);
+// (k_device: PLIF's k = sigmoid(w) in device memory, else nullptr; grad_k + k_workspace: where dL/dk goes, PLIF only)
 int launch_bn_lif_forward(int neuron, const sjhip_neuron_params &p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
-                          const float *scale, const float *shift, const float *v_init, float *spike_seq, uint8_t *spike_bits,
-                          float *v_last, hipStream_t stream);
+                          const float *scale, const float *shift, const float *v_init, const float *k_device, float *spike_seq,
+                          uint8_t *spike_bits, float *v_last, hipStream_t stream);
+int64_t bn_lif_backward_k_workspace_floats(int64_t B, int64_t C, int64_t L);
 int launch_bn_lif_backward(int neuron, const sjhip_neuron_params &p, int64_t T, int64_t B, int64_t C, int64_t L, const float *y,
-                           const float *scale, const float *shift, const float *v_init, const float *grad_spike_seq,
-                           const float *grad_v_last, float *grad_z, float *grad_v_init, float *partial, hipStream_t stream);
+                           const float *scale, const float *shift, const float *v_init, const float *k_device,
+                           const float *grad_spike_seq, const float *grad_v_last, float *grad_z, float *grad_v_init, float *partial,
+                           float *grad_k, float *k_workspace, hipStream_t stream);
 int launch_bn_backward_finalize(const float *partial, int64_t T, int64_t B, int64_t C, int64_t L, int training, const float *gamma,
                                 const float *mean, const float *invstd, float *dgamma, float *dbeta, float *coef,
                                 float *amax_reset, hipStream_t stream);

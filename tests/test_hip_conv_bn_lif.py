@@ -571,6 +571,91 @@ def test_bn_lif_against_float64(C, T, B, Cc, Lp, training, v_reset, decay_input,
     torch.testing.assert_close(bd.grad.cpu().double(), b64.grad, rtol=1e-4, atol=1e-5 * float(b64.grad.abs().max()))
 
 
+@pytest.mark.parametrize("T,B,Cc,Lp", [(4, 3, 10, 12), (7, 2, 33, 20), (16, 2, 6, 260), (4, 2, 12, 196), (33, 1, 6, 196), (20, 2, 5, 36)])
+@pytest.mark.parametrize("v_reset,decay_input,init_tau,sg", [(0.0, True, 2.0, "sigmoid"), (None, False, 3.0, "atan"), (-0.2, True, 2.5, "erf")])
+def test_bn_plif_against_float64(C, T, B, Cc, Lp, v_reset, decay_input, init_tau, sg):
+    """Batch norm + parametric LIF (``k = 1 / init_tau`` read from device memory): spikes, state and the gradients of
+    the input, of the batch-norm parameters and of ``k`` against autograd through the float64 oracle
+    (``neuron_oracle.multi_step('plif_k')``, restating functional/neuron.py:1215-1297)."""
+    from spikingjelly_amd.activation_based.hip_kernel import neuron_kernel as K
+
+    gamma, beta = seeded_randn((Cc,), 132, 1.0, 0.2), seeded_randn((Cc,), 133, 0.6, 0.3)
+    gs = seeded_randn((T, B, Cc, Lp), 136)
+    gl = seeded_randn((B, Cc, Lp), 137, 0.0, 0.3)
+    alpha = no.SG_DEFAULT_ALPHA[sg]
+    detach = v_reset is None
+    k32 = torch.tensor([1.0 / init_tau], dtype=torch.float32)
+    start = 0.0 if v_reset is None else v_reset
+    for seed in range(131, 3200, 100):  # the first input whose membrane potentials all keep the margin from the threshold
+        y = seeded_randn((T, B, Cc, Lp), seed, 0.4, 1.5)
+        y64 = y.double().requires_grad_()
+        g64, b64 = gamma.double().requires_grad_(), beta.double().requires_grad_()
+        k64 = k32.double().requires_grad_()
+        z, _, _ = co.batch_norm(y64, g64, b64, torch.zeros(Cc, dtype=torch.float64), torch.ones(Cc, dtype=torch.float64), True)
+        s64, v64, h64 = no.multi_step("plif_k", z.flatten(1), torch.full((B * Cc * Lp,), start, dtype=torch.float64), k64[0],
+                                      decay_input, 1.0, v_reset, no.surrogate(sg, alpha), detach)
+        if _no_borderline(h64.detach(), 1.0):
+            break
+    else:
+        pytest.fail("no input without a neuron within the margin of the threshold")
+    torch.autograd.backward([s64, v64[-1]], [gs.double().flatten(1), gl.double().flatten()])
+
+    soft = v_reset is None
+    spec = (0.0, 1.0, 0.0 if soft else v_reset, K._flags(soft, detach, decay_input, 0), no.SG_IDS[sg], alpha)
+    yd = y.cuda().requires_grad_()
+    gd, bd = gamma.cuda().requires_grad_(), beta.cuda().requires_grad_()
+    kd = k32.cuda().requires_grad_()
+    v0 = torch.full((1,), start, device="cuda").expand(B, Cc, Lp)
+    spikes, v_last = C.bn_lif(yd, gd, bd, v0, (torch.zeros(Cc, device="cuda"), torch.ones(Cc, device="cuda"), True, 0.1, 1e-5),
+                              spec, kd)
+    torch.autograd.backward([spikes, v_last], [gs.cuda(), gl.cuda()])
+    assert torch.equal(spikes.detach().cpu().double().flatten(1), s64.detach())
+    torch.testing.assert_close(v_last.detach().cpu().double().flatten(), v64[-1].detach(), rtol=1e-5, atol=1e-5)
+    scale = float(y64.grad.abs().max())
+    torch.testing.assert_close(yd.grad.cpu().double(), y64.grad, rtol=1e-4, atol=1e-5 * scale)
+    torch.testing.assert_close(gd.grad.cpu().double(), g64.grad, rtol=1e-4, atol=1e-5 * float(g64.grad.abs().max()))
+    torch.testing.assert_close(bd.grad.cpu().double(), b64.grad, rtol=1e-4, atol=1e-5 * float(b64.grad.abs().max()))
+    # dL/dk: a sum over every neuron-step (fp32 terms, fp64 reduction): 1e-4 of the sum of the terms' magnitudes is far
+    # below what a dropped step, a wrong v[t-1] or a missing division by k would change
+    assert float(kd.grad.cpu().double() - k64.grad) == pytest.approx(0.0, abs=1e-4 * max(1.0, float(k64.grad.abs())) + 1e-3)
+    assert abs(float(k64.grad)) > 1e-2
+
+
+def test_parametric_lif_at_the_end_of_the_chains_runs_fused_and_trains_its_parameter(monkeypatch):
+    """A block whose ``qkv_lif`` and ``proj_lif`` are ``ParametricLIFNode``s: both chains stay fused, the spikes are
+    those of the unfused modules (torch's convolution and batch norm around the hip neurons) outside the margin, and
+    ``w.grad`` of both neurons agrees with the unfused path."""
+    from spikingjelly_amd.activation_based.layer import fused
+
+    def make():
+        block = _make_block(64, 2, 71)
+        block.qkv_lif = neuron.ParametricLIFNode(init_tau=2.5, step_mode="m", backend="hip")
+        block.proj_lif = neuron.ParametricLIFNode(init_tau=3.0, step_mode="m", backend="hip")
+        return block.cuda().train()
+
+    fused_block, plain_block = make(), make()
+    ran, real_a, real_b = [], fused.conv_bn_lif, fused.lif_conv_bn_lif
+    monkeypatch.setattr(fused, "conv_bn_lif", lambda *a, **k: (lambda r: ran.append(("qkv", r is not None)) or r)(real_a(*a, **k)))
+    monkeypatch.setattr(fused, "lif_conv_bn_lif", lambda *a, **k: (lambda r: ran.append(("proj", r is not None)) or r)(real_b(*a, **k)))
+    x = seeded_randn((4, 3, 64, 36), 72, 0.0, 2.0).cuda()
+    g = seeded_randn((4, 3, 64, 36), 73).cuda()
+    monkeypatch.setattr(configure, "hip_fuse_conv_bn_lif", True)
+    xa = x.clone().requires_grad_()
+    out_a = fused_block(xa)
+    out_a.backward(g)
+    assert ("qkv", True) in ran and ("proj", True) in ran
+    monkeypatch.setattr(configure, "hip_fuse_conv_bn_lif", False)
+    xb = x.clone().requires_grad_()
+    out_b = plain_block(xb)
+    out_b.backward(g)
+    assert float((out_a.detach() != out_b.detach()).float().mean()) < 2e-3 and 0.02 < float(out_a.detach().mean()) < 0.9
+    for name in ("qkv_lif", "proj_lif"):
+        wa, wb = getattr(fused_block, name).w.grad, getattr(plain_block, name).w.grad
+        assert wa is not None and abs(float(wb)) > 1e-4
+        assert float(wa) == pytest.approx(float(wb), rel=5e-2, abs=1e-3)
+    torch.testing.assert_close(xa.grad, xb.grad, rtol=5e-2, atol=5e-3 * float(xb.grad.abs().max()))
+
+
 def test_bn_lif_bit_packed_spikes_equal_the_dense_ones(C):
     from spikingjelly_amd.activation_based.hip_kernel import neuron_kernel as K
     from spikingjelly_amd.activation_based.hip_kernel.compress import bit_spike_compress
