@@ -696,8 +696,7 @@ def lif_conv_bn_lif(pre_seq: torch.Tensor, pre_v_init: torch.Tensor, weight: tor
     if torch.compiler.is_compiling():
         from . import fused_ops as O
 
-        _eager_only(k)
-        return O.lif_conv_bn_lif(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec)
+        return O.lif_conv_bn_lif(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec, k)
     out = _LifConvBnLif.apply(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec, k)
     return out[0], out[1], out[2]
 
@@ -711,20 +710,13 @@ def lif_conv_bn_lif_supported(pre_seq: torch.Tensor, need_grad: bool) -> bool:
     return (Cin * Lp) % 8 == 0
 
 
-def _eager_only(k):
-    if k is not None:
-        raise NotImplementedError("the fused chain with a parametric LIF has no traceable operator form: run it eagerly "
-                                  "(layer/fused.py steps aside for it while a graph is traced)")
-
-
 def bn_lif(y_seq: torch.Tensor, gamma, beta, v_init: torch.Tensor, bn, spec, k: Optional[torch.Tensor] = None):
     """``y_seq [T, B, C, L]`` (a convolution output) -> ``(spikes, v_last)``.  ``k``: ``sigmoid(w)`` of a parametric LIF
     (one element on the device; its gradient comes back through autograd), in which case ``spec[0]`` is unused."""
     if torch.compiler.is_compiling():
         from . import fused_ops as O
 
-        _eager_only(k)
-        return O.bn_lif(y_seq, gamma, beta, v_init, bn, spec)
+        return O.bn_lif(y_seq, gamma, beta, v_init, bn, spec, k)
     spikes, v_last, _ = _BnLif.apply(y_seq, gamma, beta, v_init, bn, spec, k)
     return spikes, v_last
 
@@ -736,8 +728,7 @@ def conv_bn_lif(x_seq: torch.Tensor, weight: torch.Tensor, gamma, beta, v_init: 
     if torch.compiler.is_compiling():
         from . import fused_ops as O
 
-        _eager_only(k)
-        return O.conv_bn_lif(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, None)
+        return O.conv_bn_lif(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, None, k)
     spikes, v_last, _, _, _ = _ConvBnLif.apply(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, k)
     return spikes, v_last
 
@@ -749,8 +740,7 @@ def conv_bn_lif_ssa(x_seq: torch.Tensor, weight: torch.Tensor, gamma, beta, v_in
     if torch.compiler.is_compiling():
         from . import fused_ops as O
 
-        _eager_only(k)
-        return O.conv_bn_lif(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, (heads, channels_per_head, scale))
+        return O.conv_bn_lif(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, (heads, channels_per_head, scale), k)
     out, v_last, _, _, _, _ = _ConvBnLifSsa.apply(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact,
                                                (heads, channels_per_head, scale), k)
     return out, v_last

@@ -68,11 +68,13 @@ def _write_back(bn, new_mean, new_var) -> None:
 def hip_bn_lif_forward(y: torch.Tensor, gamma: Optional[torch.Tensor], beta: Optional[torch.Tensor], v_init: torch.Tensor,
                        running_mean: Optional[torch.Tensor], running_var: Optional[torch.Tensor], batch_stats: bool,
                        momentum: float, eps: float, tau: float, v_th: float, v_reset: float, flags: int, sg_id: int,
-                       sg_alpha: float) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
-    """``(spikes, v_last, bn_map, new running mean, new running variance)`` (the last two empty when not updated)."""
+                       sg_alpha: float, k: Optional[torch.Tensor] = None
+                       ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(spikes, v_last, bn_map, new running mean, new running variance)`` (the last two empty when not updated).
+    ``k``: ``sigmoid(w)`` of a parametric LIF, one element (``tau`` is then unused)."""
     spec = (tau, v_th, v_reset, flags, sg_id, sg_alpha)
     rm, rv, upd = _updated(batch_stats, running_mean, running_var)
-    spikes, v_last, bn_map = C._BnLif.forward(y, gamma, beta, v_init, (rm, rv, batch_stats, momentum, eps, None), spec)
+    spikes, v_last, bn_map = C._BnLif.forward(y, gamma, beta, v_init, (rm, rv, batch_stats, momentum, eps, None), spec, k)
     return spikes, v_last, bn_map, rm if upd else _e(y), rv if upd else _e(y)
 
 
@@ -82,7 +84,8 @@ def _fake_running(ref, batch_stats, running_mean, running_var):
 
 
 @hip_bn_lif_forward.register_fake
-def _(y, gamma, beta, v_init, running_mean, running_var, batch_stats, momentum, eps, tau, v_th, v_reset, flags, sg_id, sg_alpha):
+def _(y, gamma, beta, v_init, running_mean, running_var, batch_stats, momentum, eps, tau, v_th, v_reset, flags, sg_id, sg_alpha,
+      k=None):
     T, B, Cc, Lp = y.shape
     return (torch.empty_like(y), y.new_empty((B, Cc, Lp)), y.new_empty((4, Cc)),
             *_fake_running(y, batch_stats, running_mean, running_var))
@@ -92,44 +95,50 @@ def _(y, gamma, beta, v_init, running_mean, running_var, batch_stats, momentum, 
 def hip_bn_lif_backward(grad_spikes: Optional[torch.Tensor], grad_v_last: Optional[torch.Tensor], y: torch.Tensor,
                         gamma: Optional[torch.Tensor], v_init: torch.Tensor, bn_map: torch.Tensor, batch_stats: bool,
                         tau: float, v_th: float, v_reset: float, flags: int, sg_id: int, sg_alpha: float,
-                        need_gvi: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+                        need_gvi: bool, k: Optional[torch.Tensor] = None
+                        ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(dy, dgamma, dbeta, grad_v_init or empty, dL/dk or empty)``."""
     spec = (tau, v_th, v_reset, flags, sg_id, sg_alpha)
-    dy, dgamma, dbeta, gvi = C._bn_lif_backward(L.aligned16(y), bn_map, gamma, v_init, spec, batch_stats, grad_spikes,
-                                                grad_v_last, need_gvi)
-    return dy, dgamma.clone(), dbeta.clone(), _or_empty(gvi, y)   # (dgamma and dbeta are rows of one buffer)
+    dy, dgamma, dbeta, gvi, *grad_k = C._bn_lif_backward(L.aligned16(y), bn_map, gamma, v_init, spec, batch_stats, grad_spikes,
+                                                         grad_v_last, need_gvi, False, k)
+    # (dgamma and dbeta are rows of one buffer)
+    return dy, dgamma.clone(), dbeta.clone(), _or_empty(gvi, y), grad_k[0] if grad_k else _e(y)
 
 
 @hip_bn_lif_backward.register_fake
-def _(grad_spikes, grad_v_last, y, gamma, v_init, bn_map, batch_stats, tau, v_th, v_reset, flags, sg_id, sg_alpha, need_gvi):
+def _(grad_spikes, grad_v_last, y, gamma, v_init, bn_map, batch_stats, tau, v_th, v_reset, flags, sg_id, sg_alpha, need_gvi,
+      k=None):
     T, B, Cc, Lp = y.shape
-    return torch.empty_like(y), y.new_empty((Cc,)), y.new_empty((Cc,)), y.new_empty((B, Cc, Lp) if need_gvi else (0,))
+    return (torch.empty_like(y), y.new_empty((Cc,)), y.new_empty((Cc,)), y.new_empty((B, Cc, Lp) if need_gvi else (0,)),
+            y.new_empty((1,) if k is not None else (0,)))
 
 
 def _bn_lif_setup(ctx, inputs, output):
     (y, gamma, beta, v_init, running_mean, running_var, batch_stats, momentum, eps, tau, v_th, v_reset, flags, sg_id,
-     sg_alpha) = inputs
+     sg_alpha, k) = inputs
     ctx.scalars = (batch_stats, tau, v_th, v_reset, flags, sg_id, sg_alpha)
     ctx.has_gamma = gamma is not None
-    ctx.save_for_backward(y, gamma, v_init, output[2])
+    ctx.save_for_backward(y, gamma, v_init, output[2], k)
     ctx.set_materialize_grads(False)
 
 
 def _bn_lif_formula(ctx, grad_spikes, grad_v_last, grad_map, _rm, _rv):
     del grad_map
-    y, gamma, v_init, bn_map = ctx.saved_tensors
+    y, gamma, v_init, bn_map, k = ctx.saved_tensors
     need = ctx.needs_input_grad
-    dy, dgamma, dbeta, gvi = hip_bn_lif_backward(grad_spikes, grad_v_last, y, gamma, v_init, bn_map, *ctx.scalars, bool(need[3]))
+    dy, dgamma, dbeta, gvi, grad_k = hip_bn_lif_backward(grad_spikes, grad_v_last, y, gamma, v_init, bn_map, *ctx.scalars,
+                                                         bool(need[3]), k)
     return (dy if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None, gvi if need[3] else None) + \
-        (None,) * 11
+        (None,) * 11 + (grad_k if k is not None and need[15] else None,)
 
 
 torch.library.register_autograd("sj::hip_bn_lif_forward", _bn_lif_formula, setup_context=_bn_lif_setup)
 
 
-def bn_lif(y_seq, gamma, beta, v_init, bn, spec):
+def bn_lif(y_seq, gamma, beta, v_init, bn, spec, k=None):
     running_mean, running_var, batch_stats, momentum, eps, _ = C._bn_config(bn)
     spikes, v_last, _, new_mean, new_var = hip_bn_lif_forward(y_seq, gamma, beta, v_init, running_mean, running_var, batch_stats,
-                                                              momentum, eps, *spec)
+                                                              momentum, eps, *spec, k)
     _write_back(bn, new_mean, new_var)
     return spikes, v_last
 
@@ -146,7 +155,7 @@ def hip_conv_bn_lif_forward(x_seq: torch.Tensor, weight: torch.Tensor, gamma: Op
                             beta: Optional[torch.Tensor], v_init: torch.Tensor, running_mean: Optional[torch.Tensor],
                             running_var: Optional[torch.Tensor], batch_stats: bool, momentum: float, eps: float, tau: float,
                             v_th: float, v_reset: float, flags: int, sg_id: int, sg_alpha: float, x_exact: bool, terms: int,
-                            heads: int, cph: int, scale: float
+                            heads: int, cph: int, scale: float, k: Optional[torch.Tensor] = None
                             ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
                                        torch.Tensor, torch.Tensor]:
     """``(out, v_last, y, bn_map, bits, x_amax, new running mean, new running variance)``: ``out`` is the dense spikes
@@ -158,14 +167,14 @@ def hip_conv_bn_lif_forward(x_seq: torch.Tensor, weight: torch.Tensor, gamma: Op
     bn = (rm, rv, batch_stats, momentum, eps, None)
     new = (rm if upd else _e(x_seq), rv if upd else _e(x_seq))
     if heads == 0:
-        spikes, v_last, y, bn_map, x_amax = C._ConvBnLif.forward(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact)
+        spikes, v_last, y, bn_map, x_amax = C._ConvBnLif.forward(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, k)
         return (spikes, v_last, y, bn_map, torch.empty((0,), dtype=torch.uint8, device=x_seq.device), x_amax, *new)
-    return (*C._ConvBnLifSsa.forward(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, (heads, cph, scale)), *new)
+    return (*C._ConvBnLifSsa.forward(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact, (heads, cph, scale), k), *new)
 
 
 @hip_conv_bn_lif_forward.register_fake
 def _(x_seq, weight, gamma, beta, v_init, running_mean, running_var, batch_stats, momentum, eps, tau, v_th, v_reset,
-      flags, sg_id, sg_alpha, x_exact, terms, heads, cph, scale):
+      flags, sg_id, sg_alpha, x_exact, terms, heads, cph, scale, k=None):
     T, B, _, Lp = x_seq.shape
     Cout = weight.shape[0]
     out = x_seq.new_empty((T, B, Cout, Lp) if heads == 0 else (T * B, heads, cph, Lp))
@@ -180,53 +189,57 @@ def hip_conv_bn_lif_backward(grad_out: Optional[torch.Tensor], grad_v_last: Opti
                              weight: torch.Tensor, gamma: Optional[torch.Tensor], v_init: torch.Tensor, y: torch.Tensor,
                              bn_map: torch.Tensor, bits: torch.Tensor, x_amax: torch.Tensor, batch_stats: bool, tau: float,
                              v_th: float, v_reset: float, flags: int, sg_id: int, sg_alpha: float, x_exact: bool, terms: int,
-                             heads: int, cph: int, scale: float, need_dx: bool, need_dw: bool, need_gvi: bool
-                             ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+                             heads: int, cph: int, scale: float, need_dx: bool, need_dw: bool, need_gvi: bool,
+                             k: Optional[torch.Tensor] = None
+                             ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     if terms != C._terms():
         raise RuntimeError("configure.hip_conv_split / hip_conv_terms changed after this call was compiled")
     spec = (tau, v_th, v_reset, flags, sg_id, sg_alpha)
     ssa = (heads, cph, scale) if heads else None
-    dx, dw, dgamma, dbeta, gvi = C._conv_chain_backward(L.aligned16(x_seq), weight, gamma, v_init, y, bn_map, bits, x_amax, spec,
-                                                        batch_stats, x_exact, ssa, grad_out, grad_v_last, need_dx, need_dw,
-                                                        need_gvi)
-    return _or_empty(dx, y), _or_empty(dw, y), dgamma.clone(), dbeta.clone(), _or_empty(gvi, y)
+    dx, dw, dgamma, dbeta, gvi, *grad_k = C._conv_chain_backward(L.aligned16(x_seq), weight, gamma, v_init, y, bn_map, bits, x_amax,
+                                                                 spec, batch_stats, x_exact, ssa, grad_out, grad_v_last, need_dx,
+                                                                 need_dw, need_gvi, k)
+    return (_or_empty(dx, y), _or_empty(dw, y), dgamma.clone(), dbeta.clone(), _or_empty(gvi, y),
+            grad_k[0] if grad_k else _e(y))
 
 
 @hip_conv_bn_lif_backward.register_fake
 def _(grad_out, grad_v_last, x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax, batch_stats, tau, v_th, v_reset, flags,
-      sg_id, sg_alpha, x_exact, terms, heads, cph, scale, need_dx, need_dw, need_gvi):
+      sg_id, sg_alpha, x_exact, terms, heads, cph, scale, need_dx, need_dw, need_gvi, k=None):
     T, B, Cout, Lp = y.shape
     return (torch.empty_like(x_seq) if need_dx else _e(y), y.new_empty(tuple(weight.shape[:2])) if need_dw else _e(y),
-            y.new_empty((Cout,)), y.new_empty((Cout,)), y.new_empty((B, Cout, Lp) if need_gvi else (0,)))
+            y.new_empty((Cout,)), y.new_empty((Cout,)), y.new_empty((B, Cout, Lp) if need_gvi else (0,)),
+            y.new_empty((1,) if k is not None else (0,)))
 
 
 def _conv_setup(ctx, inputs, output):
     (x_seq, weight, gamma, beta, v_init, running_mean, running_var, batch_stats, momentum, eps, tau, v_th, v_reset,
-     flags, sg_id, sg_alpha, x_exact, terms, heads, cph, scale) = inputs
+     flags, sg_id, sg_alpha, x_exact, terms, heads, cph, scale, k) = inputs
     ctx.scalars = (batch_stats, tau, v_th, v_reset, flags, sg_id, sg_alpha, x_exact, terms, heads, cph, scale)
-    ctx.save_for_backward(x_seq, weight, gamma, v_init, output[2], output[3], output[4], output[5])
+    ctx.save_for_backward(x_seq, weight, gamma, v_init, output[2], output[3], output[4], output[5], k)
     ctx.set_materialize_grads(False)
 
 
 def _conv_formula(ctx, grad_out, grad_v_last, _y, _map, _bits, _amax, _rm, _rv):
-    x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax = ctx.saved_tensors
+    x_seq, weight, gamma, v_init, y, bn_map, bits, x_amax, k = ctx.saved_tensors
     need = ctx.needs_input_grad
-    dx, dw, dgamma, dbeta, gvi = hip_conv_bn_lif_backward(grad_out, grad_v_last, x_seq, weight, gamma, v_init, y, bn_map, bits,
-                                                          x_amax, *ctx.scalars, bool(need[0]), bool(need[1]), bool(need[4]))
+    dx, dw, dgamma, dbeta, gvi, grad_k = hip_conv_bn_lif_backward(grad_out, grad_v_last, x_seq, weight, gamma, v_init, y, bn_map,
+                                                                  bits, x_amax, *ctx.scalars, bool(need[0]), bool(need[1]),
+                                                                  bool(need[4]), k)
     dw = dw.view(weight.shape) if need[1] else None
     return (dx if need[0] else None, dw, dgamma if need[2] else None, dbeta if need[3] else None,
-            gvi if need[4] else None) + (None,) * 16
+            gvi if need[4] else None) + (None,) * 16 + (grad_k if k is not None and need[21] else None,)
 
 
 torch.library.register_autograd("sj::hip_conv_bn_lif_forward", _conv_formula, setup_context=_conv_setup)
 
 
-def conv_bn_lif(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact: bool, ssa):
+def conv_bn_lif(x_seq, weight, gamma, beta, v_init, bn, spec, x_exact: bool, ssa, k=None):
     """``(spikes, v_last)``, or with ``ssa = (heads, channels per head, scale)`` ``(contraction output, v_last)``."""
     running_mean, running_var, batch_stats, momentum, eps, _ = C._bn_config(bn)
     heads, cph, scale = ssa if ssa is not None else (0, 0, 0.0)
     out = hip_conv_bn_lif_forward(x_seq, weight, gamma, beta, v_init, running_mean, running_var, batch_stats, momentum,
-                                  eps, *spec, x_exact, C._terms(), heads, cph, scale)
+                                  eps, *spec, x_exact, C._terms(), heads, cph, scale, k)
     _write_back(bn, out[6], out[7])
     return out[0], out[1]
 
@@ -241,7 +254,7 @@ def hip_lif_conv_bn_lif_forward(pre_seq: torch.Tensor, pre_v_init: torch.Tensor,
                                 batch_stats: bool, momentum: float, eps: float,
                                 pre_tau: float, pre_v_th: float, pre_v_reset: float, pre_flags: int, pre_sg_id: int,
                                 pre_sg_alpha: float, tau: float, v_th: float, v_reset: float, flags: int, sg_id: int,
-                                sg_alpha: float, terms: int
+                                sg_alpha: float, terms: int, k: Optional[torch.Tensor] = None
                                 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
                                            torch.Tensor, torch.Tensor]:
     """``(spikes, v_last, first neuron's v_last, y, bn_map, bits, new running mean, new running variance)``."""
@@ -251,13 +264,13 @@ def hip_lif_conv_bn_lif_forward(pre_seq: torch.Tensor, pre_v_init: torch.Tensor,
     out = C._LifConvBnLif.forward(pre_seq, pre_v_init, weight, gamma, beta, v_init,
                                   (rm, rv, batch_stats, momentum, eps, None),
                                   (pre_tau, pre_v_th, pre_v_reset, pre_flags, pre_sg_id, pre_sg_alpha),
-                                  (tau, v_th, v_reset, flags, sg_id, sg_alpha))
+                                  (tau, v_th, v_reset, flags, sg_id, sg_alpha), k)
     return (*out, rm if upd else _e(pre_seq), rv if upd else _e(pre_seq))
 
 
 @hip_lif_conv_bn_lif_forward.register_fake
 def _(pre_seq, pre_v_init, weight, gamma, beta, v_init, running_mean, running_var, batch_stats, momentum, eps, pre_tau,
-      pre_v_th, pre_v_reset, pre_flags, pre_sg_id, pre_sg_alpha, tau, v_th, v_reset, flags, sg_id, sg_alpha, terms):
+      pre_v_th, pre_v_reset, pre_flags, pre_sg_id, pre_sg_alpha, tau, v_th, v_reset, flags, sg_id, sg_alpha, terms, k=None):
     T, B, Cin, Lp = pre_seq.shape
     Cout = weight.shape[0]
     new = pre_seq.new_empty
@@ -273,54 +286,57 @@ def hip_lif_conv_bn_lif_backward(grad_spikes: Optional[torch.Tensor], grad_v_las
                                  bn_map: torch.Tensor, bits: torch.Tensor, batch_stats: bool, pre_tau: float, pre_v_th: float,
                                  pre_v_reset: float, pre_flags: int, pre_sg_id: int, pre_sg_alpha: float, tau: float,
                                  v_th: float, v_reset: float, flags: int, sg_id: int, sg_alpha: float, terms: int,
-                                 need_gx: bool, need_gpv: bool, need_dw: bool, need_gvi: bool
-                                 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+                                 need_gx: bool, need_gpv: bool, need_dw: bool, need_gvi: bool, k: Optional[torch.Tensor] = None
+                                 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
+                                            torch.Tensor]:
     if terms != C._terms():
         raise RuntimeError("configure.hip_conv_split / hip_conv_terms changed after this call was compiled")
-    gx, gpv, dw, dgamma, dbeta, gvi = C._lif_conv_chain_backward(
+    gx, gpv, dw, dgamma, dbeta, gvi, *grad_k = C._lif_conv_chain_backward(
         L.aligned16(pre_seq), pre_v_init, weight, gamma, v_init, y, bn_map, bits,
         (pre_tau, pre_v_th, pre_v_reset, pre_flags, pre_sg_id, pre_sg_alpha), (tau, v_th, v_reset, flags, sg_id, sg_alpha),
-        batch_stats, grad_spikes, grad_v_last, grad_pre_v_last, need_gx, need_gpv, need_dw, need_gvi)
-    return _or_empty(gx, y), _or_empty(gpv, y), _or_empty(dw, y), dgamma.clone(), dbeta.clone(), _or_empty(gvi, y)
+        batch_stats, grad_spikes, grad_v_last, grad_pre_v_last, need_gx, need_gpv, need_dw, need_gvi, k)
+    return (_or_empty(gx, y), _or_empty(gpv, y), _or_empty(dw, y), dgamma.clone(), dbeta.clone(), _or_empty(gvi, y),
+            grad_k[0] if grad_k else _e(y))
 
 
 @hip_lif_conv_bn_lif_backward.register_fake
 def _(grad_spikes, grad_v_last, grad_pre_v_last, pre_seq, pre_v_init, weight, gamma, v_init, y, bn_map, bits, batch_stats,
       pre_tau, pre_v_th, pre_v_reset, pre_flags, pre_sg_id, pre_sg_alpha, tau, v_th, v_reset, flags, sg_id, sg_alpha, terms,
-      need_gx, need_gpv, need_dw, need_gvi):
+      need_gx, need_gpv, need_dw, need_gvi, k=None):
     T, B, Cin, Lp = pre_seq.shape
     Cout = weight.shape[0]
     new = y.new_empty
     return (torch.empty_like(pre_seq) if need_gx else _e(y), new((B, Cin, Lp)) if need_gpv else _e(y),
-            new((Cout, Cin)) if need_dw else _e(y), new((Cout,)), new((Cout,)), new((B, Cout, Lp)) if need_gvi else _e(y))
+            new((Cout, Cin)) if need_dw else _e(y), new((Cout,)), new((Cout,)), new((B, Cout, Lp)) if need_gvi else _e(y),
+            new((1,) if k is not None else (0,)))
 
 
 def _lif_conv_setup(ctx, inputs, output):
     (pre_seq, pre_v_init, weight, gamma, beta, v_init, running_mean, running_var, batch_stats, momentum, eps,
-     *scalars) = inputs
+     *scalars, k) = inputs
     ctx.scalars = (batch_stats, *scalars)
-    ctx.save_for_backward(pre_seq, pre_v_init, weight, gamma, v_init, output[3], output[4], output[5])
+    ctx.save_for_backward(pre_seq, pre_v_init, weight, gamma, v_init, output[3], output[4], output[5], k)
     ctx.set_materialize_grads(False)
 
 
 def _lif_conv_formula(ctx, grad_spikes, grad_v_last, grad_pre_v_last, _y, _map, _bits, _rm, _rv):
-    pre_seq, pre_v_init, weight, gamma, v_init, y, bn_map, bits = ctx.saved_tensors
+    pre_seq, pre_v_init, weight, gamma, v_init, y, bn_map, bits, k = ctx.saved_tensors
     need = ctx.needs_input_grad
-    gx, gpv, dw, dgamma, dbeta, gvi = hip_lif_conv_bn_lif_backward(
+    gx, gpv, dw, dgamma, dbeta, gvi, grad_k = hip_lif_conv_bn_lif_backward(
         grad_spikes, grad_v_last, grad_pre_v_last, pre_seq, pre_v_init, weight, gamma, v_init, y, bn_map, bits, *ctx.scalars,
-        bool(need[0]), bool(need[1]), bool(need[2]), bool(need[5]))
+        bool(need[0]), bool(need[1]), bool(need[2]), bool(need[5]), k)
     dw = dw.view(weight.shape) if need[2] else None
     return (gx if need[0] else None, gpv if need[1] else None, dw, dgamma if need[3] else None, dbeta if need[4] else None,
-            gvi if need[5] else None) + (None,) * 18
+            gvi if need[5] else None) + (None,) * 18 + (grad_k if k is not None and need[24] else None,)
 
 
 torch.library.register_autograd("sj::hip_lif_conv_bn_lif_forward", _lif_conv_formula, setup_context=_lif_conv_setup)
 
 
-def lif_conv_bn_lif(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec):
+def lif_conv_bn_lif(pre_seq, pre_v_init, weight, gamma, beta, v_init, bn, pre_spec, spec, k=None):
     running_mean, running_var, batch_stats, momentum, eps, _ = C._bn_config(bn)
     out = hip_lif_conv_bn_lif_forward(pre_seq, pre_v_init, weight, gamma, beta, v_init, running_mean, running_var,
-                                      batch_stats, momentum, eps, *pre_spec, *spec, C._terms())
+                                      batch_stats, momentum, eps, *pre_spec, *spec, C._terms(), k)
     _write_back(bn, out[6], out[7])
     return out[0], out[1], out[2]
 

@@ -84,11 +84,8 @@ def _lif_spec(node: nn.Module, x_like: torch.Tensor, need_grad: bool):
 
 
 def _chain_neuron(node: nn.Module) -> bool:
-    """The neuron at the end of a fused chain: a plain LIF, or a parametric LIF outside a traced graph (the operator
-    forms of the chain take no learnable ``k``)."""
-    if type(node) is neuron.ParametricLIFNode:
-        return not torch.compiler.is_compiling()
-    return type(node) is neuron.LIFNode
+    """The neuron at the end of a fused chain: a plain or a parametric LIF."""
+    return type(node) in (neuron.LIFNode, neuron.ParametricLIFNode)
 
 
 def _neuron_k(node: nn.Module, x_like: torch.Tensor) -> Optional[torch.Tensor]:

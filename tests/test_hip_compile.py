@@ -159,9 +159,13 @@ def test_inductor_compiles_linear_then_hip_node(shape):
                                atol=1e-3 * float(eager.fc.weight.grad.abs().max()))
 
 
-def _attention_block(dim, heads, seed):
+def _attention_block(dim, heads, seed, parametric=False):
     torch.manual_seed(seed)
-    block = layer.SpikingSelfAttention(dim, heads, backend="hip").cuda().train()
+    block = layer.SpikingSelfAttention(dim, heads, backend="hip")
+    if parametric:  # the neurons at the end of the two chains learn their time constant
+        block.qkv_lif = neuron.ParametricLIFNode(init_tau=2.5, step_mode="m", backend="hip")
+        block.proj_lif = neuron.ParametricLIFNode(init_tau=3.0, step_mode="m", backend="hip")
+    block = block.cuda().train()
     with torch.no_grad():
         block.qkv_conv_bn[1].weight.fill_(2.0)
         block.proj_conv_bn[1].weight.fill_(3.0)
@@ -175,8 +179,9 @@ def _launch_counts(L):
 
 
 @pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
-@pytest.mark.parametrize("dim,heads,T,B,tokens", [(64, 2, 4, 2, 36), (384, 12, 4, 2, 196)])
-def test_compiled_attention_block_keeps_the_fused_chain(backend, dim, heads, T, B, tokens):
+@pytest.mark.parametrize("dim,heads,T,B,tokens,parametric", [(64, 2, 4, 2, 36, False), (384, 12, 4, 2, 196, False),
+                                                             (64, 2, 4, 2, 36, True)])
+def test_compiled_attention_block_keeps_the_fused_chain(backend, dim, heads, T, B, tokens, parametric):
     """``torch.compile(SpikingSelfAttention(..., backend='hip'), fullgraph=True)`` launches the kernels of the fused
     convolution / batch norm / LIF chain that the eager module launches (counted by the library's own launch counters:
     the convolution GEMMs, the batch-norm + LIF kernels, the contraction), in forward and backward, with results equal
@@ -187,7 +192,7 @@ def test_compiled_attention_block_keeps_the_fused_chain(backend, dim, heads, T, 
 
     if backend == "inductor" and not _triton_available():
         pytest.skip("the inductor backend generates triton kernels and triton is not importable")
-    eager, traced = _attention_block(dim, heads, 7), _attention_block(dim, heads, 7)
+    eager, traced = _attention_block(dim, heads, 7, parametric), _attention_block(dim, heads, 7, parametric)
     fn = torch.compile(traced, fullgraph=True, backend=backend)
     x = seeded_randn((T, B, dim, tokens), 19).cuda()
     g = seeded_randn((T, B, dim, tokens), 20).cuda()
@@ -214,6 +219,11 @@ def test_compiled_attention_block_keeps_the_fused_chain(backend, dim, heads, T, 
     assert float(out_e.mean()) > 0.02
     assert torch.equal(out_c, out_e) and torch.equal(gx_c, gx_e)
     for a, b in zip(gp_c, gp_e):
-        assert torch.equal(a, b)
+        if a.dim() == 0:  # a parametric LIF's w: dL/dk times the sigmoid's derivative, which the code generator may fuse
+            torch.testing.assert_close(a, b, rtol=1e-5, atol=0.0)
+        else:
+            assert torch.equal(a, b)
     for a, b in zip(buf_c, buf_e):   # running statistics and the batch counter
         assert torch.equal(a, b)
+    if parametric:
+        assert abs(float(eager.qkv_lif.w.grad)) > 0 and abs(float(eager.proj_lif.w.grad)) > 0

@@ -154,6 +154,16 @@ def test_fused_chain_ops():
     pre_v0 = torch.zeros((2, 8, 8), device="cuda")
     torch.library.opcheck(O.hip_lif_conv_bn_lif_forward,
                           (pre, pre_v0, w, gamma, beta, v0, rm, rv, True, 0.1, 1e-5, *spec, *spec, terms), test_utils=TESTS)
+    # the same chains ending in a parametric LIF: k = sigmoid(w) as one more (differentiable) tensor argument
+    k = torch.tensor([0.4], device="cuda", requires_grad=True)
+    plif = (0.0, *spec[1:])
+    torch.library.opcheck(O.hip_bn_lif_forward, (y, gamma, beta, v0, rm, rv, True, 0.1, 1e-5, *plif, k), test_utils=TESTS)
+    for heads, cph in ((0, 0), (2, 2)):
+        torch.library.opcheck(O.hip_conv_bn_lif_forward,
+                              (x, w, gamma, beta, v0, rm, rv, True, 0.1, 1e-5, *plif, False, terms, heads, cph, 0.125, k),
+                              test_utils=TESTS)
+    torch.library.opcheck(O.hip_lif_conv_bn_lif_forward,
+                          (pre, pre_v0, w, gamma, beta, v0, rm, rv, True, 0.1, 1e-5, *spec, *plif, terms, k), test_utils=TESTS)
     x2 = seeded_randn((3, 2 * 3 * 2 * 2 * 8), 37, 0.6, 1.0).cuda().requires_grad_()   # B = 2, 3 x 2 heads x 2 channels x 8 tokens
     torch.library.opcheck(O.hip_lif_ssa_forward, (x2, torch.zeros(x2.shape[1], device="cuda"), *spec, 6, 2, 2, 8, 0.125),
                           test_utils=TESTS)
