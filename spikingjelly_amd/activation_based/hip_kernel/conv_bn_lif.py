@@ -296,6 +296,12 @@ def _lif_params(spec, flags_extra: int = 0) -> L.NeuronParams:
     return K._params(tau, v_th, v_reset, sg_alpha, sg_id, flags | flags_extra)
 
 
+def _neuron_id(spec, k) -> int:
+    """The neuron a spec stands for: a time constant of 0 means there is none, i.e. an IF neuron (a parametric LIF, whose
+    spec carries 0 as well, brings its ``k`` as a tensor and is launched through its own entry points)."""
+    return L.NEURON_IF if spec[0] == 0.0 and k is None else L.NEURON_LIF
+
+
 def _bn_lif_forward(y: torch.Tensor, bn_map: torch.Tensor, v_init: torch.Tensor, spec, packed: bool,
                     k: Optional[torch.Tensor] = None):
     """``y [T, B, C, L]`` -> (spikes ``[T, B, C, L]`` fp32 or the bit-packed byte array, ``v_last [B, C, L]``).
@@ -311,7 +317,7 @@ def _bn_lif_forward(y: torch.Tensor, bn_map: torch.Tensor, v_init: torch.Tensor,
     k_keep, k_ptr = K._k_pointer(k, y)
     with torch.cuda.device(y.device):
         if k is None:
-            rc = L.load().sjhip_bn_lif_forward(L.NEURON_LIF, ctypes.byref(params), T, B, C, Lp, y.data_ptr(), bn_map[0].data_ptr(),
+            rc = L.load().sjhip_bn_lif_forward(_neuron_id(spec, k), ctypes.byref(params), T, B, C, Lp, y.data_ptr(), bn_map[0].data_ptr(),
                                                bn_map[1].data_ptr(), v_keep.data_ptr(), None if packed else spikes.data_ptr(),
                                                spikes.data_ptr() if packed else None, v_last.data_ptr(), _stream(y))
         else:
@@ -346,7 +352,7 @@ def _bn_lif_backward(y: torch.Tensor, bn_map: torch.Tensor, gamma, v_init: torch
         stream = _stream(y)
         grad_k = None
         if k is None:
-            L.check(lib.sjhip_bn_lif_backward(L.NEURON_LIF, ctypes.byref(params), T, B, C, Lp, y.data_ptr(), bn_map[0].data_ptr(),
+            L.check(lib.sjhip_bn_lif_backward(_neuron_id(spec, k), ctypes.byref(params), T, B, C, Lp, y.data_ptr(), bn_map[0].data_ptr(),
                                               bn_map[1].data_ptr(), v_keep.data_ptr(), grad_spikes.data_ptr(), L.ptr(grad_v_last),
                                               g.data_ptr(), L.ptr(grad_v_init), partial.data_ptr(), stream), "bn_lif_backward")
         else:
@@ -378,7 +384,7 @@ def _bn_lif_backward(y: torch.Tensor, bn_map: torch.Tensor, gamma, v_init: torch
 # autograd
 # ------------------------------------------------------------------------------------------------
 # bn: (running_mean | None, running_var | None, batch_stats, momentum, eps[, num_batches_tracked | None])
-# lif spec: (tau, v_threshold, v_reset, flags, sg_id, sg_alpha)
+# lif spec: (tau, v_threshold, v_reset, flags, sg_id, sg_alpha); tau = 0: an IF neuron, or with k a parametric LIF
 def _bn_config(bn):
     """The batch-norm tuple with its optional sixth element (the counter of batches, incremented by the launch that
     updates the running statistics)."""

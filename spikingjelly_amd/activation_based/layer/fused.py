@@ -77,15 +77,16 @@ def _lif_spec(node: nn.Module, x_like: torch.Tensor, need_grad: bool):
     from ..hip_kernel.surrogate_registry import resolve_sg_hip_id_and_alpha
 
     soft = node.v_reset is None
-    flags = K._flags(soft, node.detach_reset, node.decay_input, F._hip_mode_flags(x_like))
+    flags = K._flags(soft, node.detach_reset, getattr(node, "decay_input", False), F._hip_mode_flags(x_like))
     sg_id, sg_alpha = resolve_sg_hip_id_and_alpha(node.surrogate_function) if need_grad else (0, 0.0)
-    tau = 0.0 if type(node) is neuron.ParametricLIFNode else float(node.tau)  # (a parametric LIF's k travels as a tensor)
+    # (no time constant in the spec: an IF neuron has none, a parametric LIF's k travels as a tensor)
+    tau = float(node.tau) if type(node) is neuron.LIFNode else 0.0
     return (tau, node.v_threshold, 0.0 if soft else float(node.v_reset), flags, sg_id, sg_alpha)
 
 
 def _chain_neuron(node: nn.Module) -> bool:
-    """The neuron at the end of a fused chain: a plain or a parametric LIF."""
-    return type(node) in (neuron.LIFNode, neuron.ParametricLIFNode)
+    """The neuron at the end of a fused chain: an IF neuron, a plain or a parametric LIF."""
+    return type(node) in (neuron.IFNode, neuron.LIFNode, neuron.ParametricLIFNode)
 
 
 def _neuron_k(node: nn.Module, x_like: torch.Tensor) -> Optional[torch.Tensor]:

@@ -621,6 +621,59 @@ def test_bn_plif_against_float64(C, T, B, Cc, Lp, v_reset, decay_input, init_tau
     assert abs(float(k64.grad)) > 1e-2
 
 
+@pytest.mark.parametrize("T,B,Cc,Lp", [(4, 3, 10, 12), (16, 2, 6, 260), (4, 2, 12, 196), (20, 2, 5, 36)])
+@pytest.mark.parametrize("v_reset,sg", [(0.0, "sigmoid"), (None, "atan")])
+def test_bn_if_against_float64(C, T, B, Cc, Lp, v_reset, sg):
+    """Batch norm + IF neuron (a spec without a time constant) against the float64 oracle (functional/neuron.py:242-312)."""
+    from spikingjelly_amd.activation_based.hip_kernel import neuron_kernel as K
+
+    gamma, beta = seeded_randn((Cc,), 232, 0.5, 0.1), seeded_randn((Cc,), 233, 0.3, 0.2)
+    gs = seeded_randn((T, B, Cc, Lp), 236)
+    alpha = no.SG_DEFAULT_ALPHA[sg]
+    detach = v_reset is None
+    start = 0.0 if v_reset is None else v_reset
+    for seed in range(231, 3300, 100):
+        y = seeded_randn((T, B, Cc, Lp), seed, 0.4, 1.5)
+        y64, g64, b64 = y.double().requires_grad_(), gamma.double().requires_grad_(), beta.double().requires_grad_()
+        z, _, _ = co.batch_norm(y64, g64, b64, torch.zeros(Cc, dtype=torch.float64), torch.ones(Cc, dtype=torch.float64), True)
+        s64, v64, h64 = no.multi_step("if", z.flatten(1), torch.full((B * Cc * Lp,), start, dtype=torch.float64), None, False, 1.0,
+                                      v_reset, no.surrogate(sg, alpha), detach)
+        if _no_borderline(h64.detach(), 1.0):
+            break
+    else:
+        pytest.fail("no input without a neuron within the margin of the threshold")
+    s64.backward(gs.double().flatten(1))
+    soft = v_reset is None
+    spec = (0.0, 1.0, 0.0 if soft else v_reset, K._flags(soft, detach, False, 0), no.SG_IDS[sg], alpha)
+    yd, gd, bd = y.cuda().requires_grad_(), gamma.cuda().requires_grad_(), beta.cuda().requires_grad_()
+    v0 = torch.full((1,), start, device="cuda").expand(B, Cc, Lp)
+    spikes, v_last = C.bn_lif(yd, gd, bd, v0, (torch.zeros(Cc, device="cuda"), torch.ones(Cc, device="cuda"), True, 0.1, 1e-5), spec)
+    spikes.backward(gs.cuda())
+    assert torch.equal(spikes.detach().cpu().double().flatten(1), s64.detach())
+    torch.testing.assert_close(v_last.detach().cpu().double().flatten(), v64[-1].detach(), rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(yd.grad.cpu().double(), y64.grad, rtol=1e-4, atol=1e-5 * float(y64.grad.abs().max()))
+    torch.testing.assert_close(gd.grad.cpu().double(), g64.grad, rtol=1e-4, atol=1e-5 * float(g64.grad.abs().max()))
+    torch.testing.assert_close(bd.grad.cpu().double(), b64.grad, rtol=1e-4, atol=1e-5 * float(b64.grad.abs().max()))
+
+
+def test_if_neuron_at_the_end_of_a_chain_runs_fused(monkeypatch):
+    """``Conv1d(k=1) -> BatchNorm1d -> IFNode``: fused, and equal to the modules called one by one outside the margin."""
+    from spikingjelly_amd.activation_based.layer import fused
+
+    torch.manual_seed(5)
+    conv, bn = nn.Conv1d(32, 48, 1, bias=False).cuda(), nn.BatchNorm1d(48).cuda()
+    with torch.no_grad():
+        bn.weight.fill_(0.6)
+        bn.bias.fill_(0.3)
+    node = neuron.IFNode(step_mode="m", backend="hip").cuda()
+    x = seeded_randn((4, 3, 32, 36), 6, 0.0, 1.0).cuda()
+    out = fused.conv_bn_lif(x.clone().requires_grad_(), conv, bn, node)
+    assert out is not None and 0.02 < float(out.detach().mean()) < 0.9
+    functional.reset_net(node)
+    ref = node(bn(conv(x.flatten(0, 1))).view(4, 3, 48, 36))
+    assert float((out.detach() != ref.detach()).float().mean()) < 1e-3
+
+
 def test_parametric_lif_at_the_end_of_the_chains_runs_fused_and_trains_its_parameter(monkeypatch):
     """A block whose ``qkv_lif`` and ``proj_lif`` are ``ParametricLIFNode``s: both chains stay fused, the spikes are
     those of the unfused modules (torch's convolution and batch norm around the hip neurons) outside the margin, and
