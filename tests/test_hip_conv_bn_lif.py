@@ -526,7 +526,7 @@ def _no_borderline(h, v_th):
 
 # (more than 16 steps: the backward walks the sequence in pieces of 16, one kernel variant per row shape)
 @pytest.mark.parametrize("T,B,Cc,Lp", [(4, 3, 10, 12), (1, 2, 5, 4), (7, 2, 33, 20), (16, 2, 6, 260), (4, 2, 12, 196),
-                                       (17, 2, 5, 36), (33, 1, 6, 196), (40, 1, 3, 260), (64, 2, 3, 8)])
+                                       (17, 2, 5, 36), (33, 1, 6, 196), (40, 1, 3, 260), (64, 2, 3, 8), (256, 1, 2, 196), (250, 1, 3, 16)])
 @pytest.mark.parametrize("training", [True, False])
 @pytest.mark.parametrize("v_reset,decay_input,tau,sg", [(0.0, True, 2.0, "sigmoid"), (None, False, 3.0, "atan"), (-0.2, True, 2.5, "erf")])
 def test_bn_lif_against_float64(C, T, B, Cc, Lp, training, v_reset, decay_input, tau, sg):
