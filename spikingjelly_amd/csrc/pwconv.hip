@@ -68,6 +68,7 @@ namespace sjhip {
 
 namespace {
 
+
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -99,6 +100,9 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 // one tile in flight instead of two it fits without spilling and takes the same 244 us, and the attention block's
 // step 1.50 instead of 1.46 ms.
 constexpr int pw_waves(bool h) { return h ? SJHIP_PW_F16_WAVES : 2; }
+#ifndef SJHIP_PW_ROWS
+#define SJHIP_PW_ROWS 1
+#endif
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   bf16x2 p;
@@ -726,6 +730,250 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
   }
 }
 
+// LDS of pw_gemm_rows_kernel: two B tiles (or the output staging of the epilogue, whichever is larger), then 128 floats
+constexpr unsigned rows_inverse_offset(int tb) { return 2u * tb * kRowPlane > kOutLds ? 2u * tb * kRowPlane : kOutLds; }
+
+// pw_gemm_rows_kernel: the same product, term order and batch-norm sums as pw_gemm_kernel<2, TB, true, kBFloat> (bit for
+// bit), laid out for what a compute unit can move.  Measured per compute unit: LDS reads of 16 bytes per lane run at
+// 256 bytes per cycle but writes at 64-78, and the vector memory path issues one wavefront load of 8 or 16 bytes per lane
+// every 16 cycles (58 bytes per cycle from L1), so in pw_gemm_kernel a K step of a block costs about as many cycles of LDS
+// (16 KB of A and 16 KB of B written, 64 KB read) and of the load path (32 eight-byte loads of B, 16 of A) as of the matrix
+// cores (768 per SIMD).  Here
+//   * a wavefront owns 32 rows of the tile and all 128 columns, and fetches its A fragments straight from the weight
+//     planes (the 16 bytes a lane needs are contiguous in the tile-ordered planes): A never passes through LDS and no two
+//     wavefronts fetch the same fragment;
+//   * B is fetched as 16-byte pieces of a k row (four positions of one sample; L is a multiple of 4), half the load
+//     instructions, split, and stored as it lies in memory (k rows of 128 columns); the wavefronts fetch their
+//     fragments with the transposing LDS read, as pw_gemm_kernel does for term planes;
+//   * two B tiles alternate in LDS, so a K step has one barrier.
+// Per K step of a block: 16 KB written to and 64 KB read from LDS, 16 + 16 load instructions; 146 registers, three
+// wavefronts per SIMD.
+template <int TB>
+__global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) pw_gemm_rows_kernel(const PwGemmArgs a) {
+  constexpr int TA = 2;
+  constexpr int kBuf = TB * kRowPlane;  // one B tile: [TB][32 k][kPlanePitch]
+  extern __shared__ __align__(16) uint8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t logical = xcd_order(blockIdx.x, gridDim.x);
+  const int mb = (int)(logical % a.m_blocks);
+  const int64_t nb = logical / a.m_blocks;
+  const int64_t j0 = nb * kTile;
+  const int M = a.M, K = a.K, L = a.L;
+  const int steps = a.K_pad / kTileK;
+
+  // the inverse row scales of the tile wait in LDS (beyond the operand tiles) for the epilogue
+  float *inverse_lds = reinterpret_cast<float *>(lds + rows_inverse_offset(TB));
+  const float inverse_mine = tid < kTile ? a.a_inverse[mb * kTile + tid] : 0.0f;
+
+  // A: lane (r, g) wants k chunk 2 ks + g (eight k, 16 bytes) of row r of the wavefront's 32 rows
+  const char *a_base = reinterpret_cast<const char *>(a.a_planes) + (int64_t)mb * steps * (kTile * kTileK * 2);
+  const uint32_t a_lane = (uint32_t)(((wave * 32 + (lane & 31)) * kTileK + (lane >> 5) * 8) * 2);
+  // B: the 16 bytes of columns 4 (tid % 32) .. + 3 in the k rows tid / 32 + 8 i
+  const int q4 = tid & 31, kr = tid >> 5;
+  const int64_t jc = j0 + 4 * q4;
+  const bool col_ok = jc < a.ncols;
+  uint32_t b_off = 0;
+  if (col_ok) {
+    const int64_t s = jc / L;
+    b_off = (uint32_t)(((s * K) * (int64_t)L + (jc - s * L)) * 4);
+  }
+  const uint32_t row_bytes = (uint32_t)L * 4u;
+  const bool edge_cols = __builtin_amdgcn_readfirstlane(j0 + kTile > a.ncols ? 1 : 0) != 0;
+  const char *b_base = reinterpret_cast<const char *>(a.b);
+  float b_scale = 1.0f, b_inverse = 1.0f;
+  const bool per_sample = TB > 1 && a.b_amax_samples != nullptr;
+  if (TB > 1 && !per_sample && a.b_amax != nullptr) scale_for(tensor_amax(a.b_amax), b_scale, b_inverse);
+  const bool two_samples = L >= kTile;
+  const int64_t tile_sample = j0 / L, next_sample_col = (tile_sample + 1) * L;
+  float tile_amax[2] = {0.0f, 0.0f};
+  if (per_sample && two_samples) {
+    const int64_t s_a = a.amax_s0 + tile_sample, s_b = s_a + 1 < a.amax_S ? s_a + 1 : s_a;
+    tile_amax[0] = sample_amax(a.b_amax_samples, s_a);
+    tile_amax[1] = sample_amax(a.b_amax_samples, s_b);
+  }
+  auto column_amax = [&](int64_t j) {
+    return two_samples ? (j < next_sample_col ? tile_amax[0] : tile_amax[1]) : sample_amax(a.b_amax_samples, a.amax_s0 + j / L);
+  };
+  if (per_sample && col_ok) scale_for(column_amax(jc), b_scale, b_inverse);
+
+  u32x4 af[2][TA];  // [ks][term]: the fragments of the step being multiplied, refilled as they are used up
+  u32x4 rb[2][4];   // [set][i]: k row kr + 8 i of a tile, fp32 bit patterns of four columns
+  auto fetch_a = [&](int tile, int ks) {  // every request is unconditional: k steps beyond the last repeat it
+    const int t_ = tile < steps ? tile : steps - 1;
+    const char *src = a_base + (int64_t)t_ * (kTile * kTileK * 2) + ks * 32;
+#pragma unroll
+    for (int ta = 0; ta < TA; ++ta) af[ks][ta] = *reinterpret_cast<const u32x4 *>(src + (int64_t)ta * a.plane_stride * 2 + a_lane);
+  };
+  auto fetch_b = [&](int tile, int set) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = tile * kTileK + kr + 8 * i;
+      rb[set][i] = *reinterpret_cast<const u32x4 *>(b_base + (b_off + (uint32_t)(k < K ? k : K - 1) * row_bytes));
+    }
+  };
+  auto stage = [&](int tile, int set) {
+    uint8_t *Bs = lds + (tile & 1) * kBuf;
+    if (edge_cols || (tile + 1) * kTileK > K) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (!(col_ok && tile * kTileK + kr + 8 * i < K)) rb[set][i] = (u32x4)(0u);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      // (the components go through scalars first: a bit cast applied to a vector component directly reads component 0)
+      const uint32_t u0 = rb[set][i].x, u1 = rb[set][i].y, u2 = rb[set][i].z, u3 = rb[set][i].w;
+      float x0 = __builtin_bit_cast(float, u0), x1 = __builtin_bit_cast(float, u1);
+      float x2 = __builtin_bit_cast(float, u2), x3 = __builtin_bit_cast(float, u3);
+      if (TB > 1) { x0 *= b_scale; x1 *= b_scale; x2 *= b_scale; x3 *= b_scale; }
+      uint32_t w01[TB], w23[TB];
+      split_pair<TB, true>(x0, x1, w01);
+      split_pair<TB, true>(x2, x3, w23);
+#pragma unroll
+      for (int tb = 0; tb < TB; ++tb) {
+        u32x2 v;
+        v.x = w01[tb]; v.y = w23[tb];
+        *reinterpret_cast<u32x2 *>(Bs + tb * kRowPlane + (kr + 8 * i) * kPlanePitch + q4 * 8) = v;
+      }
+    }
+  };
+
+  f32x16 acc[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int q = 0; q < 16; ++q) acc[nt][q] = 0.0f;
+  // the transposing read: group g = lane / 16 fetches columns 16 (g % 2) + 0..15 of the 32, k rows 8 (g / 2) + 0..3 (and
+  // + 4 in the second read) of the 16; lane i of the group points at columns 4 (i % 4) + 0..3 of row i / 4
+  const int tr_g = lane >> 4, tr_i = lane & 15;
+  const uint32_t tr_off = (uint32_t)((8 * (tr_g >> 1) + (tr_i >> 2)) * kPlanePitch + (16 * (tr_g & 1) + 4 * (tr_i & 3)) * 2);
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  auto multiply = [&](int tile, int next_a) {
+    const uint8_t *Bs = lds + (tile & 1) * kBuf + tr_off;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      u32x4 bf[4][TB];
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb) {
+          const uint8_t *src = Bs + tb * kRowPlane + ks * 16 * kPlanePitch + nt * 64;
+          const u32x2 k03 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(src)));
+          const u32x2 k47 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(src + 4 * kPlanePitch)));
+          bf[nt][tb].x = k03.x; bf[nt][tb].y = k03.y; bf[nt][tb].z = k47.x; bf[nt][tb].w = k47.y;
+        }
+      // smallest terms first, as mfma_step
+#pragma unroll
+      for (int order = Pairs<TA, TB>::kMax; order >= 0; --order) {
+#pragma unroll
+        for (int ta = 0; ta < TA; ++ta) {
+          const int tb = order - ta;
+          if (tb < 0 || tb >= TB) continue;
+#pragma unroll
+          for (int nt = 0; nt < 4; ++nt)
+            acc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[ks][ta]),
+                                                              __builtin_bit_cast(f16x8, bf[nt][tb]), acc[nt], 0, 0, 0);
+        }
+      }
+      fetch_a(next_a, ks);
+      __builtin_amdgcn_sched_barrier(0);  // (the requests stay here: left alone, the compiler moves them to the end of the step)
+    }
+  };
+
+  fetch_b(0, 0);
+  fetch_a(0, 0);
+  fetch_a(0, 1);
+  fetch_b(1, 1);
+  stage(0, 0);
+  if (tid < kTile) inverse_lds[tid] = inverse_mine;
+  fetch_b(2, 0);
+  __syncthreads();
+  // step i: tile i + 1 (requested two steps ago) goes into the other LDS buffer, tile i + 3 is requested into the registers
+  // that frees, tile i is multiplied while the A fragments of tile i + 1 replace the ones used up
+  int i = 0;
+  for (; i + 1 < steps; i += 2) {
+    stage(i + 1, 1);
+    fetch_b(i + 3, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(i, i + 1);
+    __syncthreads();
+    if (i + 2 < steps) stage(i + 2, 0);
+    fetch_b(i + 4, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(i + 1, i + 2);
+    __syncthreads();
+  }
+  if (i < steps) {
+    multiply(i, i);
+    __syncthreads();
+  }
+
+  // accumulator register q of a 32 x 32 tile: row 8 (q / 4) + 4 (lane / 32) + q % 4, column lane % 32
+  float b_inv_col[4] = {b_inverse, b_inverse, b_inverse, b_inverse};
+  if (per_sample) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const int64_t j = j0 + nt * 32 + (lane & 31);
+      float unused;
+      b_inv_col[nt] = 1.0f;
+      if (j < a.ncols) scale_for(column_amax(j), unused, b_inv_col[nt]);
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const f32x4 inv4 = *reinterpret_cast<const f32x4 *>(inverse_lds + wave * 32 + 8 * g + 4 * (lane >> 5));
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float inv = e == 0 ? inv4.x : (e == 1 ? inv4.y : (e == 2 ? inv4.z : inv4.w));
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) acc[nt][4 * g + e] = acc[nt][4 * g + e] * inv * b_inv_col[nt];
+    }
+  }
+  // The tile leaves through LDS (the operand tiles are no longer read: the barrier above) in pieces of 32 rows x 64
+  // columns per wavefront, as in pw_gemm_kernel: a store instruction writes four rows of 256 contiguous bytes, and lane i
+  // adds row i of the staged piece for the batch-norm sums, in the same order.
+  float *buf = reinterpret_cast<float *>(lds) + wave * (32 * kOutPitch);
+  const int c4 = 4 * (lane & 15), rsub = lane >> 4;
+  const int wave_row0 = mb * kTile + wave * 32;
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const int64_t j4 = j0 + half * 64 + c4;
+    const bool ok4 = j4 < a.ncols;
+    const int64_t s4 = ok4 ? j4 / L : 0;
+    float *cp4 = a.c + (s4 * M) * (int64_t)L + (ok4 ? (int)(j4 - s4 * L) : 0);
+    __builtin_amdgcn_wave_barrier();  // the piece staged before has been read (LDS serves a wavefront's accesses in order)
+#pragma unroll
+    for (int ntl = 0; ntl < 2; ++ntl)
+#pragma unroll
+      for (int q = 0; q < 16; ++q)
+        buf[(8 * (q >> 2) + 4 * (lane >> 5) + (q & 3)) * kOutPitch + ntl * 32 + (lane & 31)] = acc[2 * half + ntl][q];
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int row_local = 4 * q + rsub;
+      const int row = wave_row0 + row_local;
+      const f32x4 v = *reinterpret_cast<const f32x4 *>(buf + row_local * kOutPitch + c4);
+      if (ok4 && row < M) *reinterpret_cast<f32x4 *>(cp4 + (int64_t)row * L) = v;
+    }
+    if (a.stats && lane < 32) {
+      const float *rowp = buf + lane * kOutPitch;
+      float sum = 0.0f, squares = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const f32x4 v = *reinterpret_cast<const f32x4 *>(rowp + 4 * j);
+        sum += (v.x + v.y) + (v.z + v.w);
+        squares = fmaf(v.x, v.x, squares); squares = fmaf(v.y, v.y, squares);
+        squares = fmaf(v.z, v.z, squares); squares = fmaf(v.w, v.w, squares);
+      }
+      const int row = wave_row0 + lane;
+      if (row < M) {
+        float *out = a.stats + ((2 * nb + half) * (int64_t)M + row) * 2;
+        out[0] = sum;
+        out[1] = squares;
+      }
+    }
+  }
+}
+
 struct PwDwArgs {
   const float *dy;   // [S][M][L]
   const float *x;    // [S][N][L]
@@ -1198,6 +1446,12 @@ int launch_gemm_terms(const PwGemmArgs &a, int64_t blocks, hipStream_t stream) {
   return check_launch("pwconv_gemm");
 }
 
+template <int TB>
+int launch_gemm_rows(const PwGemmArgs &a, int64_t blocks, hipStream_t stream) {
+  hipLaunchKernelGGL((pw_gemm_rows_kernel<TB>), dim3((unsigned)blocks), dim3(kPwThreads), rows_inverse_offset(TB) + kTile * 4, stream, a);
+  return check_launch("pwconv_gemm");
+}
+
 template <int TA, int TB, bool H = false, bool BITS = false>
 int launch_dw_terms(const PwDwArgs &a, int64_t blocks, hipStream_t stream) {
   const unsigned lds = (TA + TB) * kRowPlane;
@@ -1301,6 +1555,13 @@ int launch_pwconv_gemm(const uint16_t *a_planes, int a_terms, int64_t M, int64_t
     const int64_t blocks = a.m_blocks * ((a.ncols + kTile - 1) / kTile);
     if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "pwconv_gemm: %lld blocks", (long long)blocks);
     int rc;
+    // real fp32 activations, positions in fours, everything 16-byte aligned: the kernel that keeps A out of LDS
+    const bool rows_kernel = SJHIP_PW_ROWS != 0 && a_terms == (SJHIP_PW_F16 | 2) && !b_bits && L % 4 == 0 && aligned16(b) && aligned16(c);
+    if (rows_kernel && (b_terms == 1 || b_terms == 2)) {
+      rc = b_terms == 2 ? launch_gemm_rows<2>(a, blocks, stream) : launch_gemm_rows<1>(a, blocks, stream);
+      if (rc != SJHIP_OK) return rc;
+      continue;
+    }
     switch (a_terms * 10 + b_terms) {
       case 33: rc = launch_gemm_terms<3, 3>(a, blocks, stream); break;
       case 31: rc = launch_gemm_terms<3, 1>(a, blocks, stream); break;
