@@ -139,6 +139,28 @@ template <int TERMS, bool H = false> __device__ __forceinline__ void split_pair(
   }
 }
 
+// The terms of (s x0, s x1) for a power of two s, for the kernels' inner loops.  With two fp16 terms the remainder is one
+// fused multiply-add per value, lo = fp16(fma(x, s, -hi)): s x and s x - hi are both exact in fp32, so this is the value
+// that the separate product, conversion back and difference of split_pair give, and it compiles to the mixed-precision
+// instruction that reads hi as fp16 and writes lo as fp16 (five vector instructions per pair of values instead of ten).
+// Otherwise s is not applied (operands of one term, and bf16 terms, are not scaled).
+template <int TERMS, bool H> __device__ __forceinline__ void split_scaled_pair(float x0, float x1, float s, uint32_t (&w)[TERMS]) {
+  if constexpr (H && TERMS == 2) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    f32x2 y;
+    y.x = x0 * s;
+    y.y = x1 * s;
+    const f16x2 hi = __builtin_convertvector(y, f16x2);
+    f16x2 lo;
+    lo.x = (_Float16)__builtin_fmaf(x0, s, -(float)hi.x);
+    lo.y = (_Float16)__builtin_fmaf(x1, s, -(float)hi.y);
+    w[0] = __builtin_bit_cast(uint32_t, hi);
+    w[1] = __builtin_bit_cast(uint32_t, lo);
+  } else {
+    split_pair<TERMS, H>(x0, x1, w);
+  }
+}
+
 // |x| of a number, 0 for an infinity or a NaN: non-finite elements take no part in choosing a scale (they still
 // propagate through the products as they would in fp32).
 __device__ __forceinline__ float finite_abs(float x) {
@@ -537,11 +559,7 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
           x0 = (float)((lo.x >> (lo.y + c)) & 1u);
           x1 = (float)((hi.x >> (hi.y + c)) & 1u);
         }
-        if (H && TB > 1) {
-          x0 *= b_scale;
-          x1 *= b_scale;
-        }
-        split_pair<TB, H>(x0, x1, w[i]);
+        split_scaled_pair<TB, H>(x0, x1, b_scale, w[i]);
       }
 #pragma unroll
       for (int t = 0; t < TB; ++t) {
@@ -824,10 +842,9 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       const uint32_t u0 = rb[set][i].x, u1 = rb[set][i].y, u2 = rb[set][i].z, u3 = rb[set][i].w;
       float x0 = __builtin_bit_cast(float, u0), x1 = __builtin_bit_cast(float, u1);
       float x2 = __builtin_bit_cast(float, u2), x3 = __builtin_bit_cast(float, u3);
-      if (TB > 1) { x0 *= b_scale; x1 *= b_scale; x2 *= b_scale; x3 *= b_scale; }
       uint32_t w01[TB], w23[TB];
-      split_pair<TB, true>(x0, x1, w01);
-      split_pair<TB, true>(x2, x3, w23);
+      split_scaled_pair<TB, true>(x0, x1, b_scale, w01);
+      split_scaled_pair<TB, true>(x2, x3, b_scale, w23);
 #pragma unroll
       for (int tb = 0; tb < TB; ++tb) {
         u32x2 v;
@@ -1107,10 +1124,9 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
       const int off = (rr + 32 * i) * kRowBytes + q4 * 8;
       {
         uint32_t w01[TA], w23[TA];
-        f32x4 v = ra[set][i];
-        if (H && TA > 1) v *= a_scale;
-        split_pair<TA, H>(v.x, v.y, w01);
-        split_pair<TA, H>(v.z, v.w, w23);
+        const f32x4 v = ra[set][i];
+        split_scaled_pair<TA, H>(v.x, v.y, a_scale, w01);
+        split_scaled_pair<TA, H>(v.z, v.w, a_scale, w23);
 #pragma unroll
         for (int t = 0; t < TA; ++t) {
           u32x2 w;
@@ -1130,9 +1146,8 @@ __global__ void __launch_bounds__(kPwThreads) __attribute__((amdgpu_waves_per_eu
           v.z = (float)((four >> 2) & 1u);
           v.w = (float)((four >> 3) & 1u);
         }
-        if (H && TB > 1) v *= b_scale;
-        split_pair<TB, H>(v.x, v.y, w01);
-        split_pair<TB, H>(v.z, v.w, w23);
+        split_scaled_pair<TB, H>(v.x, v.y, b_scale, w01);
+        split_scaled_pair<TB, H>(v.z, v.w, b_scale, w23);
 #pragma unroll
         for (int t = 0; t < TB; ++t) {
           u32x2 w;
