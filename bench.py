@@ -93,6 +93,24 @@ def recorded_traffic():
     return rec if rec.get("kernel_source_sha256") == kernel_source_digest() else None
 
 
+def measure_mfma_ceiling(torch, L, random_operands: bool = True, iterations: int = 20000, repeats: int = 3):
+    """TFLOP/s that the matrix cores sustain on v_mfma_f32_32x32x16_f16 alone (sjhip_mfma_probe: one wavefront per SIMD
+    issuing nothing else, register operands), here and now: the chip lowers its clock under their power draw, by how much
+    depends on the operands, so the published 2.5 PFLOP/s is not what a kernel on real data can be held against."""
+    sink = torch.empty(4096, dtype=torch.float32, device="cuda:0")
+    L.mfma_probe(random_operands, 1, 2000, sink)
+    torch.cuda.synchronize()
+    L.profile_reset()
+    L.profile_enable(True)
+    flop = 0
+    for _ in range(repeats):
+        flop = L.mfma_probe(random_operands, 1, iterations, sink)
+    torch.cuda.synchronize()
+    L.profile_enable(False)
+    n, ms = L.profile_read(L.KC_MFMA_PROBE)
+    return flop / (ms / max(n, 1) * 1e-3) / 1e12
+
+
 def measure_ceilings(torch, L, floats_per_stream: int, repeats: int = 5):
     """GB/s of the library's plain streaming kernel (sjhip_stream_probe) for the access mixes of the neuron kernels,
     over streams of the size of one [T, N] tensor of the workload; best cache policy of the two for each mix."""
@@ -200,7 +218,7 @@ def secondary_measurements(args):
                      "kernel": r["kernel"], "kernel_ms": r["kernel_ms"], "bound": r["bound"], "achieved": r["achieved"],
                      "peak": r["peak"], "roofline_unit": r["unit"], "frac": r["frac"]}
         for extra in ("forward_ms", "backward_ms", "graph_replay_ms_per_step", "fused_forward_packed_ms", "fused_forward_packed_GBs", "gemm_ms_per_step",
-                      "ssa_backward_ms", "ssa_backward_GBs"):
+                      "ssa_backward_ms", "ssa_backward_GBs", "mfma_sustained_random_operands_TFLOPs", "frac_of_sustained"):
             if extra in r:
                 out[name][extra] = r[extra]
     return out
@@ -480,12 +498,15 @@ def other_workload(args) -> int:
         floats = 16 * 256 * 128 * 32 * 32
         t0 = time.perf_counter()
         c = measure_ceilings(torch, L, floats, repeats=args.steps)
+        c["mfma_f16_zero_operands_TFLOPs"] = measure_mfma_ceiling(torch, L, False)
+        c["mfma_f16_random_operands_TFLOPs"] = measure_mfma_ceiling(torch, L, True)
         elapsed = time.perf_counter() - t0
-        top = max(c.values())
+        top = max(v for k, v in c.items() if not k.startswith("mfma"))
         _emit(args, "GB/s of plain fp32 streams (sjhip_stream_probe), 2.1 GB per stream, 1 MI355X", "GB/s", top, elapsed, "f32",
               {"workload": "one 16-byte access per work-item and stream; read-only, write-only, copy and the read:write "
                            "mixes of the neuron kernels (1:2 forward, 1:3 forward saving h_seq, 3:1 backward); best of "
-                           "default and streaming cache policy", **{k: round(v, 1) for k, v in c.items()}},
+                           "default and streaming cache policy; mfma_*: what the matrix cores sustain on "
+                           "v_mfma_f32_32x32x16_f16 alone (sjhip_mfma_probe)", **{k: round(v, 1) for k, v in c.items()}},
               {"bound": "hbm", "achieved": top, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": top / HBM_PEAK_GBS,
                "traffic": None, "kernel": "stream_probe"})
         return 0
@@ -509,6 +530,7 @@ def other_workload(args) -> int:
 
         elapsed = _time_steps(torch, L, step, args.steps, args.warmup)
         g_ms, d_ms = _kernel_ms(L, L.KC_PW_GEMM), _kernel_ms(L, L.KC_PW_GRAD_WEIGHT)
+        sustained = measure_mfma_ceiling(torch, L, True)
         flop = 2.0 * S * Cin * Cout * tokens                      # of one GEMM, counted once per fp32 product
         products = {3: 6, 2: 3, 1: 1, CB.F16 | 2: 3}[terms]      # 16-bit matrix-core products per fp32 product
         split = "2 fp16 terms per scaled operand" if terms & CB.F16 else f"{terms} bf16 terms per operand"
@@ -519,7 +541,9 @@ def other_workload(args) -> int:
                "frac": products * flop / (g_ms * 1e-3) / 1e12 / 2500.0, "traffic": None, "kernel": "pw_gemm",
                "kernel_ms": g_ms, "grad_weight_ms": d_ms,
                "grad_weight_TFLOPs": products * flop / (d_ms * 1e-3) / 1e12,
-               "fp32_equivalent_TFLOPs": flop / (g_ms * 1e-3) / 1e12})
+               "fp32_equivalent_TFLOPs": flop / (g_ms * 1e-3) / 1e12,
+               "mfma_sustained_random_operands_TFLOPs": sustained,
+               "frac_of_sustained": products * flop / (g_ms * 1e-3) / 1e12 / sustained})
         return 0
 
     if args.workload == "config5":
@@ -553,6 +577,7 @@ def other_workload(args) -> int:
         n_d, ms_d = L.profile_read(L.KC_PW_GRAD_WEIGHT)
         gemm_ms_per_step = (ms_g + ms_d) / args.steps
         gemm_tflops = gemm_products / (gemm_ms_per_step * 1e-3) / 1e12 if gemm_ms_per_step else 0.0
+        sustained = measure_mfma_ceiling(torch, L, True)
         cph = D // H
         probs = T * B * H
         n = T * B * D * tokens
@@ -569,6 +594,7 @@ def other_workload(args) -> int:
                "traffic": None, "kernel": "pw_gemm + pw_dw (the six convolution GEMM launches of a step)",
                "kernel_ms": gemm_ms_per_step / max((n_g + n_d) / args.steps, 1), "gemm_ms_per_step": gemm_ms_per_step,
                "gemm_launches_per_step": (n_g + n_d) / args.steps, "gemm_16bit_product_flops_per_step": gemm_products,
+               "mfma_sustained_random_operands_TFLOPs": sustained, "frac_of_sustained": gemm_tflops / sustained,
                "ssa_backward_ms": sb, "ssa_backward_GBs": bytes_b / (sb * 1e-3) / 1e9,
                "ssa_backward_frac_of_hbm": bytes_b / (sb * 1e-3) / 1e9 / HBM_PEAK_GBS, "ssa_backward_bytes": bytes_b,
                "ssa_backward_TFLOPs": 4 * product / (sb * 1e-3) / 1e12,

@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define SJHIP_ABI_VERSION 6
+#define SJHIP_ABI_VERSION 7
 
 typedef enum sjhip_status {
   SJHIP_OK = 0,
@@ -684,10 +684,21 @@ int sjhip_stream_probe(int reads, int writes, int nontemporal, int64_t floats_pe
                        float *const *out, void *stream);
 
 /*
+ * Matrix-core probe: sjhip_mfma_probe_blocks(w) blocks (compute units x w, each four wavefronts, one per SIMD) issue
+ * iterations x 16 v_mfma_f32_32x32x16_f16 per wavefront on register operands and nothing else: 2 x 32 x 32 x 16 flop
+ * per instruction.  operands: 0 all zero, 1 uniform random in [-1, 1) (the clock, and with it the sustained rate,
+ * depends on what the matrix cores are fed).  Every block writes one float to sink (at least that many floats).
+ * No counterpart in the reference: like sjhip_stream_probe it measures, on the device and in the run that quotes it,
+ * the ceiling that the convolution GEMMs' rate is compared with (kernel class 14 of sjhip_profile_read).
+ */
+int64_t sjhip_mfma_probe_blocks(int wavefronts_per_simd);
+int sjhip_mfma_probe(int operands, int wavefronts_per_simd, int iterations, float *sink, int64_t sink_floats, void *stream);
+
+/*
  * Optional per-kernel timing.  While enabled every launch is bracketed by HIP events on its own
  * stream.  sjhip_profile_read() synchronises those events and returns, for kernel class `which`
  * (0 forward, 1 backward, 2 plif-reduce, 3 bit_pack, 4 bit_unpack, 5 ssa forward, 6 ssa backward, 7 pwconv gemm,
- * 8 pwconv grad_weight, 9 bn stats, 10 bn_lif forward, 11 bn_lif backward, 12 bn grad_input, 13 stream probe), the launch count and total
+ * 8 pwconv grad_weight, 9 bn stats, 10 bn_lif forward, 11 bn_lif backward, 12 bn grad_input, 13 stream probe, 14 matrix-core probe), the launch count and total
  * milliseconds since the last sjhip_profile_reset().
  */
 int sjhip_profile_enable(int on);

@@ -14,7 +14,7 @@ from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64
 
 import torch
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 # enums of include/sjhip.h
 NEURON_IF, NEURON_LIF, NEURON_PLIF, NEURON_QIF, NEURON_ILIF, NEURON_EIF = 0, 1, 2, 3, 4, 5
@@ -35,7 +35,8 @@ FLAG_GRAD_STORAGE = 0x1000
 STATIC_WORKSPACE_MAX_NEURONS = 1 << 26
 
 (KC_FORWARD, KC_BACKWARD, KC_PLIF_REDUCE, KC_BIT_PACK, KC_BIT_UNPACK, KC_SSA_FORWARD, KC_SSA_BACKWARD, KC_PW_GEMM,
- KC_PW_GRAD_WEIGHT, KC_BN_STATS, KC_BN_LIF_FORWARD, KC_BN_LIF_BACKWARD, KC_BN_GRAD_INPUT, KC_STREAM_PROBE) = range(14)
+ KC_PW_GRAD_WEIGHT, KC_BN_STATS, KC_BN_LIF_FORWARD, KC_BN_LIF_BACKWARD, KC_BN_GRAD_INPUT, KC_STREAM_PROBE,
+ KC_MFMA_PROBE) = range(15)
 
 EXPORTED_SYMBOLS = (
     "sjhip_abi_version",
@@ -66,6 +67,8 @@ EXPORTED_SYMBOLS = (
     "sjhip_izhikevich_backward",
     "sjhip_izhikevich_backward_replay",
     "sjhip_stream_probe",
+    "sjhip_mfma_probe_blocks",
+    "sjhip_mfma_probe",
     "sjhip_pwconv_planes_elems",
     "sjhip_pwconv_split_weight",
     "sjhip_pwconv_gemm",
@@ -244,6 +247,10 @@ def load() -> ctypes.CDLL:
                                                          + [c_void_p] * 12)
         lib.sjhip_stream_probe.restype = c_int
         lib.sjhip_stream_probe.argtypes = [c_int, c_int, c_int, c_int64, POINTER(c_void_p), POINTER(c_void_p), c_void_p]
+        lib.sjhip_mfma_probe_blocks.restype = c_int64
+        lib.sjhip_mfma_probe_blocks.argtypes = [c_int]
+        lib.sjhip_mfma_probe.restype = c_int
+        lib.sjhip_mfma_probe.argtypes = [c_int, c_int, c_int, c_void_p, c_int64, c_void_p]
         lib.sjhip_ssa_lif_forward_packed.restype = c_int
         lib.sjhip_ssa_lif_forward_packed.argtypes = [c_int, POINTER(NeuronParams), c_int64, c_int64, c_int, c_int, c_int64, c_float] + \
                                                     [c_void_p] * 6
@@ -396,6 +403,16 @@ def aligned16(t: torch.Tensor) -> torch.Tensor:
     """``t`` made contiguous and 16-byte aligned (a fresh allocation always is)."""
     t = t.contiguous()
     return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
+def mfma_probe(random_operands: bool, wavefronts_per_simd: int, iterations: int, sink) -> int:
+    """One launch of the matrix-core probe (see ``sjhip_mfma_probe``); returns the floating-point operations it performs.
+    ``sink`` is an fp32 device tensor of at least ``sjhip_mfma_probe_blocks(wavefronts_per_simd)`` elements."""
+    with torch.cuda.device(sink.device):
+        rc = load().sjhip_mfma_probe(1 if random_operands else 0, wavefronts_per_simd, iterations, sink.data_ptr(), sink.numel(),
+                                     current_stream_ptr(sink.device))
+    check(rc, "mfma_probe")
+    return load().sjhip_mfma_probe_blocks(wavefronts_per_simd) * 4 * iterations * 16 * 2 * 32 * 32 * 16
 
 
 def stream_probe(reads: int, writes: int, nontemporal: bool, inputs, outputs) -> None:

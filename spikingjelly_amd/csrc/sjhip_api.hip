@@ -599,6 +599,14 @@ int sjhip_stream_probe(int reads, int writes, int nontemporal, int64_t floats_pe
   return launch_stream_probe(reads, writes, nontemporal, floats_per_stream, in, out, static_cast<hipStream_t>(stream));
 }
 
+int64_t sjhip_mfma_probe_blocks(int wavefronts_per_simd) {
+  return wavefronts_per_simd >= 1 && wavefronts_per_simd <= 8 ? mfma_probe_blocks(wavefronts_per_simd) : 0;
+}
+
+int sjhip_mfma_probe(int operands, int wavefronts_per_simd, int iterations, float *sink, int64_t sink_floats, void *stream) {
+  return launch_mfma_probe(operands, wavefronts_per_simd, iterations, sink, sink_floats, static_cast<hipStream_t>(stream));
+}
+
 int64_t sjhip_pwconv_planes_elems(int64_t rows, int64_t cols) {
   if (rows < 1 || cols < 1) return 0;
   return pwconv_planes_elems(rows, cols);

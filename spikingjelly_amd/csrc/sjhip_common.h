@@ -292,7 +292,7 @@ inline int column_spread(int64_t row_bytes, int64_t T);
 
 enum KernelClass { KC_FORWARD = 0, KC_BACKWARD = 1, KC_PLIF_REDUCE = 2, KC_BIT_PACK = 3, KC_BIT_UNPACK = 4,
                    KC_SSA_FORWARD = 5, KC_SSA_BACKWARD = 6, KC_PW_GEMM = 7, KC_PW_GRAD_WEIGHT = 8, KC_BN_STATS = 9,
-                   KC_BN_LIF_FORWARD = 10, KC_BN_LIF_BACKWARD = 11, KC_BN_GRAD_INPUT = 12, KC_STREAM_PROBE = 13, KC_COUNT = 14 };
+                   KC_BN_LIF_FORWARD = 10, KC_BN_LIF_BACKWARD = 11, KC_BN_GRAD_INPUT = 12, KC_STREAM_PROBE = 13, KC_MFMA_PROBE = 14, KC_COUNT = 15 };
 
 // Brackets one launch with events when profiling is on; free otherwise.
 class ProfileScope {
@@ -452,6 +452,8 @@ int launch_bit_pack(int dtype, int64_t n, const void *src, uint8_t *dst, hipStre
 int launch_bit_unpack(int dtype, int64_t n, const uint8_t *src, void *dst, hipStream_t stream);
 int launch_stream_probe(int reads, int writes, int nontemporal, int64_t floats_per_stream, const float *const *in,
                         float *const *out, hipStream_t stream);
+int64_t mfma_probe_blocks(int wavefronts_per_simd);
+int launch_mfma_probe(int operands, int wavefronts_per_simd, int iterations, float *sink, int64_t sink_floats, hipStream_t stream);
 int64_t pwconv_planes_elems(int64_t rows, int64_t cols);
 int launch_pwconv_split_weight(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, hipStream_t stream);
 int launch_pwconv_split_weight_f16(const float *w, int64_t rows, int64_t cols, int transpose, uint16_t *planes, float *amax_reset,

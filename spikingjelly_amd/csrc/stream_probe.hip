@@ -29,6 +29,48 @@ template <int R, int W, bool NT> __global__ void __launch_bounds__(256) stream_p
   }
 }
 
+// Matrix-core probe: a wavefront issues 16 v_mfma_f32_32x32x16_f16 per iteration (four operand pairs on four independent
+// accumulators, so no instruction waits for another) and nothing else; one block of four wavefronts per SIMD slot.
+// What it sustains depends on the operands, because the chip lowers its clock under the matrix cores' power draw.
+typedef _Float16 probe_f16x8 __attribute__((ext_vector_type(8)));
+typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ uint32_t probe_hash(uint32_t x) {
+  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+  return x;
+}
+__global__ void __launch_bounds__(256) mfma_probe_kernel(int operands, int iterations, float *sink) {
+  probe_f16x8 a[4], b[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float va = 0.0f, vb = 0.0f;
+      if (operands != 0) {  // uniform in [-1, 1), different for every lane, element and operand
+        va = (float)(probe_hash(blockIdx.x * 977u + threadIdx.x * 31u + s * 8u + i) & 0xffffu) / 32768.0f - 1.0f;
+        vb = (float)(probe_hash(blockIdx.x * 613u + threadIdx.x * 17u + s * 8u + i + 99u) & 0xffffu) / 32768.0f - 1.0f;
+      }
+      a[s][i] = (_Float16)va;
+      b[s][i] = (_Float16)vb;
+    }
+  probe_f32x16 acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
+  for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s], b[(s + i) & 3], acc[i], 0, 0, 0);
+  }
+  float x = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) x += acc[i][r];
+  if (threadIdx.x == 0) sink[blockIdx.x] = x;  // keeps the products alive
+}
+
 template <int R, int W> int launch_probe(const ProbeArgs &a, bool nt, hipStream_t stream) {
   const int64_t blocks = (a.quads + 255) / 256;
   if (blocks > 0x7fffffffLL) return fail(SJHIP_ERR_TOO_LARGE, "stream_probe: %lld words", (long long)a.quads);
@@ -72,6 +114,22 @@ int launch_stream_probe(int reads, int writes, int nontemporal, int64_t floats_p
     case 3 * 4 + 1: return launch_probe<3, 1>(a, nt, stream);
     default: return fail(SJHIP_ERR_UNSUPPORTED, "stream_probe: mix %d reads : %d writes is not instantiated", reads, writes);
   }
+}
+
+int64_t mfma_probe_blocks(int wavefronts_per_simd) {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
+  return (int64_t)cus * wavefronts_per_simd;
+}
+
+int launch_mfma_probe(int operands, int wavefronts_per_simd, int iterations, float *sink, int64_t sink_floats, hipStream_t stream) {
+  if (operands < 0 || operands > 1 || wavefronts_per_simd < 1 || wavefronts_per_simd > 8 || iterations < 1 || iterations > (1 << 24))
+    return fail(SJHIP_ERR_INVALID, "mfma_probe: operands %d (0 zeros, 1 random), %d wavefronts per SIMD (1..8), %d iterations (1..2^24)", operands, wavefronts_per_simd, iterations);
+  const int64_t blocks = mfma_probe_blocks(wavefronts_per_simd);
+  if (!sink || sink_floats < blocks) return fail(SJHIP_ERR_INVALID, "mfma_probe: sink holds %lld floats, %lld blocks write one each", (long long)sink_floats, (long long)blocks);
+  ProfileScope prof(KC_MFMA_PROBE, stream);
+  hipLaunchKernelGGL(mfma_probe_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, operands, iterations, sink);
+  return check_launch("mfma_probe");
 }
 
 }  // namespace sjhip

@@ -414,3 +414,30 @@ def test_replay_path_with_misaligned_and_non_contiguous_input():
     b(xb).backward(g.cuda())
     torch.testing.assert_close(xb.grad.cpu(), xa.grad, rtol=GRAD_RTOL, atol=GRAD_ATOL)
 
+
+
+@pytest.mark.gpu
+def test_matrix_core_probe_runs_and_refuses_bad_arguments():
+    """sjhip_mfma_probe (no counterpart in the reference: the ceiling bench.py holds the convolution GEMMs against) performs
+    the flops it reports, writes one float per block and rejects what it cannot launch."""
+    from spikingjelly_amd.activation_based.hip_kernel import library as L
+    lib = L.load()
+    blocks = lib.sjhip_mfma_probe_blocks(1)
+    assert blocks >= 1 and lib.sjhip_mfma_probe_blocks(2) == 2 * blocks and lib.sjhip_mfma_probe_blocks(0) == 0
+    sink = torch.full((2 * blocks,), float("nan"), device="cuda:0")
+    L.profile_reset()
+    L.profile_enable(True)
+    flop_zero = L.mfma_probe(False, 1, 500, sink)
+    flop_random = L.mfma_probe(True, 2, 500, sink)
+    torch.cuda.synchronize()
+    L.profile_enable(False)
+    n, ms = L.profile_read(L.KC_MFMA_PROBE)
+    assert n == 2 and ms > 0.0
+    assert flop_zero == blocks * 4 * 500 * 16 * 32768 and flop_random == 2 * flop_zero
+    assert torch.isfinite(sink).all()  # every block of the larger launch wrote its float
+    tflops = (flop_zero + flop_random) / (ms * 1e-3) / 1e12
+    assert 100.0 < tflops < 2600.0, tflops  # between a tenth of and the published fp16 peak of an MI355X
+    st = L.current_stream_ptr(torch.device("cuda:0"))
+    for bad in [(2, 1, 10, sink.data_ptr(), sink.numel()), (0, 0, 10, sink.data_ptr(), sink.numel()), (0, 9, 10, sink.data_ptr(), sink.numel()),
+                (0, 1, 0, sink.data_ptr(), sink.numel()), (0, 1, 10, None, sink.numel()), (0, 1, 10, sink.data_ptr(), blocks - 1)]:
+        assert lib.sjhip_mfma_probe(*bad, st) != 0
